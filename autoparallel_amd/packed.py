@@ -1,0 +1,501 @@
+"""Packed structure-of-arrays form of a sharding-search problem.
+
+This is the data format on both sides of the cost engine: the HIP kernels read
+it from HBM, the host builds it from ``{node: OpStrategy}`` (or directly from
+a shape-level generator).  It flattens what the reference keeps as Python
+objects:
+
+* ``DTensorSpec.placements``          -> one byte per mesh dim (``spec_plc``)
+* ``DTensorSpec.tensor_meta``         -> a row of the tensor-meta table
+* ``OpSpec.input_specs / output_specs`` -> runs of spec ids in ``lists``
+* ``strats[node]`` / ``_all_input_nodes(node)[argi]`` -> the edge table
+  (reference: autoparallel/optimize_sharding.py:306-354, 380-398, 481-552)
+
+Placement byte (equality of bytes == Python equality of placements, which is
+what the reference's ``current == target`` test needs,
+autoparallel/cost_models/collective_runtime_estimation.py:157):
+
+    0x00          Replicate
+    0x40 | dim    Shard(dim)                 dim < 64
+    0x80 | id     Partial; id 0 = "sum" (the default ``Partial()``), 1 = "avg",
+                  2 = "min", 3 = "max", 4 = "product", >= 8 interned others
+    0xC0 | id     any other placement class (is_shard/is_replicate/is_partial
+                  all False, e.g. _StridedShard)
+
+Entry layout: edge e owns ``sdst[e] * ssrc[e]`` consecutive entries starting at
+``edge_off[e]``, row-major ``[out_idx][inp_idx]``; edges are ordered by
+(node, argi).  That is the order of the reference's ``walk_over_options``
+(optimize_sharding.py:400-410); ``decision_var_order`` gives the permutation to
+the ``decision_vars`` dict order (node, out_idx, argi, inp_idx; :511-520).
+"""
+from __future__ import annotations
+
+import dataclasses
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import numpy as np
+
+MAX_MESH_DIMS = 4
+MAX_RANK = 8
+
+# ---- placement codes -------------------------------------------------------
+PLC_R = 0x00
+PLC_SHARD = 0x40
+PLC_PARTIAL = 0x80
+PLC_OTHER = 0xC0
+PLC_KIND_MASK = 0xC0
+PLC_ARG_MASK = 0x3F
+
+PARTIAL_SUM = PLC_PARTIAL | 0
+PARTIAL_AVG = PLC_PARTIAL | 1
+_REDUCE_OP_IDS = {"sum": 0, "avg": 1, "min": 2, "max": 3, "product": 4}
+
+
+def shard(dim: int) -> int:
+    assert 0 <= dim < 64
+    return PLC_SHARD | dim
+
+
+def partial(reduce_op: str = "sum") -> int:
+    return PLC_PARTIAL | _REDUCE_OP_IDS[reduce_op]
+
+
+def is_shard(code: int) -> bool:
+    return (code & PLC_KIND_MASK) == PLC_SHARD
+
+
+def is_partial(code: int) -> bool:
+    return (code & PLC_KIND_MASK) == PLC_PARTIAL
+
+
+def is_replicate(code: int) -> bool:
+    return code == PLC_R
+
+
+def plc_str(code: int) -> str:
+    if code == PLC_R:
+        return "R"
+    if is_shard(code):
+        return f"S({code & PLC_ARG_MASK})"
+    if is_partial(code):
+        names = {v: k for k, v in _REDUCE_OP_IDS.items()}
+        return f"P({names.get(code & PLC_ARG_MASK, code & PLC_ARG_MASK)})"
+    return f"X({code & PLC_ARG_MASK})"
+
+
+# ---- dtype codes -----------------------------------------------------------
+# Codes 0..4 are the dtypes the reference's device table prices GEMMs in
+# (autoparallel/cost_models/compute_estimation.py:226-239); anything else has
+# no tflops entry and is only legal on zero-flop nodes.
+DT_F64, DT_F32, DT_F16, DT_BF16, DT_I8, DT_OTHER = 0, 1, 2, 3, 4, 5
+DTYPE_ITEMSIZE = {DT_F64: 8, DT_F32: 4, DT_F16: 2, DT_BF16: 2, DT_I8: 1}
+
+# ---- edge flags ------------------------------------------------------------
+EDGE_HAS_PRODUCER = 1  # comm is computed from specs (else default row kept)
+EDGE_SCORE_TRANSITION = 2  # producer output is a single spec: the plan scorer
+#                            counts a transition (optimize_sharding.py:1097-1104)
+
+# ---- compute programs ------------------------------------------------------
+# A node's compute estimate needs flops and bytes of the op run on the sharded
+# inputs (compute_estimation.py:438-493).  Both are written as small programs
+# over the local (sharded) sizes of the tensor args:
+#   flops  = sum_t coeff_t * prod_j size(arg a_tj, dim d_tj)
+#   out[k] = shape whose dims are each: a constant, size(arg, dim), or the
+#            broadcast of all tensor args at a right-aligned position
+OP_ZERO = 0  # placeholder / get_attr / view / non-OpOverload: cost is int 0
+OP_PROGRAM = 1  # flops and output shapes from the program
+OP_EXPLICIT = 2  # host supplies flops[o], bytes[o] (ops without a closed form)
+
+DIM_CONST = 0  # value
+DIM_ARG = 1  # (arg, dim)
+DIM_BCAST = 2  # right-aligned position (0 = last dim)
+
+
+@dataclasses.dataclass
+class PackedGraph:
+    # mesh
+    mesh_shape: np.ndarray  # int32[ndim]
+    devices_per_host: int
+    # tensor metas
+    meta_rank: np.ndarray  # int32[M]
+    meta_shape: np.ndarray  # int64[M, MAX_RANK]
+    meta_stride: np.ndarray  # int64[M, MAX_RANK]
+    meta_itemsize: np.ndarray  # int32[M]
+    meta_dtype: np.ndarray  # int32[M]
+    # specs
+    spec_meta: np.ndarray  # int32[NSPEC]
+    spec_plc: np.ndarray  # uint8[NSPEC, MAX_MESH_DIMS]
+    # runs of spec ids (-1 = no DTensorSpec at that position)
+    lists: np.ndarray  # int32[L]
+    # nodes
+    node_nstrat: np.ndarray  # int32[N]
+    node_nargs: np.ndarray  # int32[N]   len(strategies[0].input_specs)
+    node_comp_off: np.ndarray  # int64[N+1] prefix sum of node_nstrat
+    node_edge_off: np.ndarray  # int32[N+1] edges of node v, ordered by argi
+    node_op: np.ndarray  # int32[N]   OP_*
+    node_prog_off: np.ndarray  # int64[N]   offset into prog (-1 if none)
+    prog: np.ndarray  # int64[...] compute programs
+    # explicit flops/bytes (OP_EXPLICIT), indexed like the compute vector
+    explicit_flops: Optional[np.ndarray] = None  # int64[sum S]
+    explicit_bytes: Optional[np.ndarray] = None  # int64[sum S]
+    # edges
+    edge_node: np.ndarray = None  # int32[NE] consumer
+    edge_arg: np.ndarray = None  # int32[NE]
+    edge_src_node: np.ndarray = None  # int32[NE] producer or -1
+    edge_sdst: np.ndarray = None  # int32[NE]
+    edge_ssrc: np.ndarray = None  # int32[NE]
+    edge_dst_list: np.ndarray = None  # int64[NE] offset into lists (sdst ids)
+    edge_src_list: np.ndarray = None  # int64[NE] offset into lists (ssrc ids) or -1
+    edge_off: np.ndarray = None  # int64[NE+1]
+    edge_flags: np.ndarray = None  # int32[NE]
+    edge_default_off: np.ndarray = None  # int64[NE] offset into default_vals or -1
+    default_vals: np.ndarray = None  # float64[...]
+    # prefetch-discount mask per edge (producer param-derived or consumer
+    # terminal-derived; optimize_sharding.py:853-860)
+    edge_prefetchable: Optional[np.ndarray] = None  # uint8[NE]
+    # cluster multiplicity per node: 1 + number of linked copies (:883)
+    node_multiplier: Optional[np.ndarray] = None  # int32[N]
+    node_names: Optional[List[str]] = None
+
+    # -- derived sizes -------------------------------------------------------
+    @property
+    def ndim(self) -> int:
+        return int(self.mesh_shape.shape[0])
+
+    @property
+    def num_nodes(self) -> int:
+        return int(self.node_nstrat.shape[0])
+
+    @property
+    def num_edges(self) -> int:
+        return int(self.edge_node.shape[0])
+
+    @property
+    def num_entries(self) -> int:
+        return int(self.edge_off[-1])
+
+    @property
+    def num_compute(self) -> int:
+        return int(self.node_comp_off[-1])
+
+    def entry_keys(self) -> np.ndarray:
+        """int32[E, 4] keys (node_idx, argi, out_idx, inp_idx) in entry order
+        (the key layout of autoparallel/serialization.py:150-157)."""
+        E = self.num_entries
+        sizes = (self.edge_sdst.astype(np.int64) * self.edge_ssrc).astype(np.int64)
+        eid = np.repeat(np.arange(self.num_edges, dtype=np.int64), sizes)
+        local = np.arange(E, dtype=np.int64) - self.edge_off[:-1][eid]
+        ssrc = self.edge_ssrc[eid].astype(np.int64)
+        keys = np.empty((E, 4), dtype=np.int32)
+        keys[:, 0] = self.edge_node[eid]
+        keys[:, 1] = self.edge_arg[eid]
+        keys[:, 2] = local // ssrc
+        keys[:, 3] = local % ssrc
+        return keys
+
+    def decision_var_order(self) -> np.ndarray:
+        """Permutation p such that entries[p] is in the reference's
+        ``decision_vars`` insertion order: node, out_idx, argi, inp_idx
+        (optimize_sharding.py:511-520)."""
+        k = self.entry_keys().astype(np.int64)
+        return np.lexsort((k[:, 3], k[:, 1], k[:, 2], k[:, 0]))
+
+    def validate(self) -> None:
+        """Host-side shape checks run before any kernel launch: every index a
+        kernel dereferences must be in range."""
+        nd = self.ndim
+        assert 1 <= nd <= MAX_MESH_DIMS
+        assert (self.mesh_shape >= 1).all()
+        M = self.meta_rank.shape[0]
+        assert self.meta_shape.shape == (M, MAX_RANK)
+        assert self.meta_stride.shape == (M, MAX_RANK)
+        assert ((self.meta_rank >= 0) & (self.meta_rank <= MAX_RANK)).all()
+        nspec = self.spec_meta.shape[0]
+        assert self.spec_plc.shape == (nspec, MAX_MESH_DIMS)
+        if nspec:
+            assert self.spec_meta.min() >= 0 and self.spec_meta.max() < M
+            sh = (self.spec_plc & PLC_KIND_MASK) == PLC_SHARD
+            dims = (self.spec_plc & PLC_ARG_MASK).astype(np.int32)
+            rank = self.meta_rank[self.spec_meta][:, None]
+            assert (~sh | (dims < rank)).all(), "Shard(dim) out of tensor rank"
+            assert (self.spec_plc[:, nd:] == 0).all()
+        L = self.lists.shape[0]
+        if L:
+            assert self.lists.min() >= -1 and self.lists.max() < nspec
+        N, NE = self.num_nodes, self.num_edges
+        assert self.node_comp_off.shape == (N + 1,)
+        assert self.node_edge_off.shape == (N + 1,)
+        assert int(self.node_edge_off[-1]) == NE
+        assert self.edge_off.shape == (NE + 1,)
+        if NE:
+            assert (self.edge_sdst >= 1).all() and (self.edge_ssrc >= 1).all()
+            sizes = self.edge_sdst.astype(np.int64) * self.edge_ssrc
+            assert (np.diff(self.edge_off) == sizes).all()
+            assert (self.edge_dst_list >= 0).all()
+            assert (self.edge_dst_list + self.edge_sdst <= L).all()
+            hp = (self.edge_flags & EDGE_HAS_PRODUCER) != 0
+            assert (self.edge_src_list[hp] >= 0).all()
+            assert (self.edge_src_list[hp] + self.edge_ssrc[hp] <= L).all()
+            assert (self.edge_sdst == self.node_nstrat[self.edge_node]).all()
+            src = self.edge_src_node[hp]
+            assert (src >= 0).all() and (src < N).all()
+            assert (self.edge_ssrc[hp] == self.node_nstrat[src]).all()
+            # entries whose spec is missing need a default value
+            need_default = ~hp
+            assert (self.edge_default_off[need_default] >= 0).all()
+            d = self.edge_default_off >= 0
+            assert (
+                self.edge_default_off[d] + sizes[d] <= self.default_vals.shape[0]
+            ).all()
+        assert (np.diff(self.node_comp_off) == self.node_nstrat).all()
+
+
+# ---------------------------------------------------------------------------
+# Builder: strategy-level description -> PackedGraph
+# ---------------------------------------------------------------------------
+TensorMetaT = Tuple[Tuple[int, ...], Tuple[int, ...], int, int]  # shape, stride, itemsize, dtype
+
+
+@dataclasses.dataclass
+class NodeDesc:
+    """One graph node with its strategies, as the packer consumes it.
+
+    ``in_specs[o][a]`` / ``out_specs[o][k]`` are spec ids from
+    :meth:`GraphBuilder.spec` (or -1 where the reference has ``None`` or a
+    non-``DTensorSpec``).  ``inputs[a]`` is the producer node index of arg a
+    (what ``_all_input_nodes(node)[a]`` returns), ``out_index`` the element of
+    a tuple-producing producer that ``operator.getitem`` selects.
+    """
+
+    name: str
+    in_specs: List[List[int]]
+    out_specs: List[List[int]]
+    inputs: List[int]
+    getitem_index: Optional[int] = None
+    op: int = OP_ZERO
+    program: Optional[List[int]] = None
+    default_rows: Optional[List[List[List[float]]]] = None  # [o][a][j]
+    flops: Optional[List[int]] = None
+    nbytes: Optional[List[int]] = None
+    tuple_output: bool = False  # output_specs is a tuple (not a single spec)
+    nargs: Optional[int] = None
+
+
+class GraphBuilder:
+    def __init__(self, mesh_shape: Sequence[int], devices_per_host: int = 8):
+        self.mesh_shape = tuple(int(x) for x in mesh_shape)
+        assert 1 <= len(self.mesh_shape) <= MAX_MESH_DIMS
+        self.devices_per_host = int(devices_per_host)
+        self._metas: Dict[TensorMetaT, int] = {}
+        self._meta_rows: List[TensorMetaT] = []
+        self._specs: Dict[Tuple[int, Tuple[int, ...]], int] = {}
+        self._spec_rows: List[Tuple[int, Tuple[int, ...]]] = []
+        self.nodes: List[NodeDesc] = []
+        self.prefetchable_edges: set = set()  # (node_idx, argi)
+        self.multiplier: Dict[int, int] = {}
+
+    def meta(self, shape, stride, itemsize: int, dtype: int) -> int:
+        key = (tuple(int(s) for s in shape), tuple(int(s) for s in stride), int(itemsize), int(dtype))
+        assert len(key[0]) == len(key[1]) <= MAX_RANK
+        i = self._metas.get(key)
+        if i is None:
+            i = len(self._meta_rows)
+            self._metas[key] = i
+            self._meta_rows.append(key)
+        return i
+
+    def spec(self, meta_id: int, placements: Sequence[int]) -> int:
+        key = (int(meta_id), tuple(int(p) for p in placements))
+        assert len(key[1]) == len(self.mesh_shape)
+        i = self._specs.get(key)
+        if i is None:
+            i = len(self._spec_rows)
+            self._specs[key] = i
+            self._spec_rows.append(key)
+        return i
+
+    def spec_placements(self, spec_id: int) -> Tuple[int, ...]:
+        return self._spec_rows[spec_id][1]
+
+    def spec_meta_row(self, spec_id: int) -> TensorMetaT:
+        return self._meta_rows[self._spec_rows[spec_id][0]]
+
+    def add_node(self, node: NodeDesc) -> int:
+        self.nodes.append(node)
+        return len(self.nodes) - 1
+
+    def pack(self) -> PackedGraph:
+        nd = len(self.mesh_shape)
+        M = len(self._meta_rows)
+        meta_rank = np.zeros(M, np.int32)
+        meta_shape = np.ones((M, MAX_RANK), np.int64)
+        meta_stride = np.zeros((M, MAX_RANK), np.int64)
+        meta_itemsize = np.zeros(M, np.int32)
+        meta_dtype = np.zeros(M, np.int32)
+        for i, (shape, stride, itemsize, dtype) in enumerate(self._meta_rows):
+            r = len(shape)
+            meta_rank[i] = r
+            meta_shape[i, :r] = shape
+            meta_stride[i, :r] = stride
+            meta_itemsize[i] = itemsize
+            meta_dtype[i] = dtype
+        ns = len(self._spec_rows)
+        spec_meta = np.zeros(ns, np.int32)
+        spec_plc = np.zeros((ns, MAX_MESH_DIMS), np.uint8)
+        for i, (m, plc) in enumerate(self._spec_rows):
+            spec_meta[i] = m
+            spec_plc[i, :nd] = plc
+
+        N = len(self.nodes)
+        lists: List[int] = []
+        node_nstrat = np.zeros(N, np.int32)
+        node_nargs = np.zeros(N, np.int32)
+        node_op = np.zeros(N, np.int32)
+        node_prog_off = np.full(N, -1, np.int64)
+        node_edge_off = np.zeros(N + 1, np.int32)
+        prog: List[int] = []
+        # per node, per output index: offset of its run of output spec ids
+        out_runs: List[Dict[int, int]] = []
+        e_node, e_arg, e_src, e_sdst, e_ssrc = [], [], [], [], []
+        e_dst_list, e_src_list, e_flags, e_def = [], [], [], []
+        defaults: List[float] = []
+        any_explicit = False
+        for v, nd_ in enumerate(self.nodes):
+            S = len(nd_.in_specs)
+            assert S == len(nd_.out_specs) and S >= 1
+            node_nstrat[v] = S
+            node_nargs[v] = nd_.nargs if nd_.nargs is not None else len(nd_.in_specs[0])
+            node_op[v] = nd_.op
+            if nd_.program is not None:
+                node_prog_off[v] = len(prog)
+                prog.extend(int(x) for x in nd_.program)
+            if nd_.op == OP_EXPLICIT:
+                any_explicit = True
+            nout = len(nd_.out_specs[0])
+            runs = {}
+            for k in range(nout):
+                runs[k] = len(lists)
+                lists.extend(nd_.out_specs[o][k] for o in range(S))
+            out_runs.append(runs)
+            # edges: one per row of redistribute_cost (== per arg)
+            n_rows = len(nd_.in_specs[0])
+            if nd_.default_rows is not None:
+                n_rows = len(nd_.default_rows[0])
+            node_edge_off[v] = len(e_node)
+            for a in range(n_rows):
+                has_prod = a < len(nd_.inputs) and nd_.inputs[a] is not None and nd_.inputs[a] >= 0
+                e_node.append(v)
+                e_arg.append(a)
+                e_sdst.append(S)
+                e_dst_list.append(len(lists))
+                lists.extend(
+                    (nd_.in_specs[o][a] if a < len(nd_.in_specs[o]) else -1) for o in range(S)
+                )
+                flags = 0
+                if has_prod:
+                    u = nd_.inputs[a]
+                    assert u < v, "producers must precede consumers"
+                    prod = self.nodes[u]
+                    k = nd_.getitem_index if nd_.getitem_index is not None else 0
+                    if prod.tuple_output and nd_.getitem_index is None:
+                        # tuple-valued producer consumed directly: not a
+                        # DTensorSpec -> default row kept (:473)
+                        src_run = -1
+                    else:
+                        src_run = out_runs[u][k]
+                    ssrc = len(prod.in_specs)
+                    e_src.append(u)
+                    e_ssrc.append(ssrc)
+                    if src_run >= 0:
+                        flags |= EDGE_HAS_PRODUCER
+                    if not prod.tuple_output:
+                        flags |= EDGE_SCORE_TRANSITION
+                    e_src_list.append(src_run)
+                else:
+                    e_src.append(-1)
+                    ssrc = (
+                        len(nd_.default_rows[0][a]) if nd_.default_rows is not None else 1
+                    )
+                    e_ssrc.append(ssrc)
+                    e_src_list.append(-1)
+                need_default = (flags & EDGE_HAS_PRODUCER) == 0 or any(
+                    (a >= len(nd_.in_specs[o]) or nd_.in_specs[o][a] < 0) for o in range(S)
+                ) or (
+                    (flags & EDGE_HAS_PRODUCER)
+                    and any(
+                        lists[e_src_list[-1] + j] < 0 for j in range(e_ssrc[-1])
+                    )
+                )
+                if need_default:
+                    e_def.append(len(defaults))
+                    for o in range(S):
+                        if nd_.default_rows is not None:
+                            row = nd_.default_rows[o][a]
+                            assert len(row) == e_ssrc[-1]
+                            defaults.extend(float(x) for x in row)
+                        else:
+                            defaults.extend([0.0] * e_ssrc[-1])
+                else:
+                    e_def.append(-1)
+                e_flags.append(flags)
+        node_edge_off[N] = len(e_node)
+        NE = len(e_node)
+        edge_sdst = np.asarray(e_sdst, np.int32)
+        edge_ssrc = np.asarray(e_ssrc, np.int32)
+        edge_off = np.zeros(NE + 1, np.int64)
+        np.cumsum(edge_sdst.astype(np.int64) * edge_ssrc, out=edge_off[1:])
+        node_comp_off = np.zeros(N + 1, np.int64)
+        np.cumsum(node_nstrat, out=node_comp_off[1:])
+        pref = np.zeros(NE, np.uint8)
+        for i, (v, a) in enumerate(zip(e_node, e_arg)):
+            if (v, a) in self.prefetchable_edges:
+                pref[i] = 1
+        mult = np.ones(N, np.int32)
+        for v, m in self.multiplier.items():
+            mult[v] = m
+        ef = eb = None
+        if any_explicit:
+            ef = np.zeros(int(node_comp_off[-1]), np.int64)
+            eb = np.zeros(int(node_comp_off[-1]), np.int64)
+            for v, nd_ in enumerate(self.nodes):
+                if nd_.op == OP_EXPLICIT:
+                    o0 = int(node_comp_off[v])
+                    ef[o0 : o0 + len(nd_.flops)] = nd_.flops
+                    eb[o0 : o0 + len(nd_.nbytes)] = nd_.nbytes
+        g = PackedGraph(
+            mesh_shape=np.asarray(self.mesh_shape, np.int32),
+            devices_per_host=self.devices_per_host,
+            meta_rank=meta_rank,
+            meta_shape=meta_shape,
+            meta_stride=meta_stride,
+            meta_itemsize=meta_itemsize,
+            meta_dtype=meta_dtype,
+            spec_meta=spec_meta,
+            spec_plc=spec_plc,
+            lists=np.asarray(lists, np.int32),
+            node_nstrat=node_nstrat,
+            node_nargs=node_nargs,
+            node_comp_off=node_comp_off,
+            node_edge_off=node_edge_off,
+            node_op=node_op,
+            node_prog_off=node_prog_off,
+            prog=np.asarray(prog, np.int64),
+            explicit_flops=ef,
+            explicit_bytes=eb,
+            edge_node=np.asarray(e_node, np.int32),
+            edge_arg=np.asarray(e_arg, np.int32),
+            edge_src_node=np.asarray(e_src, np.int32),
+            edge_sdst=edge_sdst,
+            edge_ssrc=edge_ssrc,
+            edge_dst_list=np.asarray(e_dst_list, np.int64),
+            edge_src_list=np.asarray(e_src_list, np.int64),
+            edge_off=edge_off,
+            edge_flags=np.asarray(e_flags, np.int32),
+            edge_default_off=np.asarray(e_def, np.int64),
+            default_vals=np.asarray(defaults, np.float64),
+            edge_prefetchable=pref,
+            node_multiplier=mult,
+            node_names=[n.name for n in self.nodes],
+        )
+        g.validate()
+        return g
