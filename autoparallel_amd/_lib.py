@@ -1,0 +1,127 @@
+"""ctypes binding of libapc_hip.so (the C ABI declared in include/apc.h).
+
+There is no fallback: if the library is missing, loading raises.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libapc_hip.so")
+
+MAX_MESH_DIMS = 4
+NUM_DTYPES = 8
+
+
+class ApcModel(C.Structure):
+    _fields_ = [
+        ("ndim", C.c_int32),
+        ("mesh_shape", C.c_int32 * MAX_MESH_DIMS),
+        ("mesh_bw", C.c_double * MAX_MESH_DIMS),
+        ("mesh_lat", C.c_double * MAX_MESH_DIMS),
+        ("gmem_bw", C.c_double),
+        ("tflops", C.c_double * NUM_DTYPES),
+    ]
+
+
+class ApcProblem(C.Structure):
+    _fields_ = [
+        ("model", ApcModel),
+        ("n_meta", C.c_int32),
+        ("meta_rank", C.c_void_p),
+        ("meta_shape", C.c_void_p),
+        ("meta_stride", C.c_void_p),
+        ("meta_itemsize", C.c_void_p),
+        ("meta_dtype", C.c_void_p),
+        ("n_tuple", C.c_int32),
+        ("tuple_plc", C.c_void_p),
+        ("n_list", C.c_int64),
+        ("lists", C.c_void_p),
+        ("n_node", C.c_int32),
+        ("node_nstrat", C.c_void_p),
+        ("node_nargs", C.c_void_p),
+        ("node_op", C.c_void_p),
+        ("node_comp_off", C.c_void_p),
+        ("node_edge_off", C.c_void_p),
+        ("node_prog_off", C.c_void_p),
+        ("node_multiplier", C.c_void_p),
+        ("n_prog", C.c_int64),
+        ("prog", C.c_void_p),
+        ("explicit_flops", C.c_void_p),
+        ("explicit_bytes", C.c_void_p),
+        ("n_edge", C.c_int32),
+        ("edges", C.c_void_p),
+        ("n_entry", C.c_int64),
+        ("n_tile", C.c_int32),
+        ("tile_edge", C.c_void_p),
+        ("n_default", C.c_int64),
+        ("default_vals", C.c_void_p),
+    ]
+
+
+_SIGNATURES = {
+    "apc_version": (C.c_int, []),
+    "apc_last_error": (C.c_char_p, []),
+    "apc_mesh_topology": (C.c_int, [C.c_void_p, C.c_int32, C.c_int32, C.c_void_p, C.c_void_p]),
+    "apc_device_limits": (C.c_int, [C.c_char_p, C.POINTER(ApcModel)]),
+    "apc_pair_table_size": (C.c_int64, [C.POINTER(ApcProblem)]),
+    "apc_build_pair_table": (C.c_int, [C.POINTER(ApcProblem), C.c_void_p, C.c_void_p]),
+    "apc_node_compute_costs": (
+        C.c_int, [C.POINTER(ApcProblem), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
+    "apc_edge_costs": (
+        C.c_int,
+        [C.POINTER(ApcProblem), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+         C.c_int32, C.c_void_p]),
+    "apc_apply_prefetch_discount": (
+        C.c_int,
+        [C.POINTER(ApcProblem), C.c_void_p, C.c_double, C.c_void_p, C.c_void_p, C.c_void_p,
+         C.c_void_p, C.c_void_p]),
+    "apc_objective_coeffs": (C.c_int, [C.POINTER(ApcProblem), C.c_void_p, C.c_void_p, C.c_void_p]),
+    "apc_score_assignments": (
+        C.c_int,
+        [C.POINTER(ApcProblem), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+         C.c_int64, C.c_void_p, C.c_void_p]),
+    "apc_score_random_assignments": (
+        C.c_int,
+        [C.POINTER(ApcProblem), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint64,
+         C.c_int64, C.c_int64, C.c_void_p, C.c_void_p]),
+    "apc_random_assignment": (C.c_uint32, [C.c_uint64, C.c_int64, C.c_int32, C.c_int32]),
+    "apc_enumerate_input_options": (
+        C.c_int,
+        [C.POINTER(ApcModel), C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+         C.c_void_p, C.c_void_p]),
+}
+
+EXPORTED_SYMBOLS = tuple(_SIGNATURES)
+
+_lib = None
+
+
+class ApcError(RuntimeError):
+    pass
+
+
+def load() -> C.CDLL:
+    """Load libapc_hip.so; raise (never fall back) if it is not built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise ApcError(
+            f"{LIB_PATH} is missing: build it with `python -m autoparallel_amd.csrc.build` "
+            "(hipcc, gfx950). There is no CPU fallback."
+        )
+    lib = C.CDLL(LIB_PATH)
+    for name, (res, args) in _SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    _lib = lib
+    return lib
+
+
+def check(rc: int, what: str) -> None:
+    if rc != 0:
+        msg = load().apc_last_error().decode(errors="replace")
+        raise ApcError(f"{what} failed ({rc}): {msg}")

@@ -1,0 +1,255 @@
+"""Host driver of the HIP cost engine: holds a packed problem in HBM and runs
+the kernels through the C ABI.  PyTorch is used only for device memory and the
+current HIP stream."""
+from __future__ import annotations
+
+import ctypes as C
+from typing import Dict, Optional
+
+import numpy as np
+import torch
+
+from . import _lib
+from .packed import MAX_MESH_DIMS, PackedGraph, TILE_SHIFT
+
+# Build the pair table when it is at most this many times the entry count (and
+# small in absolute terms); otherwise every entry is evaluated directly.
+_TABLE_MAX_RATIO = 1.0
+_TABLE_MAX_DOUBLES = 1 << 28
+
+
+def make_model(mesh_shape, devices_per_host: int, device_name: str) -> _lib.ApcModel:
+    """Cost-model constants for a mesh on a named device (raises ApcError for a
+    device the reference's table does not know either)."""
+    lib = _lib.load()
+    m = _lib.ApcModel()
+    nd = len(mesh_shape)
+    assert 1 <= nd <= MAX_MESH_DIMS
+    m.ndim = nd
+    shape = (C.c_int32 * MAX_MESH_DIMS)(*([int(x) for x in mesh_shape] + [1] * (MAX_MESH_DIMS - nd)))
+    m.mesh_shape = shape
+    bw = (C.c_double * MAX_MESH_DIMS)()
+    lat = (C.c_double * MAX_MESH_DIMS)()
+    _lib.check(
+        lib.apc_mesh_topology(C.addressof(shape), nd, int(devices_per_host), C.addressof(bw), C.addressof(lat)),
+        "apc_mesh_topology",
+    )
+    m.mesh_bw = bw
+    m.mesh_lat = lat
+    _lib.check(lib.apc_device_limits(device_name.encode(), C.byref(m)), "apc_device_limits")
+    return m
+
+
+def detect_device_name(device=None) -> str:
+    """Marketing name of the HIP device, as the reference's device table keys
+    on it (autoparallel/cost_models/compute_estimation.py:258-275).  Hosts
+    without the amdgpu id database report every card as "AMD Radeon Graphics";
+    the architecture name then decides (gfx950 is MI355X)."""
+    name = torch.cuda.get_device_name(device)
+    if "Instinct" not in name:
+        arch = getattr(torch.cuda.get_device_properties(device), "gcnArchName", "")
+        if arch.startswith("gfx950"):
+            return "AMD Instinct MI355X"
+        if arch.startswith("gfx942"):
+            return "AMD Instinct MI300X"
+    return name
+
+
+class CostEngine:
+    def __init__(
+        self,
+        g: PackedGraph,
+        device: str = "cuda",
+        device_name: Optional[str] = None,
+        use_table: Optional[bool] = None,
+    ):
+        self.lib = _lib.load()
+        self.g = g
+        self.device = torch.device(device)
+        if self.device.type != "cuda":
+            raise _lib.ApcError("CostEngine needs a HIP device; there is no CPU path")
+        if device_name is None:
+            device_name = detect_device_name(self.device)
+        self.device_name = device_name
+        g.validate()
+        sizes = g.edge_sdst.astype(np.int64) * g.edge_ssrc
+        assert g.num_edges == 0 or int(sizes.max()) < 2**31, "edge block too large for 32-bit local index"
+
+        self._keep: Dict[str, torch.Tensor] = {}
+
+        def up(name, arr, dtype=None):
+            a = np.ascontiguousarray(arr if dtype is None else arr.astype(dtype))
+            if a.dtype == np.uint32:
+                t = torch.from_numpy(a.view(np.int32)).to(self.device)
+            elif a.dtype.fields is not None:
+                t = torch.from_numpy(a.view(np.uint8)).to(self.device)
+            else:
+                t = torch.from_numpy(a).to(self.device)
+            self._keep[name] = t
+            return t.data_ptr() if t.numel() else None
+
+        p = _lib.ApcProblem()
+        p.model = make_model([int(x) for x in g.mesh_shape], g.devices_per_host, device_name)
+        p.n_meta = g.meta_rank.shape[0]
+        p.meta_rank = up("meta_rank", g.meta_rank)
+        p.meta_shape = up("meta_shape", g.meta_shape)
+        p.meta_stride = up("meta_stride", g.meta_stride)
+        p.meta_itemsize = up("meta_itemsize", g.meta_itemsize)
+        p.meta_dtype = up("meta_dtype", g.meta_dtype)
+        p.n_tuple = g.tuple_plc.shape[0]
+        p.tuple_plc = up("tuple_plc", g.tuple_plc)
+        p.n_list = g.lists.shape[0]
+        p.lists = up("lists", g.lists)
+        p.n_node = g.num_nodes
+        p.node_nstrat = up("node_nstrat", g.node_nstrat)
+        p.node_nargs = up("node_nargs", g.node_nargs)
+        p.node_op = up("node_op", g.node_op)
+        p.node_comp_off = up("node_comp_off", g.node_comp_off)
+        p.node_edge_off = up("node_edge_off", g.node_edge_off)
+        p.node_prog_off = up("node_prog_off", g.node_prog_off)
+        mult = g.node_multiplier if g.node_multiplier is not None else np.ones(g.num_nodes, np.int32)
+        p.node_multiplier = up("node_multiplier", mult)
+        p.n_prog = g.prog.shape[0]
+        p.prog = up("prog", g.prog)
+        p.explicit_flops = up("explicit_flops", g.explicit_flops) if g.explicit_flops is not None else None
+        p.explicit_bytes = up("explicit_bytes", g.explicit_bytes) if g.explicit_bytes is not None else None
+        p.n_edge = g.num_edges
+        p.edges = up("edges", g.edge_records())
+        p.n_entry = g.num_entries
+        tile_edge = g.tile_edge_index()
+        p.n_tile = tile_edge.shape[0]
+        assert p.n_tile == (g.num_entries + (1 << TILE_SHIFT) - 1) >> TILE_SHIFT
+        p.tile_edge = up("tile_edge", tile_edge)
+        p.n_default = g.default_vals.shape[0]
+        p.default_vals = up("default_vals", g.default_vals)
+        self.problem = p
+
+        E, NC = g.num_entries, g.num_compute
+        self.compute = torch.empty(NC, dtype=torch.float64, device=self.device)
+        self.per_arg = torch.empty(NC, dtype=torch.float64, device=self.device)
+        self.comm = torch.empty(E, dtype=torch.float64, device=self.device)
+        self.cost = torch.empty(E, dtype=torch.float64, device=self.device)
+        self.flags = torch.empty(E, dtype=torch.uint8, device=self.device)
+        self.status = torch.zeros(1, dtype=torch.int32, device=self.device)
+        tsize = int(self.lib.apc_pair_table_size(C.byref(p)))
+        if use_table is None:
+            use_table = tsize <= _TABLE_MAX_DOUBLES and tsize <= max(_TABLE_MAX_RATIO * E, 1 << 16)
+        self.use_table = bool(use_table)
+        self.table = (
+            torch.empty(tsize, dtype=torch.float64, device=self.device) if self.use_table else None
+        )
+        self.built = False
+
+    # -- raw stream -----------------------------------------------------------
+    def _stream(self):
+        return C.c_void_p(torch.cuda.current_stream(self.device).cuda_stream)
+
+    @staticmethod
+    def _ptr(t: Optional[torch.Tensor]):
+        return None if t is None or t.numel() == 0 else C.c_void_p(t.data_ptr())
+
+    # -- kernels --------------------------------------------------------------
+    def build_pair_table(self):
+        if self.table is not None:
+            _lib.check(
+                self.lib.apc_build_pair_table(C.byref(self.problem), self._ptr(self.table), self._stream()),
+                "apc_build_pair_table",
+            )
+
+    def node_compute(self):
+        _lib.check(
+            self.lib.apc_node_compute_costs(
+                C.byref(self.problem), self._ptr(self.compute), self._ptr(self.per_arg),
+                self._ptr(self.status), self._stream()),
+            "apc_node_compute_costs",
+        )
+
+    def edge_costs(self, clamp_inf: bool = True, want_comm: bool = True, want_flags: bool = True):
+        _lib.check(
+            self.lib.apc_edge_costs(
+                C.byref(self.problem), self._ptr(self.table), self._ptr(self.per_arg),
+                self._ptr(self.comm) if want_comm else None, self._ptr(self.cost),
+                self._ptr(self.flags) if want_flags else None, int(bool(clamp_inf)), self._stream()),
+            "apc_edge_costs",
+        )
+
+    def build(self, clamp_inf: bool = True):
+        """All coefficients: pair table, node compute vectors, entry arrays."""
+        self.build_pair_table()
+        self.node_compute()
+        self.edge_costs(clamp_inf)
+        self.built = True
+        return self
+
+    def check_status(self):
+        if int(self.status.item()) != 0:
+            raise ValueError(
+                "a node with flops has an input dtype without a tflops entry on "
+                f"{self.device_name} (the reference raises ValueError for it)"
+            )
+
+    def apply_prefetch_discount(self, scale: float = 0.0) -> int:
+        assert self.built
+        n = torch.zeros(1, dtype=torch.int64, device=self.device)
+        _lib.check(
+            self.lib.apc_apply_prefetch_discount(
+                C.byref(self.problem), self._ptr(self.per_arg), float(scale), self._ptr(self.comm),
+                self._ptr(self.cost), self._ptr(self.flags), self._ptr(n), self._stream()),
+            "apc_apply_prefetch_discount",
+        )
+        return int(n.item())
+
+    def objective_coeffs(self) -> torch.Tensor:
+        assert self.built
+        obj = torch.empty_like(self.cost)
+        _lib.check(
+            self.lib.apc_objective_coeffs(C.byref(self.problem), self._ptr(self.cost), self._ptr(obj), self._stream()),
+            "apc_objective_coeffs",
+        )
+        return obj
+
+    def score(self, assign: torch.Tensor) -> torch.Tensor:
+        """assign: uint16/int16 [n_node, n_assign] on the device -> float64 [n_assign, 6]."""
+        assert self.built
+        assert assign.dim() == 2 and assign.shape[0] == self.g.num_nodes and assign.is_contiguous()
+        assert assign.dtype in (torch.int16, torch.uint16) and assign.device == self.comm.device
+        A = assign.shape[1]
+        out = torch.empty((A, 6), dtype=torch.float64, device=self.device)
+        _lib.check(
+            self.lib.apc_score_assignments(
+                C.byref(self.problem), self._ptr(self.per_arg), self._ptr(self.comm), self._ptr(self.cost),
+                self._ptr(self.flags), self._ptr(assign), A, self._ptr(out), self._stream()),
+            "apc_score_assignments",
+        )
+        return out
+
+    def score_random(self, seed: int, first: int, count: int) -> torch.Tensor:
+        assert self.built
+        out = torch.empty((count, 6), dtype=torch.float64, device=self.device)
+        _lib.check(
+            self.lib.apc_score_random_assignments(
+                C.byref(self.problem), self._ptr(self.per_arg), self._ptr(self.comm), self._ptr(self.cost),
+                self._ptr(self.flags), int(seed), int(first), int(count), self._ptr(out), self._stream()),
+            "apc_score_random_assignments",
+        )
+        return out
+
+    def random_assignment(self, seed: int, a: int) -> np.ndarray:
+        """The out_idx per node that score_random draws for assignment a."""
+        g = self.g
+        return np.asarray(
+            [self.lib.apc_random_assignment(int(seed), int(a), v, int(g.node_nstrat[v])) for v in range(g.num_nodes)],
+            dtype=np.int64,
+        )
+
+    # -- results on host --------------------------------------------------------
+    def results(self) -> Dict[str, np.ndarray]:
+        torch.cuda.synchronize(self.device)
+        self.check_status()
+        return {
+            "comm": self.comm.cpu().numpy(),
+            "cost": self.cost.cpu().numpy(),
+            "flags": self.flags.cpu().numpy(),
+            "compute": self.compute.cpu().numpy(),
+            "per_arg": self.per_arg.cpu().numpy(),
+        }

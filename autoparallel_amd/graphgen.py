@@ -1,0 +1,858 @@
+"""Shape-level generators for the benchmark graphs.
+
+The reference obtains its joint forward+backward graph from Dynamo/AOTAutograd
+and its per-node strategies from DTensor's sharding propagator
+(autoparallel/api.py:157-228, autoparallel/shardings/placement_options.py:279-359);
+neither is part of the cost engine.  This module produces inputs of the same
+shape without either: a small tape-based tracer records aten-granularity ops
+on symbolic (shape, stride, dtype) tensors, differentiates them, and
+enumerates per-op strategies as the product over mesh dims of single-dim
+options, the way DTensor's ``expand_to_full_mesh_op_strategy`` does, followed
+by the reference's validity filter and de-duplication
+(autoparallel/shardings/propagation_rules.py:127-158,
+autoparallel/shardings/placement_options.py:151-170).  Linear layers appear as
+two-operand einsums, as after the reference's view-mm-view rewrite
+(autoparallel/graph_passes/graph_utils.py:415-439), with the single-dim
+options of autoparallel/shardings/propagation_rules.py:573-590 (no Partial
+inputs).
+
+Strategy sets are *input data* for the cost engine; what is checked against
+the reference is the cost of every entry given these inputs.
+"""
+from __future__ import annotations
+
+import dataclasses
+import itertools
+import math
+from typing import Callable, Dict, List, Optional, Sequence, Tuple
+
+import numpy as np
+
+from . import opprog
+from .packed import (
+    DT_BF16,
+    DT_F32,
+    DT_OTHER,
+    OP_PROGRAM,
+    OP_ZERO,
+    PARTIAL_SUM,
+    PARTIAL_AVG,
+    PLC_PARTIAL,
+    PLC_R,
+    GraphBuilder,
+    NodeDesc,
+    PackedGraph,
+    is_shard,
+    shard,
+)
+
+R = PLC_R
+P = PARTIAL_SUM
+MASK_PARTIAL = PLC_PARTIAL | 8  # embedding's MaskPartial: equal only to itself
+
+_ITEMSIZE = {DT_BF16: 2, DT_F32: 4, DT_OTHER: 8}
+
+
+def contiguous_stride(shape: Sequence[int]) -> Tuple[int, ...]:
+    st = []
+    acc = 1
+    for s in reversed(shape):
+        st.append(acc)
+        acc *= max(int(s), 1)
+    return tuple(reversed(st))
+
+
+@dataclasses.dataclass
+class T:
+    """Symbolic tensor: which node (and tuple element) produces it."""
+
+    node: int
+    out_index: Optional[int]
+    shape: Tuple[int, ...]
+    stride: Tuple[int, ...]
+    dtype: int
+    requires_grad: bool = False
+
+    @property
+    def rank(self) -> int:
+        return len(self.shape)
+
+    @property
+    def itemsize(self) -> int:
+        return _ITEMSIZE[self.dtype]
+
+
+# one single-mesh-dim option: (placements of the outputs, placements of the args)
+Option = Tuple[Tuple[Optional[int], ...], Tuple[Optional[int], ...]]
+
+
+def _valid(shape: Sequence[int], plc: Sequence[int], mesh_shape: Sequence[int]) -> bool:
+    # per-spec rule of remove_invalid_configs (propagation_rules.py:143-154)
+    shape = list(shape)
+    for n, p in zip(mesh_shape, plc):
+        if is_shard(p):
+            d = p & 0x3F
+            if shape[d] >= n:
+                shape[d] = (shape[d] + n - 1) // n
+            else:
+                return False
+    return True
+
+
+class Tracer:
+    def __init__(self, mesh_shape: Sequence[int], devices_per_host: int = 8):
+        self.mesh_shape = tuple(int(x) for x in mesh_shape)
+        self.ndim = len(self.mesh_shape)
+        self.b = GraphBuilder(self.mesh_shape, devices_per_host)
+        self._tape: List[Tuple[List[T], List[T], Callable]] = []
+        self._strategy_cache: Dict[tuple, tuple] = {}
+        self.param_nodes: List[int] = []
+        self.grad_nodes: Dict[int, int] = {}  # param node -> grad node
+        self.node_users: Dict[int, List[int]] = {}
+        self.node_inputs: Dict[int, List[int]] = {}
+        self.outputs: List[T] = []
+
+    # -- strategy expansion --------------------------------------------------
+    def _expand(
+        self,
+        sig: tuple,
+        options: List[Option],
+        out_metas: List[Optional[T]],
+        in_metas: List[Optional[T]],
+    ):
+        """Product over mesh dims of single-dim options -> validity filter ->
+        dedup.  Returns (in_plcs[o][a], out_plcs[o][k])."""
+        key = (sig, tuple(options), tuple((t.shape if t else None) for t in out_metas),
+               tuple((t.shape if t else None) for t in in_metas))
+        hit = self._strategy_cache.get(key)
+        if hit is not None:
+            return hit
+        seen = set()
+        ins_all, outs_all = [], []
+        for combo in itertools.product(options, repeat=self.ndim):
+            outs = tuple(
+                None if combo[0][0][k] is None else tuple(c[0][k] for c in combo)
+                for k in range(len(out_metas))
+            )
+            ins = tuple(
+                None if combo[0][1][a] is None else tuple(c[1][a] for c in combo)
+                for a in range(len(in_metas))
+            )
+            ok = True
+            for plc, t in list(zip(outs, out_metas)) + list(zip(ins, in_metas)):
+                if plc is None or t is None:
+                    continue
+                if not _valid(t.shape, plc, self.mesh_shape):
+                    ok = False
+                    break
+            if not ok:
+                continue
+            k2 = (ins, outs)
+            if k2 in seen:
+                continue
+            seen.add(k2)
+            ins_all.append(ins)
+            outs_all.append(outs)
+        assert ins_all, f"no valid strategy for {sig}"
+        res = (ins_all, outs_all)
+        self._strategy_cache[key] = res
+        return res
+
+    # -- node emission -------------------------------------------------------
+    def _emit(
+        self,
+        name: str,
+        args: List[T],
+        outs_meta: List[Tuple[Tuple[int, ...], Tuple[int, ...], int]],
+        options: List[Option],
+        program: Optional[List[int]],
+        tuple_output: bool = False,
+        sig_extra: tuple = (),
+    ) -> List[T]:
+        v = len(self.b.nodes)
+        out_ts = [
+            T(v, (k if tuple_output else None), tuple(s), tuple(st), dt)
+            for k, (s, st, dt) in enumerate(outs_meta)
+        ]
+        ins_all, outs_all = self._expand((name.split(".")[0],) + sig_extra, options, out_ts, args)
+        in_meta_ids = [self.b.meta(a.shape, a.stride, a.itemsize, a.dtype) for a in args]
+        out_meta_ids = [self.b.meta(t.shape, t.stride, t.itemsize, t.dtype) for t in out_ts]
+        in_specs, out_specs = [], []
+        for ins, outs in zip(ins_all, outs_all):
+            in_specs.append([
+                -1 if plc is None else self.b.spec(m, plc) for plc, m in zip(ins, in_meta_ids)
+            ])
+            out_specs.append([
+                -1 if plc is None else self.b.spec(m, plc) for plc, m in zip(outs, out_meta_ids)
+            ])
+        inputs, getitem = [], None
+        for a in args:
+            inputs.append(a.node)
+        nd = NodeDesc(
+            name=f"{name}_{v}",
+            in_specs=in_specs,
+            out_specs=out_specs,
+            inputs=inputs,
+            op=OP_PROGRAM if program is not None else OP_ZERO,
+            program=program,
+            tuple_output=tuple_output,
+        )
+        self.b.add_node(nd)
+        self.node_inputs[v] = list(inputs)
+        for u in inputs:
+            self.node_users.setdefault(u, []).append(v)
+        return out_ts
+
+    def placeholder(self, name: str, shape, dtype: int, param: bool = False, requires_grad=False) -> T:
+        """Parameters and inputs: every {Replicate, Shard(d)} combination that
+        survives the validity filter (propagation_rules.py:184-201)."""
+        shape = tuple(int(s) for s in shape)
+        stride = contiguous_stride(shape)
+        v = len(self.b.nodes)
+        t = T(v, None, shape, stride, dtype, requires_grad=requires_grad or param)
+        m = self.b.meta(shape, stride, t.itemsize, dtype)
+        opts = [R] + [shard(i) for i in range(len(shape))]
+        specs = []
+        for plc in itertools.product(opts, repeat=self.ndim):
+            if _valid(shape, plc, self.mesh_shape):
+                specs.append(self.b.spec(m, plc))
+        self.b.add_node(
+            NodeDesc(
+                name=name,
+                in_specs=[[s] for s in specs],
+                out_specs=[[s] for s in specs],
+                inputs=[],
+                default_rows=[[[0.0]] for _ in specs],
+            )
+        )
+        self.node_inputs[v] = []
+        if param:
+            self.param_nodes.append(v)
+        return t
+
+    def getitem(self, src: T) -> T:
+        """operator.getitem on a tuple-producing node: follows the producer's
+        strategies one to one (propagation_rules.py:209+)."""
+        assert src.out_index is not None
+        prod = self.b.nodes[src.node]
+        v = len(self.b.nodes)
+        k = src.out_index
+        specs = [o[k] for o in prod.out_specs]
+        # strategies with equal (input, output) collapse (keep_unique_configs)
+        uniq = list(dict.fromkeys(specs))
+        self.b.add_node(
+            NodeDesc(
+                name=f"getitem_{v}",
+                in_specs=[[s] for s in uniq],
+                out_specs=[[s] for s in uniq],
+                inputs=[src.node],
+                getitem_index=k,
+            )
+        )
+        self.node_inputs[v] = [src.node]
+        self.node_users.setdefault(src.node, []).append(v)
+        return T(v, None, src.shape, src.stride, src.dtype)
+
+    # -- autograd tape -------------------------------------------------------
+    def _record(self, ins: List[T], outs: List[T], vjp: Callable):
+        if any(t.requires_grad for t in ins):
+            for o in outs:
+                o.requires_grad = True
+            self._tape.append((ins, outs, vjp))
+
+    def backward(self, roots: List[Tuple[T, T]]):
+        """Differentiate: ``roots`` pairs each output with its tangent."""
+        grads: Dict[Tuple[int, Optional[int]], T] = {}
+
+        def key(t: T):
+            return (t.node, t.out_index)
+
+        def acc(t: T, g: Optional[T]):
+            if g is None or not t.requires_grad:
+                return
+            k = key(t)
+            if k in grads:
+                grads[k] = self.add(grads[k], g)
+            else:
+                grads[k] = g
+
+        for out, tangent in roots:
+            acc(out, tangent)
+        for ins, outs, vjp in reversed(self._tape):
+            gouts = [grads.get(key(o)) for o in outs]
+            if all(g is None for g in gouts):
+                continue
+            gins = vjp(gouts)
+            for t, g in zip(ins, gins):
+                acc(t, g)
+        self._tape = []
+        return grads
+
+    # ======================= primitive ops ==================================
+    @staticmethod
+    def _bshape(shapes: List[Tuple[int, ...]]) -> Tuple[int, ...]:
+        r = max(len(s) for s in shapes)
+        out = [1] * r
+        for s in shapes:
+            for i, x in enumerate(s):
+                j = r - len(s) + i
+                if x != 1:
+                    out[j] = x
+        return tuple(out)
+
+    def pointwise(self, name: str, args: List[T], partial: str = "none", out_dtype: Optional[int] = None,
+                  vjp: Optional[Callable] = None) -> T:
+        shape = self._bshape([a.shape for a in args])
+        r = len(shape)
+        dt = args[0].dtype if out_dtype is None else out_dtype
+        opts: List[Option] = [((R,), tuple(R for _ in args))]
+        for d in range(r):
+            if shape[d] == 1:
+                continue
+            ins = []
+            for a in args:
+                da = d - (r - a.rank)
+                ins.append(shard(da) if da >= 0 and a.shape[da] != 1 else R)
+            opts.append(((shard(d),), tuple(ins)))
+        if partial == "add":
+            opts.append(((P,), tuple(P for _ in args)))
+        elif partial == "mul":
+            for i in range(len(args)):
+                opts.append(((P,), tuple(P if j == i else R for j in range(len(args)))))
+        elif partial == "unary":
+            opts.append(((P,), (P,) + tuple(R for _ in args[1:])))
+        out = self._emit(name, args, [(shape, contiguous_stride(shape), dt)], opts,
+                         opprog.pointwise(r, _ITEMSIZE[dt]), sig_extra=(partial, dt))[0]
+        if vjp is not None:
+            self._record(args, [out], vjp)
+        return out
+
+    def _unbroadcast(self, g: T, like: T) -> T:
+        if g.shape == like.shape:
+            return g
+        lead = g.rank - like.rank
+        dims = list(range(lead)) + [lead + i for i, s in enumerate(like.shape) if s == 1 and g.shape[lead + i] != 1]
+        out = self.sum(g, dims, keepdim=False) if lead and len(dims) == lead else self.sum(g, dims, keepdim=True)
+        if out.shape != like.shape:
+            out = self.view(out, like.shape)
+        return out
+
+    def add(self, a: T, b: T) -> T:
+        return self.pointwise("add", [a, b], "add",
+                              vjp=lambda g: [self._unbroadcast(g[0], a), self._unbroadcast(g[0], b)])
+
+    def mul(self, a: T, b: T) -> T:
+        return self.pointwise(
+            "mul", [a, b], "mul",
+            vjp=lambda g: [
+                self._unbroadcast(self.mul(g[0], b), a) if a.requires_grad else None,
+                self._unbroadcast(self.mul(g[0], a), b) if b.requires_grad else None,
+            ])
+
+    def scale(self, a: T, name: str = "mul_scalar") -> T:
+        """a * python scalar (also add-scalar-free linear unary ops)."""
+        return self.pointwise(name, [a], "unary", vjp=lambda g: [self.scale(g[0], name)])
+
+    def neg(self, a: T) -> T:
+        return self.pointwise("neg", [a], "unary", vjp=lambda g: [self.neg(g[0])])
+
+    def unary(self, name: str, a: T, bwd_name: Optional[str] = None) -> T:
+        """Non-linear unary op; backward is one fused binary op (grad, saved)."""
+        bn = bwd_name or (name + "_backward")
+        return self.pointwise(name, [a], "none",
+                              vjp=lambda g: [self.pointwise(bn, [g[0], a], "none")])
+
+    def add_scalar(self, a: T) -> T:
+        return self.pointwise("add_scalar", [a], "none", vjp=lambda g: [g[0]])
+
+    def to_dtype(self, a: T, dtype: int) -> T:
+        if a.dtype == dtype:
+            return a
+        src = a.dtype
+        return self.pointwise("_to_copy", [a], "unary", out_dtype=dtype,
+                              vjp=lambda g: [self.to_dtype(g[0], src)])
+
+    def alias(self, a: T) -> T:
+        """View-like identity (alias/detach): zero compute cost."""
+        opts: List[Option] = [((R,), (R,))] + [((shard(d),), (shard(d),)) for d in range(a.rank)] + [((P,), (P,))]
+        return self._emit("alias", [a], [(a.shape, a.stride, a.dtype)], opts, None)[0]
+
+    # ---- einsum (linear layers) -------------------------------------------
+    def einsum_fwd(self, x: T, w: T) -> T:
+        """"{batch}k,kn->{batch}n"."""
+        assert w.rank == 2 and x.shape[-1] == w.shape[0]
+        r = x.rank
+        opts: List[Option] = [((R,), (R, R))]
+        for d in range(r - 1):
+            opts.append(((shard(d),), (shard(d), R)))
+        opts.append(((shard(r - 1),), (R, shard(1))))  # n
+        opts.append(((P,), (shard(r - 1), shard(0))))  # k -> Partial
+        shape = x.shape[:-1] + (w.shape[1],)
+        out = self._emit("einsum_fwd", [x, w], [(shape, contiguous_stride(shape), x.dtype)], opts,
+                         opprog.einsum_fwd(r, x.itemsize))[0]
+
+        def vjp(g):
+            gx = self.einsum_fwd(g[0], self.permute(w, [1, 0])) if x.requires_grad else None
+            gw = self.einsum_bwd(g[0], x) if w.requires_grad else None  # [k, n]
+            return [gx, gw]
+
+        self._record([x, w], [out], vjp)
+        return out
+
+    def einsum_bwd(self, a: T, b: T) -> T:
+        """"{batch}n,{batch}k->kn" (weight gradient)."""
+        assert a.shape[:-1] == b.shape[:-1]
+        r = a.rank
+        opts: List[Option] = [((R,), (R, R))]
+        for d in range(r - 1):
+            opts.append(((P,), (shard(d), shard(d))))
+        opts.append(((shard(1),), (shard(r - 1), R)))  # n
+        opts.append(((shard(0),), (R, shard(r - 1))))  # k
+        shape = (b.shape[-1], a.shape[-1])
+        return self._emit("einsum_bwd", [a, b], [(shape, contiguous_stride(shape), a.dtype)], opts,
+                          opprog.einsum_bwd(r, a.itemsize))[0]
+
+    # ---- views --------------------------------------------------------------
+    def permute(self, x: T, perm: Sequence[int]) -> T:
+        perm = [p % x.rank for p in perm]
+        shape = tuple(x.shape[p] for p in perm)
+        stride = tuple(x.stride[p] for p in perm)
+        opts: List[Option] = [((R,), (R,)), ((P,), (P,))]
+        for j, p in enumerate(perm):
+            opts.append(((shard(j),), (shard(p),)))
+        out = self._emit("permute", [x], [(shape, stride, x.dtype)], opts, None, sig_extra=(tuple(perm),))[0]
+        inv = [perm.index(i) for i in range(x.rank)]
+        self._record([x], [out], lambda g: [self.permute(g[0], inv)])
+        return out
+
+    def transpose(self, x: T, d0: int, d1: int) -> T:
+        perm = list(range(x.rank))
+        perm[d0], perm[d1] = perm[d1], perm[d0]
+        return self.permute(x, perm)
+
+    def view(self, x: T, shape: Sequence[int]) -> T:
+        """Reshape.  Sharding follows DTensor's dim-map rule: in a flatten
+        group only the leading input dim may stay sharded; in a split group
+        the shard moves to the leading output dim."""
+        shape = tuple(int(s) for s in shape)
+        assert math.prod(shape) == math.prod(x.shape), (x.shape, shape)
+        opts: List[Option] = [((R,), (R,)), ((P,), (P,))]
+        i = j = 0
+        while i < x.rank and j < len(shape):
+            i0, j0 = i, j
+            pi, pj = x.shape[i], shape[j]
+            i += 1
+            j += 1
+            while pi != pj:
+                if pi < pj:
+                    pi *= x.shape[i]
+                    i += 1
+                else:
+                    pj *= shape[j]
+                    j += 1
+            # leading non-1 dims of the group map to each other
+            ii = next((t for t in range(i0, i) if x.shape[t] != 1), None)
+            jj = next((t for t in range(j0, j) if shape[t] != 1), None)
+            if ii is not None and jj is not None:
+                opts.append(((shard(jj),), (shard(ii),)))
+        out = self._emit("view", [x], [(shape, contiguous_stride(shape), x.dtype)], opts, None,
+                         sig_extra=(shape,))[0]
+        src_shape = x.shape
+        self._record([x], [out], lambda g: [self.view(g[0], src_shape)])
+        return out
+
+    def slice(self, x: T, dim: int, start: int, end: int) -> T:
+        dim %= x.rank
+        shape = tuple((end - start) if i == dim else s for i, s in enumerate(x.shape))
+        opts: List[Option] = [((R,), (R,)), ((P,), (P,))]
+        for d in range(x.rank):
+            if d != dim:
+                opts.append(((shard(d),), (shard(d),)))
+        out = self._emit("slice", [x], [(shape, x.stride, x.dtype)], opts, None, sig_extra=(dim, start, end))[0]
+        self._record([x], [out], lambda g: [self.slice_backward(g[0], x.shape, dim)])
+        return out
+
+    def slice_backward(self, g: T, shape: Tuple[int, ...], dim: int) -> T:
+        opts: List[Option] = [((R,), (R,)), ((P,), (P,))]
+        for d in range(g.rank):
+            if d != dim:
+                opts.append(((shard(d),), (shard(d),)))
+        prog = opprog.program([], [(g.itemsize, [opprog.const(shape[i]) if i == dim else opprog.argdim(0, i)
+                                                 for i in range(len(shape))])])
+        return self._emit("slice_backward", [g], [(shape, contiguous_stride(shape), g.dtype)], opts, prog,
+                          sig_extra=(dim, shape[dim]))[0]
+
+    def cat(self, xs: List[T], dim: int) -> T:
+        dim %= xs[0].rank
+        shape = tuple(sum(x.shape[dim] for x in xs) if i == dim else s for i, s in enumerate(xs[0].shape))
+        n = len(xs)
+        opts: List[Option] = [((R,), (R,) * n), ((P,), (P,) * n)]
+        for d in range(xs[0].rank):
+            if d != dim:
+                opts.append(((shard(d),), (shard(d),) * n))
+        # output numel = sum of input numels: written as one output per input
+        prog = opprog.program([], [(x.itemsize, [opprog.argdim(k, i) for i in range(x.rank)])
+                                   for k, x in enumerate(xs)])
+        out = self._emit("cat", xs, [(shape, contiguous_stride(shape), xs[0].dtype)], opts, prog,
+                         sig_extra=(dim, n))[0]
+
+        def vjp(g):
+            res, off = [], 0
+            for x in xs:
+                res.append(self.slice(g[0], dim, off, off + x.shape[dim]))
+                off += x.shape[dim]
+            return res
+
+        self._record(xs, [out], vjp)
+        return out
+
+    def expand(self, x: T, dim: int, n: int) -> T:
+        """expand a size-1 dim to n (view, stride 0)."""
+        assert x.shape[dim] == 1
+        shape = tuple(n if i == dim else s for i, s in enumerate(x.shape))
+        stride = tuple(0 if i == dim else s for i, s in enumerate(x.stride))
+        opts: List[Option] = [((R,), (R,)), ((P,), (P,))]
+        for d in range(x.rank):
+            if d != dim and x.shape[d] != 1:
+                opts.append(((shard(d),), (shard(d),)))
+        out = self._emit("expand", [x], [(shape, stride, x.dtype)], opts, None, sig_extra=(dim, n))[0]
+        self._record([x], [out], lambda g: [self.sum(g[0], [dim], keepdim=True)])
+        return out
+
+    def clone(self, x: T) -> T:
+        shape = x.shape
+        opts: List[Option] = [((R,), (R,)), ((P,), (P,))] + [((shard(d),), (shard(d),)) for d in range(x.rank)]
+        out = self._emit("clone", [x], [(shape, contiguous_stride(shape), x.dtype)], opts,
+                         opprog.same_as_arg(0, x.rank, x.itemsize))[0]
+        self._record([x], [out], lambda g: [g[0]])
+        return out
+
+    # ---- reductions -----------------------------------------------------------
+    def sum(self, x: T, dims: Sequence[int], keepdim: bool, mean: bool = False) -> T:
+        dims = sorted({d % x.rank for d in dims})
+        shape = tuple(
+            (1 if i in dims else s) for i, s in enumerate(x.shape) if keepdim or i not in dims
+        )
+        pcode = PARTIAL_AVG if mean else P
+        opts: List[Option] = [((R,), (R,)), ((pcode,), (pcode,))]
+        j = 0
+        for d in range(x.rank):
+            if d in dims:
+                opts.append(((pcode,), (shard(d),)))
+                if keepdim:
+                    j += 1
+            else:
+                opts.append(((shard(j),), (shard(d),)))
+                j += 1
+        out = self._emit("mean" if mean else "sum", [x], [(shape, contiguous_stride(shape), x.dtype)], opts,
+                         opprog.reduction(x.rank, dims, keepdim, x.itemsize),
+                         sig_extra=(tuple(dims), keepdim))[0]
+        src = x.shape
+
+        def vjp(g):
+            gg = g[0]
+            if not keepdim:
+                gg = self.view(gg, tuple(1 if i in dims else s for i, s in enumerate(src)))
+            for d in dims:
+                gg = self.expand(gg, d, src[d])
+            if mean:
+                gg = self.scale(gg, "div_scalar")
+            return [gg]
+
+        self._record([x], [out], vjp)
+        return out
+
+    def softmax_like(self, name: str, args: List[T], dim: int, n_out: int = 1) -> T:
+        x = args[0]
+        dim %= x.rank
+        opts: List[Option] = [((R,), (R,) * len(args))]
+        for d in range(x.rank):
+            if d != dim:
+                opts.append(((shard(d),), (shard(d),) * len(args)))
+        return self._emit(name, args, [(x.shape, contiguous_stride(x.shape), x.dtype)], opts,
+                          opprog.same_as_arg(0, x.rank, x.itemsize), sig_extra=(dim,))[0]
+
+    # ---- attention ------------------------------------------------------------
+    def sdpa(self, q: T, k: T, v: T) -> T:
+        """aten._scaled_dot_product_flash_attention: tuple output (out, lse)."""
+        b, h, sq, d = q.shape
+        opts: List[Option] = [
+            ((R, R), (R, R, R)),
+            ((shard(0), shard(0)), (shard(0),) * 3),
+            ((shard(1), shard(1)), (shard(1),) * 3),
+        ]
+        out_shape = (b, h, sq, v.shape[3])
+        lse_shape = (b, h, sq)
+        outs = self._emit(
+            "sdpa_flash", [q, k, v],
+            [(out_shape, contiguous_stride(out_shape), q.dtype), (lse_shape, contiguous_stride(lse_shape), DT_F32)],
+            opts, opprog.sdpa_flash_fwd(q.itemsize), tuple_output=True)
+        o = self.getitem(outs[0])
+        lse = self.getitem(outs[1])
+
+        def vjp(g):
+            bopts: List[Option] = [
+                ((R, R, R), (R,) * 6),
+                ((shard(0),) * 3, (shard(0),) * 6),
+                ((shard(1),) * 3, (shard(1),) * 6),
+            ]
+            gs = self._emit(
+                "sdpa_flash_backward", [g[0], q, k, v, o, lse],
+                [(q.shape, contiguous_stride(q.shape), q.dtype), (k.shape, contiguous_stride(k.shape), k.dtype),
+                 (v.shape, contiguous_stride(v.shape), v.dtype)],
+                bopts, opprog.sdpa_flash_bwd(q.itemsize), tuple_output=True)
+            return [self.getitem(t) for t in gs]
+
+        self._record([q, k, v], [o], vjp)
+        return o
+
+    # ---- embedding ------------------------------------------------------------
+    def embedding(self, w: T, idx: T) -> T:
+        r = idx.rank
+        shape = idx.shape + (w.shape[1],)
+        opts: List[Option] = [((R,), (R, R))]
+        for d in range(r):
+            opts.append(((shard(d),), (R, shard(d))))
+        opts.append(((shard(r),), (shard(1), R)))
+        opts.append(((MASK_PARTIAL,), (shard(0), R)))
+        out = self._emit("embedding", [w, idx], [(shape, contiguous_stride(shape), w.dtype)], opts,
+                         opprog.embedding(r, w.itemsize))[0]
+
+        def vjp(g):
+            bopts: List[Option] = [((R,), (R, R))]
+            for d in range(r):
+                bopts.append(((P,), (shard(d), shard(d))))
+            bopts.append(((shard(1),), (shard(r), R)))
+            gw = self._emit("embedding_dense_backward", [g[0], idx],
+                            [(w.shape, contiguous_stride(w.shape), w.dtype)], bopts,
+                            opprog.embedding_dense_backward(w.shape[0], w.itemsize, g[0].rank))[0]
+            return [gw, None]
+
+        self._record([w, idx], [out], vjp)
+        return out
+
+    # ---- finishing ---------------------------------------------------------
+    def finish(self, param_grads: Dict[int, T], outputs: List[T]) -> PackedGraph:
+        """Mark prefetchable edges and pack.
+
+        Param-derived: every input is a parameter or param-derived
+        (autoparallel/graph_passes/graph_utils.py:447-459).  Terminal-derived:
+        every user is a parameter-gradient node or terminal-derived (:462-484);
+        the graph's output node counts as the only user of a gradient node."""
+        n = len(self.b.nodes)
+        param_derived = set(self.param_nodes)
+        for v in range(n):
+            ins = self.node_inputs.get(v, [])
+            if ins and all(u in param_derived for u in ins):
+                param_derived.add(v)
+        terminal = set(t.node for t in param_grads.values())
+        out_nodes = set(t.node for t in outputs) | terminal
+        for v in reversed(range(n)):
+            users = self.node_users.get(v, [])
+            if v in out_nodes and v not in terminal:
+                continue  # also used by the output node
+            if users and all(u in terminal for u in users):
+                terminal.add(v)
+        for v in range(n):
+            for a, u in enumerate(self.node_inputs.get(v, [])):
+                if u in param_derived or v in terminal:
+                    self.b.prefetchable_edges.add((v, a))
+        self.param_derived = param_derived
+        self.terminal_derived = terminal
+        return self.b.pack()
+
+
+# ===========================================================================
+# Model graphs
+# ===========================================================================
+def _rmsnorm(t: Tracer, x: T, w: T) -> T:
+    xf = t.to_dtype(x, DT_F32)
+    sq = t.unary("pow", xf)
+    ms = t.sum(sq, [-1], keepdim=True, mean=True)
+    ms = t.add_scalar(ms)
+    rs = t.unary("rsqrt", ms)
+    y = t.mul(xf, rs)
+    y = t.to_dtype(y, x.dtype)
+    return t.mul(y, w)
+
+
+def _linear(t: Tracer, x: T, w: T) -> T:
+    # nn.Linear weight is [out, in]; the einsum consumes its transposed view
+    return t.einsum_fwd(x, t.permute(w, [1, 0]))
+
+
+def _rope(t: Tracer, x: T, cos: T, sin: T) -> T:
+    # rotate-half formulation in fp32, cast back
+    xf = t.to_dtype(x, DT_F32)
+    d = x.shape[-1]
+    x1 = t.slice(xf, -1, 0, d // 2)
+    x2 = t.slice(xf, -1, d // 2, d)
+    rot = t.cat([t.neg(x2), x1], -1)
+    out = t.add(t.mul(xf, cos), t.mul(rot, sin))
+    return t.to_dtype(out, x.dtype)
+
+
+def _repeat_kv(t: Tracer, x: T, n_rep: int) -> T:
+    if n_rep == 1:
+        return x
+    b, s, h, d = x.shape
+    x = t.view(x, (b, s, h, 1, d))
+    x = t.expand(x, 3, n_rep)
+    x = t.clone(x)
+    return t.view(x, (b, s, h * n_rep, d))
+
+
+def llama_graph(
+    mesh_shape: Sequence[int],
+    n_layers: int,
+    dim: int,
+    n_heads: int,
+    n_kv_heads: int,
+    ffn_dim: int,
+    vocab: int,
+    seq: int,
+    batch: int,
+    devices_per_host: int = 8,
+    dtype: int = DT_BF16,
+) -> PackedGraph:
+    """Llama-3-style decoder (RMSNorm, RoPE, GQA, SwiGLU), forward + backward,
+    logits as the output with a tangent input, as an AOT joint graph has."""
+    t = Tracer(mesh_shape, devices_per_host)
+    hd = dim // n_heads
+    params: Dict[str, T] = {}
+
+    def P_(name, shape):
+        params[name] = t.placeholder(name, shape, dtype, param=True)
+        return params[name]
+
+    tok_emb = P_("tok_embeddings.weight", (vocab, dim))
+    layers = []
+    for i in range(n_layers):
+        layers.append(
+            dict(
+                attn_norm=P_(f"layers.{i}.attention_norm.weight", (dim,)),
+                wq=P_(f"layers.{i}.attention.wq.weight", (n_heads * hd, dim)),
+                wk=P_(f"layers.{i}.attention.wk.weight", (n_kv_heads * hd, dim)),
+                wv=P_(f"layers.{i}.attention.wv.weight", (n_kv_heads * hd, dim)),
+                wo=P_(f"layers.{i}.attention.wo.weight", (dim, n_heads * hd)),
+                ffn_norm=P_(f"layers.{i}.ffn_norm.weight", (dim,)),
+                w1=P_(f"layers.{i}.feed_forward.w1.weight", (ffn_dim, dim)),
+                w2=P_(f"layers.{i}.feed_forward.w2.weight", (dim, ffn_dim)),
+                w3=P_(f"layers.{i}.feed_forward.w3.weight", (ffn_dim, dim)),
+            )
+        )
+    norm_w = P_("norm.weight", (dim,))
+    out_w = P_("output.weight", (vocab, dim))
+    cos = t.placeholder("rope_cos", (1, seq, 1, hd), DT_F32)
+    sin = t.placeholder("rope_sin", (1, seq, 1, hd), DT_F32)
+    tokens = t.placeholder("tokens", (batch, seq), DT_OTHER)
+    tangent = t.placeholder("tangents_1", (batch, seq, vocab), dtype)
+
+    h = t.embedding(tok_emb, tokens)
+    for L in layers:
+        x = _rmsnorm(t, h, L["attn_norm"])
+        q = t.view(_linear(t, x, L["wq"]), (batch, seq, n_heads, hd))
+        k = t.view(_linear(t, x, L["wk"]), (batch, seq, n_kv_heads, hd))
+        v = t.view(_linear(t, x, L["wv"]), (batch, seq, n_kv_heads, hd))
+        q = _rope(t, q, cos, sin)
+        k = _rope(t, k, cos, sin)
+        k = _repeat_kv(t, k, n_heads // n_kv_heads)
+        v = _repeat_kv(t, v, n_heads // n_kv_heads)
+        q, k, v = (t.transpose(z, 1, 2) for z in (q, k, v))
+        o = t.sdpa(q, k, v)
+        o = t.clone(t.transpose(o, 1, 2))
+        o = t.view(o, (batch, seq, n_heads * hd))
+        h = t.add(h, _linear(t, o, L["wo"]))
+        x = _rmsnorm(t, h, L["ffn_norm"])
+        g = t.unary("silu", _linear(t, x, L["w1"]))
+        u = _linear(t, x, L["w3"])
+        h = t.add(h, _linear(t, t.mul(g, u), L["w2"]))
+    h = _rmsnorm(t, h, norm_w)
+    logits = _linear(t, h, out_w)
+    grads = t.backward([(logits, tangent)])
+    param_grads = {}
+    for name, p in params.items():
+        g = grads.get((p.node, None))
+        if g is not None:
+            param_grads[p.node] = t.alias(g)
+    return t.finish(param_grads, [logits])
+
+
+def _layernorm(t: Tracer, x: T, w: T, b: T) -> T:
+    xf = t.to_dtype(x, DT_F32)
+    mu = t.sum(xf, [-1], keepdim=True, mean=True)
+    xc = t.add(xf, t.neg(mu))
+    var = t.sum(t.unary("pow", xc), [-1], keepdim=True, mean=True)
+    rs = t.unary("rsqrt", t.add_scalar(var))
+    y = t.to_dtype(t.mul(xc, rs), x.dtype)
+    return t.add(t.mul(y, w), b)
+
+
+def gpt2_graph(
+    mesh_shape: Sequence[int],
+    n_layers: int = 12,
+    dim: int = 768,
+    n_heads: int = 12,
+    ffn_dim: int = 3072,
+    vocab: int = 50257,
+    seq: int = 1024,
+    batch: int = 8,
+    devices_per_host: int = 8,
+) -> PackedGraph:
+    """GPT-2-style decoder: fp32 master parameters cast to bf16 for compute
+    (so gradients come back in fp32), LayerNorm, GELU MLP, learned positions,
+    tied output embedding."""
+    t = Tracer(mesh_shape, devices_per_host)
+    hd = dim // n_heads
+    params: Dict[str, T] = {}
+
+    def P_(name, shape):
+        params[name] = t.placeholder(name, shape, DT_F32, param=True)
+        return t.to_dtype(params[name], DT_BF16)
+
+    wte = P_("wte.weight", (vocab, dim))
+    wpe = P_("wpe.weight", (seq, dim))
+    tokens = t.placeholder("tokens", (batch, seq), DT_OTHER)
+    pos = t.placeholder("positions", (1, seq), DT_OTHER)
+    tangent = t.placeholder("tangents_1", (batch, seq, vocab), DT_BF16)
+    h = t.add(t.embedding(wte, tokens), t.embedding(wpe, pos))
+    for i in range(n_layers):
+        ln1w, ln1b = P_(f"h.{i}.ln_1.weight", (dim,)), P_(f"h.{i}.ln_1.bias", (dim,))
+        wqkv, bqkv = P_(f"h.{i}.attn.c_attn.weight", (3 * dim, dim)), P_(f"h.{i}.attn.c_attn.bias", (3 * dim,))
+        wo, bo = P_(f"h.{i}.attn.c_proj.weight", (dim, dim)), P_(f"h.{i}.attn.c_proj.bias", (dim,))
+        ln2w, ln2b = P_(f"h.{i}.ln_2.weight", (dim,)), P_(f"h.{i}.ln_2.bias", (dim,))
+        wfc, bfc = P_(f"h.{i}.mlp.c_fc.weight", (ffn_dim, dim)), P_(f"h.{i}.mlp.c_fc.bias", (ffn_dim,))
+        wpr, bpr = P_(f"h.{i}.mlp.c_proj.weight", (dim, ffn_dim)), P_(f"h.{i}.mlp.c_proj.bias", (dim,))
+        x = _layernorm(t, h, ln1w, ln1b)
+        qkv = t.add(_linear(t, x, wqkv), bqkv)
+        q, k, v = (t.slice(qkv, -1, j * dim, (j + 1) * dim) for j in range(3))
+        q, k, v = (t.transpose(t.view(z, (batch, seq, n_heads, hd)), 1, 2) for z in (q, k, v))
+        o = t.sdpa(q, k, v)
+        o = t.view(t.clone(t.transpose(o, 1, 2)), (batch, seq, dim))
+        h = t.add(h, t.add(_linear(t, o, wo), bo))
+        x = _layernorm(t, h, ln2w, ln2b)
+        m = t.unary("gelu", t.add(_linear(t, x, wfc), bfc))
+        h = t.add(h, t.add(_linear(t, m, wpr), bpr))
+    lnfw, lnfb = P_("ln_f.weight", (dim,)), P_("ln_f.bias", (dim,))
+    h = _layernorm(t, h, lnfw, lnfb)
+    logits = _linear(t, h, wte)
+    grads = t.backward([(logits, tangent)])
+    param_grads = {}
+    for name, p in params.items():
+        g = grads.get((p.node, None))
+        if g is not None:
+            param_grads[p.node] = t.alias(g)
+    return t.finish(param_grads, [logits])
+
+
+# ---- named benchmark configurations ----------------------------------------
+def config_gpt2_small() -> PackedGraph:
+    return gpt2_graph((8,))
+
+
+def config_llama3_8b(n_layers: int = 32) -> PackedGraph:
+    return llama_graph((8, 8), n_layers, 4096, 32, 8, 14336, 128256, 8192, 64)
+
+
+def config_llama3_70b(n_layers: int = 80) -> PackedGraph:
+    return llama_graph((4, 8, 8), n_layers, 8192, 64, 8, 28672, 128256, 8192, 256)

@@ -5,9 +5,12 @@ it from HBM, the host builds it from ``{node: OpStrategy}`` (or directly from
 a shape-level generator).  It flattens what the reference keeps as Python
 objects:
 
-* ``DTensorSpec.placements``          -> one byte per mesh dim (``spec_plc``)
+* ``DTensorSpec.placements``          -> a row of the interned placement-tuple
+                                         table (``tuple_plc``, one byte per mesh dim)
 * ``DTensorSpec.tensor_meta``         -> a row of the tensor-meta table
-* ``OpSpec.input_specs / output_specs`` -> runs of spec ids in ``lists``
+* a ``DTensorSpec``                   -> one 32-bit word ``meta_id << 12 | tuple_id``
+                                         (``SPEC_NONE`` where the reference has ``None``)
+* ``OpSpec.input_specs / output_specs`` -> runs of spec words in ``lists``
 * ``strats[node]`` / ``_all_input_nodes(node)[argi]`` -> the edge table
   (reference: autoparallel/optimize_sharding.py:306-354, 380-398, 481-552)
 
@@ -37,6 +40,15 @@ import numpy as np
 
 MAX_MESH_DIMS = 4
 MAX_RANK = 8
+TUPLE_BITS = 12
+MAX_TUPLES = 1 << TUPLE_BITS
+MAX_METAS = 1 << (32 - TUPLE_BITS)
+SPEC_NONE = 0xFFFFFFFF
+TILE_SHIFT = 10  # entries per tile of the entry->edge index = 1 << TILE_SHIFT
+
+
+def spec_word(meta_id: int, tuple_id: int) -> int:
+    return (int(meta_id) << TUPLE_BITS) | int(tuple_id)
 
 # ---- placement codes -------------------------------------------------------
 PLC_R = 0x00
@@ -94,6 +106,7 @@ DTYPE_ITEMSIZE = {DT_F64: 8, DT_F32: 4, DT_F16: 2, DT_BF16: 2, DT_I8: 1}
 EDGE_HAS_PRODUCER = 1  # comm is computed from specs (else default row kept)
 EDGE_SCORE_TRANSITION = 2  # producer output is a single spec: the plan scorer
 #                            counts a transition (optimize_sharding.py:1097-1104)
+EDGE_PREFETCHABLE = 4  # set in the device records from ``edge_prefetchable``
 
 # ---- compute programs ------------------------------------------------------
 # A node's compute estimate needs flops and bytes of the op run on the sharded
@@ -122,11 +135,10 @@ class PackedGraph:
     meta_stride: np.ndarray  # int64[M, MAX_RANK]
     meta_itemsize: np.ndarray  # int32[M]
     meta_dtype: np.ndarray  # int32[M]
-    # specs
-    spec_meta: np.ndarray  # int32[NSPEC]
-    spec_plc: np.ndarray  # uint8[NSPEC, MAX_MESH_DIMS]
-    # runs of spec ids (-1 = no DTensorSpec at that position)
-    lists: np.ndarray  # int32[L]
+    # interned placement tuples
+    tuple_plc: np.ndarray  # uint8[NT, MAX_MESH_DIMS]
+    # runs of spec words (SPEC_NONE = no DTensorSpec at that position)
+    lists: np.ndarray  # uint32[L]
     # nodes
     node_nstrat: np.ndarray  # int32[N]
     node_nargs: np.ndarray  # int32[N]   len(strategies[0].input_specs)
@@ -144,8 +156,8 @@ class PackedGraph:
     edge_src_node: np.ndarray = None  # int32[NE] producer or -1
     edge_sdst: np.ndarray = None  # int32[NE]
     edge_ssrc: np.ndarray = None  # int32[NE]
-    edge_dst_list: np.ndarray = None  # int64[NE] offset into lists (sdst ids)
-    edge_src_list: np.ndarray = None  # int64[NE] offset into lists (ssrc ids) or -1
+    edge_dst_list: np.ndarray = None  # int64[NE] offset into lists (sdst words)
+    edge_src_list: np.ndarray = None  # int64[NE] offset into lists (ssrc words) or -1
     edge_off: np.ndarray = None  # int64[NE+1]
     edge_flags: np.ndarray = None  # int32[NE]
     edge_default_off: np.ndarray = None  # int64[NE] offset into default_vals or -1
@@ -200,6 +212,51 @@ class PackedGraph:
         k = self.entry_keys().astype(np.int64)
         return np.lexsort((k[:, 3], k[:, 1], k[:, 2], k[:, 0]))
 
+    # -- device-side views ----------------------------------------------------
+    EDGE_DTYPE = np.dtype(
+        [
+            ("off", "<i8"),
+            ("default_off", "<i8"),
+            ("src_list", "<u4"),
+            ("dst_list", "<u4"),
+            ("ssrc", "<i4"),
+            ("sdst", "<i4"),
+            ("comp_base", "<i4"),
+            ("flags", "<i4"),
+            ("node", "<i4"),
+            ("src_node", "<i4"),
+        ]
+    )
+
+    def edge_records(self) -> np.ndarray:
+        """Edges as 48-byte records (the ``apc_edge`` struct of include/apc.h)."""
+        NE = self.num_edges
+        rec = np.zeros(NE, self.EDGE_DTYPE)
+        assert rec.dtype.itemsize == 48
+        rec["off"] = self.edge_off[:-1]
+        rec["default_off"] = self.edge_default_off
+        rec["src_list"] = np.where(self.edge_src_list >= 0, self.edge_src_list, 0).astype(np.uint32)
+        rec["dst_list"] = self.edge_dst_list.astype(np.uint32)
+        rec["ssrc"] = self.edge_ssrc
+        rec["sdst"] = self.edge_sdst
+        rec["comp_base"] = self.node_comp_off[self.edge_node].astype(np.int32)
+        flags = self.edge_flags.astype(np.int32).copy()
+        if self.edge_prefetchable is not None:
+            flags |= (self.edge_prefetchable.astype(np.int32) != 0) * EDGE_PREFETCHABLE
+        rec["flags"] = flags
+        rec["node"] = self.edge_node
+        rec["src_node"] = self.edge_src_node
+        return rec
+
+    def tile_edge_index(self) -> np.ndarray:
+        """int32[ceil(E / 2**TILE_SHIFT)]: the edge that owns the first entry
+        of each tile, so a kernel thread finds its edge with a short forward
+        walk instead of a binary search."""
+        E = self.num_entries
+        nt = (E + (1 << TILE_SHIFT) - 1) >> TILE_SHIFT
+        starts = np.arange(nt, dtype=np.int64) << TILE_SHIFT
+        return (np.searchsorted(self.edge_off, starts, side="right") - 1).astype(np.int32)
+
     def validate(self) -> None:
         """Host-side shape checks run before any kernel launch: every index a
         kernel dereferences must be in range."""
@@ -210,18 +267,23 @@ class PackedGraph:
         assert self.meta_shape.shape == (M, MAX_RANK)
         assert self.meta_stride.shape == (M, MAX_RANK)
         assert ((self.meta_rank >= 0) & (self.meta_rank <= MAX_RANK)).all()
-        nspec = self.spec_meta.shape[0]
-        assert self.spec_plc.shape == (nspec, MAX_MESH_DIMS)
-        if nspec:
-            assert self.spec_meta.min() >= 0 and self.spec_meta.max() < M
-            sh = (self.spec_plc & PLC_KIND_MASK) == PLC_SHARD
-            dims = (self.spec_plc & PLC_ARG_MASK).astype(np.int32)
-            rank = self.meta_rank[self.spec_meta][:, None]
-            assert (~sh | (dims < rank)).all(), "Shard(dim) out of tensor rank"
-            assert (self.spec_plc[:, nd:] == 0).all()
+        NT = self.tuple_plc.shape[0]
+        assert self.tuple_plc.shape == (NT, MAX_MESH_DIMS) and NT <= MAX_TUPLES
+        assert M <= MAX_METAS
+        assert (self.tuple_plc[:, nd:] == 0).all()
         L = self.lists.shape[0]
+        assert self.lists.dtype == np.uint32
         if L:
-            assert self.lists.min() >= -1 and self.lists.max() < nspec
+            words = np.unique(self.lists)
+            words = words[words != SPEC_NONE]
+            wm = (words >> TUPLE_BITS).astype(np.int64)
+            wt = (words & (MAX_TUPLES - 1)).astype(np.int64)
+            assert (wm < M).all() and (wt < NT).all()
+            plc = self.tuple_plc[wt]
+            sh = (plc & PLC_KIND_MASK) == PLC_SHARD
+            dims = (plc & PLC_ARG_MASK).astype(np.int32)
+            rank = self.meta_rank[wm][:, None]
+            assert (~sh | (dims < rank)).all(), "Shard(dim) out of tensor rank"
         N, NE = self.num_nodes, self.num_edges
         assert self.node_comp_off.shape == (N + 1,)
         assert self.node_edge_off.shape == (N + 1,)
@@ -229,6 +291,7 @@ class PackedGraph:
         assert self.edge_off.shape == (NE + 1,)
         if NE:
             assert (self.edge_sdst >= 1).all() and (self.edge_ssrc >= 1).all()
+            assert (self.node_nargs >= 1).all(), "per-arg compute divides by num_args"
             sizes = self.edge_sdst.astype(np.int64) * self.edge_ssrc
             assert (np.diff(self.edge_off) == sizes).all()
             assert (self.edge_dst_list >= 0).all()
@@ -247,6 +310,14 @@ class PackedGraph:
             assert (
                 self.edge_default_off[d] + sizes[d] <= self.default_vals.shape[0]
             ).all()
+            # a missing spec inside a run is only legal with a default row
+            none_csum = np.concatenate([[0], np.cumsum(self.lists == SPEC_NONE)])
+            nd_run = none_csum[self.edge_dst_list + self.edge_sdst] - none_csum[self.edge_dst_list]
+            ns_run = np.zeros(NE, np.int64)
+            ns_run[hp] = (
+                none_csum[self.edge_src_list[hp] + self.edge_ssrc[hp]] - none_csum[self.edge_src_list[hp]]
+            )
+            assert (((nd_run == 0) & (ns_run == 0)) | d).all()
         assert (np.diff(self.node_comp_off) == self.node_nstrat).all()
 
 
@@ -260,7 +331,7 @@ TensorMetaT = Tuple[Tuple[int, ...], Tuple[int, ...], int, int]  # shape, stride
 class NodeDesc:
     """One graph node with its strategies, as the packer consumes it.
 
-    ``in_specs[o][a]`` / ``out_specs[o][k]`` are spec ids from
+    ``in_specs[o][a]`` / ``out_specs[o][k]`` are spec words from
     :meth:`GraphBuilder.spec` (or -1 where the reference has ``None`` or a
     non-``DTensorSpec``).  ``inputs[a]`` is the producer node index of arg a
     (what ``_all_input_nodes(node)[a]`` returns), ``out_index`` the element of
@@ -288,8 +359,8 @@ class GraphBuilder:
         self.devices_per_host = int(devices_per_host)
         self._metas: Dict[TensorMetaT, int] = {}
         self._meta_rows: List[TensorMetaT] = []
-        self._specs: Dict[Tuple[int, Tuple[int, ...]], int] = {}
-        self._spec_rows: List[Tuple[int, Tuple[int, ...]]] = []
+        self._tuples: Dict[Tuple[int, ...], int] = {}
+        self._tuple_rows: List[Tuple[int, ...]] = []
         self.nodes: List[NodeDesc] = []
         self.prefetchable_edges: set = set()  # (node_idx, argi)
         self.multiplier: Dict[int, int] = {}
@@ -304,21 +375,26 @@ class GraphBuilder:
             self._meta_rows.append(key)
         return i
 
-    def spec(self, meta_id: int, placements: Sequence[int]) -> int:
-        key = (int(meta_id), tuple(int(p) for p in placements))
-        assert len(key[1]) == len(self.mesh_shape)
-        i = self._specs.get(key)
+    def tuple_id(self, placements: Sequence[int]) -> int:
+        key = tuple(int(p) for p in placements)
+        assert len(key) == len(self.mesh_shape)
+        i = self._tuples.get(key)
         if i is None:
-            i = len(self._spec_rows)
-            self._specs[key] = i
-            self._spec_rows.append(key)
+            i = len(self._tuple_rows)
+            assert i < MAX_TUPLES, "too many distinct placement tuples"
+            self._tuples[key] = i
+            self._tuple_rows.append(key)
         return i
 
-    def spec_placements(self, spec_id: int) -> Tuple[int, ...]:
-        return self._spec_rows[spec_id][1]
+    def spec(self, meta_id: int, placements: Sequence[int]) -> int:
+        """Spec word of (tensor meta, placements); -1 stands for None."""
+        return spec_word(meta_id, self.tuple_id(placements))
 
-    def spec_meta_row(self, spec_id: int) -> TensorMetaT:
-        return self._meta_rows[self._spec_rows[spec_id][0]]
+    def spec_placements(self, word: int) -> Tuple[int, ...]:
+        return self._tuple_rows[word & (MAX_TUPLES - 1)]
+
+    def spec_meta_row(self, word: int) -> TensorMetaT:
+        return self._meta_rows[word >> TUPLE_BITS]
 
     def add_node(self, node: NodeDesc) -> int:
         self.nodes.append(node)
@@ -339,12 +415,11 @@ class GraphBuilder:
             meta_stride[i, :r] = stride
             meta_itemsize[i] = itemsize
             meta_dtype[i] = dtype
-        ns = len(self._spec_rows)
-        spec_meta = np.zeros(ns, np.int32)
-        spec_plc = np.zeros((ns, MAX_MESH_DIMS), np.uint8)
-        for i, (m, plc) in enumerate(self._spec_rows):
-            spec_meta[i] = m
-            spec_plc[i, :nd] = plc
+        assert M <= MAX_METAS
+        nt = len(self._tuple_rows)
+        tuple_plc = np.zeros((nt, MAX_MESH_DIMS), np.uint8)
+        for i, plc in enumerate(self._tuple_rows):
+            tuple_plc[i, :nd] = plc
 
         N = len(self.nodes)
         lists: List[int] = []
@@ -470,9 +545,8 @@ class GraphBuilder:
             meta_stride=meta_stride,
             meta_itemsize=meta_itemsize,
             meta_dtype=meta_dtype,
-            spec_meta=spec_meta,
-            spec_plc=spec_plc,
-            lists=np.asarray(lists, np.int32),
+            tuple_plc=tuple_plc,
+            lists=(np.asarray(lists, np.int64) & 0xFFFFFFFF).astype(np.uint32),
             node_nstrat=node_nstrat,
             node_nargs=node_nargs,
             node_comp_off=node_comp_off,

@@ -1,0 +1,208 @@
+/*
+ * apc.h -- C ABI of the MI355X sharding-search cost engine (libapc_hip.so).
+ *
+ * The reference (meta-pytorch/autoparallel) is pure Python and has no FFI: each
+ * entry point below replaces a Python function of the reference's cost path,
+ * cited per declaration (paths relative to the reference tree, or "torch:" for
+ * the installed torch it calls into).  All array arguments are DEVICE pointers
+ * unless marked "host"; the caller owns every buffer; calls are asynchronous on
+ * the given HIP stream (pass the raw hipStream_t, NULL = default stream).
+ * Return value: 0 on success, negative on error (apc_last_error() gives text).
+ * No entry point allocates device memory.
+ */
+#ifndef APC_H_
+#define APC_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define APC_MAX_MESH_DIMS 4
+#define APC_MAX_RANK 8
+#define APC_TUPLE_BITS 12
+#define APC_SPEC_NONE 0xFFFFFFFFu
+#define APC_TILE_SHIFT 10
+#define APC_NUM_DTYPES 8
+
+/* edge flags */
+#define APC_EDGE_HAS_PRODUCER 1
+#define APC_EDGE_SCORE_TRANSITION 2
+#define APC_EDGE_PREFETCHABLE 4
+
+/* node op classes */
+#define APC_OP_ZERO 0
+#define APC_OP_PROGRAM 1
+#define APC_OP_EXPLICIT 2
+
+/* entry flag bits written by apc_edge_costs */
+#define APC_ENTRY_TRANSITION 1 /* src placements != tgt placements        */
+#define APC_ENTRY_NONFINITE 2  /* cost was inf: variable must be pinned 0  */
+
+#define APC_ERR_INVALID (-1)
+#define APC_ERR_LAUNCH (-2)
+#define APC_ERR_UNSUPPORTED (-3)
+
+/* One (consumer node, argument) pair: an S_dst x S_src block of entries. */
+typedef struct apc_edge {
+  int64_t off;         /* index of entry (out_idx 0, inp_idx 0)                */
+  int64_t default_off; /* into default_vals, or -1                             */
+  uint32_t src_list;   /* into lists: S_src producer output spec words         */
+  uint32_t dst_list;   /* into lists: S_dst consumer input spec words          */
+  int32_t ssrc;
+  int32_t sdst;
+  int32_t comp_base; /* index of (node, out_idx 0) in the compute vector     */
+  int32_t flags;
+  int32_t node;
+  int32_t src_node; /* producer node or -1                                   */
+} apc_edge;
+
+/* Cost-model constants (host values, passed by value into the kernels). */
+typedef struct apc_model {
+  int32_t ndim;
+  int32_t mesh_shape[APC_MAX_MESH_DIMS];
+  double mesh_bw[APC_MAX_MESH_DIMS];  /* GB/s per mesh dim                  */
+  double mesh_lat[APC_MAX_MESH_DIMS]; /* us per hop per mesh dim            */
+  double gmem_bw;                     /* bytes/s                            */
+  double tflops[APC_NUM_DTYPES];      /* by dtype code; <= 0: unsupported   */
+} apc_model;
+
+/* The packed problem (see autoparallel_amd/packed.py for the layout). */
+typedef struct apc_problem {
+  apc_model model;
+  /* tensor metas */
+  int32_t n_meta;
+  const int32_t* meta_rank;
+  const int64_t* meta_shape;  /* [n_meta][APC_MAX_RANK] */
+  const int64_t* meta_stride; /* [n_meta][APC_MAX_RANK] */
+  const int32_t* meta_itemsize;
+  const int32_t* meta_dtype;
+  /* interned placement tuples, one byte per mesh dim */
+  int32_t n_tuple;
+  const uint8_t* tuple_plc; /* [n_tuple][APC_MAX_MESH_DIMS] */
+  /* runs of spec words: meta_id << 12 | tuple_id, or APC_SPEC_NONE */
+  int64_t n_list;
+  const uint32_t* lists;
+  /* nodes */
+  int32_t n_node;
+  const int32_t* node_nstrat;
+  const int32_t* node_nargs;
+  const int32_t* node_op;
+  const int64_t* node_comp_off; /* [n_node+1] */
+  const int32_t* node_edge_off; /* [n_node+1] */
+  const int64_t* node_prog_off; /* -1 = none */
+  const int32_t* node_multiplier;
+  int64_t n_prog;
+  const int64_t* prog;
+  const int64_t* explicit_flops; /* may be NULL */
+  const int64_t* explicit_bytes; /* may be NULL */
+  /* edges */
+  int32_t n_edge;
+  const apc_edge* edges;
+  int64_t n_entry;
+  int32_t n_tile;
+  const int32_t* tile_edge; /* [n_tile] edge owning entry tile << APC_TILE_SHIFT */
+  int64_t n_default;
+  const double* default_vals;
+} apc_problem;
+
+int apc_version(void);
+const char* apc_last_error(void);
+
+/* Host helper.  Replaces MeshTopoInfo.build_from_mesh
+ * (torch:distributed/tensor/_collective_utils.py:246-278): per-mesh-dim
+ * bandwidth (GB/s) and latency (us) from the mesh shape and the number of
+ * devices per host.  bw/lat: host arrays of ndim doubles. */
+int apc_mesh_topology(const int32_t* mesh_shape, int32_t ndim, int32_t devices_per_host,
+                      double* bw, double* lat);
+
+/* Host helper.  Replaces _get_device_limit / _get_device_tflops /
+ * _get_device_gmem_bandwidth (autoparallel/cost_models/compute_estimation.py:258-297)
+ * for the devices this library knows: fills gmem_bw and tflops[] of *model.
+ * Returns APC_ERR_UNSUPPORTED for an unknown device name (the reference raises
+ * ValueError there). */
+int apc_device_limits(const char* device_name, apc_model* model);
+
+/* Number of doubles of the pair table apc_build_pair_table fills:
+ * n_meta * n_tuple * n_tuple. */
+int64_t apc_pair_table_size(const apc_problem* p);
+
+/* Replaces estimate_strategy_comms_cost + redistribute_cost + collective_comm_cost
+ * + all_to_all_cost (autoparallel/cost_models/collective_runtime_estimation.py:65-110,
+ * 115-229, 239-262), torch's allgather/allreduce/reduce_scatter_cost
+ * (torch:distributed/tensor/_collective_utils.py:281-313) and
+ * compute_read_write_time (autoparallel/cost_models/compute_estimation.py:391-403),
+ * evaluated for every (tensor meta, source placements, target placements)
+ * triple: table[(m * n_tuple + src) * n_tuple + tgt], microseconds, +inf for
+ * forbidden transitions. */
+int apc_build_pair_table(const apc_problem* p, double* table, void* stream);
+
+/* Replaces estimate_strategy_runtime_cost
+ * (autoparallel/cost_models/compute_estimation.py:438-493, with
+ * _get_sharded_shape_stride :300-318 and compute_memory_cost :321-331) for
+ * every (node, out_idx): compute[node_comp_off[v] + o] in microseconds, and
+ * per_arg = compute / num_args (autoparallel/optimize_sharding.py:516).
+ * status (device int32[1], zeroed by the caller) is set non-zero if a node
+ * with flops has an input dtype without a tflops entry (ValueError in the
+ * reference, compute_estimation.py:287-291). */
+int apc_node_compute_costs(const apc_problem* p, double* compute, double* per_arg,
+                           int32_t* status, void* stream);
+
+/* Replaces the entry loop of ShardingOptimizer._build_decision_vars and
+ * _compute_edge_costs (autoparallel/optimize_sharding.py:446-479, 511-552):
+ * for every entry (node, argi, out_idx, inp_idx)
+ *     comm  = table lookup / direct evaluation / default row value
+ *     flags = APC_ENTRY_TRANSITION | APC_ENTRY_NONFINITE
+ *     cost  = comm + per_arg + transition
+ * and, if clamp_inf != 0, add_inf_cost_constraint's rewrite of non-finite cost
+ * to 10000.0 (:803-812).  table may be NULL: every entry is then evaluated
+ * directly (same arithmetic, no table memory).  comm / cost / flags may each
+ * be NULL to skip that output. */
+int apc_edge_costs(const apc_problem* p, const double* table, const double* per_arg,
+                   double* comm, double* cost, uint8_t* flags, int32_t clamp_inf, void* stream);
+
+/* Replaces apply_prefetch_discount (autoparallel/optimize_sharding.py:824-875)
+ * on the entry arrays, for edges flagged APC_EDGE_PREFETCHABLE: comm *= scale
+ * and cost = comm + per_arg + transition where 0 < comm < inf.  n_modified:
+ * device uint64[1], zeroed by the caller, receives the number of entries changed. */
+int apc_apply_prefetch_discount(const apc_problem* p, const double* per_arg, double scale,
+                                double* comm, double* cost, const uint8_t* flags,
+                                unsigned long long* n_modified, void* stream);
+
+/* Replaces the coefficient rule of _set_objective
+ * (autoparallel/optimize_sharding.py:879-885): obj = cost * node_multiplier. */
+int apc_objective_coeffs(const apc_problem* p, const double* cost, double* obj, void* stream);
+
+/* Replaces _compute_solution_cost (autoparallel/optimize_sharding.py:1056-1111)
+ * and evaluates the ILP objective (:879-885) with its inf-cost rows (:803-812)
+ * for a batch of assignments.  assign: uint16 [n_node][n_assign] (node-major),
+ * the chosen out_idx per node.  out: double [n_assign][6] =
+ * (total, compute, comm, transition, ilp_objective, n_forbidden_selected).
+ * Sums run in graph node order then argument order, as the reference's loop. */
+int apc_score_assignments(const apc_problem* p, const double* per_arg, const double* comm,
+                          const double* cost, const uint8_t* flags, const uint16_t* assign,
+                          int64_t n_assign, double* out, void* stream);
+
+/* As apc_score_assignments, with assignment a drawn on the fly: out_idx of node
+ * v = mix(seed, a, v) mod node_nstrat[v] (counter-based, nothing materialised).
+ * apc_random_assignment (host) gives the same draw for checking. */
+int apc_score_random_assignments(const apc_problem* p, const double* per_arg, const double* comm,
+                                 const double* cost, const uint8_t* flags, uint64_t seed,
+                                 int64_t first, int64_t n_assign, double* out, void* stream);
+uint32_t apc_random_assignment(uint64_t seed, int64_t a, int32_t node, int32_t nstrat);
+
+/* Replaces _create_all_options + remove_invalid_configs for input/parameter
+ * nodes (autoparallel/shardings/propagation_rules.py:127-158, 184-201): for
+ * each of n tensors (rank[i], shape[i][APC_MAX_RANK]) writes, for every
+ * candidate c in itertools.product order over {R, S(0..rank-1)}^ndim,
+ * valid[cand_off[i] + c] (uint8) and its placement bytes
+ * plc[(cand_off[i] + c) * APC_MAX_MESH_DIMS ..]. */
+int apc_enumerate_input_options(const apc_model* model, int32_t n, const int32_t* rank,
+                                const int64_t* shape, const int64_t* cand_off, uint8_t* valid,
+                                uint8_t* plc, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* APC_H_ */

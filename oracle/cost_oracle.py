@@ -348,9 +348,9 @@ class GraphOracle:
         self.ndim = len(self.topo.mesh_shape)
         self._comm_cache: Dict[tuple, float] = {}
         self._compute_cache: Dict[tuple, float] = {}
-        # plain-Python views (tuple per spec) so the timed loop does no numpy
-        self._spec_plc = [tuple(int(x) for x in row[: self.ndim]) for row in g.spec_plc]
-        self._spec_meta = [int(x) for x in g.spec_meta]
+        # plain-Python views so the timed loop does no numpy.  A spec is a
+        # 32-bit word: meta id in the high 20 bits, placement-tuple id below.
+        self._tuple_plc = [tuple(int(x) for x in row[: self.ndim]) for row in g.tuple_plc]
         self._meta = []
         for m in range(g.meta_rank.shape[0]):
             r = int(g.meta_rank[m])
@@ -362,7 +362,7 @@ class GraphOracle:
                     int(g.meta_dtype[m]),
                 )
             )
-        self._lists = [int(x) for x in g.lists]
+        self._lists = [(-1 if int(x) == 0xFFFFFFFF else int(x)) for x in g.lists]
 
     def reset_caches(self):
         self._comm_cache.clear()
@@ -370,18 +370,15 @@ class GraphOracle:
 
     # -- per-entry pieces ----------------------------------------------------
     def comm_cost(self, src_id: int, tgt_id: int) -> float:
-        key = (
-            self._spec_plc[src_id],
-            self._spec_meta[src_id],
-            self._spec_plc[tgt_id],
-            self._spec_meta[tgt_id],
-        )
+        # (placements, tensor meta) of both sides, as the reference's memo key
+        key = (src_id, tgt_id)
         c = self._comm_cache.get(key)
         if c is not None:
             return c
-        shape, stride, itemsize, _ = self._meta[self._spec_meta[src_id]]
+        shape, stride, itemsize, _ = self._meta[src_id >> 12]
         c = estimate_strategy_comms_cost(
-            self._spec_plc[src_id], shape, stride, itemsize, self._spec_plc[tgt_id], self.topo, self.dev
+            self._tuple_plc[src_id & 0xFFF], shape, stride, itemsize,
+            self._tuple_plc[tgt_id & 0xFFF], self.topo, self.dev
         )
         self._comm_cache[key] = c
         return c
@@ -409,8 +406,8 @@ class GraphOracle:
                 shapes.append(None)
                 isz.append(0)
                 continue
-            shape, stride, itemsize, _ = self._meta[self._spec_meta[sid]]
-            ls, _ = sharded_shape_stride(shape, stride, self._spec_plc[sid], self.topo.mesh_shape)
+            shape, stride, itemsize, _ = self._meta[sid >> 12]
+            ls, _ = sharded_shape_stride(shape, stride, self._tuple_plc[sid & 0xFFF], self.topo.mesh_shape)
             shapes.append(ls)
             isz.append(itemsize)
         flops, nbytes = run_program(self._prog_slice(po), shapes, isz)
@@ -421,7 +418,7 @@ class GraphOracle:
     def _first_dtype(self, in_ids) -> int:
         for sid in in_ids:
             if sid >= 0:
-                return self._meta[self._spec_meta[sid]][3]
+                return self._meta[sid >> 12][3]
         return 1  # torch.float32 default (compute_estimation.py:418-419)
 
     def _prog_len(self, po: int) -> int:
@@ -458,7 +455,7 @@ class GraphOracle:
         cost = np.zeros(E, np.float64)
         compute = np.zeros(g.num_compute, np.float64)
         lists = self._lists
-        spec_plc = self._spec_plc
+        tuple_plc = self._tuple_plc
         node_range = range(g.num_nodes) if nodes is None else nodes
         for v in node_range:
             S = int(g.node_nstrat[v])
@@ -481,7 +478,7 @@ class GraphOracle:
                         src_id = lists[src_list + j] if (flags & 1) else -1
                         if src_id >= 0 and tgt_id >= 0:
                             c = self.comm_cost(src_id, tgt_id)
-                            if spec_plc[src_id] != spec_plc[tgt_id]:
+                            if tuple_plc[src_id & 0xFFF] != tuple_plc[tgt_id & 0xFFF]:
                                 t = 1
                         else:
                             c = float(g.default_vals[doff + o * ssrc + j])
