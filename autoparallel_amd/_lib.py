@@ -45,6 +45,12 @@ class ApcProblem(C.Structure):
         ("node_comp_off", C.c_void_p),
         ("node_edge_off", C.c_void_p),
         ("node_prog_off", C.c_void_p),
+        ("node_prog_len", C.c_void_p),
+        ("max_node_args", C.c_int32),
+        ("max_rank", C.c_int32),
+        ("n_compute", C.c_int64),
+        ("n_comp_node", C.c_int32),
+        ("comp_nodes", C.c_void_p),
         ("node_multiplier", C.c_void_p),
         ("n_prog", C.c_int64),
         ("prog", C.c_void_p),
@@ -53,10 +59,18 @@ class ApcProblem(C.Structure):
         ("n_edge", C.c_int32),
         ("edges", C.c_void_p),
         ("n_entry", C.c_int64),
-        ("n_tile", C.c_int32),
-        ("tile_edge", C.c_void_p),
+        ("n_slot", C.c_int64),
+        ("n_chunk", C.c_int64),
+        ("chunk_edge", C.c_void_p),
+        ("n_item", C.c_int32),
+        ("items", C.c_void_p),
         ("n_default", C.c_int64),
         ("default_vals", C.c_void_p),
+        ("n_run", C.c_int32),
+        ("run_list", C.c_void_p),
+        ("run_len", C.c_void_p),
+        ("run_table_off", C.c_void_p),
+        ("table_size", C.c_int64),
     ]
 
 
@@ -73,6 +87,14 @@ _SIGNATURES = {
         C.c_int,
         [C.POINTER(ApcProblem), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
          C.c_int32, C.c_void_p]),
+    "apc_prepare": (
+        C.c_int,
+        [C.POINTER(ApcProblem), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
+    "apc_build_all": (
+        C.c_int,
+        [C.POINTER(ApcProblem), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+         C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]),
+    "apc_calibration_copy": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p]),
     "apc_apply_prefetch_discount": (
         C.c_int,
         [C.POINTER(ApcProblem), C.c_void_p, C.c_double, C.c_void_p, C.c_void_p, C.c_void_p,

@@ -1,11 +1,12 @@
 // HIP kernels and C ABI of the sharding-search cost engine (gfx950 / CDNA4).
 //
 // Everything here is HBM-bound integer/fp64 scalar work: no matrix cores.  The
-// entry kernel is a flat scan over the E cost entries: consecutive lanes own
-// consecutive entries, so every store instruction writes 512 contiguous bytes
-// (fp64) or 64 bytes (flag bytes).  All floating-point code is compiled with
-// -ffp-contract=off: the reference is a chain of separately rounded binary64
-// operations, and the results here are bit-identical to it.
+// entry kernel is a flat scan over the E cost entries: every lane owns 4
+// consecutive entries, so a wavefront writes 2 KB of contiguous fp64 per output
+// array with 16-byte stores, and 256 contiguous flag bytes with 4-byte stores.
+// All floating-point code is compiled with -ffp-contract=off: the reference is
+// a chain of separately rounded binary64 operations, and the results here are
+// bit-identical to it.
 #include <hip/hip_runtime.h>
 #include <math.h>
 #include <stdint.h>
@@ -35,6 +36,10 @@ int check_launch(const char* what) {
 constexpr uint32_t kTupleMask = (1u << APC_TUPLE_BITS) - 1u;
 constexpr int kKindMask = 0xC0, kShard = 0x40, kPartial = 0x80, kArgMask = 0x3F;
 constexpr int kPartialSum = 0x80;
+constexpr int kBlock = 256;
+
+typedef double double2_t __attribute__((ext_vector_type(2)));
+typedef long long ll2_t __attribute__((ext_vector_type(2)));
 
 // ---------------------------------------------------------------------------
 // Cost model, scalar device functions (order of operations is the contract)
@@ -146,90 +151,171 @@ __device__ __forceinline__ bool meta_contiguous(const apc_problem& p, uint32_t m
                        p.meta_stride + (size_t)mid * APC_MAX_RANK, p.meta_rank[mid]);
 }
 
-// ---------------------------------------------------------------------------
-// Kernel: pair table  T[m][src tuple][tgt tuple]
-// ---------------------------------------------------------------------------
-__global__ void __launch_bounds__(256) pair_table_kernel(apc_problem p, double* __restrict__ table) {
-  const int64_t nt = p.n_tuple;
-  const int64_t per_meta = nt * nt;
-  const int64_t total = per_meta * p.n_meta;
-  for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
-       idx += (int64_t)gridDim.x * blockDim.x) {
-    const uint32_t mid = (uint32_t)(idx / per_meta);
-    const int64_t r = idx - (int64_t)mid * per_meta;
-    const uint32_t s = (uint32_t)(r / nt), t = (uint32_t)(r - (int64_t)s * nt);
-    table[idx] = redistribute_cost(load_tuple(p.tuple_plc, s), load_tuple(p.tuple_plc, t),
-                                   meta_bytes(p, mid), meta_contiguous(p, mid), p.model);
-  }
+__device__ __forceinline__ int64_t ceil_div_pos(int64_t s, int64_t n) {
+  // sizes are almost always below 2^31: a 32-bit divide is several times cheaper
+  if (s <= 0x7FFFFFFF && n <= 0x7FFFFFFF)
+    return (int64_t)(((uint32_t)s + (uint32_t)n - 1u) / (uint32_t)n);
+  return (s + n - 1) / n;
 }
 
 // ---------------------------------------------------------------------------
-// Kernel: node compute estimate
+// Kernel: pair table T[m][src tuple][tgt tuple] and node compute estimate
 // ---------------------------------------------------------------------------
 // Local size of dim d of the tensor behind spec word w: the global size, ceil-
 // divided by each mesh dim that shards d, in mesh-dim order
 // (_get_sharded_shape_stride, compute_estimation.py:300-318).
 __device__ __forceinline__ int64_t local_size(const apc_problem& p, uint32_t w, int d) {
+  if (w == APC_SPEC_NONE) return 1;  // a program never names a non-tensor arg
   const uint32_t mid = w >> APC_TUPLE_BITS;
   int64_t s = p.meta_shape[(size_t)mid * APC_MAX_RANK + d];
   const uint32_t plc = load_tuple(p.tuple_plc, w & kTupleMask);
   for (int i = 0; i < p.model.ndim; ++i) {
     const int c = (plc >> (8 * i)) & 0xFF;
-    if ((c & kKindMask) == kShard && (c & kArgMask) == d) {
-      const int64_t n = p.model.mesh_shape[i];
-      s = (s + n - 1) / n;
-    }
+    if ((c & kKindMask) == kShard && (c & kArgMask) == d)
+      s = ceil_div_pos(s, p.model.mesh_shape[i]);
   }
   return s;
 }
 
-__device__ __forceinline__ int64_t local_numel(const apc_problem& p, uint32_t w) {
-  const int rank = p.meta_rank[w >> APC_TUPLE_BITS];
-  int64_t n = 1;
-  for (int d = 0; d < rank; ++d) n *= local_size(p, w, d);
-  return n;
+// Roofline tail of estimate_strategy_runtime_cost (compute_estimation.py:474-489).
+__device__ __forceinline__ double roofline(const apc_problem& p, int64_t flops, int64_t nbytes,
+                                           int dtype, int32_t* __restrict__ status) {
+  const double rw = rw_time((double)nbytes, p.model.gmem_bw);
+  if (flops == 0) return rw;
+  const double tf = (dtype >= 0 && dtype < APC_NUM_DTYPES) ? p.model.tflops[dtype] : 0.0;
+  if (!(tf > 0.0)) {
+    atomicExch(status, 1);
+    return NAN;
+  }
+  const double gpu_flops = tf * 1e12;
+  double ct = (double)flops / gpu_flops * 1e6;
+  ct = ct / 0.70;
+  return ct >= rw ? ct : rw;  // max(ct, rw): keeps ct on ties
 }
 
-__global__ void __launch_bounds__(256)
-node_compute_kernel(apc_problem p, double* __restrict__ compute, double* __restrict__ per_arg,
-                    int32_t* __restrict__ status) {
-  const int64_t total = p.node_comp_off[p.n_node];
-  for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
-       idx += (int64_t)gridDim.x * blockDim.x) {
-    // node owning idx: last v with node_comp_off[v] <= idx
-    int lo = 0, hi = p.n_node;
-    while (hi - lo > 1) {
-      int mid = (lo + hi) >> 1;
-      if (p.node_comp_off[mid] <= idx) lo = mid; else hi = mid;
+constexpr int kNodesPerBlock = 4;  // one wavefront each
+constexpr int kProgCache = 128;    // int64 words of program staged per wave
+
+// One wavefront per evaluated node.  Phase 1: the lanes split the node's
+// (strategy, argument) pairs and write each argument's local (sharded) sizes
+// to LDS as local[arg][dim][strategy-slot]; all loads of a pair are issued
+// together.  Phase 2: one lane per strategy interprets the node's compute
+// program out of LDS.  Strategies are processed 64 at a time.  `slow` (the LDS
+// layout does not fit) reads sizes from memory on demand instead.
+__device__ __forceinline__ void node_compute_wave(const apc_problem& p, int v, int lane,
+                                                  int64_t* __restrict__ s_prog,
+                                                  int64_t* __restrict__ s_local, bool slow,
+                                                  double* __restrict__ compute,
+                                                  double* __restrict__ per_arg,
+                                                  int32_t* __restrict__ status) {
+  const int S = p.node_nstrat[v];
+  const int64_t base = p.node_comp_off[v];
+  const int nargs = p.node_nargs[v];
+  const int op = p.node_op[v];
+  if (op == APC_OP_ZERO) {
+    const double pa = 0.0 / (double)nargs;
+    for (int o = lane; o < S; o += 64) {
+      compute[base + o] = 0.0;
+      per_arg[base + o] = pa;
     }
-    const int v = lo;
-    const int o = (int)(idx - p.node_comp_off[v]);
-    const int nargs = p.node_nargs[v];
-    const int op = p.node_op[v];
-    if (op == APC_OP_ZERO) {
-      compute[idx] = 0.0;
-      per_arg[idx] = 0.0 / (double)nargs;
-      continue;
+    return;
+  }
+  const int e0 = p.node_edge_off[v], e1 = p.node_edge_off[v + 1];
+  const int na = e1 - e0;
+  const int max_rank = p.max_rank;
+  const int slots = max_rank + 1;  // per argument: max_rank sizes + one info word
+  const int64_t* prog = nullptr;
+  if (op == APC_OP_PROGRAM) {
+    prog = p.prog + p.node_prog_off[v];
+    const int len = p.node_prog_len[v];
+    if (len <= kProgCache) {
+      for (int i = lane; i < len; i += 64) s_prog[i] = prog[i];
+      prog = s_prog;  // LDS operations of one wave execute in order
     }
-    const int e0 = p.node_edge_off[v], e1 = p.node_edge_off[v + 1];
+  }
+  for (int o0 = 0; o0 < S; o0 += 64) {
+    const int chunk = (S - o0 < 64) ? (S - o0) : 64;
+    if (!slow && op == APC_OP_PROGRAM) {
+      for (int t = lane; t < chunk * na; t += 64) {
+        const int a = t / chunk, oo = t - a * chunk;
+        const uint32_t w = p.lists[(size_t)p.edges[e0 + a].dst_list + o0 + oo];
+        const bool none = (w == APC_SPEC_NONE);
+        const uint32_t mid = none ? 0u : (w >> APC_TUPLE_BITS);
+        const int rank = none ? 0 : p.meta_rank[mid];
+        const uint32_t plc = load_tuple(p.tuple_plc, none ? 0u : (w & kTupleMask));
+        const ll2_t* r = reinterpret_cast<const ll2_t*>(p.meta_shape + (size_t)mid * APC_MAX_RANK);
+        ll2_t row[APC_MAX_RANK / 2];
+#pragma unroll
+        for (int q = 0; q < APC_MAX_RANK / 2; ++q) row[q] = r[q];
+#pragma unroll
+        for (int d = 0; d < APC_MAX_RANK; ++d) {
+          if (d >= max_rank) break;  // wave-uniform
+          int64_t sz = (d & 1) ? row[d >> 1].y : row[d >> 1].x;
+          if (d >= rank) {
+            sz = 1;
+          } else {
+            for (int i = 0; i < p.model.ndim; ++i) {
+              const int c = (plc >> (8 * i)) & 0xFF;
+              if ((c & kKindMask) == kShard && (c & kArgMask) == d)
+                sz = ceil_div_pos(sz, p.model.mesh_shape[i]);
+            }
+          }
+          s_local[(a * slots + d) * 64 + oo] = sz;
+        }
+        // info word: rank | itemsize << 8 | dtype << 40, or -1 for a missing spec
+        s_local[(a * slots + max_rank) * 64 + oo] =
+            none ? -1
+                 : ((int64_t)rank | ((int64_t)p.meta_itemsize[mid] << 8) |
+                    ((int64_t)p.meta_dtype[mid] << 40));
+      }
+    }
+    const int o = o0 + lane;
+    if (lane >= chunk) continue;
+    const int64_t idx = base + o;
     int64_t flops = 0, nbytes = 0;
     int dtype = 1;  // float32 when the node has no tensor argument
     bool have_dtype = false;
-    for (int e = e0; e < e1; ++e) {
-      const uint32_t w = p.lists[(size_t)p.edges[e].dst_list + o];
-      if (w == APC_SPEC_NONE) continue;
-      if (!have_dtype) { dtype = p.meta_dtype[w >> APC_TUPLE_BITS]; have_dtype = true; }
+    const bool staged = !slow && op == APC_OP_PROGRAM;
+    auto size_of = [&](int a, int d) -> int64_t {
+      if (staged) return s_local[(a * slots + d) * 64 + lane];
+      return local_size(p, p.lists[(size_t)p.edges[e0 + a].dst_list + o], d);
+    };
+    // rank of argument a, or -1 if it has no spec
+    auto rank_of = [&](int a) -> int {
+      if (staged) {
+        const int64_t info = s_local[(a * slots + max_rank) * 64 + lane];
+        return info < 0 ? -1 : (int)(info & 0xFF);
+      }
+      const uint32_t w = p.lists[(size_t)p.edges[e0 + a].dst_list + o];
+      return w == APC_SPEC_NONE ? -1 : p.meta_rank[w >> APC_TUPLE_BITS];
+    };
+    for (int a = 0; a < na; ++a) {
+      int rank, isz, dt;
+      if (staged) {
+        const int64_t info = s_local[(a * slots + max_rank) * 64 + lane];
+        if (info < 0) continue;
+        rank = (int)(info & 0xFF);
+        isz = (int)((info >> 8) & 0xFFFFFFFF);
+        dt = (int)(info >> 40);
+      } else {
+        const uint32_t w = p.lists[(size_t)p.edges[e0 + a].dst_list + o];
+        if (w == APC_SPEC_NONE) continue;
+        const uint32_t mid = w >> APC_TUPLE_BITS;
+        rank = p.meta_rank[mid];
+        isz = p.meta_itemsize[mid];
+        dt = p.meta_dtype[mid];
+      }
+      if (!have_dtype) { dtype = dt; have_dtype = true; }
+      if (op != APC_OP_PROGRAM) continue;
+      int64_t numel = 1;
+      for (int d = 0; d < rank; ++d) numel *= size_of(a, d);
+      nbytes += numel * (int64_t)isz;
     }
     if (op == APC_OP_EXPLICIT) {
       flops = p.explicit_flops[idx];
       nbytes = p.explicit_bytes[idx];
     } else {
-      for (int e = e0; e < e1; ++e) {
-        const uint32_t w = p.lists[(size_t)p.edges[e].dst_list + o];
-        if (w == APC_SPEC_NONE) continue;
-        nbytes += local_numel(p, w) * (int64_t)p.meta_itemsize[w >> APC_TUPLE_BITS];
-      }
-      const int64_t* pr = p.prog + p.node_prog_off[v];
+      const int64_t* pr = prog;
       const int n_terms = (int)pr[0], n_outs = (int)pr[1];
       pr += 2;
       for (int t = 0; t < n_terms; ++t) {
@@ -237,8 +323,7 @@ node_compute_kernel(apc_problem p, double* __restrict__ compute, double* __restr
         const int nfac = (int)pr[1];
         pr += 2;
         for (int f = 0; f < nfac; ++f) {
-          const uint32_t w = p.lists[(size_t)p.edges[e0 + (int)pr[0]].dst_list + o];
-          term *= local_size(p, w, (int)pr[1]);
+          term *= size_of((int)pr[0], (int)pr[1]);
           pr += 2;
         }
         flops += term;
@@ -254,18 +339,15 @@ node_compute_kernel(apc_problem p, double* __restrict__ compute, double* __restr
           if (kind == 0) {
             size = pr[1];
           } else if (kind == 1) {
-            const uint32_t w = p.lists[(size_t)p.edges[e0 + (int)pr[1]].dst_list + o];
-            size = local_size(p, w, (int)pr[2]);
+            size = size_of((int)pr[1], (int)pr[2]);
           } else {  // broadcast of all tensor args at a right-aligned position
             size = 1;
             const int pos = (int)pr[1];
-            for (int e = e0; e < e1; ++e) {
-              const uint32_t w = p.lists[(size_t)p.edges[e].dst_list + o];
-              if (w == APC_SPEC_NONE) continue;
-              const int r = p.meta_rank[w >> APC_TUPLE_BITS];
+            for (int a = 0; a < na; ++a) {
+              const int r = rank_of(a);
               if (pos >= r) continue;
-              const int64_t s = local_size(p, w, r - 1 - pos);
-              if (s != 1) size = s;
+              const int64_t sz = size_of(a, r - 1 - pos);
+              if (sz != 1) size = sz;
             }
           }
           numel *= size;
@@ -274,124 +356,230 @@ node_compute_kernel(apc_problem p, double* __restrict__ compute, double* __restr
         nbytes += numel * isz;
       }
     }
-    // roofline (compute_estimation.py:474-489)
-    const double rw = rw_time((double)nbytes, p.model.gmem_bw);
-    double result;
-    if (flops == 0) {
-      result = rw;
-    } else {
-      const double tf = (dtype >= 0 && dtype < APC_NUM_DTYPES) ? p.model.tflops[dtype] : 0.0;
-      if (!(tf > 0.0)) {
-        atomicExch(status, 1);
-        result = NAN;
-      } else {
-        const double gpu_flops = tf * 1e12;
-        double ct = (double)flops / gpu_flops * 1e6;
-        ct = ct / 0.70;
-        result = ct >= rw ? ct : rw;  // max(ct, rw): keeps ct on ties
-      }
-    }
+    const double result = roofline(p, flops, nbytes, dtype, status);
     compute[idx] = result;
     per_arg[idx] = result / (double)nargs;
   }
 }
 
+// Row tables: element idx of the table belongs to run r (binary search in
+// run_table_off), target tuple t and source position j.
+__device__ __forceinline__ void pair_table_block(const apc_problem& p, double* __restrict__ table,
+                                                 int block, int nblocks) {
+  const int64_t total = p.table_size;
+  for (int64_t idx = (int64_t)block * blockDim.x + threadIdx.x; idx < total;
+       idx += (int64_t)nblocks * blockDim.x) {
+    int lo = 0, hi = p.n_run;
+    while (hi - lo > 1) {
+      const int mid = (lo + hi) >> 1;
+      if (p.run_table_off[mid] <= idx) lo = mid; else hi = mid;
+    }
+    const uint32_t len = (uint32_t)p.run_len[lo];
+    const uint32_t r = (uint32_t)(idx - p.run_table_off[lo]);
+    const uint32_t t = r / len, j = r - t * len;
+    const uint32_t sw = p.lists[(size_t)p.run_list[lo] + j];
+    double c = 0.0;  // a missing spec never reads its table slot
+    if (sw != APC_SPEC_NONE) {
+      const uint32_t sm = sw >> APC_TUPLE_BITS;
+      c = redistribute_cost(load_tuple(p.tuple_plc, sw & kTupleMask), load_tuple(p.tuple_plc, t),
+                            meta_bytes(p, sm), meta_contiguous(p, sm), p.model);
+    }
+    table[idx] = c;
+  }
+}
+
+// Blocks [0, table_blocks) fill the pair table, the rest price the nodes of
+// comp_nodes: the two are independent, and one launch saves a dispatch on a
+// problem this small.  Dynamic LDS: per wave kProgCache words of program, then
+// (unless slow) max_node_args * (max_rank + 1) * 64 words of local sizes and
+// argument info.
+__global__ void __launch_bounds__(256)
+prepare_kernel(apc_problem p, double* __restrict__ table, int table_blocks, int slow,
+               double* __restrict__ compute, double* __restrict__ per_arg,
+               int32_t* __restrict__ status) {
+  extern __shared__ int64_t s_dyn[];
+  if ((int)blockIdx.x < table_blocks) {
+    pair_table_block(p, table, blockIdx.x, table_blocks);
+    return;
+  }
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int i = ((int)blockIdx.x - table_blocks) * kNodesPerBlock + wave;
+  if (i >= p.n_comp_node) return;
+  const int v = __builtin_amdgcn_readfirstlane(p.comp_nodes[i]);
+  const int per_wave = kProgCache + (slow ? 0 : p.max_node_args * (p.max_rank + 1) * 64);
+  int64_t* s_prog = s_dyn + (size_t)wave * per_wave;
+  node_compute_wave(p, v, threadIdx.x & 63, s_prog, s_prog + kProgCache, slow != 0, compute,
+                    per_arg, status);
+}
+
 // ---------------------------------------------------------------------------
 // Kernel: cost entries
 // ---------------------------------------------------------------------------
-constexpr int kTile = 1 << APC_TILE_SHIFT;  // entries per workgroup
-constexpr int kBlock = 256;
+constexpr int kPerLane = 4;                   // consecutive entries per lane
+constexpr int kItemEntries = 64 * kPerLane;   // entries per work item (one wavefront)
+static_assert(sizeof(apc_edge) == 64, "edge record layout");
+static_assert(kItemEntries == APC_ITEM_ENTRIES, "work items are built for this kernel");
 
-struct EntryOut {
-  double comm;
-  double pa;
-  int trans;
-};
+// Edge that owns slot idx.  Edge blocks start on multiples of 16 slots, so each
+// 16-slot chunk belongs to exactly one edge.
+__device__ __forceinline__ apc_edge find_edge(const apc_problem& p, int64_t idx) {
+  return p.edges[p.chunk_edge[idx >> APC_CHUNK_SHIFT]];
+}
 
-// Evaluate entry `local` of edge `ed`.
+// comm / transition of one entry, general path (direct evaluation, missing
+// specs, default rows).
 template <bool kUseTable>
-__device__ __forceinline__ EntryOut eval_entry(const apc_problem& p, const apc_edge& ed,
-                                               uint32_t local, const double* __restrict__ table,
-                                               const double* __restrict__ per_arg) {
-  const uint32_t ssrc = (uint32_t)ed.ssrc;
-  const uint32_t o = local / ssrc;
-  const uint32_t j = local - o * ssrc;
+__device__ __forceinline__ void eval_entry(const apc_problem& p, const apc_edge& ed, uint32_t o,
+                                           uint32_t j, const double* __restrict__ table,
+                                           double& comm, int& trans) {
   const uint32_t tw = p.lists[(size_t)ed.dst_list + o];
   const uint32_t sw =
       (ed.flags & APC_EDGE_HAS_PRODUCER) ? p.lists[(size_t)ed.src_list + j] : APC_SPEC_NONE;
-  EntryOut r;
-  r.pa = per_arg[ed.comp_base + o];
   if (sw != APC_SPEC_NONE && tw != APC_SPEC_NONE) {
     const uint32_t st = sw & kTupleMask, tt = tw & kTupleMask, sm = sw >> APC_TUPLE_BITS;
-    r.trans = (st != tt);
+    trans = (st != tt);
     if (kUseTable) {
-      r.comm = table[((size_t)sm * p.n_tuple + st) * p.n_tuple + tt];
+      comm = table[ed.table_off + (int64_t)tt * ed.ssrc + j];
     } else {
-      r.comm = redistribute_cost(load_tuple(p.tuple_plc, st), load_tuple(p.tuple_plc, tt),
-                                 meta_bytes(p, sm), meta_contiguous(p, sm), p.model);
+      comm = redistribute_cost(load_tuple(p.tuple_plc, st), load_tuple(p.tuple_plc, tt),
+                               meta_bytes(p, sm), meta_contiguous(p, sm), p.model);
     }
   } else {
-    r.comm = p.default_vals[ed.default_off + local];
-    r.trans = 0;
-  }
-  return r;
-}
-
-// Advance (e, ed) so that edge e contains entry idx.  Entries only move
-// forward, so this is a short walk from the tile's first edge.
-__device__ __forceinline__ void seek_edge(const apc_problem& p, int64_t idx, int& e, apc_edge& ed) {
-  while (idx >= ed.off + (int64_t)ed.ssrc * ed.sdst) {
-    ++e;
-    ed = p.edges[e];
+    comm = p.default_vals[ed.default_off + (int64_t)o * ed.ssrc + j];
+    trans = 0;
   }
 }
 
+// Entries [local0, local0 + 256) of one edge block: lane L owns entries
+// local0 + L + 64 k, k < 4, so that every load and store instruction of the
+// wavefront touches 64 consecutive entries (512 contiguous bytes of fp64):
+// measured on MI355X, stores whose 64 lanes cover one contiguous span stream
+// about 20% faster than lanes owning 32 contiguous bytes each.  The item record
+// is a copy of the edge record (plus local0), wave-uniform, so it lives in
+// scalar registers; a lane computes row/column of its entries, loads two spec
+// words, the per-arg compute term and one table element per entry, and stores.
+// Consecutive entries of a row are consecutive table elements, so the table
+// reads coalesce exactly like the stores.
+template <bool kUseTable>
+__device__ __forceinline__ void process_item(const apc_problem& p, const apc_edge& ed, int lane,
+                                             const double* __restrict__ table,
+                                             const double* __restrict__ per_arg,
+                                             double* __restrict__ comm, double* __restrict__ cost,
+                                             uint8_t* __restrict__ flags, int clamp_inf) {
+  const uint32_t ssrc = (uint32_t)ed.ssrc;
+  const uint32_t size = ssrc * (uint32_t)ed.sdst;
+  const bool prod = (ed.flags & APC_EDGE_HAS_PRODUCER) != 0;  // wave-uniform
+
+  uint32_t lk[kPerLane], ok[kPerLane], jk[kPerLane];
+  bool live[kPerLane];
+#pragma unroll
+  for (int k = 0; k < kPerLane; ++k) {
+    lk[k] = ed.local0 + (uint32_t)(k * 64 + lane);
+    live[k] = lk[k] < size;
+    const uint32_t l = live[k] ? lk[k] : 0u;
+    ok[k] = ed.magic ? __umulhi(l, ed.magic) : l / ssrc;
+    jk[k] = l - ok[k] * ssrc;
+  }
+  double v_comm[kPerLane], v_pa[kPerLane];
+  int v_trans[kPerLane];
+  if (kUseTable || !prod) {
+    uint32_t tw[kPerLane], sw[kPerLane];
+#pragma unroll
+    for (int k = 0; k < kPerLane; ++k) {
+      tw[k] = p.lists[(size_t)ed.dst_list + ok[k]];
+      v_pa[k] = per_arg[ed.comp_base + ok[k]];
+      sw[k] = prod ? p.lists[(size_t)ed.src_list + jk[k]] : APC_SPEC_NONE;
+    }
+    bool any_none = false;
+#pragma unroll
+    for (int k = 0; k < kPerLane; ++k) {
+      const bool none = (sw[k] == APC_SPEC_NONE) || (tw[k] == APC_SPEC_NONE);
+      const uint32_t st = sw[k] & kTupleMask, tt = tw[k] & kTupleMask;
+      v_comm[k] = (prod && !none) ? table[ed.table_off + (int64_t)(tt * ssrc + jk[k])] : 0.0;
+      v_trans[k] = none ? 0 : (st != tt);
+      any_none |= none;
+    }
+    if (any_none) {  // entries without a spec keep their default row value
+#pragma unroll
+      for (int k = 0; k < kPerLane; ++k) {
+        const bool none = (sw[k] == APC_SPEC_NONE) || (tw[k] == APC_SPEC_NONE);
+        if (none && live[k]) v_comm[k] = p.default_vals[ed.default_off + (int64_t)lk[k]];
+      }
+    }
+  } else {
+    // direct evaluation of every entry (no table)
+#pragma unroll
+    for (int k = 0; k < kPerLane; ++k) {
+      v_comm[k] = 0.0; v_pa[k] = 0.0; v_trans[k] = 0;
+      if (live[k]) {
+        eval_entry<false>(p, ed, ok[k], jk[k], table, v_comm[k], v_trans[k]);
+        v_pa[k] = per_arg[ed.comp_base + ok[k]];
+      }
+    }
+  }
+  // ---- assemble (optimize_sharding.py:544) and store
+#pragma unroll
+  for (int k = 0; k < kPerLane; ++k) {
+    double c = (v_comm[k] + v_pa[k]) + (double)v_trans[k];
+    const bool finite = isfinite(c);
+    if (clamp_inf && !finite) c = 10000.0;
+    if (live[k]) {
+      const int64_t idx = ed.off + lk[k];
+      if (comm) comm[idx] = v_comm[k];
+      if (cost) cost[idx] = c;
+      if (flags) flags[idx] = (uint8_t)(v_trans[k] | (finite ? 0 : APC_ENTRY_NONFINITE));
+    }
+  }
+}
+
+// Wave w takes items w, w + W, w + 2W, ... (W = waves in the grid, capped at
+// twice the chip's resident wave slots: measured slightly faster than one wave
+// per item, whose grid has tens of thousands of short-lived waves).
 template <bool kUseTable>
 __global__ void __launch_bounds__(kBlock)
 edge_cost_kernel(apc_problem p, const double* __restrict__ table,
                  const double* __restrict__ per_arg, double* __restrict__ comm,
                  double* __restrict__ cost, uint8_t* __restrict__ flags, int clamp_inf) {
-  const int64_t tile0 = (int64_t)blockIdx.x << APC_TILE_SHIFT;
-  int e = p.tile_edge[blockIdx.x];
-  apc_edge ed = p.edges[e];
-#pragma unroll
-  for (int u = 0; u < kTile / kBlock; ++u) {
-    const int64_t idx = tile0 + u * kBlock + threadIdx.x;
-    if (idx >= p.n_entry) break;
-    seek_edge(p, idx, e, ed);
-    const EntryOut r = eval_entry<kUseTable>(p, ed, (uint32_t)(idx - ed.off), table, per_arg);
-    double c = (r.comm + r.pa) + (double)r.trans;
-    const bool finite = isfinite(c);
-    if (clamp_inf && !finite) c = 10000.0;
-    if (comm) comm[idx] = r.comm;
-    if (cost) cost[idx] = c;
-    if (flags) flags[idx] = (uint8_t)(r.trans | (finite ? 0 : APC_ENTRY_NONFINITE));
+  const int n_waves = gridDim.x * (kBlock / 64);
+  const int w = __builtin_amdgcn_readfirstlane((int)(blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6)));
+  const int lane = threadIdx.x & 63;
+  for (int i = w; i < p.n_item; i += n_waves) {
+    const apc_edge item = p.items[i];
+    process_item<kUseTable>(p, item, lane, table, per_arg, comm, cost, flags, clamp_inf);
   }
 }
 
+// Plain copy kernel of known size: the reference point against which the
+// hardware traffic counters are scaled when a profile is taken.
+__global__ void __launch_bounds__(kBlock)
+calibration_copy_kernel(const double2_t* __restrict__ src, double2_t* __restrict__ dst, int64_t n) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+       i += (int64_t)gridDim.x * blockDim.x)
+    dst[i] = src[i];
+}
+
 // ---------------------------------------------------------------------------
-// Kernel: prefetch discount
+// Kernels: post-passes over the entry arrays (one entry per lane)
 // ---------------------------------------------------------------------------
 __global__ void __launch_bounds__(kBlock)
 prefetch_discount_kernel(apc_problem p, const double* __restrict__ per_arg, double scale,
                          double* __restrict__ comm, double* __restrict__ cost,
                          const uint8_t* __restrict__ flags, unsigned long long* n_modified) {
-  const int64_t tile0 = (int64_t)blockIdx.x << APC_TILE_SHIFT;
-  int e = p.tile_edge[blockIdx.x];
-  apc_edge ed = p.edges[e];
+  const int64_t idx = (int64_t)blockIdx.x * kBlock + threadIdx.x;
   unsigned int mine = 0;
-  for (int u = 0; u < kTile / kBlock; ++u) {
-    const int64_t idx = tile0 + u * kBlock + threadIdx.x;
-    if (idx >= p.n_entry) break;
-    seek_edge(p, idx, e, ed);
-    if (!(ed.flags & APC_EDGE_PREFETCHABLE) || ed.src_node < 0) continue;
-    double c = comm[idx];
-    if (c > 0.0 && isfinite(c)) {
-      const uint32_t o = (uint32_t)(idx - ed.off) / (uint32_t)ed.ssrc;
-      c = c * scale;
-      comm[idx] = c;
-      cost[idx] = (c + per_arg[ed.comp_base + o]) + (double)(flags[idx] & APC_ENTRY_TRANSITION);
-      ++mine;
+  if (idx < p.n_slot) {
+    const apc_edge ed = find_edge(p, idx);
+    const int64_t local = idx - ed.off;
+    if (local < (int64_t)ed.ssrc * ed.sdst && (ed.flags & APC_EDGE_PREFETCHABLE) &&
+        ed.src_node >= 0) {
+      double c = comm[idx];
+      if (c > 0.0 && isfinite(c)) {
+        const uint32_t o = (uint32_t)local / (uint32_t)ed.ssrc;
+        c = c * scale;
+        comm[idx] = c;
+        cost[idx] = (c + per_arg[ed.comp_base + o]) + (double)(flags[idx] & APC_ENTRY_TRANSITION);
+        mine = 1;
+      }
     }
   }
   // wavefront reduction, one atomic per wave
@@ -401,15 +589,11 @@ prefetch_discount_kernel(apc_problem p, const double* __restrict__ per_arg, doub
 
 __global__ void __launch_bounds__(kBlock)
 objective_kernel(apc_problem p, const double* __restrict__ cost, double* __restrict__ obj) {
-  const int64_t tile0 = (int64_t)blockIdx.x << APC_TILE_SHIFT;
-  int e = p.tile_edge[blockIdx.x];
-  apc_edge ed = p.edges[e];
-  for (int u = 0; u < kTile / kBlock; ++u) {
-    const int64_t idx = tile0 + u * kBlock + threadIdx.x;
-    if (idx >= p.n_entry) break;
-    seek_edge(p, idx, e, ed);
+  const int64_t idx = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (idx >= p.n_slot) return;
+  const apc_edge ed = find_edge(p, idx);
+  if (idx - ed.off < (int64_t)ed.ssrc * ed.sdst)
     obj[idx] = cost[idx] * (double)p.node_multiplier[ed.node];
-  }
 }
 
 // ---------------------------------------------------------------------------
@@ -419,7 +603,8 @@ objective_kernel(apc_problem p, const double* __restrict__ cost, double* __restr
 __host__ __device__ __forceinline__ uint32_t mix_assignment(uint64_t seed, int64_t a, int32_t node,
                                                             int32_t nstrat) {
   // splitmix64 finaliser over (seed, assignment, node)
-  uint64_t z = seed + 0x9E3779B97F4A7C15ull * (uint64_t)(a + 1) + 0xBF58476D1CE4E5B9ull * (uint64_t)(node + 1);
+  uint64_t z = seed + 0x9E3779B97F4A7C15ull * (uint64_t)(a + 1) +
+               0xBF58476D1CE4E5B9ull * (uint64_t)(node + 1);
   z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
   z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
   z = z ^ (z >> 31);
@@ -513,6 +698,9 @@ enumerate_kernel(apc_model m, int32_t n, const int32_t* __restrict__ rank,
   }
 }
 
+// ---------------------------------------------------------------------------
+// Host side
+// ---------------------------------------------------------------------------
 int validate_problem(const apc_problem* p) {
   if (!p) return fail(APC_ERR_INVALID, "null problem%s");
   if (p->model.ndim < 1 || p->model.ndim > APC_MAX_MESH_DIMS)
@@ -521,12 +709,20 @@ int validate_problem(const apc_problem* p) {
     if (p->model.mesh_shape[i] < 1) return fail(APC_ERR_INVALID, "mesh size < 1%s");
   if (p->n_meta < 0 || p->n_tuple < 0 || p->n_tuple > (1 << APC_TUPLE_BITS))
     return fail(APC_ERR_INVALID, "bad meta/tuple counts%s");
-  if (p->n_node < 0 || p->n_edge < 0 || p->n_entry < 0)
-    return fail(APC_ERR_INVALID, "negative sizes%s");
-  if (p->n_tile != (int32_t)((p->n_entry + kTile - 1) >> APC_TILE_SHIFT))
-    return fail(APC_ERR_INVALID, "n_tile does not match n_entry%s");
-  if (p->n_entry > 0 && (!p->edges || !p->tile_edge || !p->lists))
-    return fail(APC_ERR_INVALID, "null edge/list arrays%s");
+  if (p->n_node < 0 || p->n_edge < 0 || p->n_entry < 0 || p->n_comp_node < 0 ||
+      p->n_comp_node > p->n_node || p->n_compute < 0)
+    return fail(APC_ERR_INVALID, "bad sizes%s");
+  if (p->n_slot < p->n_entry || (p->n_slot & ((1 << APC_CHUNK_SHIFT) - 1)) ||
+      p->n_chunk != (p->n_slot >> APC_CHUNK_SHIFT) || p->n_item < 0)
+    return fail(APC_ERR_INVALID, "n_slot / n_chunk / n_item inconsistent%s");
+  if (p->n_entry > 0 && (!p->edges || !p->chunk_edge || !p->lists || !p->items))
+    return fail(APC_ERR_INVALID, "null edge/list/item arrays%s");
+  if (p->n_comp_node > 0 && !p->comp_nodes) return fail(APC_ERR_INVALID, "null comp_nodes%s");
+  if (p->n_run < 0 || p->table_size < 0 ||
+      (p->table_size > 0 && (!p->run_list || !p->run_len || !p->run_table_off)))
+    return fail(APC_ERR_INVALID, "bad run table description%s");
+  if (p->max_rank < 0 || p->max_rank > APC_MAX_RANK || p->max_node_args < 0)
+    return fail(APC_ERR_INVALID, "max_rank / max_node_args out of range%s");
   return 0;
 }
 
@@ -538,11 +734,50 @@ int grid_for(int64_t total, int block) {
   return (int)g;
 }
 
+int slot_grid(const apc_problem* p, int per_block, unsigned* grid) {
+  const int64_t g = (p->n_slot + per_block - 1) / per_block;
+  if (g > 0x7FFFFFFF) return fail(APC_ERR_INVALID, "too many entries for one launch%s");
+  *grid = (unsigned)g;
+  return 0;
+}
+
+int launch_prepare(const apc_problem* p, double* table, bool do_nodes, double* compute,
+                   double* per_arg, int32_t* status, hipStream_t stream) {
+  const int64_t tsize = table ? apc_pair_table_size(p) : 0;
+  int table_blocks = 0;
+  if (tsize > 0) {
+    int64_t b = (tsize + 255) / 256;
+    table_blocks = (int)(b > 2048 ? 2048 : b);
+  }
+  const int node_blocks = do_nodes ? (p->n_comp_node + kNodesPerBlock - 1) / kNodesPerBlock : 0;
+  if (table_blocks + node_blocks == 0) return 0;
+  // LDS for the local-size staging (a CU has 160 KB); beyond 96 KB per block,
+  // sizes are read on demand instead
+  const int64_t words = (int64_t)p->max_node_args * (p->max_rank + 1) * 64;
+  const int slow = ((kProgCache + words) * kNodesPerBlock * 8 > 96 * 1024 || p->n_meta == 0 ||
+                    p->n_tuple == 0) ? 1 : 0;
+  const size_t lds =
+      do_nodes ? (size_t)kNodesPerBlock * (kProgCache + (slow ? 0 : words)) * 8 : 0;
+  static bool attr_set = false;  // raise the 64 KB default limit of dynamic LDS once
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(prepare_kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
+    if (e != hipSuccess) {
+      snprintf(g_err, sizeof(g_err), "hipFuncSetAttribute: %s", hipGetErrorString(e));
+      return APC_ERR_LAUNCH;
+    }
+    attr_set = true;
+  }
+  hipLaunchKernelGGL(prepare_kernel, dim3(table_blocks + node_blocks), dim3(256), lds, stream, *p,
+                     table, table_blocks, slow, compute, per_arg, status);
+  return check_launch("prepare_kernel");
+}
+
 }  // namespace
 
 extern "C" {
 
-int apc_version(void) { return 1; }
+int apc_version(void) { return 2; }
 
 const char* apc_last_error(void) { return g_err; }
 
@@ -584,30 +819,31 @@ int apc_device_limits(const char* device_name, apc_model* model) {
 
 int64_t apc_pair_table_size(const apc_problem* p) {
   if (!p) return 0;
-  return (int64_t)p->n_meta * p->n_tuple * p->n_tuple;
+  return p->table_size;
 }
 
 int apc_build_pair_table(const apc_problem* p, double* table, void* stream) {
   if (int rc = validate_problem(p)) return rc;
-  const int64_t total = apc_pair_table_size(p);
-  if (total == 0) return 0;
+  if (apc_pair_table_size(p) == 0) return 0;
   if (!table) return fail(APC_ERR_INVALID, "apc_build_pair_table: null table%s");
-  hipLaunchKernelGGL(pair_table_kernel, dim3(grid_for(total, 256)), dim3(256), 0,
-                     (hipStream_t)stream, *p, table);
-  return check_launch("pair_table_kernel");
+  return launch_prepare(p, table, false, nullptr, nullptr, nullptr, (hipStream_t)stream);
 }
 
 int apc_node_compute_costs(const apc_problem* p, double* compute, double* per_arg,
                            int32_t* status, void* stream) {
   if (int rc = validate_problem(p)) return rc;
-  if (p->n_node == 0) return 0;
+  if (p->n_comp_node == 0) return 0;
   if (!compute || !per_arg || !status)
     return fail(APC_ERR_INVALID, "apc_node_compute_costs: null output%s");
-  // total strategies is not known on the host side of this ABI without a
-  // copy; size the grid from n_node (grid-stride loop covers the rest)
-  hipLaunchKernelGGL(node_compute_kernel, dim3(grid_for((int64_t)p->n_node * 16, 256)), dim3(256),
-                     0, (hipStream_t)stream, *p, compute, per_arg, status);
-  return check_launch("node_compute_kernel");
+  return launch_prepare(p, nullptr, true, compute, per_arg, status, (hipStream_t)stream);
+}
+
+int apc_prepare(const apc_problem* p, double* table, double* compute, double* per_arg,
+                int32_t* status, void* stream) {
+  if (int rc = validate_problem(p)) return rc;
+  if (!compute || !per_arg || !status) return fail(APC_ERR_INVALID, "apc_prepare: null output%s");
+  return launch_prepare(p, table, p->n_comp_node > 0, compute, per_arg, status,
+                        (hipStream_t)stream);
 }
 
 int apc_edge_costs(const apc_problem* p, const double* table, const double* per_arg, double* comm,
@@ -615,13 +851,31 @@ int apc_edge_costs(const apc_problem* p, const double* table, const double* per_
   if (int rc = validate_problem(p)) return rc;
   if (p->n_entry == 0) return 0;
   if (!per_arg) return fail(APC_ERR_INVALID, "apc_edge_costs: null per_arg%s");
+  unsigned grid = (unsigned)((p->n_item + (kBlock / 64) - 1) / (kBlock / 64));
+  const unsigned cap = 4096;  // 4 waves per block: twice the 8192 resident wave slots
+  if (grid > cap) grid = cap;
   if (table)
-    hipLaunchKernelGGL(edge_cost_kernel<true>, dim3(p->n_tile), dim3(kBlock), 0,
-                       (hipStream_t)stream, *p, table, per_arg, comm, cost, flags, clamp_inf);
+    hipLaunchKernelGGL(edge_cost_kernel<true>, dim3(grid), dim3(kBlock), 0, (hipStream_t)stream,
+                       *p, table, per_arg, comm, cost, flags, clamp_inf);
   else
-    hipLaunchKernelGGL(edge_cost_kernel<false>, dim3(p->n_tile), dim3(kBlock), 0,
-                       (hipStream_t)stream, *p, table, per_arg, comm, cost, flags, clamp_inf);
+    hipLaunchKernelGGL(edge_cost_kernel<false>, dim3(grid), dim3(kBlock), 0, (hipStream_t)stream,
+                       *p, table, per_arg, comm, cost, flags, clamp_inf);
   return check_launch("edge_cost_kernel");
+}
+
+int apc_build_all(const apc_problem* p, double* table, double* compute, double* per_arg,
+                  int32_t* status, double* comm, double* cost, uint8_t* flags, int32_t clamp_inf,
+                  void* stream) {
+  if (int rc = apc_prepare(p, table, compute, per_arg, status, stream)) return rc;
+  return apc_edge_costs(p, table, per_arg, comm, cost, flags, clamp_inf, stream);
+}
+
+int apc_calibration_copy(const void* src, void* dst, int64_t nbytes, void* stream) {
+  if (!src || !dst || nbytes <= 0 || (nbytes & 15))
+    return fail(APC_ERR_INVALID, "apc_calibration_copy: need non-null buffers, nbytes %% 16 == 0%s");
+  hipLaunchKernelGGL(calibration_copy_kernel, dim3(256 * 16), dim3(kBlock), 0, (hipStream_t)stream,
+                     (const double2_t*)src, (double2_t*)dst, nbytes / 16);
+  return check_launch("calibration_copy_kernel");
 }
 
 int apc_apply_prefetch_discount(const apc_problem* p, const double* per_arg, double scale,
@@ -631,8 +885,10 @@ int apc_apply_prefetch_discount(const apc_problem* p, const double* per_arg, dou
   if (p->n_entry == 0) return 0;
   if (!per_arg || !comm || !cost || !flags || !n_modified)
     return fail(APC_ERR_INVALID, "apc_apply_prefetch_discount: null argument%s");
-  hipLaunchKernelGGL(prefetch_discount_kernel, dim3(p->n_tile), dim3(kBlock), 0,
-                     (hipStream_t)stream, *p, per_arg, scale, comm, cost, flags, n_modified);
+  unsigned grid;
+  if (int rc = slot_grid(p, kBlock, &grid)) return rc;
+  hipLaunchKernelGGL(prefetch_discount_kernel, dim3(grid), dim3(kBlock), 0, (hipStream_t)stream,
+                     *p, per_arg, scale, comm, cost, flags, n_modified);
   return check_launch("prefetch_discount_kernel");
 }
 
@@ -641,8 +897,10 @@ int apc_objective_coeffs(const apc_problem* p, const double* cost, double* obj, 
   if (p->n_entry == 0) return 0;
   if (!cost || !obj || !p->node_multiplier)
     return fail(APC_ERR_INVALID, "apc_objective_coeffs: null argument%s");
-  hipLaunchKernelGGL(objective_kernel, dim3(p->n_tile), dim3(kBlock), 0, (hipStream_t)stream, *p,
-                     cost, obj);
+  unsigned grid;
+  if (int rc = slot_grid(p, kBlock, &grid)) return rc;
+  hipLaunchKernelGGL(objective_kernel, dim3(grid), dim3(kBlock), 0, (hipStream_t)stream, *p, cost,
+                     obj);
   return check_launch("objective_kernel");
 }
 

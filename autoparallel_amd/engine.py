@@ -10,7 +10,7 @@ import numpy as np
 import torch
 
 from . import _lib
-from .packed import MAX_MESH_DIMS, PackedGraph, TILE_SHIFT
+from .packed import CHUNK_SHIFT, MAX_MESH_DIMS, PackedGraph
 
 # Build the pair table when it is at most this many times the entry count (and
 # small in absolute terms); otherwise every entry is evaluated directly.
@@ -107,6 +107,12 @@ class CostEngine:
         p.node_comp_off = up("node_comp_off", g.node_comp_off)
         p.node_edge_off = up("node_edge_off", g.node_edge_off)
         p.node_prog_off = up("node_prog_off", g.node_prog_off)
+        p.node_prog_len = up("node_prog_len", g.node_prog_len)
+        p.max_node_args = g.max_node_args
+        p.max_rank = g.max_rank
+        p.n_compute = g.num_compute
+        p.n_comp_node = g.comp_nodes.shape[0]
+        p.comp_nodes = up("comp_nodes", g.comp_nodes)
         mult = g.node_multiplier if g.node_multiplier is not None else np.ones(g.num_nodes, np.int32)
         p.node_multiplier = up("node_multiplier", mult)
         p.n_prog = g.prog.shape[0]
@@ -116,24 +122,35 @@ class CostEngine:
         p.n_edge = g.num_edges
         p.edges = up("edges", g.edge_records())
         p.n_entry = g.num_entries
-        tile_edge = g.tile_edge_index()
-        p.n_tile = tile_edge.shape[0]
-        assert p.n_tile == (g.num_entries + (1 << TILE_SHIFT) - 1) >> TILE_SHIFT
-        p.tile_edge = up("tile_edge", tile_edge)
+        p.n_slot = g.num_slots
+        chunk_edge = g.chunk_edge_index()
+        p.n_chunk = chunk_edge.shape[0]
+        assert p.n_chunk == g.num_slots >> CHUNK_SHIFT
+        p.chunk_edge = up("chunk_edge", chunk_edge)
+        items = g.work_items()
+        p.n_item = items.shape[0]
+        p.items = up("items", items)
         p.n_default = g.default_vals.shape[0]
         p.default_vals = up("default_vals", g.default_vals)
+        run_list, run_len, run_table_off, _ = g.run_table()
+        p.n_run = run_list.shape[0]
+        p.run_list = up("run_list", run_list)
+        p.run_len = up("run_len", run_len)
+        p.run_table_off = up("run_table_off", run_table_off)
+        p.table_size = int(run_table_off[-1])
         self.problem = p
 
-        E, NC = g.num_entries, g.num_compute
-        self.compute = torch.empty(NC, dtype=torch.float64, device=self.device)
-        self.per_arg = torch.empty(NC, dtype=torch.float64, device=self.device)
-        self.comm = torch.empty(E, dtype=torch.float64, device=self.device)
-        self.cost = torch.empty(E, dtype=torch.float64, device=self.device)
-        self.flags = torch.empty(E, dtype=torch.uint8, device=self.device)
+        E, NC = g.num_slots, g.num_compute
+        # entry arrays hold num_slots elements; padding slots stay zero
+        self.compute = torch.zeros(NC, dtype=torch.float64, device=self.device)
+        self.per_arg = torch.zeros(NC, dtype=torch.float64, device=self.device)
+        self.comm = torch.zeros(E, dtype=torch.float64, device=self.device)
+        self.cost = torch.zeros(E, dtype=torch.float64, device=self.device)
+        self.flags = torch.zeros(E, dtype=torch.uint8, device=self.device)
         self.status = torch.zeros(1, dtype=torch.int32, device=self.device)
         tsize = int(self.lib.apc_pair_table_size(C.byref(p)))
         if use_table is None:
-            use_table = tsize <= _TABLE_MAX_DOUBLES and tsize <= max(_TABLE_MAX_RATIO * E, 1 << 16)
+            use_table = tsize <= _TABLE_MAX_DOUBLES and tsize <= max(_TABLE_MAX_RATIO * g.num_entries, 1 << 16)
         self.use_table = bool(use_table)
         self.table = (
             torch.empty(tsize, dtype=torch.float64, device=self.device) if self.use_table else None
@@ -173,11 +190,25 @@ class CostEngine:
             "apc_edge_costs",
         )
 
+    def prepare(self):
+        """Pair table and node compute vectors in one launch."""
+        _lib.check(
+            self.lib.apc_prepare(
+                C.byref(self.problem), self._ptr(self.table), self._ptr(self.compute),
+                self._ptr(self.per_arg), self._ptr(self.status), self._stream()),
+            "apc_prepare",
+        )
+
     def build(self, clamp_inf: bool = True):
-        """All coefficients: pair table, node compute vectors, entry arrays."""
-        self.build_pair_table()
-        self.node_compute()
-        self.edge_costs(clamp_inf)
+        """All coefficients: pair table and node compute vectors (one launch),
+        then the entry arrays (one launch)."""
+        _lib.check(
+            self.lib.apc_build_all(
+                C.byref(self.problem), self._ptr(self.table), self._ptr(self.compute),
+                self._ptr(self.per_arg), self._ptr(self.status), self._ptr(self.comm),
+                self._ptr(self.cost), self._ptr(self.flags), int(bool(clamp_inf)), self._stream()),
+            "apc_build_all",
+        )
         self.built = True
         return self
 
@@ -201,7 +232,7 @@ class CostEngine:
 
     def objective_coeffs(self) -> torch.Tensor:
         assert self.built
-        obj = torch.empty_like(self.cost)
+        obj = torch.zeros_like(self.cost)
         _lib.check(
             self.lib.apc_objective_coeffs(C.byref(self.problem), self._ptr(self.cost), self._ptr(obj), self._stream()),
             "apc_objective_coeffs",

@@ -25,11 +25,14 @@ autoparallel/cost_models/collective_runtime_estimation.py:157):
     0xC0 | id     any other placement class (is_shard/is_replicate/is_partial
                   all False, e.g. _StridedShard)
 
-Entry layout: edge e owns ``sdst[e] * ssrc[e]`` consecutive entries starting at
+Entry layout: edge e owns ``sdst[e] * ssrc[e]`` consecutive slots starting at
 ``edge_off[e]``, row-major ``[out_idx][inp_idx]``; edges are ordered by
-(node, argi).  That is the order of the reference's ``walk_over_options``
-(optimize_sharding.py:400-410); ``decision_var_order`` gives the permutation to
-the ``decision_vars`` dict order (node, out_idx, argi, inp_idx; :511-520).
+(node, argi), the order of the reference's ``walk_over_options``
+(optimize_sharding.py:400-410).  Every block starts on a multiple of 16 slots
+(aligned vector stores, exact 16-slot edge index), so the entry arrays have
+``num_slots >= num_entries`` elements; ``entry_slots()`` lists the real ones and
+``decision_var_order`` permutes them to the ``decision_vars`` dict order (node,
+out_idx, argi, inp_idx; :511-520).
 """
 from __future__ import annotations
 
@@ -44,7 +47,8 @@ TUPLE_BITS = 12
 MAX_TUPLES = 1 << TUPLE_BITS
 MAX_METAS = 1 << (32 - TUPLE_BITS)
 SPEC_NONE = 0xFFFFFFFF
-TILE_SHIFT = 10  # entries per tile of the entry->edge index = 1 << TILE_SHIFT
+CHUNK_SHIFT = 4  # edge blocks start on multiples of 1 << CHUNK_SHIFT slots
+ITEM_ENTRIES = 256  # entries of one edge per work item of the entry kernel
 
 
 def spec_word(meta_id: int, tuple_id: int) -> int:
@@ -142,10 +146,14 @@ class PackedGraph:
     # nodes
     node_nstrat: np.ndarray  # int32[N]
     node_nargs: np.ndarray  # int32[N]   len(strategies[0].input_specs)
-    node_comp_off: np.ndarray  # int64[N+1] prefix sum of node_nstrat
+    node_comp_off: np.ndarray  # int64[N] slot of (v, out 0) in the compute vector;
+    #                            nodes with identical program and input specs share one
+    n_compute: int  # length of the compute vector
+    comp_nodes: np.ndarray  # int32[...] one representative node per distinct slot
     node_edge_off: np.ndarray  # int32[N+1] edges of node v, ordered by argi
     node_op: np.ndarray  # int32[N]   OP_*
     node_prog_off: np.ndarray  # int64[N]   offset into prog (-1 if none)
+    node_prog_len: np.ndarray  # int32[N]   words of the node's program (0 if none)
     prog: np.ndarray  # int64[...] compute programs
     # explicit flops/bytes (OP_EXPLICIT), indexed like the compute vector
     explicit_flops: Optional[np.ndarray] = None  # int64[sum S]
@@ -158,7 +166,7 @@ class PackedGraph:
     edge_ssrc: np.ndarray = None  # int32[NE]
     edge_dst_list: np.ndarray = None  # int64[NE] offset into lists (sdst words)
     edge_src_list: np.ndarray = None  # int64[NE] offset into lists (ssrc words) or -1
-    edge_off: np.ndarray = None  # int64[NE+1]
+    edge_off: np.ndarray = None  # int64[NE+1] first slot of each block; [-1] = num_slots
     edge_flags: np.ndarray = None  # int32[NE]
     edge_default_off: np.ndarray = None  # int64[NE] offset into default_vals or -1
     default_vals: np.ndarray = None  # float64[...]
@@ -184,11 +192,25 @@ class PackedGraph:
 
     @property
     def num_entries(self) -> int:
+        """Real entries (decision variables)."""
+        return int((self.edge_sdst.astype(np.int64) * self.edge_ssrc).sum())
+
+    @property
+    def num_slots(self) -> int:
+        """Length of the entry arrays, padding included."""
         return int(self.edge_off[-1])
+
+    def entry_slots(self) -> np.ndarray:
+        """int64[E]: slot of every real entry, in (edge, out_idx, inp_idx) order."""
+        sizes = self.edge_sdst.astype(np.int64) * self.edge_ssrc
+        eid = np.repeat(np.arange(self.num_edges, dtype=np.int64), sizes)
+        start = np.concatenate([[0], np.cumsum(sizes)[:-1]])
+        local = np.arange(int(sizes.sum()), dtype=np.int64) - start[eid]
+        return self.edge_off[:-1][eid] + local
 
     @property
     def num_compute(self) -> int:
-        return int(self.node_comp_off[-1])
+        return int(self.n_compute)
 
     def entry_keys(self) -> np.ndarray:
         """int32[E, 4] keys (node_idx, argi, out_idx, inp_idx) in entry order
@@ -196,7 +218,8 @@ class PackedGraph:
         E = self.num_entries
         sizes = (self.edge_sdst.astype(np.int64) * self.edge_ssrc).astype(np.int64)
         eid = np.repeat(np.arange(self.num_edges, dtype=np.int64), sizes)
-        local = np.arange(E, dtype=np.int64) - self.edge_off[:-1][eid]
+        start = np.concatenate([[0], np.cumsum(sizes)[:-1]])
+        local = np.arange(E, dtype=np.int64) - start[eid]
         ssrc = self.edge_ssrc[eid].astype(np.int64)
         keys = np.empty((E, 4), dtype=np.int32)
         keys[:, 0] = self.edge_node[eid]
@@ -225,14 +248,22 @@ class PackedGraph:
             ("flags", "<i4"),
             ("node", "<i4"),
             ("src_node", "<i4"),
+            ("table_off", "<i8"),
+            ("magic", "<u4"),
+            ("local0", "<u4"),
         ]
     )
 
     def edge_records(self) -> np.ndarray:
-        """Edges as 48-byte records (the ``apc_edge`` struct of include/apc.h)."""
+        """Edges as 64-byte records (the ``apc_edge`` struct of include/apc.h)."""
         NE = self.num_edges
         rec = np.zeros(NE, self.EDGE_DTYPE)
-        assert rec.dtype.itemsize == 48
+        assert rec.dtype.itemsize == 64
+        rec["table_off"] = self.run_table()[3]
+        # division by ssrc as a multiply-high (exact while local * ssrc < 2**32)
+        ssrc = self.edge_ssrc.astype(np.int64)
+        ok = (ssrc > 1) & (ssrc * ssrc * self.edge_sdst < 2**32)
+        rec["magic"] = np.where(ok, (2**32) // np.maximum(ssrc, 1) + 1, 0).astype(np.uint32)
         rec["off"] = self.edge_off[:-1]
         rec["default_off"] = self.edge_default_off
         rec["src_list"] = np.where(self.edge_src_list >= 0, self.edge_src_list, 0).astype(np.uint32)
@@ -248,14 +279,52 @@ class PackedGraph:
         rec["src_node"] = self.edge_src_node
         return rec
 
-    def tile_edge_index(self) -> np.ndarray:
-        """int32[ceil(E / 2**TILE_SHIFT)]: the edge that owns the first entry
-        of each tile, so a kernel thread finds its edge with a short forward
-        walk instead of a binary search."""
-        E = self.num_entries
-        nt = (E + (1 << TILE_SHIFT) - 1) >> TILE_SHIFT
-        starts = np.arange(nt, dtype=np.int64) << TILE_SHIFT
+    @property
+    def max_node_args(self) -> int:
+        return int(np.diff(self.node_edge_off).max()) if self.num_nodes else 0
+
+    @property
+    def max_rank(self) -> int:
+        return int(self.meta_rank.max()) if self.meta_rank.shape[0] else 0
+
+    def run_table(self):
+        """Layout of the row table.  A *run* is a producer's list of output
+        specs (identified by its offset in ``lists``); its table holds, for
+        every placement tuple t, the row ``cost(run[j] -> t), j < S_src``, so an
+        output row of any edge fed by that run is one contiguous table row.
+        Returns (run_list int64[R], run_len int32[R], run_table_off int64[R+1],
+        edge_table_off int64[NE] (-1 without a producer))."""
+        hp = (self.edge_flags & EDGE_HAS_PRODUCER) != 0
+        nt = self.tuple_plc.shape[0]
+        edge_table_off = np.full(self.num_edges, -1, np.int64)
+        if not hp.any():
+            return (np.zeros(0, np.int64), np.zeros(0, np.int32), np.zeros(1, np.int64), edge_table_off)
+        offs, first, inv = np.unique(self.edge_src_list[hp], return_index=True, return_inverse=True)
+        run_len = self.edge_ssrc[hp][first].astype(np.int32)
+        assert (self.edge_ssrc[hp] == run_len[inv]).all(), "one run, two lengths"
+        run_table_off = np.zeros(offs.shape[0] + 1, np.int64)
+        np.cumsum(run_len.astype(np.int64) * nt, out=run_table_off[1:])
+        edge_table_off[hp] = run_table_off[:-1][inv]
+        return offs.astype(np.int64), run_len, run_table_off, edge_table_off
+
+    def chunk_edge_index(self) -> np.ndarray:
+        """int32[num_slots / 16]: the edge that owns each 16-slot chunk (blocks
+        are 16-slot aligned, so a chunk never spans two edges)."""
+        nt = self.num_slots >> CHUNK_SHIFT
+        starts = np.arange(nt, dtype=np.int64) << CHUNK_SHIFT
         return (np.searchsorted(self.edge_off, starts, side="right") - 1).astype(np.int32)
+
+    def work_items(self) -> np.ndarray:
+        """Work items of the entry kernel: for every 256 entries of every edge
+        block a copy of the edge record with ``local0`` set, in slot order."""
+        sizes = self.edge_sdst.astype(np.int64) * self.edge_ssrc
+        n = (sizes + ITEM_ENTRIES - 1) // ITEM_ENTRIES
+        eid = np.repeat(np.arange(self.num_edges, dtype=np.int64), n)
+        start = np.concatenate([[0], np.cumsum(n)[:-1]])
+        k = np.arange(int(n.sum()), dtype=np.int64) - start[eid]
+        items = self.edge_records()[eid]
+        items["local0"] = k * ITEM_ENTRIES
+        return items
 
     def validate(self) -> None:
         """Host-side shape checks run before any kernel launch: every index a
@@ -285,7 +354,16 @@ class PackedGraph:
             rank = self.meta_rank[wm][:, None]
             assert (~sh | (dims < rank)).all(), "Shard(dim) out of tensor rank"
         N, NE = self.num_nodes, self.num_edges
-        assert self.node_comp_off.shape == (N + 1,)
+        assert self.node_comp_off.shape == (N,)
+        if N:
+            assert (self.node_comp_off >= 0).all()
+            assert (self.node_comp_off + self.node_nstrat <= self.n_compute).all()
+            # every slot is written by exactly one evaluated node
+            covered = np.zeros(self.n_compute + 1, np.int64)
+            np.add.at(covered, self.node_comp_off[self.comp_nodes], 1)
+            np.add.at(covered, self.node_comp_off[self.comp_nodes] + self.node_nstrat[self.comp_nodes], -1)
+            assert (np.cumsum(covered)[:-1] == 1).all(), "compute slots not covered exactly once"
+            assert np.isin(self.node_comp_off, self.node_comp_off[self.comp_nodes]).all()
         assert self.node_edge_off.shape == (N + 1,)
         assert int(self.node_edge_off[-1]) == NE
         assert self.edge_off.shape == (NE + 1,)
@@ -293,7 +371,9 @@ class PackedGraph:
             assert (self.edge_sdst >= 1).all() and (self.edge_ssrc >= 1).all()
             assert (self.node_nargs >= 1).all(), "per-arg compute divides by num_args"
             sizes = self.edge_sdst.astype(np.int64) * self.edge_ssrc
-            assert (np.diff(self.edge_off) == sizes).all()
+            pad = (1 << CHUNK_SHIFT) - 1
+            assert (self.edge_off & pad == 0).all(), "edge blocks must be 16-slot aligned"
+            assert (np.diff(self.edge_off) == ((sizes + pad) & ~pad)).all()
             assert (self.edge_dst_list >= 0).all()
             assert (self.edge_dst_list + self.edge_sdst <= L).all()
             hp = (self.edge_flags & EDGE_HAS_PRODUCER) != 0
@@ -318,7 +398,37 @@ class PackedGraph:
                 none_csum[self.edge_src_list[hp] + self.edge_ssrc[hp]] - none_csum[self.edge_src_list[hp]]
             )
             assert (((nd_run == 0) & (ns_run == 0)) | d).all()
-        assert (np.diff(self.node_comp_off) == self.node_nstrat).all()
+        hasp = self.node_op == OP_PROGRAM
+        assert (self.node_prog_off[hasp] >= 0).all() and (self.node_prog_len[hasp] >= 2).all()
+        assert (self.node_prog_off[hasp] + self.node_prog_len[hasp] <= self.prog.shape[0]).all()
+        if (self.node_op == OP_EXPLICIT).any():
+            assert self.explicit_flops is not None and self.explicit_bytes is not None
+
+
+def check_program(prog: Sequence[int], n_args: int) -> None:
+    """Every (arg, dim) a compute program names must exist: the kernel indexes
+    the node's argument list and a MAX_RANK-wide shape row with them."""
+    p = 2
+    n_terms, n_outs = int(prog[0]), int(prog[1])
+    for _ in range(n_terms):
+        nfac = int(prog[p + 1])
+        p += 2
+        for _ in range(nfac):
+            assert 0 <= prog[p] < n_args and 0 <= prog[p + 1] < MAX_RANK, "program factor out of range"
+            p += 2
+    for _ in range(n_outs):
+        rank = int(prog[p + 1])
+        assert prog[p] >= 0 and 0 <= rank <= 64
+        p += 2
+        for _ in range(rank):
+            kind = int(prog[p])
+            assert kind in (DIM_CONST, DIM_ARG, DIM_BCAST)
+            if kind == DIM_ARG:
+                assert 0 <= prog[p + 1] < n_args and 0 <= prog[p + 2] < MAX_RANK, "program dim out of range"
+            elif kind == DIM_BCAST:
+                assert 0 <= prog[p + 1] < MAX_RANK
+            p += 3
+    assert p == len(prog), "program length mismatch"
 
 
 # ---------------------------------------------------------------------------
@@ -362,6 +472,7 @@ class GraphBuilder:
         self._tuples: Dict[Tuple[int, ...], int] = {}
         self._tuple_rows: List[Tuple[int, ...]] = []
         self.nodes: List[NodeDesc] = []
+        self.share_compute_slots = True
         self.prefetchable_edges: set = set()  # (node_idx, argi)
         self.multiplier: Dict[int, int] = {}
 
@@ -427,10 +538,26 @@ class GraphBuilder:
         node_nargs = np.zeros(N, np.int32)
         node_op = np.zeros(N, np.int32)
         node_prog_off = np.full(N, -1, np.int64)
+        node_prog_len = np.zeros(N, np.int32)
+        prog_cache: Dict[Tuple[int, ...], int] = {}
         node_edge_off = np.zeros(N + 1, np.int32)
         prog: List[int] = []
         # per node, per output index: offset of its run of output spec ids
         out_runs: List[Dict[int, int]] = []
+        run_cache: Dict[Tuple[int, ...], int] = {}
+
+        def add_run(words) -> int:
+            """Offset of a run of spec words; identical runs are stored once,
+            which also makes a producer's run offset the identity of its row
+            table."""
+            key = tuple(int(w) for w in words)
+            off = run_cache.get(key)
+            if off is None:
+                off = len(lists)
+                run_cache[key] = off
+                lists.extend(key)
+            return off
+
         e_node, e_arg, e_src, e_sdst, e_ssrc = [], [], [], [], []
         e_dst_list, e_src_list, e_flags, e_def = [], [], [], []
         defaults: List[float] = []
@@ -442,15 +569,21 @@ class GraphBuilder:
             node_nargs[v] = nd_.nargs if nd_.nargs is not None else len(nd_.in_specs[0])
             node_op[v] = nd_.op
             if nd_.program is not None:
-                node_prog_off[v] = len(prog)
-                prog.extend(int(x) for x in nd_.program)
+                key = tuple(int(x) for x in nd_.program)
+                check_program(key, len(nd_.in_specs[0]))
+                off = prog_cache.get(key)
+                if off is None:  # identical programs are stored once
+                    off = len(prog)
+                    prog_cache[key] = off
+                    prog.extend(key)
+                node_prog_off[v] = off
+                node_prog_len[v] = len(key)
             if nd_.op == OP_EXPLICIT:
                 any_explicit = True
             nout = len(nd_.out_specs[0])
             runs = {}
             for k in range(nout):
-                runs[k] = len(lists)
-                lists.extend(nd_.out_specs[o][k] for o in range(S))
+                runs[k] = add_run(nd_.out_specs[o][k] for o in range(S))
             out_runs.append(runs)
             # edges: one per row of redistribute_cost (== per arg)
             n_rows = len(nd_.in_specs[0])
@@ -462,10 +595,9 @@ class GraphBuilder:
                 e_node.append(v)
                 e_arg.append(a)
                 e_sdst.append(S)
-                e_dst_list.append(len(lists))
-                lists.extend(
+                e_dst_list.append(add_run(
                     (nd_.in_specs[o][a] if a < len(nd_.in_specs[o]) else -1) for o in range(S)
-                )
+                ))
                 flags = 0
                 if has_prod:
                     u = nd_.inputs[a]
@@ -518,9 +650,30 @@ class GraphBuilder:
         edge_sdst = np.asarray(e_sdst, np.int32)
         edge_ssrc = np.asarray(e_ssrc, np.int32)
         edge_off = np.zeros(NE + 1, np.int64)
-        np.cumsum(edge_sdst.astype(np.int64) * edge_ssrc, out=edge_off[1:])
-        node_comp_off = np.zeros(N + 1, np.int64)
-        np.cumsum(node_nstrat, out=node_comp_off[1:])
+        pad = (1 << CHUNK_SHIFT) - 1
+        np.cumsum((edge_sdst.astype(np.int64) * edge_ssrc + pad) & ~pad, out=edge_off[1:])
+        # compute slots: nodes with the same op class, program, arg count and
+        # input spec words produce the same estimate (the reference's memo key,
+        # compute_estimation.py:449-467) and share one slot
+        node_comp_off = np.zeros(N, np.int64)
+        slot_of: Dict[tuple, int] = {}
+        comp_nodes: List[int] = []
+        n_compute = 0
+        for v, nd_ in enumerate(self.nodes):
+            if nd_.op == OP_EXPLICIT or not self.share_compute_slots:
+                key = ("node", v)
+            elif nd_.op == OP_ZERO:
+                key = (OP_ZERO, len(nd_.in_specs), int(node_nargs[v]))
+            else:
+                key = (nd_.op, tuple(int(x) for x in nd_.program), int(node_nargs[v]),
+                       tuple(tuple(r) for r in nd_.in_specs))
+            off = slot_of.get(key)
+            if off is None:
+                off = n_compute
+                slot_of[key] = off
+                n_compute += len(nd_.in_specs)
+                comp_nodes.append(v)
+            node_comp_off[v] = off
         pref = np.zeros(NE, np.uint8)
         for i, (v, a) in enumerate(zip(e_node, e_arg)):
             if (v, a) in self.prefetchable_edges:
@@ -530,8 +683,8 @@ class GraphBuilder:
             mult[v] = m
         ef = eb = None
         if any_explicit:
-            ef = np.zeros(int(node_comp_off[-1]), np.int64)
-            eb = np.zeros(int(node_comp_off[-1]), np.int64)
+            ef = np.zeros(n_compute, np.int64)
+            eb = np.zeros(n_compute, np.int64)
             for v, nd_ in enumerate(self.nodes):
                 if nd_.op == OP_EXPLICIT:
                     o0 = int(node_comp_off[v])
@@ -550,9 +703,12 @@ class GraphBuilder:
             node_nstrat=node_nstrat,
             node_nargs=node_nargs,
             node_comp_off=node_comp_off,
+            n_compute=n_compute,
+            comp_nodes=np.asarray(comp_nodes, np.int32),
             node_edge_off=node_edge_off,
             node_op=node_op,
             node_prog_off=node_prog_off,
+            node_prog_len=node_prog_len,
             prog=np.asarray(prog, np.int64),
             explicit_flops=ef,
             explicit_bytes=eb,

@@ -1,0 +1,186 @@
+"""Benchmark of the sharding-search cost engine on one MI355X.
+
+A step is one build of every ILP coefficient of the workload graph, with the
+packed problem already resident in HBM: pair table, node compute vectors, and
+the entry kernel that writes comm / cost / flags for all E decision variables.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
+
+Prints one JSON line (see the keys below).  ``roofline`` is for the dominant
+kernel (edge_cost_kernel), timed with HIP events on the launch stream inside the
+timed steps; ``cpu_baseline`` is the per-entry Python oracle on this box's host.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published peak
+
+
+def workloads():
+    from autoparallel_amd import graphgen as G
+
+    return {
+        # BASELINE.json configs[1]: the configuration the metric is quoted on
+        "llama3_8b_fwd_bwd_mesh8x8": lambda: G.config_llama3_8b(),
+        # configs[0]
+        "gpt2_small_fwd_bwd_mesh8": lambda: G.config_gpt2_small(),
+        # configs[2] at reduced depth fits a quick run; full depth via --layers
+        "llama3_70b_fwd_bwd_mesh4x8x8": lambda: G.config_llama3_70b(),
+    }
+
+
+def read_traffic(workload):
+    """HBM bytes per launch of edge_cost_kernel from the committed rocprofv3
+    counter summary (profiles/edge_cost_kernel_<workload>_traffic.txt), if any."""
+    path = os.path.join(ROOT, "profiles", f"edge_cost_kernel_{workload}_traffic.txt")
+    if not os.path.exists(path):
+        return None
+    for line in open(path):
+        if line.startswith("traffic_bytes_per_launch="):
+            return float(line.split("=", 1)[1])
+    return None
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="llama3_8b_fwd_bwd_mesh8x8")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--direct", action="store_true", help="evaluate every entry directly (no pair table)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (the path needs no second one); use --gpus 1",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+
+    from autoparallel_amd.engine import CostEngine
+
+    t0 = time.perf_counter()
+    g = workloads()[args.workload]()
+    t_gen = time.perf_counter() - t0
+    E = g.num_entries
+
+    t0 = time.perf_counter()
+    eng = CostEngine(g, use_table=False if args.direct else None)
+    torch.cuda.synchronize()
+    t_upload = time.perf_counter() - t0
+
+    for _ in range(args.warmup):
+        eng.build()
+    torch.cuda.synchronize()
+
+    # HIP events on the launch stream (torch's current stream is the one the
+    # engine launches on) bracket the two launches of every timed step
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for k in range(args.steps):
+        ev[k][0].record()
+        eng.prepare()
+        ev[k][1].record()
+        eng.edge_costs(clamp_inf=True)
+        ev[k][2].record()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    eng.check_status()
+
+    t_prep = sum(e[0].elapsed_time(e[1]) for e in ev) / args.steps * 1e-3
+    t_edge = sum(e[1].elapsed_time(e[2]) for e in ev) / args.steps * 1e-3
+    ms_per_step = elapsed / args.steps * 1e3
+
+    # algorithmic bytes of one edge_cost_kernel launch: per entry one fp64 comm,
+    # one fp64 cost and one flag byte written (17 B); per edge its S_dst + S_src
+    # spec words (4 B each) and its 48-byte record read once
+    desc_bytes = int((g.edge_sdst.astype(np.int64) + g.edge_ssrc).sum()) * 4 + 48 * g.num_edges
+    algo_bytes = 17 * E + desc_bytes
+    achieved = algo_bytes / t_edge / 1e9
+
+    out = {
+        "metric": "cost entries/sec (all ILP coefficients of the graph built per step)",
+        "value": E / (elapsed / args.steps),
+        "unit": "entries/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f64",
+        "data": "synthetic",
+        "config": {
+            "workload": args.workload,
+            "mesh": [int(x) for x in g.mesh_shape],
+            "devices_per_host": g.devices_per_host,
+            "nodes": g.num_nodes,
+            "edges": g.num_edges,
+            "entries": E,
+            "strategies": g.num_compute,
+            "tensor_metas": int(g.meta_rank.shape[0]),
+            "placement_tuples": int(g.tuple_plc.shape[0]),
+            "pair_table": bool(eng.use_table),
+            "device": eng.device_name,
+        },
+        "coefficient_build_wall_s": elapsed / args.steps,
+        "kernel_s": {"prepare(pair_table+node_compute)": t_prep, "edge_cost": t_edge},
+        "host_s": {"graph_generation_and_pack": t_gen, "upload": t_upload},
+        "roofline": {
+            "kernel": "edge_cost_kernel",
+            "bound": "hbm",
+            "achieved": achieved,
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": achieved / HBM_PEAK_GBS,
+            "algorithmic_bytes_per_launch": algo_bytes,
+            "avg_launch_s": t_edge,
+            "traffic": read_traffic(args.workload),
+        },
+    }
+
+    if not args.no_cpu_baseline:
+        from oracle import cost_oracle as O
+
+        orc = O.GraphOracle(g)
+        orc.reset_caches()
+        # bounded sample: whole nodes in graph order until ~25 s of CPU time
+        budget = 25.0
+        done_entries = 0
+        t0 = time.perf_counter()
+        nodes_done = 0
+        chunk = max(1, g.num_nodes // 64)
+        arrays = None
+        while nodes_done < g.num_nodes and time.perf_counter() - t0 < budget:
+            hi = min(g.num_nodes, nodes_done + chunk)
+            arrays = orc.build(nodes=range(nodes_done, hi), out=arrays)
+            e_lo = int(g.node_edge_off[nodes_done])
+            e_hi = int(g.node_edge_off[hi])
+            done_entries += int((g.edge_sdst[e_lo:e_hi].astype(np.int64) * g.edge_ssrc[e_lo:e_hi]).sum())
+            nodes_done = hi
+        t_cpu = time.perf_counter() - t0
+        out["cpu_baseline"] = {
+            "value": done_entries / t_cpu,
+            "unit": "entries/s",
+            "cores": 1,
+            "host_cores_available": os.cpu_count(),
+            "kind": "port",
+            "sample": f"first {nodes_done} of {g.num_nodes} nodes in graph order "
+                      f"({done_entries} of {E} entries), memo caches cleared first",
+            "seconds": t_cpu,
+        }
+        out["speedup_vs_cpu_baseline"] = out["value"] / out["cpu_baseline"]["value"]
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -23,7 +23,8 @@ extern "C" {
 #define APC_MAX_RANK 8
 #define APC_TUPLE_BITS 12
 #define APC_SPEC_NONE 0xFFFFFFFFu
-#define APC_TILE_SHIFT 10
+#define APC_CHUNK_SHIFT 4    /* edge blocks start on multiples of 16 slots */
+#define APC_ITEM_ENTRIES 256 /* entries of one edge per work item (one wavefront) */
 #define APC_NUM_DTYPES 8
 
 /* edge flags */
@@ -44,9 +45,12 @@ extern "C" {
 #define APC_ERR_LAUNCH (-2)
 #define APC_ERR_UNSUPPORTED (-3)
 
-/* One (consumer node, argument) pair: an S_dst x S_src block of entries. */
+/* One (consumer node, argument) pair: an S_dst x S_src block of entries,
+ * row-major [out_idx][inp_idx], starting at slot `off` (a multiple of 16; the
+ * slots between one block's end and the next block's start are padding that
+ * no kernel reads or writes). */
 typedef struct apc_edge {
-  int64_t off;         /* index of entry (out_idx 0, inp_idx 0)                */
+  int64_t off;         /* slot of entry (out_idx 0, inp_idx 0)                 */
   int64_t default_off; /* into default_vals, or -1                             */
   uint32_t src_list;   /* into lists: S_src producer output spec words         */
   uint32_t dst_list;   /* into lists: S_dst consumer input spec words          */
@@ -55,8 +59,12 @@ typedef struct apc_edge {
   int32_t comp_base; /* index of (node, out_idx 0) in the compute vector     */
   int32_t flags;
   int32_t node;
-  int32_t src_node; /* producer node or -1                                   */
-} apc_edge;
+  int32_t src_node;  /* producer node or -1                                   */
+  int64_t table_off; /* row table of the producer's run, or -1                */
+  uint32_t magic;    /* floor(2^32 / ssrc) + 1 if ssrc > 1 and ssrc * ssrc * sdst
+                        < 2^32 (then local / ssrc == umulhi(local, magic)), else 0 */
+  uint32_t local0;   /* 0 in the edge table; in a work item, its first entry  */
+} apc_edge; /* 64 bytes */
 
 /* Cost-model constants (host values, passed by value into the kernels). */
 typedef struct apc_model {
@@ -89,9 +97,17 @@ typedef struct apc_problem {
   const int32_t* node_nstrat;
   const int32_t* node_nargs;
   const int32_t* node_op;
-  const int64_t* node_comp_off; /* [n_node+1] */
+  const int64_t* node_comp_off; /* [n_node] slot of (v, out_idx 0) in the compute
+                                   vector; nodes with identical program and
+                                   input specs may share a slot */
   const int32_t* node_edge_off; /* [n_node+1] */
   const int64_t* node_prog_off; /* -1 = none */
+  const int32_t* node_prog_len; /* words of the node's program, 0 = none */
+  int32_t max_node_args;        /* max over nodes of edges per node */
+  int32_t max_rank;             /* max tensor rank over all metas */
+  int64_t n_compute;            /* length of the compute / per_arg vectors */
+  int32_t n_comp_node;          /* nodes to evaluate: one per distinct slot */
+  const int32_t* comp_nodes;    /* [n_comp_node] */
   const int32_t* node_multiplier;
   int64_t n_prog;
   const int64_t* prog;
@@ -100,11 +116,23 @@ typedef struct apc_problem {
   /* edges */
   int32_t n_edge;
   const apc_edge* edges;
-  int64_t n_entry;
-  int32_t n_tile;
-  const int32_t* tile_edge; /* [n_tile] edge owning entry tile << APC_TILE_SHIFT */
+  int64_t n_entry;           /* real entries: sum of sdst * ssrc               */
+  int64_t n_slot;            /* length of the entry arrays (with padding)      */
+  int64_t n_chunk;           /* n_slot / 16                                    */
+  const int32_t* chunk_edge; /* [n_chunk] edge owning slots [16c, 16c + 16)    */
+  /* work items of the entry kernel: for every 256 entries of every edge block a
+   * copy of the edge record with local0 = first entry of the item, slot order */
+  int32_t n_item;
+  const apc_edge* items;     /* [n_item] */
   int64_t n_default;
   const double* default_vals;
+  /* row tables: run r is the S_src spec words at lists[run_list[r]]; its table
+   * is table[run_table_off[r] + t * run_len[r] + j] = cost(run[j] -> tuple t) */
+  int32_t n_run;
+  const int64_t* run_list;
+  const int32_t* run_len;
+  const int64_t* run_table_off; /* [n_run+1] */
+  int64_t table_size;           /* doubles: run_table_off[n_run] */
 } apc_problem;
 
 int apc_version(void);
@@ -124,8 +152,8 @@ int apc_mesh_topology(const int32_t* mesh_shape, int32_t ndim, int32_t devices_p
  * ValueError there). */
 int apc_device_limits(const char* device_name, apc_model* model);
 
-/* Number of doubles of the pair table apc_build_pair_table fills:
- * n_meta * n_tuple * n_tuple. */
+/* Number of doubles of the row table apc_build_pair_table fills
+ * (= p->table_size: sum over runs of run_len * n_tuple). */
 int64_t apc_pair_table_size(const apc_problem* p);
 
 /* Replaces estimate_strategy_comms_cost + redistribute_cost + collective_comm_cost
@@ -133,15 +161,16 @@ int64_t apc_pair_table_size(const apc_problem* p);
  * 115-229, 239-262), torch's allgather/allreduce/reduce_scatter_cost
  * (torch:distributed/tensor/_collective_utils.py:281-313) and
  * compute_read_write_time (autoparallel/cost_models/compute_estimation.py:391-403),
- * evaluated for every (tensor meta, source placements, target placements)
- * triple: table[(m * n_tuple + src) * n_tuple + tgt], microseconds, +inf for
- * forbidden transitions. */
+ * evaluated for every (producer output spec, target placements) pair that the
+ * entry kernel can ask for: table[run_table_off[r] + tgt * run_len[r] + j],
+ * microseconds, +inf for forbidden transitions. */
 int apc_build_pair_table(const apc_problem* p, double* table, void* stream);
 
 /* Replaces estimate_strategy_runtime_cost
  * (autoparallel/cost_models/compute_estimation.py:438-493, with
  * _get_sharded_shape_stride :300-318 and compute_memory_cost :321-331) for
- * every (node, out_idx): compute[node_comp_off[v] + o] in microseconds, and
+ * every (node, out_idx) of the nodes in comp_nodes: compute[node_comp_off[v] + o]
+ * in microseconds, and
  * per_arg = compute / num_args (autoparallel/optimize_sharding.py:516).
  * status (device int32[1], zeroed by the caller) is set non-zero if a node
  * with flops has an input dtype without a tflops entry (ValueError in the
@@ -161,6 +190,24 @@ int apc_node_compute_costs(const apc_problem* p, double* compute, double* per_ar
  * be NULL to skip that output. */
 int apc_edge_costs(const apc_problem* p, const double* table, const double* per_arg,
                    double* comm, double* cost, uint8_t* flags, int32_t clamp_inf, void* stream);
+
+/* apc_build_pair_table (skipped if table is NULL) and apc_node_compute_costs in
+ * one launch: the two are independent of each other. */
+int apc_prepare(const apc_problem* p, double* table, double* compute, double* per_arg,
+                int32_t* status, void* stream);
+
+/* The three steps above in two launches (pair table and node estimates share
+ * one): the whole of ShardingOptimizer._build_decision_vars' arithmetic
+ * (autoparallel/optimize_sharding.py:481-552) in one call.  table may be NULL
+ * (direct evaluation). */
+int apc_build_all(const apc_problem* p, double* table, double* compute, double* per_arg,
+                  int32_t* status, double* comm, double* cost, uint8_t* flags, int32_t clamp_inf,
+                  void* stream);
+
+/* Measurement aid, no counterpart in the reference: a plain device copy of
+ * nbytes (multiple of 16) whose HBM traffic is known (nbytes read + nbytes
+ * written), used to scale hardware traffic counters in profiles. */
+int apc_calibration_copy(const void* src, void* dst, int64_t nbytes, void* stream);
 
 /* Replaces apply_prefetch_discount (autoparallel/optimize_sharding.py:824-875)
  * on the entry arrays, for edges flagged APC_EDGE_PREFETCHABLE: comm *= scale

@@ -444,16 +444,21 @@ class GraphOracle:
         return k
 
     # -- the build -----------------------------------------------------------
-    def build(self, nodes: Optional[Sequence[int]] = None):
+    def build(self, nodes: Optional[Sequence[int]] = None, out: Optional[dict] = None):
         """Returns dict of numpy arrays in entry order:
-        comm f64[E], transition u8[E], cost f64[E] (before the inf clamp),
-        compute f64[sum S] (the per-strategy estimate, not divided)."""
+        comm f64[slots], transition u8[slots], cost f64[slots] (before the inf clamp),
+        compute f64[sum S] (the per-strategy estimate, not divided).
+        ``nodes`` restricts the build to some nodes; ``out`` reuses arrays."""
         g = self.g
-        E = g.num_entries
-        comm = np.zeros(E, np.float64)
-        trans = np.zeros(E, np.uint8)
-        cost = np.zeros(E, np.float64)
-        compute = np.zeros(g.num_compute, np.float64)
+        E = g.num_slots  # entry arrays are indexed by slot; padding stays zero
+        if out is None:
+            out = {
+                "comm": np.zeros(E, np.float64),
+                "transition": np.zeros(E, np.uint8),
+                "cost": np.zeros(E, np.float64),
+                "compute": np.zeros(g.num_compute, np.float64),
+            }
+        comm, trans, cost, compute = out["comm"], out["transition"], out["cost"], out["compute"]
         lists = self._lists
         tuple_plc = self._tuple_plc
         node_range = range(g.num_nodes) if nodes is None else nodes
@@ -485,7 +490,7 @@ class GraphOracle:
                         comm[base + j] = c
                         trans[base + j] = t
                         cost[base + j] = c + per_arg + t
-        return {"comm": comm, "transition": trans, "cost": cost, "compute": compute}
+        return out
 
 
 def clamp_inf(cost: np.ndarray) -> Tuple[np.ndarray, np.ndarray]:
