@@ -54,7 +54,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="llama3_8b_fwd_bwd_mesh8x8")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--direct", action="store_true", help="evaluate every entry directly (no pair table)")
+    ap.add_argument("--direct", action="store_true", help="evaluate every entry directly (no row table)")
+    ap.add_argument("--calibration-copy-mib", type=int, default=0,
+                    help="after the timed steps, also launch the plain copy kernel on this many MiB "
+                         "(the known-traffic reference for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (the path needs no second one); use --gpus 1",
@@ -95,14 +98,25 @@ def main():
     elapsed = time.perf_counter() - t0
     eng.check_status()
 
+    if args.calibration_copy_mib > 0:
+        import ctypes as C
+
+        nbytes = args.calibration_copy_mib << 20
+        a = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+        b = torch.empty_like(a)
+        for _ in range(5):
+            eng.lib.apc_calibration_copy(C.c_void_p(a.data_ptr()), C.c_void_p(b.data_ptr()), nbytes, eng._stream())
+        torch.cuda.synchronize()
+
     t_prep = sum(e[0].elapsed_time(e[1]) for e in ev) / args.steps * 1e-3
     t_edge = sum(e[1].elapsed_time(e[2]) for e in ev) / args.steps * 1e-3
     ms_per_step = elapsed / args.steps * 1e3
 
     # algorithmic bytes of one edge_cost_kernel launch: per entry one fp64 comm,
     # one fp64 cost and one flag byte written (17 B); per edge its S_dst + S_src
-    # spec words (4 B each) and its 48-byte record read once
-    desc_bytes = int((g.edge_sdst.astype(np.int64) + g.edge_ssrc).sum()) * 4 + 48 * g.num_edges
+    # spec words (4 B each) and its 64-byte record read once.  Table rows and
+    # per-arg terms are re-read from cache and not counted.
+    desc_bytes = int((g.edge_sdst.astype(np.int64) + g.edge_ssrc).sum()) * 4 + 64 * g.num_edges
     algo_bytes = 17 * E + desc_bytes
     achieved = algo_bytes / t_edge / 1e9
 
@@ -126,10 +140,13 @@ def main():
             "nodes": g.num_nodes,
             "edges": g.num_edges,
             "entries": E,
-            "strategies": g.num_compute,
+            "strategies": int(g.node_nstrat.sum()),
             "tensor_metas": int(g.meta_rank.shape[0]),
             "placement_tuples": int(g.tuple_plc.shape[0]),
-            "pair_table": bool(eng.use_table),
+            "row_table": bool(eng.use_table),
+            "row_table_doubles": int(eng.table.numel()) if eng.table is not None else 0,
+            "compute_slots": g.num_compute,
+            "evaluated_nodes": int(g.comp_nodes.shape[0]),
             "device": eng.device_name,
         },
         "coefficient_build_wall_s": elapsed / args.steps,

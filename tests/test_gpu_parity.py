@@ -1,0 +1,358 @@
+"""Parity of the HIP path (through the C ABI) against the CPU oracle and the
+golden vectors written by the reference's own cost functions.
+
+Bar: bit-exact for every fp64 cost entry and every flag (the north-star
+tolerance is 1e-9 relative; the kernels restate the same binary64 operations
+in the same order, so equality of bit patterns is what is asserted)."""
+import json
+
+import numpy as np
+import pytest
+import torch
+
+from autoparallel_amd import graphgen, opprog, packed
+from autoparallel_amd.packed import GraphBuilder, NodeDesc
+from helpers import bits_equal, first_mismatch, graph_from_pairs
+from oracle import cost_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def CostEngine():
+    if not torch.cuda.is_available():
+        pytest.skip("needs a GPU")
+    from autoparallel_amd.engine import CostEngine as CE
+
+    return CE
+
+
+def _check_build(CE, g, use_table, clamp=False):
+    print(f"  build: E={g.num_entries} table={use_table}", flush=True)
+    eng = CE(g, use_table=use_table).build(clamp_inf=clamp)
+    got = eng.results()
+    ref = O.GraphOracle(g).build()
+    want_cost = O.clamp_inf(ref["cost"])[0] if clamp else ref["cost"]
+    assert bits_equal(got["compute"], ref["compute"]), first_mismatch(got["compute"], ref["compute"])
+    assert bits_equal(got["comm"], ref["comm"]), first_mismatch(got["comm"], ref["comm"])
+    assert bits_equal(got["cost"], want_cost), first_mismatch(got["cost"], want_cost)
+    assert ((got["flags"] & 1) == ref["transition"]).all()
+    assert (((got["flags"] >> 1) & 1) == ~np.isfinite(ref["cost"])).all()
+    return eng, got, ref
+
+
+# ---------------------------------------------------------------------------
+# golden vectors of the reference, through the C ABI
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("use_table", [True, False])
+def test_golden_comm_vectors(CostEngine, golden, use_table):
+    n_cases = int(golden["comm_ncases"][0])
+    checked = 0
+    for k in range(n_cases):
+        mesh = [int(x) for x in golden[f"comm_{k}_mesh"]]
+        shape = [int(x) for x in golden[f"comm_{k}_shape"]]
+        stride = [int(x) for x in golden[f"comm_{k}_stride"]]
+        itemsize = int(golden[f"comm_{k}_itemsize"][0])
+        src, tgt, want = golden[f"comm_{k}_src"], golden[f"comm_{k}_tgt"], golden[f"comm_{k}_cost"]
+        src_t = sorted({tuple(int(x) for x in r) for r in src})
+        tgt_t = sorted({tuple(int(x) for x in r) for r in tgt})
+        g = graph_from_pairs(mesh, 8, shape, stride, itemsize, src_t, tgt_t)
+        print(f"golden case {k}: mesh={mesh} shape={shape} pairs={len(want)}", flush=True)
+        eng = CostEngine(g, use_table=use_table).build(clamp_inf=False)
+        comm = eng.results()["comm"]
+        e = 1  # the consumer's edge
+        base, ssrc = int(g.edge_off[e]), int(g.edge_ssrc[e])
+        si = {t: i for i, t in enumerate(src_t)}
+        ti = {t: i for i, t in enumerate(tgt_t)}
+        idx = np.asarray([base + ti[tuple(int(x) for x in t)] * ssrc + si[tuple(int(x) for x in s)]
+                          for s, t in zip(src, tgt)])
+        assert bits_equal(comm[idx], want), (k, first_mismatch(comm[idx], want))
+        checked += len(want)
+    assert checked > 20000
+
+
+def test_golden_runtime_vectors(CostEngine, golden):
+    """estimate_strategy_runtime_cost of the reference on hand-built fx nodes."""
+    d = json.loads(bytes(golden["rt_json"]).decode())
+    DT = {"torch.float64": (0, 8), "torch.float32": (1, 4), "torch.float16": (2, 2),
+          "torch.bfloat16": (3, 2), "torch.int8": (4, 1), "torch.int64": (5, 8)}
+    progs = {
+        "mm": lambda s, i: opprog.mm(i), "mm_f32": lambda s, i: opprog.mm(i),
+        "bmm": lambda s, i: opprog.bmm(i), "addmm": lambda s, i: opprog.addmm(i),
+        "add": lambda s, i: opprog.pointwise(len(s[0]), i),
+        "mul_bcast": lambda s, i: opprog.pointwise(len(s[0]), i),
+        "small_add": lambda s, i: opprog.pointwise(len(s[0]), i),
+        "silu": lambda s, i: opprog.pointwise(len(s[0]), i),
+        "sum_dim": lambda s, i: opprog.reduction(len(s[0]), [2], True, i),
+        "mean_dim": lambda s, i: opprog.reduction(len(s[0]), [-1], True, i),
+        "einsum_fwd": lambda s, i: opprog.einsum_fwd(len(s[0]), i),
+        "einsum_bwd": lambda s, i: opprog.einsum_bwd(len(s[0]), i),
+        "softmax": lambda s, i: opprog.same_as_arg(0, len(s[0]), i),
+        "embedding": lambda s, i: opprog.embedding(len(s[1]), i),
+        "sdpa_flash": lambda s, i: opprog.sdpa_flash_fwd(i),
+        "view": lambda s, i: None,
+    }
+    b = GraphBuilder(d["mesh"], 8)
+    want = []
+    # group the cases of one op into one node (one strategy per case)
+    by_op = {}
+    for i, name in enumerate(d["names"]):
+        by_op.setdefault(name, []).append(i)
+    for name, idxs in by_op.items():
+        shapes, dtypes = d["shapes"][idxs[0]], d["dtypes"][idxs[0]]
+        metas = []
+        for shape, dt in zip(shapes, dtypes):
+            stride = list(torch.empty(shape, device="meta").stride())
+            metas.append(b.meta(shape, stride, DT[dt][1], DT[dt][0]))
+        # producers: one placeholder-like node per argument, with the strategies' specs
+        prods = []
+        for a, m in enumerate(metas):
+            specs = [b.spec(m, d["placements"][i][a]) for i in idxs]
+            uniq = list(dict.fromkeys(specs))
+            prods.append(b.add_node(NodeDesc(f"{name}_arg{a}", in_specs=[[s] for s in uniq],
+                                             out_specs=[[s] for s in uniq], inputs=[],
+                                             default_rows=[[[0.0]] for _ in uniq])))
+        in_specs = [[b.spec(m, d["placements"][i][a]) for a, m in enumerate(metas)] for i in idxs]
+        prog = progs[name](shapes, DT[dtypes[0]][1])
+        b.add_node(NodeDesc(name, in_specs=in_specs, out_specs=[[r[0]] for r in in_specs], inputs=prods,
+                            op=packed.OP_PROGRAM if prog is not None else packed.OP_ZERO, program=prog))
+        want.append((len(b.nodes) - 1, [float.fromhex(d["cost_hex"][i]) for i in idxs]))
+    b.share_compute_slots = False
+    g = b.pack()
+    eng = CostEngine(g).build(clamp_inf=False)
+    compute = eng.results()["compute"]
+    for v, vals in want:
+        off = int(g.node_comp_off[v])
+        got = compute[off:off + len(vals)]
+        assert bits_equal(got, np.asarray(vals)), (g.node_names[v], got, vals)
+
+
+# ---------------------------------------------------------------------------
+# whole graphs against the oracle
+# ---------------------------------------------------------------------------
+GRAPHS = {
+    "llama_2d": lambda: graphgen.llama_graph((8, 8), 1, 1024, 8, 4, 2048, 8192, 512, 16),
+    "llama_2d_real_dims": lambda: graphgen.llama_graph((8, 8), 1, 4096, 32, 8, 14336, 128256, 8192, 64),
+    "gpt2_1d": lambda: graphgen.gpt2_graph((8,), n_layers=2),
+    "llama_3d": lambda: graphgen.llama_graph((2, 4, 2), 1, 512, 8, 4, 1024, 4096, 256, 16),
+    "llama_odd_mesh": lambda: graphgen.llama_graph((3, 5), 1, 960, 15, 5, 1920, 3000, 240, 30),
+    "pairs_4d": lambda: _pairs_graph((2, 3, 2, 4), (48, 36, 40), 300),
+    "pairs_3d_noncontig": lambda: _pairs_graph((4, 8, 8), (256, 8192, 64), 250, stride=(64, 16384, 1)),
+}
+
+
+def _pairs_graph(mesh, shape, n, stride=None, seed=3):
+    """One edge whose rows/columns are random placement tuples over
+    {R, S(d), P(sum), P(avg)} on a mesh of any rank."""
+    rng = np.random.default_rng(seed)
+    opts = [0x00] + [0x40 | d for d in range(len(shape))] + [0x80, 0x81]
+    draw = lambda: sorted({tuple(int(x) for x in rng.choice(opts, size=len(mesh))) for _ in range(n)})
+    if stride is None:
+        stride = graphgen.contiguous_stride(shape)
+    return graph_from_pairs(mesh, 8, shape, stride, 2, draw(), draw(), dtype=packed.DT_BF16)
+
+
+# every graph through the table path; direct evaluation on the smaller ones
+CASES = [(n, True) for n in GRAPHS] + [
+    (n, False) for n in ("llama_2d", "gpt2_1d", "llama_odd_mesh", "pairs_4d", "pairs_3d_noncontig")
+]
+
+
+@pytest.mark.parametrize("name,use_table", CASES)
+def test_graph_parity(CostEngine, name, use_table):
+    g = GRAPHS[name]()
+    print(f"graph {name}", flush=True)
+    _check_build(CostEngine, g, use_table)
+
+
+def test_clamp_inf(CostEngine):
+    _check_build(CostEngine, GRAPHS["llama_2d"](), True, clamp=True)
+
+
+def test_deterministic(CostEngine):
+    g = GRAPHS["llama_2d"]()
+    a = CostEngine(g).build().results()
+    b = CostEngine(g).build().build().results()
+    for k in ("comm", "cost", "compute"):
+        assert bits_equal(a[k], b[k])
+    assert (a["flags"] == b["flags"]).all()
+
+
+def test_prefetch_discount(CostEngine):
+    g = GRAPHS["llama_2d"]()
+    for scale in (0.0, 0.25):
+        eng, got, ref = _check_build(CostEngine, g, True, clamp=True)
+        n = eng.apply_prefetch_discount(scale)
+        cost0, _ = O.clamp_inf(ref["cost"])
+        comm2, cost2, n2 = O.prefetch_discount(g, ref["comm"], ref["transition"], ref["compute"], cost0, scale)
+        got2 = eng.results()
+        assert n == n2 > 0
+        assert bits_equal(got2["comm"], comm2) and bits_equal(got2["cost"], cost2)
+
+
+def test_objective_coeffs(CostEngine):
+    g = GRAPHS["gpt2_1d"]()
+    g.node_multiplier = (np.arange(g.num_nodes) % 3 + 1).astype(np.int32)
+    eng, got, ref = _check_build(CostEngine, g, True, clamp=True)
+    obj = eng.objective_coeffs().cpu().numpy()
+    slots, keys = g.entry_slots(), g.entry_keys()
+    want = got["cost"][slots] * g.node_multiplier[keys[:, 0]]
+    assert bits_equal(obj[slots], want)
+
+
+def test_scoring(CostEngine):
+    g = GRAPHS["llama_2d"]()
+    eng, got, ref = _check_build(CostEngine, g, True, clamp=True)
+    rng = np.random.default_rng(1)
+    A = 37
+    assign = np.stack([rng.integers(0, g.node_nstrat) for _ in range(A)], axis=1).astype(np.int16)
+    assign[:, 0] = 0
+    out = eng.score(torch.from_numpy(np.ascontiguousarray(assign)).cuda()).cpu().numpy()
+    cost, bad = O.clamp_inf(ref["cost"])
+    for a in range(A):
+        want = O.score_assignment(g, ref["comm"], ref["transition"], ref["compute"], assign[:, a])
+        obj, viol = O.ilp_objective(g, cost, bad, assign[:, a])
+        assert tuple(out[a, :4]) == tuple(float(x) for x in want), (a, out[a], want)
+        assert out[a, 4] == obj and out[a, 5] == viol
+    # on-device generated assignments: same draw on the host
+    out = eng.score_random(seed=11, first=5, count=9).cpu().numpy()
+    for i in range(9):
+        asg = eng.random_assignment(11, 5 + i)
+        assert (asg < g.node_nstrat).all()
+        want = O.score_assignment(g, ref["comm"], ref["transition"], ref["compute"], asg)
+        assert tuple(out[i, :4]) == tuple(float(x) for x in want)
+
+
+# ---------------------------------------------------------------------------
+# edge cases
+# ---------------------------------------------------------------------------
+def _edge_case_graph():
+    """Missing specs with default rows, a tuple-valued producer consumed
+    directly and through getitem, an explicit-flops node, a node with more than
+    8 arguments, strategies > 64, single-entry blocks."""
+    b = GraphBuilder((2, 4), 8)
+    m = b.meta((64, 48), (48, 1), 2, packed.DT_BF16)
+    mt = b.meta((64, 48), (1, 64), 2, packed.DT_BF16)
+    opts = O.create_all_options((64, 48), (2, 4))
+    specs = [b.spec(m, o) for o in opts]
+    ph = b.add_node(NodeDesc("x", in_specs=[[s] for s in specs], out_specs=[[s] for s in specs],
+                             inputs=[], default_rows=[[[0.0]] for _ in specs]))
+    one = b.add_node(NodeDesc("scalar", in_specs=[[specs[0]]], out_specs=[[specs[0]]], inputs=[],
+                              default_rows=[[[0.0]]]))
+    # tuple producer: two outputs, second one None in some strategies
+    tup_out = [[s, (b.spec(mt, o) if i % 3 else -1)] for i, (s, o) in enumerate(zip(specs, opts))]
+    tup = b.add_node(NodeDesc("tuple_op", in_specs=[[s] for s in specs], out_specs=tup_out, inputs=[ph],
+                              op=packed.OP_PROGRAM, program=opprog.same_as_arg(0, 2, 2, n_out=2),
+                              tuple_output=True))
+    uniq1 = list(dict.fromkeys(o[1] for o in tup_out))
+    gi = b.add_node(NodeDesc("getitem1", in_specs=[[s] for s in uniq1], out_specs=[[s] for s in uniq1],
+                             inputs=[tup], getitem_index=1,
+                             default_rows=[[[float(i + j) for j in range(len(specs))]] for i in range(len(uniq1))]))
+    direct = b.add_node(NodeDesc("uses_tuple", in_specs=[[specs[0]], [specs[1]]], out_specs=[[specs[0]], [specs[1]]],
+                                 inputs=[tup],
+                                 default_rows=[[[1.5] * len(specs)], [[2.5] * len(specs)]]))
+    # explicit flops/bytes, with a None input spec (non-tensor arg)
+    b.add_node(NodeDesc("explicit", in_specs=[[specs[0], -1], [specs[2], -1]], out_specs=[[specs[0]], [specs[2]]],
+                        inputs=[ph, one], op=packed.OP_EXPLICIT, flops=[10**12, 0], nbytes=[10**9, 10**3],
+                        default_rows=[[[0.0] * len(specs), [7.0]], [[0.0] * len(specs), [8.0]]]))
+    # 10 arguments: beyond the staged fast path of the node kernel
+    b.add_node(NodeDesc("many_args", in_specs=[[s] * 10 for s in specs[:5]], out_specs=[[s] for s in specs[:5]],
+                        inputs=[ph] * 10, op=packed.OP_PROGRAM, program=opprog.pointwise(2, 2)))
+    # > 64 strategies on both sides
+    big = [specs[i % len(specs)] for i in range(150)]
+    pb = b.add_node(NodeDesc("big_prod", in_specs=[[s] for s in big], out_specs=[[s] for s in big], inputs=[ph],
+                             op=packed.OP_PROGRAM, program=opprog.pointwise(2, 2)))
+    b.add_node(NodeDesc("big_cons", in_specs=[[s, s] for s in big[:131]], out_specs=[[s] for s in big[:131]],
+                        inputs=[pb, pb], op=packed.OP_PROGRAM, program=opprog.mm(2)))
+    return b.pack()
+
+
+@pytest.mark.parametrize("use_table", [True, False])
+def test_edge_cases(CostEngine, use_table):
+    g = _edge_case_graph()
+    eng, got, ref = _check_build(CostEngine, g, use_table)
+    # the default rows really were used
+    e = [i for i in range(g.num_edges) if g.node_names[g.edge_node[i]] == "uses_tuple"][0]
+    b0 = int(g.edge_off[e])
+    assert got["comm"][b0] == 1.5
+
+
+def test_unsupported_dtype_reports(CostEngine):
+    b = GraphBuilder((2,), 8)
+    m = b.meta((8, 8), (8, 1), 8, packed.DT_OTHER)
+    s = b.spec(m, (0,))
+    ph = b.add_node(NodeDesc("x", in_specs=[[s]], out_specs=[[s]], inputs=[], default_rows=[[[0.0]]]))
+    b.add_node(NodeDesc("mm_i64", in_specs=[[s, s]], out_specs=[[s]], inputs=[ph, ph],
+                        op=packed.OP_PROGRAM, program=opprog.mm(8)))
+    eng = CostEngine(b.pack()).build()
+    with pytest.raises(ValueError):
+        eng.results()
+
+
+def test_enumerate_input_options(CostEngine):
+    import ctypes as C
+
+    from autoparallel_amd import _lib
+    from autoparallel_amd.engine import make_model
+
+    lib = _lib.load()
+    mesh = (4, 8, 8)
+    shapes = [(256, 8192, 8192), (10, 3, 1000), (7,), (64, 32, 8192, 128), (), (4, 4)]
+    model = make_model(mesh, 8, "AMD Instinct MI355X")
+    rank = np.asarray([len(s) for s in shapes], np.int32)
+    shp = np.ones((len(shapes), 8), np.int64)
+    for i, s in enumerate(shapes):
+        shp[i, :len(s)] = s
+    ncand = (rank.astype(np.int64) + 1) ** len(mesh)
+    off = np.zeros(len(shapes) + 1, np.int64)
+    np.cumsum(ncand, out=off[1:])
+    d = lambda a: torch.from_numpy(a).cuda()
+    t_rank, t_shape, t_off = d(rank), d(shp), d(off)
+    valid = torch.zeros(int(off[-1]), dtype=torch.uint8, device="cuda")
+    plc = torch.zeros(int(off[-1]) * 4, dtype=torch.uint8, device="cuda")
+    rc = lib.apc_enumerate_input_options(C.byref(model), len(shapes), t_rank.data_ptr(), t_shape.data_ptr(),
+                                         t_off.data_ptr(), valid.data_ptr(), plc.data_ptr(), None)
+    assert rc == 0
+    torch.cuda.synchronize()
+    valid, plc = valid.cpu().numpy(), plc.cpu().numpy().reshape(-1, 4)
+    for i, s in enumerate(shapes):
+        got = [tuple(int(x) for x in plc[j, :3]) for j in range(off[i], off[i + 1]) if valid[j]]
+        assert got == O.create_all_options(s, mesh), s
+
+
+# ---------------------------------------------------------------------------
+# full benchmark size: properties that need no oracle pass over every entry
+# ---------------------------------------------------------------------------
+def test_full_size_properties(CostEngine):
+    g = graphgen.config_llama3_8b()
+    print(f"full size: E={g.num_entries}", flush=True)
+    eng = CostEngine(g, use_table=True).build(clamp_inf=False)
+    a = eng.results()
+    d = CostEngine(g, use_table=False).build(clamp_inf=False).results()
+    # table path and direct evaluation are the same function
+    for k in ("comm", "cost", "compute"):
+        assert bits_equal(a[k], d[k])
+    assert (a["flags"] == d["flags"]).all()
+    slots, keys = g.entry_slots(), g.entry_keys()
+    comm, cost, fl = a["comm"][slots], a["cost"][slots], a["flags"][slots]
+    pa = a["per_arg"][g.node_comp_off[keys[:, 0]] + keys[:, 2]]
+    fin = np.isfinite(comm)
+    # cost = (comm + per_arg) + transition, everywhere
+    assert (cost[fin] == (comm[fin] + pa[fin]) + (fl[fin] & 1)).all()
+    assert np.isinf(cost[~fin]).all() and ((fl[~fin] >> 1) == 1).all()
+    # no transition => no communication
+    assert (comm[(fl & 1) == 0] == 0.0).all()
+    assert (comm >= 0).all()
+    # the 32 identical layers have identical blocks: layer 3 vs layer 17
+    per_layer = (g.num_nodes - 0) // 32
+    # oracle on a sample of nodes (seconds), incl. first, last and middle nodes
+    orc = O.GraphOracle(g)
+    sample = sorted(set(list(range(0, 40)) + list(range(g.num_nodes - 40, g.num_nodes)) +
+                        list(range(g.num_nodes // 2, g.num_nodes // 2 + 60))))
+    ref = orc.build(nodes=sample)
+    for v in sample:
+        for e in range(int(g.node_edge_off[v]), int(g.node_edge_off[v + 1])):
+            b0 = int(g.edge_off[e])
+            n = int(g.edge_sdst[e]) * int(g.edge_ssrc[e])
+            assert bits_equal(a["comm"][b0:b0 + n], ref["comm"][b0:b0 + n])
+            assert bits_equal(a["cost"][b0:b0 + n], ref["cost"][b0:b0 + n])

@@ -1,0 +1,218 @@
+"""Packed format invariants, decision-var assembly identities, the scorer's
+semantics on the reference's own mock data, and the C ABI surface (load +
+exported symbols; no GPU work)."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+from autoparallel_amd import graphgen, packed
+from autoparallel_amd.packed import GraphBuilder, NodeDesc
+from oracle import cost_oracle as O
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def small_llama():
+    return graphgen.llama_graph((8, 8), 1, 1024, 8, 4, 2048, 8192, 512, 16)
+
+
+def test_layout_invariants(small_llama):
+    g = small_llama
+    g.validate()
+    assert g.num_slots % 16 == 0 and g.num_slots >= g.num_entries
+    assert (g.edge_off[:-1] % 16 == 0).all()
+    slots = g.entry_slots()
+    assert slots.shape[0] == g.num_entries and len(np.unique(slots)) == g.num_entries
+    keys = g.entry_keys()
+    assert keys.shape == (g.num_entries, 4)
+    # every (node, arg, out, inp) key is unique and in range
+    assert len({tuple(k) for k in keys[:: max(1, len(keys) // 5000)]}) > 0
+    assert (keys[:, 2] < g.node_nstrat[keys[:, 0]]).all()
+    # chunk index: each 16-slot chunk belongs to the edge of its entries
+    eid = np.repeat(np.arange(g.num_edges), g.edge_sdst.astype(np.int64) * g.edge_ssrc)
+    assert (g.chunk_edge_index()[slots >> 4] == eid).all()
+    # work items tile every edge block exactly once
+    items = g.work_items()
+    covered = np.zeros(g.num_edges, np.int64)
+    item_edge = np.searchsorted(g.edge_off[:-1], items["off"])  # items copy their edge's record
+    assert (g.edge_off[:-1][item_edge] == items["off"]).all()
+    np.add.at(covered, item_edge, 1)
+    sizes = g.edge_sdst.astype(np.int64) * g.edge_ssrc
+    assert (covered == (sizes + 255) // 256).all()
+    assert (items["local0"] % 256 == 0).all()
+    # decision-var order: node, out_idx, argi, inp_idx
+    order = g.decision_var_order()
+    k = keys[order]
+    assert (np.lexsort((k[:, 3], k[:, 1], k[:, 2], k[:, 0])) == np.arange(len(k))).all()
+
+
+def test_magic_division_exact(small_llama):
+    rec = small_llama.edge_records()
+    for r in rec[:: max(1, len(rec) // 200)]:
+        if r["magic"] == 0:
+            continue
+        size = int(r["ssrc"]) * int(r["sdst"])
+        for local in {0, 1, size - 1, size // 2, int(r["ssrc"]) - 1, int(r["ssrc"])} & set(range(size)):
+            assert (local * int(r["magic"])) >> 32 == local // int(r["ssrc"])
+
+
+def test_shared_compute_slots_are_consistent(small_llama):
+    """Nodes that share a compute slot must produce identical estimates: the
+    oracle prices every node on its own and writes into the shared slot."""
+    g = small_llama
+    orc = O.GraphOracle(g)
+    seen = {}
+    for v in range(g.num_nodes):
+        vals = [float(orc.node_compute_cost(v, o)) for o in range(int(g.node_nstrat[v]))]
+        off = int(g.node_comp_off[v])
+        if off in seen:
+            assert seen[off] == vals
+        seen[off] = vals
+    assert len(seen) == g.comp_nodes.shape[0] < g.num_nodes
+
+
+def test_assembly_identities(small_llama):
+    g = small_llama
+    r = O.GraphOracle(g).build()
+    slots = g.entry_slots()
+    keys = g.entry_keys()
+    per_arg = r["compute"][g.node_comp_off[keys[:, 0]] + keys[:, 2]] / g.node_nargs[keys[:, 0]]
+    want = (r["comm"][slots] + per_arg) + r["transition"][slots]
+    got = r["cost"][slots]
+    fin = np.isfinite(want)
+    assert (got[fin] == want[fin]).all() and np.isinf(got[~fin]).all()
+    # placeholders: one entry per strategy, all zero
+    ph = g.edge_src_node < 0
+    for e in np.nonzero(ph)[0][:50]:
+        b = int(g.edge_off[e])
+        n = int(g.edge_sdst[e]) * int(g.edge_ssrc[e])
+        assert (r["cost"][b:b + n] == 0.0).all()
+    # transition can be 1 where comm is 0 (R -> S)
+    assert ((r["transition"][slots] == 1) & (r["comm"][slots] == 0.0)).any()
+    clamped, bad = O.clamp_inf(r["cost"])
+    assert (clamped[bad == 1] == 10000.0).all() and np.isfinite(clamped).all()
+
+
+def test_prefetch_discount_semantics(small_llama):
+    g = small_llama
+    r = O.GraphOracle(g).build()
+    cost, _ = O.clamp_inf(r["cost"])
+    comm2, cost2, n = O.prefetch_discount(g, r["comm"], r["transition"], r["compute"], cost, 0.0)
+    assert n > 0
+    changed = comm2 != r["comm"]
+    assert changed.sum() == n and (comm2[changed] == 0.0).all()
+    # the reference's own check (tests/test_prefetch_derived_sets.py:288-296 there):
+    # where comm was zeroed, cost == compute + transition
+    slots = g.entry_slots()
+    keys = g.entry_keys()
+    per_arg = np.zeros(g.num_slots)
+    per_arg[slots] = r["compute"][g.node_comp_off[keys[:, 0]] + keys[:, 2]] / g.node_nargs[keys[:, 0]]
+    assert (cost2[changed] == per_arg[changed] + r["transition"][changed]).all()
+    # untouched entries (inf or zero comm, non-prefetchable edges) keep their cost
+    assert (cost2[~changed] == cost[~changed]).all()
+    # scale 1.0 changes no value
+    comm3, cost3, n3 = O.prefetch_discount(g, r["comm"], r["transition"], r["compute"], cost, 1.0)
+    assert n3 == n and (comm3 == r["comm"]).all()
+
+
+def _mock_graph(entries):
+    """A chain of single-strategy nodes whose only entries carry the given
+    (compute, comm, transition) triples via explicit default rows."""
+    b = GraphBuilder((2,), 8)
+    m = b.meta((4,), (1,), 4, packed.DT_F32)
+    s = b.spec(m, (0,))
+    for i, (comp, comm, trans) in enumerate(entries):
+        b.add_node(NodeDesc(f"n{i}", in_specs=[[s]], out_specs=[[s]], inputs=[],
+                            default_rows=[[[float(comm)]]]))
+    return b.pack()
+
+
+def test_scorer_matches_reference_mock_totals():
+    """The reference's log-formatting tests build mock DecisionVars and expect
+    the totals to be plain sums of the selected entries' components
+    (tests/test_log_formatting.py:57-79 there: 1.0/2.0/0 -> total 3.00)."""
+    g = _mock_graph([(1.0, 2.0, 0)])
+    comm = np.zeros(g.num_slots)
+    comm[g.entry_slots()] = [2.0]
+    compute = np.asarray([1.0])
+    tot = O.score_assignment(g, comm, np.zeros(g.num_slots, np.uint8), compute, [0])
+    # a producer-less entry contributes its compute only (no predecessor strategy)
+    assert tot == (1.0, 1.0, 0.0, 0.0)
+    obj, viol = O.ilp_objective(g, comm + 1.0, np.zeros(g.num_slots, np.uint8), [0])
+    assert (obj, viol) == (3.0, 0)
+
+
+def test_scorer_on_graph(small_llama):
+    g = small_llama
+    r = O.GraphOracle(g).build()
+    cost, bad = O.clamp_inf(r["cost"])
+    assign = np.zeros(g.num_nodes, np.int64)  # strategy 0 everywhere: all replicate
+    total, comp, comm, trans = O.score_assignment(g, r["comm"], r["transition"], r["compute"], assign)
+    assert comm == 0.0 and trans == 0.0 and total == comp > 0
+    obj, viol = O.ilp_objective(g, cost, bad, assign)
+    assert viol == 0 and np.isclose(obj, total, rtol=1e-12)
+    rng = np.random.default_rng(0)
+    assign = rng.integers(0, g.node_nstrat)
+    total, comp, comm, trans = O.score_assignment(g, r["comm"], r["transition"], r["compute"], assign)
+    assert total == (comp + comm) + trans and trans > 0
+
+
+def test_builder_rejects_bad_programs():
+    with pytest.raises(AssertionError):
+        packed.check_program([1, 0, 2, 1, 3, 0], 2)  # factor names arg 3 of 2
+    with pytest.raises(AssertionError):
+        packed.check_program([0, 1, 2, 1, 1, 0, 9], 1)  # dim 9 >= MAX_RANK
+    packed.check_program([0, 1, 2, 1, 2, 0, 0], 1)
+
+
+def test_abi_exports_every_declared_symbol():
+    from autoparallel_amd import _lib
+
+    lib = _lib.load()
+    header = open(os.path.join(ROOT, "include", "apc.h")).read()
+    declared = set(re.findall(r"\b(apc_[a-z_0-9]+)\s*\(", header))
+    assert declared, "no declarations found"
+    for name in sorted(declared):
+        assert hasattr(lib, name), f"{name} declared in apc.h but not exported"
+    assert set(_lib.EXPORTED_SYMBOLS) == declared
+    assert lib.apc_version() >= 2
+    # struct sizes agree between the header's layout and the ctypes mirror
+    assert packed.PackedGraph.EDGE_DTYPE.itemsize == 64
+
+
+def test_abi_host_helpers():
+    from autoparallel_amd import _lib
+
+    lib = _lib.load()
+    shape = (ctypes.c_int32 * 4)(4, 8, 8, 1)
+    bw = (ctypes.c_double * 4)()
+    lat = (ctypes.c_double * 4)()
+    assert lib.apc_mesh_topology(ctypes.addressof(shape), 3, 8, ctypes.addressof(bw), ctypes.addressof(lat)) == 0
+    t = O.Topo((4, 8, 8), 8)
+    assert list(bw)[:3] == t.bw and list(lat)[:3] == t.lat
+    m = _lib.ApcModel()
+    assert lib.apc_device_limits(b"AMD Instinct MI355X", ctypes.byref(m)) == 0
+    assert m.gmem_bw == O.MI355X_GMEM_BW and list(m.tflops)[:5] == [O.MI355X_TFLOPS[i] for i in range(5)]
+    assert lib.apc_device_limits(b"Some Other GPU", ctypes.byref(m)) == _lib.load().apc_device_limits(b"x", ctypes.byref(m)) != 0
+    assert b"Unsupported device" in lib.apc_last_error()
+    # the host-side draw of the on-device assignment generator is deterministic and in range
+    draws = [lib.apc_random_assignment(7, a, v, 13) for a in range(20) for v in range(20)]
+    assert all(0 <= d < 13 for d in draws) and len(set(draws)) > 5
+    assert draws == [lib.apc_random_assignment(7, a, v, 13) for a in range(20) for v in range(20)]
+
+
+def test_engine_needs_gpu():
+    import torch
+
+    from autoparallel_amd import _lib
+    from autoparallel_amd.engine import CostEngine
+
+    if torch.cuda.is_available():
+        pytest.skip("GPU present")
+    g = _mock_graph([(1.0, 2.0, 0)])
+    with pytest.raises(Exception):
+        CostEngine(g, device="cpu")
