@@ -22,6 +22,8 @@ class ApcModel(C.Structure):
         ("mesh_lat", C.c_double * MAX_MESH_DIMS),
         ("gmem_bw", C.c_double),
         ("tflops", C.c_double * NUM_DTYPES),
+        ("order_mode", C.c_int32),
+        ("reserved", C.c_int32),
     ]
 
 
@@ -109,6 +111,14 @@ _SIGNATURES = {
         [C.POINTER(ApcProblem), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint64,
          C.c_int64, C.c_int64, C.c_void_p, C.c_void_p]),
     "apc_random_assignment": (C.c_uint32, [C.c_uint64, C.c_int64, C.c_int32, C.c_int32]),
+    "apc_local_shapes": (
+        C.c_int,
+        [C.POINTER(ApcModel), C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+         C.c_void_p, C.c_void_p]),
+    "apc_collective_costs": (
+        C.c_int,
+        [C.POINTER(ApcModel), C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
+    "apc_rw_times": (C.c_int, [C.POINTER(ApcModel), C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p]),
     "apc_enumerate_input_options": (
         C.c_int,
         [C.POINTER(ApcModel), C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,

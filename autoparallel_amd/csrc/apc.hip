@@ -100,8 +100,12 @@ __device__ double redistribute_cost(uint32_t src, uint32_t tgt, int64_t tensor_b
     tgt_all_shard &= (((tgt >> (8 * i)) & kKindMask) == kShard);
   }
   double gb = (double)tensor_bytes / (double)num_shards / 1024.0 / 1024.0 / 1024.0;
+  // order rule of estimate_strategy_comms_cost (:253-258), or an order forced by
+  // the caller of redistribute_cost (order_mode 1: 0..ndim-1, 2: ndim-1..0)
   const bool reversed =
-      (ndim == 2) && (src == (uint32_t)(kPartialSum | (kPartialSum << 8))) && tgt_all_shard;
+      m.order_mode == 0
+          ? ((ndim == 2) && (src == (uint32_t)(kPartialSum | (kPartialSum << 8))) && tgt_all_shard)
+          : (m.order_mode == 2);
   double cost = 0.0;
   for (int step = 0; step < ndim; ++step) {
     const int i = reversed ? (ndim - 1 - step) : step;
@@ -699,6 +703,55 @@ enumerate_kernel(apc_model m, int32_t n, const int32_t* __restrict__ rank,
 }
 
 // ---------------------------------------------------------------------------
+// Kernels: scalar cost-model functions in batch form
+// ---------------------------------------------------------------------------
+// _get_sharded_shape_stride (compute_estimation.py:300-318), including its
+// stride rule: the stride of dim d-1 is divided only when d-1 > 0.
+__global__ void __launch_bounds__(kBlock)
+local_shape_kernel(apc_model m, int32_t n, const int32_t* __restrict__ rank,
+                   const int64_t* __restrict__ shape, const int64_t* __restrict__ stride,
+                   const uint8_t* __restrict__ plc, int64_t* __restrict__ out_shape,
+                   int64_t* __restrict__ out_stride) {
+  const int t = blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= n) return;
+  const int r = rank[t];
+  for (int d = 0; d < APC_MAX_RANK; ++d) {
+    out_shape[(size_t)t * APC_MAX_RANK + d] = shape[(size_t)t * APC_MAX_RANK + d];
+    out_stride[(size_t)t * APC_MAX_RANK + d] = stride[(size_t)t * APC_MAX_RANK + d];
+  }
+  for (int i = 0; i < m.ndim; ++i) {
+    const int c = plc[(size_t)t * APC_MAX_MESH_DIMS + i];
+    if ((c & kKindMask) != kShard) continue;
+    const int d = c & kArgMask;
+    if (d >= r) continue;
+    const int64_t ms = m.mesh_shape[i];
+    int64_t* s = out_shape + (size_t)t * APC_MAX_RANK;
+    int64_t* st = out_stride + (size_t)t * APC_MAX_RANK;
+    s[d] = (s[d] + ms - 1) / ms;
+    if (d - 1 > 0) st[d - 1] = (st[d - 1] + ms - 1) / ms;
+  }
+}
+
+// collective_comm_cost, default model (collective_runtime_estimation.py:65-97):
+// kind 0 allgather, 1 all_to_all, 2 allreduce, 3 reduce_scatter, else 0.0
+__global__ void __launch_bounds__(kBlock)
+collective_kernel(apc_model m, int32_t n, const int32_t* __restrict__ kind,
+                  const int64_t* __restrict__ nbytes, const int32_t* __restrict__ dim,
+                  double* __restrict__ out) {
+  const int t = blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= n) return;
+  const int k = kind[t], d = dim[t];
+  out[t] = (k >= 0 && k <= 3 && d >= 0 && d < m.ndim) ? collective_cost(k, nbytes[t], d, m) : 0.0;
+}
+
+// compute_read_write_time (compute_estimation.py:391-403)
+__global__ void __launch_bounds__(kBlock)
+rw_time_kernel(apc_model m, int32_t n, const double* __restrict__ nbytes, double* __restrict__ out) {
+  const int t = blockIdx.x * blockDim.x + threadIdx.x;
+  if (t < n) out[t] = rw_time(nbytes[t], m.gmem_bw);
+}
+
+// ---------------------------------------------------------------------------
 // Host side
 // ---------------------------------------------------------------------------
 int validate_problem(const apc_problem* p) {
@@ -707,6 +760,8 @@ int validate_problem(const apc_problem* p) {
     return fail(APC_ERR_INVALID, "mesh ndim out of range%s");
   for (int i = 0; i < p->model.ndim; ++i)
     if (p->model.mesh_shape[i] < 1) return fail(APC_ERR_INVALID, "mesh size < 1%s");
+  if (p->model.order_mode < 0 || p->model.order_mode > 2)
+    return fail(APC_ERR_INVALID, "order_mode must be 0, 1 or 2%s");
   if (p->n_meta < 0 || p->n_tuple < 0 || p->n_tuple > (1 << APC_TUPLE_BITS))
     return fail(APC_ERR_INVALID, "bad meta/tuple counts%s");
   if (p->n_node < 0 || p->n_edge < 0 || p->n_entry < 0 || p->n_comp_node < 0 ||
@@ -934,6 +989,41 @@ int apc_score_random_assignments(const apc_problem* p, const double* per_arg, co
 
 uint32_t apc_random_assignment(uint64_t seed, int64_t a, int32_t node, int32_t nstrat) {
   return mix_assignment(seed, a, node, nstrat);
+}
+
+int apc_local_shapes(const apc_model* model, int32_t n, const int32_t* rank, const int64_t* shape,
+                     const int64_t* stride, const uint8_t* plc, int64_t* out_shape,
+                     int64_t* out_stride, void* stream) {
+  if (!model || model->ndim < 1 || model->ndim > APC_MAX_MESH_DIMS)
+    return fail(APC_ERR_INVALID, "apc_local_shapes: bad model%s");
+  if (n <= 0) return 0;
+  if (!rank || !shape || !stride || !plc || !out_shape || !out_stride)
+    return fail(APC_ERR_INVALID, "apc_local_shapes: null argument%s");
+  hipLaunchKernelGGL(local_shape_kernel, dim3((n + kBlock - 1) / kBlock), dim3(kBlock), 0,
+                     (hipStream_t)stream, *model, n, rank, shape, stride, plc, out_shape, out_stride);
+  return check_launch("local_shape_kernel");
+}
+
+int apc_collective_costs(const apc_model* model, int32_t n, const int32_t* kind,
+                         const int64_t* nbytes, const int32_t* dim, double* out, void* stream) {
+  if (!model || model->ndim < 1 || model->ndim > APC_MAX_MESH_DIMS)
+    return fail(APC_ERR_INVALID, "apc_collective_costs: bad model%s");
+  if (n <= 0) return 0;
+  if (!kind || !nbytes || !dim || !out)
+    return fail(APC_ERR_INVALID, "apc_collective_costs: null argument%s");
+  hipLaunchKernelGGL(collective_kernel, dim3((n + kBlock - 1) / kBlock), dim3(kBlock), 0,
+                     (hipStream_t)stream, *model, n, kind, nbytes, dim, out);
+  return check_launch("collective_kernel");
+}
+
+int apc_rw_times(const apc_model* model, int32_t n, const double* nbytes, double* out,
+                 void* stream) {
+  if (!model) return fail(APC_ERR_INVALID, "apc_rw_times: null model%s");
+  if (n <= 0) return 0;
+  if (!nbytes || !out) return fail(APC_ERR_INVALID, "apc_rw_times: null argument%s");
+  hipLaunchKernelGGL(rw_time_kernel, dim3((n + kBlock - 1) / kBlock), dim3(kBlock), 0,
+                     (hipStream_t)stream, *model, n, nbytes, out);
+  return check_launch("rw_time_kernel");
 }
 
 int apc_enumerate_input_options(const apc_model* model, int32_t n, const int32_t* rank,

@@ -18,7 +18,7 @@ _TABLE_MAX_RATIO = 1.0
 _TABLE_MAX_DOUBLES = 1 << 28
 
 
-def make_model(mesh_shape, devices_per_host: int, device_name: str) -> _lib.ApcModel:
+def make_model(mesh_shape, devices_per_host: int, device_name: str, order_mode: int = 0) -> _lib.ApcModel:
     """Cost-model constants for a mesh on a named device (raises ApcError for a
     device the reference's table does not know either)."""
     lib = _lib.load()
@@ -26,6 +26,7 @@ def make_model(mesh_shape, devices_per_host: int, device_name: str) -> _lib.ApcM
     nd = len(mesh_shape)
     assert 1 <= nd <= MAX_MESH_DIMS
     m.ndim = nd
+    m.order_mode = int(order_mode)
     shape = (C.c_int32 * MAX_MESH_DIMS)(*([int(x) for x in mesh_shape] + [1] * (MAX_MESH_DIMS - nd)))
     m.mesh_shape = shape
     bw = (C.c_double * MAX_MESH_DIMS)()
@@ -62,6 +63,7 @@ class CostEngine:
         device: str = "cuda",
         device_name: Optional[str] = None,
         use_table: Optional[bool] = None,
+        order_mode: int = 0,
     ):
         self.lib = _lib.load()
         self.g = g
@@ -89,7 +91,7 @@ class CostEngine:
             return t.data_ptr() if t.numel() else None
 
         p = _lib.ApcProblem()
-        p.model = make_model([int(x) for x in g.mesh_shape], g.devices_per_host, device_name)
+        p.model = make_model([int(x) for x in g.mesh_shape], g.devices_per_host, device_name, order_mode)
         p.n_meta = g.meta_rank.shape[0]
         p.meta_rank = up("meta_rank", g.meta_rank)
         p.meta_shape = up("meta_shape", g.meta_shape)

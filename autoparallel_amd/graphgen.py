@@ -659,7 +659,48 @@ class Tracer:
                     self.b.prefetchable_edges.add((v, a))
         self.param_derived = param_derived
         self.terminal_derived = terminal
-        return self.b.pack()
+        g = self.b.pack()
+        g.roles = self._roles(param_grads, outputs)
+        return g
+
+    def _roles(self, param_grads: Dict[int, T], outputs: List[T]):
+        """Forward/backward pairs and dtype-cast chains, as the reference derives
+        them from the AOT graph (autoparallel/optimize_sharding.py:1463-1606)."""
+        from .sharding_problem import GraphRoles
+
+        names = [n.name for n in self.b.nodes]
+        is_cast = lambda v: names[v].startswith("_to_copy")
+        roles = GraphRoles()
+        roles.param_grad = [(p, (param_grads[p].node if p in param_grads else -1)) for p in self.param_nodes]
+        roles.output_tangent = [(o.node, t.node) for o, t in getattr(self, "_tangents", [])]
+        metas = self.b._meta_rows
+        itemsize_of = lambda v: metas[self.b.nodes[v].out_specs[0][0] >> 12][2]
+        for p in self.param_nodes:
+            # forward: param -> single-user unary chain -> cast that lowers precision
+            chain, n = [], p
+            while not is_cast(n):
+                users = list(dict.fromkeys(self.node_users.get(n, [])))
+                if len(users) != 1 or len(set(self.node_inputs[users[0]])) != 1:
+                    break
+                n = users[0]
+                chain.append(n)
+            if is_cast(n) and n != p and itemsize_of(n) < itemsize_of(p):
+                roles.fwd_pre_cast.update(chain)
+            # backward: grad <- unary chain <- cast
+            if p in param_grads:
+                g_ = param_grads[p].node
+                chain, n = [g_], g_
+                while len(set(self.node_inputs.get(n, []))) == 1:
+                    parent = self.node_inputs[n][0]
+                    if len(set(self.node_inputs.get(parent, []))) != 1:
+                        break
+                    chain.append(parent)
+                    n = parent
+                for i, v in enumerate(chain):
+                    if is_cast(v):
+                        roles.bwd_pre_cast.update(chain[i:])
+                        break
+        return roles
 
 
 # ===========================================================================
@@ -770,6 +811,7 @@ def llama_graph(
     h = _rmsnorm(t, h, norm_w)
     logits = _linear(t, h, out_w)
     grads = t.backward([(logits, tangent)])
+    t._tangents = [(logits, tangent)]
     param_grads = {}
     for name, p in params.items():
         g = grads.get((p.node, None))
@@ -837,6 +879,7 @@ def gpt2_graph(
     h = _layernorm(t, h, lnfw, lnfb)
     logits = _linear(t, h, wte)
     grads = t.backward([(logits, tangent)])
+    t._tangents = [(logits, tangent)]
     param_grads = {}
     for name, p in params.items():
         g = grads.get((p.node, None))

@@ -154,6 +154,7 @@ class PackedGraph:
     node_op: np.ndarray  # int32[N]   OP_*
     node_prog_off: np.ndarray  # int64[N]   offset into prog (-1 if none)
     node_prog_len: np.ndarray  # int32[N]   words of the node's program (0 if none)
+    node_out_list: np.ndarray  # int64[N]   run of the node's (first) output spec words
     prog: np.ndarray  # int64[...] compute programs
     # explicit flops/bytes (OP_EXPLICIT), indexed like the compute vector
     explicit_flops: Optional[np.ndarray] = None  # int64[sum S]
@@ -176,6 +177,7 @@ class PackedGraph:
     # cluster multiplicity per node: 1 + number of linked copies (:883)
     node_multiplier: Optional[np.ndarray] = None  # int32[N]
     node_names: Optional[List[str]] = None
+    roles: Optional[object] = None  # sharding_problem.GraphRoles (fwd/bwd pairs, cast chains)
 
     # -- derived sizes -------------------------------------------------------
     @property
@@ -709,6 +711,7 @@ class GraphBuilder:
             node_op=node_op,
             node_prog_off=node_prog_off,
             node_prog_len=node_prog_len,
+            node_out_list=np.asarray([r[0] for r in out_runs], np.int64),
             prog=np.asarray(prog, np.int64),
             explicit_flops=ef,
             explicit_bytes=eb,

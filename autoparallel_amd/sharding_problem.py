@@ -1,0 +1,391 @@
+"""ILP formulation of the sharding search over a packed graph.
+
+Mirrors the reference's ``ShardingOptimizer`` below the FX layer
+(autoparallel/optimize_sharding.py): coefficients come from the HIP engine,
+constraint rows are assembled from index arithmetic on the packed layout, and
+the model is handed to a MILP solver.  Decision variable (node v, arg a, out o,
+inp j) is column ``var_start[e(v, a)] + o * S_src + j``.
+
+Constraint families and their reference counterparts:
+  unique_decision          add_unique_decision_constraint            :665-688
+  same_across_args         add_same_output_across_args_constraint     :690-721
+  output_input_consistent  add_output_input_consistent_constraint     :723-801
+  inf_cases                add_inf_cost_constraint                    :803-812
+  grad_*_constraint        add_forward_backward_consistency_constraints :1463-1485
+  fwd_param_dtype / grad_reduce_dtype  add_grad_reduce_dtype_constraints  :1487-1606
+  memory_constraint_*      _apply_memory_constraint                   :1629-1671
+  user constraints         add_node_constraint / _add_node_constraint :1401-1417, 1673-1718
+"""
+from __future__ import annotations
+
+import dataclasses
+import math
+from typing import Dict, Iterable, List, Optional, Sequence, Set, Tuple
+
+import numpy as np
+
+from . import ilp
+from .packed import MAX_TUPLES, SPEC_NONE, PackedGraph, plc_str
+
+
+@dataclasses.dataclass
+class GraphRoles:
+    """What the reference reads off the AOT graph descriptors
+    (torch._functorch._aot_autograd.fx_utils): forward/backward pairs and the
+    dtype-cast chains of parameters and gradients."""
+
+    param_grad: List[Tuple[int, int]] = dataclasses.field(default_factory=list)  # grad -1 if none
+    input_grad: List[Tuple[int, int]] = dataclasses.field(default_factory=list)
+    output_tangent: List[Tuple[int, int]] = dataclasses.field(default_factory=list)
+    fwd_pre_cast: Set[int] = dataclasses.field(default_factory=set)
+    bwd_pre_cast: Set[int] = dataclasses.field(default_factory=set)
+
+
+class Coefficients:
+    """Host copy of the coefficient arrays, one element per decision variable
+    (padding slots removed), plus the per-(node, out_idx) compute vectors."""
+
+    def __init__(self, g: PackedGraph, comm, cost, flags, compute, per_arg):
+        slots = g.entry_slots()
+        self.comm = np.ascontiguousarray(comm[slots])
+        self.cost = np.ascontiguousarray(cost[slots])
+        self.flags = np.ascontiguousarray(flags[slots])
+        self.compute = np.asarray(compute)
+        self.per_arg = np.asarray(per_arg)
+
+    @classmethod
+    def from_engine(cls, eng) -> "Coefficients":
+        r = eng.results()
+        return cls(eng.g, r["comm"], r["cost"], r["flags"], r["compute"], r["per_arg"])
+
+
+class PackedShardingOptimizer:
+    def __init__(
+        self,
+        g: PackedGraph,
+        roles: Optional[GraphRoles] = None,
+        force_grad_reduce_in_higher_precision: bool = False,
+        coefficients: Optional[Coefficients] = None,
+        device: str = "cuda",
+        device_name: Optional[str] = None,
+    ):
+        self.g = g
+        self.roles = roles or getattr(g, "roles", None) or GraphRoles()
+        self.force_grad_reduce_in_higher_precision = force_grad_reduce_in_higher_precision
+        self.engine = None
+        if coefficients is None:
+            from .engine import CostEngine  # the HIP path; raises without the library / a GPU
+
+            self.engine = CostEngine(g, device=device, device_name=device_name)
+            self.engine.build(clamp_inf=True)
+            coefficients = Coefficients.from_engine(self.engine)
+        self.coef = coefficients
+        sizes = g.edge_sdst.astype(np.int64) * g.edge_ssrc
+        self.var_start = np.concatenate([[0], np.cumsum(sizes)]).astype(np.int64)
+        self.n_vars = int(self.var_start[-1])
+        self.prob = ilp.SparseILP(self.n_vars)
+        self._memory_constraint: Optional[Tuple[float, float]] = None
+        self._node_constraint_names: Dict[str, int] = {}
+        self.selected: Optional[np.ndarray] = None
+        self.add_default_constraints()
+
+    # -- indexing ---------------------------------------------------------------
+    def edge_of(self, v: int, a: int) -> int:
+        e = int(self.g.node_edge_off[v]) + a
+        assert e < int(self.g.node_edge_off[v + 1])
+        return e
+
+    def var(self, v: int, a: int, o: int, j: int) -> int:
+        e = self.edge_of(v, a)
+        return int(self.var_start[e]) + o * int(self.g.edge_ssrc[e]) + j
+
+    def _row_vars(self, e: int, o: int) -> np.ndarray:
+        """Variables of edge e with output strategy o (all inp_idx)."""
+        s = int(self.g.edge_ssrc[e])
+        b = int(self.var_start[e]) + o * s
+        return np.arange(b, b + s, dtype=np.int64)
+
+    def _col_vars(self, e: int, j: int) -> np.ndarray:
+        """Variables of edge e with input strategy j (all out_idx)."""
+        s = int(self.g.edge_ssrc[e])
+        return int(self.var_start[e]) + np.arange(int(self.g.edge_sdst[e]), dtype=np.int64) * s + j
+
+    def var_names(self) -> List[str]:
+        g = self.g
+        keys = g.entry_keys()
+        names = g.node_names or [f"node{i}" for i in range(g.num_nodes)]
+        return [f"n={names[v]},s={v},arg={a},output_p={o},input_p={j}" for v, a, o, j in keys]
+
+    # -- default constraints ------------------------------------------------------
+    def add_default_constraints(self) -> None:
+        self.add_unique_decision_constraint()
+        self.add_same_output_across_args_constraint()
+        self.add_output_input_consistent_constraint()
+        self.add_inf_cost_constraint()
+        self.add_forward_backward_consistency_constraints()
+        self.add_grad_reduce_dtype_constraints()
+
+    def add_unique_decision_constraint(self) -> None:
+        # for every (node, arg): exactly one (out, inp) pair
+        for e in range(self.g.num_edges):
+            idx = np.arange(self.var_start[e], self.var_start[e + 1], dtype=np.int64)
+            self.prob.add_row("unique_decision", idx, 1.0, ilp.EQ, 1.0)
+
+    def _num_input_nodes(self, v: int) -> int:
+        g = self.g
+        e0, e1 = int(g.node_edge_off[v]), int(g.node_edge_off[v + 1])
+        return int((g.edge_src_node[e0:e1] >= 0).sum())
+
+    def add_same_output_across_args_constraint(self) -> None:
+        # all arguments of a node pick the same output strategy
+        g = self.g
+        for v in range(g.num_nodes):
+            if self._num_input_nodes(v) <= 1:
+                continue
+            e0, e1 = int(g.node_edge_off[v]), int(g.node_edge_off[v + 1])
+            for e in range(e0 + 1, e1):
+                for o in range(int(g.node_nstrat[v])):
+                    a0, ak = self._row_vars(e0, o), self._row_vars(e, o)
+                    self.prob.add_row(
+                        "same_across_args", np.concatenate([a0, ak]),
+                        np.concatenate([np.ones(len(a0)), -np.ones(len(ak))]), ilp.EQ, 0.0)
+
+    def add_output_input_consistent_constraint(self) -> None:
+        # producer's chosen output strategy == the input strategy its consumer assumes
+        g = self.g
+        seen = set()
+        users: Dict[int, List[Tuple[int, int]]] = {}
+        for e in range(g.num_edges):
+            u = int(g.edge_src_node[e])
+            if u < 0:
+                continue
+            v = int(g.edge_node[e])
+            if (u, v) in seen:  # first matching argument only
+                continue
+            seen.add((u, v))
+            users.setdefault(u, []).append((v, e))
+        for u in sorted(users):
+            eu = int(g.node_edge_off[u])  # argument 0 of the producer
+            for v, e in users[u]:
+                assert int(g.edge_ssrc[e]) == int(g.node_nstrat[u])
+                for k in range(int(g.node_nstrat[u])):
+                    pu, cv = self._row_vars(eu, k), self._col_vars(e, k)
+                    self.prob.add_row(
+                        "output_input_consistent", np.concatenate([pu, cv]),
+                        np.concatenate([np.ones(len(pu)), -np.ones(len(cv))]), ilp.EQ, 0.0)
+
+    def add_inf_cost_constraint(self) -> None:
+        # the engine already wrote 10000.0 into cost; pin those variables to 0
+        for i in np.nonzero(self.coef.flags & 2)[0]:
+            self.prob.add_row("inf_cases", [i], 1.0, ilp.EQ, 0.0)
+
+    def _out_placements(self, v: int) -> List[Optional[int]]:
+        """Placement-tuple id of output 0 of each strategy of node v (None for
+        a missing spec): what ``str(output_specs)`` distinguishes."""
+        g = self.g
+        run = int(g.node_out_list[v])
+        words = g.lists[run : run + int(g.node_nstrat[v])]
+        return [None if int(w) == SPEC_NONE else int(w) & (MAX_TUPLES - 1) for w in words]
+
+    def _add_paired_output_constraint(self, a: int, b: int, name: str) -> None:
+        pa, pb = self._out_placements(a), self._out_placements(b)
+        ea, eb = int(self.g.node_edge_off[a]), int(self.g.node_edge_off[b])
+        for o, t in enumerate(pa):
+            va = self._row_vars(ea, o)
+            if t not in pb:
+                self.prob.add_row(name + "_disable", va, 1.0, ilp.EQ, 0.0)
+                continue
+            vb = self._row_vars(eb, pb.index(t))
+            self.prob.add_row(name, np.concatenate([vb, va]),
+                              np.concatenate([np.ones(len(vb)), -np.ones(len(va))]), ilp.EQ, 0.0)
+
+    def add_forward_backward_consistency_constraints(self) -> None:
+        for p, gnode in self.roles.param_grad:
+            if gnode >= 0:
+                self._add_paired_output_constraint(p, gnode, "grad_param_constraint")
+        for n, gnode in self.roles.input_grad:
+            if gnode >= 0:
+                self._add_paired_output_constraint(n, gnode, "grad_input_constraint")
+        for n, t in self.roles.output_tangent:
+            if t >= 0:
+                self._add_paired_output_constraint(n, t, "grad_output_constraint")
+
+    def add_grad_reduce_dtype_constraints(self) -> None:
+        keys = self.g.entry_keys()
+        comm_pos = self.coef.comm > 0
+        for nodes, name, enabled in (
+            (self.roles.fwd_pre_cast, "fwd_param_dtype", True),
+            (self.roles.bwd_pre_cast, "grad_reduce_dtype", self.force_grad_reduce_in_higher_precision),
+        ):
+            if not enabled or not nodes:
+                continue
+            mask = np.isin(keys[:, 0], np.fromiter(nodes, np.int64)) & comm_pos
+            for i in np.nonzero(mask)[0]:
+                self.prob.add_row(name, [i], 1.0, ilp.EQ, 0.0)
+
+    # -- user constraints -----------------------------------------------------------
+    def add_node_constraint(self, v: int, placement: Optional[Sequence[int]] = None,
+                            constraint_name: Optional[str] = None) -> List[str]:
+        """Force node v's output placement (placement bytes per mesh dim;
+        default Shard(0) on the first mesh dim, Replicate elsewhere)."""
+        g = self.g
+        if placement is None:
+            placement = (0x40,) + (0x00,) * (g.ndim - 1)
+        want = tuple(int(p) for p in placement)
+        allowed = [o for o, t in enumerate(self._out_placements(v))
+                   if t is not None and tuple(int(x) for x in g.tuple_plc[t, : g.ndim]) == want]
+        if not allowed:
+            raise RuntimeError(
+                f"Couldn't find appropriate constraint {g.node_names[v] if g.node_names else v} "
+                f"{constraint_name} {[plc_str(p) for p in want]}")
+        names = []
+        for e in range(int(g.node_edge_off[v]), int(g.node_edge_off[v + 1])):
+            idx = np.concatenate([self._row_vars(e, o) for o in allowed])
+            name = self.prob.add_row(constraint_name or "user_constraint", idx, 1.0, ilp.EQ, 1.0)
+            names.append(name)
+            self._node_constraint_names[name] = v
+        return names
+
+    def add_parameter_memory_constraint(self, memory_factor_low: float, memory_factor_high: float) -> None:
+        self._memory_constraint = (memory_factor_low, memory_factor_high)
+
+    def _memory_ratios(self, params: List[int]) -> List[np.ndarray]:
+        """prod(local shape) / prod(global shape) of every strategy of every
+        parameter, local shapes from the device (apc_local_shapes)."""
+        import ctypes as C
+
+        import torch
+
+        from . import _lib
+        from .engine import make_model
+
+        g = self.g
+        lib = _lib.load()
+        rows = []
+        for p in params:
+            run = int(g.edge_dst_list[int(g.node_edge_off[p])])
+            for w in g.lists[run : run + int(g.node_nstrat[p])]:
+                rows.append((int(w) >> 12, int(w) & (MAX_TUPLES - 1)))
+        mids = np.asarray([r[0] for r in rows], np.int64)
+        tids = np.asarray([r[1] for r in rows], np.int64)
+        dev = self.engine.device if self.engine is not None else torch.device("cuda")
+        up = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+        rank, shape, stride = up(g.meta_rank[mids]), up(g.meta_shape[mids]), up(g.meta_stride[mids])
+        plc = up(g.tuple_plc[tids])
+        out_shape, out_stride = torch.empty_like(shape), torch.empty_like(stride)
+        name = self.engine.device_name if self.engine is not None else "AMD Instinct MI355X"
+        model = make_model([int(x) for x in g.mesh_shape], g.devices_per_host, name)
+        _lib.check(lib.apc_local_shapes(C.byref(model), len(rows), rank.data_ptr(), shape.data_ptr(),
+                                        stride.data_ptr(), plc.data_ptr(), out_shape.data_ptr(),
+                                        out_stride.data_ptr(), None), "apc_local_shapes")
+        torch.cuda.synchronize(dev)
+        local = out_shape.cpu().numpy()
+        ratios, k = [], 0
+        for p in params:
+            S = int(g.node_nstrat[p])
+            r = []
+            for i in range(S):
+                rk = int(g.meta_rank[mids[k + i]])
+                new = math.prod(int(x) for x in local[k + i, :rk])
+                old = math.prod(int(x) for x in g.meta_shape[mids[k + i], :rk])
+                r.append(new / old)
+            ratios.append(np.asarray(r))
+            k += S
+        return ratios
+
+    def _apply_memory_constraint(self) -> None:
+        if self._memory_constraint is None:
+            return
+        low, high = self._memory_constraint
+        for name in ("memory_constraint_high", "memory_constraint_low"):
+            self.prob.constraints.pop(name, None)
+        constrained = set(self._node_constraint_names.values())
+        params = [p for p, _ in self.roles.param_grad if p not in constrained]
+        if not params:
+            return
+        idx, coef = [], []
+        budget_low = budget_high = 0.0
+        for p, ratios in zip(params, self._memory_ratios(params)):
+            for o, r in enumerate(ratios):
+                idx.append(self.var(p, 0, o, 0))
+                coef.append(r)
+            best = float(ratios.min())
+            budget_low += max(best, low)
+            budget_high += max(best, high)
+        self.prob.add_row("memory_constraint_high", idx, coef, ilp.LE, budget_high, exact_name=True)
+        self.prob.add_row("memory_constraint_low", idx, coef, ilp.GE, budget_low, exact_name=True)
+
+    def remove_constraints(self, names: Iterable[str]) -> None:
+        for name in names:
+            self.prob.remove(name)
+            self._node_constraint_names.pop(name, None)
+            if name in ("memory_constraint_high", "memory_constraint_low"):
+                self._memory_constraint = None
+
+    # -- coefficient post-passes ---------------------------------------------------
+    def apply_prefetch_discount(self, scale: float = 0.0) -> int:
+        """Needs the engine (runs on the device arrays), then refreshes the host copy."""
+        assert self.engine is not None, "coefficients were injected: no engine to run the discount on"
+        n = self.engine.apply_prefetch_discount(scale)
+        self.coef = Coefficients.from_engine(self.engine)
+        return n
+
+    # -- solve ------------------------------------------------------------------------
+    def _set_objective(self) -> None:
+        keys = self.g.entry_keys()
+        mult = self.g.node_multiplier[keys[:, 0]] if self.g.node_multiplier is not None else 1
+        self.prob.objective = self.coef.cost * mult
+
+    def _solve(self, backend: str = "auto", verbose: bool = False) -> None:
+        self._apply_memory_constraint()
+        status = self.prob.solve(backend=backend, verbose=verbose)
+        if status == ilp.STATUS_INFEASIBLE:
+            raise RuntimeError(
+                "The sharding optimizer could not find a feasible solution. This typically means "
+                "the user-specified constraints are contradictory or the device mesh is too small "
+                "for the requested sharding.")
+        self.selected = np.nonzero(self.prob.x > 0.5)[0]
+
+    def _extract(self) -> np.ndarray:
+        """out_idx per node from the selected variables; checks that each
+        (node, arg) has exactly one selection and that all args agree."""
+        keys = self.g.entry_keys()[self.selected]
+        sol = np.full(self.g.num_nodes, -1, np.int64)
+        seen = set()
+        for v, a, o, j in keys:
+            if (v, a) in seen:
+                raise RuntimeError(f"Multiple solutions for node {v}, arg {a}")
+            seen.add((int(v), int(a)))
+            if sol[v] >= 0 and sol[v] != o:
+                raise AssertionError(f"arguments of node {v} disagree on the output strategy")
+            sol[v] = o
+        return sol
+
+    def get_solution(self, backend: str = "auto", verbose: bool = False) -> np.ndarray:
+        self._set_objective()
+        self._solve(backend, verbose)
+        return self._extract()
+
+    def resolve(self, backend: str = "auto", verbose: bool = False) -> np.ndarray:
+        self._solve(backend, verbose)
+        return self._extract()
+
+    @property
+    def objective_value(self) -> float:
+        return self.prob.objective_value
+
+    def solution_placements(self, sol: np.ndarray) -> List[Optional[Tuple[str, ...]]]:
+        out = []
+        for v in range(self.g.num_nodes):
+            t = self._out_placements(v)[int(sol[v])]
+            out.append(None if t is None else tuple(plc_str(int(c)) for c in self.g.tuple_plc[t, : self.g.ndim]))
+        return out
+
+    def compute_solution_cost(self, sol: np.ndarray) -> Dict[str, float]:
+        """The reference's _compute_solution_cost for one assignment, on the device."""
+        assert self.engine is not None
+        import torch
+
+        a = torch.from_numpy(np.ascontiguousarray(sol.astype(np.int16).reshape(-1, 1))).to(self.engine.device)
+        r = self.engine.score(a).cpu().numpy()[0]
+        return {"total": r[0], "compute": r[1], "comm": r[2], "transition": r[3]}

@@ -74,6 +74,13 @@ typedef struct apc_model {
   double mesh_lat[APC_MAX_MESH_DIMS]; /* us per hop per mesh dim            */
   double gmem_bw;                     /* bytes/s                            */
   double tflops[APC_NUM_DTYPES];      /* by dtype code; <= 0: unsupported   */
+  /* mesh-dim order of the redistribution fold: 0 = the rule of
+   * estimate_strategy_comms_cost (collective_runtime_estimation.py:253-258:
+   * [1,0] for (Partial,Partial) -> all-Shard on a 2-D mesh, else 0..ndim-1);
+   * 1 = always 0..ndim-1; 2 = always ndim-1..0 (an explicit `order` argument
+   * of redistribute_cost, :115-119) */
+  int32_t order_mode;
+  int32_t reserved;
 } apc_model;
 
 /* The packed problem (see autoparallel_amd/packed.py for the layout). */
@@ -238,6 +245,26 @@ int apc_score_random_assignments(const apc_problem* p, const double* per_arg, co
                                  const double* cost, const uint8_t* flags, uint64_t seed,
                                  int64_t first, int64_t n_assign, double* out, void* stream);
 uint32_t apc_random_assignment(uint64_t seed, int64_t a, int32_t node, int32_t nstrat);
+
+/* Replaces _get_sharded_shape_stride
+ * (autoparallel/cost_models/compute_estimation.py:300-318) for n specs:
+ * rank[i], shape/stride[i][APC_MAX_RANK], plc[i][APC_MAX_MESH_DIMS] ->
+ * out_shape / out_stride[i][APC_MAX_RANK]. */
+int apc_local_shapes(const apc_model* model, int32_t n, const int32_t* rank, const int64_t* shape,
+                     const int64_t* stride, const uint8_t* plc, int64_t* out_shape,
+                     int64_t* out_stride, void* stream);
+
+/* Replaces collective_comm_cost, default model
+ * (autoparallel/cost_models/collective_runtime_estimation.py:65-110) for n
+ * queries: kind[i] 0 allgather, 1 all_to_all, 2 allreduce, 3 reduce_scatter
+ * (anything else costs 0.0), nbytes[i], mesh dim[i] -> out[i] microseconds. */
+int apc_collective_costs(const apc_model* model, int32_t n, const int32_t* kind,
+                         const int64_t* nbytes, const int32_t* dim, double* out, void* stream);
+
+/* Replaces compute_read_write_time
+ * (autoparallel/cost_models/compute_estimation.py:391-403) for n byte counts. */
+int apc_rw_times(const apc_model* model, int32_t n, const double* nbytes, double* out,
+                 void* stream);
 
 /* Replaces _create_all_options + remove_invalid_configs for input/parameter
  * nodes (autoparallel/shardings/propagation_rules.py:127-158, 184-201): for

@@ -356,3 +356,129 @@ def test_full_size_properties(CostEngine):
             n = int(g.edge_sdst[e]) * int(g.edge_ssrc[e])
             assert bits_equal(a["comm"][b0:b0 + n], ref["comm"][b0:b0 + n])
             assert bits_equal(a["cost"][b0:b0 + n], ref["cost"][b0:b0 + n])
+
+
+# ---------------------------------------------------------------------------
+# scalar cost-model entry points in batch form
+# ---------------------------------------------------------------------------
+def _model(mesh, order_mode=0):
+    from autoparallel_amd.engine import make_model
+
+    return make_model(mesh, 8, "AMD Instinct MI355X", order_mode)
+
+
+def test_forward_order_mode_matches_redistribute_cost(CostEngine, golden):
+    """redistribute_cost(src, tgt, [0..ndim)) of the reference: order_mode 1."""
+    for k in (2, 3, 10):  # two 2-D cases (where the orders differ) and a 3-D one
+        mesh = [int(x) for x in golden[f"comm_{k}_mesh"]]
+        shape = [int(x) for x in golden[f"comm_{k}_shape"]]
+        stride = [int(x) for x in golden[f"comm_{k}_stride"]]
+        src, tgt, want = golden[f"comm_{k}_src"], golden[f"comm_{k}_tgt"], golden[f"comm_{k}_cost_fwd"]
+        src_t = sorted({tuple(int(x) for x in r) for r in src})
+        tgt_t = sorted({tuple(int(x) for x in r) for r in tgt})
+        g = graph_from_pairs(mesh, 8, shape, stride, int(golden[f"comm_{k}_itemsize"][0]), src_t, tgt_t)
+        for use_table in (True, False):
+            comm = CostEngine(g, use_table=use_table, order_mode=1).build(clamp_inf=False).results()["comm"]
+            base, ssrc = int(g.edge_off[1]), int(g.edge_ssrc[1])
+            si = {t: i for i, t in enumerate(src_t)}
+            ti = {t: i for i, t in enumerate(tgt_t)}
+            idx = np.asarray([base + ti[tuple(int(x) for x in t)] * ssrc + si[tuple(int(x) for x in s)]
+                              for s, t in zip(src, tgt)])
+            assert bits_equal(comm[idx], want), (k, use_table, first_mismatch(comm[idx], want))
+
+
+def test_batch_scalar_entry_points(CostEngine, golden):
+    import ctypes as C
+
+    from autoparallel_amd import _lib
+
+    lib = _lib.load()
+    d = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    # compute_read_write_time against the reference's values
+    for key_b, key_t in (("rw_bytes", "rw_time"), ("rw_fbytes", "rw_ftime")):
+        b = d(golden[key_b].astype(np.float64))
+        out = torch.empty_like(b)
+        m = _model((8, 8))
+        assert lib.apc_rw_times(C.byref(m), b.numel(), b.data_ptr(), out.data_ptr(), None) == 0
+        torch.cuda.synchronize()
+        assert bits_equal(out.cpu().numpy(), golden[key_t])
+    # _get_sharded_shape_stride against the reference's values
+    mesh = [int(x) for x in golden["shard_mesh"]]
+    n = golden["shard_rank"].shape[0]
+    pad8 = lambda a: np.concatenate([a, np.zeros((n, 8 - a.shape[1]), np.int64)], axis=1)
+    rank = d(golden["shard_rank"].astype(np.int32))
+    shape, stride = d(pad8(golden["shard_shape"])), d(pad8(golden["shard_stride"]))
+    plc = d(np.concatenate([golden["shard_plc"], np.zeros((n, 1), np.uint8)], axis=1))
+    o_shape, o_stride = torch.zeros_like(shape), torch.zeros_like(stride)
+    m = _model(mesh)
+    assert lib.apc_local_shapes(C.byref(m), n, rank.data_ptr(), shape.data_ptr(), stride.data_ptr(),
+                                plc.data_ptr(), o_shape.data_ptr(), o_stride.data_ptr(), None) == 0
+    torch.cuda.synchronize()
+    assert (o_shape.cpu().numpy()[:, :4] == golden["shard_out_shape"]).all()
+    assert (o_stride.cpu().numpy()[:, :4] == golden["shard_out_stride"]).all()
+    # collective_comm_cost against the oracle (itself checked against torch's functions)
+    rng = np.random.default_rng(5)
+    q = 500
+    kind = rng.integers(0, 5, q).astype(np.int32)
+    nbytes = rng.integers(0, 2**36, q).astype(np.int64)
+    dim = rng.integers(0, 3, q).astype(np.int32)
+    out = torch.empty(q, dtype=torch.float64, device="cuda")
+    mesh = (4, 8, 8)
+    m = _model(mesh)
+    tk, tb, td = d(kind), d(nbytes), d(dim)
+    assert lib.apc_collective_costs(C.byref(m), q, tk.data_ptr(), tb.data_ptr(), td.data_ptr(), out.data_ptr(), None) == 0
+    torch.cuda.synchronize()
+    topo = O.Topo(mesh, 8)
+    names = ["allgather", "all_to_all", "allreduce", "reduce_scatter", "unknown"]
+    want = np.asarray([O.collective_comm_cost(names[k], int(b), topo, int(dd)) for k, b, dd in zip(kind, nbytes, dim)])
+    assert bits_equal(out.cpu().numpy(), want)
+
+
+# ---------------------------------------------------------------------------
+# ILP: the plan from the HIP coefficients is the plan from the oracle's
+# ---------------------------------------------------------------------------
+def test_solved_plan_identical(CostEngine):
+    from autoparallel_amd.sharding_problem import Coefficients, PackedShardingOptimizer
+    from test_sharding_problem import oracle_coefficients
+
+    g = graphgen.gpt2_graph((4,), n_layers=1, dim=64, n_heads=2, ffn_dim=128, vocab=256, seq=32, batch=8)
+    gpu = PackedShardingOptimizer(g)
+    ref_coef, raw = oracle_coefficients(g)
+    assert bits_equal(gpu.coef.cost, ref_coef.cost) and bits_equal(gpu.coef.comm, ref_coef.comm)
+    assert (gpu.coef.flags == ref_coef.flags).all() and bits_equal(gpu.coef.per_arg, ref_coef.per_arg)
+    cpu = PackedShardingOptimizer(g, coefficients=ref_coef)
+    s_gpu, s_cpu = gpu.get_solution(), cpu.get_solution()
+    assert (s_gpu == s_cpu).all() and gpu.objective_value == cpu.objective_value
+    # the scorer on the device agrees with the oracle on the solved plan
+    got = gpu.compute_solution_cost(s_gpu)
+    want = O.score_assignment(g, raw["comm"], raw["transition"], raw["compute"], s_gpu)
+    assert (got["total"], got["compute"], got["comm"], got["transition"]) == tuple(float(x) for x in want)
+    # prefetch discount through the optimizer, then re-solve: never more expensive
+    base = gpu.objective_value
+    assert gpu.apply_prefetch_discount(0.0) > 0
+    gpu.get_solution()
+    assert gpu.objective_value <= base + 1e-9
+
+
+def test_memory_constraint(CostEngine):
+    from autoparallel_amd.sharding_problem import PackedShardingOptimizer
+
+    g = graphgen.gpt2_graph((4,), n_layers=1, dim=64, n_heads=2, ffn_dim=128, vocab=256, seq=32, batch=8)
+    opt = PackedShardingOptimizer(g)
+    params = [p for p, _ in g.roles.param_grad]
+    ratios = opt._memory_ratios(params)
+    for p, r in zip(params, ratios):
+        run = int(g.node_out_list[p])
+        for o in range(int(g.node_nstrat[p])):
+            w = int(g.lists[run + o])
+            rk = int(g.meta_rank[w >> 12])
+            shape = [int(x) for x in g.meta_shape[w >> 12, :rk]]
+            plc = [int(x) for x in g.tuple_plc[w & 0xFFF, : g.ndim]]
+            ls, _ = O.sharded_shape_stride(shape, [1] * rk, plc, [int(x) for x in g.mesh_shape])
+            assert r[o] == np.prod(ls) / np.prod(shape)
+    # parameters sharded as much as possible: every parameter at its smallest ratio
+    opt.add_parameter_memory_constraint(0.0, 0.0)
+    sol = opt.get_solution()
+    for p, r in zip(params, ratios):
+        assert r[sol[p]] == r.min()
+    assert "memory_constraint_high" in opt.prob.constraints

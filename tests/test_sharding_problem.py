@@ -1,0 +1,135 @@
+"""ILP assembly and solver hand-off on packed graphs.  Coefficients come from
+the oracle here (CPU); tests/test_gpu_parity.py checks that the HIP engine's
+coefficients, and therefore the solved plan, are identical."""
+import os
+
+import numpy as np
+import pytest
+
+from autoparallel_amd import graphgen, ilp
+from autoparallel_amd.sharding_problem import Coefficients, PackedShardingOptimizer
+from oracle import cost_oracle as O
+
+
+def oracle_coefficients(g):
+    r = O.GraphOracle(g).build()
+    cost, bad = O.clamp_inf(r["cost"])
+    flags = (r["transition"] | (bad << 1)).astype(np.uint8)
+    per_arg = np.zeros(g.num_compute)
+    for v in range(g.num_nodes):
+        o0 = int(g.node_comp_off[v])
+        per_arg[o0:o0 + int(g.node_nstrat[v])] = r["compute"][o0:o0 + int(g.node_nstrat[v])] / int(g.node_nargs[v])
+    return Coefficients(g, r["comm"], cost, flags, r["compute"], per_arg), r
+
+
+@pytest.fixture(scope="module")
+def tiny():
+    g = graphgen.gpt2_graph((4,), n_layers=1, dim=64, n_heads=2, ffn_dim=128, vocab=256, seq=32, batch=8)
+    coef, raw = oracle_coefficients(g)
+    return g, coef, raw
+
+
+def test_row_counts(tiny):
+    g, coef, _ = tiny
+    opt = PackedShardingOptimizer(g, coefficients=coef)
+    names = list(opt.prob.constraints)
+    count = lambda p: sum(1 for n in names if n.rsplit("_", 1)[0] == p)
+    assert count("unique_decision") == g.num_edges
+    multi = [v for v in range(g.num_nodes) if opt._num_input_nodes(v) > 1]
+    want = sum((int(g.node_edge_off[v + 1]) - int(g.node_edge_off[v]) - 1) * int(g.node_nstrat[v]) for v in multi)
+    assert count("same_across_args") == want
+    pairs = {(int(u), int(v)) for u, v in zip(g.edge_src_node, g.edge_node) if u >= 0}
+    assert count("output_input_consistent") == sum(int(g.node_nstrat[u]) for u, _ in pairs)
+    assert count("inf_cases") == int(((coef.flags >> 1) & 1).sum())
+    assert count("grad_param_constraint") + count("grad_param_constraint_disable") > 0
+    assert count("fwd_param_dtype") > 0  # fp32 master weights cast to bf16
+    assert names[0] == "unique_decision_000"
+
+
+def test_solution_is_feasible_and_consistent(tiny):
+    g, coef, raw = tiny
+    opt = PackedShardingOptimizer(g, coefficients=coef)
+    sol = opt.get_solution()
+    assert (sol >= 0).all() and (sol < g.node_nstrat).all()
+    assert opt.prob.violated() == []
+    # exactly one variable per (node, arg)
+    assert len(opt.selected) == g.num_edges
+    # flow: the selected inp_idx of every edge is the producer's out_idx
+    keys = g.entry_keys()[opt.selected]
+    for v, a, o, j in keys:
+        u = int(g.edge_src_node[opt.edge_of(v, a)])
+        if u >= 0:
+            assert sol[u] == j
+        assert sol[v] == o
+    # objective == sum of selected costs; no forbidden variable selected
+    assert np.isclose(opt.objective_value, coef.cost[opt.selected].sum())
+    assert ((coef.flags[opt.selected] >> 1) & 1).sum() == 0
+    # the ILP objective of this plan equals the oracle's evaluation of it
+    cost, bad = O.clamp_inf(raw["cost"])
+    obj, viol = O.ilp_objective(g, cost, bad, sol)
+    assert viol == 0 and np.isclose(obj, opt.objective_value, rtol=1e-12)
+    # forward/backward pairs agree on placement
+    plc = opt.solution_placements(sol)
+    for p, gr in g.roles.param_grad:
+        if gr >= 0:
+            assert plc[p] == plc[gr]
+
+
+def test_optimum_not_worse_than_samples(tiny):
+    g, coef, raw = tiny
+    opt = PackedShardingOptimizer(g, coefficients=coef)
+    sol = opt.get_solution()
+    cost, bad = O.clamp_inf(raw["cost"])
+    all_rep = np.zeros(g.num_nodes, np.int64)  # strategy 0 == replicate everywhere: feasible
+    obj_rep, viol = O.ilp_objective(g, cost, bad, all_rep)
+    assert viol == 0 and opt.objective_value <= obj_rep + 1e-9
+
+
+def test_node_constraint_and_resolve(tiny):
+    g, coef, _ = tiny
+    opt = PackedShardingOptimizer(g, coefficients=coef)
+    base = opt.get_solution()
+    base_obj = opt.objective_value
+    tok = g.node_names.index("tokens")
+    names = opt.add_node_constraint(tok, (0x40,))  # Shard(0) on the batch
+    sol = opt.resolve()
+    assert opt.solution_placements(sol)[tok] == ("S(0)",)
+    assert opt.objective_value >= base_obj - 1e-9
+    opt.remove_constraints(names)
+    again = opt.resolve()
+    assert np.isclose(opt.objective_value, base_obj)
+    with pytest.raises(RuntimeError):
+        opt.add_node_constraint(tok, (0x47,))  # Shard(7) does not exist
+
+
+def test_infeasible_raises(tiny):
+    g, coef, _ = tiny
+    opt = PackedShardingOptimizer(g, coefficients=coef)
+    tok = g.node_names.index("tokens")
+    opt.add_node_constraint(tok, (0x40,))
+    opt.add_node_constraint(tok, (0x00,))
+    with pytest.raises(RuntimeError):
+        opt.get_solution()
+
+
+def test_lp_file(tiny, tmp_path):
+    g, coef, _ = tiny
+    opt = PackedShardingOptimizer(g, coefficients=coef)
+    opt._set_objective()
+    path = os.path.join(tmp_path, "model.lp")
+    opt.prob.write_lp(path, opt.var_names())
+    text = open(path).read()
+    assert text.startswith("\\* AutoParallel *\\") and "unique_decision_000:" in text and "Binaries" in text
+    assert "n_tokens_s_" in text  # reference variable naming, sanitised for the LP format
+
+
+def test_sparse_ilp_basics():
+    p = ilp.SparseILP(3)
+    p.objective = np.asarray([1.0, 2.0, 3.0])
+    p.add_row("pick", [0, 1, 2], 1.0, ilp.EQ, 1.0)
+    p.add_row("ban", [0], 1.0, ilp.EQ, 0.0)
+    assert p.solve() == ilp.STATUS_OPTIMAL and list(p.x) == [0, 1, 0]
+    p.add_row("ban", [1], 1.0, ilp.EQ, 0.0)
+    p.add_row("ban", [2], 1.0, ilp.EQ, 0.0)
+    assert p.solve() == ilp.STATUS_INFEASIBLE
+    assert list(p.constraints) == ["pick_000", "ban_000", "ban_001", "ban_002"]
