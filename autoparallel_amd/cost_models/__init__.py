@@ -1,0 +1,14 @@
+from .collective_runtime_estimation import (  # noqa: F401
+    collective_comm_cost,
+    configure,
+    estimate_strategy_comms_cost,
+    get_nccl_topo_config,
+    redistribute_cost,
+    reset_comms_cost_cache,
+    set_nccl_topo_config,
+)
+from .compute_estimation import (  # noqa: F401
+    compute_read_write_time,
+    estimate_strategy_runtime_cost,
+    reset_compute_cost_cache,
+)

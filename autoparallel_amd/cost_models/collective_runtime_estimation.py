@@ -1,0 +1,134 @@
+"""The reference's ``autoparallel.cost_models.collective_runtime_estimation``
+interface on top of the HIP engine (same names, arguments and return values;
+autoparallel/cost_models/collective_runtime_estimation.py:34-41, 65-110,
+115-229, 235-262).  Every number is computed on the device through the C ABI:
+a single query is a batch of one."""
+from __future__ import annotations
+
+import ctypes as C
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import numpy as np
+import torch
+
+from .. import _lib
+from ..dtensor_bridge import devices_per_host, placement_codes, tensor_meta_key
+from ..engine import CostEngine, detect_device_name, make_model
+from ..packed import GraphBuilder, NodeDesc
+
+_nccl_topo_config = None
+_comms_cost_cache: Dict[tuple, float] = {}
+_settings = {"devices_per_host": None, "device_name": None}
+
+_COLLECTIVES = {"allgather": 0, "all_to_all": 1, "allreduce": 2, "reduce_scatter": 3}
+
+
+def configure(devices_per_host: Optional[int] = None, device_name: Optional[str] = None) -> None:
+    """Pin the two host-dependent inputs of the model (the reference reads
+    them from the planning host: device count per host and device name)."""
+    _settings["devices_per_host"] = devices_per_host
+    _settings["device_name"] = device_name
+    _comms_cost_cache.clear()
+
+
+def _dph(mesh) -> int:
+    return _settings["devices_per_host"] if _settings["devices_per_host"] is not None else devices_per_host(mesh)
+
+
+def _device_name() -> str:
+    return _settings["device_name"] or detect_device_name()
+
+
+def set_nccl_topo_config(config) -> None:
+    global _nccl_topo_config
+    if config is not None:
+        raise NotImplementedError(
+            "the NCCL cost model is not built yet; the default (alpha-beta) model is what the "
+            "reference itself selects on MI355X")
+    _nccl_topo_config = config
+    _comms_cost_cache.clear()
+
+
+def get_nccl_topo_config():
+    return _nccl_topo_config
+
+
+def reset_comms_cost_cache() -> None:
+    _comms_cost_cache.clear()
+
+
+def comms_cost_matrix(src_specs: Sequence, tgt_specs: Sequence, order_mode: int = 0) -> np.ndarray:
+    """cost[t][s] of redistributing src_specs[s] into the placements of
+    tgt_specs[t] (all on one mesh): one edge block on the device."""
+    mesh = src_specs[0].mesh
+    b = GraphBuilder(tuple(mesh.shape), _dph(mesh))
+    src_words = [b.spec(b.meta(*tensor_meta_key(s.tensor_meta)), placement_codes(s.placements)) for s in src_specs]
+    tgt_words = [b.spec(b.meta(*tensor_meta_key(t.tensor_meta)), placement_codes(t.placements)) for t in tgt_specs]
+    b.add_node(NodeDesc("src", in_specs=[[w] for w in src_words], out_specs=[[w] for w in src_words],
+                        inputs=[], default_rows=[[[0.0]] for _ in src_words]))
+    b.add_node(NodeDesc("tgt", in_specs=[[w] for w in tgt_words], out_specs=[[w] for w in tgt_words], inputs=[0]))
+    g = b.pack()
+    eng = CostEngine(g, device_name=_device_name(), use_table=False, order_mode=order_mode)
+    eng.build(clamp_inf=False)
+    comm = eng.results()["comm"]
+    base = int(g.edge_off[1])
+    return comm[base : base + len(tgt_words) * len(src_words)].reshape(len(tgt_words), len(src_words))
+
+
+def redistribute_cost(current_spec, target_spec, order: List[int]) -> float:
+    if current_spec.mesh != target_spec.mesh:
+        return float("inf")
+    ndim = current_spec.mesh.ndim
+    if list(order) == list(range(ndim)):
+        mode = 1
+    elif list(order) == list(reversed(range(ndim))):
+        mode = 2
+    else:
+        raise NotImplementedError(f"mesh-dim order {order}: only ascending and descending orders are built")
+    return float(comms_cost_matrix([current_spec], [target_spec], order_mode=mode)[0, 0])
+
+
+def estimate_strategy_comms_cost(src_spec, tgt_spec) -> float:
+    key = (src_spec.placements, src_spec.tensor_meta, tgt_spec.placements, tgt_spec.tensor_meta,
+           tuple(src_spec.mesh.shape))
+    try:
+        hash(key)
+    except TypeError:
+        key = None
+    if key is not None:
+        cached = _comms_cost_cache.get(key)
+        if cached is not None:
+            return cached
+    if src_spec.mesh != tgt_spec.mesh:
+        cost = float("inf")
+    else:
+        cost = float(comms_cost_matrix([src_spec], [tgt_spec], order_mode=0)[0, 0])
+    if key is not None:
+        _comms_cost_cache[key] = cost
+    return cost
+
+
+def collective_comm_cost(collective: str, comm_bytes: int, mesh_shape: Tuple[int, ...], mesh_dim: int,
+                         mesh_topo=None, devices_per_host: Optional[int] = None) -> float:
+    """Cost in microseconds of one collective on one mesh dim.  ``mesh_topo``
+    (a torch MeshTopoInfo) supplies per-dim bandwidth/latency when given;
+    otherwise they are derived from ``devices_per_host``."""
+    lib = _lib.load()
+    dph = devices_per_host if devices_per_host is not None else (_settings["devices_per_host"] or 1)
+    model = make_model(tuple(mesh_shape), dph, _device_name())
+    if mesh_topo is not None:
+        for i in range(len(mesh_shape)):
+            model.mesh_bw[i] = float(mesh_topo.mesh_dim_bandwidth[i])
+            model.mesh_lat[i] = float(mesh_topo.mesh_dim_latency[i])
+    kind = torch.tensor([_COLLECTIVES.get(collective, -1)], dtype=torch.int32, device="cuda")
+    nb = torch.tensor([int(comm_bytes)], dtype=torch.int64, device="cuda")
+    dim = torch.tensor([int(mesh_dim)], dtype=torch.int32, device="cuda")
+    out = torch.empty(1, dtype=torch.float64, device="cuda")
+    _lib.check(lib.apc_collective_costs(C.byref(model), 1, kind.data_ptr(), nb.data_ptr(), dim.data_ptr(),
+                                        out.data_ptr(), None), "apc_collective_costs")
+    return float(out.item())
+
+
+def all_to_all_cost(bytes_gb: float, mesh_topo, mesh_dim: int) -> float:
+    shape = tuple(mesh_topo.mesh_dim_devices)
+    return collective_comm_cost("all_to_all", int(bytes_gb * 1024**3), shape, mesh_dim, mesh_topo)

@@ -1,0 +1,210 @@
+"""From an FX node to what the node kernel consumes: spec words of its tensor
+arguments per strategy and either a compute program (closed form) or explicit
+(flops, bytes) per strategy.
+
+The reference gets flops and bytes by running the op on sharded FakeTensors
+under ``FlopCounterMode`` for every distinct (op, input specs) key
+(autoparallel/cost_models/compute_estimation.py:334-365, 383-388, 469-473).
+Ops with a closed form here are priced on the device from a program; any other
+op takes the reference's route (meta tensors + FlopCounterMode, torch code) on
+the host to obtain the two integers, and is counted in ``fallback_ops`` so a
+caller can see which ops lack a closed form.  The roofline arithmetic itself
+always runs on the device.
+"""
+from __future__ import annotations
+
+import collections
+import ctypes as C
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import numpy as np
+import torch
+from torch.utils._pytree import tree_flatten
+
+from . import _lib, opprog
+from .dtensor_bridge import placement_codes, tensor_meta_key
+from .packed import OP_EXPLICIT, OP_PROGRAM, OP_ZERO, GraphBuilder, NodeDesc
+
+aten = torch.ops.aten
+fallback_ops: "collections.Counter[str]" = collections.Counter()
+
+
+def non_tensor_args_key(node) -> tuple:
+    def h(x):
+        if isinstance(x, (list, tuple)):
+            return tuple(h(a) for a in x)
+        if isinstance(x, torch.Tensor):
+            return (tuple(x.shape), tuple(x.stride()), x.dtype)
+        return x
+
+    return tuple(h(a) for a in tree_flatten(node.args)[0] if not isinstance(a, torch.fx.Node))
+
+
+def _tensor_arg_vals(node) -> List[torch.Tensor]:
+    vals = []
+    for a in tree_flatten(node.args)[0]:
+        if isinstance(a, torch.fx.Node) and isinstance(a.meta.get("val"), torch.Tensor):
+            vals.append(a.meta["val"])
+    return vals
+
+
+def _out_tensors(node) -> List[torch.Tensor]:
+    return [x for x in tree_flatten(node.meta.get("val"))[0] if isinstance(x, torch.Tensor)]
+
+
+def _closed_form(node) -> Optional[List[int]]:
+    """Compute program of the node's op, or None if there is no closed form."""
+    t = node.target
+    ins = _tensor_arg_vals(node)
+    outs = _out_tensors(node)
+    if not outs or not ins:
+        return None
+    o0 = outs[0]
+    osz = o0.element_size()
+    if t in (aten.mm.default,):
+        return opprog.mm(osz)
+    if t in (aten.addmm.default,) and len(ins) == 3:
+        return opprog.addmm(osz)
+    if t in (aten.bmm.default,):
+        return opprog.bmm(osz)
+    if t is aten.einsum.default and len(ins) == 2:
+        a, b = ins
+        if b.dim() == 2 and a.dim() >= 3:
+            return opprog.einsum_fwd(a.dim(), osz)
+        if a.dim() == b.dim() and a.dim() >= 3:
+            return opprog.einsum_bwd(a.dim(), osz)
+        return None
+    if t is aten._scaled_dot_product_flash_attention.default and len(ins) == 3:
+        return opprog.sdpa_flash_fwd(ins[0].element_size())
+    if t is aten._scaled_dot_product_flash_attention_backward.default and len(ins) >= 6:
+        return opprog.sdpa_flash_bwd(ins[1].element_size())
+    if t in (aten.sum.dim_IntList, aten.mean.dim) and len(ins) == 1:
+        dims = node.args[1] if len(node.args) > 1 else None
+        keep = bool(node.args[2]) if len(node.args) > 2 else bool(node.kwargs.get("keepdim", False))
+        if dims is None or len(dims) == 0:
+            dims = list(range(ins[0].dim()))
+        if ins[0].dim() == 0:
+            return None
+        return opprog.reduction(ins[0].dim(), list(dims), keep, osz)
+    if t in (aten._softmax.default, aten._log_softmax.default, aten.clone.default, aten._to_copy.default) and len(ins) == 1:
+        return opprog.same_as_arg(0, ins[0].dim(), osz)
+    if t in (aten._softmax_backward_data.default, aten._log_softmax_backward_data.default) and len(ins) == 2:
+        return opprog.same_as_arg(0, ins[0].dim(), osz)
+    if t is aten.embedding.default and len(ins) == 2:
+        return opprog.embedding(ins[1].dim(), osz)
+    if torch.Tag.pointwise in t.tags and len(outs) == 1:
+        # elementwise with broadcasting; the output shape is the broadcast of
+        # the tensor arguments only if no argument is shape-expanding by itself
+        if tuple(torch.broadcast_shapes(*[tuple(i.shape) for i in ins])) == tuple(o0.shape):
+            return opprog.pointwise(o0.dim(), osz)
+    return None
+
+
+def local_shapes(specs: Sequence) -> List[Tuple[List[int], List[int]]]:
+    """_get_sharded_shape_stride for a batch of DTensorSpecs, on the device."""
+    from .engine import make_model
+    from .cost_models.collective_runtime_estimation import _device_name
+
+    if not specs:
+        return []
+    lib = _lib.load()
+    n = len(specs)
+    rank = np.zeros(n, np.int32)
+    shape = np.ones((n, 8), np.int64)
+    stride = np.zeros((n, 8), np.int64)
+    plc = np.zeros((n, 4), np.uint8)
+    for i, s in enumerate(specs):
+        sh, st, _, _ = tensor_meta_key(s.tensor_meta)
+        rank[i] = len(sh)
+        shape[i, : len(sh)] = sh
+        stride[i, : len(st)] = st
+        codes = placement_codes(s.placements)
+        plc[i, : len(codes)] = codes
+    d = lambda a: torch.from_numpy(a).cuda()
+    t_rank, t_shape, t_stride, t_plc = d(rank), d(shape), d(stride), d(plc)
+    o_shape, o_stride = torch.empty_like(t_shape), torch.empty_like(t_stride)
+    m = make_model(tuple(specs[0].mesh.shape), 1, _device_name())
+    _lib.check(lib.apc_local_shapes(C.byref(m), n, t_rank.data_ptr(), t_shape.data_ptr(), t_stride.data_ptr(),
+                                    t_plc.data_ptr(), o_shape.data_ptr(), o_stride.data_ptr(), None),
+               "apc_local_shapes")
+    osh, ost = o_shape.cpu().numpy(), o_stride.cpu().numpy()
+    return [([int(x) for x in osh[i, : rank[i]]], [int(x) for x in ost[i, : rank[i]]]) for i in range(n)]
+
+
+def _flops_bytes_via_torch(node, strategies) -> Tuple[List[int], List[int]]:
+    """The reference's own route for ops without a closed form: run the op on
+    meta tensors of the sharded sizes under FlopCounterMode (torch code)."""
+    from torch.utils.flop_counter import FlopCounterMode
+
+    flat_specs = [s for st in strategies for s in st.input_specs if s is not None]
+    shapes = iter(local_shapes(flat_specs))
+    flops_all, bytes_all = [], []
+    flat_args, treespec = tree_flatten(node.args)
+    kwargs = {k: (v.meta["val"] if isinstance(v, torch.fx.Node) else v) for k, v in node.kwargs.items()}
+    for st in strategies:
+        new_flat, counter = [], 0
+        for a in flat_args:
+            if isinstance(a, torch.fx.Node):
+                a = a.meta["val"]
+                if isinstance(a, torch.Tensor):
+                    spec = st.input_specs[counter]
+                    counter += 1
+                    if spec is not None:
+                        sizes, strides = next(shapes)
+                        a = torch.empty_strided(sizes, strides, dtype=a.dtype, device="meta")
+                    else:
+                        a = torch.empty_strided(a.shape, a.stride(), dtype=a.dtype, device="meta")
+            new_flat.append(a)
+        args = treespec.unflatten(new_flat)
+        with FlopCounterMode(display=False) as fc:
+            out = node.target(*args, **kwargs)
+        nbytes = sum(x.numel() * x.element_size() for x in tree_flatten(args)[0] if isinstance(x, torch.Tensor))
+        nbytes += sum(x.numel() * x.element_size() for x in tree_flatten(out)[0] if isinstance(x, torch.Tensor))
+        flops_all.append(int(fc.get_total_flops()))
+        bytes_all.append(int(nbytes))
+    return flops_all, bytes_all
+
+
+def describe_node(node, strategies, b: GraphBuilder, name: Optional[str] = None) -> NodeDesc:
+    """NodeDesc (without producers) of an FX node with the given OpSpecs."""
+    in_specs, out_specs = [], []
+    for st in strategies:
+        row = []
+        for s in (st.input_specs or []):
+            if s is None or s.tensor_meta is None:
+                row.append(-1)
+            else:
+                row.append(b.spec(b.meta(*tensor_meta_key(s.tensor_meta)), placement_codes(s.placements)))
+        in_specs.append(row)
+        outs = st.output_specs
+        outs = list(outs) if isinstance(outs, (tuple, list)) else [outs]
+        orow = []
+        for s in outs:
+            if s is None or s.tensor_meta is None:
+                orow.append(-1)
+            else:
+                orow.append(b.spec(b.meta(*tensor_meta_key(s.tensor_meta)), placement_codes(s.placements)))
+        out_specs.append(orow)
+    tuple_output = isinstance(strategies[0].output_specs, (tuple, list))
+    desc = NodeDesc(name or str(node.name), in_specs=in_specs, out_specs=out_specs, inputs=[],
+                    tuple_output=tuple_output)
+    # aten._unsafe_view is a reshape that the dispatcher does not tag as a view;
+    # run with its global size list on a sharded input it cannot execute at all
+    # (the reference rewrites the view-mm-view pattern that produces it away,
+    # autoparallel/graph_passes/graph_utils.py:415-439), so it is priced as the
+    # view it is.
+    zero = (node.op != "call_function" or not isinstance(node.target, torch._ops.OpOverload)
+            or node.target.is_view or node.target is aten._unsafe_view.default)
+    if zero:
+        desc.op = OP_ZERO
+        return desc
+    prog = _closed_form(node)
+    n_tensor_specs = len(in_specs[0])
+    if prog is not None and len(_tensor_arg_vals(node)) == n_tensor_specs and all(w >= 0 for r in in_specs for w in r):
+        desc.op = OP_PROGRAM
+        desc.program = prog
+        return desc
+    fallback_ops[str(node.target)] += 1
+    desc.op = OP_EXPLICIT
+    desc.flops, desc.nbytes = _flops_bytes_via_torch(node, strategies)
+    return desc

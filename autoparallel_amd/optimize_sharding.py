@@ -1,0 +1,383 @@
+"""``ShardingOptimizer`` with the reference's constructor and public surface
+(autoparallel/optimize_sharding.py:220-291, 955-979 and the constraint adders),
+over the HIP cost engine.
+
+What happens where:
+  * strategies per node: host, torch DTensor (``shardings.placement_options``)
+  * packing of ``{node: OpStrategy}`` into SoA arrays: host (``_pack``)
+  * every coefficient (compute, comm, transition, cost, inf flags): device
+  * ILP rows and the solver hand-off: ``sharding_problem`` / ``ilp``
+``decision_vars`` is a mapping view over the coefficient arrays in the
+reference's insertion order (node, out_idx, argi, inp_idx; :511-520).
+"""
+from __future__ import annotations
+
+import collections.abc
+import logging
+import operator
+import warnings
+from typing import Any, Dict, Iterator, List, Optional, Tuple
+
+import numpy as np
+import torch
+from torch.distributed.tensor._dtensor_spec import DTensorSpec
+from torch.distributed.tensor._op_schema import OpSpec, OpStrategy
+from torch.distributed.tensor.placement_types import Replicate, Shard
+from torch.utils._pytree import tree_flatten, tree_map_only
+
+from . import fx_programs
+from .cost_models import collective_runtime_estimation as _cre
+from .dtensor_bridge import devices_per_host as _mesh_dph
+from .dtensor_bridge import placement_codes
+from .engine import detect_device_name
+from .packed import GraphBuilder, NodeDesc, PackedGraph
+from .sharding_problem import GraphRoles, PackedShardingOptimizer
+from .shardings.placement_options import _create_all_options, get_placement_options_for_node
+
+logger = logging.getLogger(__name__)
+
+
+def _produces_tensor(val) -> bool:
+    if isinstance(val, torch.Tensor):
+        return True
+    if isinstance(val, (tuple, list)):
+        return any(_produces_tensor(v) for v in val)
+    return False
+
+
+class DecisionVar:
+    """One (node, arg, out, inp) choice; attribute reads and writes go to the
+    coefficient arrays (fields of the reference's dataclass, :191-203)."""
+
+    __slots__ = ("_opt", "_i", "key")
+
+    def __init__(self, opt: "ShardingOptimizer", i: int, key: tuple):
+        self._opt, self._i, self.key = opt, i, key
+
+    @property
+    def var(self) -> int:
+        return self._i  # column of the ILP
+
+    @property
+    def cost(self) -> float:
+        return float(self._opt._core.coef.cost[self._i])
+
+    @cost.setter
+    def cost(self, v: float) -> None:
+        self._opt._core.coef.cost[self._i] = v
+
+    @property
+    def comm_cost(self) -> float:
+        return float(self._opt._core.coef.comm[self._i])
+
+    @comm_cost.setter
+    def comm_cost(self, v: float) -> None:
+        self._opt._core.coef.comm[self._i] = v
+
+    @property
+    def sharding_transition_cost(self) -> int:
+        return int(self._opt._core.coef.flags[self._i] & 1)
+
+    @property
+    def compute_cost(self) -> float:
+        v, _, o, _ = self.key
+        return float(self._opt._core.coef.per_arg[int(self._opt._packed.node_comp_off[v]) + o])
+
+    @property
+    def strategy(self) -> OpSpec:
+        v, _, o, _ = self.key
+        return self._opt.strats[self._opt.nodes[v]].strategies[o]
+
+    @property
+    def output_spec(self):
+        return self.strategy.output_specs
+
+    @property
+    def input_spec(self):
+        ins = self.strategy.input_specs
+        a = self.key[1]
+        return ins[a] if ins is not None and a < len(ins) else None
+
+    def value(self) -> Optional[float]:
+        x = self._opt._core.prob.x
+        return None if x is None else float(x[self._i])
+
+
+class DecisionVars(collections.abc.Mapping):
+    def __init__(self, opt: "ShardingOptimizer"):
+        self._opt = opt
+        g = opt._packed
+        self._keys = g.entry_keys()
+        self._order = g.decision_var_order()
+        self._index: Optional[Dict[tuple, int]] = None
+
+    def _col(self, key) -> int:
+        v, a, o, j = key
+        try:
+            return self._opt._core.var(int(v), int(a), int(o), int(j))
+        except AssertionError:
+            raise KeyError(key)
+
+    def __getitem__(self, key) -> DecisionVar:
+        g = self._opt._packed
+        v, a, o, j = key
+        if not (0 <= v < g.num_nodes) or not (0 <= o < g.node_nstrat[v]):
+            raise KeyError(key)
+        e = int(g.node_edge_off[v]) + a
+        if a < 0 or e >= int(g.node_edge_off[v + 1]) or not (0 <= j < g.edge_ssrc[e]):
+            raise KeyError(key)
+        return DecisionVar(self._opt, self._col(key), (int(v), int(a), int(o), int(j)))
+
+    def __iter__(self) -> Iterator[tuple]:
+        for i in self._order:
+            yield tuple(int(x) for x in self._keys[i])
+
+    def __len__(self) -> int:
+        return self._keys.shape[0]
+
+
+class ShardingOptimizer:
+    def __init__(self, gm, mesh, force_grad_reduce_in_higher_precision: bool = False,
+                 repeated_subgraphs: bool = False, devices_per_host: Optional[int] = None,
+                 device_name: Optional[str] = None):
+        self.orig_gm = gm
+        self.gm = gm
+        self.graph = gm.graph
+        self.mesh = mesh
+        self.force_grad_reduce_in_higher_precision = force_grad_reduce_in_higher_precision
+        if repeated_subgraphs:
+            warnings.warn("repeated_subgraphs: clustering is not built; every node is priced "
+                          "(same plan, no variable sharing)")
+        self.cluster_links: Dict[tuple, tuple] = {}
+        self._devices_per_host = devices_per_host if devices_per_host is not None else _mesh_dph(mesh)
+        self._device_name = device_name or detect_device_name()
+        _cre.configure(self._devices_per_host, self._device_name)
+        self._constraint_log: List[Tuple[str, dict]] = []
+        self.strats = self.build_sharding_metadata()
+        self.nodes = list(self.strats.keys())
+        self.node_map = {n: i for i, n in enumerate(self.nodes)}
+        self.decision_vars = self._build_decision_vars()
+        self.validate()
+
+    # -- strategies ---------------------------------------------------------------
+    def build_sharding_metadata(self) -> Dict[torch.fx.Node, Any]:
+        strats: Dict[torch.fx.Node, Any] = {}
+        for node in self.graph.nodes:
+            if node.op in ("placeholder", "get_attr"):
+                val = node.meta.get("val")
+                if isinstance(val, torch.Tensor):
+                    strats[node] = _create_all_options(self.mesh, val.shape, tensor=val)
+                elif node.op == "placeholder":
+                    strats[node] = _create_all_options(self.mesh, ())
+            elif node.op == "call_function":
+                if not _produces_tensor(node.meta.get("val")):
+                    continue
+                in_nodes = [x for x in tree_flatten(node.args)[0]
+                            if isinstance(x, torch.fx.Node) and x in strats]
+                producers = [strats[x] for x in in_nodes]
+                arg_vals = [x.meta["val"] for x in in_nodes]
+                schema_args = tree_map_only(torch.fx.Node, lambda x: strats.get(x, x.meta.get("val")), node.args)
+                strats[node] = get_placement_options_for_node(self.mesh, node, producers, arg_vals, schema_args)
+            elif node.op == "output":
+                strats[node] = tree_map_only(torch.fx.Node, lambda x: strats[x], node.args)
+            else:
+                raise ValueError(f"Unexpected node op: {node.op}")
+        return strats
+
+    def _all_input_nodes(self, node) -> List[torch.fx.Node]:
+        return [x for x in tree_flatten(node.args)[0] if isinstance(x, torch.fx.Node) and x in self.strats]
+
+    def walk_over_options(self, node, constrain_arg=None):
+        if node not in self.strats or node.op == "output":
+            return
+        st = self.strats[node]
+        for argi in range(len(st.strategies[0].input_specs)):
+            if constrain_arg is not None and argi != constrain_arg:
+                continue
+            for out_idx, s in enumerate(st.strategies):
+                for inp_idx in range(len(s.redistribute_cost[argi])):
+                    yield argi, out_idx, inp_idx
+
+    # -- packing -------------------------------------------------------------------
+    def _roles(self) -> GraphRoles:
+        from torch._functorch._aot_autograd import fx_utils
+
+        r = GraphRoles()
+        nm = self.node_map
+        try:
+            for p, g in fx_utils.get_param_and_grad_nodes(self.graph).values():
+                r.param_grad.append((nm[p], nm[g] if g is not None and g in nm else -1))
+            for n, g in fx_utils.get_plain_input_and_grad_nodes(self.graph).values():
+                r.input_grad.append((nm[n], nm[g] if g is not None and g in nm else -1))
+            for n, t in fx_utils.get_plain_output_and_tangent_nodes(self.graph).values():
+                r.output_tangent.append((nm[n], nm[t] if t is not None and t in nm else -1))
+        except Exception:  # a graph without AOT descriptors has no forward/backward pairs
+            logger.debug("no AOT descriptors on the graph: no forward/backward constraints")
+        return r
+
+    def _prefetchable(self, roles: GraphRoles) -> set:
+        """(node_idx, argi) of edges whose producer is parameter-derived or whose
+        consumer is terminal-derived (autoparallel/graph_passes/graph_utils.py:447-484)."""
+        params = {self.nodes[p] for p, _ in roles.param_grad}
+        derived = set(params)
+        for node in self.graph.nodes:
+            ins = node.all_input_nodes
+            if ins and all(i in derived for i in ins):
+                derived.add(node)
+        terminal = {self.nodes[g] for _, g in roles.param_grad if g >= 0}
+        for node in reversed(list(self.graph.nodes)):
+            if node.op == "output":
+                continue
+            if node.users and all(u in terminal for u in node.users):
+                terminal.add(node)
+        out = set()
+        for node in self.nodes:
+            if node.op == "output":
+                continue
+            for a, prod in enumerate(self._all_input_nodes(node)):
+                if prod in derived or node in terminal:
+                    out.add((self.node_map[node], a))
+        return out
+
+    def _pack(self) -> PackedGraph:
+        b = GraphBuilder(tuple(self.mesh.shape), self._devices_per_host)
+        index_of: Dict[torch.fx.Node, int] = {}
+        self._packed_index: Dict[int, int] = {}  # node_idx -> packed node
+        for node in self.nodes:
+            if node.op == "output":
+                continue
+            st: OpStrategy = self.strats[node]
+            desc = fx_programs.describe_node(node, st.strategies, b, name=node.name)
+            ins = self._all_input_nodes(node)
+            desc.inputs = [index_of[x] for x in ins]
+            if node.op == "call_function" and node.target is operator.getitem:
+                desc.getitem_index = int(node.args[1])
+            # default rows: what the strategy carried before the engine ran
+            desc.default_rows = [[list(map(float, row)) for row in s.redistribute_cost] for s in st.strategies]
+            desc.nargs = len(st.strategies[0].input_specs)
+            index_of[node] = b.add_node(desc)
+            self._packed_index[self.node_map[node]] = index_of[node]
+        assert all(self._packed_index[i] == i for i in self._packed_index), "node order must be preserved"
+        roles = self._roles()
+        b.prefetchable_edges = self._prefetchable(roles)
+        g = b.pack()
+        g.roles = roles
+        return g
+
+    # -- coefficients ----------------------------------------------------------------
+    def _build_decision_vars(self) -> DecisionVars:
+        self._packed = self._pack()
+        self._core = PackedShardingOptimizer(
+            self._packed, roles=self._packed.roles,
+            force_grad_reduce_in_higher_precision=self.force_grad_reduce_in_higher_precision,
+            device_name=self._device_name)
+        self.prob = self._core.prob
+        self._write_back_redistribute_costs()
+        return DecisionVars(self)
+
+    def _write_back_redistribute_costs(self) -> None:
+        """strategy.redistribute_cost[argi][inp_idx] = comm, as the reference's
+        loop does in place (:540)."""
+        g, comm = self._packed, self._core.coef.comm
+        vs = self._core.var_start
+        for e in range(g.num_edges):
+            node = self.nodes[int(g.edge_node[e])]
+            a, ssrc = int(g.edge_arg[e]), int(g.edge_ssrc[e])
+            block = comm[vs[e] : vs[e + 1]].reshape(-1, ssrc).tolist()
+            for s, row in zip(self.strats[node].strategies, block):
+                s.redistribute_cost[a] = row
+
+    def validate(self) -> None:
+        for node in self.graph.nodes:
+            if node.op != "call_function" or node not in self.strats:
+                continue
+            s0 = self.strats[node].strategies[0]
+            ins = self._all_input_nodes(node)
+            assert len(s0.redistribute_cost) == len(ins) or (len(ins) == 0 and len(s0.redistribute_cost) == 1), \
+                f"{node}, {len(s0.redistribute_cost)}, {len(ins)}"
+            for i, arg in enumerate(ins):
+                assert len(s0.redistribute_cost[i]) == len(self.strats[arg].strategies), f"{node} arg {i}"
+
+    # -- constraints (delegated to the packed formulation) ------------------------------
+    def add_node_constraint(self, node, placement=None, constraint_name=None):
+        self._constraint_log.append(("add_node_constraint", {"node_name": node.name, "placement": placement,
+                                                             "constraint_name": constraint_name}))
+        assert node in self.strats, node
+        codes = None if placement is None else placement_codes(placement)
+        return self._core.add_node_constraint(self.node_map[node], codes, constraint_name)
+
+    def add_sharded_input_constraint(self, input_placements=None):
+        self._io_constraints(self._packed.roles.input_grad, input_placements, "input_constraint")
+
+    def add_sharded_output_constraint(self, output_placements=None):
+        self._io_constraints(self._packed.roles.output_tangent, output_placements, "output_constraint")
+
+    def _io_constraints(self, pairs, placements, name):
+        remaining = None if placements is None else dict(enumerate(placements))
+        for i, (n, _) in enumerate(pairs):
+            plc = None if remaining is None else remaining.pop(i)
+            codes = None if plc is None else placement_codes(plc)
+            self._core.add_node_constraint(n, codes, name)
+        if remaining and any(p is not None for p in remaining.values()):
+            raise RuntimeError(f"We were unable to respect placements at indices "
+                               f"{[i for i, p in remaining.items() if p is not None]}")
+
+    def add_parameter_memory_constraint(self, memory_factor_low: float, memory_factor_high: float):
+        self._core.add_parameter_memory_constraint(memory_factor_low, memory_factor_high)
+
+    def remove_constraints(self, names):
+        self._core.remove_constraints(names)
+
+    def apply_prefetch_discount(self, scale: float = 0.0) -> int:
+        n = self._core.apply_prefetch_discount(scale)
+        self._write_back_redistribute_costs()
+        return n
+
+    # -- solve ------------------------------------------------------------------------------
+    def _solution_dict(self, sol: np.ndarray) -> Dict[torch.fx.Node, OpSpec]:
+        self.selected_keys = [tuple(int(x) for x in k) for k in self._packed.entry_keys()[self._core.selected]]
+        return {self.nodes[v]: self.strats[self.nodes[v]].strategies[int(sol[v])]
+                for v in range(self._packed.num_nodes)}
+
+    def get_solution(self, verbose: bool = False) -> Dict[torch.fx.Node, OpSpec]:
+        return self._solution_dict(self._core.get_solution(verbose=verbose))
+
+    def resolve(self, verbose: bool = False) -> Dict[torch.fx.Node, OpSpec]:
+        return self._solution_dict(self._core.resolve(verbose=verbose))
+
+    def _out_indices(self, solution: Dict[torch.fx.Node, OpSpec]) -> np.ndarray:
+        sol = np.zeros(self._packed.num_nodes, np.int64)
+        for node, spec in solution.items():
+            if node not in self.node_map or node.op == "output":
+                continue
+            for i, s in enumerate(self.strats[node].strategies):
+                if s is spec:
+                    sol[self.node_map[node]] = i
+                    break
+        return sol
+
+    def _compute_solution_cost(self, solution: Dict[torch.fx.Node, OpSpec]) -> Dict[str, float]:
+        return self._core.compute_solution_cost(self._out_indices(solution))
+
+    def diff_solutions(self, solution_a, solution_b) -> str:
+        a, b = self._compute_solution_cost(solution_a), self._compute_solution_cost(solution_b)
+        changed = sum(1 for n in solution_a if n in solution_b
+                      and isinstance(solution_a[n].output_specs, DTensorSpec)
+                      and isinstance(solution_b[n].output_specs, DTensorSpec)
+                      and solution_a[n].output_specs.placements != solution_b[n].output_specs.placements)
+        lines = [f"Objective: {a['total']:.1f} -> {b['total']:.1f} ({b['total'] - a['total']:+.1f})"]
+        for k, label in (("compute", "compute"), ("comm", "comm:   "), ("transition", "trans:  ")):
+            lines.append(f"  {label} {a[k]:.1f} -> {b[k]:.1f} ({b[k] - a[k]:+.1f})")
+        lines.append(f"Placement changes: {changed} nodes changed")
+        out = "\n".join(lines)
+        print(out)
+        return out
+
+    def print_costs_for_node(self, node, arg: int = 0) -> str:
+        v = self.node_map[node]
+        e = self._core.edge_of(v, arg)
+        g = self._packed
+        block = self._core.coef.cost[self._core.var_start[e] : self._core.var_start[e + 1]]
+        text = f"{node} arg {arg}: cost[out_idx][inp_idx]\n{block.reshape(-1, int(g.edge_ssrc[e]))}"
+        print(text)
+        return text

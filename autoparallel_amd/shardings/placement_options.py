@@ -1,0 +1,260 @@
+"""Per-node strategy enumeration on the host.
+
+The strategies of an operator come from torch's DTensor sharding propagator
+(third-party code, as in the reference:
+autoparallel/shardings/dtensor_sharding_helpers.py:327-361); this module wraps
+it with the reference's post-processing — tensor-meta fill
+(autoparallel/shardings/placement_options.py:60-127), validity filter
+(autoparallel/shardings/propagation_rules.py:127-158), de-duplication
+(placement_options.py:151-170) — and the few rules DTensor lacks or refuses
+(getitem, strict views, alias, two-operand einsum, all-Replicate fallback:
+dtensor_sharding_helpers.py:364-383).  Its output is input data for the cost
+engine.  Input/parameter options are enumerated on the device
+(apc_enumerate_input_options).
+"""
+from __future__ import annotations
+
+import ctypes as C
+import itertools
+import operator
+from typing import Dict, List, Optional, Sequence
+
+import numpy as np
+import torch
+from torch.distributed.tensor import DTensor
+from torch.distributed.tensor._dtensor_spec import DTensorSpec, TensorMeta
+from torch.distributed.tensor._op_schema import OpSchema, OpSpec, OpStrategy, TupleStrategy
+from torch.distributed.tensor.placement_types import Partial, Replicate, Shard
+from torch.utils._pytree import tree_flatten, tree_map_only
+
+from .. import _lib
+
+aten = torch.ops.aten
+fallback_nodes: List[str] = []  # nodes that got the implicit all-Replicate strategy
+
+
+def _tensor_meta(t: torch.Tensor) -> TensorMeta:
+    return TensorMeta(t.shape, t.stride(), t.dtype)
+
+
+# ---------------------------------------------------------------------------
+# inputs / parameters
+# ---------------------------------------------------------------------------
+def enumerate_input_placements(mesh_shape: Sequence[int], shapes: Sequence[Sequence[int]]) -> List[List[tuple]]:
+    """Valid {Replicate, Shard(d)} tuples of each shape, itertools.product
+    order, from the device kernel."""
+    from ..cost_models.collective_runtime_estimation import _device_name
+    from ..engine import make_model
+
+    lib = _lib.load()
+    n = len(shapes)
+    nd = len(mesh_shape)
+    rank = np.asarray([len(s) for s in shapes], np.int32)
+    shp = np.ones((n, 8), np.int64)
+    for i, s in enumerate(shapes):
+        shp[i, : len(s)] = [int(x) for x in s]
+    off = np.zeros(n + 1, np.int64)
+    np.cumsum((rank.astype(np.int64) + 1) ** nd, out=off[1:])
+    d = lambda a: torch.from_numpy(a).cuda()
+    t_rank, t_shape, t_off = d(rank), d(shp), d(off)
+    valid = torch.zeros(int(off[-1]), dtype=torch.uint8, device="cuda")
+    plc = torch.zeros(int(off[-1]) * 4, dtype=torch.uint8, device="cuda")
+    model = make_model(tuple(mesh_shape), 1, _device_name())
+    _lib.check(lib.apc_enumerate_input_options(C.byref(model), n, t_rank.data_ptr(), t_shape.data_ptr(),
+                                               t_off.data_ptr(), valid.data_ptr(), plc.data_ptr(), None),
+               "apc_enumerate_input_options")
+    valid, plc = valid.cpu().numpy(), plc.cpu().numpy().reshape(-1, 4)
+    out = []
+    for i in range(n):
+        rows = []
+        for j in range(off[i], off[i + 1]):
+            if valid[j]:
+                rows.append(tuple(Replicate() if c == 0 else Shard(int(c) & 0x3F) for c in plc[j, :nd]))
+        out.append(rows)
+    return out
+
+
+def _create_all_options(mesh, shape, tensor_meta=None, tensor=None) -> OpStrategy:
+    if tensor is not None:
+        tensor_meta = _tensor_meta(tensor)
+    if tensor_meta is None:
+        t = torch.empty(tuple(shape), device="meta")
+        tensor_meta = _tensor_meta(t)
+    rows = enumerate_input_placements(tuple(mesh.shape), [tuple(shape)])[0]
+    strats = []
+    for plc in rows:
+        spec = DTensorSpec(mesh, plc, tensor_meta=tensor_meta)
+        strats.append(OpSpec(spec, input_specs=[spec], redistribute_cost=[[0.0]]))
+    return OpStrategy(strats)
+
+
+# ---------------------------------------------------------------------------
+# post-processing of operator strategies
+# ---------------------------------------------------------------------------
+def _spec_ok(spec: DTensorSpec, mesh) -> bool:
+    shape = list(spec.tensor_meta.shape)
+    for n, p in zip(mesh.shape, spec.placements):
+        if p.is_shard():
+            if shape[p.dim] >= n:
+                shape[p.dim] = (shape[p.dim] + n - 1) // n
+            else:
+                return False
+    return True
+
+
+def remove_invalid_configs(out_strat: OpStrategy, mesh) -> OpStrategy:
+    kept = []
+    for st in out_strat.strategies:
+        outs = st.output_specs
+        outs = [outs] if isinstance(outs, DTensorSpec) else list(outs or [])
+        specs = list(st.input_specs or []) + outs
+        if all(s is None or _spec_ok(s, mesh) for s in specs):
+            kept.append(st)
+    return OpStrategy(kept)
+
+
+def keep_unique_configs(op_strat: OpStrategy) -> OpStrategy:
+    seen, kept = set(), []
+    for st in op_strat.strategies:
+        ins = tuple(st.input_specs) if st.input_specs is not None else None
+        outs = tuple(st.output_specs) if isinstance(st.output_specs, list) else st.output_specs
+        try:
+            key = (ins, outs)
+            if key in seen:
+                continue
+            seen.add(key)
+        except TypeError:
+            pass
+        kept.append(st)
+    return OpStrategy(kept)
+
+
+def propagate_tensor_meta(node, arg_vals: List[torch.Tensor], out_strat: OpStrategy) -> None:
+    out_val = node.meta.get("val")
+    for st in out_strat.strategies:
+        outs = st.output_specs
+        if isinstance(outs, DTensorSpec):
+            if isinstance(out_val, torch.Tensor):
+                outs.tensor_meta = _tensor_meta(out_val)
+        elif outs is not None:
+            vals = list(out_val) if isinstance(out_val, (tuple, list)) else [out_val]
+            for s, v in zip(outs, vals):
+                if s is not None and isinstance(v, torch.Tensor):
+                    s.tensor_meta = _tensor_meta(v)
+        if st.input_specs is not None:
+            for s, v in zip(st.input_specs, arg_vals):
+                if s is not None and s.tensor_meta is None:
+                    s.tensor_meta = _tensor_meta(v)
+
+
+def fill_redistribute_cost(out_strat: OpStrategy, producers: List[OpStrategy]) -> None:
+    """Rows of the right shape (one per tensor argument, one column per
+    producer strategy); the values are overwritten by the cost engine."""
+    for st in out_strat.strategies:
+        st.redistribute_cost = [[0.0] * len(p.strategies) for p in producers] or [[0.0]]
+
+
+# ---------------------------------------------------------------------------
+# rules
+# ---------------------------------------------------------------------------
+def _follow_input(mesh, src: OpStrategy, out_val) -> OpStrategy:
+    """One strategy per distinct producer output placement: output == input."""
+    tm = _tensor_meta(out_val)
+    seen, sts = set(), []
+    for s in src.strategies:
+        spec = s.output_specs
+        if not isinstance(spec, DTensorSpec) or spec.placements in seen:
+            continue
+        seen.add(spec.placements)
+        sts.append(OpSpec(DTensorSpec(mesh, spec.placements, tensor_meta=tm),
+                          input_specs=[DTensorSpec(mesh, spec.placements, tensor_meta=spec.tensor_meta)]))
+    return OpStrategy(sts)
+
+
+def _getitem_rule(mesh, node, src: OpStrategy) -> OpStrategy:
+    idx = node.args[1]
+    seen, sts = set(), []
+    for s in src.strategies:
+        spec = s.output_specs[idx]
+        if spec is None or spec.placements in seen:
+            continue
+        seen.add(spec.placements)
+        sts.append(OpSpec(DTensorSpec(mesh, spec.placements, tensor_meta=spec.tensor_meta),
+                          input_specs=[DTensorSpec(mesh, spec.placements, tensor_meta=spec.tensor_meta)]))
+    return OpStrategy(sts)
+
+
+def _einsum_rule(mesh, node, a: OpStrategy, b: OpStrategy) -> OpStrategy:
+    """Two-operand einsum: product over mesh dims of the single-dim options
+    without Partial inputs (the reference's rule,
+    autoparallel/shardings/propagation_rules.py:573-590)."""
+    from torch.distributed.tensor._ops._einsum_strategy import gen_einsum_strategies
+
+    eq = node.args[0]
+    full = gen_einsum_strategies(eq, mesh)
+    sts = []
+    for st in full.strategies:
+        if any(p.is_partial() for s in st.input_specs for p in s.placements):
+            continue
+        sts.append(OpSpec(st.output_specs, input_specs=list(st.input_specs)))
+    return OpStrategy(sts)
+
+
+def _replicate_fallback(mesh, node, arg_vals) -> OpStrategy:
+    rep = (Replicate(),) * mesh.ndim
+    out_val = node.meta.get("val")
+    if isinstance(out_val, torch.Tensor):
+        out = DTensorSpec(mesh, rep, tensor_meta=_tensor_meta(out_val))
+    else:
+        out = tuple(DTensorSpec(mesh, rep, tensor_meta=_tensor_meta(v)) if isinstance(v, torch.Tensor) else None
+                    for v in out_val)
+    ins = [DTensorSpec(mesh, rep, tensor_meta=_tensor_meta(v)) for v in arg_vals]
+    fallback_nodes.append(str(node.name))
+    return OpStrategy([OpSpec(out, input_specs=ins)])
+
+
+_VIEW_NONSTRICT = {aten.view.default: aten._unsafe_view.default}
+_FOLLOW = {aten.alias.default, aten.detach.default}
+
+
+def get_placement_options_for_node(mesh, node, producers: List[OpStrategy], arg_vals: List[torch.Tensor],
+                                   schema_args) -> OpStrategy:
+    """Strategies of one call_function node.  ``producers``: OpStrategy of
+    each tensor input node in flattened-args order; ``schema_args``: node.args
+    with nodes replaced by their OpStrategy (or value for non-tensors)."""
+    prop = DTensor._op_dispatcher.sharding_propagator
+    op = node.target
+    out = None
+    try:
+        if op is operator.getitem:
+            out = _getitem_rule(mesh, node, producers[0])
+        elif op in _FOLLOW and len(producers) == 1:
+            out = _follow_input(mesh, producers[0], node.meta["val"])
+        elif op is aten.einsum.default and len(producers) == 2:
+            out = _einsum_rule(mesh, node, *producers)
+        else:
+            fn = prop.op_strategy_funcs.get(_VIEW_NONSTRICT.get(op, op))
+            if fn is not None:
+                def wrap(x):
+                    if isinstance(x, (list, tuple)) and x and all(isinstance(y, OpStrategy) for y in x):
+                        return TupleStrategy(tuple(x))
+                    return x
+                args = tuple(wrap(a) for a in schema_args)
+                kwargs = {k: v for k, v in node.kwargs.items() if not isinstance(v, torch.fx.Node)}
+                res = fn(OpSchema(op, args, kwargs))
+                if isinstance(res, OpStrategy):
+                    out = res
+    except Exception:
+        out = None
+    ok = out is not None and len(out.strategies) > 0 and all(
+        st.input_specs is not None and len(st.input_specs) == len(producers) for st in out.strategies)
+    if not ok:
+        out = _replicate_fallback(mesh, node, arg_vals)
+    propagate_tensor_meta(node, arg_vals, out)
+    fill_redistribute_cost(out, producers)
+    out = remove_invalid_configs(out, mesh)
+    out = keep_unique_configs(out)
+    if not out.strategies:
+        out = _replicate_fallback(mesh, node, arg_vals)
+        fill_redistribute_cost(out, producers)
+    return out

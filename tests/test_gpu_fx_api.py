@@ -1,0 +1,179 @@
+"""The reference-shaped Python surface (ShardingOptimizer on an AOT joint
+graph, the cost_models functions on DTensorSpecs) over the HIP engine."""
+import contextlib
+
+import numpy as np
+import pytest
+import torch
+import torch.nn as nn
+
+from helpers import bits_equal
+from oracle import cost_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def mesh():
+    if not torch.cuda.is_available():
+        pytest.skip("needs a GPU")
+    import torch.distributed as dist
+    from torch.distributed.device_mesh import init_device_mesh
+    from torch.testing._internal.distributed.fake_pg import FakeStore
+
+    if not dist.is_initialized():
+        dist.init_process_group("fake", store=FakeStore(), rank=0, world_size=8)
+    yield init_device_mesh("cpu", (2, 4))
+    dist.destroy_process_group()
+
+
+class MLP(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.a = nn.Linear(64, 128, bias=False)
+        self.b = nn.Linear(128, 64, bias=False)
+
+    def forward(self, x):
+        return self.b(torch.relu(self.a(x)))
+
+
+def _joint_graph():
+    from torch._functorch.aot_autograd import aot_export_joint_with_descriptors
+    from torch._subclasses.fake_tensor import FakeTensorMode
+
+    with FakeTensorMode():
+        m, x = MLP(), torch.randn(16, 32, 64)
+        with contextlib.ExitStack() as stack:
+            jd = aot_export_joint_with_descriptors(stack, m, (x,))
+    return jd.graph_module
+
+
+def test_sharding_optimizer_on_joint_graph(mesh):
+    from autoparallel_amd.optimize_sharding import ShardingOptimizer
+
+    gm = _joint_graph()
+    opt = ShardingOptimizer(gm, mesh, devices_per_host=8, device_name="AMD Instinct MI355X")
+    g = opt._packed
+    assert len(opt.decision_vars) == g.num_entries > 1000
+    # every coefficient equals the oracle's on the same packed problem
+    ref = O.GraphOracle(g).build()
+    slots = g.entry_slots()
+    cost_ref, bad = O.clamp_inf(ref["cost"])
+    assert bits_equal(opt._core.coef.comm, ref["comm"][slots])
+    assert bits_equal(opt._core.coef.cost, cost_ref[slots])
+    # mapping view: reference key order, attribute access, strategy objects
+    keys = list(opt.decision_vars)
+    assert keys == sorted(keys, key=lambda k: (k[0], k[2], k[1], k[3]))
+    k = keys[len(keys) // 2]
+    dv = opt.decision_vars[k]
+    assert dv.cost == dv.comm_cost + dv.compute_cost + dv.sharding_transition_cost or dv.cost == 10000.0
+    assert dv.strategy is opt.strats[opt.nodes[k[0]]].strategies[k[2]]
+    assert opt.decision_vars.get((10**6, 0, 0, 0)) is None
+    # redistribute_cost rows were written back (same object the strategies carry)
+    node = opt.nodes[k[0]]
+    assert opt.strats[node].strategies[k[2]].redistribute_cost[k[1]][k[3]] == dv.comm_cost
+    # solve: one strategy per node, consistent with the flow constraints
+    sol = opt.get_solution()
+    assert set(sol) == {n for n in opt.nodes if n.op != "output"}
+    base = opt._core.objective_value
+    total = opt._compute_solution_cost(sol)["total"]
+    assert np.isclose(total, base, rtol=1e-9)  # no clusters, no inf entries selected
+    # parameters and their gradients get the same placement
+    from torch._functorch._aot_autograd import fx_utils
+
+    for p, gr in fx_utils.get_param_and_grad_nodes(gm.graph).values():
+        assert sol[p].output_specs.placements == sol[gr].output_specs.placements
+    # a user constraint moves the plan and can be removed again
+    x = next(n for n in gm.graph.nodes if n.name == "primals_3")
+    from torch.distributed.tensor.placement_types import Replicate, Shard
+
+    names = opt.add_node_constraint(x, (Shard(0), Replicate()))
+    sol2 = opt.resolve()
+    assert sol2[x].output_specs.placements == (Shard(0), Replicate())
+    assert opt._core.objective_value >= base - 1e-9
+    opt.diff_solutions(sol, sol2)
+    opt.remove_constraints(names)
+    opt.resolve()
+    assert np.isclose(opt._core.objective_value, base)
+
+
+def test_cost_models_scalar_api(mesh, golden):
+    from torch.distributed.tensor._dtensor_spec import DTensorSpec, TensorMeta
+    from torch.distributed.tensor.placement_types import Partial, Replicate, Shard
+
+    from autoparallel_amd import cost_models as cm
+
+    cm.configure(devices_per_host=8, device_name="AMD Instinct MI355X")
+    shape = (6, 10)
+    tm = TensorMeta(torch.Size(shape), (10, 1), torch.float32)
+    topo, dev = O.Topo((2, 4), 8), O.DeviceLimit()
+    code = {Replicate(): 0, Shard(0): 0x40, Shard(1): 0x41, Partial(): 0x80}
+    opts = list(code)
+    for a in [(Shard(0), Shard(1)), (Partial(), Partial()), (Replicate(), Shard(1)), (Shard(1), Partial())]:
+        for b in [(Replicate(), Replicate()), (Shard(1), Shard(0)), (Shard(0), Shard(0)), (Partial(), Replicate())]:
+            s, t = DTensorSpec(mesh, a, tensor_meta=tm), DTensorSpec(mesh, b, tensor_meta=tm)
+            got = cm.estimate_strategy_comms_cost(s, t)
+            sa, tb = tuple(code[p] for p in a), tuple(code[p] for p in b)
+            want = O.estimate_strategy_comms_cost(sa, shape, (10, 1), 4, tb, topo, dev)
+            assert got == want or (np.isinf(got) and np.isinf(want)), (a, b, got, want)
+            fwd = cm.redistribute_cost(s, t, [0, 1])
+            want_fwd = O.redistribute_cost(sa, shape, (10, 1), 4, tb, topo, dev, [0, 1])
+            assert fwd == want_fwd or (np.isinf(fwd) and np.isinf(want_fwd))
+    assert cm.compute_read_write_time(2**40) == float(O.compute_read_write_time(2**40, dev))
+    got = cm.collective_comm_cost("allreduce", 2**30, (2, 4), 1, devices_per_host=8)
+    assert got == O.collective_comm_cost("allreduce", 2**30, topo, 1)
+    from autoparallel_amd.cost_models.compute_estimation import _get_sharded_shape_stride
+
+    spec = DTensorSpec(mesh, (Shard(0), Shard(1)), tensor_meta=TensorMeta(torch.Size((64, 36)), (36, 1), torch.float32))
+    assert _get_sharded_shape_stride(spec) == ([32, 9], [36, 1])
+    with pytest.raises(NotImplementedError):
+        cm.set_nccl_topo_config(object())
+
+
+def test_runtime_cost_api_matches_reference_vectors(mesh, golden):
+    """estimate_strategy_runtime_cost on fx nodes: the closed-form ops through
+    programs, an op without one (cumsum) through the explicit route."""
+    from torch.distributed.tensor._dtensor_spec import DTensorSpec, TensorMeta
+    from torch.distributed.tensor._op_schema import OpSpec
+    from torch.distributed.tensor.placement_types import Replicate, Shard
+
+    from autoparallel_amd import cost_models as cm, fx_programs
+
+    cm.configure(devices_per_host=8, device_name="AMD Instinct MI355X")
+    aten = torch.ops.aten
+    graph = torch.fx.Graph()
+
+    def ph(name, shape, dtype):
+        n = graph.placeholder(name)
+        n.meta["val"] = torch.empty(shape, dtype=dtype, device="meta")
+        return n
+
+    a, b = ph("a", (512, 256), torch.float32), ph("b", (256, 1024), torch.float32)
+    mm = graph.call_function(aten.mm.default, (a, b))
+    mm.meta["val"] = torch.empty((512, 1024), dtype=torch.float32, device="meta")
+
+    def spec(n, plc):
+        v = n.meta["val"]
+        return DTensorSpec(mesh, plc, tensor_meta=TensorMeta(v.shape, v.stride(), v.dtype))
+
+    dev = O.DeviceLimit()
+    for pa, pb, (m_, k_, n_) in [((Replicate(), Replicate()), (Replicate(), Replicate()), (512, 256, 1024)),
+                                 ((Shard(0), Replicate()), (Replicate(), Shard(1)), (256, 256, 256))]:
+        st = OpSpec(spec(mm, pa), input_specs=[spec(a, pa), spec(b, pb)])
+        cm.reset_compute_cost_cache()
+        got = cm.estimate_strategy_runtime_cost(mm, st)
+        want = O.roofline_cost(2 * m_ * k_ * n_, 4 * (m_ * k_ + k_ * n_ + m_ * n_), 1, dev)
+        assert got == float(want)
+    # explicit route
+    x = ph("x", (4096, 4096), torch.bfloat16)
+    cs = graph.call_function(aten.cumsum.default, (x, 1))
+    cs.meta["val"] = torch.empty((4096, 4096), dtype=torch.bfloat16, device="meta")
+    st = OpSpec(spec(cs, (Shard(0), Replicate())), input_specs=[spec(x, (Shard(0), Replicate()))])
+    before = sum(fx_programs.fallback_ops.values())
+    got = cm.estimate_strategy_runtime_cost(cs, st)
+    assert sum(fx_programs.fallback_ops.values()) == before + 1
+    assert got == float(O.roofline_cost(0, 2 * (2048 * 4096 * 2), 3, dev))
+    # views cost nothing
+    v = graph.call_function(aten.view.default, (x, [16, 256, 4096]))
+    v.meta["val"] = torch.empty((16, 256, 4096), dtype=torch.bfloat16, device="meta")
+    assert cm.estimate_strategy_runtime_cost(v, st) == 0
