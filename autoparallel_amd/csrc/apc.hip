@@ -619,14 +619,14 @@ template <bool kRandom>
 __global__ void __launch_bounds__(kBlock)
 score_kernel(apc_problem p, const double* __restrict__ per_arg, const double* __restrict__ comm,
              const double* __restrict__ cost, const uint8_t* __restrict__ flags,
-             const uint16_t* __restrict__ assign, uint64_t seed, int64_t first, int64_t n_assign,
-             double* __restrict__ out) {
+             const uint16_t* __restrict__ assign, int64_t stride, uint64_t seed, int64_t first,
+             int64_t n_assign, double* __restrict__ out) {
   const int64_t a = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (a >= n_assign) return;
   double t_compute = 0.0, t_comm = 0.0, t_trans = 0.0, obj = 0.0, forbidden = 0.0;
   for (int v = 0; v < p.n_node; ++v) {
     const uint32_t o = kRandom ? mix_assignment(seed, first + a, v, p.node_nstrat[v])
-                               : (uint32_t)assign[(size_t)v * n_assign + a];
+                               : (uint32_t)assign[(size_t)v * stride + a];
     const int nargs = p.node_nargs[v];
     const double pa = per_arg[p.node_comp_off[v] + o];
     t_compute += pa * (double)(nargs > 1 ? nargs : 1);
@@ -636,7 +636,7 @@ score_kernel(apc_problem p, const double* __restrict__ per_arg, const double* __
       uint32_t j = 0;
       if (ed.src_node >= 0)
         j = kRandom ? mix_assignment(seed, first + a, ed.src_node, p.node_nstrat[ed.src_node])
-                    : (uint32_t)assign[(size_t)ed.src_node * n_assign + a];
+                    : (uint32_t)assign[(size_t)ed.src_node * stride + a];
       const int64_t idx = ed.off + (int64_t)o * ed.ssrc + j;
       const uint8_t f = flags[idx];
       obj += cost[idx] * mult;
@@ -655,6 +655,83 @@ score_kernel(apc_problem p, const double* __restrict__ per_arg, const double* __
   r[3] = t_trans;
   r[4] = obj;
   r[5] = forbidden;
+}
+
+// In-order fold of one value per lane into acc: acc = (..((acc + v0) + v1)..) + v63,
+// the association a sequential loop over 64 items has.
+__device__ __forceinline__ double fold_in_order(double acc, double v) {
+  const int lo = __double2loint(v), hi = __double2hiint(v);
+#pragma unroll
+  for (int i = 0; i < 64; ++i)
+    acc += __hiloint2double(__builtin_amdgcn_readlane(hi, i), __builtin_amdgcn_readlane(lo, i));
+  return acc;
+}
+
+// Small batches: one wavefront per assignment.  Lanes take 64 consecutive
+// nodes (then 64 consecutive edges) at a time, gather their terms in parallel,
+// and the terms are folded lane by lane in order, so the sums keep the
+// reference's sequential association (bit-identical to score_kernel) while the
+// gathers of a tile overlap.
+template <bool kRandom>
+__global__ void __launch_bounds__(kBlock)
+score_wave_kernel(apc_problem p, const double* __restrict__ per_arg,
+                  const double* __restrict__ comm, const double* __restrict__ cost,
+                  const uint8_t* __restrict__ flags, const uint16_t* __restrict__ assign,
+                  int64_t stride, uint64_t seed, int64_t first, int64_t n_assign,
+                  double* __restrict__ out) {
+  const int64_t a = (int64_t)blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6);
+  if (a >= n_assign) return;  // wave-uniform
+  const int lane = threadIdx.x & 63;
+  auto choice = [&](int v) -> uint32_t {
+    return kRandom ? mix_assignment(seed, first + a, v, p.node_nstrat[v])
+                   : (uint32_t)assign[(size_t)v * stride + a];
+  };
+  double t_compute = 0.0, t_comm = 0.0, t_trans = 0.0, obj = 0.0, forbidden = 0.0;
+  for (int v0 = 0; v0 < p.n_node; v0 += 64) {
+    const int v = v0 + lane;
+    double term = 0.0;
+    if (v < p.n_node) {
+      const int nargs = p.node_nargs[v];
+      term = per_arg[p.node_comp_off[v] + choice(v)] * (double)(nargs > 1 ? nargs : 1);
+    }
+    t_compute = fold_in_order(t_compute, term);  // + 0.0 for the lanes past the end
+  }
+  for (int e0 = 0; e0 < p.n_edge; e0 += 64) {
+    const int e = e0 + lane;
+    double c_term = 0.0, o_term = 0.0, tr = 0.0, fb = 0.0;
+    if (e < p.n_edge) {
+      const apc_edge ed = p.edges[e];
+      const uint32_t o = choice(ed.node);
+      const uint32_t j = ed.src_node >= 0 ? choice(ed.src_node) : 0u;
+      const int64_t idx = ed.off + (int64_t)o * ed.ssrc + j;
+      const uint8_t f = flags[idx];
+      o_term = cost[idx] * (double)p.node_multiplier[ed.node];
+      fb = (double)((f & APC_ENTRY_NONFINITE) != 0);
+      if (ed.src_node >= 0) {
+        const double c = comm[idx];
+        if (isfinite(c)) c_term = c;
+        if ((ed.flags & APC_EDGE_SCORE_TRANSITION) && (f & APC_ENTRY_TRANSITION)) tr = 1.0;
+      }
+    }
+    t_comm = fold_in_order(t_comm, c_term);
+    obj = fold_in_order(obj, o_term);
+    // small integers: any order is exact
+    for (int off = 32; off > 0; off >>= 1) {
+      tr += __shfl_xor(tr, off, 64);
+      fb += __shfl_xor(fb, off, 64);
+    }
+    t_trans += tr;
+    forbidden += fb;
+  }
+  if (lane == 0) {
+    double* r = out + a * 6;
+    r[0] = (t_compute + t_comm) + t_trans;
+    r[1] = t_compute;
+    r[2] = t_comm;
+    r[3] = t_trans;
+    r[4] = obj;
+    r[5] = forbidden;
+  }
 }
 
 // ---------------------------------------------------------------------------
@@ -754,6 +831,9 @@ rw_time_kernel(apc_model m, int32_t n, const double* __restrict__ nbytes, double
 // ---------------------------------------------------------------------------
 // Host side
 // ---------------------------------------------------------------------------
+// below this many assignments one wavefront per assignment is faster than one lane
+constexpr int64_t kScoreWaveBelow = 32768;
+
 int validate_problem(const apc_problem* p) {
   if (!p) return fail(APC_ERR_INVALID, "null problem%s");
   if (p->model.ndim < 1 || p->model.ndim > APC_MAX_MESH_DIMS)
@@ -959,6 +1039,39 @@ int apc_objective_coeffs(const apc_problem* p, const double* cost, double* obj, 
   return check_launch("objective_kernel");
 }
 
+// Launches in chunks: beyond a few hundred thousand lanes walking the graph at
+// once, the lanes drift apart and stop sharing cache lines of the entry arrays.
+static int launch_score(const apc_problem* p, const double* per_arg, const double* comm,
+                        const double* cost, const uint8_t* flags, const uint16_t* assign,
+                        bool random, uint64_t seed, int64_t first, int64_t n_assign, double* out,
+                        hipStream_t stream) {
+  const int64_t kChunk = 262144;
+  for (int64_t a0 = 0; a0 < n_assign; a0 += kChunk) {
+    const int64_t n = (n_assign - a0 < kChunk) ? (n_assign - a0) : kChunk;
+    const uint16_t* asg = assign ? assign + a0 : nullptr;
+    double* o = out + a0 * 6;
+    if (n_assign < kScoreWaveBelow) {
+      const unsigned grid = (unsigned)((n + (kBlock / 64) - 1) / (kBlock / 64));
+      if (random)
+        hipLaunchKernelGGL(score_wave_kernel<true>, dim3(grid), dim3(kBlock), 0, stream, *p, per_arg,
+                           comm, cost, flags, asg, n_assign, seed, first + a0, n, o);
+      else
+        hipLaunchKernelGGL(score_wave_kernel<false>, dim3(grid), dim3(kBlock), 0, stream, *p,
+                           per_arg, comm, cost, flags, asg, n_assign, seed, first + a0, n, o);
+    } else {
+      const unsigned grid = (unsigned)((n + kBlock - 1) / kBlock);
+      if (random)
+        hipLaunchKernelGGL(score_kernel<true>, dim3(grid), dim3(kBlock), 0, stream, *p, per_arg, comm,
+                           cost, flags, asg, n_assign, seed, first + a0, n, o);
+      else
+        hipLaunchKernelGGL(score_kernel<false>, dim3(grid), dim3(kBlock), 0, stream, *p, per_arg,
+                           comm, cost, flags, asg, n_assign, seed, first + a0, n, o);
+    }
+    if (int rc = check_launch("score kernel")) return rc;
+  }
+  return 0;
+}
+
 int apc_score_assignments(const apc_problem* p, const double* per_arg, const double* comm,
                           const double* cost, const uint8_t* flags, const uint16_t* assign,
                           int64_t n_assign, double* out, void* stream) {
@@ -966,11 +1079,8 @@ int apc_score_assignments(const apc_problem* p, const double* per_arg, const dou
   if (n_assign <= 0) return 0;
   if (!per_arg || !comm || !cost || !flags || !assign || !out || !p->node_multiplier)
     return fail(APC_ERR_INVALID, "apc_score_assignments: null argument%s");
-  const int64_t grid = (n_assign + kBlock - 1) / kBlock;
-  hipLaunchKernelGGL(score_kernel<false>, dim3((unsigned)grid), dim3(kBlock), 0,
-                     (hipStream_t)stream, *p, per_arg, comm, cost, flags, assign, 0ull, 0ll,
-                     n_assign, out);
-  return check_launch("score_kernel");
+  return launch_score(p, per_arg, comm, cost, flags, assign, false, 0, 0, n_assign, out,
+                      (hipStream_t)stream);
 }
 
 int apc_score_random_assignments(const apc_problem* p, const double* per_arg, const double* comm,
@@ -980,11 +1090,8 @@ int apc_score_random_assignments(const apc_problem* p, const double* per_arg, co
   if (n_assign <= 0) return 0;
   if (!per_arg || !comm || !cost || !flags || !out || !p->node_multiplier)
     return fail(APC_ERR_INVALID, "apc_score_random_assignments: null argument%s");
-  const int64_t grid = (n_assign + kBlock - 1) / kBlock;
-  hipLaunchKernelGGL(score_kernel<true>, dim3((unsigned)grid), dim3(kBlock), 0,
-                     (hipStream_t)stream, *p, per_arg, comm, cost, flags, (const uint16_t*)nullptr,
-                     seed, first, n_assign, out);
-  return check_launch("score_kernel<random>");
+  return launch_score(p, per_arg, comm, cost, flags, nullptr, true, seed, first, n_assign, out,
+                      (hipStream_t)stream);
 }
 
 uint32_t apc_random_assignment(uint64_t seed, int64_t a, int32_t node, int32_t nstrat) {

@@ -54,6 +54,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="llama3_8b_fwd_bwd_mesh8x8")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--score-assignments", type=int, default=1 << 20,
+                    help="also score this many on-device generated assignments (0 = skip)")
     ap.add_argument("--direct", action="store_true", help="evaluate every entry directly (no row table)")
     ap.add_argument("--calibration-copy-mib", type=int, default=0,
                     help="after the timed steps, also launch the plain copy kernel on this many MiB "
@@ -164,6 +166,25 @@ def main():
             "traffic": read_traffic(args.workload),
         },
     }
+
+    if args.score_assignments > 0:
+        # batch scoring of candidate assignments against the objective (secondary
+        # figure; the assignments are generated on the device, nothing is uploaded)
+        n = args.score_assignments
+        eng.score_random(1, 0, min(n, 4096))
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        scores = eng.score_random(1, 0, n)
+        torch.cuda.synchronize()
+        t_score = time.perf_counter() - t0
+        out["scoring"] = {
+            "assignments": n,
+            "seconds": t_score,
+            "assignments_per_s": n / t_score,
+            "edge_terms_per_s": n * g.num_edges / t_score,
+            "algorithmic_bytes_per_assignment": 8 * g.num_nodes + 17 * g.num_edges,
+            "feasible_fraction": float((scores[:, 5] == 0).double().mean().item()),
+        }
 
     if not args.no_cpu_baseline:
         from oracle import cost_oracle as O

@@ -214,6 +214,13 @@ def test_scoring(CostEngine):
         obj, viol = O.ilp_objective(g, cost, bad, assign[:, a])
         assert tuple(out[a, :4]) == tuple(float(x) for x in want), (a, out[a], want)
         assert out[a, 4] == obj and out[a, 5] == viol
+    # large batches take the lane-per-assignment kernel: same bits as the wave kernel
+    big = np.tile(assign, (1, 900))[:, :33000]
+    out_big = eng.score(torch.from_numpy(np.ascontiguousarray(big)).cuda()).cpu().numpy()
+    assert bits_equal(out_big[:A].ravel(), out.ravel()) and bits_equal(out_big[A:2 * A].ravel(), out.ravel())
+    r_small = eng.score_random(seed=3, first=0, count=50).cpu().numpy()
+    r_big = eng.score_random(seed=3, first=0, count=33000).cpu().numpy()
+    assert bits_equal(r_big[:50].ravel(), r_small.ravel())
     # on-device generated assignments: same draw on the host
     out = eng.score_random(seed=11, first=5, count=9).cpu().numpy()
     for i in range(9):
