@@ -899,3 +899,71 @@ def config_llama3_8b(n_layers: int = 32) -> PackedGraph:
 
 def config_llama3_70b(n_layers: int = 80) -> PackedGraph:
     return llama_graph((4, 8, 8), n_layers, 8192, 64, 8, 28672, 128256, 8192, 256)
+
+
+def stress_graph(
+    n_nodes: int,
+    mesh_shape: Sequence[int] = (4, 8, 8),
+    seed: int = 0,
+    s_min: int = 4,
+    s_max: int = 512,
+    mean_out_degree: float = 1.8,
+    devices_per_host: int = 8,
+) -> PackedGraph:
+    """Seeded random planner stress graph: a DAG whose nodes have tensor ranks
+    1-4, dims log-uniform in [64, 65536], dtype in {bf16, fp32}, op class in
+    {matmul, elementwise, reduction, view}, and ``U[s_min, s_max]`` random
+    strategies each.  No two nodes share a tensor meta, so nothing repeats:
+    the entry kernel evaluates every entry directly."""
+    rng = np.random.default_rng(seed)
+    nd = len(mesh_shape)
+    b = GraphBuilder(mesh_shape, devices_per_host)
+    b.share_compute_slots = False
+    ranks, metas, dts = [], [], []
+    n_in_total = 0
+    for v in range(n_nodes):
+        r = int(rng.integers(1, 5))
+        shape = tuple(int(2 ** rng.uniform(6, 16)) for _ in range(r))
+        dt = DT_BF16 if rng.random() < 0.5 else DT_F32
+        ranks.append(r)
+        dts.append(dt)
+        metas.append(b.meta(shape, contiguous_stride(shape), _ITEMSIZE[dt], dt))
+        S = int(rng.integers(s_min, s_max + 1))
+
+        def tuples(rank, n):
+            codes = np.asarray([R] + [shard(d) for d in range(rank)] + [P])
+            return [tuple(int(c) for c in row) for row in codes[rng.integers(0, len(codes), size=(n, nd))]]
+
+        out_specs = [[b.spec(metas[v], t)] for t in tuples(r, S)]
+        op = ("matmul", "elementwise", "reduction", "view")[int(rng.integers(0, 4))]
+        want_in = 0 if v == 0 else {"matmul": 2, "elementwise": int(rng.integers(1, 3)), "reduction": 1, "view": 1}[op]
+        # keep the mean out-degree near the target
+        if v > 0 and n_in_total / v > mean_out_degree:
+            want_in = min(want_in, 1)
+        inputs = [int(rng.integers(0, v)) for _ in range(want_in)]
+        n_in_total += len(inputs)
+        if not inputs:
+            b.add_node(NodeDesc(f"in_{v}", in_specs=[[w[0]] for w in out_specs], out_specs=out_specs, inputs=[],
+                                default_rows=[[[0.0]] for _ in out_specs]))
+            continue
+        cols = [[b.spec(metas[u], t) for t in tuples(ranks[u], S)] for u in inputs]
+        in_specs = [[c[o] for c in cols] for o in range(S)]
+        isz = _ITEMSIZE[dt]
+        if op == "view":
+            desc = NodeDesc(f"view_{v}", in_specs=in_specs, out_specs=out_specs, inputs=inputs)
+        elif op == "matmul":
+            from .packed import OP_EXPLICIT
+
+            desc = NodeDesc(f"matmul_{v}", in_specs=in_specs, out_specs=out_specs, inputs=inputs, op=OP_EXPLICIT,
+                            flops=[int(x) for x in rng.integers(1, 2**44, size=S)],
+                            nbytes=[int(x) for x in rng.integers(1, 2**34, size=S)])
+        elif op == "reduction":
+            ru = ranks[inputs[0]]
+            desc = NodeDesc(f"reduction_{v}", in_specs=in_specs, out_specs=out_specs, inputs=inputs, op=OP_PROGRAM,
+                            program=opprog.reduction(ru, [ru - 1], True, isz))
+        else:
+            ru = max(ranks[u] for u in inputs)
+            desc = NodeDesc(f"elementwise_{v}", in_specs=in_specs, out_specs=out_specs, inputs=inputs, op=OP_PROGRAM,
+                            program=opprog.pointwise(ru, isz))
+        b.add_node(desc)
+    return b.pack()

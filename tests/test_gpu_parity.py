@@ -136,6 +136,7 @@ GRAPHS = {
     "gpt2_1d": lambda: graphgen.gpt2_graph((8,), n_layers=2),
     "llama_3d": lambda: graphgen.llama_graph((2, 4, 2), 1, 512, 8, 4, 1024, 4096, 256, 16),
     "llama_odd_mesh": lambda: graphgen.llama_graph((3, 5), 1, 960, 15, 5, 1920, 3000, 240, 30),
+    "stress_3d": lambda: graphgen.stress_graph(150, (4, 8, 8), seed=1, s_max=48),
     "pairs_4d": lambda: _pairs_graph((2, 3, 2, 4), (48, 36, 40), 300),
     "pairs_3d_noncontig": lambda: _pairs_graph((4, 8, 8), (256, 8192, 64), 250, stride=(64, 16384, 1)),
 }
@@ -154,7 +155,7 @@ def _pairs_graph(mesh, shape, n, stride=None, seed=3):
 
 # every graph through the table path; direct evaluation on the smaller ones
 CASES = [(n, True) for n in GRAPHS] + [
-    (n, False) for n in ("llama_2d", "gpt2_1d", "llama_odd_mesh", "pairs_4d", "pairs_3d_noncontig")
+    (n, False) for n in ("llama_2d", "gpt2_1d", "llama_odd_mesh", "stress_3d", "pairs_4d", "pairs_3d_noncontig")
 ]
 
 
