@@ -73,6 +73,8 @@ class ApcProblem(C.Structure):
         ("run_len", C.c_void_p),
         ("run_table_off", C.c_void_p),
         ("table_size", C.c_int64),
+        ("n_table_block", C.c_int32),
+        ("table_block_run", C.c_void_p),
     ]
 
 

@@ -67,20 +67,6 @@ __device__ __forceinline__ double collective_cost(int kind, int64_t nbytes, int 
   return t;
 }
 
-// check_contiguous_sizes_strides (torch _prims_common/__init__.py:252-293)
-__device__ __forceinline__ bool is_contiguous(const int64_t* shape, const int64_t* stride,
-                                              int rank) {
-  int64_t expected = 1, expected_max = 1;
-  for (int d = rank - 1; d >= 0; --d) {
-    int64_t x = shape[d], y = stride[d];
-    if (x == 1) continue;
-    if (y != expected && y != expected_max) return false;
-    expected_max *= (x > 1 ? x : 1);
-    expected *= x;
-  }
-  return true;
-}
-
 // redistribute_cost with estimate_strategy_comms_cost's order rule
 // (collective_runtime_estimation.py:115-229, 253-258).  src/tgt: placement
 // bytes packed little-endian, one per mesh dim.
@@ -142,17 +128,35 @@ __device__ __forceinline__ uint32_t load_tuple(const uint8_t* tuple_plc, uint32_
   return *reinterpret_cast<const uint32_t*>(tuple_plc + (size_t)t * APC_MAX_MESH_DIMS);
 }
 
-__device__ __forceinline__ int64_t meta_bytes(const apc_problem& p, uint32_t mid) {
-  int rank = p.meta_rank[mid];
-  int64_t b = p.meta_itemsize[mid];
-  const int64_t* sh = p.meta_shape + (size_t)mid * APC_MAX_RANK;
-  for (int d = 0; d < rank; ++d) b *= sh[d];
-  return b;
-}
-
-__device__ __forceinline__ bool meta_contiguous(const apc_problem& p, uint32_t mid) {
-  return is_contiguous(p.meta_shape + (size_t)mid * APC_MAX_RANK,
-                       p.meta_stride + (size_t)mid * APC_MAX_RANK, p.meta_rank[mid]);
+// itemsize * prod(shape) and contiguity of tensor meta `mid`.  Both rows are
+// fetched with unconditional 16-byte loads before any element is used, so the
+// lane pays one memory latency, not one per dimension.
+__device__ __forceinline__ void meta_bytes_contig(const apc_problem& p, uint32_t mid,
+                                                  int64_t& nbytes, bool& contiguous) {
+  const int rank = p.meta_rank[mid];
+  const int64_t isz = p.meta_itemsize[mid];
+  const ll2_t* sh = reinterpret_cast<const ll2_t*>(p.meta_shape + (size_t)mid * APC_MAX_RANK);
+  const ll2_t* st = reinterpret_cast<const ll2_t*>(p.meta_stride + (size_t)mid * APC_MAX_RANK);
+  ll2_t shape[APC_MAX_RANK / 2], stride[APC_MAX_RANK / 2];
+#pragma unroll
+  for (int q = 0; q < APC_MAX_RANK / 2; ++q) { shape[q] = sh[q]; stride[q] = st[q]; }
+  int64_t b = isz, expected = 1, expected_max = 1;
+  bool ok = true;
+#pragma unroll
+  for (int d = APC_MAX_RANK - 1; d >= 0; --d) {
+    if (d >= rank) continue;
+    const int64_t x = (d & 1) ? shape[d >> 1].y : shape[d >> 1].x;
+    const int64_t y = (d & 1) ? stride[d >> 1].y : stride[d >> 1].x;
+    b *= x;
+    // check_contiguous_sizes_strides (torch _prims_common/__init__.py:252-293)
+    if (x != 1) {
+      if (y != expected && y != expected_max) ok = false;
+      expected_max *= (x > 1 ? x : 1);
+      expected *= x;
+    }
+  }
+  nbytes = b;
+  contiguous = ok;
 }
 
 __device__ __forceinline__ int64_t ceil_div_pos(int64_t s, int64_t n) {
@@ -366,30 +370,61 @@ __device__ __forceinline__ void node_compute_wave(const apc_problem& p, int v, i
   }
 }
 
-// Row tables: element idx of the table belongs to run r (binary search in
-// run_table_off), target tuple t and source position j.
+// Touch `bytes` of an array (capped) so that the dependent loads that follow
+// find it in L2: the entry arrays stream through L2 between two builds and evict
+// the small tables.  One 4-byte load per 128-byte line per lane, results kept
+// alive but unused.
+__device__ __forceinline__ uint32_t warm_lines(const void* base, int64_t bytes, int lane,
+                                               int lanes) {
+  const int64_t cap = bytes < (1 << 16) ? bytes : (1 << 16);
+  uint32_t acc = 0;
+  for (int64_t off = (int64_t)lane * 128; off + 4 <= cap; off += (int64_t)lanes * 128)
+    acc ^= *reinterpret_cast<const uint32_t*>(reinterpret_cast<const char*>(base) + off);
+  return acc;
+}
+
+__device__ __forceinline__ uint32_t warm_problem(const apc_problem& p, int lane, int lanes) {
+  uint32_t acc = 0;
+  if (p.n_list) acc ^= warm_lines(p.lists, p.n_list * 4, lane, lanes);
+  if (p.n_meta) {
+    acc ^= warm_lines(p.meta_shape, (int64_t)p.n_meta * APC_MAX_RANK * 8, lane, lanes);
+    acc ^= warm_lines(p.meta_stride, (int64_t)p.n_meta * APC_MAX_RANK * 8, lane, lanes);
+    acc ^= warm_lines(p.meta_rank, (int64_t)p.n_meta * 4, lane, lanes);
+    acc ^= warm_lines(p.meta_itemsize, (int64_t)p.n_meta * 4, lane, lanes);
+    acc ^= warm_lines(p.meta_dtype, (int64_t)p.n_meta * 4, lane, lanes);
+  }
+  if (p.n_tuple) acc ^= warm_lines(p.tuple_plc, (int64_t)p.n_tuple * APC_MAX_MESH_DIMS, lane, lanes);
+  return acc;
+}
+
+// Row tables.  Every run's table starts on a multiple of 256 elements, so a
+// block of 256 threads works on one run: the run's description is block-uniform
+// (scalar loads) and element r of the run's table is target tuple r / len,
+// source position r % len.
 __device__ __forceinline__ void pair_table_block(const apc_problem& p, double* __restrict__ table,
-                                                 int block, int nblocks) {
-  const int64_t total = p.table_size;
-  for (int64_t idx = (int64_t)block * blockDim.x + threadIdx.x; idx < total;
-       idx += (int64_t)nblocks * blockDim.x) {
-    int lo = 0, hi = p.n_run;
-    while (hi - lo > 1) {
-      const int mid = (lo + hi) >> 1;
-      if (p.run_table_off[mid] <= idx) lo = mid; else hi = mid;
-    }
-    const uint32_t len = (uint32_t)p.run_len[lo];
-    const uint32_t r = (uint32_t)(idx - p.run_table_off[lo]);
+                                                 int block) {
+  const uint32_t keep = warm_problem(p, threadIdx.x, blockDim.x);
+  const int run = p.table_block_run[block];
+  const int64_t base = p.run_table_off[run];
+  const uint32_t len = (uint32_t)p.run_len[run];
+  const int64_t r64 = (int64_t)block * 256 - base + threadIdx.x;
+  const int64_t size = (int64_t)len * p.n_tuple;
+  if (r64 < size) {
+    const uint32_t r = (uint32_t)r64;
     const uint32_t t = r / len, j = r - t * len;
-    const uint32_t sw = p.lists[(size_t)p.run_list[lo] + j];
+    const uint32_t sw = p.lists[(size_t)p.run_list[run] + j];
     double c = 0.0;  // a missing spec never reads its table slot
     if (sw != APC_SPEC_NONE) {
       const uint32_t sm = sw >> APC_TUPLE_BITS;
+      int64_t nbytes;
+      bool contig;
+      meta_bytes_contig(p, sm, nbytes, contig);
       c = redistribute_cost(load_tuple(p.tuple_plc, sw & kTupleMask), load_tuple(p.tuple_plc, t),
-                            meta_bytes(p, sm), meta_contiguous(p, sm), p.model);
+                            nbytes, contig, p.model);
     }
-    table[idx] = c;
+    table[base + r] = c;
   }
+  asm volatile("" ::"v"(keep));
 }
 
 // Blocks [0, table_blocks) fill the pair table, the rest price the nodes of
@@ -403,12 +438,14 @@ prepare_kernel(apc_problem p, double* __restrict__ table, int table_blocks, int 
                int32_t* __restrict__ status) {
   extern __shared__ int64_t s_dyn[];
   if ((int)blockIdx.x < table_blocks) {
-    pair_table_block(p, table, blockIdx.x, table_blocks);
+    pair_table_block(p, table, blockIdx.x);
     return;
   }
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int i = ((int)blockIdx.x - table_blocks) * kNodesPerBlock + wave;
   if (i >= p.n_comp_node) return;
+  const uint32_t keep = warm_problem(p, threadIdx.x & 63, 64);
+  asm volatile("" ::"v"(keep));
   const int v = __builtin_amdgcn_readfirstlane(p.comp_nodes[i]);
   const int per_wave = kProgCache + (slow ? 0 : p.max_node_args * (p.max_rank + 1) * 64);
   int64_t* s_prog = s_dyn + (size_t)wave * per_wave;
@@ -445,8 +482,11 @@ __device__ __forceinline__ void eval_entry(const apc_problem& p, const apc_edge&
     if (kUseTable) {
       comm = table[ed.table_off + (int64_t)tt * ed.ssrc + j];
     } else {
-      comm = redistribute_cost(load_tuple(p.tuple_plc, st), load_tuple(p.tuple_plc, tt),
-                               meta_bytes(p, sm), meta_contiguous(p, sm), p.model);
+      int64_t nbytes;
+      bool contig;
+      meta_bytes_contig(p, sm, nbytes, contig);
+      comm = redistribute_cost(load_tuple(p.tuple_plc, st), load_tuple(p.tuple_plc, tt), nbytes,
+                               contig, p.model);
     }
   } else {
     comm = p.default_vals[ed.default_off + (int64_t)o * ed.ssrc + j];
@@ -853,8 +893,9 @@ int validate_problem(const apc_problem* p) {
   if (p->n_entry > 0 && (!p->edges || !p->chunk_edge || !p->lists || !p->items))
     return fail(APC_ERR_INVALID, "null edge/list/item arrays%s");
   if (p->n_comp_node > 0 && !p->comp_nodes) return fail(APC_ERR_INVALID, "null comp_nodes%s");
-  if (p->n_run < 0 || p->table_size < 0 ||
-      (p->table_size > 0 && (!p->run_list || !p->run_len || !p->run_table_off)))
+  if (p->n_run < 0 || p->table_size < 0 || (p->table_size & 255) ||
+      p->n_table_block != p->table_size / 256 ||
+      (p->table_size > 0 && (!p->run_list || !p->run_len || !p->run_table_off || !p->table_block_run)))
     return fail(APC_ERR_INVALID, "bad run table description%s");
   if (p->max_rank < 0 || p->max_rank > APC_MAX_RANK || p->max_node_args < 0)
     return fail(APC_ERR_INVALID, "max_rank / max_node_args out of range%s");
@@ -878,12 +919,7 @@ int slot_grid(const apc_problem* p, int per_block, unsigned* grid) {
 
 int launch_prepare(const apc_problem* p, double* table, bool do_nodes, double* compute,
                    double* per_arg, int32_t* status, hipStream_t stream) {
-  const int64_t tsize = table ? apc_pair_table_size(p) : 0;
-  int table_blocks = 0;
-  if (tsize > 0) {
-    int64_t b = (tsize + 255) / 256;
-    table_blocks = (int)(b > 2048 ? 2048 : b);
-  }
+  const int table_blocks = (table && p->table_size > 0) ? p->n_table_block : 0;
   const int node_blocks = do_nodes ? (p->n_comp_node + kNodesPerBlock - 1) / kNodesPerBlock : 0;
   if (table_blocks + node_blocks == 0) return 0;
   // LDS for the local-size staging (a CU has 160 KB); beyond 96 KB per block,

@@ -140,6 +140,9 @@ class CostEngine:
         p.run_len = up("run_len", run_len)
         p.run_table_off = up("run_table_off", run_table_off)
         p.table_size = int(run_table_off[-1])
+        tbr = g.table_block_runs()
+        p.n_table_block = tbr.shape[0]
+        p.table_block_run = up("table_block_run", tbr)
         self.problem = p
 
         E, NC = g.num_slots, g.num_compute

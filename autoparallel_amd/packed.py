@@ -304,10 +304,18 @@ class PackedGraph:
         offs, first, inv = np.unique(self.edge_src_list[hp], return_index=True, return_inverse=True)
         run_len = self.edge_ssrc[hp][first].astype(np.int32)
         assert (self.edge_ssrc[hp] == run_len[inv]).all(), "one run, two lengths"
+        # each run's table is padded to a multiple of 256 elements so that a
+        # 256-thread block of the table kernel never spans two runs
         run_table_off = np.zeros(offs.shape[0] + 1, np.int64)
-        np.cumsum(run_len.astype(np.int64) * nt, out=run_table_off[1:])
+        np.cumsum((run_len.astype(np.int64) * nt + 255) & ~255, out=run_table_off[1:])
         edge_table_off[hp] = run_table_off[:-1][inv]
         return offs.astype(np.int64), run_len, run_table_off, edge_table_off
+
+    def table_block_runs(self) -> np.ndarray:
+        """int32[table_size / 256]: the run each 256-element block of the row
+        table belongs to."""
+        _, _, off, _ = self.run_table()
+        return np.repeat(np.arange(off.shape[0] - 1, dtype=np.int32), np.diff(off) // 256)
 
     def chunk_edge_index(self) -> np.ndarray:
         """int32[num_slots / 16]: the edge that owns each 16-slot chunk (blocks

@@ -134,12 +134,15 @@ typedef struct apc_problem {
   int64_t n_default;
   const double* default_vals;
   /* row tables: run r is the S_src spec words at lists[run_list[r]]; its table
-   * is table[run_table_off[r] + t * run_len[r] + j] = cost(run[j] -> tuple t) */
+   * is table[run_table_off[r] + t * run_len[r] + j] = cost(run[j] -> tuple t);
+   * each run's table is padded to a multiple of 256 elements */
   int32_t n_run;
   const int64_t* run_list;
   const int32_t* run_len;
-  const int64_t* run_table_off; /* [n_run+1] */
+  const int64_t* run_table_off; /* [n_run+1], multiples of 256 */
   int64_t table_size;           /* doubles: run_table_off[n_run] */
+  int32_t n_table_block;        /* table_size / 256 */
+  const int32_t* table_block_run; /* [n_table_block] run owning elements [256 b, 256 b + 256) */
 } apc_problem;
 
 int apc_version(void);
