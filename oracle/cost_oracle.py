@@ -23,6 +23,7 @@ Python ints and floats (IEEE binary64, no fused operations):
   add_inf_cost_constraint / _set_objective / apply_prefetch_discount
                       autoparallel/optimize_sharding.py:803-885
   _compute_solution_cost                              same file :1056-1111
+  NCCL collective model (selected by Topo.nccl)       oracle/nccl_oracle.py
 
 Pinning (what each function is checked against, see tests/test_oracle_*.py):
   * redistribute_cost, estimate_strategy_comms_cost, compute_read_write_time,
@@ -68,8 +69,9 @@ class DeviceLimit:
 class Topo:
     """MeshTopoInfo (torch _collective_utils.py:236-278)."""
 
-    def __init__(self, mesh_shape: Sequence[int], devices_per_host: int):
+    def __init__(self, mesh_shape: Sequence[int], devices_per_host: int, nccl=None):
         ndim = len(mesh_shape)
+        self.nccl = nccl  # oracle.nccl_oracle.NcclConfig selects the NCCL model
         base_bw = 87.7
         self.mesh_shape = tuple(int(x) for x in mesh_shape)
         self.bw = [base_bw] * ndim
@@ -120,7 +122,12 @@ def all_to_all_cost(bytes_gb: float, topo: Topo, dim: int) -> float:
 
 
 def collective_comm_cost(collective: str, comm_bytes: int, topo: Topo, dim: int) -> float:
-    """collective_runtime_estimation.py:65-97, default (alpha-beta) branch."""
+    """collective_runtime_estimation.py:65-97: NCCL model when a topology
+    config is set (:85-86), otherwise the alpha-beta functions."""
+    if topo.nccl is not None:
+        from . import nccl_oracle
+
+        return nccl_oracle.comm_cost(collective, comm_bytes, topo.mesh_shape, dim, topo.nccl)
     g = comm_bytes / 1024**3
     if collective == "allgather":
         return allgather_cost(g, topo, dim)

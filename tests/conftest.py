@@ -17,3 +17,10 @@ def golden():
     import numpy as np
 
     return np.load(os.path.join(ROOT, "tests", "golden", "cost_vectors.npz"))
+
+
+@pytest.fixture(scope="session")
+def nccl_golden():
+    import numpy as np
+
+    return np.load(os.path.join(ROOT, "tests", "golden", "nccl_vectors.npz"))
