@@ -24,6 +24,58 @@ class ApcModel(C.Structure):
         ("tflops", C.c_double * NUM_DTYPES),
         ("order_mode", C.c_int32),
         ("reserved", C.c_int32),
+        ("nccl_plan", C.c_void_p),
+    ]
+
+
+NCCL_MAX_CAND = 10
+NCCL_TABLE_LEN = 24
+
+
+class ApcNcclConfig(C.Structure):
+    _fields_ = [
+        ("arch", C.c_int32),
+        ("num_nodes", C.c_int32),
+        ("gpus_per_node", C.c_int32),
+        ("num_channels", C.c_int32),
+        ("has_nvswitch", C.c_int32),
+        ("has_collnet", C.c_int32),
+        ("bw_intra", C.c_double),
+        ("bw_inter", C.c_double),
+        ("net_latency", C.c_double),
+    ]
+
+
+class ApcNcclCand(C.Structure):
+    _fields_ = [("lat", C.c_double), ("bw", C.c_double), ("flags", C.c_int32), ("proto", C.c_int32)]
+
+
+class ApcNcclDim(C.Structure):
+    _fields_ = [
+        ("n_ranks", C.c_int32),
+        ("n_nodes", C.c_int32),
+        ("ppn", C.c_int32),
+        ("n_channels", C.c_int32),
+        ("bw_intra", C.c_double),
+        ("bw_inter", C.c_double),
+        ("n_cand", C.c_int32 * 4),
+        ("cand", (ApcNcclCand * NCCL_MAX_CAND) * 4),
+        ("ring_corr", C.c_double * NCCL_TABLE_LEN),
+        ("a2a_remote", C.c_double),
+        ("a2a_log_nodes", C.c_int32),
+        ("reserved", C.c_int32),
+    ]
+
+
+class ApcNcclPlan(C.Structure):
+    _fields_ = [
+        ("ndim", C.c_int32),
+        ("reserved", C.c_int32),
+        ("dim", ApcNcclDim * MAX_MESH_DIMS),
+        ("tree_corr", (C.c_double * NCCL_TABLE_LEN) * 3),
+        ("nvls_tree_ramp", C.c_double * NCCL_TABLE_LEN),
+        ("full_mesh_ramp", C.c_double * NCCL_TABLE_LEN),
+        ("a2a_nic_ramp", C.c_double * NCCL_TABLE_LEN),
     ]
 
 
@@ -83,6 +135,7 @@ _SIGNATURES = {
     "apc_last_error": (C.c_char_p, []),
     "apc_mesh_topology": (C.c_int, [C.c_void_p, C.c_int32, C.c_int32, C.c_void_p, C.c_void_p]),
     "apc_device_limits": (C.c_int, [C.c_char_p, C.POINTER(ApcModel)]),
+    "apc_nccl_plan_build": (C.c_int, [C.POINTER(ApcNcclConfig), C.c_void_p, C.c_int32, C.POINTER(ApcNcclPlan)]),
     "apc_pair_table_size": (C.c_int64, [C.POINTER(ApcProblem)]),
     "apc_build_pair_table": (C.c_int, [C.POINTER(ApcProblem), C.c_void_p, C.c_void_p]),
     "apc_node_compute_costs": (

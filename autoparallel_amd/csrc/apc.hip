@@ -55,8 +55,66 @@ __device__ __forceinline__ double rw_time(double nbytes, double gmem_bw) {
 // allgather / reduce_scatter / allreduce / all_to_all cost for `nbytes` on
 // mesh dim i (torch _collective_utils.py:281-313;
 // collective_runtime_estimation.py:100-110).  kind: 0 AG, 1 A2A, 2 AR, 3 RS.
+__device__ __forceinline__ int log2i64(int64_t n) {  // _log2i (nccl_cost_model.py:287-291)
+  return n <= 0 ? 0 : 63 - __clzll((unsigned long long)n);
+}
+
+// _interp_correction (nccl_cost_model.py:294-315): linear interpolation of a
+// 24-entry table indexed by log2(nbytes >> 6).  The integer part of the
+// logarithm comes from the bit position, the fraction from log2 of the
+// mantissa in [1, 2); their sum is rounded once, as the host's log2 result is.
+__device__ __forceinline__ double interp_correction(const double* __restrict__ table, int64_t nbytes) {
+  const int64_t shifted = nbytes >> 6;
+  if (shifted <= 0) return table[0];
+  const int lo = log2i64(shifted);
+  if (lo + 1 >= APC_NCCL_TABLE_LEN) return table[APC_NCCL_TABLE_LEN - 1];
+  const double mant = (double)shifted / (double)(1ll << lo);
+  const double lv = (double)lo + log2(mant);
+  const double frac = lv - (double)lo;
+  return table[lo] * (1.0 - frac) + table[lo + 1] * frac;
+}
+
+// nccl_collective_time / nccl_all_to_all_cost (nccl_cost_model.py:1163-1313):
+// minimum over the candidates the host resolved for (mesh dim, collective),
+// each with its message-size corrections (_nccl_algo_time :577-613,
+// _table_algo_time :1035-1075).
+__device__ double nccl_collective_cost(int kind, int64_t nbytes, int i,
+                                       const apc_nccl_plan* __restrict__ plan) {
+  const apc_nccl_dim& d = plan->dim[i];
+  const int nc = d.n_cand[kind];
+  double best = INFINITY;
+  for (int c = 0; c < nc; ++c) {
+    const apc_nccl_cand& k = d.cand[kind][c];
+    double bw = k.bw, lat = k.lat, t;
+    const int f = k.flags;
+    if (f & APC_NC_NIC) {
+      const int lg = log2i64((nbytes / d.n_ranks) >> 6);
+      double corr = lg < APC_NCCL_TABLE_LEN ? plan->a2a_nic_ramp[lg] : 1.0;
+      if (d.a2a_log_nodes > 1 && corr < 1.0) corr = 1.0 - (1.0 - corr) / (double)d.a2a_log_nodes;
+      t = lat + (double)nbytes * d.a2a_remote / (1000.0 * bw * corr);
+    } else {
+      if (f & (APC_NC_TREE_CORR | APC_NC_TREE_CORR24)) {
+        const int ls = log2i64(nbytes >> 6);
+        if (ls < ((f & APC_NC_TREE_CORR24) ? 24 : 23)) bw *= plan->tree_corr[k.proto][ls];
+      }
+      if (f & (APC_NC_RING_CORR | APC_NC_NVLS_RAMP | APC_NC_FULL_MESH_RAMP)) {
+        const int64_t per_rank = nbytes / d.n_ranks;
+        if (f & APC_NC_RING_CORR) bw *= interp_correction(d.ring_corr, per_rank);
+        if (f & APC_NC_NVLS_RAMP) bw *= interp_correction(plan->nvls_tree_ramp, per_rank);
+        if ((f & APC_NC_FULL_MESH_RAMP) && log2i64(per_rank >> 6) < APC_NCCL_TABLE_LEN)
+          bw *= interp_correction(plan->full_mesh_ramp, per_rank);
+      }
+      if ((f & APC_NC_PLATEAU) && (double)nbytes / (double)(d.n_channels * d.n_ranks) >= 64.0) lat *= 1.4;
+      t = lat + (double)nbytes / (1000.0 * bw);
+    }
+    best = t < best ? t : best;
+  }
+  return best;
+}
+
 __device__ __forceinline__ double collective_cost(int kind, int64_t nbytes, int i,
                                                   const apc_model& m) {
+  if (m.nccl_plan != nullptr) return nccl_collective_cost(kind, nbytes, i, m.nccl_plan);
   double g = (double)nbytes / 1073741824.0;
   int n = m.mesh_shape[i];
   int hops = (kind == 2) ? 2 * (n - 1) : (n - 1);
@@ -951,6 +1009,10 @@ extern "C" {
 int apc_version(void) { return 2; }
 
 const char* apc_last_error(void) { return g_err; }
+
+__attribute__((visibility("hidden"))) void apc_internal_set_error(const char* msg) {
+  snprintf(g_err, sizeof(g_err), "%s", msg);
+}
 
 int apc_mesh_topology(const int32_t* mesh_shape, int32_t ndim, int32_t devices_per_host,
                       double* bw, double* lat) {

@@ -23,8 +23,8 @@ HIPCC_FLAGS = [
 
 
 def build(verbose: bool = True) -> str:
-    src = os.path.join(HERE, "apc.hip")
-    cmd = ["hipcc"] + HIPCC_FLAGS + [src, "-o", LIB]
+    srcs = [os.path.join(HERE, "apc.hip"), os.path.join(HERE, "nccl_plan.cpp")]
+    cmd = ["hipcc"] + HIPCC_FLAGS + srcs + ["-o", LIB]
     if verbose:
         print(" ".join(cmd), flush=True)
     subprocess.run(cmd, check=True)

@@ -41,6 +41,47 @@ def make_model(mesh_shape, devices_per_host: int, device_name: str, order_mode: 
     return m
 
 
+def nccl_config_struct(cfg) -> _lib.ApcNcclConfig:
+    """apc_nccl_config from any object with NCCLTopoConfig's fields
+    (autoparallel/cost_models/nccl_cost_model.py:67-82); ``arch`` may be an
+    int or an enum with an int ``value``."""
+    if isinstance(cfg, _lib.ApcNcclConfig):
+        return cfg
+    c = _lib.ApcNcclConfig()
+    c.arch = int(getattr(cfg.arch, "value", cfg.arch))
+    c.num_nodes = int(cfg.num_nodes)
+    c.gpus_per_node = int(cfg.gpus_per_node)
+    c.num_channels = int(cfg.num_channels) if cfg.num_channels is not None else 0
+    c.has_nvswitch = int(bool(cfg.has_nvswitch))
+    c.has_collnet = int(bool(cfg.has_collnet))
+    c.bw_intra = float(cfg.bw_intra)
+    c.bw_inter = float(cfg.bw_inter)
+    c.net_latency = float(cfg.net_latency)
+    return c
+
+
+def build_nccl_plan(cfg, mesh_shape) -> _lib.ApcNcclPlan:
+    """Host plan of the NCCL-tuning model for a mesh (apc_nccl_plan_build)."""
+    lib = _lib.load()
+    nd = len(mesh_shape)
+    shape = (C.c_int32 * MAX_MESH_DIMS)(*([int(x) for x in mesh_shape] + [1] * (MAX_MESH_DIMS - nd)))
+    plan = _lib.ApcNcclPlan()
+    c = nccl_config_struct(cfg)
+    _lib.check(lib.apc_nccl_plan_build(C.byref(c), C.addressof(shape), nd, C.byref(plan)), "apc_nccl_plan_build")
+    return plan
+
+
+def upload_nccl_plan(model: _lib.ApcModel, cfg, device) -> torch.Tensor:
+    """Build the plan for model's mesh, copy it to ``device`` and point
+    ``model.nccl_plan`` at the copy.  The caller keeps the returned tensor alive
+    for as long as the model is used."""
+    plan = build_nccl_plan(cfg, [model.mesh_shape[i] for i in range(model.ndim)])
+    raw = np.frombuffer(bytes(plan), dtype=np.uint8).copy()
+    t = torch.from_numpy(raw).to(device)
+    model.nccl_plan = t.data_ptr()
+    return t
+
+
 def detect_device_name(device=None) -> str:
     """Marketing name of the HIP device, as the reference's device table keys
     on it (autoparallel/cost_models/compute_estimation.py:258-275).  Hosts
@@ -64,6 +105,7 @@ class CostEngine:
         device_name: Optional[str] = None,
         use_table: Optional[bool] = None,
         order_mode: int = 0,
+        nccl_config=None,
     ):
         self.lib = _lib.load()
         self.g = g
@@ -91,7 +133,10 @@ class CostEngine:
             return t.data_ptr() if t.numel() else None
 
         p = _lib.ApcProblem()
-        p.model = make_model([int(x) for x in g.mesh_shape], g.devices_per_host, device_name, order_mode)
+        model = make_model([int(x) for x in g.mesh_shape], g.devices_per_host, device_name, order_mode)
+        if nccl_config is not None:  # NCCL-tuning collectives instead of alpha-beta
+            self._keep["nccl_plan"] = upload_nccl_plan(model, nccl_config, self.device)
+        p.model = model
         p.n_meta = g.meta_rank.shape[0]
         p.meta_rank = up("meta_rank", g.meta_rank)
         p.meta_shape = up("meta_shape", g.meta_shape)

@@ -81,7 +81,69 @@ typedef struct apc_model {
    * of redistribute_cost, :115-119) */
   int32_t order_mode;
   int32_t reserved;
+  /* NULL: alpha-beta collectives from mesh_bw / mesh_lat.  Otherwise a DEVICE
+   * copy of the plan that apc_nccl_plan_build fills: collectives are priced by
+   * the NCCL-tuning model (collective_runtime_estimation.py:44-62, 85-86). */
+  const struct apc_nccl_plan* nccl_plan;
 } apc_model;
+
+/* ---- NCCL-tuning collective model (autoparallel/cost_models/nccl_cost_model.py) ----
+ * The model is min over (algorithm, protocol) candidates of
+ *     latency + n_bytes / (1000 * bandwidth)
+ * where latency and bandwidth depend on the topology only, apart from a few
+ * message-size corrections.  apc_nccl_plan_build resolves, on the host, the
+ * size-independent part for every (mesh dim, collective); the kernels apply
+ * the size-dependent corrections per entry. */
+#define APC_NCCL_MAX_CAND 10
+#define APC_NCCL_TABLE_LEN 24
+/* candidate flags: size-dependent corrections applied on the device */
+#define APC_NC_TREE_CORR 1       /* bw *= tree_corr[proto][log2i(n >> 6)] if that index < 23 (:577-580, :1038-1041) */
+#define APC_NC_TREE_CORR24 2     /* same with index < 24 (:582-589)                                */
+#define APC_NC_RING_CORR 4       /* bw *= interp(dim's ring table, n / n_ranks) (:594-601)          */
+#define APC_NC_NVLS_RAMP 8       /* bw *= interp(nvls_tree_ramp, n / n_ranks) (:1046-1048)          */
+#define APC_NC_FULL_MESH_RAMP 16 /* bw *= interp(full_mesh_ramp, n / n_ranks) below 2^30 B/rank (:1053-1061) */
+#define APC_NC_PLATEAU 32        /* lat *= 1.4 if n / (n_channels * n_ranks) >= 64 (:603-611, :1064-1071) */
+#define APC_NC_NIC 64            /* all-to-all NIC path: lat + n * remote / (1000 * bw * corr) (:1260-1285) */
+
+typedef struct apc_nccl_config { /* NCCLTopoConfig (:67-82) */
+  int32_t arch; /* 0 Ampere, 1 Hopper, 2 Blackwell */
+  int32_t num_nodes;
+  int32_t gpus_per_node;
+  int32_t num_channels; /* 0 = architecture default */
+  int32_t has_nvswitch;
+  int32_t has_collnet;
+  double bw_intra; /* GB/s per GPU inside a node */
+  double bw_inter; /* GB/s per GPU between nodes */
+  double net_latency;
+} apc_nccl_config;
+
+typedef struct apc_nccl_cand {
+  double lat;    /* us */
+  double bw;     /* GB/s */
+  int32_t flags; /* APC_NC_* */
+  int32_t proto; /* 0 LL, 1 LL128, 2 Simple: row of tree_corr */
+} apc_nccl_cand;
+
+typedef struct apc_nccl_dim { /* MeshDimTopo (:85-92) + resolved candidates */
+  int32_t n_ranks, n_nodes, ppn, n_channels;
+  double bw_intra, bw_inter; /* per channel */
+  int32_t n_cand[4];         /* by collective: 0 allgather, 1 all_to_all, 2 allreduce, 3 reduce_scatter */
+  apc_nccl_cand cand[4][APC_NCCL_MAX_CAND];
+  double ring_corr[APC_NCCL_TABLE_LEN]; /* depth-scaled when n_nodes > 4 (:700-719) */
+  double a2a_remote;                    /* (n_ranks - ppn) / n_ranks            */
+  int32_t a2a_log_nodes;
+  int32_t reserved;
+} apc_nccl_dim;
+
+typedef struct apc_nccl_plan {
+  int32_t ndim;
+  int32_t reserved;
+  apc_nccl_dim dim[APC_MAX_MESH_DIMS];
+  double tree_corr[3][APC_NCCL_TABLE_LEN];
+  double nvls_tree_ramp[APC_NCCL_TABLE_LEN];
+  double full_mesh_ramp[APC_NCCL_TABLE_LEN];
+  double a2a_nic_ramp[APC_NCCL_TABLE_LEN];
+} apc_nccl_plan;
 
 /* The packed problem (see autoparallel_amd/packed.py for the layout). */
 typedef struct apc_problem {
@@ -161,6 +223,15 @@ int apc_mesh_topology(const int32_t* mesh_shape, int32_t ndim, int32_t devices_p
  * Returns APC_ERR_UNSUPPORTED for an unknown device name (the reference raises
  * ValueError there). */
 int apc_device_limits(const char* device_name, apc_model* model);
+
+/* Host helper.  Replaces derive_mesh_dim_topo (nccl_cost_model.py:1001-1021),
+ * _compute_algo_bw (:323-465), _compute_algo_latency (:473-551), the candidate
+ * selection of nccl_collective_time (:1163-1212, :1081-1160), _eligible_algos /
+ * _eligible_protos (:616-649), _depth_scaled_ring_correction (:700-719) and the
+ * size-independent part of nccl_all_to_all_cost (:1215-1313).  plan: host
+ * memory; copy it to the device and point apc_model.nccl_plan at the copy. */
+int apc_nccl_plan_build(const apc_nccl_config* cfg, const int32_t* mesh_shape, int32_t ndim,
+                        struct apc_nccl_plan* plan);
 
 /* Number of doubles of the row table apc_build_pair_table fills
  * (= p->table_size: sum over runs of run_len * n_tuple). */
@@ -257,8 +328,10 @@ int apc_local_shapes(const apc_model* model, int32_t n, const int32_t* rank, con
                      const int64_t* stride, const uint8_t* plc, int64_t* out_shape,
                      int64_t* out_stride, void* stream);
 
-/* Replaces collective_comm_cost, default model
- * (autoparallel/cost_models/collective_runtime_estimation.py:65-110) for n
+/* Replaces collective_comm_cost
+ * (autoparallel/cost_models/collective_runtime_estimation.py:65-110), default
+ * model or, with model->nccl_plan set, _nccl_comm_cost (:44-62) and
+ * nccl_collective_time / nccl_all_to_all_cost (nccl_cost_model.py:1163-1313), for n
  * queries: kind[i] 0 allgather, 1 all_to_all, 2 allreduce, 3 reduce_scatter
  * (anything else costs 0.0), nbytes[i], mesh dim[i] -> out[i] microseconds. */
 int apc_collective_costs(const apc_model* model, int32_t n, const int32_t* kind,

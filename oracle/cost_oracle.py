@@ -348,10 +348,10 @@ class GraphOracle:
     memo caches of the reference (optimize_sharding.py:481-552;
     collective_runtime_estimation.py:239-262; compute_estimation.py:449-492)."""
 
-    def __init__(self, g, dev: Optional[DeviceLimit] = None):
+    def __init__(self, g, dev: Optional[DeviceLimit] = None, nccl=None):
         self.g = g
         self.dev = dev or DeviceLimit()
-        self.topo = Topo([int(x) for x in g.mesh_shape], g.devices_per_host)
+        self.topo = Topo([int(x) for x in g.mesh_shape], g.devices_per_host, nccl=nccl)
         self.ndim = len(self.topo.mesh_shape)
         self._comm_cache: Dict[tuple, float] = {}
         self._compute_cache: Dict[tuple, float] = {}
