@@ -136,6 +136,10 @@ _SIGNATURES = {
     "apc_mesh_topology": (C.c_int, [C.c_void_p, C.c_int32, C.c_int32, C.c_void_p, C.c_void_p]),
     "apc_device_limits": (C.c_int, [C.c_char_p, C.POINTER(ApcModel)]),
     "apc_nccl_plan_build": (C.c_int, [C.POINTER(ApcNcclConfig), C.c_void_p, C.c_int32, C.POINTER(ApcNcclPlan)]),
+    "apc_nccl_plan_for_topo": (
+        C.c_int,
+        [C.POINTER(ApcNcclConfig), C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_double, C.c_double,
+         C.POINTER(ApcNcclPlan)]),
     "apc_pair_table_size": (C.c_int64, [C.POINTER(ApcProblem)]),
     "apc_build_pair_table": (C.c_int, [C.POINTER(ApcProblem), C.c_void_p, C.c_void_p]),
     "apc_node_compute_costs": (

@@ -12,3 +12,13 @@ from .compute_estimation import (  # noqa: F401
     estimate_strategy_runtime_cost,
     reset_compute_cost_cache,
 )
+from .nccl_cost_model import (  # noqa: F401
+    GpuArch,
+    MeshDimTopo,
+    NCCLTopoConfig,
+    a100_topo_config,
+    derive_mesh_dim_topo,
+    detect_nccl_topo_config,
+    gb200_topo_config,
+    h100_topo_config,
+)

@@ -40,11 +40,10 @@ def _device_name() -> str:
 
 
 def set_nccl_topo_config(config) -> None:
+    """Select the NCCL-tuning collective model (an NCCLTopoConfig) or, with
+    None, the default alpha-beta model.  Clears the comm-cost memo, as the
+    reference does (:34-38)."""
     global _nccl_topo_config
-    if config is not None:
-        raise NotImplementedError(
-            "the NCCL cost model is not built yet; the default (alpha-beta) model is what the "
-            "reference itself selects on MI355X")
     _nccl_topo_config = config
     _comms_cost_cache.clear()
 
@@ -68,7 +67,8 @@ def comms_cost_matrix(src_specs: Sequence, tgt_specs: Sequence, order_mode: int 
                         inputs=[], default_rows=[[[0.0]] for _ in src_words]))
     b.add_node(NodeDesc("tgt", in_specs=[[w] for w in tgt_words], out_specs=[[w] for w in tgt_words], inputs=[0]))
     g = b.pack()
-    eng = CostEngine(g, device_name=_device_name(), use_table=False, order_mode=order_mode)
+    eng = CostEngine(g, device_name=_device_name(), use_table=False, order_mode=order_mode,
+                     nccl_config=_nccl_topo_config)
     eng.build(clamp_inf=False)
     comm = eng.results()["comm"]
     base = int(g.edge_off[1])
@@ -113,6 +113,10 @@ def collective_comm_cost(collective: str, comm_bytes: int, mesh_shape: Tuple[int
     """Cost in microseconds of one collective on one mesh dim.  ``mesh_topo``
     (a torch MeshTopoInfo) supplies per-dim bandwidth/latency when given;
     otherwise they are derived from ``devices_per_host``."""
+    if _nccl_topo_config is not None:
+        from .nccl_cost_model import nccl_mesh_collective_cost
+
+        return nccl_mesh_collective_cost(collective, comm_bytes, tuple(mesh_shape), mesh_dim, _nccl_topo_config)
     lib = _lib.load()
     dph = devices_per_host if devices_per_host is not None else (_settings["devices_per_host"] or 1)
     model = make_model(tuple(mesh_shape), dph, _device_name())

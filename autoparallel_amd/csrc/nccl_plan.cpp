@@ -6,6 +6,7 @@
 // and pow() is the same libm call CPython's float ** makes.
 #include <math.h>
 #include <stdint.h>
+#include <stdio.h>
 #include <string.h>
 
 #include "apc.h"
@@ -349,24 +350,60 @@ void plan_all_to_all(apc_nccl_dim& d, const Topo& t, const apc_nccl_config& c) {
   push(d, slot, ring_steps_latency(kSimple, t.n_ranks, n_inter, t, c), bus, 0, kSimple);
 }
 
-}  // namespace
+bool config_ok(const apc_nccl_config* cfg, const char* who) {
+  if (cfg && cfg->arch >= 0 && cfg->arch <= 2 && cfg->gpus_per_node >= 1 && cfg->num_channels >= 0) return true;
+  char msg[160];
+  snprintf(msg, sizeof(msg), "%s: config must have arch 0..2, gpus_per_node >= 1, num_channels >= 0", who);
+  apc_internal_set_error(msg);
+  return false;
+}
 
-extern "C" int apc_nccl_plan_build(const apc_nccl_config* cfg, const int32_t* mesh_shape, int32_t ndim,
-                                   apc_nccl_plan* plan) {
-  if (!cfg || !mesh_shape || !plan || ndim < 1 || ndim > APC_MAX_MESH_DIMS) {
-    apc_internal_set_error("apc_nccl_plan_build: null argument or mesh rank outside 1..4");
-    return APC_ERR_INVALID;
-  }
-  if (cfg->arch < 0 || cfg->arch > 2 || cfg->gpus_per_node < 1 || cfg->num_channels < 0) {
-    apc_internal_set_error("apc_nccl_plan_build: arch must be 0..2, gpus_per_node >= 1, num_channels >= 0");
-    return APC_ERR_INVALID;
-  }
+void init_plan(apc_nccl_plan* plan, int ndim) {
   memset(plan, 0, sizeof(*plan));
   plan->ndim = ndim;
   memcpy(plan->tree_corr, kTreeCorr, sizeof(kTreeCorr));
   memcpy(plan->nvls_tree_ramp, kNvlsTreeRamp, sizeof(kNvlsTreeRamp));
   memcpy(plan->full_mesh_ramp, kFullMeshRamp, sizeof(kFullMeshRamp));
   memcpy(plan->a2a_nic_ramp, kA2aNicRamp, sizeof(kA2aNicRamp));
+}
+
+// candidates and tables of one communicator
+void plan_dim(apc_nccl_dim& d, const Topo& t, const apc_nccl_config& cfg) {
+  d.n_ranks = t.n_ranks;
+  d.n_nodes = t.n_nodes;
+  d.ppn = t.ppn;
+  d.n_channels = t.nch;
+  d.bw_intra = t.bw_intra;
+  d.bw_inter = t.bw_inter;
+  // ring correction table of this communicator (:596-599, :700-719)
+  const double e = 1.0 + 0.2 * (double)(log2i(t.n_nodes) - 2);
+  for (int k = 0; k < APC_NCCL_TABLE_LEN; ++k) {
+    double corr = kRingCorr[k];
+    if (t.n_nodes > 4) {
+      if (corr < 1.0) corr = pow(corr, e);
+      if (k > 0) corr = pymin(corr, 2.0 * d.ring_corr[k - 1]);
+    }
+    d.ring_corr[k] = corr;
+  }
+  // One rank means zero ring steps: the reference's algorithm loop divides by
+  // them (ZeroDivisionError); only its measured-point paths are defined there.
+  // Undefined combinations keep zero candidates (cost +inf).
+  const bool measured = (cfg.arch == kHopper || cfg.arch == kBlackwell) && cfg.has_nvswitch && t.n_nodes == 1;
+  if (t.n_ranks >= 2 || measured)
+    for (int f = 0; f < 3; ++f) plan_collective(d, f, t, cfg);
+  plan_all_to_all(d, t, cfg);
+}
+
+}  // namespace
+
+extern "C" int apc_nccl_plan_build(const apc_nccl_config* cfg, const int32_t* mesh_shape, int32_t ndim,
+                                   apc_nccl_plan* plan) {
+  if (!mesh_shape || !plan || ndim < 1 || ndim > APC_MAX_MESH_DIMS) {
+    apc_internal_set_error("apc_nccl_plan_build: null argument or mesh rank outside 1..4");
+    return APC_ERR_INVALID;
+  }
+  if (!config_ok(cfg, "apc_nccl_plan_build")) return APC_ERR_INVALID;
+  init_plan(plan, ndim);
   for (int i = 0; i < ndim; ++i) {
     if (mesh_shape[i] < 1) {
       apc_internal_set_error("apc_nccl_plan_build: mesh dim size < 1");
@@ -384,30 +421,27 @@ extern "C" int apc_nccl_plan_build(const apc_nccl_config* cfg, const int32_t* me
     t.nch = cfg->num_channels > 0 ? cfg->num_channels : kDefaultChannels[cfg->arch];
     t.bw_intra = cfg->bw_intra / (double)t.nch;
     t.bw_inter = cfg->bw_inter / (double)t.nch;
-    apc_nccl_dim& d = plan->dim[i];
-    d.n_ranks = t.n_ranks;
-    d.n_nodes = t.n_nodes;
-    d.ppn = t.ppn;
-    d.n_channels = t.nch;
-    d.bw_intra = t.bw_intra;
-    d.bw_inter = t.bw_inter;
-    // ring correction table of this dim (:596-599, :700-719)
-    const double e = 1.0 + 0.2 * (double)(log2i(t.n_nodes) - 2);
-    for (int k = 0; k < APC_NCCL_TABLE_LEN; ++k) {
-      double corr = kRingCorr[k];
-      if (t.n_nodes > 4) {
-        if (corr < 1.0) corr = pow(corr, e);
-        if (k > 0) corr = pymin(corr, 2.0 * d.ring_corr[k - 1]);
-      }
-      d.ring_corr[k] = corr;
-    }
-    // A mesh dim of one device has zero ring steps: the reference's algorithm
-    // loop divides by them (ZeroDivisionError); only its measured-point paths are
-    // defined there.  Undefined combinations keep zero candidates (cost +inf).
-    const bool measured = (cfg->arch == kHopper || cfg->arch == kBlackwell) && cfg->has_nvswitch && t.n_nodes == 1;
-    if (t.n_ranks >= 2 || measured)
-      for (int f = 0; f < 3; ++f) plan_collective(d, f, t, *cfg);
-    plan_all_to_all(d, t, *cfg);
+    plan_dim(plan->dim[i], t, *cfg);
   }
+  return 0;
+}
+
+extern "C" int apc_nccl_plan_for_topo(const apc_nccl_config* cfg, int32_t n_ranks, int32_t n_nodes, int32_t ppn,
+                                      int32_t n_channels, double bw_intra, double bw_inter,
+                                      apc_nccl_plan* plan) {
+  if (!plan || n_ranks < 1 || n_nodes < 1 || ppn < 1 || n_channels < 1) {
+    apc_internal_set_error("apc_nccl_plan_for_topo: null plan or non-positive topology field");
+    return APC_ERR_INVALID;
+  }
+  if (!config_ok(cfg, "apc_nccl_plan_for_topo")) return APC_ERR_INVALID;
+  init_plan(plan, 1);
+  Topo t;
+  t.n_ranks = n_ranks;
+  t.n_nodes = n_nodes;
+  t.ppn = ppn;
+  t.nch = n_channels;
+  t.bw_intra = bw_intra;
+  t.bw_inter = bw_inter;
+  plan_dim(plan->dim[0], t, *cfg);
   return 0;
 }

@@ -270,7 +270,7 @@ class ShardingOptimizer:
         self._core = PackedShardingOptimizer(
             self._packed, roles=self._packed.roles,
             force_grad_reduce_in_higher_precision=self.force_grad_reduce_in_higher_precision,
-            device_name=self._device_name)
+            device_name=self._device_name, nccl_config=_cre.get_nccl_topo_config())
         self.prob = self._core.prob
         self._write_back_redistribute_costs()
         return DecisionVars(self)

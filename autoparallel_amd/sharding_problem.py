@@ -68,6 +68,7 @@ class PackedShardingOptimizer:
         coefficients: Optional[Coefficients] = None,
         device: str = "cuda",
         device_name: Optional[str] = None,
+        nccl_config=None,
     ):
         self.g = g
         self.roles = roles or getattr(g, "roles", None) or GraphRoles()
@@ -76,7 +77,7 @@ class PackedShardingOptimizer:
         if coefficients is None:
             from .engine import CostEngine  # the HIP path; raises without the library / a GPU
 
-            self.engine = CostEngine(g, device=device, device_name=device_name)
+            self.engine = CostEngine(g, device=device, device_name=device_name, nccl_config=nccl_config)
             self.engine.build(clamp_inf=True)
             coefficients = Coefficients.from_engine(self.engine)
         self.coef = coefficients

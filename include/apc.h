@@ -233,6 +233,15 @@ int apc_device_limits(const char* device_name, apc_model* model);
 int apc_nccl_plan_build(const apc_nccl_config* cfg, const int32_t* mesh_shape, int32_t ndim,
                         struct apc_nccl_plan* plan);
 
+/* Host helper.  As apc_nccl_plan_build for ONE communicator whose topology the
+ * caller states (the MeshDimTopo argument of nccl_allgather_cost /
+ * nccl_allreduce_cost / nccl_reduce_scatter_cost / nccl_all_to_all_cost,
+ * nccl_cost_model.py:1215-1336): fills plan->dim[0], plan->ndim = 1.
+ * bw_intra / bw_inter are per channel, as MeshDimTopo holds them. */
+int apc_nccl_plan_for_topo(const apc_nccl_config* cfg, int32_t n_ranks, int32_t n_nodes, int32_t ppn,
+                           int32_t n_channels, double bw_intra, double bw_inter,
+                           struct apc_nccl_plan* plan);
+
 /* Number of doubles of the row table apc_build_pair_table fills
  * (= p->table_size: sum over runs of run_len * n_tuple). */
 int64_t apc_pair_table_size(const apc_problem* p);

@@ -126,8 +126,69 @@ def test_cost_models_scalar_api(mesh, golden):
 
     spec = DTensorSpec(mesh, (Shard(0), Shard(1)), tensor_meta=TensorMeta(torch.Size((64, 36)), (36, 1), torch.float32))
     assert _get_sharded_shape_stride(spec) == ([32, 9], [36, 1])
-    with pytest.raises(NotImplementedError):
-        cm.set_nccl_topo_config(object())
+
+
+def test_nccl_model_through_reference_api(mesh):
+    """set_nccl_topo_config switches every entry point to the NCCL model; the
+    reference's own tests call these functions the same way
+    (tests/test_nccl_cost_model.py there)."""
+    from torch.distributed.tensor._dtensor_spec import DTensorSpec, TensorMeta
+    from torch.distributed.tensor.placement_types import Partial, Replicate, Shard
+
+    from autoparallel_amd import cost_models as cm
+    from autoparallel_amd.cost_models import nccl_cost_model as ncm
+    from oracle import nccl_oracle as N
+
+    cm.configure(devices_per_host=8, device_name="AMD Instinct MI355X")
+    cfg = cm.h100_topo_config(num_nodes=2)
+    ocfg = N.h100_config(num_nodes=2)
+    t = cm.derive_mesh_dim_topo(cfg, (2, 8), 0)
+    ot = N.derive_dim_topo(ocfg, (2, 8), 0)
+    assert (t.n_ranks, t.n_nodes, t.ppn, t.n_channels, t.bw_intra, t.bw_inter) == (
+        ot.n_ranks, ot.n_nodes, ot.ppn, ot.n_channels, ot.bw_intra, ot.bw_inter)
+    t16 = cm.derive_mesh_dim_topo(cfg, (16,), 0)
+    o16 = N.derive_dim_topo(ocfg, (16,), 0)
+    for nb in (1 << 12, (1 << 21) + 5, 1 << 30):
+        assert np.isclose(ncm.nccl_allreduce_cost(nb, t16, cfg), N.collective_time(N.AR, nb, o16, ocfg), rtol=1e-12)
+        assert np.isclose(ncm.nccl_allgather_cost(nb, t16, cfg), N.collective_time(N.AG, nb, o16, ocfg), rtol=1e-12)
+        assert np.isclose(ncm.nccl_reduce_scatter_cost(nb, t16, cfg), N.collective_time(N.RS, nb, o16, ocfg), rtol=1e-12)
+        assert np.isclose(ncm.nccl_all_to_all_cost(nb, t16, cfg), N.all_to_all_time(nb, o16, ocfg), rtol=1e-12)
+    # a hand-made topology with no tuning-table row falls back to the algorithm loop
+    odd = ncm.MeshDimTopo(24, 3, 8, 20.0, 50.0 / 16, 16)
+    want = N.collective_time(N.AR, 1 << 30, N.DimTopo(24, 3, 8, 20.0, 50.0 / 16, 16), ocfg)
+    assert np.isclose(ncm.nccl_allreduce_cost(1 << 30, odd, cfg), want, rtol=1e-12)
+    # the module-level switch
+    shape = (256, 512)
+    tm = TensorMeta(torch.Size(shape), (512, 1), torch.bfloat16)
+    topo, dev = O.Topo((2, 4), 8, nccl=N.h100_config(num_nodes=1)), O.DeviceLimit()
+    code = {Replicate(): 0, Shard(0): 0x40, Shard(1): 0x41, Partial(): 0x80}
+    try:
+        cm.set_nccl_topo_config(cm.h100_topo_config(num_nodes=1))
+        assert cm.get_nccl_topo_config() is not None
+        for a in [(Shard(0), Shard(1)), (Partial(), Partial()), (Shard(1), Partial())]:
+            for b in [(Replicate(), Replicate()), (Shard(1), Shard(0)), (Shard(0), Shard(0))]:
+                s, tt = DTensorSpec(mesh, a, tensor_meta=tm), DTensorSpec(mesh, b, tensor_meta=tm)
+                got = cm.estimate_strategy_comms_cost(s, tt)
+                want = O.estimate_strategy_comms_cost(tuple(code[p] for p in a), shape, (512, 1), 2,
+                                                      tuple(code[p] for p in b), topo, dev)
+                assert (np.isinf(got) and np.isinf(want)) or np.isclose(got, want, rtol=1e-12), (a, b, got, want)
+        got = cm.collective_comm_cost("allreduce", 1 << 26, (2, 4), 1)
+        assert got == N.comm_cost("allreduce", 1 << 26, (2, 4), 1, N.h100_config(num_nodes=1))
+    finally:
+        cm.set_nccl_topo_config(None)
+    alpha = cm.collective_comm_cost("allreduce", 1 << 26, (2, 4), 1, devices_per_host=8)
+    assert alpha == O.collective_comm_cost("allreduce", 1 << 26, O.Topo((2, 4), 8), 1)
+    # presets and detection
+    assert cm.a100_topo_config().bw_intra == 87.7 and cm.gb200_topo_config().gpus_per_node == 72
+
+    class _M:
+        def size(self):
+            return 16
+
+    assert cm.detect_nccl_topo_config(_M(), device_name="AMD Instinct MI355X") is None
+    h = cm.detect_nccl_topo_config(_M(), device_name="NVIDIA H100 80GB HBM3")
+    assert (h.arch, h.num_nodes, h.gpus_per_node, h.has_nvswitch) == (cm.GpuArch.HOPPER, 2, 8, True)
+    assert cm.detect_nccl_topo_config(_M(), device_name="NVIDIA GB200") is None  # 16 % 72 != 0
 
 
 def test_runtime_cost_api_matches_reference_vectors(mesh, golden):
