@@ -161,6 +161,14 @@ _SIGNATURES = {
         [C.POINTER(ApcProblem), C.c_void_p, C.c_double, C.c_void_p, C.c_void_p, C.c_void_p,
          C.c_void_p, C.c_void_p]),
     "apc_objective_coeffs": (C.c_int, [C.POINTER(ApcProblem), C.c_void_p, C.c_void_p, C.c_void_p]),
+    "apc_export_decision_vars": (
+        C.c_int,
+        [C.POINTER(ApcProblem), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+         C.c_void_p, C.c_void_p]),
+    "apc_solution_terms": (
+        C.c_int,
+        [C.POINTER(ApcProblem), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+         C.c_void_p, C.c_void_p]),
     "apc_score_assignments": (
         C.c_int,
         [C.POINTER(ApcProblem), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,

@@ -699,6 +699,66 @@ objective_kernel(apc_problem p, const double* __restrict__ cost, double* __restr
 }
 
 // ---------------------------------------------------------------------------
+// Kernel: packed twin of the decision variables, in the reference's insertion
+// order (node, out_idx, argi, inp_idx): row of entry (e, o, j) is
+// row_base[e] + o * row_stride[e] + j, where row_stride is the node's sum of
+// S_src over its arguments.  One lane per slot; the lanes of a run of inp_idx
+// write consecutive rows.
+// ---------------------------------------------------------------------------
+__global__ void __launch_bounds__(kBlock)
+export_kernel(apc_problem p, const double* __restrict__ per_arg, const double* __restrict__ comm,
+              const uint8_t* __restrict__ flags, const int64_t* __restrict__ row_base,
+              const int32_t* __restrict__ row_stride, int32_t* __restrict__ keys,
+              double* __restrict__ vals) {
+  const int64_t idx = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (idx >= p.n_slot) return;
+  const int e = p.chunk_edge[idx >> APC_CHUNK_SHIFT];
+  const apc_edge ed = p.edges[e];
+  const int64_t local = idx - ed.off;
+  if (local >= (int64_t)ed.ssrc * ed.sdst) return;
+  const uint32_t o = (uint32_t)local / (uint32_t)ed.ssrc;
+  const uint32_t j = (uint32_t)local - o * (uint32_t)ed.ssrc;
+  const int64_t row = row_base[e] + (int64_t)o * row_stride[e] + j;
+  int4 k;
+  k.x = ed.node;
+  k.y = e - p.node_edge_off[ed.node];
+  k.z = (int)o;
+  k.w = (int)j;
+  *reinterpret_cast<int4*>(keys + row * 4) = k;
+  double* v = vals + row * 3;
+  v[0] = per_arg[ed.comp_base + o];
+  v[1] = comm[idx];
+  v[2] = (double)(flags[idx] & APC_ENTRY_TRANSITION);
+}
+
+// The selected entry of every edge under one assignment (out_idx per node):
+// terms[e] = (per-arg compute, comm, transition, cost) of entry
+// (e, assign[node], assign[producer] or 0) and slot[e] = its slot.
+__global__ void __launch_bounds__(kBlock)
+solution_terms_kernel(apc_problem p, const double* __restrict__ per_arg,
+                      const double* __restrict__ comm, const double* __restrict__ cost,
+                      const uint8_t* __restrict__ flags, const uint16_t* __restrict__ assign,
+                      double* __restrict__ terms, int64_t* __restrict__ slot) {
+  const int e = blockIdx.x * kBlock + threadIdx.x;
+  if (e >= p.n_edge) return;
+  const apc_edge ed = p.edges[e];
+  const uint32_t o = assign[ed.node];
+  const uint32_t j = ed.src_node >= 0 ? assign[ed.src_node] : 0u;
+  double* t = terms + (size_t)e * 4;
+  if (o >= (uint32_t)ed.sdst || j >= (uint32_t)ed.ssrc) {  // not a strategy index of this edge
+    t[0] = t[1] = t[2] = t[3] = NAN;
+    slot[e] = -1;
+    return;
+  }
+  const int64_t idx = ed.off + (int64_t)o * ed.ssrc + j;
+  t[0] = per_arg[ed.comp_base + o];
+  t[1] = comm[idx];
+  t[2] = (double)(flags[idx] & APC_ENTRY_TRANSITION);
+  t[3] = cost[idx];
+  slot[e] = idx;
+}
+
+// ---------------------------------------------------------------------------
 // Kernel: batch scoring.  One lane per assignment; the lane walks the graph in
 // node order then argument order, so every sum has the reference's order.
 // ---------------------------------------------------------------------------
@@ -1135,6 +1195,32 @@ int apc_objective_coeffs(const apc_problem* p, const double* cost, double* obj, 
   hipLaunchKernelGGL(objective_kernel, dim3(grid), dim3(kBlock), 0, (hipStream_t)stream, *p, cost,
                      obj);
   return check_launch("objective_kernel");
+}
+
+int apc_export_decision_vars(const apc_problem* p, const double* per_arg, const double* comm,
+                             const uint8_t* flags, const int64_t* row_base,
+                             const int32_t* row_stride, int32_t* keys, double* vals, void* stream) {
+  if (int rc = validate_problem(p)) return rc;
+  if (p->n_slot == 0) return 0;
+  if (!per_arg || !comm || !flags || !row_base || !row_stride || !keys || !vals)
+    return fail(APC_ERR_INVALID, "apc_export_decision_vars: null argument%s");
+  unsigned grid;
+  if (int rc = slot_grid(p, kBlock, &grid)) return rc;
+  hipLaunchKernelGGL(export_kernel, dim3(grid), dim3(kBlock), 0, (hipStream_t)stream, *p, per_arg,
+                     comm, flags, row_base, row_stride, keys, vals);
+  return check_launch("export_kernel");
+}
+
+int apc_solution_terms(const apc_problem* p, const double* per_arg, const double* comm,
+                       const double* cost, const uint8_t* flags, const uint16_t* assign,
+                       double* terms, int64_t* slot, void* stream) {
+  if (int rc = validate_problem(p)) return rc;
+  if (p->n_edge == 0) return 0;
+  if (!per_arg || !comm || !cost || !flags || !assign || !terms || !slot)
+    return fail(APC_ERR_INVALID, "apc_solution_terms: null argument%s");
+  hipLaunchKernelGGL(solution_terms_kernel, dim3((p->n_edge + kBlock - 1) / kBlock), dim3(kBlock), 0,
+                     (hipStream_t)stream, *p, per_arg, comm, cost, flags, assign, terms, slot);
+  return check_launch("solution_terms_kernel");
 }
 
 // Launches in chunks: beyond a few hundred thousand lanes walking the graph at

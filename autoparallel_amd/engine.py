@@ -262,6 +262,20 @@ class CostEngine:
         self.built = True
         return self
 
+    def load_results(self, comm, cost, flags, compute, per_arg):
+        """Adopt coefficient arrays computed earlier (a saved optimizer): host
+        arrays of num_slots / num_compute elements are copied to the device and
+        the engine counts as built.  Nothing is recomputed."""
+        g = self.g
+        assert len(comm) == len(cost) == len(flags) == g.num_slots and len(compute) == len(per_arg) == g.num_compute
+        self.comm.copy_(torch.from_numpy(np.ascontiguousarray(comm, np.float64)))
+        self.cost.copy_(torch.from_numpy(np.ascontiguousarray(cost, np.float64)))
+        self.flags.copy_(torch.from_numpy(np.ascontiguousarray(flags, np.uint8)))
+        self.compute.copy_(torch.from_numpy(np.ascontiguousarray(compute, np.float64)))
+        self.per_arg.copy_(torch.from_numpy(np.ascontiguousarray(per_arg, np.float64)))
+        self.built = True
+        return self
+
     def check_status(self):
         if int(self.status.item()) != 0:
             raise ValueError(
@@ -303,6 +317,43 @@ class CostEngine:
             "apc_score_assignments",
         )
         return out
+
+    def export_decision_vars(self):
+        """(keys int32[E, 4], vals float64[E, 3]) on the device: the packed twin
+        of the reference's ``decision_vars`` in its insertion order."""
+        assert self.built
+        if "export_row_base" not in self._keep:
+            base, stride = self.g.export_rows()
+            self._keep["export_row_base"] = torch.from_numpy(base).to(self.device)
+            self._keep["export_row_stride"] = torch.from_numpy(stride).to(self.device)
+        E = self.g.num_entries
+        keys = torch.empty((E, 4), dtype=torch.int32, device=self.device)
+        vals = torch.empty((E, 3), dtype=torch.float64, device=self.device)
+        _lib.check(
+            self.lib.apc_export_decision_vars(
+                C.byref(self.problem), self._ptr(self.per_arg), self._ptr(self.comm), self._ptr(self.flags),
+                self._ptr(self._keep["export_row_base"]), self._ptr(self._keep["export_row_stride"]),
+                self._ptr(keys), self._ptr(vals), self._stream()),
+            "apc_export_decision_vars",
+        )
+        return keys, vals
+
+    def solution_terms(self, assign: torch.Tensor):
+        """assign: int16/uint16 [n_node] on the device -> (terms float64
+        [n_edge, 4] = compute, comm, transition, cost of each edge's selected
+        entry; slot int64[n_edge])."""
+        assert self.built
+        assert assign.dim() == 1 and assign.shape[0] == self.g.num_nodes and assign.is_contiguous()
+        assert assign.dtype in (torch.int16, torch.uint16) and assign.device == self.comm.device
+        terms = torch.empty((self.g.num_edges, 4), dtype=torch.float64, device=self.device)
+        slot = torch.empty(self.g.num_edges, dtype=torch.int64, device=self.device)
+        _lib.check(
+            self.lib.apc_solution_terms(
+                C.byref(self.problem), self._ptr(self.per_arg), self._ptr(self.comm), self._ptr(self.cost),
+                self._ptr(self.flags), self._ptr(assign), self._ptr(terms), self._ptr(slot), self._stream()),
+            "apc_solution_terms",
+        )
+        return terms, slot
 
     def score_random(self, seed: int, first: int, count: int) -> torch.Tensor:
         assert self.built

@@ -381,3 +381,72 @@ class ShardingOptimizer:
         text = f"{node} arg {arg}: cost[out_idx][inp_idx]\n{block.reshape(-1, int(g.edge_ssrc[e]))}"
         print(text)
         return text
+
+    # -- export / persistence ------------------------------------------------------------------
+    def _node_info(self) -> List[Dict[str, Any]]:
+        """Per-node fields only the FX graph carries (export_json.py:362-407 of
+        the reference): op, phase, placeholder kind, source line."""
+        import re
+
+        out = []
+        for node in self.nodes:
+            info: Dict[str, Any] = {"op": str(node.target) if node.op == "call_function" else node.op}
+            desc = type(node.meta.get("desc")).__name__ if node.meta.get("desc") is not None else None
+            kind = {"ParamAOTInput": "param", "BufferAOTInput": "buffer", "TangentAOTInput": "tangent",
+                    "PlainAOTInput": "input"}.get(desc)
+            if node.op == "placeholder" and kind:
+                info["placeholder_kind"] = kind
+            tag = node.meta.get("partitioner_tag")
+            info["phase"] = "backward" if tag == "is_backward" or kind == "tangent" else "forward"
+            st = node.meta.get("stack_trace")
+            if st:
+                frames = re.findall(r'File "([^"]+)", line (\d+), in (\w+)\n\s+(.*)', st)
+                if frames:
+                    f, line, fn, code = frames[-1]
+                    info["source"] = {"file": f, "line": int(line), "func": fn, "code": code.strip()}
+            out.append(info)
+        return out
+
+    def get_json(self) -> Dict[str, Any]:
+        from . import export_json
+
+        self._core.mesh_dim_names = list(self.mesh.mesh_dim_names) if self.mesh.mesh_dim_names else None
+        data = export_json.export_sharding_json(self._core, self._core._extract(), self._node_info())
+        out_node = next((n for n in self.graph.nodes if n.op == "output"), None)
+        if out_node is not None:  # completes the DAG; the optimizer does not solve for it
+            data["nodes"].append({"name": out_node.name, "op": "output",
+                                  "inputs": [{"name": n.name} for n in out_node.all_input_nodes]})
+        return data
+
+    def get_log(self, colored: bool = False, verbose: bool = False) -> str:
+        from . import log_formatting
+
+        sol = self._core._extract()
+        by_node: Dict[torch.fx.Node, List[DecisionVar]] = {}
+        for key in self.selected_keys:
+            by_node.setdefault(self.nodes[key[0]], []).append(self.decision_vars[key])
+        violated = self._core.prob.violated()
+        text = "\n".join(f"violated constraint: {n}" for n in violated)
+        del sol
+        return log_formatting.format_sharding_log(self.graph, by_node, colored, verbose, text)
+
+    def save(self, path: str) -> None:
+        """Packed state (graph arrays, coefficient twin, constraint log,
+        solution).  ``PackedShardingOptimizer.load(path)`` reopens it without
+        the model, mesh or process group."""
+        self._core.mesh_dim_names = list(self.mesh.mesh_dim_names) if self.mesh.mesh_dim_names else None
+        self._core.save(path)
+
+    def save_placements(self, path: str) -> None:
+        from . import serialization
+
+        names = list(self.mesh.mesh_dim_names) if self.mesh.mesh_dim_names else None
+        serialization.save_placements(self._core, self._core._extract(), path, names)
+
+    def load_placements(self, path: str) -> Dict[torch.fx.Node, OpSpec]:
+        from . import serialization
+
+        names = list(self.mesh.mesh_dim_names) if self.mesh.mesh_dim_names else None
+        sol = serialization.load_placements(self._core, path, names)
+        return {self.nodes[v]: self.strats[self.nodes[v]].strategies[int(sol[v])]
+                for v in range(self._packed.num_nodes)}

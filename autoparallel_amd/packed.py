@@ -237,6 +237,21 @@ class PackedGraph:
         k = self.entry_keys().astype(np.int64)
         return np.lexsort((k[:, 3], k[:, 1], k[:, 2], k[:, 0]))
 
+    def export_rows(self):
+        """(row_base int64[n_edge], row_stride int32[n_edge]): the row of entry
+        (e, out_idx, inp_idx) in ``decision_vars`` insertion order is
+        ``row_base[e] + out_idx * row_stride[e] + inp_idx``."""
+        ssrc = self.edge_ssrc.astype(np.int64)
+        node = self.edge_node.astype(np.int64)
+        per_node = np.zeros(self.num_nodes, np.int64)  # sum of S_src over the node's arguments
+        np.add.at(per_node, node, ssrc)
+        node_rows = per_node * self.node_nstrat.astype(np.int64)
+        node_base = np.concatenate([[0], np.cumsum(node_rows)[:-1]]) if self.num_nodes else np.zeros(0, np.int64)
+        first = self.node_edge_off[:-1].astype(np.int64)[node]  # first edge of e's node
+        csum = np.concatenate([[0], np.cumsum(ssrc)])
+        before = csum[np.arange(self.num_edges)] - csum[first]  # S_src of the node's earlier arguments
+        return (node_base[node] + before).astype(np.int64), per_node[node].astype(np.int32)
+
     # -- device-side views ----------------------------------------------------
     EDGE_DTYPE = np.dtype(
         [

@@ -58,6 +58,35 @@ class Coefficients:
         r = eng.results()
         return cls(eng.g, r["comm"], r["cost"], r["flags"], r["compute"], r["per_arg"])
 
+    @classmethod
+    def from_decision_var_arrays(cls, g: PackedGraph, keys, vals, compute, per_arg) -> "Coefficients":
+        """From the saved twin (keys int32[E, 4], vals float64[E, 3] =
+        compute, comm, transition per variable, any row order).  cost is
+        rebuilt as the reference's loader does
+        (autoparallel/serialization.py:313, then add_inf_cost_constraint)."""
+        keys = np.asarray(keys, np.int64)
+        e = g.node_edge_off[:-1].astype(np.int64)[keys[:, 0]] + keys[:, 1]
+        if (e >= g.node_edge_off[1:].astype(np.int64)[keys[:, 0]]).any():
+            raise RuntimeError("saved key names an argument its node does not have")
+        if (keys[:, 2] >= g.edge_sdst[e]).any() or (keys[:, 3] >= g.edge_ssrc[e]).any() or (keys < 0).any():
+            raise RuntimeError("saved key outside its edge block")
+        slot = g.edge_off[:-1][e] + keys[:, 2] * g.edge_ssrc[e].astype(np.int64) + keys[:, 3]
+        n = g.num_slots
+        comm, cost, flags = np.zeros(n), np.zeros(n), np.zeros(n, np.uint8)
+        seen = np.zeros(n, bool)
+        seen[slot] = True
+        if int(seen.sum()) != g.num_entries or keys.shape[0] != g.num_entries:
+            raise RuntimeError("saved keys do not cover every decision variable exactly once")
+        comm[slot] = vals[:, 1]
+        c = vals[:, 0] + vals[:, 1] + vals[:, 2]
+        bad = ~np.isfinite(c)
+        cost[slot] = np.where(bad, 10000.0, c)
+        flags[slot] = (vals[:, 2] != 0).astype(np.uint8) | (bad.astype(np.uint8) << 1)
+        out = cls(g, comm, cost, flags, compute, per_arg)
+        out.saved_arrays = (np.asarray(keys, np.int32), np.asarray(vals, np.float64))
+        out.slot_arrays = (comm, cost, flags)
+        return out
+
 
 class PackedShardingOptimizer:
     def __init__(
@@ -87,6 +116,8 @@ class PackedShardingOptimizer:
         self.prob = ilp.SparseILP(self.n_vars)
         self._memory_constraint: Optional[Tuple[float, float]] = None
         self._node_constraint_names: Dict[str, int] = {}
+        self._constraint_log: List[Tuple[str, dict]] = []  # replayed by load (serialization.py)
+        self.mesh_dim_names: Optional[List[str]] = None
         self.selected: Optional[np.ndarray] = None
         self.add_default_constraints()
 
@@ -239,6 +270,8 @@ class PackedShardingOptimizer:
             raise RuntimeError(
                 f"Couldn't find appropriate constraint {g.node_names[v] if g.node_names else v} "
                 f"{constraint_name} {[plc_str(p) for p in want]}")
+        self._constraint_log.append(("add_node_constraint", {
+            "v": int(v), "placement": [int(p) for p in want], "constraint_name": constraint_name}))
         names = []
         for e in range(int(g.node_edge_off[v]), int(g.node_edge_off[v + 1])):
             idx = np.concatenate([self._row_vars(e, o) for o in allowed])
@@ -249,6 +282,8 @@ class PackedShardingOptimizer:
 
     def add_parameter_memory_constraint(self, memory_factor_low: float, memory_factor_high: float) -> None:
         self._memory_constraint = (memory_factor_low, memory_factor_high)
+        self._constraint_log.append(("add_parameter_memory_constraint", {
+            "memory_factor_low": memory_factor_low, "memory_factor_high": memory_factor_high}))
 
     def _memory_ratios(self, params: List[int]) -> List[np.ndarray]:
         """prod(local shape) / prod(global shape) of every strategy of every
@@ -382,9 +417,82 @@ class PackedShardingOptimizer:
             out.append(None if t is None else tuple(plc_str(int(c)) for c in self.g.tuple_plc[t, : self.g.ndim]))
         return out
 
+    # -- device access for an optimizer whose coefficients were injected ---------------
+    def _ensure_engine(self):
+        """The CostEngine holding the coefficients; for a loaded optimizer the
+        saved arrays are uploaded on first use (no cost is recomputed)."""
+        if self.engine is None:
+            from .engine import CostEngine
+
+            slot_arrays = getattr(self.coef, "slot_arrays", None)
+            if slot_arrays is None:
+                raise RuntimeError("coefficients were injected without their slot arrays: no device copy to use")
+            self.engine = CostEngine(self.g)
+            self.engine.load_results(*slot_arrays, self.coef.compute, self.coef.per_arg)
+        return self.engine
+
+    def vars_of_keys(self, keys) -> np.ndarray:
+        keys = np.asarray(keys, np.int64).reshape(-1, 4)
+        e = self.g.node_edge_off[:-1].astype(np.int64)[keys[:, 0]] + keys[:, 1]
+        return self.var_start[e] + keys[:, 2] * self.g.edge_ssrc[e].astype(np.int64) + keys[:, 3]
+
+    def decision_var_arrays(self):
+        """(keys int32[E, 4], vals float64[E, 3]) in the reference's
+        decision_vars order, written by the device from the resident results."""
+        saved = getattr(self.coef, "saved_arrays", None)
+        if self.engine is None and saved is not None:
+            return saved  # loaded and untouched since
+        keys, vals = self._ensure_engine().export_decision_vars()
+        return keys.cpu().numpy(), vals.cpu().numpy()
+
+    def _spec_str(self, word: int) -> Optional[str]:
+        if int(word) == SPEC_NONE:
+            return None
+        t = int(word) & (MAX_TUPLES - 1)
+        return "".join(plc_str(int(c)) for c in self.g.tuple_plc[t, : self.g.ndim])
+
+    def output_placement_str(self, v: int, o: int) -> Optional[str]:
+        return self._spec_str(self.g.lists[int(self.g.node_out_list[v]) + o])
+
+    def input_placement_strs(self, v: int, o: int) -> List[Optional[str]]:
+        g = self.g
+        return [self._spec_str(g.lists[int(g.edge_dst_list[e]) + o])
+                for e in range(int(g.node_edge_off[v]), int(g.node_edge_off[v + 1]))]
+
+    def solution_terms(self, sol: np.ndarray):
+        """(terms float64[n_edge, 4] = compute, comm, transition, cost of the
+        selected entry of every edge; slot int64[n_edge]) from the device."""
+        import torch
+
+        eng = self._ensure_engine()
+        a = torch.from_numpy(np.ascontiguousarray(sol.astype(np.int16))).to(eng.device)
+        terms, slot = eng.solution_terms(a)
+        return terms.cpu().numpy(), slot.cpu().numpy()
+
+    def save(self, path: str) -> None:
+        from . import serialization
+
+        serialization.save_optimizer(self, path, self.mesh_dim_names)
+
+    @classmethod
+    def load(cls, path: str) -> "PackedShardingOptimizer":
+        from . import serialization
+
+        return serialization.load_optimizer(path, cls)
+
+    def get_json(self, sol: Optional[np.ndarray] = None) -> dict:
+        from . import export_json
+
+        return export_json.export_sharding_json(self, self._extract() if sol is None else sol)
+
+    def get_log(self, sol: Optional[np.ndarray] = None) -> str:
+        from . import log_formatting
+
+        return log_formatting.format_packed_log(self, self._extract() if sol is None else sol)
+
     def compute_solution_cost(self, sol: np.ndarray) -> Dict[str, float]:
         """The reference's _compute_solution_cost for one assignment, on the device."""
-        assert self.engine is not None
+        self._ensure_engine()
         import torch
 
         a = torch.from_numpy(np.ascontiguousarray(sol.astype(np.int16).reshape(-1, 1))).to(self.engine.device)

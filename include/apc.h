@@ -311,6 +311,29 @@ int apc_apply_prefetch_discount(const apc_problem* p, const double* per_arg, dou
  * (autoparallel/optimize_sharding.py:879-885): obj = cost * node_multiplier. */
 int apc_objective_coeffs(const apc_problem* p, const double* cost, double* obj, void* stream);
 
+/* Replaces the per-variable loop of save_optimizer
+ * (autoparallel/serialization.py:145-161): the packed twin of decision_vars,
+ * keys int32[E][4] = (node_idx, argi, out_idx, inp_idx) and vals double[E][3] =
+ * (compute_cost, comm_cost, sharding_transition_cost), rows in decision_vars'
+ * insertion order (node, out_idx, argi, inp_idx;
+ * autoparallel/optimize_sharding.py:511-520).  row_base[e] (int64) is the row of
+ * entry (e, 0, 0) and row_stride[e] (int32) the number of rows per out_idx of
+ * e's node (sum of S_src over the node's arguments). */
+int apc_export_decision_vars(const apc_problem* p, const double* per_arg, const double* comm,
+                             const uint8_t* flags, const int64_t* row_base,
+                             const int32_t* row_stride, int32_t* keys, double* vals, void* stream);
+
+/* Replaces the selected-variable gathers of export_sharding_json
+ * (autoparallel/export_json.py:314-361) and get_log
+ * (autoparallel/log_formatting.py:118-130) for one assignment (assign:
+ * uint16[n_node], out_idx per node): terms double[n_edge][4] = (compute_cost,
+ * comm_cost, sharding_transition_cost, cost) of the selected entry of every
+ * (node, arg) edge, slot int64[n_edge] its slot (NaN / -1 where the assignment
+ * is not a strategy index of the edge). */
+int apc_solution_terms(const apc_problem* p, const double* per_arg, const double* comm,
+                       const double* cost, const uint8_t* flags, const uint16_t* assign,
+                       double* terms, int64_t* slot, void* stream);
+
 /* Replaces _compute_solution_cost (autoparallel/optimize_sharding.py:1056-1111)
  * and evaluates the ILP objective (:879-885) with its inf-cost rows (:803-812)
  * for a batch of assignments.  assign: uint16 [n_node][n_assign] (node-major),

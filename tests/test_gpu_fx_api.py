@@ -83,6 +83,29 @@ def test_sharding_optimizer_on_joint_graph(mesh):
 
     for p, gr in fx_utils.get_param_and_grad_nodes(gm.graph).values():
         assert sol[p].output_specs.placements == sol[gr].output_specs.placements
+    # export: JSON (one record per graph node, output included), annotated log, save, placements
+    data = opt.get_json()
+    assert [n["name"] for n in data["nodes"]] == [n.name for n in gm.graph.nodes]
+    assert data["nodes"][-1]["op"] == "output" and data["mesh"]["shape"] == [2, 4]
+    assert np.isclose(data["summary"]["total"], total, rtol=1e-9)
+    kinds = {n.get("placeholder_kind") for n in data["nodes"]}
+    assert {"param", "input", "tangent"} <= kinds
+    assert any(n.get("op", "").startswith("aten.") for n in data["nodes"])
+    log = opt.get_log()
+    assert "# placement=" in log and f"total_cost: {base:.2f}" in log
+    import tempfile
+
+    from autoparallel_amd.sharding_problem import PackedShardingOptimizer
+
+    with tempfile.TemporaryDirectory() as tmp:
+        opt.save(tmp + "/opt.npz")
+        loaded = PackedShardingOptimizer.load(tmp + "/opt.npz")
+        assert loaded.n_vars == len(opt.decision_vars) and loaded.g.num_nodes == opt._packed.num_nodes == len(opt.nodes) - 1
+        assert np.isclose(loaded.objective_value, base)
+        assert loaded.get_json()["summary"] == opt._core.get_json()["summary"]
+        opt.save_placements(tmp + "/plc.json")
+        back = opt.load_placements(tmp + "/plc.json")
+        assert all(str(back[n].output_specs) == str(sol[n].output_specs) for n in sol)
     # a user constraint moves the plan and can be removed again
     x = next(n for n in gm.graph.nodes if n.name == "primals_3")
     from torch.distributed.tensor.placement_types import Replicate, Shard
