@@ -104,6 +104,7 @@ class ApcProblem(C.Structure):
         ("max_rank", C.c_int32),
         ("n_compute", C.c_int64),
         ("n_comp_node", C.c_int32),
+        ("max_nstrat", C.c_int32),
         ("comp_nodes", C.c_void_p),
         ("node_multiplier", C.c_void_p),
         ("n_prog", C.c_int64),

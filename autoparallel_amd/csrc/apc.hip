@@ -262,13 +262,14 @@ __device__ __forceinline__ double roofline(const apc_problem& p, int64_t flops, 
 constexpr int kNodesPerBlock = 4;  // one wavefront each
 constexpr int kProgCache = 128;    // int64 words of program staged per wave
 
-// One wavefront per evaluated node.  Phase 1: the lanes split the node's
+// One wavefront per 64 strategies of an evaluated node.  Phase 1: the lanes split the node's
 // (strategy, argument) pairs and write each argument's local (sharded) sizes
 // to LDS as local[arg][dim][strategy-slot]; all loads of a pair are issued
 // together.  Phase 2: one lane per strategy interprets the node's compute
-// program out of LDS.  Strategies are processed 64 at a time.  `slow` (the LDS
+// program out of LDS.  A wavefront handles the 64 strategies from o0; a node
+// with more strategies is split over several wavefronts.  `slow` (the LDS
 // layout does not fit) reads sizes from memory on demand instead.
-__device__ __forceinline__ void node_compute_wave(const apc_problem& p, int v, int lane,
+__device__ __forceinline__ void node_compute_wave(const apc_problem& p, int v, int o0, int lane,
                                                   int64_t* __restrict__ s_prog,
                                                   int64_t* __restrict__ s_local, bool slow,
                                                   double* __restrict__ compute,
@@ -278,11 +279,12 @@ __device__ __forceinline__ void node_compute_wave(const apc_problem& p, int v, i
   const int64_t base = p.node_comp_off[v];
   const int nargs = p.node_nargs[v];
   const int op = p.node_op[v];
+  if (o0 >= S) return;  // wave-uniform
   if (op == APC_OP_ZERO) {
-    const double pa = 0.0 / (double)nargs;
-    for (int o = lane; o < S; o += 64) {
+    const int o = o0 + lane;
+    if (o < S) {
       compute[base + o] = 0.0;
-      per_arg[base + o] = pa;
+      per_arg[base + o] = 0.0 / (double)nargs;
     }
     return;
   }
@@ -299,7 +301,7 @@ __device__ __forceinline__ void node_compute_wave(const apc_problem& p, int v, i
       prog = s_prog;  // LDS operations of one wave execute in order
     }
   }
-  for (int o0 = 0; o0 < S; o0 += 64) {
+  {
     const int chunk = (S - o0 < 64) ? (S - o0) : 64;
     if (!slow && op == APC_OP_PROGRAM) {
       for (int t = lane; t < chunk * na; t += 64) {
@@ -336,7 +338,7 @@ __device__ __forceinline__ void node_compute_wave(const apc_problem& p, int v, i
       }
     }
     const int o = o0 + lane;
-    if (lane >= chunk) continue;
+    if (lane >= chunk) return;
     const int64_t idx = base + o;
     int64_t flops = 0, nbytes = 0;
     int dtype = 1;  // float32 when the node has no tensor argument
@@ -500,15 +502,17 @@ prepare_kernel(apc_problem p, double* __restrict__ table, int table_blocks, int 
     return;
   }
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int i = ((int)blockIdx.x - table_blocks) * kNodesPerBlock + wave;
+  const int unit = ((int)blockIdx.x - table_blocks) * kNodesPerBlock + wave;
+  const int chunks = (p.max_nstrat + 63) >> 6;  // wavefronts per node
+  const int i = unit / chunks;
   if (i >= p.n_comp_node) return;
   const uint32_t keep = warm_problem(p, threadIdx.x & 63, 64);
   asm volatile("" ::"v"(keep));
   const int v = __builtin_amdgcn_readfirstlane(p.comp_nodes[i]);
   const int per_wave = kProgCache + (slow ? 0 : p.max_node_args * (p.max_rank + 1) * 64);
   int64_t* s_prog = s_dyn + (size_t)wave * per_wave;
-  node_compute_wave(p, v, threadIdx.x & 63, s_prog, s_prog + kProgCache, slow != 0, compute,
-                    per_arg, status);
+  node_compute_wave(p, v, (unit - i * chunks) * 64, threadIdx.x & 63, s_prog, s_prog + kProgCache,
+                    slow != 0, compute, per_arg, status);
 }
 
 // ---------------------------------------------------------------------------
@@ -1038,7 +1042,11 @@ int slot_grid(const apc_problem* p, int per_block, unsigned* grid) {
 int launch_prepare(const apc_problem* p, double* table, bool do_nodes, double* compute,
                    double* per_arg, int32_t* status, hipStream_t stream) {
   const int table_blocks = (table && p->table_size > 0) ? p->n_table_block : 0;
-  const int node_blocks = do_nodes ? (p->n_comp_node + kNodesPerBlock - 1) / kNodesPerBlock : 0;
+  const int64_t chunks = (p->max_nstrat + 63) >> 6;
+  const int64_t units = (int64_t)p->n_comp_node * chunks;  // one wavefront per 64 strategies of a node
+  if (do_nodes && (chunks < 1 || units > (1ll << 30)))
+    return fail(APC_ERR_INVALID, "launch_prepare: max_nstrat must be >= 1 and n_comp_node * chunks < 2^30%s");
+  const int node_blocks = do_nodes ? (int)((units + kNodesPerBlock - 1) / kNodesPerBlock) : 0;
   if (table_blocks + node_blocks == 0) return 0;
   // LDS for the local-size staging (a CU has 160 KB); beyond 96 KB per block,
   // sizes are read on demand instead

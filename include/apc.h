@@ -176,6 +176,7 @@ typedef struct apc_problem {
   int32_t max_rank;             /* max tensor rank over all metas */
   int64_t n_compute;            /* length of the compute / per_arg vectors */
   int32_t n_comp_node;          /* nodes to evaluate: one per distinct slot */
+  int32_t max_nstrat;           /* max of node_nstrat over comp_nodes (>= 1)  */
   const int32_t* comp_nodes;    /* [n_comp_node] */
   const int32_t* node_multiplier;
   int64_t n_prog;
