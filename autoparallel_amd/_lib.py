@@ -162,6 +162,7 @@ _SIGNATURES = {
         [C.POINTER(ApcProblem), C.c_void_p, C.c_double, C.c_void_p, C.c_void_p, C.c_void_p,
          C.c_void_p, C.c_void_p]),
     "apc_objective_coeffs": (C.c_int, [C.POINTER(ApcProblem), C.c_void_p, C.c_void_p, C.c_void_p]),
+    "apc_node_hashes": (C.c_int, [C.POINTER(ApcProblem), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
     "apc_export_decision_vars": (
         C.c_int,
         [C.POINTER(ApcProblem), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,

@@ -703,6 +703,75 @@ objective_kernel(apc_problem p, const double* __restrict__ cost, double* __restr
 }
 
 // ---------------------------------------------------------------------------
+// Kernel: structural hash of every node, the key under which repeated layers
+// are clustered.  It covers what the reference's node key covers
+// (graph_passes/graph_clustering.py:68-82: the op, the forward/backward tag, the
+// node's own strategies and its producers' strategies), read from the packed
+// arrays: op class, program, strategy counts, output/input/producer spec runs,
+// default rows.  H = mix(sum over (section, position) of mix(word ^ salt)): a
+// position-salted sum, so the lanes of a wavefront hash disjoint positions and
+// add.
+// ---------------------------------------------------------------------------
+__host__ __device__ __forceinline__ uint64_t mix64(uint64_t z) {
+  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+  z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+  return z ^ (z >> 31);
+}
+
+__device__ __forceinline__ uint64_t hash_term(uint64_t section, uint64_t pos, uint64_t w) {
+  return mix64(w ^ mix64((section << 40) + pos + 0x9E3779B97F4A7C15ull));
+}
+
+__global__ void __launch_bounds__(kBlock)
+node_hash_kernel(apc_problem p, const int64_t* __restrict__ node_out_list,
+                 const int32_t* __restrict__ node_phase, uint64_t* __restrict__ out) {
+  const int v = blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6);
+  if (v >= p.n_node) return;  // wave-uniform
+  const int lane = threadIdx.x & 63;
+  const int S = p.node_nstrat[v];
+  const int e0 = p.node_edge_off[v], e1 = p.node_edge_off[v + 1];
+  const int op = p.node_op[v];
+  uint64_t acc = 0;
+  if (lane == 0) {
+    acc += hash_term(0, 0, (uint64_t)op);
+    acc += hash_term(0, 1, (uint64_t)p.node_nargs[v]);
+    acc += hash_term(0, 2, (uint64_t)S);
+    acc += hash_term(0, 3, (uint64_t)(node_phase ? node_phase[v] : 0));
+    acc += hash_term(0, 4, (uint64_t)(e1 - e0));
+  }
+  const int plen = p.node_prog_len[v];
+  for (int i = lane; i < plen; i += 64) acc += hash_term(1, i, (uint64_t)p.prog[p.node_prog_off[v] + i]);
+  for (int k = lane; k < S; k += 64) acc += hash_term(2, k, p.lists[(size_t)node_out_list[v] + k]);
+  if (op == APC_OP_EXPLICIT) {
+    const int64_t b = p.node_comp_off[v];
+    for (int k = lane; k < S; k += 64) {
+      acc += hash_term(3, k, (uint64_t)p.explicit_flops[b + k]);
+      acc += hash_term(4, k, (uint64_t)p.explicit_bytes[b + k]);
+    }
+  }
+  for (int e = e0; e < e1; ++e) {
+    const apc_edge ed = p.edges[e];
+    const uint64_t sec = 16 + 4 * (uint64_t)(e - e0);
+    if (lane == 0) {
+      acc += hash_term(sec, 0, (uint64_t)ed.ssrc);
+      acc += hash_term(sec, 1, (uint64_t)ed.sdst);
+      acc += hash_term(sec, 2, (uint64_t)(ed.flags & (APC_EDGE_HAS_PRODUCER | APC_EDGE_SCORE_TRANSITION)));
+      acc += hash_term(sec, 3, (uint64_t)(ed.default_off >= 0));
+    }
+    for (int k = lane; k < ed.sdst; k += 64) acc += hash_term(sec + 1, k, p.lists[(size_t)ed.dst_list + k]);
+    if (ed.src_node >= 0)
+      for (int j = lane; j < ed.ssrc; j += 64) acc += hash_term(sec + 2, j, p.lists[(size_t)ed.src_list + j]);
+    if (ed.default_off >= 0) {
+      const int64_t n = (int64_t)ed.ssrc * ed.sdst;
+      for (int64_t i = lane; i < n; i += 64)
+        acc += hash_term(sec + 3, (uint64_t)i, (uint64_t)__double_as_longlong(p.default_vals[ed.default_off + i]));
+    }
+  }
+  for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor((unsigned long long)acc, off);
+  if (lane == 0) out[v] = mix64(acc);
+}
+
+// ---------------------------------------------------------------------------
 // Kernel: packed twin of the decision variables, in the reference's insertion
 // order (node, out_idx, argi, inp_idx): row of entry (e, o, j) is
 // row_base[e] + o * row_stride[e] + j, where row_stride is the node's sum of
@@ -1203,6 +1272,16 @@ int apc_objective_coeffs(const apc_problem* p, const double* cost, double* obj, 
   hipLaunchKernelGGL(objective_kernel, dim3(grid), dim3(kBlock), 0, (hipStream_t)stream, *p, cost,
                      obj);
   return check_launch("objective_kernel");
+}
+
+int apc_node_hashes(const apc_problem* p, const int64_t* node_out_list, const int32_t* node_phase,
+                    uint64_t* out, void* stream) {
+  if (int rc = validate_problem(p)) return rc;
+  if (p->n_node == 0) return 0;
+  if (!node_out_list || !out) return fail(APC_ERR_INVALID, "apc_node_hashes: null argument%s");
+  hipLaunchKernelGGL(node_hash_kernel, dim3((p->n_node + (kBlock / 64) - 1) / (kBlock / 64)), dim3(kBlock),
+                     0, (hipStream_t)stream, *p, node_out_list, node_phase, out);
+  return check_launch("node_hash_kernel");
 }
 
 int apc_export_decision_vars(const apc_problem* p, const double* per_arg, const double* comm,

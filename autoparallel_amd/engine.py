@@ -263,6 +263,12 @@ class CostEngine:
         self.built = True
         return self
 
+    def set_node_multiplier(self, mult: np.ndarray) -> None:
+        """Replace the objective multiplier per node (cluster multiplicity)."""
+        t = self._keep["node_multiplier"]
+        assert len(mult) == t.numel()
+        t.copy_(torch.from_numpy(np.ascontiguousarray(mult, np.int32)))
+
     def load_results(self, comm, cost, flags, compute, per_arg):
         """Adopt coefficient arrays computed earlier (a saved optimizer): host
         arrays of num_slots / num_compute elements are copied to the device and
@@ -318,6 +324,22 @@ class CostEngine:
             "apc_score_assignments",
         )
         return out
+
+    def node_hashes(self, node_phase: Optional[np.ndarray] = None) -> np.ndarray:
+        """uint64[n_node] structural hash of every node (the clustering key).
+        Needs only the uploaded problem, not the coefficients."""
+        g = self.g
+        out_list = torch.from_numpy(np.ascontiguousarray(g.node_out_list, np.int64)).to(self.device)
+        phase = None
+        if node_phase is not None:
+            phase = torch.from_numpy(np.ascontiguousarray(node_phase, np.int32)).to(self.device)
+        out = torch.empty(g.num_nodes, dtype=torch.int64, device=self.device)
+        _lib.check(
+            self.lib.apc_node_hashes(C.byref(self.problem), self._ptr(out_list), self._ptr(phase), self._ptr(out),
+                                     self._stream()),
+            "apc_node_hashes",
+        )
+        return out.cpu().numpy().view(np.uint64)
 
     def export_decision_vars(self):
         """(keys int32[E, 4], vals float64[E, 3]) on the device: the packed twin

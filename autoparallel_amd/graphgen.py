@@ -263,6 +263,8 @@ class Tracer:
     def backward(self, roots: List[Tuple[T, T]]):
         """Differentiate: ``roots`` pairs each output with its tangent."""
         grads: Dict[Tuple[int, Optional[int]], T] = {}
+        if getattr(self, "_bwd_start", None) is None:
+            self._bwd_start = len(self.b.nodes)  # nodes from here on belong to the backward pass
 
         def key(t: T):
             return (t.node, t.out_index)
@@ -661,6 +663,10 @@ class Tracer:
         self.terminal_derived = terminal
         g = self.b.pack()
         g.roles = self._roles(param_grads, outputs)
+        g.node_kind = np.asarray([0 if self.node_inputs.get(v) or self.b.nodes[v].op != 0 else 1 for v in range(n)],
+                                 np.uint8)
+        start = getattr(self, "_bwd_start", None)
+        g.node_phase = (np.arange(n) >= (n if start is None else start)).astype(np.int32)
         return g
 
     def _roles(self, param_grads: Dict[int, T], outputs: List[T]):

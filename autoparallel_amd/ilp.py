@@ -52,6 +52,7 @@ class SparseILP:
     def __init__(self, n_vars: int):
         self.n_vars = int(n_vars)
         self.objective = np.zeros(self.n_vars, np.float64)
+        self.upper = np.ones(self.n_vars, np.float64)  # 0 fixes a variable out of the model
         self.constraints: "collections.OrderedDict[str, Row]" = collections.OrderedDict()
         self._counters: Dict[str, int] = {}
         self.status = STATUS_NOT_SOLVED
@@ -84,7 +85,7 @@ class SparseILP:
         bounds instead of matrix rows."""
         import scipy.sparse as sp
 
-        ub = np.ones(self.n_vars)
+        ub = self.upper.copy()
         data, cols, ptr, lo, hi = [], [], [0], [], []
         for r in self.constraints.values():
             if r.sense == EQ and r.rhs == 0.0 and r.idx.shape[0] == 1 and r.coef[0] != 0:
@@ -192,5 +193,6 @@ class SparseILP:
                 f.write(f"{r.name}: {expr(r.idx, r.coef)} {_SENSE_STR[r.sense]} {r.rhs!r}\n")
             f.write("Binaries\n")
             for i in range(self.n_vars):
-                f.write(vn(i) + "\n")
+                if self.upper[i] > 0:  # variables fixed out of the model are not declared
+                    f.write(vn(i) + "\n")
             f.write("End\n")

@@ -145,9 +145,7 @@ class ShardingOptimizer:
         self.graph = gm.graph
         self.mesh = mesh
         self.force_grad_reduce_in_higher_precision = force_grad_reduce_in_higher_precision
-        if repeated_subgraphs:
-            warnings.warn("repeated_subgraphs: clustering is not built; every node is priced "
-                          "(same plan, no variable sharing)")
+        self.repeated_subgraphs = bool(repeated_subgraphs)
         self.cluster_links: Dict[tuple, tuple] = {}
         self._devices_per_host = devices_per_host if devices_per_host is not None else _mesh_dph(mesh)
         self._device_name = device_name or detect_device_name()
@@ -262,6 +260,11 @@ class ShardingOptimizer:
         b.prefetchable_edges = self._prefetchable(roles)
         g = b.pack()
         g.roles = roles
+        packed_nodes = [n for n in self.nodes if n.op != "output"]
+        g.node_kind = np.asarray([1 if n.op == "placeholder" else (2 if n.op == "get_attr" else 0)
+                                  for n in packed_nodes], np.uint8)
+        g.node_phase = np.asarray([1 if n.meta.get("partitioner_tag") == "is_backward" else 0
+                                   for n in packed_nodes], np.int32)
         return g
 
     # -- coefficients ----------------------------------------------------------------
@@ -270,7 +273,14 @@ class ShardingOptimizer:
         self._core = PackedShardingOptimizer(
             self._packed, roles=self._packed.roles,
             force_grad_reduce_in_higher_precision=self.force_grad_reduce_in_higher_precision,
-            device_name=self._device_name, nccl_config=_cre.get_nccl_topo_config())
+            device_name=self._device_name, nccl_config=_cre.get_nccl_topo_config(),
+            repeated_subgraphs=self.repeated_subgraphs)
+        # per-variable link table of the reference (:356-378): linked key -> root key
+        self.cluster_links = {}
+        for v, r in self._core.cluster_links.items():
+            for argi, out_idx, inp_idx in self.walk_over_options(self.nodes[v]):
+                self.cluster_links[(v, argi, out_idx, inp_idx)] = (r, argi, out_idx, inp_idx)
+        self._cluster_linked_node_idxs = {k[0] for k in self.cluster_links}
         self.prob = self._core.prob
         self._write_back_redistribute_costs()
         return DecisionVars(self)
@@ -336,6 +346,11 @@ class ShardingOptimizer:
     # -- solve ------------------------------------------------------------------------------
     def _solution_dict(self, sol: np.ndarray) -> Dict[torch.fx.Node, OpSpec]:
         self.selected_keys = [tuple(int(x) for x in k) for k in self._packed.entry_keys()[self._core.selected]]
+        g = self._packed
+        for v in np.nonzero(self._core.linked)[0]:  # linked nodes repeat their root's choice (:902-903)
+            for a, e in enumerate(range(int(g.node_edge_off[v]), int(g.node_edge_off[v + 1]))):
+                u = int(g.edge_src_node[e])
+                self.selected_keys.append((int(v), a, int(sol[v]), int(sol[u]) if u >= 0 else 0))
         return {self.nodes[v]: self.strats[self.nodes[v]].strategies[int(sol[v])]
                 for v in range(self._packed.num_nodes)}
 

@@ -178,6 +178,10 @@ class PackedGraph:
     node_multiplier: Optional[np.ndarray] = None  # int32[N]
     node_names: Optional[List[str]] = None
     roles: Optional[object] = None  # sharding_problem.GraphRoles (fwd/bwd pairs, cast chains)
+    # clustering inputs: 1 for placeholders (never clustered), and the
+    # forward (0) / backward (1) tag regions must not cross
+    node_kind: Optional[np.ndarray] = None  # uint8[N]
+    node_phase: Optional[np.ndarray] = None  # int32[N]
 
     # -- derived sizes -------------------------------------------------------
     @property

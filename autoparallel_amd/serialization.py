@@ -90,6 +90,7 @@ def save_optimizer(core, path: str, mesh_dim_names: Optional[List[str]] = None) 
         compute=np.asarray(core.coef.compute, np.float64),
         per_arg=np.asarray(core.coef.per_arg, np.float64),
         constraint_log=_json_arr(core._constraint_log),
+        cluster_root=np.asarray(core.root, np.int32),
         selected_keys=selected,
     )
     with open(path, "wb") as f:
@@ -114,10 +115,12 @@ def load_optimizer(path: str, cls=None):
         selected = d["selected_keys"]
         force = bool(d["force_grad_reduce_in_higher_precision"])
         dim_names = json.loads(bytes(d["mesh_dim_names"]).decode())
+        cluster_root = d["cluster_root"] if "cluster_root" in d else None
     if keys.shape != (g.num_entries, 4) or vals.shape != (g.num_entries, 3):
         raise RuntimeError("coefficient arrays do not match the packed graph")
     coef = Coefficients.from_decision_var_arrays(g, keys, vals, compute, per_arg)
-    core = cls(g, roles=g.roles, force_grad_reduce_in_higher_precision=force, coefficients=coef)
+    core = cls(g, roles=g.roles, force_grad_reduce_in_higher_precision=force, coefficients=coef,
+               cluster_root=cluster_root)
     core.mesh_dim_names = dim_names
     for method, kwargs in log:
         getattr(core, method)(**kwargs)

@@ -98,7 +98,14 @@ class PackedShardingOptimizer:
         device: str = "cuda",
         device_name: Optional[str] = None,
         nccl_config=None,
+        repeated_subgraphs: bool = False,
+        cluster_root: Optional[np.ndarray] = None,
     ):
+        """repeated_subgraphs: cluster identical regions (node hashes from the
+        device) and let every repeated node share the decision variables of its
+        root (autoparallel/optimize_sharding.py:261-266, 356-378).
+        cluster_root: the same link table given explicitly (int[N], root[v] = v
+        for unlinked nodes), e.g. from a saved file."""
         self.g = g
         self.roles = roles or getattr(g, "roles", None) or GraphRoles()
         self.force_grad_reduce_in_higher_precision = force_grad_reduce_in_higher_precision
@@ -110,10 +117,22 @@ class PackedShardingOptimizer:
             self.engine.build(clamp_inf=True)
             coefficients = Coefficients.from_engine(self.engine)
         self.coef = coefficients
+        self.region_groups: List[List[List[int]]] = []
+        if cluster_root is None and repeated_subgraphs:
+            from . import clustering
+
+            hashes = self._ensure_engine().node_hashes(g.node_phase)
+            self.region_groups = clustering.identical_regions(g, hashes)
+            cluster_root = clustering.cluster_roots(g, self.region_groups)
+        self._set_cluster_root(cluster_root)
         sizes = g.edge_sdst.astype(np.int64) * g.edge_ssrc
         self.var_start = np.concatenate([[0], np.cumsum(sizes)]).astype(np.int64)
         self.n_vars = int(self.var_start[-1])
         self.prob = ilp.SparseILP(self.n_vars)
+        if self.linked.any():  # variables of linked nodes are their root's: fixed out of the model
+            e_linked = np.nonzero(self.linked[g.edge_node])[0]
+            for e in e_linked:
+                self.prob.upper[self.var_start[e] : self.var_start[e + 1]] = 0.0
         self._memory_constraint: Optional[Tuple[float, float]] = None
         self._node_constraint_names: Dict[str, int] = {}
         self._constraint_log: List[Tuple[str, dict]] = []  # replayed by load (serialization.py)
@@ -121,11 +140,37 @@ class PackedShardingOptimizer:
         self.selected: Optional[np.ndarray] = None
         self.add_default_constraints()
 
+    # -- clusters ---------------------------------------------------------------
+    def _set_cluster_root(self, root: Optional[np.ndarray]) -> None:
+        g = self.g
+        n = g.num_nodes
+        self.root = np.arange(n, dtype=np.int64) if root is None else np.asarray(root, np.int64)
+        assert self.root.shape == (n,) and (self.root[self.root] == self.root).all(), "roots must be unlinked"
+        self.linked = self.root != np.arange(n)
+        # edge of the root node that stands in for edge e (same argument position)
+        v = g.edge_node.astype(np.int64)
+        first = g.node_edge_off[:-1].astype(np.int64)
+        self.edge_alias = first[self.root[v]] + (np.arange(g.num_edges) - first[v])
+        if self.linked.any():
+            from . import clustering
+
+            mult = clustering.multipliers(self.root)
+            g.node_multiplier = mult
+            if self.engine is not None:
+                self.engine.set_node_multiplier(mult)
+
+    @property
+    def cluster_links(self) -> Dict[int, int]:
+        """linked node -> root node (the node-level form of the reference's
+        per-variable cluster_links, as its save file stores it)."""
+        return {int(v): int(self.root[v]) for v in np.nonzero(self.linked)[0]}
+
     # -- indexing ---------------------------------------------------------------
     def edge_of(self, v: int, a: int) -> int:
+        """Edge whose variables stand for (node v, argument a): the root's for a linked node."""
         e = int(self.g.node_edge_off[v]) + a
         assert e < int(self.g.node_edge_off[v + 1])
-        return e
+        return int(self.edge_alias[e])
 
     def var(self, v: int, a: int, o: int, j: int) -> int:
         e = self.edge_of(v, a)
@@ -133,12 +178,14 @@ class PackedShardingOptimizer:
 
     def _row_vars(self, e: int, o: int) -> np.ndarray:
         """Variables of edge e with output strategy o (all inp_idx)."""
+        e = int(self.edge_alias[e])
         s = int(self.g.edge_ssrc[e])
         b = int(self.var_start[e]) + o * s
         return np.arange(b, b + s, dtype=np.int64)
 
     def _col_vars(self, e: int, j: int) -> np.ndarray:
         """Variables of edge e with input strategy j (all out_idx)."""
+        e = int(self.edge_alias[e])
         s = int(self.g.edge_ssrc[e])
         return int(self.var_start[e]) + np.arange(int(self.g.edge_sdst[e]), dtype=np.int64) * s + j
 
@@ -160,6 +207,8 @@ class PackedShardingOptimizer:
     def add_unique_decision_constraint(self) -> None:
         # for every (node, arg): exactly one (out, inp) pair
         for e in range(self.g.num_edges):
+            if self.linked[self.g.edge_node[e]]:
+                continue
             idx = np.arange(self.var_start[e], self.var_start[e + 1], dtype=np.int64)
             self.prob.add_row("unique_decision", idx, 1.0, ilp.EQ, 1.0)
 
@@ -172,7 +221,7 @@ class PackedShardingOptimizer:
         # all arguments of a node pick the same output strategy
         g = self.g
         for v in range(g.num_nodes):
-            if self._num_input_nodes(v) <= 1:
+            if self.linked[v] or self._num_input_nodes(v) <= 1:
                 continue
             e0, e1 = int(g.node_edge_off[v]), int(g.node_edge_off[v + 1])
             for e in range(e0 + 1, e1):
@@ -192,6 +241,8 @@ class PackedShardingOptimizer:
             if u < 0:
                 continue
             v = int(g.edge_node[e])
+            if self.linked[u] and self.linked[v]:  # the root-to-root edge covers it
+                continue
             if (u, v) in seen:  # first matching argument only
                 continue
             seen.add((u, v))
@@ -208,8 +259,9 @@ class PackedShardingOptimizer:
 
     def add_inf_cost_constraint(self) -> None:
         # the engine already wrote 10000.0 into cost; pin those variables to 0
-        for i in np.nonzero(self.coef.flags & 2)[0]:
-            self.prob.add_row("inf_cases", [i], 1.0, ilp.EQ, 0.0)
+        for i in np.nonzero((self.coef.flags & 2) != 0)[0]:
+            if self.prob.upper[i] > 0:  # linked nodes have no variables of their own
+                self.prob.add_row("inf_cases", [i], 1.0, ilp.EQ, 0.0)
 
     def _out_placements(self, v: int) -> List[Optional[int]]:
         """Placement-tuple id of output 0 of each strategy of node v (None for
@@ -251,7 +303,7 @@ class PackedShardingOptimizer:
         ):
             if not enabled or not nodes:
                 continue
-            mask = np.isin(keys[:, 0], np.fromiter(nodes, np.int64)) & comm_pos
+            mask = np.isin(keys[:, 0], np.fromiter(nodes, np.int64)) & comm_pos & (self.prob.upper > 0)
             for i in np.nonzero(mask)[0]:
                 self.prob.add_row(name, [i], 1.0, ilp.EQ, 0.0)
 
@@ -273,6 +325,10 @@ class PackedShardingOptimizer:
         self._constraint_log.append(("add_node_constraint", {
             "v": int(v), "placement": [int(p) for p in want], "constraint_name": constraint_name}))
         names = []
+        if self.linked[v]:
+            raise RuntimeError(
+                f"node {g.node_names[v] if g.node_names else v} shares the variables of node "
+                f"{int(self.root[v])} (repeated subgraph): constrain that node instead")
         for e in range(int(g.node_edge_off[v]), int(g.node_edge_off[v + 1])):
             idx = np.concatenate([self._row_vars(e, o) for o in allowed])
             name = self.prob.add_row(constraint_name or "user_constraint", idx, 1.0, ilp.EQ, 1.0)
@@ -387,6 +443,12 @@ class PackedShardingOptimizer:
         (node, arg) has exactly one selection and that all args agree."""
         keys = self.g.entry_keys()[self.selected]
         sol = np.full(self.g.num_nodes, -1, np.int64)
+        if self.linked.any():  # linked nodes follow their root (optimize_sharding.py:902-903)
+            k = keys[~self.linked[keys[:, 0]]]
+            for v, a, o, j in k:
+                sol[v] = o
+            sol[self.linked] = sol[self.root[self.linked]]
+
         seen = set()
         for v, a, o, j in keys:
             if (v, a) in seen:

@@ -312,6 +312,16 @@ int apc_apply_prefetch_discount(const apc_problem* p, const double* per_arg, dou
  * (autoparallel/optimize_sharding.py:879-885): obj = cost * node_multiplier. */
 int apc_objective_coeffs(const apc_problem* p, const double* cost, double* obj, void* stream);
 
+/* Replaces _hash_node (autoparallel/graph_passes/graph_clustering.py:68-82),
+ * the key under which get_identical_regions groups repeated nodes: a 64-bit
+ * structural hash per node over its op class, program, forward/backward tag
+ * (node_phase int32[n_node], may be NULL), strategy counts, output spec run
+ * (node_out_list int64[n_node]: offset of the node's output run in lists),
+ * input and producer spec runs and default rows.  Equal keys in the reference
+ * imply equal hashes here; out: uint64[n_node]. */
+int apc_node_hashes(const apc_problem* p, const int64_t* node_out_list, const int32_t* node_phase,
+                    uint64_t* out, void* stream);
+
 /* Replaces the per-variable loop of save_optimizer
  * (autoparallel/serialization.py:145-161): the packed twin of decision_vars,
  * keys int32[E][4] = (node_idx, argi, out_idx, inp_idx) and vals double[E][3] =

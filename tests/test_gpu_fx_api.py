@@ -261,3 +261,46 @@ def test_runtime_cost_api_matches_reference_vectors(mesh, golden):
     v = graph.call_function(aten.view.default, (x, [16, 256, 4096]))
     v.meta["val"] = torch.empty((16, 256, 4096), dtype=torch.bfloat16, device="meta")
     assert cm.estimate_strategy_runtime_cost(v, st) == 0
+
+
+class _Stack(nn.Module):
+    def __init__(self, n=3):
+        super().__init__()
+        self.layers = nn.ModuleList([nn.Linear(64, 64, bias=False) for _ in range(n)])
+
+    def forward(self, x):
+        for layer in self.layers:
+            x = torch.relu(layer(x))
+        return x
+
+
+def test_repeated_subgraphs_on_joint_graph(mesh):
+    """The reference's clustered mode (optimize_sharding.py:261-266): repeated
+    layers share decision variables; the plan and its cost match the
+    unclustered optimizer on identical layers."""
+    from torch._functorch.aot_autograd import aot_export_joint_with_descriptors
+    from torch._subclasses.fake_tensor import FakeTensorMode
+
+    from autoparallel_amd.optimize_sharding import ShardingOptimizer
+
+    def graph():
+        with FakeTensorMode():
+            m, x = _Stack(), torch.randn(16, 32, 64)
+            with contextlib.ExitStack() as stack:
+                return aot_export_joint_with_descriptors(stack, m, (x,)).graph_module
+
+    plain = ShardingOptimizer(graph(), mesh, devices_per_host=8, device_name="AMD Instinct MI355X")
+    plain.get_solution()
+    opt = ShardingOptimizer(graph(), mesh, devices_per_host=8, device_name="AMD Instinct MI355X",
+                            repeated_subgraphs=True)
+    assert opt.cluster_links, "three identical layers must produce links"
+    for linked, root in opt.cluster_links.items():
+        assert linked[1:] == root[1:] and linked[0] != root[0]
+        assert str(opt.nodes[linked[0]].target) == str(opt.nodes[root[0]].target)
+    sol = opt.get_solution()
+    for v in opt._cluster_linked_node_idxs:
+        r = opt._core.root[v]
+        assert str(sol[opt.nodes[v]].output_specs) == str(sol[opt.nodes[int(r)]].output_specs)
+    assert np.isclose(opt._core.objective_value, plain._core.objective_value, rtol=1e-6)
+    assert len(opt.selected_keys) == opt._packed.num_edges  # root keys plus the expanded linked keys
+    assert "total_cost:" in opt.get_log()

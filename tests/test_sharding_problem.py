@@ -133,3 +133,63 @@ def test_sparse_ilp_basics():
     p.add_row("ban", [2], 1.0, ilp.EQ, 0.0)
     assert p.solve() == ilp.STATUS_INFEASIBLE
     assert list(p.constraints) == ["pick_000", "ban_000", "ban_001", "ban_002"]
+
+
+# ---------------------------------------------------------------------------
+# repeated-subgraph clustering (host logic; hashes from the oracle here)
+# ---------------------------------------------------------------------------
+def test_clustered_ilp_matches_reference_semantics():
+    from autoparallel_amd import clustering
+    from oracle import cluster_oracle as CO
+
+    g = graphgen.llama_graph((2, 4), 3, 64, 4, 2, 128, 256, 32, 8)
+    hashes = CO.node_hashes(g, g.node_phase)
+    # the hash groups nodes exactly as the exact content key does
+    keys = [CO.node_key(g, v, g.node_phase) for v in range(g.num_nodes)]
+    by_key, by_hash = {}, {}
+    for v in range(g.num_nodes):
+        by_key.setdefault(keys[v], []).append(v)
+        by_hash.setdefault(hashes[v], []).append(v)
+    assert sorted(by_key.values()) == sorted(by_hash.values())
+    groups = clustering.identical_regions(g, hashes)
+    assert groups, "three identical decoder layers must cluster"
+    for grp in groups:
+        assert len({len(r) for r in grp}) == 1 and len(grp) >= 2 and len(grp[0]) > 1
+        for reg in grp:
+            assert reg == sorted(reg)
+            assert len({int(g.node_phase[v]) for v in reg}) == 1  # regions do not cross fwd/bwd
+        for pos in range(len(grp[0])):
+            assert len({hashes[r[pos]] for r in grp}) == 1  # identical position by position
+    flat = [v for grp in groups for r in grp for v in r]
+    assert len(flat) == len(set(flat))  # no node in two regions
+    root = clustering.cluster_roots(g, groups)
+    mult = clustering.multipliers(root)
+    assert mult.sum() == g.num_nodes and (mult[root != np.arange(g.num_nodes)] == 0).all()
+    # layers 1 and 2 link to layer 0: a good part of the graph is linked
+    assert (root != np.arange(g.num_nodes)).sum() > g.num_nodes // 4
+
+    coef, raw = oracle_coefficients(g)
+    plain = PackedShardingOptimizer(g, coefficients=coef)
+    sol_plain = plain.get_solution()
+    g2 = graphgen.llama_graph((2, 4), 3, 64, 4, 2, 128, 256, 32, 8)
+    coef2, _ = oracle_coefficients(g2)
+    opt = PackedShardingOptimizer(g2, coefficients=coef2, cluster_root=root)
+    names = list(opt.prob.constraints)
+    count = lambda p, o: sum(1 for n in list(o.prob.constraints) if n.rsplit("_", 1)[0] == p)
+    n_linked_edges = int(opt.linked[g2.edge_node].sum())
+    assert count("unique_decision", opt) == g2.num_edges - n_linked_edges
+    assert count("output_input_consistent", opt) < count("output_input_consistent", plain)
+    sol = opt.get_solution()
+    assert (sol >= 0).all()
+    assert (sol[opt.linked] == sol[opt.root[opt.linked]]).all()  # repeated nodes follow their root
+    assert opt.prob.violated() == []
+    # the ILP objective (root cost x multiplicity) is the plain objective of the expanded plan
+    cost, bad = O.clamp_inf(raw["cost"])
+    obj, viol = O.ilp_objective(g, cost, bad, sol)
+    assert viol == 0 and np.isclose(obj, opt.objective_value, rtol=1e-9)
+    # tying the layers together cannot beat the free optimum, and on identical layers it matches it
+    assert opt.objective_value >= plain.objective_value - 1e-6
+    assert np.isclose(opt.objective_value, plain.objective_value, rtol=1e-6)
+    assert opt.cluster_links and all(opt.root[r] == r for r in opt.cluster_links.values())
+    with pytest.raises(RuntimeError, match="shares the variables"):
+        opt.add_node_constraint(int(np.nonzero(opt.linked)[0][0]))
