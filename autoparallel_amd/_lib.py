@@ -121,13 +121,12 @@ class ApcProblem(C.Structure):
         ("items", C.c_void_p),
         ("n_default", C.c_int64),
         ("default_vals", C.c_void_p),
-        ("n_run", C.c_int32),
-        ("run_list", C.c_void_p),
-        ("run_len", C.c_void_p),
-        ("run_table_off", C.c_void_p),
+        ("n_block", C.c_int32),
+        ("block_edge", C.c_void_p),
+        ("block_off", C.c_void_p),
         ("table_size", C.c_int64),
-        ("n_table_block", C.c_int32),
-        ("table_block_run", C.c_void_p),
+        ("n_table_unit", C.c_int32),
+        ("table_unit_block", C.c_void_p),
     ]
 
 

@@ -1,9 +1,9 @@
 // HIP kernels and C ABI of the sharding-search cost engine (gfx950 / CDNA4).
 //
 // Everything here is HBM-bound integer/fp64 scalar work: no matrix cores.  The
-// entry kernel is a flat scan over the E cost entries: every lane owns 4
-// consecutive entries, so a wavefront writes 2 KB of contiguous fp64 per output
-// array with 16-byte stores, and 256 contiguous flag bytes with 4-byte stores.
+// entry kernel is a flat scan over the E cost entries in work items of 256
+// entries of one edge block: a wavefront owns an item, lane L the entries
+// L + 64 k, so every load and store instruction covers 64 consecutive entries.
 // All floating-point code is compiled with -ffp-contract=off: the reference is
 // a chain of separately rounded binary64 operations, and the results here are
 // bit-identical to it.
@@ -457,32 +457,34 @@ __device__ __forceinline__ uint32_t warm_problem(const apc_problem& p, int lane,
   return acc;
 }
 
-// Row tables.  Every run's table starts on a multiple of 256 elements, so a
-// block of 256 threads works on one run: the run's description is block-uniform
-// (scalar loads) and element r of the run's table is target tuple r / len,
-// source position r % len.
+// Block table.  Edges whose producer run and consumer run are the same spec
+// words have the same S_dst x S_src matrix of redistribution costs; one copy of
+// each distinct matrix is kept, in the edge block's own [out_idx][inp_idx]
+// order, padded to a multiple of 256 elements so that a workgroup works on one
+// matrix.  An element is the cost with its sign bit set when the two
+// placements differ (costs are never negative, so the sign is free to carry
+// the transition flag): the entry kernel reads comm and transition with one
+// coalesced load and no spec words.
 __device__ __forceinline__ void pair_table_block(const apc_problem& p, double* __restrict__ table,
-                                                 int block) {
+                                                 int unit) {
   const uint32_t keep = warm_problem(p, threadIdx.x, blockDim.x);
-  const int run = p.table_block_run[block];
-  const int64_t base = p.run_table_off[run];
-  const uint32_t len = (uint32_t)p.run_len[run];
-  const int64_t r64 = (int64_t)block * 256 - base + threadIdx.x;
-  const int64_t size = (int64_t)len * p.n_tuple;
-  if (r64 < size) {
-    const uint32_t r = (uint32_t)r64;
-    const uint32_t t = r / len, j = r - t * len;
-    const uint32_t sw = p.lists[(size_t)p.run_list[run] + j];
-    double c = 0.0;  // a missing spec never reads its table slot
-    if (sw != APC_SPEC_NONE) {
-      const uint32_t sm = sw >> APC_TUPLE_BITS;
-      int64_t nbytes;
-      bool contig;
-      meta_bytes_contig(p, sm, nbytes, contig);
-      c = redistribute_cost(load_tuple(p.tuple_plc, sw & kTupleMask), load_tuple(p.tuple_plc, t),
-                            nbytes, contig, p.model);
-    }
-    table[base + r] = c;
+  const int b = p.table_unit_block[unit];
+  const int64_t base = p.block_off[b];
+  const apc_edge ed = p.edges[p.block_edge[b]];  // any edge with this matrix
+  const uint32_t ssrc = (uint32_t)ed.ssrc;
+  const int64_t l64 = (int64_t)unit * 256 - base + threadIdx.x;
+  if (l64 < (int64_t)ssrc * ed.sdst) {
+    const uint32_t l = (uint32_t)l64;
+    const uint32_t o = l / ssrc, j = l - o * ssrc;
+    const uint32_t sw = p.lists[(size_t)ed.src_list + j];
+    const uint32_t tw = p.lists[(size_t)ed.dst_list + o];
+    const uint32_t st = sw & kTupleMask, tt = tw & kTupleMask;
+    int64_t nbytes;
+    bool contig;
+    meta_bytes_contig(p, sw >> APC_TUPLE_BITS, nbytes, contig);
+    const double c = redistribute_cost(load_tuple(p.tuple_plc, st), load_tuple(p.tuple_plc, tt),
+                                       nbytes, contig, p.model);
+    table[base + l] = (st != tt) ? -c : c;
   }
   asm volatile("" ::"v"(keep));
 }
@@ -531,7 +533,6 @@ __device__ __forceinline__ apc_edge find_edge(const apc_problem& p, int64_t idx)
 
 // comm / transition of one entry, general path (direct evaluation, missing
 // specs, default rows).
-template <bool kUseTable>
 __device__ __forceinline__ void eval_entry(const apc_problem& p, const apc_edge& ed, uint32_t o,
                                            uint32_t j, const double* __restrict__ table,
                                            double& comm, int& trans) {
@@ -541,15 +542,11 @@ __device__ __forceinline__ void eval_entry(const apc_problem& p, const apc_edge&
   if (sw != APC_SPEC_NONE && tw != APC_SPEC_NONE) {
     const uint32_t st = sw & kTupleMask, tt = tw & kTupleMask, sm = sw >> APC_TUPLE_BITS;
     trans = (st != tt);
-    if (kUseTable) {
-      comm = table[ed.table_off + (int64_t)tt * ed.ssrc + j];
-    } else {
-      int64_t nbytes;
-      bool contig;
-      meta_bytes_contig(p, sm, nbytes, contig);
-      comm = redistribute_cost(load_tuple(p.tuple_plc, st), load_tuple(p.tuple_plc, tt), nbytes,
-                               contig, p.model);
-    }
+    int64_t nbytes;
+    bool contig;
+    meta_bytes_contig(p, sm, nbytes, contig);
+    comm = redistribute_cost(load_tuple(p.tuple_plc, st), load_tuple(p.tuple_plc, tt), nbytes,
+                             contig, p.model);
   } else {
     comm = p.default_vals[ed.default_off + (int64_t)o * ed.ssrc + j];
     trans = 0;
@@ -562,10 +559,12 @@ __device__ __forceinline__ void eval_entry(const apc_problem& p, const apc_edge&
 // measured on MI355X, stores whose 64 lanes cover one contiguous span stream
 // about 20% faster than lanes owning 32 contiguous bytes each.  The item record
 // is a copy of the edge record (plus local0), wave-uniform, so it lives in
-// scalar registers; a lane computes row/column of its entries, loads two spec
-// words, the per-arg compute term and one table element per entry, and stores.
-// Consecutive entries of a row are consecutive table elements, so the table
-// reads coalesce exactly like the stores.
+// scalar registers.  With a block table a lane loads, per entry, one table
+// element (cost and transition flag of the entry's position in the edge's
+// matrix: same order as the output, so the reads coalesce exactly like the
+// stores) and the per-arg compute term of its row, adds and stores; no spec
+// word is read.  Edges without a matrix in the table (no producer, a missing
+// spec, or no table at all) evaluate every entry directly.
 template <bool kUseTable>
 __device__ __forceinline__ void process_item(const apc_problem& p, const apc_edge& ed, int lane,
                                              const double* __restrict__ table,
@@ -574,7 +573,6 @@ __device__ __forceinline__ void process_item(const apc_problem& p, const apc_edg
                                              uint8_t* __restrict__ flags, int clamp_inf) {
   const uint32_t ssrc = (uint32_t)ed.ssrc;
   const uint32_t size = ssrc * (uint32_t)ed.sdst;
-  const bool prod = (ed.flags & APC_EDGE_HAS_PRODUCER) != 0;  // wave-uniform
 
   uint32_t lk[kPerLane], ok[kPerLane], jk[kPerLane];
   bool live[kPerLane];
@@ -588,37 +586,24 @@ __device__ __forceinline__ void process_item(const apc_problem& p, const apc_edg
   }
   double v_comm[kPerLane], v_pa[kPerLane];
   int v_trans[kPerLane];
-  if (kUseTable || !prod) {
-    uint32_t tw[kPerLane], sw[kPerLane];
+  if (kUseTable && ed.table_off >= 0) {  // wave-uniform
+    double raw[kPerLane];
 #pragma unroll
     for (int k = 0; k < kPerLane; ++k) {
-      tw[k] = p.lists[(size_t)ed.dst_list + ok[k]];
+      raw[k] = table[ed.table_off + (int64_t)(live[k] ? lk[k] : 0u)];
       v_pa[k] = per_arg[ed.comp_base + ok[k]];
-      sw[k] = prod ? p.lists[(size_t)ed.src_list + jk[k]] : APC_SPEC_NONE;
     }
-    bool any_none = false;
 #pragma unroll
     for (int k = 0; k < kPerLane; ++k) {
-      const bool none = (sw[k] == APC_SPEC_NONE) || (tw[k] == APC_SPEC_NONE);
-      const uint32_t st = sw[k] & kTupleMask, tt = tw[k] & kTupleMask;
-      v_comm[k] = (prod && !none) ? table[ed.table_off + (int64_t)(tt * ssrc + jk[k])] : 0.0;
-      v_trans[k] = none ? 0 : (st != tt);
-      any_none |= none;
-    }
-    if (any_none) {  // entries without a spec keep their default row value
-#pragma unroll
-      for (int k = 0; k < kPerLane; ++k) {
-        const bool none = (sw[k] == APC_SPEC_NONE) || (tw[k] == APC_SPEC_NONE);
-        if (none && live[k]) v_comm[k] = p.default_vals[ed.default_off + (int64_t)lk[k]];
-      }
+      v_trans[k] = (int)((uint64_t)__double_as_longlong(raw[k]) >> 63);
+      v_comm[k] = fabs(raw[k]);
     }
   } else {
-    // direct evaluation of every entry (no table)
 #pragma unroll
     for (int k = 0; k < kPerLane; ++k) {
       v_comm[k] = 0.0; v_pa[k] = 0.0; v_trans[k] = 0;
       if (live[k]) {
-        eval_entry<false>(p, ed, ok[k], jk[k], table, v_comm[k], v_trans[k]);
+        eval_entry(p, ed, ok[k], jk[k], table, v_comm[k], v_trans[k]);
         v_pa[k] = per_arg[ed.comp_base + ok[k]];
       }
     }
@@ -638,9 +623,56 @@ __device__ __forceinline__ void process_item(const apc_problem& p, const apc_edg
   }
 }
 
+// Table path, split in two so that the loads of a wave's next item are in
+// flight while the current item is stored.
+struct ItemLoads {
+  double raw[kPerLane];
+  double pa[kPerLane];
+  uint32_t lk[kPerLane];
+  uint32_t live;  // bit k: entry k of this lane exists
+};
+
+__device__ __forceinline__ void item_load(const apc_edge& ed, int lane, const double* __restrict__ table,
+                                          const double* __restrict__ per_arg, ItemLoads& r) {
+  const uint32_t ssrc = (uint32_t)ed.ssrc;
+  const uint32_t size = ssrc * (uint32_t)ed.sdst;
+  r.live = 0;
+#pragma unroll
+  for (int k = 0; k < kPerLane; ++k) {
+    r.lk[k] = ed.local0 + (uint32_t)(k * 64 + lane);
+    const bool live = r.lk[k] < size;
+    r.live |= (uint32_t)live << k;
+    const uint32_t l = live ? r.lk[k] : 0u;
+    const uint32_t o = ed.magic ? __umulhi(l, ed.magic) : l / ssrc;
+    r.raw[k] = table[ed.table_off + (int64_t)l];
+    r.pa[k] = per_arg[ed.comp_base + o];
+  }
+}
+
+__device__ __forceinline__ void item_store(const apc_edge& ed, const ItemLoads& r,
+                                           double* __restrict__ comm, double* __restrict__ cost,
+                                           uint8_t* __restrict__ flags, int clamp_inf) {
+#pragma unroll
+  for (int k = 0; k < kPerLane; ++k) {
+    const int trans = (int)((uint64_t)__double_as_longlong(r.raw[k]) >> 63);
+    const double cm = fabs(r.raw[k]);
+    double c = (cm + r.pa[k]) + (double)trans;  // optimize_sharding.py:544
+    const bool finite = isfinite(c);
+    if (clamp_inf && !finite) c = 10000.0;
+    if ((r.live >> k) & 1) {
+      const int64_t idx = ed.off + r.lk[k];
+      if (comm) comm[idx] = cm;
+      if (cost) cost[idx] = c;
+      // byte stores: gathering a lane's four flags into one 4-byte store through
+      // cross-lane exchanges measured slower
+      if (flags) flags[idx] = (uint8_t)(trans | (finite ? 0 : APC_ENTRY_NONFINITE));
+    }
+  }
+}
+
 // Wave w takes items w, w + W, w + 2W, ... (W = waves in the grid, capped at
-// twice the chip's resident wave slots: measured slightly faster than one wave
-// per item, whose grid has tens of thousands of short-lived waves).
+// twice the chip's resident wave slots: measured faster than one wave per item,
+// whose grid has tens of thousands of short-lived waves).
 template <bool kUseTable>
 __global__ void __launch_bounds__(kBlock)
 edge_cost_kernel(apc_problem p, const double* __restrict__ table,
@@ -649,10 +681,35 @@ edge_cost_kernel(apc_problem p, const double* __restrict__ table,
   const int n_waves = gridDim.x * (kBlock / 64);
   const int w = __builtin_amdgcn_readfirstlane((int)(blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6)));
   const int lane = threadIdx.x & 63;
-  for (int i = w; i < p.n_item; i += n_waves) {
-    const apc_edge item = p.items[i];
-    process_item<kUseTable>(p, item, lane, table, per_arg, comm, cost, flags, clamp_inf);
+  if (!kUseTable) {
+    for (int i = w; i < p.n_item; i += n_waves) {
+      const apc_edge item = p.items[i];
+      process_item<false>(p, item, lane, table, per_arg, comm, cost, flags, clamp_inf);
+    }
+    return;
   }
+  // items with a matrix in the table are pipelined: loads of the next such
+  // item are issued before the current one is stored
+  bool have = false;
+  apc_edge cur;
+  ItemLoads cur_r;
+  apc_edge nxt;
+  if (w < p.n_item) nxt = p.items[w];
+  for (int i = w; i < p.n_item; i += n_waves) {
+    const apc_edge item = nxt;
+    if (i + n_waves < p.n_item) nxt = p.items[i + n_waves];  // record of the item after this one
+    if (item.table_off < 0) {  // wave-uniform
+      process_item<true>(p, item, lane, table, per_arg, comm, cost, flags, clamp_inf);
+      continue;
+    }
+    ItemLoads r;
+    item_load(item, lane, table, per_arg, r);
+    if (have) item_store(cur, cur_r, comm, cost, flags, clamp_inf);
+    cur = item;
+    cur_r = r;
+    have = true;
+  }
+  if (have) item_store(cur, cur_r, comm, cost, flags, clamp_inf);
 }
 
 // Plain copy kernel of known size: the reference point against which the
@@ -1084,10 +1141,10 @@ int validate_problem(const apc_problem* p) {
   if (p->n_entry > 0 && (!p->edges || !p->chunk_edge || !p->lists || !p->items))
     return fail(APC_ERR_INVALID, "null edge/list/item arrays%s");
   if (p->n_comp_node > 0 && !p->comp_nodes) return fail(APC_ERR_INVALID, "null comp_nodes%s");
-  if (p->n_run < 0 || p->table_size < 0 || (p->table_size & 255) ||
-      p->n_table_block != p->table_size / 256 ||
-      (p->table_size > 0 && (!p->run_list || !p->run_len || !p->run_table_off || !p->table_block_run)))
-    return fail(APC_ERR_INVALID, "bad run table description%s");
+  if (p->n_block < 0 || p->table_size < 0 || (p->table_size & 255) ||
+      p->n_table_unit != p->table_size / 256 ||
+      (p->table_size > 0 && (!p->block_edge || !p->block_off || !p->table_unit_block)))
+    return fail(APC_ERR_INVALID, "bad block table description%s");
   if (p->max_rank < 0 || p->max_rank > APC_MAX_RANK || p->max_node_args < 0)
     return fail(APC_ERR_INVALID, "max_rank / max_node_args out of range%s");
   return 0;
@@ -1110,7 +1167,7 @@ int slot_grid(const apc_problem* p, int per_block, unsigned* grid) {
 
 int launch_prepare(const apc_problem* p, double* table, bool do_nodes, double* compute,
                    double* per_arg, int32_t* status, hipStream_t stream) {
-  const int table_blocks = (table && p->table_size > 0) ? p->n_table_block : 0;
+  const int table_blocks = (table && p->table_size > 0) ? p->n_table_unit : 0;
   const int64_t chunks = (p->max_nstrat + 63) >> 6;
   const int64_t units = (int64_t)p->n_comp_node * chunks;  // one wavefront per 64 strategies of a node
   if (do_nodes && (chunks < 1 || units > (1ll << 30)))

@@ -14,7 +14,7 @@ from .packed import CHUNK_SHIFT, MAX_MESH_DIMS, PackedGraph
 
 # Build the pair table when it is at most this many times the entry count (and
 # small in absolute terms); otherwise every entry is evaluated directly.
-_TABLE_MAX_RATIO = 1.0
+_TABLE_MAX_RATIO = 0.5
 _TABLE_MAX_DOUBLES = 1 << 28
 
 
@@ -180,15 +180,13 @@ class CostEngine:
         p.items = up("items", items)
         p.n_default = g.default_vals.shape[0]
         p.default_vals = up("default_vals", g.default_vals)
-        run_list, run_len, run_table_off, _ = g.run_table()
-        p.n_run = run_list.shape[0]
-        p.run_list = up("run_list", run_list)
-        p.run_len = up("run_len", run_len)
-        p.run_table_off = up("run_table_off", run_table_off)
-        p.table_size = int(run_table_off[-1])
-        tbr = g.table_block_runs()
-        p.n_table_block = tbr.shape[0]
-        p.table_block_run = up("table_block_run", tbr)
+        block_edge, block_off, unit_block, _ = g.block_table()
+        p.n_block = block_edge.shape[0]
+        p.block_edge = up("block_edge", block_edge)
+        p.block_off = up("block_off", block_off)
+        p.table_size = int(block_off[-1])
+        p.n_table_unit = unit_block.shape[0]
+        p.table_unit_block = up("table_unit_block", unit_block)
         self.problem = p
 
         E, NC = g.num_slots, g.num_compute

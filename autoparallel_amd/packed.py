@@ -280,7 +280,7 @@ class PackedGraph:
         NE = self.num_edges
         rec = np.zeros(NE, self.EDGE_DTYPE)
         assert rec.dtype.itemsize == 64
-        rec["table_off"] = self.run_table()[3]
+        rec["table_off"] = self.block_table()[3]
         # division by ssrc as a multiply-high (exact while local * ssrc < 2**32)
         ssrc = self.edge_ssrc.astype(np.int64)
         ok = (ssrc > 1) & (ssrc * ssrc * self.edge_sdst < 2**32)
@@ -308,33 +308,43 @@ class PackedGraph:
     def max_rank(self) -> int:
         return int(self.meta_rank.max()) if self.meta_rank.shape[0] else 0
 
-    def run_table(self):
-        """Layout of the row table.  A *run* is a producer's list of output
-        specs (identified by its offset in ``lists``); its table holds, for
-        every placement tuple t, the row ``cost(run[j] -> t), j < S_src``, so an
-        output row of any edge fed by that run is one contiguous table row.
-        Returns (run_list int64[R], run_len int32[R], run_table_off int64[R+1],
-        edge_table_off int64[NE] (-1 without a producer))."""
+    def block_table(self):
+        """Layout of the block table: one S_dst x S_src cost matrix per distinct
+        (producer run, consumer run) pair among the edges that have a producer
+        and no missing spec on either side (runs are identified by their offset
+        in ``lists``: identical runs are stored once).  Every matrix is padded to
+        a multiple of 256 elements so that a 256-thread block of the table
+        kernel works on one matrix.
+        Returns (block_edge int32[B] one edge per matrix, block_off int64[B+1],
+        unit_block int32[table_size / 256], edge_table_off int64[NE] (-1 for
+        edges that are evaluated directly))."""
+        cached = getattr(self, "_block_table", None)
+        if cached is not None:
+            return cached
+        NE = self.num_edges
+        edge_table_off = np.full(NE, -1, np.int64)
+        none_before = np.concatenate([[0], np.cumsum(self.lists == SPEC_NONE)])
         hp = (self.edge_flags & EDGE_HAS_PRODUCER) != 0
-        nt = self.tuple_plc.shape[0]
-        edge_table_off = np.full(self.num_edges, -1, np.int64)
-        if not hp.any():
-            return (np.zeros(0, np.int64), np.zeros(0, np.int32), np.zeros(1, np.int64), edge_table_off)
-        offs, first, inv = np.unique(self.edge_src_list[hp], return_index=True, return_inverse=True)
-        run_len = self.edge_ssrc[hp][first].astype(np.int32)
-        assert (self.edge_ssrc[hp] == run_len[inv]).all(), "one run, two lengths"
-        # each run's table is padded to a multiple of 256 elements so that a
-        # 256-thread block of the table kernel never spans two runs
-        run_table_off = np.zeros(offs.shape[0] + 1, np.int64)
-        np.cumsum((run_len.astype(np.int64) * nt + 255) & ~255, out=run_table_off[1:])
-        edge_table_off[hp] = run_table_off[:-1][inv]
-        return offs.astype(np.int64), run_len, run_table_off, edge_table_off
-
-    def table_block_runs(self) -> np.ndarray:
-        """int32[table_size / 256]: the run each 256-element block of the row
-        table belongs to."""
-        _, _, off, _ = self.run_table()
-        return np.repeat(np.arange(off.shape[0] - 1, dtype=np.int32), np.diff(off) // 256)
+        src = np.where(hp, self.edge_src_list, 0).astype(np.int64)
+        dst = self.edge_dst_list.astype(np.int64)
+        ssrc, sdst = self.edge_ssrc.astype(np.int64), self.edge_sdst.astype(np.int64)
+        has_none = (none_before[src + ssrc] - none_before[src] > 0) | (none_before[dst + sdst] - none_before[dst] > 0)
+        ok = np.nonzero(hp & ~has_none & (ssrc * sdst > 0))[0]
+        if ok.shape[0] == 0:
+            out = (np.zeros(0, np.int32), np.zeros(1, np.int64), np.zeros(0, np.int32), edge_table_off)
+        else:
+            key = np.stack([src[ok], dst[ok], ssrc[ok], sdst[ok]], axis=1)
+            _, first, inv = np.unique(key, axis=0, return_index=True, return_inverse=True)
+            inv = inv.reshape(-1)
+            block_edge = ok[first].astype(np.int32)
+            size = ssrc[block_edge] * sdst[block_edge]
+            block_off = np.zeros(block_edge.shape[0] + 1, np.int64)
+            np.cumsum((size + 255) & ~255, out=block_off[1:])
+            edge_table_off[ok] = block_off[:-1][inv]
+            unit_block = np.repeat(np.arange(block_edge.shape[0], dtype=np.int32), np.diff(block_off) // 256)
+            out = (block_edge, block_off, unit_block, edge_table_off)
+        object.__setattr__(self, "_block_table", out)
+        return out
 
     def chunk_edge_index(self) -> np.ndarray:
         """int32[num_slots / 16]: the edge that owns each 16-slot chunk (blocks

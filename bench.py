@@ -56,7 +56,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--score-assignments", type=int, default=1 << 20,
                     help="also score this many on-device generated assignments (0 = skip)")
-    ap.add_argument("--direct", action="store_true", help="evaluate every entry directly (no row table)")
+    ap.add_argument("--direct", action="store_true", help="evaluate every entry directly (no block table)")
     ap.add_argument("--calibration-copy-mib", type=int, default=0,
                     help="after the timed steps, also launch the plain copy kernel on this many MiB "
                          "(the known-traffic reference for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)")
@@ -145,8 +145,8 @@ def main():
             "strategies": int(g.node_nstrat.sum()),
             "tensor_metas": int(g.meta_rank.shape[0]),
             "placement_tuples": int(g.tuple_plc.shape[0]),
-            "row_table": bool(eng.use_table),
-            "row_table_doubles": int(eng.table.numel()) if eng.table is not None else 0,
+            "block_table": bool(eng.use_table),
+            "block_table_doubles": int(eng.table.numel()) if eng.table is not None else 0,
             "compute_slots": g.num_compute,
             "evaluated_nodes": int(g.comp_nodes.shape[0]),
             "device": eng.device_name,

@@ -60,7 +60,7 @@ typedef struct apc_edge {
   int32_t flags;
   int32_t node;
   int32_t src_node;  /* producer node or -1                                   */
-  int64_t table_off; /* row table of the producer's run, or -1                */
+  int64_t table_off; /* first element of the edge's matrix in the block table, or -1 */
   uint32_t magic;    /* floor(2^32 / ssrc) + 1 if ssrc > 1 and ssrc * ssrc * sdst
                         < 2^32 (then local / ssrc == umulhi(local, magic)), else 0 */
   uint32_t local0;   /* 0 in the edge table; in a work item, its first entry  */
@@ -196,16 +196,18 @@ typedef struct apc_problem {
   const apc_edge* items;     /* [n_item] */
   int64_t n_default;
   const double* default_vals;
-  /* row tables: run r is the S_src spec words at lists[run_list[r]]; its table
-   * is table[run_table_off[r] + t * run_len[r] + j] = cost(run[j] -> tuple t);
-   * each run's table is padded to a multiple of 256 elements */
-  int32_t n_run;
-  const int64_t* run_list;
-  const int32_t* run_len;
-  const int64_t* run_table_off; /* [n_run+1], multiples of 256 */
-  int64_t table_size;           /* doubles: run_table_off[n_run] */
-  int32_t n_table_block;        /* table_size / 256 */
-  const int32_t* table_block_run; /* [n_table_block] run owning elements [256 b, 256 b + 256) */
+  /* block table: one S_dst x S_src matrix per distinct (producer run, consumer
+   * run) pair among the edges that have a producer and no missing spec, in the
+   * edge block's [out_idx][inp_idx] order: table[block_off[b] + out_idx * S_src
+   * + inp_idx] = comm cost, with the sign bit set when the two placements
+   * differ.  Each matrix is padded to a multiple of 256 elements;
+   * apc_edge.table_off is the matrix of the edge (-1: evaluate directly). */
+  int32_t n_block;
+  const int32_t* block_edge;       /* [n_block] an edge that owns matrix b          */
+  const int64_t* block_off;        /* [n_block+1], multiples of 256                  */
+  int64_t table_size;              /* doubles: block_off[n_block]                    */
+  int32_t n_table_unit;            /* table_size / 256                               */
+  const int32_t* table_unit_block; /* [n_table_unit] matrix owning elements [256 u, 256 u + 256) */
 } apc_problem;
 
 int apc_version(void);
@@ -243,8 +245,8 @@ int apc_nccl_plan_for_topo(const apc_nccl_config* cfg, int32_t n_ranks, int32_t 
                            int32_t n_channels, double bw_intra, double bw_inter,
                            struct apc_nccl_plan* plan);
 
-/* Number of doubles of the row table apc_build_pair_table fills
- * (= p->table_size: sum over runs of run_len * n_tuple). */
+/* Number of doubles of the block table apc_build_pair_table fills
+ * (= p->table_size). */
 int64_t apc_pair_table_size(const apc_problem* p);
 
 /* Replaces estimate_strategy_comms_cost + redistribute_cost + collective_comm_cost
@@ -252,9 +254,10 @@ int64_t apc_pair_table_size(const apc_problem* p);
  * 115-229, 239-262), torch's allgather/allreduce/reduce_scatter_cost
  * (torch:distributed/tensor/_collective_utils.py:281-313) and
  * compute_read_write_time (autoparallel/cost_models/compute_estimation.py:391-403),
- * evaluated for every (producer output spec, target placements) pair that the
- * entry kernel can ask for: table[run_table_off[r] + tgt * run_len[r] + j],
- * microseconds, +inf for forbidden transitions. */
+ * evaluated once per distinct (producer strategies, consumer strategies) matrix:
+ * table[block_off[b] + out_idx * S_src + inp_idx], microseconds, +inf for
+ * forbidden transitions, sign bit = the transition flag of
+ * _compute_edge_costs (autoparallel/optimize_sharding.py:474-478). */
 int apc_build_pair_table(const apc_problem* p, double* table, void* stream);
 
 /* Replaces estimate_strategy_runtime_cost
