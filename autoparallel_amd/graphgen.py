@@ -203,6 +203,43 @@ class Tracer:
             self.node_users.setdefault(u, []).append(v)
         return out_ts
 
+    def _emit_fixed(self, name: str, args: List[T], outs_meta, in_plcs, out_plcs, tuple_output: bool) -> List[T]:
+        """A node with exactly one strategy and no compute estimate."""
+        v = len(self.b.nodes)
+        out_ts = [T(v, (k if tuple_output else None), tuple(s), tuple(st), dt) for k, (s, st, dt) in enumerate(outs_meta)]
+        for plc, t_ in list(zip(in_plcs, args)) + list(zip(out_plcs, out_ts)):
+            assert _valid(t_.shape, plc, self.mesh_shape), (name, t_.shape, plc)
+        ins = [self.b.spec(self.b.meta(a.shape, a.stride, a.itemsize, a.dtype), tuple(p)) for a, p in zip(args, in_plcs)]
+        outs = [self.b.spec(self.b.meta(t_.shape, t_.stride, t_.itemsize, t_.dtype), tuple(p))
+                for t_, p in zip(out_ts, out_plcs)]
+        inputs = [a.node for a in args]
+        self.b.add_node(NodeDesc(name=f"{name}_{v}", in_specs=[ins], out_specs=[outs], inputs=inputs, op=OP_ZERO,
+                                 tuple_output=tuple_output))
+        self.node_inputs[v] = list(inputs)
+        for u in inputs:
+            self.node_users.setdefault(u, []).append(v)
+        return out_ts
+
+    def local_map(self, name: str, args: List[T], in_plcs, out_meta, out_plc, grad_plcs) -> T:
+        """An opaque region with declared placements, as the reference sees a
+        ``local_map`` call: one strategy (the declared input/output placements,
+        autoparallel/shardings/placement_options.py:455-490) and no compute
+        estimate (the target is a higher-order op, not an OpOverload:
+        autoparallel/cost_models/compute_estimation.py:368-380); only the
+        redistribution of its inputs into ``in_plcs`` is priced.  The backward
+        is another such node taking the output gradient and the saved inputs,
+        producing one gradient per input with placement ``grad_plcs[i]``."""
+        out = self._emit_fixed(name, args, [out_meta], in_plcs, [out_plc], tuple_output=False)[0]
+
+        def vjp(g):
+            metas = [(a.shape, a.stride, a.dtype) for a in args]
+            gs = self._emit_fixed(name + "_backward", [g[0]] + list(args), metas, [out_plc] + list(in_plcs),
+                                  list(grad_plcs), tuple_output=True)
+            return [self.getitem(x) for x in gs]
+
+        self._record(list(args), [out], vjp)
+        return out
+
     def placeholder(self, name: str, shape, dtype: int, param: bool = False, requires_grad=False) -> T:
         """Parameters and inputs: every {Replicate, Shard(d)} combination that
         survives the validity filter (propagation_rules.py:184-201)."""
@@ -574,6 +611,15 @@ class Tracer:
         return self._emit(name, args, [(x.shape, contiguous_stride(x.shape), x.dtype)], opts,
                           opprog.same_as_arg(0, x.rank, x.itemsize), sig_extra=(dim,))[0]
 
+    def softmax(self, x: T, dim: int = -1) -> T:
+        out = self.softmax_like("softmax", [x], dim)
+
+        def vjp(g):
+            return [self.softmax_like("softmax_backward", [g[0], out], dim)]
+
+        self._record([x], [out], vjp)
+        return out
+
     # ---- attention ------------------------------------------------------------
     def sdpa(self, q: T, k: T, v: T) -> T:
         """aten._scaled_dot_product_flash_attention: tuple output (out, lse)."""
@@ -824,6 +870,120 @@ def llama_graph(
         if g is not None:
             param_grads[p.node] = t.alias(g)
     return t.finish(param_grads, [logits])
+
+
+def moe_dispatch_bytes(n_layers: int, n_experts: int, top_k: int, tokens: int, dim: int, itemsize: int,
+                       dp: int, ep: int, seed: int = 0) -> np.ndarray:
+    """Bytes one expert-parallel group moves in the dispatch all-to-all of each
+    MoE layer when the tokens per expert follow a Zipf(1.1) law (a benchmark
+    extension: the reference prices a local_map region at zero and only charges
+    the redistribution of its inputs).  Per layer: expert popularity is
+    rank^-1.1 over a random permutation of the experts
+    (numpy.random.default_rng(seed)); the tokens * top_k / dp routed slots of
+    one data-parallel group are split in that proportion; the collective is as
+    slow as its most loaded rank, so the volume is ep * (slots of the most
+    loaded rank's experts) * dim * itemsize."""
+    rng = np.random.default_rng(seed)
+    w = np.arange(1, n_experts + 1, dtype=np.float64) ** -1.1
+    w /= w.sum()
+    slots = tokens * top_k // dp
+    out = np.zeros(n_layers, np.int64)
+    per_rank = n_experts // ep
+    for i in range(n_layers):
+        load = np.floor(w[rng.permutation(n_experts)] * slots).astype(np.int64)
+        rank_load = load.reshape(ep, per_rank).sum(axis=1)
+        out[i] = int(ep * rank_load.max() * dim * itemsize)
+    return out
+
+
+def moe_graph(
+    mesh_shape: Sequence[int] = (8, 8),
+    n_layers: int = 16,
+    dim: int = 2048,
+    n_heads: int = 16,
+    n_experts: int = 64,
+    top_k: int = 6,
+    expert_ffn: int = 1408,
+    vocab: int = 129280,
+    seq: int = 4096,
+    batch: int = 32,
+    devices_per_host: int = 8,
+    dtype: int = DT_BF16,
+) -> PackedGraph:
+    """DeepSeek-V3-style MoE decoder, forward + backward, on a (dp, ep) mesh:
+    attention and a dense shared expert are planned by the optimizer; the
+    routed-expert dispatch is a ``local_map`` region with the declared
+    placements of the reference's MoE recipe (docs/local_map_and_moe.md:246-268):
+    tokens and gate scores (Shard(0), Shard(0)), expert weights
+    (Replicate, Shard(0)), output (Shard(0), Shard(0))."""
+    t = Tracer(mesh_shape, devices_per_host)
+    assert t.ndim == 2, "the MoE recipe is written for a (dp, ep) mesh"
+    hd = dim // n_heads
+    params: Dict[str, T] = {}
+
+    def P_(name, shape):
+        params[name] = t.placeholder(name, shape, dtype, param=True)
+        return params[name]
+
+    S0, PS = shard(0), PARTIAL_SUM
+    tok_emb = P_("tok_embeddings.weight", (vocab, dim))
+    layers = []
+    for i in range(n_layers):
+        layers.append(dict(
+            attn_norm=P_(f"layers.{i}.attention_norm.weight", (dim,)),
+            wq=P_(f"layers.{i}.attention.wq.weight", (dim, dim)),
+            wk=P_(f"layers.{i}.attention.wk.weight", (dim, dim)),
+            wv=P_(f"layers.{i}.attention.wv.weight", (dim, dim)),
+            wo=P_(f"layers.{i}.attention.wo.weight", (dim, dim)),
+            ffn_norm=P_(f"layers.{i}.ffn_norm.weight", (dim,)),
+            gate=P_(f"layers.{i}.moe.gate.weight", (n_experts, dim)),
+            ew1=P_(f"layers.{i}.moe.expert_w1", (n_experts, dim, expert_ffn)),
+            ew2=P_(f"layers.{i}.moe.expert_w2", (n_experts, expert_ffn, dim)),
+            sw1=P_(f"layers.{i}.moe.shared.w1.weight", (expert_ffn, dim)),
+            sw2=P_(f"layers.{i}.moe.shared.w2.weight", (dim, expert_ffn)),
+            sw3=P_(f"layers.{i}.moe.shared.w3.weight", (expert_ffn, dim)),
+        ))
+    norm_w = P_("norm.weight", (dim,))
+    out_w = P_("output.weight", (vocab, dim))
+    cos = t.placeholder("rope_cos", (1, seq, 1, hd), DT_F32)
+    sin = t.placeholder("rope_sin", (1, seq, 1, hd), DT_F32)
+    tokens = t.placeholder("tokens", (batch, seq), DT_OTHER)
+    tangent = t.placeholder("tangents_1", (batch, seq, vocab), dtype)
+
+    h = t.embedding(tok_emb, tokens)
+    for L in layers:
+        x = _rmsnorm(t, h, L["attn_norm"])
+        q, k, v = (t.view(_linear(t, x, L[w]), (batch, seq, n_heads, hd)) for w in ("wq", "wk", "wv"))
+        q = _rope(t, q, cos, sin)
+        k = _rope(t, k, cos, sin)
+        q, k, v = (t.transpose(z, 1, 2) for z in (q, k, v))
+        o = t.clone(t.transpose(t.sdpa(q, k, v), 1, 2))
+        h = t.add(h, _linear(t, t.view(o, (batch, seq, dim)), L["wo"]))
+        x = _rmsnorm(t, h, L["ffn_norm"])
+        scores = t.softmax(_linear(t, x, L["gate"]))
+        x_flat = t.view(x, (batch * seq, dim))
+        g_flat = t.view(scores, (batch * seq, n_experts))
+        routed = t.local_map(
+            "local_map_moe", [x_flat, g_flat, L["ew1"], L["ew2"]],
+            in_plcs=[(S0, S0), (S0, S0), (R, S0), (R, S0)],
+            out_meta=(x_flat.shape, x_flat.stride, x_flat.dtype), out_plc=(S0, S0),
+            grad_plcs=[(S0, S0), (S0, S0), (PS, S0), (PS, S0)])
+        shared = _linear(t, t.mul(t.unary("silu", _linear(t, x, L["sw1"])), _linear(t, x, L["sw3"])), L["sw2"])
+        h = t.add(t.add(h, t.view(routed, (batch, seq, dim))), shared)
+    h = _rmsnorm(t, h, norm_w)
+    logits = _linear(t, h, out_w)
+    grads = t.backward([(logits, tangent)])
+    t._tangents = [(logits, tangent)]
+    param_grads = {}
+    for name, p in params.items():
+        g = grads.get((p.node, None))
+        if g is not None:
+            param_grads[p.node] = t.alias(g)
+    return t.finish(param_grads, [logits])
+
+
+def config_moe(n_layers: int = 16) -> PackedGraph:
+    return moe_graph((8, 8), n_layers)
 
 
 def _layernorm(t: Tracer, x: T, w: T, b: T) -> T:

@@ -137,6 +137,9 @@ GRAPHS = {
     "llama_3d": lambda: graphgen.llama_graph((2, 4, 2), 1, 512, 8, 4, 1024, 4096, 256, 16),
     "llama_odd_mesh": lambda: graphgen.llama_graph((3, 5), 1, 960, 15, 5, 1920, 3000, 240, 30),
     "stress_3d": lambda: graphgen.stress_graph(150, (4, 8, 8), seed=1, s_max=48),
+    "llama70b_1layer_3d": lambda: graphgen.config_llama3_70b(1),  # config 3 dims on (4,8,8)
+    "moe_1layer_real_dims": lambda: graphgen.config_moe(1),  # config 4 dims on (8,8), local_map nodes
+    "moe_tiny": lambda: graphgen.moe_graph((2, 4), 2, 64, 4, 8, 2, 32, 256, 32, 8),
     "pairs_4d": lambda: _pairs_graph((2, 3, 2, 4), (48, 36, 40), 300),
     "pairs_3d_noncontig": lambda: _pairs_graph((4, 8, 8), (256, 8192, 64), 250, stride=(64, 16384, 1)),
 }
@@ -155,7 +158,8 @@ def _pairs_graph(mesh, shape, n, stride=None, seed=3):
 
 # every graph through the table path; direct evaluation on the smaller ones
 CASES = [(n, True) for n in GRAPHS] + [
-    (n, False) for n in ("llama_2d", "gpt2_1d", "llama_odd_mesh", "stress_3d", "pairs_4d", "pairs_3d_noncontig")
+    (n, False) for n in ("llama_2d", "gpt2_1d", "llama_odd_mesh", "stress_3d", "pairs_4d", "pairs_3d_noncontig",
+                         "moe_tiny")
 ]
 
 
@@ -164,6 +168,41 @@ def test_graph_parity(CostEngine, name, use_table):
     g = GRAPHS[name]()
     print(f"graph {name}", flush=True)
     _check_build(CostEngine, g, use_table)
+
+
+def test_moe_local_map_nodes_and_dispatch_volume(CostEngine):
+    """Config 4: the routed-expert region is a single-strategy node priced at
+    zero compute whose inputs are redistributed into the declared placements;
+    the Zipf-weighted dispatch all-to-all is priced by the collective entry
+    point (benchmark extension, not part of the entry parity)."""
+    import ctypes as C
+
+    from autoparallel_amd import _lib
+    from autoparallel_amd.engine import make_model
+
+    g = graphgen.config_moe(1)
+    eng, got, ref = _check_build(CostEngine, g, True)
+    lm = [v for v, n in enumerate(g.node_names) if n.startswith("local_map_moe")]
+    assert len(lm) == 2  # forward and backward region
+    for v in lm:
+        assert int(g.node_nstrat[v]) == 1 and int(g.node_op[v]) == packed.OP_ZERO
+        assert got["compute"][int(g.node_comp_off[v])] == 0.0
+        for e in range(int(g.node_edge_off[v]), int(g.node_edge_off[v + 1])):
+            blk = got["comm"][int(g.edge_off[e]): int(g.edge_off[e]) + int(g.edge_ssrc[e])]
+            assert np.isfinite(blk).any() and (blk[np.isfinite(blk)] >= 0).all()
+            assert (blk == 0).any()  # the producer can already hold the declared placement
+    nbytes = graphgen.moe_dispatch_bytes(16, 64, 6, 32 * 4096, 2048, 2, 8, 8, seed=0)
+    assert nbytes.shape == (16,) and (nbytes > 0).all()
+    lib = _lib.load()
+    m = make_model((8, 8), 8, "AMD Instinct MI355X")
+    d = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    kind, dim = d(np.full(16, 1, np.int32)), d(np.full(16, 1, np.int32))
+    nb, out = d(nbytes), torch.empty(16, dtype=torch.float64, device="cuda")
+    assert lib.apc_collective_costs(C.byref(m), 16, kind.data_ptr(), nb.data_ptr(), dim.data_ptr(), out.data_ptr(), None) == 0
+    torch.cuda.synchronize()
+    topo = O.Topo((8, 8), 8)
+    want = np.asarray([O.collective_comm_cost("all_to_all", int(b), topo, 1) for b in nbytes])
+    assert bits_equal(out.cpu().numpy(), want)
 
 
 def test_clamp_inf(CostEngine):
