@@ -148,6 +148,13 @@ _SIGNATURES = {
         C.c_int,
         [C.POINTER(ApcProblem), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
          C.c_int32, C.c_void_p]),
+    "apc_timer_create": (C.c_int, [C.c_int32, C.POINTER(C.c_void_p)]),
+    "apc_timer_destroy": (C.c_int, [C.c_void_p]),
+    "apc_timer_elapsed_ms": (C.c_int, [C.c_void_p, C.c_int32, C.POINTER(C.c_float)]),
+    "apc_edge_costs_timed": (
+        C.c_int,
+        [C.POINTER(ApcProblem), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+         C.c_int32, C.c_void_p, C.c_int32, C.c_void_p]),
     "apc_prepare": (
         C.c_int,
         [C.POINTER(ApcProblem), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),

@@ -8,6 +8,7 @@
 // a chain of separately rounded binary64 operations, and the results here are
 // bit-identical to it.
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 #include <math.h>
 #include <stdint.h>
 #include <stdio.h>
@@ -1273,8 +1274,10 @@ int apc_prepare(const apc_problem* p, double* table, double* compute, double* pe
                         (hipStream_t)stream);
 }
 
-int apc_edge_costs(const apc_problem* p, const double* table, const double* per_arg, double* comm,
-                   double* cost, uint8_t* flags, int32_t clamp_inf, void* stream) {
+// start / stop: events recorded at the kernel's own begin and end (NULL: none)
+static int launch_edge_costs(const apc_problem* p, const double* table, const double* per_arg,
+                             double* comm, double* cost, uint8_t* flags, int32_t clamp_inf,
+                             hipStream_t stream, hipEvent_t start, hipEvent_t stop) {
   if (int rc = validate_problem(p)) return rc;
   if (p->n_entry == 0) return 0;
   if (!per_arg) return fail(APC_ERR_INVALID, "apc_edge_costs: null per_arg%s");
@@ -1282,12 +1285,67 @@ int apc_edge_costs(const apc_problem* p, const double* table, const double* per_
   const unsigned cap = 4096;  // 4 waves per block: twice the 8192 resident wave slots
   if (grid > cap) grid = cap;
   if (table)
-    hipLaunchKernelGGL(edge_cost_kernel<true>, dim3(grid), dim3(kBlock), 0, (hipStream_t)stream,
-                       *p, table, per_arg, comm, cost, flags, clamp_inf);
+    hipExtLaunchKernelGGL(edge_cost_kernel<true>, dim3(grid), dim3(kBlock), 0, stream, start, stop, 0,
+                          *p, table, per_arg, comm, cost, flags, clamp_inf);
   else
-    hipLaunchKernelGGL(edge_cost_kernel<false>, dim3(grid), dim3(kBlock), 0, (hipStream_t)stream,
-                       *p, table, per_arg, comm, cost, flags, clamp_inf);
+    hipExtLaunchKernelGGL(edge_cost_kernel<false>, dim3(grid), dim3(kBlock), 0, stream, start, stop, 0,
+                          *p, table, per_arg, comm, cost, flags, clamp_inf);
   return check_launch("edge_cost_kernel");
+}
+
+int apc_edge_costs(const apc_problem* p, const double* table, const double* per_arg, double* comm,
+                   double* cost, uint8_t* flags, int32_t clamp_inf, void* stream) {
+  return launch_edge_costs(p, table, per_arg, comm, cost, flags, clamp_inf, (hipStream_t)stream,
+                           nullptr, nullptr);
+}
+
+struct apc_timer {
+  int32_t n;
+  hipEvent_t* ev;  // 2 n events: start and stop of each slot
+};
+
+int apc_timer_create(int32_t n_slots, void** timer) {
+  if (n_slots <= 0 || !timer) return fail(APC_ERR_INVALID, "apc_timer_create: need n_slots > 0 and a result pointer%s");
+  apc_timer* t = new apc_timer{n_slots, new hipEvent_t[2 * (size_t)n_slots]};
+  for (int i = 0; i < 2 * n_slots; ++i) {
+    if (hipEventCreate(&t->ev[i]) != hipSuccess) {
+      for (int j = 0; j < i; ++j) (void)hipEventDestroy(t->ev[j]);
+      delete[] t->ev;
+      delete t;
+      return fail(APC_ERR_LAUNCH, "apc_timer_create: hipEventCreate failed%s");
+    }
+  }
+  *timer = t;
+  return 0;
+}
+
+int apc_timer_destroy(void* timer) {
+  apc_timer* t = static_cast<apc_timer*>(timer);
+  if (!t) return 0;
+  for (int i = 0; i < 2 * t->n; ++i) (void)hipEventDestroy(t->ev[i]);
+  delete[] t->ev;
+  delete t;
+  return 0;
+}
+
+int apc_timer_elapsed_ms(void* timer, int32_t slot, float* ms) {
+  apc_timer* t = static_cast<apc_timer*>(timer);
+  if (!t || slot < 0 || slot >= t->n || !ms) return fail(APC_ERR_INVALID, "apc_timer_elapsed_ms: bad timer or slot%s");
+  hipError_t e = hipEventElapsedTime(ms, t->ev[2 * slot], t->ev[2 * slot + 1]);
+  if (e != hipSuccess) {
+    snprintf(g_err, sizeof(g_err), "apc_timer_elapsed_ms: %s", hipGetErrorString(e));
+    return APC_ERR_LAUNCH;
+  }
+  return 0;
+}
+
+int apc_edge_costs_timed(const apc_problem* p, const double* table, const double* per_arg,
+                         double* comm, double* cost, uint8_t* flags, int32_t clamp_inf, void* timer,
+                         int32_t slot, void* stream) {
+  apc_timer* t = static_cast<apc_timer*>(timer);
+  if (!t || slot < 0 || slot >= t->n) return fail(APC_ERR_INVALID, "apc_edge_costs_timed: bad timer or slot%s");
+  return launch_edge_costs(p, table, per_arg, comm, cost, flags, clamp_inf, (hipStream_t)stream,
+                           t->ev[2 * slot], t->ev[2 * slot + 1]);
 }
 
 int apc_build_all(const apc_problem* p, double* table, double* compute, double* per_arg,

@@ -239,6 +239,17 @@ class CostEngine:
             "apc_edge_costs",
         )
 
+    def edge_costs_timed(self, timer, slot: int, clamp_inf: bool = True):
+        """edge_costs with HIP events at the kernel's begin and end (a timer from
+        apc_timer_create); the launch is otherwise identical."""
+        _lib.check(
+            self.lib.apc_edge_costs_timed(
+                C.byref(self.problem), self._ptr(self.table), self._ptr(self.per_arg), self._ptr(self.comm),
+                self._ptr(self.cost), self._ptr(self.flags), int(bool(clamp_inf)), timer, int(slot),
+                self._stream()),
+            "apc_edge_costs_timed",
+        )
+
     def prepare(self):
         """Pair table and node compute vectors in one launch."""
         _lib.check(
@@ -280,6 +291,21 @@ class CostEngine:
         self.per_arg.copy_(torch.from_numpy(np.ascontiguousarray(per_arg, np.float64)))
         self.built = True
         return self
+
+    def capture_build(self, clamp_inf: bool = True) -> "torch.cuda.CUDAGraph":
+        """The two launches of build() recorded in a HIP graph, for callers that
+        replay a whole planning step from a graph (measured here, a replay takes
+        41.7 us against 38 us for the two eager launches: no gain on its own).
+        The graph holds kernel
+        nodes only (no memset nodes); it is valid while this engine's buffers
+        live.  build() is run once eagerly first so that one-time function
+        attributes are set outside the capture."""
+        self.build(clamp_inf)
+        torch.cuda.synchronize(self.device)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            self.build(clamp_inf)
+        return graph
 
     def check_status(self):
         if int(self.status.item()) != 0:

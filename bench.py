@@ -86,23 +86,39 @@ def main():
     torch.cuda.synchronize()
 
     # HIP events on the launch stream (torch's current stream is the one the
-    # engine launches on) bracket the two launches of every timed step
-    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
+    # engine launches on), recorded at the begin and end of the dominant kernel
+    # of every timed step (apc_edge_costs_timed: the events are attached to the
+    # kernel's own dispatch, so dispatch latency is not counted)
+    import ctypes as C
+
+    timer = C.c_void_p()
+    assert eng.lib.apc_timer_create(args.steps, C.byref(timer)) == 0
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for k in range(args.steps):
-        ev[k][0].record()
         eng.prepare()
-        ev[k][1].record()
-        eng.edge_costs(clamp_inf=True)
-        ev[k][2].record()
+        eng.edge_costs_timed(timer, k, clamp_inf=True)
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     eng.check_status()
+    ms = C.c_float()
+    t_edge = 0.0
+    for k in range(args.steps):
+        assert eng.lib.apc_timer_elapsed_ms(timer, k, C.byref(ms)) == 0
+        t_edge += ms.value
+    t_edge = t_edge / args.steps * 1e-3
+    eng.lib.apc_timer_destroy(timer)
+
+    # outside the timed region: the prepare kernel bracketed the same way, for the report
+    pe = [[torch.cuda.Event(enable_timing=True) for _ in range(2)] for _ in range(20)]
+    for a, b in pe:
+        a.record()
+        eng.prepare()
+        b.record()
+        eng.edge_costs(clamp_inf=True)
+    torch.cuda.synchronize()
 
     if args.calibration_copy_mib > 0:
-        import ctypes as C
-
         nbytes = args.calibration_copy_mib << 20
         a = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
         b = torch.empty_like(a)
@@ -110,8 +126,7 @@ def main():
             eng.lib.apc_calibration_copy(C.c_void_p(a.data_ptr()), C.c_void_p(b.data_ptr()), nbytes, eng._stream())
         torch.cuda.synchronize()
 
-    t_prep = sum(e[0].elapsed_time(e[1]) for e in ev) / args.steps * 1e-3
-    t_edge = sum(e[1].elapsed_time(e[2]) for e in ev) / args.steps * 1e-3
+    t_prep = sum(a.elapsed_time(b) for a, b in pe) / len(pe) * 1e-3
     ms_per_step = elapsed / args.steps * 1e3
 
     # algorithmic bytes of one edge_cost_kernel launch: per entry one fp64 comm,

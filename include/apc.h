@@ -298,6 +298,19 @@ int apc_build_all(const apc_problem* p, double* table, double* compute, double* 
                   int32_t* status, double* comm, double* cost, uint8_t* flags, int32_t clamp_inf,
                   void* stream);
 
+/* Measurement aids, no counterpart in the reference.  A timer owns n_slots
+ * pairs of HIP events (host objects, no device memory).  apc_edge_costs_timed
+ * is apc_edge_costs with the pair of `slot` recorded at the kernel's own begin
+ * and end on the launch stream (hipExtLaunchKernelGGL's start/stop events), so
+ * the elapsed time is the kernel's duration without dispatch latency; read it
+ * with apc_timer_elapsed_ms after synchronising the stream. */
+int apc_timer_create(int32_t n_slots, void** timer);
+int apc_timer_destroy(void* timer);
+int apc_timer_elapsed_ms(void* timer, int32_t slot, float* ms);
+int apc_edge_costs_timed(const apc_problem* p, const double* table, const double* per_arg,
+                         double* comm, double* cost, uint8_t* flags, int32_t clamp_inf, void* timer,
+                         int32_t slot, void* stream);
+
 /* Measurement aid, no counterpart in the reference: a plain device copy of
  * nbytes (multiple of 16) whose HBM traffic is known (nbytes read + nbytes
  * written), used to scale hardware traffic counters in profiles. */

@@ -205,6 +205,56 @@ def test_moe_local_map_nodes_and_dispatch_volume(CostEngine):
     assert bits_equal(out.cpu().numpy(), want)
 
 
+def test_graph_replay_matches_eager(CostEngine):
+    """The build captured in a HIP graph: every replay, with eager work and
+    synchronisations in between, gives the eager bits."""
+    g = GRAPHS["llama_2d"]()
+    eng = CostEngine(g)
+    eng.build(clamp_inf=True)
+    want = {k: v.copy() for k, v in eng.results().items()}
+    graph = eng.capture_build(clamp_inf=True)
+    for rep in range(4):
+        for t in (eng.comm, eng.cost, eng.compute, eng.per_arg):
+            t.fill_(-1.0)
+        eng.flags.fill_(255)
+        if eng.table is not None:
+            eng.table.fill_(-7.0)
+        torch.cuda.synchronize()
+        graph.replay()
+        got = eng.results()
+        slots = g.entry_slots()
+        for k in ("comm", "cost", "flags"):
+            assert bits_equal(got[k][slots], want[k][slots]), (rep, k)
+        assert bits_equal(got["compute"], want["compute"]) and bits_equal(got["per_arg"], want["per_arg"])
+        # eager work between replays
+        eng.build(clamp_inf=False)
+        torch.cuda.synchronize()
+
+
+def test_timed_launch_is_the_same_launch(CostEngine):
+    import ctypes as C
+
+    g = GRAPHS["llama_2d"]()
+    eng = CostEngine(g).build(clamp_inf=True)
+    want = eng.results()
+    timer = C.c_void_p()
+    assert eng.lib.apc_timer_create(3, C.byref(timer)) == 0
+    eng.cost.fill_(-1.0)
+    for k in range(3):
+        eng.edge_costs_timed(timer, k, clamp_inf=True)
+    got = eng.results()
+    slots = g.entry_slots()
+    assert bits_equal(got["cost"][slots], want["cost"][slots])
+    ms = C.c_float()
+    for k in range(3):
+        assert eng.lib.apc_timer_elapsed_ms(timer, k, C.byref(ms)) == 0
+        assert 0.0 < ms.value < 100.0
+    assert eng.lib.apc_timer_elapsed_ms(timer, 3, C.byref(ms)) != 0  # slot out of range
+    with pytest.raises(Exception):
+        eng.edge_costs_timed(timer, 7)
+    assert eng.lib.apc_timer_destroy(timer) == 0
+
+
 def test_clamp_inf(CostEngine):
     _check_build(CostEngine, GRAPHS["llama_2d"](), True, clamp=True)
 
