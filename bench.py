@@ -232,6 +232,23 @@ def main():
             "seconds": t_cpu,
         }
         out["speedup_vs_cpu_baseline"] = out["value"] / out["cpu_baseline"]["value"]
+        # also reported, and not the reference: the compiled (C, no memo cache)
+        # restatement on the same graph, one thread and all cores of the box's share
+        try:
+            from oracle import c_oracle
+
+            co = c_oracle.COracle(g)
+            arrays_c = co.build(threads=1)  # warm-up, and the output buffers to reuse
+            res = {}
+            for label, threads in (("1_thread", 1), ("all_cores", min(os.cpu_count() or 1, 16))):
+                reps, t0 = 0, time.perf_counter()
+                while reps < 3 or (time.perf_counter() - t0 < 2.0 and reps < 50):
+                    co.build(threads=threads, out=arrays_c)
+                    reps += 1
+                res[label] = {"threads": threads, "entries_per_s": E * reps / (time.perf_counter() - t0)}
+            out["cpu_baseline"]["compiled_port"] = res
+        except Exception as exc:  # the checker library is optional for the benchmark
+            out["cpu_baseline"]["compiled_port"] = {"error": str(exc)}
     print(json.dumps(out))
 
 
