@@ -32,6 +32,9 @@ def workloads():
         "gpt2_small_fwd_bwd_mesh8": lambda: G.config_gpt2_small(),
         # configs[2] at reduced depth fits a quick run; full depth via --layers
         "llama3_70b_fwd_bwd_mesh4x8x8": lambda: G.config_llama3_70b(),
+        # configs[3] and a seeded slice of configs[4] (3 000 of its 200 000 nodes)
+        "moe_16l_fwd_bwd_mesh8x8": lambda: G.config_moe(),
+        "stress_3k_mesh4x8x8": lambda: G.stress_graph(3000, (4, 8, 8), seed=0),
     }
 
 
