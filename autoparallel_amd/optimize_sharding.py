@@ -216,18 +216,13 @@ class ShardingOptimizer:
     def _prefetchable(self, roles: GraphRoles) -> set:
         """(node_idx, argi) of edges whose producer is parameter-derived or whose
         consumer is terminal-derived (autoparallel/graph_passes/graph_utils.py:447-484)."""
-        params = {self.nodes[p] for p, _ in roles.param_grad}
-        derived = set(params)
-        for node in self.graph.nodes:
-            ins = node.all_input_nodes
-            if ins and all(i in derived for i in ins):
-                derived.add(node)
-        terminal = {self.nodes[g] for _, g in roles.param_grad if g >= 0}
-        for node in reversed(list(self.graph.nodes)):
-            if node.op == "output":
-                continue
-            if node.users and all(u in terminal for u in node.users):
-                terminal.add(node)
+        from .graph_utils import build_param_derived_set, build_terminal_derived_set
+
+        try:
+            derived = build_param_derived_set(self.graph)
+            terminal = build_terminal_derived_set(self.graph)
+        except Exception:  # a graph without AOT descriptors has no parameters to prefetch
+            derived, terminal = set(), set()
         out = set()
         for node in self.nodes:
             if node.op == "output":

@@ -304,3 +304,54 @@ def test_repeated_subgraphs_on_joint_graph(mesh):
     assert np.isclose(opt._core.objective_value, plain._core.objective_value, rtol=1e-6)
     assert len(opt.selected_keys) == opt._packed.num_edges  # root keys plus the expanded linked keys
     assert "total_cost:" in opt.get_log()
+
+
+def test_prefetch_discount_on_joint_graph(mesh):
+    """apply_prefetch_discount(0) (reference tests/test_prefetch_derived_sets.py:262-296):
+    discounted variables have comm 0 and cost == compute + transition."""
+    from autoparallel_amd.optimize_sharding import ShardingOptimizer
+
+    opt = ShardingOptimizer(_joint_graph(), mesh, devices_per_host=8, device_name="AMD Instinct MI355X")
+    before = {k: dv.comm_cost for k, dv in opt.decision_vars.items() if 0 < dv.comm_cost < float("inf")}
+    assert before
+    n = opt.apply_prefetch_discount(scale=0.0)
+    assert n > 0
+    zeroed = 0
+    for k, dv in opt.decision_vars.items():
+        if k in before and dv.comm_cost == 0.0:
+            assert dv.cost == dv.compute_cost + dv.sharding_transition_cost
+            zeroed += 1
+    assert zeroed == n
+    # the strategies' redistribute_cost rows follow the discount
+    k = next(k for k in before if opt.decision_vars[k].comm_cost == 0.0)
+    assert opt.strats[opt.nodes[k[0]]].strategies[k[2]].redistribute_cost[k[1]][k[3]] == 0.0
+
+
+def test_rebuild_after_mutating_strategies(mesh):
+    """_build_decision_vars is re-entrant (reference tests/test_paired_output_constraint.py:30-158):
+    after removing one placement from a gradient node's strategies, the rebuilt
+    ILP disables the parameter strategies without a partner and the solution
+    never picks them."""
+    from torch._functorch._aot_autograd import fx_utils
+
+    from autoparallel_amd.optimize_sharding import ShardingOptimizer
+
+    gm = _joint_graph()
+    opt = ShardingOptimizer(gm, mesh, devices_per_host=8, device_name="AMD Instinct MI355X")
+    param, grad = next((p, g) for p, g in fx_utils.get_param_and_grad_nodes(gm.graph).values() if g is not None)
+    removed = str(opt.strats[grad].strategies[-1].output_specs.placements)
+    n_before = len(opt.decision_vars)
+    opt.strats[grad].strategies = [s for s in opt.strats[grad].strategies
+                                   if str(s.output_specs.placements) != removed]
+    opt.decision_vars = opt._build_decision_vars()
+    assert len(opt.decision_vars) < n_before
+    assert any("grad_param_constraint_disable" in name for name in opt.prob.constraints)
+    sol = opt.get_solution()
+    grad_plc = {str(s.output_specs.placements) for s in opt.strats[grad].strategies}
+    chosen = str(sol[param].output_specs.placements)
+    assert chosen in grad_plc and chosen != removed
+    # every variable of the unmatched parameter strategy is zero
+    pidx = opt.node_map[param]
+    bad = [i for i, s in enumerate(opt.strats[param].strategies) if str(s.output_specs.placements) == removed]
+    assert len(bad) == 1
+    assert all(k[2] != bad[0] for k in opt.selected_keys if k[0] == pidx)

@@ -1,0 +1,86 @@
+"""Host post-processing of operator strategies: the known answers of the
+reference's tests/test_placement_options_utils.py (:28-150), restated for
+autoparallel_amd.shardings.placement_options on a fake (CPU) mesh."""
+import pytest
+import torch
+from torch.distributed.tensor._dtensor_spec import DTensorSpec, TensorMeta
+from torch.distributed.tensor._op_schema import OpSpec, OpStrategy
+from torch.distributed.tensor.placement_types import Replicate, Shard
+
+from autoparallel_amd.shardings.placement_options import (
+    fill_redistribute_cost,
+    keep_unique_configs,
+    remove_invalid_configs,
+)
+from oracle import cost_oracle as O
+
+
+@pytest.fixture(scope="module")
+def meshes():
+    import torch.distributed as dist
+    from torch.distributed.device_mesh import init_device_mesh
+    from torch.testing._internal.distributed.fake_pg import FakeStore
+
+    if dist.is_initialized():
+        dist.destroy_process_group()
+    dist.init_process_group("fake", store=FakeStore(), rank=0, world_size=256)
+    yield init_device_mesh("cpu", (256,)), init_device_mesh("cpu", (32, 8))
+    dist.destroy_process_group()
+
+
+def _tm(shape, dtype=torch.float32):
+    t = torch.empty(shape, dtype=dtype, device="meta")
+    return TensorMeta(t.shape, t.stride(), t.dtype)
+
+
+def _one(mesh, shape, plc):
+    spec = DTensorSpec(mesh, plc, tensor_meta=_tm(shape))
+    return OpSpec(spec, input_specs=[spec], redistribute_cost=[[0.0]])
+
+
+@pytest.mark.parametrize("which,shape,plc,kept", [
+    (0, (256, 64), (Shard(0),), 1),            # divisible
+    (0, (100, 64), (Shard(0),), 0),            # 100 < 256: empty shards
+    (0, (7, 3), (Replicate(),), 1),            # replicate always kept
+    (1, (256, 10), (Shard(0), Shard(1)), 1),   # 10 >= 8: uneven but non-empty
+    (1, (257, 64), (Shard(0), Replicate()), 1),
+    (1, (31, 64), (Shard(0), Replicate()), 0),
+    (1, (64, 64), (Shard(0), Shard(0)), 0),    # 64/32 = 2, then 2 < 8
+    (1, (256, 64), (Shard(0), Shard(0)), 1),   # 256/32 = 8, then 8 >= 8
+])
+def test_remove_invalid_configs_known_answers(meshes, which, shape, plc, kept):
+    mesh = meshes[which]
+    out = remove_invalid_configs(OpStrategy([_one(mesh, shape, plc)]), mesh)
+    assert len(out.strategies) == kept
+    # the same rule as the oracle's per-spec test (and the device enumeration kernel's)
+    code = tuple(0 if isinstance(p, Replicate) else 0x40 | p.dim for p in plc)
+    assert O.is_valid_spec(shape, code, tuple(mesh.shape)) == bool(kept)
+
+
+def test_remove_invalid_configs_none_output_and_mix(meshes):
+    mesh = meshes[0]
+    spec = DTensorSpec(mesh, (Replicate(),), tensor_meta=_tm((256,)))
+    out = remove_invalid_configs(OpStrategy([OpSpec(None, input_specs=[spec], redistribute_cost=[[0.0]])]), mesh)
+    assert len(out.strategies) == 1
+    mix = OpStrategy([_one(mesh, (256, 64), (Shard(0),)), _one(mesh, (100, 64), (Shard(0),))])
+    assert len(remove_invalid_configs(mix, mesh).strategies) == 1
+
+
+def test_keep_unique_configs_known_answers(meshes):
+    mesh = meshes[0]
+    a = _one(mesh, (4, 8), (Replicate(),))
+    assert len(keep_unique_configs(OpStrategy([a, a])).strategies) == 1
+    b = _one(mesh, (256, 64), (Replicate(),))
+    c = _one(mesh, (256, 64), (Shard(0),))
+    assert len(keep_unique_configs(OpStrategy([b, c])).strategies) == 2
+    # equal content in distinct objects is still a duplicate
+    assert len(keep_unique_configs(OpStrategy([_one(mesh, (4, 8), (Replicate(),)), a])).strategies) == 1
+
+
+def test_fill_redistribute_cost_shapes(meshes):
+    mesh = meshes[0]
+    prod = OpStrategy([_one(mesh, (256, 64), (Replicate(),)), _one(mesh, (256, 64), (Shard(0),))])
+    spec = DTensorSpec(mesh, (Replicate(),), tensor_meta=_tm((256, 64)))
+    st = OpStrategy([OpSpec(spec, input_specs=[spec, spec])])
+    fill_redistribute_cost(st, [prod, prod])
+    assert st.strategies[0].redistribute_cost == [[0.0, 0.0], [0.0, 0.0]]
