@@ -460,3 +460,65 @@ class ShardingOptimizer:
         sol = serialization.load_placements(self._core, path, names)
         return {self.nodes[v]: self.strats[self.nodes[v]].strategies[int(sol[v])]
                 for v in range(self._packed.num_nodes)}
+
+    def explain_placement(self, target_placement, start_node=None, max_nodes=None) -> str:
+        """Why the optimizer did not choose ``target_placement``: per node, the
+        chosen placement with its compute and communication cost next to the
+        cost the target would have if every node that offers it used it (a node
+        that does not keeps its chosen strategy), as the reference's
+        explain_placement (:1227-1397).  The two plans' per-edge terms come from
+        the device (apc_solution_terms).  Call after get_solution()."""
+        from tabulate import tabulate
+        from torch.distributed.tensor._op_schema import _pretty_print_spec
+
+        g, core = self._packed, self._core
+        target = tuple(target_placement)
+        chosen = core._extract()
+        tgt_idx = np.full(g.num_nodes, -1, np.int64)
+        for v in range(g.num_nodes):
+            for i, s in enumerate(self.strats[self.nodes[v]].strategies):
+                if isinstance(s.output_specs, DTensorSpec) and s.output_specs.placements == target:
+                    tgt_idx[v] = i
+                    break
+        what_if = np.where(tgt_idx >= 0, tgt_idx, chosen)
+        terms_c, _ = core.solution_terms(chosen)
+        terms_t, _ = core.solution_terms(what_if)
+        rows, started = [], start_node is None
+        for v in range(g.num_nodes):
+            node = self.nodes[v]
+            if not started:
+                if node is not start_node:
+                    continue
+                started = True
+            if max_nodes is not None and len(rows) >= max_nodes:
+                break
+            spec = self.strats[node].strategies[int(chosen[v])].output_specs
+            if not isinstance(spec, DTensorSpec):
+                continue  # tuple-output nodes are skipped
+            e0, e1 = int(g.node_edge_off[v]), int(g.node_edge_off[v + 1])
+            prod = g.edge_src_node[e0:e1] >= 0
+            c_comp, c_comm = float(terms_c[e0:e1, 0].sum()), float(terms_c[e0:e1, 1][prod].sum())
+            shape = str(list(spec.tensor_meta.shape)) if spec.tensor_meta is not None else "?"
+            if tgt_idx[v] >= 0:
+                t_comp, t_comm = float(terms_t[e0:e1, 0].sum()), float(terms_t[e0:e1, 1][prod].sum())
+                if spec.placements == target:
+                    status = "CHOSEN"
+                elif abs((c_comp + c_comm) - (t_comp + t_comm)) < 0.01:
+                    status = "TIE"
+                elif t_comp + t_comm < c_comp + c_comm:
+                    status = "TARGET CHEAPER"
+                else:
+                    status = "CHOSEN CHEAPER"
+                if abs(t_comp - 7.0) < 0.01 and abs(c_comp - 7.0) < 0.01:
+                    status += " [floor]"
+                t_comp_s, t_comm_s = f"{t_comp:.1f}", f"{t_comm:.1f}"
+            else:
+                t_comp_s = t_comm_s = "N/A"
+                status = "UNAVAILABLE"
+            rows.append([str(node), shape, _pretty_print_spec(spec), f"{c_comp:.1f}", f"{c_comm:.1f}", t_comp_s,
+                         t_comm_s, status])
+        text = f"explain_placement: target={_pretty_print_spec(DTensorSpec(self.mesh, target))}\n\n"
+        text += tabulate(rows, headers=["Node", "Shape", "Chosen", "Ch.Comp", "Ch.Comm", "Tgt.Comp", "Tgt.Comm",
+                                        "Status"])
+        print(text)
+        return text

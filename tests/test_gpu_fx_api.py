@@ -106,6 +106,13 @@ def test_sharding_optimizer_on_joint_graph(mesh):
         opt.save_placements(tmp + "/plc.json")
         back = opt.load_placements(tmp + "/plc.json")
         assert all(str(back[n].output_specs) == str(sol[n].output_specs) for n in sol)
+    # counterfactual report: the all-Replicate plan is available everywhere and never cheaper in total
+    from torch.distributed.tensor.placement_types import Replicate as _R
+
+    text = opt.explain_placement((_R(), _R()))
+    assert text.startswith("explain_placement: target=") and "Tgt.Comm" in text
+    assert "UNAVAILABLE" not in text and ("CHOSEN CHEAPER" in text or "TIE" in text or "CHOSEN" in text)
+    assert len(opt.explain_placement((_R(), _R()), max_nodes=3).strip().split("\n")) == 2 + 2 + 3
     # a user constraint moves the plan and can be removed again
     x = next(n for n in gm.graph.nodes if n.name == "primals_3")
     from torch.distributed.tensor.placement_types import Replicate, Shard
