@@ -462,10 +462,11 @@ __device__ __forceinline__ uint32_t warm_problem(const apc_problem& p, int lane,
 // words have the same S_dst x S_src matrix of redistribution costs; one copy of
 // each distinct matrix is kept, in the edge block's own [out_idx][inp_idx]
 // order, padded to a multiple of 256 elements so that a workgroup works on one
-// matrix.  An element is the cost with its sign bit set when the two
-// placements differ (costs are never negative, so the sign is free to carry
-// the transition flag): the entry kernel reads comm and transition with one
-// coalesced load and no spec words.
+// matrix.  An edge with a producer and a missing spec has a matrix of its own
+// (the missing positions hold its default values).  An element is the cost
+// with its sign bit set when the two placements differ (costs are never
+// negative, so the sign is free to carry the transition flag): the entry kernel
+// reads comm and transition with one coalesced load and no spec words.
 __device__ __forceinline__ void pair_table_block(const apc_problem& p, double* __restrict__ table,
                                                  int unit) {
   const uint32_t keep = warm_problem(p, threadIdx.x, blockDim.x);
@@ -479,13 +480,17 @@ __device__ __forceinline__ void pair_table_block(const apc_problem& p, double* _
     const uint32_t o = l / ssrc, j = l - o * ssrc;
     const uint32_t sw = p.lists[(size_t)ed.src_list + j];
     const uint32_t tw = p.lists[(size_t)ed.dst_list + o];
-    const uint32_t st = sw & kTupleMask, tt = tw & kTupleMask;
-    int64_t nbytes;
-    bool contig;
-    meta_bytes_contig(p, sw >> APC_TUPLE_BITS, nbytes, contig);
-    const double c = redistribute_cost(load_tuple(p.tuple_plc, st), load_tuple(p.tuple_plc, tt),
-                                       nbytes, contig, p.model);
-    table[base + l] = (st != tt) ? -c : c;
+    if (sw != APC_SPEC_NONE && tw != APC_SPEC_NONE) {
+      const uint32_t st = sw & kTupleMask, tt = tw & kTupleMask;
+      int64_t nbytes;
+      bool contig;
+      meta_bytes_contig(p, sw >> APC_TUPLE_BITS, nbytes, contig);
+      const double c = redistribute_cost(load_tuple(p.tuple_plc, st), load_tuple(p.tuple_plc, tt),
+                                         nbytes, contig, p.model);
+      table[base + l] = (st != tt) ? -c : c;
+    } else {  // a missing spec keeps the default row's value and is no transition
+      table[base + l] = p.default_vals[ed.default_off + (int64_t)l];
+    }
   }
   asm volatile("" ::"v"(keep));
 }
@@ -535,8 +540,7 @@ __device__ __forceinline__ apc_edge find_edge(const apc_problem& p, int64_t idx)
 // comm / transition of one entry, general path (direct evaluation, missing
 // specs, default rows).
 __device__ __forceinline__ void eval_entry(const apc_problem& p, const apc_edge& ed, uint32_t o,
-                                           uint32_t j, const double* __restrict__ table,
-                                           double& comm, int& trans) {
+                                           uint32_t j, double& comm, int& trans) {
   const uint32_t tw = p.lists[(size_t)ed.dst_list + o];
   const uint32_t sw =
       (ed.flags & APC_EDGE_HAS_PRODUCER) ? p.lists[(size_t)ed.src_list + j] : APC_SPEC_NONE;
@@ -560,15 +564,9 @@ __device__ __forceinline__ void eval_entry(const apc_problem& p, const apc_edge&
 // measured on MI355X, stores whose 64 lanes cover one contiguous span stream
 // about 20% faster than lanes owning 32 contiguous bytes each.  The item record
 // is a copy of the edge record (plus local0), wave-uniform, so it lives in
-// scalar registers.  With a block table a lane loads, per entry, one table
-// element (cost and transition flag of the entry's position in the edge's
-// matrix: same order as the output, so the reads coalesce exactly like the
-// stores) and the per-arg compute term of its row, adds and stores; no spec
-// word is read.  Edges without a matrix in the table (no producer, a missing
-// spec, or no table at all) evaluate every entry directly.
-template <bool kUseTable>
+// scalar registers.  Without a block table every entry is evaluated directly
+// from its two spec words.
 __device__ __forceinline__ void process_item(const apc_problem& p, const apc_edge& ed, int lane,
-                                             const double* __restrict__ table,
                                              const double* __restrict__ per_arg,
                                              double* __restrict__ comm, double* __restrict__ cost,
                                              uint8_t* __restrict__ flags, int clamp_inf) {
@@ -587,26 +585,12 @@ __device__ __forceinline__ void process_item(const apc_problem& p, const apc_edg
   }
   double v_comm[kPerLane], v_pa[kPerLane];
   int v_trans[kPerLane];
-  if (kUseTable && ed.table_off >= 0) {  // wave-uniform
-    double raw[kPerLane];
 #pragma unroll
-    for (int k = 0; k < kPerLane; ++k) {
-      raw[k] = table[ed.table_off + (int64_t)(live[k] ? lk[k] : 0u)];
+  for (int k = 0; k < kPerLane; ++k) {
+    v_comm[k] = 0.0; v_pa[k] = 0.0; v_trans[k] = 0;
+    if (live[k]) {
+      eval_entry(p, ed, ok[k], jk[k], v_comm[k], v_trans[k]);
       v_pa[k] = per_arg[ed.comp_base + ok[k]];
-    }
-#pragma unroll
-    for (int k = 0; k < kPerLane; ++k) {
-      v_trans[k] = (int)((uint64_t)__double_as_longlong(raw[k]) >> 63);
-      v_comm[k] = fabs(raw[k]);
-    }
-  } else {
-#pragma unroll
-    for (int k = 0; k < kPerLane; ++k) {
-      v_comm[k] = 0.0; v_pa[k] = 0.0; v_trans[k] = 0;
-      if (live[k]) {
-        eval_entry(p, ed, ok[k], jk[k], table, v_comm[k], v_trans[k]);
-        v_pa[k] = per_arg[ed.comp_base + ok[k]];
-      }
     }
   }
   // ---- assemble (optimize_sharding.py:544) and store
@@ -624,8 +608,15 @@ __device__ __forceinline__ void process_item(const apc_problem& p, const apc_edg
   }
 }
 
-// Table path, split in two so that the loads of a wave's next item are in
-// flight while the current item is stored.
+// Table path.  A lane loads, per entry, one element of the edge's matrix (cost
+// and transition flag of the entry's position: same order as the output, so
+// the reads coalesce exactly like the stores) and the per-arg compute term of
+// its row, adds and stores; no spec word is read.  The matrix of an edge with a
+// producer is in the block table; an edge without one has no specs to compare,
+// and its matrix is its rows of default_vals as they are.  Split in two so that
+// the loads of a wave's next item are in flight while the current item is
+// stored.  The kernel needs a third of the registers of the direct one, which
+// is why the two do not share a body: eight waves per SIMD instead of three.
 struct ItemLoads {
   double raw[kPerLane];
   double pa[kPerLane];
@@ -634,9 +625,12 @@ struct ItemLoads {
 };
 
 __device__ __forceinline__ void item_load(const apc_edge& ed, int lane, const double* __restrict__ table,
+                                          const double* __restrict__ default_vals,
                                           const double* __restrict__ per_arg, ItemLoads& r) {
   const uint32_t ssrc = (uint32_t)ed.ssrc;
   const uint32_t size = ssrc * (uint32_t)ed.sdst;
+  const double* __restrict__ matrix =  // wave-uniform
+      ed.table_off >= 0 ? table + ed.table_off : default_vals + ed.default_off;
   r.live = 0;
 #pragma unroll
   for (int k = 0; k < kPerLane; ++k) {
@@ -645,7 +639,7 @@ __device__ __forceinline__ void item_load(const apc_edge& ed, int lane, const do
     r.live |= (uint32_t)live << k;
     const uint32_t l = live ? r.lk[k] : 0u;
     const uint32_t o = ed.magic ? __umulhi(l, ed.magic) : l / ssrc;
-    r.raw[k] = table[ed.table_off + (int64_t)l];
+    r.raw[k] = matrix[l];
     r.pa[k] = per_arg[ed.comp_base + o];
   }
 }
@@ -671,9 +665,8 @@ __device__ __forceinline__ void item_store(const apc_edge& ed, const ItemLoads& 
   }
 }
 
-// Wave w takes items w, w + W, w + 2W, ... (W = waves in the grid, capped at
-// twice the chip's resident wave slots: measured faster than one wave per item,
-// whose grid has tens of thousands of short-lived waves).
+// Wave w takes items w, w + W, w + 2W, ... (W = waves in the grid, which the
+// launcher caps).
 template <bool kUseTable>
 __global__ void __launch_bounds__(kBlock)
 edge_cost_kernel(apc_problem p, const double* __restrict__ table,
@@ -685,26 +678,24 @@ edge_cost_kernel(apc_problem p, const double* __restrict__ table,
   if (!kUseTable) {
     for (int i = w; i < p.n_item; i += n_waves) {
       const apc_edge item = p.items[i];
-      process_item<false>(p, item, lane, table, per_arg, comm, cost, flags, clamp_inf);
+      process_item(p, item, lane, per_arg, comm, cost, flags, clamp_inf);
     }
     return;
   }
-  // items with a matrix in the table are pipelined: loads of the next such
-  // item are issued before the current one is stored
+  // pipelined: the loads of the next item are issued before the current one is stored
+  const apc_edge* __restrict__ items = p.items;
+  const double* __restrict__ default_vals = p.default_vals;
+  const int n_item = p.n_item;
   bool have = false;
   apc_edge cur;
   ItemLoads cur_r;
   apc_edge nxt;
-  if (w < p.n_item) nxt = p.items[w];
-  for (int i = w; i < p.n_item; i += n_waves) {
+  if (w < n_item) nxt = items[w];
+  for (int i = w; i < n_item; i += n_waves) {
     const apc_edge item = nxt;
-    if (i + n_waves < p.n_item) nxt = p.items[i + n_waves];  // record of the item after this one
-    if (item.table_off < 0) {  // wave-uniform
-      process_item<true>(p, item, lane, table, per_arg, comm, cost, flags, clamp_inf);
-      continue;
-    }
+    if (i + n_waves < n_item) nxt = items[i + n_waves];  // record of the item after this one
     ItemLoads r;
-    item_load(item, lane, table, per_arg, r);
+    item_load(item, lane, table, default_vals, per_arg, r);
     if (have) item_store(cur, cur_r, comm, cost, flags, clamp_inf);
     cur = item;
     cur_r = r;
@@ -1282,7 +1273,10 @@ static int launch_edge_costs(const apc_problem* p, const double* table, const do
   if (p->n_entry == 0) return 0;
   if (!per_arg) return fail(APC_ERR_INVALID, "apc_edge_costs: null per_arg%s");
   unsigned grid = (unsigned)((p->n_item + (kBlock / 64) - 1) / (kBlock / 64));
-  const unsigned cap = 4096;  // 4 waves per block: twice the 8192 resident wave slots
+  // Measured on MI355X: the table kernel (8 waves per SIMD) is fastest with one
+  // wave per item, the direct kernel (4 per SIMD, long-lived waves) with a few
+  // items per wave; the caps only bound the grid of very large problems.
+  const unsigned cap = table ? (1u << 22) : (1u << 14);
   if (grid > cap) grid = cap;
   if (table)
     hipExtLaunchKernelGGL(edge_cost_kernel<true>, dim3(grid), dim3(kBlock), 0, stream, start, stop, 0,

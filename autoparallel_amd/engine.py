@@ -198,8 +198,15 @@ class CostEngine:
         self.flags = torch.zeros(E, dtype=torch.uint8, device=self.device)
         self.status = torch.zeros(1, dtype=torch.int32, device=self.device)
         tsize = int(self.lib.apc_pair_table_size(C.byref(p)))
+        # the table path carries the transition flag in the sign bit of a cost and
+        # reads default rows the same way: a default value with its sign bit set
+        # (nothing the reference produces) is only exact on the direct path
+        signed_defaults = bool(np.signbit(g.default_vals).any())
         if use_table is None:
-            use_table = tsize <= _TABLE_MAX_DOUBLES and tsize <= max(_TABLE_MAX_RATIO * g.num_entries, 1 << 16)
+            use_table = (not signed_defaults and tsize <= _TABLE_MAX_DOUBLES
+                         and tsize <= max(_TABLE_MAX_RATIO * g.num_entries, 1 << 16))
+        elif use_table and signed_defaults:
+            raise ValueError("use_table=True needs default values with a clear sign bit")
         self.use_table = bool(use_table)
         self.table = (
             torch.empty(tsize, dtype=torch.float64, device=self.device) if self.use_table else None

@@ -312,12 +312,15 @@ class PackedGraph:
         """Layout of the block table: one S_dst x S_src cost matrix per distinct
         (producer run, consumer run) pair among the edges that have a producer
         and no missing spec on either side (runs are identified by their offset
-        in ``lists``: identical runs are stored once).  Every matrix is padded to
-        a multiple of 256 elements so that a 256-thread block of the table
-        kernel works on one matrix.
+        in ``lists``: identical runs are stored once), and a matrix of its own
+        for every edge with a producer and a missing spec.  Every matrix is
+        padded to a multiple of 256 elements so that a 256-thread block of the
+        table kernel works on one matrix.  Edges without a producer need no
+        matrix: their costs are their rows of ``default_vals``, already in
+        entry order.
         Returns (block_edge int32[B] one edge per matrix, block_off int64[B+1],
         unit_block int32[table_size / 256], edge_table_off int64[NE] (-1 for
-        edges that are evaluated directly))."""
+        edges without a producer and for empty edges))."""
         cached = getattr(self, "_block_table", None)
         if cached is not None:
             return cached
@@ -329,11 +332,13 @@ class PackedGraph:
         dst = self.edge_dst_list.astype(np.int64)
         ssrc, sdst = self.edge_ssrc.astype(np.int64), self.edge_sdst.astype(np.int64)
         has_none = (none_before[src + ssrc] - none_before[src] > 0) | (none_before[dst + sdst] - none_before[dst] > 0)
-        ok = np.nonzero(hp & ~has_none & (ssrc * sdst > 0))[0]
+        ok = np.nonzero(hp & (ssrc * sdst > 0))[0]
         if ok.shape[0] == 0:
             out = (np.zeros(0, np.int32), np.zeros(1, np.int64), np.zeros(0, np.int32), edge_table_off)
         else:
-            key = np.stack([src[ok], dst[ok], ssrc[ok], sdst[ok]], axis=1)
+            # an edge with a missing spec reads its own default rows: its key is its own index
+            own = np.where(has_none[ok], ok, -1)
+            key = np.stack([src[ok], dst[ok], ssrc[ok], sdst[ok], own], axis=1)
             _, first, inv = np.unique(key, axis=0, return_index=True, return_inverse=True)
             inv = inv.reshape(-1)
             block_edge = ok[first].astype(np.int32)

@@ -60,7 +60,9 @@ typedef struct apc_edge {
   int32_t flags;
   int32_t node;
   int32_t src_node;  /* producer node or -1                                   */
-  int64_t table_off; /* first element of the edge's matrix in the block table, or -1 */
+  int64_t table_off; /* first element of the edge's matrix in the block table;
+                        -1 for an edge without a producer (its matrix is its
+                        rows of default_vals)                                   */
   uint32_t magic;    /* floor(2^32 / ssrc) + 1 if ssrc > 1 and ssrc * ssrc * sdst
                         < 2^32 (then local / ssrc == umulhi(local, magic)), else 0 */
   uint32_t local0;   /* 0 in the edge table; in a work item, its first entry  */
@@ -197,11 +199,14 @@ typedef struct apc_problem {
   int64_t n_default;
   const double* default_vals;
   /* block table: one S_dst x S_src matrix per distinct (producer run, consumer
-   * run) pair among the edges that have a producer and no missing spec, in the
-   * edge block's [out_idx][inp_idx] order: table[block_off[b] + out_idx * S_src
-   * + inp_idx] = comm cost, with the sign bit set when the two placements
-   * differ.  Each matrix is padded to a multiple of 256 elements;
-   * apc_edge.table_off is the matrix of the edge (-1: evaluate directly). */
+   * run) pair among the edges that have a producer and no missing spec, and one
+   * of its own for each edge with a producer and a missing spec, in the edge
+   * block's [out_idx][inp_idx] order: table[block_off[b] + out_idx * S_src +
+   * inp_idx] = comm cost, with the sign bit set when the two placements differ.
+   * Each matrix is padded to a multiple of 256 elements; apc_edge.table_off is
+   * the matrix of the edge.  A caller that passes a table to apc_edge_costs
+   * gives every edge with a producer a matrix, and keeps every default value's
+   * sign bit clear (the table path reads default rows with the same decoding). */
   int32_t n_block;
   const int32_t* block_edge;       /* [n_block] an edge that owns matrix b          */
   const int64_t* block_off;        /* [n_block+1], multiples of 256                  */
@@ -280,8 +285,8 @@ int apc_node_compute_costs(const apc_problem* p, double* compute, double* per_ar
  *     cost  = comm + per_arg + transition
  * and, if clamp_inf != 0, add_inf_cost_constraint's rewrite of non-finite cost
  * to 10000.0 (:803-812).  table may be NULL: every entry is then evaluated
- * directly (same arithmetic, no table memory).  comm / cost / flags may each
- * be NULL to skip that output. */
+ * directly (same arithmetic, no table memory, any default values).  comm /
+ * cost / flags may each be NULL to skip that output. */
 int apc_edge_costs(const apc_problem* p, const double* table, const double* per_arg,
                    double* comm, double* cost, uint8_t* flags, int32_t clamp_inf, void* stream);
 
