@@ -127,6 +127,9 @@ class ApcProblem(C.Structure):
         ("table_size", C.c_int64),
         ("n_table_unit", C.c_int32),
         ("table_unit_block", C.c_void_p),
+        ("list_uidx", C.c_void_p),
+        ("list_ufirst", C.c_void_p),
+        ("block_udst", C.c_void_p),
     ]
 
 

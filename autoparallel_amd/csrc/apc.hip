@@ -261,6 +261,7 @@ __device__ __forceinline__ double roofline(const apc_problem& p, int64_t flops, 
 }
 
 constexpr int kNodesPerBlock = 4;  // one wavefront each
+constexpr int kFusedTableBlocks = 2048;  // larger tables are built by a launch of their own
 constexpr int kProgCache = 128;    // int64 words of program staged per wave
 
 // One wavefront per 64 strategies of an evaluated node.  Phase 1: the lanes split the node's
@@ -467,17 +468,25 @@ __device__ __forceinline__ uint32_t warm_problem(const apc_problem& p, int lane,
 // with its sign bit set when the two placements differ (costs are never
 // negative, so the sign is free to carry the transition flag): the entry kernel
 // reads comm and transition with one coalesced load and no spec words.
+template <bool kWarm>
 __device__ __forceinline__ void pair_table_block(const apc_problem& p, double* __restrict__ table,
                                                  int unit) {
-  const uint32_t keep = warm_problem(p, threadIdx.x, blockDim.x);
+  const uint32_t keep = kWarm ? warm_problem(p, threadIdx.x, blockDim.x) : 0u;
   const int b = p.table_unit_block[unit];
   const int64_t base = p.block_off[b];
   const apc_edge ed = p.edges[p.block_edge[b]];  // any edge with this matrix
-  const uint32_t ssrc = (uint32_t)ed.ssrc;
+  // a compressed matrix has one column / row per distinct word of the two runs
+  const bool squeezed = (ed.flags & APC_EDGE_COMPRESSED) != 0;
+  const uint32_t ncol = squeezed ? (uint32_t)ed.flags >> APC_EDGE_USRC_SHIFT : (uint32_t)ed.ssrc;
+  const uint32_t nrow = squeezed ? (uint32_t)p.block_udst[b] : (uint32_t)ed.sdst;
   const int64_t l64 = (int64_t)unit * 256 - base + threadIdx.x;
-  if (l64 < (int64_t)ssrc * ed.sdst) {
+  if (l64 < (int64_t)ncol * nrow) {
     const uint32_t l = (uint32_t)l64;
-    const uint32_t o = l / ssrc, j = l - o * ssrc;
+    uint32_t o = l / ncol, j = l - o * ncol;
+    if (squeezed) {  // position in its run of an occurrence of that word
+      o = (uint32_t)p.list_ufirst[(size_t)ed.dst_list + o];
+      j = (uint32_t)p.list_ufirst[(size_t)ed.src_list + j];
+    }
     const uint32_t sw = p.lists[(size_t)ed.src_list + j];
     const uint32_t tw = p.lists[(size_t)ed.dst_list + o];
     if (sw != APC_SPEC_NONE && tw != APC_SPEC_NONE) {
@@ -489,7 +498,7 @@ __device__ __forceinline__ void pair_table_block(const apc_problem& p, double* _
                                          nbytes, contig, p.model);
       table[base + l] = (st != tt) ? -c : c;
     } else {  // a missing spec keeps the default row's value and is no transition
-      table[base + l] = p.default_vals[ed.default_off + (int64_t)l];
+      table[base + l] = p.default_vals[ed.default_off + (int64_t)l];  // never squeezed
     }
   }
   asm volatile("" ::"v"(keep));
@@ -506,7 +515,7 @@ prepare_kernel(apc_problem p, double* __restrict__ table, int table_blocks, int 
                int32_t* __restrict__ status) {
   extern __shared__ int64_t s_dyn[];
   if ((int)blockIdx.x < table_blocks) {
-    pair_table_block(p, table, blockIdx.x);
+    pair_table_block<true>(p, table, blockIdx.x);
     return;
   }
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -521,6 +530,15 @@ prepare_kernel(apc_problem p, double* __restrict__ table, int table_blocks, int 
   int64_t* s_prog = s_dyn + (size_t)wave * per_wave;
   node_compute_wave(p, v, (unit - i * chunks) * 64, threadIdx.x & 63, s_prog, s_prog + kProgCache,
                     slow != 0, compute, per_arg, status);
+}
+
+// The block table alone, for tables of many units: no dynamic LDS (which in
+// prepare_kernel limits the blocks per CU to what the node wavefronts need) and
+// no cache warming (thousands of blocks keep the descriptor arrays in L2 by
+// themselves).
+__global__ void __launch_bounds__(256)
+pair_table_kernel(apc_problem p, double* __restrict__ table) {
+  pair_table_block<false>(p, table, blockIdx.x);
 }
 
 // ---------------------------------------------------------------------------
@@ -624,23 +642,42 @@ struct ItemLoads {
   uint32_t live;  // bit k: entry k of this lane exists
 };
 
+template <bool kSqueezed>
 __device__ __forceinline__ void item_load(const apc_edge& ed, int lane, const double* __restrict__ table,
                                           const double* __restrict__ default_vals,
+                                          const int32_t* __restrict__ list_uidx,
                                           const double* __restrict__ per_arg, ItemLoads& r) {
   const uint32_t ssrc = (uint32_t)ed.ssrc;
   const uint32_t size = ssrc * (uint32_t)ed.sdst;
   const double* __restrict__ matrix =  // wave-uniform
       ed.table_off >= 0 ? table + ed.table_off : default_vals + ed.default_off;
   r.live = 0;
+  uint32_t lv[kPerLane], ov[kPerLane];
 #pragma unroll
   for (int k = 0; k < kPerLane; ++k) {
     r.lk[k] = ed.local0 + (uint32_t)(k * 64 + lane);
     const bool live = r.lk[k] < size;
     r.live |= (uint32_t)live << k;
-    const uint32_t l = live ? r.lk[k] : 0u;
-    const uint32_t o = ed.magic ? __umulhi(l, ed.magic) : l / ssrc;
-    r.raw[k] = matrix[l];
-    r.pa[k] = per_arg[ed.comp_base + o];
+    lv[k] = live ? r.lk[k] : 0u;
+    ov[k] = ed.magic ? __umulhi(lv[k], ed.magic) : lv[k] / ssrc;
+    r.pa[k] = per_arg[ed.comp_base + ov[k]];
+  }
+  if (kSqueezed && (ed.flags & APC_EDGE_COMPRESSED)) {  // wave-uniform
+    // the matrix has one row / column per distinct spec word of the two runs:
+    // two index loads, then a gather inside the (cache-resident) matrix
+    const uint32_t usrc = (uint32_t)ed.flags >> APC_EDGE_USRC_SHIFT;
+    uint32_t at[kPerLane];
+#pragma unroll
+    for (int k = 0; k < kPerLane; ++k) {
+      const uint32_t uo = (uint32_t)list_uidx[(size_t)ed.dst_list + ov[k]];
+      const uint32_t uj = (uint32_t)list_uidx[(size_t)ed.src_list + (lv[k] - ov[k] * ssrc)];
+      at[k] = uo * usrc + uj;
+    }
+#pragma unroll
+    for (int k = 0; k < kPerLane; ++k) r.raw[k] = matrix[at[k]];
+  } else {
+#pragma unroll
+    for (int k = 0; k < kPerLane; ++k) r.raw[k] = matrix[lv[k]];
   }
 }
 
@@ -667,7 +704,8 @@ __device__ __forceinline__ void item_store(const apc_edge& ed, const ItemLoads& 
 
 // Wave w takes items w, w + W, w + 2W, ... (W = waves in the grid, which the
 // launcher caps).
-template <bool kUseTable>
+// kMode 0: direct evaluation; 1: block table; 2: block table with compressed matrices
+template <int kMode>
 __global__ void __launch_bounds__(kBlock)
 edge_cost_kernel(apc_problem p, const double* __restrict__ table,
                  const double* __restrict__ per_arg, double* __restrict__ comm,
@@ -675,7 +713,7 @@ edge_cost_kernel(apc_problem p, const double* __restrict__ table,
   const int n_waves = gridDim.x * (kBlock / 64);
   const int w = __builtin_amdgcn_readfirstlane((int)(blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6)));
   const int lane = threadIdx.x & 63;
-  if (!kUseTable) {
+  if (kMode == 0) {
     for (int i = w; i < p.n_item; i += n_waves) {
       const apc_edge item = p.items[i];
       process_item(p, item, lane, per_arg, comm, cost, flags, clamp_inf);
@@ -685,6 +723,7 @@ edge_cost_kernel(apc_problem p, const double* __restrict__ table,
   // pipelined: the loads of the next item are issued before the current one is stored
   const apc_edge* __restrict__ items = p.items;
   const double* __restrict__ default_vals = p.default_vals;
+  const int32_t* __restrict__ list_uidx = p.list_uidx;
   const int n_item = p.n_item;
   bool have = false;
   apc_edge cur;
@@ -695,7 +734,7 @@ edge_cost_kernel(apc_problem p, const double* __restrict__ table,
     const apc_edge item = nxt;
     if (i + n_waves < n_item) nxt = items[i + n_waves];  // record of the item after this one
     ItemLoads r;
-    item_load(item, lane, table, default_vals, per_arg, r);
+    item_load<kMode == 2>(item, lane, table, default_vals, list_uidx, per_arg, r);
     if (have) item_store(cur, cur_r, comm, cost, flags, clamp_inf);
     cur = item;
     cur_r = r;
@@ -1137,6 +1176,9 @@ int validate_problem(const apc_problem* p) {
       p->n_table_unit != p->table_size / 256 ||
       (p->table_size > 0 && (!p->block_edge || !p->block_off || !p->table_unit_block)))
     return fail(APC_ERR_INVALID, "bad block table description%s");
+  if ((p->list_uidx != nullptr) != (p->list_ufirst != nullptr) ||
+      (p->list_uidx != nullptr) != (p->block_udst != nullptr))
+    return fail(APC_ERR_INVALID, "compressed block table: list_uidx, list_ufirst and block_udst go together%s");
   if (p->max_rank < 0 || p->max_rank > APC_MAX_RANK || p->max_node_args < 0)
     return fail(APC_ERR_INVALID, "max_rank / max_node_args out of range%s");
   return 0;
@@ -1159,7 +1201,12 @@ int slot_grid(const apc_problem* p, int per_block, unsigned* grid) {
 
 int launch_prepare(const apc_problem* p, double* table, bool do_nodes, double* compute,
                    double* per_arg, int32_t* status, hipStream_t stream) {
-  const int table_blocks = (table && p->table_size > 0) ? p->n_table_unit : 0;
+  int table_blocks = (table && p->table_size > 0) ? p->n_table_unit : 0;
+  if (table_blocks > kFusedTableBlocks) {  // a launch of its own: see pair_table_kernel
+    hipLaunchKernelGGL(pair_table_kernel, dim3(table_blocks), dim3(256), 0, stream, *p, table);
+    if (int rc = check_launch("pair_table_kernel")) return rc;
+    table_blocks = 0;
+  }
   const int64_t chunks = (p->max_nstrat + 63) >> 6;
   const int64_t units = (int64_t)p->n_comp_node * chunks;  // one wavefront per 64 strategies of a node
   if (do_nodes && (chunks < 1 || units > (1ll << 30)))
@@ -1278,11 +1325,14 @@ static int launch_edge_costs(const apc_problem* p, const double* table, const do
   // items per wave; the caps only bound the grid of very large problems.
   const unsigned cap = table ? (1u << 22) : (1u << 14);
   if (grid > cap) grid = cap;
-  if (table)
-    hipExtLaunchKernelGGL(edge_cost_kernel<true>, dim3(grid), dim3(kBlock), 0, stream, start, stop, 0,
+  if (table && p->list_uidx)
+    hipExtLaunchKernelGGL(edge_cost_kernel<2>, dim3(grid), dim3(kBlock), 0, stream, start, stop, 0,
+                          *p, table, per_arg, comm, cost, flags, clamp_inf);
+  else if (table)
+    hipExtLaunchKernelGGL(edge_cost_kernel<1>, dim3(grid), dim3(kBlock), 0, stream, start, stop, 0,
                           *p, table, per_arg, comm, cost, flags, clamp_inf);
   else
-    hipExtLaunchKernelGGL(edge_cost_kernel<false>, dim3(grid), dim3(kBlock), 0, stream, start, stop, 0,
+    hipExtLaunchKernelGGL(edge_cost_kernel<0>, dim3(grid), dim3(kBlock), 0, stream, start, stop, 0,
                           *p, table, per_arg, comm, cost, flags, clamp_inf);
   return check_launch("edge_cost_kernel");
 }

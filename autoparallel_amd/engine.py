@@ -106,7 +106,13 @@ class CostEngine:
         use_table: Optional[bool] = None,
         order_mode: int = 0,
         nccl_config=None,
+        table_mode: Optional[str] = None,
     ):
+        """``table_mode``: "full" (one S_dst x S_src matrix per distinct pair of
+        runs), "compressed" (matrices by distinct spec word, read by gather),
+        "direct" (no table: every entry evaluated), or None: the first of the
+        three whose table is small against the entry count.  ``use_table`` is
+        the older switch: True = "full", False = "direct"."""
         self.lib = _lib.load()
         self.g = g
         self.device = torch.device(device)
@@ -168,19 +174,48 @@ class CostEngine:
         p.explicit_flops = up("explicit_flops", g.explicit_flops) if g.explicit_flops is not None else None
         p.explicit_bytes = up("explicit_bytes", g.explicit_bytes) if g.explicit_bytes is not None else None
         p.n_edge = g.num_edges
-        p.edges = up("edges", g.edge_records())
         p.n_entry = g.num_entries
         p.n_slot = g.num_slots
         chunk_edge = g.chunk_edge_index()
         p.n_chunk = chunk_edge.shape[0]
         assert p.n_chunk == g.num_slots >> CHUNK_SHIFT
         p.chunk_edge = up("chunk_edge", chunk_edge)
-        items = g.work_items()
+        # the table path carries the transition flag in the sign bit of a cost and
+        # reads default rows the same way: a default value with its sign bit set
+        # (nothing the reference produces) is only exact on the direct path
+        signed_defaults = bool(np.signbit(g.default_vals).any())
+        if table_mode is None and use_table is not None:
+            table_mode = "full" if use_table else "direct"
+        if table_mode is None:
+            def small(t):
+                return t <= _TABLE_MAX_DOUBLES and t <= max(_TABLE_MAX_RATIO * g.num_entries, 1 << 16)
+
+            if signed_defaults:
+                table_mode = "direct"
+            elif small(int(g.block_table(False)[1][-1])):
+                table_mode = "full"
+            elif g.run_unique_index() is not None and small(int(g.block_table(True)[1][-1])):
+                table_mode = "compressed"
+            else:
+                table_mode = "direct"
+        if table_mode not in ("direct", "full", "compressed"):
+            raise ValueError(f"unknown table_mode {table_mode!r}")
+        if table_mode != "direct" and signed_defaults:
+            raise ValueError("a block table needs default values with a clear sign bit")
+        self.table_mode = table_mode
+        squeezed = table_mode == "compressed"
+        p.edges = up("edges", g.edge_records(squeezed))
+        items = g.work_items(squeezed)
         p.n_item = items.shape[0]
         p.items = up("items", items)
         p.n_default = g.default_vals.shape[0]
         p.default_vals = up("default_vals", g.default_vals)
-        block_edge, block_off, unit_block, _ = g.block_table()
+        block_edge, block_off, unit_block, _, _, block_udst = g.block_table(squeezed)
+        if squeezed:
+            uidx, ufirst, _ = g.run_unique_index()
+            p.list_uidx = up("list_uidx", uidx)
+            p.list_ufirst = up("list_ufirst", ufirst)
+            p.block_udst = up("block_udst", block_udst)
         p.n_block = block_edge.shape[0]
         p.block_edge = up("block_edge", block_edge)
         p.block_off = up("block_off", block_off)
@@ -198,16 +233,7 @@ class CostEngine:
         self.flags = torch.zeros(E, dtype=torch.uint8, device=self.device)
         self.status = torch.zeros(1, dtype=torch.int32, device=self.device)
         tsize = int(self.lib.apc_pair_table_size(C.byref(p)))
-        # the table path carries the transition flag in the sign bit of a cost and
-        # reads default rows the same way: a default value with its sign bit set
-        # (nothing the reference produces) is only exact on the direct path
-        signed_defaults = bool(np.signbit(g.default_vals).any())
-        if use_table is None:
-            use_table = (not signed_defaults and tsize <= _TABLE_MAX_DOUBLES
-                         and tsize <= max(_TABLE_MAX_RATIO * g.num_entries, 1 << 16))
-        elif use_table and signed_defaults:
-            raise ValueError("use_table=True needs default values with a clear sign bit")
-        self.use_table = bool(use_table)
+        self.use_table = table_mode != "direct"
         self.table = (
             torch.empty(tsize, dtype=torch.float64, device=self.device) if self.use_table else None
         )

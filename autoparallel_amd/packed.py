@@ -111,6 +111,10 @@ EDGE_HAS_PRODUCER = 1  # comm is computed from specs (else default row kept)
 EDGE_SCORE_TRANSITION = 2  # producer output is a single spec: the plan scorer
 #                            counts a transition (optimize_sharding.py:1097-1104)
 EDGE_PREFETCHABLE = 4  # set in the device records from ``edge_prefetchable``
+EDGE_COMPRESSED = 8  # device records only: the edge's matrix in the block table has one
+#                      row / column per distinct spec word; its row length is in
+#                      flags >> EDGE_USRC_SHIFT
+EDGE_USRC_SHIFT = 8
 
 # ---- compute programs ------------------------------------------------------
 # A node's compute estimate needs flops and bytes of the op run on the sharded
@@ -275,12 +279,15 @@ class PackedGraph:
         ]
     )
 
-    def edge_records(self) -> np.ndarray:
-        """Edges as 64-byte records (the ``apc_edge`` struct of include/apc.h)."""
+    def edge_records(self, compressed: bool = False) -> np.ndarray:
+        """Edges as 64-byte records (the ``apc_edge`` struct of include/apc.h).
+        ``compressed``: records for the compressed block table (``table_off``
+        of that layout; EDGE_COMPRESSED and the matrix's row length in
+        ``flags`` for the edges whose matrix is stored by distinct spec word)."""
         NE = self.num_edges
         rec = np.zeros(NE, self.EDGE_DTYPE)
         assert rec.dtype.itemsize == 64
-        rec["table_off"] = self.block_table()[3]
+        rec["table_off"] = self.block_table(compressed)[3]
         # division by ssrc as a multiply-high (exact while local * ssrc < 2**32)
         ssrc = self.edge_ssrc.astype(np.int64)
         ok = (ssrc > 1) & (ssrc * ssrc * self.edge_sdst < 2**32)
@@ -295,6 +302,9 @@ class PackedGraph:
         flags = self.edge_flags.astype(np.int32).copy()
         if self.edge_prefetchable is not None:
             flags |= (self.edge_prefetchable.astype(np.int32) != 0) * EDGE_PREFETCHABLE
+        if compressed:
+            usrc = self.block_table(True)[4]
+            flags |= np.where(usrc > 0, EDGE_COMPRESSED | (usrc << EDGE_USRC_SHIFT), 0).astype(np.int32)
         rec["flags"] = flags
         rec["node"] = self.edge_node
         rec["src_node"] = self.edge_src_node
@@ -308,7 +318,51 @@ class PackedGraph:
     def max_rank(self) -> int:
         return int(self.meta_rank.max()) if self.meta_rank.shape[0] else 0
 
-    def block_table(self):
+    def run_unique_index(self):
+        """Distinct spec words of every run an edge names (producer runs and
+        consumer runs).  Returns (uidx int32[L], ufirst int32[L], nuniq
+        int32[L]): ``uidx[p]`` is the rank of ``lists[p]`` among the distinct
+        words of its run, ``ufirst[run + k]`` the position inside the run of an
+        occurrence of the run's k-th distinct word, ``nuniq[run]`` their number
+        (at the run's first position).  None if two runs of different extent
+        overlap: a position then has no single rank."""
+        cached = getattr(self, "_run_unique", False)
+        if cached is not False:
+            return cached
+        L = self.lists.shape[0]
+        hp = (self.edge_flags & EDGE_HAS_PRODUCER) != 0
+        runs = np.concatenate([
+            np.stack([self.edge_src_list[hp].astype(np.int64), self.edge_ssrc[hp].astype(np.int64)], 1),
+            np.stack([self.edge_dst_list.astype(np.int64), self.edge_sdst.astype(np.int64)], 1)])
+        runs = np.unique(runs, axis=0)  # sorted by offset, then length
+        off, ln = runs[:, 0], runs[:, 1]
+        out = None
+        if runs.shape[0] == 0 or (off[:-1] + ln[:-1] <= off[1:]).all():
+            rid = np.repeat(np.arange(runs.shape[0], dtype=np.int64), ln)
+            start = np.concatenate([[0], np.cumsum(ln)[:-1]]) if runs.shape[0] else np.zeros(0, np.int64)
+            pos = off[rid] + (np.arange(int(ln.sum()), dtype=np.int64) - start[rid])
+            words = self.lists[pos].astype(np.int64)
+            order = np.lexsort((pos, words, rid))
+            rs, ws, ps = rid[order], words[order], pos[order]
+            new = np.ones(rs.shape[0], bool)
+            new[1:] = (rs[1:] != rs[:-1]) | (ws[1:] != ws[:-1])
+            gid = np.cumsum(new) - 1
+            run_first = np.zeros(runs.shape[0], np.int64)
+            first_of_run = np.ones(rs.shape[0], bool)
+            first_of_run[1:] = rs[1:] != rs[:-1]
+            run_first[rs[first_of_run]] = gid[first_of_run]
+            rank = gid - run_first[rs]
+            uidx = np.zeros(L, np.int32)
+            uidx[ps] = rank
+            ufirst = np.zeros(L, np.int32)
+            ufirst[off[rs[new]] + rank[new]] = ps[new] - off[rs[new]]
+            nuniq = np.zeros(L, np.int32)
+            np.maximum.at(nuniq, off[rs], (rank + 1).astype(np.int32))
+            out = (uidx, ufirst, nuniq)
+        object.__setattr__(self, "_run_unique", out)
+        return out
+
+    def block_table(self, compressed: bool = False):
         """Layout of the block table: one S_dst x S_src cost matrix per distinct
         (producer run, consumer run) pair among the edges that have a producer
         and no missing spec on either side (runs are identified by their offset
@@ -318,23 +372,44 @@ class PackedGraph:
         table kernel works on one matrix.  Edges without a producer need no
         matrix: their costs are their rows of ``default_vals``, already in
         entry order.
+
+        ``compressed``: the matrices of the first kind keep one row per distinct
+        consumer spec word and one column per distinct producer spec word of
+        their runs (``run_unique_index``); strategies that differ elsewhere
+        (other arguments, other outputs) repeat spec words, and the cost depends
+        on the two words only.
+
         Returns (block_edge int32[B] one edge per matrix, block_off int64[B+1],
         unit_block int32[table_size / 256], edge_table_off int64[NE] (-1 for
-        edges without a producer and for empty edges))."""
-        cached = getattr(self, "_block_table", None)
-        if cached is not None:
-            return cached
+        edges without a producer and for empty edges), edge_usrc int32[NE] row
+        length of the edge's compressed matrix (0: not compressed), block_udst
+        int32[B] rows of every matrix)."""
+        cache = self.__dict__.setdefault("_block_tables", {})
+        if compressed in cache:
+            return cache[compressed]
         NE = self.num_edges
         edge_table_off = np.full(NE, -1, np.int64)
+        edge_usrc = np.zeros(NE, np.int32)
         none_before = np.concatenate([[0], np.cumsum(self.lists == SPEC_NONE)])
         hp = (self.edge_flags & EDGE_HAS_PRODUCER) != 0
         src = np.where(hp, self.edge_src_list, 0).astype(np.int64)
         dst = self.edge_dst_list.astype(np.int64)
         ssrc, sdst = self.edge_ssrc.astype(np.int64), self.edge_sdst.astype(np.int64)
         has_none = (none_before[src + ssrc] - none_before[src] > 0) | (none_before[dst + sdst] - none_before[dst] > 0)
+        cols, rows = ssrc.copy(), sdst.copy()
+        if compressed:
+            ru = self.run_unique_index()
+            if ru is None:
+                raise ValueError("runs of spec words overlap: no compressed block table for this graph")
+            squeeze = hp & ~has_none
+            cols[squeeze] = ru[2][src[squeeze]]
+            rows[squeeze] = ru[2][dst[squeeze]]
+            edge_usrc[squeeze] = cols[squeeze]
+            assert (cols < (1 << (31 - EDGE_USRC_SHIFT))).all()
         ok = np.nonzero(hp & (ssrc * sdst > 0))[0]
         if ok.shape[0] == 0:
-            out = (np.zeros(0, np.int32), np.zeros(1, np.int64), np.zeros(0, np.int32), edge_table_off)
+            out = (np.zeros(0, np.int32), np.zeros(1, np.int64), np.zeros(0, np.int32), edge_table_off,
+                   edge_usrc, np.zeros(0, np.int32))
         else:
             # an edge with a missing spec reads its own default rows: its key is its own index
             own = np.where(has_none[ok], ok, -1)
@@ -342,13 +417,13 @@ class PackedGraph:
             _, first, inv = np.unique(key, axis=0, return_index=True, return_inverse=True)
             inv = inv.reshape(-1)
             block_edge = ok[first].astype(np.int32)
-            size = ssrc[block_edge] * sdst[block_edge]
+            size = cols[block_edge] * rows[block_edge]
             block_off = np.zeros(block_edge.shape[0] + 1, np.int64)
             np.cumsum((size + 255) & ~255, out=block_off[1:])
             edge_table_off[ok] = block_off[:-1][inv]
             unit_block = np.repeat(np.arange(block_edge.shape[0], dtype=np.int32), np.diff(block_off) // 256)
-            out = (block_edge, block_off, unit_block, edge_table_off)
-        object.__setattr__(self, "_block_table", out)
+            out = (block_edge, block_off, unit_block, edge_table_off, edge_usrc, rows[block_edge].astype(np.int32))
+        cache[compressed] = out
         return out
 
     def chunk_edge_index(self) -> np.ndarray:
@@ -358,7 +433,7 @@ class PackedGraph:
         starts = np.arange(nt, dtype=np.int64) << CHUNK_SHIFT
         return (np.searchsorted(self.edge_off, starts, side="right") - 1).astype(np.int32)
 
-    def work_items(self) -> np.ndarray:
+    def work_items(self, compressed: bool = False) -> np.ndarray:
         """Work items of the entry kernel: for every 256 entries of every edge
         block a copy of the edge record with ``local0`` set, in slot order."""
         sizes = self.edge_sdst.astype(np.int64) * self.edge_ssrc
@@ -366,7 +441,7 @@ class PackedGraph:
         eid = np.repeat(np.arange(self.num_edges, dtype=np.int64), n)
         start = np.concatenate([[0], np.cumsum(n)[:-1]])
         k = np.arange(int(n.sum()), dtype=np.int64) - start[eid]
-        items = self.edge_records()[eid]
+        items = self.edge_records(compressed)[eid]
         items["local0"] = k * ITEM_ENTRIES
         return items
 

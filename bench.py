@@ -60,6 +60,8 @@ def main():
     ap.add_argument("--score-assignments", type=int, default=1 << 20,
                     help="also score this many on-device generated assignments (0 = skip)")
     ap.add_argument("--direct", action="store_true", help="evaluate every entry directly (no block table)")
+    ap.add_argument("--table-mode", choices=["full", "compressed", "direct"], default=None,
+                    help="force the block-table layout (default: chosen from the table sizes)")
     ap.add_argument("--calibration-copy-mib", type=int, default=0,
                     help="after the timed steps, also launch the plain copy kernel on this many MiB "
                          "(the known-traffic reference for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)")
@@ -80,7 +82,7 @@ def main():
     E = g.num_entries
 
     t0 = time.perf_counter()
-    eng = CostEngine(g, use_table=False if args.direct else None)
+    eng = CostEngine(g, table_mode="direct" if args.direct else args.table_mode)
     torch.cuda.synchronize()
     t_upload = time.perf_counter() - t0
 
@@ -164,6 +166,7 @@ def main():
             "tensor_metas": int(g.meta_rank.shape[0]),
             "placement_tuples": int(g.tuple_plc.shape[0]),
             "block_table": bool(eng.use_table),
+            "table_mode": eng.table_mode,
             "block_table_doubles": int(eng.table.numel()) if eng.table is not None else 0,
             "compute_slots": g.num_compute,
             "evaluated_nodes": int(g.comp_nodes.shape[0]),

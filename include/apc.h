@@ -31,6 +31,10 @@ extern "C" {
 #define APC_EDGE_HAS_PRODUCER 1
 #define APC_EDGE_SCORE_TRANSITION 2
 #define APC_EDGE_PREFETCHABLE 4
+/* the edge's matrix in the block table is stored by distinct spec word (see
+ * apc_problem.list_uidx); its row length is flags >> APC_EDGE_USRC_SHIFT */
+#define APC_EDGE_COMPRESSED 8
+#define APC_EDGE_USRC_SHIFT 8
 
 /* node op classes */
 #define APC_OP_ZERO 0
@@ -213,6 +217,17 @@ typedef struct apc_problem {
   int64_t table_size;              /* doubles: block_off[n_block]                    */
   int32_t n_table_unit;            /* table_size / 256                               */
   const int32_t* table_unit_block; /* [n_table_unit] matrix owning elements [256 u, 256 u + 256) */
+  /* compressed block table (all three NULL otherwise).  Strategies of a node
+   * that differ in other arguments or outputs repeat spec words, and a cost
+   * depends on the two words only (the key of the reference's own memo,
+   * autoparallel/cost_models/collective_runtime_estimation.py:232-246): the
+   * matrix of an edge flagged APC_EDGE_COMPRESSED has one row per distinct
+   * word of the consumer run and one column per distinct word of the producer
+   * run, table[table_off + list_uidx[dst_list + out_idx] * usrc +
+   * list_uidx[src_list + inp_idx]].  Runs are disjoint ranges of lists. */
+  const int32_t* list_uidx;   /* [n_list] rank of the word among its run's distinct words */
+  const int32_t* list_ufirst; /* [n_list] at run + k: position in the run of its k-th distinct word */
+  const int32_t* block_udst;  /* [n_block] rows of matrix b */
 } apc_problem;
 
 int apc_version(void);

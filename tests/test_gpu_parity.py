@@ -29,7 +29,11 @@ def CostEngine():
 
 def _check_build(CE, g, use_table, clamp=False):
     print(f"  build: E={g.num_entries} table={use_table}", flush=True)
-    eng = CE(g, use_table=use_table).build(clamp_inf=clamp)
+    # use_table: True / False, or the name of a table mode
+    kw = dict(table_mode=use_table) if isinstance(use_table, str) else dict(use_table=use_table)
+    eng = CE(g, **kw).build(clamp_inf=clamp)
+    if isinstance(use_table, str):
+        assert eng.table_mode == use_table
     got = eng.results()
     ref = O.GraphOracle(g).build()
     want_cost = O.clamp_inf(ref["cost"])[0] if clamp else ref["cost"]
@@ -156,10 +160,13 @@ def _pairs_graph(mesh, shape, n, stride=None, seed=3):
     return graph_from_pairs(mesh, 8, shape, stride, 2, draw(), draw(), dtype=packed.DT_BF16)
 
 
-# every graph through the table path; direct evaluation on the smaller ones
+# every graph through the table path; direct evaluation and the compressed
+# table (matrices by distinct spec word, read by gather) on the smaller ones
 CASES = [(n, True) for n in GRAPHS] + [
     (n, False) for n in ("llama_2d", "gpt2_1d", "llama_odd_mesh", "stress_3d", "pairs_4d", "pairs_3d_noncontig",
                          "moe_tiny")
+] + [
+    (n, "compressed") for n in ("llama_2d", "gpt2_1d", "llama_3d", "stress_3d", "moe_tiny", "pairs_3d_noncontig")
 ]
 
 
@@ -364,7 +371,7 @@ def _edge_case_graph():
     return b.pack()
 
 
-@pytest.mark.parametrize("use_table", [True, False])
+@pytest.mark.parametrize("use_table", [True, False, "compressed"])
 def test_edge_cases(CostEngine, use_table):
     g = _edge_case_graph()
     eng, got, ref = _check_build(CostEngine, g, use_table)

@@ -60,6 +60,50 @@ def test_magic_division_exact(small_llama):
             assert (local * int(r["magic"])) >> 32 == local // int(r["ssrc"])
 
 
+@pytest.mark.parametrize("make", [
+    lambda: graphgen.llama_graph((2, 4), 1, 64, 4, 2, 128, 256, 32, 16),
+    lambda: graphgen.stress_graph(60, (4, 8, 8), seed=2, s_max=40),
+    lambda: graphgen.moe_graph((2, 4), 2, 64, 4, 8, 2, 32, 256, 32, 8),
+])
+def test_compressed_block_table_layout(make):
+    """The compressed block table against its definition: matrix element
+    [uidx[o]][uidx[j]] of an edge stands for the pair (lists[src + j],
+    lists[dst + o]), whatever o and j reach it."""
+    g = make()
+    uidx, ufirst, nuniq = g.run_unique_index()
+    block_edge, block_off, unit_block, table_off, usrc, block_udst = g.block_table(True)
+    full = g.block_table(False)
+    assert block_off[-1] <= full[1][-1] and (block_off % 256 == 0).all()
+    assert unit_block.shape[0] == block_off[-1] // 256
+    hp = (g.edge_flags & packed.EDGE_HAS_PRODUCER) != 0
+    assert ((table_off >= 0) == hp).all()
+    # element -> the word pair it stands for, filled from every entry of every edge
+    cell = {}
+    rec = g.edge_records(True)
+    for e in np.nonzero(hp)[0]:
+        s0, d0, ns, nd = int(g.edge_src_list[e]), int(g.edge_dst_list[e]), int(g.edge_ssrc[e]), int(g.edge_sdst[e])
+        sw, tw = g.lists[s0:s0 + ns], g.lists[d0:d0 + nd]
+        if usrc[e] == 0:  # not compressed: a missing spec somewhere
+            assert (sw == packed.SPEC_NONE).any() or (tw == packed.SPEC_NONE).any()
+            assert not rec["flags"][e] & packed.EDGE_COMPRESSED
+            continue
+        assert rec["flags"][e] & packed.EDGE_COMPRESSED and rec["flags"][e] >> packed.EDGE_USRC_SHIFT == usrc[e]
+        assert usrc[e] == np.unique(sw).shape[0] == nuniq[s0]
+        assert nuniq[d0] == np.unique(tw).shape[0]
+        at = table_off[e] + uidx[d0:d0 + nd].astype(np.int64)[:, None] * usrc[e] + uidx[s0:s0 + ns][None, :]
+        assert at.max() < table_off[e] + int(usrc[e]) * nuniq[d0]
+        pair = (sw.astype(np.int64)[None, :] << 32) | tw.astype(np.int64)[:, None]
+        for a, w in zip(at.ravel().tolist(), pair.ravel().tolist()):
+            assert cell.setdefault(a, w) == w
+        # and the table kernel's way back: element -> a position holding that word
+        k = np.arange(usrc[e])
+        assert (uidx[s0 + ufirst[s0 + k]] == k).all()
+    for b, e in enumerate(block_edge):
+        if usrc[e]:
+            assert block_udst[b] == nuniq[int(g.edge_dst_list[e])]
+            assert block_off[b + 1] - block_off[b] >= int(usrc[e]) * int(block_udst[b])
+
+
 def test_shared_compute_slots_are_consistent(small_llama):
     """Nodes that share a compute slot must produce identical estimates: the
     oracle prices every node on its own and writes into the shared slot."""
