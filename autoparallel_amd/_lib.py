@@ -133,6 +133,28 @@ class ApcProblem(C.Structure):
     ]
 
 
+class ApcSchedule(C.Structure):
+    """apc_schedule of include/apc.h."""
+
+    _fields_ = [
+        ("n_node", C.c_int32),
+        ("n_stream", C.c_int32),
+        ("dur", C.c_void_p),
+        ("stream", C.c_void_p),
+        ("flags", C.c_void_p),
+        ("wait_src", C.c_void_p),
+        ("n_storage", C.c_int32),
+        ("st_bytes", C.c_void_p),
+        ("st_freeable", C.c_void_p),
+        ("st_users", C.c_void_p),
+        ("alloc_off", C.c_void_p),
+        ("alloc_st", C.c_void_p),
+        ("use_off", C.c_void_p),
+        ("use_st", C.c_void_p),
+        ("initial_bytes", C.c_int64),
+    ]
+
+
 _SIGNATURES = {
     "apc_version": (C.c_int, []),
     "apc_last_error": (C.c_char_p, []),
@@ -201,6 +223,10 @@ _SIGNATURES = {
         C.c_int,
         [C.POINTER(ApcModel), C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
          C.c_void_p, C.c_void_p]),
+    "apc_schedule_metrics": (
+        C.c_int,
+        [C.POINTER(ApcSchedule), C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+         C.c_void_p]),
 }
 
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)

@@ -59,6 +59,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--score-assignments", type=int, default=1 << 20,
                     help="also score this many on-device generated assignments (0 = skip)")
+    ap.add_argument("--schedules", type=int, default=16384,
+                    help="also price this many candidate orders of a lowered 32-layer schedule (0 = skip)")
     ap.add_argument("--direct", action="store_true", help="evaluate every entry directly (no block table)")
     ap.add_argument("--table-mode", choices=["full", "compressed", "direct"], default=None,
                     help="force the block-table layout (default: chosen from the table sizes)")
@@ -206,6 +208,33 @@ def main():
             "algorithmic_bytes_per_assignment": 8 * g.num_nodes + 17 * g.num_edges,
             "feasible_fraction": float((scores[:, 5] == 0).double().mean().item()),
         }
+
+    if args.schedules > 0:
+        # next row of the path: the lowered-graph estimator as a batch scorer of
+        # candidate orders (secondary figure)
+        from autoparallel_amd import schedule_metrics as SM
+
+        ps = SM.synthetic_schedule(32, seed=0)
+        base = ps.random_orders(256, seed=1)
+        orders = np.tile(base, ((args.schedules + 255) // 256, 1))[:args.schedules]
+        est = SM.ScheduleEstimator(ps)
+        est.evaluate(orders[:256])
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        times, peak = est.evaluate(orders)
+        t_sched = time.perf_counter() - t0
+        out["schedule_estimator"] = {
+            "nodes": ps.n_node, "orders": int(orders.shape[0]), "seconds_including_upload_and_readback": t_sched,
+            "orders_per_s": orders.shape[0] / t_sched,
+            "best_total_time_us": float(times[:, 0].min()), "graph_order_total_time_us": float(times[0, 0]),
+        }
+        if not args.no_cpu_baseline:
+            from oracle import schedule_oracle as SO
+
+            t0 = time.perf_counter()
+            for o in base[:64]:
+                SO.schedule_metrics(ps, o)
+            out["schedule_estimator"]["cpu_port_orders_per_s"] = 64 / (time.perf_counter() - t0)
 
     if not args.no_cpu_baseline:
         from oracle import cost_oracle as O

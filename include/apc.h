@@ -431,6 +431,57 @@ int apc_enumerate_input_options(const apc_model* model, int32_t n, const int32_t
                                 const int64_t* shape, const int64_t* cand_off, uint8_t* valid,
                                 uint8_t* plc, void* stream);
 
+/* ---------------------------------------------------------------------------
+ * Schedule estimator: timeline and peak memory of a lowered graph (collectives
+ * as nodes) under many candidate orders.
+ * ------------------------------------------------------------------------- */
+#define APC_SCHED_MAX_STREAMS 8
+/* node flags */
+#define APC_SCHED_COMM 1    /* a communication node (collective or wait_tensor)      */
+#define APC_SCHED_WAIT 2    /* wait_tensor on the compute stream whose argument is
+                               not a graph input: stalls until wait_src has ended  */
+#define APC_SCHED_SYNC 4    /* blocking collective: the compute stream waits for it */
+#define APC_SCHED_NO_MEM 8  /* placeholder / get_attr / output: allocates and frees
+                               nothing when scheduled                               */
+
+typedef struct apc_schedule {
+  int32_t n_node;
+  int32_t n_stream;        /* streams in use, <= APC_SCHED_MAX_STREAMS; 0 = compute   */
+  const double* dur;       /* [n_node] runtime estimate of the node, microseconds    */
+  const int32_t* stream;   /* [n_node] stream the node runs on                        */
+  const uint8_t* flags;    /* [n_node] APC_SCHED_*                                    */
+  const int32_t* wait_src; /* [n_node] for APC_SCHED_WAIT: the collective waited for, or -1 */
+  /* storages (liveness as torch's MemoryTracker keeps it) */
+  int32_t n_storage;
+  const int64_t* st_bytes;    /* [n_storage]                                          */
+  const uint8_t* st_freeable; /* [n_storage] on a tracked device and releasable       */
+  const int32_t* st_users;    /* [n_storage] number of nodes that read the storage    */
+  const int32_t* alloc_off;   /* [n_node+1] into alloc_st: storages the node allocates */
+  const int32_t* alloc_st;
+  const int32_t* use_off;     /* [n_node+1] into use_st: storages the node reads       */
+  const int32_t* use_st;
+  int64_t initial_bytes;      /* live before the first node (graph inputs, attributes) */
+} apc_schedule;
+
+/* Replaces estimate_graph_metrics
+ * (autoparallel/graph_passes/estimate_graph_metrics.py:30-89; the same timeline
+ * as create_execution_trace, graph_passes/debug_helpers.py:336-420) for n_sched
+ * orders of the same nodes at once: order[b * n_node + t] is the node scheduled
+ * t-th in order b (NULL: the graph's own order, n_sched must be 1).  A compute
+ * stream (0) and one stream per communication group advance by dur + 1 us of
+ * launch overhead per node; a wait_tensor stalls the compute stream until its
+ * collective has ended; peak memory follows torch's MemoryTracker
+ * (torch/_inductor/fx_passes/memory_estimator.py: a storage is allocated when
+ * its allocator is scheduled and freed at the last scheduled of its readers).
+ * times[b * 4 ..] = total_time, compute_time, communication_time,
+ * exposed_comm_time; peak[b] = peak_memory.  Scratch, device memory the caller
+ * provides and the call overwrites: end_scratch double[n_sched * n_node],
+ * remaining_scratch int32[n_sched * n_storage].  Every order must be a
+ * permutation that schedules a storage's allocator before its readers. */
+int apc_schedule_metrics(const apc_schedule* s, const int32_t* order, int64_t n_sched,
+                         double* end_scratch, int32_t* remaining_scratch, double* times,
+                         int64_t* peak, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
