@@ -991,6 +991,52 @@ __device__ __forceinline__ double fold_in_order(double acc, double v) {
 // and the terms are folded lane by lane in order, so the sums keep the
 // reference's sequential association (bit-identical to score_kernel) while the
 // gathers of a tile overlap.
+// score_kernel<true> over a window of a larger graph: global node ids for the
+// draw, sums continued from the previous window's.
+__global__ void __launch_bounds__(kBlock)
+score_window_kernel(apc_problem p, const double* __restrict__ per_arg,
+                    const double* __restrict__ comm, const double* __restrict__ cost,
+                    const uint8_t* __restrict__ flags, uint64_t seed, int64_t first,
+                    int64_t n_assign, const int32_t* __restrict__ node_gid, int first_node,
+                    const double* __restrict__ init, double* __restrict__ out) {
+  const int64_t a = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (a >= n_assign) return;
+  double t_compute = 0.0, t_comm = 0.0, t_trans = 0.0, obj = 0.0, forbidden = 0.0;
+  if (init) {
+    const double* r = init + a * 6;
+    t_compute = r[1]; t_comm = r[2]; t_trans = r[3]; obj = r[4]; forbidden = r[5];
+  }
+  for (int v = first_node; v < p.n_node; ++v) {
+    const uint32_t o = mix_assignment(seed, first + a, node_gid[v], p.node_nstrat[v]);
+    const int nargs = p.node_nargs[v];
+    const double pa = per_arg[p.node_comp_off[v] + o];
+    t_compute += pa * (double)(nargs > 1 ? nargs : 1);
+    const double mult = (double)p.node_multiplier[v];
+    for (int e = p.node_edge_off[v]; e < p.node_edge_off[v + 1]; ++e) {
+      const apc_edge ed = p.edges[e];
+      uint32_t j = 0;
+      if (ed.src_node >= 0)
+        j = mix_assignment(seed, first + a, node_gid[ed.src_node], p.node_nstrat[ed.src_node]);
+      const int64_t idx = ed.off + (int64_t)o * ed.ssrc + j;
+      const uint8_t f = flags[idx];
+      obj += cost[idx] * mult;
+      forbidden += (double)((f & APC_ENTRY_NONFINITE) != 0);
+      if (ed.src_node >= 0) {
+        const double c = comm[idx];
+        if (isfinite(c)) t_comm += c;
+        if ((ed.flags & APC_EDGE_SCORE_TRANSITION) && (f & APC_ENTRY_TRANSITION)) t_trans += 1.0;
+      }
+    }
+  }
+  double* r = out + a * 6;
+  r[0] = (t_compute + t_comm) + t_trans;
+  r[1] = t_compute;
+  r[2] = t_comm;
+  r[3] = t_trans;
+  r[4] = obj;
+  r[5] = forbidden;
+}
+
 template <bool kRandom>
 __global__ void __launch_bounds__(kBlock)
 score_wave_kernel(apc_problem p, const double* __restrict__ per_arg,
@@ -1522,6 +1568,27 @@ int apc_score_random_assignments(const apc_problem* p, const double* per_arg, co
     return fail(APC_ERR_INVALID, "apc_score_random_assignments: null argument%s");
   return launch_score(p, per_arg, comm, cost, flags, nullptr, true, seed, first, n_assign, out,
                       (hipStream_t)stream);
+}
+
+int apc_score_random_window(const apc_problem* p, const double* per_arg, const double* comm,
+                            const double* cost, const uint8_t* flags, uint64_t seed,
+                            int64_t first, int64_t n_assign, const int32_t* node_gid,
+                            int32_t first_node, const double* init, double* out, void* stream) {
+  if (int rc = validate_problem(p)) return rc;
+  if (n_assign <= 0) return 0;
+  if (!per_arg || !comm || !cost || !flags || !out || !node_gid || !p->node_multiplier)
+    return fail(APC_ERR_INVALID, "apc_score_random_window: null argument%s");
+  if (first_node < 0 || first_node > p->n_node)
+    return fail(APC_ERR_INVALID, "apc_score_random_window: first_node out of range%s");
+  const int64_t kChunk = 262144;  // as launch_score
+  for (int64_t a0 = 0; a0 < n_assign; a0 += kChunk) {
+    const int64_t n = (n_assign - a0 < kChunk) ? (n_assign - a0) : kChunk;
+    hipLaunchKernelGGL(score_window_kernel, dim3((unsigned)((n + kBlock - 1) / kBlock)), dim3(kBlock),
+                       0, (hipStream_t)stream, *p, per_arg, comm, cost, flags, seed, first + a0, n,
+                       node_gid, first_node, init ? init + a0 * 6 : nullptr, out + a0 * 6);
+    if (int rc = check_launch("score_window_kernel")) return rc;
+  }
+  return 0;
 }
 
 uint32_t apc_random_assignment(uint64_t seed, int64_t a, int32_t node, int32_t nstrat) {

@@ -446,6 +446,26 @@ class CostEngine:
         )
         return out
 
+    def score_random_window(self, seed: int, first: int, count: int, node_gid: np.ndarray, first_node: int,
+                            init: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """score_random for a window of a larger graph (apc_score_random_window):
+        draws by global node id, skips the first ``first_node`` stand-in nodes and
+        continues the sums of ``init`` (the previous window's result)."""
+        assert self.built
+        gid = np.ascontiguousarray(node_gid, np.int32)
+        assert gid.shape == (self.g.num_nodes,) and 0 <= first_node <= self.g.num_nodes
+        assert init is None or (init.shape == (count, 6) and init.dtype == torch.float64 and init.is_contiguous())
+        d_gid = torch.from_numpy(gid).to(self.device)
+        out = torch.empty((count, 6), dtype=torch.float64, device=self.device)
+        _lib.check(
+            self.lib.apc_score_random_window(
+                C.byref(self.problem), self._ptr(self.per_arg), self._ptr(self.comm), self._ptr(self.cost),
+                self._ptr(self.flags), int(seed), int(first), int(count), self._ptr(d_gid), int(first_node),
+                self._ptr(init), self._ptr(out), self._stream()),
+            "apc_score_random_window",
+        )
+        return out
+
     def random_assignment(self, seed: int, a: int) -> np.ndarray:
         """The out_idx per node that score_random draws for assignment a."""
         g = self.g

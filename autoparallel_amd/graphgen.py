@@ -1133,3 +1133,121 @@ def stress_graph(
                             program=opprog.pointwise(ru, isz))
         b.add_node(desc)
     return b.pack()
+
+
+# ---------------------------------------------------------------------------
+# The stress DAG in windows: every node is drawn from its own counter-based
+# generator, so any range of nodes can be produced without the rest.
+# ---------------------------------------------------------------------------
+def _stress_header(seed: int, v: int, nd: int, s_min: int, s_max: int):
+    """(rank, shape, dtype, out placement tuples) of node v, from (seed, v) alone."""
+    rng = np.random.default_rng([seed, v, 0])
+    r = int(rng.integers(1, 5))
+    shape = tuple(int(2 ** rng.uniform(6, 16)) for _ in range(r))
+    dt = DT_BF16 if rng.random() < 0.5 else DT_F32
+    S = int(rng.integers(s_min, s_max + 1))
+    codes = np.asarray([R] + [shard(d) for d in range(r)] + [P])
+    out = [tuple(int(c) for c in row) for row in codes[rng.integers(0, len(codes), size=(S, nd))]]
+    return r, shape, dt, out
+
+
+def stress_dag_window(
+    n_total: int,
+    lo: int,
+    hi: int,
+    mesh_shape: Sequence[int] = (4, 8, 8),
+    seed: int = 0,
+    s_min: int = 4,
+    s_max: int = 512,
+    devices_per_host: int = 8,
+):
+    """Nodes [lo, hi) of the seeded n_total-node stress DAG (ranks 1-4, dims
+    log-uniform in [64, 65536], bf16 / fp32, op class uniform over {matmul,
+    elementwise, reduction, view}, U[s_min, s_max] strategies per node, mean
+    in-degree 1.8 with producers uniform over the earlier nodes), as a packed
+    graph of its own.  Producers below ``lo`` come first as stand-in input nodes
+    with the producer's real output specs, so every edge of the window has its
+    producer run; ``window(0, n_total)`` is the whole DAG.
+    Returns (graph, node_gid int32[N] index of every local node in the whole
+    DAG, n_standin)."""
+    assert 0 <= lo < hi <= n_total
+    nd = len(mesh_shape)
+    headers = {}
+
+    def header(v):
+        if v not in headers:
+            headers[v] = _stress_header(seed, v, nd, s_min, s_max)
+        return headers[v]
+
+    bodies = []
+    external = set()
+    for v in range(lo, hi):
+        rng = np.random.default_rng([seed, v, 1])
+        op = ("matmul", "elementwise", "reduction", "view")[int(rng.integers(0, 4))]
+        if v == 0:
+            want_in = 0
+        elif op == "matmul":
+            want_in = 3 if rng.random() < 0.7 else 2  # with or without a bias
+        elif op == "elementwise":
+            want_in = int(rng.integers(1, 5))
+        else:
+            want_in = 1
+        inputs = [int(rng.integers(0, v)) for _ in range(want_in)]
+        external.update(u for u in inputs if u < lo)
+        bodies.append((v, op, inputs, rng))
+    standins = sorted(external)
+    local = {u: i for i, u in enumerate(standins)}
+    local.update({v: len(standins) + (v - lo) for v in range(lo, hi)})
+
+    b = GraphBuilder(mesh_shape, devices_per_host)
+    b.share_compute_slots = False
+    metas = {}
+
+    def specs_of(v, tuples):
+        if v not in metas:
+            r, shape, dt, _ = header(v)
+            metas[v] = b.meta(shape, contiguous_stride(shape), _ITEMSIZE[dt], dt)
+        return [b.spec(metas[v], t) for t in tuples]
+
+    def add_input(v):
+        out = [[w] for w in specs_of(v, header(v)[3])]
+        b.add_node(NodeDesc(f"in_{v}", in_specs=out, out_specs=out, inputs=[],
+                            default_rows=[[[0.0]] for _ in out]))
+
+    for u in standins:
+        add_input(u)
+    for v, op, inputs, rng in bodies:
+        r, shape, dt, out_tuples = header(v)
+        if not inputs:
+            add_input(v)
+            continue
+        S = len(out_tuples)
+        out_specs = [[w] for w in specs_of(v, out_tuples)]
+        cols = []
+        for u in inputs:
+            ru = header(u)[0]
+            codes = np.asarray([R] + [shard(d) for d in range(ru)] + [P])
+            cols.append(specs_of(u, [tuple(int(c) for c in row)
+                                     for row in codes[rng.integers(0, len(codes), size=(S, nd))]]))
+        in_specs = [[c[o] for c in cols] for o in range(S)]
+        loc = [local[u] for u in inputs]
+        isz = _ITEMSIZE[dt]
+        if op == "view":
+            desc = NodeDesc(f"view_{v}", in_specs=in_specs, out_specs=out_specs, inputs=loc)
+        elif op == "matmul":
+            from .packed import OP_EXPLICIT
+
+            desc = NodeDesc(f"matmul_{v}", in_specs=in_specs, out_specs=out_specs, inputs=loc, op=OP_EXPLICIT,
+                            flops=[int(x) for x in rng.integers(1, 2**44, size=S)],
+                            nbytes=[int(x) for x in rng.integers(1, 2**34, size=S)])
+        elif op == "reduction":
+            ru = header(inputs[0])[0]
+            desc = NodeDesc(f"reduction_{v}", in_specs=in_specs, out_specs=out_specs, inputs=loc, op=OP_PROGRAM,
+                            program=opprog.reduction(ru, [ru - 1], True, isz))
+        else:
+            ru = max(header(u)[0] for u in inputs)
+            desc = NodeDesc(f"elementwise_{v}", in_specs=in_specs, out_specs=out_specs, inputs=loc, op=OP_PROGRAM,
+                            program=opprog.pointwise(ru, isz))
+        b.add_node(desc)
+    gid = np.asarray(standins + list(range(lo, hi)), np.int32)
+    return b.pack(), gid, len(standins)

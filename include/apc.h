@@ -399,6 +399,19 @@ int apc_score_random_assignments(const apc_problem* p, const double* per_arg, co
                                  int64_t first, int64_t n_assign, double* out, void* stream);
 uint32_t apc_random_assignment(uint64_t seed, int64_t a, int32_t node, int32_t nstrat);
 
+/* apc_score_random_assignments for a graph too large to keep its coefficients
+ * resident: the problem holds a window of the graph's nodes (preceded by
+ * first_node stand-ins for producers outside the window, which are not scored),
+ * node_gid[v] is the node's index in the whole graph (the draw uses it, so a
+ * node gets the same out_idx in every window), and the sums continue from
+ * init (the out of the previous window; NULL = start at zero): scoring the
+ * windows in node order forms every sum in the order of one pass over the whole
+ * graph, bit for bit.  One lane per assignment. */
+int apc_score_random_window(const apc_problem* p, const double* per_arg, const double* comm,
+                            const double* cost, const uint8_t* flags, uint64_t seed,
+                            int64_t first, int64_t n_assign, const int32_t* node_gid,
+                            int32_t first_node, const double* init, double* out, void* stream);
+
 /* Replaces _get_sharded_shape_stride
  * (autoparallel/cost_models/compute_estimation.py:300-318) for n specs:
  * rank[i], shape/stride[i][APC_MAX_RANK], plc[i][APC_MAX_MESH_DIMS] ->

@@ -1,0 +1,50 @@
+"""A graph scored in windows of nodes gives, bit for bit, the sums of one pass
+over the whole graph."""
+import numpy as np
+import pytest
+import torch
+
+from autoparallel_amd import graphgen, windowed
+from oracle import cost_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+N_TOTAL, S_MAX, SEED, N_ASSIGN = 240, 24, 5, 40000
+
+
+def test_windows_equal_one_pass():
+    from autoparallel_amd.engine import CostEngine
+
+    g, gid, n_standin = graphgen.stress_dag_window(N_TOTAL, 0, N_TOTAL, (4, 8, 8), SEED, 4, S_MAX)
+    assert n_standin == 0 and (gid == np.arange(N_TOTAL)).all()
+    eng = CostEngine(g).build(clamp_inf=True)
+    whole = eng.score_random(seed=1, first=0, count=N_ASSIGN).cpu().numpy()
+    again = eng.score_random_window(1, 0, N_ASSIGN, gid, 0).cpu().numpy()
+    assert (whole.view(np.uint64) == again.view(np.uint64)).all()
+    for window in (60, 97):
+        print(f"  windows of {window}", flush=True)
+        got, st = windowed.score_in_windows(N_TOTAL, window, N_ASSIGN, seed=SEED, assign_seed=1, s_max=S_MAX,
+                                            workers=1)
+        assert st["nodes"] == N_TOTAL and st["edges"] == g.num_edges and st["entries"] == g.num_entries
+        assert st["standin_nodes"] > 0
+        assert (got.view(np.uint64) == whole.view(np.uint64)).all()
+    # and the whole-graph sums are the oracle's for a few of the drawn assignments
+    ref = O.GraphOracle(g).build()
+    cost, bad = O.clamp_inf(ref["cost"])
+    for a in (0, 1, 39999):
+        asg = eng.random_assignment(1, a)
+        want = O.score_assignment(g, ref["comm"], ref["transition"], ref["compute"], asg)
+        obj, viol = O.ilp_objective(g, cost, bad, asg)
+        assert tuple(whole[a, :4]) == tuple(float(x) for x in want)
+        assert whole[a, 4] == obj and whole[a, 5] == viol
+
+
+def test_window_arguments_are_checked():
+    from autoparallel_amd.engine import CostEngine
+
+    g, gid, ns = graphgen.stress_dag_window(60, 30, 60, (4, 8, 8), SEED, 4, 12)
+    eng = CostEngine(g).build(clamp_inf=True)
+    with pytest.raises(AssertionError):
+        eng.score_random_window(1, 0, 16, gid[:-1], ns)
+    with pytest.raises(AssertionError):
+        eng.score_random_window(1, 0, 16, gid, ns, init=torch.zeros(8, 6, dtype=torch.float64, device="cuda"))

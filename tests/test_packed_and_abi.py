@@ -260,3 +260,41 @@ def test_engine_needs_gpu():
     g = _mock_graph([(1.0, 2.0, 0)])
     with pytest.raises(Exception):
         CostEngine(g, device="cpu")
+
+
+def test_stress_dag_windows_are_slices_of_one_graph():
+    """A window holds the nodes of its range as the whole DAG has them:
+    same strategies, same producers (by global id), same spec words' content."""
+    n, seed = 90, 3
+    whole, gid_w, ns_w = graphgen.stress_dag_window(n, 0, n, (4, 8, 8), seed, 4, 16)
+    assert ns_w == 0 and whole.num_nodes == n
+
+    def content(g, v):
+        """(strategy count, per edge: producer gid, decoded consumer specs) of local node v."""
+        out = []
+        for e in range(int(g.node_edge_off[v]), int(g.node_edge_off[v + 1])):
+            words = g.lists[int(g.edge_dst_list[e]):int(g.edge_dst_list[e]) + int(g.edge_sdst[e])]
+            metas = words >> packed.TUPLE_BITS
+            dec = [(tuple(g.meta_shape[m][:g.meta_rank[m]]), int(g.meta_dtype[m]), tuple(g.tuple_plc[w & 0xFFF]))
+                   for m, w in zip(metas, words)]
+            src = ()
+            if g.edge_src_node[e] >= 0:  # the producer's run: the stand-in must carry the real specs
+                sw = g.lists[int(g.edge_src_list[e]):int(g.edge_src_list[e]) + int(g.edge_ssrc[e])]
+                src = tuple((tuple(g.meta_shape[w >> packed.TUPLE_BITS][:g.meta_rank[w >> packed.TUPLE_BITS]]),
+                             tuple(g.tuple_plc[w & 0xFFF])) for w in sw)
+            out.append((int(g.edge_src_node[e]), dec + [src]))
+        return int(g.node_nstrat[v]), out
+
+    edges = 0
+    for lo, hi in ((0, 30), (30, 61), (61, 90)):
+        g, gid, ns = graphgen.stress_dag_window(n, lo, hi, (4, 8, 8), seed, 4, 16)
+        g.validate()
+        assert (gid[ns:] == np.arange(lo, hi)).all() and (gid[:ns] < lo).all() and (np.diff(gid[:ns]) > 0).all()
+        for v in range(ns, g.num_nodes):
+            s_loc, e_loc = content(g, v)
+            s_all, e_all = content(whole, int(gid[v]))
+            assert s_loc == s_all and len(e_loc) == len(e_all)
+            for (src_l, dec_l), (src_a, dec_a) in zip(e_loc, e_all):
+                assert (int(gid[src_l]) if src_l >= 0 else -1) == src_a and dec_l == dec_a
+        edges += int((g.edge_node >= ns).sum())
+    assert edges == whole.num_edges
