@@ -1445,6 +1445,13 @@ int apc_build_all(const apc_problem* p, double* table, double* compute, double* 
   return apc_edge_costs(p, table, per_arg, comm, cost, flags, clamp_inf, stream);
 }
 
+int apc_build_all_timed(const apc_problem* p, double* table, double* compute, double* per_arg,
+                        int32_t* status, double* comm, double* cost, uint8_t* flags,
+                        int32_t clamp_inf, void* timer, int32_t slot, void* stream) {
+  if (int rc = apc_prepare(p, table, compute, per_arg, status, stream)) return rc;
+  return apc_edge_costs_timed(p, table, per_arg, comm, cost, flags, clamp_inf, timer, slot, stream);
+}
+
 int apc_calibration_copy(const void* src, void* dst, int64_t nbytes, void* stream) {
   if (!src || !dst || nbytes <= 0 || (nbytes & 15))
     return fail(APC_ERR_INVALID, "apc_calibration_copy: need non-null buffers, nbytes %% 16 == 0%s");

@@ -305,6 +305,20 @@ class CostEngine:
         self.built = True
         return self
 
+    def build_timed(self, timer, slot: int, clamp_inf: bool = True):
+        """build() with HIP events at the begin and end of the entry kernel (a
+        timer from apc_timer_create); the launches are otherwise identical."""
+        _lib.check(
+            self.lib.apc_build_all_timed(
+                C.byref(self.problem), self._ptr(self.table), self._ptr(self.compute),
+                self._ptr(self.per_arg), self._ptr(self.status), self._ptr(self.comm),
+                self._ptr(self.cost), self._ptr(self.flags), int(bool(clamp_inf)), timer, int(slot),
+                self._stream()),
+            "apc_build_all_timed",
+        )
+        self.built = True
+        return self
+
     def set_node_multiplier(self, mult: np.ndarray) -> None:
         """Replace the objective multiplier per node (cluster multiplicity)."""
         t = self._keep["node_multiplier"]

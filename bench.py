@@ -94,7 +94,7 @@ def main():
 
     # HIP events on the launch stream (torch's current stream is the one the
     # engine launches on), recorded at the begin and end of the dominant kernel
-    # of every timed step (apc_edge_costs_timed: the events are attached to the
+    # of every timed step (apc_build_all_timed: the events are attached to the
     # kernel's own dispatch, so dispatch latency is not counted)
     import ctypes as C
 
@@ -103,8 +103,7 @@ def main():
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for k in range(args.steps):
-        eng.prepare()
-        eng.edge_costs_timed(timer, k, clamp_inf=True)
+        eng.build_timed(timer, k, clamp_inf=True)
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     eng.check_status()

@@ -330,6 +330,10 @@ int apc_timer_elapsed_ms(void* timer, int32_t slot, float* ms);
 int apc_edge_costs_timed(const apc_problem* p, const double* table, const double* per_arg,
                          double* comm, double* cost, uint8_t* flags, int32_t clamp_inf, void* timer,
                          int32_t slot, void* stream);
+/* apc_build_all with the entry kernel timed as apc_edge_costs_timed does. */
+int apc_build_all_timed(const apc_problem* p, double* table, double* compute, double* per_arg,
+                        int32_t* status, double* comm, double* cost, uint8_t* flags,
+                        int32_t clamp_inf, void* timer, int32_t slot, void* stream);
 
 /* Measurement aid, no counterpart in the reference: a plain device copy of
  * nbytes (multiple of 16) whose HBM traffic is known (nbytes read + nbytes

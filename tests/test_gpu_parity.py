@@ -48,7 +48,7 @@ def _check_build(CE, g, use_table, clamp=False):
 # ---------------------------------------------------------------------------
 # golden vectors of the reference, through the C ABI
 # ---------------------------------------------------------------------------
-@pytest.mark.parametrize("use_table", [True, False])
+@pytest.mark.parametrize("use_table", [True, False, "compressed"])
 def test_golden_comm_vectors(CostEngine, golden, use_table):
     n_cases = int(golden["comm_ncases"][0])
     checked = 0
@@ -62,7 +62,8 @@ def test_golden_comm_vectors(CostEngine, golden, use_table):
         tgt_t = sorted({tuple(int(x) for x in r) for r in tgt})
         g = graph_from_pairs(mesh, 8, shape, stride, itemsize, src_t, tgt_t)
         print(f"golden case {k}: mesh={mesh} shape={shape} pairs={len(want)}", flush=True)
-        eng = CostEngine(g, use_table=use_table).build(clamp_inf=False)
+        kw = dict(table_mode=use_table) if isinstance(use_table, str) else dict(use_table=use_table)
+        eng = CostEngine(g, **kw).build(clamp_inf=False)
         comm = eng.results()["comm"]
         e = 1  # the consumer's edge
         base, ssrc = int(g.edge_off[e]), int(g.edge_ssrc[e])
