@@ -130,6 +130,7 @@ class ApcProblem(C.Structure):
         ("list_uidx", C.c_void_p),
         ("list_ufirst", C.c_void_p),
         ("block_udst", C.c_void_p),
+        ("comp_recs", C.c_void_p),
     ]
 
 

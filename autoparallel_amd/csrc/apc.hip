@@ -263,6 +263,8 @@ __device__ __forceinline__ double roofline(const apc_problem& p, int64_t flops, 
 constexpr int kNodesPerBlock = 4;  // one wavefront each
 constexpr int kFusedTableBlocks = 2048;  // larger tables are built by a launch of their own
 constexpr int kProgCache = 128;    // int64 words of program staged per wave
+constexpr int kRecWords = 8;       // int64 words of LDS for the record's argument runs
+static_assert(kRecWords * 2 >= APC_REC_ARGS && sizeof(apc_comp_rec) == 96, "record layout");
 
 // One wavefront per 64 strategies of an evaluated node.  Phase 1: the lanes split the node's
 // (strategy, argument) pairs and write each argument's local (sharded) sizes
@@ -271,16 +273,37 @@ constexpr int kProgCache = 128;    // int64 words of program staged per wave
 // program out of LDS.  A wavefront handles the 64 strategies from o0; a node
 // with more strategies is split over several wavefronts.  `slow` (the LDS
 // layout does not fit) reads sizes from memory on demand instead.
-__device__ __forceinline__ void node_compute_wave(const apc_problem& p, int v, int o0, int lane,
-                                                  int64_t* __restrict__ s_prog,
+// The record of evaluated node i: read as it is, or gathered from the node
+// arrays when the caller keeps none.
+__device__ __forceinline__ apc_comp_rec load_comp_rec(const apc_problem& p, int i) {
+  if (p.comp_recs) return p.comp_recs[i];
+  apc_comp_rec r;
+  const int v = __builtin_amdgcn_readfirstlane(p.comp_nodes[i]);
+  r.node = v;
+  r.nstrat = p.node_nstrat[v];
+  r.nargs = p.node_nargs[v];
+  r.op = p.node_op[v];
+  r.comp_off = p.node_comp_off[v];
+  r.prog_off = p.node_prog_off[v];
+  r.prog_len = p.node_prog_len[v];
+  const int e0 = p.node_edge_off[v];
+  r.n_edge = p.node_edge_off[v + 1] - e0;
+#pragma unroll
+  for (int a = 0; a < APC_REC_ARGS; ++a) r.dst_list[a] = a < r.n_edge ? p.edges[e0 + a].dst_list : 0u;
+  return r;
+}
+
+__device__ __forceinline__ void node_compute_wave(const apc_problem& p, const apc_comp_rec& rec,
+                                                  int o0, int lane, int64_t* __restrict__ s_prog,
+                                                  uint32_t* __restrict__ s_dst,
                                                   int64_t* __restrict__ s_local, bool slow,
                                                   double* __restrict__ compute,
                                                   double* __restrict__ per_arg,
                                                   int32_t* __restrict__ status) {
-  const int S = p.node_nstrat[v];
-  const int64_t base = p.node_comp_off[v];
-  const int nargs = p.node_nargs[v];
-  const int op = p.node_op[v];
+  const int S = rec.nstrat;
+  const int64_t base = rec.comp_off;
+  const int nargs = rec.nargs;
+  const int op = rec.op;
   if (o0 >= S) return;  // wave-uniform
   if (op == APC_OP_ZERO) {
     const int o = o0 + lane;
@@ -290,17 +313,29 @@ __device__ __forceinline__ void node_compute_wave(const apc_problem& p, int v, i
     }
     return;
   }
-  const int e0 = p.node_edge_off[v], e1 = p.node_edge_off[v + 1];
-  const int na = e1 - e0;
+  const int na = rec.n_edge;
+  // lanes look the run of an argument up by a lane-varying index: through LDS
+  if (lane == 0) {  // constant indices: the record stays in scalar registers
+#pragma unroll
+    for (int a = 0; a < APC_REC_ARGS; ++a) s_dst[a] = rec.dst_list[a];
+  }
+  const int e0 = na > APC_REC_ARGS ? p.node_edge_off[rec.node] : 0;  // only for the arguments past the record
+  auto dst_of = [&](int a) -> uint32_t {
+    return a < APC_REC_ARGS ? s_dst[a] : p.edges[e0 + a].dst_list;
+  };
   const int max_rank = p.max_rank;
   const int slots = max_rank + 1;  // per argument: max_rank sizes + one info word
+  // program words: loaded now, parked in LDS after the argument loads below are
+  // on their way
   const int64_t* prog = nullptr;
+  int64_t pw0 = 0, pw1 = 0;
+  bool cached = false;
   if (op == APC_OP_PROGRAM) {
-    prog = p.prog + p.node_prog_off[v];
-    const int len = p.node_prog_len[v];
-    if (len <= kProgCache) {
-      for (int i = lane; i < len; i += 64) s_prog[i] = prog[i];
-      prog = s_prog;  // LDS operations of one wave execute in order
+    prog = p.prog + rec.prog_off;
+    cached = rec.prog_len <= kProgCache;
+    if (cached) {
+      if (lane < rec.prog_len) pw0 = prog[lane];
+      if (lane + 64 < rec.prog_len) pw1 = prog[lane + 64];
     }
   }
   {
@@ -308,7 +343,7 @@ __device__ __forceinline__ void node_compute_wave(const apc_problem& p, int v, i
     if (!slow && op == APC_OP_PROGRAM) {
       for (int t = lane; t < chunk * na; t += 64) {
         const int a = t / chunk, oo = t - a * chunk;
-        const uint32_t w = p.lists[(size_t)p.edges[e0 + a].dst_list + o0 + oo];
+        const uint32_t w = p.lists[(size_t)dst_of(a) + o0 + oo];
         const bool none = (w == APC_SPEC_NONE);
         const uint32_t mid = none ? 0u : (w >> APC_TUPLE_BITS);
         const int rank = none ? 0 : p.meta_rank[mid];
@@ -339,6 +374,11 @@ __device__ __forceinline__ void node_compute_wave(const apc_problem& p, int v, i
                     ((int64_t)p.meta_dtype[mid] << 40));
       }
     }
+    if (cached) {  // LDS operations of one wave execute in order
+      if (lane < rec.prog_len) s_prog[lane] = pw0;
+      if (lane + 64 < rec.prog_len) s_prog[lane + 64] = pw1;
+      prog = s_prog;
+    }
     const int o = o0 + lane;
     if (lane >= chunk) return;
     const int64_t idx = base + o;
@@ -348,7 +388,7 @@ __device__ __forceinline__ void node_compute_wave(const apc_problem& p, int v, i
     const bool staged = !slow && op == APC_OP_PROGRAM;
     auto size_of = [&](int a, int d) -> int64_t {
       if (staged) return s_local[(a * slots + d) * 64 + lane];
-      return local_size(p, p.lists[(size_t)p.edges[e0 + a].dst_list + o], d);
+      return local_size(p, p.lists[(size_t)dst_of(a) + o], d);
     };
     // rank of argument a, or -1 if it has no spec
     auto rank_of = [&](int a) -> int {
@@ -356,7 +396,7 @@ __device__ __forceinline__ void node_compute_wave(const apc_problem& p, int v, i
         const int64_t info = s_local[(a * slots + max_rank) * 64 + lane];
         return info < 0 ? -1 : (int)(info & 0xFF);
       }
-      const uint32_t w = p.lists[(size_t)p.edges[e0 + a].dst_list + o];
+      const uint32_t w = p.lists[(size_t)dst_of(a) + o];
       return w == APC_SPEC_NONE ? -1 : p.meta_rank[w >> APC_TUPLE_BITS];
     };
     for (int a = 0; a < na; ++a) {
@@ -368,7 +408,7 @@ __device__ __forceinline__ void node_compute_wave(const apc_problem& p, int v, i
         isz = (int)((info >> 8) & 0xFFFFFFFF);
         dt = (int)(info >> 40);
       } else {
-        const uint32_t w = p.lists[(size_t)p.edges[e0 + a].dst_list + o];
+        const uint32_t w = p.lists[(size_t)dst_of(a) + o];
         if (w == APC_SPEC_NONE) continue;
         const uint32_t mid = w >> APC_TUPLE_BITS;
         rank = p.meta_rank[mid];
@@ -523,12 +563,11 @@ prepare_kernel(apc_problem p, double* __restrict__ table, int table_blocks, int 
   const int chunks = (p.max_nstrat + 63) >> 6;  // wavefronts per node
   const int i = unit / chunks;
   if (i >= p.n_comp_node) return;
-  const uint32_t keep = warm_problem(p, threadIdx.x & 63, 64);
-  asm volatile("" ::"v"(keep));
-  const int v = __builtin_amdgcn_readfirstlane(p.comp_nodes[i]);
-  const int per_wave = kProgCache + (slow ? 0 : p.max_node_args * (p.max_rank + 1) * 64);
+  const apc_comp_rec rec = load_comp_rec(p, i);
+  const int per_wave = kProgCache + kRecWords + (slow ? 0 : p.max_node_args * (p.max_rank + 1) * 64);
   int64_t* s_prog = s_dyn + (size_t)wave * per_wave;
-  node_compute_wave(p, v, (unit - i * chunks) * 64, threadIdx.x & 63, s_prog, s_prog + kProgCache,
+  node_compute_wave(p, rec, (unit - i * chunks) * 64, threadIdx.x & 63, s_prog,
+                    reinterpret_cast<uint32_t*>(s_prog + kProgCache), s_prog + kProgCache + kRecWords,
                     slow != 0, compute, per_arg, status);
 }
 
@@ -1262,10 +1301,10 @@ int launch_prepare(const apc_problem* p, double* table, bool do_nodes, double* c
   // LDS for the local-size staging (a CU has 160 KB); beyond 96 KB per block,
   // sizes are read on demand instead
   const int64_t words = (int64_t)p->max_node_args * (p->max_rank + 1) * 64;
-  const int slow = ((kProgCache + words) * kNodesPerBlock * 8 > 96 * 1024 || p->n_meta == 0 ||
-                    p->n_tuple == 0) ? 1 : 0;
+  const int slow = ((kProgCache + kRecWords + words) * kNodesPerBlock * 8 > 96 * 1024 ||
+                    p->n_meta == 0 || p->n_tuple == 0) ? 1 : 0;
   const size_t lds =
-      do_nodes ? (size_t)kNodesPerBlock * (kProgCache + (slow ? 0 : words)) * 8 : 0;
+      do_nodes ? (size_t)kNodesPerBlock * (kProgCache + kRecWords + (slow ? 0 : words)) * 8 : 0;
   static bool attr_set = false;  // raise the 64 KB default limit of dynamic LDS once
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(prepare_kernel),

@@ -166,6 +166,7 @@ class CostEngine:
         p.n_compute = g.num_compute
         p.n_comp_node = g.comp_nodes.shape[0]
         p.comp_nodes = up("comp_nodes", g.comp_nodes)
+        p.comp_recs = up("comp_recs", g.comp_records())
         p.max_nstrat = int(g.node_nstrat[g.comp_nodes].max()) if g.comp_nodes.shape[0] else 1
         mult = g.node_multiplier if g.node_multiplier is not None else np.ones(g.num_nodes, np.int32)
         p.node_multiplier = up("node_multiplier", mult)

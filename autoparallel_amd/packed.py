@@ -310,6 +310,28 @@ class PackedGraph:
         rec["src_node"] = self.edge_src_node
         return rec
 
+    REC_ARGS = 14
+    COMP_REC_DTYPE = np.dtype([
+        ("node", "<i4"), ("nstrat", "<i4"), ("nargs", "<i4"), ("op", "<i4"), ("comp_off", "<i8"),
+        ("prog_off", "<i8"), ("prog_len", "<i4"), ("n_edge", "<i4"), ("dst_list", "<u4", (14,)),
+    ])
+
+    def comp_records(self) -> np.ndarray:
+        """One 96-byte record per evaluated node (``apc_comp_rec`` of
+        include/apc.h): what the node kernel reads about the node, gathered."""
+        v = self.comp_nodes.astype(np.int64)
+        rec = np.zeros(v.shape[0], self.COMP_REC_DTYPE)
+        assert rec.dtype.itemsize == 96
+        e0 = self.node_edge_off[:-1].astype(np.int64)[v]
+        n_edge = (self.node_edge_off[1:].astype(np.int64)[v] - e0)
+        rec["node"], rec["nstrat"], rec["nargs"] = v, self.node_nstrat[v], self.node_nargs[v]
+        rec["op"], rec["comp_off"] = self.node_op[v], self.node_comp_off[v]
+        rec["prog_off"], rec["prog_len"], rec["n_edge"] = self.node_prog_off[v], self.node_prog_len[v], n_edge
+        for a in range(self.REC_ARGS):
+            has = n_edge > a
+            rec["dst_list"][has, a] = self.edge_dst_list[(e0 + a)[has]].astype(np.uint32)
+        return rec
+
     @property
     def max_node_args(self) -> int:
         return int(np.diff(self.node_edge_off).max()) if self.num_nodes else 0

@@ -72,6 +72,22 @@ typedef struct apc_edge {
   uint32_t local0;   /* 0 in the edge table; in a work item, its first entry  */
 } apc_edge; /* 64 bytes */
 
+/* Everything the node estimate reads about one evaluated node, in one record,
+ * so that a wavefront starts with one load instead of a chain through the
+ * node, edge-offset and edge arrays. */
+#define APC_REC_ARGS 14
+typedef struct apc_comp_rec {
+  int32_t node;      /* the evaluated node                                    */
+  int32_t nstrat;
+  int32_t nargs;     /* len(input_specs): the divisor of per_arg              */
+  int32_t op;        /* APC_OP_*                                              */
+  int64_t comp_off;  /* slot of (node, out_idx 0) in the compute vector       */
+  int64_t prog_off;  /* into prog, -1 if none                                 */
+  int32_t prog_len;
+  int32_t n_edge;    /* arguments with an edge                                */
+  uint32_t dst_list[APC_REC_ARGS]; /* dst_list of the node's first edges      */
+} apc_comp_rec; /* 96 bytes */
+
 /* Cost-model constants (host values, passed by value into the kernels). */
 typedef struct apc_model {
   int32_t ndim;
@@ -228,6 +244,9 @@ typedef struct apc_problem {
   const int32_t* list_uidx;   /* [n_list] rank of the word among its run's distinct words */
   const int32_t* list_ufirst; /* [n_list] at run + k: position in the run of its k-th distinct word */
   const int32_t* block_udst;  /* [n_block] rows of matrix b */
+  /* optional: one record per entry of comp_nodes (NULL: the kernel gathers the
+   * same fields from the arrays above) */
+  const apc_comp_rec* comp_recs;
 } apc_problem;
 
 int apc_version(void);

@@ -382,6 +382,31 @@ def test_edge_cases(CostEngine, use_table):
     assert got["comm"][b0] == 1.5
 
 
+@pytest.mark.parametrize("rank,n_args", [(1, 15), (2, 16)])
+def test_more_arguments_than_the_node_record_holds(CostEngine, rank, n_args):
+    """Arguments past the 14 runs kept in a node's record are found through the
+    edge table: with rank-1 tensors the local sizes are still staged in LDS, with
+    rank 2 and 16 arguments they are read on demand."""
+    b = GraphBuilder((2, 4), 8)
+    shape = (64, 48)[:rank]
+    m = b.meta(shape, graphgen.contiguous_stride(shape), 2, packed.DT_BF16)
+    opts = O.create_all_options(shape, (2, 4))
+    specs = [b.spec(m, o) for o in opts]
+    phs = [b.add_node(NodeDesc(f"x{k}", in_specs=[[s] for s in specs], out_specs=[[s] for s in specs], inputs=[],
+                               default_rows=[[[0.0]] for _ in specs])) for k in range(3)]
+    rng = np.random.default_rng(rank)
+    S = 40
+    in_specs = [[specs[int(rng.integers(len(specs)))] for _ in range(n_args)] for _ in range(S)]
+    out_specs = [[specs[int(rng.integers(len(specs)))]] for _ in range(S)]
+    b.add_node(NodeDesc("wide", in_specs=in_specs, out_specs=out_specs,
+                        inputs=[phs[k % 3] for k in range(n_args)], op=packed.OP_PROGRAM,
+                        program=opprog.pointwise(rank, 2)))
+    g = b.pack()
+    assert g.max_node_args == n_args > packed.PackedGraph.REC_ARGS
+    _check_build(CostEngine, g, True)
+    _check_build(CostEngine, g, False)
+
+
 def test_unsupported_dtype_reports(CostEngine):
     b = GraphBuilder((2,), 8)
     m = b.meta((8, 8), (8, 1), 8, packed.DT_OTHER)
