@@ -260,7 +260,9 @@ __device__ __forceinline__ double roofline(const apc_problem& p, int64_t flops, 
   return ct >= rw ? ct : rw;  // max(ct, rw): keeps ct on ties
 }
 
-constexpr int kNodesPerBlock = 4;  // one wavefront each
+constexpr int kNodesPerBlock = 2;  // one wavefront each; the other wavefronts of a node block exit at once:
+                                   // the block table's blocks share the launch and its LDS size per block,
+                                   // which decides how many of them a CU holds
 constexpr int kFusedTableBlocks = 2048;  // larger tables are built by a launch of their own
 constexpr int kProgCache = 128;    // int64 words of program staged per wave
 constexpr int kRecWords = 8;       // int64 words of LDS for the record's argument runs
@@ -324,7 +326,7 @@ __device__ __forceinline__ void node_compute_wave(const apc_problem& p, const ap
     return a < APC_REC_ARGS ? s_dst[a] : p.edges[e0 + a].dst_list;
   };
   const int max_rank = p.max_rank;
-  const int slots = max_rank + 1;  // per argument: max_rank sizes + one info word
+  const int slots = max_rank + 2;  // per argument: max_rank sizes, an info word, its local bytes
   // program words: loaded now, parked in LDS after the argument loads below are
   // on their way
   const int64_t* prog = nullptr;
@@ -352,6 +354,7 @@ __device__ __forceinline__ void node_compute_wave(const apc_problem& p, const ap
         ll2_t row[APC_MAX_RANK / 2];
 #pragma unroll
         for (int q = 0; q < APC_MAX_RANK / 2; ++q) row[q] = r[q];
+        int64_t numel = 1;
 #pragma unroll
         for (int d = 0; d < APC_MAX_RANK; ++d) {
           if (d >= max_rank) break;  // wave-uniform
@@ -366,12 +369,15 @@ __device__ __forceinline__ void node_compute_wave(const apc_problem& p, const ap
             }
           }
           s_local[(a * slots + d) * 64 + oo] = sz;
+          numel *= sz;  // sizes past the rank are 1
         }
         // info word: rank | itemsize << 8 | dtype << 40, or -1 for a missing spec
+        const int64_t isz = p.meta_itemsize[mid];
         s_local[(a * slots + max_rank) * 64 + oo] =
-            none ? -1
-                 : ((int64_t)rank | ((int64_t)p.meta_itemsize[mid] << 8) |
-                    ((int64_t)p.meta_dtype[mid] << 40));
+            none ? -1 : ((int64_t)rank | (isz << 8) | ((int64_t)p.meta_dtype[mid] << 40));
+        // numel * itemsize of the local tensor, formed here where the sizes are
+        // in registers: phase 2 adds one word per argument
+        s_local[(a * slots + max_rank + 1) * 64 + oo] = numel * isz;
       }
     }
     if (cached) {  // LDS operations of one wave execute in order
@@ -404,9 +410,9 @@ __device__ __forceinline__ void node_compute_wave(const apc_problem& p, const ap
       if (staged) {
         const int64_t info = s_local[(a * slots + max_rank) * 64 + lane];
         if (info < 0) continue;
-        rank = (int)(info & 0xFF);
-        isz = (int)((info >> 8) & 0xFFFFFFFF);
-        dt = (int)(info >> 40);
+        if (!have_dtype) { dtype = (int)(info >> 40); have_dtype = true; }
+        nbytes += s_local[(a * slots + max_rank + 1) * 64 + lane];
+        continue;
       } else {
         const uint32_t w = p.lists[(size_t)dst_of(a) + o];
         if (w == APC_SPEC_NONE) continue;
@@ -547,7 +553,7 @@ __device__ __forceinline__ void pair_table_block(const apc_problem& p, double* _
 // Blocks [0, table_blocks) fill the pair table, the rest price the nodes of
 // comp_nodes: the two are independent, and one launch saves a dispatch on a
 // problem this small.  Dynamic LDS: per wave kProgCache words of program, then
-// (unless slow) max_node_args * (max_rank + 1) * 64 words of local sizes and
+// (unless slow) max_node_args * (max_rank + 2) * 64 words of local sizes, local bytes and
 // argument info.
 __global__ void __launch_bounds__(256)
 prepare_kernel(apc_problem p, double* __restrict__ table, int table_blocks, int slow,
@@ -559,12 +565,13 @@ prepare_kernel(apc_problem p, double* __restrict__ table, int table_blocks, int 
     return;
   }
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  if (wave >= kNodesPerBlock) return;
   const int unit = ((int)blockIdx.x - table_blocks) * kNodesPerBlock + wave;
   const int chunks = (p.max_nstrat + 63) >> 6;  // wavefronts per node
   const int i = unit / chunks;
   if (i >= p.n_comp_node) return;
   const apc_comp_rec rec = load_comp_rec(p, i);
-  const int per_wave = kProgCache + kRecWords + (slow ? 0 : p.max_node_args * (p.max_rank + 1) * 64);
+  const int per_wave = kProgCache + kRecWords + (slow ? 0 : p.max_node_args * (p.max_rank + 2) * 64);
   int64_t* s_prog = s_dyn + (size_t)wave * per_wave;
   node_compute_wave(p, rec, (unit - i * chunks) * 64, threadIdx.x & 63, s_prog,
                     reinterpret_cast<uint32_t*>(s_prog + kProgCache), s_prog + kProgCache + kRecWords,
@@ -1300,7 +1307,7 @@ int launch_prepare(const apc_problem* p, double* table, bool do_nodes, double* c
   if (table_blocks + node_blocks == 0) return 0;
   // LDS for the local-size staging (a CU has 160 KB); beyond 96 KB per block,
   // sizes are read on demand instead
-  const int64_t words = (int64_t)p->max_node_args * (p->max_rank + 1) * 64;
+  const int64_t words = (int64_t)p->max_node_args * (p->max_rank + 2) * 64;
   const int slow = ((kProgCache + kRecWords + words) * kNodesPerBlock * 8 > 96 * 1024 ||
                     p->n_meta == 0 || p->n_tuple == 0) ? 1 : 0;
   const size_t lds =
