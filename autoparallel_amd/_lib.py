@@ -131,6 +131,7 @@ class ApcProblem(C.Structure):
         ("list_ufirst", C.c_void_p),
         ("block_udst", C.c_void_p),
         ("comp_recs", C.c_void_p),
+        ("item_entries", C.c_int32),
     ]
 
 

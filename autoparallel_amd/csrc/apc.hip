@@ -590,10 +590,9 @@ pair_table_kernel(apc_problem p, double* __restrict__ table) {
 // ---------------------------------------------------------------------------
 // Kernel: cost entries
 // ---------------------------------------------------------------------------
-constexpr int kPerLane = 4;                   // consecutive entries per lane
-constexpr int kItemEntries = 64 * kPerLane;   // entries per work item (one wavefront)
+constexpr int kPerLane = 4;  // entries per lane of a work item of APC_ITEM_ENTRIES entries
 static_assert(sizeof(apc_edge) == 64, "edge record layout");
-static_assert(kItemEntries == APC_ITEM_ENTRIES, "work items are built for this kernel");
+static_assert(64 * kPerLane == APC_ITEM_ENTRIES, "work items are built for this kernel");
 
 // Edge that owns slot idx.  Edge blocks start on multiples of 16 slots, so each
 // 16-slot chunk belongs to exactly one edge.
@@ -681,26 +680,32 @@ __device__ __forceinline__ void process_item(const apc_problem& p, const apc_edg
 // the loads of a wave's next item are in flight while the current item is
 // stored.  The kernel needs a third of the registers of the direct one, which
 // is why the two do not share a body: eight waves per SIMD instead of three.
+// Work items of the table path hold 256 or 512 entries (apc_problem.item_entries):
+// measured on MI355X, 256 is faster while the whole launch is a few tens of
+// microseconds (more wavefronts to spread), 512 from some tens of millions of
+// entries on (half the wavefronts, twice the bytes in flight per wavefront:
+// 1.44 ms against 1.67 ms at 418 M entries).
+template <int kN>
 struct ItemLoads {
-  double raw[kPerLane];
-  double pa[kPerLane];
-  uint32_t lk[kPerLane];
+  double raw[kN];
+  double pa[kN];
+  uint32_t lk[kN];
   uint32_t live;  // bit k: entry k of this lane exists
 };
 
-template <bool kSqueezed>
+template <bool kSqueezed, int kN>
 __device__ __forceinline__ void item_load(const apc_edge& ed, int lane, const double* __restrict__ table,
                                           const double* __restrict__ default_vals,
                                           const int32_t* __restrict__ list_uidx,
-                                          const double* __restrict__ per_arg, ItemLoads& r) {
+                                          const double* __restrict__ per_arg, ItemLoads<kN>& r) {
   const uint32_t ssrc = (uint32_t)ed.ssrc;
   const uint32_t size = ssrc * (uint32_t)ed.sdst;
   const double* __restrict__ matrix =  // wave-uniform
       ed.table_off >= 0 ? table + ed.table_off : default_vals + ed.default_off;
   r.live = 0;
-  uint32_t lv[kPerLane], ov[kPerLane];
+  uint32_t lv[kN], ov[kN];
 #pragma unroll
-  for (int k = 0; k < kPerLane; ++k) {
+  for (int k = 0; k < kN; ++k) {
     r.lk[k] = ed.local0 + (uint32_t)(k * 64 + lane);
     const bool live = r.lk[k] < size;
     r.live |= (uint32_t)live << k;
@@ -712,26 +717,27 @@ __device__ __forceinline__ void item_load(const apc_edge& ed, int lane, const do
     // the matrix has one row / column per distinct spec word of the two runs:
     // two index loads, then a gather inside the (cache-resident) matrix
     const uint32_t usrc = (uint32_t)ed.flags >> APC_EDGE_USRC_SHIFT;
-    uint32_t at[kPerLane];
+    uint32_t at[kN];
 #pragma unroll
-    for (int k = 0; k < kPerLane; ++k) {
+    for (int k = 0; k < kN; ++k) {
       const uint32_t uo = (uint32_t)list_uidx[(size_t)ed.dst_list + ov[k]];
       const uint32_t uj = (uint32_t)list_uidx[(size_t)ed.src_list + (lv[k] - ov[k] * ssrc)];
       at[k] = uo * usrc + uj;
     }
 #pragma unroll
-    for (int k = 0; k < kPerLane; ++k) r.raw[k] = matrix[at[k]];
+    for (int k = 0; k < kN; ++k) r.raw[k] = matrix[at[k]];
   } else {
 #pragma unroll
-    for (int k = 0; k < kPerLane; ++k) r.raw[k] = matrix[lv[k]];
+    for (int k = 0; k < kN; ++k) r.raw[k] = matrix[lv[k]];
   }
 }
 
-__device__ __forceinline__ void item_store(const apc_edge& ed, const ItemLoads& r,
+template <int kN>
+__device__ __forceinline__ void item_store(const apc_edge& ed, const ItemLoads<kN>& r,
                                            double* __restrict__ comm, double* __restrict__ cost,
                                            uint8_t* __restrict__ flags, int clamp_inf) {
 #pragma unroll
-  for (int k = 0; k < kPerLane; ++k) {
+  for (int k = 0; k < kN; ++k) {
     const int trans = (int)((uint64_t)__double_as_longlong(r.raw[k]) >> 63);
     const double cm = fabs(r.raw[k]);
     double c = (cm + r.pa[k]) + (double)trans;  // optimize_sharding.py:544
@@ -750,8 +756,9 @@ __device__ __forceinline__ void item_store(const apc_edge& ed, const ItemLoads& 
 
 // Wave w takes items w, w + W, w + 2W, ... (W = waves in the grid, which the
 // launcher caps).
-// kMode 0: direct evaluation; 1: block table; 2: block table with compressed matrices
-template <int kMode>
+// kMode 0: direct evaluation; 1: block table; 2: block table with compressed matrices.
+// kN: entries per lane of a work item (table modes; the direct path has 4).
+template <int kMode, int kN>
 __global__ void __launch_bounds__(kBlock)
 edge_cost_kernel(apc_problem p, const double* __restrict__ table,
                  const double* __restrict__ per_arg, double* __restrict__ comm,
@@ -773,14 +780,14 @@ edge_cost_kernel(apc_problem p, const double* __restrict__ table,
   const int n_item = p.n_item;
   bool have = false;
   apc_edge cur;
-  ItemLoads cur_r;
+  ItemLoads<kN> cur_r;
   apc_edge nxt;
   if (w < n_item) nxt = items[w];
   for (int i = w; i < n_item; i += n_waves) {
     const apc_edge item = nxt;
     if (i + n_waves < n_item) nxt = items[i + n_waves];  // record of the item after this one
-    ItemLoads r;
-    item_load<kMode == 2>(item, lane, table, default_vals, list_uidx, per_arg, r);
+    ItemLoads<kN> r;
+    item_load<kMode == 2, kN>(item, lane, table, default_vals, list_uidx, per_arg, r);
     if (have) item_store(cur, cur_r, comm, cost, flags, clamp_inf);
     cur = item;
     cur_r = r;
@@ -1268,6 +1275,9 @@ int validate_problem(const apc_problem* p) {
       p->n_table_unit != p->table_size / 256 ||
       (p->table_size > 0 && (!p->block_edge || !p->block_off || !p->table_unit_block)))
     return fail(APC_ERR_INVALID, "bad block table description%s");
+  if (p->item_entries != 0 && p->item_entries != APC_ITEM_ENTRIES &&
+      p->item_entries != 2 * APC_ITEM_ENTRIES)
+    return fail(APC_ERR_INVALID, "item_entries must be 0, 256 or 512%s");
   if ((p->list_uidx != nullptr) != (p->list_ufirst != nullptr) ||
       (p->list_uidx != nullptr) != (p->block_udst != nullptr))
     return fail(APC_ERR_INVALID, "compressed block table: list_uidx, list_ufirst and block_udst go together%s");
@@ -1417,15 +1427,20 @@ static int launch_edge_costs(const apc_problem* p, const double* table, const do
   // items per wave; the caps only bound the grid of very large problems.
   const unsigned cap = table ? (1u << 22) : (1u << 14);
   if (grid > cap) grid = cap;
-  if (table && p->list_uidx)
-    hipExtLaunchKernelGGL(edge_cost_kernel<2>, dim3(grid), dim3(kBlock), 0, stream, start, stop, 0,
-                          *p, table, per_arg, comm, cost, flags, clamp_inf);
-  else if (table)
-    hipExtLaunchKernelGGL(edge_cost_kernel<1>, dim3(grid), dim3(kBlock), 0, stream, start, stop, 0,
-                          *p, table, per_arg, comm, cost, flags, clamp_inf);
-  else
-    hipExtLaunchKernelGGL(edge_cost_kernel<0>, dim3(grid), dim3(kBlock), 0, stream, start, stop, 0,
-                          *p, table, per_arg, comm, cost, flags, clamp_inf);
+  const bool wide = p->item_entries == 2 * APC_ITEM_ENTRIES;
+  if (wide && !table)
+    return fail(APC_ERR_INVALID, "apc_edge_costs: work items of 512 entries need a block table%s");
+#define APC_LAUNCH_EDGE(MODE, N)                                                                   \
+  hipExtLaunchKernelGGL((edge_cost_kernel<MODE, N>), dim3(grid), dim3(kBlock), 0, stream, start,   \
+                        stop, 0, *p, table, per_arg, comm, cost, flags, clamp_inf)
+  if (table && p->list_uidx) {
+    if (wide) APC_LAUNCH_EDGE(2, 2 * kPerLane); else APC_LAUNCH_EDGE(2, kPerLane);
+  } else if (table) {
+    if (wide) APC_LAUNCH_EDGE(1, 2 * kPerLane); else APC_LAUNCH_EDGE(1, kPerLane);
+  } else {
+    APC_LAUNCH_EDGE(0, kPerLane);
+  }
+#undef APC_LAUNCH_EDGE
   return check_launch("edge_cost_kernel");
 }
 

@@ -10,12 +10,13 @@ import numpy as np
 import torch
 
 from . import _lib
-from .packed import CHUNK_SHIFT, MAX_MESH_DIMS, PackedGraph
+from .packed import CHUNK_SHIFT, ITEM_ENTRIES, MAX_MESH_DIMS, PackedGraph
 
 # Build the pair table when it is at most this many times the entry count (and
 # small in absolute terms); otherwise every entry is evaluated directly.
 _TABLE_MAX_RATIO = 0.5
 _TABLE_MAX_DOUBLES = 1 << 28
+_WIDE_ITEMS_FROM = 32_000_000  # entries
 
 
 def make_model(mesh_shape, devices_per_host: int, device_name: str, order_mode: int = 0) -> _lib.ApcModel:
@@ -107,12 +108,15 @@ class CostEngine:
         order_mode: int = 0,
         nccl_config=None,
         table_mode: Optional[str] = None,
+        item_entries: Optional[int] = None,
     ):
         """``table_mode``: "full" (one S_dst x S_src matrix per distinct pair of
         runs), "compressed" (matrices by distinct spec word, read by gather),
         "direct" (no table: every entry evaluated), or None: the first of the
         three whose table is small against the entry count.  ``use_table`` is
-        the older switch: True = "full", False = "direct"."""
+        the older switch: True = "full", False = "direct".  ``item_entries``:
+        entries per work item of the entry kernel, 256 or 512 (512 needs a
+        table); None: by problem size."""
         self.lib = _lib.load()
         self.g = g
         self.device = torch.device(device)
@@ -206,7 +210,11 @@ class CostEngine:
         self.table_mode = table_mode
         squeezed = table_mode == "compressed"
         p.edges = up("edges", g.edge_records(squeezed))
-        items = g.work_items(squeezed)
+        # work items of 512 entries pay off from some tens of millions of entries on
+        self.item_entries = (2 * ITEM_ENTRIES if table_mode != "direct" and g.num_entries >= _WIDE_ITEMS_FROM
+                             else ITEM_ENTRIES) if item_entries is None else int(item_entries)
+        items = g.work_items(squeezed, self.item_entries)
+        p.item_entries = self.item_entries
         p.n_item = items.shape[0]
         p.items = up("items", items)
         p.n_default = g.default_vals.shape[0]

@@ -455,16 +455,18 @@ class PackedGraph:
         starts = np.arange(nt, dtype=np.int64) << CHUNK_SHIFT
         return (np.searchsorted(self.edge_off, starts, side="right") - 1).astype(np.int32)
 
-    def work_items(self, compressed: bool = False) -> np.ndarray:
-        """Work items of the entry kernel: for every 256 entries of every edge
-        block a copy of the edge record with ``local0`` set, in slot order."""
+    def work_items(self, compressed: bool = False, item_entries: int = ITEM_ENTRIES) -> np.ndarray:
+        """Work items of the entry kernel: for every ``item_entries`` (256 or 512)
+        entries of every edge block a copy of the edge record with ``local0``
+        set, in slot order."""
+        assert item_entries in (ITEM_ENTRIES, 2 * ITEM_ENTRIES)
         sizes = self.edge_sdst.astype(np.int64) * self.edge_ssrc
-        n = (sizes + ITEM_ENTRIES - 1) // ITEM_ENTRIES
+        n = (sizes + item_entries - 1) // item_entries
         eid = np.repeat(np.arange(self.num_edges, dtype=np.int64), n)
         start = np.concatenate([[0], np.cumsum(n)[:-1]])
         k = np.arange(int(n.sum()), dtype=np.int64) - start[eid]
         items = self.edge_records(compressed)[eid]
-        items["local0"] = k * ITEM_ENTRIES
+        items["local0"] = k * item_entries
         return items
 
     def validate(self) -> None:

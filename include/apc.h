@@ -24,7 +24,8 @@ extern "C" {
 #define APC_TUPLE_BITS 12
 #define APC_SPEC_NONE 0xFFFFFFFFu
 #define APC_CHUNK_SHIFT 4    /* edge blocks start on multiples of 16 slots */
-#define APC_ITEM_ENTRIES 256 /* entries of one edge per work item (one wavefront) */
+#define APC_ITEM_ENTRIES 256 /* entries of one edge per work item (one wavefront);
+                                apc_problem.item_entries may double it */
 #define APC_NUM_DTYPES 8
 
 /* edge flags */
@@ -212,8 +213,9 @@ typedef struct apc_problem {
   int64_t n_slot;            /* length of the entry arrays (with padding)      */
   int64_t n_chunk;           /* n_slot / 16                                    */
   const int32_t* chunk_edge; /* [n_chunk] edge owning slots [16c, 16c + 16)    */
-  /* work items of the entry kernel: for every 256 entries of every edge block a
-   * copy of the edge record with local0 = first entry of the item, slot order */
+  /* work items of the entry kernel: for every 256 (or item_entries) entries of
+   * every edge block a copy of the edge record with local0 = first entry of
+   * the item, slot order */
   int32_t n_item;
   const apc_edge* items;     /* [n_item] */
   int64_t n_default;
@@ -247,6 +249,9 @@ typedef struct apc_problem {
   /* optional: one record per entry of comp_nodes (NULL: the kernel gathers the
    * same fields from the arrays above) */
   const apc_comp_rec* comp_recs;
+  /* entries per work item: 0 or APC_ITEM_ENTRIES, or 2 * APC_ITEM_ENTRIES (block
+   * table only), as the items array was built */
+  int32_t item_entries;
 } apc_problem;
 
 int apc_version(void);

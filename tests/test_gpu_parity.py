@@ -382,6 +382,23 @@ def test_edge_cases(CostEngine, use_table):
     assert got["comm"][b0] == 1.5
 
 
+@pytest.mark.parametrize("mode", ["full", "compressed"])
+def test_work_items_of_512_entries(CostEngine, mode):
+    """Large problems use work items of 512 entries: same bits."""
+    for make in (GRAPHS["llama_2d"], GRAPHS["stress_3d"], _edge_case_graph):
+        g = make()
+        eng = CostEngine(g, table_mode=mode, item_entries=512).build(clamp_inf=False)
+        assert eng.problem.item_entries == 512
+        assert eng.problem.n_item < CostEngine(g, table_mode=mode, item_entries=256).problem.n_item
+        got = eng.results()
+        ref = O.GraphOracle(g).build()
+        assert bits_equal(got["comm"], ref["comm"]) and bits_equal(got["cost"], ref["cost"])
+        assert ((got["flags"] & 1) == ref["transition"]).all()
+    from autoparallel_amd import _lib
+    with pytest.raises(_lib.ApcError):
+        CostEngine(g, table_mode="direct", item_entries=512).build()
+
+
 @pytest.mark.parametrize("rank,n_args", [(1, 15), (2, 16)])
 def test_more_arguments_than_the_node_record_holds(CostEngine, rank, n_args):
     """Arguments past the 14 runs kept in a node's record are found through the
