@@ -198,7 +198,10 @@ class CostEngine:
             if signed_defaults:
                 table_mode = "direct"
             elif small(int(g.block_table(False)[1][-1])):
-                table_mode = "full"
+                # once the outputs stream past every cache, the smaller compressed
+                # table costs less than its gathers (measured at 84 M and 418 M entries)
+                big = g.num_entries >= _WIDE_ITEMS_FROM and g.run_unique_index() is not None
+                table_mode = "compressed" if big and g.block_table(True)[1][-1] < g.block_table(False)[1][-1] else "full"
             elif g.run_unique_index() is not None and small(int(g.block_table(True)[1][-1])):
                 table_mode = "compressed"
             else:
