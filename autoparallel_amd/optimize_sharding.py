@@ -435,10 +435,12 @@ class ShardingOptimizer:
         by_node: Dict[torch.fx.Node, List[DecisionVar]] = {}
         for key in self.selected_keys:
             by_node.setdefault(self.nodes[key[0]], []).append(self.decision_vars[key])
-        violated = self._core.prob.violated()
-        text = "\n".join(f"violated constraint: {n}" for n in violated)
         del sol
-        return log_formatting.format_sharding_log(self.graph, by_node, colored, verbose, text)
+        return log_formatting.format_sharding_log(self.graph, by_node, colored, verbose,
+                                                  self.get_violated_constraints_log())
+
+    def get_violated_constraints_log(self) -> str:
+        return self._core.get_violated_constraints_log()
 
     def save(self, path: str) -> None:
         """Packed state (graph arrays, coefficient twin, constraint log,

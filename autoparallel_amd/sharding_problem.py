@@ -547,10 +547,24 @@ class PackedShardingOptimizer:
 
         return export_json.export_sharding_json(self, self._extract() if sol is None else sol)
 
+    def get_violated_constraints_log(self) -> str:
+        """The rows the current solution violates, with their terms, in the
+        reference's layout (optimize_sharding.py:1115-1124)."""
+        x = self.prob.x
+        violated = [(n, r) for n, r in self.prob.constraints.items() if x is not None and not r.valid(x)]
+        out = f"Violated constraints: {[n for n, _ in violated]}"
+        names = self.var_names() if violated else []
+        for name, r in violated:
+            out += f"\n========= {name} ============="
+            for i, c in zip(r.idx, r.coef):
+                out += f"\n{names[int(i)]}, coeff={c}, value={x[int(i)]}"
+        return out
+
     def get_log(self, sol: Optional[np.ndarray] = None) -> str:
         from . import log_formatting
 
-        return log_formatting.format_packed_log(self, self._extract() if sol is None else sol)
+        return log_formatting.format_packed_log(self, self._extract() if sol is None else sol,
+                                                self.get_violated_constraints_log() if sol is None else "")
 
     def compute_solution_cost(self, sol: np.ndarray) -> Dict[str, float]:
         """The reference's _compute_solution_cost for one assignment, on the device."""

@@ -193,3 +193,22 @@ def test_clustered_ilp_matches_reference_semantics():
     assert opt.cluster_links and all(opt.root[r] == r for r in opt.cluster_links.values())
     with pytest.raises(RuntimeError, match="shares the variables"):
         opt.add_node_constraint(int(np.nonzero(opt.linked)[0][0]))
+
+
+def test_violated_constraints_log(tiny):
+    """The reference's layout (optimize_sharding.py:1115-1124): a list of the
+    violated row names, then each row's terms with coefficient and value."""
+    g, coef, _ = tiny
+    opt = PackedShardingOptimizer(g, coefficients=coef)
+    opt.get_solution()
+    assert opt.get_violated_constraints_log() == "Violated constraints: []"
+    # deselect the variable chosen for the first (node, arg): its uniqueness row now sums to 0
+    first = int(opt.selected[0])
+    opt.prob.x[first] = 0.0
+    log = opt.get_violated_constraints_log()
+    head, *rest = log.split("\n")
+    assert head.startswith("Violated constraints: ['unique_decision_000'")
+    assert rest[0] == "========= unique_decision_000 ============="
+    names = opt.var_names()
+    assert f"{names[first]}, coeff=1.0, value=0.0" in rest
+    opt.prob.x[first] = 1.0
