@@ -8,7 +8,10 @@ from .collective_runtime_estimation import (  # noqa: F401
     set_nccl_topo_config,
 )
 from .compute_estimation import (  # noqa: F401
+    DeviceLimit,
+    compute_memory_cost,
     compute_read_write_time,
+    einsum_flop,
     estimate_strategy_runtime_cost,
     reset_compute_cost_cache,
 )

@@ -27,6 +27,74 @@ def _model(mesh_shape=(1,)):
     return make_model(tuple(mesh_shape), 1, _device_name())
 
 
+# dtype order of apc_model.tflops (packed.DT_*: float64, float32, float16, bfloat16, int8)
+_TFLOPS_DTYPES = (torch.float64, torch.float32, torch.float16, torch.bfloat16, torch.int8)
+
+
+class DeviceLimit:
+    """Bandwidth and GEMM throughput of the current device, as the reference's
+    DeviceLimit carries them (compute_estimation.py:47-66), read from the
+    engine's device table (apc_device_limits)."""
+
+    def __init__(self, name: str, gmem_bandwidth: float, gemm_tflops: Dict[torch.dtype, float]):
+        self.name, self.gmem_bandwidth, self.gemm_tflops = name, gmem_bandwidth, gemm_tflops
+
+
+def _get_device_limit() -> DeviceLimit:
+    """Raises ValueError for a device the table does not know, as the reference
+    does (compute_estimation.py:258-275)."""
+    from .collective_runtime_estimation import _device_name
+
+    name = _device_name()
+    try:
+        m = _model()
+    except _lib.ApcError as exc:
+        raise ValueError(str(exc)) from None
+    tf = {dt: float(m.tflops[i]) for i, dt in enumerate(_TFLOPS_DTYPES) if m.tflops[i] > 0.0}
+    return DeviceLimit(name, float(m.gmem_bw), tf)
+
+
+def _get_device_tflops(dtype) -> float:
+    limit = _get_device_limit()
+    if dtype not in limit.gemm_tflops:
+        raise ValueError(f"Dtype {dtype} not supported on {limit.name}. "
+                         f"Supported dtypes: {list(limit.gemm_tflops.keys())}")
+    return limit.gemm_tflops[dtype]
+
+
+def _get_device_gmem_bandwidth() -> float:
+    return _get_device_limit().gmem_bandwidth
+
+
+def einsum_flop(equation, tensors, out=None, **kwargs) -> int:
+    """Flops of the two einsum forms a linear layer lowers to (reference
+    compute_estimation.py:17-44): "{batch}k,kn->{batch}n" and
+    "{batch}n,{batch}k->kn", 2 * batch * n * k each.  The device evaluates the
+    same products from opprog.einsum_fwd / einsum_bwd."""
+    assert len(tensors) == 2
+    a, b = (tuple(t.shape) for t in tensors)
+    batch = 1
+    for d in a[:-1]:
+        batch *= d
+    if len(b) == 2 and len(a) >= 3:
+        assert a[-1] == b[0], f"Contracting dim mismatch: {a[-1]} vs {b[0]}"
+        return batch * b[1] * a[-1] * 2
+    if len(a) == len(b) and len(a) >= 3:
+        assert a[:-1] == b[:-1], f"Batch dims mismatch: {a[:-1]} vs {b[:-1]}"
+        return batch * a[-1] * b[-1] * 2
+    raise NotImplementedError(f"Unsupported einsum shapes: {a} {b}")
+
+
+def compute_memory_cost(op, args, outs) -> int:
+    """Bytes read plus bytes written by an op (reference compute_estimation.py:321-331)."""
+    from torch.utils._pytree import tree_flatten
+
+    def nbytes(data):
+        return sum(x.numel() * x.element_size() for x in tree_flatten(data)[0] if isinstance(x, torch.Tensor))
+
+    return nbytes(args) + nbytes(outs)
+
+
 def compute_read_write_time(read_write_bytes) -> float:
     lib = _lib.load()
     b = torch.tensor([float(read_write_bytes)], dtype=torch.float64, device="cuda")

@@ -84,3 +84,45 @@ def test_fill_redistribute_cost_shapes(meshes):
     st = OpStrategy([OpSpec(spec, input_specs=[spec, spec])])
     fill_redistribute_cost(st, [prod, prod])
     assert st.strategies[0].redistribute_cost == [[0.0, 0.0], [0.0, 0.0]]
+
+
+def test_device_limit_interface():
+    """The reference's device table values for the MI355X
+    (compute_estimation.py:226-239) through the engine's table, and its errors."""
+    import torch
+
+    from autoparallel_amd.cost_models import compute_estimation as CE
+    from autoparallel_amd.cost_models import collective_runtime_estimation as CRE
+
+    CRE.configure(device_name="AMD Instinct MI355X")
+    try:
+        limit = CE._get_device_limit()
+        assert limit.gmem_bandwidth == 8.0 * 1024**4
+        assert limit.gemm_tflops == {torch.float64: 78.6, torch.float32: 157.3, torch.float16: 2516.6,
+                                     torch.bfloat16: 2516.6, torch.int8: 5033.2}
+        assert CE._get_device_tflops(torch.bfloat16) == 2516.6
+        assert CE._get_device_gmem_bandwidth() == limit.gmem_bandwidth
+        with pytest.raises(ValueError, match="not supported"):
+            CE._get_device_tflops(torch.int64)
+        CRE.configure(device_name="Some Unknown Accelerator")
+        with pytest.raises(ValueError):
+            CE._get_device_limit()
+    finally:
+        CRE.configure(device_name=None)
+
+
+def test_einsum_flop_and_memory_cost_known_answers():
+    import torch
+
+    from autoparallel_amd.cost_models import compute_memory_cost, einsum_flop
+
+    a, b = torch.empty(4, 8, 16, device="meta"), torch.empty(16, 32, device="meta")
+    assert einsum_flop("bsk,kn->bsn", (a, b)) == 4 * 8 * 32 * 16 * 2
+    g, x = torch.empty(4, 8, 32, device="meta"), torch.empty(4, 8, 16, device="meta")
+    assert einsum_flop("bsn,bsk->kn", (g, x)) == 4 * 8 * 32 * 16 * 2
+    with pytest.raises(NotImplementedError):
+        einsum_flop("ij,jk->ik", (torch.empty(2, 3, device="meta"), torch.empty(3, 4, device="meta")))
+    with pytest.raises(AssertionError):
+        einsum_flop("bsk,kn->bsn", (a, torch.empty(15, 32, device="meta")))
+    bf = torch.empty(8, 4, dtype=torch.bfloat16, device="meta")
+    assert compute_memory_cost(None, (a, [bf, 3]), {"out": b}) == 4 * 8 * 16 * 4 + 8 * 4 * 2 + 16 * 32 * 4
