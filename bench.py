@@ -53,8 +53,8 @@ def read_traffic(workload):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="llama3_8b_fwd_bwd_mesh8x8")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--score-assignments", type=int, default=1 << 20,
