@@ -233,6 +233,12 @@ _SIGNATURES = {
         C.c_int,
         [C.POINTER(ApcProblem), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint64, C.c_int64, C.c_int64,
          C.c_void_p, C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p]),
+    "apc_pack_score_records": (
+        C.c_int, [C.POINTER(ApcProblem), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
+    "apc_score_packed": (
+        C.c_int,
+        [C.POINTER(ApcProblem), C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint64, C.c_int64, C.c_int64, C.c_void_p,
+         C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p]),
     "apc_schedule_metrics": (
         C.c_int,
         [C.POINTER(ApcSchedule), C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,

@@ -978,13 +978,21 @@ solution_terms_kernel(apc_problem p, const double* __restrict__ per_arg,
 // ---------------------------------------------------------------------------
 __host__ __device__ __forceinline__ uint32_t mix_assignment(uint64_t seed, int64_t a, int32_t node,
                                                             int32_t nstrat) {
-  // splitmix64 finaliser over (seed, assignment, node)
-  uint64_t z = seed + 0x9E3779B97F4A7C15ull * (uint64_t)(a + 1) +
-               0xBF58476D1CE4E5B9ull * (uint64_t)(node + 1);
-  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
-  z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
-  z = z ^ (z >> 31);
-  return (uint32_t)((z >> 32) % (uint64_t)nstrat);
+  // counter-based draw: a 32-bit mix of (seed, assignment, node) through
+  // murmur3's finaliser, scaled to [0, nstrat) by a multiply-high.  The part
+  // that does not depend on the node is loop-invariant in the scorers; the
+  // walk is instruction-bound, and the 64-bit mix with a modulo that was
+  // here before took a quarter of it.
+  uint32_t h = (uint32_t)seed ^ ((uint32_t)(seed >> 32) * 0x27D4EB2Fu);
+  h ^= (uint32_t)(uint64_t)a * 0x9E3779B1u;
+  h ^= (uint32_t)((uint64_t)a >> 32) * 0x85EBCA77u;
+  h ^= (uint32_t)(node + 1) * 0xC2B2AE3Du;
+  h ^= h >> 16;
+  h *= 0x85EBCA6Bu;
+  h ^= h >> 13;
+  h *= 0xC2B2AE35u;
+  h ^= h >> 16;
+  return (uint32_t)(((uint64_t)h * (uint64_t)(uint32_t)nstrat) >> 32);
 }
 
 template <bool kRandom>
@@ -1077,6 +1085,68 @@ score_window_kernel(apc_problem p, const double* __restrict__ per_arg,
       if (ed.src_node >= 0) {
         const double c = comm[idx];
         if (isfinite(c)) t_comm += c;
+        if ((ed.flags & APC_EDGE_SCORE_TRANSITION) && (f & APC_ENTRY_TRANSITION)) t_trans += 1.0;
+      }
+    }
+  }
+  double* r = out + a * 6;
+  r[0] = (t_compute + t_comm) + t_trans;
+  r[1] = t_compute;
+  r[2] = t_comm;
+  r[3] = t_trans;
+  r[4] = obj;
+  r[5] = forbidden;
+}
+
+// The lane-per-assignment walk over interleaved records (apc_score_rec): one
+// gather per drawn entry.  Covers explicit assignments, drawn ones, and windows
+// of a larger graph (global ids for the draw, sums continued from init).
+__global__ void __launch_bounds__(kBlock)
+score_pack_kernel(int64_t n, const double* __restrict__ comm, const double* __restrict__ cost,
+                  const uint8_t* __restrict__ flags, apc_score_rec* __restrict__ recs) {
+  const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (i >= n) return;
+  apc_score_rec r;
+  r.comm = comm[i];
+  r.cost = cost[i];
+  r.flags = flags[i];
+  r.reserved = 0;
+  recs[i] = r;
+}
+
+template <bool kRandom>
+__global__ void __launch_bounds__(kBlock)
+score_packed_kernel(apc_problem p, const double* __restrict__ per_arg,
+                    const apc_score_rec* __restrict__ recs, const uint16_t* __restrict__ assign,
+                    int64_t stride, uint64_t seed, int64_t first, int64_t n_assign,
+                    const int32_t* __restrict__ node_gid, int first_node,
+                    const double* __restrict__ init, double* __restrict__ out) {
+  const int64_t a = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (a >= n_assign) return;
+  double t_compute = 0.0, t_comm = 0.0, t_trans = 0.0, obj = 0.0, forbidden = 0.0;
+  if (init) {
+    const double* r = init + a * 6;
+    t_compute = r[1]; t_comm = r[2]; t_trans = r[3]; obj = r[4]; forbidden = r[5];
+  }
+  auto choice = [&](int v) -> uint32_t {
+    return kRandom ? mix_assignment(seed, first + a, node_gid ? node_gid[v] : v, p.node_nstrat[v])
+                   : (uint32_t)assign[(size_t)v * stride + a];
+  };
+  for (int v = first_node; v < p.n_node; ++v) {
+    const uint32_t o = choice(v);
+    const int nargs = p.node_nargs[v];
+    const double pa = per_arg[p.node_comp_off[v] + o];
+    t_compute += pa * (double)(nargs > 1 ? nargs : 1);
+    const double mult = (double)p.node_multiplier[v];
+    for (int e = p.node_edge_off[v]; e < p.node_edge_off[v + 1]; ++e) {
+      const apc_edge ed = p.edges[e];
+      const uint32_t j = ed.src_node >= 0 ? choice(ed.src_node) : 0u;
+      const apc_score_rec r = recs[ed.off + (int64_t)o * ed.ssrc + j];
+      const uint32_t f = (uint32_t)r.flags;
+      obj += r.cost * mult;
+      forbidden += (double)((f & APC_ENTRY_NONFINITE) != 0);
+      if (ed.src_node >= 0) {
+        if (isfinite(r.comm)) t_comm += r.comm;
         if ((ed.flags & APC_EDGE_SCORE_TRANSITION) && (f & APC_ENTRY_TRANSITION)) t_trans += 1.0;
       }
     }
@@ -1655,6 +1725,47 @@ int apc_score_random_window(const apc_problem* p, const double* per_arg, const d
                        0, (hipStream_t)stream, *p, per_arg, comm, cost, flags, seed, first + a0, n,
                        node_gid, first_node, init ? init + a0 * 6 : nullptr, out + a0 * 6);
     if (int rc = check_launch("score_window_kernel")) return rc;
+  }
+  return 0;
+}
+
+int apc_pack_score_records(const apc_problem* p, const double* comm, const double* cost,
+                           const uint8_t* flags, apc_score_rec* recs, void* stream) {
+  if (int rc = validate_problem(p)) return rc;
+  if (p->n_slot == 0) return 0;
+  if (!comm || !cost || !flags || !recs)
+    return fail(APC_ERR_INVALID, "apc_pack_score_records: null argument%s");
+  unsigned grid;
+  if (int rc = slot_grid(p, kBlock, &grid)) return rc;
+  hipLaunchKernelGGL(score_pack_kernel, dim3(grid), dim3(kBlock), 0, (hipStream_t)stream, p->n_slot,
+                     comm, cost, flags, recs);
+  return check_launch("score_pack_kernel");
+}
+
+int apc_score_packed(const apc_problem* p, const double* per_arg, const apc_score_rec* recs,
+                     const uint16_t* assign, uint64_t seed, int64_t first, int64_t n_assign,
+                     const int32_t* node_gid, int32_t first_node, const double* init,
+                     double* out, void* stream) {
+  if (int rc = validate_problem(p)) return rc;
+  if (n_assign <= 0) return 0;
+  if (!per_arg || !recs || !out || !p->node_multiplier)
+    return fail(APC_ERR_INVALID, "apc_score_packed: null argument%s");
+  if (first_node < 0 || first_node > p->n_node)
+    return fail(APC_ERR_INVALID, "apc_score_packed: first_node out of range%s");
+  const int64_t kChunk = 262144;  // as launch_score
+  for (int64_t a0 = 0; a0 < n_assign; a0 += kChunk) {
+    const int64_t n = (n_assign - a0 < kChunk) ? (n_assign - a0) : kChunk;
+    const dim3 grid((unsigned)((n + kBlock - 1) / kBlock));
+    const double* in = init ? init + a0 * 6 : nullptr;
+    if (assign)
+      hipLaunchKernelGGL(score_packed_kernel<false>, grid, dim3(kBlock), 0, (hipStream_t)stream, *p,
+                         per_arg, recs, assign + a0, n_assign, seed, first + a0, n, node_gid,
+                         first_node, in, out + a0 * 6);
+    else
+      hipLaunchKernelGGL(score_packed_kernel<true>, grid, dim3(kBlock), 0, (hipStream_t)stream, *p,
+                         per_arg, recs, assign, n_assign, seed, first + a0, n, node_gid, first_node,
+                         in, out + a0 * 6);
+    if (int rc = check_launch("score_packed_kernel")) return rc;
   }
   return 0;
 }

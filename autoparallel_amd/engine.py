@@ -17,6 +17,8 @@ from .packed import CHUNK_SHIFT, ITEM_ENTRIES, MAX_MESH_DIMS, PackedGraph
 _TABLE_MAX_RATIO = 0.5
 _TABLE_MAX_DOUBLES = 1 << 28
 _WIDE_ITEMS_FROM = 32_000_000  # entries
+_PACKED_SCORING_FROM = 8192  # mean entries per edge block
+_SCORE_LANES_FROM = 32768  # assignments: below, one wavefront per assignment (entry arrays as they are)
 
 
 def make_model(mesh_shape, devices_per_host: int, device_name: str, order_mode: int = 0) -> _lib.ApcModel:
@@ -250,6 +252,12 @@ class CostEngine:
             torch.empty(tsize, dtype=torch.float64, device=self.device) if self.use_table else None
         )
         self.built = False
+        # interleaved copy of the entry arrays for scoring (apc_score_rec), made on
+        # first use when the edge blocks are large; stale after anything rewrites
+        # the entry arrays
+        self.packed_scoring = g.num_edges > 0 and g.num_entries / g.num_edges >= _PACKED_SCORING_FROM
+        self._recs: Optional[torch.Tensor] = None
+        self._recs_valid = False
 
     # -- raw stream -----------------------------------------------------------
     def _stream(self):
@@ -276,6 +284,7 @@ class CostEngine:
         )
 
     def edge_costs(self, clamp_inf: bool = True, want_comm: bool = True, want_flags: bool = True):
+        self._recs_valid = False
         _lib.check(
             self.lib.apc_edge_costs(
                 C.byref(self.problem), self._ptr(self.table), self._ptr(self.per_arg),
@@ -287,6 +296,7 @@ class CostEngine:
     def edge_costs_timed(self, timer, slot: int, clamp_inf: bool = True):
         """edge_costs with HIP events at the kernel's begin and end (a timer from
         apc_timer_create); the launch is otherwise identical."""
+        self._recs_valid = False
         _lib.check(
             self.lib.apc_edge_costs_timed(
                 C.byref(self.problem), self._ptr(self.table), self._ptr(self.per_arg), self._ptr(self.comm),
@@ -307,6 +317,7 @@ class CostEngine:
     def build(self, clamp_inf: bool = True):
         """All coefficients: pair table and node compute vectors (one launch),
         then the entry arrays (one launch)."""
+        self._recs_valid = False
         _lib.check(
             self.lib.apc_build_all(
                 C.byref(self.problem), self._ptr(self.table), self._ptr(self.compute),
@@ -320,6 +331,7 @@ class CostEngine:
     def build_timed(self, timer, slot: int, clamp_inf: bool = True):
         """build() with HIP events at the begin and end of the entry kernel (a
         timer from apc_timer_create); the launches are otherwise identical."""
+        self._recs_valid = False
         _lib.check(
             self.lib.apc_build_all_timed(
                 C.byref(self.problem), self._ptr(self.table), self._ptr(self.compute),
@@ -349,6 +361,7 @@ class CostEngine:
         self.compute.copy_(torch.from_numpy(np.ascontiguousarray(compute, np.float64)))
         self.per_arg.copy_(torch.from_numpy(np.ascontiguousarray(per_arg, np.float64)))
         self.built = True
+        self._recs_valid = False
         return self
 
     def capture_build(self, clamp_inf: bool = True) -> "torch.cuda.CUDAGraph":
@@ -375,6 +388,7 @@ class CostEngine:
 
     def apply_prefetch_discount(self, scale: float = 0.0) -> int:
         assert self.built
+        self._recs_valid = False
         n = torch.zeros(1, dtype=torch.int64, device=self.device)
         _lib.check(
             self.lib.apc_apply_prefetch_discount(
@@ -400,12 +414,34 @@ class CostEngine:
         assert assign.dtype in (torch.int16, torch.uint16) and assign.device == self.comm.device
         A = assign.shape[1]
         out = torch.empty((A, 6), dtype=torch.float64, device=self.device)
+        if self.packed_scoring and A >= _SCORE_LANES_FROM:
+            return self._score_packed(assign, 0, 0, A, None, 0, None, out)
         _lib.check(
             self.lib.apc_score_assignments(
                 C.byref(self.problem), self._ptr(self.per_arg), self._ptr(self.comm), self._ptr(self.cost),
                 self._ptr(self.flags), self._ptr(assign), A, self._ptr(out), self._stream()),
             "apc_score_assignments",
         )
+        return out
+
+    def _score_packed(self, assign, seed, first, count, d_gid, first_node, init, out) -> torch.Tensor:
+        """Scoring from the interleaved records (apc_score_packed); they are
+        (re)made here if the entry arrays changed since."""
+        if not self._recs_valid:
+            if self._recs is None:
+                self._recs = torch.empty(self.g.num_slots * 4, dtype=torch.float64, device=self.device)
+            _lib.check(
+                self.lib.apc_pack_score_records(
+                    C.byref(self.problem), self._ptr(self.comm), self._ptr(self.cost), self._ptr(self.flags),
+                    self._ptr(self._recs), self._stream()),
+                "apc_pack_score_records")
+            self._recs_valid = True
+        _lib.check(
+            self.lib.apc_score_packed(
+                C.byref(self.problem), self._ptr(self.per_arg), self._ptr(self._recs), self._ptr(assign),
+                int(seed), int(first), int(count), self._ptr(d_gid), int(first_node), self._ptr(init),
+                self._ptr(out), self._stream()),
+            "apc_score_packed")
         return out
 
     def node_hashes(self, node_phase: Optional[np.ndarray] = None) -> np.ndarray:
@@ -464,6 +500,8 @@ class CostEngine:
     def score_random(self, seed: int, first: int, count: int) -> torch.Tensor:
         assert self.built
         out = torch.empty((count, 6), dtype=torch.float64, device=self.device)
+        if self.packed_scoring and count >= _SCORE_LANES_FROM:
+            return self._score_packed(None, seed, first, count, None, 0, None, out)
         _lib.check(
             self.lib.apc_score_random_assignments(
                 C.byref(self.problem), self._ptr(self.per_arg), self._ptr(self.comm), self._ptr(self.cost),
@@ -483,6 +521,8 @@ class CostEngine:
         assert init is None or (init.shape == (count, 6) and init.dtype == torch.float64 and init.is_contiguous())
         d_gid = torch.from_numpy(gid).to(self.device)
         out = torch.empty((count, 6), dtype=torch.float64, device=self.device)
+        if self.packed_scoring:
+            return self._score_packed(None, seed, first, count, d_gid, first_node, init, out)
         _lib.check(
             self.lib.apc_score_random_window(
                 C.byref(self.problem), self._ptr(self.per_arg), self._ptr(self.comm), self._ptr(self.cost),

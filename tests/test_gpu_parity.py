@@ -328,6 +328,41 @@ def test_scoring(CostEngine):
         assert tuple(out[i, :4]) == tuple(float(x) for x in want)
 
 
+def test_scoring_from_interleaved_records(CostEngine):
+    """apc_score_packed against the scorers that read the three entry arrays:
+    explicit assignments, drawn ones, a window with continued sums; and the
+    records follow the entry arrays when those are rewritten."""
+    for name in ("stress_3d", "llama_2d"):
+        g = GRAPHS[name]()
+        eng = CostEngine(g).build(clamp_inf=True)
+        n = 40000
+        rng = np.random.default_rng(2)
+        assign = np.stack([rng.integers(0, g.node_nstrat) for _ in range(64)], axis=1).astype(np.int16)
+        big = torch.from_numpy(np.ascontiguousarray(np.tile(assign, (1, n // 64 + 1))[:, :n])).cuda()
+        gid = np.arange(g.num_nodes, dtype=np.int32) + 1000
+        half = torch.rand(n, 6, dtype=torch.float64, device="cuda")
+
+        def run():
+            return [eng.score(big), eng.score_random(3, 5, n), eng.score_random_window(3, 0, n, gid, 7, init=half)]
+
+        eng.packed_scoring = False
+        want = run()
+        eng.packed_scoring = True
+        got = run()
+        for a, b in zip(got, want):
+            assert torch.equal(a.view(torch.int64), b.view(torch.int64))
+        assert eng._recs_valid
+        if name == "llama_2d":
+            eng = CostEngine(g).build(clamp_inf=True)
+            eng.packed_scoring = True
+            before = eng.score_random(3, 5, n)
+            assert eng.apply_prefetch_discount(0.25) > 0 and not eng._recs_valid
+            after = eng.score_random(3, 5, n)
+            eng.packed_scoring = False
+            assert torch.equal(after.view(torch.int64), eng.score_random(3, 5, n).view(torch.int64))
+            assert not torch.equal(after, before)
+
+
 # ---------------------------------------------------------------------------
 # edge cases
 # ---------------------------------------------------------------------------
