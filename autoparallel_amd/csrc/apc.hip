@@ -995,6 +995,17 @@ __host__ __device__ __forceinline__ uint32_t mix_assignment(uint64_t seed, int64
   return (uint32_t)(((uint64_t)h * (uint64_t)(uint32_t)nstrat) >> 32);
 }
 
+// An edge record through one 64-byte load.  In the scorers the index is
+// wave-uniform, so this is a single scalar load instead of one per field with a
+// wait after each, and the record of the next edge is requested before the
+// current one is used.
+typedef uint32_t u32x16_t __attribute__((ext_vector_type(16)));
+__device__ __forceinline__ apc_edge load_edge(const apc_edge* __restrict__ e) {
+  union { u32x16_t raw; apc_edge ed; } u;
+  u.raw = *reinterpret_cast<const u32x16_t*>(e);
+  return u.ed;
+}
+
 template <bool kRandom>
 __global__ void __launch_bounds__(kBlock)
 score_kernel(apc_problem p, const double* __restrict__ per_arg, const double* __restrict__ comm,
@@ -1004,6 +1015,8 @@ score_kernel(apc_problem p, const double* __restrict__ per_arg, const double* __
   const int64_t a = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (a >= n_assign) return;
   double t_compute = 0.0, t_comm = 0.0, t_trans = 0.0, obj = 0.0, forbidden = 0.0;
+  apc_edge nxt;  // edges are visited in index order
+  if (p.n_edge > 0) nxt = load_edge(p.edges);
   for (int v = 0; v < p.n_node; ++v) {
     const uint32_t o = kRandom ? mix_assignment(seed, first + a, v, p.node_nstrat[v])
                                : (uint32_t)assign[(size_t)v * stride + a];
@@ -1012,10 +1025,11 @@ score_kernel(apc_problem p, const double* __restrict__ per_arg, const double* __
     t_compute += pa * (double)(nargs > 1 ? nargs : 1);
     const double mult = (double)p.node_multiplier[v];
     for (int e = p.node_edge_off[v]; e < p.node_edge_off[v + 1]; ++e) {
-      const apc_edge ed = p.edges[e];
+      const apc_edge ed = nxt;
+      if (e + 1 < p.n_edge) nxt = load_edge(p.edges + e + 1);
       uint32_t j = 0;
-      if (ed.src_node >= 0)
-        j = kRandom ? mix_assignment(seed, first + a, ed.src_node, p.node_nstrat[ed.src_node])
+      if (ed.src_node >= 0)  // ssrc is the producer's strategy count
+        j = kRandom ? mix_assignment(seed, first + a, ed.src_node, ed.ssrc)
                     : (uint32_t)assign[(size_t)ed.src_node * stride + a];
       const int64_t idx = ed.off + (int64_t)o * ed.ssrc + j;
       const uint8_t f = flags[idx];
@@ -1067,6 +1081,9 @@ score_window_kernel(apc_problem p, const double* __restrict__ per_arg,
     const double* r = init + a * 6;
     t_compute = r[1]; t_comm = r[2]; t_trans = r[3]; obj = r[4]; forbidden = r[5];
   }
+  apc_edge nxt;
+  if (first_node < p.n_node && p.node_edge_off[first_node] < p.n_edge)
+    nxt = load_edge(p.edges + p.node_edge_off[first_node]);
   for (int v = first_node; v < p.n_node; ++v) {
     const uint32_t o = mix_assignment(seed, first + a, node_gid[v], p.node_nstrat[v]);
     const int nargs = p.node_nargs[v];
@@ -1074,10 +1091,11 @@ score_window_kernel(apc_problem p, const double* __restrict__ per_arg,
     t_compute += pa * (double)(nargs > 1 ? nargs : 1);
     const double mult = (double)p.node_multiplier[v];
     for (int e = p.node_edge_off[v]; e < p.node_edge_off[v + 1]; ++e) {
-      const apc_edge ed = p.edges[e];
+      const apc_edge ed = nxt;
+      if (e + 1 < p.n_edge) nxt = load_edge(p.edges + e + 1);
       uint32_t j = 0;
       if (ed.src_node >= 0)
-        j = mix_assignment(seed, first + a, node_gid[ed.src_node], p.node_nstrat[ed.src_node]);
+        j = mix_assignment(seed, first + a, node_gid[ed.src_node], ed.ssrc);
       const int64_t idx = ed.off + (int64_t)o * ed.ssrc + j;
       const uint8_t f = flags[idx];
       obj += cost[idx] * mult;
@@ -1128,19 +1146,23 @@ score_packed_kernel(apc_problem p, const double* __restrict__ per_arg,
     const double* r = init + a * 6;
     t_compute = r[1]; t_comm = r[2]; t_trans = r[3]; obj = r[4]; forbidden = r[5];
   }
-  auto choice = [&](int v) -> uint32_t {
-    return kRandom ? mix_assignment(seed, first + a, node_gid ? node_gid[v] : v, p.node_nstrat[v])
+  auto choice = [&](int v, int nstrat) -> uint32_t {
+    return kRandom ? mix_assignment(seed, first + a, node_gid ? node_gid[v] : v, nstrat)
                    : (uint32_t)assign[(size_t)v * stride + a];
   };
+  apc_edge nxt;
+  if (first_node < p.n_node && p.node_edge_off[first_node] < p.n_edge)
+    nxt = load_edge(p.edges + p.node_edge_off[first_node]);
   for (int v = first_node; v < p.n_node; ++v) {
-    const uint32_t o = choice(v);
+    const uint32_t o = choice(v, p.node_nstrat[v]);
     const int nargs = p.node_nargs[v];
     const double pa = per_arg[p.node_comp_off[v] + o];
     t_compute += pa * (double)(nargs > 1 ? nargs : 1);
     const double mult = (double)p.node_multiplier[v];
     for (int e = p.node_edge_off[v]; e < p.node_edge_off[v + 1]; ++e) {
-      const apc_edge ed = p.edges[e];
-      const uint32_t j = ed.src_node >= 0 ? choice(ed.src_node) : 0u;
+      const apc_edge ed = nxt;
+      if (e + 1 < p.n_edge) nxt = load_edge(p.edges + e + 1);
+      const uint32_t j = ed.src_node >= 0 ? choice(ed.src_node, ed.ssrc) : 0u;  // ssrc: the producer's count
       const apc_score_rec r = recs[ed.off + (int64_t)o * ed.ssrc + j];
       const uint32_t f = (uint32_t)r.flags;
       obj += r.cost * mult;

@@ -526,6 +526,10 @@ class PackedGraph:
             src = self.edge_src_node[hp]
             assert (src >= 0).all() and (src < N).all()
             assert (self.edge_ssrc[hp] == self.node_nstrat[src]).all()
+            # inp_idx counts the producer's strategies on every edge that names one
+            # (the scorers draw the producer's choice from ssrc)
+            named = self.edge_src_node >= 0
+            assert (self.edge_ssrc[named] == self.node_nstrat[self.edge_src_node[named]]).all()
             # entries whose spec is missing need a default value
             need_default = ~hp
             assert (self.edge_default_off[need_default] >= 0).all()
