@@ -36,6 +36,15 @@ def bcast(pos_from_right: int) -> Dim:
 
 
 def program(terms: Sequence[Tuple[int, Sequence[Tuple[int, int]]]], outs: Sequence[Tuple[int, Sequence[Dim]]]) -> List[int]:
+    # Terms over the same multiset of factors are one term with the sum of their
+    # coefficients (the five matmuls of an attention backward are two distinct
+    # products): the same integer, and a shorter walk for the lane that
+    # interprets the program, whose length sets the length of the launch.
+    merged: dict = {}
+    for coeff, facs in terms:
+        key = tuple(sorted((int(a), int(d)) for a, d in facs))
+        merged[key] = merged.get(key, 0) + int(coeff)
+    terms = [(c, list(k)) for k, c in merged.items()]
     p: List[int] = [len(terms), len(outs)]
     for coeff, facs in terms:
         p += [int(coeff), len(facs)]
