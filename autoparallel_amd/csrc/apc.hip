@@ -152,7 +152,7 @@ __device__ __forceinline__ void node_compute_wave(const apc_problem& p, const ap
     return a < APC_REC_ARGS ? s_dst[a] : p.edges[e0 + a].dst_list;
   };
   const int max_rank = p.max_rank;
-  const int slots = max_rank + 2;  // per argument: max_rank sizes, an info word, its local bytes
+  const int slots = max_rank + 2;  // per argument: max_rank sizes, an info word, its local element count
   // program words: loaded now, parked in LDS after the argument loads below are
   // on their way
   const int64_t* prog = nullptr;
@@ -201,9 +201,9 @@ __device__ __forceinline__ void node_compute_wave(const apc_problem& p, const ap
         const int64_t isz = p.meta_itemsize[mid];
         s_local[(a * slots + max_rank) * 64 + oo] =
             none ? -1 : ((int64_t)rank | (isz << 8) | ((int64_t)p.meta_dtype[mid] << 40));
-        // numel * itemsize of the local tensor, formed here where the sizes are
-        // in registers: phase 2 adds one word per argument
-        s_local[(a * slots + max_rank + 1) * 64 + oo] = numel * isz;
+        // element count of the local tensor, formed here where the sizes are in
+        // registers: phase 2 reads one word per argument
+        s_local[(a * slots + max_rank + 1) * 64 + oo] = numel;
       }
     }
     if (cached) {  // LDS operations of one wave execute in order
@@ -237,7 +237,7 @@ __device__ __forceinline__ void node_compute_wave(const apc_problem& p, const ap
         const int64_t info = s_local[(a * slots + max_rank) * 64 + lane];
         if (info < 0) continue;
         if (!have_dtype) { dtype = (int)(info >> 40); have_dtype = true; }
-        nbytes += s_local[(a * slots + max_rank + 1) * 64 + lane];
+        nbytes += s_local[(a * slots + max_rank + 1) * 64 + lane] * (int64_t)((info >> 8) & 0xFFFFFFFF);
         continue;
       } else {
         const uint32_t w = p.lists[(size_t)dst_of(a) + o];
@@ -282,6 +282,15 @@ __device__ __forceinline__ void node_compute_wave(const apc_problem& p, const ap
             size = pr[1];
           } else if (kind == 1) {
             size = size_of((int)pr[1], (int)pr[2]);
+          } else if (kind == 3) {  // all local sizes of an argument
+            const int a = (int)pr[1];
+            if (staged) {
+              size = s_local[(a * slots + max_rank + 1) * 64 + lane];
+            } else {
+              size = 1;
+              const int r = rank_of(a);
+              for (int d = 0; d < r; ++d) size *= size_of(a, d);
+            }
           } else {  // broadcast of all tensor args at a right-aligned position
             size = 1;
             const int pos = (int)pr[1];

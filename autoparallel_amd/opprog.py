@@ -18,7 +18,7 @@ from __future__ import annotations
 
 from typing import List, Sequence, Tuple
 
-from .packed import DIM_ARG, DIM_BCAST, DIM_CONST
+from .packed import DIM_ARG, DIM_ARGNUMEL, DIM_BCAST, DIM_CONST
 
 Dim = Tuple[int, int, int]
 
@@ -33,6 +33,12 @@ def argdim(arg: int, dim: int) -> Dim:
 
 def bcast(pos_from_right: int) -> Dim:
     return (DIM_BCAST, int(pos_from_right), 0)
+
+
+def argnumel(arg: int) -> Dim:
+    """All local sizes of an argument as one factor: an output shaped like the
+    argument is ``[argnumel(arg)]``, one program word triple whatever its rank."""
+    return (DIM_ARGNUMEL, int(arg), 0)
 
 
 def program(terms: Sequence[Tuple[int, Sequence[Tuple[int, int]]]], outs: Sequence[Tuple[int, Sequence[Dim]]]) -> List[int]:
@@ -66,7 +72,7 @@ def pointwise(out_rank: int, out_itemsize: int) -> List[int]:
 def same_as_arg(arg: int, rank: int, out_itemsize: int, n_out: int = 1) -> List[int]:
     """Zero-flop op whose outputs have the (local) shape of one argument
     (softmax, dtype conversion, clone, ...)."""
-    return program([], [(out_itemsize, [argdim(arg, i) for i in range(rank)])] * n_out)
+    return program([], [(out_itemsize, [argnumel(arg)])] * n_out)
 
 
 def mm(out_itemsize: int, a: int = 0, b: int = 1) -> List[int]:
@@ -162,9 +168,5 @@ def sdpa_flash_bwd(itemsize: int) -> List[int]:
         # grad_scores^T @ q -> dk
         (2, [(q, 0), (q, 1), (k, 2), (q, 2), (q, 3)]),
     ]
-    outs = [
-        (itemsize, [argdim(q, i) for i in range(4)]),
-        (itemsize, [argdim(k, i) for i in range(4)]),
-        (itemsize, [argdim(v, i) for i in range(4)]),
-    ]
+    outs = [(itemsize, [argnumel(q)]), (itemsize, [argnumel(k)]), (itemsize, [argnumel(v)])]
     return program(terms, outs)

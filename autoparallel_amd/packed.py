@@ -121,8 +121,9 @@ EDGE_USRC_SHIFT = 8
 # inputs (compute_estimation.py:438-493).  Both are written as small programs
 # over the local (sharded) sizes of the tensor args:
 #   flops  = sum_t coeff_t * prod_j size(arg a_tj, dim d_tj)
-#   out[k] = shape whose dims are each: a constant, size(arg, dim), or the
-#            broadcast of all tensor args at a right-aligned position
+#   out[k] = shape whose dims are each: a constant, size(arg, dim), the
+#            broadcast of all tensor args at a right-aligned position, or the
+#            whole element count of an argument
 OP_ZERO = 0  # placeholder / get_attr / view / non-OpOverload: cost is int 0
 OP_PROGRAM = 1  # flops and output shapes from the program
 OP_EXPLICIT = 2  # host supplies flops[o], bytes[o] (ops without a closed form)
@@ -130,6 +131,7 @@ OP_EXPLICIT = 2  # host supplies flops[o], bytes[o] (ops without a closed form)
 DIM_CONST = 0  # value
 DIM_ARG = 1  # (arg, dim)
 DIM_BCAST = 2  # right-aligned position (0 = last dim)
+DIM_ARGNUMEL = 3  # (arg): all of an argument's local sizes as one factor (an output shaped like it)
 
 
 @dataclasses.dataclass
@@ -569,8 +571,10 @@ def check_program(prog: Sequence[int], n_args: int) -> None:
         p += 2
         for _ in range(rank):
             kind = int(prog[p])
-            assert kind in (DIM_CONST, DIM_ARG, DIM_BCAST)
-            if kind == DIM_ARG:
+            assert kind in (DIM_CONST, DIM_ARG, DIM_BCAST, DIM_ARGNUMEL)
+            if kind == DIM_ARGNUMEL:
+                assert 0 <= prog[p + 1] < n_args, "program dim out of range"
+            elif kind == DIM_ARG:
                 assert 0 <= prog[p + 1] < n_args and 0 <= prog[p + 2] < MAX_RANK, "program dim out of range"
             elif kind == DIM_BCAST:
                 assert 0 <= prog[p + 1] < MAX_RANK

@@ -240,6 +240,9 @@ static double node_compute(const oc_graph* g, int v, int o, int* bad) {
           size = p[1];
         } else if (p[0] == 1) {
           size = shp[p[1]][p[2]];
+        } else if (p[0] == 3) { /* all local sizes of an argument */
+          size = 1;
+          for (int q = 0; q < rk[p[1]]; ++q) size *= shp[p[1]][q];
         } else {
           size = 1;
           for (int a = 0; a < na; ++a) {

@@ -289,7 +289,7 @@ def roofline_cost(flops: int, nbytes: int, dtype: int, dev: DeviceLimit):
 # ---------------------------------------------------------------------------
 # Compute programs (see autoparallel_amd/packed.py for the encoding)
 # ---------------------------------------------------------------------------
-DIM_CONST, DIM_ARG, DIM_BCAST = 0, 1, 2
+DIM_CONST, DIM_ARG, DIM_BCAST, DIM_ARGNUMEL = 0, 1, 2, 3
 
 
 def run_program(prog: Sequence[int], local_shapes: List[Optional[List[int]]], itemsizes: List[int]):
@@ -327,6 +327,8 @@ def run_program(prog: Sequence[int], local_shapes: List[Optional[List[int]]], it
                 size = a
             elif kind == DIM_ARG:
                 size = local_shapes[a][b]
+            elif kind == DIM_ARGNUMEL:
+                size = math.prod(local_shapes[a])
             else:
                 size = 1
                 for shp in local_shapes:

@@ -90,11 +90,26 @@ def test_sdpa_bwd_terms_distinct_dims():
     # torch's closed form with all dims different (flop_counter.py:478-512)
     b, h, sq, sk, dq, dv = 3, 5, 7, 11, 13, 17
     want = 2 * b * h * (sq * dq * sk + sq * dv * sk + sk * sq * dv + sq * sk * dq + dq * sq * sk)
-    f, _ = O.run_program(
+    f, nb = O.run_program(
         opprog.sdpa_flash_bwd(2),
         [[b, h, sq, dv], [b, h, sq, dq], [b, h, sk, dq], [b, h, sk, dv]],
         [2, 2, 2, 2])
     assert f == want
+    # bytes: the four inputs read, dq / dk / dv (shaped like q / k / v) written
+    nq, nk, nv = b * h * sq * dq, b * h * sk * dq, b * h * sk * dv
+    assert nb == 2 * (b * h * sq * dv + nq + nk + nv) + 2 * (nq + nk + nv)
+
+
+def test_output_shaped_like_an_argument():
+    """``argnumel`` stands for all of an argument's local sizes: the same bytes as
+    the output written dim by dim."""
+    shapes = [[3, 5, 7], [11, 13]]
+    whole = O.run_program(opprog.same_as_arg(1, 2, 4, n_out=2), shapes, [2, 4])
+    by_dim = O.run_program(opprog.program([], [(4, [opprog.argdim(1, 0), opprog.argdim(1, 1)])] * 2), shapes, [2, 4])
+    assert whole == by_dim == (0, 3 * 5 * 7 * 2 + 11 * 13 * 4 + 2 * 11 * 13 * 4)
+    # equal terms are merged when a program is built: the same flops
+    merged = opprog.program([(2, [(0, 0), (1, 1)]), (3, [(1, 1), (0, 0)])], [])
+    assert merged[:2] == [1, 0] and O.run_program(merged, shapes, [2, 4])[0] == 5 * 3 * 13
 
 
 def test_mm_family_vs_flop_counter():
