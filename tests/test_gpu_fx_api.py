@@ -362,3 +362,57 @@ def test_rebuild_after_mutating_strategies(mesh):
     bad = [i for i, s in enumerate(opt.strats[param].strategies) if str(s.output_specs.placements) == removed]
     assert len(bad) == 1
     assert all(k[2] != bad[0] for k in opt.selected_keys if k[0] == pidx)
+
+
+class _Block(nn.Module):
+    """Embedding, layer norms, attention through scaled_dot_product_attention,
+    a GELU MLP with biases: the op mix of a decoder block."""
+
+    def __init__(self, d=64, h=4):
+        super().__init__()
+        self.h = h
+        self.ln1, self.ln2 = nn.LayerNorm(d), nn.LayerNorm(d)
+        self.qkv, self.o = nn.Linear(d, 3 * d, bias=False), nn.Linear(d, d, bias=False)
+        self.up, self.down = nn.Linear(d, 4 * d), nn.Linear(4 * d, d)
+        self.emb = nn.Embedding(128, d)
+
+    def forward(self, tok):
+        import torch.nn.functional as F
+
+        x = self.emb(tok)
+        b, s, d = x.shape
+        q, k, v = self.qkv(self.ln1(x)).view(b, s, 3, self.h, d // self.h).permute(2, 0, 3, 1, 4)
+        a = F.scaled_dot_product_attention(q, k, v, is_causal=True)
+        x = x + self.o(a.transpose(1, 2).reshape(b, s, d))
+        x = x + self.down(F.gelu(self.up(self.ln2(x))))
+        return x.float().pow(2).mean()
+
+
+def test_transformer_block_joint_graph(mesh):
+    """A decoder block traced fwd+bwd: every coefficient the facade builds equals
+    the oracle's on the same packed problem, and the plan solves."""
+    from torch._functorch.aot_autograd import aot_export_joint_with_descriptors
+    from torch._subclasses.fake_tensor import FakeTensorMode
+
+    from autoparallel_amd.optimize_sharding import ShardingOptimizer
+
+    with FakeTensorMode():
+        m, tok = _Block(), torch.randint(0, 128, (8, 32))
+        with contextlib.ExitStack() as stack:
+            gm = aot_export_joint_with_descriptors(stack, m, (tok,)).graph_module
+    ops = {str(n.target) for n in gm.graph.nodes if n.op == "call_function"}
+    assert any("scaled_dot_product" in o for o in ops) and any("layer_norm" in o for o in ops)
+    assert any("embedding" in o for o in ops)
+    opt = ShardingOptimizer(gm, mesh, devices_per_host=8, device_name="AMD Instinct MI355X")
+    g = opt._packed
+    ref = O.GraphOracle(g).build()
+    slots = g.entry_slots()
+    cost_ref, _ = O.clamp_inf(ref["cost"])
+    assert g.num_entries > 10000
+    assert bits_equal(opt._core.coef.comm, ref["comm"][slots])
+    assert bits_equal(opt._core.coef.cost, cost_ref[slots])
+    assert bits_equal(opt._core.coef.compute, ref["compute"])
+    assert (ref["compute"] > 0).any()
+    sol = opt.get_solution()
+    assert set(sol) == {n for n in opt.nodes if n.op != "output"}
+    assert np.isclose(opt._compute_solution_cost(sol)["total"], opt._core.objective_value, rtol=1e-9)
