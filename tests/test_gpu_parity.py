@@ -540,6 +540,35 @@ def test_full_size_properties(CostEngine):
             assert bits_equal(a["cost"][b0:b0 + n], ref["cost"][b0:b0 + n])
 
 
+@pytest.mark.parametrize("name", ["llama3_8b", "llama3_70b_8layers", "moe_16l", "llama3_70b"])
+def test_full_size_every_entry_against_compiled_oracle(CostEngine, name):
+    """Every entry of the benchmark graphs (not a sample) against the compiled C
+    restatement, itself bit-identical to the Python oracle on the test graphs
+    (tests/test_oracle_c.py); and the other table layouts give the same bits."""
+    from oracle import c_oracle
+
+    g = {"llama3_8b": lambda: graphgen.config_llama3_8b(), "llama3_70b_8layers": lambda: graphgen.config_llama3_70b(8),
+         "moe_16l": lambda: graphgen.config_moe(), "llama3_70b": lambda: graphgen.config_llama3_70b()}[name]()
+    print(f"  {name}: E={g.num_entries}", flush=True)
+    want = c_oracle.COracle(g).build(threads=16)
+    eng = CostEngine(g).build(clamp_inf=False)
+    got = eng.results()
+    assert bits_equal(got["comm"], want["comm"]), first_mismatch(got["comm"], want["comm"])
+    assert bits_equal(got["cost"], want["cost"]), first_mismatch(got["cost"], want["cost"])
+    assert bits_equal(got["compute"], want["compute"])
+    assert ((got["flags"] & 1) == want["transition"]).all()
+    del got, want
+    if g.num_entries > 10**8:  # the largest config once, in the layout the engine picks
+        return
+    for kw in (dict(table_mode="compressed", item_entries=512), dict(table_mode="full", item_entries=512),
+               dict(table_mode="compressed", item_entries=256)):
+        other = CostEngine(g, **kw).build(clamp_inf=False)
+        assert torch.equal(other.comm.view(torch.int64), eng.comm.view(torch.int64)), kw
+        assert torch.equal(other.cost.view(torch.int64), eng.cost.view(torch.int64)), kw
+        assert torch.equal(other.flags, eng.flags), kw
+        del other
+
+
 # ---------------------------------------------------------------------------
 # scalar cost-model entry points in batch form
 # ---------------------------------------------------------------------------
