@@ -540,7 +540,7 @@ def test_full_size_properties(CostEngine):
             assert bits_equal(a["cost"][b0:b0 + n], ref["cost"][b0:b0 + n])
 
 
-@pytest.mark.parametrize("name", ["llama3_8b", "llama3_70b_8layers", "moe_16l", "llama3_70b"])
+@pytest.mark.parametrize("name", ["llama3_8b", "llama3_70b_8layers", "moe_16l", "llama3_70b", "stress_3k"])
 def test_full_size_every_entry_against_compiled_oracle(CostEngine, name):
     """Every entry of the benchmark graphs (not a sample) against the compiled C
     restatement, itself bit-identical to the Python oracle on the test graphs
@@ -548,7 +548,8 @@ def test_full_size_every_entry_against_compiled_oracle(CostEngine, name):
     from oracle import c_oracle
 
     g = {"llama3_8b": lambda: graphgen.config_llama3_8b(), "llama3_70b_8layers": lambda: graphgen.config_llama3_70b(8),
-         "moe_16l": lambda: graphgen.config_moe(), "llama3_70b": lambda: graphgen.config_llama3_70b()}[name]()
+         "moe_16l": lambda: graphgen.config_moe(), "llama3_70b": lambda: graphgen.config_llama3_70b(),
+         "stress_3k": lambda: graphgen.stress_graph(3000, (4, 8, 8), seed=0)}[name]()
     print(f"  {name}: E={g.num_entries}", flush=True)
     want = c_oracle.COracle(g).build(threads=16)
     eng = CostEngine(g).build(clamp_inf=False)
