@@ -1067,6 +1067,18 @@ def config_llama3_70b(n_layers: int = 80) -> PackedGraph:
     return llama_graph((4, 8, 8), n_layers, 8192, 64, 8, 28672, 128256, 8192, 256)
 
 
+def _cap_numel(shape: Tuple[int, ...], limit: int = 2**48) -> Tuple[int, ...]:
+    """Four dims drawn up to 65536 each can describe a tensor of 2**64 elements,
+    which no device holds and int64 byte counts cannot express: the largest dim
+    is halved until the tensor has at most ``limit`` elements (no random draw is
+    consumed, so everything else about the graph is as before)."""
+    shape = list(shape)
+    while math.prod(shape) > limit:
+        k = shape.index(max(shape))
+        shape[k] = max(shape[k] // 2, 1)
+    return tuple(shape)
+
+
 def stress_graph(
     n_nodes: int,
     mesh_shape: Sequence[int] = (4, 8, 8),
@@ -1089,7 +1101,7 @@ def stress_graph(
     n_in_total = 0
     for v in range(n_nodes):
         r = int(rng.integers(1, 5))
-        shape = tuple(int(2 ** rng.uniform(6, 16)) for _ in range(r))
+        shape = _cap_numel(tuple(int(2 ** rng.uniform(6, 16)) for _ in range(r)))
         dt = DT_BF16 if rng.random() < 0.5 else DT_F32
         ranks.append(r)
         dts.append(dt)
@@ -1143,7 +1155,7 @@ def _stress_header(seed: int, v: int, nd: int, s_min: int, s_max: int):
     """(rank, shape, dtype, out placement tuples) of node v, from (seed, v) alone."""
     rng = np.random.default_rng([seed, v, 0])
     r = int(rng.integers(1, 5))
-    shape = tuple(int(2 ** rng.uniform(6, 16)) for _ in range(r))
+    shape = _cap_numel(tuple(int(2 ** rng.uniform(6, 16)) for _ in range(r)))
     dt = DT_BF16 if rng.random() < 0.5 else DT_F32
     S = int(rng.integers(s_min, s_max + 1))
     codes = np.asarray([R] + [shard(d) for d in range(r)] + [P])

@@ -481,6 +481,16 @@ class PackedGraph:
         assert self.meta_shape.shape == (M, MAX_RANK)
         assert self.meta_stride.shape == (M, MAX_RANK)
         assert ((self.meta_rank >= 0) & (self.meta_rank <= MAX_RANK)).all()
+        if M:
+            # The kernels hold a tensor's byte count in int64 (the reference in a
+            # Python int), and the block table keeps the transition flag in the sign
+            # of a cost: a tensor of 2**62 bytes or more would wrap and turn costs
+            # negative.  (Beyond 2**53 bytes the two also round differently.)
+            dims = np.where(np.arange(MAX_RANK)[None, :] < self.meta_rank[:, None], np.maximum(self.meta_shape, 1), 1)
+            log2_bytes = np.log2(dims.astype(np.float64)).sum(axis=1) + np.log2(np.maximum(self.meta_itemsize, 1))
+            if not (log2_bytes < 62).all():
+                raise ValueError(f"tensor meta {int(np.argmax(log2_bytes))} has 2**{log2_bytes.max():.1f} bytes: "
+                                 "beyond the int64 range of the cost engine")
         NT = self.tuple_plc.shape[0]
         assert self.tuple_plc.shape == (NT, MAX_MESH_DIMS) and NT <= MAX_TUPLES
         assert M <= MAX_METAS

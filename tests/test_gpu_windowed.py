@@ -48,3 +48,20 @@ def test_window_arguments_are_checked():
         eng.score_random_window(1, 0, 16, gid[:-1], ns)
     with pytest.raises(AssertionError):
         eng.score_random_window(1, 0, 16, gid, ns, init=torch.zeros(8, 6, dtype=torch.float64, device="cuda"))
+
+
+def test_a_window_of_the_full_dag_against_the_compiled_oracle():
+    """One window deep inside the 200 000-node DAG (stand-in producers from all
+    over the graph): every entry against the compiled C restatement."""
+    from autoparallel_amd.engine import CostEngine
+    from oracle import c_oracle
+
+    g, gid, n_standin = graphgen.stress_dag_window(200000, 150000, 151000)
+    assert n_standin > 1000 and int(gid[:n_standin].min()) < 50000
+    print(f"  window: {g.num_nodes} nodes, E={g.num_entries}", flush=True)
+    want = c_oracle.COracle(g).build(threads=16)
+    eng = CostEngine(g).build(clamp_inf=False)
+    got = eng.results()
+    for k in ("comm", "cost", "compute"):
+        assert (got[k].view(np.uint64) == want[k].view(np.uint64)).all(), k
+    assert ((got["flags"] & 1) == want["transition"]).all()

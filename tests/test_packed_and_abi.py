@@ -298,3 +298,14 @@ def test_stress_dag_windows_are_slices_of_one_graph():
                 assert (int(gid[src_l]) if src_l >= 0 else -1) == src_a and dec_l == dec_a
         edges += int((g.edge_node >= ns).sum())
     assert edges == whole.num_edges
+
+
+def test_tensors_beyond_int64_bytes_are_refused():
+    b = GraphBuilder((2, 4), 8)
+    m = b.meta((65536, 65536, 65536, 32768), graphgen.contiguous_stride((65536, 65536, 65536, 32768)), 4, packed.DT_F32)
+    s = b.spec(m, (0, 0))
+    b.add_node(NodeDesc("x", in_specs=[[s]], out_specs=[[s]], inputs=[], default_rows=[[[0.0]]]))
+    with pytest.raises(ValueError, match="int64 range"):
+        b.pack().validate()
+    assert graphgen._cap_numel((65536, 65536, 65536, 65536)) == (8192, 8192, 8192, 8192) or \
+        np.prod([float(x) for x in graphgen._cap_numel((65536, 65536, 65536, 65536))]) <= 2.0**48
