@@ -7,7 +7,8 @@ it with the reference's post-processing — tensor-meta fill
 (autoparallel/shardings/placement_options.py:60-127), validity filter
 (autoparallel/shardings/propagation_rules.py:127-158), de-duplication
 (placement_options.py:151-170) — and the few rules DTensor lacks or refuses
-(getitem, strict views, alias, two-operand einsum, all-Replicate fallback:
+(getitem, strict views, alias, two-operand einsum, operators without tensor
+inputs: propagation_rules.py:412-554; all-Replicate fallback:
 dtensor_sharding_helpers.py:364-383).  Its output is input data for the cost
 engine.  Input/parameter options are enumerated on the device
 (apc_enumerate_input_options).
@@ -31,6 +32,7 @@ from .. import _lib
 
 aten = torch.ops.aten
 fallback_nodes: List[str] = []  # nodes that got the implicit all-Replicate strategy
+fallback_reasons: Dict[str, str] = {}  # node name -> why its operator strategy was not used
 
 
 def _tensor_meta(t: torch.Tensor) -> TensorMeta:
@@ -136,11 +138,29 @@ def propagate_tensor_meta(node, arg_vals: List[torch.Tensor], out_strat: OpStrat
         if isinstance(outs, DTensorSpec):
             if isinstance(out_val, torch.Tensor):
                 outs.tensor_meta = _tensor_meta(out_val)
+            elif isinstance(out_val, (tuple, list)):
+                # one spec given for an operator with several outputs (the norms:
+                # "out, mean and rstd have the same placements"): one per tensor output
+                st.output_specs = tuple(
+                    DTensorSpec(outs.mesh, outs.placements, tensor_meta=_tensor_meta(v))
+                    if isinstance(v, torch.Tensor) else None for v in out_val)
         elif outs is not None:
             vals = list(out_val) if isinstance(out_val, (tuple, list)) else [out_val]
+            # an output DTensor leaves without a spec is Replicate; a spec for an
+            # output that does not exist is dropped
+            # (autoparallel/shardings/placement_options.py:72-101)
+            mesh = st.mesh
+            fixed = []
             for s, v in zip(outs, vals):
-                if s is not None and isinstance(v, torch.Tensor):
-                    s.tensor_meta = _tensor_meta(v)
+                if isinstance(v, torch.Tensor):
+                    if s is None:
+                        s = DTensorSpec(mesh, (Replicate(),) * mesh.ndim)
+                    if s.tensor_meta is None or s.tensor_meta != _tensor_meta(v):
+                        s.tensor_meta = _tensor_meta(v)
+                else:
+                    s = None
+                fixed.append(s)
+            st.output_specs = tuple(fixed) + tuple(outs[len(fixed):])
         if st.input_specs is not None:
             for s, v in zip(st.input_specs, arg_vals):
                 if s is not None and s.tensor_meta is None:
@@ -208,12 +228,118 @@ def _replicate_fallback(mesh, node, arg_vals) -> OpStrategy:
     else:
         out = tuple(DTensorSpec(mesh, rep, tensor_meta=_tensor_meta(v)) if isinstance(v, torch.Tensor) else None
                     for v in out_val)
-    ins = [DTensorSpec(mesh, rep, tensor_meta=_tensor_meta(v)) for v in arg_vals]
+    ins = [DTensorSpec(mesh, rep, tensor_meta=_tensor_meta(v) if isinstance(v, torch.Tensor) else None)
+           for v in arg_vals]
     fallback_nodes.append(str(node.name))
     return OpStrategy([OpSpec(out, input_specs=ins)])
 
 
-_VIEW_NONSTRICT = {aten.view.default: aten._unsafe_view.default}
+_SHAPE_FACTORY_OPS = {aten.zeros.default, aten.ones.default, aten.full.default, aten.empty.memory_format,
+                      aten.rand.default, aten.randn.default}
+
+
+def _inputless_rule(mesh, node) -> OpStrategy:
+    """Operators without tensor inputs.  The per-argument loops of the
+    coefficient build want one argument, so every strategy carries its output
+    spec as a stand-in input spec with a row of zero costs (no producer: the
+    zeros stay).  Factories that take a size (zeros, ones, full, empty, rand,
+    randn) get every {Shard(d), Replicate} combination over the mesh, Replicate
+    last on each mesh dim, and a row as long as that product before filtering
+    (autoparallel/shardings/propagation_rules.py:486-554); anything whose values
+    depend on the position (iota, :412-421; arange and other generators are
+    treated the same way here) and scalar_tensor (:453-484) are Replicate only."""
+    tm = _tensor_meta(node.meta["val"])
+    if node.target in _SHAPE_FACTORY_OPS:
+        from torch.distributed.tensor._ops.utils import is_tensor_shardable
+
+        shape = tuple(tm.shape)
+        per_dim = [Shard(i) for i in range(len(shape))] + [Replicate()]
+        combs = list(itertools.product(per_dim, repeat=mesh.ndim))
+        sts = []
+        for plc in combs:
+            spec = DTensorSpec(mesh, tuple(plc), tensor_meta=tm)
+            if not is_tensor_shardable(shape, spec):
+                continue
+            sts.append(OpSpec(spec, input_specs=[spec], redistribute_cost=[[0.0] * len(combs)]))
+        return OpStrategy(sts)
+    spec = DTensorSpec(mesh, (Replicate(),) * mesh.ndim, tensor_meta=tm)
+    return OpStrategy([OpSpec(spec, input_specs=[spec], redistribute_cost=[[0.0]])])
+
+
+def _view_rule(mesh, node, src: OpStrategy) -> OpStrategy:
+    """view as the reference prices it
+    (autoparallel/shardings/propagation_rules.py:239-287): one strategy per
+    producer strategy, the input demoted to what the view can keep
+    (strict_view=False) instead of the refusal of DTensor's own rule; a producer
+    strategy the propagation rejects is skipped."""
+    from torch.distributed.tensor._ops._view_ops import dim_maps, propagate_shape_and_sharding
+
+    rules = dim_maps[torch.Tensor.view](src, node.args[1])
+    out_tm = _tensor_meta(node.meta["val"])
+    sts = []
+    for s in src.strategies:
+        spec = s.output_specs
+        try:
+            in_plc, out_plc = propagate_shape_and_sharding(spec.placements, tuple(src.shape), rules,
+                                                           tuple(mesh.shape), strict_view=False)
+        except (AssertionError, RuntimeError):
+            continue
+        sts.append(OpSpec(DTensorSpec(mesh, tuple(out_plc), tensor_meta=out_tm),
+                          input_specs=(DTensorSpec(mesh, tuple(in_plc), tensor_meta=spec.tensor_meta),)))
+    return OpStrategy(sts)
+
+
+def _one_strategy_at_a_time(fn, op, args, kwargs, producers: List[OpStrategy]) -> Optional[OpStrategy]:
+    """Some of DTensor's strategy functions (the norms, nll_loss_backward, ...)
+    index every tensor argument's strategies with the position in the first
+    one's, which holds in eager DTensor (one placement per argument) and fails
+    on arguments with different numbers of candidates.  Those are asked once
+    per strategy of the argument with the most candidates, every other argument
+    standing in with one placement, as at run time: on each mesh dim the lead's
+    Shard where it means the same thing for the argument (same rank, same extent
+    of that tensor dim), else Replicate.  What the function then asks of an
+    argument is priced against the argument's real candidates by the cost engine."""
+    if not producers:
+        return None
+    lead = max(producers, key=lambda p: len(p.strategies))
+
+    def pick(p: OpStrategy, lead_sp: DTensorSpec) -> OpStrategy:
+        if p is lead:
+            return OpStrategy([lead_st])
+        sp = p.strategies[0].output_specs
+        if not isinstance(sp, DTensorSpec):
+            return OpStrategy([p.strategies[0]])
+        a, b = sp.tensor_meta, lead_sp.tensor_meta
+        same_rank = a is not None and b is not None and len(a.shape) == len(b.shape)
+        plc = tuple(x if same_rank and x.is_shard() and a.shape[x.dim] == b.shape[x.dim] else Replicate()
+                    for x in lead_sp.placements)
+        spec = DTensorSpec(sp.mesh, plc, tensor_meta=a)
+        return OpStrategy([OpSpec(spec, input_specs=(spec,), redistribute_cost=[[0.0]])])
+
+    def narrow(a, plc):
+        if isinstance(a, OpStrategy):
+            return pick(a, plc)
+        if isinstance(a, TupleStrategy):
+            return TupleStrategy(tuple(narrow(c, plc) for c in a.children))
+        return a
+
+    sts = []
+    for lead_st in lead.strategies:
+        if not isinstance(lead_st.output_specs, DTensorSpec):
+            return None
+        plc = lead_st.output_specs
+        res = fn(OpSchema(op, tuple(narrow(a, plc) for a in args), kwargs))
+        if not isinstance(res, OpStrategy):
+            return None
+        sts.extend(res.strategies)
+    return OpStrategy(sts)
+
+
+_NONSTRICT_VIEWS = {aten.view.default, aten._unsafe_view.default}
+# strategy functions of the installed torch that pair the arguments' strategies by index
+_INDEX_PAIRED = {getattr(getattr(aten, name), "default") for name in (
+    "native_layer_norm", "native_layer_norm_backward", "_fused_rms_norm", "_fused_rms_norm_backward",
+    "nll_loss_forward", "nll_loss_backward", "nll_loss2d_forward", "nll_loss2d_backward") if hasattr(aten, name)}
 _FOLLOW = {aten.alias.default, aten.detach.default}
 
 
@@ -224,6 +350,8 @@ def get_placement_options_for_node(mesh, node, producers: List[OpStrategy], arg_
     with nodes replaced by their OpStrategy (or value for non-tensors)."""
     prop = DTensor._op_dispatcher.sharding_propagator
     op = node.target
+    if not producers and isinstance(node.meta.get("val"), torch.Tensor):
+        return keep_unique_configs(remove_invalid_configs(_inputless_rule(mesh, node), mesh))
     out = None
     try:
         if op is operator.getitem:
@@ -232,8 +360,10 @@ def get_placement_options_for_node(mesh, node, producers: List[OpStrategy], arg_
             out = _follow_input(mesh, producers[0], node.meta["val"])
         elif op is aten.einsum.default and len(producers) == 2:
             out = _einsum_rule(mesh, node, *producers)
+        elif op in _NONSTRICT_VIEWS and len(producers) == 1:
+            out = _view_rule(mesh, node, producers[0])
         else:
-            fn = prop.op_strategy_funcs.get(_VIEW_NONSTRICT.get(op, op))
+            fn = prop.op_strategy_funcs.get(op)
             if fn is not None:
                 def wrap(x):
                     if isinstance(x, (list, tuple)) and x and all(isinstance(y, OpStrategy) for y in x):
@@ -241,20 +371,39 @@ def get_placement_options_for_node(mesh, node, producers: List[OpStrategy], arg_
                     return x
                 args = tuple(wrap(a) for a in schema_args)
                 kwargs = {k: v for k, v in node.kwargs.items() if not isinstance(v, torch.fx.Node)}
-                res = fn(OpSchema(op, args, kwargs))
+                if op in _INDEX_PAIRED and len(producers) > 1:
+                    res = _one_strategy_at_a_time(fn, op, args, kwargs, producers)
+                else:
+                    try:
+                        res = fn(OpSchema(op, args, kwargs))
+                    except IndexError:
+                        res = _one_strategy_at_a_time(fn, op, args, kwargs, producers)
                 if isinstance(res, OpStrategy):
                     out = res
-    except Exception:
-        out = None
+                    if len(producers) == 1:
+                        # a strategy without input specs follows its output
+                        # (autoparallel/shardings/placement_options.py:104-116)
+                        for st in out.strategies:
+                            if st.input_specs is None and isinstance(st.output_specs, DTensorSpec):
+                                st.input_specs = (st.output_specs,)
+        why = "no strategy registered" if out is None else ""
+    except Exception as exc:
+        out, why = None, f"{type(exc).__name__}: {exc}"
     ok = out is not None and len(out.strategies) > 0 and all(
         st.input_specs is not None and len(st.input_specs) == len(producers) for st in out.strategies)
     if not ok:
+        if out is not None:
+            why = "no strategies" if not out.strategies else (
+                f"{len(producers)} tensor inputs, input specs of "
+                f"{sorted({-1 if st.input_specs is None else len(st.input_specs) for st in out.strategies})}")
+        fallback_reasons[str(node.name)] = why
         out = _replicate_fallback(mesh, node, arg_vals)
     propagate_tensor_meta(node, arg_vals, out)
     fill_redistribute_cost(out, producers)
     out = remove_invalid_configs(out, mesh)
     out = keep_unique_configs(out)
     if not out.strategies:
+        fallback_reasons[str(node.name)] = "no strategy is valid for the shapes"
         out = _replicate_fallback(mesh, node, arg_vals)
         fill_redistribute_cost(out, producers)
     return out

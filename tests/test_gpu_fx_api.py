@@ -396,14 +396,28 @@ def test_transformer_block_joint_graph(mesh):
 
     from autoparallel_amd.optimize_sharding import ShardingOptimizer
 
+    from autoparallel_amd.shardings import placement_options as PO
+
+    # traced on fake tensors of the GPU, so that attention is the fused kernel
+    # DTensor has a strategy for (the CPU kernel has none)
     with FakeTensorMode():
-        m, tok = _Block(), torch.randint(0, 128, (8, 32))
+        with torch.device("cuda"):
+            m = _Block()
+        tok = torch.randint(0, 128, (8, 32), device="cuda")
         with contextlib.ExitStack() as stack:
             gm = aot_export_joint_with_descriptors(stack, m, (tok,)).graph_module
     ops = {str(n.target) for n in gm.graph.nodes if n.op == "call_function"}
     assert any("scaled_dot_product" in o for o in ops) and any("layer_norm" in o for o in ops)
     assert any("embedding" in o for o in ops)
+    PO.fallback_nodes.clear()
+    PO.fallback_reasons.clear()
     opt = ShardingOptimizer(gm, mesh, devices_per_host=8, device_name="AMD Instinct MI355X")
+    # no operator was left with the all-Replicate stand-in, and the norms offer
+    # more than one strategy although their arguments have different numbers of candidates
+    assert PO.fallback_nodes == [], PO.fallback_reasons
+    ln = next(n for n in gm.graph.nodes if "native_layer_norm.default" in str(n.target))
+    assert len(opt.strats[ln].strategies) > 1
+    assert all(isinstance(s.output_specs, tuple) and len(s.output_specs) == 3 for s in opt.strats[ln].strategies)
     g = opt._packed
     ref = O.GraphOracle(g).build()
     slots = g.entry_slots()
@@ -416,3 +430,145 @@ def test_transformer_block_joint_graph(mesh):
     sol = opt.get_solution()
     assert set(sol) == {n for n in opt.nodes if n.op != "output"}
     assert np.isclose(opt._compute_solution_cost(sol)["total"], opt._core.objective_value, rtol=1e-9)
+
+
+class _WithFactories(nn.Module):
+    """Operators without tensor inputs next to ordinary ones."""
+
+    def __init__(self):
+        super().__init__()
+        self.w = nn.Linear(64, 64, bias=False)
+
+    def forward(self, x):
+        pos = torch.arange(x.shape[1], device=x.device)
+        bias = torch.full((32, 64), 0.5, device=x.device)
+        mask = torch.zeros(16, 32, 64, device=x.device)
+        y = self.w(x) + bias + mask
+        return (y * pos[None, :, None].to(y.dtype)).sum()
+
+
+def test_operators_without_tensor_inputs(mesh):
+    """Factories get the Shard/Replicate product with a stand-in input spec and a
+    zero row as long as the unfiltered product; generators are Replicate only
+    (autoparallel/shardings/propagation_rules.py:412-554).  The coefficients of
+    the whole graph equal the oracle's and the plan solves."""
+    from torch._functorch.aot_autograd import aot_export_joint_with_descriptors
+    from torch._subclasses.fake_tensor import FakeTensorMode
+    from torch.distributed.tensor.placement_types import Replicate
+
+    from autoparallel_amd.optimize_sharding import ShardingOptimizer
+
+    with FakeTensorMode():
+        m, x = _WithFactories(), torch.randn(16, 32, 64)
+        with contextlib.ExitStack() as stack:
+            gm = aot_export_joint_with_descriptors(stack, m, (x,)).graph_module
+    by_op = {}
+    for n in gm.graph.nodes:
+        if n.op == "call_function":
+            by_op.setdefault(str(n.target), n)
+    assert "aten.full.default" in by_op and "aten.zeros.default" in by_op and "aten.arange.default" in by_op
+    opt = ShardingOptimizer(gm, mesh, devices_per_host=8, device_name="AMD Instinct MI355X")
+    full = opt.strats[by_op["aten.full.default"]].strategies
+    # rank 2 on a 2-dim mesh: (2 + 1)^2 combinations, all valid for (32, 64) on (2, 4)
+    assert len(full) == 9 and all(len(s.redistribute_cost[0]) == 9 for s in full)
+    assert all(s.input_specs[0] is s.output_specs for s in full)
+    assert full[-1].output_specs.placements == (Replicate(), Replicate())
+    zeros = opt.strats[by_op["aten.zeros.default"]].strategies
+    assert len(zeros) == 16 and all(len(s.redistribute_cost[0]) == 16 for s in zeros)
+    ar = opt.strats[by_op["aten.arange.default"]].strategies
+    assert len(ar) == 1 and ar[0].output_specs.placements == (Replicate(), Replicate())
+    assert ar[0].redistribute_cost == [[0.0]]
+    g = opt._packed
+    v = opt.node_map[by_op["aten.full.default"]]
+    e = int(g.node_edge_off[v])
+    assert g.node_nargs[v] == 1 and g.edge_src_node[e] < 0 and g.edge_ssrc[e] == 9
+    ref = O.GraphOracle(g).build()
+    slots = g.entry_slots()
+    cost_ref, _ = O.clamp_inf(ref["cost"])
+    assert bits_equal(opt._core.coef.comm, ref["comm"][slots])
+    assert bits_equal(opt._core.coef.cost, cost_ref[slots])
+    assert bits_equal(opt._core.coef.compute, ref["compute"])
+    sol = opt.get_solution()
+    assert set(sol) == {n for n in opt.nodes if n.op != "output"}
+    assert np.isclose(opt._compute_solution_cost(sol)["total"], opt._core.objective_value, rtol=1e-9)
+
+
+def test_hf_gpt2_small_joint_graph():
+    """GPT-2 small as transformers defines it (12 layers, d 768, vocab 50257,
+    random weights), batch 8 x 1024 tokens, forward and backward, on a mesh of 8:
+    every operator gets DTensor strategies, every coefficient equals the
+    oracle's, and the solved plan shards the large matrices."""
+    transformers = pytest.importorskip("transformers")
+    import torch.distributed as dist
+    from torch._functorch.aot_autograd import aot_export_joint_with_descriptors
+    from torch._subclasses.fake_tensor import FakeTensorMode
+    from torch.distributed.device_mesh import init_device_mesh
+    from torch.testing._internal.distributed.fake_pg import FakeStore
+
+    from autoparallel_amd.optimize_sharding import ShardingOptimizer
+    from autoparallel_amd.shardings import placement_options as PO
+
+    if not torch.cuda.is_available():
+        pytest.skip("needs a GPU")
+
+    class Wrap(nn.Module):
+        def __init__(self, lm):
+            super().__init__()
+            self.lm = lm
+
+        def forward(self, ids):
+            t = self.lm.transformer
+            x = t.wte(ids) + t.wpe(torch.arange(ids.shape[1], device=ids.device))[None]
+            for blk in t.h:
+                out = blk(x)
+                x = out[0] if isinstance(out, tuple) else out
+            logits = self.lm.lm_head(t.ln_f(x))
+            return torch.nn.functional.cross_entropy(
+                logits[:, :-1].reshape(-1, logits.shape[-1]).float(), ids[:, 1:].reshape(-1))
+
+    cfg = transformers.GPT2Config(attn_pdrop=0.0, embd_pdrop=0.0, resid_pdrop=0.0, use_cache=False,
+                                  attn_implementation="sdpa")
+    assert (cfg.n_layer, cfg.n_embd, cfg.n_head, cfg.vocab_size) == (12, 768, 12, 50257)
+    with FakeTensorMode():
+        torch.manual_seed(0)
+        with torch.device("cuda"):
+            m = Wrap(transformers.GPT2LMHeadModel(cfg))
+        ids = torch.randint(0, cfg.vocab_size, (8, 1024), device="cuda")
+        with contextlib.ExitStack() as stack:
+            gm = aot_export_joint_with_descriptors(stack, m, (ids,)).graph_module
+    own_pg = not dist.is_initialized()
+    if own_pg:
+        dist.init_process_group("fake", store=FakeStore(), rank=0, world_size=8)
+    try:
+        mesh8 = init_device_mesh("cpu", (8,))
+        PO.fallback_nodes.clear()
+        PO.fallback_reasons.clear()
+        opt = ShardingOptimizer(gm, mesh8, devices_per_host=8, device_name="AMD Instinct MI355X")
+        assert PO.fallback_nodes == [], PO.fallback_reasons
+        g = opt._packed
+        assert g.num_nodes > 1500 and g.num_entries > 15000
+        ref = O.GraphOracle(g).build()
+        slots = g.entry_slots()
+        cost_ref, _ = O.clamp_inf(ref["cost"])
+        assert bits_equal(opt._core.coef.comm, ref["comm"][slots])
+        assert bits_equal(opt._core.coef.cost, cost_ref[slots])
+        assert bits_equal(opt._core.coef.compute, ref["compute"])
+        assert (ref["compute"] > 0).sum() > 300
+        sol = opt.get_solution()
+        # the objective counts a transition on an edge out of a tuple-valued producer
+        # (autoparallel/optimize_sharding.py:470-477, through getitem), the reference's
+        # scorer does not (:1099-1104, pred_spec is a tuple there)
+        import operator
+
+        uncounted = sum(
+            1 for n, st in sol.items()
+            if n.op == "call_function" and n.target is operator.getitem
+            and sol[n.args[0]].output_specs[n.args[1]].placements != st.input_specs[0].placements)
+        assert np.isclose(opt._compute_solution_cost(sol)["total"] + uncounted, opt._core.objective_value, rtol=1e-9)
+        big = [n for n in sol if n.op == "placeholder" and n.meta["val"].ndim == 2
+               and n.meta["val"].numel() in (768 * 3072, 768 * 2304)]
+        assert len(big) == 12 * 3
+        assert all(any(p.is_shard() for p in sol[n].output_specs.placements) for n in big)
+    finally:
+        if own_pg:
+            dist.destroy_process_group()

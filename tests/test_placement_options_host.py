@@ -126,3 +126,96 @@ def test_einsum_flop_and_memory_cost_known_answers():
         einsum_flop("bsk,kn->bsn", (a, torch.empty(15, 32, device="meta")))
     bf = torch.empty(8, 4, dtype=torch.bfloat16, device="meta")
     assert compute_memory_cost(None, (a, [bf, 3]), {"out": b}) == 4 * 8 * 16 * 4 + 8 * 4 * 2 + 16 * 32 * 4
+
+
+def _fx_node(target, args, val, name=None):
+    g = torch.fx.Graph()
+    n = g.call_function(target, args)
+    n.meta["val"] = val
+    if name:
+        n.name = name
+    return n
+
+
+def _candidates(mesh, shape, placements):
+    return OpStrategy([_one(mesh, shape, p) for p in placements])
+
+
+def test_operators_without_tensor_inputs_rules(meshes):
+    """Size-taking factories: every {Shard(d), Replicate} combination, Replicate
+    last per mesh dim, invalid ones dropped, a stand-in input spec that is the
+    output spec, and a zero row as long as the unfiltered product
+    (autoparallel/shardings/propagation_rules.py:486-554).  Generators and
+    scalar_tensor: Replicate only with one zero (:412-421, :453-484)."""
+    from autoparallel_amd.shardings.placement_options import get_placement_options_for_node
+
+    aten = torch.ops.aten
+    mesh = meshes[1]  # (32, 8)
+    val = torch.empty(64, 16, device="meta")
+    node = _fx_node(aten.zeros.default, ([64, 16],), val)
+    out = get_placement_options_for_node(mesh, node, [], [], ([64, 16],))
+    plcs = [s.output_specs.placements for s in out.strategies]
+    # (S0|S1|R)^2 = 9; dim 1 (16) cannot take the mesh dim of 32; 64/32 = 2 cannot take 8 more
+    assert plcs == [(Shard(0), Shard(1)), (Shard(0), Replicate()),
+                    (Replicate(), Shard(0)), (Replicate(), Shard(1)), (Replicate(), Replicate())]
+    assert all(s.input_specs[0] is s.output_specs and s.redistribute_cost == [[0.0] * 9] for s in out.strategies)
+    assert out.strategies[0].output_specs.tensor_meta.shape == (64, 16)
+    for target, args, v in ((aten.arange.default, (128,), torch.empty(128, dtype=torch.int64, device="meta")),
+                            (aten.scalar_tensor.default, (1.0,), torch.empty((), device="meta"))):
+        out = get_placement_options_for_node(mesh, _fx_node(target, args, v), [], [], args)
+        assert len(out.strategies) == 1 and out.strategies[0].redistribute_cost == [[0.0]]
+        assert out.strategies[0].output_specs.placements == (Replicate(), Replicate())
+        assert out.strategies[0].output_specs.tensor_meta.dtype == v.dtype
+
+
+def test_view_is_not_strict(meshes):
+    """A view that splits a sharded dim keeps the strategy with the input demoted
+    (autoparallel/shardings/propagation_rules.py:239-287) where DTensor's own
+    rule refuses the whole operator."""
+    from autoparallel_amd.shardings.placement_options import fallback_nodes, get_placement_options_for_node
+
+    mesh = meshes[0]  # (256,)
+    src = _candidates(mesh, (512, 1024, 768), [(Replicate(),), (Shard(0),), (Shard(2),)])
+    val = torch.empty(512, 1024, 12, 64, device="meta")
+    g = torch.fx.Graph()
+    x = g.placeholder("x")
+    x.meta["val"] = torch.empty(512, 1024, 768, device="meta")
+    node = g.call_function(torch.ops.aten.view.default, (x, [512, 1024, 12, 64]))
+    node.meta["val"] = val
+    before = list(fallback_nodes)
+    out = get_placement_options_for_node(mesh, node, [src], [x.meta["val"]], (src, [512, 1024, 12, 64]))
+    assert fallback_nodes == before
+    got = {(s.input_specs[0].placements, s.output_specs.placements) for s in out.strategies}
+    # 768 -> (12, 64): 12 < 256, so Shard(2) cannot follow; the input is asked to be Replicate
+    assert got == {((Replicate(),), (Replicate(),)), ((Shard(0),), (Shard(0),))}
+    assert all(len(s.redistribute_cost[0]) == 3 for s in out.strategies)
+    assert all(s.output_specs.tensor_meta.shape == (512, 1024, 12, 64) for s in out.strategies)
+
+
+def test_norm_strategies_with_unequal_candidate_counts(meshes):
+    """DTensor's layer-norm functions pair the arguments' strategies by index;
+    with 3 candidates for the input and 2 for weight and bias they are asked one
+    input strategy at a time: one strategy per input placement, weight and bias
+    Replicate, three outputs that follow the input on the outer dims."""
+    from autoparallel_amd.shardings.placement_options import fallback_nodes, get_placement_options_for_node
+
+    mesh = meshes[1]  # (32, 8)
+    x_val = torch.empty(256, 64, 128, device="meta")
+    w_val = torch.empty(128, device="meta")
+    xs = _candidates(mesh, (256, 64, 128), [(Replicate(), Replicate()), (Shard(0), Replicate()),
+                                            (Shard(0), Shard(1)), (Replicate(), Shard(2))])
+    ws = _candidates(mesh, (128,), [(Replicate(), Replicate()), (Replicate(), Shard(0))])
+    g = torch.fx.Graph()
+    x, w, b = g.placeholder("x"), g.placeholder("w"), g.placeholder("b")
+    x.meta["val"], w.meta["val"], b.meta["val"] = x_val, w_val, w_val
+    node = g.call_function(torch.ops.aten.native_layer_norm.default, (x, [128], w, b, 1e-5))
+    node.meta["val"] = (x_val, torch.empty(256, 64, 1, device="meta"), torch.empty(256, 64, 1, device="meta"))
+    before = list(fallback_nodes)
+    out = get_placement_options_for_node(mesh, node, [xs, ws, ws], [x_val, w_val, w_val], (xs, [128], ws, ws, 1e-5))
+    assert fallback_nodes == before
+    got = [(tuple(s.placements for s in st.input_specs), tuple(s.placements for s in st.output_specs))
+           for st in out.strategies]
+    rr = (Replicate(), Replicate())
+    assert got == [((p, rr, rr), (p, p, p)) for p in (rr, (Shard(0), Replicate()), (Shard(0), Shard(1)))]
+    assert [len(r) for r in out.strategies[0].redistribute_cost] == [4, 2, 2]
+    assert out.strategies[0].output_specs[1].tensor_meta.shape == (256, 64, 1)
