@@ -46,6 +46,100 @@ class Row:
         return lhs >= self.rhs - tol
 
 
+class _Block:
+    """Rows added together, as CSR: names ``{prefix}_{first + i:03}`` (or one exact
+    name), one sense, a rhs and a liveness flag per row."""
+
+    __slots__ = ("prefix", "first", "exact", "indptr", "idx", "coef", "sense", "rhs", "alive", "n_alive")
+
+    def __init__(self, prefix, first, exact, indptr, idx, coef, sense, rhs):
+        self.prefix, self.first, self.exact = prefix, first, exact
+        self.indptr, self.idx, self.coef, self.sense, self.rhs = indptr, idx, coef, sense, rhs
+        self.alive = np.ones(rhs.shape[0], bool)
+        self.n_alive = int(rhs.shape[0])
+
+    def name(self, i: int) -> str:
+        return self.exact if self.exact is not None else f"{self.prefix}_{self.first + i:03}"
+
+    def row(self, i: int) -> Row:
+        a, b = self.indptr[i], self.indptr[i + 1]
+        return Row(self.name(i), self.idx[a:b], self.coef[a:b], self.sense, self.rhs[i])
+
+
+class _Rows:
+    """The model's rows as an ordered name -> Row mapping (insertion order) over
+    the blocks; Row objects are made on access."""
+
+    def __init__(self):
+        self.blocks: List[_Block] = []
+        self.by_prefix: Dict[str, List[_Block]] = {}
+        self.exact: Dict[str, _Block] = {}
+
+    def _find(self, name: str) -> Optional[Tuple[_Block, int]]:
+        b = self.exact.get(name)
+        if b is not None:
+            return (b, 0) if b.alive[0] else None
+        prefix, _, num = name.rpartition("_")
+        if not num.isdigit() or name != f"{prefix}_{int(num):03}":
+            return None
+        k = int(num)
+        for b in self.by_prefix.get(prefix, ()):
+            if b.first <= k < b.first + b.rhs.shape[0]:
+                return (b, k - b.first) if b.alive[k - b.first] else None
+        return None
+
+    def __contains__(self, name) -> bool:
+        return self._find(name) is not None
+
+    def __getitem__(self, name) -> Row:
+        hit = self._find(name)
+        if hit is None:
+            raise KeyError(name)
+        return hit[0].row(hit[1])
+
+    def __delitem__(self, name) -> None:
+        hit = self._find(name)
+        if hit is None:
+            raise KeyError(name)
+        b, i = hit
+        b.alive[i] = False
+        b.n_alive -= 1
+        if b.exact is not None:
+            del self.exact[name]
+
+    def pop(self, name, default=None):
+        hit = self._find(name)
+        if hit is None:
+            return default
+        row = hit[0].row(hit[1])
+        del self[name]
+        return row
+
+    def __len__(self) -> int:
+        return sum(b.n_alive for b in self.blocks)
+
+    def items(self):
+        for b in self.blocks:
+            if b.n_alive == 0:
+                continue
+            for i in (range(b.rhs.shape[0]) if b.n_alive == b.rhs.shape[0] else np.nonzero(b.alive)[0]):
+                r = b.row(int(i))
+                yield r.name, r
+
+    def __iter__(self):
+        for b in self.blocks:
+            if b.n_alive == 0:
+                continue
+            for i in (range(b.rhs.shape[0]) if b.n_alive == b.rhs.shape[0] else np.nonzero(b.alive)[0]):
+                yield b.name(int(i))
+
+    keys = __iter__
+
+    def values(self):
+        for _, r in self.items():
+            yield r
+
+
 class SparseILP:
     """Minimise c.x over binary x subject to named rows."""
 
@@ -53,7 +147,7 @@ class SparseILP:
         self.n_vars = int(n_vars)
         self.objective = np.zeros(self.n_vars, np.float64)
         self.upper = np.ones(self.n_vars, np.float64)  # 0 fixes a variable out of the model
-        self.constraints: "collections.OrderedDict[str, Row]" = collections.OrderedDict()
+        self.constraints = _Rows()
         self._counters: Dict[str, int] = {}
         self.status = STATUS_NOT_SOLVED
         self.x: Optional[np.ndarray] = None
@@ -66,15 +160,40 @@ class SparseILP:
         return f"{prefix}_{i:03}"
 
     # -- rows -----------------------------------------------------------------
-    def add_row(self, prefix_or_name: str, idx, coef, sense: int, rhs: float, exact_name: bool = False) -> str:
-        name = prefix_or_name if exact_name else self.next_name(prefix_or_name)
-        idx = np.asarray(idx, np.int64)
-        if np.isscalar(coef):
-            coef = np.full(idx.shape[0], float(coef))
-        assert idx.shape[0] == len(coef)
+    def add_rows(self, prefix: str, indptr, idx, coef, sense: int, rhs) -> List[str]:
+        """A block of rows at once: row i has variables ``idx[indptr[i]:indptr[i+1]]``
+        with coefficients ``coef`` (an array as long as idx, or one value) and
+        right-hand side ``rhs`` (an array or one value).  Names continue the
+        prefix's counter.  Returns the names."""
+        indptr = np.ascontiguousarray(indptr, np.int64)
+        idx = np.ascontiguousarray(idx, np.int64)
+        n = indptr.shape[0] - 1
+        if n <= 0:
+            return []
+        coef = np.full(idx.shape[0], float(coef)) if np.isscalar(coef) else np.ascontiguousarray(coef, np.float64)
+        rhs = np.full(n, float(rhs)) if np.isscalar(rhs) else np.ascontiguousarray(rhs, np.float64)
+        assert indptr[0] == 0 and indptr[-1] == idx.shape[0] == coef.shape[0] and (np.diff(indptr) >= 0).all()
         assert idx.size == 0 or (0 <= idx.min() and idx.max() < self.n_vars)
-        self.constraints[name] = Row(name, idx, coef, sense, rhs)
-        return name
+        first = self._counters.get(prefix, 0)
+        self._counters[prefix] = first + n
+        b = _Block(prefix, first, None, indptr, idx, coef, sense, rhs)
+        self.constraints.blocks.append(b)
+        self.constraints.by_prefix.setdefault(prefix, []).append(b)
+        return [b.name(i) for i in range(n)]
+
+    def add_row(self, prefix_or_name: str, idx, coef, sense: int, rhs: float, exact_name: bool = False) -> str:
+        idx = np.asarray(idx, np.int64)
+        if not exact_name:
+            return self.add_rows(prefix_or_name, [0, idx.shape[0]], idx, coef, sense, rhs)[0]
+        coef = np.full(idx.shape[0], float(coef)) if np.isscalar(coef) else np.asarray(coef, np.float64)
+        assert idx.shape[0] == coef.shape[0]
+        assert idx.size == 0 or (0 <= idx.min() and idx.max() < self.n_vars)
+        self.constraints.pop(prefix_or_name, None)  # an exact name replaces its row
+        b = _Block(None, 0, prefix_or_name, np.asarray([0, idx.shape[0]], np.int64), idx, coef, sense,
+                   np.asarray([float(rhs)]))
+        self.constraints.blocks.append(b)
+        self.constraints.exact[prefix_or_name] = b
+        return prefix_or_name
 
     def remove(self, name: str) -> None:
         del self.constraints[name]
@@ -86,27 +205,36 @@ class SparseILP:
         import scipy.sparse as sp
 
         ub = self.upper.copy()
-        data, cols, ptr, lo, hi = [], [], [0], [], []
-        for r in self.constraints.values():
-            if r.sense == EQ and r.rhs == 0.0 and r.idx.shape[0] == 1 and r.coef[0] != 0:
-                ub[r.idx[0]] = 0.0
+        data, cols, lens, lo, hi = [], [], [], [], []
+        for b in self.constraints.blocks:
+            if b.n_alive == 0:
                 continue
-            data.append(r.coef)
-            cols.append(r.idx)
-            ptr.append(ptr[-1] + r.idx.shape[0])
-            if r.sense == EQ:
-                lo.append(r.rhs); hi.append(r.rhs)
-            elif r.sense == LE:
-                lo.append(-np.inf); hi.append(r.rhs)
+            ln = np.diff(b.indptr)
+            keep = b.alive.copy()
+            if b.sense == EQ:
+                # a single variable pinned to zero is a bound, not a row
+                pin = keep & (ln == 1) & (b.rhs == 0.0)
+                if pin.any():
+                    at = b.indptr[:-1][pin]
+                    pin[pin] = b.coef[at] != 0
+                    ub[b.idx[b.indptr[:-1][pin]]] = 0.0
+                    keep &= ~pin
+            if not keep.any():
+                continue
+            if keep.all():
+                data.append(b.coef); cols.append(b.idx); lens.append(ln)
             else:
-                lo.append(r.rhs); hi.append(np.inf)
-        n_rows = len(lo)
-        A = sp.csr_matrix(
-            (np.concatenate(data) if data else np.zeros(0), np.concatenate(cols) if cols else np.zeros(0, np.int64),
-             np.asarray(ptr, np.int64)),
-            shape=(n_rows, self.n_vars),
-        )
-        return A, np.asarray(lo), np.asarray(hi), ub
+                ent = np.repeat(keep, ln)
+                data.append(b.coef[ent]); cols.append(b.idx[ent]); lens.append(ln[keep])
+            r = b.rhs[keep]
+            lo.append(r if b.sense != LE else np.full(r.shape[0], -np.inf))
+            hi.append(r if b.sense != GE else np.full(r.shape[0], np.inf))
+        cat = lambda xs, dt: np.concatenate(xs) if xs else np.zeros(0, dt)
+        lens = cat(lens, np.int64)
+        ptr = np.zeros(lens.shape[0] + 1, np.int64)
+        np.cumsum(lens, out=ptr[1:])
+        A = sp.csr_matrix((cat(data, np.float64), cat(cols, np.int64), ptr), shape=(lens.shape[0], self.n_vars))
+        return A, cat(lo, np.float64), cat(hi, np.float64), ub
 
     # -- solve ------------------------------------------------------------------
     def solve(self, backend: str = "auto", time_limit: Optional[float] = None, verbose: bool = False) -> int:

@@ -204,13 +204,38 @@ class PackedShardingOptimizer:
         self.add_forward_backward_consistency_constraints()
         self.add_grad_reduce_dtype_constraints()
 
+    @staticmethod
+    def _segments(start, count, stride=None):
+        """Concatenation of start[k] + stride[k] * arange(count[k]) over k, and
+        the offsets of the pieces."""
+        start = np.asarray(start, np.int64)
+        count = np.asarray(count, np.int64)
+        ptr = np.zeros(count.shape[0] + 1, np.int64)
+        np.cumsum(count, out=ptr[1:])
+        seg = np.repeat(np.arange(count.shape[0], dtype=np.int64), count)
+        local = np.arange(int(ptr[-1]), dtype=np.int64) - ptr[:-1][seg]
+        if stride is not None:
+            local = local * np.asarray(stride, np.int64)[seg]
+        return start[seg] + local, ptr
+
+    def _add_difference_rows(self, prefix, plus_start, plus_count, minus_start, minus_count, minus_stride) -> None:
+        """Rows  sum(plus piece) - sum(minus piece) = 0, one per pair of pieces."""
+        n = len(plus_start)
+        if n == 0:
+            return
+        start = np.empty(2 * n, np.int64); start[0::2] = plus_start; start[1::2] = minus_start
+        count = np.empty(2 * n, np.int64); count[0::2] = plus_count; count[1::2] = minus_count
+        stride = np.ones(2 * n, np.int64); stride[1::2] = minus_stride
+        idx, ptr = self._segments(start, count, stride)
+        sign = np.ones(2 * n); sign[1::2] = -1.0
+        self.prob.add_rows(prefix, ptr[0::2], idx, np.repeat(sign, count), ilp.EQ, 0.0)
+
     def add_unique_decision_constraint(self) -> None:
         # for every (node, arg): exactly one (out, inp) pair
-        for e in range(self.g.num_edges):
-            if self.linked[self.g.edge_node[e]]:
-                continue
-            idx = np.arange(self.var_start[e], self.var_start[e + 1], dtype=np.int64)
-            self.prob.add_row("unique_decision", idx, 1.0, ilp.EQ, 1.0)
+        g = self.g
+        e = np.nonzero(~self.linked[g.edge_node])[0]
+        idx, ptr = self._segments(self.var_start[e], self.var_start[e + 1] - self.var_start[e])
+        self.prob.add_rows("unique_decision", ptr, idx, 1.0, ilp.EQ, 1.0)
 
     def _num_input_nodes(self, v: int) -> int:
         g = self.g
@@ -218,50 +243,55 @@ class PackedShardingOptimizer:
         return int((g.edge_src_node[e0:e1] >= 0).sum())
 
     def add_same_output_across_args_constraint(self) -> None:
-        # all arguments of a node pick the same output strategy
+        # all arguments of a node pick the same output strategy: for every later
+        # argument e and output strategy o, row o of argument 0 minus row o of e
         g = self.g
-        for v in range(g.num_nodes):
-            if self.linked[v] or self._num_input_nodes(v) <= 1:
-                continue
-            e0, e1 = int(g.node_edge_off[v]), int(g.node_edge_off[v + 1])
-            for e in range(e0 + 1, e1):
-                for o in range(int(g.node_nstrat[v])):
-                    a0, ak = self._row_vars(e0, o), self._row_vars(e, o)
-                    self.prob.add_row(
-                        "same_across_args", np.concatenate([a0, ak]),
-                        np.concatenate([np.ones(len(a0)), -np.ones(len(ak))]), ilp.EQ, 0.0)
+        first = g.node_edge_off[:-1].astype(np.int64)
+        n_in = np.add.reduceat(np.concatenate([(g.edge_src_node >= 0).astype(np.int64), [0]]),
+                               np.minimum(first, g.num_edges))[: g.num_nodes]
+        n_in[np.diff(g.node_edge_off) == 0] = 0
+        v = g.edge_node.astype(np.int64)
+        later = np.nonzero((np.arange(g.num_edges) != first[v]) & ~self.linked[v] & (n_in[v] > 1))[0]
+        if later.size == 0:
+            return
+        S = g.node_nstrat[v[later]].astype(np.int64)
+        e = np.repeat(later, S)
+        o = np.arange(int(S.sum()), dtype=np.int64) - np.repeat(np.cumsum(S) - S, S)
+        e0 = self.edge_alias[first[v[e]]]
+        ek = self.edge_alias[e]
+        s0, sk = g.edge_ssrc[e0].astype(np.int64), g.edge_ssrc[ek].astype(np.int64)
+        self._add_difference_rows("same_across_args", self.var_start[e0] + o * s0, s0,
+                                  self.var_start[ek] + o * sk, sk, np.ones_like(sk))
 
     def add_output_input_consistent_constraint(self) -> None:
-        # producer's chosen output strategy == the input strategy its consumer assumes
+        # producer's chosen output strategy == the input strategy its consumer assumes:
+        # for the first edge of every (producer u, consumer v) pair and every strategy k
+        # of u, row k of u's argument 0 minus column k of the edge; producers in order
         g = self.g
-        seen = set()
-        users: Dict[int, List[Tuple[int, int]]] = {}
-        for e in range(g.num_edges):
-            u = int(g.edge_src_node[e])
-            if u < 0:
-                continue
-            v = int(g.edge_node[e])
-            if self.linked[u] and self.linked[v]:  # the root-to-root edge covers it
-                continue
-            if (u, v) in seen:  # first matching argument only
-                continue
-            seen.add((u, v))
-            users.setdefault(u, []).append((v, e))
-        for u in sorted(users):
-            eu = int(g.node_edge_off[u])  # argument 0 of the producer
-            for v, e in users[u]:
-                assert int(g.edge_ssrc[e]) == int(g.node_nstrat[u])
-                for k in range(int(g.node_nstrat[u])):
-                    pu, cv = self._row_vars(eu, k), self._col_vars(e, k)
-                    self.prob.add_row(
-                        "output_input_consistent", np.concatenate([pu, cv]),
-                        np.concatenate([np.ones(len(pu)), -np.ones(len(cv))]), ilp.EQ, 0.0)
+        u = g.edge_src_node.astype(np.int64)
+        v = g.edge_node.astype(np.int64)
+        has = np.nonzero(u >= 0)[0]
+        has = has[~(self.linked[u[has]] & self.linked[v[has]])]  # the root-to-root edge covers those
+        if has.size == 0:
+            return
+        _, firsts = np.unique(u[has] * g.num_nodes + v[has], return_index=True)  # first matching argument only
+        edges = has[np.sort(firsts)]
+        edges = edges[np.argsort(u[edges], kind="stable")]
+        assert (g.edge_ssrc[edges] == g.node_nstrat[u[edges]]).all()
+        S = g.node_nstrat[u[edges]].astype(np.int64)
+        e = np.repeat(edges, S)
+        k = np.arange(int(S.sum()), dtype=np.int64) - np.repeat(np.cumsum(S) - S, S)
+        eu = self.edge_alias[g.node_edge_off[u[e]].astype(np.int64)]  # argument 0 of the producer
+        ev = self.edge_alias[e]
+        su, sv = g.edge_ssrc[eu].astype(np.int64), g.edge_ssrc[ev].astype(np.int64)
+        self._add_difference_rows("output_input_consistent", self.var_start[eu] + k * su, su,
+                                  self.var_start[ev] + k, g.edge_sdst[ev].astype(np.int64), sv)
 
     def add_inf_cost_constraint(self) -> None:
         # the engine already wrote 10000.0 into cost; pin those variables to 0
-        for i in np.nonzero((self.coef.flags & 2) != 0)[0]:
-            if self.prob.upper[i] > 0:  # linked nodes have no variables of their own
-                self.prob.add_row("inf_cases", [i], 1.0, ilp.EQ, 0.0)
+        # (linked nodes have no variables of their own)
+        i = np.nonzero(((self.coef.flags & 2) != 0) & (self.prob.upper > 0))[0]
+        self.prob.add_rows("inf_cases", np.arange(i.shape[0] + 1), i, 1.0, ilp.EQ, 0.0)
 
     def _out_placements(self, v: int) -> List[Optional[int]]:
         """Placement-tuple id of output 0 of each strategy of node v (None for
@@ -304,8 +334,8 @@ class PackedShardingOptimizer:
             if not enabled or not nodes:
                 continue
             mask = np.isin(keys[:, 0], np.fromiter(nodes, np.int64)) & comm_pos & (self.prob.upper > 0)
-            for i in np.nonzero(mask)[0]:
-                self.prob.add_row(name, [i], 1.0, ilp.EQ, 0.0)
+            i = np.nonzero(mask)[0]
+            self.prob.add_rows(name, np.arange(i.shape[0] + 1), i, 1.0, ilp.EQ, 0.0)
 
     # -- user constraints -----------------------------------------------------------
     def add_node_constraint(self, v: int, placement: Optional[Sequence[int]] = None,

@@ -343,11 +343,68 @@ _INDEX_PAIRED = {getattr(getattr(aten, name), "default") for name in (
 _FOLLOW = {aten.alias.default, aten.detach.default}
 
 
+def _fingerprint(x):
+    """Hashable summary of one argument of a strategy query."""
+    if isinstance(x, OpStrategy):
+        return ("S",) + tuple(_fingerprint(st.output_specs) for st in x.strategies)
+    if isinstance(x, DTensorSpec):
+        return (x.placements, x.tensor_meta)
+    if isinstance(x, torch.Tensor):
+        return ("T", tuple(x.shape), tuple(x.stride()), x.dtype)
+    if isinstance(x, (list, tuple)):
+        return tuple(_fingerprint(y) for y in x)
+    if isinstance(x, dict):
+        return tuple((k, _fingerprint(v)) for k, v in x.items())
+    return x
+
+
+def _copy_strategy(src: OpStrategy) -> OpStrategy:
+    """New OpSpec wrappers and cost rows (both are written per node); the specs are shared."""
+    return OpStrategy([OpSpec(st.output_specs, input_specs=st.input_specs,
+                              redistribute_cost=[list(r) for r in st.redistribute_cost]) for st in src.strategies])
+
+
+# strategies by query, as the reference keeps them
+# (autoparallel/shardings/placement_options.py:183-217, 279-302): the layers of a
+# model repeat the same queries, and one answer from the propagator costs
+# milliseconds.  Values: (strategies, why the all-Replicate stand-in was used or None).
+_strategy_cache: Dict[tuple, tuple] = {}
+strategy_cache_stats = {"hits": 0, "misses": 0}
+
+
+def reset_placement_options_cache() -> None:
+    _strategy_cache.clear()
+    strategy_cache_stats.update(hits=0, misses=0)
+
+
 def get_placement_options_for_node(mesh, node, producers: List[OpStrategy], arg_vals: List[torch.Tensor],
                                    schema_args) -> OpStrategy:
     """Strategies of one call_function node.  ``producers``: OpStrategy of
     each tensor input node in flattened-args order; ``schema_args``: node.args
     with nodes replaced by their OpStrategy (or value for non-tensors)."""
+    try:
+        key = (id(mesh), tuple(mesh.shape), node.target, _fingerprint(schema_args),
+               _fingerprint({k: v for k, v in node.kwargs.items() if not isinstance(v, torch.fx.Node)}),
+               _fingerprint(node.meta.get("val")), _fingerprint(arg_vals))
+        hit = _strategy_cache.get(key)
+    except TypeError:  # something unhashable (a SymInt, ...) in the query
+        key = hit = None
+    if hit is not None:
+        strategy_cache_stats["hits"] += 1
+        if hit[1] is not None:
+            fallback_nodes.append(str(node.name))
+            fallback_reasons[str(node.name)] = hit[1]
+        return _copy_strategy(hit[0])
+    strategy_cache_stats["misses"] += 1
+    n_fallback = len(fallback_nodes)
+    out = _placement_options_uncached(mesh, node, producers, arg_vals, schema_args)
+    if key is not None:
+        why = fallback_reasons.get(str(node.name), "") if len(fallback_nodes) > n_fallback else None
+        _strategy_cache[key] = (_copy_strategy(out), why)
+    return out
+
+
+def _placement_options_uncached(mesh, node, producers, arg_vals, schema_args) -> OpStrategy:
     prop = DTensor._op_dispatcher.sharding_propagator
     op = node.target
     if not producers and isinstance(node.meta.get("val"), torch.Tensor):

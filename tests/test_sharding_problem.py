@@ -212,3 +212,107 @@ def test_violated_constraints_log(tiny):
     names = opt.var_names()
     assert f"{names[first]}, coeff=1.0, value=0.0" in rest
     opt.prob.x[first] = 1.0
+
+
+def _rows_one_at_a_time(opt):
+    """The default rows written as the reference's loops write them
+    (autoparallel/optimize_sharding.py:665-801), one row per iteration: what the
+    block builders must reproduce, names and order included."""
+    g = opt.g
+    rows = []
+    count = {}
+
+    def add(prefix, idx, coef, rhs):
+        k = count.get(prefix, 0)
+        count[prefix] = k + 1
+        rows.append((f"{prefix}_{k:03}", [int(i) for i in idx], [float(c) for c in coef], ilp.EQ, float(rhs)))
+
+    def row_vars(e, o):
+        e = int(opt.edge_alias[e])
+        s = int(g.edge_ssrc[e])
+        b = int(opt.var_start[e]) + o * s
+        return list(range(b, b + s))
+
+    def col_vars(e, j):
+        e = int(opt.edge_alias[e])
+        s = int(g.edge_ssrc[e])
+        return [int(opt.var_start[e]) + o * s + j for o in range(int(g.edge_sdst[e]))]
+
+    for e in range(g.num_edges):
+        if not opt.linked[g.edge_node[e]]:
+            idx = range(int(opt.var_start[e]), int(opt.var_start[e + 1]))
+            add("unique_decision", idx, [1.0] * len(idx), 1.0)
+    for v in range(g.num_nodes):
+        e0, e1 = int(g.node_edge_off[v]), int(g.node_edge_off[v + 1])
+        if opt.linked[v] or int((g.edge_src_node[e0:e1] >= 0).sum()) <= 1:
+            continue
+        for e in range(e0 + 1, e1):
+            for o in range(int(g.node_nstrat[v])):
+                a0, ak = row_vars(e0, o), row_vars(e, o)
+                add("same_across_args", a0 + ak, [1.0] * len(a0) + [-1.0] * len(ak), 0.0)
+    seen, users = set(), {}
+    for e in range(g.num_edges):
+        u, v = int(g.edge_src_node[e]), int(g.edge_node[e])
+        if u < 0 or (opt.linked[u] and opt.linked[v]) or (u, v) in seen:
+            continue
+        seen.add((u, v))
+        users.setdefault(u, []).append(e)
+    for u in sorted(users):
+        eu = int(g.node_edge_off[u])
+        for e in users[u]:
+            for k in range(int(g.node_nstrat[u])):
+                pu, cv = row_vars(eu, k), col_vars(e, k)
+                add("output_input_consistent", pu + cv, [1.0] * len(pu) + [-1.0] * len(cv), 0.0)
+    for i in np.nonzero((opt.coef.flags & 2) != 0)[0]:
+        if opt.prob.upper[i] > 0:
+            add("inf_cases", [i], [1.0], 0.0)
+    return rows
+
+
+@pytest.mark.parametrize("clustered", [False, True])
+def test_block_rows_equal_the_loops(tiny, clustered):
+    g, coef, _ = tiny
+    root = None
+    if clustered:  # link every third node to an earlier node of the same shape
+        root, first = np.arange(g.num_nodes), {}
+        for v in range(g.num_nodes):
+            e0, e1 = int(g.node_edge_off[v]), int(g.node_edge_off[v + 1])
+            key = (int(g.node_nstrat[v]), tuple(g.edge_ssrc[e0:e1].tolist()), tuple(g.edge_sdst[e0:e1].tolist()))
+            if key in first and v % 3 == 0:
+                root[v] = first[key]
+            first.setdefault(key, v)
+        assert (root != np.arange(g.num_nodes)).sum() > 5
+    opt = PackedShardingOptimizer(g, coefficients=coef, cluster_root=root)
+    want = _rows_one_at_a_time(opt)
+    got = [(n, r.idx.tolist(), r.coef.tolist(), r.sense, r.rhs) for n, r in opt.prob.constraints.items()]
+    assert got[: len(want)] == want
+    assert all(n.rsplit("_", 1)[0] not in ("unique_decision", "same_across_args", "output_input_consistent",
+                                            "inf_cases") for n, *_ in got[len(want):])
+
+
+def test_row_container():
+    """Rows live in blocks; the mapping view finds, removes and replaces them by name."""
+    p = ilp.SparseILP(6)
+    names = p.add_rows("pair", [0, 2, 4, 6], [0, 1, 2, 3, 4, 5], 1.0, ilp.LE, [1.0, 2.0, 3.0])
+    assert names == ["pair_000", "pair_001", "pair_002"] and p.add_row("pair", [0], 1.0, ilp.GE, 0.0) == "pair_003"
+    p.add_row("cap", [0, 5], [2.0, 3.0], ilp.LE, 4.0, exact_name=True)
+    p.add_rows("pin", [0, 1, 2], [1, 4], 1.0, ilp.EQ, 0.0)
+    assert list(p.constraints) == ["pair_000", "pair_001", "pair_002", "pair_003", "cap", "pin_000", "pin_001"]
+    assert len(p.constraints) == 7 and "pair_001" in p.constraints and "pair_004" not in p.constraints
+    assert "pair_1" not in p.constraints and "nothing" not in p.constraints
+    r = p.constraints["pair_001"]
+    assert (r.name, r.idx.tolist(), r.coef.tolist(), r.sense, r.rhs) == ("pair_001", [2, 3], [1.0, 1.0], ilp.LE, 2.0)
+    p.remove("pair_001")
+    assert "pair_001" not in p.constraints and len(p.constraints) == 6
+    with pytest.raises(KeyError):
+        p.remove("pair_001")
+    assert p.constraints.pop("pair_001", None) is None and p.constraints.pop("cap").rhs == 4.0
+    p.add_row("cap", [1], 1.0, ilp.LE, 1.0, exact_name=True)
+    p.add_row("cap", [2], 1.0, ilp.LE, 1.0, exact_name=True)  # replaces
+    assert [n for n in p.constraints].count("cap") == 1 and p.constraints["cap"].idx.tolist() == [2]
+    A, lo, hi, ub = p.to_matrix()
+    # pins become bounds; the rest in insertion order
+    assert ub.tolist() == [1, 0, 1, 1, 0, 1] and A.shape == (4, 6)
+    assert A.toarray().tolist() == [[1, 1, 0, 0, 0, 0], [0, 0, 0, 0, 1, 1], [1, 0, 0, 0, 0, 0], [0, 0, 1, 0, 0, 0]]
+    assert lo.tolist() == [-np.inf, -np.inf, 0.0, -np.inf] and hi.tolist() == [1.0, 3.0, np.inf, 1.0]
+    assert p.next_name("pair") == "pair_004"
