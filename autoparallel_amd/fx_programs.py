@@ -165,26 +165,29 @@ def _flops_bytes_via_torch(node, strategies) -> Tuple[List[int], List[int]]:
     return flops_all, bytes_all
 
 
-def describe_node(node, strategies, b: GraphBuilder, name: Optional[str] = None) -> NodeDesc:
-    """NodeDesc (without producers) of an FX node with the given OpSpecs."""
+def describe_node(node, strategies, b: GraphBuilder, name: Optional[str] = None,
+                  memo: Optional[dict] = None) -> NodeDesc:
+    """NodeDesc (without producers) of an FX node with the given OpSpecs.
+    ``memo``: a dict kept by the caller over the nodes of one graph (whose specs
+    stay alive meanwhile): spec words by spec object, explicit flop/byte counts
+    by (operator, spec words, other arguments), so that the repeated layers of a
+    model are converted once."""
+    words = memo.setdefault("words", {}) if memo is not None else {}
+
+    def word(s) -> int:
+        if s is None or s.tensor_meta is None:
+            return -1
+        w = words.get(id(s))
+        if w is None:
+            w = b.spec(b.meta(*tensor_meta_key(s.tensor_meta)), placement_codes(s.placements))
+            words[id(s)] = w
+        return w
+
     in_specs, out_specs = [], []
     for st in strategies:
-        row = []
-        for s in (st.input_specs or []):
-            if s is None or s.tensor_meta is None:
-                row.append(-1)
-            else:
-                row.append(b.spec(b.meta(*tensor_meta_key(s.tensor_meta)), placement_codes(s.placements)))
-        in_specs.append(row)
+        in_specs.append([word(s) for s in (st.input_specs or [])])
         outs = st.output_specs
-        outs = list(outs) if isinstance(outs, (tuple, list)) else [outs]
-        orow = []
-        for s in outs:
-            if s is None or s.tensor_meta is None:
-                orow.append(-1)
-            else:
-                orow.append(b.spec(b.meta(*tensor_meta_key(s.tensor_meta)), placement_codes(s.placements)))
-        out_specs.append(orow)
+        out_specs.append([word(s) for s in (outs if isinstance(outs, (tuple, list)) else [outs])])
     tuple_output = isinstance(strategies[0].output_specs, (tuple, list))
     desc = NodeDesc(name or str(node.name), in_specs=in_specs, out_specs=out_specs, inputs=[],
                     tuple_output=tuple_output)
@@ -206,5 +209,20 @@ def describe_node(node, strategies, b: GraphBuilder, name: Optional[str] = None)
         return desc
     fallback_ops[str(node.target)] += 1
     desc.op = OP_EXPLICIT
+    key = None
+    if memo is not None:
+        try:
+            others = tuple(repr(a) if not isinstance(a, torch.fx.Node) else
+                           ("T", tuple(a.meta["val"].shape), a.meta["val"].dtype) if isinstance(a.meta.get("val"), torch.Tensor)
+                           else ("N",) for a in tree_flatten((node.args, node.kwargs))[0])
+            key = (node.target, tuple(map(tuple, in_specs)), others)
+            hit = memo.setdefault("explicit", {}).get(key)
+            if hit is not None:
+                desc.flops, desc.nbytes = list(hit[0]), list(hit[1])
+                return desc
+        except Exception:
+            key = None
     desc.flops, desc.nbytes = _flops_bytes_via_torch(node, strategies)
+    if key is not None:
+        memo["explicit"][key] = (list(desc.flops), list(desc.nbytes))
     return desc

@@ -236,11 +236,12 @@ class ShardingOptimizer:
         b = GraphBuilder(tuple(self.mesh.shape), self._devices_per_host)
         index_of: Dict[torch.fx.Node, int] = {}
         self._packed_index: Dict[int, int] = {}  # node_idx -> packed node
+        memo: Dict[str, dict] = {}
         for node in self.nodes:
             if node.op == "output":
                 continue
             st: OpStrategy = self.strats[node]
-            desc = fx_programs.describe_node(node, st.strategies, b, name=node.name)
+            desc = fx_programs.describe_node(node, st.strategies, b, name=node.name, memo=memo)
             ins = self._all_input_nodes(node)
             desc.inputs = [index_of[x] for x in ins]
             if node.op == "call_function" and node.target is operator.getitem:

@@ -572,3 +572,88 @@ def test_hf_gpt2_small_joint_graph():
     finally:
         if own_pg:
             dist.destroy_process_group()
+
+
+def test_hf_llama3_8b_layers_joint_graph():
+    """Llama-3-8B as transformers defines it (d 4096, 32 query / 8 key-value heads,
+    SwiGLU 14336, RMSNorm, rotary embedding, vocab 128256, bf16), four of its
+    layers, batch 64 x 8192 tokens, forward and backward, on an (8, 8) mesh:
+    every operator gets DTensor strategies (the layers after the first from the
+    query cache), and every coefficient equals the oracle's."""
+    transformers = pytest.importorskip("transformers")
+    import torch.distributed as dist
+    from torch._functorch.aot_autograd import aot_export_joint_with_descriptors
+    from torch._subclasses.fake_tensor import FakeTensorMode
+    from torch.distributed.device_mesh import init_device_mesh
+    from torch.testing._internal.distributed.fake_pg import FakeStore
+
+    from autoparallel_amd.optimize_sharding import ShardingOptimizer
+    from autoparallel_amd.shardings import placement_options as PO
+
+    if not torch.cuda.is_available():
+        pytest.skip("needs a GPU")
+
+    class Wrap(nn.Module):
+        def __init__(self, lm):
+            super().__init__()
+            self.lm = lm
+
+        def forward(self, ids):
+            m = self.lm.model
+            x = m.embed_tokens(ids)
+            pos = torch.arange(ids.shape[1], device=ids.device)[None]
+            pe = m.rotary_emb(x, pos)
+            for layer in m.layers:
+                out = layer(x, attention_mask=None, position_ids=pos, position_embeddings=pe)
+                x = out[0] if isinstance(out, tuple) else out
+            logits = self.lm.lm_head(m.norm(x))
+            return torch.nn.functional.cross_entropy(
+                logits[:, :-1].reshape(-1, logits.shape[-1]).float(), ids[:, 1:].reshape(-1))
+
+    cfg = transformers.LlamaConfig(
+        vocab_size=128256, hidden_size=4096, intermediate_size=14336, num_hidden_layers=4, num_attention_heads=32,
+        num_key_value_heads=8, max_position_embeddings=8192, rope_theta=500000.0, attention_dropout=0.0,
+        use_cache=False, attn_implementation="sdpa")
+    with FakeTensorMode():
+        torch.manual_seed(0)
+        torch.set_default_dtype(torch.bfloat16)
+        try:
+            with torch.device("cuda"):
+                m = Wrap(transformers.LlamaForCausalLM(cfg))
+        finally:
+            torch.set_default_dtype(torch.float32)
+        ids = torch.randint(0, cfg.vocab_size, (64, 8192), device="cuda")
+        with contextlib.ExitStack() as stack:
+            gm = aot_export_joint_with_descriptors(stack, m, (ids,)).graph_module
+    ops = {str(n.target) for n in gm.graph.nodes if n.op == "call_function"}
+    assert any("scaled_dot_product" in o for o in ops) and "aten.silu.default" in ops and "aten.rsqrt.default" in ops
+    had_pg = dist.is_initialized()
+    if had_pg:  # the module's 8-rank fake group: this mesh needs 64
+        dist.destroy_process_group()
+    dist.init_process_group("fake", store=FakeStore(), rank=0, world_size=64)
+    try:
+        mesh88 = init_device_mesh("cpu", (8, 8))
+        PO.fallback_nodes.clear()
+        PO.fallback_reasons.clear()
+        PO.reset_placement_options_cache()
+        opt = ShardingOptimizer(gm, mesh88, devices_per_host=8, device_name="AMD Instinct MI355X")
+        assert PO.fallback_nodes == [], PO.fallback_reasons
+        assert PO.strategy_cache_stats["hits"] > 2 * PO.strategy_cache_stats["misses"]
+        g = opt._packed
+        assert g.num_nodes > 900 and g.num_entries > 200000
+        ref = O.GraphOracle(g).build()
+        slots = g.entry_slots()
+        cost_ref, _ = O.clamp_inf(ref["cost"])
+        assert bits_equal(opt._core.coef.comm, ref["comm"][slots])
+        assert bits_equal(opt._core.coef.cost, cost_ref[slots])
+        assert bits_equal(opt._core.coef.compute, ref["compute"])
+        # the first and the last layer's nodes got the same strategy sets
+        mms = [n for n in gm.graph.nodes if n.op == "call_function" and n.target is torch.ops.aten.mm.default]
+        per_layer = {}
+        for n in mms:
+            per_layer.setdefault(tuple(n.meta["val"].shape), []).append(len(opt.strats[n].strategies))
+        assert all(len(set(v)) == 1 for v in per_layer.values())
+    finally:
+        dist.destroy_process_group()
+        if had_pg:
+            dist.init_process_group("fake", store=FakeStore(), rank=0, world_size=8)
