@@ -131,7 +131,7 @@ def keep_unique_configs(op_strat: OpStrategy) -> OpStrategy:
     return OpStrategy(kept)
 
 
-def propagate_tensor_meta(node, arg_vals: List[torch.Tensor], out_strat: OpStrategy) -> None:
+def propagate_tensor_meta(node, arg_vals: List[torch.Tensor], out_strat: OpStrategy, mesh=None) -> None:
     out_val = node.meta.get("val")
     for st in out_strat.strategies:
         outs = st.output_specs
@@ -149,7 +149,8 @@ def propagate_tensor_meta(node, arg_vals: List[torch.Tensor], out_strat: OpStrat
             # an output DTensor leaves without a spec is Replicate; a spec for an
             # output that does not exist is dropped
             # (autoparallel/shardings/placement_options.py:72-101)
-            mesh = st.mesh
+            if mesh is None:
+                mesh = st.mesh
             fixed = []
             for s, v in zip(outs, vals):
                 if isinstance(v, torch.Tensor):
@@ -335,6 +336,18 @@ def _one_strategy_at_a_time(fn, op, args, kwargs, producers: List[OpStrategy]) -
     return OpStrategy(sts)
 
 
+def _without_partial(a):
+    """The argument with its Partial candidates left out (itself if it has none, or nothing else)."""
+    if isinstance(a, TupleStrategy):
+        kids = tuple(_without_partial(c) for c in a.children)
+        return a if all(x is y for x, y in zip(kids, a.children)) else TupleStrategy(kids)
+    if not isinstance(a, OpStrategy):
+        return a
+    keep = [st for st in a.strategies if isinstance(st.output_specs, DTensorSpec)
+            and not any(p.is_partial() for p in st.output_specs.placements)]
+    return a if not keep or len(keep) == len(a.strategies) else OpStrategy(keep)
+
+
 _NONSTRICT_VIEWS = {aten.view.default, aten._unsafe_view.default}
 # strategy functions of the installed torch that pair the arguments' strategies by index
 _INDEX_PAIRED = {getattr(getattr(aten, name), "default") for name in (
@@ -435,6 +448,14 @@ def _placement_options_uncached(mesh, node, producers, arg_vals, schema_args) ->
                         res = fn(OpSchema(op, args, kwargs))
                     except IndexError:
                         res = _one_strategy_at_a_time(fn, op, args, kwargs, producers)
+                    except RuntimeError:
+                        # some functions (the random ones) refuse an argument that may
+                        # arrive Partial: ask again without those candidates; what it
+                        # costs to bring a Partial producer there is priced per entry
+                        narrowed = tuple(_without_partial(a) for a in args)
+                        if all(x is y for x, y in zip(narrowed, args)):
+                            raise
+                        res = fn(OpSchema(op, narrowed, kwargs))
                 if isinstance(res, OpStrategy):
                     out = res
                     if len(producers) == 1:
@@ -455,7 +476,7 @@ def _placement_options_uncached(mesh, node, producers, arg_vals, schema_args) ->
                 f"{sorted({-1 if st.input_specs is None else len(st.input_specs) for st in out.strategies})}")
         fallback_reasons[str(node.name)] = why
         out = _replicate_fallback(mesh, node, arg_vals)
-    propagate_tensor_meta(node, arg_vals, out)
+    propagate_tensor_meta(node, arg_vals, out, mesh)
     fill_redistribute_cost(out, producers)
     out = remove_invalid_configs(out, mesh)
     out = keep_unique_configs(out)

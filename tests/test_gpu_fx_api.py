@@ -574,6 +574,47 @@ def test_hf_gpt2_small_joint_graph():
             dist.destroy_process_group()
 
 
+def test_encoder_layer_with_dropout_joint_graph(mesh):
+    """torch's TransformerEncoderLayer in training mode (dropout, whose DTensor
+    rule refuses Partial arguments): no operator on the all-Replicate stand-in,
+    coefficients equal to the oracle's, and the plan solves."""
+    from torch._functorch.aot_autograd import aot_export_joint_with_descriptors
+    from torch._subclasses.fake_tensor import FakeTensorMode
+
+    from autoparallel_amd.optimize_sharding import ShardingOptimizer
+    from autoparallel_amd.shardings import placement_options as PO
+
+    class Enc(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.layer = nn.TransformerEncoderLayer(64, 4, 128, dropout=0.1, batch_first=True)
+            self.head = nn.Linear(64, 1)
+
+        def forward(self, x):
+            return self.head(self.layer(x)).mean()
+
+    with FakeTensorMode():
+        with torch.device("cuda"):
+            m = Enc()
+        x = torch.randn(8, 16, 64, device="cuda")
+        with contextlib.ExitStack() as stack:
+            gm = aot_export_joint_with_descriptors(stack, m, (x,)).graph_module
+    assert any("native_dropout" in str(n.target) for n in gm.graph.nodes)
+    PO.fallback_nodes.clear()
+    PO.fallback_reasons.clear()
+    opt = ShardingOptimizer(gm, mesh, devices_per_host=8, device_name="AMD Instinct MI355X")
+    assert PO.fallback_nodes == [], PO.fallback_reasons
+    g = opt._packed
+    ref = O.GraphOracle(g).build()
+    slots = g.entry_slots()
+    cost_ref, _ = O.clamp_inf(ref["cost"])
+    assert bits_equal(opt._core.coef.comm, ref["comm"][slots])
+    assert bits_equal(opt._core.coef.cost, cost_ref[slots])
+    assert bits_equal(opt._core.coef.compute, ref["compute"])
+    sol = opt.get_solution()
+    assert set(sol) == {n for n in opt.nodes if n.op != "output"}
+
+
 def test_hf_llama3_8b_layers_joint_graph():
     """Llama-3-8B as transformers defines it (d 4096, 32 query / 8 key-value heads,
     SwiGLU 14336, RMSNorm, rotary embedding, vocab 128256, bf16), four of its

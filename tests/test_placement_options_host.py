@@ -219,3 +219,25 @@ def test_norm_strategies_with_unequal_candidate_counts(meshes):
     assert got == [((p, rr, rr), (p, p, p)) for p in (rr, (Shard(0), Replicate()), (Shard(0), Shard(1)))]
     assert [len(r) for r in out.strategies[0].redistribute_cost] == [4, 2, 2]
     assert out.strategies[0].output_specs[1].tensor_meta.shape == (256, 64, 1)
+
+
+def test_partial_candidates_do_not_cost_the_operator_its_strategies(meshes):
+    """DTensor's dropout rule raises when an argument may arrive Partial; the
+    query is repeated without those candidates instead of giving the operator up
+    to the all-Replicate stand-in (rows keep one column per real candidate)."""
+    from torch.distributed.tensor.placement_types import Partial
+
+    from autoparallel_amd.shardings.placement_options import fallback_nodes, get_placement_options_for_node
+
+    mesh = meshes[0]
+    src = _candidates(mesh, (512, 64), [(Replicate(),), (Shard(0),), (Partial(),)])
+    g = torch.fx.Graph()
+    x = g.placeholder("x")
+    x.meta["val"] = torch.empty(512, 64, device="meta")
+    node = g.call_function(torch.ops.aten.native_dropout.default, (x, 0.1, True))
+    node.meta["val"] = (torch.empty(512, 64, device="meta"), torch.empty(512, 64, dtype=torch.bool, device="meta"))
+    before = list(fallback_nodes)
+    out = get_placement_options_for_node(mesh, node, [src], [x.meta["val"]], (src, 0.1, True))
+    assert fallback_nodes == before
+    assert {st.input_specs[0].placements for st in out.strategies} == {(Replicate(),), (Shard(0),)}
+    assert all(len(st.redistribute_cost[0]) == 3 and len(st.output_specs) == 2 for st in out.strategies)
