@@ -396,7 +396,7 @@ def get_placement_options_for_node(mesh, node, producers: List[OpStrategy], arg_
     each tensor input node in flattened-args order; ``schema_args``: node.args
     with nodes replaced by their OpStrategy (or value for non-tensors)."""
     try:
-        key = (id(mesh), tuple(mesh.shape), node.target, _fingerprint(schema_args),
+        key = (mesh, node.target, _fingerprint(schema_args),
                _fingerprint({k: v for k, v in node.kwargs.items() if not isinstance(v, torch.fx.Node)}),
                _fingerprint(node.meta.get("val")), _fingerprint(arg_vals))
         hit = _strategy_cache.get(key)
