@@ -8,7 +8,7 @@ it with the reference's post-processing — tensor-meta fill
 (autoparallel/shardings/propagation_rules.py:127-158), de-duplication
 (placement_options.py:151-170) — and the few rules DTensor lacks or refuses
 (getitem, strict views, alias, two-operand einsum, operators without tensor
-inputs: propagation_rules.py:412-554; all-Replicate fallback:
+inputs: propagation_rules.py:412-554; local_map regions: placement_options.py:380-490; all-Replicate fallback:
 dtensor_sharding_helpers.py:364-383).  Its output is input data for the cost
 engine.  Input/parameter options are enumerated on the device
 (apc_enumerate_input_options).
@@ -336,6 +336,49 @@ def _one_strategy_at_a_time(fn, op, args, kwargs, producers: List[OpStrategy]) -
     return OpStrategy(sts)
 
 
+def _local_map_rule(mesh, node, schema_args, kw) -> OpStrategy:
+    """The single strategy of a ``local_map`` region: the placements its author
+    declared (autoparallel/shardings/placement_options.py:380-490).  Arguments
+    before the declared ones (the backward region's saved activations) are
+    Replicate, as are outputs after the declared ones; an argument or output
+    without a placement, or that is not a tensor, has no spec; a tensor with an
+    unbacked symbolic size has none either."""
+    in_plc, out_plc = kw["in_placements"], kw["out_placements"]
+    assert in_plc is not None and out_plc is not None
+    assert kw.get("in_grad_placements") is None, "Not yet implemented"
+    assert kw.get("device_mesh") in (mesh, None), "Not yet implemented"
+    assert "call_local_map" in str(node.target)
+    rep = (Replicate(),) * mesh.ndim
+
+    def meta_of(t):
+        if any(isinstance(x, torch.SymInt) for x in t.shape) or any(isinstance(x, torch.SymInt) for x in t.stride()):
+            return None
+        return _tensor_meta(t)
+
+    def spec_of(val, plc):
+        if plc is None or not isinstance(val, torch.Tensor):
+            return None
+        tm = meta_of(val)
+        if tm is None:
+            return None
+        plc = (plc,) if isinstance(plc, (Replicate, Shard, Partial)) else tuple(plc)
+        return DTensorSpec(mesh, plc, tensor_meta=tm)
+
+    vals = [a.meta.get("val") if isinstance(a, torch.fx.Node) else a for a in node.args]
+    n_act = len(vals) - len(in_plc)
+    assert n_act >= 0
+    in_specs = [spec_of(v, rep) for v in vals[:n_act]] + [spec_of(v, p) for v, p in zip(vals[n_act:], in_plc)]
+    out_val = node.meta["val"]
+    outs = list(out_val) if isinstance(out_val, (list, tuple)) else [out_val]
+    out_specs = [spec_of(v, p) for v, p in zip(outs, out_plc)] + [spec_of(v, rep) for v in outs[len(out_plc):]]
+    kept, rows = [], []
+    for arg, spec in zip(schema_args, in_specs):
+        if isinstance(arg, OpStrategy):  # other arguments have no sharding and no edge
+            kept.append(spec)
+            rows.append([0.0] * len(arg.strategies))
+    return OpStrategy([OpSpec(tuple(out_specs), input_specs=tuple(kept), redistribute_cost=rows)])
+
+
 def _without_partial(a):
     """The argument with its Partial candidates left out (itself if it has none, or nothing else)."""
     if isinstance(a, TupleStrategy):
@@ -395,6 +438,9 @@ def get_placement_options_for_node(mesh, node, producers: List[OpStrategy], arg_
     """Strategies of one call_function node.  ``producers``: OpStrategy of
     each tensor input node in flattened-args order; ``schema_args``: node.args
     with nodes replaced by their OpStrategy (or value for non-tensors)."""
+    if node.meta.get("local_map_kwargs"):
+        assert not node.kwargs
+        return _local_map_rule(mesh, node, schema_args, node.meta["local_map_kwargs"])
     try:
         key = (mesh, node.target, _fingerprint(schema_args),
                _fingerprint({k: v for k, v in node.kwargs.items() if not isinstance(v, torch.fx.Node)}),

@@ -698,3 +698,56 @@ def test_hf_llama3_8b_layers_joint_graph():
         dist.destroy_process_group()
         if had_pg:
             dist.init_process_group("fake", store=FakeStore(), rank=0, world_size=8)
+
+
+def test_local_map_region_in_a_graph(mesh):
+    """A graph with a local_map region (one declared strategy, zero compute, a
+    non-tensor argument, an output without a spec): coefficients equal the
+    oracle's, the region's inputs are redistributed to the declared placements,
+    and the plan solves."""
+    from torch.distributed.tensor.placement_types import Replicate, Shard
+
+    from autoparallel_amd.optimize_sharding import ShardingOptimizer
+
+    def call_local_map(*args):  # stands in for the higher-order operator; never run
+        raise AssertionError
+
+    aten = torch.ops.aten
+    g = torch.fx.Graph()
+    x, w = g.placeholder("x"), g.placeholder("w")
+    x.meta["val"] = torch.empty(256, 64, device="meta")
+    w.meta["val"] = torch.empty(64, 64, device="meta")
+    h = g.call_function(aten.mm.default, (x, w))
+    h.meta["val"] = torch.empty(256, 64, device="meta")
+    region = g.call_function(call_local_map, (h, w, 3))
+    region.meta["val"] = (torch.empty(256, 64, device="meta"), torch.empty(4, device="meta"))
+    region.meta["local_map_kwargs"] = {"in_placements": ((Shard(0), Replicate()), (Replicate(), Replicate()), None),
+                                       "out_placements": ((Shard(0), Replicate()),)}
+    y = g.call_function(__import__("operator").getitem, (region, 0))
+    y.meta["val"] = region.meta["val"][0]
+    r = g.call_function(aten.relu.default, (y,))
+    r.meta["val"] = torch.empty(256, 64, device="meta")
+    g.output((r,))
+    gm = torch.fx.GraphModule(torch.nn.Module(), g)
+    opt = ShardingOptimizer(gm, mesh, devices_per_host=8, device_name="AMD Instinct MI355X")
+    reg = region
+    assert len(opt.strats[reg].strategies) == 1
+    pk = opt._packed
+    ref = O.GraphOracle(pk).build()
+    slots = pk.entry_slots()
+    cost_ref, _ = O.clamp_inf(ref["cost"])
+    assert bits_equal(opt._core.coef.comm, ref["comm"][slots])
+    assert bits_equal(opt._core.coef.cost, cost_ref[slots])
+    v = opt.node_map[reg]
+    o0 = int(pk.node_comp_off[v])
+    assert opt._core.coef.compute[o0] == 0.0  # a region is not priced (not an OpOverload)
+    # the edge from the matmul into the region: free only from producer strategies that are (S(0), R) up to a local slice
+    e = int(pk.node_edge_off[v])
+    block = opt._core.coef.comm[opt._core.var_start[e]:opt._core.var_start[e + 1]]
+    src = [s.output_specs.placements for s in opt.strats[h].strategies]
+    tgt = (Shard(0), Replicate())
+    free = [all(a == b or (a.is_replicate() and b.is_shard()) for a, b in zip(p, tgt)) for p in src]  # R -> S is a local slice
+    assert [c == 0.0 for c in block] == free and not all(free) and sum(free) >= 2
+    sol = opt.get_solution()
+    assert sol[h].output_specs.placements == (Shard(0), Replicate())
+    assert sol[r].output_specs.placements == (Shard(0), Replicate())

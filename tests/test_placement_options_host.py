@@ -241,3 +241,48 @@ def test_partial_candidates_do_not_cost_the_operator_its_strategies(meshes):
     assert fallback_nodes == before
     assert {st.input_specs[0].placements for st in out.strategies} == {(Replicate(),), (Shard(0),)}
     assert all(len(st.redistribute_cost[0]) == 3 and len(st.output_specs) == 2 for st in out.strategies)
+
+
+def test_local_map_region_has_its_declared_strategy(meshes):
+    """A local_map region offers exactly the placements its author declared
+    (autoparallel/shardings/placement_options.py:380-490): leading arguments
+    beyond the declared ones are Replicate, an argument with placement None or a
+    non-tensor has no spec, trailing outputs are Replicate, and the cost rows
+    have one zero per candidate of each tensor argument."""
+    from torch.distributed.tensor.placement_types import Partial
+
+    from autoparallel_amd.shardings.placement_options import get_placement_options_for_node
+
+    mesh = meshes[1]  # (32, 8)
+
+    def call_local_map(*args):  # stands in for the higher-order operator
+        raise AssertionError("never run")
+
+    g = torch.fx.Graph()
+    sub = g.get_attr("body")  # the region's graph module: not a tensor
+    act, x, w, n = g.placeholder("act"), g.placeholder("x"), g.placeholder("w"), g.placeholder("n")
+    act.meta["val"] = torch.empty(64, 32, device="meta")
+    x.meta["val"] = torch.empty(256, 64, device="meta")
+    w.meta["val"] = torch.empty(64, 64, device="meta")
+    n.meta["val"] = 7
+    node = g.call_function(call_local_map, (sub, act, x, w, n))
+    node.meta["val"] = (torch.empty(256, 64, device="meta"), None, torch.empty(8, device="meta"))
+    node.meta["local_map_kwargs"] = {
+        "in_placements": ((Shard(0), Replicate()), None, None),
+        "out_placements": ((Shard(0), Partial()), None),
+    }
+    cands = {
+        act: _candidates(mesh, (64, 32), [(Replicate(), Replicate()), (Shard(0), Replicate())]),
+        x: _candidates(mesh, (256, 64), [(Replicate(), Replicate()), (Shard(0), Replicate()), (Shard(0), Shard(1))]),
+        w: _candidates(mesh, (64, 64), [(Replicate(), Replicate())]),
+    }
+    schema = (None, cands[act], cands[x], cands[w], 7)
+    out = get_placement_options_for_node(mesh, node, [cands[act], cands[x], cands[w]],
+                                         [act.meta["val"], x.meta["val"], w.meta["val"]], schema)
+    assert len(out.strategies) == 1
+    st = out.strategies[0]
+    rr = (Replicate(), Replicate())
+    assert [None if s is None else s.placements for s in st.input_specs] == [rr, (Shard(0), Replicate()), None]
+    assert st.input_specs[1].tensor_meta.shape == (256, 64)
+    assert [None if s is None else s.placements for s in st.output_specs] == [(Shard(0), Partial()), None, rr]
+    assert st.redistribute_cost == [[0.0, 0.0], [0.0, 0.0, 0.0], [0.0]]
