@@ -168,6 +168,45 @@ def propagate_tensor_meta(node, arg_vals: List[torch.Tensor], out_strat: OpStrat
                     s.tensor_meta = _tensor_meta(v)
 
 
+def _unshare_specs(out_strat: OpStrategy, producers: List[OpStrategy]) -> None:
+    """Some strategy functions hand back a producer's own spec object as the
+    input spec, or one object as both input and output spec (DTensor's select
+    when the selected dim is not sharded; the reference copies it there,
+    autoparallel/shardings/propagation_rules.py:318-355).  The tensor-meta fill
+    writes into specs, so every spec of the new strategies gets an object of its
+    own first."""
+    import dataclasses
+
+    taken = set()
+    for p in producers:
+        for st in p.strategies:
+            outs = st.output_specs
+            for sp in (outs if isinstance(outs, (tuple, list)) else (outs,)):
+                if sp is not None:
+                    taken.add(id(sp))
+
+    def own(sp):
+        if sp is None:
+            return None
+        if id(sp) in taken:
+            sp = dataclasses.replace(sp)
+        taken.add(id(sp))
+        return sp
+
+    for st in out_strat.strategies:
+        if st.input_specs is not None:
+            ins = [own(sp) for sp in st.input_specs]
+            if any(a is not b for a, b in zip(ins, st.input_specs)):
+                st.input_specs = tuple(ins) if isinstance(st.input_specs, tuple) else ins
+        outs = st.output_specs
+        if isinstance(outs, DTensorSpec):
+            st.output_specs = own(outs)
+        elif outs is not None:
+            new = tuple(own(sp) for sp in outs)
+            if any(a is not b for a, b in zip(new, outs)):
+                st.output_specs = new
+
+
 def fill_redistribute_cost(out_strat: OpStrategy, producers: List[OpStrategy]) -> None:
     """Rows of the right shape (one per tensor argument, one column per
     producer strategy); the values are overwritten by the cost engine."""
@@ -379,6 +418,82 @@ def _local_map_rule(mesh, node, schema_args, kw) -> OpStrategy:
     return OpStrategy([OpSpec(tuple(out_specs), input_specs=tuple(kept), redistribute_cost=rows)])
 
 
+def _product_rule(mesh, rows, n_out: int) -> OpStrategy:
+    """Every combination over the mesh dims of single-dim rows
+    ``[output placements..., input placements...]``; tensor metas and the
+    validity filter come afterwards."""
+    sts = []
+    for comb in itertools.product(rows, repeat=mesh.ndim):
+        specs = [DTensorSpec(mesh, tuple(plc)) for plc in zip(*comb)]
+        outs = specs[0] if n_out == 1 else tuple(specs[:n_out])
+        sts.append(OpSpec(outs, input_specs=list(specs[n_out:])))
+    return OpStrategy(sts)
+
+
+def _stack_rule(mesh, node, producers: List[OpStrategy]) -> OpStrategy:
+    """stack: inputs all Replicate or all sharded on the same dim, the output on
+    that dim shifted past the new one (autoparallel/shardings/propagation_rules.py:621-656;
+    DTensor's own rule only follows the first input's first candidate)."""
+    ndim = len(producers[0].shape)
+    dim = node.args[1] if len(node.args) > 1 else node.kwargs.get("dim", 0)
+    dim = dim + ndim + 1 if dim < 0 else dim
+    rows = [[Replicate()] * (1 + len(producers))]
+    rows += [[Shard(i if i < dim else i + 1)] + [Shard(i)] * len(producers) for i in range(ndim)]
+    return _product_rule(mesh, rows, 1)
+
+
+def _uniform_rule(mesh, node, src: OpStrategy) -> OpStrategy:
+    """uniform_: the output keeps any sharding of the input
+    (autoparallel/shardings/propagation_rules.py:663-680)."""
+    rows = [[Replicate(), Replicate()]] + [[Shard(d), Shard(d)] for d in range(len(src.shape))]
+    return _product_rule(mesh, rows, 1)
+
+
+def _split_with_sizes_rule(mesh, node, src: OpStrategy) -> OpStrategy:
+    """split_with_sizes: the pieces keep the input's placements; candidates sharded
+    on the split dim or Partial are not offered
+    (autoparallel/shardings/propagation_rules.py:375-409)."""
+    dim = node.args[2] if len(node.args) > 2 else node.kwargs.get("dim", 0)
+    dim = dim + len(src.shape) if dim < 0 else dim
+    n_out = len(node.meta["val"])
+    seen, sts = set(), []
+    for st in src.strategies:
+        plc = st.output_specs.placements
+        if plc in seen or any(p.is_shard(dim) or p.is_partial() for p in plc):
+            continue
+        seen.add(plc)
+        sts.append(OpSpec(tuple(DTensorSpec(mesh, plc) for _ in range(n_out)),
+                          input_specs=(DTensorSpec(mesh, plc, tensor_meta=st.output_specs.tensor_meta),)))
+    return OpStrategy(sts)
+
+
+def _view_dtype_rule(mesh, node, src: OpStrategy) -> OpStrategy:
+    """view(dtype): the bytes of the last dim are regrouped, so candidates sharded
+    on it are not offered; the others carry over
+    (autoparallel/shardings/propagation_rules.py:289-315)."""
+    last = len(src.shape) - 1
+    seen, sts = set(), []
+    for st in src.strategies:
+        plc = st.output_specs.placements
+        if plc in seen or any(p.is_shard(last) for p in plc):
+            continue
+        seen.add(plc)
+        sts.append(OpSpec(DTensorSpec(mesh, plc),
+                          input_specs=(DTensorSpec(mesh, plc, tensor_meta=st.output_specs.tensor_meta),)))
+    return OpStrategy(sts)
+
+
+def _alias_rule(mesh, node, src: OpStrategy) -> OpStrategy:
+    """alias: every valid placement of the tensor, output as input
+    (autoparallel/shardings/propagation_rules.py:358-372)."""
+    tm = _tensor_meta(node.meta["val"])
+    sts = []
+    for st in _create_all_options(mesh, tm.shape, tensor_meta=tm).strategies:
+        plc = st.output_specs.placements
+        sts.append(OpSpec(DTensorSpec(mesh, plc, tensor_meta=tm), input_specs=(DTensorSpec(mesh, plc, tensor_meta=tm),)))
+    return OpStrategy(sts)
+
+
 def _without_partial(a):
     """The argument with its Partial candidates left out (itself if it has none, or nothing else)."""
     if isinstance(a, TupleStrategy):
@@ -396,7 +511,8 @@ _NONSTRICT_VIEWS = {aten.view.default, aten._unsafe_view.default}
 _INDEX_PAIRED = {getattr(getattr(aten, name), "default") for name in (
     "native_layer_norm", "native_layer_norm_backward", "_fused_rms_norm", "_fused_rms_norm_backward",
     "nll_loss_forward", "nll_loss_backward", "nll_loss2d_forward", "nll_loss2d_backward") if hasattr(aten, name)}
-_FOLLOW = {aten.alias.default, aten.detach.default}
+_FOLLOW = {aten.detach.default} | ({torch.ops.prims.convert_element_type.default}
+                                  if hasattr(torch.ops.prims, "convert_element_type") else set())
 
 
 def _fingerprint(x):
@@ -478,6 +594,16 @@ def _placement_options_uncached(mesh, node, producers, arg_vals, schema_args) ->
             out = _einsum_rule(mesh, node, *producers)
         elif op in _NONSTRICT_VIEWS and len(producers) == 1:
             out = _view_rule(mesh, node, producers[0])
+        elif op is aten.alias.default and len(producers) == 1:
+            out = _alias_rule(mesh, node, producers[0])
+        elif op is aten.stack.default and producers:
+            out = _stack_rule(mesh, node, producers)
+        elif op is aten.uniform.default and len(producers) == 1:
+            out = _uniform_rule(mesh, node, producers[0])
+        elif op is aten.split_with_sizes.default and len(producers) == 1:
+            out = _split_with_sizes_rule(mesh, node, producers[0])
+        elif op is aten.view.dtype and len(producers) == 1:
+            out = _view_dtype_rule(mesh, node, producers[0])
         else:
             fn = prop.op_strategy_funcs.get(op)
             if fn is not None:
@@ -486,6 +612,13 @@ def _placement_options_uncached(mesh, node, producers, arg_vals, schema_args) ->
                         return TupleStrategy(tuple(x))
                     return x
                 args = tuple(wrap(a) for a in schema_args)
+                if op is aten.select.int and isinstance(args[0], OpStrategy):
+                    # DTensor's rule does not take a negative dim or index
+                    # (autoparallel/shardings/propagation_rules.py:318-343)
+                    d, i = args[1], args[2]
+                    d = d + len(args[0].shape) if isinstance(d, int) and d < 0 else d
+                    i = i + args[0].shape[d] if isinstance(i, int) and i < 0 else i
+                    args = (args[0], d, i) + args[3:]
                 kwargs = {k: v for k, v in node.kwargs.items() if not isinstance(v, torch.fx.Node)}
                 if op in _INDEX_PAIRED and len(producers) > 1:
                     res = _one_strategy_at_a_time(fn, op, args, kwargs, producers)
@@ -522,6 +655,7 @@ def _placement_options_uncached(mesh, node, producers, arg_vals, schema_args) ->
                 f"{sorted({-1 if st.input_specs is None else len(st.input_specs) for st in out.strategies})}")
         fallback_reasons[str(node.name)] = why
         out = _replicate_fallback(mesh, node, arg_vals)
+    _unshare_specs(out, producers)
     propagate_tensor_meta(node, arg_vals, out, mesh)
     fill_redistribute_cost(out, producers)
     out = remove_invalid_configs(out, mesh)

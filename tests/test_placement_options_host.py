@@ -286,3 +286,104 @@ def test_local_map_region_has_its_declared_strategy(meshes):
     assert st.input_specs[1].tensor_meta.shape == (256, 64)
     assert [None if s is None else s.placements for s in st.output_specs] == [(Shard(0), Partial()), None, rr]
     assert st.redistribute_cost == [[0.0, 0.0], [0.0, 0.0, 0.0], [0.0]]
+
+
+def test_select_does_not_write_into_its_producer(meshes):
+    """DTensor's select hands back one spec object as input and output when the
+    selected dim is not sharded; the tensor-meta fill must not reach the
+    producer's or the input's meta through it."""
+    from autoparallel_amd.shardings.placement_options import get_placement_options_for_node
+
+    mesh = meshes[1]
+    src = _candidates(mesh, (256, 16, 64), [(Replicate(), Replicate()), (Shard(0), Replicate()), (Shard(0), Shard(2))])
+    g = torch.fx.Graph()
+    x = g.placeholder("x")
+    x.meta["val"] = torch.empty(256, 16, 64, device="meta")
+    node = g.call_function(torch.ops.aten.select.int, (x, 1, 3))
+    node.meta["val"] = torch.empty(256, 64, device="meta")
+    out = get_placement_options_for_node(mesh, node, [src], [x.meta["val"]], (src, 1, 3))
+    assert len(out.strategies) >= 3
+    for st in src.strategies:
+        assert st.output_specs.tensor_meta.shape == (256, 16, 64)
+    for st in out.strategies:
+        assert st.output_specs.tensor_meta.shape == (256, 64)
+        assert st.input_specs[0].tensor_meta.shape == (256, 16, 64)
+        assert st.input_specs[0] is not st.output_specs
+    assert {st.output_specs.placements for st in out.strategies} >= {(Replicate(), Replicate()), (Shard(0), Shard(1))}
+
+
+def _plcs(strategy):
+    out = []
+    for st in strategy.strategies:
+        o = st.output_specs[0] if isinstance(st.output_specs, tuple) else st.output_specs
+        out.append((tuple(s.placements for s in st.input_specs), o.placements))
+    return out
+
+
+def test_rules_the_reference_keeps_for_itself(meshes):
+    """stack, uniform_, split_with_sizes, view(dtype) and alias as the reference's
+    own rules define them (autoparallel/shardings/propagation_rules.py:289-315,
+    358-409, 621-680), on a (32, 8) mesh."""
+    from torch.distributed.tensor.placement_types import Partial
+
+    from autoparallel_amd.shardings import placement_options as PO
+
+    mesh = meshes[1]
+    aten = torch.ops.aten
+    R, S = Replicate(), Shard
+    g = torch.fx.Graph()
+    a, b = g.placeholder("a"), g.placeholder("b")
+    a.meta["val"] = b.meta["val"] = torch.empty(256, 64, device="meta")
+    two = _candidates(mesh, (256, 64), [(R, R), (S(0), R)])
+
+    # stack at dim 1: inputs alike, the output's shard dim moves past the new dim
+    node = g.call_function(aten.stack.default, ([a, b], 1))
+    node.meta["val"] = torch.empty(256, 2, 64, device="meta")
+    out = PO.get_placement_options_for_node(mesh, node, [two, two], [a.meta["val"]] * 2, ([two, two], 1))
+    got = _plcs(out)
+    # 3 x 3 combinations less (S(1), S(1)): 64 / 32 = 2 rows cannot be split 8 ways
+    assert len(got) == 8 and all(i[0] == i[1] for i, _ in got)
+    assert ((((S(0), S(1)),) * 2, (S(0), S(2))) in got) and ((((R, R),) * 2, (R, R)) in got)
+    assert all(len(r) == 2 for st in out.strategies for r in st.redistribute_cost)
+
+    # uniform_: output as input, every sharding of the tensor
+    node = g.call_function(aten.uniform.default, (a, 0.0, 1.0))
+    node.meta["val"] = a.meta["val"]
+    got = _plcs(PO.get_placement_options_for_node(mesh, node, [two], [a.meta["val"]], (two, 0.0, 1.0)))
+    assert len(got) == 8 and all(i == (o,) for i, o in got) and ((S(1), S(1)),) not in [i for i, _ in got]
+
+    # split_with_sizes on dim 1: no candidate sharded there, none Partial
+    many = _candidates(mesh, (256, 64), [(R, R), (S(0), R), (S(1), R), (R, Partial()), (S(0), S(0)), (S(0), R)])
+    node = g.call_function(aten.split_with_sizes.default, (a, [32, 32], 1))
+    node.meta["val"] = (torch.empty(256, 32, device="meta"), torch.empty(256, 32, device="meta"))
+    out = PO.get_placement_options_for_node(mesh, node, [many], [a.meta["val"]], (many, [32, 32], 1))
+    assert [st.input_specs[0].placements for st in out.strategies] == [(R, R), (S(0), R), (S(0), S(0))]
+    assert all(len(st.output_specs) == 2 and st.output_specs[1].tensor_meta.shape == (256, 32) and
+               st.output_specs[0].placements == st.input_specs[0].placements for st in out.strategies)
+    assert all(len(st.redistribute_cost[0]) == 6 for st in out.strategies)
+
+    # view(dtype): nothing sharded on the last dim
+    node = g.call_function(aten.view.dtype, (a, torch.int32))
+    node.meta["val"] = torch.empty(256, 64, dtype=torch.int32, device="meta")
+    out = PO.get_placement_options_for_node(mesh, node, [many], [a.meta["val"]], (many, torch.int32))
+    assert [st.output_specs.placements for st in out.strategies] == [(R, R), (S(0), R), (R, Partial()), (S(0), S(0))]
+    assert all(st.output_specs.tensor_meta.dtype == torch.int32 and st.input_specs[0].tensor_meta.dtype == torch.float32
+               for st in out.strategies)
+
+
+def test_select_takes_negative_dim_and_index(meshes):
+    from autoparallel_amd.shardings.placement_options import fallback_nodes, get_placement_options_for_node
+
+    mesh = meshes[1]
+    src = _candidates(mesh, (256, 16, 64), [(Replicate(), Replicate()), (Shard(0), Shard(2))])
+    g = torch.fx.Graph()
+    x = g.placeholder("x")
+    x.meta["val"] = torch.empty(256, 16, 64, device="meta")
+    outs = []
+    for dim, index in ((1, 15), (-2, -1)):
+        node = g.call_function(torch.ops.aten.select.int, (x, dim, index))
+        node.meta["val"] = torch.empty(256, 64, device="meta")
+        before = list(fallback_nodes)
+        outs.append(_plcs(get_placement_options_for_node(mesh, node, [src], [x.meta["val"]], (src, dim, index))))
+        assert fallback_nodes == before
+    assert outs[0] == outs[1] and (((Shard(0), Shard(2)),), (Shard(0), Shard(1))) in outs[0]
