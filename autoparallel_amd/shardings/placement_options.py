@@ -608,7 +608,9 @@ def _placement_options_uncached(mesh, node, producers, arg_vals, schema_args) ->
             fn = prop.op_strategy_funcs.get(op)
             if fn is not None:
                 def wrap(x):
-                    if isinstance(x, (list, tuple)) and x and all(isinstance(y, OpStrategy) for y in x):
+                    # a list argument with tensors in it, e.g. index_put's indices with None for
+                    # the dims it leaves alone (autoparallel/shardings/placement_options.py:306-316)
+                    if isinstance(x, (list, tuple)) and any(isinstance(y, OpStrategy) for y in x):
                         return TupleStrategy(tuple(x))
                     return x
                 args = tuple(wrap(a) for a in schema_args)
