@@ -699,21 +699,42 @@ int apc_mesh_topology(const int32_t* mesh_shape, int32_t ndim, int32_t devices_p
   return 0;
 }
 
+namespace {
+// Device table of autoparallel/cost_models/compute_estimation.py:66-255, in its
+// order (the first entry whose name occurs in the device name wins): memory
+// bandwidth in bytes/s and dense GEMM TFLOP/s for f64, f32 (tf32 where the
+// device has it), f16, bf16, int8; 0 = the reference lists no figure.
+struct DeviceRow { const char* name; double gmem_bw; double tflops[APC_NUM_DTYPES]; };
+constexpr double kGiB = 1024.0 * 1024.0 * 1024.0, kTiB = 1024.0 * kGiB;
+const DeviceRow kDevices[] = {
+    {"H100", 3.35 * kTiB, {67, 989 / 2, 1979 / 2, 1979 / 2, 3958 / 2}},  // integer halves, as written there
+    {"B200", 7.7 * kTiB, {37, 2200 / 2, 4500 / 2, 4500 / 2, 9000 / 2}},
+    {"A100", 2 * kTiB, {19.5, 156, 312, 312, 624}},
+    {"A30", 933 * kGiB, {10.3, 82, 165, 165, 330}},
+    {"A10G", 933 * kGiB, {0, 31.2, 125, 125, 250}},
+    {"T4", 300 * kGiB, {0, 8.1, 65, 0, 130}},
+    {"V100", 900 * kGiB, {7.8, 15.7, 125, 0, 0}},
+    {"P100", 732 * kGiB, {5.3, 10.6, 21.2, 0, 0}},
+    {"AMD Instinct MI200X", 1.6 * kTiB, {45.3, 45.3, 181.0, 181.0, 181.0}},
+    {"AMD Instinct MI300X", 5.3 * kTiB, {163.4, 653.7, 1307.4, 1307.4, 2614.9}},
+    {"AMD Instinct MI325X", 6.0 * kTiB, {163.4, 653.7, 1307.4, 1307.4, 2614.9}},
+    {"AMD Instinct MI350X", 8.0 * kTiB, {72.1, 144.2, 2309.6, 2309.6, 4614.0}},
+    {"AMD Instinct MI355X", 8.0 * kTiB, {78.6, 157.3, 2516.6, 2516.6, 5033.2}},
+    {"Max 1550", 3.3 * kTiB, {46, 46, 367, 367, 734}},
+};
+}  // namespace
+
 int apc_device_limits(const char* device_name, apc_model* model) {
   if (!device_name || !model) return fail(APC_ERR_INVALID, "apc_device_limits: null argument%s");
   for (int i = 0; i < APC_NUM_DTYPES; ++i) model->tflops[i] = 0.0;
   // dtype codes: 0 f64, 1 f32, 2 f16, 3 bf16, 4 int8
-  if (strstr(device_name, "AMD Instinct MI355X")) {
-    model->gmem_bw = 8.0 * (1024.0 * 1024.0 * 1024.0 * 1024.0);
-    model->tflops[0] = 78.6; model->tflops[1] = 157.3; model->tflops[2] = 2516.6;
-    model->tflops[3] = 2516.6; model->tflops[4] = 5033.2;
-    return 0;
-  }
-  if (strstr(device_name, "AMD Instinct MI300X")) {
-    model->gmem_bw = 5.3 * (1024.0 * 1024.0 * 1024.0 * 1024.0);
-    model->tflops[0] = 81.7; model->tflops[1] = 163.4; model->tflops[2] = 1307.4;
-    model->tflops[3] = 1307.4; model->tflops[4] = 2614.9;
-    return 0;
+  for (const DeviceRow& d : kDevices) {
+    // compute_estimation.py:262-266: substring match, and PG509 boards are A100s
+    if (strstr(device_name, d.name) || (!strcmp(d.name, "A100") && strstr(device_name, "PG509"))) {
+      model->gmem_bw = d.gmem_bw;
+      for (int i = 0; i < APC_NUM_DTYPES; ++i) model->tflops[i] = d.tflops[i];
+      return 0;
+    }
   }
   return fail(APC_ERR_UNSUPPORTED, "Unsupported device: %s", device_name);
 }

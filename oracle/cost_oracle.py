@@ -60,10 +60,39 @@ MI355X_GMEM_BW = 8.0 * (1024**4)
 MI355X_TFLOPS = {0: 78.6, 1: 157.3, 2: 2516.6, 3: 2516.6, 4: 5033.2}
 
 
+# The whole table (compute_estimation.py:66-255), in its order: name ->
+# (bytes/s, {dtype code: TFLOPS}); the halves are integer halves there.
+DEVICE_TABLE = (
+    ("H100", 3.35 * (1024**4), {0: 67, 1: 989 // 2, 2: 1979 // 2, 3: 1979 // 2, 4: 3958 // 2}),
+    ("B200", 7.7 * (1024**4), {0: 37, 1: 2200 // 2, 2: 4500 // 2, 3: 4500 // 2, 4: 9000 // 2}),
+    ("A100", 2 * (1024**4), {0: 19.5, 1: 156, 2: 312, 3: 312, 4: 624}),
+    ("A30", 933 * (1024**3), {0: 10.3, 1: 82, 2: 165, 3: 165, 4: 330}),
+    ("A10G", 933 * (1024**3), {1: 31.2, 2: 125, 3: 125, 4: 250}),
+    ("T4", 300 * (1024**3), {1: 8.1, 2: 65, 4: 130}),
+    ("V100", 900 * (1024**3), {0: 7.8, 1: 15.7, 2: 125}),
+    ("P100", 732 * (1024**3), {0: 5.3, 1: 10.6, 2: 21.2}),
+    ("AMD Instinct MI200X", 1.6 * (1024**4), {0: 45.3, 1: 45.3, 2: 181.0, 3: 181.0, 4: 181.0}),
+    ("AMD Instinct MI300X", 5.3 * (1024**4), {0: 163.4, 1: 653.7, 2: 1307.4, 3: 1307.4, 4: 2614.9}),
+    ("AMD Instinct MI325X", 6.0 * (1024**4), {0: 163.4, 1: 653.7, 2: 1307.4, 3: 1307.4, 4: 2614.9}),
+    ("AMD Instinct MI350X", 8.0 * (1024**4), {0: 72.1, 1: 144.2, 2: 2309.6, 3: 2309.6, 4: 4614.0}),
+    ("AMD Instinct MI355X", MI355X_GMEM_BW, MI355X_TFLOPS),
+    ("Max 1550", 3.3 * (1024**4), {0: 46, 1: 46, 2: 367, 3: 367, 4: 734}),
+)
+
+
 class DeviceLimit:
     def __init__(self, gmem_bandwidth=MI355X_GMEM_BW, tflops=None):
         self.gmem_bandwidth = gmem_bandwidth
         self.tflops = dict(MI355X_TFLOPS if tflops is None else tflops)
+
+    @classmethod
+    def named(cls, device_name: str) -> "DeviceLimit":
+        """First row whose name occurs in device_name; PG509 boards are A100s
+        (compute_estimation.py:258-275)."""
+        for name, bw, tf in DEVICE_TABLE:
+            if name in device_name or (name == "A100" and "PG509" in device_name):
+                return cls(bw, {k: float(v) for k, v in tf.items()})
+        raise ValueError(f"Unsupported device: {device_name}")
 
 
 class Topo:

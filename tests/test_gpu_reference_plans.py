@@ -1,0 +1,163 @@
+"""The solved plans the reference's own tests expect
+(tests/test_optimize_placement.py:67-299 there), reproduced through
+ShardingOptimizer on this stack: same models, sizes, meshes (256 ranks, 8 per
+host, planning device H100 with its NCCL model, as that suite's patches and the
+default cost model set it up), same constraints, and the joint graph prepared
+with alias nodes as the reference prepares it.  The expected placements below
+are that file's expectations, not this repository's output."""
+import contextlib
+
+import pytest
+import torch
+import torch.nn as nn
+from torch.distributed.tensor.placement_types import Partial, Replicate, Shard
+
+pytestmark = pytest.mark.gpu
+
+
+class FFN(nn.Module):
+    def __init__(self, dim1, dim2):
+        super().__init__()
+        self.linear1 = nn.Linear(dim1, dim2, bias=False)
+        self.linear2 = nn.Linear(dim2, dim1, bias=False)
+
+    def forward(self, x, y):
+        return y + 2, self.linear2(self.linear1(x)), y + 2
+
+
+class TransformerBlock(nn.Module):
+    def __init__(self, nheads, dim1, dim2):
+        super().__init__()
+        self.nheads = nheads
+        self.wq, self.wk, self.wv, self.wo = (nn.Linear(dim1, dim1, bias=False) for _ in range(4))
+        self.w1, self.w2 = nn.Linear(dim1, dim2, bias=False), nn.Linear(dim2, dim1, bias=False)
+
+    def forward(self, x):
+        heads = lambda t: t.unflatten(-1, (self.nheads, -1)).permute(0, 2, 1, 3)
+        o = nn.functional.scaled_dot_product_attention(heads(self.wq(x)), heads(self.wk(x)), heads(self.wv(x)))
+        o0 = self.wo(o.permute(0, 2, 1, 3).flatten(-2)) + x
+        return o0 + self.w2(torch.relu(self.w1(o0)))
+
+
+@pytest.fixture(scope="module")
+def meshes():
+    if not torch.cuda.is_available():
+        pytest.skip("needs a GPU")
+    import torch.distributed as dist
+    from torch.distributed.device_mesh import init_device_mesh
+    from torch.testing._internal.distributed.fake_pg import FakeStore
+
+    from autoparallel_amd.cost_models import get_nccl_topo_config, set_nccl_topo_config
+
+    if dist.is_initialized():
+        dist.destroy_process_group()
+    dist.init_process_group("fake", store=FakeStore(), rank=0, world_size=256)
+    before = get_nccl_topo_config()
+    yield (init_device_mesh("cpu", (256,), mesh_dim_names=("dp",)),
+           init_device_mesh("cpu", (32, 8), mesh_dim_names=("dp", "tp")))
+    set_nccl_topo_config(before)
+    dist.destroy_process_group()
+
+
+def _optimizer(mesh, model_type, high_mem):
+    from torch._functorch.aot_autograd import aot_export_joint_with_descriptors
+    from torch._subclasses.fake_tensor import FakeTensorMode
+
+    from autoparallel_amd.cost_models import detect_nccl_topo_config, set_nccl_topo_config
+    from autoparallel_amd.graph_utils import add_alias_nodes
+    from autoparallel_amd.optimize_sharding import ShardingOptimizer
+    from autoparallel_amd.shardings import placement_options as PO
+
+    lead = mesh.shape[0]
+    with FakeTensorMode():
+        with torch.device("cuda"):
+            m = FFN(1024, 4096) if model_type == "ffn" else TransformerBlock(48, 6144, 6144 * 4)
+        if model_type == "ffn":
+            xs = (torch.randn(2048 * lead, 1024, device="cuda"), torch.randn(2048 * lead, 1, device="cuda"))
+        else:
+            xs = (torch.randn(8 * lead, 256, 6144, device="cuda", requires_grad=True),)
+        with contextlib.ExitStack() as stack:
+            gm = aot_export_joint_with_descriptors(stack, m, xs).graph_module
+    add_alias_nodes(gm)
+    set_nccl_topo_config(detect_nccl_topo_config(mesh, "H100"))
+    PO.fallback_nodes.clear()
+    opt = ShardingOptimizer(gm, mesh, devices_per_host=8, device_name="H100")
+    assert PO.fallback_nodes == [], PO.fallback_reasons
+    batch = (Shard(0),) + (Replicate(),) * (mesh.ndim - 1)
+    n_in, n_out = (2, 3) if model_type == "ffn" else (1, 1)
+    opt.add_sharded_input_constraint([batch] * n_in)
+    opt.add_sharded_output_constraint([batch] * n_out)
+    opt.add_parameter_memory_constraint(0, 1.0 / mesh.size() if high_mem is None else high_mem)  # api.py:371-382
+    return gm, opt
+
+
+def _mm_nodes(gm):
+    return [n for n in gm.graph.nodes if n.op == "call_function" and n.target is torch.ops.aten.mm.default]
+
+
+@pytest.mark.parametrize("model_type", ["ffn", "transformer_block"])
+@pytest.mark.parametrize("high_mem", [None, 1.0])
+def test_fsdp_and_ddp_on_one_mesh_dim(meshes, model_type, high_mem):
+    """tests/test_optimize_placement.py:100-183: parameters sharded (budget 1/256)
+    or replicated (budget 1), forward matmuls batch-sharded with the whole weight,
+    weight gradients Partial, input gradients batch-sharded."""
+    from torch._functorch._aot_autograd.fx_utils import get_param_nodes
+
+    gm, opt = _optimizer(meshes[0], model_type, high_mem)
+    sol = opt.get_solution()
+    want = (Shard(0),) if high_mem is None else (Replicate(),)
+    for node in get_param_nodes(gm.graph):
+        assert sol[node].output_specs.placements == want
+    mms = _mm_nodes(gm)
+    n_fwd = 2 if model_type == "ffn" else 6
+    assert len(mms) == (5 if model_type == "ffn" else 18)
+    for node in mms[:n_fwd]:
+        p = sol[node]
+        assert (p.input_specs[0].placements, p.input_specs[1].placements, p.output_specs.placements) == \
+            ((Shard(0),), (Replicate(),), (Shard(0),))
+    for node in mms[n_fwd::2]:  # weight gradients
+        p = sol[node]
+        assert (p.input_specs[0].placements, p.input_specs[1].placements, p.output_specs.placements) == \
+            ((Shard(1),), (Shard(0),), (Partial("sum"),))
+    for node in mms[n_fwd + 1::2]:  # input gradients
+        p = sol[node]
+        assert (p.input_specs[0].placements, p.input_specs[1].placements, p.output_specs.placements) == \
+            ((Shard(0),), (Replicate(),), (Shard(0),))
+
+
+_S, _R, _P = Shard, Replicate(), Partial("sum")
+# matmul placements (input 0, input 1, output) of tests/test_optimize_placement.py:189-192
+_MM1 = ((_S(0), _R), (_R, _S(1)), (_S(0), _S(1)))
+_MM2 = ((_S(0), _S(1)), (_R, _S(0)), (_S(0), _P))
+_MM3 = ((_S(1), _R), (_S(0), _S(1)), (_P, _S(1)))
+_MM4 = ((_S(1), _S(0)), (_S(0), _R), (_P, _S(0)))
+_EXPECTED_2D = {  # :186-233
+    "ffn": ([(_S(0), _S(0)), (_S(0), _S(1))], [_MM1, _MM2, _MM3, _MM1, _MM4]),
+    "transformer_block": (
+        [(_S(0), _S(0))] * 3 + [(_S(0), _S(1)), (_S(0), _S(0)), (_S(0), _S(1))],
+        [_MM1, _MM1, _MM1, _MM2, _MM1, _MM2, _MM3, _MM1, _MM4, _MM2, _MM3, _MM1, _MM4, _MM2, _MM4, _MM2, _MM4, _MM2]),
+}
+
+
+@pytest.mark.parametrize("model_type", ["ffn", "transformer_block"])
+def test_fsdp_with_tensor_parallel_on_two_mesh_dims(meshes, model_type):
+    """tests/test_optimize_placement.py:236-299: every parameter's placement,
+    every matmul's input and output placements, and attention sharded on batch
+    and heads."""
+    from torch._functorch._aot_autograd.fx_utils import get_param_nodes
+
+    gm, opt = _optimizer(meshes[1], model_type, None)
+    sol = opt.get_solution()
+    params, mms = _EXPECTED_2D[model_type]
+    got = [sol[n].output_specs.placements for n in get_param_nodes(gm.graph)]
+    assert got == params
+    got = [(sol[n].input_specs[0].placements, sol[n].input_specs[1].placements, sol[n].output_specs.placements)
+           for n in _mm_nodes(gm)]
+    assert got == mms
+    sdpa = [n for n in gm.graph.nodes if n.op == "call_function"
+            and n.target is torch.ops.aten._scaled_dot_product_efficient_attention.default]
+    assert len(sdpa) == (0 if model_type == "ffn" else 1)
+    for node in sdpa:
+        p = sol[node]
+        assert [s.placements for s in p.input_specs[:3]] == [(_S(0), _S(1))] * 3
+        assert p.output_specs[0].placements == (_S(0), _S(1))

@@ -96,3 +96,43 @@ def test_terminal_derived_known_answers():
     _out(g, [fwd, ga, gb], [PlainAOTOutput(0), GradAOTOutput(grad_of=da), GradAOTOutput(grad_of=db)])
     t = build_terminal_derived_set(g)
     assert {ga, ca, gb, cb} <= t and fwd not in t
+
+
+def test_add_alias_nodes():
+    """An alias after every tensor node with two or more users (the users read
+    the alias) and after every returned node
+    (autoparallel/graph_passes/graph_utils.py:99-183, "v2")."""
+    import torch
+
+    from autoparallel_amd.graph_utils import add_alias_nodes
+
+    aten = torch.ops.aten
+    g = torch.fx.Graph()
+    x = g.placeholder("x")
+    x.meta["val"] = torch.empty(4, 4, device="meta")
+    a = g.call_function(aten.relu.default, (x,))
+    a.meta["val"] = torch.empty(4, 4, device="meta")
+    b = g.call_function(aten.add.Tensor, (a, x))
+    b.meta["val"] = torch.empty(4, 4, device="meta")
+    c = g.call_function(aten.mul.Tensor, (a, b))
+    c.meta["val"] = torch.empty(4, 4, device="meta")
+    g.output((c, b))
+    gm = add_alias_nodes(torch.fx.GraphModule(torch.nn.Module(), g))
+    gm.graph.lint()
+    nodes = list(gm.graph.nodes)
+    alias = [n for n in nodes if n.op == "call_function" and n.target is aten.alias.default]
+    # x (relu, add), relu (add, mul) and add (mul, output) fan out; mul and add's alias are returned
+    assert len(alias) == 5
+    of = lambda n: [al for al in alias if al.args[0] is n]
+    assert len(of(x)) == 1 and set(of(x)[0].users) == {a, b} and list(x.users) == of(x)
+    assert len(of(a)) == 1 and set(of(a)[0].users) == {b, c}
+    fan = of(b)[0]
+    out = nodes[-1]
+    returned = list(out.all_input_nodes)
+    assert all(r.target is aten.alias.default for r in returned)
+    # the returned add already fans out: its second alias takes over every user of the first, as in the reference
+    assert returned[0].args[0] is c and returned[1].args[0] is fan and c.args[1] is returned[1]
+    assert list(fan.users) == [returned[1]]
+    assert all(al.meta["val"].shape == (4, 4) for al in alias)
+    # the alias of a fanned-out node sits before its first user
+    assert nodes.index(of(x)[0]) < nodes.index(a)

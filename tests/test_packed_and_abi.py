@@ -241,6 +241,17 @@ def test_abi_host_helpers():
     m = _lib.ApcModel()
     assert lib.apc_device_limits(b"AMD Instinct MI355X", ctypes.byref(m)) == 0
     assert m.gmem_bw == O.MI355X_GMEM_BW and list(m.tflops)[:5] == [O.MI355X_TFLOPS[i] for i in range(5)]
+    # the whole device table of the reference, matched by substring in its order
+    for name, bw, tf in O.DEVICE_TABLE:
+        for full in (name, "NVIDIA " + name + " 80GB HBM3"):
+            assert lib.apc_device_limits(full.encode(), ctypes.byref(m)) == 0, full
+            assert m.gmem_bw == bw and list(m.tflops)[:5] == [float(tf.get(i, 0.0)) for i in range(5)], full
+    assert lib.apc_device_limits(b"NVIDIA PG509-210", ctypes.byref(m)) == 0 and m.tflops[3] == 312.0
+    assert lib.apc_device_limits(b"NVIDIA H100 and A100", ctypes.byref(m)) == 0 and m.tflops[0] == 67.0
+    # figures the reference's own documentation and tests quote
+    h100 = O.DeviceLimit.named("NVIDIA H100 80GB HBM3")
+    assert h100.tflops[3] == 989.0 and h100.tflops[1] == 494.0 and h100.gmem_bandwidth == 3.35 * 1024**4
+    assert O.DeviceLimit.named("AMD Instinct MI300X").tflops[1] == 653.7
     assert lib.apc_device_limits(b"Some Other GPU", ctypes.byref(m)) == _lib.load().apc_device_limits(b"x", ctypes.byref(m)) != 0
     assert b"Unsupported device" in lib.apc_last_error()
     # the host-side draw of the on-device assignment generator is deterministic and in range
