@@ -161,3 +161,123 @@ def test_fsdp_with_tensor_parallel_on_two_mesh_dims(meshes, model_type):
         p = sol[node]
         assert [s.placements for s in p.input_specs[:3]] == [(_S(0), _S(1))] * 3
         assert p.output_specs[0].placements == (_S(0), _S(1))
+
+
+class _TwoLinear(nn.Module):
+    def __init__(self, dim1, dim2, bias):
+        super().__init__()
+        self.linear1, self.linear2 = nn.Linear(dim1, dim2, bias=bias), nn.Linear(dim2, dim1, bias=bias)
+
+    def forward(self, x):
+        return self.linear2(torch.relu(self.linear1(x)))
+
+
+def _two_linear(mesh, dim1=1024, dim2=4096, bias=False, rows=None, memory=True):
+    """Model, constraints and defaults of tests/test_optimize_placement.py:518-556, 598-655."""
+    from torch._functorch.aot_autograd import aot_export_joint_with_descriptors
+    from torch._subclasses.fake_tensor import FakeTensorMode
+
+    from autoparallel_amd.cost_models import detect_nccl_topo_config, set_nccl_topo_config
+    from autoparallel_amd.graph_utils import add_alias_nodes
+    from autoparallel_amd.optimize_sharding import ShardingOptimizer
+
+    with FakeTensorMode():
+        with torch.device("cuda"):
+            m = _TwoLinear(dim1, dim2, bias)
+        x = torch.rand((2048 if rows is None else rows) * mesh.shape[0], dim1, device="cuda", requires_grad=True)
+        with contextlib.ExitStack() as stack:
+            gm = aot_export_joint_with_descriptors(stack, m, (x,)).graph_module
+    add_alias_nodes(gm)
+    set_nccl_topo_config(detect_nccl_topo_config(mesh, "H100"))
+    opt = ShardingOptimizer(gm, mesh, devices_per_host=8, device_name="H100")
+    batch = (Shard(0),) + (Replicate(),) * (mesh.ndim - 1)
+    opt.add_sharded_input_constraint([batch])
+    opt.add_sharded_output_constraint([batch])
+    if memory:
+        opt.add_parameter_memory_constraint(0.0, 1.0 / mesh.size())
+    return gm, opt
+
+
+def test_memory_budget_with_a_parameter_that_does_not_divide(meshes):
+    """:518-556: a bias of 280 elements on 256 ranks cannot be sharded all the
+    way; the budget takes each parameter's best achievable ratio, so the problem
+    stays feasible."""
+    from torch._functorch._aot_autograd.fx_utils import get_param_nodes
+
+    gm, opt = _two_linear(meshes[1], 1024, 280, bias=True, rows=8)
+    sol = opt.get_solution()
+    params = get_param_nodes(gm.graph)
+    assert len(params) == 4 and all(p in sol for p in params)
+
+
+def test_parameter_smaller_than_the_mesh_stays_replicated(meshes):
+    """:559-595: a parameter of 128 elements on 256 ranks."""
+    from torch._functorch.aot_autograd import aot_export_joint_with_descriptors
+    from torch._functorch._aot_autograd.fx_utils import get_param_nodes
+    from torch._subclasses.fake_tensor import FakeTensorMode
+
+    from autoparallel_amd.graph_utils import add_alias_nodes
+    from autoparallel_amd.optimize_sharding import ShardingOptimizer
+
+    class Model(nn.Module):
+        def __init__(self, dim):
+            super().__init__()
+            self.param = nn.Parameter(torch.rand(dim))
+
+        def forward(self, x):
+            return x + self.param
+
+    mesh = meshes[0]
+    with FakeTensorMode():
+        with torch.device("cuda"):
+            m = Model(128)
+        x = torch.rand(512, 128, device="cuda")
+        with contextlib.ExitStack() as stack:
+            gm = aot_export_joint_with_descriptors(stack, m, (x,)).graph_module
+    add_alias_nodes(gm)
+    opt = ShardingOptimizer(gm, mesh, devices_per_host=8, device_name="H100")
+    opt.add_sharded_input_constraint([(Shard(0),)])
+    opt.add_sharded_output_constraint([(Shard(0),)])
+    opt.add_parameter_memory_constraint(0.0, 1.0 / mesh.size())
+    sol = opt.get_solution()
+    for node in get_param_nodes(gm.graph):
+        assert sol[node].output_specs.placements == (Replicate(),)
+
+
+@pytest.mark.parametrize("memory_first", [True, False])
+def test_node_constraint_is_left_out_of_the_memory_budget(meshes, memory_first):
+    """:598-696: a parameter forced to Replicate does not make the sharding budget
+    infeasible, whichever constraint was added first, on the first solve and on a
+    re-solve."""
+    from torch._functorch._aot_autograd.fx_utils import get_param_nodes
+
+    gm, opt = _two_linear(meshes[0], memory=False)
+    node = get_param_nodes(gm.graph)[0]
+    if memory_first:
+        opt.add_parameter_memory_constraint(0.0, 1.0 / 256)
+        opt.add_node_constraint(node, placement=(Replicate(),))
+    else:
+        opt.add_node_constraint(node, placement=(Replicate(),))
+        opt.add_parameter_memory_constraint(0.0, 1.0 / 256)
+    assert opt.get_solution()[node].output_specs.placements == (Replicate(),)
+    assert opt.resolve()[node].output_specs.placements == (Replicate(),)
+
+
+def test_constraints_added_and_removed_between_solves(meshes):
+    """:699-843: a node constraint added after a solve is honoured by resolve();
+    removing it puts the parameter back under the budget (sharded again);
+    removing the memory rows by name keeps them from being rebuilt."""
+    from torch._functorch._aot_autograd.fx_utils import get_param_nodes
+
+    gm, opt = _two_linear(meshes[0])
+    params = get_param_nodes(gm.graph)
+    sol = opt.get_solution()
+    assert all(sol[p].output_specs.placements == (Shard(0),) for p in params)
+    names = opt.add_node_constraint(params[0], placement=(Replicate(),))
+    assert opt.resolve()[params[0]].output_specs.placements == (Replicate(),)
+    opt.remove_constraints(names)
+    assert opt.resolve()[params[0]].output_specs.placements == (Shard(0),)
+    opt.remove_constraints(["memory_constraint_high", "memory_constraint_low"])
+    opt.resolve()
+    assert "memory_constraint_high" not in opt.prob.constraints
+    assert "memory_constraint_low" not in opt.prob.constraints
