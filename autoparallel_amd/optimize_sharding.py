@@ -209,9 +209,56 @@ class ShardingOptimizer:
                 r.input_grad.append((nm[n], nm[g] if g is not None and g in nm else -1))
             for n, t in fx_utils.get_plain_output_and_tangent_nodes(self.graph).values():
                 r.output_tangent.append((nm[n], nm[t] if t is not None and t in nm else -1))
+            self._mark_pre_cast_nodes(r)
         except Exception:  # a graph without AOT descriptors has no forward/backward pairs
             logger.debug("no AOT descriptors on the graph: no forward/backward constraints")
         return r
+
+    # operators that stand for the mixed-precision cast of a parameter or its gradient
+    # (the reference's parametrization inserts torch.ops.autoparallel.dtype_cast)
+    dtype_cast_targets: set = set()
+
+    def _mark_pre_cast_nodes(self, r: GraphRoles) -> None:
+        """Nodes before the mixed-precision cast, on which a redistribution would
+        run in the larger dtype (autoparallel/optimize_sharding.py:1487-1606).
+        Forward: from a parameter along single-user, single-input nodes to a cast
+        that narrows the dtype, cast included.  Backward: from a gradient back
+        along single-input nodes, the cast and everything before it in that
+        chain except the first producer with more than one input."""
+        from torch._functorch._aot_autograd import fx_utils
+
+        casts = set(self.dtype_cast_targets)
+        ns = getattr(torch.ops, "autoparallel", None)
+        if ns is not None and hasattr(ns, "dtype_cast"):
+            casts.add(ns.dtype_cast.default)
+        if not casts:
+            return
+        nm = self.node_map
+        for param, grad in fx_utils.get_param_and_grad_nodes(self.graph).values():
+            n = param
+            while n.target not in casts:
+                users = list(n.users)
+                if len(users) != 1 or len(users[0].all_input_nodes) != 1:
+                    break
+                n = users[0]
+            if n.target in casts and n.meta["val"].dtype.itemsize < param.meta["val"].dtype.itemsize:
+                node = n
+                while node is not param:
+                    if node in nm:
+                        r.fwd_pre_cast.add(nm[node])
+                    node = node.all_input_nodes[0]
+            if grad is None:
+                continue
+            chain, n = [grad], grad
+            while len(n.all_input_nodes) == 1:
+                parent = n.all_input_nodes[0]
+                if len(parent.all_input_nodes) != 1:
+                    break
+                chain.append(parent)
+                n = parent
+            at = next((i for i, node in enumerate(chain) if node.target in casts), None)
+            if at is not None:
+                r.bwd_pre_cast.update(nm[node] for node in chain[at:] if node in nm)
 
     def _prefetchable(self, roles: GraphRoles) -> set:
         """(node_idx, argi) of edges whose producer is parameter-derived or whose

@@ -615,6 +615,71 @@ def test_encoder_layer_with_dropout_joint_graph(mesh):
     assert set(sol) == {n for n in opt.nodes if n.op != "output"}
 
 
+def test_collectives_stay_on_the_narrow_side_of_a_cast(mesh):
+    """fp32 parameters cast to bf16 for compute, gradients cast back to fp32
+    (what the reference's mixed-precision parametrization produces, with
+    aten._to_copy standing in for its cast operator): no redistribution on the
+    nodes before the forward cast, nor, when reduction is asked for in the wider
+    dtype, on the backward cast and the single-input nodes that precede it
+    (autoparallel/optimize_sharding.py:1487-1606)."""
+    from torch._functorch._aot_autograd import fx_utils
+    from torch._functorch.aot_autograd import aot_export_joint_with_descriptors
+    from torch._subclasses.fake_tensor import FakeTensorMode
+
+    from autoparallel_amd.optimize_sharding import ShardingOptimizer
+
+    class Mixed(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.w1 = nn.Parameter(torch.randn(256, 128))
+            self.w2 = nn.Parameter(torch.randn(128, 256))
+
+        def forward(self, x):
+            h = torch.relu(x @ self.w1.to(torch.bfloat16).t())
+            return (h @ self.w2.to(torch.bfloat16).t()).float().pow(2).mean()
+
+    with FakeTensorMode():
+        with torch.device("cuda"):
+            m = Mixed()
+        x = torch.randn(64, 128, device="cuda", dtype=torch.bfloat16)
+        with contextlib.ExitStack() as stack:
+            gm = aot_export_joint_with_descriptors(stack, m, (x,)).graph_module
+    cast = torch.ops.aten._to_copy.default
+    pairs = list(fx_utils.get_param_and_grad_nodes(gm.graph).values())
+    assert len(pairs) == 2 and all(g is not None and g.target is cast for _, g in pairs)
+    old = ShardingOptimizer.dtype_cast_targets
+    ShardingOptimizer.dtype_cast_targets = {cast}
+    try:
+        plain = ShardingOptimizer(gm, mesh, devices_per_host=8, device_name="AMD Instinct MI355X")
+        wide = ShardingOptimizer(gm, mesh, True, devices_per_host=8, device_name="AMD Instinct MI355X")
+    finally:
+        ShardingOptimizer.dtype_cast_targets = old
+    for opt in (plain, wide):
+        roles = opt._packed.roles
+        fwd = {opt.nodes[i] for i in roles.fwd_pre_cast}
+        assert fwd == {next(iter(p.users)) for p, _ in pairs} and all(n.target is cast for n in fwd)
+        bwd = {opt.nodes[i] for i in roles.bwd_pre_cast}
+        # the cast and the transposes between it and the weight-gradient matmul, which stays out
+        assert {g for _, g in pairs} <= bwd and {n.target for n in bwd} == {cast, torch.ops.aten.t.default}
+        heads = [n for n in bwd if n.all_input_nodes[0] not in bwd]
+        assert len(heads) == 2 and all(n.all_input_nodes[0].target is torch.ops.aten.mm.default for n in heads)
+        names = list(opt.prob.constraints)
+        n_fwd = sum(1 for n in names if n.startswith("fwd_param_dtype_"))
+        n_bwd = sum(1 for n in names if n.startswith("grad_reduce_dtype_"))
+        comm = opt._core.coef.comm
+        keys = opt._packed.entry_keys()
+        on = lambda idx: int(((comm > 0) & np.isin(keys[:, 0], list(idx))).sum())
+        assert n_fwd == on(roles.fwd_pre_cast) > 0
+        assert n_bwd == (on(roles.bwd_pre_cast) if opt is wide else 0)
+        sol = opt.get_solution()
+        for p, g in pairs:
+            c = next(iter(p.users))
+            assert sol[c].input_specs[0].placements == sol[p].output_specs.placements  # gathered after the cast
+        if opt is wide:
+            for n in bwd:  # reduced after the cast: nothing moves on the way to it
+                assert sol[n].input_specs[0].placements == sol[n.all_input_nodes[0]].output_specs.placements
+
+
 def test_hf_llama3_8b_layers_joint_graph():
     """Llama-3-8B as transformers defines it (d 4096, 32 query / 8 key-value heads,
     SwiGLU 14336, RMSNorm, rotary embedding, vocab 128256, bf16), four of its
