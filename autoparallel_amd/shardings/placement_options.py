@@ -8,7 +8,7 @@ it with the reference's post-processing — tensor-meta fill
 (autoparallel/shardings/propagation_rules.py:127-158), de-duplication
 (placement_options.py:151-170) — and the few rules DTensor lacks or refuses
 (getitem, strict views, alias, two-operand einsum, operators without tensor
-inputs: propagation_rules.py:412-554; local_map regions: placement_options.py:380-490; all-Replicate fallback:
+inputs: propagation_rules.py:412-554; local_map regions and flex_attention: placement_options.py:380-650; all-Replicate fallback:
 dtensor_sharding_helpers.py:364-383).  Its output is input data for the cost
 engine.  Input/parameter options are enumerated on the device
 (apc_enumerate_input_options).
@@ -494,6 +494,61 @@ def _alias_rule(mesh, node, src: OpStrategy) -> OpStrategy:
     return OpStrategy(sts)
 
 
+def _is_flex_attention(node) -> bool:
+    t = node.target
+    return isinstance(t, torch._ops.HigherOrderOperator) and t.name() in ("flex_attention", "flex_attention_backward")
+
+
+def _flex_attention_rule(mesh, node) -> OpStrategy:
+    """flex_attention and its backward: attention is independent per (batch,
+    head), so every combination of {Replicate, Shard(0), Shard(1)} over the mesh
+    dims is a strategy.  A tensor takes a Shard only where it can (more than one
+    element on that dim, the query's extent a multiple of it, itself a multiple
+    of the mesh dim: grouped key/value heads, broadcast dims); the buffers the
+    score and mask functions index, and tensors of rank below two, are Replicate
+    (autoparallel/shardings/placement_options.py:493-650)."""
+    import inspect
+
+    from torch._higher_order_ops.flex_attention import (
+        flex_attention_backward_fake_tensor_mode,
+        flex_attention_fake_impl,
+    )
+
+    impl = flex_attention_fake_impl if node.target.name() == "flex_attention" else flex_attention_backward_fake_tensor_mode
+    params = list(inspect.signature(impl).parameters)
+    buffers = set()
+    for name in ("score_mod_other_buffers", "mask_mod_other_buffers"):
+        if name in params and params.index(name) < len(node.args):
+            arg = node.args[params.index(name)]
+            if isinstance(arg, (tuple, list)):
+                buffers.update(x for x in tree_flatten(arg)[0] if isinstance(x, torch.fx.Node))
+    tensors = [(a, a.meta["val"]) for a in tree_flatten(node.args)[0]
+               if isinstance(a, torch.fx.Node) and isinstance(a.meta.get("val"), torch.Tensor)]
+    q = node.args[0].meta["val"]
+    ref = {0: q.shape[0], 1: q.shape[1]}
+    rep = (Replicate(),) * mesh.ndim
+
+    def fit(t, plc):
+        out = []
+        for size, p in zip(mesh.shape, plc):
+            if p.is_shard() and p.dim in ref:
+                n = t.shape[p.dim]
+                p = p if n > 1 and ref[p.dim] % n == 0 and n % size == 0 else Replicate()
+            out.append(p)
+        return tuple(out)
+
+    outs = node.meta["val"]
+    assert isinstance(outs, (tuple, list))
+    sts = []
+    for plc in itertools.product((Replicate(), Shard(0), Shard(1)), repeat=mesh.ndim):
+        ins = [DTensorSpec(mesh, rep if (a in buffers or t.ndim < 2) else fit(t, plc), tensor_meta=_tensor_meta(t))
+               for a, t in tensors]
+        out_specs = tuple(DTensorSpec(mesh, fit(o, plc), tensor_meta=_tensor_meta(o)) if isinstance(o, torch.Tensor) else None
+                          for o in outs)
+        sts.append(OpSpec(out_specs, input_specs=tuple(ins)))
+    return OpStrategy(sts)
+
+
 def _without_partial(a):
     """The argument with its Partial candidates left out (itself if it has none, or nothing else)."""
     if isinstance(a, TupleStrategy):
@@ -557,6 +612,10 @@ def get_placement_options_for_node(mesh, node, producers: List[OpStrategy], arg_
     if node.meta.get("local_map_kwargs"):
         assert not node.kwargs
         return _local_map_rule(mesh, node, schema_args, node.meta["local_map_kwargs"])
+    if _is_flex_attention(node):
+        out = _flex_attention_rule(mesh, node)
+        fill_redistribute_cost(out, producers)
+        return out
     try:
         key = (mesh, node.target, _fingerprint(schema_args),
                _fingerprint({k: v for k, v in node.kwargs.items() if not isinstance(v, torch.fx.Node)}),

@@ -387,3 +387,45 @@ def test_select_takes_negative_dim_and_index(meshes):
         outs.append(_plcs(get_placement_options_for_node(mesh, node, [src], [x.meta["val"]], (src, dim, index))))
         assert fallback_nodes == before
     assert outs[0] == outs[1] and (((Shard(0), Shard(2)),), (Shard(0), Shard(1))) in outs[0]
+
+
+def test_flex_attention_strategies(meshes):
+    """flex_attention: {Replicate, Shard(batch), Shard(head)} per mesh dim; grouped
+    key/value heads shard only where they divide; block-mask tensors and the
+    buffers of the score function are Replicate
+    (autoparallel/shardings/placement_options.py:493-650).  Mesh (32, 8), 64 query
+    heads over 8 key/value heads, batch 64."""
+    from torch._higher_order_ops.flex_attention import flex_attention
+
+    from autoparallel_amd.shardings.placement_options import get_placement_options_for_node
+
+    mesh = meshes[1]
+    R, S = Replicate(), Shard
+    g = torch.fx.Graph()
+    mk = lambda name, *shape, dtype=torch.bfloat16: (lambda n: (n.meta.__setitem__("val", torch.empty(*shape, dtype=dtype, device="meta")), n)[1])(g.placeholder(name))
+    q, k, v = mk("q", 64, 64, 128, 32), mk("k", 64, 8, 128, 32), mk("v", 64, 8, 128, 32)
+    kv_num = mk("kv_num_blocks", 1, 1, 4, dtype=torch.int32)
+    kv_idx = mk("kv_indices", 1, 1, 4, 4, dtype=torch.int32)
+    bias = mk("bias", 64, 128)
+    score_mod = g.get_attr("score_mod")
+    mask_mod = g.get_attr("mask_mod")
+    block_mask = (128, 128, kv_num, kv_idx, None, None, None, None, None, None, 32, 32, mask_mod)
+    node = g.call_function(flex_attention, (q, k, v, score_mod, block_mask, 0.17, {}, (bias,), ()))
+    node.meta["val"] = (torch.empty(64, 64, 128, 32, dtype=torch.bfloat16, device="meta"),
+                        torch.empty(64, 64, 128, device="meta"), torch.empty(64, 64, 128, device="meta"))
+    tens = [q, k, v, kv_num, kv_idx, bias]
+    cands = [_candidates(mesh, tuple(t.meta["val"].shape), [(R, R), (S(0), R)]) for t in tens]
+    out = get_placement_options_for_node(mesh, node, cands, [t.meta["val"] for t in tens], None)
+    assert len(out.strategies) == 9
+    by_q = {st.input_specs[0].placements: st for st in out.strategies}
+    assert set(by_q) == set(__import__("itertools").product((R, S(0), S(1)), repeat=2))
+    for plc, st in by_q.items():
+        ins = [s.placements for s in st.input_specs]
+        # 8 key/value heads: Shard(1) holds on the mesh dim of 8 only, not on the one of 32
+        kv = tuple(R if (p.is_shard() and p.dim == 1 and n != 8) else p for p, n in zip(plc, mesh.shape))
+        assert ins[1] == ins[2] == kv
+        assert ins[3] == ins[4] == (R, R)  # block-mask tensors have extent 1 on batch and heads
+        assert ins[5] == (R, R)            # a buffer of the score function
+        assert [s.placements for s in st.output_specs] == [plc, plc, plc]
+        assert [len(r) for r in st.redistribute_cost] == [2] * 6
+    assert by_q[(S(0), S(1))].output_specs[1].tensor_meta.shape == (64, 64, 128)
