@@ -680,6 +680,59 @@ def test_collectives_stay_on_the_narrow_side_of_a_cast(mesh):
                 assert sol[n].input_specs[0].placements == sol[n.all_input_nodes[0]].output_specs.placements
 
 
+def test_hf_gpt2_layers_under_the_default_memory_budget(mesh):
+    """Two GPT-2 layers prepared as the reference prepares its graph (alias nodes)
+    with the batch-sharded input and the default parameter budget of 1 / mesh size
+    (autoparallel/api.py:371-382): every parameter ends fully sharded, the
+    layer-norm weights too, whose gradients leave layer_norm_backward Partial and
+    reach their Shard on the alias edge."""
+    transformers = pytest.importorskip("transformers")
+    from torch._functorch._aot_autograd.fx_utils import get_param_and_grad_nodes
+    from torch._functorch.aot_autograd import aot_export_joint_with_descriptors
+    from torch._subclasses.fake_tensor import FakeTensorMode
+    from torch.distributed.tensor.placement_types import Replicate, Shard
+
+    from autoparallel_amd.graph_utils import add_alias_nodes
+    from autoparallel_amd.optimize_sharding import ShardingOptimizer
+
+    class Wrap(nn.Module):
+        def __init__(self, lm):
+            super().__init__()
+            self.lm = lm
+
+        def forward(self, ids):
+            t = self.lm.transformer
+            x = t.wte(ids) + t.wpe(torch.arange(ids.shape[1], device=ids.device))[None]
+            for blk in t.h:
+                out = blk(x)
+                x = out[0] if isinstance(out, tuple) else out
+            logits = self.lm.lm_head(t.ln_f(x))
+            return torch.nn.functional.cross_entropy(
+                logits[:, :-1].reshape(-1, logits.shape[-1]).float(), ids[:, 1:].reshape(-1))
+
+    cfg = transformers.GPT2Config(n_layer=2, attn_pdrop=0.0, embd_pdrop=0.0, resid_pdrop=0.0, use_cache=False,
+                                  attn_implementation="sdpa")
+    with FakeTensorMode():
+        with torch.device("cuda"):
+            m = Wrap(transformers.GPT2LMHeadModel(cfg))
+        ids = torch.randint(0, cfg.vocab_size, (8, 1024), device="cuda")
+        with contextlib.ExitStack() as stack:
+            gm = aot_export_joint_with_descriptors(stack, m, (ids,)).graph_module
+    add_alias_nodes(gm)
+    opt = ShardingOptimizer(gm, mesh, devices_per_host=8, device_name="AMD Instinct MI355X")
+    opt.add_sharded_input_constraint([(Shard(0), Replicate())])
+    opt.add_parameter_memory_constraint(0.0, 1.0 / mesh.size())
+    sol = opt.get_solution()
+    pairs = list(get_param_and_grad_nodes(gm.graph).values())
+    assert len(pairs) >= 28
+    for p, g in pairs:
+        plc = sol[p].output_specs.placements
+        assert all(x.is_shard() for x in plc), (p.name, plc)
+        assert g.target is torch.ops.aten.alias.default and sol[g].output_specs.placements == plc
+    norm_w = [p for p, g in pairs if p.meta["val"].shape == (768,)]
+    assert len(norm_w) >= 10
+
+
 def test_hf_llama3_8b_layers_joint_graph():
     """Llama-3-8B as transformers defines it (d 4096, 32 query / 8 key-value heads,
     SwiGLU 14336, RMSNorm, rotary embedding, vocab 128256, bf16), four of its
