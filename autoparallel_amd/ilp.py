@@ -13,7 +13,6 @@ receive the identical matrix.
 """
 from __future__ import annotations
 
-import collections
 import re
 from typing import Dict, List, Optional, Sequence, Tuple
 

@@ -15,14 +15,12 @@ from __future__ import annotations
 import collections.abc
 import logging
 import operator
-import warnings
 from typing import Any, Dict, Iterator, List, Optional, Tuple
 
 import numpy as np
 import torch
 from torch.distributed.tensor._dtensor_spec import DTensorSpec
 from torch.distributed.tensor._op_schema import OpSpec, OpStrategy
-from torch.distributed.tensor.placement_types import Replicate, Shard
 from torch.utils._pytree import tree_flatten, tree_map_only
 
 from . import fx_programs
@@ -30,7 +28,7 @@ from .cost_models import collective_runtime_estimation as _cre
 from .dtensor_bridge import devices_per_host as _mesh_dph
 from .dtensor_bridge import placement_codes
 from .engine import detect_device_name
-from .packed import GraphBuilder, NodeDesc, PackedGraph
+from .packed import GraphBuilder, PackedGraph
 from .sharding_problem import GraphRoles, PackedShardingOptimizer
 from .shardings.placement_options import _create_all_options, get_placement_options_for_node
 

@@ -26,7 +26,7 @@ from torch.distributed.tensor import DTensor
 from torch.distributed.tensor._dtensor_spec import DTensorSpec, TensorMeta
 from torch.distributed.tensor._op_schema import OpSchema, OpSpec, OpStrategy, TupleStrategy
 from torch.distributed.tensor.placement_types import Partial, Replicate, Shard
-from torch.utils._pytree import tree_flatten, tree_map_only
+from torch.utils._pytree import tree_flatten
 
 from .. import _lib
 
