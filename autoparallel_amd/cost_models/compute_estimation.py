@@ -130,6 +130,28 @@ def _has_zero_cost(node) -> bool:
     return bool(node.target.is_view) or node.target is torch.ops.aten._unsafe_view.default
 
 
+def _unsharded_strategy(node):
+    """Stand-in strategy for an operator evaluated on its traced arguments:
+    Replicate on a mesh of one device (the local shape is the traced shape)."""
+    from types import SimpleNamespace
+
+    from torch.distributed.tensor._dtensor_spec import TensorMeta
+    from torch.distributed.tensor.placement_types import Replicate
+    from torch.utils._pytree import tree_flatten
+
+    one = SimpleNamespace(shape=(1,), ndim=1)
+    spec = lambda t: SimpleNamespace(mesh=one, placements=(Replicate(),),
+                                     tensor_meta=TensorMeta(t.shape, t.stride(), t.dtype))
+    ins = [spec(a.meta["val"]) for a in tree_flatten(node.args)[0]
+           if isinstance(a, torch.fx.Node) and isinstance(a.meta.get("val"), torch.Tensor)]
+    val = node.meta.get("val")
+    if isinstance(val, torch.Tensor):
+        outs = spec(val)
+    else:
+        outs = tuple(spec(v) if isinstance(v, torch.Tensor) else None for v in val)
+    return SimpleNamespace(input_specs=ins, output_specs=outs)
+
+
 def runtime_cost_vector(node, strategies) -> np.ndarray:
     """estimate_strategy_runtime_cost for every strategy of one node: one
     compute slot evaluated on the device."""
@@ -137,8 +159,12 @@ def runtime_cost_vector(node, strategies) -> np.ndarray:
         return np.zeros(len(strategies))
     from .collective_runtime_estimation import _device_name, _dph
 
-    mesh = next(s for st in strategies for s in st.input_specs if s is not None).mesh
-    b = GraphBuilder(tuple(mesh.shape), _dph(mesh))
+    mesh = next((s for st in strategies for s in st.input_specs if s is not None), None)
+    if mesh is None:  # no tensor argument: a factory, priced on its output alone
+        mesh = next(s for s in (lambda o: o if isinstance(o, (tuple, list)) else (o,))(strategies[0].output_specs)
+                    if s is not None)
+    mesh = mesh.mesh
+    b = GraphBuilder(tuple(mesh.shape), _dph(mesh) if hasattr(mesh, "device_type") else 1)
     desc = fx_programs.describe_node(node, strategies, b)
     prods = []
     n_args = len(desc.in_specs[0])
@@ -165,7 +191,9 @@ def estimate_strategy_runtime_cost(node, strategy):
     if _has_zero_cost(node):
         return 0
     if strategy is None:
-        raise NotImplementedError("unsharded runtime estimates (strategy=None) are not built")
+        # the operator on its arguments as traced, no sharding
+        # (compute_estimation.py:334-339): every tensor argument whole on one device
+        return float(runtime_cost_vector(node, [_unsharded_strategy(node)])[0])
     key = None
     try:
         key = (node.target, tuple((s.placements, s.tensor_meta) for s in strategy.input_specs),

@@ -368,3 +368,51 @@ def estimate_graph_metrics(
         total_time=float(times[0, 0]), compute_time=float(times[0, 1]),
         communication_time=float(times[0, 2]), exposed_comm_time=float(times[0, 3]),
         peak_memory=int(peak[0]))
+
+
+def make_custom_runtime_estimation(mesh):
+    """The runtime estimator the reference hands to its lowered-graph passes
+    (graph_passes/debug_helpers.py:170-224): a collective is priced with
+    ``collective_comm_cost`` on the mesh dim its process group belongs to (the
+    flattened mesh when the group is none of the mesh's own; all-gather volume
+    is the input shard times the group size), ``wait_tensor`` and unknown
+    collectives cost nothing, and every other operator gets the unsharded
+    compute estimate.  ``override_size`` (GiB) replaces the traced volume."""
+    from torch._inductor.fx_passes.overlap_scheduling import get_group_name
+    from torch.distributed.tensor._collective_utils import MeshTopoInfo
+
+    from .cost_models.collective_runtime_estimation import collective_comm_cost
+    from .cost_models.compute_estimation import estimate_strategy_runtime_cost
+
+    c10d, dt = torch.ops._c10d_functional, torch.ops._dtensor
+    kinds = {
+        c10d.all_gather_into_tensor.default: "allgather",
+        c10d.all_gather_into_tensor_out.default: "allgather",
+        c10d.reduce_scatter_tensor.default: "reduce_scatter",
+        c10d.all_reduce.default: "allreduce",
+        dt.shard_dim_alltoall.default: "all_to_all",
+    }
+
+    def custom_runtime_estimation(node: fx.Node, override_size=None):
+        if node.op != "call_function" or not isinstance(node.target, torch._ops.OpOverload):
+            return 0
+        if not is_communication_node(node):
+            return estimate_strategy_runtime_cost(node, None)
+        kind = kinds.get(node.target)
+        if kind is None:  # wait_tensor and collectives the cost model does not know
+            return 0
+        group = get_group_name(node)
+        names = tuple(g.group_name for g in mesh.get_all_groups())
+        if group in names:
+            cost_mesh, dim = mesh, names.index(group)
+        elif mesh.ndim > 1:
+            cost_mesh, dim = mesh._flatten(), 0
+        else:
+            return 0
+        t = node.args[0].meta["val"]
+        nbytes = t.numel() * t.itemsize if override_size is None else int(override_size * 2**30)
+        if kind == "allgather":
+            nbytes *= cost_mesh.shape[dim]
+        return collective_comm_cost(kind, nbytes, tuple(cost_mesh.shape), dim, MeshTopoInfo.build_from_mesh(cost_mesh))
+
+    return custom_runtime_estimation

@@ -733,6 +733,30 @@ def test_hf_gpt2_layers_under_the_default_memory_budget(mesh):
     assert len(norm_w) >= 10
 
 
+def test_unsharded_runtime_estimate(mesh):
+    """estimate_strategy_runtime_cost(node, None) prices the operator on its
+    traced arguments (autoparallel/cost_models/compute_estimation.py:334-339,
+    438-493): the same figure as the all-Replicate strategy, whose local shapes
+    are the traced ones."""
+    from autoparallel_amd.cost_models.compute_estimation import estimate_strategy_runtime_cost
+    from autoparallel_amd.optimize_sharding import ShardingOptimizer
+
+    gm = _joint_graph()
+    opt = ShardingOptimizer(gm, mesh, devices_per_host=8, device_name="AMD Instinct MI355X")
+    checked = 0
+    for node in gm.graph.nodes:
+        if node.op != "call_function" or node not in opt.strats:
+            continue
+        rep = [st for st in opt.strats[node].strategies
+               if all(s is None or all(p.is_replicate() for p in s.placements) for s in st.input_specs)]
+        if not rep:
+            continue
+        a, b = estimate_strategy_runtime_cost(node, None), estimate_strategy_runtime_cost(node, rep[0])
+        assert a == b, (node, a, b)
+        checked += a > 0
+    assert checked >= 4
+
+
 def test_hf_llama3_8b_layers_joint_graph():
     """Llama-3-8B as transformers defines it (d 4096, 32 query / 8 key-value heads,
     SwiGLU 14336, RMSNorm, rotary embedding, vocab 128256, bf16), four of its

@@ -119,3 +119,85 @@ def test_bad_arguments_are_refused():
     rc = est.lib.apc_schedule_metrics(C.byref(s), None, 2, C.c_void_p(out.data_ptr()), None,
                                       C.c_void_p(out.data_ptr()), C.c_void_p(pk.data_ptr()), None)
     assert rc == -1 and b"one schedule" in est.lib.apc_last_error()
+
+
+def test_runtime_estimator_of_a_lowered_graph():
+    """make_custom_runtime_estimation (reference: graph_passes/debug_helpers.py:170-224):
+    collectives priced on the mesh dim of their group with the oracle's
+    alpha-beta forms (all-gather on the gathered volume), waits free, compute
+    nodes at the unsharded roofline estimate; and the whole graph through
+    estimate_graph_metrics with it."""
+    import torch.distributed as dist
+    import torch.fx as fx
+    from torch._subclasses.fake_tensor import FakeTensorMode
+    from torch.distributed.device_mesh import init_device_mesh
+    from torch.testing._internal.distributed.fake_pg import FakeStore
+
+    from autoparallel_amd.cost_models import collective_runtime_estimation as cre
+    from autoparallel_amd.schedule_metrics import estimate_graph_metrics, make_custom_runtime_estimation
+    from oracle import cost_oracle as O
+
+    if not torch.cuda.is_available():
+        pytest.skip("needs a GPU")
+    had = dist.is_initialized()
+    if had:
+        dist.destroy_process_group()
+    dist.init_process_group("fake", store=FakeStore(), rank=0, world_size=16)
+    try:
+        mesh = init_device_mesh("cpu", (2, 8), mesh_dim_names=("dp", "tp"))
+        cre.configure(8, "AMD Instinct MI355X")
+        names = [g.group_name for g in mesh.get_all_groups()]
+        ops = torch.ops
+        g = fx.Graph()
+        with FakeTensorMode():
+            x = g.placeholder("x")
+            x.meta["val"] = torch.empty(512, 1024, dtype=torch.bfloat16, device="cuda")
+            w = g.placeholder("w")
+            w.meta["val"] = torch.empty(1024, 2048, dtype=torch.bfloat16, device="cuda")
+            ag = g.call_function(ops._c10d_functional.all_gather_into_tensor.default, (x, 8, names[1]))
+            ag.meta["val"] = torch.empty(4096, 1024, dtype=torch.bfloat16, device="cuda")
+            wt = g.call_function(ops._c10d_functional.wait_tensor.default, (ag,))
+            wt.meta["val"] = ag.meta["val"]
+            mm = g.call_function(ops.aten.mm.default, (wt, w))
+            mm.meta["val"] = torch.empty(4096, 2048, dtype=torch.bfloat16, device="cuda")
+            ar = g.call_function(ops._c10d_functional.all_reduce.default, (mm, "sum", names[0]))
+            ar.meta["val"] = mm.meta["val"]
+            wt2 = g.call_function(ops._c10d_functional.wait_tensor.default, (ar,))
+            wt2.meta["val"] = mm.meta["val"]
+            other = g.call_function(ops._c10d_functional.all_reduce.default, (wt2, "sum", "not a group of this mesh"))
+            other.meta["val"] = mm.meta["val"]
+            v = g.call_function(ops.aten.view.default, (other, [2048, 4096]))
+            v.meta["val"] = torch.empty(2048, 4096, dtype=torch.bfloat16, device="cuda")
+            g.output((v,))
+        gm = fx.GraphModule(torch.nn.Module(), g)
+        est = make_custom_runtime_estimation(mesh)
+        from torch.distributed.tensor._collective_utils import MeshTopoInfo
+
+        def topo_of(m):  # bandwidth and latency as torch derives them for this mesh on this host, as the reference passes them
+            t, mt = O.Topo(tuple(m.shape), 8), MeshTopoInfo.build_from_mesh(m)
+            t.bw, t.lat = list(mt.mesh_dim_bandwidth), list(mt.mesh_dim_latency)
+            return t
+
+        topo = topo_of(mesh)
+        dev = O.DeviceLimit()
+        want_ag = O.collective_comm_cost("allgather", 512 * 1024 * 2 * 8, topo, 1)
+        want_ar = O.collective_comm_cost("allreduce", 4096 * 2048 * 2, topo, 0)
+        flat = O.collective_comm_cost("allreduce", 4096 * 2048 * 2, topo_of(mesh._flatten()), 0)  # the flattened mesh
+        flops = 2 * 4096 * 1024 * 2048
+        nbytes = 2 * (4096 * 1024 + 1024 * 2048 + 4096 * 2048)
+        want_mm = O.roofline_cost(flops, nbytes, 3, dev)
+        assert want_mm == max(flops / (2516.6e12) * 1e6 / 0.70, O.compute_read_write_time(nbytes, dev))
+        assert est(ag) == want_ag and est(ar) == want_ar and est(other) == flat
+        assert est(wt) == 0 and est(v) == 0 and est(x) == 0
+        assert est(mm) == want_mm
+        assert est(ag, override_size=0.5) == O.collective_comm_cost("allgather", 2**29 * 8, topo, 1)
+        m = estimate_graph_metrics(gm, est)
+        assert m.compute_time == want_mm and m.communication_time == want_ag + want_ar + flat
+        assert abs(m.exposed_comm_time - (want_ag + want_ar)) < 1e-9 * m.exposed_comm_time  # both waited for right away; the last one never
+        # the chain end to end (the last collective runs out on its own stream), plus 1 us of launch per node passed
+        chain = want_ag + want_mm + want_ar + flat
+        assert chain < m.total_time <= chain + len(list(gm.graph.nodes))
+    finally:
+        dist.destroy_process_group()
+        if had:
+            dist.init_process_group("fake", store=FakeStore(), rank=0, world_size=8)
