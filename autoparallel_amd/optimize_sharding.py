@@ -134,6 +134,43 @@ class DecisionVars(collections.abc.Mapping):
         return self._keys.shape[0]
 
 
+class _Variables(collections.abc.Mapping):
+    """``pulp_variables`` of the reference (autoparallel/optimize_sharding.py:412-444):
+    key -> an object with the variable's name and, after a solve, ``varValue``.
+    The variables themselves are columns of the packed problem."""
+
+    class _Var:
+        __slots__ = ("name", "index", "_prob")
+
+        def __init__(self, name, index, prob):
+            self.name, self.index, self._prob = name, index, prob
+
+        @property
+        def varValue(self):
+            x = self._prob.x
+            return None if x is None else float(x[self.index])
+
+        def value(self):
+            return self.varValue
+
+    def __init__(self, opt: "ShardingOptimizer"):
+        self._opt = opt
+
+    def __getitem__(self, key):
+        opt = self._opt
+        col = opt.decision_vars._col(opt.cluster_links.get(key, key)) if key in opt.decision_vars else None
+        if col is None:
+            raise KeyError(key)
+        v, a, o, j = key
+        return self._Var(f"n={opt.nodes[v]},s={v},arg={a},output_p={o},input_p={j}", col, opt.prob)
+
+    def __iter__(self):
+        return iter(self._opt.decision_vars)
+
+    def __len__(self):
+        return len(self._opt.decision_vars)
+
+
 class ShardingOptimizer:
     def __init__(self, gm, mesh, force_grad_reduce_in_higher_precision: bool = False,
                  repeated_subgraphs: bool = False, devices_per_host: Optional[int] = None,
@@ -154,6 +191,37 @@ class ShardingOptimizer:
         self.node_map = {n: i for i, n in enumerate(self.nodes)}
         self.decision_vars = self._build_decision_vars()
         self.validate()
+
+    # -- accessors of the reference's class ----------------------------------------
+    @property
+    def pulp_variables(self) -> _Variables:
+        return _Variables(self)
+
+    @property
+    def _concrete_to_orig(self) -> Dict[torch.fx.Node, torch.fx.Node]:
+        """Graphs are planned as given (no symbolic sizes are made concrete
+        here), so the two graphs of the reference are one."""
+        return {n: n for n in self.nodes}
+
+    _orig_to_concrete = _concrete_to_orig
+
+    def _normalize_node(self, node):
+        return node
+
+    def get_strategy(self, node):
+        return self.strats[self._normalize_node(node)]
+
+    def _get_pulp_variable(self, key):
+        return self.pulp_variables[key]
+
+    def _resolve_decision_var(self, key) -> DecisionVar:
+        return self.decision_vars[key]
+
+    @classmethod
+    def load(cls, path: str):
+        """A saved optimizer, reopened without the model, mesh or process group
+        (the packed form: PackedShardingOptimizer)."""
+        return PackedShardingOptimizer.load(path)
 
     # -- strategies ---------------------------------------------------------------
     def build_sharding_metadata(self) -> Dict[torch.fx.Node, Any]:

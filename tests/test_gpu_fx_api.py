@@ -76,6 +76,14 @@ def test_sharding_optimizer_on_joint_graph(mesh):
     sol = opt.get_solution()
     assert set(sol) == {n for n in opt.nodes if n.op != "output"}
     base = opt._core.objective_value
+    # the reference's accessors: variables by key with their solved values, strategies by node
+    chosen = set(opt.selected_keys)
+    assert all(opt.pulp_variables[key].varValue == 1.0 for key in list(chosen)[:50])
+    others = [key for key in keys[:400] if key not in chosen]
+    assert others and all(opt.pulp_variables[key].varValue == 0.0 for key in others)
+    assert opt.pulp_variables[k].name == f"n={opt.nodes[k[0]]},s={k[0]},arg={k[1]},output_p={k[2]},input_p={k[3]}"
+    assert opt.get_strategy(node) is opt.strats[node] and opt._concrete_to_orig[node] is node
+    assert opt._resolve_decision_var(k).cost == dv.cost
     total = opt._compute_solution_cost(sol)["total"]
     assert np.isclose(total, base, rtol=1e-9)  # no clusters, no inf entries selected
     # parameters and their gradients get the same placement
