@@ -134,6 +134,60 @@ class DecisionVars(collections.abc.Mapping):
         return self._keys.shape[0]
 
 
+def concretize_symint(val):
+    """A SymInt becomes its hint; one without a hint (unbacked) and anything
+    else pass through (autoparallel/optimize_sharding.py:111-120)."""
+    if isinstance(val, torch.SymInt):
+        hint = val.node.hint
+        return val if hint is None else hint
+    return val
+
+
+def concretize_args(args):
+    """The same tree with SymInts replaced by their hints and fake tensors of
+    symbolic shape replaced by fake tensors of the hinted shape and stride (left
+    alone when a size has no hint) (:123-150)."""
+    from torch._subclasses.fake_tensor import FakeTensor
+
+    def one(x):
+        if isinstance(x, torch.SymInt):
+            return concretize_symint(x)
+        if isinstance(x, FakeTensor) and any(isinstance(d, torch.SymInt) for d in x.shape):
+            shape = [concretize_symint(d) for d in x.shape]
+            stride = [concretize_symint(d) for d in x.stride()]
+            if not all(isinstance(d, int) for d in shape):
+                return x
+            with x.fake_mode:
+                return torch.empty_strided(shape, stride, dtype=x.dtype, device=x.device)
+        return x
+
+    return tree_map_only((torch.SymInt, FakeTensor), one, args)
+
+
+def concretize_gm(gm):
+    """(copy of gm with every ``meta['val']`` made concrete, original -> copy,
+    copy -> original).  The planner works on the copy; the caller keeps the
+    symbolic graph (:162-189)."""
+    graph = torch.fx.Graph()
+    to_concrete: Dict[torch.fx.Node, torch.fx.Node] = {}
+    for node in gm.graph.nodes:
+        twin = graph.node_copy(node, lambda n: to_concrete[n])
+        to_concrete[node] = twin
+        if twin.meta.get("val") is not None:  # node_copy made a shallow copy of meta
+            twin.meta["val"] = concretize_args(twin.meta["val"])
+    return torch.fx.GraphModule(gm, graph), to_concrete, {v: k for k, v in to_concrete.items()}
+
+
+def _has_symbolic_sizes(gm) -> bool:
+    for node in gm.graph.nodes:
+        for x in tree_flatten(node.meta.get("val"))[0]:
+            if isinstance(x, torch.SymInt):
+                return True
+            if isinstance(x, torch.Tensor) and any(isinstance(d, torch.SymInt) for d in tuple(x.shape) + tuple(x.stride())):
+                return True
+    return False
+
+
 class _Variables(collections.abc.Mapping):
     """``pulp_variables`` of the reference (autoparallel/optimize_sharding.py:412-444):
     key -> an object with the variable's name and, after a solve, ``varValue``.
@@ -176,6 +230,14 @@ class ShardingOptimizer:
                  repeated_subgraphs: bool = False, devices_per_host: Optional[int] = None,
                  device_name: Optional[str] = None):
         self.orig_gm = gm
+        # planning needs concrete sizes: a graph with symbolic ones is planned on a
+        # copy at their hints, and plans are handed back on the caller's nodes
+        # (autoparallel/optimize_sharding.py:228-237); a static graph is planned as it is
+        if _has_symbolic_sizes(gm):
+            gm, self._orig_to_concrete, self._concrete_to_orig = concretize_gm(gm)
+        else:
+            self._orig_to_concrete = {n: n for n in gm.graph.nodes}
+            self._concrete_to_orig = dict(self._orig_to_concrete)
         self.gm = gm
         self.graph = gm.graph
         self.mesh = mesh
@@ -197,16 +259,15 @@ class ShardingOptimizer:
     def pulp_variables(self) -> _Variables:
         return _Variables(self)
 
-    @property
-    def _concrete_to_orig(self) -> Dict[torch.fx.Node, torch.fx.Node]:
-        """Graphs are planned as given (no symbolic sizes are made concrete
-        here), so the two graphs of the reference are one."""
-        return {n: n for n in self.nodes}
-
-    _orig_to_concrete = _concrete_to_orig
-
     def _normalize_node(self, node):
-        return node
+        """The planner's node for a node of either graph (:298-304)."""
+        return self._orig_to_concrete.get(node, node)
+
+    def _to_orig_solution(self, solution):
+        return {self._concrete_to_orig.get(n, n): spec for n, spec in solution.items()}
+
+    def _to_concrete_solution(self, solution):
+        return {self._orig_to_concrete.get(n, n): spec for n, spec in solution.items()}
 
     def get_strategy(self, node):
         return self.strats[self._normalize_node(node)]
@@ -419,6 +480,7 @@ class ShardingOptimizer:
 
     # -- constraints (delegated to the packed formulation) ------------------------------
     def add_node_constraint(self, node, placement=None, constraint_name=None):
+        node = self._normalize_node(node)
         self._constraint_log.append(("add_node_constraint", {"node_name": node.name, "placement": placement,
                                                              "constraint_name": constraint_name}))
         assert node in self.strats, node
@@ -460,18 +522,18 @@ class ShardingOptimizer:
             for a, e in enumerate(range(int(g.node_edge_off[v]), int(g.node_edge_off[v + 1]))):
                 u = int(g.edge_src_node[e])
                 self.selected_keys.append((int(v), a, int(sol[v]), int(sol[u]) if u >= 0 else 0))
-        return {self.nodes[v]: self.strats[self.nodes[v]].strategies[int(sol[v])]
-                for v in range(self._packed.num_nodes)}
+        return self._to_orig_solution({self.nodes[v]: self.strats[self.nodes[v]].strategies[int(sol[v])]
+                                       for v in range(self._packed.num_nodes)})
 
     def get_solution(self, verbose: bool = False) -> Dict[torch.fx.Node, OpSpec]:
-        return self._solution_dict(self._core.get_solution(verbose=verbose))
+        return self._to_orig_solution(self._solution_dict(self._core.get_solution(verbose=verbose)))
 
     def resolve(self, verbose: bool = False) -> Dict[torch.fx.Node, OpSpec]:
-        return self._solution_dict(self._core.resolve(verbose=verbose))
+        return self._to_orig_solution(self._solution_dict(self._core.resolve(verbose=verbose)))
 
     def _out_indices(self, solution: Dict[torch.fx.Node, OpSpec]) -> np.ndarray:
         sol = np.zeros(self._packed.num_nodes, np.int64)
-        for node, spec in solution.items():
+        for node, spec in self._to_concrete_solution(solution).items():
             if node not in self.node_map or node.op == "output":
                 continue
             for i, s in enumerate(self.strats[node].strategies):
@@ -498,7 +560,7 @@ class ShardingOptimizer:
         return out
 
     def print_costs_for_node(self, node, arg: int = 0) -> str:
-        v = self.node_map[node]
+        v = self.node_map[self._normalize_node(node)]
         e = self._core.edge_of(v, arg)
         g = self._packed
         block = self._core.coef.cost[self._core.var_start[e] : self._core.var_start[e + 1]]
@@ -574,8 +636,8 @@ class ShardingOptimizer:
 
         names = list(self.mesh.mesh_dim_names) if self.mesh.mesh_dim_names else None
         sol = serialization.load_placements(self._core, path, names)
-        return {self.nodes[v]: self.strats[self.nodes[v]].strategies[int(sol[v])]
-                for v in range(self._packed.num_nodes)}
+        return self._to_orig_solution({self.nodes[v]: self.strats[self.nodes[v]].strategies[int(sol[v])]
+                                       for v in range(self._packed.num_nodes)})
 
     def explain_placement(self, target_placement, start_node=None, max_nodes=None) -> str:
         """Why the optimizer did not choose ``target_placement``: per node, the
@@ -599,6 +661,7 @@ class ShardingOptimizer:
         what_if = np.where(tgt_idx >= 0, tgt_idx, chosen)
         terms_c, _ = core.solution_terms(chosen)
         terms_t, _ = core.solution_terms(what_if)
+        start_node = None if start_node is None else self._normalize_node(start_node)
         rows, started = [], start_node is None
         for v in range(g.num_nodes):
             node = self.nodes[v]

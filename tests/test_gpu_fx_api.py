@@ -765,6 +765,65 @@ def test_unsharded_runtime_estimate(mesh):
     assert checked >= 4
 
 
+def test_graph_with_symbolic_sizes_is_planned_on_a_concrete_copy(mesh):
+    """A graph whose batch size is symbolic: the planner works on a copy at the
+    hinted sizes (autoparallel/optimize_sharding.py:162-189, 228-237) and gives
+    the same coefficients and plan as the static graph; the plan comes back on
+    the caller's nodes, and nodes of either graph are accepted."""
+    import torch.fx as fx
+    from torch._subclasses import FakeTensorMode
+    from torch.distributed.tensor.placement_types import Replicate, Shard
+    from torch.fx.experimental.symbolic_shapes import DimDynamic, ShapeEnv, StatelessSymbolicContext
+
+    from autoparallel_amd.optimize_sharding import ShardingOptimizer
+
+    aten = torch.ops.aten
+
+    def build(symbolic):
+        if symbolic:
+            mode = FakeTensorMode(shape_env=ShapeEnv(), static_shapes=False)
+            ctx = StatelessSymbolicContext(dynamic_sizes=[DimDynamic.DYNAMIC, DimDynamic.STATIC])
+            xv = mode.from_tensor(torch.empty(64, 128, device="meta"), symbolic_context=ctx)
+        else:
+            mode = FakeTensorMode()
+            xv = mode.from_tensor(torch.empty(64, 128, device="meta"))
+        wv = mode.from_tensor(torch.empty(128, 256, device="meta"))
+        g = fx.Graph()
+        x, w = g.placeholder("x"), g.placeholder("w")
+        x.meta["val"], w.meta["val"] = xv, wv
+        with mode:
+            h = g.call_function(aten.mm.default, (x, w))
+            h.meta["val"] = aten.mm.default(xv, wv)
+            r = g.call_function(aten.relu.default, (h,))
+            r.meta["val"] = aten.relu.default(h.meta["val"])
+            t = g.call_function(aten.sum.dim_IntList, (r, [1]))
+            t.meta["val"] = aten.sum.dim_IntList(r.meta["val"], [1])
+        g.output((t,))
+        return fx.GraphModule(torch.nn.Module(), g)
+
+    sym, static = build(True), build(False)
+    assert isinstance(next(iter(sym.graph.nodes)).meta["val"].shape[0], torch.SymInt)
+    a = ShardingOptimizer(sym, mesh, devices_per_host=8, device_name="AMD Instinct MI355X")
+    b = ShardingOptimizer(static, mesh, devices_per_host=8, device_name="AMD Instinct MI355X")
+    assert a.gm is not sym and a.orig_gm is sym and b.gm is static
+    assert all(type(d) is int for n in a.graph.nodes for v in [n.meta.get("val")] if isinstance(v, torch.Tensor)
+               for d in v.shape)
+    assert a._packed.num_entries == b._packed.num_entries > 0
+    assert bits_equal(a._core.coef.cost, b._core.coef.cost) and bits_equal(a._core.coef.comm, b._core.coef.comm)
+    x_sym = next(iter(sym.graph.nodes))
+    names = a.add_node_constraint(x_sym, (Shard(0), Replicate()))  # a node of the caller's graph
+    b.add_node_constraint(next(iter(static.graph.nodes)), (Shard(0), Replicate()))
+    sa, sb = a.get_solution(), b.get_solution()
+    assert set(sa) == {n for n in sym.graph.nodes if n.op != "output"}  # keyed by the caller's nodes
+    assert [str(sa[n].output_specs) for n in sym.graph.nodes if n.op != "output"] == \
+        [str(sb[n].output_specs) for n in static.graph.nodes if n.op != "output"]
+    assert sa[x_sym].output_specs.placements == (Shard(0), Replicate())
+    assert a.get_strategy(x_sym) is a.strats[a._orig_to_concrete[x_sym]]
+    assert np.isclose(a._compute_solution_cost(sa)["total"], b._compute_solution_cost(sb)["total"], rtol=1e-12)
+    a.remove_constraints(names)
+    assert set(a.resolve()) == set(sa)
+
+
 def test_hf_llama3_8b_layers_joint_graph():
     """Llama-3-8B as transformers defines it (d 4096, 32 query / 8 key-value heads,
     SwiGLU 14336, RMSNorm, rotary embedding, vocab 128256, bf16), four of its

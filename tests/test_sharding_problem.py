@@ -316,3 +316,60 @@ def test_row_container():
     assert A.toarray().tolist() == [[1, 1, 0, 0, 0, 0], [0, 0, 0, 0, 1, 1], [1, 0, 0, 0, 0, 0], [0, 0, 1, 0, 0, 0]]
     assert lo.tolist() == [-np.inf, -np.inf, 0.0, -np.inf] and hi.tolist() == [1.0, 3.0, np.inf, 1.0]
     assert p.next_name("pair") == "pair_004"
+
+
+# -- symbolic sizes made concrete (known answers of the reference's
+#    tests/test_dynamic_shapes.py:296-480, restated) ---------------------------------
+def _symbolic(shape, dynamic):
+    import torch
+    from torch._subclasses import FakeTensorMode
+    from torch.fx.experimental.symbolic_shapes import DimDynamic, ShapeEnv, StatelessSymbolicContext
+
+    mode = FakeTensorMode(shape_env=ShapeEnv(), static_shapes=False)
+    ctx = StatelessSymbolicContext(dynamic_sizes=[DimDynamic.DYNAMIC if d else DimDynamic.STATIC for d in dynamic])
+    return mode, mode.from_tensor(torch.empty(*shape, device="meta"), symbolic_context=ctx)
+
+
+def test_concretize_args():
+    import torch
+
+    from autoparallel_amd.optimize_sharding import _produces_tensor, concretize_args, concretize_symint
+
+    _, x = _symbolic((16, 128), (True, True))
+    assert all(isinstance(d, torch.SymInt) for d in x.shape)
+    out = concretize_args((x, x.shape[0], [x.shape[1], 32]))
+    assert isinstance(out[0], torch.Tensor) and all(type(d) is int for d in out[0].shape) and out[0].shape == (16, 128)
+    assert type(out[1]) is int and out[1] == 16
+    assert type(out[2][0]) is int and out[2] == [128, 32]
+    assert out[0].stride() == (128, 1) and out[0].dtype == x.dtype
+    plain = concretize_args((torch.randn(4, 4), 42, [1, 2, 3]))
+    assert plain[1] == 42 and plain[2] == [1, 2, 3]
+    assert concretize_symint(7) == 7 and concretize_symint("s") == "s"
+    assert _produces_tensor(torch.randn(4)) and _produces_tensor((torch.randn(4), None))
+    assert not _produces_tensor(42) and not _produces_tensor(None) and not _produces_tensor((1, None))
+
+
+def test_concretize_gm():
+    import torch
+    from torch.fx import Graph, GraphModule
+
+    from autoparallel_amd.optimize_sharding import concretize_gm
+
+    mode, t = _symbolic((16, 128), (True, False))
+    graph = Graph()
+    x = graph.placeholder("x")
+    x.meta.update(val=t, desc="descriptor", custom_key=42)
+    y = graph.call_function(torch.relu, (x,))
+    with mode:
+        y.meta["val"] = torch.relu(t)
+    graph.output(y)
+    gm = GraphModule({}, graph)
+    concrete, to_c, to_o = concretize_gm(gm)
+    orig, conc = list(gm.graph.nodes), list(concrete.graph.nodes)
+    assert [(n.op, n.target) for n in orig] == [(n.op, n.target) for n in conc]
+    assert all(to_c[a] is b and to_o[b] is a for a, b in zip(orig, conc)) and len(to_c) == len(to_o) == 3
+    assert conc[1].args == (conc[0],)  # edges follow the copy
+    for n in conc[:2]:
+        assert all(type(d) is int for d in n.meta["val"].shape) and n.meta["val"].shape == (16, 128)
+    assert isinstance(orig[0].meta["val"].shape[0], torch.SymInt)  # the caller's graph is untouched
+    assert conc[0].meta["desc"] == "descriptor" and conc[0].meta["custom_key"] == 42
