@@ -332,10 +332,15 @@ class ShardingOptimizer:
         try:
             for p, g in fx_utils.get_param_and_grad_nodes(self.graph).values():
                 r.param_grad.append((nm[p], nm[g] if g is not None and g in nm else -1))
-            for n, g in fx_utils.get_plain_input_and_grad_nodes(self.graph).values():
+            # position of each plain input / output among the traced function's own
+            # (an input without a placeholder of its own, e.g. an alias, leaves a gap)
+            self._input_idx, self._output_idx = [], []
+            for desc, (n, g) in fx_utils.get_plain_input_and_grad_nodes(self.graph).items():
                 r.input_grad.append((nm[n], nm[g] if g is not None and g in nm else -1))
-            for n, t in fx_utils.get_plain_output_and_tangent_nodes(self.graph).values():
+                self._input_idx.append(getattr(desc, "idx", len(self._input_idx)))
+            for desc, (n, t) in fx_utils.get_plain_output_and_tangent_nodes(self.graph).items():
                 r.output_tangent.append((nm[n], nm[t] if t is not None and t in nm else -1))
+                self._output_idx.append(getattr(desc, "idx", len(self._output_idx)))
             self._mark_pre_cast_nodes(r)
         except Exception:  # a graph without AOT descriptors has no forward/backward pairs
             logger.debug("no AOT descriptors on the graph: no forward/backward constraints")
@@ -488,20 +493,27 @@ class ShardingOptimizer:
         return self._core.add_node_constraint(self.node_map[node], codes, constraint_name)
 
     def add_sharded_input_constraint(self, input_placements=None):
-        self._io_constraints(self._packed.roles.input_grad, input_placements, "input_constraint")
+        self._io_constraints(self._packed.roles.input_grad, input_placements, "input_constraint",
+                             getattr(self, "_input_idx", None), "inputs")
 
     def add_sharded_output_constraint(self, output_placements=None):
-        self._io_constraints(self._packed.roles.output_tangent, output_placements, "output_constraint")
+        self._io_constraints(self._packed.roles.output_tangent, output_placements, "output_constraint",
+                             getattr(self, "_output_idx", None), "outputs")
 
-    def _io_constraints(self, pairs, placements, name):
+    def _io_constraints(self, pairs, placements, name, idx=None, what="inputs"):
+        """Forward-side nodes only; their gradients / tangents follow through the
+        forward-backward rows (autoparallel/optimize_sharding.py:1720-1752)."""
         remaining = None if placements is None else dict(enumerate(placements))
         for i, (n, _) in enumerate(pairs):
-            plc = None if remaining is None else remaining.pop(i)
+            plc = None if remaining is None else remaining.pop(i if not idx else idx[i])
             codes = None if plc is None else placement_codes(plc)
             self._core.add_node_constraint(n, codes, name)
-        if remaining and any(p is not None for p in remaining.values()):
-            raise RuntimeError(f"We were unable to respect placements at indices "
-                               f"{[i for i, p in remaining.items() if p is not None]}")
+        ignored = [] if not remaining else [i for i, p in remaining.items() if p is not None]
+        if ignored:
+            raise RuntimeError(
+                f"We were unable to respect placements for {what} at indices {ignored}.  This is because the "
+                f"traced joint graph did not actually have a dedicated node for them, typically because some "
+                f"{what} aliased each other.  Replace the placement with None, or clone the tensors.")
 
     def add_parameter_memory_constraint(self, memory_factor_low: float, memory_factor_high: float):
         self._core.add_parameter_memory_constraint(memory_factor_low, memory_factor_high)
@@ -526,10 +538,10 @@ class ShardingOptimizer:
                                        for v in range(self._packed.num_nodes)})
 
     def get_solution(self, verbose: bool = False) -> Dict[torch.fx.Node, OpSpec]:
-        return self._to_orig_solution(self._solution_dict(self._core.get_solution(verbose=verbose)))
+        return self._solution_dict(self._core.get_solution(verbose=verbose))
 
     def resolve(self, verbose: bool = False) -> Dict[torch.fx.Node, OpSpec]:
-        return self._to_orig_solution(self._solution_dict(self._core.resolve(verbose=verbose)))
+        return self._solution_dict(self._core.resolve(verbose=verbose))
 
     def _out_indices(self, solution: Dict[torch.fx.Node, OpSpec]) -> np.ndarray:
         sol = np.zeros(self._packed.num_nodes, np.int64)
