@@ -480,8 +480,13 @@ class ShardingOptimizer:
             ins = self._all_input_nodes(node)
             assert len(s0.redistribute_cost) == len(ins) or (len(ins) == 0 and len(s0.redistribute_cost) == 1), \
                 f"{node}, {len(s0.redistribute_cost)}, {len(ins)}"
+            # every spec the first strategy carries knows its tensor (:205-218, 651-654)
+            for label, specs in (("output_specs", s0.output_specs), ("input_spec", tuple(s0.input_specs))):
+                for spec in (specs if isinstance(specs, (list, tuple)) else (specs,)):
+                    assert not spec or spec.tensor_meta is not None, f"{node} {label} doesn't have a tensor_meta"
             for i, arg in enumerate(ins):
-                assert len(s0.redistribute_cost[i]) == len(self.strats[arg].strategies), f"{node} arg {i}"
+                assert len(s0.redistribute_cost[i]) == len(self.strats[arg].strategies), \
+                    f"{node}, {len(s0.redistribute_cost[i])}, {len(self.strats[arg].strategies)}"
 
     # -- constraints (delegated to the packed formulation) ------------------------------
     def add_node_constraint(self, node, placement=None, constraint_name=None):
