@@ -19,6 +19,7 @@ Constraint families and their reference counterparts:
 from __future__ import annotations
 
 import dataclasses
+import logging
 import math
 from typing import Dict, Iterable, List, Optional, Sequence, Set, Tuple
 
@@ -26,6 +27,8 @@ import numpy as np
 
 from . import ilp
 from .packed import MAX_TUPLES, SPEC_NONE, PackedGraph, plc_str
+
+logger = logging.getLogger(__name__)
 
 
 @dataclasses.dataclass
@@ -462,10 +465,12 @@ class PackedShardingOptimizer:
         self._apply_memory_constraint()
         status = self.prob.solve(backend=backend, verbose=verbose)
         if status == ilp.STATUS_INFEASIBLE:
+            logger.warning(self.get_violated_constraints_log())
             raise RuntimeError(
                 "The sharding optimizer could not find a feasible solution. This typically means "
                 "the user-specified constraints are contradictory or the device mesh is too small "
-                "for the requested sharding.")
+                "for the requested sharding. Check the WARNING log above for the list of violated "
+                "constraints, and consider relaxing input/output constraints or using a larger mesh.")
         self.selected = np.nonzero(self.prob.x > 0.5)[0]
 
     def _extract(self) -> np.ndarray:
