@@ -62,6 +62,9 @@ def main():
                     help="also score this many on-device generated assignments (0 = skip)")
     ap.add_argument("--schedules", type=int, default=16384,
                     help="also price this many candidate orders of a lowered 32-layer schedule (0 = skip)")
+    ap.add_argument("--fx-layers", type=int, default=32,
+                    help="also plan the traced transformers Llama-3-8B with this many layers through "
+                         "ShardingOptimizer and report its host time (0 = skip)")
     ap.add_argument("--direct", action="store_true", help="evaluate every entry directly (no block table)")
     ap.add_argument("--table-mode", choices=["full", "compressed", "direct"], default=None,
                     help="force the block-table layout (default: chosen from the table sizes)")
@@ -295,7 +298,86 @@ def main():
             out["cpu_baseline"]["compiled_port"] = res
         except Exception as exc:  # the checker library is optional for the benchmark
             out["cpu_baseline"]["compiled_port"] = {"error": str(exc)}
+    if args.fx_layers > 0 and args.workload == "llama3_8b_fwd_bwd_mesh8x8":
+        # secondary figure: the same model through the reference-shaped interface, from
+        # the traced joint graph to coefficients and ILP rows (strategy sets of the
+        # installed torch, so fewer entries than the generator's graph above)
+        try:
+            out["fx_path"] = _fx_path_figure(args.fx_layers)
+        except Exception as exc:  # transformers or the fake process group unavailable
+            out["fx_path"] = {"error": f"{type(exc).__name__}: {exc}"[:300]}
     print(json.dumps(out))
+
+
+def _fx_path_figure(n_layers: int) -> dict:
+    import contextlib
+
+    import torch
+    import torch.distributed as dist
+    import transformers
+    from torch._functorch.aot_autograd import aot_export_joint_with_descriptors
+    from torch._subclasses.fake_tensor import FakeTensorMode
+    from torch.distributed.device_mesh import init_device_mesh
+    from torch.testing._internal.distributed.fake_pg import FakeStore
+
+    from autoparallel_amd.optimize_sharding import ShardingOptimizer
+    from autoparallel_amd.shardings import placement_options as PO
+
+    class Wrap(torch.nn.Module):
+        def __init__(self, lm):
+            super().__init__()
+            self.lm = lm
+
+        def forward(self, ids):
+            m = self.lm.model
+            x = m.embed_tokens(ids)
+            pos = torch.arange(ids.shape[1], device=ids.device)[None]
+            pe = m.rotary_emb(x, pos)
+            for layer in m.layers:
+                o = layer(x, attention_mask=None, position_ids=pos, position_embeddings=pe)
+                x = o[0] if isinstance(o, tuple) else o
+            logits = self.lm.lm_head(m.norm(x))
+            return torch.nn.functional.cross_entropy(
+                logits[:, :-1].reshape(-1, logits.shape[-1]).float(), ids[:, 1:].reshape(-1))
+
+    cfg = transformers.LlamaConfig(
+        vocab_size=128256, hidden_size=4096, intermediate_size=14336, num_hidden_layers=n_layers,
+        num_attention_heads=32, num_key_value_heads=8, max_position_embeddings=8192, rope_theta=500000.0,
+        attention_dropout=0.0, use_cache=False, attn_implementation="sdpa")
+    t0 = time.perf_counter()
+    with FakeTensorMode():
+        torch.set_default_dtype(torch.bfloat16)
+        try:
+            with torch.device("cuda"):
+                m = Wrap(transformers.LlamaForCausalLM(cfg))
+        finally:
+            torch.set_default_dtype(torch.float32)
+        ids = torch.randint(0, cfg.vocab_size, (64, 8192), device="cuda")
+        with contextlib.ExitStack() as stack:
+            gm = aot_export_joint_with_descriptors(stack, m, (ids,)).graph_module
+    t_trace = time.perf_counter() - t0
+    own = not dist.is_initialized()
+    if own:
+        dist.init_process_group("fake", store=FakeStore(), rank=0, world_size=64)
+    try:
+        mesh = init_device_mesh("cpu", (8, 8))
+        PO.fallback_nodes.clear()
+        PO.reset_placement_options_cache()
+        t0 = time.perf_counter()
+        opt = ShardingOptimizer(gm, mesh, devices_per_host=8, device_name="AMD Instinct MI355X")
+        t_opt = time.perf_counter() - t0
+        g = opt._packed
+        return {
+            "workload": f"transformers LlamaForCausalLM, Llama-3-8B dimensions, {n_layers} layers, bf16, "
+                        f"batch 64 x 8192, joint graph, mesh (8,8)",
+            "nodes": g.num_nodes, "edges": g.num_edges, "entries": g.num_entries,
+            "trace_s": t_trace, "sharding_optimizer_s": t_opt,
+            "strategy_queries": dict(PO.strategy_cache_stats), "replicate_stand_ins": len(PO.fallback_nodes),
+            "ilp_rows": len(opt.prob.constraints),
+        }
+    finally:
+        if own:
+            dist.destroy_process_group()
 
 
 if __name__ == "__main__":
