@@ -56,11 +56,14 @@ def reset_comms_cost_cache() -> None:
     _comms_cost_cache.clear()
 
 
-def comms_cost_matrix(src_specs: Sequence, tgt_specs: Sequence, order_mode: int = 0) -> np.ndarray:
+def comms_cost_matrix(src_specs: Sequence, tgt_specs: Sequence, order_mode: int = 0,
+                      bandwidth_latency=None) -> np.ndarray:
     """cost[t][s] of redistributing src_specs[s] into the placements of
-    tgt_specs[t] (all on one mesh): one edge block on the device."""
+    tgt_specs[t] (all on one mesh): one edge block on the device.
+    ``bandwidth_latency``: (GB/s per mesh dim, us per mesh dim) in place of what
+    the mesh shape and the devices per host give."""
     mesh = src_specs[0].mesh
-    b = GraphBuilder(tuple(mesh.shape), _dph(mesh))
+    b = GraphBuilder(tuple(mesh.shape), _dph(mesh) if hasattr(mesh, "device_type") else (_settings["devices_per_host"] or 1))
     src_words = [b.spec(b.meta(*tensor_meta_key(s.tensor_meta)), placement_codes(s.placements)) for s in src_specs]
     tgt_words = [b.spec(b.meta(*tensor_meta_key(t.tensor_meta)), placement_codes(t.placements)) for t in tgt_specs]
     b.add_node(NodeDesc("src", in_specs=[[w] for w in src_words], out_specs=[[w] for w in src_words],
@@ -69,6 +72,9 @@ def comms_cost_matrix(src_specs: Sequence, tgt_specs: Sequence, order_mode: int 
     g = b.pack()
     eng = CostEngine(g, device_name=_device_name(), use_table=False, order_mode=order_mode,
                      nccl_config=_nccl_topo_config)
+    if bandwidth_latency is not None:
+        for i, (bw, lat) in enumerate(zip(*bandwidth_latency)):
+            eng.problem.model.mesh_bw[i], eng.problem.model.mesh_lat[i] = float(bw), float(lat)
     eng.build(clamp_inf=False)
     comm = eng.results()["comm"]
     base = int(g.edge_off[1])
@@ -79,13 +85,38 @@ def redistribute_cost(current_spec, target_spec, order: List[int]) -> float:
     if current_spec.mesh != target_spec.mesh:
         return float("inf")
     ndim = current_spec.mesh.ndim
-    if list(order) == list(range(ndim)):
-        mode = 1
-    elif list(order) == list(reversed(range(ndim))):
-        mode = 2
-    else:
-        raise NotImplementedError(f"mesh-dim order {order}: only ascending and descending orders are built")
-    return float(comms_cost_matrix([current_spec], [target_spec], order_mode=mode)[0, 0])
+    order = [int(i) for i in order]
+    if order == list(range(ndim)):
+        return float(comms_cost_matrix([current_spec], [target_spec], order_mode=1)[0, 0])
+    if order == list(reversed(range(ndim))):
+        return float(comms_cost_matrix([current_spec], [target_spec], order_mode=2)[0, 0])
+    return _redistribute_cost_in_order(current_spec, target_spec, order)
+
+
+def _redistribute_cost_in_order(current_spec, target_spec, order: List[int]) -> float:
+    """Any other visiting order of the mesh dims (a permutation, or a subset: the
+    dims left out are never touched, :154-156).  The fold only sees, per step, the
+    two placements, the size, bandwidth and latency of the dim it visits, and the
+    running volume; so it is evaluated in ascending order on the mesh relabelled
+    in visiting order, with the bandwidth and latency each dim has on the real
+    mesh carried along."""
+    from types import SimpleNamespace
+
+    if _nccl_topo_config is not None:
+        raise NotImplementedError("an explicit mesh-dim order with the NCCL model is not built")
+    mesh = current_spec.mesh
+    ndim = mesh.ndim
+    assert len(set(order)) == len(order) and all(0 <= i < ndim for i in order), order
+    rest = [i for i in range(ndim) if i not in order]
+    perm = order + rest
+    model = make_model(tuple(mesh.shape), _dph(mesh), _device_name())
+    bw, lat = [model.mesh_bw[i] for i in perm], [model.mesh_lat[i] for i in perm]
+    relabelled = SimpleNamespace(shape=tuple(mesh.shape[i] for i in perm), ndim=ndim)
+    src_plc = tuple(current_spec.placements[i] for i in perm)
+    tgt_plc = tuple(target_spec.placements[i] if i in order else current_spec.placements[i] for i in perm)
+    src = SimpleNamespace(mesh=relabelled, placements=src_plc, tensor_meta=current_spec.tensor_meta)
+    tgt = SimpleNamespace(mesh=relabelled, placements=tgt_plc, tensor_meta=target_spec.tensor_meta)
+    return float(comms_cost_matrix([src], [tgt], order_mode=1, bandwidth_latency=(bw, lat))[0, 0])
 
 
 def estimate_strategy_comms_cost(src_spec, tgt_spec) -> float:

@@ -824,6 +824,48 @@ def test_graph_with_symbolic_sizes_is_planned_on_a_concrete_copy(mesh):
     assert set(a.resolve()) == set(sa)
 
 
+def test_redistribute_cost_in_any_mesh_dim_order(mesh):
+    """redistribute_cost(current, target, order) for every permutation of a 3-D
+    mesh's dims and for orders that leave dims out, against the oracle's fold
+    in that order (autoparallel/cost_models/collective_runtime_estimation.py:115-229):
+    ascending and descending run on the device as they are, the others on the
+    relabelled mesh."""
+    import itertools
+
+    from torch.distributed.device_mesh import init_device_mesh
+    from torch.distributed.tensor._dtensor_spec import DTensorSpec, TensorMeta
+    from torch.distributed.tensor.placement_types import Partial, Replicate, Shard
+
+    from autoparallel_amd.cost_models import collective_runtime_estimation as cre
+    from autoparallel_amd.dtensor_bridge import placement_codes
+
+    m3 = init_device_mesh("cpu", (2, 2, 2))
+    cre.configure(4, "AMD Instinct MI355X")  # 4 per host: the outer dim crosses hosts, the inner two do not
+    try:
+        topo, dev = O.Topo((2, 2, 2), 4), O.DeviceLimit()
+        metas = [((1024, 512, 64), (512 * 64, 64, 1)), ((1024, 512, 64), (64, 65536, 1))]  # contiguous, permuted
+        R, P, S = Replicate(), Partial(), Shard
+        pairs = [((S(0), S(1), P), (R, S(0), S(2))), ((P, P, S(1)), (S(0), R, R)), ((S(2), S(0), S(1)), (S(0), S(1), R)),
+                 ((P, S(0), R), (R, R, S(0))), ((S(0), R, P), (S(0), P, R))]
+        orders = [list(p) for p in itertools.permutations(range(3))] + [[1], [2, 0], [0, 2], []]
+        checked = 0
+        for shape, stride in metas:
+            tm = TensorMeta(torch.Size(shape), stride, torch.bfloat16)
+            for src, tgt in pairs:
+                a, b = DTensorSpec(m3, src, tensor_meta=tm), DTensorSpec(m3, tgt, tensor_meta=tm)
+                for order in orders:
+                    got = cre.redistribute_cost(a, b, order)
+                    want = O.redistribute_cost(placement_codes(src), shape, stride, 2, placement_codes(tgt), topo, dev, order)
+                    assert got == want or (np.isinf(got) and np.isinf(want)), (src, tgt, order, got, want)
+                    checked += np.isfinite(want) and want > 0
+        assert checked > 60
+        # the order changes the price: gathering before or after the reduce-scatter moves different volumes
+        a, b = DTensorSpec(m3, pairs[0][0], tensor_meta=tm), DTensorSpec(m3, pairs[0][1], tensor_meta=tm)
+        assert len({cre.redistribute_cost(a, b, o) for o in orders[:6]}) > 1
+    finally:
+        cre.configure(8, "AMD Instinct MI355X")
+
+
 def test_hf_llama3_8b_layers_joint_graph():
     """Llama-3-8B as transformers defines it (d 4096, 32 query / 8 key-value heads,
     SwiGLU 14336, RMSNorm, rotary embedding, vocab 128256, bf16), four of its
