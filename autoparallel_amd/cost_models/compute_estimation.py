@@ -207,3 +207,45 @@ def estimate_strategy_runtime_cost(node, strategy):
     if key is not None:
         _compute_cost_cache[key] = cost
     return cost
+
+
+def benchmark_fn(fn, *args, **kwargs) -> float:
+    """Mean time of ``fn(*args, **kwargs)`` on the current stream in
+    microseconds: 3 untimed calls, then 10 between two events
+    (compute_estimation.py:513-529)."""
+    for _ in range(3):
+        fn(*args, **kwargs)
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(10):
+        fn(*args, **kwargs)
+    end.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(end) / 10 * 1e3
+
+
+def benchmark_strategy_runtime_cost(node, strategy) -> float:
+    """The measured counterpart of estimate_strategy_runtime_cost, for checking
+    the model against the device: the operator is run on random tensors of the
+    sizes the strategy leaves on one device (compute_estimation.py:496-510)."""
+    if _has_zero_cost(node):
+        return 0
+    from torch._subclasses.fake_tensor import unset_fake_temporarily
+    from torch.utils._pytree import tree_flatten, tree_map_only
+
+    args = tree_map_only(torch.fx.Node, lambda x: x.meta["val"], node.args)
+    kwargs = tree_map_only(torch.fx.Node, lambda x: x.meta["val"], node.kwargs)
+    flat, spec = tree_flatten(args)
+    with unset_fake_temporarily():
+        specs = iter(strategy.input_specs if strategy is not None else ())
+        real = []
+        for x in flat:
+            if isinstance(x, torch.Tensor):
+                if strategy is None:
+                    sizes, strides = list(x.shape), list(x.stride())
+                else:
+                    sizes, strides = _get_sharded_shape_stride(next(specs))
+                t = torch.empty_strided(sizes, strides, dtype=x.dtype, device="cuda")
+                x = t.normal_() if t.dtype.is_floating_point else t.random_(0, 256)
+            real.append(x)
+        return benchmark_fn(node.target, *spec.unflatten(real), **kwargs)

@@ -866,6 +866,28 @@ def test_redistribute_cost_in_any_mesh_dim_order(mesh):
         cre.configure(8, "AMD Instinct MI355X")
 
 
+def test_measured_runtime_of_a_strategy(mesh):
+    """benchmark_strategy_runtime_cost (autoparallel/cost_models/compute_estimation.py:496-529)
+    runs the operator at the strategy's local sizes on the device: a matmul takes
+    time, sharded or whole; a view takes none."""
+    from autoparallel_amd.cost_models.compute_estimation import (
+        benchmark_strategy_runtime_cost,
+        estimate_strategy_runtime_cost,
+    )
+    from autoparallel_amd.optimize_sharding import ShardingOptimizer
+
+    gm = _joint_graph()
+    opt = ShardingOptimizer(gm, mesh, devices_per_host=8, device_name="AMD Instinct MI355X")
+    mm = next(n for n in gm.graph.nodes if n.op == "call_function" and n.target is torch.ops.aten.mm.default)
+    view = next(n for n in gm.graph.nodes if n.op == "call_function" and n.target is torch.ops.aten.view.default)
+    sts = opt.strats[mm].strategies
+    whole = next(s for s in sts if all(p.is_replicate() for sp in s.input_specs for p in sp.placements))
+    t_whole = benchmark_strategy_runtime_cost(mm, whole)
+    assert t_whole > 0 and benchmark_strategy_runtime_cost(mm, None) > 0
+    assert benchmark_strategy_runtime_cost(view, opt.strats[view].strategies[0]) == 0
+    assert estimate_strategy_runtime_cost(mm, whole) > 0
+
+
 def test_hf_llama3_8b_layers_joint_graph():
     """Llama-3-8B as transformers defines it (d 4096, 32 query / 8 key-value heads,
     SwiGLU 14336, RMSNorm, rotary embedding, vocab 128256, bf16), four of its
