@@ -224,6 +224,61 @@ def benchmark_fn(fn, *args, **kwargs) -> float:
     return start.elapsed_time(end) / 10 * 1e3
 
 
+def _shard_args_for_node(node, strategy=None, rand_init: bool = False):
+    """(args, kwargs) of the node with every tensor argument at the size and
+    stride the strategy leaves on one device (the traced ones without a
+    strategy); real random ones on the device with
+    ``rand_init`` (compute_estimation.py:334-365).  Without it the tensors are on
+    the meta device."""
+    from torch.utils._pytree import tree_flatten, tree_map_only
+
+    args = tree_map_only(torch.fx.Node, lambda x: x.meta["val"], node.args)
+    kwargs = tree_map_only(torch.fx.Node, lambda x: x.meta["val"], node.kwargs)
+    assert not any(isinstance(v, torch.Tensor) for v in kwargs.values()), f"{node}: tensors are expected in args"
+    flat, spec = tree_flatten(args)
+    specs = iter(strategy.input_specs if strategy is not None else ())
+    out = []
+    for x in flat:
+        if isinstance(x, torch.Tensor):
+            sizes, strides = (list(x.shape), list(x.stride())) if strategy is None else _get_sharded_shape_stride(next(specs))
+            if rand_init:
+                t = torch.empty_strided(sizes, strides, dtype=x.dtype, device="cuda")
+                x = t.normal_() if t.dtype.is_floating_point else t.random_(0, 256)
+            else:
+                x = torch.empty_strided(sizes, strides, dtype=x.dtype, device="meta")  # sizes are all the counters need
+        out.append(x)
+    return spec.unflatten(out), kwargs
+
+
+def _compute_flops(fn, *args, **kwargs):
+    """(flops torch counts for fn on these arguments, its output) (:383-388)."""
+    from torch.utils.flop_counter import FlopCounterMode
+
+    with FlopCounterMode(display=False) as counter:
+        out = fn(*args, **kwargs)
+    return counter.get_total_flops(), out
+
+
+def compare_estimated_with_benchmarked_throughput(graph, sharding_placement, tgt_ops="mm"):
+    """For the chosen strategy of every node of the target operators: measured
+    time, estimated time, achieved TFLOP/s, the device's figure and their ratio
+    (:532-556)."""
+    if tgt_ops == "mm":
+        tgt_ops = [torch.ops.aten.mm.default, torch.ops.aten.bmm.default]
+    data = {}
+    for node in graph.nodes:
+        if node.op != "call_function" or (tgt_ops is not None and node.target not in tgt_ops):
+            continue
+        strategy = sharding_placement[node]
+        args, kwargs = _shard_args_for_node(node, strategy)
+        flops = _compute_flops(node.target, *args, **kwargs)[0]
+        real_us = benchmark_strategy_runtime_cost(node, strategy)
+        throughput = flops / (real_us / 1e6) * 1e-12
+        peak = _get_device_tflops(strategy.input_specs[0].tensor_meta.dtype)
+        data[node] = (real_us, estimate_strategy_runtime_cost(node, strategy), throughput, peak, throughput / peak)
+    return data
+
+
 def benchmark_strategy_runtime_cost(node, strategy) -> float:
     """The measured counterpart of estimate_strategy_runtime_cost, for checking
     the model against the device: the operator is run on random tensors of the
@@ -231,21 +286,7 @@ def benchmark_strategy_runtime_cost(node, strategy) -> float:
     if _has_zero_cost(node):
         return 0
     from torch._subclasses.fake_tensor import unset_fake_temporarily
-    from torch.utils._pytree import tree_flatten, tree_map_only
 
-    args = tree_map_only(torch.fx.Node, lambda x: x.meta["val"], node.args)
-    kwargs = tree_map_only(torch.fx.Node, lambda x: x.meta["val"], node.kwargs)
-    flat, spec = tree_flatten(args)
     with unset_fake_temporarily():
-        specs = iter(strategy.input_specs if strategy is not None else ())
-        real = []
-        for x in flat:
-            if isinstance(x, torch.Tensor):
-                if strategy is None:
-                    sizes, strides = list(x.shape), list(x.stride())
-                else:
-                    sizes, strides = _get_sharded_shape_stride(next(specs))
-                t = torch.empty_strided(sizes, strides, dtype=x.dtype, device="cuda")
-                x = t.normal_() if t.dtype.is_floating_point else t.random_(0, 256)
-            real.append(x)
-        return benchmark_fn(node.target, *spec.unflatten(real), **kwargs)
+        args, kwargs = _shard_args_for_node(node, strategy, rand_init=True)
+        return benchmark_fn(node.target, *args, **kwargs)

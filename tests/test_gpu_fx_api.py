@@ -886,6 +886,14 @@ def test_measured_runtime_of_a_strategy(mesh):
     assert t_whole > 0 and benchmark_strategy_runtime_cost(mm, None) > 0
     assert benchmark_strategy_runtime_cost(view, opt.strats[view].strategies[0]) == 0
     assert estimate_strategy_runtime_cost(mm, whole) > 0
+    from autoparallel_amd.cost_models.compute_estimation import compare_estimated_with_benchmarked_throughput
+
+    sol = opt.get_solution()
+    table = compare_estimated_with_benchmarked_throughput(gm.graph, sol)
+    mms = [n for n in gm.graph.nodes if n.op == "call_function" and n.target is torch.ops.aten.mm.default]
+    assert set(table) == set(mms)
+    for real_us, est_us, tflops, peak, eff in table.values():
+        assert real_us > 0 and est_us > 0 and peak == 157.3 and np.isclose(eff, tflops / peak)  # fp32 model
 
 
 def test_hf_llama3_8b_layers_joint_graph():
