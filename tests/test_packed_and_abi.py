@@ -320,3 +320,25 @@ def test_tensors_beyond_int64_bytes_are_refused():
         b.pack().validate()
     assert graphgen._cap_numel((65536, 65536, 65536, 65536)) == (8192, 8192, 8192, 8192) or \
         np.prod([float(x) for x in graphgen._cap_numel((65536, 65536, 65536, 65536))]) <= 2.0**48
+
+
+def test_missing_library_is_an_error_not_a_fallback(monkeypatch, tmp_path):
+    """Without the built HIP library every entry into the product path raises:
+    nothing is computed on the host instead."""
+    from autoparallel_amd import _lib
+
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "libapc_hip.so"))
+    with pytest.raises(_lib.ApcError, match="no CPU fallback"):
+        _lib.load()
+    from autoparallel_amd.engine import make_model
+
+    with pytest.raises(_lib.ApcError):
+        make_model((8, 8), 8, "AMD Instinct MI355X")
+    # the package itself never reaches for the oracle
+    import pathlib
+    import re
+
+    root = pathlib.Path(_lib.__file__).parent
+    for path in root.rglob("*.py"):
+        assert not re.search(r"^\s*(from|import)\s+oracle\b", path.read_text(), re.M), path
