@@ -248,7 +248,8 @@ def test_abi_host_helpers():
             assert m.gmem_bw == bw and list(m.tflops)[:5] == [float(tf.get(i, 0.0)) for i in range(5)], full
     assert lib.apc_device_limits(b"NVIDIA PG509-210", ctypes.byref(m)) == 0 and m.tflops[3] == 312.0
     assert lib.apc_device_limits(b"NVIDIA H100 and A100", ctypes.byref(m)) == 0 and m.tflops[0] == 67.0
-    # figures the reference's own documentation and tests quote
+    # the H100 row against the figures the reference's documentation quotes (989 TFLOPS bf16, 3.35 TB/s:
+    # docs/how_autoparallel_chooses_a_strategy.md:34-39); the other rows are data restated from the table
     h100 = O.DeviceLimit.named("NVIDIA H100 80GB HBM3")
     assert h100.tflops[3] == 989.0 and h100.tflops[1] == 494.0 and h100.gmem_bandwidth == 3.35 * 1024**4
     assert O.DeviceLimit.named("AMD Instinct MI300X").tflops[1] == 653.7
