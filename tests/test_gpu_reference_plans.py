@@ -281,3 +281,51 @@ def test_constraints_added_and_removed_between_solves(meshes):
     opt.resolve()
     assert "memory_constraint_high" not in opt.prob.constraints
     assert "memory_constraint_low" not in opt.prob.constraints
+
+
+def test_tensor_created_in_the_graph_and_a_buffer(meshes):
+    """The model of tests/test_optimize_placement.py:302-335 (a tensor made by
+    torch.full inside forward, a registered buffer): the factory gets its
+    Shard/Replicate product, the buffer is planned like an input, and the plan
+    solves with the batch-sharded input."""
+    from torch._functorch.aot_autograd import aot_export_joint_with_descriptors
+    from torch._subclasses.fake_tensor import FakeTensorMode
+
+    from autoparallel_amd.graph_utils import add_alias_nodes
+    from autoparallel_amd.optimize_sharding import ShardingOptimizer
+    from autoparallel_amd.shardings import placement_options as PO
+
+    dim = 128
+
+    class Model(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.linear = nn.Linear(dim, dim)
+            self.register_buffer("buf", torch.empty(dim))
+
+        def forward(self, x):
+            x = x + torch.full([256, 256, 6144], 0, dtype=torch.bfloat16, device=x.device).sum()
+            return self.linear(x) + self.buf
+
+    mesh = meshes[0]
+    with FakeTensorMode():
+        with torch.device("cuda"):
+            m = Model()
+        x = torch.rand(512, dim, device="cuda")
+        with contextlib.ExitStack() as stack:
+            gm = aot_export_joint_with_descriptors(stack, m, (x,)).graph_module
+    add_alias_nodes(gm)
+    PO.fallback_nodes.clear()
+    opt = ShardingOptimizer(gm, mesh, devices_per_host=8, device_name="H100")
+    assert PO.fallback_nodes == [], PO.fallback_reasons
+    full = next(n for n in gm.graph.nodes if n.op == "call_function" and n.target is torch.ops.aten.full.default)
+    sts = opt.strats[full].strategies
+    # rank 3 on one mesh dim: Shard(0), Shard(1), Shard(2), Replicate; 256 ranks split 256, 256 and 6144
+    assert [s.output_specs.placements for s in sts] == [(Shard(0),), (Shard(1),), (Shard(2),), (Replicate(),)]
+    assert all(s.output_specs.tensor_meta.dtype == torch.bfloat16 and len(s.redistribute_cost[0]) == 4 for s in sts)
+    opt.add_sharded_input_constraint([(Shard(0),)])
+    opt.add_sharded_output_constraint([(Shard(0),)])
+    sol = opt.get_solution()
+    assert sol[full].output_specs.placements != (Replicate(),)  # 200 MB of zeros are cheaper to make in shards
+    inputs = [n for n in gm.graph.nodes if n.op == "placeholder"]
+    assert len(inputs) >= 4 and all(n in sol for n in inputs)
