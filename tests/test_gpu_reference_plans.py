@@ -329,3 +329,41 @@ def test_tensor_created_in_the_graph_and_a_buffer(meshes):
     assert sol[full].output_specs.placements != (Replicate(),)  # 200 MB of zeros are cheaper to make in shards
     inputs = [n for n in gm.graph.nodes if n.op == "placeholder"]
     assert len(inputs) >= 4 and all(n in sol for n in inputs)
+
+
+def test_constant_tensor_attribute_of_the_graph(meshes):
+    """tests/test_optimize_placement.py:470-516: a constant made by new_tensor is
+    an attribute of the traced graph; it gets placements like any input and, being
+    eight elements broadcast over the batch, ends up Replicate."""
+    from torch._functorch.aot_autograd import aot_export_joint_with_descriptors
+    from torch._subclasses.fake_tensor import FakeTensorMode
+
+    from autoparallel_amd.graph_utils import add_alias_nodes
+    from autoparallel_amd.optimize_sharding import ShardingOptimizer
+
+    class Model(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.linear = nn.Linear(256, 1024)
+
+        def forward(self, x):
+            y = x.new_tensor([0, 1, 2, 3, 4, 5, 6, 7])[None, :, None]
+            return self.linear(x) + y
+
+    mesh = meshes[0]
+    with FakeTensorMode(allow_non_fake_inputs=True):
+        with torch.device("cuda"):
+            m = Model()
+        x = torch.rand(8 * 256, 8, 256, device="cuda", requires_grad=True)
+        with contextlib.ExitStack() as stack:
+            gm = aot_export_joint_with_descriptors(stack, m, (x,)).graph_module
+    add_alias_nodes(gm)
+    consts = [n for n in gm.graph.nodes if n.op == "get_attr"]
+    assert consts, [n.op for n in gm.graph.nodes]
+    opt = ShardingOptimizer(gm, mesh, devices_per_host=8, device_name="H100")
+    opt.add_parameter_memory_constraint(0.0, 1.0 / mesh.size())
+    opt.add_sharded_input_constraint([(Shard(0),)])
+    opt.add_sharded_output_constraint([(Shard(0),)])
+    sol = opt.get_solution()
+    for node in consts:
+        assert node in sol and sol[node].output_specs.placements == (Replicate(),)
