@@ -11,6 +11,8 @@
 // L + 64 k, so every load and store instruction covers 64 consecutive entries.
 #include "apc_device.h"
 
+#include <mutex>
+
 namespace apc_impl {
 
 thread_local char g_err[512] = "";
@@ -82,6 +84,27 @@ int slot_grid(const apc_problem* p, int per_block, unsigned* grid) {
 namespace {
 
 using apc_impl::g_err;
+
+// What the library remembers per device (a kernel attribute that is set once,
+// the address of the static scratch array): looked up by the current device of
+// the calling thread, guarded by a mutex of its own.
+struct DeviceState {
+  std::mutex mu;
+  bool lds_limit_raised = false;
+  double* scratch = nullptr;  // device address of `scratch` on this device
+};
+constexpr int kMaxDevices = 64;
+DeviceState g_devices[kMaxDevices];
+
+DeviceState* current_device_state() {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    snprintf(g_err, sizeof(g_err), "hipGetDevice: %s (device %d)", hipGetErrorString(e), dev);
+    return nullptr;
+  }
+  return &g_devices[dev];
+}
 
 // ---------------------------------------------------------------------------
 // Kernel: block table and node compute estimate
@@ -655,15 +678,19 @@ int launch_prepare(const apc_problem* p, double* table, bool do_nodes, double* c
                     p->n_meta == 0 || p->n_tuple == 0) ? 1 : 0;
   const size_t lds =
       do_nodes ? (size_t)kNodesPerBlock * (kProgCache + kRecWords + (slow ? 0 : words)) * 8 : 0;
-  static bool attr_set = false;  // raise the 64 KB default limit of dynamic LDS once
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(prepare_kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
-    if (e != hipSuccess) {
-      snprintf(g_err, sizeof(g_err), "hipFuncSetAttribute: %s", hipGetErrorString(e));
-      return APC_ERR_LAUNCH;
+  if (lds > 0) {  // dynamic LDS beyond the 64 KB default needs the limit raised: once per device
+    DeviceState* dev = current_device_state();
+    if (!dev) return APC_ERR_LAUNCH;
+    std::lock_guard<std::mutex> lock(dev->mu);
+    if (!dev->lds_limit_raised) {
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(prepare_kernel),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
+      if (e != hipSuccess) {
+        snprintf(g_err, sizeof(g_err), "hipFuncSetAttribute: %s", hipGetErrorString(e));
+        return APC_ERR_LAUNCH;
+      }
+      dev->lds_limit_raised = true;
     }
-    attr_set = true;
   }
   hipLaunchKernelGGL(prepare_kernel, dim3(table_blocks + node_blocks), dim3(256), lds, stream, *p,
                      table, table_blocks, slow, compute, per_arg, status);
