@@ -106,6 +106,30 @@ DeviceState* current_device_state() {
   return &g_devices[dev];
 }
 
+// Scratch of apc_build_all_noalloc: the block table of one build.  Every GPU
+// the library runs on holds its own copy (8 MiB) until the process ends.  The
+// name is a host-side stand-in, not a device address: host code uses the
+// address hipGetSymbolAddress returns for the current device (resolve_scratch).
+__device__ __align__(256) static double scratch[APC_NOALLOC_MAX_TABLE];
+
+// Device address of `scratch` on the calling thread's current device, resolved
+// on the first call there.
+double* resolve_scratch() {
+  DeviceState* dev = current_device_state();
+  if (!dev) return nullptr;
+  std::lock_guard<std::mutex> lock(dev->mu);
+  if (!dev->scratch) {
+    void* ptr = nullptr;
+    hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr) {
+      snprintf(g_err, sizeof(g_err), "hipGetSymbolAddress(scratch): %s", hipGetErrorString(e));
+      return nullptr;
+    }
+    dev->scratch = static_cast<double*>(ptr);
+  }
+  return dev->scratch;
+}
+
 // ---------------------------------------------------------------------------
 // Kernel: block table and node compute estimate
 // ---------------------------------------------------------------------------
@@ -885,6 +909,27 @@ int apc_build_all(const apc_problem* p, double* table, double* compute, double* 
                   void* stream) {
   if (int rc = apc_prepare(p, table, compute, per_arg, status, stream)) return rc;
   return apc_edge_costs(p, table, per_arg, comm, cost, flags, clamp_inf, stream);
+}
+
+int apc_build_all_noalloc(const apc_problem* p, double* compute, double* per_arg, int32_t* status,
+                          double* comm, double* cost, uint8_t* flags, int32_t clamp_inf,
+                          void* stream) {
+  if (int rc = validate_problem(p)) return rc;
+  if (p->table_size > APC_NOALLOC_MAX_TABLE) {
+    snprintf(g_err, sizeof(g_err),
+             "apc_build_all_noalloc: the block table has %lld doubles, the static scratch holds %lld; "
+             "use apc_build_all with a table of the caller's",
+             (long long)p->table_size, (long long)APC_NOALLOC_MAX_TABLE);
+    return APC_ERR_INVALID;
+  }
+  // without a block table (table_size 0) every edge is evaluated directly, as
+  // apc_build_all does with table == NULL
+  double* table = nullptr;
+  if (p->table_size > 0) {
+    table = resolve_scratch();
+    if (!table) return APC_ERR_LAUNCH;
+  }
+  return apc_build_all(p, table, compute, per_arg, status, comm, cost, flags, clamp_inf, stream);
 }
 
 int apc_build_all_timed(const apc_problem* p, double* table, double* compute, double* per_arg,

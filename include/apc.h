@@ -342,6 +342,24 @@ int apc_build_all(const apc_problem* p, double* table, double* compute, double* 
                   int32_t* status, double* comm, double* cost, uint8_t* flags, int32_t clamp_inf,
                   void* stream);
 
+/* apc_build_all for callers that cannot allocate device memory (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc): no
+ * counterpart in the reference.  The block table, the one buffer of the build
+ * that is neither input nor output, lives in a static device array of
+ * APC_NOALLOC_MAX_TABLE doubles (8 MiB per GPU, held until the process ends)
+ * instead of a buffer of the caller's; everything else is passed as for
+ * apc_build_all, and the results are the same bit for bit.  Returns
+ * APC_ERR_INVALID when p->table_size exceeds APC_NOALLOC_MAX_TABLE; with
+ * table_size == 0 every entry is evaluated directly.  The call allocates
+ * nothing (the first call on a device looks the array's address up).  Every
+ * call on a GPU shares that GPU's array: calls that overlap on one GPU (two
+ * streams, two threads) race; a build reads only the table elements it wrote
+ * itself, so nothing needs clearing between calls. */
+#define APC_NOALLOC_MAX_TABLE (1 << 20)
+int apc_build_all_noalloc(const apc_problem* p, double* compute, double* per_arg, int32_t* status,
+                          double* comm, double* cost, uint8_t* flags, int32_t clamp_inf,
+                          void* stream);
+
 /* Measurement aids, no counterpart in the reference.  A timer owns n_slots
  * pairs of HIP events (host objects, no device memory).  apc_edge_costs_timed
  * is apc_edge_costs with the pair of `slot` recorded at the kernel's own begin
