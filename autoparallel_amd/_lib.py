@@ -132,6 +132,10 @@ class ApcProblem(C.Structure):
         ("block_udst", C.c_void_p),
         ("comp_recs", C.c_void_p),
         ("item_entries", C.c_int32),
+        ("table_units", C.c_void_p),
+        ("spec_recs", C.c_void_p),
+        ("n_prog_term", C.c_int64),
+        ("prog_terms", C.c_void_p),
     ]
 
 

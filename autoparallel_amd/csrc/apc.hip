@@ -62,6 +62,8 @@ int validate_problem(const apc_problem* p) {
     return fail(APC_ERR_INVALID, "compressed block table: list_uidx, list_ufirst and block_udst go together%s");
   if (p->max_rank < 0 || p->max_rank > APC_MAX_RANK || p->max_node_args < 0)
     return fail(APC_ERR_INVALID, "max_rank / max_node_args out of range%s");
+  if (p->n_prog_term < 0 || (p->n_prog_term > 0 && !p->prog_terms))
+    return fail(APC_ERR_INVALID, "n_prog_term without prog_terms%s");
   return 0;
 }
 
@@ -133,13 +135,15 @@ double* resolve_scratch() {
 // ---------------------------------------------------------------------------
 // Kernel: block table and node compute estimate
 // ---------------------------------------------------------------------------
-constexpr int kNodesPerBlock = 2;  // one wavefront each; the other wavefronts of a node block exit at once:
-                                   // the block table's blocks share the launch and its LDS size per block,
-                                   // which decides how many of them a CU holds
 constexpr int kFusedTableBlocks = 2048;  // larger tables are built by a launch of their own
-constexpr int kProgCache = 128;    // int64 words of program staged per wave
+constexpr int kProgCache = 128;    // int64 words of program (or 64 product terms) staged per node block
 constexpr int kRecWords = 8;       // int64 words of LDS for the record's argument runs
-static_assert(kRecWords * 2 >= APC_REC_ARGS && sizeof(apc_comp_rec) == 96, "record layout");
+constexpr int kHintWords = 4;      // and for its 16 meta hints
+constexpr int kPartWords = 4 * 3 * 64;  // per wavefront and lane: partial flops, bytes, first argument with a spec
+constexpr int kNodeHeader = kProgCache + kRecWords + kHintWords + kPartWords;  // words before the value table
+static_assert(kRecWords * 2 >= APC_REC_ARGS && sizeof(apc_comp_rec) == 160, "record layout");
+static_assert(sizeof(apc_prog_term) == 16 && 2 * APC_TERMS_MAX <= kProgCache, "term layout");
+static_assert(sizeof(apc_spec_rec) == 16 && sizeof(apc_table_unit) == 32, "record layout");
 
 // One wavefront per 64 strategies of an evaluated node.  Phase 1: the lanes split the node's
 // (strategy, argument) pairs and write each argument's local (sharded) sizes
@@ -154,6 +158,9 @@ __device__ __forceinline__ apc_comp_rec load_comp_rec(const apc_problem& p, int 
   if (p.comp_recs) return p.comp_recs[i];
   apc_comp_rec r;
   const int v = __builtin_amdgcn_readfirstlane(p.comp_nodes[i]);
+  r.term_off = 0; r.n_term = 0; r.term_flags = 0;
+#pragma unroll
+  for (int a = 0; a < 16; ++a) r.arg_meta[a] = 0xFFFF;
   r.node = v;
   r.nstrat = p.node_nstrat[v];
   r.nargs = p.node_nargs[v];
@@ -360,31 +367,177 @@ __device__ __forceinline__ void node_compute_wave(const apc_problem& p, const ap
   }
 }
 
-// Touch `bytes` of an array (capped) so that the dependent loads that follow
-// find it in L2: the entry arrays stream through L2 between two builds and evict
-// the small tables.  One 4-byte load per 128-byte line per lane, results kept
-// alive but unused.
-__device__ __forceinline__ uint32_t warm_lines(const void* base, int64_t bytes, int lane,
-                                               int lanes) {
-  const int64_t cap = bytes < (1 << 16) ? bytes : (1 << 16);
-  uint32_t acc = 0;
-  for (int64_t off = (int64_t)lane * 128; off + 4 <= cap; off += (int64_t)lanes * 128)
-    acc ^= *reinterpret_cast<const uint32_t*>(reinterpret_cast<const char*>(base) + off);
-  return acc;
-}
-
-__device__ __forceinline__ uint32_t warm_problem(const apc_problem& p, int lane, int lanes) {
-  uint32_t acc = 0;
-  if (p.n_list) acc ^= warm_lines(p.lists, p.n_list * 4, lane, lanes);
-  if (p.n_meta) {
-    acc ^= warm_lines(p.meta_shape, (int64_t)p.n_meta * APC_MAX_RANK * 8, lane, lanes);
-    acc ^= warm_lines(p.meta_stride, (int64_t)p.n_meta * APC_MAX_RANK * 8, lane, lanes);
-    acc ^= warm_lines(p.meta_rank, (int64_t)p.n_meta * 4, lane, lanes);
-    acc ^= warm_lines(p.meta_itemsize, (int64_t)p.n_meta * 4, lane, lanes);
-    acc ^= warm_lines(p.meta_dtype, (int64_t)p.n_meta * 4, lane, lanes);
+// One workgroup (four wavefronts) per 64 strategies of an evaluated node whose
+// program has the product-term form.  Phase 1: the 256 lanes split the node's
+// (strategy, argument) pairs and write each argument's local sizes, an info
+// word and its local element count into the value table in LDS (row layout:
+// apc_prog_term in include/apc.h).  Phase 1b, only for programs that read a
+// broadcast size: one lane per (position, strategy).  Phase 2: lane = strategy,
+// the wavefronts share the terms (term t goes to wavefront t mod 4); each term
+// is one 16-byte LDS read, then independent reads of its factors.  Integer
+// sums do not depend on their order, so the partial sums per wavefront add up
+// to the interpreter's flops and bytes exactly.  Wavefront 0 folds them and
+// writes the estimate.  Nodes without that form (or when the table does not fit
+// in LDS) are interpreted by wavefront 0 alone.
+__device__ __forceinline__ void node_compute_block(const apc_problem& p, const apc_comp_rec& rec,
+                                                   int o0, int tid, int64_t* __restrict__ s_dyn,
+                                                   bool slow, double* __restrict__ compute,
+                                                   double* __restrict__ per_arg,
+                                                   int32_t* __restrict__ status) {
+  const int S = rec.nstrat;
+  if (o0 >= S) return;  // uniform over the workgroup
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+  int64_t* s_prog = s_dyn;
+  uint32_t* s_dst = reinterpret_cast<uint32_t*>(s_dyn + kProgCache);
+  uint16_t* s_hint = reinterpret_cast<uint16_t*>(s_dyn + kProgCache + kRecWords);
+  int64_t* s_part = s_dyn + kProgCache + kRecWords + kHintWords;
+  int64_t* s_val = s_dyn + kNodeHeader;
+  const bool fast = !slow && rec.op == APC_OP_PROGRAM && rec.n_term > 0 && p.prog_terms != nullptr;
+  if (!fast) {
+    if (wave == 0)
+      node_compute_wave(p, rec, o0, lane, s_prog, s_dst, s_val, slow, compute, per_arg, status);
+    return;
   }
-  if (p.n_tuple) acc ^= warm_lines(p.tuple_plc, (int64_t)p.n_tuple * APC_MAX_MESH_DIMS, lane, lanes);
-  return acc;
+  const int na = rec.n_edge;  // at most APC_REC_ARGS on this path
+  const int R = p.max_rank, slots = R + 2;
+  const int chunk = (S - o0 < 64) ? (S - o0) : 64;
+  const int n_words = 2 * rec.n_term;
+  int64_t term_word = 0;
+  if (tid < n_words) term_word = reinterpret_cast<const int64_t*>(p.prog_terms + rec.term_off)[tid];
+  if (tid == 0) {  // constant indices: the record stays in scalar registers
+#pragma unroll
+    for (int a = 0; a < APC_REC_ARGS; ++a) {
+      s_dst[a] = rec.dst_list[a];
+      s_hint[a] = rec.arg_meta[a];
+    }
+  }
+  __syncthreads();
+  for (int t = tid; t < chunk * na; t += 256) {
+    const int a = t / chunk, oo = t - a * chunk;
+    const size_t pos = (size_t)s_dst[a] + o0 + oo;
+    // The rows of the hinted meta are fetched together with the spec word, not
+    // after it; a word that names another meta fetches its own.
+    uint32_t mid = s_hint[a];
+    const bool hinted = mid != 0xFFFFu;
+    if (!hinted) mid = 0;
+    uint32_t w, plc = 0;
+    if (p.spec_recs) {
+      const apc_spec_rec sr = p.spec_recs[pos];
+      w = sr.word;
+      plc = sr.plc;
+    } else {
+      w = p.lists[pos];
+    }
+    int rank = p.meta_rank[mid];
+    int64_t isz = p.meta_itemsize[mid];
+    int64_t dt = p.meta_dtype[mid];
+    const ll2_t* r = reinterpret_cast<const ll2_t*>(p.meta_shape + (size_t)mid * APC_MAX_RANK);
+    ll2_t row[APC_MAX_RANK / 2];
+#pragma unroll
+    for (int q = 0; q < APC_MAX_RANK / 2; ++q) row[q] = r[q];
+    const bool none = (w == APC_SPEC_NONE);
+    if (!none && (!hinted || (w >> APC_TUPLE_BITS) != mid)) {
+      mid = w >> APC_TUPLE_BITS;
+      rank = p.meta_rank[mid];
+      isz = p.meta_itemsize[mid];
+      dt = p.meta_dtype[mid];
+      r = reinterpret_cast<const ll2_t*>(p.meta_shape + (size_t)mid * APC_MAX_RANK);
+#pragma unroll
+      for (int q = 0; q < APC_MAX_RANK / 2; ++q) row[q] = r[q];
+    }
+    if (!p.spec_recs) plc = load_tuple(p.tuple_plc, none ? 0u : (w & kTupleMask));
+    if (none) rank = 0;
+    int64_t numel = 1;
+    int64_t* col = s_val + (size_t)(R + a * slots) * 64 + oo;
+#pragma unroll
+    for (int d = 0; d < APC_MAX_RANK; ++d) {
+      if (d >= R) break;  // uniform
+      int64_t sz = (d & 1) ? row[d >> 1].y : row[d >> 1].x;
+      if (d >= rank) {
+        sz = 1;
+      } else {
+        for (int i = 0; i < p.model.ndim; ++i) {
+          const int c = (plc >> (8 * i)) & 0xFF;
+          if ((c & kKindMask) == kShard && (c & kArgMask) == d) sz = ceil_div_pos(sz, p.model.mesh_shape[i]);
+        }
+      }
+      col[d * 64] = sz;
+      numel *= sz;  // sizes past the rank are 1
+    }
+    // info word: rank | itemsize << 8 | dtype << 40, or -1 for a missing spec
+    col[R * 64] = none ? -1 : ((int64_t)rank | (isz << 8) | (dt << 40));
+    col[(R + 1) * 64] = numel;
+  }
+  if (tid < n_words) s_prog[tid] = term_word;
+  __syncthreads();
+  if (rec.term_flags & APC_TERMS_BCAST) {
+    // broadcast of all arguments at a right-aligned position: the size of the last
+    // argument that reaches the position with a size other than 1
+    for (int t = tid; t < chunk * R; t += 256) {
+      const int pos = t / chunk, oo = t - pos * chunk;
+      int64_t size = 1;
+      for (int a = 0; a < na; ++a) {
+        const int64_t* col = s_val + (size_t)(R + a * slots) * 64 + oo;
+        const int64_t info = col[R * 64];
+        const int r = info < 0 ? -1 : (int)(info & 0xFF);
+        if (pos >= r) continue;
+        const int64_t sz = col[(r - 1 - pos) * 64];
+        if (sz != 1) size = sz;
+      }
+      s_val[pos * 64 + oo] = size;
+    }
+    __syncthreads();
+  }
+  // Phase 2.  Wavefront w takes the terms and the arguments congruent to w mod 4;
+  // `first` is its lowest argument that has a spec (the node's dtype is that of
+  // the lowest over all wavefronts) or 255.
+  int64_t flops = 0, nbytes = 0;
+  int first = 255, dtype = 1;  // float32 when the node has no tensor argument
+  if (lane < chunk) {
+    for (int t = wave; t < rec.n_term; t += 4) {
+      const ll2_t tw = *reinterpret_cast<const ll2_t*>(s_prog + 2 * t);
+      int64_t term = tw.x;
+      // the term is the same for every lane: its factor list goes to scalar registers
+      const uint32_t ilo = __builtin_amdgcn_readfirstlane((uint32_t)tw.y);
+      const uint32_t ihi = __builtin_amdgcn_readfirstlane((uint32_t)((uint64_t)tw.y >> 32));
+      int64_t v[7];
+#pragma unroll
+      for (int f = 0; f < 7; ++f) {
+        const uint32_t i = ((f < 4 ? ilo >> (8 * f) : ihi >> (8 * (f - 4))) & 0xFF);
+        v[f] = (i != 0xFF) ? s_val[i * 64 + lane] : 1;
+      }
+#pragma unroll
+      for (int f = 0; f < 7; ++f) term *= v[f];
+      if (ihi >> 24) nbytes += term; else flops += term;
+    }
+    for (int a = wave; a < na; a += 4) {
+      const int64_t* col = s_val + (size_t)(R + a * slots) * 64 + lane;
+      const int64_t info = col[R * 64];
+      const int64_t numel = col[(R + 1) * 64];
+      if (info < 0) continue;
+      if (first == 255) { first = a; dtype = (int)(info >> 40); }
+      nbytes += numel * (int64_t)((info >> 8) & 0xFFFFFFFF);
+    }
+  }
+  if (wave != 0) {
+    s_part[(wave * 3 + 0) * 64 + lane] = flops;
+    s_part[(wave * 3 + 1) * 64 + lane] = nbytes;
+    s_part[(wave * 3 + 2) * 64 + lane] = (int64_t)first | ((int64_t)dtype << 8);
+  }
+  __syncthreads();
+  if (wave == 0 && lane < chunk) {
+#pragma unroll
+    for (int w = 1; w < 4; ++w) {
+      flops += s_part[(w * 3 + 0) * 64 + lane];
+      nbytes += s_part[(w * 3 + 1) * 64 + lane];
+      const int64_t fd = s_part[(w * 3 + 2) * 64 + lane];
+      if ((int)(fd & 0xFF) < first) { first = (int)(fd & 0xFF); dtype = (int)(fd >> 8); }
+    }
+    const int64_t idx = rec.comp_off + o0 + lane;
+    const double result = roofline(p, flops, nbytes, dtype, status);
+    compute[idx] = result;
+    per_arg[idx] = result / (double)rec.nargs;
+  }
 }
 
 // Block table.  Edges whose producer run and consumer run are the same spec
@@ -396,40 +549,59 @@ __device__ __forceinline__ uint32_t warm_problem(const apc_problem& p, int lane,
 // with its sign bit set when the two placements differ (costs are never
 // negative, so the sign is free to carry the transition flag): the entry kernel
 // reads comm and transition with one coalesced load and no spec words.
-template <bool kWarm>
 __device__ __forceinline__ void pair_table_block(const apc_problem& p, double* __restrict__ table,
                                                  int unit) {
-  const uint32_t keep = kWarm ? warm_problem(p, threadIdx.x, blockDim.x) : 0u;
-  const int b = p.table_unit_block[unit];
-  const int64_t base = p.block_off[b];
-  const apc_edge ed = p.edges[p.block_edge[b]];  // any edge with this matrix
-  // a compressed matrix has one column / row per distinct word of the two runs
-  const bool squeezed = (ed.flags & APC_EDGE_COMPRESSED) != 0;
-  const uint32_t ncol = squeezed ? (uint32_t)ed.flags >> APC_EDGE_USRC_SHIFT : (uint32_t)ed.ssrc;
-  const uint32_t nrow = squeezed ? (uint32_t)p.block_udst[b] : (uint32_t)ed.sdst;
-  const int64_t l64 = (int64_t)unit * 256 - base + threadIdx.x;
-  if (l64 < (int64_t)ncol * nrow) {
-    const uint32_t l = (uint32_t)l64;
-    uint32_t o = l / ncol, j = l - o * ncol;
-    if (squeezed) {  // position in its run of an occurrence of that word
-      o = (uint32_t)p.list_ufirst[(size_t)ed.dst_list + o];
-      j = (uint32_t)p.list_ufirst[(size_t)ed.src_list + j];
-    }
-    const uint32_t sw = p.lists[(size_t)ed.src_list + j];
-    const uint32_t tw = p.lists[(size_t)ed.dst_list + o];
+  const int tid = threadIdx.x;
+  apc_table_unit u;
+  if (p.table_units) {
+    u = p.table_units[unit];
+  } else {  // the same fields through the block and edge arrays
+    const int b = p.table_unit_block[unit];
+    const apc_edge ed = p.edges[p.block_edge[b]];  // any edge with this matrix
+    const bool squeezed = (ed.flags & APC_EDGE_COMPRESSED) != 0;
+    u.default_off = ed.default_off;
+    u.src_list = ed.src_list;
+    u.dst_list = ed.dst_list;
+    u.ncol = squeezed ? (uint32_t)ed.flags >> APC_EDGE_USRC_SHIFT : (uint32_t)ed.ssrc;
+    u.nrow = squeezed ? (uint32_t)p.block_udst[b] : (uint32_t)ed.sdst;
+    u.first = (uint32_t)((int64_t)unit * 256 - p.block_off[b]);
+    u.flags = squeezed ? APC_EDGE_COMPRESSED : 0;
+  }
+  const uint32_t l = u.first + (uint32_t)tid;
+  if (l >= u.ncol * u.nrow) return;  // a matrix has fewer than 2^31 elements
+  uint32_t o = l / u.ncol, j = l - o * u.ncol;
+  if (u.flags & APC_EDGE_COMPRESSED) {  // position in its run of an occurrence of that word
+    o = (uint32_t)p.list_ufirst[(size_t)u.dst_list + o];
+    j = (uint32_t)p.list_ufirst[(size_t)u.src_list + j];
+  }
+  // the two specs: a record per side when the caller made them, else the word,
+  // then its tuple row and its tensor's shape and stride rows
+  uint32_t sw, tw, src_plc, tgt_plc;
+  int64_t nbytes;
+  bool contig;
+  if (p.spec_recs) {
+    const apc_spec_rec rs = p.spec_recs[(size_t)u.src_list + j];
+    const apc_spec_rec rt = p.spec_recs[(size_t)u.dst_list + o];
+    sw = rs.word; tw = rt.word;
+    src_plc = rs.plc; tgt_plc = rt.plc;
+    nbytes = rs.nbytes2 >> 1;
+    contig = (rs.nbytes2 & 1) != 0;
+  } else {
+    sw = p.lists[(size_t)u.src_list + j];
+    tw = p.lists[(size_t)u.dst_list + o];
     if (sw != APC_SPEC_NONE && tw != APC_SPEC_NONE) {
-      const uint32_t st = sw & kTupleMask, tt = tw & kTupleMask;
-      int64_t nbytes;
-      bool contig;
+      src_plc = load_tuple(p.tuple_plc, sw & kTupleMask);
+      tgt_plc = load_tuple(p.tuple_plc, tw & kTupleMask);
       meta_bytes_contig(p, sw >> APC_TUPLE_BITS, nbytes, contig);
-      const double c = redistribute_cost(load_tuple(p.tuple_plc, st), load_tuple(p.tuple_plc, tt),
-                                         nbytes, contig, p.model);
-      table[base + l] = (st != tt) ? -c : c;
-    } else {  // a missing spec keeps the default row's value and is no transition
-      table[base + l] = p.default_vals[ed.default_off + (int64_t)l];  // never squeezed
     }
   }
-  asm volatile("" ::"v"(keep));
+  double* out = table + (int64_t)unit * 256 + tid;
+  if (sw != APC_SPEC_NONE && tw != APC_SPEC_NONE) {
+    const double c = redistribute_cost(src_plc, tgt_plc, nbytes, contig, p.model);
+    *out = ((sw & kTupleMask) != (tw & kTupleMask)) ? -c : c;
+  } else {  // a missing spec keeps the default row's value and is no transition
+    *out = p.default_vals[u.default_off + (int64_t)l];  // never a compressed matrix
+  }
 }
 
 // Blocks [0, table_blocks) fill the pair table, the rest price the nodes of
@@ -443,21 +615,16 @@ prepare_kernel(apc_problem p, double* __restrict__ table, int table_blocks, int 
                int32_t* __restrict__ status) {
   extern __shared__ int64_t s_dyn[];
   if ((int)blockIdx.x < table_blocks) {
-    pair_table_block<true>(p, table, blockIdx.x);
+    pair_table_block(p, table, blockIdx.x);
     return;
   }
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  if (wave >= kNodesPerBlock) return;
-  const int unit = ((int)blockIdx.x - table_blocks) * kNodesPerBlock + wave;
-  const int chunks = (p.max_nstrat + 63) >> 6;  // wavefronts per node
+  const int unit = (int)blockIdx.x - table_blocks;
+  const int chunks = (p.max_nstrat + 63) >> 6;  // workgroups per node
   const int i = unit / chunks;
   if (i >= p.n_comp_node) return;
   const apc_comp_rec rec = load_comp_rec(p, i);
-  const int per_wave = kProgCache + kRecWords + (slow ? 0 : p.max_node_args * (p.max_rank + 2) * 64);
-  int64_t* s_prog = s_dyn + (size_t)wave * per_wave;
-  node_compute_wave(p, rec, (unit - i * chunks) * 64, threadIdx.x & 63, s_prog,
-                    reinterpret_cast<uint32_t*>(s_prog + kProgCache), s_prog + kProgCache + kRecWords,
-                    slow != 0, compute, per_arg, status);
+  node_compute_block(p, rec, (unit - i * chunks) * 64, threadIdx.x, s_dyn, slow != 0, compute, per_arg,
+                     status);
 }
 
 // The block table alone, for tables of many units: no dynamic LDS (which in
@@ -466,7 +633,7 @@ prepare_kernel(apc_problem p, double* __restrict__ table, int table_blocks, int 
 // themselves).
 __global__ void __launch_bounds__(256)
 pair_table_kernel(apc_problem p, double* __restrict__ table) {
-  pair_table_block<false>(p, table, blockIdx.x);
+  pair_table_block(p, table, blockIdx.x);
 }
 
 // ---------------------------------------------------------------------------
@@ -690,18 +857,16 @@ int launch_prepare(const apc_problem* p, double* table, bool do_nodes, double* c
     table_blocks = 0;
   }
   const int64_t chunks = (p->max_nstrat + 63) >> 6;
-  const int64_t units = (int64_t)p->n_comp_node * chunks;  // one wavefront per 64 strategies of a node
+  const int64_t units = (int64_t)p->n_comp_node * chunks;  // one workgroup per 64 strategies of a node
   if (do_nodes && (chunks < 1 || units > (1ll << 30)))
     return fail(APC_ERR_INVALID, "launch_prepare: max_nstrat must be >= 1 and n_comp_node * chunks < 2^30%s");
-  const int node_blocks = do_nodes ? (int)((units + kNodesPerBlock - 1) / kNodesPerBlock) : 0;
+  const int node_blocks = do_nodes ? (int)units : 0;
   if (table_blocks + node_blocks == 0) return 0;
-  // LDS for the local-size staging (a CU has 160 KB); beyond 96 KB per block,
-  // sizes are read on demand instead
-  const int64_t words = (int64_t)p->max_node_args * (p->max_rank + 2) * 64;
-  const int slow = ((kProgCache + kRecWords + words) * kNodesPerBlock * 8 > 96 * 1024 ||
-                    p->n_meta == 0 || p->n_tuple == 0) ? 1 : 0;
-  const size_t lds =
-      do_nodes ? (size_t)kNodesPerBlock * (kProgCache + kRecWords + (slow ? 0 : words)) * 8 : 0;
+  // LDS for the value table of a node workgroup (a CU has 160 KB); beyond 96 KB
+  // per workgroup, sizes are read on demand instead
+  const int64_t words = ((int64_t)p->max_rank + (int64_t)p->max_node_args * (p->max_rank + 2)) * 64;
+  const int slow = ((kNodeHeader + words) * 8 > 96 * 1024 || p->n_meta == 0 || p->n_tuple == 0) ? 1 : 0;
+  const size_t lds = do_nodes ? (size_t)(kNodeHeader + (slow ? 0 : words)) * 8 : 0;
   if (lds > 0) {  // dynamic LDS beyond the 64 KB default needs the limit raised: once per device
     DeviceState* dev = current_device_state();
     if (!dev) return APC_ERR_LAUNCH;

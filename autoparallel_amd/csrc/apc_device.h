@@ -47,9 +47,31 @@ typedef long long ll2_t __attribute__((ext_vector_type(2)));
 // Cost model, scalar device functions (order of operations is the contract)
 // ---------------------------------------------------------------------------
 
+// x / d, correctly rounded.  A quotient by a power of two is the product with
+// its reciprocal, bit for bit (both are the one correctly rounded value of the
+// same real number), and costs one instruction instead of a division sequence:
+// mesh sizes, shard counts and the MI355X memory bandwidth (8 * 1024^4 B/s) are
+// powers of two.  The branch is on the divisor, which is the same for every
+// lane of a wavefront wherever this is called with a model constant.
+__device__ __forceinline__ double div_exact(double x, double d) {
+  const uint64_t bits = (uint64_t)__double_as_longlong(d);
+  const uint64_t exp = (bits >> 52) & 0x7FF;
+  // a normal power of two whose reciprocal is normal too
+  if ((bits & 0x800FFFFFFFFFFFFFull) == 0 && exp >= 2 && exp <= 2044)
+    return x * __longlong_as_double((long long)((2046 - exp) << 52));
+  return x / d;
+}
+
+// x / n for a positive integer n
+__device__ __forceinline__ double div_int(double x, int64_t n) {
+  if ((n & (n - 1)) == 0 && n > 0 && n < (1ll << 62))
+    return x * __longlong_as_double((long long)((uint64_t)(1023 - (63 - __clzll((unsigned long long)n))) << 52));
+  return x / (double)n;
+}
+
 // compute_read_write_time (compute_estimation.py:391-403)
 __device__ __forceinline__ double rw_time(double nbytes, double gmem_bw) {
-  double t = nbytes / gmem_bw * 1e6;
+  double t = div_exact(nbytes, gmem_bw) * 1e6;
   t = t / 0.70;
   return t >= 7.0 ? t : 7.0;  // max(t, 7): keeps t on ties, as Python's max
 }
@@ -121,7 +143,7 @@ __device__ __forceinline__ double collective_cost(int kind, int64_t nbytes, int 
   int n = m.mesh_shape[i];
   int hops = (kind == 2) ? 2 * (n - 1) : (n - 1);
   double latency = 6.6 + (double)hops * m.mesh_lat[i];
-  double bw = (g * (double)hops / (double)n) / m.mesh_bw[i];
+  double bw = div_int(g * (double)hops, n) / m.mesh_bw[i];
   double t = latency + bw * 1e6;
   if (kind == 1) t = t * 5.0;
   return t;
@@ -145,43 +167,53 @@ __device__ double redistribute_cost(uint32_t src, uint32_t tgt, int64_t tensor_b
     if (((src >> (8 * i)) & kKindMask) == kShard) num_shards *= m.mesh_shape[i];
     tgt_all_shard &= (((tgt >> (8 * i)) & kKindMask) == kShard);
   }
-  double gb = (double)tensor_bytes / (double)num_shards / 1024.0 / 1024.0 / 1024.0;
+  double gb = div_int((double)tensor_bytes, num_shards) / 1024.0 / 1024.0 / 1024.0;
   // order rule of estimate_strategy_comms_cost (:253-258), or an order forced by
   // the caller of redistribute_cost (order_mode 1: 0..ndim-1, 2: ndim-1..0)
   const bool reversed =
       m.order_mode == 0
           ? ((ndim == 2) && (src == (uint32_t)(kPartialSum | (kPartialSum << 8))) && tgt_all_shard)
           : (m.order_mode == 2);
+  // The lanes of a wavefront hold unrelated (source, target) pairs, so a branch
+  // per transition kind would make every wavefront walk all of them, each with
+  // its own divisions.  Instead a step selects the operands of the one
+  // collective and the one read/write time it may need and evaluates those
+  // once; which of the reference's additions happen is decided by predicates.
+  // An addition that the reference does not make is skipped, not made with
+  // zero, except `copies * rw` of Shard -> Shard, which the reference also adds
+  // when copies is 0.
   double cost = 0.0;
+  bool forbidden = false;
   for (int step = 0; step < ndim; ++step) {
     const int i = reversed ? (ndim - 1 - step) : step;
     const int cur = (src >> (8 * i)) & 0xFF, tg = (tgt >> (8 * i)) & 0xFF;
     if (cur == tg) continue;
     const int n = m.mesh_shape[i];
-    if (!contiguous) cost += rw_time(gb * 2.0 * 1073741824.0, m.gmem_bw);
     const int ck = cur & kKindMask, tk = tg & kKindMask;
-    if (ck == kShard && tg == 0) {
-      gb = gb * (double)n;
-      cost += collective_cost(0, (int64_t)(gb * 1073741824.0), i, m);
-      if ((cur & kArgMask) != 0) cost += rw_time(gb * 2.0 * 1073741824.0, m.gmem_bw);
-    } else if (ck == kShard && tk == kShard) {
-      cost += collective_cost(1, (int64_t)(gb * 1073741824.0), i, m);
-      int copies = ((cur & kArgMask) != 0) + ((tg & kArgMask) != 0);
-      cost += (double)copies * rw_time(gb * 2.0 * 1073741824.0, m.gmem_bw);
-    } else if (ck == kPartial && tg == 0) {
-      cost += collective_cost(2, (int64_t)(gb * 1073741824.0), i, m);
-    } else if (ck == kPartial && tk == kShard) {
-      cost += collective_cost(3, (int64_t)(gb * 1073741824.0), i, m);
-      if ((tg & kArgMask) != 0) cost += rw_time(gb * 2.0 * 1073741824.0, m.gmem_bw);
-      gb = gb / (double)n;
-    } else if (ck == kShard && tk == kPartial) {
-      return INFINITY;
-    } else if (cur == 0 && tk == kPartial) {
-      return INFINITY;
+    const bool s_r = ck == kShard && tg == 0;      // allgather, on gb * n
+    const bool s_s = ck == kShard && tk == kShard;  // all_to_all
+    const bool p_r = ck == kPartial && tg == 0;     // allreduce
+    const bool p_s = ck == kPartial && tk == kShard;  // reduce_scatter, then gb / n
+    forbidden |= (ck == kShard && tk == kPartial) || (cur == 0 && tk == kPartial);
+    if (!contiguous) cost += rw_time(gb * 2.0 * 1073741824.0, m.gmem_bw);
+    if (s_r | s_s | p_r | p_s) {
+      if (s_r) gb = gb * (double)n;
+      const int kind = s_r ? 0 : s_s ? 1 : p_r ? 2 : 3;
+      cost += collective_cost(kind, (int64_t)(gb * 1073741824.0), i, m);
+      // reshuffle penalties: S(d != 0) -> R on the gathered bytes, each side of
+      // S(d) -> S(d') that is not dim 0, P -> S(d' != 0)
+      const int copies = s_r ? ((cur & kArgMask) != 0)
+                             : s_s ? ((cur & kArgMask) != 0) + ((tg & kArgMask) != 0)
+                                   : p_s ? ((tg & kArgMask) != 0) : 0;
+      if (s_s | (copies != 0)) {
+        const double rw = rw_time(gb * 2.0 * 1073741824.0, m.gmem_bw);
+        cost += s_s ? (double)copies * rw : rw;
+      }
+      if (p_s) gb = div_int(gb, n);
     }
     contiguous = true;
   }
-  return cost;
+  return forbidden ? INFINITY : cost;
 }
 
 __device__ __forceinline__ uint32_t load_tuple(const uint8_t* tuple_plc, uint32_t t) {

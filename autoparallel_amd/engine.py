@@ -173,6 +173,10 @@ class CostEngine:
         p.n_comp_node = g.comp_nodes.shape[0]
         p.comp_nodes = up("comp_nodes", g.comp_nodes)
         p.comp_recs = up("comp_recs", g.comp_records())
+        terms, _ = g.program_terms()
+        p.n_prog_term = terms.shape[0]
+        p.prog_terms = up("prog_terms", terms)
+        p.spec_recs = up("spec_recs", g.spec_records())
         p.max_nstrat = int(g.node_nstrat[g.comp_nodes].max()) if g.comp_nodes.shape[0] else 1
         mult = g.node_multiplier if g.node_multiplier is not None else np.ones(g.num_nodes, np.int32)
         p.node_multiplier = up("node_multiplier", mult)
@@ -236,6 +240,7 @@ class CostEngine:
         p.table_size = int(block_off[-1])
         p.n_table_unit = unit_block.shape[0]
         p.table_unit_block = up("table_unit_block", unit_block)
+        p.table_units = up("table_units", g.table_unit_records(squeezed))
         self.problem = p
 
         E, NC = g.num_slots, g.num_compute

@@ -316,14 +316,26 @@ class PackedGraph:
     COMP_REC_DTYPE = np.dtype([
         ("node", "<i4"), ("nstrat", "<i4"), ("nargs", "<i4"), ("op", "<i4"), ("comp_off", "<i8"),
         ("prog_off", "<i8"), ("prog_len", "<i4"), ("n_edge", "<i4"), ("dst_list", "<u4", (14,)),
+        ("term_off", "<i4"), ("n_term", "<i4"), ("term_flags", "<i4"), ("arg_meta", "<u2", (16,)),
+        ("reserved", "<i4", (5,)),
     ])
+    PROG_TERM_DTYPE = np.dtype([("coeff", "<i8"), ("idx", "u1", (7,)), ("to_bytes", "u1")])
+    SPEC_REC_DTYPE = np.dtype([("word", "<u4"), ("plc", "<u4"), ("nbytes2", "<i8")])
+    TABLE_UNIT_DTYPE = np.dtype([
+        ("default_off", "<i8"), ("src_list", "<u4"), ("dst_list", "<u4"), ("ncol", "<u4"), ("nrow", "<u4"),
+        ("first", "<u4"), ("flags", "<u4"),
+    ])
+    TERMS_BCAST = 1
+    TERMS_MAX = 64
 
     def comp_records(self) -> np.ndarray:
-        """One 96-byte record per evaluated node (``apc_comp_rec`` of
-        include/apc.h): what the node kernel reads about the node, gathered."""
+        """One 160-byte record per evaluated node (``apc_comp_rec`` of
+        include/apc.h): what the node kernel reads about the node, gathered,
+        and where its program stands as product terms (``program_terms``)."""
         v = self.comp_nodes.astype(np.int64)
         rec = np.zeros(v.shape[0], self.COMP_REC_DTYPE)
-        assert rec.dtype.itemsize == 96
+        assert rec.dtype.itemsize == 160
+        rec["arg_meta"] = 0xFFFF
         e0 = self.node_edge_off[:-1].astype(np.int64)[v]
         n_edge = (self.node_edge_off[1:].astype(np.int64)[v] - e0)
         rec["node"], rec["nstrat"], rec["nargs"] = v, self.node_nstrat[v], self.node_nargs[v]
@@ -332,6 +344,144 @@ class PackedGraph:
         for a in range(self.REC_ARGS):
             has = n_edge > a
             rec["dst_list"][has, a] = self.edge_dst_list[(e0 + a)[has]].astype(np.uint32)
+            # meta of the argument's first spec, if it has one and it fits the field
+            first = self.lists[self.edge_dst_list[(e0 + a)[has]]].astype(np.int64)
+            mid = first >> TUPLE_BITS
+            rec["arg_meta"][np.nonzero(has)[0], a] = np.where((first != SPEC_NONE) & (mid < 0xFFFF), mid, 0xFFFF)
+        _, where = self.program_terms()
+        for i, node in enumerate(v):
+            if self.node_op[node] != OP_PROGRAM or n_edge[i] > self.REC_ARGS:
+                continue
+            # a node with more arguments than rows of the value table can name keeps the interpreter
+            if self.max_rank + int(n_edge[i]) * (self.max_rank + 2) > 0xFF:
+                continue
+            hit = where.get(int(self.node_prog_off[node]))
+            if hit is not None:
+                rec["term_off"][i], rec["n_term"][i], rec["term_flags"][i] = hit
+        return rec
+
+    def program_terms(self):
+        """Every distinct compute program as product terms (``apc_prog_term`` of
+        include/apc.h).  Returns (terms, where): ``where[prog_off] = (term_off,
+        n_term, flags)`` for the programs that have this form; one with a term
+        of more than 7 factors or more than TERMS_MAX terms has none and is
+        interpreted word by word."""
+        cached = self.__dict__.get("_program_terms")
+        if cached is not None:
+            return cached
+        R = self.max_rank
+        slots = R + 2
+        out: List[tuple] = []
+        where: Dict[int, Tuple[int, int, int]] = {}
+        has_prog = self.node_op == OP_PROGRAM
+        offs = np.unique(self.node_prog_off[has_prog]) if has_prog.any() else np.zeros(0, np.int64)
+        lens = {int(o): int(l) for o, l in zip(self.node_prog_off[has_prog], self.node_prog_len[has_prog])}
+        for off in offs:
+            off = int(off)
+            pr = [int(x) for x in self.prog[off:off + lens[off]]]
+            terms, flags, ok = [], 0, True
+            q = 2
+            for _ in range(pr[0]):
+                coeff, nfac = pr[q], pr[q + 1]
+                q += 2
+                idx = []
+                for _ in range(nfac):
+                    a, d = pr[q], pr[q + 1]
+                    q += 2
+                    if d < R:  # no tensor of the graph has that dim otherwise: its size is 1
+                        idx.append(R + a * slots + d)
+                terms.append((coeff, idx, 0))
+            for _ in range(pr[1]):
+                coeff, rank = pr[q], pr[q + 1]
+                q += 2
+                idx = []
+                for _ in range(rank):
+                    kind, x, y = pr[q], pr[q + 1], pr[q + 2]
+                    q += 3
+                    if kind == DIM_CONST:
+                        coeff *= x
+                    elif kind == DIM_ARG:
+                        if y < R:
+                            idx.append(R + x * slots + y)
+                    elif kind == DIM_ARGNUMEL:
+                        idx.append(R + x * slots + R + 1)
+                    else:  # DIM_BCAST: no tensor reaches a position past the largest rank
+                        if x < R:
+                            idx.append(x)
+                            flags |= self.TERMS_BCAST
+                terms.append((coeff, idx, 1))
+            assert q == len(pr)
+            if len(terms) > self.TERMS_MAX or any(len(t[1]) > 7 or max(t[1], default=0) > 0xFE for t in terms):
+                ok = False
+            if not (-(2**63) <= min((t[0] for t in terms), default=0) and max((t[0] for t in terms), default=0) < 2**63):
+                ok = False
+            if ok and terms:
+                where[off] = (len(out), len(terms), flags)
+                out.extend(terms)
+        arr = np.zeros(len(out), self.PROG_TERM_DTYPE)
+        assert arr.dtype.itemsize == 16
+        for i, (coeff, idx, to_bytes) in enumerate(out):
+            arr["coeff"][i] = coeff
+            arr["idx"][i] = idx + [0xFF] * (7 - len(idx))
+            arr["to_bytes"][i] = to_bytes
+        object.__setattr__(self, "_program_terms", (arr, where))
+        return arr, where
+
+    def meta_bytes_contiguous(self):
+        """(nbytes int64[M], contiguous bool[M]) per tensor meta: itemsize *
+        prod(shape), and whether its strides are those of a contiguous tensor
+        (torch ``check_contiguous_sizes_strides``,
+        _prims_common/__init__.py:252-293: dims of size 1 are skipped, the others
+        must have the running product of the sizes to their right as stride)."""
+        M = self.meta_rank.shape[0]
+        nbytes = self.meta_itemsize.astype(np.int64).copy()
+        expected = np.ones(M, np.int64)
+        expected_max = np.ones(M, np.int64)
+        ok = np.ones(M, bool)
+        with np.errstate(over="ignore"):
+            for d in range(MAX_RANK - 1, -1, -1):
+                live = d < self.meta_rank
+                x, y = self.meta_shape[:, d], self.meta_stride[:, d]
+                nbytes = np.where(live, nbytes * x, nbytes)
+                check = live & (x != 1)
+                ok &= ~(check & (y != expected) & (y != expected_max))
+                expected_max = np.where(check, expected_max * np.maximum(x, 1), expected_max)
+                expected = np.where(check, expected * x, expected)
+        return nbytes, ok
+
+    def spec_records(self) -> np.ndarray:
+        """One ``apc_spec_rec`` per position of ``lists``: the spec word, its
+        placement bytes and its tensor's byte count and contiguity."""
+        L = self.lists.shape[0]
+        rec = np.zeros(L, self.SPEC_REC_DTYPE)
+        assert rec.dtype.itemsize == 16
+        rec["word"] = self.lists
+        some = self.lists != SPEC_NONE
+        w = self.lists[some].astype(np.int64)
+        plc = np.ascontiguousarray(self.tuple_plc).view("<u4").reshape(-1)
+        nbytes, contig = self.meta_bytes_contiguous()
+        rec["plc"][some] = plc[w & (MAX_TUPLES - 1)]
+        rec["nbytes2"][some] = (nbytes[w >> TUPLE_BITS] << 1) | contig[w >> TUPLE_BITS]
+        return rec
+
+    def table_unit_records(self, compressed: bool = False) -> np.ndarray:
+        """One ``apc_table_unit`` per 256 elements of the block table: the two
+        runs, the matrix extent and the unit's first element, so that a
+        workgroup of the table build starts from one load."""
+        block_edge, block_off, unit_block, _, edge_usrc, block_udst = self.block_table(compressed)
+        rec = np.zeros(unit_block.shape[0], self.TABLE_UNIT_DTYPE)
+        assert rec.dtype.itemsize == 32
+        if unit_block.shape[0] == 0:
+            return rec
+        e = block_edge[unit_block].astype(np.int64)
+        squeezed = edge_usrc[e] > 0
+        rec["default_off"] = self.edge_default_off[e]
+        rec["src_list"] = self.edge_src_list[e].astype(np.uint32)
+        rec["dst_list"] = self.edge_dst_list[e].astype(np.uint32)
+        rec["ncol"] = np.where(squeezed, edge_usrc[e], self.edge_ssrc[e])
+        rec["nrow"] = np.where(squeezed, block_udst[unit_block], self.edge_sdst[e])
+        rec["first"] = np.arange(unit_block.shape[0], dtype=np.int64) * 256 - block_off[:-1][unit_block]
+        rec["flags"] = np.where(squeezed, EDGE_COMPRESSED, 0)
         return rec
 
     @property

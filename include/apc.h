@@ -74,7 +74,7 @@ typedef struct apc_edge {
 } apc_edge; /* 64 bytes */
 
 /* Everything the node estimate reads about one evaluated node, in one record,
- * so that a wavefront starts with one load instead of a chain through the
+ * so that a workgroup starts with one load instead of a chain through the
  * node, edge-offset and edge arrays. */
 #define APC_REC_ARGS 14
 typedef struct apc_comp_rec {
@@ -87,7 +87,61 @@ typedef struct apc_comp_rec {
   int32_t prog_len;
   int32_t n_edge;    /* arguments with an edge                                */
   uint32_t dst_list[APC_REC_ARGS]; /* dst_list of the node's first edges      */
-} apc_comp_rec; /* 96 bytes */
+  int32_t term_off;  /* into prog_terms: the node's program as product terms  */
+  int32_t n_term;    /* 0: none, the kernel interprets prog                   */
+  int32_t term_flags; /* APC_TERMS_*                                          */
+  /* the tensor meta behind argument a's specs (all strategies of a node see the
+   * same tensor per argument), so that its rows are fetched together with the
+   * spec words instead of after them; 0xFFFF: none or not uniform.  A hint: a
+   * spec whose meta differs is looked up by its own. */
+  uint16_t arg_meta[16];
+  int32_t reserved[5];
+} apc_comp_rec; /* 160 bytes */
+
+/* A compute program as independent product terms, so that the wavefronts of a
+ * workgroup can share them: value = coeff * product of the per-strategy values
+ * idx[k] names (0xFF: no factor), added to the node's flops, or to its bytes
+ * when `to_bytes` is set.  The per-strategy values are rows of the workgroup's
+ * table of local sizes: rows [0, max_rank) the broadcast of all arguments'
+ * sizes at a right-aligned position (row = position from the right), then per
+ * argument a the rows max_rank + a * (max_rank + 2) + d: d < max_rank the local
+ * size of dim d, d == max_rank + 1 the local element count.  Constant dims of
+ * an output are folded into coeff.  Made from `prog` by the host
+ * (PackedGraph.program_terms); same integers as the interpreted program. */
+typedef struct apc_prog_term {
+  int64_t coeff;
+  uint8_t idx[7];
+  uint8_t to_bytes;
+} apc_prog_term; /* 16 bytes */
+#define APC_TERMS_BCAST 1 /* some term reads a broadcast row */
+#define APC_TERMS_MAX 64  /* terms per program                 */
+
+/* A spec word of `lists` with what the redistribution cost reads behind it:
+ * the placement bytes of its tuple, and itemsize * prod(shape) and the
+ * contiguity of its tensor meta (spec_to_bytes,
+ * torch:distributed/tensor/_collective_utils.py:230-232, and
+ * check_contiguous_sizes_strides, torch:_prims_common/__init__.py:252-293).
+ * One 16-byte load per side of a table element instead of the word, then its
+ * tuple row, then two shape/stride rows.  Made per position of `lists` by the
+ * host (PackedGraph.spec_records). */
+typedef struct apc_spec_rec {
+  uint32_t word;   /* lists[k]                                              */
+  uint32_t plc;    /* tuple_plc row of the word, one byte per mesh dim      */
+  int64_t nbytes2; /* nbytes << 1 | contiguous; 0 for APC_SPEC_NONE          */
+} apc_spec_rec; /* 16 bytes */
+
+/* What a workgroup of the block-table build reads about its 256 elements, in
+ * one record instead of a chain through table_unit_block, block_off,
+ * block_edge and the edge array. */
+typedef struct apc_table_unit {
+  int64_t default_off; /* default rows of the matrix's edge, or -1            */
+  uint32_t src_list;   /* the two runs of spec words                          */
+  uint32_t dst_list;
+  uint32_t ncol;       /* columns / rows of the stored matrix (of distinct    */
+  uint32_t nrow;       /* words when compressed)                              */
+  uint32_t first;      /* element of the matrix that the unit starts at       */
+  uint32_t flags;      /* APC_EDGE_COMPRESSED or 0                            */
+} apc_table_unit; /* 32 bytes */
 
 /* Cost-model constants (host values, passed by value into the kernels). */
 typedef struct apc_model {
@@ -252,6 +306,12 @@ typedef struct apc_problem {
   /* entries per work item: 0 or APC_ITEM_ENTRIES, or 2 * APC_ITEM_ENTRIES (block
    * table only), as the items array was built */
   int32_t item_entries;
+  /* optional accelerators of the prepare launch, each derived from the arrays
+   * above by the host (NULL: the kernels walk those arrays instead) */
+  const apc_table_unit* table_units; /* [n_table_unit]                          */
+  const apc_spec_rec* spec_recs;     /* [n_list]                                */
+  int64_t n_prog_term;
+  const apc_prog_term* prog_terms;   /* named by apc_comp_rec.term_off / n_term */
 } apc_problem;
 
 int apc_version(void);

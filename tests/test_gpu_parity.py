@@ -459,6 +459,61 @@ def test_more_arguments_than_the_node_record_holds(CostEngine, rank, n_args):
     _check_build(CostEngine, g, False)
 
 
+@pytest.mark.parametrize("mode", ["full", "compressed"])
+def test_problem_without_the_derived_records(CostEngine, mode):
+    """A caller of the C ABI may leave out every record the host derives for the
+    prepare launch (table units, spec records, product terms, node records): the
+    kernels then walk the arrays those were made from.  Same bits either way."""
+    g = graphgen.llama_graph((2, 2, 4), 1, 64, 4, 2, 128, 256, 32, 16)
+    eng = CostEngine(g, table_mode=mode).build(clamp_inf=False)
+    want = eng.results()
+    ref = O.GraphOracle(g).build()
+    assert bits_equal(want["comm"], ref["comm"]) and bits_equal(want["compute"], ref["compute"])
+    for drop in (("table_units",), ("spec_recs",), ("prog_terms", "n_prog_term"),
+                 ("comp_recs",), ("table_units", "spec_recs", "prog_terms", "n_prog_term", "comp_recs")):
+        e2 = CostEngine(g, table_mode=mode)
+        for f in drop:
+            setattr(e2.problem, f, 0 if f == "n_prog_term" else None)
+        got = e2.build(clamp_inf=False).results()
+        for k in ("comm", "cost", "compute", "per_arg"):
+            assert bits_equal(got[k], want[k]), (drop, k, first_mismatch(got[k], want[k]))
+        assert (got["flags"] == want["flags"]).all()
+
+
+def test_node_program_paths(CostEngine):
+    """The node estimate by product terms, by the interpreter (a term over more
+    factors than a term record names), with an argument whose strategies see
+    different tensors (the record's meta hint then misses), a missing spec and a
+    broadcast output, all in one graph."""
+    b = GraphBuilder((2, 4), 8)
+    big = (4,) * 8
+    m8 = b.meta(big, graphgen.contiguous_stride(big), 2, packed.DT_BF16)
+    ma = b.meta((64, 48), (48, 1), 2, packed.DT_BF16)
+    mb = b.meta((64, 1), (1, 1), 4, packed.DT_F32)
+    mc = b.meta((32, 48), (48, 1), 2, packed.DT_BF16)
+    o8 = [b.spec(m8, o) for o in O.create_all_options(big, (2, 4))[:12]]
+    oa = [b.spec(ma, o) for o in O.create_all_options((64, 48), (2, 4))]
+    ob = [b.spec(mb, o) for o in O.create_all_options((64, 1), (2, 4))]
+    oc = [b.spec(mc, o) for o in O.create_all_options((32, 48), (2, 4))]
+    x8 = b.add_node(NodeDesc("x8", [[s] for s in o8], [[s] for s in o8], inputs=[], default_rows=[[[0.0]] for _ in o8]))
+    xa = b.add_node(NodeDesc("xa", [[s] for s in oa], [[s] for s in oa], inputs=[], default_rows=[[[0.0]] for _ in oa]))
+    xb = b.add_node(NodeDesc("xb", [[s] for s in ob], [[s] for s in ob], inputs=[], default_rows=[[[0.0]] for _ in ob]))
+    # eight factors in one term: interpreted word by word
+    prog8 = opprog.program([(2, [(0, d) for d in range(8)])], [(2, [opprog.argnumel(0)])])
+    b.add_node(NodeDesc("eight", [[s] for s in o8], [[s] for s in o8], inputs=[x8], op=packed.OP_PROGRAM, program=prog8))
+    # broadcast add of [64, 48] and [64, 1]; argument 0 sees tensor ma or mc by strategy
+    mixed = [[(oa + oc)[k % (len(oa) + len(oc))], ob[k % len(ob)], -1] for k in range(70)]
+    rows = [[[0.0] * len(oa), [0.0] * len(ob), [0.0]] for _ in range(70)]
+    b.add_node(NodeDesc("bcast_add", mixed, [[r[0]] for r in mixed], inputs=[xa, xb, None], op=packed.OP_PROGRAM,
+                        program=opprog.pointwise(2, 2), default_rows=rows, nargs=3))
+    g = b.pack()
+    rec = g.comp_records()
+    by_node = {int(r["node"]): r for r in rec}
+    assert by_node[3]["n_term"] == 0 and by_node[4]["n_term"] > 0 and by_node[4]["term_flags"] & 1
+    for mode in (True, False, "compressed"):
+        _check_build(CostEngine, g, mode)
+
+
 def test_unsupported_dtype_reports(CostEngine):
     b = GraphBuilder((2,), 8)
     m = b.meta((8, 8), (8, 1), 8, packed.DT_OTHER)

@@ -1,0 +1,149 @@
+"""The records the host derives from a packed problem for the prepare launch
+(product terms of compute programs, per-position spec records, table units):
+each against the definition it stands for, on the CPU."""
+import math
+
+import numpy as np
+import pytest
+
+from autoparallel_amd import graphgen, packed
+from autoparallel_amd.packed import DT_BF16, DT_F32, GraphBuilder, NodeDesc
+from oracle import cost_oracle as O
+
+GRAPHS = {
+    "llama": lambda: graphgen.llama_graph((8, 8), 1, 1024, 8, 4, 2048, 8192, 512, 16),
+    "llama_3d": lambda: graphgen.llama_graph((2, 2, 4), 1, 64, 4, 2, 128, 256, 32, 16),
+    "moe": lambda: graphgen.moe_graph((2, 4), 2, 64, 4, 8, 2, 32, 256, 32, 8),
+    "stress": lambda: graphgen.stress_graph(60, (4, 8, 8), seed=2, s_max=40),
+}
+
+
+@pytest.mark.parametrize("name", list(GRAPHS))
+def test_program_terms_equal_the_interpreter(name):
+    """flops and bytes from the product terms, evaluated on the rows of the
+    value table the kernel builds, equal run_program on the same local shapes."""
+    g = GRAPHS[name]()
+    orc = O.GraphOracle(g)
+    terms, where = g.program_terms()
+    recs = g.comp_records()
+    R, slots = g.max_rank, g.max_rank + 2
+    checked = 0
+    for rec in recs:
+        if rec["n_term"] == 0:
+            continue
+        v = int(rec["node"])
+        e0, e1 = int(g.node_edge_off[v]), int(g.node_edge_off[v + 1])
+        po = int(g.node_prog_off[v])
+        prog = [int(x) for x in g.prog[po:po + int(g.node_prog_len[v])]]
+        for o in range(0, int(g.node_nstrat[v]), max(1, int(g.node_nstrat[v]) // 7)):
+            words = [int(g.lists[int(g.edge_dst_list[e]) + o]) for e in range(e0, e1)]
+            shapes, isz, rows = [], [], {}
+            for a, w in enumerate(words):
+                if w == packed.SPEC_NONE:
+                    shapes.append(None)
+                    isz.append(0)
+                    local = []
+                else:
+                    m = w >> packed.TUPLE_BITS
+                    r = int(g.meta_rank[m])
+                    local, _ = O.sharded_shape_stride(
+                        [int(x) for x in g.meta_shape[m, :r]], [int(x) for x in g.meta_stride[m, :r]],
+                        [int(x) for x in g.tuple_plc[w & 0xFFF, :g.ndim]], [int(x) for x in g.mesh_shape])
+                    shapes.append(list(local))
+                    isz.append(int(g.meta_itemsize[m]))
+                for d in range(R):
+                    rows[R + a * slots + d] = local[d] if d < len(local) else 1
+                rows[R + a * slots + R + 1] = math.prod(local)
+            for pos in range(R):  # broadcast rows
+                size = 1
+                for shp in shapes:
+                    if shp is None or pos >= len(shp):
+                        continue
+                    if shp[len(shp) - 1 - pos] != 1:
+                        size = shp[len(shp) - 1 - pos]
+                rows[pos] = size
+            flops = nbytes = 0
+            for t in terms[int(rec["term_off"]):int(rec["term_off"]) + int(rec["n_term"])]:
+                val = int(t["coeff"])
+                for i in t["idx"]:
+                    if i != 0xFF:
+                        val *= rows[int(i)]
+                if t["to_bytes"]:
+                    nbytes += val
+                else:
+                    flops += val
+            nbytes += sum(math.prod(s) * z for s, z in zip(shapes, isz) if s is not None)
+            assert (flops, nbytes) == O.run_program(prog, shapes, isz), (name, v, o)
+            checked += 1
+    assert checked > 0
+    # every program has the term form on these graphs
+    prog_nodes = g.comp_nodes[g.node_op[g.comp_nodes] == packed.OP_PROGRAM]
+    assert (recs["n_term"][g.node_op[g.comp_nodes] == packed.OP_PROGRAM] > 0).all(), len(prog_nodes)
+
+
+def test_program_without_term_form_keeps_the_interpreter():
+    b = GraphBuilder((2, 2))
+    m = b.meta((4,) * 8, tuple(4 ** (7 - i) for i in range(8)), 2, DT_BF16)
+    s = b.spec(m, (0, 0))
+    b.add_node(NodeDesc("x", [[s]], [[s]], inputs=[], default_rows=[[[0.0]]]))
+    # a term over eight factors: more than a 16-byte term record names
+    prog = [1, 0, 2, 8] + [v for d in range(8) for v in (0, d)]
+    b.add_node(NodeDesc("y", [[s]], [[s]], inputs=[0], op=packed.OP_PROGRAM, program=prog))
+    g = b.pack()
+    rec = g.comp_records()
+    y = rec[rec["node"] == 1][0]
+    assert y["n_term"] == 0 and g.program_terms()[0].shape[0] == 0
+
+
+def test_spec_records():
+    b = GraphBuilder((2, 4))
+    metas = [
+        b.meta((8, 16, 4), (64, 4, 1), 4, DT_F32),  # contiguous
+        b.meta((8, 16, 4), (4, 32, 1), 2, DT_BF16),  # transposed
+        b.meta((8, 1, 4), (4, 999, 1), 4, DT_F32),  # size-1 dim: its stride does not count
+        b.meta((), (), 8, packed.DT_F64),  # scalar
+        b.meta((5, 0, 3), (3, 3, 1), 4, DT_F32),  # no elements
+    ]
+    specs = [b.spec(m, plc) for m in metas for plc in ((0, 0), (packed.PARTIAL_SUM, 0))]
+    b.add_node(NodeDesc("p", [[s] for s in specs], [[s] for s in specs], inputs=[],
+                        default_rows=[[[0.0]] for _ in specs]))
+    b.add_node(NodeDesc("c", [[specs[0], -1]], [[specs[0]]], inputs=[0, None],
+                        default_rows=[[[0.0] * len(specs), [0.0]]]))
+    g = b.pack()
+    rec = g.spec_records()
+    assert rec.shape[0] == g.lists.shape[0] and (rec["word"] == g.lists).all()
+    assert (g.lists == packed.SPEC_NONE).any()
+    for k, w in enumerate(g.lists):
+        if w == packed.SPEC_NONE:
+            assert rec["plc"][k] == 0 and rec["nbytes2"][k] == 0
+            continue
+        m, t = int(w) >> packed.TUPLE_BITS, int(w) & 0xFFF
+        r = int(g.meta_rank[m])
+        shape, stride = [int(x) for x in g.meta_shape[m, :r]], [int(x) for x in g.meta_stride[m, :r]]
+        assert int(rec["plc"][k]) == int.from_bytes(bytes(g.tuple_plc[t]), "little")
+        assert int(rec["nbytes2"][k]) >> 1 == int(g.meta_itemsize[m]) * math.prod(shape)
+        assert bool(int(rec["nbytes2"][k]) & 1) == O.check_contiguous(shape, stride)
+    contig = {int(w) >> packed.TUPLE_BITS: bool(int(n) & 1) for w, n in zip(g.lists, rec["nbytes2"]) if w != packed.SPEC_NONE}
+    assert contig == {0: True, 1: False, 2: True, 3: True, 4: True}
+
+
+@pytest.mark.parametrize("name", list(GRAPHS))
+@pytest.mark.parametrize("compressed", [False, True])
+def test_table_units_tile_every_matrix(name, compressed):
+    g = GRAPHS[name]()
+    block_edge, block_off, unit_block, _, edge_usrc, block_udst = g.block_table(compressed)
+    units = g.table_unit_records(compressed)
+    assert units.shape[0] == unit_block.shape[0] == block_off[-1] // 256
+    for b in range(block_edge.shape[0]):
+        e = int(block_edge[b])
+        mine = units[unit_block == b]
+        squeezed = compressed and edge_usrc[e] > 0
+        ncol = int(edge_usrc[e]) if squeezed else int(g.edge_ssrc[e])
+        nrow = int(block_udst[b]) if squeezed else int(g.edge_sdst[e])
+        assert (mine["ncol"] == ncol).all() and (mine["nrow"] == nrow).all()
+        assert (mine["src_list"] == g.edge_src_list[e]).all() and (mine["dst_list"] == g.edge_dst_list[e]).all()
+        assert (mine["default_off"] == g.edge_default_off[e]).all()
+        assert (mine["flags"] == (packed.EDGE_COMPRESSED if squeezed else 0)).all()
+        # the units of a matrix start every 256 elements and reach past its last one
+        assert (mine["first"] == np.arange(mine.shape[0]) * 256).all()
+        assert mine.shape[0] * 256 >= ncol * nrow > (mine.shape[0] - 1) * 256
