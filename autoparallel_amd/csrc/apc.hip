@@ -647,17 +647,33 @@ static_assert(64 * kPerLane == APC_ITEM_ENTRIES, "work items are built for this 
 // specs, default rows).
 __device__ __forceinline__ void eval_entry(const apc_problem& p, const apc_edge& ed, uint32_t o,
                                            uint32_t j, double& comm, int& trans) {
-  const uint32_t tw = p.lists[(size_t)ed.dst_list + o];
-  const uint32_t sw =
-      (ed.flags & APC_EDGE_HAS_PRODUCER) ? p.lists[(size_t)ed.src_list + j] : APC_SPEC_NONE;
+  const bool has_producer = (ed.flags & APC_EDGE_HAS_PRODUCER) != 0;  // wave-uniform
+  uint32_t sw = APC_SPEC_NONE, tw, src_plc = 0, tgt_plc = 0;
+  int64_t nbytes = 0;
+  bool contig = true;
+  if (p.spec_recs) {  // one record per side
+    const apc_spec_rec rt = p.spec_recs[(size_t)ed.dst_list + o];
+    tw = rt.word;
+    tgt_plc = rt.plc;
+    if (has_producer) {
+      const apc_spec_rec rs = p.spec_recs[(size_t)ed.src_list + j];
+      sw = rs.word;
+      src_plc = rs.plc;
+      nbytes = rs.nbytes2 >> 1;
+      contig = (rs.nbytes2 & 1) != 0;
+    }
+  } else {
+    tw = p.lists[(size_t)ed.dst_list + o];
+    if (has_producer) sw = p.lists[(size_t)ed.src_list + j];
+    if (sw != APC_SPEC_NONE && tw != APC_SPEC_NONE) {
+      src_plc = load_tuple(p.tuple_plc, sw & kTupleMask);
+      tgt_plc = load_tuple(p.tuple_plc, tw & kTupleMask);
+      meta_bytes_contig(p, sw >> APC_TUPLE_BITS, nbytes, contig);
+    }
+  }
   if (sw != APC_SPEC_NONE && tw != APC_SPEC_NONE) {
-    const uint32_t st = sw & kTupleMask, tt = tw & kTupleMask, sm = sw >> APC_TUPLE_BITS;
-    trans = (st != tt);
-    int64_t nbytes;
-    bool contig;
-    meta_bytes_contig(p, sm, nbytes, contig);
-    comm = redistribute_cost(load_tuple(p.tuple_plc, st), load_tuple(p.tuple_plc, tt), nbytes,
-                             contig, p.model);
+    trans = ((sw & kTupleMask) != (tw & kTupleMask));
+    comm = redistribute_cost(src_plc, tgt_plc, nbytes, contig, p.model);
   } else {
     comm = p.default_vals[ed.default_off + (int64_t)o * ed.ssrc + j];
     trans = 0;

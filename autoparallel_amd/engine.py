@@ -257,12 +257,16 @@ class CostEngine:
             torch.empty(tsize, dtype=torch.float64, device=self.device) if self.use_table else None
         )
         self.built = False
+        self._build_args = None
         # interleaved copy of the entry arrays for scoring (apc_score_rec), made on
         # first use when the edge blocks are large; stale after anything rewrites
         # the entry arrays
         self.packed_scoring = g.num_edges > 0 and g.num_entries / g.num_edges >= _PACKED_SCORING_FROM
         self._recs: Optional[torch.Tensor] = None
         self._recs_valid = False
+
+    def synchronize(self) -> None:
+        torch.cuda.synchronize(self.device)
 
     # -- raw stream -----------------------------------------------------------
     def _stream(self):
@@ -319,32 +323,36 @@ class CostEngine:
             "apc_prepare",
         )
 
+    def build_args(self):
+        if self._build_args is None:
+            self._build_args = (
+                C.byref(self.problem), self._ptr(self.table), self._ptr(self.compute), self._ptr(self.per_arg),
+                self._ptr(self.status), self._ptr(self.comm), self._ptr(self.cost), self._ptr(self.flags))
+        return self._build_args
+
     def build(self, clamp_inf: bool = True):
         """All coefficients: pair table and node compute vectors (one launch),
         then the entry arrays (one launch)."""
         self._recs_valid = False
-        _lib.check(
-            self.lib.apc_build_all(
-                C.byref(self.problem), self._ptr(self.table), self._ptr(self.compute),
-                self._ptr(self.per_arg), self._ptr(self.status), self._ptr(self.comm),
-                self._ptr(self.cost), self._ptr(self.flags), int(bool(clamp_inf)), self._stream()),
-            "apc_build_all",
-        )
+        # the argument list is the same from call to call apart from the stream:
+        # made once, so that issuing a step costs less host time than the step takes
+        args = self._build_args or self.build_args()
+        rc = self.lib.apc_build_all(*args, 1 if clamp_inf else 0,
+                                    torch.cuda.current_stream(self.device).cuda_stream)
+        if rc:
+            _lib.check(rc, "apc_build_all")
         self.built = True
         return self
 
     def build_timed(self, timer, slot: int, clamp_inf: bool = True):
         """build() with HIP events at the begin and end of the entry kernel (a
         timer from apc_timer_create); the launches are otherwise identical."""
+        self.build_args()
+        rc = self.lib.apc_build_all_timed(*self._build_args, 1 if clamp_inf else 0, timer, int(slot),
+                                          torch.cuda.current_stream(self.device).cuda_stream)
+        if rc:
+            _lib.check(rc, "apc_build_all_timed")
         self._recs_valid = False
-        _lib.check(
-            self.lib.apc_build_all_timed(
-                C.byref(self.problem), self._ptr(self.table), self._ptr(self.compute),
-                self._ptr(self.per_arg), self._ptr(self.status), self._ptr(self.comm),
-                self._ptr(self.cost), self._ptr(self.flags), int(bool(clamp_inf)), timer, int(slot),
-                self._stream()),
-            "apc_build_all_timed",
-        )
         self.built = True
         return self
 

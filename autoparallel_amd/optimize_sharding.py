@@ -14,6 +14,7 @@ from __future__ import annotations
 
 import collections.abc
 import logging
+import time
 import operator
 from typing import Any, Dict, Iterator, List, Optional, Tuple
 
@@ -248,11 +249,19 @@ class ShardingOptimizer:
         self._device_name = device_name or detect_device_name()
         _cre.configure(self._devices_per_host, self._device_name)
         self._constraint_log: List[Tuple[str, dict]] = []
+        # seconds per phase, the split the reference logs at DEBUG
+        # (autoparallel/optimize_sharding.py:249-291, 579-587)
+        self.phase_s: Dict[str, float] = {}
+        t0 = time.perf_counter()
         self.strats = self.build_sharding_metadata()
+        self.phase_s["strategy_enumeration"] = time.perf_counter() - t0
         self.nodes = list(self.strats.keys())
         self.node_map = {n: i for i, n in enumerate(self.nodes)}
         self.decision_vars = self._build_decision_vars()
+        t0 = time.perf_counter()
         self.validate()
+        self.phase_s["validate"] = time.perf_counter() - t0
+        logger.debug("ShardingOptimizer phases (s): %s", self.phase_s)
 
     # -- accessors of the reference's class ----------------------------------------
     @property
@@ -444,7 +453,9 @@ class ShardingOptimizer:
 
     # -- coefficients ----------------------------------------------------------------
     def _build_decision_vars(self) -> DecisionVars:
+        t0 = time.perf_counter()
         self._packed = self._pack()
+        self.phase_s["pack"] = time.perf_counter() - t0
         self._core = PackedShardingOptimizer(
             self._packed, roles=self._packed.roles,
             force_grad_reduce_in_higher_precision=self.force_grad_reduce_in_higher_precision,
@@ -457,7 +468,10 @@ class ShardingOptimizer:
                 self.cluster_links[(v, argi, out_idx, inp_idx)] = (r, argi, out_idx, inp_idx)
         self._cluster_linked_node_idxs = {k[0] for k in self.cluster_links}
         self.prob = self._core.prob
+        self.phase_s.update(self._core.phase_s)
+        t0 = time.perf_counter()
         self._write_back_redistribute_costs()
+        self.phase_s["write_back_redistribute_cost"] = time.perf_counter() - t0
         return DecisionVars(self)
 
     def _write_back_redistribute_costs(self) -> None:

@@ -21,6 +21,7 @@ from __future__ import annotations
 import dataclasses
 import logging
 import math
+import time
 from typing import Dict, Iterable, List, Optional, Sequence, Set, Tuple
 
 import numpy as np
@@ -113,14 +114,21 @@ class PackedShardingOptimizer:
         self.roles = roles or getattr(g, "roles", None) or GraphRoles()
         self.force_grad_reduce_in_higher_precision = force_grad_reduce_in_higher_precision
         self.engine = None
+        self.phase_s: Dict[str, float] = {}  # seconds per phase of the construction
         if coefficients is None:
             from .engine import CostEngine  # the HIP path; raises without the library / a GPU
 
+            t0 = time.perf_counter()
             self.engine = CostEngine(g, device=device, device_name=device_name, nccl_config=nccl_config)
+            t1 = time.perf_counter()
             self.engine.build(clamp_inf=True)
+            self.engine.synchronize()
+            t2 = time.perf_counter()
             coefficients = Coefficients.from_engine(self.engine)
+            self.phase_s.update(engine_construct=t1 - t0, device_build=t2 - t1, readback=time.perf_counter() - t2)
         self.coef = coefficients
         self.region_groups: List[List[List[int]]] = []
+        t0 = time.perf_counter()
         if cluster_root is None and repeated_subgraphs:
             from . import clustering
 
@@ -128,6 +136,8 @@ class PackedShardingOptimizer:
             self.region_groups = clustering.identical_regions(g, hashes)
             cluster_root = clustering.cluster_roots(g, self.region_groups)
         self._set_cluster_root(cluster_root)
+        self.phase_s["clustering"] = time.perf_counter() - t0
+        t0 = time.perf_counter()
         sizes = g.edge_sdst.astype(np.int64) * g.edge_ssrc
         self.var_start = np.concatenate([[0], np.cumsum(sizes)]).astype(np.int64)
         self.n_vars = int(self.var_start[-1])
@@ -142,6 +152,7 @@ class PackedShardingOptimizer:
         self.mesh_dim_names: Optional[List[str]] = None
         self.selected: Optional[np.ndarray] = None
         self.add_default_constraints()
+        self.phase_s["ilp_rows"] = time.perf_counter() - t0
 
     # -- clusters ---------------------------------------------------------------
     def _set_cluster_root(self, root: Optional[np.ndarray]) -> None:

@@ -3,13 +3,20 @@
 A step is one build of every ILP coefficient of the workload graph, with the
 packed problem already resident in HBM: pair table, node compute vectors, and
 the entry kernel that writes comm / cost / flags for all E decision variables.
+``value`` is that resident rebuild (``value_is``); ``end_to_end`` is the same
+work from the packed problem on the host to the coefficients back on the host
+(engine construction with its descriptor upload, one build, read-back), and
+``cpu_baseline`` the per-entry Python oracle on this box's host, which pays its
+memoisation inside its timed region as the reference does.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
 
-Prints one JSON line (see the keys below).  ``roofline`` is for the dominant
+Prints one JSON line (see the keys below).  A step issues the two launches
+(``--launch graph`` replays a HIP graph of them instead: measured slower on
+this stack, 29.8 us against 25.8 us per step); ``roofline`` is for the dominant
 kernel (edge_cost_kernel), timed with HIP events on the launch stream inside the
-timed steps (on a sample of them: every 4th step of a short region, 25 steps of a
-long one); ``cpu_baseline`` is the per-entry Python oracle on this box's host.
+timed steps (on a sample of them, launched with the event pair attached to the
+kernel's dispatch: every 6th step of a short region, 25 steps of a long one).
 """
 import argparse
 import json
@@ -65,6 +72,8 @@ def main():
     ap.add_argument("--fx-layers", type=int, default=32,
                     help="also plan the traced transformers Llama-3-8B with this many layers through "
                          "ShardingOptimizer and report its host time (0 = skip)")
+    ap.add_argument("--launch", choices=["graph", "eager"], default="eager",
+                    help="how a step is issued: replay of a HIP graph of its launches, or the launches themselves")
     ap.add_argument("--direct", action="store_true", help="evaluate every entry directly (no block table)")
     ap.add_argument("--table-mode", choices=["full", "compressed", "direct"], default=None,
                     help="force the block-table layout (default: chosen from the table sizes)")
@@ -90,11 +99,52 @@ def main():
     t0 = time.perf_counter()
     eng = CostEngine(g, table_mode="direct" if args.direct else args.table_mode)
     torch.cuda.synchronize()
-    t_upload = time.perf_counter() - t0
+    t_first_engine = time.perf_counter() - t0  # includes the creation of the HIP context
+
+    # End to end, on a warm process: a second engine from the packed problem on the
+    # host (layout records, descriptor upload), one build, and the five result
+    # arrays copied into pinned host memory (allocated before the clock starts).
+    pinned = {k: torch.empty(t.shape, dtype=t.dtype, pin_memory=True)
+              for k, t in (("comm", eng.comm), ("cost", eng.cost), ("flags", eng.flags),
+                           ("compute", eng.compute), ("per_arg", eng.per_arg))}
+    e2e = {"engine_construct": [], "build": [], "readback": []}
+    for _ in range(3):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        eng2 = CostEngine(g, table_mode=eng.table_mode)
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        eng2.build(clamp_inf=True)
+        torch.cuda.synchronize()
+        t2 = time.perf_counter()
+        for k, dst in pinned.items():
+            dst.copy_(getattr(eng2, k), non_blocking=True)
+        torch.cuda.synchronize()
+        t3 = time.perf_counter()
+        e2e["engine_construct"].append(t1 - t0)
+        e2e["build"].append(t2 - t1)
+        e2e["readback"].append(t3 - t2)
+        del eng2
+    e2e = {k: min(v) for k, v in e2e.items()}
+    t_e2e = sum(e2e.values())
+
+    # before the timed region: the prepare kernel bracketed the same way, for the report
+    pe = [[torch.cuda.Event(enable_timing=True) for _ in range(2)] for _ in range(20)]
+    for a, b in pe:
+        a.record()
+        eng.prepare()
+        b.record()
+        eng.edge_costs(clamp_inf=True)
+    torch.cuda.synchronize()
 
     for _ in range(args.warmup):
         eng.build()
     torch.cuda.synchronize()
+    graph = eng.capture_build(clamp_inf=True) if args.launch == "graph" else None
+    if graph is not None:
+        for _ in range(3):
+            graph.replay()
+        torch.cuda.synchronize()
 
     # HIP events on the launch stream (torch's current stream is the one the
     # engine launches on), recorded at the begin and end of the dominant kernel
@@ -103,19 +153,22 @@ def main():
     import ctypes as C
 
     # The event pair costs about 30 us of host time per launch on this stack, more
-    # than the whole step: on every launch it would make the loop host-bound (the
-    # step then reads 40 us, of which the GPU is busy 28).  So a sample of the
-    # timed region's launches carries events: every `stride`-th step (every 4th
-    # of a short region, 25 of a long one).
-    stride = max(4, args.steps // 25) if args.steps >= 4 else 1
+    # than the whole step: on every launch it would make the loop host-bound.  So
+    # a sample of the timed region's steps carries events: every `stride`-th step
+    # (every 6th of a short region, 25 of a long one).
+    stride = max(6, args.steps // 25) if args.steps >= 6 else 1
     n_timed = (args.steps + stride - 1) // stride
     timer = C.c_void_p()
     assert eng.lib.apc_timer_create(n_timed, C.byref(timer)) == 0
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for k in range(args.steps):
-        if k % stride == 0:
+        # the sampled step is the last of its group, when the queue holds the steps
+        # issued ahead and the event pair's host time is hidden behind them
+        if k % stride == stride - 1 or (k == args.steps - 1 and k // stride == n_timed - 1 and k % stride != stride - 1):
             eng.build_timed(timer, k // stride, clamp_inf=True)
+        elif graph is not None:
+            graph.replay()
         else:
             eng.build(clamp_inf=True)
     torch.cuda.synchronize()
@@ -128,15 +181,6 @@ def main():
         t_edge += ms.value
     t_edge = t_edge / n_timed * 1e-3
     eng.lib.apc_timer_destroy(timer)
-
-    # outside the timed region: the prepare kernel bracketed the same way, for the report
-    pe = [[torch.cuda.Event(enable_timing=True) for _ in range(2)] for _ in range(20)]
-    for a, b in pe:
-        a.record()
-        eng.prepare()
-        b.record()
-        eng.edge_costs(clamp_inf=True)
-    torch.cuda.synchronize()
 
     if args.calibration_copy_mib > 0:
         nbytes = args.calibration_copy_mib << 20
@@ -160,6 +204,9 @@ def main():
     out = {
         "metric": "cost entries/sec (all ILP coefficients of the graph built per step)",
         "value": E / (elapsed / args.steps),
+        "value_is": "resident_rebuild: packed problem, block-table layout and work items already in HBM; "
+                    "see end_to_end for the figure from host arrays to host arrays",
+        "launch": args.launch,
         "unit": "entries/s",
         "n_gpus": 1,
         "steps": args.steps,
@@ -189,7 +236,15 @@ def main():
         },
         "coefficient_build_wall_s": elapsed / args.steps,
         "kernel_s": {"prepare(pair_table+node_compute)": t_prep, "edge_cost": t_edge},
-        "host_s": {"graph_generation_and_pack": t_gen, "upload": t_upload},
+        "host_s": {"graph_generation_and_pack": t_gen, "first_engine_with_hip_context": t_first_engine,
+                   "engine_construct": e2e["engine_construct"], "single_build_synchronised": e2e["build"],
+                   "readback_to_pinned_host": e2e["readback"]},
+        "end_to_end": {
+            "what": "CostEngine(packed problem on the host) + one build + copy of comm, cost, flags, compute, "
+                    "per_arg to pinned host memory; best of 3 on a warm process",
+            "seconds": t_e2e,
+            "entries_per_s": E / t_e2e,
+        },
         "roofline": {
             "kernel": "edge_cost_kernel",
             "bound": "hbm",
@@ -198,9 +253,18 @@ def main():
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBS,
             "algorithmic_bytes_per_launch": algo_bytes,
+            "bytes_per_entry": 17,
             "avg_launch_s": t_edge,
             "timed_launches": n_timed,
+            # the same bytes over the whole step (prepare launch included), and both
+            # with 8 B per entry (the cost alone) instead of the 17 B this build writes
+            "step_frac": algo_bytes / (elapsed / args.steps) / 1e9 / HBM_PEAK_GBS,
+            "frac_at_8B": (8 * E + desc_bytes) / t_edge / 1e9 / HBM_PEAK_GBS,
+            "step_frac_at_8B": (8 * E + desc_bytes) / (elapsed / args.steps) / 1e9 / HBM_PEAK_GBS,
             "traffic": read_traffic(args.workload),
+            "traffic_source": "profiles/edge_cost_kernel_%s_traffic.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE "
+                              "runs of this command, scaled by the copy kernel; not a quantity of this run)"
+                              % args.workload,
         },
     }
 
@@ -220,7 +284,9 @@ def main():
             "assignments_per_s": n / t_score,
             "edge_terms_per_s": n * g.num_edges / t_score,
             "algorithmic_bytes_per_assignment": 8 * g.num_nodes + 17 * g.num_edges,
-            "feasible_fraction": float((scores[:, 5] == 0).double().mean().item()),
+            "assignments_are": "independent uniform draws of one strategy per node (flow-consistent by "
+                               "construction: each edge's inp_idx is its producer's draw), not ILP-feasible plans",
+            "fraction_without_forbidden_entry": float((scores[:, 5] == 0).double().mean().item()),
         }
 
     if args.schedules > 0:
@@ -281,6 +347,7 @@ def main():
             "seconds": t_cpu,
         }
         out["speedup_vs_cpu_baseline"] = out["value"] / out["cpu_baseline"]["value"]
+        out["speedup_vs_cpu_baseline_end_to_end"] = out["end_to_end"]["entries_per_s"] / out["cpu_baseline"]["value"]
         # also reported, and not the reference: the compiled (C, no memo cache)
         # restatement on the same graph, one thread and all cores of the box's share
         try:
@@ -303,13 +370,13 @@ def main():
         # the traced joint graph to coefficients and ILP rows (strategy sets of the
         # installed torch, so fewer entries than the generator's graph above)
         try:
-            out["fx_path"] = _fx_path_figure(args.fx_layers)
+            out["fx_path"] = _fx_path_figure(args.fx_layers, not args.no_cpu_baseline)
         except Exception as exc:  # transformers or the fake process group unavailable
             out["fx_path"] = {"error": f"{type(exc).__name__}: {exc}"[:300]}
     print(json.dumps(out))
 
 
-def _fx_path_figure(n_layers: int) -> dict:
+def _fx_path_figure(n_layers: int, cpu_port: bool) -> dict:
     import contextlib
 
     import torch
@@ -367,14 +434,36 @@ def _fx_path_figure(n_layers: int) -> dict:
         opt = ShardingOptimizer(gm, mesh, devices_per_host=8, device_name="AMD Instinct MI355X")
         t_opt = time.perf_counter() - t0
         g = opt._packed
-        return {
+        res = {
             "workload": f"transformers LlamaForCausalLM, Llama-3-8B dimensions, {n_layers} layers, bf16, "
                         f"batch 64 x 8192, joint graph, mesh (8,8)",
             "nodes": g.num_nodes, "edges": g.num_edges, "entries": g.num_entries,
             "trace_s": t_trace, "sharding_optimizer_s": t_opt,
+            # the split the reference logs for the same constructor
+            # (autoparallel/optimize_sharding.py:249-291, 579-587)
+            "phase_s": {k: round(v, 6) for k, v in opt.phase_s.items()},
+            "entries_per_s_through_the_api": g.num_entries / t_opt,
             "strategy_queries": dict(PO.strategy_cache_stats), "replicate_stand_ins": len(PO.fallback_nodes),
             "ilp_rows": len(opt.prob.constraints),
         }
+        if cpu_port:
+            # the per-entry Python port on this same packed problem: what the reference's
+            # _build_decision_vars loop costs after strategy enumeration
+            from oracle import cost_oracle as O
+
+            orc = O.GraphOracle(g)
+            orc.reset_caches()
+            t0 = time.perf_counter()
+            orc.build()
+            t_cpu = time.perf_counter() - t0
+            coeff_s = sum(opt.phase_s.get(k, 0.0) for k in ("pack", "engine_construct", "device_build", "readback"))
+            res["cpu_baseline"] = {
+                "kind": "port", "cores": 1, "seconds": t_cpu, "entries_per_s": g.num_entries / t_cpu,
+                "what": "oracle.cost_oracle.GraphOracle(opt._packed).build(), memo caches cleared first",
+                "coefficient_phases_s": coeff_s,
+                "speedup_of_coefficient_phases": t_cpu / coeff_s if coeff_s > 0 else None,
+            }
+        return res
     finally:
         if own:
             dist.destroy_process_group()
