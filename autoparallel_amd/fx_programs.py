@@ -131,37 +131,46 @@ def local_shapes(specs: Sequence) -> List[Tuple[List[int], List[int]]]:
     return [([int(x) for x in osh[i, : rank[i]]], [int(x) for x in ost[i, : rank[i]]]) for i in range(n)]
 
 
-def _flops_bytes_via_torch(node, strategies) -> Tuple[List[int], List[int]]:
+def _flops_bytes_via_torch(node, strategies, shapes_fn=None) -> Tuple[List[int], List[int]]:
     """The reference's own route for ops without a closed form: run the op on
-    meta tensors of the sharded sizes under FlopCounterMode (torch code)."""
+    meta tensors of the sharded sizes under FlopCounterMode (torch code).
+    ``shapes_fn``: what turns a list of DTensorSpecs into their local (shape,
+    stride) pairs; the device's batch form of _get_sharded_shape_stride unless a
+    caller brings its own."""
     from torch.utils.flop_counter import FlopCounterMode
 
+    from torch._subclasses.fake_tensor import FakeTensorMode
+
     flat_specs = [s for st in strategies for s in st.input_specs if s is not None]
-    shapes = iter(local_shapes(flat_specs))
+    shapes = iter((shapes_fn or local_shapes)(flat_specs))
     flops_all, bytes_all = [], []
     flat_args, treespec = tree_flatten(node.args)
     kwargs = {k: (v.meta["val"] if isinstance(v, torch.fx.Node) else v) for k, v in node.kwargs.items()}
-    for st in strategies:
-        new_flat, counter = [], 0
-        for a in flat_args:
-            if isinstance(a, torch.fx.Node):
-                a = a.meta["val"]
-                if isinstance(a, torch.Tensor):
-                    spec = st.input_specs[counter]
-                    counter += 1
-                    if spec is not None:
-                        sizes, strides = next(shapes)
-                        a = torch.empty_strided(sizes, strides, dtype=a.dtype, device="meta")
-                    else:
-                        a = torch.empty_strided(a.shape, a.stride(), dtype=a.dtype, device="meta")
-            new_flat.append(a)
-        args = treespec.unflatten(new_flat)
-        with FlopCounterMode(display=False) as fc:
-            out = node.target(*args, **kwargs)
-        nbytes = sum(x.numel() * x.element_size() for x in tree_flatten(args)[0] if isinstance(x, torch.Tensor))
-        nbytes += sum(x.numel() * x.element_size() for x in tree_flatten(out)[0] if isinstance(x, torch.Tensor))
-        flops_all.append(int(fc.get_total_flops()))
-        bytes_all.append(int(nbytes))
+    # Fake tensors on the traced tensors' own device, as the reference runs the
+    # operator (compute_estimation.py:334-365): an operator that names a device in
+    # its arguments (_to_copy) cannot run on meta tensors.
+    with FakeTensorMode(allow_non_fake_inputs=True):
+        for st in strategies:
+            new_flat, counter = [], 0
+            for a in flat_args:
+                if isinstance(a, torch.fx.Node):
+                    a = a.meta["val"]
+                    if isinstance(a, torch.Tensor):
+                        spec = st.input_specs[counter]
+                        counter += 1
+                        if spec is not None:
+                            sizes, strides = next(shapes)
+                        else:
+                            sizes, strides = a.shape, a.stride()
+                        a = torch.empty_strided(sizes, strides, dtype=a.dtype, device=a.device)
+                new_flat.append(a)
+            args = treespec.unflatten(new_flat)
+            with FlopCounterMode(display=False) as fc:
+                out = node.target(*args, **kwargs)
+            nbytes = sum(x.numel() * x.element_size() for x in tree_flatten(args)[0] if isinstance(x, torch.Tensor))
+            nbytes += sum(x.numel() * x.element_size() for x in tree_flatten(out)[0] if isinstance(x, torch.Tensor))
+            flops_all.append(int(fc.get_total_flops()))
+            bytes_all.append(int(nbytes))
     return flops_all, bytes_all
 
 

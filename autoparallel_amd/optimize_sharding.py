@@ -226,6 +226,33 @@ class _Variables(collections.abc.Mapping):
         return len(self._opt.decision_vars)
 
 
+def enumerate_strategies(graph, mesh) -> Dict[torch.fx.Node, Any]:
+    """Placement strategies of every node that carries a tensor, in graph order
+    (build_sharding_metadata, autoparallel/optimize_sharding.py:306-354)."""
+    strats: Dict[torch.fx.Node, Any] = {}
+    for node in graph.nodes:
+        if node.op in ("placeholder", "get_attr"):
+            val = node.meta.get("val")
+            if isinstance(val, torch.Tensor):
+                strats[node] = _create_all_options(mesh, val.shape, tensor=val)
+            elif node.op == "placeholder":
+                strats[node] = _create_all_options(mesh, ())
+        elif node.op == "call_function":
+            if not _produces_tensor(node.meta.get("val")):
+                continue
+            in_nodes = [x for x in tree_flatten(node.args)[0]
+                        if isinstance(x, torch.fx.Node) and x in strats]
+            producers = [strats[x] for x in in_nodes]
+            arg_vals = [x.meta["val"] for x in in_nodes]
+            schema_args = tree_map_only(torch.fx.Node, lambda x: strats.get(x, x.meta.get("val")), node.args)
+            strats[node] = get_placement_options_for_node(mesh, node, producers, arg_vals, schema_args)
+        elif node.op == "output":
+            strats[node] = tree_map_only(torch.fx.Node, lambda x: strats[x], node.args)
+        else:
+            raise ValueError(f"Unexpected node op: {node.op}")
+    return strats
+
+
 class ShardingOptimizer:
     def __init__(self, gm, mesh, force_grad_reduce_in_higher_precision: bool = False,
                  repeated_subgraphs: bool = False, devices_per_host: Optional[int] = None,
@@ -295,28 +322,7 @@ class ShardingOptimizer:
 
     # -- strategies ---------------------------------------------------------------
     def build_sharding_metadata(self) -> Dict[torch.fx.Node, Any]:
-        strats: Dict[torch.fx.Node, Any] = {}
-        for node in self.graph.nodes:
-            if node.op in ("placeholder", "get_attr"):
-                val = node.meta.get("val")
-                if isinstance(val, torch.Tensor):
-                    strats[node] = _create_all_options(self.mesh, val.shape, tensor=val)
-                elif node.op == "placeholder":
-                    strats[node] = _create_all_options(self.mesh, ())
-            elif node.op == "call_function":
-                if not _produces_tensor(node.meta.get("val")):
-                    continue
-                in_nodes = [x for x in tree_flatten(node.args)[0]
-                            if isinstance(x, torch.fx.Node) and x in strats]
-                producers = [strats[x] for x in in_nodes]
-                arg_vals = [x.meta["val"] for x in in_nodes]
-                schema_args = tree_map_only(torch.fx.Node, lambda x: strats.get(x, x.meta.get("val")), node.args)
-                strats[node] = get_placement_options_for_node(self.mesh, node, producers, arg_vals, schema_args)
-            elif node.op == "output":
-                strats[node] = tree_map_only(torch.fx.Node, lambda x: strats[x], node.args)
-            else:
-                raise ValueError(f"Unexpected node op: {node.op}")
-        return strats
+        return enumerate_strategies(self.graph, self.mesh)
 
     def _all_input_nodes(self, node) -> List[torch.fx.Node]:
         return [x for x in tree_flatten(node.args)[0] if isinstance(x, torch.fx.Node) and x in self.strats]

@@ -229,9 +229,11 @@ def test_nccl_model_through_reference_api(mesh):
     assert cm.detect_nccl_topo_config(_M(), device_name="NVIDIA GB200") is None  # 16 % 72 != 0
 
 
-def test_runtime_cost_api_matches_reference_vectors(mesh, golden):
-    """estimate_strategy_runtime_cost on fx nodes: the closed-form ops through
-    programs, an op without one (cumsum) through the explicit route."""
+def test_runtime_cost_api_routes(mesh):
+    """estimate_strategy_runtime_cost on fx nodes: a closed-form operator through
+    its program, one without (cumsum) through the explicit route, a view for
+    nothing, each against the oracle's roofline.  (The reference's own vectors
+    are reproduced through this function in test_gpu_fx_dispatch.py.)"""
     from torch.distributed.tensor._dtensor_spec import DTensorSpec, TensorMeta
     from torch.distributed.tensor._op_schema import OpSpec
     from torch.distributed.tensor.placement_types import Replicate, Shard

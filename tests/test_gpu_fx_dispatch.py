@@ -1,0 +1,314 @@
+"""From an FX node to its compute program: the choice fx_programs._closed_form
+makes, pinned two ways.
+
+1. The reference's own estimate_strategy_runtime_cost on hand-built fx nodes
+   (tests/golden/cost_vectors.npz, ``rt_json``: written by the reference with the
+   device patched to MI355X), reproduced through this package's
+   cost_models.estimate_strategy_runtime_cost on the same nodes, bit for bit.
+2. On traced joint graphs (GPT-2 small and four layers of Llama-3-8B as
+   transformers defines them), for every node that gets a program and every
+   one of its strategies: the program evaluated by the oracle on the oracle's
+   local shapes equals what the reference's route gives for that node, the
+   operator run on meta tensors of the sharded sizes under FlopCounterMode
+   (autoparallel/cost_models/compute_estimation.py:321-388, 438-493).
+"""
+import collections
+import contextlib
+import json
+
+import pytest
+import torch
+import torch.nn as nn
+
+from oracle import cost_oracle as O
+
+pytestmark = pytest.mark.gpu
+aten = torch.ops.aten
+
+
+@contextlib.contextmanager
+def _fake_group(world):
+    import torch.distributed as dist
+    from torch.testing._internal.distributed.fake_pg import FakeStore
+
+    if dist.is_initialized():
+        dist.destroy_process_group()
+    dist.init_process_group("fake", store=FakeStore(), rank=0, world_size=world)
+    try:
+        yield
+    finally:
+        dist.destroy_process_group()
+
+
+# the operators of the golden runtime cases: name -> (target, arguments after the tensors,
+# or the equation before them for einsum), as tests/golden/make_cost_vectors.py builds them
+_RT_OPS = {
+    "mm": (aten.mm.default, ()), "mm_f32": (aten.mm.default, ()), "bmm": (aten.bmm.default, ()),
+    "addmm": (aten.addmm.default, ()), "add": (aten.add.Tensor, ()), "mul_bcast": (aten.mul.Tensor, ()),
+    "small_add": (aten.add.Tensor, ()), "silu": (aten.silu.default, ()),
+    "sum_dim": (aten.sum.dim_IntList, ([2], True)), "mean_dim": (aten.mean.dim, ([-1], True)),
+    "einsum_fwd": (aten.einsum.default, "bsk,kn->bsn"), "einsum_bwd": (aten.einsum.default, "bsn,bsk->kn"),
+    "softmax": (aten._softmax.default, (-1, False)), "embedding": (aten.embedding.default, ()),
+    "view": (aten.view.default, ([64, 8192, 32, 128],)),
+    "sdpa_flash": (aten._scaled_dot_product_flash_attention.default, (0.0, True)),
+}
+
+
+def _placements(codes):
+    from torch.distributed.tensor.placement_types import Partial, Replicate, Shard
+
+    out = []
+    for c in codes:
+        out.append(Replicate() if c == 0 else Shard(c & 0x3F) if (c & 0xC0) == 0x40 else Partial())
+    return tuple(out)
+
+
+def test_runtime_cost_api_reproduces_the_reference_vectors(golden):
+    if not torch.cuda.is_available():
+        pytest.skip("needs a GPU")
+    from torch.distributed.device_mesh import init_device_mesh
+    from torch.distributed.tensor._dtensor_spec import DTensorSpec, TensorMeta
+    from torch.distributed.tensor._op_schema import OpSpec
+
+    from autoparallel_amd import cost_models as cm, fx_programs
+
+    d = json.loads(bytes(golden["rt_json"]).decode())
+    assert set(d["names"]) == set(_RT_OPS)
+    with _fake_group(64):
+        mesh = init_device_mesh("cpu", tuple(d["mesh"]))
+        cm.configure(devices_per_host=8, device_name="AMD Instinct MI355X")
+        before = sum(fx_programs.fallback_ops.values())
+        nodes = {}
+        for i, name in enumerate(d["names"]):
+            if name not in nodes:
+                target, extra = _RT_OPS[name]
+                graph = torch.fx.Graph()
+                phs = []
+                for k, (shape, dt) in enumerate(zip(d["shapes"][i], d["dtypes"][i])):
+                    ph = graph.placeholder(f"x{k}")
+                    ph.meta["val"] = torch.empty(shape, dtype=getattr(torch, dt.split(".")[1]), device="meta")
+                    phs.append(ph)
+                args = (extra, phs) if isinstance(extra, str) else tuple(phs) + tuple(extra)
+                node = graph.call_function(target, args)
+                vals = [p.meta["val"] for p in phs]
+                node.meta["val"] = target(extra, vals) if isinstance(extra, str) else target(*vals, *extra)
+                nodes[name] = (node, phs)
+            node, phs = nodes[name]
+            in_specs = []
+            for ph, codes in zip(phs, d["placements"][i]):
+                v = ph.meta["val"]
+                in_specs.append(DTensorSpec(mesh, _placements(codes), tensor_meta=TensorMeta(v.shape, v.stride(), v.dtype)))
+            cm.reset_compute_cost_cache()
+            got = cm.estimate_strategy_runtime_cost(node, OpSpec(output_specs=in_specs[0], input_specs=in_specs))
+            want = float.fromhex(d["cost_hex"][i])
+            assert float(got).hex() == want.hex(), (name, d["placements"][i], got, want)
+        # every one of these operators has a closed form: none took the explicit route
+        assert sum(fx_programs.fallback_ops.values()) == before
+
+
+def _oracle_shapes(st, mesh_shape):
+    from autoparallel_amd.dtensor_bridge import placement_codes, tensor_meta_key
+
+    shapes, isz = [], []
+    for s in st.input_specs:
+        shape, stride, itemsize, _ = tensor_meta_key(s.tensor_meta)
+        local, _ = O.sharded_shape_stride(list(shape), list(stride), list(placement_codes(s.placements)), list(mesh_shape))
+        shapes.append(list(local))
+        isz.append(itemsize)
+    return shapes, isz
+
+
+def _check_programs_of(gm, mesh):
+    """Every node of the graph that describe_node would give a program: program
+    on oracle shapes == FlopCounterMode route, for every strategy.  Returns the
+    operators checked, with the number of distinct nodes of each."""
+    from autoparallel_amd import fx_programs
+    from autoparallel_amd.optimize_sharding import enumerate_strategies
+
+    strats = enumerate_strategies(gm.graph, mesh)
+    seen, checked, explicit, refused = set(), collections.Counter(), collections.Counter(), collections.Counter()
+    for node in gm.graph.nodes:
+        if node.op != "call_function" or node not in strats:
+            continue
+        t = node.target
+        if not isinstance(t, torch._ops.OpOverload) or t.is_view or t is aten._unsafe_view.default:
+            continue
+        prog = fx_programs._closed_form(node)
+        sts = strats[node].strategies
+        tensors = fx_programs._tensor_arg_vals(node)
+        if prog is None or len(tensors) != len(sts[0].input_specs) or any(s is None for st in sts for s in st.input_specs):
+            explicit[str(t)] += 1  # priced from FlopCounterMode's own numbers: nothing chosen here
+            continue
+        key = (t, tuple((tuple(v.shape), tuple(v.stride()), v.dtype) for v in tensors),
+               fx_programs.non_tensor_args_key(node),
+               tuple(tuple(s.placements for s in st.input_specs) for st in sts))
+        try:
+            if key in seen:
+                continue
+            seen.add(key)
+        except TypeError:
+            pass
+        try:
+            flops, nbytes = fx_programs._flops_bytes_via_torch(node, sts)
+        except AssertionError as exc:
+            # torch's flop formula for attention refuses grouped-query shapes (fewer
+            # key/value heads than query heads): the reference's route raises on such a
+            # node, so there is nothing to compare the program with
+            assert "scaled_dot_product" in str(t) and ("incompatible" in str(exc) or "mismatch" in str(exc)), (str(t), exc)
+            q, k_ = tensors[0], tensors[1]
+            if "backward" in str(t):
+                q, k_ = tensors[1], tensors[2]
+            assert q.shape[1] != k_.shape[1]
+            refused[str(t)] += 1
+            continue
+        for k, st in enumerate(sts):
+            shapes, isz = _oracle_shapes(st, mesh.shape)
+            assert O.run_program(prog, shapes, isz) == (flops[k], nbytes[k]), \
+                (str(t), node.name, k, [str(s) for s in st.input_specs], O.run_program(prog, shapes, isz),
+                 (flops[k], nbytes[k]))
+        checked[str(t)] += 1
+    print("explicit route:", dict(explicit))
+    print("refused by torch's flop counter:", dict(refused))
+    return checked, refused
+
+
+def _trace(module, ids):
+    from torch._functorch.aot_autograd import aot_export_joint_with_descriptors
+
+    with contextlib.ExitStack() as stack:
+        return aot_export_joint_with_descriptors(stack, module, (ids,)).graph_module
+
+
+def test_programs_of_the_traced_gpt2_small_graph():
+    transformers = pytest.importorskip("transformers")
+    if not torch.cuda.is_available():
+        pytest.skip("needs a GPU")
+    from torch._subclasses.fake_tensor import FakeTensorMode
+    from torch.distributed.device_mesh import init_device_mesh
+
+    class Wrap(nn.Module):
+        def __init__(self, lm):
+            super().__init__()
+            self.lm = lm
+
+        def forward(self, ids):
+            t = self.lm.transformer
+            x = t.wte(ids) + t.wpe(torch.arange(ids.shape[1], device=ids.device))[None]
+            for blk in t.h:
+                out = blk(x)
+                x = out[0] if isinstance(out, tuple) else out
+            logits = self.lm.lm_head(t.ln_f(x))
+            return torch.nn.functional.cross_entropy(
+                logits[:, :-1].reshape(-1, logits.shape[-1]).float(), ids[:, 1:].reshape(-1))
+
+    cfg = transformers.GPT2Config(attn_pdrop=0.0, embd_pdrop=0.0, resid_pdrop=0.0, use_cache=False,
+                                  attn_implementation="sdpa")
+    with FakeTensorMode():
+        with torch.device("cuda"):
+            m = Wrap(transformers.GPT2LMHeadModel(cfg))
+        gm = _trace(m, torch.randint(0, cfg.vocab_size, (8, 1024), device="cuda"))
+    with _fake_group(8):
+        checked, refused = _check_programs_of(gm, init_device_mesh("cpu", (8,)))
+    print(dict(checked))
+    # (this fp32 model's attention is the memory-efficient kernel, which has no program)
+    families = {"aten.addmm.default", "aten.mm.default", "aten.embedding.default", "aten.sum.dim_IntList",
+                "aten.add.Tensor", "aten.mul.Tensor", "aten.tanh.default", "aten.clone.default",
+                "aten._log_softmax.default", "aten._log_softmax_backward_data.default"}
+    assert families <= set(checked), families - set(checked)
+    assert not refused
+
+
+class _LlamaLoss(nn.Module):
+    def __init__(self, lm):
+        super().__init__()
+        self.lm = lm
+
+    def forward(self, ids):
+        m = self.lm.model
+        x = m.embed_tokens(ids)
+        pos = torch.arange(ids.shape[1], device=ids.device)[None]
+        pe = m.rotary_emb(x, pos)
+        for layer in m.layers:
+            out = layer(x, attention_mask=None, position_ids=pos, position_embeddings=pe)
+            x = out[0] if isinstance(out, tuple) else out
+        logits = self.lm.lm_head(m.norm(x))
+        return torch.nn.functional.cross_entropy(
+            logits[:, :-1].reshape(-1, logits.shape[-1]).float(), ids[:, 1:].reshape(-1))
+
+
+def test_programs_of_flash_attention_forward_and_backward():
+    """A bf16 decoder layer with as many key/value heads as query heads: its
+    attention is the flash kernel, forward and backward, which the flop counter
+    has formulas for."""
+    transformers = pytest.importorskip("transformers")
+    if not torch.cuda.is_available():
+        pytest.skip("needs a GPU")
+    from torch._subclasses.fake_tensor import FakeTensorMode
+    from torch.distributed.device_mesh import init_device_mesh
+
+    cfg = transformers.LlamaConfig(
+        vocab_size=4096, hidden_size=512, intermediate_size=1024, num_hidden_layers=1, num_attention_heads=8,
+        num_key_value_heads=8, max_position_embeddings=512, attention_dropout=0.0, use_cache=False,
+        attn_implementation="sdpa")
+    with FakeTensorMode():
+        torch.set_default_dtype(torch.bfloat16)
+        try:
+            with torch.device("cuda"):
+                m = _LlamaLoss(transformers.LlamaForCausalLM(cfg))
+        finally:
+            torch.set_default_dtype(torch.float32)
+        gm = _trace(m, torch.randint(0, cfg.vocab_size, (16, 256), device="cuda"))
+    with _fake_group(8):
+        checked, refused = _check_programs_of(gm, init_device_mesh("cpu", (2, 4)))
+    print(dict(checked))
+    assert {"aten._scaled_dot_product_flash_attention.default",
+            "aten._scaled_dot_product_flash_attention_backward.default"} <= set(checked)
+    assert not refused
+
+
+def test_programs_of_the_traced_llama3_8b_graph():
+    transformers = pytest.importorskip("transformers")
+    if not torch.cuda.is_available():
+        pytest.skip("needs a GPU")
+    from torch._subclasses.fake_tensor import FakeTensorMode
+    from torch.distributed.device_mesh import init_device_mesh
+
+    class Wrap(nn.Module):
+        def __init__(self, lm):
+            super().__init__()
+            self.lm = lm
+
+        def forward(self, ids):
+            m = self.lm.model
+            x = m.embed_tokens(ids)
+            pos = torch.arange(ids.shape[1], device=ids.device)[None]
+            pe = m.rotary_emb(x, pos)
+            for layer in m.layers:
+                out = layer(x, attention_mask=None, position_ids=pos, position_embeddings=pe)
+                x = out[0] if isinstance(out, tuple) else out
+            logits = self.lm.lm_head(m.norm(x))
+            return torch.nn.functional.cross_entropy(
+                logits[:, :-1].reshape(-1, logits.shape[-1]).float(), ids[:, 1:].reshape(-1))
+
+    cfg = transformers.LlamaConfig(
+        vocab_size=128256, hidden_size=4096, intermediate_size=14336, num_hidden_layers=4, num_attention_heads=32,
+        num_key_value_heads=8, max_position_embeddings=8192, rope_theta=500000.0, attention_dropout=0.0,
+        use_cache=False, attn_implementation="sdpa")
+    with FakeTensorMode():
+        torch.set_default_dtype(torch.bfloat16)
+        try:
+            with torch.device("cuda"):
+                m = Wrap(transformers.LlamaForCausalLM(cfg))
+        finally:
+            torch.set_default_dtype(torch.float32)
+        gm = _trace(m, torch.randint(0, cfg.vocab_size, (64, 8192), device="cuda"))
+    with _fake_group(64):
+        checked, refused = _check_programs_of(gm, init_device_mesh("cpu", (8, 8)))
+    print(dict(checked))
+    families = {"aten.mm.default", "aten.embedding.default", "aten.mean.dim", "aten.sum.dim_IntList",
+                "aten._to_copy.default", "aten.silu.default", "aten.mul.Tensor", "aten.rsqrt.default"}
+    assert families <= set(checked), families - set(checked)
+    # 32 query heads on 8 key/value heads: the flop counter the reference relies on has no
+    # formula for it
+    assert set(refused) == {"aten._scaled_dot_product_flash_attention.default",
+                            "aten._scaled_dot_product_flash_attention_backward.default"}
