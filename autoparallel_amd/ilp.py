@@ -151,6 +151,7 @@ class SparseILP:
         self.status = STATUS_NOT_SOLVED
         self.x: Optional[np.ndarray] = None
         self.objective_value: Optional[float] = None
+        self.mip_rel_gap = 0.0  # relative optimality gap HiGHS may stop at
 
     # -- naming ---------------------------------------------------------------
     def next_name(self, prefix: str) -> str:
@@ -250,7 +251,9 @@ class SparseILP:
 
         A, lo, hi, ub = self.to_matrix()
         cons = [LinearConstraint(A, lo, hi)] if A.shape[0] else []
-        opts = {"disp": bool(verbose)}
+        # no optimality gap: the reference's solver (CBC at its defaults) stops at a
+        # proven optimum, so a near-tie must not be decided by a tolerance here
+        opts = {"disp": bool(verbose), "mip_rel_gap": float(self.mip_rel_gap)}
         if time_limit is not None:
             opts["time_limit"] = float(time_limit)
         res = milp(self.objective, constraints=cons, integrality=np.ones(self.n_vars),
@@ -282,6 +285,8 @@ class SparseILP:
             prob.solve(solver)
         if prob.status == -1:
             self.status = STATUS_INFEASIBLE
+            self.x = None
+            self.objective_value = None
             return self.status
         self.x = np.asarray([round(v.value() or 0.0) for v in xs], np.float64)
         self.objective_value = float(self.objective @ self.x)
@@ -308,7 +313,7 @@ class SparseILP:
                 if c == 0:
                     continue
                 sign = "-" if c < 0 else "+"
-                mag = abs(c)
+                mag = abs(float(c))  # a Python float: numpy scalars print as np.float64(...)
                 parts.append(f"{sign} {vn(i)}" if mag == 1 else f"{sign} {mag!r} {vn(i)}")
             return " ".join(parts) if parts else "0"
 
@@ -317,7 +322,7 @@ class SparseILP:
             nz = np.nonzero(self.objective)[0]
             f.write(expr(nz, self.objective[nz]) + "\nSubject To\n")
             for r in self.constraints.values():
-                f.write(f"{r.name}: {expr(r.idx, r.coef)} {_SENSE_STR[r.sense]} {r.rhs!r}\n")
+                f.write(f"{r.name}: {expr(r.idx, r.coef)} {_SENSE_STR[r.sense]} {float(r.rhs)!r}\n")
             f.write("Binaries\n")
             for i in range(self.n_vars):
                 if self.upper[i] > 0:  # variables fixed out of the model are not declared

@@ -339,26 +339,37 @@ class ShardingOptimizer:
                     yield argi, out_idx, inp_idx
 
     # -- packing -------------------------------------------------------------------
+    def _has_aot_descriptors(self) -> bool:
+        """Whether the graph is an AOT joint graph with input/output descriptors
+        (meta['desc'] on its placeholders): the source of the forward/backward
+        pairs.  A hand-built graph has none, and then no such pairs exist."""
+        phs = [n for n in self.graph.nodes if n.op == "placeholder"]
+        return bool(phs) and all("desc" in n.meta for n in phs)
+
     def _roles(self) -> GraphRoles:
         from torch._functorch._aot_autograd import fx_utils
 
+        self._input_idx, self._output_idx = [], []
+        if not self._has_aot_descriptors():
+            logger.debug("no AOT descriptors on the graph: no forward/backward constraints")
+            return GraphRoles()
+        # With descriptors, anything that goes wrong below is an error, as in the
+        # reference: a plan without the parameter/gradient rows would be wrong silently.
         r = GraphRoles()
         nm = self.node_map
-        try:
-            for p, g in fx_utils.get_param_and_grad_nodes(self.graph).values():
-                r.param_grad.append((nm[p], nm[g] if g is not None and g in nm else -1))
-            # position of each plain input / output among the traced function's own
-            # (an input without a placeholder of its own, e.g. an alias, leaves a gap)
-            self._input_idx, self._output_idx = [], []
-            for desc, (n, g) in fx_utils.get_plain_input_and_grad_nodes(self.graph).items():
-                r.input_grad.append((nm[n], nm[g] if g is not None and g in nm else -1))
-                self._input_idx.append(getattr(desc, "idx", len(self._input_idx)))
-            for desc, (n, t) in fx_utils.get_plain_output_and_tangent_nodes(self.graph).items():
-                r.output_tangent.append((nm[n], nm[t] if t is not None and t in nm else -1))
-                self._output_idx.append(getattr(desc, "idx", len(self._output_idx)))
-            self._mark_pre_cast_nodes(r)
-        except Exception:  # a graph without AOT descriptors has no forward/backward pairs
-            logger.debug("no AOT descriptors on the graph: no forward/backward constraints")
+        input_idx, output_idx = [], []
+        for p, g in fx_utils.get_param_and_grad_nodes(self.graph).values():
+            r.param_grad.append((nm[p], nm[g] if g is not None and g in nm else -1))
+        # position of each plain input / output among the traced function's own
+        # (an input without a placeholder of its own, e.g. an alias, leaves a gap)
+        for desc, (n, g) in fx_utils.get_plain_input_and_grad_nodes(self.graph).items():
+            r.input_grad.append((nm[n], nm[g] if g is not None and g in nm else -1))
+            input_idx.append(getattr(desc, "idx", len(input_idx)))
+        for desc, (n, t) in fx_utils.get_plain_output_and_tangent_nodes(self.graph).items():
+            r.output_tangent.append((nm[n], nm[t] if t is not None and t in nm else -1))
+            output_idx.append(getattr(desc, "idx", len(output_idx)))
+        self._mark_pre_cast_nodes(r)
+        self._input_idx, self._output_idx = input_idx, output_idx
         return r
 
     # operators that stand for the mixed-precision cast of a parameter or its gradient
@@ -412,10 +423,10 @@ class ShardingOptimizer:
         consumer is terminal-derived (autoparallel/graph_passes/graph_utils.py:447-484)."""
         from .graph_utils import build_param_derived_set, build_terminal_derived_set
 
-        try:
+        if self._has_aot_descriptors():
             derived = build_param_derived_set(self.graph)
             terminal = build_terminal_derived_set(self.graph)
-        except Exception:  # a graph without AOT descriptors has no parameters to prefetch
+        else:  # a graph without AOT descriptors has no parameters to prefetch
             derived, terminal = set(), set()
         out = set()
         for node in self.nodes:
@@ -511,11 +522,13 @@ class ShardingOptimizer:
     # -- constraints (delegated to the packed formulation) ------------------------------
     def add_node_constraint(self, node, placement=None, constraint_name=None):
         node = self._normalize_node(node)
-        self._constraint_log.append(("add_node_constraint", {"node_name": node.name, "placement": placement,
-                                                             "constraint_name": constraint_name}))
         assert node in self.strats, node
         codes = None if placement is None else placement_codes(placement)
-        return self._core.add_node_constraint(self.node_map[node], codes, constraint_name)
+        names = self._core.add_node_constraint(self.node_map[node], codes, constraint_name)
+        # logged once the rows exist: a refused constraint must not be replayed from a saved file
+        self._constraint_log.append(("add_node_constraint", {"node_name": node.name, "placement": placement,
+                                                             "constraint_name": constraint_name}))
+        return names
 
     def add_sharded_input_constraint(self, input_placements=None):
         self._io_constraints(self._packed.roles.input_grad, input_placements, "input_constraint",

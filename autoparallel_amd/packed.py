@@ -188,6 +188,9 @@ class PackedGraph:
     # forward (0) / backward (1) tag regions must not cross
     node_kind: Optional[np.ndarray] = None  # uint8[N]
     node_phase: Optional[np.ndarray] = None  # int32[N]
+    # runs of every output of a tuple-valued node (column k: output k, -1 past the
+    # node's outputs); column 0 is node_out_list
+    node_out_runs: Optional[np.ndarray] = None  # int64[N, max outputs]
 
     # -- derived sizes -------------------------------------------------------
     @property
@@ -1038,6 +1041,9 @@ class GraphBuilder:
             edge_prefetchable=pref,
             node_multiplier=mult,
             node_names=[n.name for n in self.nodes],
+            node_out_runs=np.asarray(
+                [[r.get(k, -1) for k in range(max((len(x) for x in out_runs), default=1))] for r in out_runs],
+                np.int64).reshape(len(out_runs), -1),
         )
         g.validate()
         return g

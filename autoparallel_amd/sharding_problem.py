@@ -315,6 +315,21 @@ class PackedShardingOptimizer:
         words = g.lists[run : run + int(g.node_nstrat[v])]
         return [None if int(w) == SPEC_NONE else int(w) & (MAX_TUPLES - 1) for w in words]
 
+    def _first_out_placements(self, v: int) -> List[Optional[int]]:
+        """Per strategy of node v, the placement-tuple id of its first output
+        that has a spec (None if none has): what a node constraint is matched
+        against for a tuple-valued node (autoparallel/optimize_sharding.py:1696-1706)."""
+        g = self.g
+        runs = None if g.node_out_runs is None else [int(r) for r in g.node_out_runs[v] if r >= 0]
+        if not runs or len(runs) == 1:
+            return self._out_placements(v)
+        out: List[Optional[int]] = []
+        for o in range(int(g.node_nstrat[v])):
+            words = [int(g.lists[r + o]) for r in runs]
+            first = next((w for w in words if w != SPEC_NONE), None)
+            out.append(None if first is None else first & (MAX_TUPLES - 1))
+        return out
+
     def _add_paired_output_constraint(self, a: int, b: int, name: str) -> None:
         pa, pb = self._out_placements(a), self._out_placements(b)
         ea, eb = int(self.g.node_edge_off[a]), int(self.g.node_edge_off[b])
@@ -360,24 +375,24 @@ class PackedShardingOptimizer:
         if placement is None:
             placement = (0x40,) + (0x00,) * (g.ndim - 1)
         want = tuple(int(p) for p in placement)
-        allowed = [o for o, t in enumerate(self._out_placements(v))
+        allowed = [o for o, t in enumerate(self._first_out_placements(v))
                    if t is not None and tuple(int(x) for x in g.tuple_plc[t, : g.ndim]) == want]
         if not allowed:
             raise RuntimeError(
                 f"Couldn't find appropriate constraint {g.node_names[v] if g.node_names else v} "
                 f"{constraint_name} {[plc_str(p) for p in want]}")
-        self._constraint_log.append(("add_node_constraint", {
-            "v": int(v), "placement": [int(p) for p in want], "constraint_name": constraint_name}))
+        # A node of a repeated subgraph has no variables of its own: the rows go on
+        # its root's (edge_alias), as the reference's variable lookup resolves a
+        # linked key to its root (autoparallel/optimize_sharding.py:1401-1417).
         names = []
-        if self.linked[v]:
-            raise RuntimeError(
-                f"node {g.node_names[v] if g.node_names else v} shares the variables of node "
-                f"{int(self.root[v])} (repeated subgraph): constrain that node instead")
         for e in range(int(g.node_edge_off[v]), int(g.node_edge_off[v + 1])):
             idx = np.concatenate([self._row_vars(e, o) for o in allowed])
             name = self.prob.add_row(constraint_name or "user_constraint", idx, 1.0, ilp.EQ, 1.0)
             names.append(name)
             self._node_constraint_names[name] = v
+        # logged once the rows exist: a refused constraint is not replayed by load()
+        self._constraint_log.append(("add_node_constraint", {
+            "v": int(v), "placement": [int(p) for p in want], "constraint_name": constraint_name}))
         return names
 
     def add_parameter_memory_constraint(self, memory_factor_low: float, memory_factor_high: float) -> None:

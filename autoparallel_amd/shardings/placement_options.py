@@ -15,8 +15,10 @@ engine.  Input/parameter options are enumerated on the device
 """
 from __future__ import annotations
 
+import contextlib
 import ctypes as C
 import itertools
+import logging
 import operator
 from typing import Dict, List, Optional, Sequence
 
@@ -31,8 +33,33 @@ from torch.utils._pytree import tree_flatten
 from .. import _lib
 
 aten = torch.ops.aten
+logger = logging.getLogger(__name__)
+
 fallback_nodes: List[str] = []  # nodes that got the implicit all-Replicate strategy
 fallback_reasons: Dict[str, str] = {}  # node name -> why its operator strategy was not used
+
+# An operator without a registered strategy function gets the all-Replicate
+# stand-in, with a warning, as the reference's driver arranges
+# (autoparallel/shardings/placement_options.py:331 inside with_implicit_strategies,
+# dtensor_sharding_helpers.py:327-361).  Anything else that goes wrong for a
+# node (a rule or strategy function that raises, strategies whose input specs do
+# not match the node's tensor inputs, no strategy left after the validity
+# filter) is an error, as it is there, unless a caller opts into the stand-in
+# for those as well.
+_stand_in_on_error = False
+
+
+@contextlib.contextmanager
+def replicate_stand_in_on_error():
+    """Inside: a node whose strategies cannot be produced gets the
+    all-Replicate stand-in (logged as a warning, reason kept in
+    ``fallback_reasons``) instead of raising."""
+    global _stand_in_on_error
+    old, _stand_in_on_error = _stand_in_on_error, True
+    try:
+        yield
+    finally:
+        _stand_in_on_error = old
 
 
 def _tensor_meta(t: torch.Tensor) -> TensorMeta:
@@ -706,7 +733,11 @@ def _placement_options_uncached(mesh, node, producers, arg_vals, schema_args) ->
                                 st.input_specs = (st.output_specs,)
         why = "no strategy registered" if out is None else ""
     except Exception as exc:
+        if not _stand_in_on_error:
+            logger.error("strategies of node %s (%s) failed: %s: %s", node.name, op, type(exc).__name__, exc)
+            raise
         out, why = None, f"{type(exc).__name__}: {exc}"
+    unregistered = out is None and why == "no strategy registered"
     ok = out is not None and len(out.strategies) > 0 and all(
         st.input_specs is not None and len(st.input_specs) == len(producers) for st in out.strategies)
     if not ok:
@@ -714,6 +745,9 @@ def _placement_options_uncached(mesh, node, producers, arg_vals, schema_args) ->
             why = "no strategies" if not out.strategies else (
                 f"{len(producers)} tensor inputs, input specs of "
                 f"{sorted({-1 if st.input_specs is None else len(st.input_specs) for st in out.strategies})}")
+        if not unregistered and not _stand_in_on_error:
+            raise ValueError(f"node {node.name} ({op}): {why}")
+        logger.warning("node %s: all-Replicate stand-in for `%s` (%s)", node.name, op, why)
         fallback_reasons[str(node.name)] = why
         out = _replicate_fallback(mesh, node, arg_vals)
     _unshare_specs(out, producers)
@@ -722,7 +756,11 @@ def _placement_options_uncached(mesh, node, producers, arg_vals, schema_args) ->
     out = remove_invalid_configs(out, mesh)
     out = keep_unique_configs(out)
     if not out.strategies:
-        fallback_reasons[str(node.name)] = "no strategy is valid for the shapes"
+        why = "no strategy is valid for the shapes"
+        if not _stand_in_on_error:
+            raise ValueError(f"node {node.name} ({op}): {why}")
+        logger.warning("node %s: all-Replicate stand-in for `%s` (%s)", node.name, op, why)
+        fallback_reasons[str(node.name)] = why
         out = _replicate_fallback(mesh, node, arg_vals)
         fill_redistribute_cost(out, producers)
     return out

@@ -243,6 +243,53 @@ def test_partial_candidates_do_not_cost_the_operator_its_strategies(meshes):
     assert all(len(st.redistribute_cost[0]) == 3 and len(st.output_specs) == 2 for st in out.strategies)
 
 
+def test_failures_raise_and_only_unregistered_operators_get_the_stand_in(meshes, caplog, monkeypatch):
+    """As in the reference (dtensor_sharding_helpers.py:327-361 under
+    with_implicit_strategies, placement_options.py:328-346): an operator without
+    a registered strategy function is planned all-Replicate, with a warning; a
+    rule that raises is an error, unless the caller opts into the stand-in."""
+    import logging
+
+    from autoparallel_amd.shardings import placement_options as PO
+
+    mesh = meshes[0]
+    PO.reset_placement_options_cache()
+    src = _candidates(mesh, (512, 64), [(Replicate(),), (Shard(0),)])
+    g = torch.fx.Graph()
+    x = g.placeholder("x")
+    x.meta["val"] = torch.empty(512, 64, device="meta")
+    # 1. no strategy function: stand-in + warning
+    prop = PO.DTensor._op_dispatcher.sharding_propagator
+    op = torch.ops.aten.flip.default
+    assert op not in prop.op_strategy_funcs
+    node = g.call_function(op, (x, [0]))
+    node.meta["val"] = torch.empty(512, 64, device="meta")
+    PO.fallback_nodes.clear()
+    with caplog.at_level(logging.WARNING, logger=PO.logger.name):
+        out = PO.get_placement_options_for_node(mesh, node, [src], [x.meta["val"]], (src, [0]))
+    assert PO.fallback_nodes == [node.name] and "no strategy registered" in PO.fallback_reasons[node.name]
+    assert any("all-Replicate stand-in" in r.message for r in caplog.records)
+    assert [st.output_specs.placements for st in out.strategies] == [(Replicate(),)]
+    # 2. a rule that raises: the error reaches the caller
+    def broken(mesh, node, producer):
+        raise KeyError("boom")
+
+    monkeypatch.setattr(PO, "_view_rule", broken)
+    view = g.call_function(torch.ops.aten.view.default, (x, [64, 512]))
+    view.meta["val"] = torch.empty(64, 512, device="meta")
+    PO.fallback_nodes.clear()
+    with pytest.raises(KeyError, match="boom"):
+        PO.get_placement_options_for_node(mesh, view, [src], [x.meta["val"]], (src, [64, 512]))
+    assert PO.fallback_nodes == []
+    # 3. ... unless asked for the stand-in
+    with PO.replicate_stand_in_on_error(), caplog.at_level(logging.WARNING, logger=PO.logger.name):
+        out = PO.get_placement_options_for_node(mesh, view, [src], [x.meta["val"]], (src, [64, 512]))
+    assert PO.fallback_nodes == [view.name] and "KeyError" in PO.fallback_reasons[view.name]
+    assert [st.output_specs.placements for st in out.strategies] == [(Replicate(),)]
+    PO.reset_placement_options_cache()
+    PO.fallback_nodes.clear()
+
+
 def test_local_map_region_has_its_declared_strategy(meshes):
     """A local_map region offers exactly the placements its author declared
     (autoparallel/shardings/placement_options.py:380-490): leading arguments

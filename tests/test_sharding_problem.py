@@ -123,6 +123,36 @@ def test_lp_file(tiny, tmp_path):
     assert "n_tokens_s_" in text  # reference variable naming, sanitised for the LP format
 
 
+def test_lp_file_text_of_a_three_variable_model(tmp_path):
+    """The LP text, character for character: objective with a unit, a fractional
+    and a negative coefficient, one row of each sense, a negative right-hand
+    side, a variable fixed out of the model (not declared binary), names
+    sanitised for the format."""
+    p = ilp.SparseILP(3)
+    p.objective = np.asarray([1.0, 2.5, -3.0])
+    p.add_row("pick", [0, 1, 2], 1.0, ilp.EQ, 1.0)
+    p.add_row("cap", [0, 2], [2.0, -1.0], ilp.LE, 1.5)
+    p.add_row("floor", [1], [1.0], ilp.GE, -2.0)
+    p.upper[2] = 0.0
+    path = os.path.join(tmp_path, "m.lp")
+    p.write_lp(path, ["n=a,s=0,arg=0,output_p=0,input_p=0", "n=a,s=0,arg=0,output_p=0,input_p=1", "z z"])
+    x0, x1 = "n_a_s_0_arg_0_output_p_0_input_p_0", "n_a_s_0_arg_0_output_p_0_input_p_1"
+    assert open(path).read() == (
+        "\\* AutoParallel *\\\n"
+        "Minimize\n"
+        f"OBJ: + {x0} + 2.5 {x1} - 3.0 z_z\n"
+        "Subject To\n"
+        f"pick_000: + {x0} + {x1} + z_z = 1.0\n"
+        f"cap_000: + 2.0 {x0} - z_z <= 1.5\n"
+        f"floor_000: + {x1} >= -2.0\n"
+        "Binaries\n"
+        f"{x0}\n{x1}\n"
+        "End\n")
+    # and without names
+    p.write_lp(path)
+    assert "OBJ: + x0 + 2.5 x1 - 3.0 x2\n" in open(path).read()
+
+
 def test_sparse_ilp_basics():
     p = ilp.SparseILP(3)
     p.objective = np.asarray([1.0, 2.0, 3.0])
@@ -191,8 +221,46 @@ def test_clustered_ilp_matches_reference_semantics():
     assert opt.objective_value >= plain.objective_value - 1e-6
     assert np.isclose(opt.objective_value, plain.objective_value, rtol=1e-6)
     assert opt.cluster_links and all(opt.root[r] == r for r in opt.cluster_links.values())
-    with pytest.raises(RuntimeError, match="shares the variables"):
-        opt.add_node_constraint(int(np.nonzero(opt.linked)[0][0]))
+    # a constraint on a repeated node lands on its root's variables
+    # (autoparallel/optimize_sharding.py:1401-1417: the variable lookup resolves links)
+    v = next(int(x) for x in np.nonzero(opt.linked)[0] if opt._first_out_placements(int(x))[int(sol[x])] is not None)
+    r = int(opt.root[v])
+    other = next(o for o, t in enumerate(opt._first_out_placements(v))
+                 if t is not None and t != opt._first_out_placements(v)[int(sol[v])])
+    want = tuple(int(x) for x in g2.tuple_plc[opt._first_out_placements(v)[other], : g2.ndim])
+    n_log = len(opt._constraint_log)
+    names = opt.add_node_constraint(v, want, "pin_linked")
+    assert len(names) == int(g2.node_edge_off[v + 1] - g2.node_edge_off[v]) and len(opt._constraint_log) == n_log + 1
+    for name, e in zip(names, range(int(g2.node_edge_off[r]), int(g2.node_edge_off[r + 1]))):
+        row = opt.prob.constraints[name]
+        assert int(opt.var_start[e]) <= row.idx.min() and row.idx.max() < int(opt.var_start[e + 1])
+    sol2 = opt.get_solution()
+    chosen = tuple(int(x) for x in g2.tuple_plc[opt._first_out_placements(v)[int(sol2[v])], : g2.ndim])
+    assert chosen == want and sol2[v] == sol2[r]
+    # a constraint that cannot be met is refused and leaves no trace in the log
+    with pytest.raises(RuntimeError, match="Couldn't find"):
+        opt.add_node_constraint(v, (0x47,) * g2.ndim)
+    assert len(opt._constraint_log) == n_log + 1
+
+
+def test_node_constraint_matches_the_first_output_that_has_a_spec():
+    """For a tuple-valued node the placement is matched against the first output
+    with a spec in each strategy (autoparallel/optimize_sharding.py:1696-1706)."""
+    from autoparallel_amd.packed import DT_F32, GraphBuilder, NodeDesc
+
+    b = GraphBuilder((2,), 8)
+    m = b.meta((8, 8), (8, 1), 4, DT_F32)
+    r_, s0 = b.spec(m, (0x00,)), b.spec(m, (0x40,))
+    b.add_node(NodeDesc("x", [[r_], [s0]], [[r_], [s0]], inputs=[], default_rows=[[[0.0]], [[0.0]]]))
+    # two outputs; strategy 1 has no spec for output 0, its first output with a spec is Shard(0)
+    b.add_node(NodeDesc("pair", [[r_], [s0]], [[r_, r_], [-1, s0]], inputs=[0], tuple_output=True))
+    g = b.pack()
+    assert g.node_out_runs.shape == (2, 2) and g.node_out_runs[0, 1] == -1
+    coef, _ = oracle_coefficients(g)
+    opt = PackedShardingOptimizer(g, coefficients=coef)
+    assert opt._out_placements(1)[1] is None and opt._first_out_placements(1)[1] is not None
+    opt.add_node_constraint(1, (0x40,))
+    assert opt.get_solution()[1] == 1
 
 
 def test_violated_constraints_log(tiny):
