@@ -25,6 +25,18 @@ class ApcModel(C.Structure):
         ("order_mode", C.c_int32),
         ("reserved", C.c_int32),
         ("nccl_plan", C.c_void_p),
+        ("mesh_a2a_bw", C.c_double * MAX_MESH_DIMS),
+    ]
+
+
+class ApcXgmiConfig(C.Structure):
+    _fields_ = [
+        ("gpus_per_node", C.c_int32),
+        ("links_per_gpu", C.c_int32),
+        ("link_gbps", C.c_double),
+        ("nic_gbps", C.c_double),
+        ("lat_intra_us", C.c_double),
+        ("lat_inter_us", C.c_double),
     ]
 
 
@@ -166,6 +178,8 @@ _SIGNATURES = {
     "apc_last_error": (C.c_char_p, []),
     "apc_mesh_topology": (C.c_int, [C.c_void_p, C.c_int32, C.c_int32, C.c_void_p, C.c_void_p]),
     "apc_device_limits": (C.c_int, [C.c_char_p, C.POINTER(ApcModel)]),
+    "apc_xgmi_topology": (
+        C.c_int, [C.POINTER(ApcXgmiConfig), C.c_void_p, C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p]),
     "apc_nccl_plan_build": (C.c_int, [C.POINTER(ApcNcclConfig), C.c_void_p, C.c_int32, C.POINTER(ApcNcclPlan)]),
     "apc_nccl_plan_for_topo": (
         C.c_int,

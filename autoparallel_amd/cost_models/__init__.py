@@ -1,10 +1,17 @@
 from .collective_runtime_estimation import (  # noqa: F401
+    XGMITopoConfig,
     collective_comm_cost,
     configure,
+    detect_mesh_topo_config,
     estimate_strategy_comms_cost,
+    get_mesh_topo_config,
     get_nccl_topo_config,
+    mi300x_topo_config,
+    mi355x_topo,
+    mi355x_topo_config,
     redistribute_cost,
     reset_comms_cost_cache,
+    set_mesh_topo_config,
     set_nccl_topo_config,
 )
 from .compute_estimation import (  # noqa: F401

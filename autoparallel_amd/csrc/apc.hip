@@ -931,6 +931,32 @@ int apc_mesh_topology(const int32_t* mesh_shape, int32_t ndim, int32_t devices_p
   return 0;
 }
 
+int apc_xgmi_topology(const apc_xgmi_config* cfg, const int32_t* mesh_shape, int32_t ndim, double* bw,
+                      double* lat, double* a2a_bw) {
+  if (!cfg || !mesh_shape || !bw || !lat || !a2a_bw || ndim < 1 || ndim > APC_MAX_MESH_DIMS)
+    return fail(APC_ERR_INVALID, "apc_xgmi_topology: bad arguments%s");
+  if (cfg->gpus_per_node < 1 || cfg->links_per_gpu < 1 || !(cfg->link_gbps > 0.0) || !(cfg->nic_gbps > 0.0))
+    return fail(APC_ERR_INVALID, "apc_xgmi_topology: gpus_per_node, links_per_gpu, link_gbps, nic_gbps must be positive%s");
+  const double one_way = cfg->link_gbps / 2.0;
+  int64_t total = 1;
+  for (int i = ndim - 1; i >= 0; --i) {
+    const int n = mesh_shape[i];
+    if (n < 1) return fail(APC_ERR_INVALID, "apc_xgmi_topology: mesh size < 1%s");
+    total *= n;
+    if (total <= cfg->gpus_per_node) {
+      const int links = n - 1 < cfg->links_per_gpu ? n - 1 : cfg->links_per_gpu;
+      bw[i] = one_way;
+      a2a_bw[i] = one_way * (double)(links > 1 ? links : 1);
+      lat[i] = cfg->lat_intra_us;
+    } else {
+      bw[i] = cfg->nic_gbps;
+      a2a_bw[i] = cfg->nic_gbps;
+      lat[i] = cfg->lat_inter_us;
+    }
+  }
+  return 0;
+}
+
 namespace {
 // Device table of autoparallel/cost_models/compute_estimation.py:66-255, in its
 // order (the first entry whose name occurs in the device name wins): memory

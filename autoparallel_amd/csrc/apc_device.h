@@ -143,7 +143,9 @@ __device__ __forceinline__ double collective_cost(int kind, int64_t nbytes, int 
   int n = m.mesh_shape[i];
   int hops = (kind == 2) ? 2 * (n - 1) : (n - 1);
   double latency = 6.6 + (double)hops * m.mesh_lat[i];
-  double bw = div_int(g * (double)hops, n) / m.mesh_bw[i];
+  // an all_to_all may see another bandwidth than the ring collectives (direct links)
+  const double dim_bw = (kind == 1 && m.mesh_a2a_bw[i] > 0.0) ? m.mesh_a2a_bw[i] : m.mesh_bw[i];
+  double bw = div_int(g * (double)hops, n) / dim_bw;
   double t = latency + bw * 1e6;
   if (kind == 1) t = t * 5.0;
   return t;

@@ -21,9 +21,23 @@ _PACKED_SCORING_FROM = 8192  # mean entries per edge block
 _SCORE_LANES_FROM = 32768  # assignments: below, one wavefront per assignment (entry arrays as they are)
 
 
-def make_model(mesh_shape, devices_per_host: int, device_name: str, order_mode: int = 0) -> _lib.ApcModel:
+def xgmi_config_struct(cfg) -> _lib.ApcXgmiConfig:
+    """apc_xgmi_config from any object with XGMITopoConfig's fields."""
+    if isinstance(cfg, _lib.ApcXgmiConfig):
+        return cfg
+    c = _lib.ApcXgmiConfig()
+    c.gpus_per_node, c.links_per_gpu = int(cfg.gpus_per_node), int(cfg.links_per_gpu)
+    c.link_gbps, c.nic_gbps = float(cfg.link_gbps), float(cfg.nic_gbps)
+    c.lat_intra_us, c.lat_inter_us = float(cfg.lat_intra_us), float(cfg.lat_inter_us)
+    return c
+
+
+def make_model(mesh_shape, devices_per_host: int, device_name: str, order_mode: int = 0,
+               topo_config=None) -> _lib.ApcModel:
     """Cost-model constants for a mesh on a named device (raises ApcError for a
-    device the reference's table does not know either)."""
+    device the reference's table does not know either).  ``topo_config``: an
+    XGMITopoConfig whose link constants replace the reference's NVLink-era ones
+    (then ``devices_per_host`` is not used)."""
     lib = _lib.load()
     m = _lib.ApcModel()
     nd = len(mesh_shape)
@@ -38,6 +52,14 @@ def make_model(mesh_shape, devices_per_host: int, device_name: str, order_mode: 
         lib.apc_mesh_topology(C.addressof(shape), nd, int(devices_per_host), C.addressof(bw), C.addressof(lat)),
         "apc_mesh_topology",
     )
+    if topo_config is not None:
+        a2a = (C.c_double * MAX_MESH_DIMS)()
+        xc = xgmi_config_struct(topo_config)
+        _lib.check(
+            lib.apc_xgmi_topology(C.byref(xc), C.addressof(shape), nd, C.addressof(bw), C.addressof(lat),
+                                  C.addressof(a2a)),
+            "apc_xgmi_topology")
+        m.mesh_a2a_bw = a2a
     m.mesh_bw = bw
     m.mesh_lat = lat
     _lib.check(lib.apc_device_limits(device_name.encode(), C.byref(m)), "apc_device_limits")
@@ -111,11 +133,13 @@ class CostEngine:
         nccl_config=None,
         table_mode: Optional[str] = None,
         item_entries: Optional[int] = None,
+        topo_config=None,
     ):
         """``table_mode``: "full" (one S_dst x S_src matrix per distinct pair of
         runs), "compressed" (matrices by distinct spec word, read by gather),
         "direct" (no table: every entry evaluated), or None: the first of the
-        three whose table is small against the entry count.  ``use_table`` is
+        three whose table is small against the entry count.  ``topo_config``:
+        an XGMITopoConfig for the alpha-beta constants (make_model).  ``use_table`` is
         the older switch: True = "full", False = "direct".  ``item_entries``:
         entries per work item of the entry kernel, 256 or 512 (512 needs a
         table); None: by problem size."""
@@ -145,7 +169,8 @@ class CostEngine:
             return t.data_ptr() if t.numel() else None
 
         p = _lib.ApcProblem()
-        model = make_model([int(x) for x in g.mesh_shape], g.devices_per_host, device_name, order_mode)
+        model = make_model([int(x) for x in g.mesh_shape], g.devices_per_host, device_name, order_mode,
+                           topo_config=topo_config)
         if nccl_config is not None:  # NCCL-tuning collectives instead of alpha-beta
             self._keep["nccl_plan"] = upload_nccl_plan(model, nccl_config, self.device)
         p.model = model

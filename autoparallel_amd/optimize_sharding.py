@@ -477,6 +477,7 @@ class ShardingOptimizer:
             self._packed, roles=self._packed.roles,
             force_grad_reduce_in_higher_precision=self.force_grad_reduce_in_higher_precision,
             device_name=self._device_name, nccl_config=_cre.get_nccl_topo_config(),
+            topo_config=_cre.get_mesh_topo_config(),
             repeated_subgraphs=self.repeated_subgraphs)
         # per-variable link table of the reference (:356-378): linked key -> root key
         self.cluster_links = {}

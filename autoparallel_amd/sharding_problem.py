@@ -104,6 +104,7 @@ class PackedShardingOptimizer:
         nccl_config=None,
         repeated_subgraphs: bool = False,
         cluster_root: Optional[np.ndarray] = None,
+        topo_config=None,
     ):
         """repeated_subgraphs: cluster identical regions (node hashes from the
         device) and let every repeated node share the decision variables of its
@@ -119,7 +120,8 @@ class PackedShardingOptimizer:
             from .engine import CostEngine  # the HIP path; raises without the library / a GPU
 
             t0 = time.perf_counter()
-            self.engine = CostEngine(g, device=device, device_name=device_name, nccl_config=nccl_config)
+            self.engine = CostEngine(g, device=device, device_name=device_name, nccl_config=nccl_config,
+                                     topo_config=topo_config)
             t1 = time.perf_counter()
             self.engine.build(clamp_inf=True)
             self.engine.synchronize()

@@ -162,6 +162,11 @@ typedef struct apc_model {
    * copy of the plan that apc_nccl_plan_build fills: collectives are priced by
    * the NCCL-tuning model (collective_runtime_estimation.py:44-62, 85-86). */
   const struct apc_nccl_plan* nccl_plan;
+  /* GB/s that all_to_all sees on each mesh dim, where it differs from mesh_bw
+   * (a fabric of direct links, on which an all-to-all drives every link at once
+   * while a ring drives one); 0 = mesh_bw, the reference's model.  Filled by
+   * apc_xgmi_topology. */
+  double mesh_a2a_bw[APC_MAX_MESH_DIMS];
 } apc_model;
 
 /* ---- NCCL-tuning collective model (autoparallel/cost_models/nccl_cost_model.py) ----
@@ -323,6 +328,30 @@ const char* apc_last_error(void);
  * devices per host.  bw/lat: host arrays of ndim doubles. */
 int apc_mesh_topology(const int32_t* mesh_shape, int32_t ndim, int32_t devices_per_host,
                       double* bw, double* lat);
+
+/* Host helper, no counterpart in the reference, which has topology presets for
+ * NVLink/NVSwitch systems only (nccl_cost_model.py:1413-1470) and detects none
+ * on an MI355X (:1341-1410), leaving that user with NVLink constants.  Per-dim
+ * constants of the alpha-beta model for nodes whose GPUs are joined pairwise
+ * by xGMI links: walking the mesh dims from the innermost out, a dim lies inside
+ * a node while the product of the sizes so far is at most gpus_per_node.
+ * Inside a node a ring collective (allgather, reduce_scatter, allreduce) moves
+ * every byte over one link per rank and direction: bw = link_gbps / 2 (a link's
+ * figure counts both directions); an all_to_all among the n ranks of the dim
+ * drives min(n - 1, links_per_gpu) links of every rank at once: a2a_bw = that
+ * many times bw.  Between nodes both are nic_gbps (per GPU).  lat: lat_intra_us
+ * / lat_inter_us per hop.  bw, lat, a2a_bw: host arrays of ndim doubles, to be
+ * copied into apc_model.mesh_bw / mesh_lat / mesh_a2a_bw. */
+typedef struct apc_xgmi_config {
+  int32_t gpus_per_node; /* 8 */
+  int32_t links_per_gpu; /* 7: one direct link to every peer of the node */
+  double link_gbps;      /* one link, both directions together: 153.6 on MI355X */
+  double nic_gbps;       /* per GPU between nodes */
+  double lat_intra_us;   /* per hop inside a node */
+  double lat_inter_us;   /* per hop between nodes */
+} apc_xgmi_config;
+int apc_xgmi_topology(const apc_xgmi_config* cfg, const int32_t* mesh_shape, int32_t ndim, double* bw,
+                      double* lat, double* a2a_bw);
 
 /* Host helper.  Replaces _get_device_limit / _get_device_tflops /
  * _get_device_gmem_bandwidth (autoparallel/cost_models/compute_estimation.py:258-297)

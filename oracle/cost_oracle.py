@@ -101,9 +101,10 @@ class DeviceLimit:
 class Topo:
     """MeshTopoInfo (torch _collective_utils.py:236-278)."""
 
-    def __init__(self, mesh_shape: Sequence[int], devices_per_host: int, nccl=None):
+    def __init__(self, mesh_shape: Sequence[int], devices_per_host: int, nccl=None, xgmi=None):
         ndim = len(mesh_shape)
         self.nccl = nccl  # oracle.nccl_oracle.NcclConfig selects the NCCL model
+        self.a2a_bw = None  # per dim, where all_to_all sees another bandwidth (xgmi)
         base_bw = 87.7
         self.mesh_shape = tuple(int(x) for x in mesh_shape)
         self.bw = [base_bw] * ndim
@@ -117,6 +118,25 @@ class Topo:
             if total > devices_per_host:
                 self.bw[d] *= 0.22
                 self.lat[d] = 2.7
+        if xgmi is not None:
+            # Not in the reference (an extension of this build, outside the parity
+            # claim): nodes of GPUs joined pairwise by xGMI links.  xgmi: an object
+            # with gpus_per_node, links_per_gpu, link_gbps (both directions), nic_gbps,
+            # lat_intra_us, lat_inter_us.  A ring moves every byte over one link per
+            # direction; an all_to_all among n ranks drives min(n - 1, links) links.
+            one_way = xgmi.link_gbps / 2.0
+            self.a2a_bw = [0.0] * ndim
+            total = 1
+            for d in reversed(range(ndim)):
+                n = self.mesh_shape[d]
+                total *= n
+                if total <= xgmi.gpus_per_node:
+                    self.bw[d] = one_way
+                    self.a2a_bw[d] = one_way * float(max(1, min(n - 1, xgmi.links_per_gpu)))
+                    self.lat[d] = xgmi.lat_intra_us
+                else:
+                    self.bw[d] = self.a2a_bw[d] = xgmi.nic_gbps
+                    self.lat[d] = xgmi.lat_inter_us
 
 
 def allgather_cost(bytes_gb: float, topo: Topo, dim: int) -> float:
@@ -147,7 +167,8 @@ def all_to_all_cost(bytes_gb: float, topo: Topo, dim: int) -> float:
     n = topo.devices[dim]
     hops = n - 1
     latency = 6.6 + hops * topo.lat[dim]
-    bw = (bytes_gb * hops / n) / topo.bw[dim]
+    dim_bw = topo.a2a_bw[dim] if topo.a2a_bw is not None and topo.a2a_bw[dim] > 0 else topo.bw[dim]
+    bw = (bytes_gb * hops / n) / dim_bw
     total = latency + bw * 1e6
     total *= 5
     return total
@@ -382,10 +403,10 @@ class GraphOracle:
     memo caches of the reference (optimize_sharding.py:481-552;
     collective_runtime_estimation.py:239-262; compute_estimation.py:449-492)."""
 
-    def __init__(self, g, dev: Optional[DeviceLimit] = None, nccl=None):
+    def __init__(self, g, dev: Optional[DeviceLimit] = None, nccl=None, xgmi=None):
         self.g = g
         self.dev = dev or DeviceLimit()
-        self.topo = Topo([int(x) for x in g.mesh_shape], g.devices_per_host, nccl=nccl)
+        self.topo = Topo([int(x) for x in g.mesh_shape], g.devices_per_host, nccl=nccl, xgmi=xgmi)
         self.ndim = len(self.topo.mesh_shape)
         self._comm_cache: Dict[tuple, float] = {}
         self._compute_cache: Dict[tuple, float] = {}

@@ -514,6 +514,26 @@ def test_node_program_paths(CostEngine):
         _check_build(CostEngine, g, mode)
 
 
+@pytest.mark.parametrize("mode", ["full", "direct"])
+def test_xgmi_topology_on_the_device(CostEngine, mode):
+    """With the xGMI link constants selected, the device and the oracle still
+    agree bit for bit, every all_to_all entry changes and nothing else does
+    that has no collective on a dim whose constants moved."""
+    from autoparallel_amd import cost_models as cm
+
+    cfg = cm.mi355x_topo_config()
+    g = graphgen.llama_graph((8, 8), 1, 1024, 8, 4, 2048, 8192, 512, 16)
+    got = CostEngine(g, table_mode=mode, topo_config=cfg).build(clamp_inf=False).results()
+    ref = O.GraphOracle(g, xgmi=cfg).build()
+    assert bits_equal(got["comm"], ref["comm"]), first_mismatch(got["comm"], ref["comm"])
+    assert bits_equal(got["cost"], ref["cost"])
+    plain = O.GraphOracle(g).build()
+    assert bits_equal(got["compute"], plain["compute"])  # the compute estimate does not see the links
+    finite = np.isfinite(plain["comm"])
+    assert (ref["comm"][finite] != plain["comm"][finite]).any()
+    assert ((ref["comm"] == 0) == (plain["comm"] == 0)).all() and (np.isfinite(ref["comm"]) == finite).all()
+
+
 def test_unsupported_dtype_reports(CostEngine):
     b = GraphBuilder((2,), 8)
     m = b.meta((8, 8), (8, 1), 8, packed.DT_OTHER)
