@@ -134,12 +134,16 @@ class CostEngine:
         table_mode: Optional[str] = None,
         item_entries: Optional[int] = None,
         topo_config=None,
+        allocate_results: bool = True,
     ):
         """``table_mode``: "full" (one S_dst x S_src matrix per distinct pair of
         runs), "compressed" (matrices by distinct spec word, read by gather),
         "direct" (no table: every entry evaluated), or None: the first of the
         three whose table is small against the entry count.  ``topo_config``:
-        an XGMITopoConfig for the alpha-beta constants (make_model).  ``use_table`` is
+        an XGMITopoConfig for the alpha-beta constants (make_model).
+        ``allocate_results=False``: only the problem is uploaded (for the node
+        hashes, which are taken before it is decided which edges get entries);
+        such an engine cannot build.  ``use_table`` is
         the older switch: True = "full", False = "direct".  ``item_entries``:
         entries per work item of the entry kernel, 256 or 512 (512 needs a
         table); None: by problem size."""
@@ -268,7 +272,8 @@ class CostEngine:
         p.table_units = up("table_units", g.table_unit_records(squeezed))
         self.problem = p
 
-        E, NC = g.num_slots, g.num_compute
+        E, NC = (g.num_slots, g.num_compute) if allocate_results else (0, 0)
+        self.can_build = bool(allocate_results)
         # entry arrays hold num_slots elements; padding slots stay zero
         self.compute = torch.zeros(NC, dtype=torch.float64, device=self.device)
         self.per_arg = torch.zeros(NC, dtype=torch.float64, device=self.device)
@@ -279,7 +284,8 @@ class CostEngine:
         tsize = int(self.lib.apc_pair_table_size(C.byref(p)))
         self.use_table = table_mode != "direct"
         self.table = (
-            torch.empty(tsize, dtype=torch.float64, device=self.device) if self.use_table else None
+            torch.empty(tsize, dtype=torch.float64, device=self.device)
+            if self.use_table and allocate_results else None
         )
         self.built = False
         self._build_args = None
@@ -349,6 +355,8 @@ class CostEngine:
         )
 
     def build_args(self):
+        if not self.can_build:
+            raise _lib.ApcError("this engine holds the problem only (allocate_results=False)")
         if self._build_args is None:
             self._build_args = (
                 C.byref(self.problem), self._ptr(self.table), self._ptr(self.compute), self._ptr(self.per_arg),

@@ -142,36 +142,46 @@ def _flops_bytes_via_torch(node, strategies, shapes_fn=None) -> Tuple[List[int],
     from torch._subclasses.fake_tensor import FakeTensorMode
 
     flat_specs = [s for st in strategies for s in st.input_specs if s is not None]
-    shapes = iter((shapes_fn or local_shapes)(flat_specs))
-    flops_all, bytes_all = [], []
+    shapes = (shapes_fn or local_shapes)(flat_specs)
     flat_args, treespec = tree_flatten(node.args)
     kwargs = {k: (v.meta["val"] if isinstance(v, torch.fx.Node) else v) for k, v in node.kwargs.items()}
-    # Fake tensors on the traced tensors' own device, as the reference runs the
-    # operator (compute_estimation.py:334-365): an operator that names a device in
-    # its arguments (_to_copy) cannot run on meta tensors.
-    with FakeTensorMode(allow_non_fake_inputs=True):
-        for st in strategies:
-            new_flat, counter = [], 0
-            for a in flat_args:
-                if isinstance(a, torch.fx.Node):
-                    a = a.meta["val"]
-                    if isinstance(a, torch.Tensor):
-                        spec = st.input_specs[counter]
-                        counter += 1
-                        if spec is not None:
-                            sizes, strides = next(shapes)
-                        else:
-                            sizes, strides = a.shape, a.stride()
-                        a = torch.empty_strided(sizes, strides, dtype=a.dtype, device=a.device)
-                new_flat.append(a)
-            args = treespec.unflatten(new_flat)
-            with FlopCounterMode(display=False) as fc:
-                out = node.target(*args, **kwargs)
-            nbytes = sum(x.numel() * x.element_size() for x in tree_flatten(args)[0] if isinstance(x, torch.Tensor))
-            nbytes += sum(x.numel() * x.element_size() for x in tree_flatten(out)[0] if isinstance(x, torch.Tensor))
-            flops_all.append(int(fc.get_total_flops()))
-            bytes_all.append(int(nbytes))
-    return flops_all, bytes_all
+    # Meta tensors carry all the counters need (sizes and dtypes).  An operator that
+    # names a device in its arguments (_to_copy) cannot run on them: it runs on fake
+    # tensors of the traced tensors' own device instead, as the reference runs
+    # every operator (compute_estimation.py:334-365).
+    def run(make, mode):
+        flops_all, bytes_all = [], []
+        it = iter(shapes)
+        with mode:
+            for st in strategies:
+                new_flat, counter = [], 0
+                for a in flat_args:
+                    if isinstance(a, torch.fx.Node):
+                        a = a.meta["val"]
+                        if isinstance(a, torch.Tensor):
+                            spec = st.input_specs[counter]
+                            counter += 1
+                            sizes, strides = next(it) if spec is not None else (a.shape, a.stride())
+                            a = make(sizes, strides, a)
+                    new_flat.append(a)
+                args = treespec.unflatten(new_flat)
+                with FlopCounterMode(display=False) as fc:
+                    out = node.target(*args, **kwargs)
+                nbytes = sum(x.numel() * x.element_size() for x in tree_flatten(args)[0] if isinstance(x, torch.Tensor))
+                nbytes += sum(x.numel() * x.element_size() for x in tree_flatten(out)[0] if isinstance(x, torch.Tensor))
+                flops_all.append(int(fc.get_total_flops()))
+                bytes_all.append(int(nbytes))
+        return flops_all, bytes_all
+
+    import contextlib
+
+    shapes = list(shapes)
+    try:
+        return run(lambda sizes, strides, a: torch.empty_strided(sizes, strides, dtype=a.dtype, device="meta"),
+                   contextlib.nullcontext())
+    except NotImplementedError:
+        return run(lambda sizes, strides, a: torch.empty_strided(sizes, strides, dtype=a.dtype, device=a.device),
+                   FakeTensorMode(allow_non_fake_inputs=True))
 
 
 def describe_node(node, strategies, b: GraphBuilder, name: Optional[str] = None,

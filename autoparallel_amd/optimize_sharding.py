@@ -13,6 +13,7 @@ reference's insertion order (node, out_idx, argi, inp_idx; :511-520).
 from __future__ import annotations
 
 import collections.abc
+import dataclasses
 import logging
 import time
 import operator
@@ -29,7 +30,7 @@ from .cost_models import collective_runtime_estimation as _cre
 from .dtensor_bridge import devices_per_host as _mesh_dph
 from .dtensor_bridge import placement_codes
 from .engine import detect_device_name
-from .packed import GraphBuilder, PackedGraph
+from .packed import GraphBuilder, NodeDesc, PackedGraph
 from .sharding_problem import GraphRoles, PackedShardingOptimizer
 from .shardings.placement_options import _create_all_options, get_placement_options_for_node
 
@@ -133,6 +134,38 @@ class DecisionVars(collections.abc.Mapping):
 
     def __len__(self) -> int:
         return self._keys.shape[0]
+
+
+class _ClusterLinks(collections.abc.Mapping):
+    """The reference's per-variable link table (linked key -> root key,
+    autoparallel/optimize_sharding.py:356-378) as a view over the node-level
+    links: a repeated node's key maps to the same (arg, out, inp) of its root.
+    Keys are produced on iteration, not stored (a 32-layer model has millions)."""
+
+    def __init__(self, opt: "ShardingOptimizer", node_links: Dict[int, int]):
+        self._opt, self._nodes = opt, dict(node_links)
+
+    def __getitem__(self, key):
+        v, a, o, j = key
+        r = self._nodes.get(int(v))
+        if r is None or key not in self._opt.decision_vars:
+            raise KeyError(key)
+        return (r, int(a), int(o), int(j))
+
+    def __iter__(self):
+        for v in self._nodes:
+            for a, o, j in self._opt.walk_over_options(self._opt.nodes[v]):
+                yield (v, a, o, j)
+
+    def __len__(self) -> int:
+        g = self._opt._packed
+        sizes = g.edge_sdst.astype(np.int64) * g.edge_ssrc
+        linked = np.zeros(g.num_nodes, bool)
+        linked[list(self._nodes)] = True
+        return int(sizes[linked[g.edge_node]].sum())
+
+    def __bool__(self) -> bool:
+        return bool(self._nodes)
 
 
 def concretize_symint(val):
@@ -442,17 +475,26 @@ class ShardingOptimizer:
         index_of: Dict[torch.fx.Node, int] = {}
         self._packed_index: Dict[int, int] = {}  # node_idx -> packed node
         memo: Dict[str, dict] = {}
+        described: Dict[tuple, NodeDesc] = {}  # by strategy query: the repeated layers of a model
         for node in self.nodes:
             if node.op == "output":
                 continue
             st: OpStrategy = self.strats[node]
-            desc = fx_programs.describe_node(node, st.strategies, b, name=node.name, memo=memo)
+            qkey = getattr(st, "_apc_query_key", None)
+            seen = described.get(qkey) if qkey is not None else None
+            if seen is not None:  # same operator, arguments and candidates: same specs and program
+                desc = dataclasses.replace(seen, name=node.name, inputs=[], getitem_index=None)
+            else:
+                desc = fx_programs.describe_node(node, st.strategies, b, name=node.name, memo=memo)
+                if qkey is not None:
+                    described[qkey] = desc
             ins = self._all_input_nodes(node)
             desc.inputs = [index_of[x] for x in ins]
             if node.op == "call_function" and node.target is operator.getitem:
                 desc.getitem_index = int(node.args[1])
-            # default rows: what the strategy carried before the engine ran
-            desc.default_rows = [[list(map(float, row)) for row in s.redistribute_cost] for s in st.strategies]
+            # default rows: what the strategy carried before the engine ran (the packer
+            # reads them where an edge has no producer or a spec is missing; not copied)
+            desc.default_rows = [s.redistribute_cost for s in st.strategies]
             desc.nargs = len(st.strategies[0].input_specs)
             index_of[node] = b.add_node(desc)
             self._packed_index[self.node_map[node]] = index_of[node]
@@ -479,12 +521,10 @@ class ShardingOptimizer:
             device_name=self._device_name, nccl_config=_cre.get_nccl_topo_config(),
             topo_config=_cre.get_mesh_topo_config(),
             repeated_subgraphs=self.repeated_subgraphs)
+        self._packed = self._core.g  # with the entry blocks of repeated nodes dropped, if any
         # per-variable link table of the reference (:356-378): linked key -> root key
-        self.cluster_links = {}
-        for v, r in self._core.cluster_links.items():
-            for argi, out_idx, inp_idx in self.walk_over_options(self.nodes[v]):
-                self.cluster_links[(v, argi, out_idx, inp_idx)] = (r, argi, out_idx, inp_idx)
-        self._cluster_linked_node_idxs = {k[0] for k in self.cluster_links}
+        self.cluster_links = _ClusterLinks(self, self._core.cluster_links)
+        self._cluster_linked_node_idxs = set(self._core.cluster_links)
         self.prob = self._core.prob
         self.phase_s.update(self._core.phase_s)
         t0 = time.perf_counter()
@@ -496,11 +536,12 @@ class ShardingOptimizer:
         """strategy.redistribute_cost[argi][inp_idx] = comm, as the reference's
         loop does in place (:540)."""
         g, comm = self._packed, self._core.coef.comm
-        vs = self._core.var_start
+        vs, alias = self._core.var_start, self._core.edge_alias
         for e in range(g.num_edges):
             node = self.nodes[int(g.edge_node[e])]
             a, ssrc = int(g.edge_arg[e]), int(g.edge_ssrc[e])
-            block = comm[vs[e] : vs[e + 1]].reshape(-1, ssrc).tolist()
+            r = int(alias[e])  # a repeated node's rows are its root's (:554-571)
+            block = comm[vs[r] : vs[r + 1]].reshape(-1, ssrc).tolist()
             for s, row in zip(self.strats[node].strategies, block):
                 s.redistribute_cost[a] = row
 

@@ -191,6 +191,12 @@ class PackedGraph:
     # runs of every output of a tuple-valued node (column k: output k, -1 past the
     # node's outputs); column 0 is node_out_list
     node_out_runs: Optional[np.ndarray] = None  # int64[N, max outputs]
+    # Repeated subgraphs: edge_alias[e] is the edge whose entry block stands for e
+    # (e itself for an edge that owns one).  An aliased edge owns no slots: its
+    # edge_off is its alias's, and only owning ("priced") edges count in
+    # num_entries, entry_slots, entry_keys and the work items.  None: every edge
+    # owns its block.  Set through with_edge_alias().
+    edge_alias: Optional[np.ndarray] = None  # int64[NE]
 
     # -- derived sizes -------------------------------------------------------
     @property
@@ -206,9 +212,57 @@ class PackedGraph:
         return int(self.edge_node.shape[0])
 
     @property
+    def priced(self) -> np.ndarray:
+        """bool[NE]: the edge owns an entry block (is not an alias of another)."""
+        if self.edge_alias is None:
+            return np.ones(self.num_edges, bool)
+        return self.edge_alias == np.arange(self.num_edges)
+
+    def block_sizes(self) -> np.ndarray:
+        """int64[NE]: entries of each edge's own block (0 for an aliased edge)."""
+        sizes = self.edge_sdst.astype(np.int64) * self.edge_ssrc
+        return sizes if self.edge_alias is None else np.where(self.priced, sizes, 0)
+
+    @property
     def num_entries(self) -> int:
-        """Real entries (decision variables)."""
-        return int((self.edge_sdst.astype(np.int64) * self.edge_ssrc).sum())
+        """Real entries (decision variables): those of the edges that own a block."""
+        return int(self.block_sizes().sum())
+
+    def with_edge_alias(self, alias: np.ndarray) -> "PackedGraph":
+        """The same graph with the entry blocks of aliased edges dropped: edge e
+        reads the block of edge alias[e], which must have the same strategies on
+        both sides (same spec words, same default rows).  Blocks of the owning
+        edges are laid out compactly, in edge order."""
+        NE = self.num_edges
+        alias = np.asarray(alias, np.int64)
+        assert alias.shape == (NE,) and (alias[alias] == alias).all(), "an alias must own its block"
+        own = alias == np.arange(NE)
+        sizes = self.edge_sdst.astype(np.int64) * self.edge_ssrc
+        a = alias[~own]
+        e = np.nonzero(~own)[0]
+        assert (self.edge_sdst[e] == self.edge_sdst[a]).all() and (self.edge_ssrc[e] == self.edge_ssrc[a]).all()
+        assert ((self.edge_flags[e] & EDGE_HAS_PRODUCER) == (self.edge_flags[a] & EDGE_HAS_PRODUCER)).all()
+        for x, y in zip(e, a):  # same words on both sides, same default rows
+            n_d, n_s = int(self.edge_sdst[x]), int(self.edge_ssrc[x])
+            if self.edge_dst_list[x] != self.edge_dst_list[y]:
+                assert np.array_equal(self.lists[self.edge_dst_list[x]:self.edge_dst_list[x] + n_d],
+                                      self.lists[self.edge_dst_list[y]:self.edge_dst_list[y] + n_d])
+            if self.edge_src_list[x] != self.edge_src_list[y]:
+                assert self.edge_src_list[x] >= 0 and self.edge_src_list[y] >= 0
+                assert np.array_equal(self.lists[self.edge_src_list[x]:self.edge_src_list[x] + n_s],
+                                      self.lists[self.edge_src_list[y]:self.edge_src_list[y] + n_s])
+            dx, dy = int(self.edge_default_off[x]), int(self.edge_default_off[y])
+            assert (dx < 0) == (dy < 0)
+            if dx >= 0:
+                assert np.array_equal(self.default_vals[dx:dx + n_d * n_s], self.default_vals[dy:dy + n_d * n_s])
+        pad = (1 << CHUNK_SHIFT) - 1
+        padded = np.where(own, (sizes + pad) & ~pad, 0)
+        edge_off = np.zeros(NE + 1, np.int64)
+        np.cumsum(padded, out=edge_off[1:])
+        total = int(edge_off[-1])
+        edge_off[:-1][~own] = edge_off[:-1][a]
+        edge_off[-1] = total
+        return dataclasses.replace(self, edge_off=edge_off, edge_alias=alias)
 
     @property
     def num_slots(self) -> int:
@@ -217,7 +271,7 @@ class PackedGraph:
 
     def entry_slots(self) -> np.ndarray:
         """int64[E]: slot of every real entry, in (edge, out_idx, inp_idx) order."""
-        sizes = self.edge_sdst.astype(np.int64) * self.edge_ssrc
+        sizes = self.block_sizes()
         eid = np.repeat(np.arange(self.num_edges, dtype=np.int64), sizes)
         start = np.concatenate([[0], np.cumsum(sizes)[:-1]])
         local = np.arange(int(sizes.sum()), dtype=np.int64) - start[eid]
@@ -231,7 +285,7 @@ class PackedGraph:
         """int32[E, 4] keys (node_idx, argi, out_idx, inp_idx) in entry order
         (the key layout of autoparallel/serialization.py:150-157)."""
         E = self.num_entries
-        sizes = (self.edge_sdst.astype(np.int64) * self.edge_ssrc).astype(np.int64)
+        sizes = self.block_sizes()
         eid = np.repeat(np.arange(self.num_edges, dtype=np.int64), sizes)
         start = np.concatenate([[0], np.cumsum(sizes)[:-1]])
         local = np.arange(E, dtype=np.int64) - start[eid]
@@ -254,7 +308,7 @@ class PackedGraph:
         """(row_base int64[n_edge], row_stride int32[n_edge]): the row of entry
         (e, out_idx, inp_idx) in ``decision_vars`` insertion order is
         ``row_base[e] + out_idx * row_stride[e] + inp_idx``."""
-        ssrc = self.edge_ssrc.astype(np.int64)
+        ssrc = np.where(self.priced, self.edge_ssrc, 0).astype(np.int64)  # an aliased edge has no rows
         node = self.edge_node.astype(np.int64)
         per_node = np.zeros(self.num_nodes, np.int64)  # sum of S_src over the node's arguments
         np.add.at(per_node, node, ssrc)
@@ -583,7 +637,7 @@ class PackedGraph:
             rows[squeeze] = ru[2][dst[squeeze]]
             edge_usrc[squeeze] = cols[squeeze]
             assert (cols < (1 << (31 - EDGE_USRC_SHIFT))).all()
-        ok = np.nonzero(hp & (ssrc * sdst > 0))[0]
+        ok = np.nonzero(hp & (ssrc * sdst > 0) & self.priced)[0]  # an aliased edge reads its alias's matrix
         if ok.shape[0] == 0:
             out = (np.zeros(0, np.int32), np.zeros(1, np.int64), np.zeros(0, np.int32), edge_table_off,
                    edge_usrc, np.zeros(0, np.int32))
@@ -598,6 +652,9 @@ class PackedGraph:
             block_off = np.zeros(block_edge.shape[0] + 1, np.int64)
             np.cumsum((size + 255) & ~255, out=block_off[1:])
             edge_table_off[ok] = block_off[:-1][inv]
+            if self.edge_alias is not None:
+                edge_table_off[~self.priced] = edge_table_off[self.edge_alias[~self.priced]]
+                edge_usrc[~self.priced] = edge_usrc[self.edge_alias[~self.priced]]
             unit_block = np.repeat(np.arange(block_edge.shape[0], dtype=np.int32), np.diff(block_off) // 256)
             out = (block_edge, block_off, unit_block, edge_table_off, edge_usrc, rows[block_edge].astype(np.int32))
         cache[compressed] = out
@@ -608,14 +665,17 @@ class PackedGraph:
         are 16-slot aligned, so a chunk never spans two edges)."""
         nt = self.num_slots >> CHUNK_SHIFT
         starts = np.arange(nt, dtype=np.int64) << CHUNK_SHIFT
-        return (np.searchsorted(self.edge_off, starts, side="right") - 1).astype(np.int32)
+        if self.edge_alias is None:
+            return (np.searchsorted(self.edge_off, starts, side="right") - 1).astype(np.int32)
+        own = np.nonzero(self.priced)[0]  # their blocks are laid out in this order
+        return own[np.searchsorted(self.edge_off[:-1][own], starts, side="right") - 1].astype(np.int32)
 
     def work_items(self, compressed: bool = False, item_entries: int = ITEM_ENTRIES) -> np.ndarray:
         """Work items of the entry kernel: for every ``item_entries`` (256 or 512)
         entries of every edge block a copy of the edge record with ``local0``
         set, in slot order."""
         assert item_entries in (ITEM_ENTRIES, 2 * ITEM_ENTRIES)
-        sizes = self.edge_sdst.astype(np.int64) * self.edge_ssrc
+        sizes = self.block_sizes()
         n = (sizes + item_entries - 1) // item_entries
         eid = np.repeat(np.arange(self.num_edges, dtype=np.int64), n)
         start = np.concatenate([[0], np.cumsum(n)[:-1]])
@@ -681,7 +741,14 @@ class PackedGraph:
             sizes = self.edge_sdst.astype(np.int64) * self.edge_ssrc
             pad = (1 << CHUNK_SHIFT) - 1
             assert (self.edge_off & pad == 0).all(), "edge blocks must be 16-slot aligned"
-            assert (np.diff(self.edge_off) == ((sizes + pad) & ~pad)).all()
+            if self.edge_alias is None:
+                assert (np.diff(self.edge_off) == ((sizes + pad) & ~pad)).all()
+            else:
+                own = self.priced
+                assert self.edge_alias.shape == (NE,) and own[self.edge_alias].all()
+                ends = np.concatenate([self.edge_off[:-1][own][1:], self.edge_off[-1:]])
+                assert (ends - self.edge_off[:-1][own] == ((sizes[own] + pad) & ~pad)).all()
+                assert (self.edge_off[:-1][~own] == self.edge_off[:-1][self.edge_alias[~own]]).all()
             assert (self.edge_dst_list >= 0).all()
             assert (self.edge_dst_list + self.edge_sdst <= L).all()
             hp = (self.edge_flags & EDGE_HAS_PRODUCER) != 0
@@ -1004,6 +1071,7 @@ class GraphBuilder:
                     o0 = int(node_comp_off[v])
                     ef[o0 : o0 + len(nd_.flops)] = nd_.flops
                     eb[o0 : o0 + len(nd_.nbytes)] = nd_.nbytes
+        max_outs = max((len(x) for x in out_runs), default=1)
         g = PackedGraph(
             mesh_shape=np.asarray(self.mesh_shape, np.int32),
             devices_per_host=self.devices_per_host,
@@ -1041,9 +1109,8 @@ class GraphBuilder:
             edge_prefetchable=pref,
             node_multiplier=mult,
             node_names=[n.name for n in self.nodes],
-            node_out_runs=np.asarray(
-                [[r.get(k, -1) for k in range(max((len(x) for x in out_runs), default=1))] for r in out_runs],
-                np.int64).reshape(len(out_runs), -1),
+            node_out_runs=np.asarray([[r.get(k, -1) for k in range(max_outs)] for r in out_runs],
+                                     np.int64).reshape(len(out_runs), max_outs),
         )
         g.validate()
         return g

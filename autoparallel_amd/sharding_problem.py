@@ -57,6 +57,14 @@ class Coefficients:
         self.compute = np.asarray(compute)
         self.per_arg = np.asarray(per_arg)
 
+    def subset(self, keep: np.ndarray) -> "Coefficients":
+        """The coefficients of the variables ``keep`` marks (bool per variable),
+        in order: what is left when some edges lose their entry blocks."""
+        out = object.__new__(Coefficients)
+        out.comm, out.cost, out.flags = self.comm[keep].copy(), self.cost[keep].copy(), self.flags[keep].copy()
+        out.compute, out.per_arg = self.compute, self.per_arg
+        return out
+
     @classmethod
     def from_engine(cls, eng) -> "Coefficients":
         r = eng.results()
@@ -116,12 +124,33 @@ class PackedShardingOptimizer:
         self.force_grad_reduce_in_higher_precision = force_grad_reduce_in_higher_precision
         self.engine = None
         self.phase_s: Dict[str, float] = {}  # seconds per phase of the construction
+        self.region_groups: List[List[List[int]]] = []
+        engine_kw = dict(device=device, device_name=device_name, nccl_config=nccl_config, topo_config=topo_config)
+        # Repeated subgraphs are found before anything is priced: the hashes need the
+        # problem on the device, not its coefficients.  The nodes of a repeat then get
+        # no entries of their own: their edges read the entry blocks of their root
+        # (autoparallel/optimize_sharding.py:501-507, 554-577).
+        t0 = time.perf_counter()
+        if cluster_root is None and repeated_subgraphs:
+            from . import clustering
+            from .engine import CostEngine
+
+            assert g.edge_alias is None, "the graph already carries a clustering"
+            hashes = CostEngine(g, allocate_results=False, **engine_kw).node_hashes(g.node_phase)
+            self.region_groups = clustering.identical_regions(g, hashes)
+            cluster_root = clustering.cluster_roots(g, self.region_groups)
+        g_in = g
+        self._set_cluster_root(cluster_root)
+        g = self.g  # with the entry blocks of linked nodes dropped, if any are linked
+        if coefficients is not None and g is not g_in and coefficients.cost.shape[0] == g_in.num_entries:
+            # coefficients of every node were handed in: keep those of the edges that still own a block
+            coefficients = coefficients.subset(np.repeat(g.priced, g_in.block_sizes()))
+        self.phase_s["clustering"] = time.perf_counter() - t0
         if coefficients is None:
             from .engine import CostEngine  # the HIP path; raises without the library / a GPU
 
             t0 = time.perf_counter()
-            self.engine = CostEngine(g, device=device, device_name=device_name, nccl_config=nccl_config,
-                                     topo_config=topo_config)
+            self.engine = CostEngine(g, **engine_kw)
             t1 = time.perf_counter()
             self.engine.build(clamp_inf=True)
             self.engine.synchronize()
@@ -129,25 +158,11 @@ class PackedShardingOptimizer:
             coefficients = Coefficients.from_engine(self.engine)
             self.phase_s.update(engine_construct=t1 - t0, device_build=t2 - t1, readback=time.perf_counter() - t2)
         self.coef = coefficients
-        self.region_groups: List[List[List[int]]] = []
         t0 = time.perf_counter()
-        if cluster_root is None and repeated_subgraphs:
-            from . import clustering
-
-            hashes = self._ensure_engine().node_hashes(g.node_phase)
-            self.region_groups = clustering.identical_regions(g, hashes)
-            cluster_root = clustering.cluster_roots(g, self.region_groups)
-        self._set_cluster_root(cluster_root)
-        self.phase_s["clustering"] = time.perf_counter() - t0
-        t0 = time.perf_counter()
-        sizes = g.edge_sdst.astype(np.int64) * g.edge_ssrc
-        self.var_start = np.concatenate([[0], np.cumsum(sizes)]).astype(np.int64)
+        self.var_start = np.concatenate([[0], np.cumsum(g.block_sizes())]).astype(np.int64)
         self.n_vars = int(self.var_start[-1])
+        assert self.coef.cost.shape[0] == self.n_vars, "coefficients do not match the graph's decision variables"
         self.prob = ilp.SparseILP(self.n_vars)
-        if self.linked.any():  # variables of linked nodes are their root's: fixed out of the model
-            e_linked = np.nonzero(self.linked[g.edge_node])[0]
-            for e in e_linked:
-                self.prob.upper[self.var_start[e] : self.var_start[e + 1]] = 0.0
         self._memory_constraint: Optional[Tuple[float, float]] = None
         self._node_constraint_names: Dict[str, int] = {}
         self._constraint_log: List[Tuple[str, dict]] = []  # replayed by load (serialization.py)
@@ -170,10 +185,13 @@ class PackedShardingOptimizer:
         if self.linked.any():
             from . import clustering
 
-            mult = clustering.multipliers(self.root)
-            g.node_multiplier = mult
-            if self.engine is not None:
-                self.engine.set_node_multiplier(mult)
+            if g.edge_alias is None:
+                g = self.g = g.with_edge_alias(self.edge_alias)
+            else:  # a graph saved with its clustering
+                assert np.array_equal(g.edge_alias, self.edge_alias), "the graph's aliases are not this clustering's"
+            g.node_multiplier = clustering.multipliers(self.root)
+        else:
+            assert g.edge_alias is None, "the graph aliases edges but no node is linked"
 
     @property
     def cluster_links(self) -> Dict[int, int]:

@@ -655,13 +655,16 @@ def get_placement_options_for_node(mesh, node, producers: List[OpStrategy], arg_
         if hit[1] is not None:
             fallback_nodes.append(str(node.name))
             fallback_reasons[str(node.name)] = hit[1]
-        return _copy_strategy(hit[0])
+        out = _copy_strategy(hit[0])
+        out._apc_query_key = key  # equal keys: equal strategies (what a packer may memoise on)
+        return out
     strategy_cache_stats["misses"] += 1
     n_fallback = len(fallback_nodes)
     out = _placement_options_uncached(mesh, node, producers, arg_vals, schema_args)
     if key is not None:
         why = fallback_reasons.get(str(node.name), "") if len(fallback_nodes) > n_fallback else None
         _strategy_cache[key] = (_copy_strategy(out), why)
+        out._apc_query_key = key
     return out
 
 

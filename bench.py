@@ -430,40 +430,57 @@ def _fx_path_figure(n_layers: int, cpu_port: bool) -> dict:
         mesh = init_device_mesh("cpu", (8, 8))
         PO.fallback_nodes.clear()
         PO.reset_placement_options_cache()
-        t0 = time.perf_counter()
-        opt = ShardingOptimizer(gm, mesh, devices_per_host=8, device_name="AMD Instinct MI355X")
-        t_opt = time.perf_counter() - t0
-        g = opt._packed
-        res = {
+        def leg(repeated_subgraphs: bool) -> dict:
+            PO.fallback_nodes.clear()
+            PO.reset_placement_options_cache()
+            t0 = time.perf_counter()
+            opt = ShardingOptimizer(gm, mesh, devices_per_host=8, device_name="AMD Instinct MI355X",
+                                    repeated_subgraphs=repeated_subgraphs)
+            t_opt = time.perf_counter() - t0
+            g = opt._packed
+            priced_nodes = sorted(set(int(v) for v in g.edge_node[g.priced]))
+            res = {
+                "nodes": g.num_nodes, "edges": g.num_edges, "priced_nodes": len(priced_nodes),
+                # decision variables = entries the engine builds: every node's, or with
+                # repeated_subgraphs those of one representative per repeated node
+                "entries": g.num_entries,
+                "sharding_optimizer_s": t_opt,
+                # the split the reference logs for the same constructor
+                # (autoparallel/optimize_sharding.py:249-291, 579-587)
+                "phase_s": {k: round(v, 6) for k, v in opt.phase_s.items()},
+                "entries_per_s_through_the_api": g.num_entries / t_opt,
+                "strategy_queries": dict(PO.strategy_cache_stats), "replicate_stand_ins": len(PO.fallback_nodes),
+                "ilp_rows": len(opt.prob.constraints),
+            }
+            if cpu_port:
+                # the per-entry Python port on this same packed problem and the same set of
+                # nodes: what the reference's _build_decision_vars loop costs after strategy
+                # enumeration
+                from oracle import cost_oracle as O
+
+                orc = O.GraphOracle(g)
+                orc.reset_caches()
+                t0 = time.perf_counter()
+                orc.build(nodes=priced_nodes)
+                t_cpu = time.perf_counter() - t0
+                coeff_s = sum(opt.phase_s.get(k, 0.0) for k in ("pack", "engine_construct", "device_build", "readback"))
+                device_s = sum(opt.phase_s.get(k, 0.0) for k in ("engine_construct", "device_build", "readback"))
+                res["cpu_baseline"] = {
+                    "kind": "port", "cores": 1, "seconds": t_cpu, "entries_per_s": g.num_entries / t_cpu,
+                    "what": "oracle.cost_oracle.GraphOracle(opt._packed).build(nodes=priced nodes), memo caches "
+                            "cleared first",
+                    "pack_plus_device_phases_s": coeff_s, "device_phases_s": device_s,
+                    "speedup_of_device_phases": t_cpu / device_s if device_s > 0 else None,
+                }
+            return res
+
+        return {
             "workload": f"transformers LlamaForCausalLM, Llama-3-8B dimensions, {n_layers} layers, bf16, "
                         f"batch 64 x 8192, joint graph, mesh (8,8)",
-            "nodes": g.num_nodes, "edges": g.num_edges, "entries": g.num_entries,
-            "trace_s": t_trace, "sharding_optimizer_s": t_opt,
-            # the split the reference logs for the same constructor
-            # (autoparallel/optimize_sharding.py:249-291, 579-587)
-            "phase_s": {k: round(v, 6) for k, v in opt.phase_s.items()},
-            "entries_per_s_through_the_api": g.num_entries / t_opt,
-            "strategy_queries": dict(PO.strategy_cache_stats), "replicate_stand_ins": len(PO.fallback_nodes),
-            "ilp_rows": len(opt.prob.constraints),
+            "trace_s": t_trace,
+            "all_nodes": leg(False),
+            "cluster_roots_only": leg(True),
         }
-        if cpu_port:
-            # the per-entry Python port on this same packed problem: what the reference's
-            # _build_decision_vars loop costs after strategy enumeration
-            from oracle import cost_oracle as O
-
-            orc = O.GraphOracle(g)
-            orc.reset_caches()
-            t0 = time.perf_counter()
-            orc.build()
-            t_cpu = time.perf_counter() - t0
-            coeff_s = sum(opt.phase_s.get(k, 0.0) for k in ("pack", "engine_construct", "device_build", "readback"))
-            res["cpu_baseline"] = {
-                "kind": "port", "cores": 1, "seconds": t_cpu, "entries_per_s": g.num_entries / t_cpu,
-                "what": "oracle.cost_oracle.GraphOracle(opt._packed).build(), memo caches cleared first",
-                "coefficient_phases_s": coeff_s,
-                "speedup_of_coefficient_phases": t_cpu / coeff_s if coeff_s > 0 else None,
-            }
-        return res
     finally:
         if own:
             dist.destroy_process_group()

@@ -56,16 +56,65 @@ def test_full_size_grouping(engine_mod):
     assert clustering.multipliers(root).max() >= 32  # 65 for the norm blocks: two per layer and the final one
 
 
+def _clustered(g, engine_mod):
+    eng = engine_mod.CostEngine(g, allocate_results=False)  # the problem alone is enough for the hashes
+    groups = clustering.identical_regions(g, eng.node_hashes(g.node_phase))
+    root = clustering.cluster_roots(g, groups).astype(np.int64)
+    first = g.node_edge_off[:-1].astype(np.int64)
+    v = g.edge_node.astype(np.int64)
+    return root, first[root[v]] + (np.arange(g.num_edges) - first[v])
+
+
+@pytest.mark.parametrize("mode", ["full", "compressed", "direct"])
+def test_only_cluster_roots_are_priced(engine_mod, mode):
+    """With the edges of repeated nodes aliased to their root's, the build
+    writes the roots' entries only, bit-equal to the same entries of the build of
+    every node; and in that build every repeated edge's block equals its
+    root's, which is what makes reading the root's block for it exact."""
+    from helpers import bits_equal
+    from oracle import cost_oracle as O
+
+    g = GRAPHS["llama_3layer_2x4"]()
+    root, alias = _clustered(g, engine_mod)
+    ga = g.with_edge_alias(alias)
+    assert 0 < ga.num_entries < 0.6 * g.num_entries and ga.num_slots < 0.6 * g.num_slots
+    full = engine_mod.CostEngine(g, table_mode=mode).build(clamp_inf=False).results()
+    part = engine_mod.CostEngine(ga, table_mode=mode).build(clamp_inf=False).results()
+    sizes = g.edge_sdst.astype(np.int64) * g.edge_ssrc
+    for e in range(g.num_edges):
+        a = int(alias[e])
+        lo, n = int(g.edge_off[e]), int(sizes[e])
+        ro, po = int(g.edge_off[a]), int(ga.edge_off[e])
+        assert po == int(ga.edge_off[a])
+        for k in ("comm", "cost"):
+            assert bits_equal(full[k][lo:lo + n], full[k][ro:ro + n]), (k, e, a)  # the premise
+            assert bits_equal(part[k][po:po + n], full[k][lo:lo + n]), (k, e, a)
+        assert (part["flags"][po:po + n] == full["flags"][lo:lo + n]).all()
+    assert bits_equal(part["compute"], full["compute"])
+    # and the oracle, run over the aliased graph, fills the same arrays
+    ref = O.GraphOracle(ga).build()
+    assert bits_equal(part["comm"], ref["comm"]) and bits_equal(part["cost"], ref["cost"])
+    # the exported twin holds the roots' variables only, in decision_vars order
+    eng = engine_mod.CostEngine(ga).build(clamp_inf=False)
+    keys, vals = (t.cpu().numpy() for t in eng.export_decision_vars())
+    assert keys.shape == (ga.num_entries, 4) and not (root[keys[:, 0]] != keys[:, 0]).any()
+    order = ga.decision_var_order()
+    assert np.array_equal(keys, ga.entry_keys()[order])
+    assert bits_equal(vals[:, 1], part["comm"][ga.entry_slots()][order])
+
+
 def test_clustered_optimizer_end_to_end(engine_mod):
     from autoparallel_amd.sharding_problem import PackedShardingOptimizer
 
     plain = PackedShardingOptimizer(GRAPHS["llama_3layer_2x4"]())
-    plain.get_solution()
+    sol_plain = plain.get_solution()
     g = GRAPHS["llama_3layer_2x4"]()
     opt = PackedShardingOptimizer(g, repeated_subgraphs=True)
     assert opt.region_groups and opt.linked.sum() > g.num_nodes // 4
-    n_free = int((opt.prob.upper > 0).sum())
-    assert n_free < 0.8 * opt.n_vars  # linked nodes have no variables of their own
+    # linked nodes have no variables of their own, and no entries were built for them
+    assert opt.n_vars == opt.g.num_entries < 0.6 * plain.n_vars
+    assert opt.engine.comm.numel() == opt.g.num_slots < 0.6 * g.num_slots
+    assert not opt.linked[opt.g.entry_keys()[:, 0]].any()
     sol = opt.get_solution()
     assert (sol[opt.linked] == sol[opt.root[opt.linked]]).all()
     # objective (root cost x multiplicity) == the device's objective of the expanded plan
@@ -74,12 +123,24 @@ def test_clustered_optimizer_end_to_end(engine_mod):
     assert r[5] == 0
     assert np.isclose(r[4], opt.objective_value, rtol=1e-9)
     assert np.isclose(opt.objective_value, plain.objective_value, rtol=1e-6)
+    # the expanded plan scores the same on the engine that priced every node: sums of the
+    # reference's _compute_solution_cost, bit for bit (linked rows are read from the root)
+    r_plain = plain.engine.score(a).cpu().numpy()[0]
+    assert (r[:4] == r_plain[:4]).all()
+    # the identical layers make the free optimum a clustered plan too: same placements
+    assert plain.solution_placements(sol_plain) == opt.solution_placements(sol)
+    # per-edge terms of the plan: a linked edge reports its root's entry
+    terms, slot = opt.solution_terms(sol)
+    terms_plain, _ = plain.solution_terms(sol)
+    assert np.array_equal(terms, terms_plain) and (slot >= 0).all()
+    linked_e = np.nonzero(opt.linked[g.edge_node])[0]
+    assert linked_e.size and (slot[linked_e] == slot[opt.edge_alias[linked_e]]).all()
     # save / load keeps the links
     import tempfile
 
     with tempfile.TemporaryDirectory() as tmp:
         opt.save(tmp + "/c.npz")
         back = PackedShardingOptimizer.load(tmp + "/c.npz")
-    assert back.cluster_links == opt.cluster_links
+    assert back.cluster_links == opt.cluster_links and back.n_vars == opt.n_vars
     assert np.array_equal(back._extract(), sol)
     assert set(back.prob.constraints) == set(opt.prob.constraints)

@@ -977,6 +977,37 @@ def test_hf_llama3_8b_layers_joint_graph():
         for n in mms:
             per_layer.setdefault(tuple(n.meta["val"].shape), []).append(len(opt.strats[n].strategies))
         assert all(len(set(v)) == 1 for v in per_layer.values())
+        # With repeated_subgraphs only the first copy of every layer node is priced
+        # (autoparallel/optimize_sharding.py:501-507): far fewer entries, the same
+        # coefficients where both have them, and the same plan.
+        PO.reset_placement_options_cache()
+        clustered = ShardingOptimizer(gm, mesh88, devices_per_host=8, device_name="AMD Instinct MI355X",
+                                      repeated_subgraphs=True)
+        gc = clustered._packed
+        assert gc.edge_alias is not None and gc.num_entries < 0.45 * g.num_entries
+        assert len(clustered.decision_vars) == gc.num_entries == clustered._core.n_vars
+        own = np.repeat(gc.priced, g.block_sizes())
+        assert bits_equal(clustered._core.coef.comm, opt._core.coef.comm[own])
+        assert bits_equal(clustered._core.coef.cost, opt._core.coef.cost[own])
+        # a repeated node's strategies carry its root's redistribution rows (:554-571)
+        v = int(np.nonzero(clustered._core.linked)[0][-1])
+        r = int(clustered._core.root[v])
+        for s_l, s_r, s_p in zip(clustered.strats[clustered.nodes[v]].strategies,
+                                 clustered.strats[clustered.nodes[r]].strategies,
+                                 opt.strats[opt.nodes[v]].strategies):
+            assert s_l.redistribute_cost == s_r.redistribute_cost == s_p.redistribute_cost
+        sol_c = clustered.get_solution()
+        opt.get_solution()
+        # Tying the layers together is a restriction of the free problem (here the first and the
+        # last layer would rather differ from the middle ones): its optimum cannot be lower, and
+        # its plan, expanded to every node, costs on the optimizer that priced every node exactly
+        # what the clustered objective says (root cost x multiplicity).
+        assert clustered._core.objective_value >= opt._core.objective_value * (1 - 1e-9)
+        idx = torch.from_numpy(clustered._out_indices(sol_c).astype(np.int16).reshape(-1, 1)).cuda()
+        r = opt._core.engine.score(idx).cpu().numpy()[0]
+        assert r[5] == 0 and np.isclose(r[4], clustered._core.objective_value, rtol=1e-9)
+        rc = clustered._core.engine.score(idx).cpu().numpy()[0]
+        assert (rc[:4] == r[:4]).all() and np.isclose(rc[4], r[4], rtol=1e-12)
     finally:
         dist.destroy_process_group()
         if had_pg:

@@ -147,3 +147,50 @@ def test_table_units_tile_every_matrix(name, compressed):
         # the units of a matrix start every 256 elements and reach past its last one
         assert (mine["first"] == np.arange(mine.shape[0]) * 256).all()
         assert mine.shape[0] * 256 >= ncol * nrow > (mine.shape[0] - 1) * 256
+
+
+def test_edge_alias_layout():
+    """with_edge_alias: aliased edges own no slots, the owning edges' blocks are
+    laid out compactly, and every index structure covers exactly those."""
+    from autoparallel_amd import clustering
+    from oracle import cluster_oracle as CO
+
+    g = graphgen.llama_graph((2, 4), 3, 64, 4, 2, 128, 256, 32, 8)
+    groups = clustering.identical_regions(g, CO.node_hashes(g, g.node_phase))
+    root = clustering.cluster_roots(g, groups).astype(np.int64)
+    first = g.node_edge_off[:-1].astype(np.int64)
+    v = g.edge_node.astype(np.int64)
+    alias = first[root[v]] + (np.arange(g.num_edges) - first[v])
+    ga = g.with_edge_alias(alias)
+    ga.validate()
+    own = ga.priced
+    assert own.sum() < g.num_edges and (own == (root[v] == v)).all()
+    sizes = g.edge_sdst.astype(np.int64) * g.edge_ssrc
+    assert ga.num_entries == int(sizes[own].sum()) and ga.num_slots == int(((sizes[own] + 15) & ~15).sum())
+    assert (ga.edge_off[:-1][~own] == ga.edge_off[:-1][alias[~own]]).all()
+    slots, keys = ga.entry_slots(), ga.entry_keys()
+    assert slots.shape[0] == keys.shape[0] == ga.num_entries and len(np.unique(slots)) == ga.num_entries
+    assert (root[keys[:, 0]] == keys[:, 0]).all()  # keys of owning nodes only
+    eid = np.repeat(np.arange(g.num_edges), ga.block_sizes())
+    assert (ga.chunk_edge_index()[slots >> 4] == eid).all()
+    items = ga.work_items()
+    assert items.shape[0] == int(((sizes[own] + 255) // 256).sum())
+    assert set(items["off"].tolist()) == set(ga.edge_off[:-1][own].tolist())
+    base, stride = ga.export_rows()
+    rows = base[eid] + keys[:, 2] * stride[eid] + keys[:, 3]
+    assert np.array_equal(np.sort(rows), np.arange(ga.num_entries))
+    assert np.array_equal(np.argsort(rows), ga.decision_var_order())
+    # edge records: an aliased edge points at its alias's block and matrix
+    rec = ga.edge_records()
+    assert (rec["off"][~own] == rec["off"][alias[~own]]).all()
+    assert (rec["table_off"][~own] == rec["table_off"][alias[~own]]).all()
+    # the oracle over the aliased graph writes each owning block once and the same
+    # values again for its aliases: equal to the owning blocks of the plain build
+    a, b = O.GraphOracle(ga).build(), O.GraphOracle(g).build()
+    assert np.array_equal(a["comm"][slots], b["comm"][g.entry_slots()[np.repeat(own, sizes)]])
+    # an alias between edges with different strategies is refused
+    bad = np.arange(g.num_edges)
+    x = int(np.nonzero(g.edge_ssrc != g.edge_ssrc[0])[0][0])
+    bad[x] = 0
+    with pytest.raises(AssertionError):
+        g.with_edge_alias(bad)

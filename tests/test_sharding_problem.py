@@ -341,12 +341,14 @@ def _rows_one_at_a_time(opt):
 def test_block_rows_equal_the_loops(tiny, clustered):
     g, coef, _ = tiny
     root = None
-    if clustered:  # link every third node to an earlier node of the same shape
+    if clustered:  # link every other node to an earlier node with the same strategies on every edge
         root, first = np.arange(g.num_nodes), {}
         for v in range(g.num_nodes):
             e0, e1 = int(g.node_edge_off[v]), int(g.node_edge_off[v + 1])
-            key = (int(g.node_nstrat[v]), tuple(g.edge_ssrc[e0:e1].tolist()), tuple(g.edge_sdst[e0:e1].tolist()))
-            if key in first and v % 3 == 0:
+            key = (int(g.node_nstrat[v]), tuple(g.edge_ssrc[e0:e1].tolist()),
+                   tuple(g.edge_dst_list[e0:e1].tolist()), tuple(g.edge_src_list[e0:e1].tolist()),
+                   tuple(g.edge_default_off[e0:e1].tolist() if (g.edge_default_off[e0:e1] < 0).all() else [v]))
+            if key in first and v % 2 == 0:
                 root[v] = first[key]
             first.setdefault(key, v)
         assert (root != np.arange(g.num_nodes)).sum() > 5
