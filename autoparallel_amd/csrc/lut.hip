@@ -1,0 +1,245 @@
+// Redistribution costs of whole matrices through a per-source lookup table in
+// LDS: the block table of large problems, and the direct evaluation of entries
+// when no block table applies (gfx950 / CDNA4).
+//
+// A redistribution cost is a walk over the mesh dims that adds, per dim whose
+// placement changes, one collective and up to two read/write times, all of them
+// functions of the bytes in flight at that step.  For a fixed source spec the
+// bytes at step s take at most 2^s values: every earlier step either left them
+// alone or, if the source is sharded (partial) there and the target replicated
+// (sharded), multiplied (divided) them by that dim's size.  So the terms depend
+// on the source spec, the step and which earlier steps changed the bytes, not on
+// the target: a workgroup owns a tile of one matrix (up to 64 source columns, a
+// chunk of target rows), computes those terms once per source column into LDS
+// with the cost model's own functions, and an element is then the reference's
+// additions in the reference's order over looked-up terms: bit-identical to the
+// per-element fold, at a fraction of its arithmetic.
+#include "apc_device.h"
+
+namespace {
+
+constexpr int kLutCols = 64;                     // source columns per tile
+constexpr int kLutStates = (1 << APC_MAX_MESH_DIMS) - 1;  // (step, changed-mask) pairs
+constexpr int kLutStride = kLutStates * 4 + 2;   // doubles per column: 16-byte aligned, and not a multiple of the 32 banks
+constexpr int kLutRows = 1024;                   // target rows per tile
+static_assert(sizeof(apc_lut_tile) == 64, "tile record layout");
+
+struct Terms {  // of one (source column, step, mask)
+  double coll_a;  // Shard -> Replicate: allgather of the gathered bytes; Partial -> Replicate: allreduce
+  double rw_a;    // read/write time of the gathered bytes (S(d != 0) -> R)
+  double coll_b;  // Shard -> Shard: all_to_all; Partial -> Shard: reduce_scatter
+  double rw_b;    // read/write time of the bytes as they are (non-contiguous source, reshuffles)
+};
+
+__device__ __forceinline__ int step_dim(const apc_model& m, int step) {
+  return m.order_mode == 2 ? m.ndim - 1 - step : step;
+}
+
+// The walk of redistribute_cost (apc_device.h) over looked-up terms.  `lut`: the
+// source column's terms, 4 doubles per state, state (step, mask) at
+// (1 << step) - 1 + mask.  Branch-free: every step reads its four terms and adds
+// three values, each either the term the reference adds at that point or +0.0
+// (which leaves a non-negative sum as it is, bit for bit); the lanes of a
+// wavefront hold unrelated pairs, so branches would only serialise them.
+template <int kNdim>
+__device__ __forceinline__ double walk_lut(const double* __restrict__ lut, uint32_t src, uint32_t tgt,
+                                           bool contiguous, bool reversed) {
+  double cost = 0.0;
+  bool forbidden = false;
+  uint32_t mask = 0;
+#pragma unroll
+  for (int step = 0; step < kNdim; ++step) {
+    const int i = reversed ? kNdim - 1 - step : step;
+    const int cur = (src >> (8 * i)) & 0xFF, tg = (tgt >> (8 * i)) & 0xFF;
+    const bool active = cur != tg;
+    const double2_t* q = reinterpret_cast<const double2_t*>(lut + (((1u << step) - 1u + mask) << 2));
+    const double2_t qa = q[0], qb = q[1];  // coll_a, rw_a | coll_b, rw_b
+    const int ck = cur & kKindMask, tk = tg & kKindMask;
+    const bool s_r = active && ck == kShard && tg == 0;
+    const bool s_s = active && ck == kShard && tk == kShard;
+    const bool p_r = active && ck == kPartial && tg == 0;
+    const bool p_s = active && ck == kPartial && tk == kShard;
+    forbidden |= active && ((ck == kShard && tk == kPartial) || (cur == 0 && tk == kPartial));
+    const double pre = (active && !contiguous) ? qb.y : 0.0;
+    const double coll = (s_r | p_r) ? qa.x : ((s_s | p_s) ? qb.x : 0.0);
+    const bool cur_off0 = (cur & kArgMask) != 0, tg_off0 = (tg & kArgMask) != 0;
+    const double copies = (double)((int)cur_off0 + (int)tg_off0);
+    const double rw = s_r ? (cur_off0 ? qa.y : 0.0) : s_s ? copies * qb.y : ((p_s && tg_off0) ? qb.y : 0.0);
+    cost = ((cost + pre) + coll) + rw;
+    if (s_r | p_s) mask |= 1u << step;
+    contiguous |= active;
+  }
+  return forbidden ? INFINITY : cost;
+}
+
+template <bool kEntries, int kNdim>
+__global__ void __launch_bounds__(256)
+lut_kernel(apc_problem p, const apc_lut_tile* __restrict__ tiles, double* __restrict__ table,
+           const double* __restrict__ per_arg, double* __restrict__ comm, double* __restrict__ cost,
+           uint8_t* __restrict__ flags, int clamp_inf) {
+  __shared__ __align__(16) double s_lut[kLutCols * kLutStride];
+  __shared__ apc_spec_rec s_src[kLutCols];
+  __shared__ uint2 s_tgt[kLutRows];  // per target row of the tile: spec word, placement bytes
+  const apc_lut_tile t = tiles[blockIdx.x];  // the same for the whole workgroup: scalar registers
+  const int tid = threadIdx.x;
+  const apc_model& m = p.model;
+  constexpr int ndim = kNdim;  // == m.ndim: the launcher picks the instance
+  constexpr int nstate = (1 << ndim) - 1;
+  const bool reversed = m.order_mode == 2;
+  const bool has_producer = (t.flags & APC_EDGE_HAS_PRODUCER) != 0;
+  const bool squeezed = (t.flags & APC_EDGE_COMPRESSED) != 0;
+  // 1. the tile's source columns
+  if (tid < (int)t.ncols) {
+    apc_spec_rec r = {APC_SPEC_NONE, 0u, 0};
+    if (has_producer) {
+      uint32_t j = t.col0 + (uint32_t)tid;
+      if (squeezed) j = (uint32_t)p.list_ufirst[(size_t)t.src_list + j];
+      r = p.spec_recs[(size_t)t.src_list + j];
+    }
+    s_src[tid] = r;
+  }
+  // ... and its target rows
+  for (uint32_t rr = tid; rr < t.nrows; rr += 256) {
+    uint2 w = make_uint2(APC_SPEC_NONE, 0u);
+    if (has_producer) {
+      uint32_t o = t.row0 + rr;
+      if (squeezed) o = (uint32_t)p.list_ufirst[(size_t)t.dst_list + o];
+      const apc_spec_rec rt = p.spec_recs[(size_t)t.dst_list + o];
+      w = make_uint2(rt.word, rt.plc);
+    }
+    s_tgt[rr] = w;
+  }
+  __syncthreads();
+  // 2. their terms: one task per (column, step, mask)
+  if (has_producer) {
+    for (int task = tid; task < (int)t.ncols * nstate; task += 256) {
+      const int c = task / nstate, st = task - c * nstate;
+      const apc_spec_rec r = s_src[c];
+      const uint32_t src = r.plc;
+      if (r.word == APC_SPEC_NONE || src == 0u) continue;  // no walk from a missing or fully replicated source
+      const int step = 31 - __clz(st + 1);
+      const uint32_t mask = (uint32_t)(st + 1) - (1u << step);
+      int64_t num_shards = 1;
+      for (int i = 0; i < ndim; ++i)
+        if (((src >> (8 * i)) & kKindMask) == kShard) num_shards *= m.mesh_shape[i];
+      double gb = div_int((double)(r.nbytes2 >> 1), num_shards) / 1024.0 / 1024.0 / 1024.0;
+      bool reachable = true;  // a step changes the bytes only from a Shard or a Partial
+      for (int k = 0; k < step; ++k) {
+        if (!((mask >> k) & 1)) continue;
+        const int i = step_dim(m, k);
+        const int ck = (src >> (8 * i)) & kKindMask;
+        if (ck == kShard) gb = gb * (double)m.mesh_shape[i];
+        else if (ck == kPartial) gb = div_int(gb, m.mesh_shape[i]);
+        else reachable = false;
+      }
+      if (!reachable) continue;
+      const int i = step_dim(m, step);
+      const int ck = (src >> (8 * i)) & kKindMask;
+      Terms q = {0.0, 0.0, 0.0, 0.0};
+      q.rw_b = rw_time(gb * 2.0 * 1073741824.0, m.gmem_bw);
+      if (ck == kShard) {
+        const double gathered = gb * (double)m.mesh_shape[i];
+        q.coll_a = collective_cost(0, (int64_t)(gathered * 1073741824.0), i, m);
+        q.rw_a = rw_time(gathered * 2.0 * 1073741824.0, m.gmem_bw);
+        q.coll_b = collective_cost(1, (int64_t)(gb * 1073741824.0), i, m);
+      } else if (ck == kPartial) {
+        q.coll_a = collective_cost(2, (int64_t)(gb * 1073741824.0), i, m);
+        q.coll_b = collective_cost(3, (int64_t)(gb * 1073741824.0), i, m);
+      }
+      double* out = s_lut + c * kLutStride + st * 4;
+      out[0] = q.coll_a; out[1] = q.rw_a; out[2] = q.coll_b; out[3] = q.rw_b;
+    }
+  }
+  __syncthreads();
+  // 3. the tile's elements, row-major: consecutive lanes write consecutive elements
+  const uint32_t total = t.nrows * t.ncols;
+  const bool pp_rule = m.order_mode == 0 && ndim == 2;  // (Partial, Partial) -> all-Shard walks the dims backwards
+  for (uint32_t idx = tid; idx < total; idx += 256) {
+    const uint32_t rr = t.magic ? __umulhi(idx, t.magic) : idx, c = idx - rr * t.ncols;
+    const uint32_t o = t.row0 + rr, j = t.col0 + c;
+    const int64_t at = (int64_t)o * t.ncol + j;  // element of the matrix
+    const apc_spec_rec rs = s_src[c];
+    double value;
+    int trans = 0;
+    bool from_specs = false;
+    if (has_producer) {
+      const uint2 rt = s_tgt[rr];  // x: word, y: placement bytes
+      if (rs.word != APC_SPEC_NONE && rt.x != APC_SPEC_NONE) {
+        from_specs = true;
+        trans = (rs.word & kTupleMask) != (rt.x & kTupleMask);
+        const uint32_t src = rs.plc, tgt = rt.y;
+        const bool contig = (rs.nbytes2 & 1) != 0;
+        if (src == 0u) {
+          bool any_partial = false;
+          for (int i = 0; i < ndim; ++i) any_partial |= (((tgt >> (8 * i)) & kKindMask) == kPartial);
+          value = any_partial ? INFINITY : 0.0;
+        } else if (pp_rule && src == (uint32_t)(kPartialSum | (kPartialSum << 8)) &&
+                   (tgt & kKindMask) == kShard && ((tgt >> 8) & kKindMask) == kShard) {
+          value = redistribute_cost(src, tgt, rs.nbytes2 >> 1, contig, m);  // the one pair with its own order
+        } else {
+          value = walk_lut<kNdim>(s_lut + c * kLutStride, src, tgt, contig, reversed);
+        }
+      }
+    }
+    if (!from_specs) value = p.default_vals[t.default_off + at];  // a missing spec keeps the default row's value
+    if (kEntries) {
+      const double pa = per_arg[t.comp_base + (int64_t)o];
+      double total_cost = (value + pa) + (double)trans;  // optimize_sharding.py:544
+      const bool finite = isfinite(total_cost);
+      if (clamp_inf && !finite) total_cost = 10000.0;
+      const int64_t slot = t.out + at;
+      if (comm) comm[slot] = value;
+      if (cost) cost[slot] = total_cost;
+      if (flags) flags[slot] = (uint8_t)(trans | (finite ? 0 : APC_ENTRY_NONFINITE));
+    } else {
+      table[t.out + at] = trans ? -value : value;
+    }
+  }
+}
+
+template <bool kEntries>
+void launch_lut(const apc_problem* p, const apc_lut_tile* tiles, int64_t n_tile, double* table, const double* per_arg,
+                double* comm, double* cost, uint8_t* flags, int clamp_inf, hipStream_t stream) {
+#define APC_LAUNCH_LUT(N)                                                                                      \
+  hipLaunchKernelGGL((lut_kernel<kEntries, N>), dim3((unsigned)n_tile), dim3(256), 0, stream, *p, tiles, table, \
+                     per_arg, comm, cost, flags, clamp_inf)
+  switch (p->model.ndim) {  // validate_problem has checked the range
+    case 1: APC_LAUNCH_LUT(1); break;
+    case 2: APC_LAUNCH_LUT(2); break;
+    case 3: APC_LAUNCH_LUT(3); break;
+    default: APC_LAUNCH_LUT(4); break;
+  }
+#undef APC_LAUNCH_LUT
+}
+
+int check_tiles(const apc_problem* p, const apc_lut_tile* tiles, int64_t n_tile, const char* what) {
+  if (int rc = validate_problem(p)) return rc;
+  if (n_tile < 0 || n_tile > 0x7FFFFFFF || (n_tile > 0 && !tiles)) return fail(APC_ERR_INVALID, "%s: bad tile list", what);
+  if (n_tile > 0 && !p->spec_recs) return fail(APC_ERR_INVALID, "%s: needs apc_problem.spec_recs", what);
+  // (a tile has at most 64 columns and 1024 rows: the host that made the list guarantees it)
+  return 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+int apc_build_pair_table_lut(const apc_problem* p, const apc_lut_tile* tiles, int64_t n_tile, double* table,
+                             void* stream) {
+  if (int rc = check_tiles(p, tiles, n_tile, "apc_build_pair_table_lut")) return rc;
+  if (n_tile == 0) return 0;
+  if (!table) return fail(APC_ERR_INVALID, "apc_build_pair_table_lut: null table%s");
+  launch_lut<false>(p, tiles, n_tile, table, nullptr, nullptr, nullptr, nullptr, 0, (hipStream_t)stream);
+  return check_launch("lut_kernel<table>");
+}
+
+int apc_edge_costs_lut(const apc_problem* p, const apc_lut_tile* tiles, int64_t n_tile, const double* per_arg,
+                       double* comm, double* cost, uint8_t* flags, int32_t clamp_inf, void* stream) {
+  if (int rc = check_tiles(p, tiles, n_tile, "apc_edge_costs_lut")) return rc;
+  if (n_tile == 0) return 0;
+  if (!per_arg) return fail(APC_ERR_INVALID, "apc_edge_costs_lut: null per_arg%s");
+  launch_lut<true>(p, tiles, n_tile, nullptr, per_arg, comm, cost, flags, clamp_inf, (hipStream_t)stream);
+  return check_launch("lut_kernel<entries>");
+}
+
+}  // extern "C"

@@ -19,6 +19,7 @@ _TABLE_MAX_DOUBLES = 1 << 28
 _WIDE_ITEMS_FROM = 32_000_000  # entries
 _PACKED_SCORING_FROM = 8192  # mean entries per edge block
 _SCORE_LANES_FROM = 32768  # assignments: below, one wavefront per assignment (entry arrays as they are)
+_LUT_TABLE_FROM = 2048  # table units: larger tables are built tile by tile with per-source terms in LDS
 
 
 def xgmi_config_struct(cfg) -> _lib.ApcXgmiConfig:
@@ -135,6 +136,7 @@ class CostEngine:
         item_entries: Optional[int] = None,
         topo_config=None,
         allocate_results: bool = True,
+        lut: Optional[bool] = None,
     ):
         """``table_mode``: "full" (one S_dst x S_src matrix per distinct pair of
         runs), "compressed" (matrices by distinct spec word, read by gather),
@@ -143,7 +145,9 @@ class CostEngine:
         an XGMITopoConfig for the alpha-beta constants (make_model).
         ``allocate_results=False``: only the problem is uploaded (for the node
         hashes, which are taken before it is decided which edges get entries);
-        such an engine cannot build.  ``use_table`` is
+        such an engine cannot build.  ``lut``: build the block table (or, without
+        one, the entries) with the lookup-table kernels; None: for tables of
+        more than 2 048 units and for direct evaluation.  ``use_table`` is
         the older switch: True = "full", False = "direct".  ``item_entries``:
         entries per work item of the entry kernel, 256 or 512 (512 needs a
         table); None: by problem size."""
@@ -271,6 +275,13 @@ class CostEngine:
         p.table_unit_block = up("table_unit_block", unit_block)
         p.table_units = up("table_units", g.table_unit_records(squeezed))
         self.problem = p
+        # Large tables, and direct evaluation, go through the lookup-table kernels:
+        # tiles of whole matrices instead of one element per lane.
+        self._lut_tiles = None
+        self.lut = lut if lut is not None else (table_mode == "direct" or p.n_table_unit > _LUT_TABLE_FROM)
+        if self.lut and g.num_entries > 0:
+            tiles = g.lut_tiles(squeezed, entries=(table_mode == "direct"))
+            self._lut_tiles = (up("lut_tiles", tiles), int(tiles.shape[0]))
 
         E, NC = (g.num_slots, g.num_compute) if allocate_results else (0, 0)
         self.can_build = bool(allocate_results)
@@ -370,12 +381,30 @@ class CostEngine:
         # the argument list is the same from call to call apart from the stream:
         # made once, so that issuing a step costs less host time than the step takes
         args = self._build_args or self.build_args()
-        rc = self.lib.apc_build_all(*args, 1 if clamp_inf else 0,
-                                    torch.cuda.current_stream(self.device).cuda_stream)
-        if rc:
-            _lib.check(rc, "apc_build_all")
+        stream = torch.cuda.current_stream(self.device).cuda_stream
+        if self._lut_tiles is None:
+            rc = self.lib.apc_build_all(*args, 1 if clamp_inf else 0, stream)
+            if rc:
+                _lib.check(rc, "apc_build_all")
+        else:
+            self._build_with_lut(1 if clamp_inf else 0, stream)
         self.built = True
         return self
+
+    def _build_with_lut(self, clamp_inf: int, stream) -> None:
+        """The same results through the lookup-table kernels: the block table tile
+        by tile, then the usual node and entry launches; or, without a table, the
+        entries themselves tile by tile."""
+        p, table, compute, per_arg, status, comm, cost, flags = self.build_args()
+        tiles, n_tile = self._lut_tiles
+        lib = self.lib
+        _lib.check(lib.apc_node_compute_costs(p, compute, per_arg, status, stream), "apc_node_compute_costs")
+        if self.use_table:
+            _lib.check(lib.apc_build_pair_table_lut(p, tiles, n_tile, table, stream), "apc_build_pair_table_lut")
+            _lib.check(lib.apc_edge_costs(p, table, per_arg, comm, cost, flags, clamp_inf, stream), "apc_edge_costs")
+        else:
+            _lib.check(lib.apc_edge_costs_lut(p, tiles, n_tile, per_arg, comm, cost, flags, clamp_inf, stream),
+                       "apc_edge_costs_lut")
 
     def build_timed(self, timer, slot: int, clamp_inf: bool = True):
         """build() with HIP events at the begin and end of the entry kernel (a

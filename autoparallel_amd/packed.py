@@ -521,6 +521,62 @@ class PackedGraph:
         rec["nbytes2"][some] = (nbytes[w >> TUPLE_BITS] << 1) | contig[w >> TUPLE_BITS]
         return rec
 
+    LUT_TILE_DTYPE = np.dtype([
+        ("out", "<i8"), ("default_off", "<i8"), ("src_list", "<u4"), ("dst_list", "<u4"), ("ncol", "<u4"),
+        ("nrow", "<u4"), ("col0", "<u4"), ("ncols", "<u4"), ("row0", "<u4"), ("nrows", "<u4"), ("flags", "<u4"),
+        ("comp_base", "<i4"), ("magic", "<u4"), ("reserved", "<u4"),
+    ])
+    LUT_COLS = 64
+    LUT_ROWS = 1024
+    LUT_TILE_ELEMENTS = 16384
+
+    def lut_tiles(self, compressed: bool = False, entries: bool = False) -> np.ndarray:
+        """Tiles (``apc_lut_tile`` of include/apc.h) for the lookup-table kernels:
+        of every matrix of the block table (``entries=False``; ``compressed`` as
+        for block_table), or of every edge block that owns entries
+        (``entries=True``: direct evaluation, edges without a producer included).
+        A tile has at most LUT_COLS source columns and about LUT_TILE_ELEMENTS
+        elements."""
+        if entries:
+            e = np.nonzero(self.priced & (self.block_sizes() > 0))[0].astype(np.int64)
+            ncol, nrow = self.edge_ssrc[e].astype(np.int64), self.edge_sdst[e].astype(np.int64)
+            out = self.edge_off[:-1][e]
+            flags = (self.edge_flags[e] & EDGE_HAS_PRODUCER).astype(np.int64)
+            comp_base = self.node_comp_off[self.edge_node[e]].astype(np.int64)
+        else:
+            block_edge, block_off, _, _, edge_usrc, block_udst = self.block_table(compressed)
+            e = block_edge.astype(np.int64)
+            squeezed = edge_usrc[e] > 0
+            ncol = np.where(squeezed, edge_usrc[e], self.edge_ssrc[e]).astype(np.int64)
+            nrow = np.where(squeezed, block_udst, self.edge_sdst[e]).astype(np.int64)
+            out = block_off[:-1]
+            flags = EDGE_HAS_PRODUCER | np.where(squeezed, EDGE_COMPRESSED, 0).astype(np.int64)
+            comp_base = np.full(e.shape[0], -1, np.int64)
+        n_ct = (ncol + self.LUT_COLS - 1) // self.LUT_COLS
+        rows_per = np.minimum(np.minimum(nrow, self.LUT_ROWS),
+                              np.maximum(1, self.LUT_TILE_ELEMENTS // np.minimum(ncol, self.LUT_COLS)))
+        n_rt = (nrow + rows_per - 1) // np.maximum(rows_per, 1)
+        per = n_ct * n_rt
+        k = np.repeat(np.arange(e.shape[0], dtype=np.int64), per)
+        start = np.concatenate([[0], np.cumsum(per)[:-1]]) if e.shape[0] else np.zeros(0, np.int64)
+        local = np.arange(int(per.sum()), dtype=np.int64) - start[k]
+        ct, rt = local % n_ct[k], local // n_ct[k]
+        rec = np.zeros(k.shape[0], self.LUT_TILE_DTYPE)
+        assert rec.dtype.itemsize == 64
+        rec["out"], rec["default_off"] = out[k], self.edge_default_off[e[k]]
+        rec["src_list"] = np.maximum(self.edge_src_list[e[k]], 0).astype(np.uint32)
+        rec["dst_list"] = self.edge_dst_list[e[k]].astype(np.uint32)
+        rec["ncol"], rec["nrow"] = ncol[k], nrow[k]
+        rec["col0"] = ct * self.LUT_COLS
+        rec["ncols"] = np.minimum(self.LUT_COLS, ncol[k] - ct * self.LUT_COLS)
+        rec["row0"] = rt * rows_per[k]
+        rec["nrows"] = np.minimum(rows_per[k], nrow[k] - rt * rows_per[k])
+        rec["flags"], rec["comp_base"] = flags[k], comp_base[k]
+        nc = rec["ncols"].astype(np.int64)
+        rec["magic"] = np.where(nc > 1, (2**32) // np.maximum(nc, 1) + 1, 0)  # one column: the row is the index
+        assert (rec["nrows"].astype(np.int64) * rec["ncols"] < 2**20).all() and (rec["nrows"] <= self.LUT_ROWS).all()
+        return rec
+
     def table_unit_records(self, compressed: bool = False) -> np.ndarray:
         """One ``apc_table_unit`` per 256 elements of the block table: the two
         runs, the matrix extent and the unit's first element, so that a

@@ -393,6 +393,42 @@ int64_t apc_pair_table_size(const apc_problem* p);
  * _compute_edge_costs (autoparallel/optimize_sharding.py:474-478). */
 int apc_build_pair_table(const apc_problem* p, double* table, void* stream);
 
+/* A tile of one cost matrix for the lookup-table kernels below: columns
+ * [col0, col0 + ncols) (ncols <= 64) and rows [row0, row0 + nrows) (nrows <= 1024) of an
+ * S_dst x S_src matrix (nrow x ncol; of distinct words when APC_EDGE_COMPRESSED),
+ * whose element (o, j) goes to out + o * ncol + j. */
+typedef struct apc_lut_tile {
+  int64_t out;         /* table: first element of the matrix; entries: slot of entry (0, 0) */
+  int64_t default_off; /* default rows of the edge, or -1                       */
+  uint32_t src_list;
+  uint32_t dst_list;
+  uint32_t ncol;
+  uint32_t nrow;
+  uint32_t col0;
+  uint32_t ncols;
+  uint32_t row0;
+  uint32_t nrows;
+  uint32_t flags;      /* APC_EDGE_HAS_PRODUCER | APC_EDGE_COMPRESSED            */
+  int32_t comp_base;   /* entries: index of (node, out_idx 0) in per_arg         */
+  uint32_t magic;      /* floor(2^32 / ncols) + 1: idx / ncols == umulhi(idx, magic) for idx < 2^20;
+                          0 for ncols == 1 */
+  uint32_t reserved;
+} apc_lut_tile; /* 64 bytes */
+
+/* apc_build_pair_table for large tables: the same table, bit for bit, built
+ * tile by tile with the terms of each source spec computed once per tile into
+ * LDS (replaces the same reference functions as apc_build_pair_table).  tiles:
+ * device array covering every matrix of the block table exactly once
+ * (PackedGraph.lut_tiles).  Needs apc_problem.spec_recs. */
+int apc_build_pair_table_lut(const apc_problem* p, const apc_lut_tile* tiles, int64_t n_tile, double* table,
+                             void* stream);
+
+/* apc_edge_costs with table == NULL (direct evaluation), bit for bit, tile by
+ * tile the same way: tiles cover every edge block exactly once, edges without
+ * a producer included (their entries are their default rows). */
+int apc_edge_costs_lut(const apc_problem* p, const apc_lut_tile* tiles, int64_t n_tile, const double* per_arg,
+                       double* comm, double* cost, uint8_t* flags, int32_t clamp_inf, void* stream);
+
 /* Replaces estimate_strategy_runtime_cost
  * (autoparallel/cost_models/compute_estimation.py:438-493, with
  * _get_sharded_shape_stride :300-318 and compute_memory_cost :321-331) for

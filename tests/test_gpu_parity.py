@@ -48,8 +48,9 @@ def _check_build(CE, g, use_table, clamp=False):
 # ---------------------------------------------------------------------------
 # golden vectors of the reference, through the C ABI
 # ---------------------------------------------------------------------------
+@pytest.mark.parametrize("lut", [False, True])
 @pytest.mark.parametrize("use_table", [True, False, "compressed"])
-def test_golden_comm_vectors(CostEngine, golden, use_table):
+def test_golden_comm_vectors(CostEngine, golden, use_table, lut):
     n_cases = int(golden["comm_ncases"][0])
     checked = 0
     for k in range(n_cases):
@@ -63,7 +64,7 @@ def test_golden_comm_vectors(CostEngine, golden, use_table):
         g = graph_from_pairs(mesh, 8, shape, stride, itemsize, src_t, tgt_t)
         print(f"golden case {k}: mesh={mesh} shape={shape} pairs={len(want)}", flush=True)
         kw = dict(table_mode=use_table) if isinstance(use_table, str) else dict(use_table=use_table)
-        eng = CostEngine(g, **kw).build(clamp_inf=False)
+        eng = CostEngine(g, lut=lut, **kw).build(clamp_inf=False)  # lut: per-source terms in LDS, or the fold per element
         comm = eng.results()["comm"]
         e = 1  # the consumer's edge
         base, ssrc = int(g.edge_off[e]), int(g.edge_ssrc[e])
@@ -431,7 +432,7 @@ def test_work_items_of_512_entries(CostEngine, mode):
         assert ((got["flags"] & 1) == ref["transition"]).all()
     from autoparallel_amd import _lib
     with pytest.raises(_lib.ApcError):
-        CostEngine(g, table_mode="direct", item_entries=512).build()
+        CostEngine(g, table_mode="direct", item_entries=512, lut=False).build()
 
 
 @pytest.mark.parametrize("rank,n_args", [(1, 15), (2, 16)])
@@ -465,13 +466,13 @@ def test_problem_without_the_derived_records(CostEngine, mode):
     prepare launch (table units, spec records, product terms, node records): the
     kernels then walk the arrays those were made from.  Same bits either way."""
     g = graphgen.llama_graph((2, 2, 4), 1, 64, 4, 2, 128, 256, 32, 16)
-    eng = CostEngine(g, table_mode=mode).build(clamp_inf=False)
+    eng = CostEngine(g, table_mode=mode, lut=False).build(clamp_inf=False)  # the kernels with one element per lane
     want = eng.results()
     ref = O.GraphOracle(g).build()
     assert bits_equal(want["comm"], ref["comm"]) and bits_equal(want["compute"], ref["compute"])
     for drop in (("table_units",), ("spec_recs",), ("prog_terms", "n_prog_term"),
                  ("comp_recs",), ("table_units", "spec_recs", "prog_terms", "n_prog_term", "comp_recs")):
-        e2 = CostEngine(g, table_mode=mode)
+        e2 = CostEngine(g, table_mode=mode, lut=False)
         for f in drop:
             setattr(e2.problem, f, 0 if f == "n_prog_term" else None)
         got = e2.build(clamp_inf=False).results()
@@ -532,6 +533,32 @@ def test_xgmi_topology_on_the_device(CostEngine, mode):
     finite = np.isfinite(plain["comm"])
     assert (ref["comm"][finite] != plain["comm"][finite]).any()
     assert ((ref["comm"] == 0) == (plain["comm"] == 0)).all() and (np.isfinite(ref["comm"]) == finite).all()
+
+
+@pytest.mark.parametrize("name", ["llama_2d", "llama_3d", "llama_odd_mesh", "moe_tiny", "pairs_4d", "pairs_3d_noncontig",
+                                  "stress_3d"])
+def test_lookup_table_kernels(CostEngine, name):
+    """The tile kernels (terms per source spec in LDS) against the oracle, for the
+    block table in both layouts and for direct evaluation, with the inf clamp on
+    the direct path; and the edge cases graph (missing specs, tuple outputs, default
+    rows, an edge without a producer)."""
+    g = GRAPHS[name]()
+    ref = O.GraphOracle(g).build()
+    for mode in ("full", "compressed", "direct"):
+        eng = CostEngine(g, table_mode=mode, lut=True)
+        assert eng._lut_tiles is not None
+        got = eng.build(clamp_inf=False).results()
+        assert bits_equal(got["comm"], ref["comm"]), (mode, first_mismatch(got["comm"], ref["comm"]))
+        assert bits_equal(got["cost"], ref["cost"]), mode
+        assert ((got["flags"] & 1) == ref["transition"]).all() and bits_equal(got["compute"], ref["compute"])
+    clamped = CostEngine(g, table_mode="direct", lut=True).build(clamp_inf=True).results()
+    assert bits_equal(clamped["cost"], O.clamp_inf(ref["cost"])[0])
+    ge = _edge_case_graph()
+    re_ = O.GraphOracle(ge).build()
+    for mode in ("full", "compressed", "direct"):
+        got = CostEngine(ge, table_mode=mode, lut=True).build(clamp_inf=False).results()
+        assert bits_equal(got["comm"], re_["comm"]) and bits_equal(got["cost"], re_["cost"]), mode
+        assert ((got["flags"] & 1) == re_["transition"]).all()
 
 
 def test_unsupported_dtype_reports(CostEngine):
@@ -657,12 +684,13 @@ def test_seeded_graphs_on_many_meshes_every_layout(CostEngine, seed):
     g = graphgen.stress_graph([120, 300, 700][seed % 3], meshes[seed % len(meshes)], seed=1000 + seed, s_min=2,
                               s_max=[40, 120, 260][(seed // 3) % 3])
     want = c_oracle.COracle(g).build(threads=16)
-    for mode, items in (("direct", 256), ("full", 256), ("full", 512), ("compressed", 256), ("compressed", 512)):
-        got = CostEngine(g, table_mode=mode, item_entries=items).build(clamp_inf=False).results()
-        assert bits_equal(got["comm"], want["comm"]), (mode, items, first_mismatch(got["comm"], want["comm"]))
-        assert bits_equal(got["cost"], want["cost"]), (mode, items)
-        assert bits_equal(got["compute"], want["compute"]), (mode, items)
-        assert ((got["flags"] & 1) == want["transition"]).all(), (mode, items)
+    for mode, items, lut in (("direct", 256, False), ("direct", 256, True), ("full", 256, False), ("full", 512, True),
+                             ("compressed", 256, True), ("compressed", 512, False)):
+        got = CostEngine(g, table_mode=mode, item_entries=items, lut=lut).build(clamp_inf=False).results()
+        assert bits_equal(got["comm"], want["comm"]), (mode, items, lut, first_mismatch(got["comm"], want["comm"]))
+        assert bits_equal(got["cost"], want["cost"]), (mode, items, lut)
+        assert bits_equal(got["compute"], want["compute"]), (mode, items, lut)
+        assert ((got["flags"] & 1) == want["transition"]).all(), (mode, items, lut)
 
 
 # ---------------------------------------------------------------------------
