@@ -214,6 +214,415 @@ score_packed_kernel(apc_problem p, const double* __restrict__ per_arg,
   r[5] = forbidden;
 }
 
+// ---------------------------------------------------------------------------
+// Compact records and the walk over them: what scoring falls back to on a graph
+// with large blocks when it cannot read the block table (no table, or entry
+// arrays that something changed after the build).
+//
+// A drawn entry is one random read inside its edge's block, and the walk runs at
+// the rate at which a CU has cache misses served, wherever the line comes from
+// (measured: with the blocks kept in L2, 93% hits instead of 27%, the same time).
+// What helps is fewer and better used requests:
+//   - the record is {comm, flags}, 16 bytes: the cost of an entry is (comm +
+//     per_arg) + transition, clamped or not, and the lane holds per_arg of its
+//     node's choice already, so cost need not be stored;
+//   - a lane carries kPer assignments, whose reads of an edge are independent and
+//     issued back to back, and the whole batch walks the graph once.
+// Measured on a 3000-node window of the stress DAG, 2^20 assignments: 99 ms from
+// 32-byte records in launches of 2^18 lanes, 70-80 ms here with kPer = 8.
+// The sums of an assignment run in node order, then argument order, as in
+// score_kernel: same results, bit for bit.
+// ---------------------------------------------------------------------------
+
+// One lane per slot.  mismatch[0] is set if some cost is neither (comm + per_arg)
+// + transition nor that sum's clamp: then the compact records cannot stand for
+// the arrays and the caller must not use them.
+__global__ void __launch_bounds__(kBlock)
+score_pack16_kernel(apc_problem p, const double* __restrict__ per_arg, const double* __restrict__ comm,
+                    const double* __restrict__ cost, const uint8_t* __restrict__ flags,
+                    apc_score_rec16* __restrict__ recs, int32_t* __restrict__ mismatch) {
+  const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (i >= p.n_slot) return;
+  const apc_edge* ed = p.edges + p.chunk_edge[i >> 4];
+  const int64_t l = i - ed->off;
+  const int ssrc = ed->ssrc;
+  apc_score_rec16 r;
+  r.comm = 0.0;
+  r.flags = 0;
+  if (l < (int64_t)ssrc * ed->sdst) {  // else padding behind the block
+    const uint32_t o = (uint32_t)l / (uint32_t)ssrc;
+    const double cm = comm[i], c = cost[i];
+    const uint32_t f = flags[i];
+    const double want = (cm + per_arg[ed->comp_base + o]) + (double)(int)(f & APC_ENTRY_TRANSITION);
+    bool bad = ((f & APC_ENTRY_NONFINITE) != 0) != !isfinite(want);
+    uint64_t extra = 0;
+    if (__double_as_longlong(c) != __double_as_longlong(want)) {
+      if (c == 10000.0 && !isfinite(want)) extra = APC_SCORE_CLAMPED;
+      else bad = true;
+    }
+    if (bad) atomicOr(mismatch, 1);
+    r.comm = cm;
+    r.flags = (uint64_t)f | extra;
+  }
+  recs[i] = r;
+}
+
+__global__ void clear_flag_kernel(int32_t* flag) { *flag = 0; }
+
+template <bool kRandom, int kPer>
+__global__ void __launch_bounds__(kBlock)
+score_compact_kernel(apc_problem p, const double* __restrict__ per_arg,
+                     const apc_score_rec16* __restrict__ recs, const uint16_t* __restrict__ assign,
+                     int64_t stride, uint64_t seed, int64_t first, int64_t n_assign,
+                     const int32_t* __restrict__ node_gid, int first_node, int end_node,
+                     const double* __restrict__ init, double* __restrict__ out) {
+  const int64_t lanes = (int64_t)gridDim.x * blockDim.x;
+  const int64_t t_raw = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (t_raw >= n_assign) return;
+  const int64_t t = t_raw;
+  // assignment k of this lane; a lane past the end repeats another one and stores nothing
+  auto asg = [&](int k) -> int64_t {
+    const int64_t ak = t_raw + k * lanes;
+    return ak < n_assign ? ak : t;
+  };
+  double t_compute[kPer], t_comm[kPer], t_trans[kPer], obj[kPer], forbidden[kPer];
+  uint32_t h0[kPer];
+#pragma unroll
+  for (int k = 0; k < kPer; ++k) {
+    t_compute[k] = 0.0; t_comm[k] = 0.0; t_trans[k] = 0.0; obj[k] = 0.0; forbidden[k] = 0.0;
+    if (init) {
+      const double* r = init + asg(k) * 6;
+      t_compute[k] = r[1]; t_comm[k] = r[2]; t_trans[k] = r[3]; obj[k] = r[4]; forbidden[k] = r[5];
+    }
+    // the part of mix_assignment that does not depend on the node
+    const uint64_t ua = (uint64_t)(first + asg(k));
+    uint32_t h = (uint32_t)seed ^ ((uint32_t)(seed >> 32) * 0x27D4EB2Fu);
+    h ^= (uint32_t)ua * 0x9E3779B1u;
+    h ^= (uint32_t)(ua >> 32) * 0x85EBCA77u;
+    h0[k] = h;
+  }
+  auto choice = [&](int k, int v, int nstrat) -> uint32_t {
+    if (!kRandom) return (uint32_t)assign[(size_t)v * stride + asg(k)];
+    uint32_t h = h0[k] ^ ((uint32_t)((node_gid ? node_gid[v] : v) + 1) * 0xC2B2AE3Du);
+    h ^= h >> 16;
+    h *= 0x85EBCA6Bu;
+    h ^= h >> 13;
+    h *= 0xC2B2AE35u;
+    h ^= h >> 16;
+    return (uint32_t)(((uint64_t)h * (uint64_t)(uint32_t)nstrat) >> 32);
+  };
+  apc_edge nxt;
+  if (first_node < p.n_node && p.node_edge_off[first_node] < p.n_edge)
+    nxt = load_edge(p.edges + p.node_edge_off[first_node]);
+  for (int v = first_node; v < end_node; ++v) {
+    const int nstrat = p.node_nstrat[v];
+    const int nargs = p.node_nargs[v];
+    const double fargs = (double)(nargs > 1 ? nargs : 1);
+    const double mult = (double)p.node_multiplier[v];
+    const int64_t comp_off = p.node_comp_off[v];
+    uint32_t o[kPer];
+    double pa[kPer];
+#pragma unroll
+    for (int k = 0; k < kPer; ++k) {
+      o[k] = choice(k, v, nstrat);
+      pa[k] = per_arg[comp_off + o[k]];
+    }
+#pragma unroll
+    for (int k = 0; k < kPer; ++k) t_compute[k] += pa[k] * fargs;
+    for (int e = p.node_edge_off[v]; e < p.node_edge_off[v + 1]; ++e) {
+      const apc_edge ed = nxt;
+      if (e + 1 < p.n_edge) nxt = load_edge(p.edges + e + 1);
+      const bool has_src = ed.src_node >= 0;
+      apc_score_rec16 r[kPer];
+#pragma unroll
+      for (int k = 0; k < kPer; ++k) {
+        const uint32_t j = has_src ? choice(k, ed.src_node, ed.ssrc) : 0u;  // ssrc: the producer's count
+        r[k] = recs[ed.off + (int64_t)o[k] * ed.ssrc + j];
+      }
+      const bool count_trans = has_src && (ed.flags & APC_EDGE_SCORE_TRANSITION);
+#pragma unroll
+      for (int k = 0; k < kPer; ++k) {
+        const uint32_t f = (uint32_t)r[k].flags;
+        double c = (r[k].comm + pa[k]) + (double)(int)(f & APC_ENTRY_TRANSITION);
+        if (f & (uint32_t)APC_SCORE_CLAMPED) c = 10000.0;
+        obj[k] += c * mult;
+        forbidden[k] += (double)((f & APC_ENTRY_NONFINITE) != 0);
+        if (has_src && isfinite(r[k].comm)) t_comm[k] += r[k].comm;
+        if (count_trans && (f & APC_ENTRY_TRANSITION)) t_trans[k] += 1.0;
+      }
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < kPer; ++k) {
+    if (t_raw + k * lanes >= n_assign) continue;
+    double* r = out + asg(k) * 6;
+    r[0] = (t_compute[k] + t_comm[k]) + t_trans[k];
+    r[1] = t_compute[k];
+    r[2] = t_comm[k];
+    r[3] = t_trans[k];
+    r[4] = obj[k];
+    r[5] = forbidden[k];
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Scoring from the block table, for graphs whose blocks are large.
+//
+// A drawn entry of a block of 10^5 entries is a random read that misses the
+// CU's cache, and the walk over such records runs at the rate at which a CU
+// can have misses served (measured: one per 8 cycles per CU whether the line
+// comes from L2 or from memory; 7e10 draws/s on the whole chip).  The block
+// table holds the same numbers in far less room: an edge's matrix has one row
+// per distinct consumer spec word and one column per distinct producer spec
+// word (8 times fewer elements than the blocks on the stress DAG, 63 KB a
+// matrix on average), and an entry is (|m| + per_arg) + transition with the
+// transition flag in m's sign, clamped or not: what the build makes of it
+// (item_store in apc.hip).  So one workgroup per CU, 1024 lanes with kPer
+// assignments each, has the matrix of the current edge in LDS and draws from
+// there.  The matrix comes in by loads that write LDS directly
+// (global_load_lds: no registers in between), into one of two buffers: the
+// loads of the next edge's matrix are issued before the draws of the current
+// one.  Matrices larger than a buffer are taken in several tiles; very large
+// ones and the default rows of edges without a producer are read in place.
+// The sums of an assignment run in node order, then argument order, as in
+// score_kernel: same results, bit for bit, as scoring the entry arrays that a
+// build with the same clamp_inf wrote.
+// ---------------------------------------------------------------------------
+constexpr int kTableBlock = 1024;
+constexpr int kTileDoubles = 8192;  // 64 KB: four 16-byte loads per lane
+constexpr int kListInts = 1024;     // one 4-byte load per lane
+constexpr int kTableLds = 2 * kTileDoubles * 8 + 4 * kListInts * 4;  // 144 KB
+
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+
+// Lane i's 16 (4) bytes src[i] -> LDS, for the lanes with i < n.  lds_wave is the LDS
+// byte address of the element of the wave's first lane; the hardware adds lane * 16
+// (lane * 4).  The load is written out by hand because the compiler, which cannot
+// tell these LDS writes from the LDS reads of the draws, would wait for it before the
+// next LDS read, and the point is that it stays in flight while the lanes draw from
+// the other buffer.  So the compiler does not count it either: the code that needs
+// the data waits with s_waitcnt vmcnt(0) itself.  (Loads complete in order, so the
+// compiler's own counts for its own loads only ever wait longer than they must.)
+__device__ __forceinline__ void copy16_to_lds(const double2_t* __restrict__ src, uint32_t lds_wave, int i, int n) {
+  if (i < n) {
+    const uint32_t m = __builtin_amdgcn_readfirstlane(lds_wave);
+    const double2_t* g = src + i;
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 3\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(m), "v"(g) : "memory");
+  }
+}
+__device__ __forceinline__ void copy4_to_lds(const int32_t* __restrict__ src, uint32_t lds_wave, int i, int n) {
+  if (i < n) {
+    const uint32_t m = __builtin_amdgcn_readfirstlane(lds_wave);
+    const int32_t* g = src + i;
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 3\n\tglobal_load_lds_dword %1, off" ::"s"(m), "v"(g) : "memory");
+  }
+}
+
+template <bool kRandom, int kPer>
+__global__ void __launch_bounds__(kTableBlock)
+score_table_kernel(apc_problem p, const double* __restrict__ per_arg, const double* __restrict__ table,
+                   const int32_t* __restrict__ edge_msize, const int32_t* __restrict__ next_staged,
+                   const uint16_t* __restrict__ assign, int64_t stride, uint64_t seed, int64_t first,
+                   int64_t n_assign, const int32_t* __restrict__ node_gid, int first_node, int end_node,
+                   int clamp_inf, const double* __restrict__ init, double* __restrict__ out) {
+  extern __shared__ __align__(16) double s_all[];
+  // [2][kTileDoubles] doubles, then [2][2][kListInts] ints
+  int32_t* const s_lists = reinterpret_cast<int32_t*>(s_all + 2 * kTileDoubles);
+  const int tid = threadIdx.x;
+  const int wave0 = tid & ~63;
+  const uint32_t lds_mat = (uint32_t)(uintptr_t)(lds_ptr_t)s_all;  // byte addresses inside LDS
+  const uint32_t lds_lists = lds_mat + 2 * kTileDoubles * 8;
+  const int64_t lanes = (int64_t)gridDim.x * kTableBlock;
+  const int64_t t_raw = (int64_t)blockIdx.x * kTableBlock + tid;
+  const int64_t t = t_raw < n_assign ? t_raw : 0;  // no lane leaves early: the workgroup meets at barriers
+  // assignment k of this lane; a lane past the end repeats another one and stores nothing
+  auto asg = [&](int k) -> int64_t {
+    const int64_t ak = t_raw + k * lanes;
+    return ak < n_assign ? ak : t;
+  };
+  double t_compute[kPer], t_comm[kPer], t_trans[kPer], obj[kPer], forbidden[kPer];
+  uint32_t h0[kPer];
+#pragma unroll
+  for (int k = 0; k < kPer; ++k) {
+    t_compute[k] = 0.0; t_comm[k] = 0.0; t_trans[k] = 0.0; obj[k] = 0.0; forbidden[k] = 0.0;
+    if (init) {
+      const double* r = init + asg(k) * 6;
+      t_compute[k] = r[1]; t_comm[k] = r[2]; t_trans[k] = r[3]; obj[k] = r[4]; forbidden[k] = r[5];
+    }
+    // the part of mix_assignment that does not depend on the node
+    const uint64_t ua = (uint64_t)(first + asg(k));
+    uint32_t h = (uint32_t)seed ^ ((uint32_t)(seed >> 32) * 0x27D4EB2Fu);
+    h ^= (uint32_t)ua * 0x9E3779B1u;
+    h ^= (uint32_t)(ua >> 32) * 0x85EBCA77u;
+    h0[k] = h;
+  }
+  auto choice = [&](int k, int v, int nstrat) -> uint32_t {
+    if (!kRandom) return (uint32_t)assign[(size_t)v * stride + asg(k)];
+    uint32_t h = h0[k] ^ ((uint32_t)((node_gid ? node_gid[v] : v) + 1) * 0xC2B2AE3Du);
+    h ^= h >> 16;
+    h *= 0x85EBCA6Bu;
+    h ^= h >> 13;
+    h *= 0xC2B2AE35u;
+    h ^= h >> 16;
+    return (uint32_t)(((uint64_t)h * (uint64_t)(uint32_t)nstrat) >> 32);
+  };
+  // Whether the two index lists of a compressed matrix go through LDS too.
+  auto lists_staged = [](const apc_edge& x) {
+    return (x.flags & APC_EDGE_COMPRESSED) && x.sdst <= kListInts && x.ssrc <= kListInts;
+  };
+  // The loads of tile `base` of edge x's matrix (and, with its first tile, of its index
+  // lists) into buffer b.  Nothing waits here.
+  auto issue = [&](const apc_edge& x, int msize, int base, int b) {
+    const int n = msize - base < kTileDoubles ? msize - base : kTileDoubles;
+    const double2_t* __restrict__ src2 = reinterpret_cast<const double2_t*>(table + x.table_off + base);
+#pragma unroll
+    for (int r = 0; r < kTileDoubles / 2 / kTableBlock; ++r)
+      copy16_to_lds(src2, lds_mat + (uint32_t)(b * kTileDoubles + 2 * (r * kTableBlock + wave0)) * 8u,
+                    r * kTableBlock + tid, n >> 1);
+    if (base == 0 && lists_staged(x)) {
+      copy4_to_lds(p.list_uidx + x.dst_list, lds_lists + (uint32_t)((b * 2 + 0) * kListInts + wave0) * 4u, tid, x.sdst);
+      copy4_to_lds(p.list_uidx + x.src_list, lds_lists + (uint32_t)((b * 2 + 1) * kListInts + wave0) * 4u, tid, x.ssrc);
+    }
+  };
+  const int e_begin = first_node < end_node ? p.node_edge_off[first_node] : 0;
+  const int e_end = first_node < end_node ? p.node_edge_off[end_node] : 0;
+  apc_edge nxt;
+  if (e_begin < e_end) nxt = load_edge(p.edges + e_begin);
+  int buf = 0;
+  {
+    const int s0 = e_begin < e_end ? next_staged[e_begin] : -1;  // the first edge that goes through LDS
+    if (s0 >= 0 && s0 < e_end) issue(s0 == e_begin ? nxt : load_edge(p.edges + s0), edge_msize[s0], 0, buf);
+  }
+  for (int v = first_node; v < end_node; ++v) {
+    const int nstrat = p.node_nstrat[v];
+    const int nargs = p.node_nargs[v];
+    const double fargs = (double)(nargs > 1 ? nargs : 1);
+    const double mult = (double)p.node_multiplier[v];
+    const int64_t comp_off = p.node_comp_off[v];
+    uint32_t o[kPer];
+    double pa[kPer];
+#pragma unroll
+    for (int k = 0; k < kPer; ++k) {
+      o[k] = choice(k, v, nstrat);
+      pa[k] = per_arg[comp_off + o[k]];
+    }
+#pragma unroll
+    for (int k = 0; k < kPer; ++k) t_compute[k] += pa[k] * fargs;
+    for (int e = p.node_edge_off[v]; e < p.node_edge_off[v + 1]; ++e) {
+      const apc_edge ed = nxt;
+      if (e + 1 < e_end) nxt = load_edge(p.edges + e + 1);
+      const int msize = edge_msize[e];  // elements that go through LDS; 0: read the matrix in place
+      const bool has_src = ed.src_node >= 0;
+      const bool squeezed = (ed.flags & APC_EDGE_COMPRESSED) != 0;
+      const uint32_t usrc = (uint32_t)ed.flags >> APC_EDGE_USRC_SHIFT;
+      uint32_t j[kPer], at[kPer];
+#pragma unroll
+      for (int k = 0; k < kPer; ++k) j[k] = has_src ? choice(k, ed.src_node, ed.ssrc) : 0u;
+      double raw[kPer];
+      if (msize > 0) {  // uniform over the workgroup, as everything that decides a barrier below
+        const double* const mat = s_all + buf * kTileDoubles;
+        __builtin_amdgcn_s_waitcnt(0);  // this lane's part of the first tile has arrived,
+        __syncthreads();                // and everyone's; and the draws of the edge before are done,
+        {                               // so its buffer can take the next matrix
+          const int s1 = next_staged[e + 1];
+          if (s1 >= 0 && s1 < e_end) issue(s1 == e + 1 ? nxt : load_edge(p.edges + s1), edge_msize[s1], 0, buf ^ 1);
+        }
+        if (squeezed && lists_staged(ed)) {
+          const int32_t* const ud = s_lists + (buf * 2 + 0) * kListInts;
+          const int32_t* const us = s_lists + (buf * 2 + 1) * kListInts;
+#pragma unroll
+          for (int k = 0; k < kPer; ++k) at[k] = (uint32_t)ud[o[k]] * usrc + (uint32_t)us[j[k]];
+        } else if (squeezed) {
+#pragma unroll
+          for (int k = 0; k < kPer; ++k)
+            at[k] = (uint32_t)p.list_uidx[(size_t)ed.dst_list + o[k]] * usrc +
+                    (uint32_t)p.list_uidx[(size_t)ed.src_list + j[k]];
+        } else {
+#pragma unroll
+          for (int k = 0; k < kPer; ++k) at[k] = o[k] * (uint32_t)ed.ssrc + j[k];
+        }
+        for (int base = 0;;) {
+          const int n = msize - base < kTileDoubles ? msize - base : kTileDoubles;
+#pragma unroll
+          for (int k = 0; k < kPer; ++k) {
+            const uint32_t local = at[k] - (uint32_t)base;
+            if (local < (uint32_t)n) raw[k] = mat[local];
+          }
+          base += kTileDoubles;
+          if (base >= msize) break;
+          __syncthreads();  // the draws from this tile are done
+          issue(ed, msize, base, buf);
+          __builtin_amdgcn_s_waitcnt(0);
+          __syncthreads();
+        }
+        buf ^= 1;
+      } else {
+        const double* __restrict__ matrix =
+            ed.table_off >= 0 ? table + ed.table_off : p.default_vals + ed.default_off;
+#pragma unroll
+        for (int k = 0; k < kPer; ++k) {
+          if (squeezed)
+            at[k] = (uint32_t)p.list_uidx[(size_t)ed.dst_list + o[k]] * usrc +
+                    (uint32_t)p.list_uidx[(size_t)ed.src_list + j[k]];
+          else at[k] = o[k] * (uint32_t)ed.ssrc + j[k];
+        }
+#pragma unroll
+        for (int k = 0; k < kPer; ++k) raw[k] = matrix[at[k]];
+      }
+      const bool count_trans = has_src && (ed.flags & APC_EDGE_SCORE_TRANSITION);
+#pragma unroll
+      for (int k = 0; k < kPer; ++k) {
+        // as item_store makes an entry from its matrix element
+        const uint32_t trans = (uint32_t)((uint64_t)__double_as_longlong(raw[k]) >> 63);
+        const double cm = fabs(raw[k]);
+        double c = (cm + pa[k]) + (double)(int)trans;
+        const bool finite = isfinite(c);
+        if (clamp_inf && !finite) c = 10000.0;
+        obj[k] += c * mult;
+        forbidden[k] += (double)!finite;
+        if (has_src && isfinite(cm)) t_comm[k] += cm;
+        if (count_trans && trans) t_trans[k] += 1.0;
+      }
+    }
+  }
+  __builtin_amdgcn_s_waitcnt(0);  // nothing is in flight towards LDS when the workgroup ends
+#pragma unroll
+  for (int k = 0; k < kPer; ++k) {
+    if (t_raw + k * lanes >= n_assign) continue;
+    double* r = out + asg(k) * 6;
+    r[0] = (t_compute[k] + t_comm[k]) + t_trans[k];
+    r[1] = t_compute[k];
+    r[2] = t_comm[k];
+    r[3] = t_trans[k];
+    r[4] = obj[k];
+    r[5] = forbidden[k];
+  }
+}
+
+template <bool kRandom, int kPer>
+int launch_table_k(dim3 grid, hipStream_t stream, const apc_problem& p, const double* per_arg, const double* table,
+                   const int32_t* edge_msize, const int32_t* next_staged, const uint16_t* assign, int64_t stride,
+                   uint64_t seed, int64_t first, int64_t n_assign, const int32_t* node_gid, int first_node,
+                   int end_node, int clamp_inf, const double* init, double* out) {
+  // dynamic LDS beyond 64 KB needs the limit raised, per kernel and device; cheap enough to do per launch
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(score_table_kernel<kRandom, kPer>),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, kTableLds);
+  if (e != hipSuccess) return fail(APC_ERR_LAUNCH, "hipFuncSetAttribute(score_table_kernel): %s", hipGetErrorString(e));
+  hipLaunchKernelGGL((score_table_kernel<kRandom, kPer>), grid, dim3(kTableBlock), kTableLds, stream, p, per_arg,
+                     table, edge_msize, next_staged, assign, stride, seed, first, n_assign, node_gid, first_node,
+                     end_node, clamp_inf, init, out);
+  return check_launch("score_table_kernel");
+}
+
+template <bool kRandom, typename... Args>
+int launch_table(int per, Args... args) {
+  switch (per) {
+    case 1: return launch_table_k<kRandom, 1>(args...);
+    case 2: return launch_table_k<kRandom, 2>(args...);
+    default: return launch_table_k<kRandom, 4>(args...);
+  }
+}
+
 template <bool kRandom>
 __global__ void __launch_bounds__(kBlock)
 score_wave_kernel(apc_problem p, const double* __restrict__ per_arg,
@@ -278,6 +687,24 @@ score_wave_kernel(apc_problem p, const double* __restrict__ per_arg,
 
 // below this many assignments one wavefront per assignment is faster than one lane
 constexpr int64_t kScoreWaveBelow = 32768;
+
+template <bool kRandom>
+int launch_compact(int per, dim3 grid, hipStream_t stream, const apc_problem& p, const double* per_arg,
+                          const apc_score_rec16* recs, const uint16_t* assign, int64_t stride, uint64_t seed,
+                          int64_t first, int64_t n_assign, const int32_t* node_gid, int first_node, int end_node,
+                          const double* init, double* out) {
+#define APC_COMPACT(K)                                                                                     \
+  hipLaunchKernelGGL((score_compact_kernel<kRandom, K>), grid, dim3(kBlock), 0, stream, p, per_arg, recs, \
+                     assign, stride, seed, first, n_assign, node_gid, first_node, end_node, init, out)
+  switch (per) {
+    case 1: APC_COMPACT(1); break;
+    case 2: APC_COMPACT(2); break;
+    case 4: APC_COMPACT(4); break;
+    default: APC_COMPACT(8); break;
+  }
+#undef APC_COMPACT
+  return check_launch("score_compact_kernel");
+}
 
 }  // namespace
 
@@ -396,6 +823,89 @@ int apc_score_packed(const apc_problem* p, const double* per_arg, const apc_scor
                          per_arg, recs, assign, n_assign, seed, first + a0, n, node_gid, first_node,
                          in, out + a0 * 6);
     if (int rc = check_launch("score_packed_kernel")) return rc;
+  }
+  return 0;
+}
+
+int apc_pack_score_records16(const apc_problem* p, const double* per_arg, const double* comm,
+                             const double* cost, const uint8_t* flags, apc_score_rec16* recs,
+                             int32_t* mismatch, void* stream) {
+  if (int rc = validate_problem(p)) return rc;
+  if (!per_arg || !comm || !cost || !flags || !recs || !mismatch)
+    return fail(APC_ERR_INVALID, "apc_pack_score_records16: null argument%s");
+  hipLaunchKernelGGL(clear_flag_kernel, dim3(1), dim3(1), 0, (hipStream_t)stream, mismatch);
+  if (p->n_slot == 0) return check_launch("clear_flag_kernel");
+  if (!p->chunk_edge) return fail(APC_ERR_INVALID, "apc_pack_score_records16: the problem has no chunk_edge%s");
+  unsigned grid;
+  if (int rc = slot_grid(p, kBlock, &grid)) return rc;
+  hipLaunchKernelGGL(score_pack16_kernel, dim3(grid), dim3(kBlock), 0, (hipStream_t)stream, *p, per_arg, comm,
+                     cost, flags, recs, mismatch);
+  return check_launch("score_pack16_kernel");
+}
+
+int apc_score_compact(const apc_problem* p, const double* per_arg, const apc_score_rec16* recs,
+                      const uint16_t* assign, uint64_t seed, int64_t first, int64_t n_assign,
+                      const int32_t* node_gid, int32_t first_node, int32_t end_node, int32_t per_lane,
+                      const double* init, double* out, void* stream) {
+  if (int rc = validate_problem(p)) return rc;
+  if (n_assign <= 0) return 0;
+  if (!per_arg || !recs || !out || !p->node_multiplier)
+    return fail(APC_ERR_INVALID, "apc_score_compact: null argument%s");
+  if (first_node < 0 || first_node > end_node || end_node > p->n_node)
+    return fail(APC_ERR_INVALID, "apc_score_compact: need 0 <= first_node <= end_node <= n_node%s");
+  // Batches of up to kResident * 8 assignments per launch: kResident lanes are what the
+  // 256 CUs hold at once with this kernel's registers, so that no workgroup waits for
+  // another to finish and all of them walk the graph together.
+  const int64_t kResident = 262144;
+  for (int64_t a0 = 0; a0 < n_assign; a0 += kResident * 8) {
+    const int64_t n = (n_assign - a0 < kResident * 8) ? (n_assign - a0) : kResident * 8;
+    int per = per_lane;
+    if (per <= 0) per = n <= kResident ? 1 : n <= 2 * kResident ? 2 : n <= 4 * kResident ? 4 : 8;
+    if (per != 1 && per != 2 && per != 4 && per != 8)
+      return fail(APC_ERR_INVALID, "apc_score_compact: per_lane must be 0 (choose), 1, 2, 4 or 8%s");
+    const int64_t lanes = (n + per - 1) / per;
+    const dim3 grid((unsigned)((lanes + kBlock - 1) / kBlock));
+    const double* in = init ? init + a0 * 6 : nullptr;
+    int rc = assign ? launch_compact<false>(per, grid, (hipStream_t)stream, *p, per_arg, recs, assign + a0, n_assign,
+                                            seed, first + a0, n, node_gid, first_node, end_node, in, out + a0 * 6)
+                    : launch_compact<true>(per, grid, (hipStream_t)stream, *p, per_arg, recs, assign, n_assign,
+                                           seed, first + a0, n, node_gid, first_node, end_node, in, out + a0 * 6);
+    if (rc) return rc;
+  }
+  return 0;
+}
+
+int apc_score_table_tile(void) { return kTileDoubles; }
+
+int apc_score_table(const apc_problem* p, const double* per_arg, const double* table,
+                    const int32_t* edge_msize, const int32_t* next_staged, const uint16_t* assign,
+                    uint64_t seed, int64_t first, int64_t n_assign, const int32_t* node_gid,
+                    int32_t first_node, int32_t end_node, int32_t clamp_inf, int32_t per_lane,
+                    const double* init, double* out, void* stream) {
+  if (int rc = validate_problem(p)) return rc;
+  if (n_assign <= 0) return 0;
+  if (!per_arg || !edge_msize || !next_staged || !out || !p->node_multiplier || (p->table_size > 0 && !table))
+    return fail(APC_ERR_INVALID, "apc_score_table: null argument%s");
+  if (first_node < 0 || first_node > end_node || end_node > p->n_node)
+    return fail(APC_ERR_INVALID, "apc_score_table: need 0 <= first_node <= end_node <= n_node%s");
+  if (per_lane != 0 && per_lane != 1 && per_lane != 2 && per_lane != 4)
+    return fail(APC_ERR_INVALID, "apc_score_table: per_lane must be 0 (choose), 1, 2 or 4%s");
+  // 262144 lanes are one workgroup on each of the 256 CUs; four assignments a lane is
+  // what the registers of that many waves allow.
+  const int64_t kLanes = 262144;
+  for (int64_t a0 = 0; a0 < n_assign; a0 += kLanes * 4) {
+    const int64_t n = (n_assign - a0 < kLanes * 4) ? (n_assign - a0) : kLanes * 4;
+    const int per = per_lane ? per_lane : n <= kLanes ? 1 : n <= 2 * kLanes ? 2 : 4;
+    const int64_t lanes = (n + per - 1) / per;
+    const dim3 grid((unsigned)((lanes + kTableBlock - 1) / kTableBlock));
+    const double* in = init ? init + a0 * 6 : nullptr;
+    int rc = assign ? launch_table<false>(per, grid, (hipStream_t)stream, *p, per_arg, table, edge_msize, next_staged,
+                                          assign + a0, n_assign, seed, first + a0, n, node_gid, (int)first_node,
+                                          (int)end_node, (int)clamp_inf, in, out + a0 * 6)
+                    : launch_table<true>(per, grid, (hipStream_t)stream, *p, per_arg, table, edge_msize, next_staged,
+                                         assign, n_assign, seed, first + a0, n, node_gid, (int)first_node,
+                                         (int)end_node, (int)clamp_inf, in, out + a0 * 6);
+    if (rc) return rc;
   }
   return 0;
 }

@@ -19,6 +19,10 @@ _TABLE_MAX_DOUBLES = 1 << 28
 _WIDE_ITEMS_FROM = 32_000_000  # entries
 _PACKED_SCORING_FROM = 8192  # mean entries per edge block
 _SCORE_LANES_FROM = 32768  # assignments: below, one wavefront per assignment (entry arrays as they are)
+_SCORE_FROM_TABLE = True  # the three ways of scoring a graph with large blocks can be switched off (tests do)
+_SCORE_COMPACT = True
+_SCORE_STAGE_TILES = 8  # matrices of up to this many LDS tiles go through LDS in the table scorer
+_SCORE_PER_LANE = 0  # assignments per lane of the compact scorer; 0: the library chooses
 _LUT_TABLE_FROM = 2048  # table units: larger tables are built tile by tile with per-source terms in LDS
 
 
@@ -306,6 +310,10 @@ class CostEngine:
         self.packed_scoring = g.num_edges > 0 and g.num_entries / g.num_edges >= _PACKED_SCORING_FROM
         self._recs: Optional[torch.Tensor] = None
         self._recs_valid = False
+        self._recs_compact = False
+        # clamp_inf of the build whose table path wrote the entry arrays as they are now,
+        # None once anything else has written them: then scoring cannot read the table instead
+        self._table_clamp: Optional[int] = None
 
     def synchronize(self) -> None:
         torch.cuda.synchronize(self.device)
@@ -336,6 +344,7 @@ class CostEngine:
 
     def edge_costs(self, clamp_inf: bool = True, want_comm: bool = True, want_flags: bool = True):
         self._recs_valid = False
+        self._table_clamp = None
         _lib.check(
             self.lib.apc_edge_costs(
                 C.byref(self.problem), self._ptr(self.table), self._ptr(self.per_arg),
@@ -348,6 +357,7 @@ class CostEngine:
         """edge_costs with HIP events at the kernel's begin and end (a timer from
         apc_timer_create); the launch is otherwise identical."""
         self._recs_valid = False
+        self._table_clamp = None
         _lib.check(
             self.lib.apc_edge_costs_timed(
                 C.byref(self.problem), self._ptr(self.table), self._ptr(self.per_arg), self._ptr(self.comm),
@@ -389,6 +399,7 @@ class CostEngine:
         else:
             self._build_with_lut(1 if clamp_inf else 0, stream)
         self.built = True
+        self._table_clamp = (1 if clamp_inf else 0) if self.table is not None else None
         return self
 
     def _build_with_lut(self, clamp_inf: int, stream) -> None:
@@ -416,6 +427,7 @@ class CostEngine:
             _lib.check(rc, "apc_build_all_timed")
         self._recs_valid = False
         self.built = True
+        self._table_clamp = (1 if clamp_inf else 0) if self.table is not None else None
         return self
 
     def set_node_multiplier(self, mult: np.ndarray) -> None:
@@ -437,6 +449,7 @@ class CostEngine:
         self.per_arg.copy_(torch.from_numpy(np.ascontiguousarray(per_arg, np.float64)))
         self.built = True
         self._recs_valid = False
+        self._table_clamp = None
         return self
 
     def capture_build(self, clamp_inf: bool = True) -> "torch.cuda.CUDAGraph":
@@ -464,6 +477,7 @@ class CostEngine:
     def apply_prefetch_discount(self, scale: float = 0.0) -> int:
         assert self.built
         self._recs_valid = False
+        self._table_clamp = None
         n = torch.zeros(1, dtype=torch.int64, device=self.device)
         _lib.check(
             self.lib.apc_apply_prefetch_discount(
@@ -500,17 +514,55 @@ class CostEngine:
         return out
 
     def _score_packed(self, assign, seed, first, count, d_gid, first_node, init, out) -> torch.Tensor:
-        """Scoring from the interleaved records (apc_score_packed); they are
-        (re)made here if the entry arrays changed since."""
-        if not self._recs_valid:
-            if self._recs is None:
-                self._recs = torch.empty(self.g.num_slots * 4, dtype=torch.float64, device=self.device)
+        """Scoring of a graph with large blocks: from the block table while the
+        entry arrays are what the last build made of it (apc_score_table); else
+        from records made here if the entry arrays changed since: compact 16-byte
+        records, several assignments per lane (apc_score_compact), while every
+        cost is (comm + per_arg) + transition or its clamp (checked on the device
+        when the records are made); else the 32-byte records that carry the cost
+        (apc_score_packed)."""
+        if self._table_clamp is not None and _SCORE_FROM_TABLE:
+            msize, next_staged = self._score_msize()
             _lib.check(
-                self.lib.apc_pack_score_records(
-                    C.byref(self.problem), self._ptr(self.comm), self._ptr(self.cost), self._ptr(self.flags),
-                    self._ptr(self._recs), self._stream()),
-                "apc_pack_score_records")
+                self.lib.apc_score_table(
+                    C.byref(self.problem), self._ptr(self.per_arg), self._ptr(self.table),
+                    C.c_void_p(msize.data_ptr()), C.c_void_p(next_staged.data_ptr()), self._ptr(assign),
+                    int(seed), int(first), int(count), self._ptr(d_gid), int(first_node), self.g.num_nodes,
+                    self._table_clamp, min(_SCORE_PER_LANE, 4),
+                    self._ptr(init), self._ptr(out), self._stream()),
+                "apc_score_table")
+            return out
+        if not self._recs_valid:
+            self._recs = None  # one kind at a time: either is as large as the entry arrays
+            recs = None
+            self._recs_compact = False
+            if _SCORE_COMPACT:
+                recs = torch.empty(self.g.num_slots * 2, dtype=torch.float64, device=self.device)
+                mismatch = torch.empty(1, dtype=torch.int32, device=self.device)
+                _lib.check(
+                    self.lib.apc_pack_score_records16(
+                        C.byref(self.problem), self._ptr(self.per_arg), self._ptr(self.comm), self._ptr(self.cost),
+                        self._ptr(self.flags), self._ptr(recs), self._ptr(mismatch), self._stream()),
+                    "apc_pack_score_records16")
+                self._recs_compact = int(mismatch.item()) == 0
+            if not self._recs_compact:
+                del recs
+                recs = torch.empty(self.g.num_slots * 4, dtype=torch.float64, device=self.device)
+                _lib.check(
+                    self.lib.apc_pack_score_records(
+                        C.byref(self.problem), self._ptr(self.comm), self._ptr(self.cost), self._ptr(self.flags),
+                        self._ptr(recs), self._stream()),
+                    "apc_pack_score_records")
+            self._recs = recs
             self._recs_valid = True
+        if self._recs_compact:
+            _lib.check(
+                self.lib.apc_score_compact(
+                    C.byref(self.problem), self._ptr(self.per_arg), self._ptr(self._recs), self._ptr(assign),
+                    int(seed), int(first), int(count), self._ptr(d_gid), int(first_node), self.g.num_nodes,
+                    _SCORE_PER_LANE, self._ptr(init), self._ptr(out), self._stream()),
+                "apc_score_compact")
+            return out
         _lib.check(
             self.lib.apc_score_packed(
                 C.byref(self.problem), self._ptr(self.per_arg), self._ptr(self._recs), self._ptr(assign),
@@ -518,6 +570,27 @@ class CostEngine:
                 self._ptr(out), self._stream()),
             "apc_score_packed")
         return out
+
+    def _score_msize(self):
+        """(edge_msize, next_staged) of apc_score_table: the padded size of an
+        edge's matrix in the block table if it is worth taking through LDS (eight
+        tiles at most), and the first such edge from each edge on."""
+        hit = self._keep.get("score_msize")
+        if hit is None:
+            g = self.g
+            _, block_off, _, edge_table_off, _, _ = g.block_table(self.table_mode == "compressed")
+            msize = np.zeros(g.num_edges, np.int32)
+            has = edge_table_off >= 0
+            b = np.searchsorted(block_off, edge_table_off[has], side="right") - 1
+            size = (block_off[b + 1] - block_off[b]).astype(np.int64)
+            limit = _SCORE_STAGE_TILES * int(self.lib.apc_score_table_tile())
+            msize[has] = np.where(size <= limit, size, 0).astype(np.int32)
+            idx = np.where(msize > 0, np.arange(g.num_edges), g.num_edges)
+            nxt = np.minimum.accumulate(np.concatenate([idx, [g.num_edges]])[::-1])[::-1]
+            next_staged = np.where(nxt < g.num_edges, nxt, -1).astype(np.int32)
+            hit = self._keep["score_msize"] = (torch.from_numpy(msize).to(self.device),
+                                               torch.from_numpy(next_staged).to(self.device))
+        return hit
 
     def node_hashes(self, node_phase: Optional[np.ndarray] = None) -> np.ndarray:
         """uint64[n_node] structural hash of every node (the clustering key).

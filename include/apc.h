@@ -607,6 +607,53 @@ int apc_score_packed(const apc_problem* p, const double* per_arg, const apc_scor
                      const int32_t* node_gid, int32_t first_node, const double* init,
                      double* out, void* stream);
 
+/* Compact records for graphs with large blocks: cost is not stored, because
+ * the cost of an entry is (comm + per_arg[comp_base + out_idx]) + transition
+ * (autoparallel/optimize_sharding.py:544), or the clamp 10000 where that sum
+ * is not finite, and the scorer holds per_arg of its node's choice already. */
+#define APC_SCORE_CLAMPED 4 /* in apc_score_rec16.flags beside APC_ENTRY_*: cost is the clamp */
+typedef struct apc_score_rec16 {
+  double comm;
+  uint64_t flags;
+} apc_score_rec16; /* 16 bytes */
+
+/* recs[slot] = {comm[slot], flags[slot] | clamped}; mismatch[0] (device) = 0,
+ * or 1 if some cost[slot] is neither that sum nor its clamp (arrays changed
+ * after the build): then the records must not be used.  p needs chunk_edge. */
+int apc_pack_score_records16(const apc_problem* p, const double* per_arg, const double* comm,
+                             const double* cost, const uint8_t* flags, apc_score_rec16* recs,
+                             int32_t* mismatch, void* stream);
+
+/* apc_score_packed over the compact records, for the nodes [first_node,
+ * end_node), per_lane assignments per lane (1, 2, 4, 8; 0: chosen so that a
+ * batch of up to 2^21 walks the graph once, larger batches in launches of
+ * 2^21).  Same sums, bit for bit. */
+int apc_score_compact(const apc_problem* p, const double* per_arg, const apc_score_rec16* recs,
+                      const uint16_t* assign, uint64_t seed, int64_t first, int64_t n_assign,
+                      const int32_t* node_gid, int32_t first_node, int32_t end_node, int32_t per_lane,
+                      const double* init, double* out, void* stream);
+
+/* The same sums from the block table instead of the entry arrays, for graphs
+ * with large blocks: an entry is (|m| + per_arg) + transition with the flag in
+ * the sign of its matrix element m, clamped to 10000 if clamp_inf and not finite
+ * (what apc_edge_costs writes from the table), so the result equals, bit for
+ * bit, that of apc_score_packed on the arrays of a build with this clamp_inf.
+ * One workgroup of 1024 lanes per CU, per_lane assignments each (1, 2, 4; 0:
+ * chosen), has the current edge's matrix in LDS and draws from there.
+ * edge_msize[e] (device, int32[n_edge]): the number of elements of edge e's
+ * matrix to take through LDS, tile by tile (apc_score_table_tile() elements a
+ * tile): even, and only for an edge with table_off >= 0 (the matrix's padded
+ * size in the table will do); or 0 to read the matrix in place (no matrix:
+ * default rows; or too large to be worth it).  next_staged[e] (device,
+ * int32[n_edge + 1]): the first edge >= e with edge_msize > 0, or -1.  table as
+ * for apc_edge_costs; p carries list_uidx if it has compressed matrices. */
+int apc_score_table(const apc_problem* p, const double* per_arg, const double* table,
+                    const int32_t* edge_msize, const int32_t* next_staged, const uint16_t* assign,
+                    uint64_t seed, int64_t first, int64_t n_assign, const int32_t* node_gid,
+                    int32_t first_node, int32_t end_node, int32_t clamp_inf, int32_t per_lane,
+                    const double* init, double* out, void* stream);
+int apc_score_table_tile(void);
+
 /* Replaces _get_sharded_shape_stride
  * (autoparallel/cost_models/compute_estimation.py:300-318) for n specs:
  * rank[i], shape/stride[i][APC_MAX_RANK], plc[i][APC_MAX_MESH_DIMS] ->

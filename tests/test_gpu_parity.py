@@ -329,10 +329,16 @@ def test_scoring(CostEngine):
         assert tuple(out[i, :4]) == tuple(float(x) for x in want)
 
 
-def test_scoring_from_interleaved_records(CostEngine):
+def test_scoring_from_interleaved_records(CostEngine, monkeypatch):
     """apc_score_packed against the scorers that read the three entry arrays:
     explicit assignments, drawn ones, a window with continued sums; and the
-    records follow the entry arrays when those are rewritten."""
+    records follow the entry arrays when those are rewritten.  (The scorers
+    that come before it for a graph with large blocks are switched off here;
+    test_gpu_scoring_large_blocks.py covers them.)"""
+    from autoparallel_amd import engine as engine_mod
+
+    monkeypatch.setattr(engine_mod, "_SCORE_FROM_TABLE", False)
+    monkeypatch.setattr(engine_mod, "_SCORE_COMPACT", False)
     for name in ("stress_3d", "llama_2d"):
         g = GRAPHS[name]()
         eng = CostEngine(g).build(clamp_inf=True)
