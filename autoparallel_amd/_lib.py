@@ -216,6 +216,10 @@ _SIGNATURES = {
         C.c_int,
         [C.POINTER(ApcProblem), C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32,
          C.c_void_p]),
+    "apc_edge_costs_lut_timed": (
+        C.c_int,
+        [C.POINTER(ApcProblem), C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32,
+         C.c_void_p, C.c_int32, C.c_void_p]),
     "apc_calibration_copy": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p]),
     "apc_apply_prefetch_discount": (
         C.c_int,

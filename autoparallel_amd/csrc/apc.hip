@@ -1067,6 +1067,18 @@ struct apc_timer {
   hipEvent_t* ev;  // 2 n events: start and stop of each slot
 };
 
+}  // extern "C"
+namespace apc_impl {
+bool timer_events(void* timer, int slot, hipEvent_t* start, hipEvent_t* stop) {
+  apc_timer* t = static_cast<apc_timer*>(timer);
+  if (!t || slot < 0 || slot >= t->n) return false;
+  *start = t->ev[2 * slot];
+  *stop = t->ev[2 * slot + 1];
+  return true;
+}
+}  // namespace apc_impl
+extern "C" {
+
 int apc_timer_create(int32_t n_slots, void** timer) {
   if (n_slots <= 0 || !timer) return fail(APC_ERR_INVALID, "apc_timer_create: need n_slots > 0 and a result pointer%s");
   apc_timer* t = new apc_timer{n_slots, new hipEvent_t[2 * (size_t)n_slots]};

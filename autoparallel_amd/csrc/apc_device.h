@@ -25,6 +25,8 @@ APC_HIDDEN int check_launch(const char* what);
 APC_HIDDEN int validate_problem(const apc_problem* p);
 APC_HIDDEN int grid_for(int64_t total, int block);
 APC_HIDDEN int slot_grid(const apc_problem* p, int per_block, unsigned* grid);
+// The two events of a timer's slot (apc_timer_create); false for a bad timer or slot.
+APC_HIDDEN bool timer_events(void* timer, int slot, hipEvent_t* start, hipEvent_t* stop);
 }  // namespace apc_impl
 
 namespace {

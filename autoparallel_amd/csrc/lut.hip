@@ -199,10 +199,11 @@ lut_kernel(apc_problem p, const apc_lut_tile* __restrict__ tiles, double* __rest
 
 template <bool kEntries>
 void launch_lut(const apc_problem* p, const apc_lut_tile* tiles, int64_t n_tile, double* table, const double* per_arg,
-                double* comm, double* cost, uint8_t* flags, int clamp_inf, hipStream_t stream) {
-#define APC_LAUNCH_LUT(N)                                                                                      \
-  hipLaunchKernelGGL((lut_kernel<kEntries, N>), dim3((unsigned)n_tile), dim3(256), 0, stream, *p, tiles, table, \
-                     per_arg, comm, cost, flags, clamp_inf)
+                double* comm, double* cost, uint8_t* flags, int clamp_inf, hipStream_t stream,
+                hipEvent_t start = nullptr, hipEvent_t stop = nullptr) {
+#define APC_LAUNCH_LUT(N)                                                                                   \
+  hipExtLaunchKernelGGL((lut_kernel<kEntries, N>), dim3((unsigned)n_tile), dim3(256), 0, stream, start, stop, \
+                        0, *p, tiles, table, per_arg, comm, cost, flags, clamp_inf)
   switch (p->model.ndim) {  // validate_problem has checked the range
     case 1: APC_LAUNCH_LUT(1); break;
     case 2: APC_LAUNCH_LUT(2); break;
@@ -239,6 +240,20 @@ int apc_edge_costs_lut(const apc_problem* p, const apc_lut_tile* tiles, int64_t 
   if (n_tile == 0) return 0;
   if (!per_arg) return fail(APC_ERR_INVALID, "apc_edge_costs_lut: null per_arg%s");
   launch_lut<true>(p, tiles, n_tile, nullptr, per_arg, comm, cost, flags, clamp_inf, (hipStream_t)stream);
+  return check_launch("lut_kernel<entries>");
+}
+
+/* apc_edge_costs_lut with the timer's events of `slot` at the kernel's begin and end. */
+int apc_edge_costs_lut_timed(const apc_problem* p, const apc_lut_tile* tiles, int64_t n_tile, const double* per_arg,
+                             double* comm, double* cost, uint8_t* flags, int32_t clamp_inf, void* timer,
+                             int32_t slot, void* stream) {
+  if (int rc = check_tiles(p, tiles, n_tile, "apc_edge_costs_lut_timed")) return rc;
+  hipEvent_t start, stop;
+  if (!apc_impl::timer_events(timer, slot, &start, &stop))
+    return fail(APC_ERR_INVALID, "apc_edge_costs_lut_timed: bad timer or slot%s");
+  if (n_tile == 0) return 0;
+  if (!per_arg) return fail(APC_ERR_INVALID, "apc_edge_costs_lut_timed: null per_arg%s");
+  launch_lut<true>(p, tiles, n_tile, nullptr, per_arg, comm, cost, flags, clamp_inf, (hipStream_t)stream, start, stop);
   return check_launch("lut_kernel<entries>");
 }
 

@@ -17,7 +17,7 @@ from .packed import CHUNK_SHIFT, ITEM_ENTRIES, MAX_MESH_DIMS, PackedGraph
 _TABLE_MAX_RATIO = 0.5
 _TABLE_MAX_DOUBLES = 1 << 28
 _WIDE_ITEMS_FROM = 32_000_000  # entries
-_PACKED_SCORING_FROM = 8192  # mean entries per edge block
+_LARGE_BLOCKS_FROM = 8192  # mean entries per edge block
 _SCORE_LANES_FROM = 32768  # assignments: below, one wavefront per assignment (entry arrays as they are)
 _SCORE_FROM_TABLE = True  # the three ways of scoring a graph with large blocks can be switched off (tests do)
 _SCORE_COMPACT = True
@@ -304,16 +304,19 @@ class CostEngine:
         )
         self.built = False
         self._build_args = None
-        # interleaved copy of the entry arrays for scoring (apc_score_rec), made on
-        # first use when the edge blocks are large; stale after anything rewrites
-        # the entry arrays
-        self.packed_scoring = g.num_edges > 0 and g.num_entries / g.num_edges >= _PACKED_SCORING_FROM
+        # Batches of _SCORE_LANES_FROM assignments and more are scored from something
+        # denser than the three entry arrays: the block table itself when the blocks
+        # are large (_score_packed), else records made from the arrays on first use,
+        # stale after anything rewrites the arrays.
+        self.packed_scoring = g.num_edges > 0 and g.num_entries > 0
+        self.large_blocks = g.num_edges > 0 and g.num_entries / g.num_edges >= _LARGE_BLOCKS_FROM
         self._recs: Optional[torch.Tensor] = None
         self._recs_valid = False
         self._recs_compact = False
         # clamp_inf of the build whose table path wrote the entry arrays as they are now,
         # None once anything else has written them: then scoring cannot read the table instead
         self._table_clamp: Optional[int] = None
+        self.last_score_backend = "entry_arrays"  # what the last large batch was scored from
 
     def synchronize(self) -> None:
         torch.cuda.synchronize(self.device)
@@ -367,13 +370,22 @@ class CostEngine:
         )
 
     def prepare(self):
-        """Pair table and node compute vectors in one launch."""
-        _lib.check(
-            self.lib.apc_prepare(
-                C.byref(self.problem), self._ptr(self.table), self._ptr(self.compute),
-                self._ptr(self.per_arg), self._ptr(self.status), self._stream()),
-            "apc_prepare",
-        )
+        """Pair table and node compute vectors, as build() makes them: one launch,
+        or, with the lookup-table kernels, the node launch and the table by tiles."""
+        if self._lut_tiles is None:
+            _lib.check(
+                self.lib.apc_prepare(
+                    C.byref(self.problem), self._ptr(self.table), self._ptr(self.compute),
+                    self._ptr(self.per_arg), self._ptr(self.status), self._stream()),
+                "apc_prepare",
+            )
+            return
+        p, table, compute, per_arg, status = self.build_args()[:5]
+        stream = torch.cuda.current_stream(self.device).cuda_stream
+        _lib.check(self.lib.apc_node_compute_costs(p, compute, per_arg, status, stream), "apc_node_compute_costs")
+        if self.use_table:
+            tiles, n_tile = self._lut_tiles
+            _lib.check(self.lib.apc_build_pair_table_lut(p, tiles, n_tile, table, stream), "apc_build_pair_table_lut")
 
     def build_args(self):
         if not self.can_build:
@@ -418,16 +430,31 @@ class CostEngine:
                        "apc_edge_costs_lut")
 
     def build_timed(self, timer, slot: int, clamp_inf: bool = True):
-        """build() with HIP events at the begin and end of the entry kernel (a
-        timer from apc_timer_create); the launches are otherwise identical."""
+        """build() with HIP events at the begin and end of the kernel that writes
+        the entries (a timer from apc_timer_create); the launches are otherwise
+        identical."""
         self.build_args()
-        rc = self.lib.apc_build_all_timed(*self._build_args, 1 if clamp_inf else 0, timer, int(slot),
-                                          torch.cuda.current_stream(self.device).cuda_stream)
-        if rc:
-            _lib.check(rc, "apc_build_all_timed")
+        stream = torch.cuda.current_stream(self.device).cuda_stream
+        clamp = 1 if clamp_inf else 0
+        if self._lut_tiles is None:
+            rc = self.lib.apc_build_all_timed(*self._build_args, clamp, timer, int(slot), stream)
+            if rc:
+                _lib.check(rc, "apc_build_all_timed")
+        else:
+            p, table, compute, per_arg, status, comm, cost, flags = self._build_args
+            tiles, n_tile = self._lut_tiles
+            lib = self.lib
+            _lib.check(lib.apc_node_compute_costs(p, compute, per_arg, status, stream), "apc_node_compute_costs")
+            if self.use_table:
+                _lib.check(lib.apc_build_pair_table_lut(p, tiles, n_tile, table, stream), "apc_build_pair_table_lut")
+                _lib.check(lib.apc_edge_costs_timed(p, table, per_arg, comm, cost, flags, clamp, timer, int(slot),
+                                                    stream), "apc_edge_costs_timed")
+            else:
+                _lib.check(lib.apc_edge_costs_lut_timed(p, tiles, n_tile, per_arg, comm, cost, flags, clamp, timer,
+                                                        int(slot), stream), "apc_edge_costs_lut_timed")
         self._recs_valid = False
         self.built = True
-        self._table_clamp = (1 if clamp_inf else 0) if self.table is not None else None
+        self._table_clamp = clamp if self.table is not None else None
         return self
 
     def set_node_multiplier(self, mult: np.ndarray) -> None:
@@ -514,14 +541,18 @@ class CostEngine:
         return out
 
     def _score_packed(self, assign, seed, first, count, d_gid, first_node, init, out) -> torch.Tensor:
-        """Scoring of a graph with large blocks: from the block table while the
-        entry arrays are what the last build made of it (apc_score_table); else
-        from records made here if the entry arrays changed since: compact 16-byte
+        """Scoring of a large batch.  A graph with large blocks: from the block
+        table while the entry arrays are what the last build made of it
+        (apc_score_table, 5x the rate of any walk over records there).  Else,
+        and for graphs with small blocks (where the records win: 15.6 ms against
+        18.0 ms from the table and 31.2 ms from the three arrays for 2^20
+        assignments of the Llama-3-8B graph), from records made here if the entry
+        arrays changed since: compact 16-byte
         records, several assignments per lane (apc_score_compact), while every
         cost is (comm + per_arg) + transition or its clamp (checked on the device
         when the records are made); else the 32-byte records that carry the cost
         (apc_score_packed)."""
-        if self._table_clamp is not None and _SCORE_FROM_TABLE:
+        if self._table_clamp is not None and _SCORE_FROM_TABLE and (self.large_blocks or not _SCORE_COMPACT):
             msize, next_staged = self._score_msize()
             _lib.check(
                 self.lib.apc_score_table(
@@ -531,6 +562,7 @@ class CostEngine:
                     self._table_clamp, min(_SCORE_PER_LANE, 4),
                     self._ptr(init), self._ptr(out), self._stream()),
                 "apc_score_table")
+            self.last_score_backend = "block_table"
             return out
         if not self._recs_valid:
             self._recs = None  # one kind at a time: either is as large as the entry arrays
@@ -562,6 +594,7 @@ class CostEngine:
                     int(seed), int(first), int(count), self._ptr(d_gid), int(first_node), self.g.num_nodes,
                     _SCORE_PER_LANE, self._ptr(init), self._ptr(out), self._stream()),
                 "apc_score_compact")
+            self.last_score_backend = "compact_records"
             return out
         _lib.check(
             self.lib.apc_score_packed(
@@ -569,6 +602,7 @@ class CostEngine:
                 int(seed), int(first), int(count), self._ptr(d_gid), int(first_node), self._ptr(init),
                 self._ptr(out), self._stream()),
             "apc_score_packed")
+        self.last_score_backend = "records"
         return out
 
     def _score_msize(self):

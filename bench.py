@@ -246,7 +246,7 @@ def main():
             "entries_per_s": E / t_e2e,
         },
         "roofline": {
-            "kernel": "edge_cost_kernel",
+            "kernel": "edge_cost_kernel" if eng.use_table or eng._lut_tiles is None else "lut_kernel<entries>",
             "bound": "hbm",
             "achieved": achieved,
             "peak": HBM_PEAK_GBS,
@@ -280,6 +280,7 @@ def main():
         t_score = time.perf_counter() - t0
         out["scoring"] = {
             "assignments": n,
+            "scored_from": eng.last_score_backend,
             "seconds": t_score,
             "assignments_per_s": n / t_score,
             "edge_terms_per_s": n * g.num_edges / t_score,

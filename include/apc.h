@@ -497,6 +497,10 @@ int apc_timer_elapsed_ms(void* timer, int32_t slot, float* ms);
 int apc_edge_costs_timed(const apc_problem* p, const double* table, const double* per_arg,
                          double* comm, double* cost, uint8_t* flags, int32_t clamp_inf, void* timer,
                          int32_t slot, void* stream);
+/* apc_edge_costs_lut with the events at the begin and end of its kernel. */
+int apc_edge_costs_lut_timed(const apc_problem* p, const apc_lut_tile* tiles, int64_t n_tile,
+                             const double* per_arg, double* comm, double* cost, uint8_t* flags,
+                             int32_t clamp_inf, void* timer, int32_t slot, void* stream);
 /* apc_build_all with the entry kernel timed as apc_edge_costs_timed does. */
 int apc_build_all_timed(const apc_problem* p, double* table, double* compute, double* per_arg,
                         int32_t* status, double* comm, double* cost, uint8_t* flags,

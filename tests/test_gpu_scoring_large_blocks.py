@@ -65,6 +65,7 @@ def test_every_backend_gives_the_sums_of_the_entry_arrays(knobs, name, table_mod
         eng.packed_scoring = False
         want = _calls(eng, g, assign, half)
         eng.packed_scoring = True
+        eng.large_blocks = True  # the table scorer also for the graph with small blocks
         assert eng._table_clamp == int(clamp)
         # the table, its matrices through LDS (one tile, several tiles) or read in place
         E._SCORE_FROM_TABLE = True
