@@ -480,13 +480,14 @@ class CostEngine:
         return self
 
     def capture_build(self, clamp_inf: bool = True) -> "torch.cuda.CUDAGraph":
-        """The two launches of build() recorded in a HIP graph, for callers that
-        replay a whole planning step from a graph (measured here, a replay takes
-        41.7 us against 38 us for the two eager launches: no gain on its own).
-        The graph holds kernel
-        nodes only (no memset nodes); it is valid while this engine's buffers
-        live.  build() is run once eagerly first so that one-time function
-        attributes are set outside the capture."""
+        """The launches of build() recorded in a HIP graph, for callers that
+        replay a whole planning step from a graph.  On its own a replay is no
+        faster than the eager launches (measured on the headline graph: 29.8 us
+        a replay against 25.8 us for the two launches issued eagerly with cached
+        argument lists).  The graph holds kernel nodes only (no memset nodes);
+        it is valid while this engine's buffers live.  build() is run once
+        eagerly first so that one-time function attributes are set outside the
+        capture."""
         self.build(clamp_inf)
         torch.cuda.synchronize(self.device)
         graph = torch.cuda.CUDAGraph()
