@@ -597,10 +597,25 @@ _FOLLOW = {aten.detach.default} | ({torch.ops.prims.convert_element_type.default
                                   if hasattr(torch.ops.prims, "convert_element_type") else set())
 
 
+# content of an OpStrategy's output specs -> a small token.  A strategy object is
+# summarised once (its specs do not change after it has been returned) and copies
+# made from the query cache inherit the token, so a query key holds one token per
+# tensor argument instead of a tuple over all of the argument's strategies.
+_fp_intern: Dict[tuple, tuple] = {}
+_fp_serial = itertools.count()  # never restarts: a token given out once is not given to other content
+
+
 def _fingerprint(x):
     """Hashable summary of one argument of a strategy query."""
     if isinstance(x, OpStrategy):
-        return ("S",) + tuple(_fingerprint(st.output_specs) for st in x.strategies)
+        fp = getattr(x, "_apc_fp", None)
+        if fp is None:
+            content = ("S",) + tuple(_fingerprint(st.output_specs) for st in x.strategies)
+            fp = _fp_intern.get(content)
+            if fp is None:
+                fp = _fp_intern[content] = ("S#", next(_fp_serial))
+            x._apc_fp = fp
+        return fp
     if isinstance(x, DTensorSpec):
         return (x.placements, x.tensor_meta)
     if isinstance(x, torch.Tensor):
@@ -613,9 +628,16 @@ def _fingerprint(x):
 
 
 def _copy_strategy(src: OpStrategy) -> OpStrategy:
-    """New OpSpec wrappers and cost rows (both are written per node); the specs are shared."""
-    return OpStrategy([OpSpec(st.output_specs, input_specs=st.input_specs,
-                              redistribute_cost=[list(r) for r in st.redistribute_cost]) for st in src.strategies])
+    """New OpSpec wrappers and a new list of cost rows each (a node's rows are
+    replaced when its costs are written back); the specs are shared, and so are
+    the rows themselves until then: they hold zeros, and copying 1.7 M of them
+    for a Llama-3-8B graph took longer than everything else a cache hit does."""
+    out = OpStrategy([OpSpec(st.output_specs, input_specs=st.input_specs,
+                             redistribute_cost=list(st.redistribute_cost)) for st in src.strategies])
+    fp = getattr(src, "_apc_fp", None)
+    if fp is not None:
+        out._apc_fp = fp
+    return out
 
 
 # strategies by query, as the reference keeps them
@@ -628,6 +650,7 @@ strategy_cache_stats = {"hits": 0, "misses": 0}
 
 def reset_placement_options_cache() -> None:
     _strategy_cache.clear()
+    _fp_intern.clear()
     strategy_cache_stats.update(hits=0, misses=0)
 
 
@@ -663,12 +686,51 @@ def get_placement_options_for_node(mesh, node, producers: List[OpStrategy], arg_
     out = _placement_options_uncached(mesh, node, producers, arg_vals, schema_args)
     if key is not None:
         why = fallback_reasons.get(str(node.name), "") if len(fallback_nodes) > n_fallback else None
+        _fingerprint(out)  # summarised here, once: the cached copy and every later copy inherit it
         _strategy_cache[key] = (_copy_strategy(out), why)
         out._apc_query_key = key
     return out
 
 
+def _zero_cost_rows(src_strategy, dst_spec):
+    return [0.0] * len(src_strategy.strategies)
+
+
+_cost_row_users: List = []  # modules of torch's strategy functions that hold generate_redistribute_costs
+_cost_row_users_at = -1     # len(sys.modules) when the list was made
+
+
+@contextlib.contextmanager
+def _without_torch_cost_rows():
+    """torch's strategy functions price every (strategy, producer strategy) pair
+    with torch's own redistribute_cost while they build their answer; the rows
+    are replaced below (fill_redistribute_cost) and priced by the cost engine,
+    so for the duration of a query they are made of zeros instead: half of the
+    time the propagator takes on a transformer graph."""
+    import sys
+
+    global _cost_row_users, _cost_row_users_at
+    if _cost_row_users_at != len(sys.modules):  # strategy modules are imported lazily
+        _cost_row_users = [mod for name, mod in list(sys.modules.items())
+                           if name.startswith("torch.distributed.tensor._ops") and mod is not None
+                           and "generate_redistribute_costs" in getattr(mod, "__dict__", {})]
+        _cost_row_users_at = len(sys.modules)
+    saved = [(mod, mod.__dict__["generate_redistribute_costs"]) for mod in _cost_row_users]
+    for mod, _ in saved:
+        mod.generate_redistribute_costs = _zero_cost_rows
+    try:
+        yield
+    finally:
+        for mod, fn in saved:
+            mod.generate_redistribute_costs = fn
+
+
 def _placement_options_uncached(mesh, node, producers, arg_vals, schema_args) -> OpStrategy:
+    with _without_torch_cost_rows():
+        return _placement_options_uncached_inner(mesh, node, producers, arg_vals, schema_args)
+
+
+def _placement_options_uncached_inner(mesh, node, producers, arg_vals, schema_args) -> OpStrategy:
     prop = DTensor._op_dispatcher.sharding_propagator
     op = node.target
     if not producers and isinstance(node.meta.get("val"), torch.Tensor):

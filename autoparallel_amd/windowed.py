@@ -32,11 +32,21 @@ import numpy as np
 
 
 def _make_window(task):
+    import gc
+
     from autoparallel_amd import graphgen
 
     n_total, lo, hi, mesh, seed, s_min, s_max = task
-    g, gid, n_standin = graphgen.stress_dag_window(n_total, lo, hi, mesh, seed, s_min, s_max)
-    g.validate()
+    # millions of small objects that all live until the window is packed: the cyclic
+    # collector only walks them over and over (a quarter of the time of a window)
+    was = gc.isenabled()
+    gc.disable()
+    try:
+        g, gid, n_standin = graphgen.stress_dag_window(n_total, lo, hi, mesh, seed, s_min, s_max)
+        g.validate()
+    finally:
+        if was:
+            gc.enable()
     return lo, hi, g, gid, n_standin
 
 
