@@ -476,3 +476,87 @@ def test_flex_attention_strategies(meshes):
         assert [s.placements for s in st.output_specs] == [plc, plc, plc]
         assert [len(r) for r in st.redistribute_cost] == [2] * 6
     assert by_q[(S(0), S(1))].output_specs[1].tensor_meta.shape == (64, 64, 128)
+
+
+def test_flat_args_and_map_nodes_equal_pytree():
+    """The argument walks of the strategy enumeration against torch's pytree on
+    the structures FX arguments have (nested tuples, lists, dicts, slices,
+    repeated nodes, None)."""
+    from torch.utils._pytree import tree_flatten, tree_map_only
+
+    from autoparallel_amd.optimize_sharding import _flat_args, _map_nodes
+
+    g = torch.fx.Graph()
+    a, b = g.placeholder("a"), g.placeholder("b")
+    cases = [
+        (a, b), (a, a, 1.5), ([a, None, b], 2), ((a, [b, (a, 3)]), {"k": b, "j": [a]}), (slice(0, 4, None), a),
+        (), (None,), ("ij,jk->ik", [a, b]),
+    ]
+    for args in cases:
+        node = g.call_function(torch.ops.aten.add.Tensor, args)  # FX turns the lists into immutable ones
+        assert _flat_args(node.args, []) == tree_flatten(node.args)[0]
+        f = lambda n: ("strategy of", n.name)
+        assert _map_nodes(node.args, f) == tree_map_only(torch.fx.Node, f, node.args)
+
+
+def test_torch_cost_rows_are_restored(meshes):
+    """While a query runs torch's strategy functions fill their rows with zeros;
+    afterwards, and after an error inside the query, torch's own function is
+    back in every module that imported it."""
+    import torch.distributed.tensor._ops._matrix_ops as MO
+    import torch.distributed.tensor._ops.utils as OU
+
+    from autoparallel_amd.shardings import placement_options as PO
+
+    real = OU.generate_redistribute_costs
+    assert MO.generate_redistribute_costs is real
+    with PO._without_torch_cost_rows():
+        assert OU.generate_redistribute_costs is PO._zero_cost_rows and MO.generate_redistribute_costs is PO._zero_cost_rows
+        with PO._without_torch_cost_rows():  # nested: the inner exit must not bring the real one back early
+            pass
+        assert MO.generate_redistribute_costs is PO._zero_cost_rows
+    assert OU.generate_redistribute_costs is real and MO.generate_redistribute_costs is real
+    with pytest.raises(KeyError):
+        with PO._without_torch_cost_rows():
+            raise KeyError("inside")
+    assert OU.generate_redistribute_costs is real and MO.generate_redistribute_costs is real
+
+
+def test_strategy_summaries_keep_the_cache_hits(meshes):
+    """A query key holds one token per argument strategy; strategies with the
+    same output specs get the same token wherever they come from, and tokens
+    are not reused after the cache is reset."""
+    from autoparallel_amd.shardings import placement_options as PO
+
+    mesh = meshes[0]
+    R, S = Replicate(), Shard
+    x = _candidates(mesh, (64, 32), [(R, R), (S(0), R)])
+    y = _candidates(mesh, (64, 32), [(R, R), (S(0), R)])  # other objects, same content
+    z = _candidates(mesh, (64, 32), [(R, R), (S(1), R)])
+    assert PO._fingerprint(x) == PO._fingerprint(y) != PO._fingerprint(z)
+    assert PO._fingerprint(PO._copy_strategy(x)) == PO._fingerprint(x)
+    old = PO._fingerprint(x)
+    PO.reset_placement_options_cache()
+    w = _candidates(mesh, (64, 32), [(R, S(1))])
+    assert PO._fingerprint(w) != old  # x still carries `old`; nothing else may get it
+
+
+def test_collector_state_is_restored():
+    import gc
+
+    from autoparallel_amd.optimize_sharding import _gc_paused
+
+    assert gc.isenabled()
+    with _gc_paused():
+        assert not gc.isenabled()
+        with _gc_paused():
+            pass
+        assert not gc.isenabled()
+    assert gc.isenabled()
+    gc.disable()
+    try:
+        with _gc_paused():
+            pass
+        assert not gc.isenabled()  # it was off before: stays off
+    finally:
+        gc.enable()
