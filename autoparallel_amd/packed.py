@@ -719,12 +719,13 @@ class PackedGraph:
     def chunk_edge_index(self) -> np.ndarray:
         """int32[num_slots / 16]: the edge that owns each 16-slot chunk (blocks
         are 16-slot aligned, so a chunk never spans two edges)."""
-        nt = self.num_slots >> CHUNK_SHIFT
-        starts = np.arange(nt, dtype=np.int64) << CHUNK_SHIFT
-        if self.edge_alias is None:
-            return (np.searchsorted(self.edge_off, starts, side="right") - 1).astype(np.int32)
-        own = np.nonzero(self.priced)[0]  # their blocks are laid out in this order
-        return own[np.searchsorted(self.edge_off[:-1][own], starts, side="right") - 1].astype(np.int32)
+        pad = (1 << CHUNK_SHIFT) - 1
+        # an edge that owns a block owns ceil(size / 16) consecutive chunks, in edge order
+        # (the order the blocks are laid out in); an aliased edge owns none
+        chunks = (self.block_sizes() + pad) >> CHUNK_SHIFT
+        out = np.repeat(np.arange(self.num_edges, dtype=np.int32), chunks)
+        assert out.shape[0] == self.num_slots >> CHUNK_SHIFT
+        return out
 
     def work_items(self, compressed: bool = False, item_entries: int = ITEM_ENTRIES) -> np.ndarray:
         """Work items of the entry kernel: for every ``item_entries`` (256 or 512)
