@@ -38,6 +38,13 @@ __device__ __forceinline__ apc_edge load_edge(const apc_edge* __restrict__ e) {
   return u.ed;
 }
 
+typedef int32_t i32x4_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ apc_score_edge_aux load_aux(const apc_score_edge_aux* __restrict__ a) {
+  union { i32x4_t raw; apc_score_edge_aux aux; } u;
+  u.raw = *reinterpret_cast<const i32x4_t*>(a);
+  return u.aux;
+}
+
 template <bool kRandom>
 __global__ void __launch_bounds__(kBlock)
 score_kernel(apc_problem p, const double* __restrict__ per_arg, const double* __restrict__ comm,
@@ -421,7 +428,7 @@ __device__ __forceinline__ void copy4_to_lds(const int32_t* __restrict__ src, ui
 template <bool kRandom, int kPer>
 __global__ void __launch_bounds__(kTableBlock)
 score_table_kernel(apc_problem p, const double* __restrict__ per_arg, const double* __restrict__ table,
-                   const int32_t* __restrict__ edge_msize, const int32_t* __restrict__ next_staged,
+                   const apc_score_edge_aux* __restrict__ edge_aux,
                    const uint16_t* __restrict__ assign, int64_t stride, uint64_t seed, int64_t first,
                    int64_t n_assign, const int32_t* __restrict__ node_gid, int first_node, int end_node,
                    int clamp_inf, const double* __restrict__ init, double* __restrict__ out) {
@@ -456,9 +463,10 @@ score_table_kernel(apc_problem p, const double* __restrict__ per_arg, const doub
     h ^= (uint32_t)(ua >> 32) * 0x85EBCA77u;
     h0[k] = h;
   }
-  auto choice = [&](int k, int v, int nstrat) -> uint32_t {
+  // the choice of assignment k at node v, whose id for the draw is gid
+  auto choice = [&](int k, int v, int gid, int nstrat) -> uint32_t {
     if (!kRandom) return (uint32_t)assign[(size_t)v * stride + asg(k)];
-    uint32_t h = h0[k] ^ ((uint32_t)((node_gid ? node_gid[v] : v) + 1) * 0xC2B2AE3Du);
+    uint32_t h = h0[k] ^ ((uint32_t)(gid + 1) * 0xC2B2AE3Du);
     h ^= h >> 16;
     h *= 0x85EBCA6Bu;
     h ^= h >> 13;
@@ -486,12 +494,19 @@ score_table_kernel(apc_problem p, const double* __restrict__ per_arg, const doub
   };
   const int e_begin = first_node < end_node ? p.node_edge_off[first_node] : 0;
   const int e_end = first_node < end_node ? p.node_edge_off[end_node] : 0;
+  // The record of an edge and what else the walk needs to know about it (apc_score_edge_aux)
+  // are requested one edge ahead, so that an edge starts with everything in scalar registers.
   apc_edge nxt;
-  if (e_begin < e_end) nxt = load_edge(p.edges + e_begin);
+  apc_score_edge_aux aux_nxt = {0, -1, 0, 0};
+  if (e_begin < e_end) {
+    nxt = load_edge(p.edges + e_begin);
+    aux_nxt = load_aux(edge_aux + e_begin);
+  }
   int buf = 0;
   {
-    const int s0 = e_begin < e_end ? next_staged[e_begin] : -1;  // the first edge that goes through LDS
-    if (s0 >= 0 && s0 < e_end) issue(s0 == e_begin ? nxt : load_edge(p.edges + s0), edge_msize[s0], 0, buf);
+    const int s0 = aux_nxt.next_staged;  // the first edge that goes through LDS
+    if (s0 >= 0 && s0 < e_end)
+      issue(s0 == e_begin ? nxt : load_edge(p.edges + s0), s0 == e_begin ? aux_nxt.msize : edge_aux[s0].msize, 0, buf);
   }
   for (int v = first_node; v < end_node; ++v) {
     const int nstrat = p.node_nstrat[v];
@@ -503,29 +518,33 @@ score_table_kernel(apc_problem p, const double* __restrict__ per_arg, const doub
     double pa[kPer];
 #pragma unroll
     for (int k = 0; k < kPer; ++k) {
-      o[k] = choice(k, v, nstrat);
+      o[k] = choice(k, v, node_gid ? node_gid[v] : v, nstrat);
       pa[k] = per_arg[comp_off + o[k]];
     }
 #pragma unroll
     for (int k = 0; k < kPer; ++k) t_compute[k] += pa[k] * fargs;
     for (int e = p.node_edge_off[v]; e < p.node_edge_off[v + 1]; ++e) {
       const apc_edge ed = nxt;
+      const apc_score_edge_aux aux = aux_nxt;
       if (e + 1 < e_end) nxt = load_edge(p.edges + e + 1);
-      const int msize = edge_msize[e];  // elements that go through LDS; 0: read the matrix in place
+      aux_nxt = load_aux(edge_aux + e + 1);  // the list ends with a record of its own
+      const int msize = aux.msize;  // elements that go through LDS; 0: read the matrix in place
       const bool has_src = ed.src_node >= 0;
       const bool squeezed = (ed.flags & APC_EDGE_COMPRESSED) != 0;
       const uint32_t usrc = (uint32_t)ed.flags >> APC_EDGE_USRC_SHIFT;
       uint32_t j[kPer], at[kPer];
 #pragma unroll
-      for (int k = 0; k < kPer; ++k) j[k] = has_src ? choice(k, ed.src_node, ed.ssrc) : 0u;
+      for (int k = 0; k < kPer; ++k) j[k] = has_src ? choice(k, ed.src_node, aux.src_gid, ed.ssrc) : 0u;
       double raw[kPer];
       if (msize > 0) {  // uniform over the workgroup, as everything that decides a barrier below
         const double* const mat = s_all + buf * kTileDoubles;
         __builtin_amdgcn_s_waitcnt(0);  // this lane's part of the first tile has arrived,
         __syncthreads();                // and everyone's; and the draws of the edge before are done,
         {                               // so its buffer can take the next matrix
-          const int s1 = next_staged[e + 1];
-          if (s1 >= 0 && s1 < e_end) issue(s1 == e + 1 ? nxt : load_edge(p.edges + s1), edge_msize[s1], 0, buf ^ 1);
+          const int s1 = aux_nxt.next_staged;
+          if (s1 >= 0 && s1 < e_end)
+            issue(s1 == e + 1 ? nxt : load_edge(p.edges + s1), s1 == e + 1 ? aux_nxt.msize : edge_aux[s1].msize, 0,
+                  buf ^ 1);
         }
         if (squeezed && lists_staged(ed)) {
           const int32_t* const ud = s_lists + (buf * 2 + 0) * kListInts;
@@ -601,7 +620,7 @@ score_table_kernel(apc_problem p, const double* __restrict__ per_arg, const doub
 
 template <bool kRandom, int kPer>
 int launch_table_k(dim3 grid, hipStream_t stream, const apc_problem& p, const double* per_arg, const double* table,
-                   const int32_t* edge_msize, const int32_t* next_staged, const uint16_t* assign, int64_t stride,
+                   const apc_score_edge_aux* edge_aux, const uint16_t* assign, int64_t stride,
                    uint64_t seed, int64_t first, int64_t n_assign, const int32_t* node_gid, int first_node,
                    int end_node, int clamp_inf, const double* init, double* out) {
   // dynamic LDS beyond 64 KB needs the limit raised, per kernel and device; cheap enough to do per launch
@@ -609,7 +628,7 @@ int launch_table_k(dim3 grid, hipStream_t stream, const apc_problem& p, const do
                                      hipFuncAttributeMaxDynamicSharedMemorySize, kTableLds);
   if (e != hipSuccess) return fail(APC_ERR_LAUNCH, "hipFuncSetAttribute(score_table_kernel): %s", hipGetErrorString(e));
   hipLaunchKernelGGL((score_table_kernel<kRandom, kPer>), grid, dim3(kTableBlock), kTableLds, stream, p, per_arg,
-                     table, edge_msize, next_staged, assign, stride, seed, first, n_assign, node_gid, first_node,
+                     table, edge_aux, assign, stride, seed, first, n_assign, node_gid, first_node,
                      end_node, clamp_inf, init, out);
   return check_launch("score_table_kernel");
 }
@@ -878,13 +897,13 @@ int apc_score_compact(const apc_problem* p, const double* per_arg, const apc_sco
 int apc_score_table_tile(void) { return kTileDoubles; }
 
 int apc_score_table(const apc_problem* p, const double* per_arg, const double* table,
-                    const int32_t* edge_msize, const int32_t* next_staged, const uint16_t* assign,
+                    const apc_score_edge_aux* edge_aux, const uint16_t* assign,
                     uint64_t seed, int64_t first, int64_t n_assign, const int32_t* node_gid,
                     int32_t first_node, int32_t end_node, int32_t clamp_inf, int32_t per_lane,
                     const double* init, double* out, void* stream) {
   if (int rc = validate_problem(p)) return rc;
   if (n_assign <= 0) return 0;
-  if (!per_arg || !edge_msize || !next_staged || !out || !p->node_multiplier || (p->table_size > 0 && !table))
+  if (!per_arg || !edge_aux || !out || !p->node_multiplier || (p->table_size > 0 && !table))
     return fail(APC_ERR_INVALID, "apc_score_table: null argument%s");
   if (first_node < 0 || first_node > end_node || end_node > p->n_node)
     return fail(APC_ERR_INVALID, "apc_score_table: need 0 <= first_node <= end_node <= n_node%s");
@@ -899,10 +918,10 @@ int apc_score_table(const apc_problem* p, const double* per_arg, const double* t
     const int64_t lanes = (n + per - 1) / per;
     const dim3 grid((unsigned)((lanes + kTableBlock - 1) / kTableBlock));
     const double* in = init ? init + a0 * 6 : nullptr;
-    int rc = assign ? launch_table<false>(per, grid, (hipStream_t)stream, *p, per_arg, table, edge_msize, next_staged,
+    int rc = assign ? launch_table<false>(per, grid, (hipStream_t)stream, *p, per_arg, table, edge_aux,
                                           assign + a0, n_assign, seed, first + a0, n, node_gid, (int)first_node,
                                           (int)end_node, (int)clamp_inf, in, out + a0 * 6)
-                    : launch_table<true>(per, grid, (hipStream_t)stream, *p, per_arg, table, edge_msize, next_staged,
+                    : launch_table<true>(per, grid, (hipStream_t)stream, *p, per_arg, table, edge_aux,
                                          assign, n_assign, seed, first + a0, n, node_gid, (int)first_node,
                                          (int)end_node, (int)clamp_inf, in, out + a0 * 6);
     if (rc) return rc;

@@ -554,11 +554,11 @@ class CostEngine:
         when the records are made); else the 32-byte records that carry the cost
         (apc_score_packed)."""
         if self._table_clamp is not None and _SCORE_FROM_TABLE and (self.large_blocks or not _SCORE_COMPACT):
-            msize, next_staged = self._score_msize()
+            aux = self._score_edge_aux(d_gid)
             _lib.check(
                 self.lib.apc_score_table(
                     C.byref(self.problem), self._ptr(self.per_arg), self._ptr(self.table),
-                    C.c_void_p(msize.data_ptr()), C.c_void_p(next_staged.data_ptr()), self._ptr(assign),
+                    C.c_void_p(aux.data_ptr()), self._ptr(assign),
                     int(seed), int(first), int(count), self._ptr(d_gid), int(first_node), self.g.num_nodes,
                     self._table_clamp, min(_SCORE_PER_LANE, 4),
                     self._ptr(init), self._ptr(out), self._stream()),
@@ -606,26 +606,41 @@ class CostEngine:
         self.last_score_backend = "records"
         return out
 
-    def _score_msize(self):
-        """(edge_msize, next_staged) of apc_score_table: the padded size of an
-        edge's matrix in the block table if it is worth taking through LDS (eight
-        tiles at most), and the first such edge from each edge on."""
-        hit = self._keep.get("score_msize")
-        if hit is None:
-            g = self.g
-            _, block_off, _, edge_table_off, _, _ = g.block_table(self.table_mode == "compressed")
-            msize = np.zeros(g.num_edges, np.int32)
-            has = edge_table_off >= 0
-            b = np.searchsorted(block_off, edge_table_off[has], side="right") - 1
-            size = (block_off[b + 1] - block_off[b]).astype(np.int64)
-            limit = _SCORE_STAGE_TILES * int(self.lib.apc_score_table_tile())
-            msize[has] = np.where(size <= limit, size, 0).astype(np.int32)
+    def _score_msize(self) -> np.ndarray:
+        """int32[num_edges]: the padded size of an edge's matrix in the block table
+        if it is worth taking through LDS (_SCORE_STAGE_TILES tiles at most), else 0."""
+        g = self.g
+        _, block_off, _, edge_table_off, _, _ = g.block_table(self.table_mode == "compressed")
+        msize = np.zeros(g.num_edges, np.int32)
+        has = edge_table_off >= 0
+        b = np.searchsorted(block_off, edge_table_off[has], side="right") - 1
+        size = (block_off[b + 1] - block_off[b]).astype(np.int64)
+        limit = _SCORE_STAGE_TILES * int(self.lib.apc_score_table_tile())
+        msize[has] = np.where(size <= limit, size, 0).astype(np.int32)
+        return msize
+
+    def _score_edge_aux(self, d_gid: Optional[torch.Tensor]) -> torch.Tensor:
+        """apc_score_edge_aux records of apc_score_table (int32[num_edges + 1, 4] on
+        the device): what does not depend on the call is made once; the producers'
+        ids for the draw follow the call's node ids."""
+        g = self.g
+        base = self._keep.get("score_edge_aux")
+        if base is None:
+            msize = self._score_msize()
             idx = np.where(msize > 0, np.arange(g.num_edges), g.num_edges)
             nxt = np.minimum.accumulate(np.concatenate([idx, [g.num_edges]])[::-1])[::-1]
-            next_staged = np.where(nxt < g.num_edges, nxt, -1).astype(np.int32)
-            hit = self._keep["score_msize"] = (torch.from_numpy(msize).to(self.device),
-                                               torch.from_numpy(next_staged).to(self.device))
-        return hit
+            aux = np.zeros((g.num_edges + 1, 4), np.int32)
+            aux[:-1, 0] = msize
+            aux[:, 1] = np.where(nxt < g.num_edges, nxt, -1)
+            aux[:-1, 2] = g.edge_src_node
+            base = self._keep["score_edge_aux"] = torch.from_numpy(aux).to(self.device)
+            self._keep["score_edge_src"] = torch.from_numpy(
+                np.maximum(g.edge_src_node, 0).astype(np.int64)).to(self.device)
+        if d_gid is None:
+            return base
+        aux = base.clone()
+        aux[:-1, 2] = d_gid[self._keep["score_edge_src"]]
+        return aux
 
     def node_hashes(self, node_phase: Optional[np.ndarray] = None) -> np.ndarray:
         """uint64[n_node] structural hash of every node (the clustering key).

@@ -637,6 +637,21 @@ int apc_score_compact(const apc_problem* p, const double* per_arg, const apc_sco
                       const int32_t* node_gid, int32_t first_node, int32_t end_node, int32_t per_lane,
                       const double* init, double* out, void* stream);
 
+/* What the table scorer needs to know about an edge beside its apc_edge record,
+ * in one 16-byte load. */
+typedef struct apc_score_edge_aux {
+  int32_t msize;       /* elements of the edge's matrix to take through LDS, tile by tile
+                          (apc_score_table_tile() elements a tile): even, and only for an
+                          edge with table_off >= 0 (the matrix's padded size in the table
+                          will do); 0: read the matrix in place (no matrix: default rows;
+                          or too large to be worth it)                                   */
+  int32_t next_staged; /* the first edge >= this one with msize > 0, or -1            */
+  int32_t src_gid;     /* id of the producer node for the draw: node_gid[src_node], or
+                          src_node itself when the draw uses local ids; unused without
+                          a producer                                                  */
+  int32_t reserved;
+} apc_score_edge_aux; /* 16 bytes */
+
 /* The same sums from the block table instead of the entry arrays, for graphs
  * with large blocks: an entry is (|m| + per_arg) + transition with the flag in
  * the sign of its matrix element m, clamped to 10000 if clamp_inf and not finite
@@ -644,15 +659,10 @@ int apc_score_compact(const apc_problem* p, const double* per_arg, const apc_sco
  * bit, that of apc_score_packed on the arrays of a build with this clamp_inf.
  * One workgroup of 1024 lanes per CU, per_lane assignments each (1, 2, 4; 0:
  * chosen), has the current edge's matrix in LDS and draws from there.
- * edge_msize[e] (device, int32[n_edge]): the number of elements of edge e's
- * matrix to take through LDS, tile by tile (apc_score_table_tile() elements a
- * tile): even, and only for an edge with table_off >= 0 (the matrix's padded
- * size in the table will do); or 0 to read the matrix in place (no matrix:
- * default rows; or too large to be worth it).  next_staged[e] (device,
- * int32[n_edge + 1]): the first edge >= e with edge_msize > 0, or -1.  table as
+ * edge_aux (device): n_edge + 1 records, the last one {0, -1, 0, 0}.  table as
  * for apc_edge_costs; p carries list_uidx if it has compressed matrices. */
 int apc_score_table(const apc_problem* p, const double* per_arg, const double* table,
-                    const int32_t* edge_msize, const int32_t* next_staged, const uint16_t* assign,
+                    const apc_score_edge_aux* edge_aux, const uint16_t* assign,
                     uint64_t seed, int64_t first, int64_t n_assign, const int32_t* node_gid,
                     int32_t first_node, int32_t end_node, int32_t clamp_inf, int32_t per_lane,
                     const double* init, double* out, void* stream);

@@ -71,8 +71,8 @@ def test_every_backend_gives_the_sums_of_the_entry_arrays(knobs, name, table_mod
         E._SCORE_FROM_TABLE = True
         for tiles, per in ((8, 0), (0, 4), (1, 2), (64, 4), (8, 1)):
             E._SCORE_STAGE_TILES, E._SCORE_PER_LANE = tiles, per
-            eng._keep.pop("score_msize", None)
-            msize = eng._score_msize()[0].cpu().numpy()
+            eng._keep.pop("score_edge_aux", None)
+            msize = eng._score_msize()
             if name == "stress" and tiles in (8, 64):
                 tile = int(eng.lib.apc_score_table_tile())
                 assert (msize > tile).any() and (msize > 0).any()  # several tiles do occur
