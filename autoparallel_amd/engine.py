@@ -18,6 +18,8 @@ _TABLE_MAX_RATIO = 0.5
 _TABLE_MAX_DOUBLES = 1 << 28
 _WIDE_ITEMS_FROM = 32_000_000  # entries
 _LARGE_BLOCKS_FROM = 8192  # mean entries per edge block
+_UPLOAD_ARENA_BYTES = 8 << 20  # descriptor arrays of one problem that go up in one copy
+_UPLOAD_ARENA_MAX_ARRAY = 2 << 20
 _SCORE_LANES_FROM = 32768  # assignments: below, one wavefront per assignment (entry arrays as they are)
 _SCORE_FROM_TABLE = True  # the three ways of scoring a graph with large blocks can be switched off (tests do)
 _SCORE_COMPACT = True
@@ -112,6 +114,19 @@ def upload_nccl_plan(model: _lib.ApcModel, cfg, device) -> torch.Tensor:
     return t
 
 
+_stage_buffer: Optional[torch.Tensor] = None
+
+
+def _upload_stage(nbytes: int) -> torch.Tensor:
+    """Pinned staging buffer of the upload arena, kept between engines (pinning
+    memory costs more than the copy it serves); an engine is done with it when
+    its constructor returns."""
+    global _stage_buffer
+    if _stage_buffer is None or _stage_buffer.numel() < nbytes:
+        _stage_buffer = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, pin_memory=True)
+    return _stage_buffer
+
+
 def detect_device_name(device=None) -> str:
     """Marketing name of the HIP device, as the reference's device table keys
     on it (autoparallel/cost_models/compute_estimation.py:258-275).  Hosts
@@ -169,16 +184,42 @@ class CostEngine:
 
         self._keep: Dict[str, torch.Tensor] = {}
 
+        # The problem is some thirty arrays, most of them a few kilobytes: they go up in
+        # one copy.  An array is laid into a pinned staging buffer and gets its address
+        # inside a device arena at once (the struct fields below need it); the arena is
+        # filled by _flush_uploads when all of them are known.  Large arrays (and what
+        # does not fit any more) are copied on their own.
+        arena_bytes = int(min(_UPLOAD_ARENA_BYTES, (256 << 10) + 32 * g.lists.shape[0] + 160 * g.num_edges
+                              + 320 * g.num_nodes + 8 * g.default_vals.shape[0]))
+        stage = _upload_stage(arena_bytes)
+        arena = torch.empty(arena_bytes, dtype=torch.uint8, device=self.device)
+        stage_np = stage.numpy()
+        used = [0]
+
         def up(name, arr, dtype=None):
             a = np.ascontiguousarray(arr if dtype is None else arr.astype(dtype))
             if a.dtype == np.uint32:
-                t = torch.from_numpy(a.view(np.int32)).to(self.device)
-            elif a.dtype.fields is not None:
-                t = torch.from_numpy(a.view(np.uint8)).to(self.device)
+                a = a.view(np.int32)
+            raw = a.reshape(-1).view(np.uint8) if a.dtype.fields is None else a.view(np.uint8).reshape(-1)
+            n = raw.shape[0]
+            off = (used[0] + 255) & ~255
+            if n == 0 or n > _UPLOAD_ARENA_MAX_ARRAY or off + n > arena_bytes:
+                t = torch.from_numpy(raw if a.dtype.fields is not None else a).to(self.device)
             else:
-                t = torch.from_numpy(a).to(self.device)
+                stage_np[off:off + n] = raw
+                used[0] = off + n
+                t = arena[off:off + n]
+                if a.dtype.fields is None:
+                    t = t.view(torch.from_numpy(a[:0].reshape(-1)).dtype).view(a.shape)
             self._keep[name] = t
             return t.data_ptr() if t.numel() else None
+
+        def flush_uploads():
+            if used[0]:
+                arena[:used[0]].copy_(stage[:used[0]], non_blocking=True)
+                # the staging buffer is let go once the copy has run
+                torch.cuda.current_stream(self.device).synchronize()
+            self._keep["upload_arena"] = arena
 
         p = _lib.ApcProblem()
         model = make_model([int(x) for x in g.mesh_shape], g.devices_per_host, device_name, order_mode,
@@ -286,6 +327,7 @@ class CostEngine:
         if self.lut and g.num_entries > 0:
             tiles = g.lut_tiles(squeezed, entries=(table_mode == "direct"))
             self._lut_tiles = (up("lut_tiles", tiles), int(tiles.shape[0]))
+        flush_uploads()
 
         E, NC = (g.num_slots, g.num_compute) if allocate_results else (0, 0)
         self.can_build = bool(allocate_results)

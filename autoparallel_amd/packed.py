@@ -732,6 +732,9 @@ class PackedGraph:
         entries of every edge block a copy of the edge record with ``local0``
         set, in slot order."""
         assert item_entries in (ITEM_ENTRIES, 2 * ITEM_ENTRIES)
+        cache = self.__dict__.setdefault("_work_items", {})  # as the block table: made once per layout
+        if (compressed, item_entries) in cache:
+            return cache[(compressed, item_entries)]
         sizes = self.block_sizes()
         n = (sizes + item_entries - 1) // item_entries
         eid = np.repeat(np.arange(self.num_edges, dtype=np.int64), n)
@@ -739,6 +742,7 @@ class PackedGraph:
         k = np.arange(int(n.sum()), dtype=np.int64) - start[eid]
         items = self.edge_records(compressed)[eid]
         items["local0"] = k * item_entries
+        cache[(compressed, item_entries)] = items
         return items
 
     def validate(self) -> None:
