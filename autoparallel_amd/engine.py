@@ -4,6 +4,7 @@ current HIP stream."""
 from __future__ import annotations
 
 import ctypes as C
+import threading
 from typing import Dict, Optional
 
 import numpy as np
@@ -114,17 +115,17 @@ def upload_nccl_plan(model: _lib.ApcModel, cfg, device) -> torch.Tensor:
     return t
 
 
-_stage_buffer: Optional[torch.Tensor] = None
+_stage = threading.local()  # .buffer: this thread's pinned staging buffer
 
 
 def _upload_stage(nbytes: int) -> torch.Tensor:
-    """Pinned staging buffer of the upload arena, kept between engines (pinning
-    memory costs more than the copy it serves); an engine is done with it when
-    its constructor returns."""
-    global _stage_buffer
-    if _stage_buffer is None or _stage_buffer.numel() < nbytes:
-        _stage_buffer = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, pin_memory=True)
-    return _stage_buffer
+    """Pinned staging buffer of the upload arena, kept between the engines a
+    thread makes (pinning memory costs more than the copy it serves); an engine
+    is done with it when its copy has run, before its constructor returns."""
+    buf = getattr(_stage, "buffer", None)
+    if buf is None or buf.numel() < nbytes:
+        buf = _stage.buffer = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, pin_memory=True)
+    return buf
 
 
 def detect_device_name(device=None) -> str:
