@@ -34,7 +34,7 @@ def workloads():
     from autoparallel_amd import graphgen as G
 
     return {
-        # BASELINE.json configs[1]: the configuration the metric is quoted on
+        # the configuration the metric is quoted on
         "llama3_8b_fwd_bwd_mesh8x8": lambda: G.config_llama3_8b(),
         # configs[0]
         "gpt2_small_fwd_bwd_mesh8": lambda: G.config_gpt2_small(),

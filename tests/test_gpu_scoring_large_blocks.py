@@ -177,3 +177,60 @@ def test_twelve_thousand_nodes_in_four_windows():
     eng.packed_scoring = False  # and the one pass over the entry arrays themselves
     plain = eng.score_random(seed=1, first=0, count=n_assign).cpu().numpy()
     assert (plain.view(np.uint64) == whole.view(np.uint64)).all()
+
+
+def test_small_batches_and_node_ranges(knobs):
+    """A batch smaller than a workgroup, and the walk cut into node ranges through
+    the C entry points (sums continued from the previous range's result): the
+    sums of one walk, bit for bit."""
+    import ctypes as C
+
+    from autoparallel_amd import _lib
+
+    E = knobs
+    g = GRAPHS["stress"]()
+    eng = E.CostEngine(g).build(clamp_inf=True)
+    gid = np.arange(g.num_nodes, dtype=np.int32) * 3 + 5
+    for n in (1, 7, 1000):
+        eng.packed_scoring = False
+        want = eng.score_random_window(3, 11, n, gid, 0)
+        eng.packed_scoring = True
+        for from_table in (True, False):
+            E._SCORE_FROM_TABLE = from_table
+            assert _same(eng.score_random_window(3, 11, n, gid, 0), want), (n, from_table)
+            assert eng.last_score_backend == ("block_table" if from_table else "compact_records")
+    # node ranges [0, a), [a, b), [b, N) chained through init
+    n = 5000
+    eng.packed_scoring = False
+    want = eng.score_random_window(3, 0, n, gid, 0)
+    d_gid = torch.from_numpy(gid).cuda()
+    aux = eng._score_edge_aux(d_gid)
+    cuts = [0, g.num_nodes // 3, g.num_nodes // 3 + 1, 2 * g.num_nodes // 3, g.num_nodes]
+    out = torch.empty(n, 6, dtype=torch.float64, device="cuda")
+    prev = None
+    for lo, hi in zip(cuts[:-1], cuts[1:]):
+        _lib.check(eng.lib.apc_score_table(
+            C.byref(eng.problem), eng._ptr(eng.per_arg), eng._ptr(eng.table), C.c_void_p(aux.data_ptr()), None,
+            3, 0, n, eng._ptr(d_gid), lo, hi, 1, 0, eng._ptr(prev), eng._ptr(out), eng._stream()), "apc_score_table")
+        prev = out
+    assert _same(out, want)
+    E._SCORE_FROM_TABLE = False
+    eng.packed_scoring = True
+    eng.score_random(1, 0, 40000)  # makes the compact records
+    assert eng._recs_compact
+    prev = None
+    for lo, hi in zip(cuts[:-1], cuts[1:]):
+        _lib.check(eng.lib.apc_score_compact(
+            C.byref(eng.problem), eng._ptr(eng.per_arg), eng._ptr(eng._recs), None, 3, 0, n, eng._ptr(d_gid), lo, hi,
+            2, eng._ptr(prev), eng._ptr(out), eng._stream()), "apc_score_compact")
+        prev = out
+    assert _same(out, want)
+    # argument checks
+    rc = eng.lib.apc_score_table(C.byref(eng.problem), eng._ptr(eng.per_arg), eng._ptr(eng.table),
+                                 C.c_void_p(aux.data_ptr()), None, 3, 0, n, None, 5, 4, 1, 0, None, eng._ptr(out),
+                                 eng._stream())
+    assert rc == -1 and b"first_node" in eng.lib.apc_last_error()
+    rc = eng.lib.apc_score_table(C.byref(eng.problem), eng._ptr(eng.per_arg), eng._ptr(eng.table),
+                                 C.c_void_p(aux.data_ptr()), None, 3, 0, n, None, 0, g.num_nodes, 1, 3, None,
+                                 eng._ptr(out), eng._stream())
+    assert rc == -1 and b"per_lane" in eng.lib.apc_last_error()
