@@ -447,14 +447,16 @@ score_table_kernel(apc_problem p, const double* __restrict__ per_arg, const doub
     const int64_t ak = t_raw + k * lanes;
     return ak < n_assign ? ak : t;
   };
-  double t_compute[kPer], t_comm[kPer], t_trans[kPer], obj[kPer], forbidden[kPer];
-  uint32_t h0[kPer];
+  // t_trans and forbidden only ever grow by ones: counted in integers and added to the
+  // carried sums at the end, exactly as the ones would have been (see below)
+  double t_compute[kPer], t_comm[kPer], obj[kPer];
+  uint32_t n_trans[kPer], n_forbidden[kPer], h0[kPer];
 #pragma unroll
   for (int k = 0; k < kPer; ++k) {
-    t_compute[k] = 0.0; t_comm[k] = 0.0; t_trans[k] = 0.0; obj[k] = 0.0; forbidden[k] = 0.0;
+    t_compute[k] = 0.0; t_comm[k] = 0.0; obj[k] = 0.0; n_trans[k] = 0; n_forbidden[k] = 0;
     if (init) {
       const double* r = init + asg(k) * 6;
-      t_compute[k] = r[1]; t_comm[k] = r[2]; t_trans[k] = r[3]; obj[k] = r[4]; forbidden[k] = r[5];
+      t_compute[k] = r[1]; t_comm[k] = r[2]; obj[k] = r[4];
     }
     // the part of mix_assignment that does not depend on the node
     const uint64_t ua = (uint64_t)(first + asg(k));
@@ -598,23 +600,37 @@ score_table_kernel(apc_problem p, const double* __restrict__ per_arg, const doub
         const bool finite = isfinite(c);
         if (clamp_inf && !finite) c = 10000.0;
         obj[k] += c * mult;
-        forbidden[k] += (double)!finite;
+        n_forbidden[k] += finite ? 0u : 1u;
         if (has_src && isfinite(cm)) t_comm[k] += cm;
-        if (count_trans && trans) t_trans[k] += 1.0;
+        n_trans[k] += count_trans ? trans : 0u;
       }
     }
   }
   __builtin_amdgcn_s_waitcnt(0);  // nothing is in flight towards LDS when the workgroup ends
+  // x + 1.0 n times over.  While x is a whole number below 2^52 every step is exact, and so
+  // is x + n in one step (what the carried sums are in practice: counts); anything else is
+  // added one by one, as the other scorers do.
+  auto add_ones = [](double x, uint32_t n) -> double {
+    if (x == floor(x) && fabs(x) < 4503599627370496.0 - 4294967296.0) return x + (double)n;
+    for (uint32_t i = 0; i < n; ++i) x += 1.0;
+    return x;
+  };
 #pragma unroll
   for (int k = 0; k < kPer; ++k) {
     if (t_raw + k * lanes >= n_assign) continue;
+    const double t_trans = add_ones(init ? init[asg(k) * 6 + 3] : 0.0, n_trans[k]);
+    // the other scorers add 0.0 or 1.0 for every edge: what an edge without a forbidden
+    // entry adds changes nothing, except the sign of a carried -0.0
+    double forbidden = init ? init[asg(k) * 6 + 5] : 0.0;
+    if (e_end > e_begin) forbidden += 0.0;
+    forbidden = add_ones(forbidden, n_forbidden[k]);
     double* r = out + asg(k) * 6;
-    r[0] = (t_compute[k] + t_comm[k]) + t_trans[k];
+    r[0] = (t_compute[k] + t_comm[k]) + t_trans;
     r[1] = t_compute[k];
     r[2] = t_comm[k];
-    r[3] = t_trans[k];
+    r[3] = t_trans;
     r[4] = obj[k];
-    r[5] = forbidden[k];
+    r[5] = forbidden;
   }
 }
 
