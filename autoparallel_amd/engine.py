@@ -783,12 +783,15 @@ class CostEngine:
 
     # -- results on host --------------------------------------------------------
     def results(self) -> Dict[str, np.ndarray]:
-        torch.cuda.synchronize(self.device)
+        """The five result arrays on the host.  They are copied into pinned memory
+        (torch keeps freed pinned blocks, so only a process's first call pays for
+        pinning) by copies that run back to back; the arrays returned own it."""
         self.check_status()
-        return {
-            "comm": self.comm.cpu().numpy(),
-            "cost": self.cost.cpu().numpy(),
-            "flags": self.flags.cpu().numpy(),
-            "compute": self.compute.cpu().numpy(),
-            "per_arg": self.per_arg.cpu().numpy(),
-        }
+        out = {}
+        for name in ("comm", "cost", "flags", "compute", "per_arg"):
+            src = getattr(self, name)
+            dst = torch.empty(src.shape, dtype=src.dtype, pin_memory=True)
+            dst.copy_(src, non_blocking=True)
+            out[name] = dst
+        torch.cuda.current_stream(self.device).synchronize()
+        return {k: v.numpy() for k, v in out.items()}

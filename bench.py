@@ -425,6 +425,13 @@ def _fx_path_figure(n_layers: int, cpu_port: bool) -> dict:
         with contextlib.ExitStack() as stack:
             gm = aot_export_joint_with_descriptors(stack, m, (ids,)).graph_module
     t_trace = time.perf_counter() - t0
+    # as the reference prepares its joint graph before planning (autoparallel/api.py:208):
+    # linear layers become einsums, so that batch and sequence can be sharded separately
+    from autoparallel_amd.graph_utils import replace_view_mm_view_with_einsum
+
+    t0 = time.perf_counter()
+    n_einsum = replace_view_mm_view_with_einsum(gm)
+    t_rewrite = time.perf_counter() - t0
     own = not dist.is_initialized()
     if own:
         dist.init_process_group("fake", store=FakeStore(), rank=0, world_size=64)
@@ -480,6 +487,8 @@ def _fx_path_figure(n_layers: int, cpu_port: bool) -> dict:
             "workload": f"transformers LlamaForCausalLM, Llama-3-8B dimensions, {n_layers} layers, bf16, "
                         f"batch 64 x 8192, joint graph, mesh (8,8)",
             "trace_s": t_trace,
+            "linear_layers_as_einsums": n_einsum,
+            "einsum_rewrite_s": t_rewrite,
             "all_nodes": leg(False),
             "cluster_roots_only": leg(True),
         }

@@ -1065,3 +1065,92 @@ def test_local_map_region_in_a_graph(mesh):
     sol = opt.get_solution()
     assert sol[h].output_specs.placements == (Shard(0), Replicate())
     assert sol[r].output_specs.placements == (Shard(0), Replicate())
+
+
+def test_hf_llama_linears_as_einsums():
+    """Two layers of the traced Llama-3-8B with its linear layers rewritten as
+    einsums, the way the reference prepares a joint graph before planning
+    (autoparallel/api.py:208): no matmul is left, the einsums are offered
+    strategies that shard batch and sequence on different mesh dims, nothing
+    falls back, and every coefficient equals the oracle's."""
+    transformers = pytest.importorskip("transformers")
+    import torch.distributed as dist
+    from torch._functorch.aot_autograd import aot_export_joint_with_descriptors
+    from torch._subclasses.fake_tensor import FakeTensorMode
+    from torch.distributed.device_mesh import init_device_mesh
+    from torch.distributed.tensor.placement_types import Shard
+    from torch.testing._internal.distributed.fake_pg import FakeStore
+
+    from autoparallel_amd.graph_utils import replace_view_mm_view_with_einsum
+    from autoparallel_amd.optimize_sharding import ShardingOptimizer
+    from autoparallel_amd.shardings import placement_options as PO
+
+    if not torch.cuda.is_available():
+        pytest.skip("needs a GPU")
+
+    class Wrap(nn.Module):
+        def __init__(self, lm):
+            super().__init__()
+            self.lm = lm
+
+        def forward(self, ids):
+            m = self.lm.model
+            x = m.embed_tokens(ids)
+            pos = torch.arange(ids.shape[1], device=ids.device)[None]
+            pe = m.rotary_emb(x, pos)
+            for layer in m.layers:
+                out = layer(x, attention_mask=None, position_ids=pos, position_embeddings=pe)
+                x = out[0] if isinstance(out, tuple) else out
+            logits = self.lm.lm_head(m.norm(x))
+            return torch.nn.functional.cross_entropy(
+                logits[:, :-1].reshape(-1, logits.shape[-1]).float(), ids[:, 1:].reshape(-1))
+
+    n_layers = 2
+    cfg = transformers.LlamaConfig(
+        vocab_size=128256, hidden_size=4096, intermediate_size=14336, num_hidden_layers=n_layers,
+        num_attention_heads=32, num_key_value_heads=8, max_position_embeddings=8192, rope_theta=500000.0,
+        attention_dropout=0.0, use_cache=False, attn_implementation="sdpa")
+    with FakeTensorMode():
+        torch.set_default_dtype(torch.bfloat16)
+        try:
+            with torch.device("cuda"):
+                m = Wrap(transformers.LlamaForCausalLM(cfg))
+        finally:
+            torch.set_default_dtype(torch.float32)
+        ids = torch.randint(0, cfg.vocab_size, (64, 8192), device="cuda")
+        with contextlib.ExitStack() as stack:
+            gm = aot_export_joint_with_descriptors(stack, m, (ids,)).graph_module
+    n_mm = len(gm.graph.find_nodes(op="call_function", target=torch.ops.aten.mm.default))
+    # seven linear layers per block and the head; each with its input and its weight gradient
+    assert n_mm == 3 * (7 * n_layers + 1)
+    assert replace_view_mm_view_with_einsum(gm) == n_mm
+    assert not gm.graph.find_nodes(op="call_function", target=torch.ops.aten.mm.default)
+    eins = gm.graph.find_nodes(op="call_function", target=torch.ops.aten.einsum.default)
+    assert sorted({n.args[0] for n in eins}) == ["abk,kn->abn", "abn,abk->kn"]
+    had_pg = dist.is_initialized()
+    if had_pg:
+        dist.destroy_process_group()
+    dist.init_process_group("fake", store=FakeStore(), rank=0, world_size=64)
+    try:
+        mesh88 = init_device_mesh("cpu", (8, 8))
+        PO.fallback_nodes.clear()
+        PO.fallback_reasons.clear()
+        PO.reset_placement_options_cache()
+        opt = ShardingOptimizer(gm, mesh88, devices_per_host=8, device_name="AMD Instinct MI355X")
+        assert PO.fallback_nodes == [], PO.fallback_reasons
+        for n in eins:
+            activations = {s.input_specs[0].placements for s in opt.strats[n].strategies}
+            assert (Shard(0), Shard(1)) in activations and (Shard(1), Shard(0)) in activations, n
+        g = opt._packed
+        ref = O.GraphOracle(g).build()
+        slots = g.entry_slots()
+        cost_ref, _ = O.clamp_inf(ref["cost"])
+        assert bits_equal(opt._core.coef.comm, ref["comm"][slots])
+        assert bits_equal(opt._core.coef.cost, cost_ref[slots])
+        assert bits_equal(opt._core.coef.compute, ref["compute"])
+        sol = opt.get_solution()
+        assert all(n in sol for n in eins)
+    finally:
+        dist.destroy_process_group()
+        if had_pg:
+            dist.init_process_group("fake", store=FakeStore(), rank=0, world_size=8)
