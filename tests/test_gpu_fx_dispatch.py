@@ -302,12 +302,19 @@ def test_programs_of_the_traced_llama3_8b_graph():
         finally:
             torch.set_default_dtype(torch.float32)
         gm = _trace(m, torch.randint(0, cfg.vocab_size, (64, 8192), device="cuda"))
+    from autoparallel_amd.graph_utils import replace_view_mm_view_with_einsum
+
     with _fake_group(64):
-        checked, refused = _check_programs_of(gm, init_device_mesh("cpu", (8, 8)))
+        mesh = init_device_mesh("cpu", (8, 8))
+        checked, refused = _check_programs_of(gm, mesh)
+        # and with the linear layers as einsums, the way the graph is planned
+        assert replace_view_mm_view_with_einsum(gm) > 0
+        checked_einsum, _ = _check_programs_of(gm, mesh)
     print(dict(checked))
     families = {"aten.mm.default", "aten.embedding.default", "aten.mean.dim", "aten.sum.dim_IntList",
                 "aten._to_copy.default", "aten.silu.default", "aten.mul.Tensor", "aten.rsqrt.default"}
     assert families <= set(checked), families - set(checked)
+    assert "aten.einsum.default" in checked_einsum and "aten.mm.default" not in checked_einsum
     # 32 query heads on 8 key/value heads: the flop counter the reference relies on has no
     # formula for it
     assert set(refused) == {"aten._scaled_dot_product_flash_attention.default",
