@@ -293,6 +293,9 @@ EXPORTED_SYMBOLS = tuple(_SIGNATURES)
 _lib = None
 
 
+ABI_VERSION = 3  # apc_version() of the library whose struct layouts this module mirrors
+
+
 class ApcError(RuntimeError):
     pass
 
@@ -308,6 +311,12 @@ def load() -> C.CDLL:
             "(hipcc, gfx950). There is no CPU fallback."
         )
     lib = C.CDLL(LIB_PATH)
+    lib.apc_version.restype = C.c_int
+    if lib.apc_version() != ABI_VERSION:
+        # the structs mirrored here are the ones of include/apc.h at this version: a library
+        # built from other sources would read them wrongly
+        raise ApcError(f"{LIB_PATH} has ABI version {lib.apc_version()}, this package needs {ABI_VERSION}: "
+                       "rebuild it with `python -m autoparallel_amd.csrc.build`")
     for name, (res, args) in _SIGNATURES.items():
         fn = getattr(lib, name)
         fn.restype = res

@@ -319,6 +319,7 @@ typedef struct apc_problem {
   const apc_prog_term* prog_terms;   /* named by apc_comp_rec.term_off / n_term */
 } apc_problem;
 
+/* Version of the ABI (struct layouts and signatures of this header): 3. */
 int apc_version(void);
 const char* apc_last_error(void);
 
