@@ -535,8 +535,9 @@ class PackedGraph:
         of every matrix of the block table (``entries=False``; ``compressed`` as
         for block_table), or of every edge block that owns entries
         (``entries=True``: direct evaluation, edges without a producer included).
-        A tile has at most LUT_COLS source columns and about LUT_TILE_ELEMENTS
-        elements."""
+        A tile has at most LUT_COLS source columns and LUT_ROWS target rows, and
+        about LUT_TILE_ELEMENTS elements, more when there is work for more than a
+        few thousand tiles."""
         if entries:
             e = np.nonzero(self.priced & (self.block_sizes() > 0))[0].astype(np.int64)
             ncol, nrow = self.edge_ssrc[e].astype(np.int64), self.edge_sdst[e].astype(np.int64)
@@ -553,8 +554,12 @@ class PackedGraph:
             flags = EDGE_HAS_PRODUCER | np.where(squeezed, EDGE_COMPRESSED, 0).astype(np.int64)
             comp_base = np.full(e.shape[0], -1, np.int64)
         n_ct = (ncol + self.LUT_COLS - 1) // self.LUT_COLS
+        # a tile's lookup tables are made once per tile: tiles as tall as the work allows
+        # while there are still a few thousand of them to spread over the chip
+        total = int((ncol * nrow).sum())
+        tile_elements = int(min(self.LUT_COLS * self.LUT_ROWS, max(self.LUT_TILE_ELEMENTS, total // 3072)))
         rows_per = np.minimum(np.minimum(nrow, self.LUT_ROWS),
-                              np.maximum(1, self.LUT_TILE_ELEMENTS // np.minimum(ncol, self.LUT_COLS)))
+                              np.maximum(1, tile_elements // np.minimum(ncol, self.LUT_COLS)))
         n_rt = (nrow + rows_per - 1) // np.maximum(rows_per, 1)
         per = n_ct * n_rt
         k = np.repeat(np.arange(e.shape[0], dtype=np.int64), per)
