@@ -321,8 +321,27 @@ def load() -> C.CDLL:
         fn = getattr(lib, name)
         fn.restype = res
         fn.argtypes = args
+    _warn_if_stale()
     _lib = lib
     return lib
+
+
+def _warn_if_stale() -> None:
+    """A library older than a source next to it runs kernels those sources no
+    longer describe (an edited kernel, a record laid out differently): say so."""
+    here = os.path.dirname(LIB_PATH)
+    srcs = [os.path.join(here, "csrc", f) for f in os.listdir(os.path.join(here, "csrc"))
+            if f.endswith((".hip", ".cpp", ".h"))] if os.path.isdir(os.path.join(here, "csrc")) else []
+    header = os.path.join(os.path.dirname(here), "include", "apc.h")
+    if os.path.exists(header):
+        srcs.append(header)
+    built = os.path.getmtime(LIB_PATH)
+    newer = [os.path.basename(f) for f in srcs if os.path.getmtime(f) > built]
+    if newer:
+        import warnings
+
+        warnings.warn(f"{LIB_PATH} is older than {', '.join(sorted(newer))}: rebuild it with "
+                      "`python -m autoparallel_amd.csrc.build`", RuntimeWarning, stacklevel=3)
 
 
 def check(rc: int, what: str) -> None:

@@ -733,20 +733,26 @@ class PackedGraph:
         return out
 
     def work_items(self, compressed: bool = False, item_entries: int = ITEM_ENTRIES) -> np.ndarray:
-        """Work items of the entry kernel: for every ``item_entries`` (256 or 512)
-        entries of every edge block a copy of the edge record with ``local0``
-        set, in slot order."""
+        """Work items of the entry kernel: copies of the edge record with ``local0``
+        set, in slot order, each covering ``item_entries`` (256 or 512) slots.
+        An item starts at a multiple of 64 slots of the entry arrays, so that
+        every store instruction of a wave writes whole aligned 512-byte (costs)
+        and 64-byte (flags) pieces; blocks start at multiples of 16 slots, so the
+        first item of a block may start up to 48 slots before it: its ``local0``
+        is then negative modulo 2**32, and the kernel's ``entry < size`` test
+        switches those lanes off like the ones past the block's end."""
         assert item_entries in (ITEM_ENTRIES, 2 * ITEM_ENTRIES)
         cache = self.__dict__.setdefault("_work_items", {})  # as the block table: made once per layout
         if (compressed, item_entries) in cache:
             return cache[(compressed, item_entries)]
         sizes = self.block_sizes()
-        n = (sizes + item_entries - 1) // item_entries
+        lead = np.where(sizes > 0, self.edge_off[:-1] % 64, 0).astype(np.int64)
+        n = (sizes + lead + item_entries - 1) // item_entries
         eid = np.repeat(np.arange(self.num_edges, dtype=np.int64), n)
         start = np.concatenate([[0], np.cumsum(n)[:-1]])
         k = np.arange(int(n.sum()), dtype=np.int64) - start[eid]
         items = self.edge_records(compressed)[eid]
-        items["local0"] = k * item_entries
+        items["local0"] = ((k * item_entries - lead[eid]) & 0xFFFFFFFF).astype(np.uint32)
         cache[(compressed, item_entries)] = items
         return items
 

@@ -70,7 +70,8 @@ typedef struct apc_edge {
                         rows of default_vals)                                   */
   uint32_t magic;    /* floor(2^32 / ssrc) + 1 if ssrc > 1 and ssrc * ssrc * sdst
                         < 2^32 (then local / ssrc == umulhi(local, magic)), else 0 */
-  uint32_t local0;   /* 0 in the edge table; in a work item, its first entry  */
+  uint32_t local0;   /* 0 in the edge table; in a work item, its first entry
+                        (modulo 2^32: see apc_problem.items)                 */
 } apc_edge; /* 64 bytes */
 
 /* Everything the node estimate reads about one evaluated node, in one record,
@@ -272,9 +273,11 @@ typedef struct apc_problem {
   int64_t n_slot;            /* length of the entry arrays (with padding)      */
   int64_t n_chunk;           /* n_slot / 16                                    */
   const int32_t* chunk_edge; /* [n_chunk] edge owning slots [16c, 16c + 16)    */
-  /* work items of the entry kernel: for every 256 (or item_entries) entries of
-   * every edge block a copy of the edge record with local0 = first entry of
-   * the item, slot order */
+  /* work items of the entry kernel: copies of the edge record, slot order, each
+   * covering 256 (or item_entries) slots from entry local0 of its block on.  An
+   * item may start before its block (local0 negative modulo 2^32, so that it
+   * starts at a multiple of 64 slots of the entry arrays) and end after it:
+   * lanes whose entry local0 + i is not below sdst * ssrc (unsigned) are idle */
   int32_t n_item;
   const apc_edge* items;     /* [n_item] */
   int64_t n_default;

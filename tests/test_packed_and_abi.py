@@ -42,8 +42,17 @@ def test_layout_invariants(small_llama):
     assert (g.edge_off[:-1][item_edge] == items["off"]).all()
     np.add.at(covered, item_edge, 1)
     sizes = g.edge_sdst.astype(np.int64) * g.edge_ssrc
-    assert (covered == (sizes + 255) // 256).all()
-    assert (items["local0"] % 256 == 0).all()
+    lead = g.edge_off[:-1] % 64  # an item starts at a multiple of 64 slots, up to 48 before its block
+    assert (covered == (sizes + lead + 255) // 256).all()
+    first_slot = items["off"] + items["local0"].astype(np.int32)
+    assert (first_slot % 64 == 0).all() and (first_slot + 64 > items["off"]).all()
+    # the entries an item's 256 lanes-times-four reach, kept where 0 <= entry < size: every entry once
+    hit = np.zeros(g.num_slots, np.int32)
+    for it, e in zip(items, item_edge):
+        local = (np.arange(256, dtype=np.int64) + int(np.int32(it["local0"])))
+        local = local[(local >= 0) & (local < sizes[e])]
+        hit[it["off"] + local] += 1
+    assert (hit[slots] == 1).all() and hit.sum() == len(slots)
     # decision-var order: node, out_idx, argi, inp_idx
     order = g.decision_var_order()
     k = keys[order]
