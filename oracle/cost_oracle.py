@@ -61,10 +61,9 @@ MI355X_TFLOPS = {0: 78.6, 1: 157.3, 2: 2516.6, 3: 2516.6, 4: 5033.2}
 
 
 # The whole table (compute_estimation.py:66-255), in its order: name ->
-# (bytes/s, {dtype code: TFLOPS}); the halves are integer halves there.  Data, restated:
-# only the H100 row has an independent pin (the 989 TFLOPS bf16 and 3.35 TB/s that
-# docs/how_autoparallel_chooses_a_strategy.md:34-39 quotes) and the MI355X row the golden
-# cost vectors; the other rows are parity unpinned.
+# (bytes/s, {dtype code: TFLOPS}); the halves are integer halves there.  Pinned row by
+# row, with the substring matching and its order, by tests/golden/device_table_vectors.json:
+# what the reference's own lookups answer for 38 device names (tests/test_device_table_golden.py).
 DEVICE_TABLE = (
     ("H100", 3.35 * (1024**4), {0: 67, 1: 989 // 2, 2: 1979 // 2, 3: 1979 // 2, 4: 3958 // 2}),
     ("B200", 7.7 * (1024**4), {0: 37, 1: 2200 // 2, 2: 4500 // 2, 3: 4500 // 2, 4: 9000 // 2}),
