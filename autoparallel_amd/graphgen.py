@@ -1159,7 +1159,7 @@ def _stress_header(seed: int, v: int, nd: int, s_min: int, s_max: int):
     dt = DT_BF16 if rng.random() < 0.5 else DT_F32
     S = int(rng.integers(s_min, s_max + 1))
     codes = np.asarray([R] + [shard(d) for d in range(r)] + [P])
-    out = [tuple(int(c) for c in row) for row in codes[rng.integers(0, len(codes), size=(S, nd))]]
+    out = codes[rng.integers(0, len(codes), size=(S, nd))]  # int array [S, nd]
     return r, shape, dt, out
 
 
@@ -1219,7 +1219,7 @@ def stress_dag_window(
         if v not in metas:
             r, shape, dt, _ = header(v)
             metas[v] = b.meta(shape, contiguous_stride(shape), _ITEMSIZE[dt], dt)
-        return [b.spec(metas[v], t) for t in tuples]
+        return b.specs(metas[v], tuples)
 
     def add_input(v):
         out = [[w] for w in specs_of(v, header(v)[3])]
@@ -1239,9 +1239,8 @@ def stress_dag_window(
         for u in inputs:
             ru = header(u)[0]
             codes = np.asarray([R] + [shard(d) for d in range(ru)] + [P])
-            cols.append(specs_of(u, [tuple(int(c) for c in row)
-                                     for row in codes[rng.integers(0, len(codes), size=(S, nd))]]))
-        in_specs = [[c[o] for c in cols] for o in range(S)]
+            cols.append(specs_of(u, codes[rng.integers(0, len(codes), size=(S, nd))]))
+        in_specs = [list(row) for row in zip(*cols)]
         loc = [local[u] for u in inputs]
         isz = _ITEMSIZE[dt]
         if op == "view":

@@ -954,6 +954,24 @@ class GraphBuilder:
         """Spec word of (tensor meta, placements); -1 stands for None."""
         return spec_word(meta_id, self.tuple_id(placements))
 
+    def specs(self, meta_id: int, placements) -> List[int]:
+        """Spec words of one tensor meta under many placement tuples
+        (``placements``: int array [n, mesh dims]): the same words, and the same
+        tuple ids in the same order, as ``spec`` called row by row."""
+        rows = np.ascontiguousarray(placements, dtype=np.int64).reshape(-1, len(self.mesh_shape))
+        if rows.shape[0] == 0:
+            return []
+        assert ((rows >= 0) & (rows < 256)).all()
+        key = rows @ (256 ** np.arange(rows.shape[1], dtype=np.int64))
+        uniq, first, inverse = np.unique(key, return_index=True, return_inverse=True)
+        known = self.__dict__.setdefault("_tuple_of_key", {})  # packed placements -> tuple id
+        ids = [known.get(k) for k in uniq.tolist()]
+        if None in ids:
+            for i in np.argsort(first, kind="stable").tolist():  # new tuples get their ids in order of first use
+                if ids[i] is None:
+                    ids[i] = known[int(uniq[i])] = self.tuple_id(rows[first[i]].tolist())
+        return ((int(meta_id) << TUPLE_BITS) | np.asarray(ids, np.int64)[inverse.reshape(-1)]).tolist()
+
     def spec_placements(self, word: int) -> Tuple[int, ...]:
         return self._tuple_rows[word & (MAX_TUPLES - 1)]
 
@@ -1003,7 +1021,7 @@ class GraphBuilder:
             """Offset of a run of spec words; identical runs are stored once,
             which also makes a producer's run offset the identity of its row
             table."""
-            key = tuple(int(w) for w in words)
+            key = tuple(map(int, words))
             off = run_cache.get(key)
             if off is None:
                 off = len(lists)
@@ -1036,7 +1054,7 @@ class GraphBuilder:
             nout = len(nd_.out_specs[0])
             runs = {}
             for k in range(nout):
-                runs[k] = add_run(nd_.out_specs[o][k] for o in range(S))
+                runs[k] = add_run([row[k] for row in nd_.out_specs])
             out_runs.append(runs)
             # edges: one per row of redistribute_cost (== per arg)
             n_rows = len(nd_.in_specs[0])
@@ -1048,9 +1066,8 @@ class GraphBuilder:
                 e_node.append(v)
                 e_arg.append(a)
                 e_sdst.append(S)
-                e_dst_list.append(add_run(
-                    (nd_.in_specs[o][a] if a < len(nd_.in_specs[o]) else -1) for o in range(S)
-                ))
+                dst_words = [int(row[a]) if a < len(row) else -1 for row in nd_.in_specs]
+                e_dst_list.append(add_run(dst_words))
                 flags = 0
                 if has_prod:
                     u = nd_.inputs[a]
@@ -1078,14 +1095,9 @@ class GraphBuilder:
                     )
                     e_ssrc.append(ssrc)
                     e_src_list.append(-1)
-                need_default = (flags & EDGE_HAS_PRODUCER) == 0 or any(
-                    (a >= len(nd_.in_specs[o]) or nd_.in_specs[o][a] < 0) for o in range(S)
-                ) or (
-                    (flags & EDGE_HAS_PRODUCER)
-                    and any(
-                        lists[e_src_list[-1] + j] < 0 for j in range(e_ssrc[-1])
-                    )
-                )
+                # a missing spec on either side (-1) keeps the default row
+                need_default = ((flags & EDGE_HAS_PRODUCER) == 0 or min(dst_words) < 0
+                                or min(lists[e_src_list[-1]:e_src_list[-1] + e_ssrc[-1]]) < 0)
                 if need_default:
                     e_def.append(len(defaults))
                     for o in range(S):

@@ -352,3 +352,19 @@ def test_missing_library_is_an_error_not_a_fallback(monkeypatch, tmp_path):
     root = pathlib.Path(_lib.__file__).parent
     for path in root.rglob("*.py"):
         assert not re.search(r"^\s*(from|import)\s+oracle\b", path.read_text(), re.M), path
+
+
+def test_specs_in_bulk_equal_specs_one_by_one():
+    """GraphBuilder.specs gives the words, and hands out the tuple ids in the order, of spec called per row."""
+    rng = np.random.default_rng(5)
+    one, bulk = packed.GraphBuilder((4, 8, 8)), packed.GraphBuilder((4, 8, 8))
+    codes = np.asarray([packed.PLC_R, packed.shard(0), packed.shard(1), packed.shard(2), packed.PARTIAL_SUM])
+    for k in range(40):
+        shape = (64 + k, 128, 32)
+        m1 = one.meta(shape, (128 * 32, 32, 1), 2, packed.DT_BF16)
+        m2 = bulk.meta(shape, (128 * 32, 32, 1), 2, packed.DT_BF16)
+        rows = codes[rng.integers(0, 2 + k % 4, size=(int(rng.integers(1, 300)), 3))]
+        assert [one.spec(m1, tuple(int(c) for c in r)) for r in rows] == bulk.specs(m2, rows)
+        if k % 7 == 0:  # the two ways of interning mix
+            assert one.spec(m1, (codes[4], codes[4], codes[0])) == bulk.spec(m2, (codes[4], codes[4], codes[0]))
+    assert one._tuple_rows == bulk._tuple_rows and bulk.specs(0, np.zeros((0, 3), np.int64)) == []
