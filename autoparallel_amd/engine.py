@@ -13,11 +13,6 @@ import torch
 from . import _lib
 from .packed import CHUNK_SHIFT, ITEM_ENTRIES, MAX_MESH_DIMS, PackedGraph
 
-# Build the pair table when it is at most this many times the entry count (and
-# small in absolute terms); otherwise every entry is evaluated directly.
-_TABLE_MAX_RATIO = 0.5
-_TABLE_MAX_DOUBLES = 1 << 28
-_WIDE_ITEMS_FROM = 32_000_000  # entries
 _LARGE_BLOCKS_FROM = 8192  # mean entries per edge block
 _UPLOAD_ARENA_BYTES = 8 << 20  # descriptor arrays of one problem that go up in one copy
 _UPLOAD_ARENA_MAX_ARRAY = 2 << 20
@@ -270,27 +265,11 @@ class CostEngine:
         p.n_chunk = chunk_edge.shape[0]
         assert p.n_chunk == g.num_slots >> CHUNK_SHIFT
         p.chunk_edge = up("chunk_edge", chunk_edge)
-        # the table path carries the transition flag in the sign bit of a cost and
-        # reads default rows the same way: a default value with its sign bit set
-        # (nothing the reference produces) is only exact on the direct path
         signed_defaults = bool(np.signbit(g.default_vals).any())
         if table_mode is None and use_table is not None:
             table_mode = "full" if use_table else "direct"
         if table_mode is None:
-            def small(t):
-                return t <= _TABLE_MAX_DOUBLES and t <= max(_TABLE_MAX_RATIO * g.num_entries, 1 << 16)
-
-            if signed_defaults:
-                table_mode = "direct"
-            elif small(int(g.block_table(False)[1][-1])):
-                # once the outputs stream past every cache, the smaller compressed
-                # table costs less than its gathers (measured at 84 M and 418 M entries)
-                big = g.num_entries >= _WIDE_ITEMS_FROM and g.run_unique_index() is not None
-                table_mode = "compressed" if big and g.block_table(True)[1][-1] < g.block_table(False)[1][-1] else "full"
-            elif g.run_unique_index() is not None and small(int(g.block_table(True)[1][-1])):
-                table_mode = "compressed"
-            else:
-                table_mode = "direct"
+            table_mode = g.default_table_mode()
         if table_mode not in ("direct", "full", "compressed"):
             raise ValueError(f"unknown table_mode {table_mode!r}")
         if table_mode != "direct" and signed_defaults:
@@ -298,9 +277,7 @@ class CostEngine:
         self.table_mode = table_mode
         squeezed = table_mode == "compressed"
         p.edges = up("edges", g.edge_records(squeezed))
-        # work items of 512 entries pay off from some tens of millions of entries on
-        self.item_entries = (2 * ITEM_ENTRIES if table_mode != "direct" and g.num_entries >= _WIDE_ITEMS_FROM
-                             else ITEM_ENTRIES) if item_entries is None else int(item_entries)
+        self.item_entries = g.default_item_entries(table_mode) if item_entries is None else int(item_entries)
         items = g.work_items(squeezed, self.item_entries)
         p.item_entries = self.item_entries
         p.n_item = items.shape[0]

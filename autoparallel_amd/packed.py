@@ -49,6 +49,11 @@ MAX_METAS = 1 << (32 - TUPLE_BITS)
 SPEC_NONE = 0xFFFFFFFF
 CHUNK_SHIFT = 4  # edge blocks start on multiples of 1 << CHUNK_SHIFT slots
 ITEM_ENTRIES = 256  # entries of one edge per work item of the entry kernel
+# A block table is built when it is at most this many times the entry count (and
+# small in absolute terms); otherwise every entry is evaluated directly.
+TABLE_MAX_RATIO = 0.5
+TABLE_MAX_DOUBLES = 1 << 28
+WIDE_ITEMS_FROM = 32_000_000  # entries: from here on work items of 512 entries and, if smaller, the compressed table
 
 
 def spec_word(meta_id: int, tuple_id: int) -> int:
@@ -406,13 +411,12 @@ class PackedGraph:
             mid = first >> TUPLE_BITS
             rec["arg_meta"][np.nonzero(has)[0], a] = np.where((first != SPEC_NONE) & (mid < 0xFFFF), mid, 0xFFFF)
         _, where = self.program_terms()
-        for i, node in enumerate(v):
-            if self.node_op[node] != OP_PROGRAM or n_edge[i] > self.REC_ARGS:
-                continue
-            # a node with more arguments than rows of the value table can name keeps the interpreter
-            if self.max_rank + int(n_edge[i]) * (self.max_rank + 2) > 0xFF:
-                continue
-            hit = where.get(int(self.node_prog_off[node]))
+        R = self.max_rank
+        # a node with more arguments than rows of the value table can name keeps the interpreter
+        as_terms = (self.node_op[v] == OP_PROGRAM) & (n_edge <= self.REC_ARGS) & (R + n_edge * (R + 2) <= 0xFF)
+        prog_off = self.node_prog_off[v]
+        for i in np.nonzero(as_terms)[0].tolist():
+            hit = where.get(int(prog_off[i]))
             if hit is not None:
                 rec["term_off"][i], rec["n_term"][i], rec["term_flags"][i] = hit
         return rec
@@ -634,7 +638,9 @@ class PackedGraph:
             start = np.concatenate([[0], np.cumsum(ln)[:-1]]) if runs.shape[0] else np.zeros(0, np.int64)
             pos = off[rid] + (np.arange(int(ln.sum()), dtype=np.int64) - start[rid])
             words = self.lists[pos].astype(np.int64)
-            order = np.lexsort((pos, words, rid))
+            # by run, then word, then position: positions already ascend within a run, so a
+            # stable sort on (run, word) in one 64-bit key does it (words are 32-bit)
+            order = np.argsort((rid << 32) | (words & 0xFFFFFFFF), kind="stable")
             rs, ws, ps = rid[order], words[order], pos[order]
             new = np.ones(rs.shape[0], bool)
             new[1:] = (rs[1:] != rs[:-1]) | (ws[1:] != ws[:-1])
@@ -756,9 +762,49 @@ class PackedGraph:
         cache[(compressed, item_entries)] = items
         return items
 
+    def default_table_mode(self) -> str:
+        """The block-table layout the engine uses unless told otherwise: "full",
+        "compressed" (matrices by distinct spec word) or "direct" (no table)."""
+        def small(t):
+            return t <= TABLE_MAX_DOUBLES and t <= max(TABLE_MAX_RATIO * self.num_entries, 1 << 16)
+
+        # the table path carries the transition flag in the sign bit of a cost and
+        # reads default rows the same way: a default value with its sign bit set
+        # (nothing the reference produces) is only exact on the direct path
+        if bool(np.signbit(self.default_vals).any()):
+            return "direct"
+        if small(int(self.block_table(False)[1][-1])):
+            # once the outputs stream past every cache, the smaller compressed
+            # table costs less than its gathers (measured at 84 M and 418 M entries)
+            big = self.num_entries >= WIDE_ITEMS_FROM and self.run_unique_index() is not None
+            return "compressed" if big and self.block_table(True)[1][-1] < self.block_table(False)[1][-1] else "full"
+        if self.run_unique_index() is not None and small(int(self.block_table(True)[1][-1])):
+            return "compressed"
+        return "direct"
+
+    def default_item_entries(self, table_mode: str) -> int:
+        """Work items of 512 entries pay off from some tens of millions of entries on."""
+        return 2 * ITEM_ENTRIES if table_mode != "direct" and self.num_entries >= WIDE_ITEMS_FROM else ITEM_ENTRIES
+
+    def warm_host_layout(self) -> None:
+        """Makes, and caches on the graph, the layouts the engine would derive for
+        its default choices (they travel with the graph when it is pickled): for
+        graphs packed in worker processes."""
+        mode = self.default_table_mode()
+        if mode != "direct":
+            self.block_table(mode == "compressed")
+        self.work_items(mode == "compressed", self.default_item_entries(mode))
+
     def validate(self) -> None:
         """Host-side shape checks run before any kernel launch: every index a
-        kernel dereferences must be in range."""
+        kernel dereferences must be in range.  A graph that passed is marked, and
+        not checked again (its arrays are not meant to be written to)."""
+        if self.__dict__.get("_validated"):
+            return
+        self._validate()
+        object.__setattr__(self, "_validated", True)
+
+    def _validate(self) -> None:
         nd = self.ndim
         assert 1 <= nd <= MAX_MESH_DIMS
         assert (self.mesh_shape >= 1).all()

@@ -44,6 +44,9 @@ def _make_window(task):
     try:
         g, gid, n_standin = graphgen.stress_dag_window(n_total, lo, hi, mesh, seed, s_min, s_max)
         g.validate()
+        # the layouts the engine derives on the host are cached on the graph and travel with
+        # it: made here, in the worker, instead of in the one process that drives the device
+        g.warm_host_layout()
     finally:
         if was:
             gc.enable()
@@ -75,7 +78,8 @@ def score_in_windows(
     if max_windows is not None:
         tasks = tasks[:max_windows]
     stats = {"nodes": 0, "edges": 0, "entries": 0, "standin_nodes": 0, "windows": 0, "table_doubles": 0,
-             "build_device_s": 0.0, "score_device_s": 0.0, "modes": {}}
+             "build_device_s": 0.0, "score_device_s": 0.0, "wait_for_window_s": 0.0, "engine_construct_s": 0.0,
+             "modes": {}}
     out = None
     t_wall = time.perf_counter()
     pool = None
@@ -85,8 +89,12 @@ def score_in_windows(
     else:
         results = map(_make_window, tasks)
     try:
+        t_mark = time.perf_counter()
         for lo, hi, g, gid, n_standin in results:
+            stats["wait_for_window_s"] += time.perf_counter() - t_mark  # the host's generation and packing
+            t_mark = time.perf_counter()
             eng = CostEngine(g)
+            stats["engine_construct_s"] += time.perf_counter() - t_mark  # layout of the problem and its upload
             ev = [torch.cuda.Event(enable_timing=True) for _ in range(3)]
             ev[0].record()
             eng.build(clamp_inf=True)
@@ -108,6 +116,7 @@ def score_in_windows(
             if progress:
                 progress(stats, time.perf_counter() - t_wall)
             del eng
+            t_mark = time.perf_counter()
     finally:
         if pool is not None:
             pool.terminate()
