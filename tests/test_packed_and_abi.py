@@ -368,3 +368,30 @@ def test_specs_in_bulk_equal_specs_one_by_one():
         if k % 7 == 0:  # the two ways of interning mix
             assert one.spec(m1, (codes[4], codes[4], codes[0])) == bulk.spec(m2, (codes[4], codes[4], codes[0]))
     assert one._tuple_rows == bulk._tuple_rows and bulk.specs(0, np.zeros((0, 3), np.int64)) == []
+
+
+def test_layout_choice_and_caches_travel_with_the_graph(small_llama):
+    """The engine's default layout is a property of the packed graph, and the
+    layouts made for it in a worker process arrive with the pickled graph."""
+    import pickle
+
+    # one layer: the full table would be more than half as large as the entry arrays; four layers share it
+    assert small_llama.default_table_mode() == "compressed"
+    four = graphgen.llama_graph((8, 8), 4, 1024, 8, 4, 2048, 8192, 512, 16)
+    assert four.default_table_mode() == "full" and four.default_item_entries("full") == 256
+    g = graphgen.stress_graph(60, (4, 8, 8), seed=2, s_min=64, s_max=300)
+    mode = g.default_table_mode()
+    assert mode == "compressed"  # no two edges share a matrix: only the matrices of distinct words are small enough
+    assert g.default_item_entries(mode) == (512 if g.num_entries >= packed.WIDE_ITEMS_FROM else 256)
+    assert g.default_item_entries("direct") == 256
+    g.validate()
+    g.warm_host_layout()
+    h = pickle.loads(pickle.dumps(g))
+    assert h.__dict__.get("_validated") and h.__dict__["_run_unique"] is not None
+    assert (True, g.default_item_entries(mode)) in h.__dict__["_work_items"] and True in h.__dict__["_block_tables"]
+    for a, b in zip(h.run_unique_index(), g.run_unique_index()):
+        assert np.array_equal(a, b)
+    assert np.array_equal(h.work_items(True, g.default_item_entries(mode)), g.work_items(True, g.default_item_entries(mode)))
+    # a graph derived from it starts without them
+    alias = np.arange(g.num_edges)
+    assert "_work_items" not in g.with_edge_alias(alias).__dict__
