@@ -120,9 +120,9 @@ def _create_all_options(mesh, shape, tensor_meta=None, tensor=None) -> OpStrateg
 # ---------------------------------------------------------------------------
 # post-processing of operator strategies
 # ---------------------------------------------------------------------------
-def _spec_ok(spec: DTensorSpec, mesh) -> bool:
+def _spec_ok(spec: DTensorSpec, mesh_shape) -> bool:
     shape = list(spec.tensor_meta.shape)
-    for n, p in zip(mesh.shape, spec.placements):
+    for n, p in zip(mesh_shape, spec.placements):
         if p.is_shard():
             if shape[p.dim] >= n:
                 shape[p.dim] = (shape[p.dim] + n - 1) // n
@@ -133,11 +133,12 @@ def _spec_ok(spec: DTensorSpec, mesh) -> bool:
 
 def remove_invalid_configs(out_strat: OpStrategy, mesh) -> OpStrategy:
     kept = []
+    mesh_shape = tuple(mesh.shape)  # DeviceMesh.shape rebuilds its layout on every access
     for st in out_strat.strategies:
         outs = st.output_specs
         outs = [outs] if isinstance(outs, DTensorSpec) else list(outs or [])
         specs = list(st.input_specs or []) + outs
-        if all(s is None or _spec_ok(s, mesh) for s in specs):
+        if all(s is None or _spec_ok(s, mesh_shape) for s in specs):
             kept.append(st)
     return OpStrategy(kept)
 
