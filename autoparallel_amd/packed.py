@@ -655,7 +655,9 @@ class PackedGraph:
             ufirst = np.zeros(L, np.int32)
             ufirst[off[rs[new]] + rank[new]] = ps[new] - off[rs[new]]
             nuniq = np.zeros(L, np.int32)
-            np.maximum.at(nuniq, off[rs], (rank + 1).astype(np.int32))
+            last_of_run = np.ones(rs.shape[0], bool)  # ranks ascend within a run: its last one is the largest
+            last_of_run[:-1] = rs[1:] != rs[:-1]
+            nuniq[off[rs[last_of_run]]] = (rank[last_of_run] + 1).astype(np.int32)
             out = (uidx, ufirst, nuniq)
         object.__setattr__(self, "_run_unique", out)
         return out
