@@ -590,7 +590,6 @@ class ShardingOptimizer:
         # per-variable link table of the reference (:356-378): linked key -> root key
         self.cluster_links = _ClusterLinks(self, self._core.cluster_links)
         self._cluster_linked_node_idxs = set(self._core.cluster_links)
-        self.prob = self._core.prob
         self.phase_s.update(self._core.phase_s)
         t0 = time.perf_counter()
         self._write_back_redistribute_costs()
@@ -627,6 +626,60 @@ class ShardingOptimizer:
                     f"{node}, {len(s0.redistribute_cost[i])}, {len(self.strats[arg].strategies)}"
 
     # -- constraints (delegated to the packed formulation) ------------------------------
+    @property
+    def prob(self):
+        """The ILP of the current decision variables (``ilp.SparseILP``)."""
+        return self._core.prob
+
+    @prob.setter
+    def prob(self, value):
+        """The reference's rebuild sequence assigns a new problem before it adds the
+        default rows again (``opt.prob = pulp.LpProblem(...)``,
+        tests/test_paired_output_constraint.py:58-62, serialization.py:330-337): an
+        assignment starts an empty problem over the current decision variables.  A
+        SparseILP of that size is taken as it is; anything else only marks the restart."""
+        from . import ilp
+
+        core = self._core
+        if value is core.prob:
+            return
+        core.reset_problem(value if isinstance(value, ilp.SparseILP) and value.n_vars == core.n_vars else None)
+        self._constraint_log.clear()  # the rows it would replay are gone
+
+    @property
+    def _name_counters(self) -> Dict[str, int]:
+        """Next index per constraint-name prefix (autoparallel/optimize_sharding.py:248, 293-296)."""
+        return self._core.prob._counters
+
+    @_name_counters.setter
+    def _name_counters(self, value) -> None:
+        counters = self._core.prob._counters
+        counters.clear()
+        counters.update(value)
+
+    def add_default_constraints(self):
+        """The six groups of rows every problem has (autoparallel/optimize_sharding.py:814-822).
+        ``_build_decision_vars`` leaves them in place; a caller that assigned ``prob`` adds them here."""
+        self._core.add_default_constraints()
+
+    def add_unique_decision_constraint(self):  # :665-688
+        self._core.add_unique_decision_constraint()
+
+    def add_same_output_across_args_constraint(self):  # :690-721
+        self._core.add_same_output_across_args_constraint()
+
+    def add_output_input_consistent_constraint(self):  # :723-801
+        self._core.add_output_input_consistent_constraint()
+
+    def add_inf_cost_constraint(self):  # :803-812
+        self._core.add_inf_cost_constraint()
+
+    def add_forward_backward_consistency_constraints(self):  # :1460-1485
+        self._core.add_forward_backward_consistency_constraints()
+
+    def add_grad_reduce_dtype_constraints(self):  # :1487-1627
+        self._core.add_grad_reduce_dtype_constraints()
+
     def add_node_constraint(self, node, placement=None, constraint_name=None):
         node = self._normalize_node(node)
         assert node in self.strats, node

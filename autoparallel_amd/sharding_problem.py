@@ -486,6 +486,16 @@ class PackedShardingOptimizer:
         self.prob.add_row("memory_constraint_high", idx, coef, ilp.LE, budget_high, exact_name=True)
         self.prob.add_row("memory_constraint_low", idx, coef, ilp.GE, budget_low, exact_name=True)
 
+    def reset_problem(self, prob: Optional[ilp.SparseILP] = None) -> None:
+        """An empty problem over the same decision variables (or ``prob``): no rows,
+        no variable fixed, no memory budget, no logged constraint."""
+        assert prob is None or prob.n_vars == self.n_vars
+        self.prob = prob if prob is not None else ilp.SparseILP(self.n_vars)
+        self._memory_constraint = None
+        self._node_constraint_names = {}
+        self._constraint_log = []
+        self.selected = None
+
     def remove_constraints(self, names: Iterable[str]) -> None:
         for name in names:
             self.prob.remove(name)

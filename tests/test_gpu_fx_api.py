@@ -372,6 +372,28 @@ def test_rebuild_after_mutating_strategies(mesh):
     bad = [i for i, s in enumerate(opt.strats[param].strategies) if str(s.output_specs.placements) == removed]
     assert len(bad) == 1
     assert all(k[2] != bad[0] for k in opt.selected_keys if k[0] == pidx)
+    # the reference's own sequence, statement by statement (tests/test_paired_output_constraint.py:58-62):
+    # counters cleared, variables rebuilt, a new problem assigned, the default rows added to it
+    rows = sorted(opt.prob.constraints)
+    objective = opt.prob.objective_value
+    opt.add_node_constraint(param, constraint_name="gone_with_the_old_problem")
+    opt._name_counters.clear()
+    opt.decision_vars = opt._build_decision_vars()
+    opt.prob = object()  # pulp.LpProblem("AutoParallel", pulp.LpMinimize) there
+    assert len(opt.prob.constraints) == 0 and opt._name_counters == {}
+    opt.add_default_constraints()
+    assert sorted(opt.prob.constraints) == rows  # the same rows under the same names, none twice
+    sol2 = opt.get_solution()
+    assert opt.prob.objective_value == objective
+    assert {n.name: str(s.output_specs) for n, s in sol2.items()} == {n.name: str(s.output_specs) for n, s in sol.items()}
+    # one group at a time, and counters that can be assigned (serialization.py:266)
+    opt.prob = None
+    opt._name_counters = {}
+    for add in (opt.add_unique_decision_constraint, opt.add_same_output_across_args_constraint,
+                opt.add_output_input_consistent_constraint, opt.add_inf_cost_constraint,
+                opt.add_forward_backward_consistency_constraints, opt.add_grad_reduce_dtype_constraints):
+        add()
+    assert sorted(opt.prob.constraints) == rows
 
 
 class _Block(nn.Module):
