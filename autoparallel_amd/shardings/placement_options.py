@@ -342,7 +342,9 @@ def _view_rule(mesh, node, src: OpStrategy) -> OpStrategy:
     strategy the propagation rejects is skipped."""
     from torch.distributed.tensor._ops._view_ops import dim_maps, propagate_shape_and_sharding
 
-    rules = dim_maps[torch.Tensor.view](src, node.args[1])
+    # the target sizes from the result: in a graph traced with symbolic sizes the
+    # argument holds nodes (a product of sizes), and a -1 is resolved there already
+    rules = dim_maps[torch.Tensor.view](src, tuple(int(d) for d in node.meta["val"].shape))
     out_tm = _tensor_meta(node.meta["val"])
     sts = []
     for s in src.strategies:

@@ -396,6 +396,48 @@ def test_rebuild_after_mutating_strategies(mesh):
     assert sorted(opt.prob.constraints) == rows
 
 
+def test_joint_graph_with_symbolic_batch_is_planned_on_its_concrete_twin(mesh):
+    """A joint graph traced with symbolic input sizes (the reference's dynamic=True,
+    autoparallel/api.py:129-154) is planned on a twin with the sizes' hints
+    (optimize_sharding.py:160-218): the same coefficients and the same plan as
+    the graph traced with plain sizes, and a solution keyed by the nodes of the
+    graph that was handed in."""
+    from torch._functorch.aot_autograd import aot_export_joint_with_descriptors
+    from torch._subclasses.fake_tensor import FakeTensorMode
+    from torch.fx.experimental.symbolic_shapes import DimDynamic, ShapeEnv, StatelessSymbolicContext
+
+    from autoparallel_amd.optimize_sharding import ShardingOptimizer, _has_symbolic_sizes
+
+    mode = FakeTensorMode(shape_env=ShapeEnv(), static_shapes=False)
+    with mode:
+        m = MLP()
+    meta = torch.empty(16, 32, 64, device="meta")
+    x = mode.from_tensor(meta, symbolic_context=StatelessSymbolicContext(dynamic_sizes=[DimDynamic.DYNAMIC] * 3))
+    with mode:
+        x = x.to("cpu")
+        with contextlib.ExitStack() as stack:
+            gm = aot_export_joint_with_descriptors(stack, m, (x,)).graph_module
+    assert _has_symbolic_sizes(gm)
+    dyn = ShardingOptimizer(gm, mesh, devices_per_host=8, device_name="AMD Instinct MI355X")
+    static = ShardingOptimizer(_joint_graph(), mesh, devices_per_host=8, device_name="AMD Instinct MI355X")
+    # planned on the twin: its graph is not the one handed in, and the maps between the two are total
+    assert dyn.graph is not gm.graph and set(dyn._concrete_to_orig.values()) == set(gm.graph.nodes)
+    assert all(not isinstance(d, torch.SymInt) for n in dyn.graph.nodes if isinstance(n.meta.get("val"), torch.Tensor)
+               for d in n.meta["val"].shape)
+    sol_d, sol_s = dyn.get_solution(), static.get_solution()
+    assert set(sol_d) <= set(gm.graph.nodes)  # keyed by the caller's nodes
+    assert dyn._core.objective_value == static._core.objective_value
+    from autoparallel_amd.optimize_sharding import _produces_tensor
+
+    # the symbolic trace only adds size arithmetic (sym_size, products of sizes): nodes without a tensor, not planned
+    ops = lambda opt: [str(n.target) for n in opt.graph.nodes if n.op == "call_function" and _produces_tensor(n.meta.get("val"))]
+    assert ops(dyn) == ops(static) and len(list(dyn.graph.nodes)) > len(list(static.graph.nodes))
+    assert len(dyn.decision_vars) == len(static.decision_vars)
+    assert bits_equal(dyn._core.coef.cost, static._core.coef.cost) and bits_equal(dyn._core.coef.comm, static._core.coef.comm)
+    by_name = lambda sol: [(str(n.target), str(s.output_specs)) for n, s in sol.items() if n.op == "call_function"]
+    assert by_name(sol_d) == by_name(sol_s)
+
+
 class _Block(nn.Module):
     """Embedding, layer norms, attention through scaled_dot_product_attention,
     a GELU MLP with biases: the op mix of a decoder block."""
