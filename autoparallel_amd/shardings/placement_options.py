@@ -593,6 +593,8 @@ def _without_partial(a):
 
 _NONSTRICT_VIEWS = {aten.view.default, aten._unsafe_view.default}
 # strategy functions of the installed torch that pair the arguments' strategies by index
+_INDEX_PUTS = {getattr(getattr(aten, name), "default") for name in ("index_put", "index_put_", "_index_put_impl_")
+               if hasattr(aten, name)}
 _INDEX_PAIRED = {getattr(getattr(aten, name), "default") for name in (
     "native_layer_norm", "native_layer_norm_backward", "_fused_rms_norm", "_fused_rms_norm_backward",
     "nll_loss_forward", "nll_loss_backward", "nll_loss2d_forward", "nll_loss2d_backward") if hasattr(aten, name)}
@@ -760,6 +762,11 @@ def _placement_options_uncached_inner(mesh, node, producers, arg_vals, schema_ar
             out = _view_dtype_rule(mesh, node, producers[0])
         else:
             fn = prop.op_strategy_funcs.get(op)
+            if fn is not None and op in _INDEX_PUTS and len(schema_args) > 1 and any(i is None for i in schema_args[1]):
+                # `out[:, idx] = ...`: a None among the indices for a dim that is left alone.  The rule
+                # of the installed torch takes tensors only (it asserts on the None), so for this
+                # form it is as if none were registered: the node gets the all-Replicate stand-in.
+                fn = None
             if fn is not None:
                 def wrap(x):
                     # a list argument with tensors in it, e.g. index_put's indices with None for

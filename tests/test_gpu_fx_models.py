@@ -1,0 +1,133 @@
+"""Small models of the reference's own end-to-end tests, traced the way the
+reference traces (its decomposition choices, autoparallel/tracing.py:14-36) and
+planned through ShardingOptimizer: the permute / LayerNorm / permute block with
+its non-contiguous strides, torch.arange (prims.iota), advanced indexing
+(index / index_put with a None among the indices), an MLP with biases (addmm
+taken apart so that the matmul can be sharded) (tests/test_propagation_rules.py:15-193)."""
+import contextlib
+import copy
+
+import numpy as np
+import pytest
+import torch
+import torch.nn as nn
+
+from helpers import bits_equal
+from oracle import cost_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def reference_style_decompositions():
+    from torch._inductor.decomposition import select_decomp_table
+
+    aten = torch.ops.aten
+    table = copy.copy(select_decomp_table())
+    for op in (aten.full_like.default, aten.empty_like.default, aten.threshold_backward.default,
+               aten.native_layer_norm.default, aten.embedding_dense_backward.default,
+               aten.native_layer_norm_backward.default, aten._softmax_backward_data.default, aten._softmax.default,
+               aten.stack.default, aten.addmm.default):
+        table.pop(op, None)
+    table[aten.addmm.default] = lambda self, mat1, mat2, beta=1, alpha=1: self + mat1 @ mat2
+    return table
+
+
+class PermuteLayerNorm(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.norm = nn.LayerNorm(96, eps=1e-6)
+
+    def forward(self, x):  # (N, C, H, W) -> (N, H, W, C) -> norm over C -> back
+        return self.norm(x.permute(0, 2, 3, 1)).permute(0, 3, 1, 2)
+
+
+class ArangeEmbedding(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.embed = nn.Embedding(256, 64)
+
+    def forward(self, x):
+        return x + self.embed(torch.arange(x.shape[1], device=x.device))
+
+
+class IndexPut(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.weight = nn.Parameter(torch.randn(32, 64))
+
+    def forward(self, x):
+        out = torch.zeros_like(x)
+        idx = torch.arange(x.shape[1], device=x.device)
+        out[:, idx] = x[:, idx]
+        return out @ self.weight
+
+
+class BiasedMLP(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.a, self.b = nn.Linear(64, 128), nn.Linear(128, 64)
+
+    def forward(self, x):
+        return self.b(torch.nn.functional.gelu(self.a(x)))
+
+
+CASES = {
+    # model, input shape, operators the trace must hold, nodes that get the all-Replicate stand-in
+    "permute_layer_norm": (PermuteLayerNorm, (256, 96, 56, 56), ("aten.permute.default", "aten.native_layer_norm.default"), set()),
+    "arange_embedding": (ArangeEmbedding, (256, 256, 64), ("prims.iota.default", "aten.embedding.default"), set()),
+    # torch 2.10 registers no strategy for index.Tensor, and its index_put rule takes no None index
+    "index_put": (IndexPut, (256, 32), ("aten.index_put.default", "aten.index.Tensor"), {"index", "index_put"}),
+    "biased_mlp": (BiasedMLP, (64, 128, 64), ("aten.mm.default", "aten.add.Tensor"), set()),
+}
+
+
+@pytest.fixture(scope="module")
+def meshes():
+    if not torch.cuda.is_available():
+        pytest.skip("needs a GPU")
+    import torch.distributed as dist
+    from torch.distributed.device_mesh import init_device_mesh
+    from torch.testing._internal.distributed.fake_pg import FakeStore
+
+    own = not dist.is_initialized()
+    if own:
+        dist.init_process_group("fake", store=FakeStore(), rank=0, world_size=8)
+    yield {"1d": init_device_mesh("cpu", (8,)), "2d": init_device_mesh("cpu", (2, 4))}
+    if own:
+        dist.destroy_process_group()
+
+
+@pytest.mark.parametrize("mesh_name", ["1d", "2d"])
+@pytest.mark.parametrize("case", list(CASES))
+def test_reference_style_trace_is_planned(meshes, case, mesh_name):
+    from torch._functorch.aot_autograd import aot_export_joint_with_descriptors
+    from torch._subclasses.fake_tensor import FakeTensorMode
+
+    from autoparallel_amd.optimize_sharding import ShardingOptimizer
+    from autoparallel_amd.shardings import placement_options as PO
+
+    cls, shape, must_have, stand_ins = CASES[case]
+    with FakeTensorMode():
+        model, x = cls(), torch.rand(*shape)
+        with contextlib.ExitStack() as stack:
+            gm = aot_export_joint_with_descriptors(stack, model, (x,), decompositions=reference_style_decompositions()).graph_module
+    targets = {str(n.target) for n in gm.graph.nodes if n.op == "call_function"}
+    assert set(must_have) <= targets, targets
+    assert "aten.addmm.default" not in targets
+    PO.fallback_nodes.clear()
+    PO.fallback_reasons.clear()
+    opt = ShardingOptimizer(gm, meshes[mesh_name], devices_per_host=8, device_name="AMD Instinct MI355X")
+    assert set(PO.fallback_reasons) == stand_ins, PO.fallback_reasons
+    # every coefficient against the oracle on the same packed problem
+    g = opt._packed
+    ref = O.GraphOracle(g).build()
+    slots = g.entry_slots()
+    cost_ref, _ = O.clamp_inf(ref["cost"])
+    assert bits_equal(opt._core.coef.comm, ref["comm"][slots]) and bits_equal(opt._core.coef.cost, cost_ref[slots])
+    sol = opt.get_solution()
+    assert set(sol) == {n for n in opt.nodes if n.op != "output"}
+    assert np.isfinite(opt._core.objective_value) and not opt._core.prob.violated()
+    # a node with the stand-in is Replicate on every mesh dim, inputs and output
+    for n, spec in sol.items():
+        if n.name in stand_ins:
+            assert all(p.is_replicate() for p in spec.output_specs.placements)
