@@ -405,6 +405,30 @@ def _one_strategy_at_a_time(fn, op, args, kwargs, producers: List[OpStrategy]) -
     return OpStrategy(sts)
 
 
+_reduction_rule_leaks: Optional[bool] = None
+
+
+def _reduction_rule_carries_state(mesh) -> bool:
+    """Whether the installed torch's rule for sum / mean / max ... decides once per call,
+    instead of per candidate, if a pending reduction has to be cleared first: one candidate
+    that is Partial with another reduce op then makes every later candidate lose its
+    shards on the reduced dims (and all of them collapse to the same Replicate answer).
+    The reference's tests state the per-candidate behaviour
+    (tests/test_reduction_strategies.py:63-117); probed once, on two candidates."""
+    global _reduction_rule_leaks
+    if _reduction_rule_leaks is None:
+        from torch.distributed.tensor._ops._math_ops import common_reduction_strategy
+
+        nd = mesh.ndim
+        tm = _tensor_meta(torch.empty((4 * mesh.size(), 4 * mesh.size()), device="meta"))
+        cands = [(Partial("avg"),) + (Replicate(),) * (nd - 1), (Shard(0),) + (Replicate(),) * (nd - 1)]
+        src = OpStrategy([OpSpec(DTensorSpec(mesh, c, tensor_meta=tm), input_specs=(), redistribute_cost=[]) for c in cands])
+        with _without_torch_cost_rows():
+            out = common_reduction_strategy(src, reduce_dims=[0], reduction_op="sum")
+        _reduction_rule_leaks = not out.strategies[1].output_specs.placements[0].is_partial()
+    return _reduction_rule_leaks
+
+
 def _local_map_rule(mesh, node, schema_args, kw) -> OpStrategy:
     """The single strategy of a ``local_map`` region: the placements its author
     declared (autoparallel/shardings/placement_options.py:380-490).  Arguments
@@ -784,6 +808,10 @@ def _placement_options_uncached_inner(mesh, node, producers, arg_vals, schema_ar
                     args = (args[0], d, i) + args[3:]
                 kwargs = {k: v for k, v in node.kwargs.items() if not isinstance(v, torch.fx.Node)}
                 if op in _INDEX_PAIRED and len(producers) > 1:
+                    res = _one_strategy_at_a_time(fn, op, args, kwargs, producers)
+                elif (getattr(fn, "__name__", "") == "linear_reduction_strategy" and len(producers) == 1
+                      and len(producers[0].strategies) > 1 and _reduction_rule_carries_state(mesh)):
+                    # each candidate of the input on its own, as the rule is meant to treat them
                     res = _one_strategy_at_a_time(fn, op, args, kwargs, producers)
                 else:
                     try:

@@ -560,3 +560,64 @@ def test_collector_state_is_restored():
         assert not gc.isenabled()  # it was off before: stays off
     finally:
         gc.enable()
+
+
+def _reduce_node(target, shape, args, out_shape):
+    g = torch.fx.Graph()
+    x = g.placeholder("x")
+    x.meta["val"] = torch.empty(shape, device="meta")
+    node = g.call_function(target, (x,) + tuple(args))
+    node.meta["val"] = torch.empty(out_shape, device="meta")
+    return x, node
+
+
+@pytest.mark.parametrize("cands, must_have", [
+    # both sharded dims are reduced: pending sums on both mesh dims
+    ([(Shard(0), Shard(1))], [("P(sum)", "P(sum)")]),
+    # the shards are on the dim that stays: it is dim 0 of the result
+    ([(Shard(2), Shard(2))], [("S(0)", "S(0)")]),
+    # a candidate that is Partial(avg) must not cost the later ones their shards
+    ([(Replicate(), Replicate()), (Replicate(), "avg"), (Shard(0), Shard(1)), (Shard(0), Shard(2))],
+     [("P(sum)", "P(sum)"), ("P(sum)", "S(0)"), ("R", "R")]),
+    ([(Replicate(), "avg"), (Shard(0), Shard(1))], [("R", "R"), ("P(sum)", "P(sum)")]),
+])
+def test_sum_treats_every_candidate_on_its_own(meshes, cands, must_have):
+    """The known answers of the reference's tests/test_reduction_strategies.py:38-117 for
+    sum over dims [0, 1] of a (32, 8192, 4096) tensor on a 2-D mesh, asked through the node
+    query: each candidate of the input keeps its own answer, whatever precedes it in the
+    list (torch 2.10's rule decides once per call; the query then asks candidate by candidate)."""
+    from torch.distributed.tensor.placement_types import Partial
+
+    from autoparallel_amd.shardings.placement_options import get_placement_options_for_node, reset_placement_options_cache
+
+    mesh = meshes[1]
+    shape = (32, 8192, 4096)
+    as_plc = lambda c: tuple(Partial(p) if isinstance(p, str) else p for p in c)
+    src = OpStrategy([_one(mesh, shape, as_plc(c)) for c in cands])
+    x, node = _reduce_node(torch.ops.aten.sum.dim_IntList, shape, ([0, 1],), (4096,))
+    reset_placement_options_cache()
+    out = get_placement_options_for_node(mesh, node, [src], [x.meta["val"]], (src, [0, 1]))
+
+    def short(p):
+        return "R" if p.is_replicate() else (f"S({p.dim})" if p.is_shard() else f"P({p.reduce_op})")
+
+    got = {tuple(short(p) for p in st.output_specs.placements) for st in out.strategies}
+    assert set(must_have) <= got, got
+    # one column per candidate of the input in every cost row
+    assert all(len(st.redistribute_cost) == 1 and len(st.redistribute_cost[0]) == len(cands) for st in out.strategies)
+
+
+def test_mean_of_sharded_and_replicated_candidates(meshes):
+    """mean over [0, 1] (tests/test_reduction_strategies.py:119-140): the replicated candidate
+    stays replicated, the one sharded on the reduced dims ends in a pending average."""
+    from autoparallel_amd.shardings.placement_options import get_placement_options_for_node, reset_placement_options_cache
+
+    mesh = meshes[1]
+    shape = (32, 8192, 4096)
+    src = OpStrategy([_one(mesh, shape, (Replicate(), Replicate())), _one(mesh, shape, (Shard(0), Shard(1)))])
+    x, node = _reduce_node(torch.ops.aten.mean.dim, shape, ([0, 1],), (4096,))
+    reset_placement_options_cache()
+    out = get_placement_options_for_node(mesh, node, [src], [x.meta["val"]], (src, [0, 1]))
+    got = {st.output_specs.placements for st in out.strategies}
+    assert (Replicate(), Replicate()) in got
+    assert any(all(p.is_partial() and p.reduce_op == "avg" for p in plc) for plc in got), got
