@@ -1050,6 +1050,21 @@ def test_hf_llama3_8b_layers_joint_graph():
         gc = clustered._packed
         assert gc.edge_alias is not None and gc.num_entries < 0.45 * g.num_entries
         assert len(clustered.decision_vars) == gc.num_entries == clustered._core.n_vars
+        # what the reference asks of its clustering on such a model (tests/test_graph_clustering.py:231-297):
+        # no region mixes forward and backward nodes, no node sits in two regions, the regions of a
+        # group are as long as each other, and most of the graph is covered
+        groups = clustered._core.region_groups
+        assert groups
+        seen = set()
+        for group in groups:
+            assert len(group) >= 2 and len({len(region) for region in group}) == 1
+            for region in group:
+                tags = {clustered.nodes[v].meta.get("partitioner_tag") for v in region} - {None}
+                assert len(tags) <= 1, tags
+                assert not (seen & set(region))
+                seen |= set(region)
+        n_ops = sum(1 for n in clustered.nodes if n.op == "call_function")
+        assert len(seen) >= 0.5 * n_ops, (len(seen), n_ops)
         own = np.repeat(gc.priced, g.block_sizes())
         assert bits_equal(clustered._core.coef.comm, opt._core.coef.comm[own])
         assert bits_equal(clustered._core.coef.cost, opt._core.coef.cost[own])
