@@ -48,61 +48,98 @@ def _produces_tensor(val) -> bool:
 
 
 class DecisionVar:
-    """One (node, arg, out, inp) choice; attribute reads and writes go to the
-    coefficient arrays (fields of the reference's dataclass, :191-203)."""
+    """One (node, arg, out, inp) choice.  Made by the optimizer it is a view:
+    attribute reads and writes go to the coefficient arrays.  Made from the
+    fields of the reference's dataclass (``DecisionVar(var=..., cost=...,
+    compute_cost=..., comm_cost=..., sharding_transition_cost=..., strategy=...,
+    output_spec=..., input_spec=...)``, autoparallel/optimize_sharding.py:191-203)
+    it is a record of its own that holds them."""
 
-    __slots__ = ("_opt", "_i", "key")
+    __slots__ = ("_opt", "_i", "key", "_own")
+    _FIELDS = ("var", "cost", "compute_cost", "comm_cost", "sharding_transition_cost", "strategy",
+               "output_spec", "input_spec")
 
-    def __init__(self, opt: "ShardingOptimizer", i: int, key: tuple):
-        self._opt, self._i, self.key = opt, i, key
+    def __init__(self, opt: Optional["ShardingOptimizer"] = None, i: Optional[int] = None, key: Optional[tuple] = None,
+                 **fields):
+        if opt is None:
+            unknown = set(fields) - set(self._FIELDS)
+            if unknown:
+                raise TypeError(f"DecisionVar got unexpected fields {sorted(unknown)}")
+            missing = [f for f in self._FIELDS if f not in fields]
+            if missing:
+                raise TypeError(f"DecisionVar is missing fields {missing}")
+            self._opt, self._i, self.key, self._own = None, None, key, dict(fields)
+        else:
+            assert not fields, "a view takes its fields from the optimizer"
+            self._opt, self._i, self.key, self._own = opt, i, key, None
 
     @property
-    def var(self) -> int:
-        return self._i  # column of the ILP
+    def var(self):
+        return self._i if self._own is None else self._own["var"]  # column of the ILP
 
     @property
     def cost(self) -> float:
-        return float(self._opt._core.coef.cost[self._i])
+        return float(self._opt._core.coef.cost[self._i]) if self._own is None else self._own["cost"]
 
     @cost.setter
     def cost(self, v: float) -> None:
-        self._opt._core.coef.cost[self._i] = v
+        if self._own is None:
+            self._opt._core.coef.cost[self._i] = v
+        else:
+            self._own["cost"] = v
 
     @property
     def comm_cost(self) -> float:
-        return float(self._opt._core.coef.comm[self._i])
+        return float(self._opt._core.coef.comm[self._i]) if self._own is None else self._own["comm_cost"]
 
     @comm_cost.setter
     def comm_cost(self, v: float) -> None:
-        self._opt._core.coef.comm[self._i] = v
+        if self._own is None:
+            self._opt._core.coef.comm[self._i] = v
+        else:
+            self._own["comm_cost"] = v
 
     @property
-    def sharding_transition_cost(self) -> int:
+    def sharding_transition_cost(self):
+        if self._own is not None:
+            return self._own["sharding_transition_cost"]
         return int(self._opt._core.coef.flags[self._i] & 1)
 
     @property
     def compute_cost(self) -> float:
+        if self._own is not None:
+            return self._own["compute_cost"]
         v, _, o, _ = self.key
         return float(self._opt._core.coef.per_arg[int(self._opt._packed.node_comp_off[v]) + o])
 
     @property
-    def strategy(self) -> OpSpec:
+    def strategy(self):
+        if self._own is not None:
+            return self._own["strategy"]
         v, _, o, _ = self.key
         return self._opt.strats[self._opt.nodes[v]].strategies[o]
 
     @property
     def output_spec(self):
-        return self.strategy.output_specs
+        return self.strategy.output_specs if self._own is None else self._own["output_spec"]
 
     @property
     def input_spec(self):
+        if self._own is not None:
+            return self._own["input_spec"]
         ins = self.strategy.input_specs
         a = self.key[1]
         return ins[a] if ins is not None and a < len(ins) else None
 
     def value(self) -> Optional[float]:
+        if self._own is not None:
+            v = self._own["var"]
+            return v.value() if hasattr(v, "value") else None
         x = self._opt._core.prob.x
         return None if x is None else float(x[self._i])
+
+    def __repr__(self) -> str:
+        return "DecisionVar(" + ", ".join(f"{f}={getattr(self, f)!r}" for f in self._FIELDS) + ")"
 
 
 class DecisionVars(collections.abc.Mapping):
