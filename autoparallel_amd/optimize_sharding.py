@@ -817,28 +817,12 @@ class ShardingOptimizer:
 
     # -- export / persistence ------------------------------------------------------------------
     def _node_info(self) -> List[Dict[str, Any]]:
-        """Per-node fields only the FX graph carries (export_json.py:362-407 of
-        the reference): op, phase, placeholder kind, source line."""
-        import re
+        """Per-node fields only the FX graph carries (export_json.py:362-407 of the
+        reference), and the cluster of every repeated node."""
+        from . import export_json
 
-        out = []
-        for node in self.nodes:
-            info: Dict[str, Any] = {"op": str(node.target) if node.op == "call_function" else node.op}
-            desc = type(node.meta.get("desc")).__name__ if node.meta.get("desc") is not None else None
-            kind = {"ParamAOTInput": "param", "BufferAOTInput": "buffer", "TangentAOTInput": "tangent",
-                    "PlainAOTInput": "input"}.get(desc)
-            if node.op == "placeholder" and kind:
-                info["placeholder_kind"] = kind
-            tag = node.meta.get("partitioner_tag")
-            info["phase"] = "backward" if tag == "is_backward" or kind == "tangent" else "forward"
-            st = node.meta.get("stack_trace")
-            if st:
-                frames = re.findall(r'File "([^"]+)", line (\d+), in (\w+)\n\s+(.*)', st)
-                if frames:
-                    f, line, fn, code = frames[-1]
-                    info["source"] = {"file": f, "line": int(line), "func": fn, "code": code.strip()}
-            out.append(info)
-        return out
+        linked = {self.nodes[v]: self.nodes[r] for v, r in self._core.cluster_links.items()}
+        return export_json.fx_node_info(self.nodes, linked)
 
     def get_json(self) -> Dict[str, Any]:
         from . import export_json

@@ -1,0 +1,133 @@
+"""The fields of the plan export that come from the FX graph (module path,
+phase, repeated-layer index, cluster roots): autoparallel_amd.export_json against
+the scenarios of the reference's tests/test_export_json.py:44-128 and the rules
+of its export_json.py:23-215."""
+import contextlib
+from types import SimpleNamespace
+
+import torch
+from torch import nn
+
+from autoparallel_amd import export_json as X
+
+
+class Repeated(nn.Module):
+    def __init__(self, dim, n_layers):
+        super().__init__()
+        self.embed = nn.Linear(dim, dim, bias=False)
+        self.layers = nn.ModuleList([nn.Linear(dim, dim, bias=False) for _ in range(n_layers)])
+        self.head = nn.Linear(dim, dim, bias=False)
+
+    def forward(self, x):
+        x = self.embed(x)
+        for layer in self.layers:
+            x = layer(x)
+        return self.head(x)
+
+
+def _joint(n_layers):
+    from torch._functorch.aot_autograd import aot_export_joint_with_descriptors
+    from torch._subclasses.fake_tensor import FakeTensorMode
+
+    with FakeTensorMode():
+        m, x = Repeated(64, n_layers), torch.rand(16, 64)
+        with contextlib.ExitStack() as stack:
+            return aot_export_joint_with_descriptors(stack, m, (x,)).graph_module
+
+
+def test_layer_index_from_the_module_stack():
+    gm = torch.fx.symbolic_trace(Repeated(64, 3))  # a tracer that records the module stack
+    layers, outside = set(), 0
+    for n in gm.graph.nodes:
+        i = X.layer_index(n)
+        if i is not None:
+            layers.add(i)
+        elif n.op not in ("placeholder", "output"):
+            outside += 1
+    assert layers == {0, 1, 2} and outside == 2  # embed and head are in no numbered layer
+    assert {X.module_path(n) for n in gm.graph.nodes if n.op == "call_module"} == {"embed", "layers.0", "layers.1", "layers.2", "head"}
+    assert X.layer_index(SimpleNamespace(meta={})) is None
+    assert X.layer_index(SimpleNamespace(meta={"nn_module_stack": {}})) is None
+    assert X.layer_index(SimpleNamespace(meta={"fwd_nn_module_stack": {"a": ("model.layers.17.mlp", nn.Linear)}})) == 17
+
+
+def test_phase_module_path_and_kinds_on_a_joint_graph():
+    gm = _joint(2)
+    nodes = list(gm.graph.nodes)
+    info = X.fx_node_info(nodes)
+    assert len(info) == len(nodes)
+    by_name = {n.name: i for n, i in zip(nodes, info)}
+    params = [n for n in nodes if n.op == "placeholder" and X.placeholder_kind(n) == "param"]
+    assert len(params) == 4 and all(by_name[p.name]["phase"] == "forward" for p in params)
+    assert {by_name[p.name]["module_path"] for p in params} == {"embed.weight", "layers.0.weight", "layers.1.weight", "head.weight"}
+    tangents = [n for n in nodes if X.placeholder_kind(n) == "tangent"]
+    assert tangents and all(by_name[t.name]["phase"] == "backward" and by_name[t.name]["placeholder_kind"] == "tangent" for t in tangents)
+    assert {i["phase"] for i in info} == {"forward", "backward"}
+    # this tracer records no module stack: a node next to a parameter is placed by it, the parameter counted by its module
+    first_use = [next(iter(p.users)) for p in params]
+    assert {by_name[n.name]["module_path"] for n in first_use} == {"embed", "layers.0", "layers.1", "head"}
+    assert all(i["op"] for i in info) and all("placeholder_kind" not in i for n, i in zip(nodes, info) if n.op != "placeholder")
+
+
+class _Node(SimpleNamespace):
+    __hash__ = object.__hash__  # nodes are dictionary keys, by identity
+
+    def __eq__(self, other):
+        return self is other
+
+
+def _fake(name, layer=None, op="call_function", inputs=(), users=(), **meta):
+    if layer is not None:
+        meta["nn_module_stack"] = {"m": (f"layers.{layer}.ffn", nn.Linear)}
+    return _Node(name=name, op=op, target=name, meta=meta, all_input_nodes=list(inputs), users=list(users))
+
+
+def test_module_path_of_a_node_that_lost_its_stack():
+    a = _fake("a", nn_module_stack={"m": ("model.layers.3.attn.wq", nn.Linear)})
+    b = _fake("b", op="placeholder", desc=SimpleNamespace(target="model.layers.3.attn.wq.weight"))
+    c = _fake("c", nn_module_stack={"m": ("model.layers.3.mlp", nn.Linear)})
+    assert X.module_path(a) == "model.layers.3.attn.wq" and X.module_path(b) == "model.layers.3.attn.wq.weight"
+    assert X.module_path(_fake("lost", inputs=[a, b])) == "model.layers.3.attn.wq"  # the parameter counts by its module
+    assert X.module_path(_fake("lost", inputs=[a], users=[c])) == "model.layers.3"
+    assert X.module_path(_fake("lost", inputs=[a], users=[_fake("z", nn_module_stack={"m": ("other.block", nn.Linear)})])) is None
+    assert X.module_path(_fake("lost", inputs=[_fake("r", nn_module_stack={"m": ("L['self']", nn.Module)})])) is None
+    assert X.module_path(_fake("alone")) is None
+    assert X.module_path(_fake("saved", module_path="kept.as.written")) == "kept.as.written"
+
+
+def test_phase_rules_in_their_order():
+    assert X.phase(_fake("n", phase="backward", partitioner_tag="is_forward")) == "backward"  # what a saved graph says wins
+    assert X.phase(_fake("n", partitioner_tag="is_backward")) == "backward"
+    assert X.phase(_fake("n", partitioner_tag="is_forward")) == "forward"
+    assert X.phase(_fake("tangents_1", op="placeholder")) == "backward" and X.phase(_fake("primals_1", op="placeholder")) == "forward"
+    assert X.phase(_fake("n", layer=0)) == "forward"
+    assert X.phase(_fake("n", fwd_nn_module_stack={"m": ("layers.0", nn.Linear)})) == "backward"
+    # nothing to go by: position relative to the first tangent input
+    graph = SimpleNamespace()
+    seq = [_fake("primals_1", op="placeholder"), _fake("x"), _fake("tangents_1", op="placeholder"), _fake("y")]
+    graph.nodes = seq
+    for n in seq:
+        n.graph = graph
+    assert X.phase(seq[1]) == "forward" and X.phase(seq[3]) == "backward"
+
+
+def test_clusters_are_rerooted_at_the_lowest_layer():
+    X.normalize_cluster_layer({})
+    # forward cluster rooted in layer 0, backward cluster rooted in layer 3 (topological order)
+    f = [_fake(f"f{i}", layer=i) for i in range(4)]
+    b = [_fake(f"b{i}", layer=i) for i in range(4)]
+    roots = {f[1]: f[0], f[2]: f[0], f[3]: f[0], b[0]: b[3], b[1]: b[3], b[2]: b[3]}
+    X.normalize_cluster_layer(roots)
+    assert roots == {f[1]: f[0], f[2]: f[0], f[3]: f[0], b[1]: b[0], b[2]: b[0], b[3]: b[0]}
+    # a cluster without a copy in the lowest layer moves to its nearest one; nodes outside numbered layers stay
+    c = [_fake(f"c{i}", layer=i) for i in (1, 2, 3)]
+    u = [_fake("u0"), _fake("u1")]
+    roots = {f[1]: f[0], c[0]: c[2], c[1]: c[2], u[1]: u[0]}
+    X.normalize_cluster_layer(roots)
+    assert roots == {f[1]: f[0], c[1]: c[0], c[2]: c[0], u[1]: u[0]}
+    # the export numbers clusters by root and names the root on the linked nodes only
+    info = X.fx_node_info(f + b, {f[1]: f[0], b[0]: b[3], b[1]: b[3]})
+    by = {n.name: i for n, i in zip(f + b, info)}
+    assert by["f0"]["cluster_id"] == by["f1"]["cluster_id"] and by["f1"]["cluster_root"] == "f0" and "cluster_root" not in by["f0"]
+    assert by["b0"]["cluster_id"] == by["b1"]["cluster_id"] == by["b3"]["cluster_id"] != by["f0"]["cluster_id"]
+    assert by["b1"]["cluster_root"] == by["b3"]["cluster_root"] == "b0" and "cluster_id" not in by["f2"]

@@ -321,6 +321,18 @@ def test_repeated_subgraphs_on_joint_graph(mesh):
     assert np.isclose(opt._core.objective_value, plain._core.objective_value, rtol=1e-6)
     assert len(opt.selected_keys) == opt._packed.num_edges  # root keys plus the expanded linked keys
     assert "total_cost:" in opt.get_log()
+    # the export names the cluster of every repeated node (autoparallel/export_json.py:396-401):
+    # a linked node carries its root's name, root and linked nodes share the cluster's number
+    data = opt.get_json()
+    by_name = {n["name"]: n for n in data["nodes"]}
+    linked = [n for n in data["nodes"] if "cluster_root" in n]
+    assert len(linked) == len(opt._cluster_linked_node_idxs) > 0
+    for n in linked:
+        root = by_name[n["cluster_root"]]
+        assert "cluster_root" not in root and root["cluster_id"] == n["cluster_id"] and root["op"] == n["op"]
+        assert root["placement"] == n["placement"]
+    assert all({"name", "op"} <= set(n) for n in data["nodes"]) and {"total", "comm", "compute"} <= set(data["summary"])
+    assert any(n.get("module_path") for n in data["nodes"]) and {n.get("phase") for n in data["nodes"]} >= {"forward", "backward"}
 
 
 def test_prefetch_discount_on_joint_graph(mesh):
