@@ -18,10 +18,12 @@ Constraint families and their reference counterparts:
 """
 from __future__ import annotations
 
+import collections.abc
 import dataclasses
 import logging
 import math
 import time
+import types
 from typing import Dict, Iterable, List, Optional, Sequence, Set, Tuple
 
 import numpy as np
@@ -98,6 +100,59 @@ class Coefficients:
         out.saved_arrays = (np.asarray(keys, np.int32), np.asarray(vals, np.float64))
         out.slot_arrays = (comm, cost, flags)
         return out
+
+
+class MeshPlaceholder:
+    """What a plan needs of a DeviceMesh when none exists (a problem reopened
+    without a process group): shape, dim names, ndim, size()
+    (autoparallel/serialization.py:25-42)."""
+
+    def __init__(self, shape, dim_names=None):
+        self.shape = tuple(int(x) for x in shape)
+        self.mesh_dim_names = tuple(dim_names) if dim_names else None
+        self.ndim = len(self.shape)
+
+    def size(self) -> int:
+        return int(np.prod(self.shape, dtype=np.int64)) if self.shape else 1
+
+
+class PackedDecisionVars(collections.abc.Mapping):
+    """(node, arg, out_idx, inp_idx) -> the variable's coefficients, in the
+    reference's key order, over the packed arrays."""
+
+    def __init__(self, core: "PackedShardingOptimizer"):
+        self._core = core
+        self._keys = None
+
+    def _all(self) -> np.ndarray:
+        if self._keys is None:
+            self._keys = self._core.g.entry_keys()[self._core.g.decision_var_order()]
+        return self._keys
+
+    def __len__(self) -> int:
+        return self._core.n_vars
+
+    def __iter__(self):
+        return (tuple(int(x) for x in k) for k in self._all())
+
+    def __getitem__(self, key):
+        core, g = self._core, self._core.g
+        try:
+            v, a, o, j = (int(x) for x in key)
+        except (TypeError, ValueError):
+            raise KeyError(key) from None
+        if not (0 <= v < g.num_nodes and 0 <= a < int(g.node_edge_off[v + 1]) - int(g.node_edge_off[v])):
+            raise KeyError(key)
+        e = int(g.node_edge_off[v]) + a
+        # a linked node has no variables of its own: its root's stand for it
+        if core.linked[v] or not (0 <= o < int(g.edge_sdst[e]) and 0 <= j < int(g.edge_ssrc[e])):
+            raise KeyError(key)
+        i = int(core.var_start[e]) + o * int(g.edge_ssrc[e]) + j
+        x = core.prob.x
+        return types.SimpleNamespace(
+            var=i, cost=float(core.coef.cost[i]), comm_cost=float(core.coef.comm[i]),
+            compute_cost=float(core.coef.per_arg[int(core.g.node_comp_off[v]) + o]),
+            sharding_transition_cost=int(core.coef.flags[i] & 1), value=None if x is None else float(x[i]))
 
 
 class PackedShardingOptimizer:
@@ -621,6 +676,37 @@ class PackedShardingOptimizer:
         a = torch.from_numpy(np.ascontiguousarray(sol.astype(np.int16))).to(eng.device)
         terms, slot = eng.solution_terms(a)
         return terms.cpu().numpy(), slot.cpu().numpy()
+
+    # -- what code written for the reference reads on an optimizer it loaded (serialization.py:25-42,
+    #    tests/test_serialization.py:119-260): nodes, decision variables by key, the mesh's shape, the
+    #    selected keys
+    @property
+    def nodes(self) -> List[str]:
+        """Node names in graph order (the reference holds fx nodes there; a reloaded packed problem has their names)."""
+        return list(self.g.node_names) if self.g.node_names else [f"node{i}" for i in range(self.g.num_nodes)]
+
+    @property
+    def mesh(self) -> "MeshPlaceholder":
+        return MeshPlaceholder([int(x) for x in self.g.mesh_shape], self.mesh_dim_names)
+
+    @property
+    def selected_keys(self) -> List[Tuple[int, int, int, int]]:
+        """(node, arg, out_idx, inp_idx) of every selected variable, the expanded ones of linked nodes
+        included (optimize_sharding.py:896-905)."""
+        if self.selected is None:
+            return []
+        sol = self._extract()
+        keys = [tuple(int(x) for x in k) for k in self.g.entry_keys()[self.selected]]
+        g = self.g
+        for v in np.nonzero(self.linked)[0]:
+            for a, e in enumerate(range(int(g.node_edge_off[v]), int(g.node_edge_off[v + 1]))):
+                u = int(g.edge_src_node[e])
+                keys.append((int(v), a, int(sol[v]), int(sol[u]) if u >= 0 else 0))
+        return keys
+
+    @property
+    def decision_vars(self) -> "PackedDecisionVars":
+        return PackedDecisionVars(self)
 
     def save(self, path: str) -> None:
         from . import serialization

@@ -91,6 +91,35 @@ def test_save_load_roundtrip(tiny, tmp_path):
     assert np.isclose(loaded.objective_value, opt.objective_value, rtol=1e-12)
     loaded._memory_constraint = None
     assert np.array_equal(loaded.resolve(), sol)
+    # what code written for the reference reads on the object it loaded (its tests/test_serialization.py:136-168,
+    # 183-190): node and variable counts, a mesh stand-in with the shape, the selected keys, variables by key
+    assert len(loaded.nodes) == len(opt.nodes) == g.num_nodes and loaded.nodes == list(g.node_names)
+    assert len(loaded.decision_vars) == len(opt.decision_vars) == g.num_entries
+    assert loaded.mesh.shape == tuple(int(x) for x in g.mesh_shape) and loaded.mesh.ndim == len(g.mesh_shape)
+    assert loaded.mesh.size() == int(np.prod(g.mesh_shape)) and loaded.mesh.mesh_dim_names is None
+    keys = loaded.selected_keys
+    assert len(keys) == g.num_edges and {k[0] for k in keys} == set(range(g.num_nodes))
+    assert all(loaded.decision_vars[k].value == 1.0 and k in loaded.decision_vars for k in keys)
+    total = sum(loaded.decision_vars[k].cost for k in keys)
+    assert np.isclose(total, loaded.objective_value, rtol=1e-12)
+    order = list(loaded.decision_vars)
+    assert order == sorted(order, key=lambda k: (k[0], k[2], k[1], k[3])) and len(order) == g.num_entries
+    k0 = order[len(order) // 2]
+    dv = loaded.decision_vars[k0]
+    assert dv.cost == dv.comm_cost + dv.compute_cost + dv.sharding_transition_cost or dv.cost == 10000.0
+    for bad in ((g.num_nodes, 0, 0, 0), (0, 99, 0, 0), (k0[0], k0[1], 10**6, 0), "x"):
+        assert bad not in loaded.decision_vars
+        with pytest.raises(KeyError):
+            loaded.decision_vars[bad]
+
+
+def test_mesh_placeholder_known_answers():
+    from autoparallel_amd.sharding_problem import MeshPlaceholder
+
+    m = MeshPlaceholder((32, 8), ("dp", "tp"))
+    assert m.shape == (32, 8) and m.mesh_dim_names == ("dp", "tp") and m.ndim == 2 and m.size() == 256
+    m = MeshPlaceholder((64,), None)
+    assert m.mesh_dim_names is None and m.ndim == 1 and m.size() == 64
 
 
 def test_unsolved_save_and_version_check(tiny, tmp_path):
