@@ -131,3 +131,51 @@ def test_reference_style_trace_is_planned(meshes, case, mesh_name):
     for n, spec in sol.items():
         if n.name in stand_ins:
             assert all(p.is_replicate() for p in spec.output_specs.placements)
+
+
+def test_uneven_shards_are_offered_and_can_be_forced(meshes):
+    """A weight dim that the mesh dim does not divide is still offered sharded on it
+    while every shard is non-empty (the reference's tests/test_dynamic_shapes.py:1537-1640,
+    remove_invalid_configs: the local size is a ceiling division), and the plan can be
+    pinned to such a placement."""
+    from torch._functorch._aot_autograd.fx_utils import get_param_nodes
+    from torch._functorch.aot_autograd import aot_export_joint_with_descriptors
+    from torch._subclasses.fake_tensor import FakeTensorMode
+    from torch.distributed.tensor.placement_types import Replicate, Shard
+
+    from autoparallel_amd.optimize_sharding import ShardingOptimizer
+
+    class FFN(nn.Module):
+        def __init__(self, d1, d2):
+            super().__init__()
+            self.w1, self.w2 = nn.Linear(d1, d2, bias=False), nn.Linear(d2, d1, bias=False)
+
+        def forward(self, x):
+            return self.w2(torch.relu(self.w1(x)))
+
+    mesh = meshes["2d"]  # (2, 4)
+    d1, d2 = 102, 400    # 102 = 4 * 25 + 2: uneven on the second mesh dim, every shard non-empty
+    with FakeTensorMode():
+        model, x = FFN(d1, d2), torch.randn(16, d1)
+        with contextlib.ExitStack() as stack:
+            gm = aot_export_joint_with_descriptors(stack, model, (x,), decompositions=reference_style_decompositions()).graph_module
+    opt = ShardingOptimizer(gm, mesh, devices_per_host=8, device_name="AMD Instinct MI355X")
+    w1 = get_param_nodes(gm.graph)[0]
+    assert tuple(w1.meta["val"].shape) == (d2, d1)
+    on_tp = {s.output_specs.placements[1].dim for s in opt.strats[w1].strategies if s.output_specs.placements[1].is_shard()}
+    assert on_tp == {0, 1}
+    # a dim smaller than the mesh dim is not offered: 3 rows cannot fill 4 shards
+    with FakeTensorMode():
+        tiny, xt = FFN(3, 400), torch.randn(16, 3)
+        with contextlib.ExitStack() as stack:
+            gt = aot_export_joint_with_descriptors(stack, tiny, (xt,), decompositions=reference_style_decompositions()).graph_module
+    ot = ShardingOptimizer(gt, mesh, devices_per_host=8, device_name="AMD Instinct MI355X")
+    wt = get_param_nodes(gt.graph)[0]
+    assert {s.output_specs.placements[1].dim for s in ot.strats[wt].strategies if s.output_specs.placements[1].is_shard()} == {0}
+    # pinned to the uneven placement, the plan is found and the weight's bytes are those of the ceiling shard
+    opt.add_node_constraint(w1, (Replicate(), Shard(1)))
+    sol = opt.get_solution()
+    assert sol[w1].output_specs.placements == (Replicate(), Shard(1))
+    g = opt._packed
+    ref = O.GraphOracle(g).build()
+    assert bits_equal(opt._core.coef.comm, ref["comm"][g.entry_slots()])
