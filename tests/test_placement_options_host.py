@@ -621,3 +621,28 @@ def test_mean_of_sharded_and_replicated_candidates(meshes):
     got = {st.output_specs.placements for st in out.strategies}
     assert (Replicate(), Replicate()) in got
     assert any(all(p.is_partial() and p.reduce_op == "avg" for p in plc) for plc in got), got
+
+
+def test_tensor_meta_of_the_result_is_written_over_filled_in_or_left_alone(meshes):
+    """The three cases of the reference's tests/test_placement_options_utils.py:193-240:
+    an existing tensor meta on the output spec is replaced by the result's, a missing one
+    is filled in, a strategy without an output spec (a non-tensor getitem) is skipped."""
+    from autoparallel_amd.shardings.placement_options import propagate_tensor_meta
+
+    mesh = meshes[0]
+    val = torch.empty(4, 8, device="meta")
+    node = _fx_node(torch.ops.aten.neg.default, (), val)
+    stale = _tm((2, 2))
+    spec = DTensorSpec(mesh, (Replicate(),), tensor_meta=stale)
+    strat = OpStrategy([OpSpec(spec, input_specs=[DTensorSpec(mesh, (Replicate(),))], redistribute_cost=[[0.0]])])
+    propagate_tensor_meta(node, [val], strat, mesh)
+    got = strat.strategies[0].output_specs.tensor_meta
+    assert got is not stale and got.shape == torch.Size([4, 8]) and got.stride == (8, 1)
+    assert strat.strategies[0].input_specs[0].tensor_meta.shape == torch.Size([4, 8])  # inputs are filled in too
+    bare = OpStrategy([OpSpec(DTensorSpec(mesh, (Replicate(),)), input_specs=[spec], redistribute_cost=[[0.0]])])
+    assert bare.strategies[0].output_specs.tensor_meta is None
+    propagate_tensor_meta(node, [val], bare, mesh)
+    assert bare.strategies[0].output_specs.tensor_meta.shape == torch.Size([4, 8])
+    none = OpStrategy([OpSpec(None, input_specs=[spec], redistribute_cost=[[0.0]])])
+    propagate_tensor_meta(node, [val], none, mesh)
+    assert none.strategies[0].output_specs is None
