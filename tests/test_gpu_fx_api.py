@@ -766,6 +766,63 @@ def test_collectives_stay_on_the_narrow_side_of_a_cast(mesh):
                 assert sol[n].input_specs[0].placements == sol[n.all_input_nodes[0]].output_specs.placements
 
 
+def test_reduction_after_the_cast_holds_for_repeated_layers_too(mesh):
+    """With gradients reduced in the higher precision and repeated layers sharing their
+    variables, no selected variable on the way from a weight-gradient matmul to its cast
+    moves data, the expanded variables of linked layers included (the reference's
+    tests/test_grad_reduce_dtype.py:147-171 with its check :53-125)."""
+    from torch._functorch._aot_autograd import fx_utils
+    from torch._functorch.aot_autograd import aot_export_joint_with_descriptors
+    from torch._subclasses.fake_tensor import FakeTensorMode
+
+    from autoparallel_amd.optimize_sharding import ShardingOptimizer
+
+    class Stacked(nn.Module):
+        def __init__(self, n=4, d=128):
+            super().__init__()
+            self.ws = nn.ParameterList([nn.Parameter(torch.randn(d, d)) for _ in range(n)])
+
+        def forward(self, x):
+            for w in self.ws:
+                x = torch.relu(x @ w.to(torch.bfloat16).t())
+            return x.float().pow(2).mean()
+
+    with FakeTensorMode():
+        with torch.device("cuda"):
+            m = Stacked()
+        x = torch.randn(64, 128, device="cuda", dtype=torch.bfloat16)
+        with contextlib.ExitStack() as stack:
+            gm = aot_export_joint_with_descriptors(stack, m, (x,)).graph_module
+    cast = torch.ops.aten._to_copy.default
+    old = ShardingOptimizer.dtype_cast_targets
+    ShardingOptimizer.dtype_cast_targets = {cast}
+    try:
+        opt = ShardingOptimizer(gm, mesh, True, repeated_subgraphs=True, devices_per_host=8,
+                                device_name="AMD Instinct MI355X")
+    finally:
+        ShardingOptimizer.dtype_cast_targets = old
+    assert opt.cluster_links
+    sol = opt.get_solution()
+    checked = checked_linked = 0
+    for param, grad in fx_utils.get_param_and_grad_nodes(gm.graph).values():
+        assert grad is not None and grad.target is cast
+        chain, n = [grad], grad  # the unary chain that ends in the gradient
+        while len(n.all_input_nodes) == 1 and len(n.all_input_nodes[0].all_input_nodes) == 1:
+            n = n.all_input_nodes[0]
+            chain.append(n)
+        at = next(i for i, c in enumerate(chain) if c.target is cast)
+        before = {opt.node_map[c] for c in chain[at:] if c in opt.node_map}
+        for key in opt.selected_keys:
+            if key[0] in before:
+                dv = opt._resolve_decision_var(key)
+                checked += 1
+                checked_linked += key in opt.cluster_links
+                assert dv.comm_cost == 0, (opt.nodes[key[0]].name, dv.comm_cost)
+        assert any(p.is_partial() for p in sol[chain[at]].output_specs.placements) or \
+            all(p.is_replicate() for p in sol[param].output_specs.placements)
+    assert checked > 0 and checked_linked > 0
+
+
 def test_hf_gpt2_layers_under_the_default_memory_budget(mesh):
     """Two GPT-2 layers prepared as the reference prepares its graph (alias nodes)
     with the batch-sharded input and the default parameter budget of 1 / mesh size
