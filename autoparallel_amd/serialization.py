@@ -71,7 +71,12 @@ def _json_arr(obj) -> np.ndarray:
 
 
 def save_optimizer(core, path: str, mesh_dim_names: Optional[List[str]] = None) -> None:
-    """core: a PackedShardingOptimizer (solved or not)."""
+    """core: a PackedShardingOptimizer (solved or not), or the ShardingOptimizer that holds one
+    (the reference's call, ``save_optimizer(opt, path)``, autoparallel/serialization.py:145)."""
+    if hasattr(core, "_core"):
+        if mesh_dim_names is None and getattr(core.mesh, "mesh_dim_names", None):
+            mesh_dim_names = list(core.mesh.mesh_dim_names)
+        core = core._core
     g = core.g
     keys, vals = core.decision_var_arrays()
     names = g.node_names or [f"node{i}" for i in range(g.num_nodes)]
@@ -103,7 +108,10 @@ def load_optimizer(path: str, cls=None):
     file holds one, the saved solution."""
     from .sharding_problem import Coefficients, PackedShardingOptimizer
 
-    cls = cls or PackedShardingOptimizer
+    if isinstance(path, type) or (cls is not None and not isinstance(cls, type)):
+        path, cls = cls, path  # the reference's order: load_optimizer(cls, path) (autoparallel/serialization.py:298)
+    if cls is None or not issubclass(cls, PackedShardingOptimizer):
+        cls = PackedShardingOptimizer  # a file holds the packed problem, whichever class asked for it
     with np.load(path, allow_pickle=False) as d:
         version = int(d["version"])
         if version != FORMAT_VERSION:

@@ -113,6 +113,19 @@ def test_save_load_roundtrip(tiny, tmp_path):
             loaded.decision_vars[bad]
 
 
+def test_load_takes_the_reference_argument_order_too(tiny, tmp_path):
+    from autoparallel_amd import serialization
+
+    g, coef, _ = tiny
+    opt = PackedShardingOptimizer(g, coefficients=coef)
+    path = str(tmp_path / "o.npz")
+    serialization.save_optimizer(opt, path)
+    a = serialization.load_optimizer(path)
+    b = serialization.load_optimizer(PackedShardingOptimizer, path)  # load_optimizer(cls, path) there
+    c = serialization.load_optimizer(path, object)  # a class that is not the packed one: the packed one is made
+    assert type(a) is type(b) is type(c) is PackedShardingOptimizer and a.n_vars == b.n_vars == c.n_vars == opt.n_vars
+
+
 def test_mesh_placeholder_known_answers():
     from autoparallel_amd.sharding_problem import MeshPlaceholder
 
