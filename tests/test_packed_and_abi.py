@@ -395,3 +395,31 @@ def test_layout_choice_and_caches_travel_with_the_graph(small_llama):
     # a graph derived from it starts without them
     alias = np.arange(g.num_edges)
     assert "_work_items" not in g.with_edge_alias(alias).__dict__
+
+
+def test_every_entry_point_refuses_a_problem_it_could_not_walk():
+    """No GPU is touched: a null problem, an empty one (no mesh) and one whose counts
+    name arrays that are not there are turned away on the host, with a status below zero
+    and a message, by every entry point that takes a problem."""
+    from autoparallel_amd import _lib
+
+    lib = _lib.load()
+    ptr = ctypes.POINTER(_lib.ApcProblem)
+    ints = (ctypes.c_int, ctypes.c_int32, ctypes.c_int64, ctypes.c_uint32, ctypes.c_uint64)
+    takers = [(name, args) for name, (res, args) in _lib._SIGNATURES.items()
+              if res is ctypes.c_int and args and args[0] is ptr]
+    assert len(takers) >= 20
+
+    def call(name, args, first):
+        rest = [0 if a in ints else 0.0 if a in (ctypes.c_double, ctypes.c_float) else None for a in args[1:]]
+        return getattr(lib, name)(first, *rest)
+
+    empty = _lib.ApcProblem()
+    no_arrays = _lib.ApcProblem()
+    no_arrays.model.ndim = 2
+    no_arrays.model.mesh_shape[0], no_arrays.model.mesh_shape[1] = 2, 4
+    no_arrays.n_node, no_arrays.n_edge, no_arrays.n_entry, no_arrays.n_slot, no_arrays.n_chunk, no_arrays.n_item = 5, 7, 100, 112, 7, 1
+    for name, args in takers:
+        for what, first in (("null", None), ("empty", ctypes.byref(empty)), ("no arrays", ctypes.byref(no_arrays))):
+            rc = call(name, args, first)
+            assert rc < 0 and lib.apc_last_error(), (name, what, rc)
