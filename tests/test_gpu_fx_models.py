@@ -179,3 +179,93 @@ def test_uneven_shards_are_offered_and_can_be_forced(meshes):
     g = opt._packed
     ref = O.GraphOracle(g).build()
     assert bits_equal(opt._core.coef.comm, ref["comm"][g.entry_slots()])
+
+
+# ---------------------------------------------------------------------------
+# Architectures of the transformers library at toy sizes: encoder, encoder-decoder,
+# vision, grouped-query decoder, mixture of experts.
+# ---------------------------------------------------------------------------
+def _hf_cases():
+    import transformers as T
+
+    small = dict(hidden_size=128, num_hidden_layers=2, num_attention_heads=4, intermediate_size=256, vocab_size=512,
+                 max_position_embeddings=128)
+    return {
+        "bert": (T.BertConfig, T.BertForMaskedLM, dict(hidden_dropout_prob=0.0, attention_probs_dropout_prob=0.0, **small), torch.float32),
+        "t5": (T.T5Config, T.T5ForConditionalGeneration,
+               dict(d_model=128, d_kv=32, d_ff=256, num_layers=2, num_heads=4, vocab_size=512, dropout_rate=0.0), torch.float32),
+        "vit": (T.ViTConfig, T.ViTForImageClassification,
+                dict(hidden_size=128, num_hidden_layers=2, num_attention_heads=4, intermediate_size=256, image_size=32,
+                     patch_size=8, hidden_dropout_prob=0.0, attention_probs_dropout_prob=0.0), torch.float32),
+        "mistral": (T.MistralConfig, T.MistralForCausalLM, dict(num_key_value_heads=2, sliding_window=None, **small), torch.float32),
+        "mixtral": (T.MixtralConfig, T.MixtralForCausalLM,
+                    dict(num_key_value_heads=2, num_local_experts=4, num_experts_per_tok=2, **small), torch.bfloat16),
+    }
+
+
+class _HFLoss(nn.Module):
+    def __init__(self, model, kind):
+        super().__init__()
+        self.m, self.kind = model, kind
+
+    def forward(self, x):
+        if self.kind in ("mistral", "mixtral"):  # the decoder layers themselves: no mask is built from data
+            m = self.m.model
+            h = m.embed_tokens(x)
+            pos = torch.arange(x.shape[1], device=x.device)[None]
+            pe = m.rotary_emb(h, pos)
+            for layer in m.layers:
+                o = layer(h, attention_mask=None, position_ids=pos, position_embeddings=pe)
+                h = o[0] if isinstance(o, tuple) else o
+            logits = self.m.lm_head(m.norm(h))
+        elif self.kind == "vit":
+            logits = self.m(pixel_values=x).logits
+        elif self.kind == "t5":
+            logits = self.m(input_ids=x, decoder_input_ids=x).logits
+        else:
+            logits = self.m(input_ids=x).logits
+        return logits.float().pow(2).mean()
+
+
+# operators for which torch 2.10 registers no strategy (they get the all-Replicate stand-in)
+_NO_STRATEGY_IN_THIS_TORCH = {"aten.convolution.default", "aten.convolution_backward.default", "aten.index.Tensor",
+                              "aten.floor_divide.default"}
+
+
+@pytest.mark.parametrize("kind", ["bert", "t5", "vit", "mistral", "mixtral"])
+def test_transformers_architectures_are_planned(meshes, kind):
+    pytest.importorskip("transformers")
+    from torch._functorch.aot_autograd import aot_export_joint_with_descriptors
+    from torch._subclasses.fake_tensor import FakeTensorMode
+
+    from autoparallel_amd.optimize_sharding import ShardingOptimizer
+    from autoparallel_amd.shardings import placement_options as PO
+
+    cfg_cls, model_cls, kwargs, dtype = _hf_cases()[kind]
+    cfg = cfg_cls(**kwargs)
+    cfg.use_cache = False
+    cfg._attn_implementation = "sdpa"
+    with FakeTensorMode():
+        torch.set_default_dtype(dtype)
+        try:
+            with torch.device("cuda"):
+                model = _HFLoss(model_cls(cfg), kind)
+        finally:
+            torch.set_default_dtype(torch.float32)
+        x = torch.rand(8, 3, 32, 32, device="cuda") if kind == "vit" else torch.randint(0, 512, (8, 64), device="cuda")
+        with contextlib.ExitStack() as stack:
+            gm = aot_export_joint_with_descriptors(stack, model, (x,)).graph_module
+    PO.fallback_nodes.clear()
+    PO.fallback_reasons.clear()
+    opt = ShardingOptimizer(gm, meshes["2d"], devices_per_host=8, device_name="AMD Instinct MI355X")
+    by_name = {n.name: n for n in opt.nodes}
+    assert {str(by_name[k].target) for k in PO.fallback_reasons} <= _NO_STRATEGY_IN_THIS_TORCH, PO.fallback_reasons
+    g = opt._packed
+    assert g.num_nodes > 300 and g.num_entries > 40000
+    ref = O.GraphOracle(g).build()
+    slots = g.entry_slots()
+    cost_ref, _ = O.clamp_inf(ref["cost"])
+    assert bits_equal(opt._core.coef.comm, ref["comm"][slots]) and bits_equal(opt._core.coef.cost, cost_ref[slots])
+    assert bits_equal(opt._core.coef.compute, ref["compute"])
+    sol = opt.get_solution()
+    assert set(sol) == {n for n in opt.nodes if n.op != "output"} and not opt._core.prob.violated()
