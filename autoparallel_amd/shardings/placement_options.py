@@ -617,6 +617,19 @@ def _without_partial(a):
 
 _NONSTRICT_VIEWS = {aten.view.default, aten._unsafe_view.default}
 # strategy functions of the installed torch that pair the arguments' strategies by index
+# Elementwise operators that the installed torch may leave without a strategy (it tags some of
+# them pointwise, not all): they take DTensor's pointwise rule instead of the stand-in.
+_ELEMENTWISE_BY_NAME = {getattr(getattr(aten, name), overload) for name, overload in (
+    ("floor_divide", "default"), ("floor_divide", "Scalar"), ("hardswish", "default"), ("hardswish_backward", "default"),
+    ("leaky_relu", "default"), ("leaky_relu_backward", "default"), ("hardsigmoid", "default"),
+    ("hardsigmoid_backward", "default"), ("elu_backward", "default"), ("softplus_backward", "default"),
+    ("mish_backward", "default"), ("div", "Scalar_mode")) if hasattr(getattr(aten, name, None), overload)}
+
+
+def _is_elementwise(op) -> bool:
+    return op in _ELEMENTWISE_BY_NAME or torch.Tag.pointwise in getattr(op, "tags", ())
+
+
 _INDEX_PUTS = {getattr(getattr(aten, name), "default") for name in ("index_put", "index_put_", "_index_put_impl_")
                if hasattr(aten, name)}
 _INDEX_PAIRED = {getattr(getattr(aten, name), "default") for name in (
@@ -786,6 +799,8 @@ def _placement_options_uncached_inner(mesh, node, producers, arg_vals, schema_ar
             out = _view_dtype_rule(mesh, node, producers[0])
         else:
             fn = prop.op_strategy_funcs.get(op)
+            if fn is None and producers and _is_elementwise(op):
+                from torch.distributed.tensor._ops._pointwise_ops import pointwise_strategy as fn
             if fn is not None and op in _INDEX_PUTS and len(schema_args) > 1 and any(i is None for i in schema_args[1]):
                 # `out[:, idx] = ...`: a None among the indices for a dim that is left alone.  The rule
                 # of the installed torch takes tensors only (it asserts on the None), so for this

@@ -228,8 +228,7 @@ class _HFLoss(nn.Module):
 
 
 # operators for which torch 2.10 registers no strategy (they get the all-Replicate stand-in)
-_NO_STRATEGY_IN_THIS_TORCH = {"aten.convolution.default", "aten.convolution_backward.default", "aten.index.Tensor",
-                              "aten.floor_divide.default"}
+_NO_STRATEGY_IN_THIS_TORCH = {"aten.convolution.default", "aten.convolution_backward.default", "aten.index.Tensor"}
 
 
 @pytest.mark.parametrize("kind", ["bert", "t5", "vit", "mistral", "mixtral"])

@@ -646,3 +646,38 @@ def test_tensor_meta_of_the_result_is_written_over_filled_in_or_left_alone(meshe
     none = OpStrategy([OpSpec(None, input_specs=[spec], redistribute_cost=[[0.0]])])
     propagate_tensor_meta(node, [val], none, mesh)
     assert none.strategies[0].output_specs is None
+
+
+@pytest.mark.parametrize("target, extra", [
+    (torch.ops.aten.floor_divide.default, None), (torch.ops.aten.hardswish.default, ()), (torch.ops.aten.leaky_relu.default, (0.1,)),
+    (torch.ops.aten.mish.default, ()), (torch.ops.aten.softplus.default, ()),
+])
+def test_elementwise_operators_without_a_registered_strategy_are_pointwise(meshes, target, extra):
+    """torch 2.10 registers nothing for these; they are elementwise (some carry the pointwise
+    tag, some not), so they take DTensor's pointwise rule: the result follows the input's
+    shards instead of forcing everything to Replicate."""
+    from autoparallel_amd.shardings.placement_options import (fallback_reasons, get_placement_options_for_node,
+                                                              reset_placement_options_cache)
+
+    mesh = meshes[1]
+    shape = (256, 64)
+    cands = [(Replicate(), Replicate()), (Shard(0), Replicate()), (Shard(0), Shard(1)), (Replicate(), Shard(1))]
+    src = OpStrategy([_one(mesh, shape, c) for c in cands])
+    g = torch.fx.Graph()
+    x = g.placeholder("x")
+    x.meta["val"] = torch.empty(shape, device="meta")
+    if extra is None:  # binary: the same tensor on both sides
+        node = g.call_function(target, (x, x))
+        producers, vals, schema = [src, src], [x.meta["val"]] * 2, (src, src)
+    else:
+        node = g.call_function(target, (x,) + tuple(extra))
+        producers, vals, schema = [src], [x.meta["val"]], (src,) + tuple(extra)
+    node.meta["val"] = torch.empty(shape, device="meta")
+    reset_placement_options_cache()
+    fallback_reasons.clear()
+    out = get_placement_options_for_node(mesh, node, producers, vals, schema)
+    assert not fallback_reasons
+    got = {st.output_specs.placements for st in out.strategies}
+    assert set(cands) <= got
+    for st in out.strategies:  # elementwise: every input is placed like the output
+        assert all(s.placements == st.output_specs.placements for s in st.input_specs)
