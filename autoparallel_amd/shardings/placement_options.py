@@ -394,14 +394,24 @@ def _one_strategy_at_a_time(fn, op, args, kwargs, producers: List[OpStrategy]) -
         return a
 
     sts = []
+    refused = None
     for lead_st in lead.strategies:
         if not isinstance(lead_st.output_specs, DTensorSpec):
             return None
         plc = lead_st.output_specs
-        res = fn(OpSchema(op, tuple(narrow(a, plc) for a in args), kwargs))
+        try:
+            res = fn(OpSchema(op, tuple(narrow(a, plc) for a in args), kwargs))
+        except (ValueError, RuntimeError) as exc:
+            # the rule has no answer for this candidate (a mean over shards of unequal size, ...):
+            # the operator offers nothing that follows it, and reaching what it does offer
+            # from that candidate is priced like any other redistribution
+            refused = exc
+            continue
         if not isinstance(res, OpStrategy):
             return None
         sts.extend(res.strategies)
+    if not sts and refused is not None:
+        raise refused
     return OpStrategy(sts)
 
 
@@ -831,7 +841,9 @@ def _placement_options_uncached_inner(mesh, node, producers, arg_vals, schema_ar
                 else:
                     try:
                         res = fn(OpSchema(op, args, kwargs))
-                    except IndexError:
+                    except (IndexError, ValueError):
+                        # pairs candidates by index, or refuses one of them outright: candidate by
+                        # candidate, the refused ones dropped (raises again if none is accepted)
                         res = _one_strategy_at_a_time(fn, op, args, kwargs, producers)
                     except RuntimeError:
                         # some functions (the random ones) refuse an argument that may

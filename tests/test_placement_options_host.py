@@ -681,3 +681,35 @@ def test_elementwise_operators_without_a_registered_strategy_are_pointwise(meshe
     assert set(cands) <= got
     for st in out.strategies:  # elementwise: every input is placed like the output
         assert all(s.placements == st.output_specs.placements for s in st.input_specs)
+
+
+def test_a_candidate_the_rule_refuses_costs_only_that_candidate(meshes):
+    """nll_loss with reduction mean: torch's rule raises for an input candidate whose shards are
+    of unequal size (the mean over shards would be biased).  Asked candidate by candidate, the
+    operator simply offers nothing that follows that candidate; the others keep their answers and
+    every cost row still has a column per real candidate.  When every candidate is refused the
+    error is the rule's own."""
+    from autoparallel_amd.shardings.placement_options import get_placement_options_for_node, reset_placement_options_cache
+
+    mesh = meshes[1]  # (32, 8)
+    n, v = 16 * 2047, 512  # 32752 rows: 8 divides them, 32 does not
+    cands = [(Replicate(), Replicate()), (Replicate(), Shard(0)), (Shard(0), Replicate()), (Shard(0), Shard(0))]
+    logits = OpStrategy([_one(mesh, (n, v), c) for c in cands])
+    target = OpStrategy([_one(mesh, (n,), (Replicate(), Replicate()))])
+    g = torch.fx.Graph()
+    x, t = g.placeholder("x"), g.placeholder("t")
+    x.meta["val"] = torch.empty(n, v, device="meta")
+    t.meta["val"] = torch.empty(n, dtype=torch.int64, device="meta")
+    node = g.call_function(torch.ops.aten.nll_loss_forward.default, (x, t, None, 1, -100))
+    node.meta["val"] = (torch.empty((), device="meta"), torch.empty((), device="meta"))
+    reset_placement_options_cache()
+    out = get_placement_options_for_node(mesh, node, [logits, target], [x.meta["val"], t.meta["val"]], (logits, target, None, 1, -100))
+    followed = {st.input_specs[0].placements for st in out.strategies}
+    assert (Replicate(), Replicate()) in followed and (Replicate(), Shard(0)) in followed
+    assert (Shard(0), Replicate()) not in followed and (Shard(0), Shard(0)) not in followed
+    assert all(len(st.redistribute_cost[0]) == len(cands) and len(st.redistribute_cost[1]) == 1 for st in out.strategies)
+    only_uneven = OpStrategy([_one(mesh, (n, v), (Shard(0), Replicate()))])
+    reset_placement_options_cache()
+    with pytest.raises(ValueError, match="evenly sharded"):
+        get_placement_options_for_node(mesh, node, [only_uneven, target], [x.meta["val"], t.meta["val"]],
+                                       (only_uneven, target, None, 1, -100))
