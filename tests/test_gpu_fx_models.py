@@ -268,3 +268,53 @@ def test_transformers_architectures_are_planned(meshes, kind):
     assert bits_equal(opt._core.coef.compute, ref["compute"])
     sol = opt.get_solution()
     assert set(sol) == {n for n in opt.nodes if n.op != "output"} and not opt._core.prob.violated()
+
+
+@pytest.mark.parametrize("kind", ["bert", "mistral", "mixtral"])
+def test_the_whole_planning_sequence_on_architectures(meshes, kind, tmp_path):
+    """What a caller of the reference does around the planner, in its order: linear layers as
+    einsums, alias nodes, repeated layers sharing variables, the batch-sharded input pinned, the
+    default parameter budget, solve, the log and the export, save and reopen."""
+    pytest.importorskip("transformers")
+    from torch._functorch.aot_autograd import aot_export_joint_with_descriptors
+    from torch._subclasses.fake_tensor import FakeTensorMode
+    from torch.distributed.tensor.placement_types import Replicate, Shard
+
+    from autoparallel_amd.graph_utils import add_alias_nodes, replace_view_mm_view_with_einsum
+    from autoparallel_amd.optimize_sharding import ShardingOptimizer
+
+    cfg_cls, model_cls, kwargs, dtype = _hf_cases()[kind]
+    cfg = cfg_cls(**kwargs)
+    cfg.use_cache = False
+    cfg._attn_implementation = "sdpa"
+    with FakeTensorMode():
+        torch.set_default_dtype(dtype)
+        try:
+            with torch.device("cuda"):
+                model = _HFLoss(model_cls(cfg), kind)
+        finally:
+            torch.set_default_dtype(torch.float32)
+        x = torch.randint(0, 512, (8, 64), device="cuda")
+        with contextlib.ExitStack() as stack:
+            gm = aot_export_joint_with_descriptors(stack, model, (x,)).graph_module
+    mesh = meshes["2d"]
+    assert replace_view_mm_view_with_einsum(gm) > 10
+    add_alias_nodes(gm)
+    opt = ShardingOptimizer(gm, mesh, repeated_subgraphs=True, devices_per_host=8, device_name="AMD Instinct MI355X")
+    assert opt._cluster_linked_node_idxs
+    opt.add_sharded_input_constraint([(Shard(0), Replicate())])
+    opt.add_parameter_memory_constraint(0.0, 1.0 / mesh.size())
+    plan = opt.get_solution()
+    ids = next(n for n in opt.nodes if n.op == "placeholder" and type(n.meta.get("desc")).__name__ == "PlainAOTInput")
+    assert plan[ids].output_specs.placements == (Shard(0), Replicate())
+    assert "total_cost:" in opt.get_log() and "Violated constraints: []" in opt.get_log()
+    data = opt.get_json()
+    assert abs(data["summary"]["total"] - sum(data["summary"][k] for k in ("comm", "compute", "transition"))) < 1e-6
+    assert sum("cluster_root" in n for n in data["nodes"]) == len(opt._cluster_linked_node_idxs)
+    opt.save(str(tmp_path / "o.npz"))
+    again = type(opt).load(str(tmp_path / "o.npz"))
+    assert np.isclose(again.objective_value, opt._core.objective_value, rtol=1e-12)
+    assert len(again.decision_vars) == len(opt.decision_vars) and len(again.selected_keys) == len(opt.selected_keys)
+    opt.save_placements(str(tmp_path / "p.json"))
+    back = opt.load_placements(str(tmp_path / "p.json"))
+    assert all(str(back[n].output_specs) == str(plan[n].output_specs) for n in plan)
