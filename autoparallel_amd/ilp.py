@@ -234,6 +234,10 @@ class SparseILP:
         ptr = np.zeros(lens.shape[0] + 1, np.int64)
         np.cumsum(lens, out=ptr[1:])
         A = sp.csr_matrix((cat(data, np.float64), cat(cols, np.int64), ptr), shape=(lens.shape[0], self.n_vars))
+        # A row may name a variable twice: with repeated subgraphs sharing variables, the two sides of
+        # a difference row can stand for the same ones.  HiGHS takes such a matrix for a model error.
+        A.sum_duplicates()
+        A.eliminate_zeros()
         return A, cat(lo, np.float64), cat(hi, np.float64), ub
 
     # -- solve ------------------------------------------------------------------
@@ -259,6 +263,11 @@ class SparseILP:
         res = milp(self.objective, constraints=cons, integrality=np.ones(self.n_vars),
                    bounds=Bounds(np.zeros(self.n_vars), ub), options=opts)
         if res.x is None:
+            if res.status not in (2, 3):  # scipy's milp: 2 infeasible, 3 unbounded; anything else is not an answer
+                raise RuntimeError(f"the ILP solver did not solve the problem: {res.message}")
+            if "infeasible" not in str(res.message).lower() and res.status == 2:
+                # status 2 also stands for a model HiGHS refuses to read
+                raise RuntimeError(f"the ILP solver refused the problem: {res.message}")
             self.status = STATUS_INFEASIBLE
             self.x = None
             self.objective_value = None

@@ -360,7 +360,13 @@ class PackedShardingOptimizer:
         u = g.edge_src_node.astype(np.int64)
         v = g.edge_node.astype(np.int64)
         has = np.nonzero(u >= 0)[0]
-        has = has[~(self.linked[u[has]] & self.linked[v[has]])]  # the root-to-root edge covers those
+        # an edge between two linked nodes is covered by the edge between their roots
+        # (autoparallel/optimize_sharding.py:743-746) -- when the roots are joined by one: regions of
+        # different groups can meet so that the producer's root is not what the consumer's root
+        # reads at that argument, and then the edge needs its own rows
+        both = self.linked[u[has]] & self.linked[v[has]]
+        covered = both & (g.edge_src_node[self.edge_alias[has]].astype(np.int64) == self.root[u[has]])
+        has = has[~covered]
         if has.size == 0:
             return
         _, firsts = np.unique(u[has] * g.num_nodes + v[has], return_index=True)  # first matching argument only

@@ -494,6 +494,23 @@ def _product_rule(mesh, rows, n_out: int) -> OpStrategy:
     return OpStrategy(sts)
 
 
+def _conv_rule(mesh, node, producers: List[OpStrategy]) -> OpStrategy:
+    """Convolution where the installed torch registers no strategy for it (it has a
+    run-time propagation rule only): per mesh dim either everything Replicate, or the
+    batch sharded with weight and bias Replicate, which is exact because the operator
+    is linear in the batch: the output (and the input gradient) is sharded on the batch,
+    the weight and bias gradients are pending sums.  Sharding channels or spatial dims
+    would need halo exchanges or other collectives inside the operator and is not offered."""
+    R, S0, P = Replicate(), Shard(0), Partial()
+    if node.target is aten.convolution.default:
+        n_in = len(producers)  # input, weight, and bias when there is one
+        rows = [[R] + [R] * n_in, [S0] + [S0, R] + [R] * (n_in - 2)]
+        return _product_rule(mesh, rows, 1)
+    assert len(producers) == 3  # grad_output, input, weight -> grad_input, grad_weight, grad_bias
+    rows = [[R, R, R] + [R, R, R], [S0, P, P] + [S0, S0, R]]
+    return _product_rule(mesh, rows, 3)
+
+
 def _stack_rule(mesh, node, producers: List[OpStrategy]) -> OpStrategy:
     """stack: inputs all Replicate or all sharded on the same dim, the output on
     that dim shifted past the new one (autoparallel/shardings/propagation_rules.py:621-656;
@@ -640,6 +657,7 @@ def _is_elementwise(op) -> bool:
     return op in _ELEMENTWISE_BY_NAME or torch.Tag.pointwise in getattr(op, "tags", ())
 
 
+_CONVOLUTIONS = {aten.convolution.default, aten.convolution_backward.default}
 _INDEX_PUTS = {getattr(getattr(aten, name), "default") for name in ("index_put", "index_put_", "_index_put_impl_")
                if hasattr(aten, name)}
 _INDEX_PAIRED = {getattr(getattr(aten, name), "default") for name in (
@@ -807,6 +825,8 @@ def _placement_options_uncached_inner(mesh, node, producers, arg_vals, schema_ar
             out = _split_with_sizes_rule(mesh, node, producers[0])
         elif op is aten.view.dtype and len(producers) == 1:
             out = _view_dtype_rule(mesh, node, producers[0])
+        elif op in _CONVOLUTIONS and op not in prop.op_strategy_funcs and len(producers) >= 2:
+            out = _conv_rule(mesh, node, producers)
         else:
             fn = prop.op_strategy_funcs.get(op)
             if fn is None and producers and _is_elementwise(op):

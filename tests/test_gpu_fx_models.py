@@ -318,3 +318,52 @@ def test_the_whole_planning_sequence_on_architectures(meshes, kind, tmp_path):
     opt.save_placements(str(tmp_path / "p.json"))
     back = opt.load_placements(str(tmp_path / "p.json"))
     assert all(str(back[n].output_specs) == str(plan[n].output_specs) for n in plan)
+
+
+def test_regions_of_different_groups_that_meet(meshes):
+    """The vision model's backward holds small repeated chains (a bias gradient: view, sum, view)
+    whose producers belong to regions of another group, rooted elsewhere; and chains that hang off
+    different outputs of one attention backward.  Two things went wrong there: a difference row
+    named a variable twice, which the solver took for a broken model and the planner reported as
+    infeasible; and an edge between two linked nodes was left to an edge between their roots that
+    does not exist.  The clustered plan, expanded, must cost on the engine that priced every node
+    exactly what the clustered objective says."""
+    pytest.importorskip("transformers")
+    from torch._functorch.aot_autograd import aot_export_joint_with_descriptors
+    from torch._subclasses.fake_tensor import FakeTensorMode
+    from torch.distributed.tensor.placement_types import Replicate, Shard
+
+    from autoparallel_amd.graph_utils import add_alias_nodes, replace_view_mm_view_with_einsum
+    from autoparallel_amd.optimize_sharding import ShardingOptimizer
+
+    cfg_cls, model_cls, kwargs, dtype = _hf_cases()["vit"]
+    cfg = cfg_cls(**kwargs)
+    cfg._attn_implementation = "sdpa"
+    with FakeTensorMode():
+        with torch.device("cuda"):
+            model = _HFLoss(model_cls(cfg), "vit")
+        x = torch.rand(8, 3, 32, 32, device="cuda")
+        with contextlib.ExitStack() as stack:
+            gm = aot_export_joint_with_descriptors(stack, model, (x,)).graph_module
+    replace_view_mm_view_with_einsum(gm)
+    add_alias_nodes(gm)
+    mesh = meshes["2d"]
+    kw = dict(devices_per_host=8, device_name="AMD Instinct MI355X")
+    full = ShardingOptimizer(gm, mesh, **kw)
+    clustered = ShardingOptimizer(gm, mesh, repeated_subgraphs=True, **kw)
+    core = clustered._core
+    g = core.g
+    u, v = g.edge_src_node.astype(np.int64), g.edge_node.astype(np.int64)
+    has = np.nonzero(u >= 0)[0]
+    both = core.linked[u[has]] & core.linked[v[has]]
+    uncovered = both & (g.edge_src_node[core.edge_alias[has]] != core.root[u[has]])
+    assert uncovered.sum() > 0  # the case is present in this graph
+    for opt in (full, clustered):
+        opt.add_sharded_input_constraint([(Shard(0), Replicate())])
+        opt.add_parameter_memory_constraint(0.0, 1.0 / mesh.size())
+    plan = clustered.get_solution()
+    full.get_solution()
+    assert clustered._core.objective_value >= full._core.objective_value * (1 - 1e-9)
+    idx = torch.from_numpy(clustered._out_indices(plan).astype(np.int16).reshape(-1, 1)).cuda()
+    r = full._core.engine.score(idx).cpu().numpy()[0]
+    assert r[5] == 0 and np.isclose(r[4], clustered._core.objective_value, rtol=1e-9)

@@ -713,3 +713,47 @@ def test_a_candidate_the_rule_refuses_costs_only_that_candidate(meshes):
     with pytest.raises(ValueError, match="evenly sharded"):
         get_placement_options_for_node(mesh, node, [only_uneven, target], [x.meta["val"], t.meta["val"]],
                                        (only_uneven, target, None, 1, -100))
+
+
+def test_convolution_is_offered_replicated_or_batch_sharded(meshes):
+    """torch 2.10 registers no strategy for convolution: per mesh dim, all Replicate or the batch
+    sharded with the weights Replicate; backward the same with the weight and bias gradients as
+    pending sums, and no spec for an output the mask switches off."""
+    from torch.distributed.tensor.placement_types import Partial
+
+    from autoparallel_amd.shardings.placement_options import (fallback_reasons, get_placement_options_for_node,
+                                                              reset_placement_options_cache)
+
+    mesh = meshes[1]  # (32, 8)
+    g = torch.fx.Graph()
+    vals = {"x": (512, 3, 16, 16), "w": (8, 3, 3, 3), "b": (8,), "go": (512, 8, 16, 16)}
+    ph = {}
+    for k, shape in vals.items():
+        ph[k] = g.placeholder(k)
+        ph[k].meta["val"] = torch.empty(shape, device="meta")
+    full = lambda shape: OpStrategy([_one(mesh, shape, p) for p in
+                                    [(Replicate(), Replicate()), (Shard(0), Replicate()), (Shard(0), Shard(0)), (Shard(1), Replicate())]])
+    sx, sw, sb, sgo = full(vals["x"]), full(vals["w"]), OpStrategy([_one(mesh, vals["b"], (Replicate(), Replicate()))]), full(vals["go"])
+    conv = g.call_function(torch.ops.aten.convolution.default, (ph["x"], ph["w"], ph["b"], [1, 1], [1, 1], [1, 1], False, [0, 0], 1))
+    conv.meta["val"] = torch.empty(vals["go"], device="meta")
+    reset_placement_options_cache()
+    fallback_reasons.clear()
+    out = get_placement_options_for_node(mesh, conv, [sx, sw, sb], [ph[k].meta["val"] for k in "xwb"],
+                                         (sx, sw, sb, [1, 1], [1, 1], [1, 1], False, [0, 0], 1))
+    assert not fallback_reasons
+    got = {(st.output_specs.placements, tuple(s.placements for s in st.input_specs)) for st in out.strategies}
+    R, S0 = Replicate(), Shard(0)
+    assert got == {((a, b), ((a, b), (R, R), (R, R))) for a in (R, S0) for b in (R, S0)}
+    assert all([len(r) for r in st.redistribute_cost] == [4, 4, 1] for st in out.strategies)
+    bwd = g.call_function(torch.ops.aten.convolution_backward.default,
+                          (ph["go"], ph["x"], ph["w"], [8], [1, 1], [1, 1], [1, 1], False, [0, 0], 1, [False, True, True]))
+    bwd.meta["val"] = (None, torch.empty(vals["w"], device="meta"), torch.empty(vals["b"], device="meta"))
+    out = get_placement_options_for_node(mesh, bwd, [sgo, sx, sw], [ph[k].meta["val"] for k in ("go", "x", "w")],
+                                         (sgo, sx, sw, [8], [1, 1], [1, 1], [1, 1], False, [0, 0], 1, [False, True, True]))
+    assert not fallback_reasons and len(out.strategies) == 4
+    for st in out.strategies:
+        gi, gw, gb = st.output_specs
+        a = st.input_specs[0].placements
+        assert gi is None and st.input_specs[1].placements == a and st.input_specs[2].placements == (R, R)
+        want = tuple(Partial() if p.is_shard() else R for p in a)
+        assert gw.placements == gb.placements == want and gw.tensor_meta.shape == torch.Size(vals["w"])

@@ -168,6 +168,26 @@ def test_sparse_ilp_basics():
 # ---------------------------------------------------------------------------
 # repeated-subgraph clustering (host logic; hashes from the oracle here)
 # ---------------------------------------------------------------------------
+def test_a_row_that_names_a_variable_twice_is_merged_not_refused():
+    """With repeated subgraphs sharing variables the two sides of a difference row can stand for
+    the same variables.  The solver takes a matrix with duplicate entries for a model error, which
+    is not the same as an infeasible problem: the entries are merged, and a row that cancels
+    itself out says nothing."""
+    p = ilp.SparseILP(3)
+    p.objective[:] = [1.0, 2.0, 3.0]
+    p.add_row("twice", [0, 0, 1], [1.0, -1.0, 1.0], ilp.EQ, 1.0)  # x0 - x0 + x1 == 1
+    p.add_row("cancels", [2, 2], [1.0, -1.0], ilp.EQ, 0.0)        # x2 - x2 == 0
+    p.add_row("doubles", [0, 0, 2], [1.0, 1.0, 1.0], ilp.GE, 1.0)  # 2 x0 + x2 >= 1
+    A, lo, hi, ub = p.to_matrix()
+    assert A.has_canonical_format and A.shape == (3, 3)
+    assert A[0].toarray().tolist() == [[0.0, 1.0, 0.0]] and A[1].nnz == 0 and A[2].toarray().tolist() == [[2.0, 0.0, 1.0]]
+    assert p.solve() == ilp.STATUS_OPTIMAL and p.x.tolist() == [1.0, 1.0, 0.0] and p.objective_value == 3.0
+    # a problem without a solution is still reported as that
+    q = ilp.SparseILP(2)
+    q.add_row("too_much", [0, 1], [1.0, 1.0], ilp.EQ, 3.0)
+    assert q.solve() == ilp.STATUS_INFEASIBLE and q.x is None
+
+
 def test_clustered_ilp_matches_reference_semantics():
     from autoparallel_amd import clustering
     from oracle import cluster_oracle as CO
@@ -321,7 +341,11 @@ def _rows_one_at_a_time(opt):
     seen, users = set(), {}
     for e in range(g.num_edges):
         u, v = int(g.edge_src_node[e]), int(g.edge_node[e])
-        if u < 0 or (opt.linked[u] and opt.linked[v]) or (u, v) in seen:
+        # an edge between two linked nodes has no rows of its own when the edge between their roots
+        # stands for it (autoparallel/optimize_sharding.py:743-746); where the producer's root is not
+        # what the consumer's root reads there, it keeps them
+        covered = u >= 0 and opt.linked[u] and opt.linked[v] and int(g.edge_src_node[int(opt.edge_alias[e])]) == int(opt.root[u])
+        if u < 0 or covered or (u, v) in seen:
             continue
         seen.add((u, v))
         users.setdefault(u, []).append(e)
