@@ -494,6 +494,56 @@ def _product_rule(mesh, rows, n_out: int) -> OpStrategy:
     return OpStrategy(sts)
 
 
+def _from_propagation_rule(rule, op, mesh, schema_args, producers: List[OpStrategy]) -> Optional[OpStrategy]:
+    """Strategies of a gather (``index.Tensor``, ``index_select``) for which the installed torch
+    has a run-time propagation rule but no strategy function: the rule is asked once per candidate
+    of the indexed tensor, the index tensors Replicate; where it answers with a suggestion (the
+    candidate is sharded on an indexed dim) the suggested inputs are taken and it is asked again."""
+    if not producers:
+        return None
+
+    def replicated(a: OpStrategy) -> DTensorSpec:
+        sp = a.strategies[0].output_specs
+        return DTensorSpec(mesh, (Replicate(),) * mesh.ndim, tensor_meta=sp.tensor_meta)
+
+    def specs_in(args):
+        out = []
+        for a in args:
+            if isinstance(a, DTensorSpec):
+                out.append(a)
+            elif isinstance(a, (list, tuple)):
+                out.extend(x for x in a if isinstance(x, DTensorSpec))
+        return out
+
+    sts, seen = [], set()
+    for cand in producers[0].strategies:
+        if not isinstance(cand.output_specs, DTensorSpec):
+            return None
+        first = True
+        args = []
+        for a in schema_args:
+            if isinstance(a, OpStrategy):
+                args.append(cand.output_specs if first else replicated(a))
+                first = False
+            elif isinstance(a, (list, tuple)) and any(isinstance(y, OpStrategy) for y in a):
+                args.append([replicated(y) if isinstance(y, OpStrategy) else y for y in a])
+            else:
+                args.append(a)
+        answer = rule(OpSchema(op, tuple(args), {}))
+        if answer.output_spec is None and answer.redistribute_schema is not None:
+            args = list(answer.redistribute_schema.args_schema)
+            answer = rule(answer.redistribute_schema)
+        if not isinstance(answer.output_spec, DTensorSpec):
+            continue
+        ins = specs_in(args)
+        key = (answer.output_spec.placements, tuple(x.placements for x in ins))
+        if len(ins) == len(producers) and key not in seen:
+            seen.add(key)
+            sts.append(OpSpec(DTensorSpec(mesh, answer.output_spec.placements),
+                              input_specs=tuple(DTensorSpec(mesh, x.placements, tensor_meta=x.tensor_meta) for x in ins)))
+    return OpStrategy(sts) if sts else None
+
+
 def _conv_rule(mesh, node, producers: List[OpStrategy]) -> OpStrategy:
     """Convolution where the installed torch registers no strategy for it (it has a
     run-time propagation rule only): per mesh dim either everything Replicate, or the
@@ -657,6 +707,7 @@ def _is_elementwise(op) -> bool:
     return op in _ELEMENTWISE_BY_NAME or torch.Tag.pointwise in getattr(op, "tags", ())
 
 
+_GATHERS = {aten.index.Tensor, aten.index_select.default}
 _CONVOLUTIONS = {aten.convolution.default, aten.convolution_backward.default}
 _INDEX_PUTS = {getattr(getattr(aten, name), "default") for name in ("index_put", "index_put_", "_index_put_impl_")
                if hasattr(aten, name)}
@@ -827,6 +878,8 @@ def _placement_options_uncached_inner(mesh, node, producers, arg_vals, schema_ar
             out = _view_dtype_rule(mesh, node, producers[0])
         elif op in _CONVOLUTIONS and op not in prop.op_strategy_funcs and len(producers) >= 2:
             out = _conv_rule(mesh, node, producers)
+        elif op in _GATHERS and op not in prop.op_strategy_funcs and op in prop.op_to_rules:
+            out = _from_propagation_rule(prop.op_to_rules[op], op, mesh, schema_args, producers)
         else:
             fn = prop.op_strategy_funcs.get(op)
             if fn is None and producers and _is_elementwise(op):

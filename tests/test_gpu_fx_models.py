@@ -75,8 +75,8 @@ CASES = {
     # model, input shape, operators the trace must hold, nodes that get the all-Replicate stand-in
     "permute_layer_norm": (PermuteLayerNorm, (256, 96, 56, 56), ("aten.permute.default", "aten.native_layer_norm.default"), set()),
     "arange_embedding": (ArangeEmbedding, (256, 256, 64), ("prims.iota.default", "aten.embedding.default"), set()),
-    # torch 2.10 registers no strategy for index.Tensor, and its index_put rule takes no None index
-    "index_put": (IndexPut, (256, 32), ("aten.index_put.default", "aten.index.Tensor"), {"index", "index_put"}),
+    # torch 2.10's index_put rule takes no None index (index.Tensor is planned from its run-time rule)
+    "index_put": (IndexPut, (256, 32), ("aten.index_put.default", "aten.index.Tensor"), {"index_put"}),
     "biased_mlp": (BiasedMLP, (64, 128, 64), ("aten.mm.default", "aten.add.Tensor"), set()),
 }
 
@@ -228,7 +228,7 @@ class _HFLoss(nn.Module):
 
 
 # operators for which torch 2.10 registers no strategy (they get the all-Replicate stand-in)
-_NO_STRATEGY_IN_THIS_TORCH = {"aten.convolution.default", "aten.convolution_backward.default", "aten.index.Tensor"}
+_NO_STRATEGY_IN_THIS_TORCH = {"aten.select_scatter.default"}
 
 
 @pytest.mark.parametrize("kind", ["bert", "t5", "vit", "mistral", "mixtral"])

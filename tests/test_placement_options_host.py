@@ -757,3 +757,31 @@ def test_convolution_is_offered_replicated_or_batch_sharded(meshes):
         assert gi is None and st.input_specs[1].placements == a and st.input_specs[2].placements == (R, R)
         want = tuple(Partial() if p.is_shard() else R for p in a)
         assert gw.placements == gb.placements == want and gw.tensor_meta.shape == torch.Size(vals["w"])
+
+
+def test_gather_strategies_come_from_the_run_time_rule(meshes):
+    """``x[idx]`` (aten.index.Tensor): torch 2.10 has a propagation rule for it, no strategy
+    function.  One answer per candidate of the indexed tensor: a shard on a dim that is not
+    indexed survives (moved past the index's dims), a shard on the indexed dim is given up
+    for Replicate, the index itself Replicate."""
+    from autoparallel_amd.shardings.placement_options import (fallback_reasons, get_placement_options_for_node,
+                                                              reset_placement_options_cache)
+
+    mesh = meshes[1]
+    R = Replicate()
+    g = torch.fx.Graph()
+    x, i = g.placeholder("x"), g.placeholder("i")
+    x.meta["val"] = torch.empty(512, 256, device="meta")
+    i.meta["val"] = torch.empty(1024, dtype=torch.int64, device="meta")
+    sx = OpStrategy([_one(mesh, (512, 256), p) for p in [(R, R), (Shard(1), R), (Shard(0), R), (R, Shard(1)), (Shard(0), Shard(1))]])
+    si = OpStrategy([_one(mesh, (1024,), p) for p in [(R, R), (Shard(0), R)]])
+    node = g.call_function(torch.ops.aten.index.Tensor, (x, [i]))
+    node.meta["val"] = torch.empty(1024, 256, device="meta")
+    reset_placement_options_cache()
+    fallback_reasons.clear()
+    out = get_placement_options_for_node(mesh, node, [sx, si], [x.meta["val"], i.meta["val"]], (sx, [si]))
+    assert not fallback_reasons
+    got = {(st.input_specs[0].placements, st.input_specs[1].placements, st.output_specs.placements) for st in out.strategies}
+    assert got == {((R, R), (R, R), (R, R)), ((Shard(1), R), (R, R), (Shard(1), R)), ((R, Shard(1)), (R, R), (R, Shard(1)))}
+    assert all([len(r) for r in st.redistribute_cost] == [5, 2] for st in out.strategies)
+    assert all(st.output_specs.tensor_meta.shape == torch.Size([1024, 256]) for st in out.strategies)
