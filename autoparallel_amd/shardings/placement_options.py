@@ -707,6 +707,10 @@ def _is_elementwise(op) -> bool:
     return op in _ELEMENTWISE_BY_NAME or torch.Tag.pointwise in getattr(op, "tags", ())
 
 
+# reshapes that the installed torch may leave without a strategy: planned like a view to the result's shape
+_RESHAPES_BY_RESULT = {getattr(aten.squeeze, "dims")} if hasattr(aten.squeeze, "dims") else set()
+# (var, mean) in one operator: the strategies of var, the one spec standing for both results
+_SAME_AS = {aten.var_mean.correction: aten.var.correction} if hasattr(aten.var_mean, "correction") else {}
 _GATHERS = {aten.index.Tensor, aten.index_select.default}
 _CONVOLUTIONS = {aten.convolution.default, aten.convolution_backward.default}
 _INDEX_PUTS = {getattr(getattr(aten, name), "default") for name in ("index_put", "index_put_", "_index_put_impl_")
@@ -864,7 +868,7 @@ def _placement_options_uncached_inner(mesh, node, producers, arg_vals, schema_ar
             out = _follow_input(mesh, producers[0], node.meta["val"])
         elif op is aten.einsum.default and len(producers) == 2:
             out = _einsum_rule(mesh, node, *producers)
-        elif op in _NONSTRICT_VIEWS and len(producers) == 1:
+        elif (op in _NONSTRICT_VIEWS or (op in _RESHAPES_BY_RESULT and op not in prop.op_strategy_funcs)) and len(producers) == 1:
             out = _view_rule(mesh, node, producers[0])
         elif op is aten.alias.default and len(producers) == 1:
             out = _alias_rule(mesh, node, producers[0])
@@ -882,6 +886,8 @@ def _placement_options_uncached_inner(mesh, node, producers, arg_vals, schema_ar
             out = _from_propagation_rule(prop.op_to_rules[op], op, mesh, schema_args, producers)
         else:
             fn = prop.op_strategy_funcs.get(op)
+            if fn is None and op in _SAME_AS:
+                fn = prop.op_strategy_funcs.get(_SAME_AS[op])
             if fn is None and producers and _is_elementwise(op):
                 from torch.distributed.tensor._ops._pointwise_ops import pointwise_strategy as fn
             if fn is not None and op in _INDEX_PUTS and len(schema_args) > 1 and any(i is None for i in schema_args[1]):

@@ -785,3 +785,38 @@ def test_gather_strategies_come_from_the_run_time_rule(meshes):
     assert got == {((R, R), (R, R), (R, R)), ((Shard(1), R), (R, R), (Shard(1), R)), ((R, Shard(1)), (R, R), (R, Shard(1)))}
     assert all([len(r) for r in st.redistribute_cost] == [5, 2] for st in out.strategies)
     assert all(st.output_specs.tensor_meta.shape == torch.Size([1024, 256]) for st in out.strategies)
+
+
+def test_squeeze_of_several_dims_and_var_mean_have_strategies(meshes):
+    """Both come out of the decomposition of batch norm; torch 2.10 registers neither.  squeeze.dims
+    is a reshape to the result's shape; var_mean takes var's strategies, one spec for both results."""
+    from autoparallel_amd.shardings.placement_options import (fallback_reasons, get_placement_options_for_node,
+                                                              reset_placement_options_cache)
+
+    mesh = meshes[1]
+    R = Replicate()
+    g = torch.fx.Graph()
+    x = g.placeholder("x")
+    x.meta["val"] = torch.empty(1, 64, 1, 512, device="meta")
+    sx = OpStrategy([_one(mesh, (1, 64, 1, 512), p) for p in [(R, R), (Shard(1), R), (Shard(3), Shard(1))]])
+    sq = g.call_function(torch.ops.aten.squeeze.dims, (x, [0, 2]))
+    sq.meta["val"] = torch.empty(64, 512, device="meta")
+    reset_placement_options_cache()
+    fallback_reasons.clear()
+    out = get_placement_options_for_node(mesh, sq, [sx], [x.meta["val"]], (sx, [0, 2]))
+    assert not fallback_reasons
+    assert {(st.input_specs[0].placements, st.output_specs.placements) for st in out.strategies} == {
+        ((R, R), (R, R)), ((Shard(1), R), (Shard(0), R)), ((Shard(3), Shard(1)), (Shard(1), Shard(0)))}
+    y = g.placeholder("y")
+    y.meta["val"] = torch.empty(256, 64, 8, 8, device="meta")
+    sy = OpStrategy([_one(mesh, (256, 64, 8, 8), p) for p in [(R, R), (Shard(0), R), (Shard(1), R)]])
+    vm = g.call_function(torch.ops.aten.var_mean.correction, (y, [0, 2, 3]), {"correction": 0, "keepdim": True})
+    vm.meta["val"] = (torch.empty(1, 64, 1, 1, device="meta"), torch.empty(1, 64, 1, 1, device="meta"))
+    out = get_placement_options_for_node(mesh, vm, [sy], [y.meta["val"]], (sy, [0, 2, 3]))
+    assert not fallback_reasons
+    for st in out.strategies:
+        var, mean = st.output_specs
+        assert var.placements == mean.placements and var.tensor_meta.shape == torch.Size([1, 64, 1, 1])
+        # not linear: nothing stays sharded on a reduced dim, the channel shard survives
+        assert all(not p.is_shard() or p.dim == 1 for p in st.input_specs[0].placements)
+    assert ((Shard(1), R), (Shard(1), R)) in {(st.input_specs[0].placements, st.output_specs[0].placements) for st in out.strategies}
