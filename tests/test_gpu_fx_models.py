@@ -71,6 +71,17 @@ class BiasedMLP(nn.Module):
         return self.b(torch.nn.functional.gelu(self.a(x)))
 
 
+class ConvBatchNorm(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.c1, self.bn, self.c2 = nn.Conv2d(3, 32, 3, padding=1), nn.BatchNorm2d(32), nn.Conv2d(32, 64, 3, stride=2, padding=1)
+        self.fc = nn.Linear(64, 10)
+
+    def forward(self, x):
+        x = torch.relu(self.c2(torch.relu(self.bn(self.c1(x)))))
+        return self.fc(x.mean((2, 3)))
+
+
 CASES = {
     # model, input shape, operators the trace must hold, nodes that get the all-Replicate stand-in
     "permute_layer_norm": (PermuteLayerNorm, (256, 96, 56, 56), ("aten.permute.default", "aten.native_layer_norm.default"), set()),
@@ -78,6 +89,9 @@ CASES = {
     # torch 2.10's index_put rule takes no None index (index.Tensor is planned from its run-time rule)
     "index_put": (IndexPut, (256, 32), ("aten.index_put.default", "aten.index.Tensor"), {"index_put"}),
     "biased_mlp": (BiasedMLP, (64, 128, 64), ("aten.mm.default", "aten.add.Tensor"), set()),
+    # convolution (batch-parallel rule), batch norm taken apart into var_mean / squeeze.dims / pointwise
+    "conv_batch_norm": (ConvBatchNorm, (64, 3, 32, 32), ("aten.convolution.default", "aten.convolution_backward.default",
+                                                          "aten.var_mean.correction", "aten.squeeze.dims"), set()),
 }
 
 
