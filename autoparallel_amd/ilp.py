@@ -13,6 +13,8 @@ receive the identical matrix.
 """
 from __future__ import annotations
 
+import collections.abc
+
 import re
 from typing import Dict, List, Optional, Sequence, Tuple
 
@@ -63,6 +65,31 @@ class _Block:
     def row(self, i: int) -> Row:
         a, b = self.indptr[i], self.indptr[i + 1]
         return Row(self.name(i), self.idx[a:b], self.coef[a:b], self.sense, self.rhs[i])
+
+
+class _BlockNames(collections.abc.Sequence):
+    """The names of a block's rows, made when asked for (a block can hold millions)."""
+
+    def __init__(self, block, n: int):
+        self._block, self._n = block, n
+
+    def __len__(self) -> int:
+        return self._n
+
+    def __getitem__(self, i):
+        if isinstance(i, slice):
+            return [self._block.name(k) for k in range(*i.indices(self._n))]
+        if i < 0:
+            i += self._n
+        if not 0 <= i < self._n:
+            raise IndexError(i)
+        return self._block.name(i)
+
+    def __eq__(self, other) -> bool:
+        return list(self) == list(other) if isinstance(other, (list, tuple, _BlockNames)) else NotImplemented
+
+    def __repr__(self) -> str:
+        return repr(list(self))
 
 
 class _Rows:
@@ -179,7 +206,7 @@ class SparseILP:
         b = _Block(prefix, first, None, indptr, idx, coef, sense, rhs)
         self.constraints.blocks.append(b)
         self.constraints.by_prefix.setdefault(prefix, []).append(b)
-        return [b.name(i) for i in range(n)]
+        return _BlockNames(b, n)
 
     def add_row(self, prefix_or_name: str, idx, coef, sense: int, rhs: float, exact_name: bool = False) -> str:
         idx = np.asarray(idx, np.int64)

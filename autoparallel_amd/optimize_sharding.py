@@ -145,10 +145,7 @@ class DecisionVar:
 class DecisionVars(collections.abc.Mapping):
     def __init__(self, opt: "ShardingOptimizer"):
         self._opt = opt
-        g = opt._packed
-        self._keys = g.entry_keys()
-        self._order = g.decision_var_order()
-        self._index: Optional[Dict[tuple, int]] = None
+        self._ordered_keys: Optional[np.ndarray] = None  # made when the mapping is first iterated
 
     def _col(self, key) -> int:
         v, a, o, j = key
@@ -168,11 +165,14 @@ class DecisionVars(collections.abc.Mapping):
         return DecisionVar(self._opt, self._col(key), (int(v), int(a), int(o), int(j)))
 
     def __iter__(self) -> Iterator[tuple]:
-        for i in self._order:
-            yield tuple(int(x) for x in self._keys[i])
+        if self._ordered_keys is None:
+            g = self._opt._packed
+            self._ordered_keys = g.entry_keys()[g.decision_var_order()]
+        for k in self._ordered_keys:
+            yield tuple(int(x) for x in k)
 
     def __len__(self) -> int:
-        return self._keys.shape[0]
+        return int(self._opt._packed.num_entries)
 
 
 class _ClusterLinks(collections.abc.Mapping):

@@ -306,8 +306,33 @@ class PackedGraph:
         """Permutation p such that entries[p] is in the reference's
         ``decision_vars`` insertion order: node, out_idx, argi, inp_idx
         (optimize_sharding.py:511-520)."""
-        k = self.entry_keys().astype(np.int64)
-        return np.lexsort((k[:, 3], k[:, 1], k[:, 2], k[:, 0]))
+        # Without sorting: the order visits, per node and per out_idx, the row of every argument's
+        # block in turn, and a row is S_src consecutive entries.  Runs = (node, out_idx, arg).
+        sizes = self.block_sizes()
+        entry_start = np.concatenate([[0], np.cumsum(sizes)[:-1]]) if self.num_edges else np.zeros(0, np.int64)
+        own = np.nonzero(sizes > 0)[0]  # edges that own a block, in (node, arg) order
+        if own.size == 0:
+            return np.zeros(0, np.int64)
+        node = self.edge_node[own].astype(np.int64)
+        S = self.edge_sdst[own].astype(np.int64)           # rows of the block = strategies of its node
+        ssrc = self.edge_ssrc[own].astype(np.int64)
+        # position of each owning edge among its node's owning edges, and how many the node has
+        first_of_node = np.ones(own.size, bool)
+        first_of_node[1:] = node[1:] != node[:-1]
+        group = np.cumsum(first_of_node) - 1
+        group_start = np.nonzero(first_of_node)[0]
+        n_args = np.diff(np.append(group_start, own.size))
+        rank = np.arange(own.size) - group_start[group]
+        # runs in order: for each node group, for o in range(S), for each of its edges
+        runs_per_group = S[group_start] * n_args
+        run_group = np.repeat(np.arange(group_start.size), runs_per_group)
+        within = np.arange(int(runs_per_group.sum())) - np.repeat(np.cumsum(runs_per_group) - runs_per_group, runs_per_group)
+        o = within // n_args[run_group]
+        edge = group_start[run_group] + within % n_args[run_group]  # index into `own`
+        start = entry_start[own[edge]] + o * ssrc[edge]
+        count = ssrc[edge]
+        total = int(count.sum())
+        return np.repeat(start - (np.cumsum(count) - count), count) + np.arange(total, dtype=np.int64)
 
     def export_rows(self):
         """(row_base int64[n_edge], row_stride int32[n_edge]): the row of entry
