@@ -64,9 +64,16 @@ class _Region:
         self.ancestors |= self._anc[v]
 
 
-def identical_regions(g: PackedGraph, hashes: Sequence[int], check_cycles: bool = True) -> List[List[List[int]]]:
+def identical_regions(g: PackedGraph, hashes: Sequence[int], check_cycles: bool = True,
+                      keep_unclaimed: bool = False) -> List[List[List[int]]]:
     """Region groups, each a list of regions (node lists in graph order) that
-    are identical position by position; groups and regions in graph order."""
+    are identical position by position; groups and regions in graph order.
+
+    keep_unclaimed: the reference drops a whole list of duplicates as soon as an
+    earlier region has taken one of them (graph_clustering.py:169-176), which
+    leaves e.g. the second normalisation of every transformer layer outside any
+    region when the first one was taken.  With this set, the duplicates that are
+    still free are grown into regions of their own when two or more remain."""
     n = g.num_nodes
     args = _unique_args(g)
     users: List[List[int]] = [[] for _ in range(n)]
@@ -96,7 +103,11 @@ def identical_regions(g: PackedGraph, hashes: Sequence[int], check_cycles: bool 
     result = []
     for grp in cand:
         if any(r in seen for r in grp):
-            continue
+            if not keep_unclaimed:
+                continue
+            grp = [r for r in grp if r not in seen]
+            if len(grp) < 2:
+                continue
         ph = int(phase[grp[0]])
         regions = [_Region(r, args, anc) for r in grp]
         cur = regions[0].next()
@@ -119,6 +130,8 @@ def identical_regions(g: PackedGraph, hashes: Sequence[int], check_cycles: bool 
             cur = regions[0].next()
         if len(regions[0].nodes) > 1:
             result.append([sorted(reg.nodes) for reg in regions])
+            if keep_unclaimed:  # the roots of a kept region are taken too
+                seen.update(grp)
     for grp in result:
         grp.sort(key=lambda r: r[0])
     result.sort(key=lambda grp: grp[0][0])

@@ -399,6 +399,9 @@ class ShardingOptimizer:
         self.mesh = mesh
         self.force_grad_reduce_in_higher_precision = force_grad_reduce_in_higher_precision
         self.repeated_subgraphs = bool(repeated_subgraphs)
+        # "extended": also cluster what the reference's pass leaves out (see
+        # clustering.identical_regions); any other true value is the reference's pass
+        self._cluster_mode = "extended" if repeated_subgraphs == "extended" else self.repeated_subgraphs
         self.cluster_links: Dict[tuple, tuple] = {}
         self._devices_per_host = devices_per_host if devices_per_host is not None else _mesh_dph(mesh)
         self._device_name = device_name or detect_device_name()
@@ -610,7 +613,38 @@ class ShardingOptimizer:
                                   for n in packed_nodes], np.uint8)
         g.node_phase = np.asarray([1 if n.meta.get("partitioner_tag") == "is_backward" else 0
                                    for n in packed_nodes], np.int32)
+        if self.repeated_subgraphs:
+            g.node_cluster_key = self._cluster_keys(packed_nodes)
         return g
+
+    @staticmethod
+    def _cluster_keys(nodes) -> np.ndarray:
+        """int32 per node: an id of the parts of the reference's clustering key that
+        the packed arrays do not hold: the operator's name, the forward/backward
+        tag, the source position, and the arguments (tensor arguments by their
+        metadata, integers by value, anything else as absent)
+        (autoparallel/graph_passes/graph_clustering.py:35-52, 68-73).  Nodes with
+        different ids never fall into one group of duplicates."""
+        from torch.utils._pytree import tree_flatten
+
+        def arg_key(a):
+            if isinstance(a, torch.fx.Node):
+                v = a.meta.get("val")
+                if isinstance(v, torch.Tensor):
+                    return (tuple(str(d) for d in v.shape), tuple(str(d) for d in v.stride()), str(v.dtype))
+                return None if v is None else str(v)
+            return a if isinstance(a, int) else None
+
+        ids: Dict[tuple, int] = {}
+        out = np.empty(len(nodes), np.int32)
+        for i, n in enumerate(nodes):
+            flat, _ = tree_flatten(n.args)
+            kw = sorted(n.kwargs.items(), key=lambda kv: kv[0])
+            flat_kw, _ = tree_flatten(kw)
+            key = (str(n.target), n.meta.get("partitioner_tag"), n.meta.get("stack_trace"),
+                   tuple(k for k, _ in kw), tuple(arg_key(a) for a in flat + flat_kw))
+            out[i] = ids.setdefault(key, len(ids))
+        return out
 
     # -- coefficients ----------------------------------------------------------------
     def _build_decision_vars(self) -> DecisionVars:
@@ -622,7 +656,7 @@ class ShardingOptimizer:
             force_grad_reduce_in_higher_precision=self.force_grad_reduce_in_higher_precision,
             device_name=self._device_name, nccl_config=_cre.get_nccl_topo_config(),
             topo_config=_cre.get_mesh_topo_config(),
-            repeated_subgraphs=self.repeated_subgraphs)
+            repeated_subgraphs=self._cluster_mode)
         self._packed = self._core.g  # with the entry blocks of repeated nodes dropped, if any
         # per-variable link table of the reference (:356-378): linked key -> root key
         self.cluster_links = _ClusterLinks(self, self._core.cluster_links)

@@ -193,6 +193,10 @@ class PackedGraph:
     # forward (0) / backward (1) tag regions must not cross
     node_kind: Optional[np.ndarray] = None  # uint8[N]
     node_phase: Optional[np.ndarray] = None  # int32[N]
+    # optional id per node of whatever else must agree before two nodes may be
+    # duplicates of each other (the packer of a traced graph sets it from the
+    # operator's name, source position and arguments); hashed in place of the tag
+    node_cluster_key: Optional[np.ndarray] = None  # int32[N]
     # runs of every output of a tuple-valued node (column k: output k, -1 past the
     # node's outputs); column 0 is node_out_list
     node_out_runs: Optional[np.ndarray] = None  # int64[N, max outputs]

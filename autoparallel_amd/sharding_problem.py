@@ -171,7 +171,9 @@ class PackedShardingOptimizer:
     ):
         """repeated_subgraphs: cluster identical regions (node hashes from the
         device) and let every repeated node share the decision variables of its
-        root (autoparallel/optimize_sharding.py:261-266, 356-378).
+        root (autoparallel/optimize_sharding.py:261-266, 356-378).  The string
+        "extended" also clusters the duplicates that the reference's pass leaves
+        out because an earlier region took one of their siblings.
         cluster_root: the same link table given explicitly (int[N], root[v] = v
         for unlinked nodes), e.g. from a saved file."""
         self.g = g
@@ -191,8 +193,10 @@ class PackedShardingOptimizer:
             from .engine import CostEngine
 
             assert g.edge_alias is None, "the graph already carries a clustering"
-            hashes = CostEngine(g, allocate_results=False, **engine_kw).node_hashes(g.node_phase)
-            self.region_groups = clustering.identical_regions(g, hashes)
+            key = g.node_cluster_key if g.node_cluster_key is not None else g.node_phase
+            hashes = CostEngine(g, allocate_results=False, **engine_kw).node_hashes(key)
+            self.region_groups = clustering.identical_regions(
+                g, hashes, keep_unclaimed=repeated_subgraphs == "extended")
             cluster_root = clustering.cluster_roots(g, self.region_groups)
         g_in = g
         self._set_cluster_root(cluster_root)

@@ -131,3 +131,30 @@ def test_clusters_are_rerooted_at_the_lowest_layer():
     assert by["f0"]["cluster_id"] == by["f1"]["cluster_id"] and by["f1"]["cluster_root"] == "f0" and "cluster_root" not in by["f0"]
     assert by["b0"]["cluster_id"] == by["b1"]["cluster_id"] == by["b3"]["cluster_id"] != by["f0"]["cluster_id"]
     assert by["b1"]["cluster_root"] == by["b3"]["cluster_root"] == "b0" and "cluster_id" not in by["f2"]
+
+
+def test_cluster_keys_follow_the_reference_hash_key():
+    """What the packed arrays do not hold of the reference's clustering key
+    (graph_clustering.py:35-52, 68-73): operator name, tag, source position and arguments
+    (tensors by metadata, integers by value).  Same on all of them: same id."""
+    from torch.fx.experimental.proxy_tensor import make_fx
+
+    from autoparallel_amd.optimize_sharding import ShardingOptimizer
+
+    def f(x):
+        for _ in range(2):
+            x = torch.relu(x)  # one source line, same argument metadata: duplicates
+        s0, s1 = x.sum(0), x.sum(1)
+        return torch.sigmoid(x), s0, s1
+
+    gm = make_fx(f)(torch.randn(4, 4))
+    nodes = [n for n in gm.graph.nodes if n.op != "output"]
+    ids = dict(zip((n.name for n in nodes), ShardingOptimizer._cluster_keys(nodes)))
+    relus = [n.name for n in nodes if "relu" in n.name]
+    sums = [n.name for n in nodes if "sum" in n.name]
+    assert len(relus) == 2 and ids[relus[0]] == ids[relus[1]]
+    assert len(sums) == 2 and ids[sums[0]] != ids[sums[1]]  # the dimension is part of the key
+    assert len({ids[relus[0]], ids[sums[0]], ids[sums[1]], ids[next(n.name for n in nodes if "sigmoid" in n.name)]}) == 4
+    nodes[1].meta["partitioner_tag"] = "is_backward"
+    again = ShardingOptimizer._cluster_keys(nodes)
+    assert again[1] != again[2]  # a different tag separates them

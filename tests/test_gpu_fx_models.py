@@ -381,3 +381,55 @@ def test_regions_of_different_groups_that_meet(meshes):
     idx = torch.from_numpy(clustered._out_indices(plan).astype(np.int16).reshape(-1, 1)).cuda()
     r = full._core.engine.score(idx).cpu().numpy()[0]
     assert r[5] == 0 and np.isclose(r[4], clustered._core.objective_value, rtol=1e-9)
+
+
+def test_extended_clustering_takes_what_the_first_pass_leaves(meshes):
+    """With four decoder layers the reference's pass takes the first normalisation of every layer
+    into the large backward region and then drops the whole list of its duplicates, so the second
+    normalisation of every layer stays on its own.  repeated_subgraphs="extended" grows regions
+    from the duplicates that are still free: more nodes share variables, fewer entries are priced,
+    and the plan, expanded and scored on the engine that priced every node, costs what the
+    clustered objective says and no less than the plan of the unclustered problem."""
+    pytest.importorskip("transformers")
+    from torch._functorch.aot_autograd import aot_export_joint_with_descriptors
+    from torch._subclasses.fake_tensor import FakeTensorMode
+    from torch.distributed.tensor.placement_types import Replicate, Shard
+
+    from autoparallel_amd.graph_utils import add_alias_nodes, replace_view_mm_view_with_einsum
+    from autoparallel_amd.optimize_sharding import ShardingOptimizer
+
+    cfg_cls, model_cls, kwargs, dtype = _hf_cases()["mistral"]
+    cfg = cfg_cls(**{**kwargs, "num_hidden_layers": 4})
+    cfg.use_cache = False
+    cfg._attn_implementation = "sdpa"
+    with FakeTensorMode():
+        with torch.device("cuda"):
+            model = _HFLoss(model_cls(cfg), "mistral")
+        x = torch.randint(0, 512, (8, 64), device="cuda")
+        with contextlib.ExitStack() as stack:
+            gm = aot_export_joint_with_descriptors(stack, model, (x,)).graph_module
+    replace_view_mm_view_with_einsum(gm)
+    add_alias_nodes(gm)
+    mesh = meshes["2d"]
+    kw = dict(devices_per_host=8, device_name="AMD Instinct MI355X")
+    full = ShardingOptimizer(gm, mesh, **kw)
+    first = ShardingOptimizer(gm, mesh, repeated_subgraphs=True, **kw)
+    ext = ShardingOptimizer(gm, mesh, repeated_subgraphs="extended", **kw)
+    assert ext.repeated_subgraphs is True
+    assert len(ext._cluster_linked_node_idxs) > len(first._cluster_linked_node_idxs) > 0
+    assert ext._packed.num_entries < first._packed.num_entries < full._packed.num_entries
+    # the regions of the first pass are all still there
+    taken = {tuple(reg) for grp in ext._core.region_groups for reg in grp}
+    assert all(tuple(reg) in taken for grp in first._core.region_groups for reg in grp)
+    for opt in (full, first, ext):
+        opt.add_sharded_input_constraint([(Shard(0), Replicate())])
+        opt.add_parameter_memory_constraint(0.0, 1.0 / mesh.size())
+    plan = ext.get_solution()
+    first.get_solution()
+    full.get_solution()
+    assert "Violated constraints: []" in ext.get_log()
+    assert ext._core.objective_value >= first._core.objective_value * (1 - 1e-9)
+    assert first._core.objective_value >= full._core.objective_value * (1 - 1e-9)
+    idx = torch.from_numpy(ext._out_indices(plan).astype(np.int16).reshape(-1, 1)).cuda()
+    r = full._core.engine.score(idx).cpu().numpy()[0]
+    assert r[5] == 0 and np.isclose(r[4], ext._core.objective_value, rtol=1e-9)
