@@ -83,7 +83,20 @@ def save_optimizer(core, path: str, mesh_dim_names: Optional[List[str]] = None) 
     selected = np.zeros((0, 4), np.int32)
     if core.selected is not None:
         selected = g.entry_keys()[core.selected].astype(np.int32)
+    # local/global size of every parameter's strategies: what the memory budget
+    # rows weigh with.  They come from the device, so the file carries them and a
+    # problem read back can be solved under a memory budget where there is no GPU.
+    params = [int(p) for p, _ in core.roles.param_grad]
+    if core.engine is not None and params:
+        core._memory_ratios(params)
+    kept = [p for p in params if p in core._memory_ratio_cache]
+    ratio_vals = [core._memory_ratio_cache[p] for p in kept]
     arrays = graph_to_arrays(g)
+    arrays.update(
+        memory_ratio_node=np.asarray(kept, np.int32),
+        memory_ratio_off=np.cumsum([0] + [len(r) for r in ratio_vals]).astype(np.int64),
+        memory_ratio_val=np.concatenate(ratio_vals) if ratio_vals else np.zeros(0),
+    )
     arrays.update(
         version=np.asarray(FORMAT_VERSION),
         mesh_shape=np.asarray(g.mesh_shape, np.int64),
@@ -124,12 +137,17 @@ def load_optimizer(path: str, cls=None):
         force = bool(d["force_grad_reduce_in_higher_precision"])
         dim_names = json.loads(bytes(d["mesh_dim_names"]).decode())
         cluster_root = d["cluster_root"] if "cluster_root" in d else None
+        ratios = {}
+        if "memory_ratio_node" in d:
+            off, val = d["memory_ratio_off"], d["memory_ratio_val"]
+            ratios = {int(p): val[off[i]:off[i + 1]].copy() for i, p in enumerate(d["memory_ratio_node"])}
     if keys.shape != (g.num_entries, 4) or vals.shape != (g.num_entries, 3):
         raise RuntimeError("coefficient arrays do not match the packed graph")
     coef = Coefficients.from_decision_var_arrays(g, keys, vals, compute, per_arg)
     core = cls(g, roles=g.roles, force_grad_reduce_in_higher_precision=force, coefficients=coef,
                cluster_root=cluster_root)
     core.mesh_dim_names = dim_names
+    core._memory_ratio_cache = ratios
     for method, kwargs in log:
         getattr(core, method)(**kwargs)
     core._constraint_log = [(m, k) for m, k in log]

@@ -181,6 +181,7 @@ class PackedShardingOptimizer:
         self.force_grad_reduce_in_higher_precision = force_grad_reduce_in_higher_precision
         self.engine = None
         self.phase_s: Dict[str, float] = {}  # seconds per phase of the construction
+        self._memory_ratio_cache: Dict[int, np.ndarray] = {}  # parameter node -> local/global size per strategy
         self.region_groups: List[List[List[int]]] = []
         engine_kw = dict(device=device, device_name=device_name, nccl_config=nccl_config, topo_config=topo_config)
         # Repeated subgraphs are found before anything is priced: the hashes need the
@@ -496,6 +497,10 @@ class PackedShardingOptimizer:
         from .engine import make_model
 
         g = self.g
+        cache = self._memory_ratio_cache
+        wanted, params = params, [p for p in params if p not in cache]
+        if not params:  # computed before, or carried by the file this problem was read from
+            return [cache[p] for p in wanted]
         lib = _lib.load()
         rows = []
         for p in params:
@@ -516,7 +521,7 @@ class PackedShardingOptimizer:
                                         out_stride.data_ptr(), None), "apc_local_shapes")
         torch.cuda.synchronize(dev)
         local = out_shape.cpu().numpy()
-        ratios, k = [], 0
+        k = 0
         for p in params:
             S = int(g.node_nstrat[p])
             r = []
@@ -525,9 +530,9 @@ class PackedShardingOptimizer:
                 new = math.prod(int(x) for x in local[k + i, :rk])
                 old = math.prod(int(x) for x in g.meta_shape[mids[k + i], :rk])
                 r.append(new / old)
-            ratios.append(np.asarray(r))
+            cache[p] = np.asarray(r)
             k += S
-        return ratios
+        return [cache[p] for p in wanted]
 
     def _apply_memory_constraint(self) -> None:
         if self._memory_constraint is None:

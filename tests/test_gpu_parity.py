@@ -824,3 +824,24 @@ def test_memory_constraint(CostEngine):
     for p, r in zip(params, ratios):
         assert r[sol[p]] == r.min()
     assert "memory_constraint_high" in opt.prob.constraints
+
+
+def test_saved_problem_carries_the_memory_ratios(CostEngine, tmp_path, monkeypatch):
+    """The ratios that weigh the memory budget rows come from the device; the saved file holds
+    them, so the problem read back is solved under its budget without another device call."""
+    from autoparallel_amd import _lib
+    from autoparallel_amd.sharding_problem import PackedShardingOptimizer
+
+    g = graphgen.gpt2_graph((4,), n_layers=1, dim=64, n_heads=2, ffn_dim=128, vocab=256, seq=32, batch=8)
+    opt = PackedShardingOptimizer(g)
+    opt.add_parameter_memory_constraint(0.0, 0.0)
+    sol = opt.get_solution()
+    path = str(tmp_path / "budget.npz")
+    opt.save(path)
+    params = [p for p, _ in g.roles.param_grad]
+    want = opt._memory_ratios(params)
+    monkeypatch.setattr(_lib, "load", lambda: (_ for _ in ()).throw(AssertionError("no device call expected")))
+    back = PackedShardingOptimizer.load(path)
+    assert all(np.array_equal(a, b) for a, b in zip(back._memory_ratios(params), want))
+    assert np.array_equal(back.resolve(), sol) and "memory_constraint_high" in back.prob.constraints
+    assert np.isclose(back.objective_value, opt.objective_value, rtol=1e-12)

@@ -113,6 +113,39 @@ def test_save_load_roundtrip(tiny, tmp_path):
             loaded.decision_vars[bad]
 
 
+def test_memory_ratios_travel_with_the_file(tiny, tmp_path):
+    """A problem under a parameter-memory budget is saved with the local/global size of every
+    parameter strategy and solved again from the file alone.  Here the ratios are the oracle's
+    (sharded_shape_stride); tests/test_gpu_parity.py checks the device's against the same."""
+    g, coef, _ = tiny
+    opt = PackedShardingOptimizer(g, coefficients=coef)
+    params = [p for p, _ in g.roles.param_grad]
+    mesh = [int(x) for x in g.mesh_shape]
+    for p in params:
+        run, r = int(g.node_out_list[p]), []
+        for o in range(int(g.node_nstrat[p])):
+            w = int(g.lists[run + o])
+            rk = int(g.meta_rank[w >> 12])
+            shape = [int(x) for x in g.meta_shape[w >> 12, :rk]]
+            local, _ = O.sharded_shape_stride(shape, [1] * rk, [int(x) for x in g.tuple_plc[w & 0xFFF, : g.ndim]], mesh)
+            r.append(np.prod(local) / np.prod(shape))
+        opt._memory_ratio_cache[p] = np.asarray(r)
+    opt.add_parameter_memory_constraint(0.0, 0.0)  # every parameter at its smallest ratio
+    sol = opt.get_solution()
+    assert all(opt._memory_ratio_cache[p][sol[p]] == opt._memory_ratio_cache[p].min() for p in params)
+    path = str(tmp_path / "budget.npz")
+    opt.save(path)
+    back = PackedShardingOptimizer.load(path)
+    assert set(back._memory_ratio_cache) == set(params)
+    assert all(np.array_equal(back._memory_ratio_cache[p], opt._memory_ratio_cache[p]) for p in params)
+    assert np.array_equal(back.resolve(), sol) and "memory_constraint_high" in back.prob.constraints
+    # without the ratios the budget rows need the device: no silent stand-in
+    back._memory_ratio_cache = {}
+    if not torch.cuda.is_available():
+        with pytest.raises(Exception):
+            back.resolve()
+
+
 def test_load_takes_the_reference_argument_order_too(tiny, tmp_path):
     from autoparallel_amd import serialization
 
