@@ -439,7 +439,7 @@ def _fx_path_figure(n_layers: int, cpu_port: bool) -> dict:
         mesh = init_device_mesh("cpu", (8, 8))
         PO.fallback_nodes.clear()
         PO.reset_placement_options_cache()
-        def leg(repeated_subgraphs: bool) -> dict:
+        def leg(repeated_subgraphs) -> dict:
             PO.fallback_nodes.clear()
             PO.reset_placement_options_cache()
             t0 = time.perf_counter()
@@ -491,6 +491,8 @@ def _fx_path_figure(n_layers: int, cpu_port: bool) -> dict:
             "einsum_rewrite_s": t_rewrite,
             "all_nodes": leg(False),
             "cluster_roots_only": leg(True),
+            # the duplicates that the reference's pass drops clustered too (no counterpart in the reference)
+            "cluster_roots_only_extended_pass": leg("extended"),
         }
     finally:
         if own:
