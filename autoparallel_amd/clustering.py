@@ -73,7 +73,8 @@ def identical_regions(g: PackedGraph, hashes: Sequence[int], check_cycles: bool 
     earlier region has taken one of them (graph_clustering.py:169-176), which
     leaves e.g. the second normalisation of every transformer layer outside any
     region when the first one was taken.  With this set, the duplicates that are
-    still free are grown into regions of their own when two or more remain."""
+    still free are grown into regions of their own when two or more remain, and
+    duplicates that end up in no region at all form regions of one node each."""
     n = g.num_nodes
     args = _unique_args(g)
     users: List[List[int]] = [[] for _ in range(n)]
@@ -132,6 +133,14 @@ def identical_regions(g: PackedGraph, hashes: Sequence[int], check_cycles: bool 
             result.append([sorted(reg.nodes) for reg in regions])
             if keep_unclaimed:  # the roots of a kept region are taken too
                 seen.update(grp)
+    if keep_unclaimed:
+        # what no region took: duplicates of each other still share variables, as
+        # regions of one node (the reference keeps no such region, :188-190)
+        for grp in cand:
+            free = [r for r in grp if r not in seen]
+            if len(free) > 1:
+                result.append([[r] for r in free])
+                seen.update(free)
     for grp in result:
         grp.sort(key=lambda r: r[0])
     result.sort(key=lambda grp: grp[0][0])

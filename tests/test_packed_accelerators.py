@@ -201,25 +201,26 @@ def test_regions_from_the_duplicates_an_earlier_region_left():
     """Three layers of a = A(prev), b = N(a), c = C(b), e = E(input), d = N(c, e): the region grown
     from the C nodes takes a, b and c of every layer.  b and d are duplicates of each other, so the
     reference's pass then drops their whole list (graph_clustering.py:169-176) and d stays alone;
-    with keep_unclaimed the d nodes still grow a region of their own, through e."""
+    with keep_unclaimed the d nodes still grow a region of their own, through e, and the f nodes
+    (f = F(input), used by nothing), which no region can reach, become regions of one node."""
     from types import SimpleNamespace
 
     from autoparallel_amd import clustering
 
-    A, N, C, E = 11, 12, 13, 14
+    A, N, C, E, F = 11, 12, 13, 14, 15
     args, hashes = [[]], [0]  # node 0: the input
     prev = 0
     for _ in range(3):
         base = len(args)
-        args += [[prev], [base], [base + 1], [0], [base + 2, base + 3]]
-        hashes += [A, N, C, E, N]
+        args += [[prev], [base], [base + 1], [0], [base + 2, base + 3], [0]]
+        hashes += [A, N, C, E, N, F]
         prev = base + 4
     off = np.cumsum([0] + [len(a) for a in args])
     n = len(args)
     g = SimpleNamespace(num_nodes=n, node_edge_off=off, edge_src_node=np.asarray([u for a in args for u in a]),
                         node_kind=np.asarray([1] + [0] * (n - 1)), node_op=np.zeros(n, np.int32), node_phase=None)
-    layers = [[1 + 5 * i + k for k in range(5)] for i in range(3)]
+    layers = [[1 + 6 * i + k for k in range(6)] for i in range(3)]
     abc = [[lay[0], lay[1], lay[2]] for lay in layers]
     assert clustering.identical_regions(g, hashes) == [abc]
     ext = clustering.identical_regions(g, hashes, keep_unclaimed=True)
-    assert ext == [abc, [[lay[3], lay[4]] for lay in layers]]
+    assert ext == [abc, [[lay[3], lay[4]] for lay in layers], [[lay[5]] for lay in layers]]
