@@ -672,12 +672,20 @@ class ShardingOptimizer:
         loop does in place (:540)."""
         g, comm = self._packed, self._core.coef.comm
         vs, alias = self._core.var_start, self._core.edge_alias
+        nodes, strats = self.nodes, self.strats
+        edge_node, edge_arg, edge_ssrc = g.edge_node.tolist(), g.edge_arg.tolist(), g.edge_ssrc.tolist()
+        vs, alias = np.asarray(vs).tolist(), np.asarray(alias).tolist()
+        made: Dict[int, list] = {}  # rows of the edges that own a block, as lists
         for e in range(g.num_edges):
-            node = self.nodes[int(g.edge_node[e])]
-            a, ssrc = int(g.edge_arg[e]), int(g.edge_ssrc[e])
-            r = int(alias[e])  # a repeated node's rows are its root's (:554-571)
-            block = comm[vs[r] : vs[r + 1]].reshape(-1, ssrc).tolist()
-            for s, row in zip(self.strats[node].strategies, block):
+            r = alias[e]  # a repeated node's rows are its root's (:554-571)
+            block = made.get(r)
+            if block is None:
+                block = made[r] = comm[vs[r] : vs[r + 1]].reshape(-1, edge_ssrc[e]).tolist()
+                rows = block
+            else:  # lists of its own over the same numbers (:569-571)
+                rows = [row[:] for row in block]
+            a = edge_arg[e]
+            for s, row in zip(strats[nodes[edge_node[e]]].strategies, rows):
                 s.redistribute_cost[a] = row
 
     def validate(self) -> None:
