@@ -144,3 +144,30 @@ def test_clustered_optimizer_end_to_end(engine_mod):
     assert back.cluster_links == opt.cluster_links and back.n_vars == opt.n_vars
     assert np.array_equal(back._extract(), sol)
     assert set(back.prob.constraints) == set(opt.prob.constraints)
+
+
+@pytest.mark.parametrize("name", ["llama_3layer_2x4", "gpt2_2layer_4"])
+def test_extended_pass_on_the_packed_graphs(engine_mod, name):
+    """repeated_subgraphs="extended" keeps every region of the first pass, links at least as many
+    nodes, and its objective is the device's objective of the expanded plan, scored both on its
+    own engine (linked rows read from the root) and on the engine that priced every node."""
+    from autoparallel_amd.sharding_problem import PackedShardingOptimizer
+
+    plain = PackedShardingOptimizer(GRAPHS[name]())
+    plain.get_solution()
+    first = PackedShardingOptimizer(GRAPHS[name](), repeated_subgraphs=True)
+    ext = PackedShardingOptimizer(GRAPHS[name](), repeated_subgraphs="extended")
+    taken = {tuple(reg) for grp in ext.region_groups for reg in grp}
+    assert all(tuple(reg) in taken for grp in first.region_groups for reg in grp)
+    assert ext.linked.sum() >= first.linked.sum() > 0 and ext.n_vars <= first.n_vars
+    # regions of one node only ever hold nodes that no larger region took
+    seen = [v for grp in ext.region_groups for reg in grp for v in reg]
+    assert len(seen) == len(set(seen))
+    sol = ext.get_solution()
+    first.get_solution()
+    assert (sol[ext.linked] == sol[ext.root[ext.linked]]).all()
+    a = torch.from_numpy(sol.astype(np.int16).reshape(-1, 1)).cuda()
+    for eng in (ext.engine, plain.engine):
+        r = eng.score(a).cpu().numpy()[0]
+        assert r[5] == 0 and np.isclose(r[4], ext.objective_value, rtol=1e-9)
+    assert ext.objective_value >= first.objective_value * (1 - 1e-9) >= plain.objective_value * (1 - 1e-9) ** 2
