@@ -625,24 +625,28 @@ class ShardingOptimizer:
         metadata, integers by value, anything else as absent)
         (autoparallel/graph_passes/graph_clustering.py:35-52, 68-73).  Nodes with
         different ids never fall into one group of duplicates."""
-        from torch.utils._pytree import tree_flatten
+        of_node: Dict[torch.fx.Node, object] = {}  # a producer is described once
 
         def arg_key(a):
             if isinstance(a, torch.fx.Node):
-                v = a.meta.get("val")
-                if isinstance(v, torch.Tensor):
-                    return (tuple(str(d) for d in v.shape), tuple(str(d) for d in v.stride()), str(v.dtype))
-                return None if v is None else str(v)
+                k = of_node.get(a, of_node)
+                if k is of_node:
+                    v = a.meta.get("val")
+                    if isinstance(v, torch.Tensor):
+                        k = (tuple(str(d) for d in v.shape), tuple(str(d) for d in v.stride()), str(v.dtype))
+                    else:
+                        k = None if v is None else str(v)
+                    of_node[a] = k
+                return k
             return a if isinstance(a, int) else None
 
         ids: Dict[tuple, int] = {}
         out = np.empty(len(nodes), np.int32)
         for i, n in enumerate(nodes):
-            flat, _ = tree_flatten(n.args)
             kw = sorted(n.kwargs.items(), key=lambda kv: kv[0])
-            flat_kw, _ = tree_flatten(kw)
+            flat = _flat_args(kw, _flat_args(n.args, []))
             key = (str(n.target), n.meta.get("partitioner_tag"), n.meta.get("stack_trace"),
-                   tuple(k for k, _ in kw), tuple(arg_key(a) for a in flat + flat_kw))
+                   tuple(k for k, _ in kw), tuple(arg_key(a) for a in flat))
             out[i] = ids.setdefault(key, len(ids))
         return out
 
