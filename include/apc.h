@@ -530,7 +530,10 @@ int apc_objective_coeffs(const apc_problem* p, const double* cost, double* obj, 
 /* Replaces _hash_node (autoparallel/graph_passes/graph_clustering.py:68-82),
  * the key under which get_identical_regions groups repeated nodes: a 64-bit
  * structural hash per node over its op class, program, forward/backward tag
- * (node_phase int32[n_node], may be NULL), strategy counts, output spec run
+ * (node_phase int32[n_node], may be NULL; a caller that knows more of the
+ * reference's key than the problem holds, such as the operator's name, source
+ * position and non-tensor arguments of a traced node, passes one id per
+ * distinct combination of those and the tag here), strategy counts, output spec run
  * (node_out_list int64[n_node]: offset of the node's output run in lists),
  * input and producer spec runs and default rows.  Equal keys in the reference
  * imply equal hashes here; out: uint64[n_node]. */
