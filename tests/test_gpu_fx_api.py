@@ -766,7 +766,8 @@ def test_collectives_stay_on_the_narrow_side_of_a_cast(mesh):
                 assert sol[n].input_specs[0].placements == sol[n.all_input_nodes[0]].output_specs.placements
 
 
-def test_reduction_after_the_cast_holds_for_repeated_layers_too(mesh):
+@pytest.mark.parametrize("clusters", [True, "extended"])
+def test_reduction_after_the_cast_holds_for_repeated_layers_too(mesh, clusters):
     """With gradients reduced in the higher precision and repeated layers sharing their
     variables, no selected variable on the way from a weight-gradient matmul to its cast
     moves data, the expanded variables of linked layers included (the reference's
@@ -797,7 +798,7 @@ def test_reduction_after_the_cast_holds_for_repeated_layers_too(mesh):
     old = ShardingOptimizer.dtype_cast_targets
     ShardingOptimizer.dtype_cast_targets = {cast}
     try:
-        opt = ShardingOptimizer(gm, mesh, True, repeated_subgraphs=True, devices_per_host=8,
+        opt = ShardingOptimizer(gm, mesh, True, repeated_subgraphs=clusters, devices_per_host=8,
                                 device_name="AMD Instinct MI355X")
     finally:
         ShardingOptimizer.dtype_cast_targets = old
