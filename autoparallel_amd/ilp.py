@@ -287,8 +287,15 @@ class SparseILP:
         opts = {"disp": bool(verbose), "mip_rel_gap": float(self.mip_rel_gap)}
         if time_limit is not None:
             opts["time_limit"] = float(time_limit)
-        res = milp(self.objective, constraints=cons, integrality=np.ones(self.n_vars),
-                   bounds=Bounds(np.zeros(self.n_vars), ub), options=opts)
+        try:
+            res = milp(self.objective, constraints=cons, integrality=np.ones(self.n_vars),
+                       bounds=Bounds(np.zeros(self.n_vars), ub), options=opts)
+        except (ValueError, MemoryError) as exc:
+            # what the solver's own code raises when it runs out of room part-way (seen at
+            # 1.6 M variables and 40 M nonzeros): not an answer about the problem
+            raise RuntimeError(
+                f"the ILP solver failed inside on {self.n_vars} variables x {A.shape[0]} rows ({exc}); "
+                "write_lp() writes the problem for another solver") from exc
         if res.x is None:
             if res.status not in (2, 3):  # scipy's milp: 2 infeasible, 3 unbounded; anything else is not an answer
                 raise RuntimeError(f"the ILP solver did not solve the problem: {res.message}")

@@ -188,6 +188,21 @@ def test_a_row_that_names_a_variable_twice_is_merged_not_refused():
     assert q.solve() == ilp.STATUS_INFEASIBLE and q.x is None
 
 
+def test_a_failure_inside_the_solver_is_reported_as_that(monkeypatch):
+    """The solver's own code can give up part-way on a very large problem (an exception out of its
+    C++ side, not a status): the caller gets one error that says so and names the way out."""
+    import scipy.optimize
+
+    def broken(*a, **k):
+        raise ValueError("vector::_M_default_append")
+
+    monkeypatch.setattr(scipy.optimize, "milp", broken)
+    p = ilp.SparseILP(2)
+    p.add_row("one", [0, 1], [1.0, 1.0], ilp.EQ, 1.0)
+    with pytest.raises(RuntimeError, match="failed inside on 2 variables x 1 rows.*write_lp"):
+        p.solve(backend="highs")
+
+
 def test_clustered_ilp_matches_reference_semantics():
     from autoparallel_amd import clustering
     from oracle import cluster_oracle as CO
