@@ -182,6 +182,11 @@ class PackedShardingOptimizer:
         self.engine = None
         self.phase_s: Dict[str, float] = {}  # seconds per phase of the construction
         self._memory_ratio_cache: Dict[int, np.ndarray] = {}  # parameter node -> local/global size per strategy
+        # The reference writes the flow rows of every edge from an unlinked producer to a linked
+        # consumer, although they are the rows of the edge to that consumer's root over again
+        # (one copy per repeated layer for a tensor every layer reads).  The extended mode, which
+        # has no row numbering of the reference to keep, writes each distinct row once.
+        self._distinct_flow_rows_only = repeated_subgraphs == "extended"
         self.region_groups: List[List[List[int]]] = []
         engine_kw = dict(device=device, device_name=device_name, nccl_config=nccl_config, topo_config=topo_config)
         # Repeated subgraphs are found before anything is priced: the hashes need the
@@ -377,6 +382,11 @@ class PackedShardingOptimizer:
         _, firsts = np.unique(u[has] * g.num_nodes + v[has], return_index=True)  # first matching argument only
         edges = has[np.sort(firsts)]
         edges = edges[np.argsort(u[edges], kind="stable")]
+        if self._distinct_flow_rows_only:
+            # the rows of an edge are a function of the two blocks they name
+            pair = self.edge_alias[g.node_edge_off[u[edges]].astype(np.int64)] * g.num_edges + self.edge_alias[edges]
+            _, firsts = np.unique(pair, return_index=True)
+            edges = edges[np.sort(firsts)]
         assert (g.edge_ssrc[edges] == g.node_nstrat[u[edges]]).all()
         S = g.node_nstrat[u[edges]].astype(np.int64)
         e = np.repeat(edges, S)
