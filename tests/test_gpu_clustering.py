@@ -171,3 +171,12 @@ def test_extended_pass_on_the_packed_graphs(engine_mod, name):
         r = eng.score(a).cpu().numpy()[0]
         assert r[5] == 0 and np.isclose(r[4], ext.objective_value, rtol=1e-9)
     assert ext.objective_value >= first.objective_value * (1 - 1e-9) >= plain.objective_value * (1 - 1e-9) ** 2
+    # each distinct flow row once; the first pass, like the reference, repeats the rows of a
+    # producer outside the regions for every repeated consumer
+
+    def flow_rows(opt):
+        return [(r.idx.tobytes(), r.coef.tobytes()) for n, r in opt.prob.constraints.items()
+                if n.startswith("output_input_consistent")]
+
+    mine, theirs = flow_rows(ext), flow_rows(first)
+    assert len(set(mine)) == len(mine) > 0 and len(set(theirs)) < len(theirs)
