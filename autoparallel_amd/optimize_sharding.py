@@ -19,7 +19,7 @@ import gc
 import logging
 import time
 import operator
-from typing import Any, Dict, Iterator, List, Optional, Tuple
+from typing import Any, Dict, Iterator, List, Optional, Tuple, Union
 
 import numpy as np
 import torch
@@ -377,7 +377,7 @@ def _gc_paused():
 
 class ShardingOptimizer:
     def __init__(self, gm, mesh, force_grad_reduce_in_higher_precision: bool = False,
-                 repeated_subgraphs: bool = False, devices_per_host: Optional[int] = None,
+                 repeated_subgraphs: Union[bool, str] = False, devices_per_host: Optional[int] = None,
                  device_name: Optional[str] = None):
         with _gc_paused():
             self._construct(gm, mesh, force_grad_reduce_in_higher_precision, repeated_subgraphs,

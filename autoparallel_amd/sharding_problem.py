@@ -24,7 +24,7 @@ import logging
 import math
 import time
 import types
-from typing import Dict, Iterable, List, Optional, Sequence, Set, Tuple
+from typing import Dict, Iterable, List, Optional, Sequence, Set, Tuple, Union
 
 import numpy as np
 
@@ -165,7 +165,7 @@ class PackedShardingOptimizer:
         device: str = "cuda",
         device_name: Optional[str] = None,
         nccl_config=None,
-        repeated_subgraphs: bool = False,
+        repeated_subgraphs: Union[bool, str] = False,  # True: the reference's pass; "extended": see below
         cluster_root: Optional[np.ndarray] = None,
         topo_config=None,
     ):
