@@ -72,6 +72,9 @@ def main():
     ap.add_argument("--fx-layers", type=int, default=32,
                     help="also plan the traced transformers Llama-3-8B with this many layers through "
                          "ShardingOptimizer and report its host time (0 = skip)")
+    ap.add_argument("--fx-solve", action="store_true",
+                    help="also solve the two clustered problems of the FX figure (input pinned to "
+                         "(Shard(0), Replicate()), parameter-memory budget 1/64): minutes of one host core")
     ap.add_argument("--launch", choices=["graph", "eager"], default="eager",
                     help="how a step is issued: replay of a HIP graph of its launches, or the launches themselves")
     ap.add_argument("--direct", action="store_true", help="evaluate every entry directly (no block table)")
@@ -372,13 +375,13 @@ def main():
         # the traced joint graph to coefficients and ILP rows (strategy sets of the
         # installed torch, so fewer entries than the generator's graph above)
         try:
-            out["fx_path"] = _fx_path_figure(args.fx_layers, not args.no_cpu_baseline)
+            out["fx_path"] = _fx_path_figure(args.fx_layers, not args.no_cpu_baseline, args.fx_solve)
         except Exception as exc:  # transformers or the fake process group unavailable
             out["fx_path"] = {"error": f"{type(exc).__name__}: {exc}"[:300]}
     print(json.dumps(out))
 
 
-def _fx_path_figure(n_layers: int, cpu_port: bool) -> dict:
+def _fx_path_figure(n_layers: int, cpu_port: bool, solve: bool = False) -> dict:
     import contextlib
 
     import torch
@@ -427,11 +430,15 @@ def _fx_path_figure(n_layers: int, cpu_port: bool) -> dict:
     t_trace = time.perf_counter() - t0
     # as the reference prepares its joint graph before planning (autoparallel/api.py:208):
     # linear layers become einsums, so that batch and sequence can be sharded separately
-    from autoparallel_amd.graph_utils import replace_view_mm_view_with_einsum
+    from autoparallel_amd.graph_utils import add_alias_nodes, replace_view_mm_view_with_einsum
 
     t0 = time.perf_counter()
     n_einsum = replace_view_mm_view_with_einsum(gm)
     t_rewrite = time.perf_counter() - t0
+    # and every tensor gets an alias node, where a redistribution can sit (:209-211)
+    t0 = time.perf_counter()
+    add_alias_nodes(gm)
+    t_alias = time.perf_counter() - t0
     own = not dist.is_initialized()
     if own:
         dist.init_process_group("fake", store=FakeStore(), rank=0, world_size=64)
@@ -481,6 +488,8 @@ def _fx_path_figure(n_layers: int, cpu_port: bool) -> dict:
                     "pack_plus_device_phases_s": coeff_s, "device_phases_s": device_s,
                     "speedup_of_device_phases": t_cpu / device_s if device_s > 0 else None,
                 }
+            if solve and repeated_subgraphs:
+                res["solve"] = _timed_solve(opt, mesh)
             return res
 
         return {
@@ -489,6 +498,7 @@ def _fx_path_figure(n_layers: int, cpu_port: bool) -> dict:
             "trace_s": t_trace,
             "linear_layers_as_einsums": n_einsum,
             "einsum_rewrite_s": t_rewrite,
+            "alias_nodes_s": t_alias,
             "all_nodes": leg(False),
             "cluster_roots_only": leg(True),
             # the duplicates that the reference's pass drops clustered too (no counterpart in the reference)
@@ -497,6 +507,36 @@ def _fx_path_figure(n_layers: int, cpu_port: bool) -> dict:
     finally:
         if own:
             dist.destroy_process_group()
+
+
+def _timed_solve(opt, mesh) -> dict:
+    """The problem a caller of the reference's example poses (examples/example_llama3.py:226-236):
+    batch-sharded input, parameters within 1/mesh size of their bytes; solved by the library's
+    solver hand-off.  A line goes to stderr every minute: the solver itself prints nothing."""
+    import threading
+
+    from torch.distributed.tensor.placement_types import Replicate, Shard
+
+    opt.add_sharded_input_constraint([(Shard(0),) + (Replicate(),) * (mesh.ndim - 1)])
+    opt.add_parameter_memory_constraint(0.0, 1.0 / mesh.size())
+    done = threading.Event()
+    t0 = time.perf_counter()
+
+    def beat():
+        while not done.wait(60):
+            print(f"[bench] solving, {time.perf_counter() - t0:.0f} s", file=sys.stderr, flush=True)
+
+    threading.Thread(target=beat, daemon=True).start()
+    try:
+        plan = opt.get_solution()
+    finally:
+        done.set()
+    dt = time.perf_counter() - t0
+    params = [n for n in opt.nodes if n.op == "placeholder" and n in plan]
+    fully = sum(all(pl.is_shard() for pl in plan[n].output_specs.placements) for n in params)
+    return {"seconds": dt, "objective": opt._core.objective_value, "variables": opt._packed.num_entries,
+            "rows": len(opt.prob.constraints), "solver": "HiGHS through scipy.optimize.milp, one thread, gap 0",
+            "placeholders_sharded_on_every_mesh_dim": f"{fully} of {len(params)}"}
 
 
 if __name__ == "__main__":
