@@ -284,8 +284,9 @@ def test_transformers_architectures_are_planned(meshes, kind):
     assert set(sol) == {n for n in opt.nodes if n.op != "output"} and not opt._core.prob.violated()
 
 
-@pytest.mark.parametrize("kind", ["bert", "mistral", "mixtral"])
-def test_the_whole_planning_sequence_on_architectures(meshes, kind, tmp_path):
+@pytest.mark.parametrize("kind,clusters", [("bert", True), ("mistral", True), ("mixtral", True),
+                                           ("mistral", "extended"), ("bert", "extended")])
+def test_the_whole_planning_sequence_on_architectures(meshes, kind, clusters, tmp_path):
     """What a caller of the reference does around the planner, in its order: linear layers as
     einsums, alias nodes, repeated layers sharing variables, the batch-sharded input pinned, the
     default parameter budget, solve, the log and the export, save and reopen."""
@@ -314,7 +315,8 @@ def test_the_whole_planning_sequence_on_architectures(meshes, kind, tmp_path):
     mesh = meshes["2d"]
     assert replace_view_mm_view_with_einsum(gm) > 10
     add_alias_nodes(gm)
-    opt = ShardingOptimizer(gm, mesh, repeated_subgraphs=True, devices_per_host=8, device_name="AMD Instinct MI355X")
+    opt = ShardingOptimizer(gm, mesh, repeated_subgraphs=clusters, devices_per_host=8,
+                            device_name="AMD Instinct MI355X")
     assert opt._cluster_linked_node_idxs
     opt.add_sharded_input_constraint([(Shard(0), Replicate())])
     opt.add_parameter_memory_constraint(0.0, 1.0 / mesh.size())
