@@ -224,3 +224,88 @@ def test_regions_from_the_duplicates_an_earlier_region_left():
     assert clustering.identical_regions(g, hashes) == [abc]
     ext = clustering.identical_regions(g, hashes, keep_unclaimed=True)
     assert ext == [abc, [[lay[3], lay[4]] for lay in layers], [[lay[5]] for lay in layers]]
+
+
+def test_region_growth_equals_torchs_own():
+    """The reference grows its regions with torch's fully_expand_region_group and
+    _populate_recursive_ancestor_map (graph_clustering.py:17-27, 103, 178-183) around a few lines
+    of its own (:141-206: lists of duplicates, latest first, skip a list whose root is taken, keep
+    regions of more than one node, sort).  Here those few lines are restated around torch's two
+    functions on FX graphs made of repeated random layers plus stray nodes, and
+    clustering.identical_regions must return the same regions on the same graph and classes."""
+    nonempty = sum(_regions_mine_and_torchs(seed) for seed in range(40))
+    assert nonempty >= 20  # most of the graphs have regions to find
+
+
+def _regions_mine_and_torchs(seed) -> bool:
+    import operator
+    from types import SimpleNamespace
+
+    import torch.fx
+    from torch._dynamo.graph_region_tracker import _populate_recursive_ancestor_map, fully_expand_region_group
+
+    from autoparallel_amd import clustering
+
+    rng = np.random.default_rng(seed)
+    n_layers, width = int(rng.integers(2, 5)), int(rng.integers(5, 12))
+    # one random layer: node k reads one or two of (the layer's input, earlier nodes of the layer)
+    layer = []
+    for k in range(width):
+        srcs = sorted(set(int(x) for x in rng.integers(-1, k, size=int(rng.integers(1, 3)))))
+        layer.append((int(rng.integers(0, 4)), srcs))  # (class within the layer, sources; -1: the input)
+    graph = torch.fx.Graph()
+    x = graph.placeholder("x")
+    nodes, klass, args = [x], [None], [[]]
+    prev = 0
+    for _ in range(n_layers):
+        base = len(nodes)
+        for c, srcs in layer:
+            a = [prev if s < 0 else base + s for s in srcs]
+            nodes.append(graph.call_function(operator.add if len(a) == 2 else operator.neg, tuple(nodes[i] for i in a)))
+            klass.append((c, len(a)))
+            args.append(a)
+        prev = len(nodes) - 1
+        for _ in range(int(rng.integers(0, 3))):  # stray nodes between the layers, of the layers' classes too
+            a = [int(rng.integers(0, len(nodes)))]
+            nodes.append(graph.call_function(operator.neg, (nodes[a[0]],)))
+            klass.append((int(rng.integers(0, 4)), 1))
+            args.append(a)
+    graph.output(nodes[-1])
+    rank = {n: i for i, n in enumerate(nodes)}
+
+    # the reference's lines around torch's functions
+    dup = {}
+    for n, c in zip(nodes[1:], klass[1:]):
+        dup.setdefault(c, []).append(n)
+    of = {n: lst for lst in dup.values() for n in lst}
+    anc = _populate_recursive_ancestor_map(graph)
+    groups = sorted(([[n] for n in lst] for lst in dup.values() if len(lst) > 1),
+                    key=lambda rg: -min(rank[r[0]] for r in rg))
+    seen = set()
+    for rg in groups:
+        if any(r[0] in seen for r in rg):
+            continue
+        fully_expand_region_group(rg, seen, anc, lambda a, b: a in of and b in of and of[a] is of[b] and a is not b)
+        for r in rg:
+            r.sort(key=rank.__getitem__)
+    groups = [rg for rg in groups if len(rg[0]) > 1]
+    for rg in groups:
+        rg.sort(key=lambda r: rank[r[0]])
+    groups.sort(key=lambda rg: rank[rg[0][0]])
+    want = [[[rank[n] for n in r] for r in rg] for rg in groups]
+
+    n = len(nodes)
+    ids = {c: i + 1 for i, c in enumerate(dict.fromkeys(klass[1:]))}
+    g = SimpleNamespace(num_nodes=n, node_edge_off=np.cumsum([0] + [len(a) for a in args]),
+                        edge_src_node=np.asarray([u for a in args for u in a], np.int64),
+                        node_kind=np.asarray([1] + [0] * (n - 1)), node_op=np.zeros(n, np.int32), node_phase=None)
+    flat = [i for rg in want for r in rg for i in r]
+    if len(set(flat)) != len(flat):
+        # a root of one list taken into a region of another, later, list: the reference ends with
+        # "Duplicate node ... in region group" (:198-205), and so does this
+        with pytest.raises(RuntimeError, match="Duplicate node"):
+            clustering.identical_regions(g, [0] + [ids[c] for c in klass[1:]])
+        return False
+    got = clustering.identical_regions(g, [0] + [ids[c] for c in klass[1:]])
+    assert got == want, seed
+    return len(want) > 0
