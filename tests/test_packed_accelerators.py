@@ -272,6 +272,10 @@ def _regions_mine_and_torchs(seed) -> bool:
             args.append(a)
     graph.output(nodes[-1])
     rank = {n: i for i, n in enumerate(nodes)}
+    # a forward/backward tag: part of the key, and a barrier for the growth (:123-139, 177)
+    cut = int(rng.integers(1, len(nodes) + 1))
+    phase = [0 if i < cut else 1 for i in range(len(nodes))]
+    klass = [None] + [c + (phase[i],) for i, c in enumerate(klass) if i > 0]
 
     # the reference's lines around torch's functions
     dup = {}
@@ -285,7 +289,10 @@ def _regions_mine_and_torchs(seed) -> bool:
     for rg in groups:
         if any(r[0] in seen for r in rg):
             continue
-        fully_expand_region_group(rg, seen, anc, lambda a, b: a in of and b in of and of[a] is of[b] and a is not b)
+        expanding = phase[rank[rg[0][0]]]
+        fully_expand_region_group(
+            rg, seen, anc,
+            lambda a, b: a in of and b in of and of[a] is of[b] and a is not b and phase[rank[a]] == expanding)
         for r in rg:
             r.sort(key=rank.__getitem__)
     groups = [rg for rg in groups if len(rg[0]) > 1]
@@ -298,7 +305,8 @@ def _regions_mine_and_torchs(seed) -> bool:
     ids = {c: i + 1 for i, c in enumerate(dict.fromkeys(klass[1:]))}
     g = SimpleNamespace(num_nodes=n, node_edge_off=np.cumsum([0] + [len(a) for a in args]),
                         edge_src_node=np.asarray([u for a in args for u in a], np.int64),
-                        node_kind=np.asarray([1] + [0] * (n - 1)), node_op=np.zeros(n, np.int32), node_phase=None)
+                        node_kind=np.asarray([1] + [0] * (n - 1)), node_op=np.zeros(n, np.int32),
+                        node_phase=np.asarray(phase, np.int32))
     flat = [i for rg in want for r in rg for i in r]
     if len(set(flat)) != len(flat):
         # a root of one list taken into a region of another, later, list: the reference ends with
