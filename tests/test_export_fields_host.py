@@ -158,3 +158,48 @@ def test_cluster_keys_follow_the_reference_hash_key():
     nodes[1].meta["partitioner_tag"] = "is_backward"
     again = ShardingOptimizer._cluster_keys(nodes)
     assert again[1] != again[2]  # a different tag separates them
+
+
+def test_cluster_keys_partition_like_the_pickled_key_of_the_reference():
+    """The reference hashes a pickle, made by torch's InputPickler, of (operator name, tag, source
+    position, argument values with tensors by their fake-tensor metadata, strategies)
+    (graph_clustering.py:35-52, 68-81).  On a traced joint graph the ids of _cluster_keys group the
+    nodes exactly as the non-strategy part of that pickle does (the strategies are the packed
+    arrays' part of the key)."""
+    from torch._dynamo.graph_region_tracker import InputPickler
+    from torch.utils._pytree import tree_flatten
+
+    from autoparallel_amd.optimize_sharding import ShardingOptimizer
+
+    gm = _joint(4)
+    nodes = [n for n in gm.graph.nodes if n.op != "output"]
+    assert {n.meta.get("partitioner_tag") for n in nodes} >= {"is_forward", "is_backward"}
+    # this tracer records no source positions; give the matmuls of the layers two different ones
+    mms = [n for n in nodes if n.target is torch.ops.aten.mm.default]
+    for i, n in enumerate(mms):
+        n.meta["stack_trace"] = f'File "model.py", line {20 + i % 2}, in forward'
+    pickler = InputPickler()
+
+    def extract(a):
+        if isinstance(a, torch.fx.Node):
+            return a.meta.get("val")
+        return a if isinstance(a, (torch.Tensor, int)) else None
+
+    def pickled(n):
+        flat, _ = tree_flatten(n.args)
+        kw = sorted(n.kwargs.items(), key=lambda kv: kv[0])
+        flat_kw, _ = tree_flatten(kw)
+        key = (str(n.target), n.meta.get("partitioner_tag"), n.meta.get("stack_trace"),
+               (tuple(sorted(n.kwargs)), tuple(extract(a) for a in flat + flat_kw)))
+        return pickler.dumps(key)
+
+    theirs = {}
+    for i, n in enumerate(nodes):
+        theirs.setdefault(pickled(n), []).append(i)
+    mine = {}
+    for i, k in enumerate(ShardingOptimizer._cluster_keys(nodes)):
+        mine.setdefault(int(k), []).append(i)
+    assert sorted(theirs.values()) == sorted(mine.values())
+    assert max(len(v) for v in mine.values()) >= 4  # the repeated layers do fall together
+    by_node = dict(zip(nodes, ShardingOptimizer._cluster_keys(nodes)))
+    assert all(by_node[a] != by_node[b] for a, b in zip(mms, mms[1:]))  # neighbours differ in source position
