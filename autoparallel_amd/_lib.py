@@ -231,6 +231,10 @@ _SIGNATURES = {
         C.c_int,
         [C.POINTER(ApcProblem), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
          C.c_void_p, C.c_void_p]),
+    "apc_compact_entries": (
+        C.c_int,
+        [C.POINTER(ApcProblem), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+         C.c_void_p, C.c_void_p]),
     "apc_solution_terms": (
         C.c_int,
         [C.POINTER(ApcProblem), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,

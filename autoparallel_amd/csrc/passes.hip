@@ -113,6 +113,28 @@ node_hash_kernel(apc_problem p, const int64_t* __restrict__ node_out_list,
   if (lane == 0) out[v] = mix64(acc);
 }
 
+// Entry arrays without their padding: slot -> decision variable.  Blocks start on
+// multiples of 16 slots, variables are numbered through the real entries only;
+// var_start[e] is the first variable of edge e's block.  One lane per slot, so the
+// reads are coalesced and the writes are the same stream shifted by the padding
+// before them.
+__global__ void __launch_bounds__(kBlock)
+compact_kernel(apc_problem p, const int64_t* __restrict__ var_start, const double* __restrict__ comm,
+               const double* __restrict__ cost, const uint8_t* __restrict__ flags,
+               double* __restrict__ out_comm, double* __restrict__ out_cost,
+               uint8_t* __restrict__ out_flags) {
+  const int64_t idx = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (idx >= p.n_slot) return;
+  const int e = p.chunk_edge[idx >> APC_CHUNK_SHIFT];
+  const apc_edge* ed = p.edges + e;
+  const int64_t local = idx - ed->off;
+  if (local >= (int64_t)ed->ssrc * ed->sdst) return;
+  const int64_t v = var_start[e] + local;
+  out_comm[v] = comm[idx];
+  out_cost[v] = cost[idx];
+  out_flags[v] = flags[idx];
+}
+
 // ---------------------------------------------------------------------------
 // Kernel: packed twin of the decision variables, in the reference's insertion
 // order (node, out_idx, argi, inp_idx): row of entry (e, o, j) is
@@ -319,6 +341,20 @@ int apc_export_decision_vars(const apc_problem* p, const double* per_arg, const 
   hipLaunchKernelGGL(export_kernel, dim3(grid), dim3(kBlock), 0, (hipStream_t)stream, *p, per_arg,
                      comm, flags, row_base, row_stride, keys, vals);
   return check_launch("export_kernel");
+}
+
+int apc_compact_entries(const apc_problem* p, const int64_t* var_start, const double* comm,
+                        const double* cost, const uint8_t* flags, double* out_comm, double* out_cost,
+                        uint8_t* out_flags, void* stream) {
+  if (int rc = validate_problem(p)) return rc;
+  if (p->n_slot == 0) return 0;
+  if (!var_start || !comm || !cost || !flags || !out_comm || !out_cost || !out_flags)
+    return fail(APC_ERR_INVALID, "apc_compact_entries: null argument%s");
+  unsigned grid;
+  if (int rc = slot_grid(p, kBlock, &grid)) return rc;
+  hipLaunchKernelGGL(compact_kernel, dim3(grid), dim3(kBlock), 0, (hipStream_t)stream, *p, var_start,
+                     comm, cost, flags, out_comm, out_cost, out_flags);
+  return check_launch("compact_kernel");
 }
 
 int apc_solution_terms(const apc_problem* p, const double* per_arg, const double* comm,

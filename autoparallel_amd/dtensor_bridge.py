@@ -4,6 +4,7 @@ from __future__ import annotations
 from typing import List, Optional, Sequence, Tuple
 
 import torch
+from torch.distributed.tensor.placement_types import Partial, Replicate, Shard
 
 from .packed import DT_BF16, DT_F16, DT_F32, DT_F64, DT_I8, DT_OTHER, PLC_OTHER, PLC_PARTIAL, PLC_R, PLC_SHARD
 
@@ -36,8 +37,6 @@ def _intern(p) -> int:
 
 
 def placement_code(p) -> int:
-    from torch.distributed.tensor.placement_types import Partial, Replicate, Shard
-
     if type(p) is Replicate or (isinstance(p, Replicate) and p.is_replicate()):
         return PLC_R
     if type(p) is Shard:

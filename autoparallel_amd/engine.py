@@ -21,6 +21,7 @@ _SCORE_FROM_TABLE = True  # the three ways of scoring a graph with large blocks 
 _SCORE_COMPACT = True
 _SCORE_STAGE_TILES = 8  # matrices of up to this many LDS tiles go through LDS in the table scorer
 _SCORE_PER_LANE = 0  # assignments per lane of the compact scorer; 0: the library chooses
+_READBACK_PINNED = True  # results() copies into pinned host memory (else pageable)
 _LUT_TABLE_FROM = 2048  # table units: larger tables are built tile by tile with per-source terms in LDS
 
 
@@ -759,16 +760,41 @@ class CostEngine:
         )
 
     # -- results on host --------------------------------------------------------
-    def results(self) -> Dict[str, np.ndarray]:
-        """The five result arrays on the host.  They are copied into pinned memory
-        (torch keeps freed pinned blocks, so only a process's first call pays for
-        pinning) by copies that run back to back; the arrays returned own it."""
+    def compact_entries(self):
+        """(comm, cost, flags) on the device with one element per decision variable:
+        the entry arrays without the padding between edge blocks
+        (apc_compact_entries), in the order of the ILP's columns."""
+        assert self.built
+        g = self.g
+        if "var_start" not in self._keep:
+            start = np.zeros(g.num_edges + 1, np.int64)
+            np.cumsum(g.block_sizes(), out=start[1:])
+            self._keep["var_start"] = torch.from_numpy(start).to(self.device)
+        E = g.num_entries
+        comm = torch.empty(E, dtype=torch.float64, device=self.device)
+        cost = torch.empty(E, dtype=torch.float64, device=self.device)
+        flags = torch.empty(E, dtype=torch.uint8, device=self.device)
+        _lib.check(
+            self.lib.apc_compact_entries(
+                C.byref(self.problem), self._ptr(self._keep["var_start"]), self._ptr(self.comm), self._ptr(self.cost),
+                self._ptr(self.flags), self._ptr(comm), self._ptr(cost), self._ptr(flags), self._stream()),
+            "apc_compact_entries")
+        return comm, cost, flags
+
+    def results(self, compact: bool = False) -> Dict[str, np.ndarray]:
+        """The five result arrays on the host.  ``compact``: comm, cost and flags
+        per decision variable (padding taken out on the device) instead of per
+        slot.  They are copied into pinned memory (torch keeps freed pinned
+        blocks, so only a process's first call pays for pinning) by copies that
+        run back to back; the arrays returned own it."""
         self.check_status()
+        src = {name: getattr(self, name) for name in ("comm", "cost", "flags", "compute", "per_arg")}
+        if compact and self.g.num_slots != self.g.num_entries:
+            src["comm"], src["cost"], src["flags"] = self.compact_entries()
         out = {}
-        for name in ("comm", "cost", "flags", "compute", "per_arg"):
-            src = getattr(self, name)
-            dst = torch.empty(src.shape, dtype=src.dtype, pin_memory=True)
-            dst.copy_(src, non_blocking=True)
+        for name, t in src.items():
+            dst = torch.empty(t.shape, dtype=t.dtype, pin_memory=_READBACK_PINNED)
+            dst.copy_(t, non_blocking=_READBACK_PINNED)
             out[name] = dst
         torch.cuda.current_stream(self.device).synchronize()
         return {k: v.numpy() for k, v in out.items()}

@@ -23,7 +23,7 @@ from torch.utils._pytree import tree_flatten
 
 from . import _lib, opprog
 from .dtensor_bridge import placement_codes, tensor_meta_key
-from .packed import OP_EXPLICIT, OP_PROGRAM, OP_ZERO, GraphBuilder, NodeDesc
+from .packed import OP_EXPLICIT, OP_PROGRAM, OP_ZERO, GraphBuilder, NodeDesc, spec_word
 
 aten = torch.ops.aten
 fallback_ops: "collections.Counter[str]" = collections.Counter()
@@ -92,6 +92,18 @@ def _closed_form(node) -> Optional[List[int]]:
         return opprog.same_as_arg(0, ins[0].dim(), osz)
     if t is aten.embedding.default and len(ins) == 2:
         return opprog.embedding(ins[1].dim(), osz)
+    if t is aten.embedding_dense_backward.default and len(ins) == 2 and ins[0].dim() >= 1:
+        return opprog.embedding_dense_backward(int(node.args[2]), osz, ins[0].dim())
+    if t is aten.cat.default and len(outs) == 1 and all(i.dim() == o0.dim() and i.dtype == o0.dtype for i in ins):
+        return opprog.cat(len(ins), osz)
+    if t is aten.slice_backward.default and len(ins) == 1 and all(isinstance(x, int) for x in node.args[1]):
+        return opprog.constant_shape(node.args[1], osz)
+    if t is aten.nll_loss_forward.default and len(outs) == 2 and ins[0].dim() == 2 and isinstance(node.args[3], int):
+        # (self [N, C], target [N], weight or None, reduction, ignore_index) -> (loss, total_weight)
+        return opprog.nll_loss_forward(node.args[3] == 0, osz, outs[1].element_size())
+    if t is aten.nll_loss_backward.default and len(outs) == 1 and len(ins) >= 4:
+        # (grad_output, self, target, weight or None, reduction, ignore_index, total_weight) -> grad of self
+        return opprog.same_as_arg(1, ins[1].dim(), osz)
     if torch.Tag.pointwise in t.tags and len(outs) == 1:
         # elementwise with broadcasting; the output shape is the broadcast of
         # the tensor arguments only if no argument is shape-expanding by itself
@@ -192,13 +204,27 @@ def describe_node(node, strategies, b: GraphBuilder, name: Optional[str] = None,
     by (operator, spec words, other arguments), so that the repeated layers of a
     model are converted once."""
     words = memo.setdefault("words", {}) if memo is not None else {}
+    # tensor metas and placement tuples by value: the specs of a graph are many objects
+    # over few distinct metas and tuples, and a dictionary hit costs a tenth of the conversion
+    meta_ids = memo.setdefault("meta_ids", {}) if memo is not None else {}
+    tuple_ids = memo.setdefault("tuple_ids", {}) if memo is not None else {}
 
     def word(s) -> int:
         if s is None or s.tensor_meta is None:
             return -1
         w = words.get(id(s))
         if w is None:
-            w = b.spec(b.meta(*tensor_meta_key(s.tensor_meta)), placement_codes(s.placements))
+            tm, plc = s.tensor_meta, s.placements
+            try:
+                m = meta_ids.get(tm)
+                if m is None:
+                    m = meta_ids[tm] = b.meta(*tensor_meta_key(tm))
+                t = tuple_ids.get(plc)
+                if t is None:
+                    t = tuple_ids[plc] = b.tuple_id(placement_codes(plc))
+            except TypeError:  # a size without a hash
+                m, t = b.meta(*tensor_meta_key(tm)), b.tuple_id(placement_codes(plc))
+            w = spec_word(m, t)
             words[id(s)] = w
         return w
 

@@ -18,7 +18,7 @@ def build_param_derived_set(graph: torch.fx.Graph) -> Set[torch.fx.Node]:
     derived = set(fx_utils.get_param_nodes(graph))
     for node in graph.nodes:
         ins = node.all_input_nodes
-        if ins and all(i in derived for i in ins):
+        if ins and derived.issuperset(ins):
             derived.add(node)
     return derived
 
@@ -30,7 +30,7 @@ def build_terminal_derived_set(graph: torch.fx.Graph) -> Set[torch.fx.Node]:
     for node in reversed(list(graph.nodes)):
         if node.op == "output":
             continue
-        if node.users and all(u in terminal for u in node.users):
+        if node.users and terminal.issuperset(node.users):
             terminal.add(node)
     return terminal
 

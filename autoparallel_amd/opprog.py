@@ -130,6 +130,25 @@ def embedding_dense_backward(num_weights: int, out_itemsize: int, grad_rank: int
     return program([], [(out_itemsize, [const(num_weights), argdim(0, grad_rank - 1)])])
 
 
+def cat(n_inputs: int, out_itemsize: int) -> List[int]:
+    """aten.cat of tensors that agree outside the concatenated dim: the output
+    has as many elements as the inputs together."""
+    return program([], [(out_itemsize, [argnumel(i)]) for i in range(n_inputs)])
+
+
+def constant_shape(shape: Sequence[int], out_itemsize: int) -> List[int]:
+    """Zero-flop op whose output shape is given among its arguments, not taken from
+    the local tensor sizes (aten.slice_backward's ``input_sizes``: the operator is
+    run with the global list whatever the sharding of its tensor)."""
+    return program([], [(out_itemsize, [const(int(s)) for s in shape])])
+
+
+def nll_loss_forward(unreduced: bool, out_itemsize: int, weight_itemsize: int) -> List[int]:
+    """(loss, total_weight) of aten.nll_loss_forward on a [N, C] input: the loss
+    per row without a reduction, else a scalar; total_weight is a scalar."""
+    return program([], [(out_itemsize, [argdim(0, 0)] if unreduced else []), (weight_itemsize, [])])
+
+
 # ROCm builds of torch return the philox seed and offset of the flash kernels
 # as two scalar int64 tensors (16 bytes in total).
 _PHILOX_BYTES_ROCM = 16

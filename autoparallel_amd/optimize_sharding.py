@@ -330,9 +330,11 @@ def _map_nodes(a, fn):
     return a
 
 
-def enumerate_strategies(graph, mesh) -> Dict[torch.fx.Node, Any]:
+def enumerate_strategies(graph, mesh, input_nodes: Optional[dict] = None) -> Dict[torch.fx.Node, Any]:
     """Placement strategies of every node that carries a tensor, in graph order
-    (build_sharding_metadata, autoparallel/optimize_sharding.py:306-354)."""
+    (build_sharding_metadata, autoparallel/optimize_sharding.py:306-354).
+    ``input_nodes``: a dict that receives, per call_function node, the
+    tensor-carrying nodes among its flattened args (what the packer asks for again)."""
     strats: Dict[torch.fx.Node, Any] = {}
     for node in graph.nodes:
         if node.op in ("placeholder", "get_attr"):
@@ -346,6 +348,8 @@ def enumerate_strategies(graph, mesh) -> Dict[torch.fx.Node, Any]:
                 continue
             in_nodes = [x for x in _flat_args(node.args, [])
                         if isinstance(x, torch.fx.Node) and x in strats]
+            if input_nodes is not None:
+                input_nodes[node] = in_nodes
             producers = [strats[x] for x in in_nodes]
             arg_vals = [x.meta["val"] for x in in_nodes]
             schema_args = _map_nodes(node.args, lambda x: strats.get(x, x.meta.get("val")))
@@ -453,7 +457,8 @@ class ShardingOptimizer:
 
     # -- strategies ---------------------------------------------------------------
     def build_sharding_metadata(self) -> Dict[torch.fx.Node, Any]:
-        return enumerate_strategies(self.graph, self.mesh)
+        self._input_nodes_of: Dict[torch.fx.Node, List[torch.fx.Node]] = {}
+        return enumerate_strategies(self.graph, self.mesh, self._input_nodes_of)
 
     def _all_input_nodes(self, node) -> List[torch.fx.Node]:
         """The tensor-carrying nodes among a node's flattened args, duplicates kept
@@ -556,59 +561,55 @@ class ShardingOptimizer:
             if at is not None:
                 r.bwd_pre_cast.update(nm[node] for node in chain[at:] if node in nm)
 
-    def _prefetchable(self, roles: GraphRoles) -> set:
-        """(node_idx, argi) of edges whose producer is parameter-derived or whose
-        consumer is terminal-derived (autoparallel/graph_passes/graph_utils.py:447-484)."""
+    def _prefetchable(self, g: PackedGraph, packed_nodes) -> np.ndarray:
+        """uint8 per edge: 1 where the producer is parameter-derived or the consumer
+        terminal-derived (autoparallel/graph_passes/graph_utils.py:447-484)."""
         from .graph_utils import build_param_derived_set, build_terminal_derived_set
 
-        if self._has_aot_descriptors():
-            derived = build_param_derived_set(self.graph)
-            terminal = build_terminal_derived_set(self.graph)
-        else:  # a graph without AOT descriptors has no parameters to prefetch
-            derived, terminal = set(), set()
-        out = set()
-        for node in self.nodes:
-            if node.op == "output":
-                continue
-            for a, prod in enumerate(self._all_input_nodes(node)):
-                if prod in derived or node in terminal:
-                    out.add((self.node_map[node], a))
-        return out
+        if not self._has_aot_descriptors():  # a graph without AOT descriptors has no parameters to prefetch
+            return np.zeros(g.num_edges, np.uint8)
+        derived_set = build_param_derived_set(self.graph)
+        terminal_set = build_terminal_derived_set(self.graph)
+        derived = np.fromiter((n in derived_set for n in packed_nodes), bool, len(packed_nodes))
+        terminal = np.fromiter((n in terminal_set for n in packed_nodes), bool, len(packed_nodes))
+        # an argument row counts when it has a producer among the node's inputs (named or not)
+        src = g.edge_src_node.astype(np.int64)
+        return ((src >= 0) & (derived[np.maximum(src, 0)] | terminal[g.edge_node])).astype(np.uint8)
 
     def _pack(self) -> PackedGraph:
         b = GraphBuilder(tuple(self.mesh.shape), self._devices_per_host)
         index_of: Dict[torch.fx.Node, int] = {}
-        self._packed_index: Dict[int, int] = {}  # node_idx -> packed node
         memo: Dict[str, dict] = {}
-        described: Dict[tuple, NodeDesc] = {}  # by strategy query: the repeated layers of a model
+        # One template per strategy query: the repeated layers of a model ask the same
+        # queries (same operator, arguments and candidates: same specs and program), and
+        # a node then only adds its producers.  Everything else is array work in pack().
+        template_of: Dict[int, int] = {}
+        strats, input_nodes_of = self.strats, self._all_input_nodes
+        packed_nodes: List[torch.fx.Node] = []
         for node in self.nodes:
             if node.op == "output":
                 continue
-            st: OpStrategy = self.strats[node]
-            qkey = getattr(st, "_apc_query_key", None)
-            seen = described.get(qkey) if qkey is not None else None
-            if seen is not None:  # same operator, arguments and candidates: same specs and program
-                desc = dataclasses.replace(seen, name=node.name, inputs=[], getitem_index=None)
-            else:
+            st: OpStrategy = strats[node]
+            qkey = getattr(st, "_apc_query_id", None)
+            t = template_of.get(qkey) if qkey is not None else None
+            if t is None:
                 desc = fx_programs.describe_node(node, st.strategies, b, name=node.name, memo=memo)
+                # rows of the strategies as they stand (their number per strategy is the
+                # number of arguments; the values are read below, where an edge keeps them)
+                desc.default_rows = [s.redistribute_cost for s in st.strategies]
+                desc.nargs = len(st.strategies[0].input_specs)
+                t = b.add_template(desc)
                 if qkey is not None:
-                    described[qkey] = desc
-            ins = self._all_input_nodes(node)
-            desc.inputs = [index_of[x] for x in ins]
-            if node.op == "call_function" and node.target is operator.getitem:
-                desc.getitem_index = int(node.args[1])
-            # default rows: what the strategy carried before the engine ran (the packer
-            # reads them where an edge has no producer or a spec is missing; not copied)
-            desc.default_rows = [s.redistribute_cost for s in st.strategies]
-            desc.nargs = len(st.strategies[0].input_specs)
-            index_of[node] = b.add_node(desc)
-            self._packed_index[self.node_map[node]] = index_of[node]
-        assert all(self._packed_index[i] == i for i in self._packed_index), "node order must be preserved"
-        roles = self._roles()
-        b.prefetchable_edges = self._prefetchable(roles)
-        g = b.pack()
-        g.roles = roles
-        packed_nodes = [n for n in self.nodes if n.op != "output"]
+                    template_of[qkey] = t
+            getitem = int(node.args[1]) if node.op == "call_function" and node.target is operator.getitem else None
+            index_of[node] = b.add_instance(t, [index_of[x] for x in input_nodes_of(node)], getitem, node.name)
+            packed_nodes.append(node)
+        # default rows: what a strategy carried before the engine ran; the packer reads them
+        # where an edge has no producer or a spec is missing
+        g = b.pack(default_rows_of=lambda v: [s.redistribute_cost for s in strats[packed_nodes[v]].strategies])
+        assert self.nodes[:len(packed_nodes)] == packed_nodes, "node order must be preserved"
+        g.roles = self._roles()
+        g.edge_prefetchable = self._prefetchable(g, packed_nodes)
         g.node_kind = np.asarray([1 if n.op == "placeholder" else (2 if n.op == "get_attr" else 0)
                                   for n in packed_nodes], np.uint8)
         g.node_phase = np.asarray([1 if n.meta.get("partitioner_tag") == "is_backward" else 0

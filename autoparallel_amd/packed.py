@@ -377,6 +377,9 @@ class PackedGraph:
         ``compressed``: records for the compressed block table (``table_off``
         of that layout; EDGE_COMPRESSED and the matrix's row length in
         ``flags`` for the edges whose matrix is stored by distinct spec word)."""
+        cache = self.__dict__.setdefault("_edge_records", {})  # made once per layout, like the block table
+        if compressed in cache:
+            return cache[compressed]
         NE = self.num_edges
         rec = np.zeros(NE, self.EDGE_DTYPE)
         assert rec.dtype.itemsize == 64
@@ -401,6 +404,7 @@ class PackedGraph:
         rec["flags"] = flags
         rec["node"] = self.edge_node
         rec["src_node"] = self.edge_src_node
+        cache[compressed] = rec
         return rec
 
     REC_ARGS = 14
@@ -464,8 +468,11 @@ class PackedGraph:
         out: List[tuple] = []
         where: Dict[int, Tuple[int, int, int]] = {}
         has_prog = self.node_op == OP_PROGRAM
-        offs = np.unique(self.node_prog_off[has_prog]) if has_prog.any() else np.zeros(0, np.int64)
-        lens = {int(o): int(l) for o, l in zip(self.node_prog_off[has_prog], self.node_prog_len[has_prog])}
+        if has_prog.any():
+            offs, at = np.unique(self.node_prog_off[has_prog], return_index=True)
+            lens = dict(zip(offs.tolist(), self.node_prog_len[has_prog][at].tolist()))
+        else:
+            offs, lens = np.zeros(0, np.int64), {}
         for off in offs:
             off = int(off)
             pr = [int(x) for x in self.prog[off:off + lens[off]]]
@@ -742,9 +749,24 @@ class PackedGraph:
         else:
             # an edge with a missing spec reads its own default rows: its key is its own index
             own = np.where(has_none[ok], ok, -1)
-            key = np.stack([src[ok], dst[ok], ssrc[ok], sdst[ok], own], axis=1)
-            _, first, inv = np.unique(key, axis=0, return_index=True, return_inverse=True)
-            inv = inv.reshape(-1)
+            # distinct (src, dst, ssrc, sdst, own) rows in lexicographic order, each named by
+            # its first edge: a stable sort on three 64-bit keys (np.unique over rows sorts
+            # them as structured records, twenty times slower)
+            k_runs = src[ok] * (self.lists.shape[0] + 1) + dst[ok]
+            k_size = (ssrc[ok] << 31) | sdst[ok]
+            order = np.argsort(k_runs, kind="stable")
+            kr, ks, ko = k_runs[order], k_size[order], own[order]
+            new = np.ones(order.shape[0], bool)
+            new[1:] = (kr[1:] != kr[:-1]) | (ks[1:] != ks[:-1]) | (ko[1:] != ko[:-1])
+            if (new[1:] & (kr[1:] == kr[:-1])).any():
+                # one pair of runs at two extents, or with and without rows of its own: the
+                # sort on the runs alone does not group those, the full one does
+                order = np.lexsort((own, k_size, k_runs))
+                kr, ks, ko = k_runs[order], k_size[order], own[order]
+                new[1:] = (kr[1:] != kr[:-1]) | (ks[1:] != ks[:-1]) | (ko[1:] != ko[:-1])
+            first = order[new]
+            inv = np.empty(order.shape[0], np.int64)
+            inv[order] = np.cumsum(new) - 1
             block_edge = ok[first].astype(np.int32)
             size = cols[block_edge] * rows[block_edge]
             block_off = np.zeros(block_edge.shape[0] + 1, np.int64)
@@ -788,7 +810,9 @@ class PackedGraph:
         eid = np.repeat(np.arange(self.num_edges, dtype=np.int64), n)
         start = np.concatenate([[0], np.cumsum(n)[:-1]])
         k = np.arange(int(n.sum()), dtype=np.int64) - start[eid]
-        items = self.edge_records(compressed)[eid]
+        # rows of eight 64-bit words: gathering structured records field by field is ten times slower
+        words = np.take(self.edge_records(compressed).view(np.uint64).reshape(-1, 8), eid, axis=0)
+        items = words.reshape(-1).view(self.EDGE_DTYPE)
         items["local0"] = ((k * item_entries - lead[eid]) & 0xFFFFFFFF).astype(np.uint32)
         cache[(compressed, item_entries)] = items
         return items
@@ -876,9 +900,9 @@ class PackedGraph:
             assert (self.node_comp_off >= 0).all()
             assert (self.node_comp_off + self.node_nstrat <= self.n_compute).all()
             # every slot is written by exactly one evaluated node
-            covered = np.zeros(self.n_compute + 1, np.int64)
-            np.add.at(covered, self.node_comp_off[self.comp_nodes], 1)
-            np.add.at(covered, self.node_comp_off[self.comp_nodes] + self.node_nstrat[self.comp_nodes], -1)
+            lo = self.node_comp_off[self.comp_nodes]
+            hi = lo + self.node_nstrat[self.comp_nodes]
+            covered = (np.bincount(lo, minlength=self.n_compute + 1) - np.bincount(hi, minlength=self.n_compute + 1))
             assert (np.cumsum(covered)[:-1] == 1).all(), "compute slots not covered exactly once"
             assert np.isin(self.node_comp_off, self.node_comp_off[self.comp_nodes]).all()
         assert self.node_edge_off.shape == (N + 1,)
@@ -1005,6 +1029,7 @@ class GraphBuilder:
         self.share_compute_slots = True
         self.prefetchable_edges: set = set()  # (node_idx, argi)
         self.multiplier: Dict[int, int] = {}
+        self._reset_templates()
 
     def meta(self, shape, stride, itemsize: int, dtype: int) -> int:
         key = (tuple(int(s) for s in shape), tuple(int(s) for s in stride), int(itemsize), int(dtype))
@@ -1056,10 +1081,132 @@ class GraphBuilder:
         return self._meta_rows[word >> TUPLE_BITS]
 
     def add_node(self, node: NodeDesc) -> int:
+        """A node described on its own.  It is read when ``pack`` runs (so its fields
+        may still change until then)."""
+        assert not self._inst_tmpl, "a builder takes either nodes or template instances"
         self.nodes.append(node)
         return len(self.nodes) - 1
 
-    def pack(self) -> PackedGraph:
+    # -- templates: one description for all the nodes that share it ------------------
+    def _add_run(self, words) -> int:
+        """Offset of a run of spec words; identical runs are stored once, which also
+        makes a producer's run offset the identity of its row table."""
+        key = tuple(map(int, words))
+        off = self._run_cache.get(key)
+        if off is None:
+            off = len(self._lists)
+            self._run_cache[key] = off
+            self._lists.extend(key)
+        return off
+
+    def add_template(self, desc: NodeDesc) -> int:
+        """Registers everything about a node that does not depend on where it sits in
+        the graph: strategy count, runs of output and input spec words, program,
+        compute-slot class.  ``desc.inputs`` and ``desc.getitem_index`` are not read;
+        ``desc.default_rows`` only for the number of argument rows.  The repeated
+        layers of a model share their templates (add_instance)."""
+        S = len(desc.in_specs)
+        assert S == len(desc.out_specs) and S >= 1
+        t = len(self._t_S)
+        nargs = desc.nargs if desc.nargs is not None else len(desc.in_specs[0])
+        prog_off, prog_len = -1, 0
+        if desc.program is not None:
+            key = tuple(int(x) for x in desc.program)
+            check_program(key, len(desc.in_specs[0]))
+            prog_off = self._prog_cache.get(key)
+            if prog_off is None:  # identical programs are stored once
+                prog_off = len(self._prog)
+                self._prog_cache[key] = prog_off
+                self._prog.extend(key)
+            prog_len = len(key)
+        nout = len(desc.out_specs[0])
+        out_runs = [self._add_run([row[k] for row in desc.out_specs]) for k in range(nout)]
+        # edges: one per row of redistribute_cost (== per arg)
+        n_rows = len(desc.in_specs[0]) if desc.default_rows is None else len(desc.default_rows[0])
+        dst_runs, dst_none = [], []
+        for a in range(n_rows):
+            words = [int(row[a]) if a < len(row) else -1 for row in desc.in_specs]
+            dst_runs.append(self._add_run(words))
+            dst_none.append(min(words) < 0)
+        # compute slots: nodes with the same op class, program, arg count and input spec
+        # words produce the same estimate (the reference's memo key,
+        # compute_estimation.py:449-467) and share one slot; explicit counts are per node
+        if desc.op == OP_EXPLICIT:
+            comp_class = -1
+        else:
+            if desc.op == OP_ZERO:
+                key = (OP_ZERO, S, int(nargs))
+            else:
+                key = (desc.op, tuple(int(x) for x in desc.program), int(nargs), tuple(tuple(r) for r in desc.in_specs))
+            comp_class = self._comp_classes.setdefault(key, len(self._comp_classes))
+        self._t_S.append(S)
+        self._t_nargs.append(int(nargs))
+        self._t_op.append(int(desc.op))
+        self._t_prog.append((prog_off, prog_len))
+        self._t_out_runs.append(out_runs)
+        self._t_dst_runs.append(dst_runs)
+        self._t_dst_none.append(dst_none)
+        self._t_tuple_out.append(bool(desc.tuple_output))
+        self._t_comp_class.append(comp_class)
+        self._t_desc.append(desc)
+        return t
+
+    def add_instance(self, template: int, inputs: Sequence[Optional[int]], getitem_index: Optional[int] = None,
+                     name: Optional[str] = None, default_rows=None) -> int:
+        """A node of the graph: a template at a place.  ``inputs[a]``: the producer of
+        argument a (None or negative: none); ``default_rows``: the node's
+        ``[o][a][j]`` default costs, or None to ask ``pack``'s callback (or zeros)."""
+        assert not self.nodes, "a builder takes either nodes or template instances"
+        v = len(self._inst_tmpl)
+        self._inst_tmpl.append(template)
+        self._inst_inputs.append(inputs)
+        self._inst_getitem.append(-1 if getitem_index is None else int(getitem_index))
+        self._inst_name.append(name)
+        if default_rows is not None:
+            self._inst_defaults[v] = default_rows
+        return v
+
+    def pack(self, default_rows_of=None) -> PackedGraph:
+        """``default_rows_of(v)``: the ``[o][a][j]`` default costs of node v, asked only
+        for the arguments that keep them (no producer, or a missing spec)."""
+        if self.nodes:  # nodes described on their own: a template each, in node order
+            for nd_ in self.nodes:
+                v = len(self._inst_tmpl)
+                self._inst_tmpl.append(self.add_template(nd_))
+                self._inst_inputs.append(nd_.inputs)
+                self._inst_getitem.append(-1 if nd_.getitem_index is None else int(nd_.getitem_index))
+                self._inst_name.append(nd_.name)
+                if nd_.default_rows is not None:
+                    self._inst_defaults[v] = nd_.default_rows
+            try:
+                return self._pack(default_rows_of)
+            finally:  # the builder stays what it was: a list of nodes, packed again on the next call
+                self._reset_templates()
+        return self._pack(default_rows_of)
+
+    def _reset_templates(self) -> None:
+        self._lists: List[int] = []
+        self._run_cache: Dict[Tuple[int, ...], int] = {}
+        self._prog: List[int] = []
+        self._prog_cache: Dict[Tuple[int, ...], int] = {}
+        self._comp_classes: Dict[tuple, int] = {}
+        self._t_S: List[int] = []
+        self._t_nargs: List[int] = []
+        self._t_op: List[int] = []
+        self._t_prog: List[Tuple[int, int]] = []
+        self._t_out_runs: List[List[int]] = []
+        self._t_dst_runs: List[List[int]] = []
+        self._t_dst_none: List[List[bool]] = []
+        self._t_tuple_out: List[bool] = []
+        self._t_comp_class: List[int] = []
+        self._t_desc: List[NodeDesc] = []
+        self._inst_tmpl: List[int] = []
+        self._inst_inputs: List[Sequence[Optional[int]]] = []
+        self._inst_getitem: List[int] = []
+        self._inst_name: List[Optional[str]] = []
+        self._inst_defaults: Dict[int, object] = {}
+
+    def _pack(self, default_rows_of=None) -> PackedGraph:
         nd = len(self.mesh_shape)
         M = len(self._meta_rows)
         meta_rank = np.zeros(M, np.int32)
@@ -1080,159 +1227,137 @@ class GraphBuilder:
         for i, plc in enumerate(self._tuple_rows):
             tuple_plc[i, :nd] = plc
 
-        N = len(self.nodes)
-        lists: List[int] = []
-        node_nstrat = np.zeros(N, np.int32)
-        node_nargs = np.zeros(N, np.int32)
-        node_op = np.zeros(N, np.int32)
-        node_prog_off = np.full(N, -1, np.int64)
-        node_prog_len = np.zeros(N, np.int32)
-        prog_cache: Dict[Tuple[int, ...], int] = {}
+        def ragged(rows, dtype=np.int64):
+            """(flat, first position of every row)"""
+            cnt = np.fromiter((len(r) for r in rows), np.int64, len(rows))
+            off = np.zeros(len(rows) + 1, np.int64)
+            np.cumsum(cnt, out=off[1:])
+            flat = np.fromiter((x for r in rows for x in r), dtype, int(off[-1]))
+            return flat, off[:-1], cnt
+
+        # per template
+        T = len(self._t_S)
+        t_S = np.asarray(self._t_S, np.int64)
+        t_nargs = np.asarray(self._t_nargs, np.int32)
+        t_op = np.asarray(self._t_op, np.int32)
+        t_prog = np.asarray(self._t_prog, np.int64).reshape(T, 2)
+        t_tuple = np.asarray(self._t_tuple_out, bool)
+        t_class = np.asarray(self._t_comp_class, np.int64)
+        out_flat, t_out_off, t_nout = ragged(self._t_out_runs)
+        dst_flat, t_dst_off, t_nrows = ragged(self._t_dst_runs)
+        dst_none_flat = np.fromiter((x for r in self._t_dst_none for x in r), bool, dst_flat.shape[0])
+        lists = (np.asarray(self._lists, np.int64) & 0xFFFFFFFF).astype(np.uint32)
+        none_csum = np.concatenate([[0], np.cumsum(lists == SPEC_NONE)])
+
+        # per node
+        N = len(self._inst_tmpl)
+        tm = np.asarray(self._inst_tmpl, np.int64)
+        assert N == 0 or ((tm >= 0) & (tm < T)).all()
+        node_nstrat = t_S[tm].astype(np.int32)
+        node_nargs = t_nargs[tm]
+        node_op = t_op[tm]
+        node_prog_off = t_prog[tm, 0]
+        node_prog_len = t_prog[tm, 1].astype(np.int32)
+        getitem = np.asarray(self._inst_getitem, np.int64)
+        nrows = t_nrows[tm]
         node_edge_off = np.zeros(N + 1, np.int32)
-        prog: List[int] = []
-        # per node, per output index: offset of its run of output spec ids
-        out_runs: List[Dict[int, int]] = []
-        run_cache: Dict[Tuple[int, ...], int] = {}
+        np.cumsum(nrows, out=node_edge_off[1:])
+        NE = int(node_edge_off[-1])
+        in_flat, in_off, in_cnt = ragged([[-1 if u is None else u for u in r] for r in self._inst_inputs])
 
-        def add_run(words) -> int:
-            """Offset of a run of spec words; identical runs are stored once,
-            which also makes a producer's run offset the identity of its row
-            table."""
-            key = tuple(map(int, words))
-            off = run_cache.get(key)
-            if off is None:
-                off = len(lists)
-                run_cache[key] = off
-                lists.extend(key)
-            return off
-
-        e_node, e_arg, e_src, e_sdst, e_ssrc = [], [], [], [], []
-        e_dst_list, e_src_list, e_flags, e_def = [], [], [], []
+        # edges: one per argument row
+        e_node = np.repeat(np.arange(N, dtype=np.int64), nrows)
+        e_arg = np.arange(NE, dtype=np.int64) - node_edge_off[:-1].astype(np.int64)[e_node]
+        et = tm[e_node]
+        edge_sdst = t_S[et].astype(np.int32)
+        e_dst_list = dst_flat[t_dst_off[et] + e_arg]
+        has_in = e_arg < in_cnt[e_node]
+        u = np.full(NE, -1, np.int64)
+        u[has_in] = in_flat[(in_off[e_node] + e_arg)[has_in]]
+        has_prod = u >= 0
+        assert (u[has_prod] < e_node[has_prod]).all(), "producers must precede consumers"
+        ut = tm[np.maximum(u, 0)]
+        k = np.maximum(getitem[e_node], 0)
+        # a tuple-valued producer consumed directly is not a DTensorSpec: default row kept (:473)
+        named = has_prod & ~(t_tuple[ut] & (getitem[e_node] < 0))
+        assert (k[named] < t_nout[ut[named]]).all(), "getitem index past the producer's outputs"
+        e_src_list = np.full(NE, -1, np.int64)
+        e_src_list[named] = out_flat[(t_out_off[ut] + k)[named]]
+        edge_ssrc = np.where(has_prod, t_S[ut], 1).astype(np.int32)
+        e_flags = np.where(named, EDGE_HAS_PRODUCER, 0) | np.where(has_prod & ~t_tuple[ut], EDGE_SCORE_TRANSITION, 0)
+        # a missing spec on either side keeps the default row
+        src_none = np.zeros(NE, bool)
+        sl = e_src_list[named]
+        src_none[named] = none_csum[sl + edge_ssrc[named]] - none_csum[sl] > 0
+        need_default = ~named | dst_none_flat[t_dst_off[et] + e_arg] | src_none
+        e_def = np.full(NE, -1, np.int64)
         defaults: List[float] = []
-        any_explicit = False
-        for v, nd_ in enumerate(self.nodes):
-            S = len(nd_.in_specs)
-            assert S == len(nd_.out_specs) and S >= 1
-            node_nstrat[v] = S
-            node_nargs[v] = nd_.nargs if nd_.nargs is not None else len(nd_.in_specs[0])
-            node_op[v] = nd_.op
-            if nd_.program is not None:
-                key = tuple(int(x) for x in nd_.program)
-                check_program(key, len(nd_.in_specs[0]))
-                off = prog_cache.get(key)
-                if off is None:  # identical programs are stored once
-                    off = len(prog)
-                    prog_cache[key] = off
-                    prog.extend(key)
-                node_prog_off[v] = off
-                node_prog_len[v] = len(key)
-            if nd_.op == OP_EXPLICIT:
-                any_explicit = True
-            nout = len(nd_.out_specs[0])
-            runs = {}
-            for k in range(nout):
-                runs[k] = add_run([row[k] for row in nd_.out_specs])
-            out_runs.append(runs)
-            # edges: one per row of redistribute_cost (== per arg)
-            n_rows = len(nd_.in_specs[0])
-            if nd_.default_rows is not None:
-                n_rows = len(nd_.default_rows[0])
-            node_edge_off[v] = len(e_node)
-            for a in range(n_rows):
-                has_prod = a < len(nd_.inputs) and nd_.inputs[a] is not None and nd_.inputs[a] >= 0
-                e_node.append(v)
-                e_arg.append(a)
-                e_sdst.append(S)
-                dst_words = [int(row[a]) if a < len(row) else -1 for row in nd_.in_specs]
-                e_dst_list.append(add_run(dst_words))
-                flags = 0
-                if has_prod:
-                    u = nd_.inputs[a]
-                    assert u < v, "producers must precede consumers"
-                    prod = self.nodes[u]
-                    k = nd_.getitem_index if nd_.getitem_index is not None else 0
-                    if prod.tuple_output and nd_.getitem_index is None:
-                        # tuple-valued producer consumed directly: not a
-                        # DTensorSpec -> default row kept (:473)
-                        src_run = -1
-                    else:
-                        src_run = out_runs[u][k]
-                    ssrc = len(prod.in_specs)
-                    e_src.append(u)
-                    e_ssrc.append(ssrc)
-                    if src_run >= 0:
-                        flags |= EDGE_HAS_PRODUCER
-                    if not prod.tuple_output:
-                        flags |= EDGE_SCORE_TRANSITION
-                    e_src_list.append(src_run)
-                else:
-                    e_src.append(-1)
-                    ssrc = (
-                        len(nd_.default_rows[0][a]) if nd_.default_rows is not None else 1
-                    )
-                    e_ssrc.append(ssrc)
-                    e_src_list.append(-1)
-                # a missing spec on either side (-1) keeps the default row
-                need_default = ((flags & EDGE_HAS_PRODUCER) == 0 or min(dst_words) < 0
-                                or min(lists[e_src_list[-1]:e_src_list[-1] + e_ssrc[-1]]) < 0)
-                if need_default:
-                    e_def.append(len(defaults))
-                    for o in range(S):
-                        if nd_.default_rows is not None:
-                            row = nd_.default_rows[o][a]
-                            assert len(row) == e_ssrc[-1]
-                            defaults.extend(float(x) for x in row)
-                        else:
-                            defaults.extend([0.0] * e_ssrc[-1])
-                else:
-                    e_def.append(-1)
-                e_flags.append(flags)
-        node_edge_off[N] = len(e_node)
-        NE = len(e_node)
-        edge_sdst = np.asarray(e_sdst, np.int32)
-        edge_ssrc = np.asarray(e_ssrc, np.int32)
+        rows_of: Dict[int, object] = {}
+
+        def node_rows(v):
+            if v not in rows_of:
+                r = self._inst_defaults.get(v)
+                if r is None and default_rows_of is not None:
+                    r = default_rows_of(v)
+                rows_of[v] = r
+            return rows_of[v]
+
+        for e in np.nonzero(need_default)[0].tolist():
+            v, a = int(e_node[e]), int(e_arg[e])
+            rows = node_rows(v)
+            if not has_prod[e]:
+                edge_ssrc[e] = len(rows[0][a]) if rows is not None else 1
+            n_s = int(edge_ssrc[e])
+            e_def[e] = len(defaults)
+            if rows is None:
+                defaults.extend([0.0] * (n_s * int(edge_sdst[e])))
+            else:
+                assert len(rows) == int(edge_sdst[e]) and len(rows[0]) == int(nrows[v])
+                for o in range(int(edge_sdst[e])):
+                    row = rows[o][a]
+                    assert len(row) == n_s
+                    defaults.extend(float(x) for x in row)
         edge_off = np.zeros(NE + 1, np.int64)
         pad = (1 << CHUNK_SHIFT) - 1
         np.cumsum((edge_sdst.astype(np.int64) * edge_ssrc + pad) & ~pad, out=edge_off[1:])
-        # compute slots: nodes with the same op class, program, arg count and
-        # input spec words produce the same estimate (the reference's memo key,
-        # compute_estimation.py:449-467) and share one slot
-        node_comp_off = np.zeros(N, np.int64)
-        slot_of: Dict[tuple, int] = {}
-        comp_nodes: List[int] = []
-        n_compute = 0
-        for v, nd_ in enumerate(self.nodes):
-            if nd_.op == OP_EXPLICIT or not self.share_compute_slots:
-                key = ("node", v)
-            elif nd_.op == OP_ZERO:
-                key = (OP_ZERO, len(nd_.in_specs), int(node_nargs[v]))
-            else:
-                key = (nd_.op, tuple(int(x) for x in nd_.program), int(node_nargs[v]),
-                       tuple(tuple(r) for r in nd_.in_specs))
-            off = slot_of.get(key)
-            if off is None:
-                off = n_compute
-                slot_of[key] = off
-                n_compute += len(nd_.in_specs)
-                comp_nodes.append(v)
-            node_comp_off[v] = off
+
+        # compute slots, in the order their first nodes appear
+        own_slot = (t_class[tm] < 0) | (not self.share_compute_slots)
+        slot_key = np.where(own_slot, -1 - np.arange(N, dtype=np.int64), t_class[tm])
+        _, first, inverse = np.unique(slot_key, return_index=True, return_inverse=True)
+        order = np.argsort(first, kind="stable")
+        comp_nodes = first[order]
+        slot_off = np.zeros(comp_nodes.shape[0] + 1, np.int64)
+        np.cumsum(node_nstrat[comp_nodes], out=slot_off[1:])
+        n_compute = int(slot_off[-1])
+        rank_of = np.empty(order.shape[0], np.int64)
+        rank_of[order] = np.arange(order.shape[0])
+        node_comp_off = slot_off[:-1][rank_of[inverse.reshape(-1)]] if N else np.zeros(0, np.int64)
+
         pref = np.zeros(NE, np.uint8)
-        for i, (v, a) in enumerate(zip(e_node, e_arg)):
-            if (v, a) in self.prefetchable_edges:
-                pref[i] = 1
+        if self.prefetchable_edges:
+            pv = np.asarray(sorted(self.prefetchable_edges), np.int64).reshape(-1, 2)
+            pv = pv[(pv[:, 0] >= 0) & (pv[:, 0] < N)]
+            pv = pv[(pv[:, 1] >= 0) & (pv[:, 1] < nrows[pv[:, 0]])]
+            pref[node_edge_off[:-1].astype(np.int64)[pv[:, 0]] + pv[:, 1]] = 1
         mult = np.ones(N, np.int32)
         for v, m in self.multiplier.items():
             mult[v] = m
         ef = eb = None
-        if any_explicit:
+        explicit = np.nonzero(node_op == OP_EXPLICIT)[0]
+        if explicit.shape[0]:
             ef = np.zeros(n_compute, np.int64)
             eb = np.zeros(n_compute, np.int64)
-            for v, nd_ in enumerate(self.nodes):
-                if nd_.op == OP_EXPLICIT:
-                    o0 = int(node_comp_off[v])
-                    ef[o0 : o0 + len(nd_.flops)] = nd_.flops
-                    eb[o0 : o0 + len(nd_.nbytes)] = nd_.nbytes
-        max_outs = max((len(x) for x in out_runs), default=1)
+            for v in explicit.tolist():
+                d = self._t_desc[int(tm[v])]
+                o0 = int(node_comp_off[v])
+                ef[o0 : o0 + len(d.flops)] = d.flops
+                eb[o0 : o0 + len(d.nbytes)] = d.nbytes
+        max_outs = int(t_nout.max()) if T else 1
+        t_out_pad = np.full((T, max(max_outs, 1)), -1, np.int64)
+        for t, runs in enumerate(self._t_out_runs):
+            t_out_pad[t, : len(runs)] = runs
+        names = self._inst_name
         g = PackedGraph(
             mesh_shape=np.asarray(self.mesh_shape, np.int32),
             devices_per_host=self.devices_per_host,
@@ -1242,36 +1367,35 @@ class GraphBuilder:
             meta_itemsize=meta_itemsize,
             meta_dtype=meta_dtype,
             tuple_plc=tuple_plc,
-            lists=(np.asarray(lists, np.int64) & 0xFFFFFFFF).astype(np.uint32),
+            lists=lists,
             node_nstrat=node_nstrat,
             node_nargs=node_nargs,
             node_comp_off=node_comp_off,
             n_compute=n_compute,
-            comp_nodes=np.asarray(comp_nodes, np.int32),
+            comp_nodes=comp_nodes.astype(np.int32),
             node_edge_off=node_edge_off,
             node_op=node_op,
             node_prog_off=node_prog_off,
             node_prog_len=node_prog_len,
-            node_out_list=np.asarray([r[0] for r in out_runs], np.int64),
-            prog=np.asarray(prog, np.int64),
+            node_out_list=t_out_pad[tm, 0] if N else np.zeros(0, np.int64),
+            prog=np.asarray(self._prog, np.int64),
             explicit_flops=ef,
             explicit_bytes=eb,
-            edge_node=np.asarray(e_node, np.int32),
-            edge_arg=np.asarray(e_arg, np.int32),
-            edge_src_node=np.asarray(e_src, np.int32),
+            edge_node=e_node.astype(np.int32),
+            edge_arg=e_arg.astype(np.int32),
+            edge_src_node=u.astype(np.int32),
             edge_sdst=edge_sdst,
             edge_ssrc=edge_ssrc,
-            edge_dst_list=np.asarray(e_dst_list, np.int64),
-            edge_src_list=np.asarray(e_src_list, np.int64),
+            edge_dst_list=e_dst_list,
+            edge_src_list=e_src_list,
             edge_off=edge_off,
-            edge_flags=np.asarray(e_flags, np.int32),
-            edge_default_off=np.asarray(e_def, np.int64),
+            edge_flags=e_flags.astype(np.int32),
+            edge_default_off=e_def,
             default_vals=np.asarray(defaults, np.float64),
             edge_prefetchable=pref,
             node_multiplier=mult,
-            node_names=[n.name for n in self.nodes],
-            node_out_runs=np.asarray([[r.get(k, -1) for k in range(max_outs)] for r in out_runs],
-                                     np.int64).reshape(len(out_runs), max_outs),
+            node_names=[n if n is not None else f"node{v}" for v, n in enumerate(names)],
+            node_out_runs=t_out_pad[tm] if N else np.zeros((0, max(max_outs, 1)), np.int64),
         )
         g.validate()
         return g

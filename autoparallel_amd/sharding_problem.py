@@ -52,10 +52,14 @@ class Coefficients:
     (padding slots removed), plus the per-(node, out_idx) compute vectors."""
 
     def __init__(self, g: PackedGraph, comm, cost, flags, compute, per_arg):
-        slots = g.entry_slots()
-        self.comm = np.ascontiguousarray(comm[slots])
-        self.cost = np.ascontiguousarray(cost[slots])
-        self.flags = np.ascontiguousarray(flags[slots])
+        """comm, cost, flags: per slot of the entry arrays (padding is dropped here),
+        or already per decision variable."""
+        if len(comm) != g.num_entries:
+            slots = g.entry_slots()
+            comm, cost, flags = comm[slots], cost[slots], flags[slots]
+        self.comm = np.ascontiguousarray(comm)
+        self.cost = np.ascontiguousarray(cost)
+        self.flags = np.ascontiguousarray(flags)
         self.compute = np.asarray(compute)
         self.per_arg = np.asarray(per_arg)
 
@@ -69,7 +73,7 @@ class Coefficients:
 
     @classmethod
     def from_engine(cls, eng) -> "Coefficients":
-        r = eng.results()
+        r = eng.results(compact=True)  # padding taken out on the device: 17 B per variable cross the link
         return cls(eng.g, r["comm"], r["cost"], r["flags"], r["compute"], r["per_arg"])
 
     @classmethod

@@ -768,8 +768,9 @@ def _copy_strategy(src: OpStrategy) -> OpStrategy:
 # strategies by query, as the reference keeps them
 # (autoparallel/shardings/placement_options.py:183-217, 279-302): the layers of a
 # model repeat the same queries, and one answer from the propagator costs
-# milliseconds.  Values: (strategies, why the all-Replicate stand-in was used or None).
+# milliseconds.  Values: (strategies, why the all-Replicate stand-in was used or None, id of the answer).
 _strategy_cache: Dict[tuple, tuple] = {}
+_query_serial = itertools.count()  # never restarts: an id names one answer for the life of the process
 strategy_cache_stats = {"hits": 0, "misses": 0}
 
 
@@ -804,7 +805,7 @@ def get_placement_options_for_node(mesh, node, producers: List[OpStrategy], arg_
             fallback_nodes.append(str(node.name))
             fallback_reasons[str(node.name)] = hit[1]
         out = _copy_strategy(hit[0])
-        out._apc_query_key = key  # equal keys: equal strategies (what a packer may memoise on)
+        out._apc_query_id = hit[2]  # equal ids: equal strategies (what a packer may memoise on)
         return out
     strategy_cache_stats["misses"] += 1
     n_fallback = len(fallback_nodes)
@@ -812,8 +813,9 @@ def get_placement_options_for_node(mesh, node, producers: List[OpStrategy], arg_
     if key is not None:
         why = fallback_reasons.get(str(node.name), "") if len(fallback_nodes) > n_fallback else None
         _fingerprint(out)  # summarised here, once: the cached copy and every later copy inherit it
-        _strategy_cache[key] = (_copy_strategy(out), why)
-        out._apc_query_key = key
+        qid = next(_query_serial)
+        _strategy_cache[key] = (_copy_strategy(out), why, qid)
+        out._apc_query_id = qid
     return out
 
 

@@ -552,6 +552,17 @@ int apc_export_decision_vars(const apc_problem* p, const double* per_arg, const 
                              const uint8_t* flags, const int64_t* row_base,
                              const int32_t* row_stride, int32_t* keys, double* vals, void* stream);
 
+/* The three entry arrays with the padding between edge blocks taken out: element
+ * var_start[e] + out_idx * S_src + inp_idx of the outputs is entry (e, out_idx,
+ * inp_idx), i.e. the arrays are indexed by decision variable, in
+ * walk_over_options order (autoparallel/optimize_sharding.py:400-410), which is
+ * the column order of the ILP.  var_start: int64[n_edge], running sum of the
+ * entries of the edges that own a block.  Outputs hold n_entry elements.  This is
+ * what a host reads back (17 B per variable) instead of the padded arrays. */
+int apc_compact_entries(const apc_problem* p, const int64_t* var_start, const double* comm,
+                        const double* cost, const uint8_t* flags, double* out_comm, double* out_cost,
+                        uint8_t* out_flags, void* stream);
+
 /* Replaces the selected-variable gathers of export_sharding_json
  * (autoparallel/export_json.py:314-361) and get_log
  * (autoparallel/log_formatting.py:118-130) for one assignment (assign:

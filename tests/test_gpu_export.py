@@ -121,3 +121,35 @@ def test_full_size_export_properties(engine_mod):
     k = keys.to(torch.int64)
     code = ((k[:, 0] * 4096 + k[:, 2]) * 64 + k[:, 1]) * 4096 + k[:, 3]
     assert bool((code[1:] > code[:-1]).all())
+
+
+@pytest.mark.parametrize("name", list(GRAPHS))
+def test_compacted_entries_are_the_real_slots(engine_mod, name):
+    """apc_compact_entries: the three entry arrays per decision variable equal a
+    host gather of the padded arrays at entry_slots(), bit for bit; with repeated
+    nodes aliased to their roots too."""
+    g = GRAPHS[name]()
+    if name == "llama_1layer_8x8":
+        # alias the edges of every second node with the same strategies on both sides as an earlier one
+        from autoparallel_amd.packed import EDGE_HAS_PRODUCER
+
+        seen, alias = {}, np.arange(g.num_edges, dtype=np.int64)
+        for e in range(g.num_edges):
+            key = (int(g.edge_dst_list[e]), int(g.edge_src_list[e]), int(g.edge_sdst[e]), int(g.edge_ssrc[e]),
+                   int(g.edge_flags[e]) & EDGE_HAS_PRODUCER, int(g.edge_default_off[e]) < 0)
+            if key[5] and key in seen:
+                alias[e] = seen[key]
+            else:
+                seen.setdefault(key, e)
+        assert (alias != np.arange(g.num_edges)).sum() > 10
+        g = g.with_edge_alias(alias)
+    print(f"  compact: {name} E={g.num_entries} slots={g.num_slots}", flush=True)
+    assert g.num_slots > g.num_entries
+    eng = engine_mod.CostEngine(g).build(clamp_inf=True)
+    padded, packed = eng.results(), eng.results(compact=True)
+    slots = g.entry_slots()
+    for k in ("comm", "cost"):
+        assert packed[k].shape == (g.num_entries,) and bits_equal(packed[k], padded[k][slots]), k
+    assert np.array_equal(packed["flags"], padded["flags"][slots])
+    for k in ("compute", "per_arg"):
+        assert bits_equal(packed[k], padded[k])

@@ -312,7 +312,10 @@ def test_programs_of_the_traced_llama3_8b_graph():
         checked_einsum, _ = _check_programs_of(gm, mesh)
     print(dict(checked))
     families = {"aten.mm.default", "aten.embedding.default", "aten.mean.dim", "aten.sum.dim_IntList",
-                "aten._to_copy.default", "aten.silu.default", "aten.mul.Tensor", "aten.rsqrt.default"}
+                "aten._to_copy.default", "aten.silu.default", "aten.mul.Tensor", "aten.rsqrt.default",
+                # zero-flop operators whose output size is not that of an argument
+                "aten.cat.default", "aten.slice_backward.default", "aten.nll_loss_forward.default",
+                "aten.nll_loss_backward.default", "aten.embedding_dense_backward.default"}
     assert families <= set(checked), families - set(checked)
     assert "aten.einsum.default" in checked_einsum and "aten.mm.default" not in checked_einsum
     # 32 query heads on 8 key/value heads: the flop counter the reference relies on has no

@@ -423,3 +423,51 @@ def test_every_entry_point_refuses_a_problem_it_could_not_walk():
         for what, first in (("null", None), ("empty", ctypes.byref(empty)), ("no arrays", ctypes.byref(no_arrays))):
             rc = call(name, args, first)
             assert rc < 0 and lib.apc_last_error(), (name, what, rc)
+
+
+def test_templates_pack_like_nodes_described_one_by_one():
+    """GraphBuilder.add_template / add_instance (one description shared by the
+    repeated nodes of a model, default rows asked through a callback) give the
+    arrays that add_node gives for the same nodes, field by field."""
+    import dataclasses
+
+    from autoparallel_amd import graphgen
+    from autoparallel_amd.packed import GraphBuilder, PackedGraph
+
+    class Recorder(GraphBuilder):
+        made = []
+
+        def __init__(self, *a, **k):
+            super().__init__(*a, **k)
+            Recorder.made.append(self)
+
+    saved, graphgen.GraphBuilder = graphgen.GraphBuilder, Recorder
+    try:
+        want = graphgen.llama_graph((2, 4), 3, 256, 8, 4, 512, 1024, 128, 16)
+    finally:
+        graphgen.GraphBuilder = saved
+    src = Recorder.made[-1]
+    # the same nodes again: a template per distinct description (by content), an instance per node
+    b = GraphBuilder(src.mesh_shape, src.devices_per_host)
+    b._metas, b._meta_rows = dict(src._metas), list(src._meta_rows)
+    b._tuples, b._tuple_rows = dict(src._tuples), list(src._tuple_rows)
+    b.prefetchable_edges, b.multiplier = set(src.prefetchable_edges), dict(src.multiplier)
+    templates, rows = {}, {}
+    for v, nd in enumerate(src.nodes):
+        key = (tuple(map(tuple, nd.in_specs)), tuple(map(tuple, nd.out_specs)), nd.op,
+               None if nd.program is None else tuple(nd.program), nd.tuple_output, nd.nargs,
+               None if nd.default_rows is None else len(nd.default_rows[0]))
+        if key not in templates:
+            templates[key] = b.add_template(nd)
+        b.add_instance(templates[key], nd.inputs, nd.getitem_index, nd.name)
+        rows[v] = nd.default_rows
+    assert len(templates) < len(src.nodes) // 2
+    got = b.pack(default_rows_of=rows.get)
+    for f in dataclasses.fields(PackedGraph):
+        if f.name in ("roles", "node_kind", "node_phase", "node_cluster_key"):  # the generator sets these after packing
+            continue
+        x, y = getattr(got, f.name), getattr(want, f.name)
+        if isinstance(y, np.ndarray):
+            assert x.dtype == y.dtype and x.shape == y.shape and x.tobytes() == y.tobytes(), f.name
+        else:
+            assert x == y, f.name
