@@ -640,6 +640,7 @@ pair_table_kernel(apc_problem p, double* __restrict__ table) {
 // Kernel: cost entries
 // ---------------------------------------------------------------------------
 constexpr int kPerLane = 4;  // entries per lane of a work item of APC_ITEM_ENTRIES entries
+constexpr unsigned kXcdRun = 64;  // consecutive workgroups of wide items that share an XCD
 static_assert(sizeof(apc_edge) == 64, "edge record layout");
 static_assert(64 * kPerLane == APC_ITEM_ENTRIES, "work items are built for this kernel");
 
@@ -804,11 +805,22 @@ __device__ __forceinline__ void item_store(const apc_edge& ed, const ItemLoads<k
     if (clamp_inf && !finite) c = 10000.0;
     if ((r.live >> k) & 1) {
       const int64_t idx = ed.off + r.lk[k];
-      if (comm) comm[idx] = cm;
-      if (cost) cost[idx] = c;
-      // byte stores: gathering a lane's four flags into one 4-byte store through
-      // cross-lane exchanges measured slower
-      if (flags) flags[idx] = (uint8_t)(trans | (finite ? 0 : APC_ENTRY_NONFINITE));
+      const uint8_t f = (uint8_t)(trans | (finite ? 0 : APC_ENTRY_NONFINITE));
+      if (kN > kPerLane) {
+        // Wide items are for outputs that stream past every cache: stored as such they
+        // leave the block table in L2 (measured at 418 M entries: 1.39 -> 1.33 ms, with
+        // the workgroup order below 1.21 ms; on the 5.5 M entries of the headline graph
+        // the same stores cost 2 us of 19, which is why narrow items keep plain ones).
+        if (comm) __builtin_nontemporal_store(cm, comm + idx);
+        if (cost) __builtin_nontemporal_store(c, cost + idx);
+        if (flags) __builtin_nontemporal_store(f, flags + idx);
+      } else {
+        if (comm) comm[idx] = cm;
+        if (cost) cost[idx] = c;
+        // byte stores: gathering a lane's four flags into one 4-byte store through
+        // cross-lane exchanges measured slower
+        if (flags) flags[idx] = f;
+      }
     }
   }
 }
@@ -823,7 +835,18 @@ edge_cost_kernel(apc_problem p, const double* __restrict__ table,
                  const double* __restrict__ per_arg, double* __restrict__ comm,
                  double* __restrict__ cost, uint8_t* __restrict__ flags, int clamp_inf) {
   const int n_waves = gridDim.x * (kBlock / 64);
-  const int w = __builtin_amdgcn_readfirstlane((int)(blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6)));
+  // Workgroup b runs on XCD b mod 8, each with an L2 of its own.  With wide items
+  // (large problems) a run of kXcdRun consecutive workgroups' worth of items goes to
+  // one XCD, so that the items of an edge block, which read one matrix of the block
+  // table, mostly share an L2 instead of fetching it into all eight; the eight XCDs
+  // still write neighbouring runs (1 MB of costs each), which keeps the store stream
+  // compact.  The launcher rounds the grid up to whole groups of 8 runs.
+  unsigned wg = blockIdx.x;
+  if (kN > kPerLane) {
+    const unsigned k = wg >> 3, xcd = wg & 7;
+    wg = ((k / kXcdRun) * 8 + xcd) * kXcdRun + (k % kXcdRun);
+  }
+  const int w = __builtin_amdgcn_readfirstlane((int)(wg * (kBlock / 64) + (threadIdx.x >> 6)));
   const int lane = threadIdx.x & 63;
   if (kMode == 0) {
     for (int i = w; i < p.n_item; i += n_waves) {
@@ -1040,6 +1063,7 @@ static int launch_edge_costs(const apc_problem* p, const double* table, const do
   const unsigned cap = table ? (1u << 22) : (1u << 14);
   if (grid > cap) grid = cap;
   const bool wide = p->item_entries == 2 * APC_ITEM_ENTRIES;
+  if (wide) grid = (grid + 8 * kXcdRun - 1) / (8 * kXcdRun) * (8 * kXcdRun);  // whole groups of runs: see the kernel
   if (wide && !table)
     return fail(APC_ERR_INVALID, "apc_edge_costs: work items of 512 entries need a block table%s");
 #define APC_LAUNCH_EDGE(MODE, N)                                                                   \
