@@ -148,6 +148,10 @@ class ApcProblem(C.Structure):
         ("spec_recs", C.c_void_p),
         ("n_prog_term", C.c_int64),
         ("prog_terms", C.c_void_p),
+        ("lut_table_tiles", C.c_void_p),
+        ("n_lut_table_tile", C.c_int64),
+        ("lut_entry_tiles", C.c_void_p),
+        ("n_lut_entry_tile", C.c_int64),
     ]
 
 
@@ -297,7 +301,7 @@ EXPORTED_SYMBOLS = tuple(_SIGNATURES)
 _lib = None
 
 
-ABI_VERSION = 3  # apc_version() of the library whose struct layouts this module mirrors
+ABI_VERSION = 4  # apc_version() of the library whose struct layouts this module mirrors
 
 
 class ApcError(RuntimeError):

@@ -64,6 +64,12 @@ int validate_problem(const apc_problem* p) {
     return fail(APC_ERR_INVALID, "max_rank / max_node_args out of range%s");
   if (p->n_prog_term < 0 || (p->n_prog_term > 0 && !p->prog_terms))
     return fail(APC_ERR_INVALID, "n_prog_term without prog_terms%s");
+  if (p->n_lut_table_tile < 0 || p->n_lut_table_tile > 0x7FFFFFFF || p->n_lut_entry_tile < 0 ||
+      p->n_lut_entry_tile > 0x7FFFFFFF || (p->n_lut_table_tile > 0 && !p->lut_table_tiles) ||
+      (p->n_lut_entry_tile > 0 && !p->lut_entry_tiles))
+    return fail(APC_ERR_INVALID, "bad lookup-table tile lists%s");
+  if ((p->n_lut_table_tile > 0 || p->n_lut_entry_tile > 0) && !p->spec_recs)
+    return fail(APC_ERR_INVALID, "lookup-table tiles need apc_problem.spec_recs%s");
   return 0;
 }
 
@@ -890,6 +896,10 @@ calibration_copy_kernel(const double2_t* __restrict__ src, double2_t* __restrict
 int launch_prepare(const apc_problem* p, double* table, bool do_nodes, double* compute,
                    double* per_arg, int32_t* status, hipStream_t stream) {
   int table_blocks = (table && p->table_size > 0) ? p->n_table_unit : 0;
+  if (table_blocks > 0 && p->n_lut_table_tile > 0) {  // tile by tile, per-source terms in LDS (lut.hip)
+    if (int rc = apc_impl::launch_lut_table(p, table, stream)) return rc;
+    table_blocks = 0;
+  }
   if (table_blocks > kFusedTableBlocks) {  // a launch of its own: see pair_table_kernel
     hipLaunchKernelGGL(pair_table_kernel, dim3(table_blocks), dim3(256), 0, stream, *p, table);
     if (int rc = check_launch("pair_table_kernel")) return rc;
@@ -929,7 +939,7 @@ int launch_prepare(const apc_problem* p, double* table, bool do_nodes, double* c
 
 extern "C" {
 
-int apc_version(void) { return 3; }
+int apc_version(void) { return 4; }
 
 const char* apc_last_error(void) { return g_err; }
 
@@ -1056,6 +1066,8 @@ static int launch_edge_costs(const apc_problem* p, const double* table, const do
   if (int rc = validate_problem(p)) return rc;
   if (p->n_entry == 0) return 0;
   if (!per_arg) return fail(APC_ERR_INVALID, "apc_edge_costs: null per_arg%s");
+  if (!table && p->n_lut_entry_tile > 0)  // direct evaluation by tiles (lut.hip), same bits
+    return apc_impl::launch_lut_entries(p, per_arg, comm, cost, flags, clamp_inf, stream, start, stop);
   unsigned grid = (unsigned)((p->n_item + (kBlock / 64) - 1) / (kBlock / 64));
   // Measured on MI355X: the table kernel (8 waves per SIMD) is fastest with one
   // wave per item, the direct kernel (4 per SIMD, long-lived waves) with a few

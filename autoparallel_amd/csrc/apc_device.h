@@ -27,6 +27,11 @@ APC_HIDDEN int grid_for(int64_t total, int block);
 APC_HIDDEN int slot_grid(const apc_problem* p, int per_block, unsigned* grid);
 // The two events of a timer's slot (apc_timer_create); false for a bad timer or slot.
 APC_HIDDEN bool timer_events(void* timer, int slot, hipEvent_t* start, hipEvent_t* stop);
+// The lookup-table kernels over the problem's own tile lists (lut.hip).
+APC_HIDDEN int launch_lut_table(const apc_problem* p, double* table, hipStream_t stream);
+APC_HIDDEN int launch_lut_entries(const apc_problem* p, const double* per_arg, double* comm, double* cost,
+                                  uint8_t* flags, int clamp_inf, hipStream_t stream, hipEvent_t start,
+                                  hipEvent_t stop);
 }  // namespace apc_impl
 
 namespace {

@@ -323,6 +323,21 @@ int check_tiles(const apc_problem* p, const apc_lut_tile* tiles, int64_t n_tile,
 
 }  // namespace
 
+namespace apc_impl {
+// The problem's own tile lists, for the entry points that take no list (apc.hip).
+int launch_lut_table(const apc_problem* p, double* table, hipStream_t stream) {
+  launch_lut<false>(p, p->lut_table_tiles, p->n_lut_table_tile, table, nullptr, nullptr, nullptr, nullptr, 0, stream);
+  return check_launch("lut_kernel<table>");
+}
+
+int launch_lut_entries(const apc_problem* p, const double* per_arg, double* comm, double* cost, uint8_t* flags,
+                       int clamp_inf, hipStream_t stream, hipEvent_t start, hipEvent_t stop) {
+  launch_lut<true>(p, p->lut_entry_tiles, p->n_lut_entry_tile, nullptr, per_arg, comm, cost, flags, clamp_inf, stream,
+                   start, stop);
+  return check_launch("lut_kernel<entries>");
+}
+}  // namespace apc_impl
+
 extern "C" {
 
 int apc_build_pair_table_lut(const apc_problem* p, const apc_lut_tile* tiles, int64_t n_tile, double* table,

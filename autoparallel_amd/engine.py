@@ -301,11 +301,16 @@ class CostEngine:
         self.problem = p
         # Large tables, and direct evaluation, go through the lookup-table kernels:
         # tiles of whole matrices instead of one element per lane.
+        # The library takes that route by itself when the problem carries the tile list.
         self._lut_tiles = None
         self.lut = lut if lut is not None else (table_mode == "direct" or p.n_table_unit > _LUT_TABLE_FROM)
         if self.lut and g.num_entries > 0:
             tiles = g.lut_tiles(squeezed, entries=(table_mode == "direct"))
             self._lut_tiles = (up("lut_tiles", tiles), int(tiles.shape[0]))
+            if table_mode == "direct":
+                p.lut_entry_tiles, p.n_lut_entry_tile = self._lut_tiles
+            else:
+                p.lut_table_tiles, p.n_lut_table_tile = self._lut_tiles
         flush_uploads()
 
         E, NC = (g.num_slots, g.num_compute) if allocate_results else (0, 0)
@@ -392,21 +397,13 @@ class CostEngine:
 
     def prepare(self):
         """Pair table and node compute vectors, as build() makes them: one launch,
-        or, with the lookup-table kernels, the node launch and the table by tiles."""
-        if self._lut_tiles is None:
-            _lib.check(
-                self.lib.apc_prepare(
-                    C.byref(self.problem), self._ptr(self.table), self._ptr(self.compute),
-                    self._ptr(self.per_arg), self._ptr(self.status), self._stream()),
-                "apc_prepare",
-            )
-            return
-        p, table, compute, per_arg, status = self.build_args()[:5]
-        stream = torch.cuda.current_stream(self.device).cuda_stream
-        _lib.check(self.lib.apc_node_compute_costs(p, compute, per_arg, status, stream), "apc_node_compute_costs")
-        if self.use_table:
-            tiles, n_tile = self._lut_tiles
-            _lib.check(self.lib.apc_build_pair_table_lut(p, tiles, n_tile, table, stream), "apc_build_pair_table_lut")
+        or, with the lookup-table kernels, the table by tiles and the node launch."""
+        _lib.check(
+            self.lib.apc_prepare(
+                C.byref(self.problem), self._ptr(self.table), self._ptr(self.compute),
+                self._ptr(self.per_arg), self._ptr(self.status), self._stream()),
+            "apc_prepare",
+        )
 
     def build_args(self):
         if not self.can_build:
@@ -418,37 +415,19 @@ class CostEngine:
         return self._build_args
 
     def build(self, clamp_inf: bool = True):
-        """All coefficients: pair table and node compute vectors (one launch),
-        then the entry arrays (one launch)."""
+        """All coefficients: pair table and node compute vectors, then the entry
+        arrays (apc_build_all: two launches, three when the table is built by tiles)."""
         self._recs_valid = False
         # the argument list is the same from call to call apart from the stream:
         # made once, so that issuing a step costs less host time than the step takes
         args = self._build_args or self.build_args()
         stream = torch.cuda.current_stream(self.device).cuda_stream
-        if self._lut_tiles is None:
-            rc = self.lib.apc_build_all(*args, 1 if clamp_inf else 0, stream)
-            if rc:
-                _lib.check(rc, "apc_build_all")
-        else:
-            self._build_with_lut(1 if clamp_inf else 0, stream)
+        rc = self.lib.apc_build_all(*args, 1 if clamp_inf else 0, stream)
+        if rc:
+            _lib.check(rc, "apc_build_all")
         self.built = True
         self._table_clamp = (1 if clamp_inf else 0) if self.table is not None else None
         return self
-
-    def _build_with_lut(self, clamp_inf: int, stream) -> None:
-        """The same results through the lookup-table kernels: the block table tile
-        by tile, then the usual node and entry launches; or, without a table, the
-        entries themselves tile by tile."""
-        p, table, compute, per_arg, status, comm, cost, flags = self.build_args()
-        tiles, n_tile = self._lut_tiles
-        lib = self.lib
-        _lib.check(lib.apc_node_compute_costs(p, compute, per_arg, status, stream), "apc_node_compute_costs")
-        if self.use_table:
-            _lib.check(lib.apc_build_pair_table_lut(p, tiles, n_tile, table, stream), "apc_build_pair_table_lut")
-            _lib.check(lib.apc_edge_costs(p, table, per_arg, comm, cost, flags, clamp_inf, stream), "apc_edge_costs")
-        else:
-            _lib.check(lib.apc_edge_costs_lut(p, tiles, n_tile, per_arg, comm, cost, flags, clamp_inf, stream),
-                       "apc_edge_costs_lut")
 
     def build_timed(self, timer, slot: int, clamp_inf: bool = True):
         """build() with HIP events at the begin and end of the kernel that writes
@@ -457,22 +436,9 @@ class CostEngine:
         self.build_args()
         stream = torch.cuda.current_stream(self.device).cuda_stream
         clamp = 1 if clamp_inf else 0
-        if self._lut_tiles is None:
-            rc = self.lib.apc_build_all_timed(*self._build_args, clamp, timer, int(slot), stream)
-            if rc:
-                _lib.check(rc, "apc_build_all_timed")
-        else:
-            p, table, compute, per_arg, status, comm, cost, flags = self._build_args
-            tiles, n_tile = self._lut_tiles
-            lib = self.lib
-            _lib.check(lib.apc_node_compute_costs(p, compute, per_arg, status, stream), "apc_node_compute_costs")
-            if self.use_table:
-                _lib.check(lib.apc_build_pair_table_lut(p, tiles, n_tile, table, stream), "apc_build_pair_table_lut")
-                _lib.check(lib.apc_edge_costs_timed(p, table, per_arg, comm, cost, flags, clamp, timer, int(slot),
-                                                    stream), "apc_edge_costs_timed")
-            else:
-                _lib.check(lib.apc_edge_costs_lut_timed(p, tiles, n_tile, per_arg, comm, cost, flags, clamp, timer,
-                                                        int(slot), stream), "apc_edge_costs_lut_timed")
+        rc = self.lib.apc_build_all_timed(*self._build_args, clamp, timer, int(slot), stream)
+        if rc:
+            _lib.check(rc, "apc_build_all_timed")
         self._recs_valid = False
         self.built = True
         self._table_clamp = clamp if self.table is not None else None

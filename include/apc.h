@@ -320,9 +320,51 @@ typedef struct apc_problem {
   const apc_spec_rec* spec_recs;     /* [n_list]                                */
   int64_t n_prog_term;
   const apc_prog_term* prog_terms;   /* named by apc_comp_rec.term_off / n_term */
+  /* optional: tile lists for the lookup-table kernels (both need spec_recs).
+   * With lut_table_tiles (every matrix of the block table covered exactly once)
+   * apc_prepare / apc_build_pair_table / apc_build_all build the table tile by
+   * tile (lut_kernel<table>) instead of element by element; worth it from a few
+   * thousand table units on.  With lut_entry_tiles (every edge block that owns
+   * entries covered exactly once, edges without a producer included)
+   * apc_edge_costs / apc_build_all called with table == NULL evaluate the
+   * entries tile by tile (lut_kernel<entries>, three times the rate of the
+   * per-entry fold).  NULL: the element-by-element kernels, same bits. */
+  const struct apc_lut_tile* lut_table_tiles;
+  int64_t n_lut_table_tile;
+  const struct apc_lut_tile* lut_entry_tiles;
+  int64_t n_lut_entry_tile;
 } apc_problem;
 
-/* Version of the ABI (struct layouts and signatures of this header): 3. */
+/* What is checked, and what is the caller's to check.  Every entry point that
+ * takes an apc_problem checks sizes, counts and null pointers on the host and
+ * refuses what is inconsistent (APC_ERR_INVALID).  The CONTENTS of the index
+ * arrays are not read on the host (they live in device memory): chunk_edge,
+ * edges[].off / src_list / dst_list / default_off / table_off / comp_base, items,
+ * node_edge_off, node_comp_off, block_off, list_uidx / list_ufirst, the tile
+ * lists and the program words must name positions inside the arrays they index,
+ * or a kernel reads or writes outside them.  The Python packer validates all of
+ * them before it uploads (PackedGraph.validate); a C caller that fills the
+ * arrays itself owns that check.
+ *
+ * Which kernel an entry point launches (all on `stream`, asynchronously):
+ *   apc_prepare             prepare_kernel: table blocks + node blocks in one launch;
+ *                           tables of more than 2 048 units get pair_table_kernel of
+ *                           their own first; with lut_table_tiles the table is built
+ *                           by lut_kernel<table> instead (then prepare_kernel prices
+ *                           the nodes only)
+ *   apc_build_pair_table    the table part of the above alone
+ *   apc_node_compute_costs  the node part of the above alone
+ *   apc_edge_costs          with a table: edge_cost_kernel<1,n> (full matrices) or
+ *                           <2,n> (compressed: list_uidx set), n = 4 or 8 entries per
+ *                           lane by item_entries; table == NULL: lut_kernel<entries>
+ *                           when the problem carries lut_entry_tiles, else
+ *                           edge_cost_kernel<0,4>, the per-entry fold (the fallback
+ *                           for problems without spec_recs; a third of the rate)
+ *   apc_build_all           apc_prepare, then apc_edge_costs
+ *   apc_build_pair_table_lut / apc_edge_costs_lut   lut_kernel over a list passed as
+ *                           an argument instead of the problem's own
+ *
+ * Version of the ABI (struct layouts and signatures of this header): 4. */
 int apc_version(void);
 const char* apc_last_error(void);
 
@@ -464,9 +506,10 @@ int apc_prepare(const apc_problem* p, double* table, double* compute, double* pe
                 int32_t* status, void* stream);
 
 /* The three steps above in two launches (pair table and node estimates share
- * one): the whole of ShardingOptimizer._build_decision_vars' arithmetic
+ * one; three when the table is built by tiles): the whole of
+ * ShardingOptimizer._build_decision_vars' arithmetic
  * (autoparallel/optimize_sharding.py:481-552) in one call.  table may be NULL
- * (direct evaluation). */
+ * (direct evaluation: by tiles if the problem carries lut_entry_tiles). */
 int apc_build_all(const apc_problem* p, double* table, double* compute, double* per_arg,
                   int32_t* status, double* comm, double* cost, uint8_t* flags, int32_t clamp_inf,
                   void* stream);
@@ -480,7 +523,10 @@ int apc_build_all(const apc_problem* p, double* table, double* compute, double* 
  * apc_build_all, and the results are the same bit for bit.  Returns
  * APC_ERR_INVALID when p->table_size exceeds APC_NOALLOC_MAX_TABLE; with
  * table_size == 0 every entry is evaluated directly.  The call allocates
- * nothing (the first call on a device looks the array's address up).  Every
+ * nothing.  The first call on a device looks the array's address up
+ * (hipGetSymbolAddress) and sets a kernel attribute once: make one eager call
+ * per device before capturing calls into a HIP graph, where those two host
+ * calls may be refused.  Every
  * call on a GPU shares that GPU's array: calls that overlap on one GPU (two
  * streams, two threads) race; a build reads only the table elements it wrote
  * itself, so nothing needs clearing between calls. */

@@ -567,6 +567,60 @@ def test_lookup_table_kernels(CostEngine, name):
         assert ((got["flags"] & 1) == re_["transition"]).all()
 
 
+def test_build_all_takes_the_tile_route_from_the_problem(CostEngine):
+    """One build entry point: apc_build_all through the C ABI with table == NULL
+    evaluates by tiles when the problem carries lut_entry_tiles and entry by entry
+    when it does not, and with a table builds it by tiles when the problem carries
+    lut_table_tiles; the same bits each way, and as the entry points that take a
+    tile list as an argument."""
+    import ctypes as C
+
+    import torch
+
+    from autoparallel_amd import _lib
+
+    g = graphgen.stress_graph(200, (4, 8, 8), seed=11, s_min=8, s_max=160)
+    ref = O.GraphOracle(g).build()
+
+    def run(eng, table):
+        for t in (eng.comm, eng.cost, eng.flags):
+            t.zero_()
+        _lib.check(eng.lib.apc_build_all(
+            C.byref(eng.problem), table, eng._ptr(eng.compute), eng._ptr(eng.per_arg), eng._ptr(eng.status),
+            eng._ptr(eng.comm), eng._ptr(eng.cost), eng._ptr(eng.flags), 0, eng._stream()), "apc_build_all")
+        eng.built = True
+        return eng.results()
+
+    for lut in (True, False):
+        eng = CostEngine(g, table_mode="direct", lut=lut)
+        assert (eng.problem.n_lut_entry_tile > 0) == lut and eng.problem.n_lut_table_tile == 0
+        got = run(eng, None)
+        assert bits_equal(got["comm"], ref["comm"]) and bits_equal(got["cost"], ref["cost"]), lut
+        assert ((got["flags"] & 1) == ref["transition"]).all()
+    # the explicit entry point with the same list
+    eng = CostEngine(g, table_mode="direct", lut=True)
+    eng.node_compute()
+    tiles, n_tile = eng._lut_tiles
+    for t in (eng.comm, eng.cost, eng.flags):
+        t.zero_()
+    _lib.check(eng.lib.apc_edge_costs_lut(C.byref(eng.problem), tiles, n_tile, eng._ptr(eng.per_arg), eng._ptr(eng.comm),
+                                          eng._ptr(eng.cost), eng._ptr(eng.flags), 0, eng._stream()), "apc_edge_costs_lut")
+    eng.built = True
+    got = eng.results()
+    assert bits_equal(got["comm"], ref["comm"]) and bits_equal(got["cost"], ref["cost"])
+    for mode in ("full", "compressed"):
+        tables = []
+        for lut in (True, False):
+            eng = CostEngine(g, table_mode=mode, lut=lut)
+            assert (eng.problem.n_lut_table_tile > 0) == lut and eng.problem.n_lut_entry_tile == 0
+            eng.table.zero_()  # the padding between matrices is nobody's to write
+            got = run(eng, eng._ptr(eng.table))
+            assert bits_equal(got["comm"], ref["comm"]) and bits_equal(got["cost"], ref["cost"]), (mode, lut)
+            tables.append(eng.table.cpu().numpy())
+        assert bits_equal(tables[0], tables[1]), mode
+        torch.cuda.synchronize()
+
+
 def test_unsupported_dtype_reports(CostEngine):
     b = GraphBuilder((2,), 8)
     m = b.meta((8, 8), (8, 1), 8, packed.DT_OTHER)

@@ -61,3 +61,37 @@ def test_noalloc_build_refuses_a_table_beyond_the_static_array():
         eng._ptr(eng.comm), eng._ptr(eng.cost), eng._ptr(eng.flags), 1, eng._stream())
     assert rc == -1
     assert b"static scratch" in eng.lib.apc_last_error()
+
+
+def test_noalloc_build_of_a_problem_without_a_block_table():
+    """table_size == 0: every entry is evaluated directly, as apc_build_all does
+    with table == NULL; with and without the problem's tile list."""
+    import torch
+
+    from autoparallel_amd import _lib
+    from autoparallel_amd.engine import CostEngine
+
+    g = graphgen.stress_graph(60, (2, 4, 4), seed=3, s_max=48)
+    for lut in (False, True):
+        eng = CostEngine(g, table_mode="direct", lut=lut)
+        assert eng.table is None
+        # the problem as a caller without a block table describes it
+        eng.problem.table_size, eng.problem.n_table_unit, eng.problem.n_block = 0, 0, 0
+        assert (eng.problem.n_lut_entry_tile > 0) == lut
+        rc = eng.lib.apc_build_all(
+            C.byref(eng.problem), None, eng._ptr(eng.compute), eng._ptr(eng.per_arg), eng._ptr(eng.status),
+            eng._ptr(eng.comm), eng._ptr(eng.cost), eng._ptr(eng.flags), 1, eng._stream())
+        _lib.check(rc, "apc_build_all")
+        eng.built = True
+        want = {k: v.copy() for k, v in eng.results().items()}
+        for t in (eng.comm, eng.cost, eng.flags, eng.compute, eng.per_arg, eng.status):
+            t.zero_()
+        torch.cuda.synchronize()
+        rc = eng.lib.apc_build_all_noalloc(
+            C.byref(eng.problem), eng._ptr(eng.compute), eng._ptr(eng.per_arg), eng._ptr(eng.status),
+            eng._ptr(eng.comm), eng._ptr(eng.cost), eng._ptr(eng.flags), 1, eng._stream())
+        _lib.check(rc, "apc_build_all_noalloc")
+        got = eng.results()
+        for k in ("comm", "cost", "compute", "per_arg"):
+            assert (got[k].view(np.uint64) == want[k].view(np.uint64)).all(), (lut, k)
+        assert (got["flags"] == want["flags"]).all()
