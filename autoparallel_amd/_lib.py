@@ -252,6 +252,11 @@ _SIGNATURES = {
         [C.POINTER(ApcProblem), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint64,
          C.c_int64, C.c_int64, C.c_void_p, C.c_void_p]),
     "apc_random_assignment": (C.c_uint32, [C.c_uint64, C.c_int64, C.c_int32, C.c_int32]),
+    "apc_sample_feasible": (
+        C.c_int,
+        [C.POINTER(ApcProblem), C.c_void_p, C.c_uint64, C.c_int64, C.c_int64, C.c_void_p, C.c_int32, C.c_void_p,
+         C.c_void_p, C.c_void_p]),
+    "apc_sample_takes": (C.c_int32, [C.c_uint64, C.c_int64, C.c_int32, C.c_uint32]),
     "apc_local_shapes": (
         C.c_int,
         [C.POINTER(ApcModel), C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,

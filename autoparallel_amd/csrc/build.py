@@ -23,7 +23,7 @@ HIPCC_FLAGS = [
 
 
 def build(verbose: bool = True) -> str:
-    srcs = [os.path.join(HERE, f) for f in ("apc.hip", "lut.hip", "score.hip", "passes.hip", "schedule.hip", "nccl_plan.cpp")]
+    srcs = [os.path.join(HERE, f) for f in ("apc.hip", "lut.hip", "score.hip", "sample.hip", "passes.hip", "schedule.hip", "nccl_plan.cpp")]
     cmd = ["hipcc"] + HIPCC_FLAGS + srcs + ["-o", LIB]
     if verbose:
         print(" ".join(cmd), flush=True)

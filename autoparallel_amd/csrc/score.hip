@@ -395,10 +395,15 @@ score_compact_kernel(apc_problem p, const double* __restrict__ per_arg,
 // score_kernel: same results, bit for bit, as scoring the entry arrays that a
 // build with the same clamp_inf wrote.
 // ---------------------------------------------------------------------------
-constexpr int kTableBlock = 1024;
-constexpr int kTileDoubles = 8192;  // 64 KB: four 16-byte loads per lane
-constexpr int kListInts = 1024;     // one 4-byte load per lane
-constexpr int kTableLds = 2 * kTileDoubles * 8 + 4 * kListInts * 4;  // 144 KB
+constexpr int kTileDoubles = 8192;  // 64 KB: a tile of a matrix
+constexpr int kListInts = 1024;     // an index list that goes through LDS
+constexpr int kLanes = 1024;        // one workgroup per CU
+constexpr int kBufs = 2;            // tile buffers: the next edge's matrix arrives while the lanes draw from this one
+constexpr int kTableLds = kBufs * kTileDoubles * 8 + kBufs * 2 * kListInts * 4;  // 144 KB
+// Measured on a 3 000-node window of the stress DAG, 2^20 assignments, where this shape
+// takes 18.3 ms: two workgroups of 512 lanes per CU with one buffer each, which overlap
+// each other instead of prefetching, 24.4 ms; a quarter of the waves (by turns) issuing
+// the whole copy while the others go on to their draws, 25.0 ms.
 
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 
@@ -408,39 +413,52 @@ typedef __attribute__((address_space(3))) void* lds_ptr_t;
 // tell these LDS writes from the LDS reads of the draws, would wait for it before the
 // next LDS read, and the point is that it stays in flight while the lanes draw from
 // the other buffer.  So the compiler does not count it either: the code that needs
-// the data waits with s_waitcnt vmcnt(0) itself.  (Loads complete in order, so the
+// the data waits for the vector-memory counter itself.  (Loads complete in order, so the
 // compiler's own counts for its own loads only ever wait longer than they must.)
+// m0 holds the LDS address for the load; the compiler keeps m0 for its own uses
+// (it is a reserved register, which a clobber list cannot name), so the statement
+// puts back what it found there.
 __device__ __forceinline__ void copy16_to_lds(const double2_t* __restrict__ src, uint32_t lds_wave, int i, int n) {
   if (i < n) {
     const uint32_t m = __builtin_amdgcn_readfirstlane(lds_wave);
     const double2_t* g = src + i;
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 3\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(m), "v"(g) : "memory");
+    uint32_t saved;
+    asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %1\n\ts_nop 3\n\tglobal_load_lds_dwordx4 %2, off\n\ts_mov_b32 m0, %0"
+                 : "=&s"(saved) : "s"(m), "v"(g) : "memory");
   }
 }
 __device__ __forceinline__ void copy4_to_lds(const int32_t* __restrict__ src, uint32_t lds_wave, int i, int n) {
   if (i < n) {
     const uint32_t m = __builtin_amdgcn_readfirstlane(lds_wave);
     const int32_t* g = src + i;
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 3\n\tglobal_load_lds_dword %1, off" ::"s"(m), "v"(g) : "memory");
+    uint32_t saved;
+    asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %1\n\ts_nop 3\n\tglobal_load_lds_dword %2, off\n\ts_mov_b32 m0, %0"
+                 : "=&s"(saved) : "s"(m), "v"(g) : "memory");
   }
 }
 
+// Every vector-memory operation of this wave has completed (the copies into LDS
+// among them); scalar loads requested ahead (the next edge's and node's records)
+// stay in flight.  s_waitcnt fields of gfx9: vmcnt [3:0] and [15:14], expcnt [6:4],
+// lgkmcnt [11:8].
+__device__ __forceinline__ void wait_vector_memory() { __builtin_amdgcn_s_waitcnt(0x0F70); }
+
 template <bool kRandom, int kPer>
-__global__ void __launch_bounds__(kTableBlock)
+__global__ void __launch_bounds__(kLanes)
 score_table_kernel(apc_problem p, const double* __restrict__ per_arg, const double* __restrict__ table,
                    const apc_score_edge_aux* __restrict__ edge_aux,
                    const uint16_t* __restrict__ assign, int64_t stride, uint64_t seed, int64_t first,
                    int64_t n_assign, const int32_t* __restrict__ node_gid, int first_node, int end_node,
                    int clamp_inf, const double* __restrict__ init, double* __restrict__ out) {
   extern __shared__ __align__(16) double s_all[];
-  // [2][kTileDoubles] doubles, then [2][2][kListInts] ints
-  int32_t* const s_lists = reinterpret_cast<int32_t*>(s_all + 2 * kTileDoubles);
+  // [kBufs][kTileDoubles] doubles, then [kBufs][2][kListInts] ints
+  int32_t* const s_lists = reinterpret_cast<int32_t*>(s_all + kBufs * kTileDoubles);
   const int tid = threadIdx.x;
   const int wave0 = tid & ~63;
   const uint32_t lds_mat = (uint32_t)(uintptr_t)(lds_ptr_t)s_all;  // byte addresses inside LDS
-  const uint32_t lds_lists = lds_mat + 2 * kTileDoubles * 8;
-  const int64_t lanes = (int64_t)gridDim.x * kTableBlock;
-  const int64_t t_raw = (int64_t)blockIdx.x * kTableBlock + tid;
+  const uint32_t lds_lists = lds_mat + kBufs * kTileDoubles * 8;
+  const int64_t lanes = (int64_t)gridDim.x * kLanes;
+  const int64_t t_raw = (int64_t)blockIdx.x * kLanes + tid;
   const int64_t t = t_raw < n_assign ? t_raw : 0;  // no lane leaves early: the workgroup meets at barriers
   // assignment k of this lane; a lane past the end repeats another one and stores nothing
   auto asg = [&](int k) -> int64_t {
@@ -486,18 +504,33 @@ score_table_kernel(apc_problem p, const double* __restrict__ per_arg, const doub
     const int n = msize - base < kTileDoubles ? msize - base : kTileDoubles;
     const double2_t* __restrict__ src2 = reinterpret_cast<const double2_t*>(table + x.table_off + base);
 #pragma unroll
-    for (int r = 0; r < kTileDoubles / 2 / kTableBlock; ++r)
-      copy16_to_lds(src2, lds_mat + (uint32_t)(b * kTileDoubles + 2 * (r * kTableBlock + wave0)) * 8u,
-                    r * kTableBlock + tid, n >> 1);
+    for (int r = 0; r < kTileDoubles / 2 / kLanes; ++r)
+      copy16_to_lds(src2, lds_mat + (uint32_t)(b * kTileDoubles + 2 * (r * kLanes + wave0)) * 8u,
+                    r * kLanes + tid, n >> 1);
     if (base == 0 && lists_staged(x)) {
-      copy4_to_lds(p.list_uidx + x.dst_list, lds_lists + (uint32_t)((b * 2 + 0) * kListInts + wave0) * 4u, tid, x.sdst);
-      copy4_to_lds(p.list_uidx + x.src_list, lds_lists + (uint32_t)((b * 2 + 1) * kListInts + wave0) * 4u, tid, x.ssrc);
+#pragma unroll
+      for (int r = 0; r < kListInts / kLanes; ++r) {
+        copy4_to_lds(p.list_uidx + x.dst_list, lds_lists + (uint32_t)((b * 2 + 0) * kListInts + r * kLanes + wave0) * 4u,
+                     r * kLanes + tid, x.sdst);
+        copy4_to_lds(p.list_uidx + x.src_list, lds_lists + (uint32_t)((b * 2 + 1) * kListInts + r * kLanes + wave0) * 4u,
+                     r * kLanes + tid, x.ssrc);
+      }
     }
   };
   const int e_begin = first_node < end_node ? p.node_edge_off[first_node] : 0;
   const int e_end = first_node < end_node ? p.node_edge_off[end_node] : 0;
   // The record of an edge and what else the walk needs to know about it (apc_score_edge_aux)
-  // are requested one edge ahead, so that an edge starts with everything in scalar registers.
+  // are requested one edge ahead, and what it needs to know about a node one node ahead, so
+  // that an edge and a node start with everything in scalar registers.
+  struct NodeInfo { int nstrat, nargs, mult, gid, e_end; int64_t comp_off; };
+  auto load_node = [&](int v) -> NodeInfo {
+    NodeInfo n;
+    n.nstrat = p.node_nstrat[v]; n.nargs = p.node_nargs[v]; n.mult = p.node_multiplier[v];
+    n.gid = node_gid ? node_gid[v] : v; n.e_end = p.node_edge_off[v + 1]; n.comp_off = p.node_comp_off[v];
+    return n;
+  };
+  NodeInfo node_nxt = {1, 1, 1, 0, 0, 0};
+  if (first_node < end_node) node_nxt = load_node(first_node);
   apc_edge nxt;
   apc_score_edge_aux aux_nxt = {0, -1, 0, 0};
   if (e_begin < e_end) {
@@ -510,22 +543,20 @@ score_table_kernel(apc_problem p, const double* __restrict__ per_arg, const doub
     if (s0 >= 0 && s0 < e_end)
       issue(s0 == e_begin ? nxt : load_edge(p.edges + s0), s0 == e_begin ? aux_nxt.msize : edge_aux[s0].msize, 0, buf);
   }
+  int e = e_begin;
   for (int v = first_node; v < end_node; ++v) {
-    const int nstrat = p.node_nstrat[v];
-    const int nargs = p.node_nargs[v];
-    const double fargs = (double)(nargs > 1 ? nargs : 1);
-    const double mult = (double)p.node_multiplier[v];
-    const int64_t comp_off = p.node_comp_off[v];
+    const NodeInfo node = node_nxt;
+    if (v + 1 < end_node) node_nxt = load_node(v + 1);
+    const double fargs = (double)(node.nargs > 1 ? node.nargs : 1);
+    const double mult = (double)node.mult;
     uint32_t o[kPer];
     double pa[kPer];
 #pragma unroll
     for (int k = 0; k < kPer; ++k) {
-      o[k] = choice(k, v, node_gid ? node_gid[v] : v, nstrat);
-      pa[k] = per_arg[comp_off + o[k]];
+      o[k] = choice(k, v, node.gid, node.nstrat);
+      pa[k] = per_arg[node.comp_off + o[k]];  // first needed when the node's first edge has drawn
     }
-#pragma unroll
-    for (int k = 0; k < kPer; ++k) t_compute[k] += pa[k] * fargs;
-    for (int e = p.node_edge_off[v]; e < p.node_edge_off[v + 1]; ++e) {
+    for (; e < node.e_end; ++e) {
       const apc_edge ed = nxt;
       const apc_score_edge_aux aux = aux_nxt;
       if (e + 1 < e_end) nxt = load_edge(p.edges + e + 1);
@@ -540,9 +571,9 @@ score_table_kernel(apc_problem p, const double* __restrict__ per_arg, const doub
       double raw[kPer];
       if (msize > 0) {  // uniform over the workgroup, as everything that decides a barrier below
         const double* const mat = s_all + buf * kTileDoubles;
-        __builtin_amdgcn_s_waitcnt(0);  // this lane's part of the first tile has arrived,
-        __syncthreads();                // and everyone's; and the draws of the edge before are done,
-        {                               // so its buffer can take the next matrix
+        wait_vector_memory();  // this lane's part of the first tile has arrived,
+        __syncthreads();       // and everyone's; and the draws of the edge before are done,
+        {                      // so its buffer can take the next matrix
           const int s1 = aux_nxt.next_staged;
           if (s1 >= 0 && s1 < e_end)
             issue(s1 == e + 1 ? nxt : load_edge(p.edges + s1), s1 == e + 1 ? aux_nxt.msize : edge_aux[s1].msize, 0,
@@ -573,7 +604,7 @@ score_table_kernel(apc_problem p, const double* __restrict__ per_arg, const doub
           if (base >= msize) break;
           __syncthreads();  // the draws from this tile are done
           issue(ed, msize, base, buf);
-          __builtin_amdgcn_s_waitcnt(0);
+          wait_vector_memory();
           __syncthreads();
         }
         buf ^= 1;
@@ -605,6 +636,10 @@ score_table_kernel(apc_problem p, const double* __restrict__ per_arg, const doub
         n_trans[k] += count_trans ? trans : 0u;
       }
     }
+    // the node's own term, added where its compute terms have long arrived (nothing else
+    // is added to this sum in between, so its order is the walk's)
+#pragma unroll
+    for (int k = 0; k < kPer; ++k) t_compute[k] += pa[k] * fargs;
   }
   __builtin_amdgcn_s_waitcnt(0);  // nothing is in flight towards LDS when the workgroup ends
   // x + 1.0 n times over.  While x is a whole number below 2^52 every step is exact, and so
@@ -635,7 +670,7 @@ score_table_kernel(apc_problem p, const double* __restrict__ per_arg, const doub
 }
 
 template <bool kRandom, int kPer>
-int launch_table_k(dim3 grid, hipStream_t stream, const apc_problem& p, const double* per_arg, const double* table,
+int launch_table_k(int64_t lanes, hipStream_t stream, const apc_problem& p, const double* per_arg, const double* table,
                    const apc_score_edge_aux* edge_aux, const uint16_t* assign, int64_t stride,
                    uint64_t seed, int64_t first, int64_t n_assign, const int32_t* node_gid, int first_node,
                    int end_node, int clamp_inf, const double* init, double* out) {
@@ -643,7 +678,8 @@ int launch_table_k(dim3 grid, hipStream_t stream, const apc_problem& p, const do
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(score_table_kernel<kRandom, kPer>),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, kTableLds);
   if (e != hipSuccess) return fail(APC_ERR_LAUNCH, "hipFuncSetAttribute(score_table_kernel): %s", hipGetErrorString(e));
-  hipLaunchKernelGGL((score_table_kernel<kRandom, kPer>), grid, dim3(kTableBlock), kTableLds, stream, p, per_arg,
+  const dim3 grid((unsigned)((lanes + kLanes - 1) / kLanes));
+  hipLaunchKernelGGL((score_table_kernel<kRandom, kPer>), grid, dim3(kLanes), kTableLds, stream, p, per_arg,
                      table, edge_aux, assign, stride, seed, first, n_assign, node_gid, first_node,
                      end_node, clamp_inf, init, out);
   return check_launch("score_table_kernel");
@@ -925,19 +961,18 @@ int apc_score_table(const apc_problem* p, const double* per_arg, const double* t
     return fail(APC_ERR_INVALID, "apc_score_table: need 0 <= first_node <= end_node <= n_node%s");
   if (per_lane != 0 && per_lane != 1 && per_lane != 2 && per_lane != 4)
     return fail(APC_ERR_INVALID, "apc_score_table: per_lane must be 0 (choose), 1, 2 or 4%s");
-  // 262144 lanes are one workgroup on each of the 256 CUs; four assignments a lane is
-  // what the registers of that many waves allow.
-  const int64_t kLanes = 262144;
-  for (int64_t a0 = 0; a0 < n_assign; a0 += kLanes * 4) {
-    const int64_t n = (n_assign - a0 < kLanes * 4) ? (n_assign - a0) : kLanes * 4;
-    const int per = per_lane ? per_lane : n <= kLanes ? 1 : n <= 2 * kLanes ? 2 : 4;
+  // 262144 lanes are one workgroup of 1024 on each of the 256 CUs; four
+  // assignments a lane is what the registers of that many waves allow.
+  const int64_t kResident = 262144;
+  for (int64_t a0 = 0; a0 < n_assign; a0 += kResident * 4) {
+    const int64_t n = (n_assign - a0 < kResident * 4) ? (n_assign - a0) : kResident * 4;
+    const int per = per_lane ? per_lane : n <= kResident ? 1 : n <= 2 * kResident ? 2 : 4;
     const int64_t lanes = (n + per - 1) / per;
-    const dim3 grid((unsigned)((lanes + kTableBlock - 1) / kTableBlock));
     const double* in = init ? init + a0 * 6 : nullptr;
-    int rc = assign ? launch_table<false>(per, grid, (hipStream_t)stream, *p, per_arg, table, edge_aux,
+    int rc = assign ? launch_table<false>(per, lanes, (hipStream_t)stream, *p, per_arg, table, edge_aux,
                                           assign + a0, n_assign, seed, first + a0, n, node_gid, (int)first_node,
                                           (int)end_node, (int)clamp_inf, in, out + a0 * 6)
-                    : launch_table<true>(per, grid, (hipStream_t)stream, *p, per_arg, table, edge_aux,
+                    : launch_table<true>(per, lanes, (hipStream_t)stream, *p, per_arg, table, edge_aux,
                                          assign, n_assign, seed, first + a0, n, node_gid, (int)first_node,
                                          (int)end_node, (int)clamp_inf, in, out + a0 * 6);
     if (rc) return rc;

@@ -717,6 +717,31 @@ class CostEngine:
         )
         return out
 
+    def sample_feasible(self, seed: int, first: int, count: int, node_gid: Optional[np.ndarray] = None,
+                        first_node: int = 0, assign: Optional[torch.Tensor] = None):
+        """``count`` assignments drawn node by node among the strategies that select
+        no forbidden (non-finite) entry against the choices made for the node's
+        producers (apc_sample_feasible).  Returns (assign uint16[n_node, count] on
+        the device, n_fallback int32[count]: nodes that had no such strategy and
+        took the plain draw).  ``assign``/``first_node``: rows below first_node are
+        given (a window of a larger graph); ``node_gid``: ids for the hashes."""
+        assert self.built
+        N = self.g.num_nodes
+        if assign is None:
+            assert first_node == 0
+            assign = torch.empty((N, count), dtype=torch.uint16, device=self.device)
+        assert assign.shape == (N, count) and assign.dtype == torch.uint16 and assign.is_contiguous()
+        d_gid = None
+        if node_gid is not None:
+            d_gid = torch.from_numpy(np.ascontiguousarray(node_gid, np.int32)).to(self.device)
+        fallback = torch.empty(count, dtype=torch.int32, device=self.device)
+        _lib.check(
+            self.lib.apc_sample_feasible(
+                C.byref(self.problem), self._ptr(self.flags), int(seed), int(first), int(count), self._ptr(d_gid),
+                int(first_node), self._ptr(assign), self._ptr(fallback), self._stream()),
+            "apc_sample_feasible")
+        return assign, fallback
+
     def random_assignment(self, seed: int, a: int) -> np.ndarray:
         """The out_idx per node that score_random draws for assignment a."""
         g = self.g

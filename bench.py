@@ -335,6 +335,32 @@ def main():
                                "construction: each edge's inp_idx is its producer's draw), not ILP-feasible plans",
             "fraction_without_forbidden_entry": float((scores[:, 5] == 0).double().mean().item()),
         }
+        # the same batch drawn so that no forbidden (non-finite) entry is selected where the
+        # graph allows it: node by node, uniformly among the strategies allowed against the
+        # producers' choices (apc_sample_feasible), then scored from the assignment matrix
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        assign, fallbacks = eng.sample_feasible(1, 0, n)
+        torch.cuda.synchronize()
+        t_sample = time.perf_counter() - t0
+        t0 = time.perf_counter()
+        fscores = eng.score(assign)
+        torch.cuda.synchronize()
+        t_fscore = time.perf_counter() - t0
+        out["scoring"]["feasible_draws"] = {
+            "assignments": n,
+            "sample_seconds": t_sample,
+            "score_seconds": t_fscore,
+            "scored_from": eng.last_score_backend,
+            "assignments_per_s_sampled_and_scored": n / (t_sample + t_fscore),
+            "fraction_without_forbidden_entry": float((fscores[:, 5] == 0).double().mean().item()),
+            "fraction_without_fallback_node": float((fallbacks == 0).double().mean().item()),
+            "mean_fallback_nodes_per_assignment": float(fallbacks.double().mean().item()),
+            "objective_min": float(fscores[:, 4].min().item()),
+            "objective_mean": float(fscores[:, 4].mean().item()),
+            "objective_mean_of_the_plain_draws": float(scores[:, 4].mean().item()),
+        }
+        del assign, fscores
 
     if args.schedules > 0:
         # next row of the path: the lowered-graph estimator as a batch scorer of

@@ -638,6 +638,27 @@ int apc_score_random_assignments(const apc_problem* p, const double* per_arg, co
                                  int64_t first, int64_t n_assign, double* out, void* stream);
 uint32_t apc_random_assignment(uint64_t seed, int64_t a, int32_t node, int32_t nstrat);
 
+/* Candidate assignments that select no forbidden variable, where the graph allows
+ * it.  No function of the reference does this; "forbidden" is the reference's own
+ * notion: a decision variable whose cost is not finite, which
+ * add_inf_cost_constraint pins to zero (autoparallel/optimize_sharding.py:803-812;
+ * the APC_ENTRY_NONFINITE bit of flags).  For assignment a (counter first + a) the
+ * nodes from first_node on are walked in order and node v gets, uniformly, one of
+ * the strategies out_idx whose entries (v, arg, out_idx, choice of the producer of
+ * arg) are all finite; a node without such a strategy takes the plain draw of
+ * apc_random_assignment and is counted in n_fallback[a].  The choice among the
+ * allowed strategies is a reservoir walk in out_idx order: the k-th allowed one
+ * replaces the pick when apc_sample_takes(seed, first + a, id of v, k) is 1.
+ * assign: uint16[n_node][n_assign], written for v >= first_node; the rows below
+ * first_node are read (choices made earlier, e.g. for the stand-in nodes of a
+ * window of a larger graph).  node_gid: id of every node for the hashes (NULL:
+ * its index).  Score the result with apc_score_assignments or the batch scorers
+ * that take explicit assignments: element 5 of a row is 0 where n_fallback is. */
+int apc_sample_feasible(const apc_problem* p, const uint8_t* flags, uint64_t seed, int64_t first,
+                        int64_t n_assign, const int32_t* node_gid, int32_t first_node, uint16_t* assign,
+                        int32_t* n_fallback, void* stream);
+int32_t apc_sample_takes(uint64_t seed, int64_t a, int32_t node, uint32_t k);
+
 /* apc_score_random_assignments for a graph too large to keep its coefficients
  * resident: the problem holds a window of the graph's nodes (preceded by
  * first_node stand-ins for producers outside the window, which are not scored),

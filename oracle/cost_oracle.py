@@ -35,6 +35,11 @@ Pinning (what each function is checked against, see tests/test_oracle_*.py):
   * flop programs: ``torch.utils.flop_counter.FlopCounterMode`` on meta tensors.
   * decision-var assembly, scorer: algebraic identities and the reference
     tests' mock DecisionVar sums (tests/test_log_formatting.py:57-148 there).
+  * sample_feasible: no counterpart in the reference (which has no sampler); it
+    restates this library's own definition, and is pinned by what that definition
+    implies: no forbidden variable selected unless a node is counted as a
+    fallback, every allowed strategy of a node reached, and the frequencies of a
+    node's choices flat over many assignments (tests/test_oracle_closed_forms.py).
 """
 from __future__ import annotations
 
@@ -631,3 +636,77 @@ def ilp_objective(g, cost_clamped, forbidden, assign: Sequence[int]):
             obj += cost_clamped[i] * mult
             viol += int(forbidden[i])
     return obj, viol
+
+
+# ---------------------------------------------------------------------------
+# Candidate assignments without a forbidden variable
+# ---------------------------------------------------------------------------
+_M32 = 0xFFFFFFFF
+
+
+def _finalise32(h: int) -> int:
+    h ^= h >> 16
+    h = (h * 0x85EBCA6B) & _M32
+    h ^= h >> 13
+    h = (h * 0xC2B2AE35) & _M32
+    h ^= h >> 16
+    return h
+
+
+def _assignment_hash(seed: int, a: int) -> int:
+    seed &= 0xFFFFFFFFFFFFFFFF
+    a &= 0xFFFFFFFFFFFFFFFF
+    h = (seed & _M32) ^ (((seed >> 32) * 0x27D4EB2F) & _M32)
+    h ^= ((a & _M32) * 0x9E3779B1) & _M32
+    h ^= ((a >> 32) * 0x85EBCA77) & _M32
+    return h
+
+
+def plain_draw(seed: int, a: int, gid: int, nstrat: int) -> int:
+    """Uniform draw of the scorers: a 32-bit mix of (seed, assignment, node)
+    scaled to [0, nstrat) by a multiply-high."""
+    h = _finalise32(_assignment_hash(seed, a) ^ (((gid + 1) * 0xC2B2AE3D) & _M32))
+    return (h * nstrat) >> 32
+
+
+def reservoir_takes(seed: int, a: int, gid: int, k: int) -> bool:
+    """Whether the k-th allowed strategy (k >= 1) of node gid replaces the pick."""
+    h = _finalise32(_assignment_hash(seed, a) ^ (((gid + 1) * 0xC2B2AE3D) & _M32) ^ ((k * 0x9E3779B1) & _M32)
+                    ^ 0x68E31DA4)
+    return ((h * k) >> 32) == 0
+
+
+def sample_feasible(g, forbidden, seed: int, a: int, node_gid=None, first_node: int = 0, given=None):
+    """One assignment, node by node in graph order: node v gets, uniformly, one of
+    its strategies whose entries against the choices of its producers are all
+    allowed (``forbidden``: uint8 per slot, the non-finite costs that
+    add_inf_cost_constraint pins to zero, optimize_sharding.py:803-812); a node
+    without one takes the plain draw and is counted.  ``given``: the choices of
+    the nodes below first_node.  Returns (choices per node, number of fallbacks)."""
+    N = g.num_nodes
+    assign = [0] * N
+    for v in range(first_node):
+        assign[v] = int(given[v])
+    fallbacks = 0
+    for v in range(first_node, N):
+        gid = int(node_gid[v]) if node_gid is not None else v
+        S = int(g.node_nstrat[v])
+        count, pick = 0, 0
+        edges = range(int(g.node_edge_off[v]), int(g.node_edge_off[v + 1]))
+        for o in range(S):
+            ok = True
+            for e in edges:
+                u = int(g.edge_src_node[e])
+                j = assign[u] if u >= 0 else 0
+                if forbidden[int(g.edge_off[e]) + o * int(g.edge_ssrc[e]) + j]:
+                    ok = False
+                    break
+            if ok:
+                count += 1
+                if reservoir_takes(seed, a, gid, count):
+                    pick = o
+        if count == 0:
+            pick = plain_draw(seed, a, gid, S)
+            fallbacks += 1
+        assign[v] = pick
+    return assign, fallbacks

@@ -1,0 +1,77 @@
+"""apc_sample_feasible through the C ABI: the device's assignments equal the
+oracle's node by node, none selects a forbidden variable unless a node is counted
+as a fallback, and their scores are the oracle's bit for bit."""
+import numpy as np
+import pytest
+import torch
+
+from autoparallel_amd import graphgen
+from oracle import cost_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+GRAPHS = {
+    "llama_1layer_2x4": lambda: graphgen.llama_graph((2, 4), 1, 64, 4, 2, 128, 256, 32, 16),
+    "llama_1layer_8x8": lambda: graphgen.llama_graph((8, 8), 1, 1024, 8, 4, 2048, 8192, 512, 16),
+    "moe_tiny": lambda: graphgen.moe_graph((2, 4), 2, 64, 4, 8, 2, 32, 256, 32, 8),
+    "stress_3d": lambda: graphgen.stress_graph(150, (2, 2, 4), seed=4, s_min=2, s_max=60),
+}
+
+
+@pytest.fixture(scope="module")
+def CostEngine():
+    if not torch.cuda.is_available():
+        pytest.skip("needs a GPU")
+    from autoparallel_amd.engine import CostEngine
+
+    return CostEngine
+
+
+@pytest.mark.parametrize("name", list(GRAPHS))
+def test_sampled_assignments_equal_the_oracles(CostEngine, name):
+    g = GRAPHS[name]()
+    print(f"  sampler: {name} nodes={g.num_nodes} E={g.num_entries}", flush=True)
+    eng = CostEngine(g).build(clamp_inf=True)
+    ref = O.GraphOracle(g).build()
+    clamped, forbidden = O.clamp_inf(ref["cost"])
+    n = 96
+    assign, fallback = eng.sample_feasible(seed=9, first=1000, count=n)
+    assign, fallback = assign.cpu().numpy(), fallback.cpu().numpy()
+    # uint16 has no signed twin in numpy < 2; the tensor came back as uint16
+    scores = eng.score(torch.from_numpy(assign).to(eng.device)).cpu().numpy()
+    some_clean = False
+    for a in list(range(12)) + [n - 1]:
+        want, want_fb = O.sample_feasible(g, forbidden, 9, 1000 + a)
+        assert assign[:, a].tolist() == want, (name, a)
+        assert int(fallback[a]) == want_fb
+        tot = O.score_assignment(g, ref["comm"], ref["transition"], ref["compute"], want)
+        obj, viol = O.ilp_objective(g, clamped, forbidden, want)
+        assert tuple(scores[a, :4]) == tuple(float(x) for x in tot), (name, a)
+        assert scores[a, 4] == obj and scores[a, 5] == viol
+        if want_fb == 0:
+            assert viol == 0
+            some_clean = True
+    # over the whole batch: no fallback, nothing forbidden selected
+    assert ((fallback == 0) <= (scores[:, 5] == 0)).all()
+    if name != "stress_3d":
+        assert some_clean and (fallback == 0).any()
+    # and the plain draws of the same counters do select forbidden variables on these graphs
+    plain = eng.score_random(9, 1000, n).cpu().numpy()
+    assert (plain[:, 5] > 0).mean() > (scores[:, 5] > 0).mean()
+
+
+def test_sampler_continues_from_given_rows(CostEngine):
+    """Rows below first_node are taken as given (the stand-in nodes of a window):
+    sampling the tail of a graph from the head's choices gives the whole-graph
+    sample back."""
+    g = GRAPHS["llama_1layer_2x4"]()
+    eng = CostEngine(g).build(clamp_inf=True)
+    n, cut = 64, g.num_nodes // 2
+    whole, fb_whole = eng.sample_feasible(seed=3, first=0, count=n)
+    part = whole.clone()
+    part[cut:] = 0xFFFF
+    gid = np.arange(g.num_nodes, dtype=np.int32)
+    part, fb_part = eng.sample_feasible(seed=3, first=0, count=n, node_gid=gid, first_node=cut, assign=part)
+    assert torch.equal(part, whole)
+    # the tail's fallbacks are a part of the whole's
+    assert bool((fb_part <= fb_whole).all())

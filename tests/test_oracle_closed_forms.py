@@ -190,3 +190,68 @@ def test_roofline_closed_form():
     assert O.roofline_cost(0, 10, 3, dev) == 7
     with pytest.raises(ValueError):
         O.roofline_cost(10, 10, 5, dev)
+
+
+# ---------------------------------------------------------------------------
+# the sampler of assignments without a forbidden variable (no reference counterpart)
+# ---------------------------------------------------------------------------
+def _sampler_graph():
+    from autoparallel_amd import graphgen
+
+    g = graphgen.llama_graph((2, 4), 1, 64, 4, 2, 128, 256, 32, 16)
+    ref = O.GraphOracle(g).build()
+    _, forbidden = O.clamp_inf(ref["cost"])
+    return g, ref, forbidden
+
+
+def test_sampled_assignments_select_no_forbidden_variable():
+    g, ref, forbidden = _sampler_graph()
+    assert forbidden.any()
+    clamped, _ = O.clamp_inf(ref["cost"])
+    plain_hits = clean = 0
+    for a in range(40):
+        assign, fallbacks = O.sample_feasible(g, forbidden, 11, a)
+        _, viol = O.ilp_objective(g, clamped, forbidden, assign)
+        if fallbacks == 0:  # every node found an allowed strategy: nothing forbidden is selected
+            assert viol == 0
+            clean += 1
+        plain = [O.plain_draw(11, a, v, int(g.node_nstrat[v])) for v in range(g.num_nodes)]
+        plain_hits += O.ilp_objective(g, clamped, forbidden, plain)[1] > 0
+    assert clean > 0
+    assert plain_hits == 40  # the plain draws all select something forbidden on this graph
+
+
+def test_sampler_is_uniform_over_the_allowed_strategies_of_a_node():
+    """Frequencies of a node's choice over many assignments with its producer's
+    choice given: every allowed strategy is reached, no other one is, and none is
+    favoured (chi-square against the flat distribution).  The forbidden mask is
+    made by hand, so the allowed set is known without the sampler."""
+    from helpers import graph_from_pairs
+
+    n_src, n_tgt = 3, 12
+    g = graph_from_pairs((2, 4), 8, (64, 64), (64, 1), 4, [(0, 0), (0x40, 0), (0, 0x41)],
+                         [(0, 0)] * n_tgt)
+    assert g.num_nodes == 2 and int(g.node_nstrat[1]) == n_tgt
+    e = int(g.node_edge_off[1])
+    forbidden = np.zeros(g.num_slots, np.uint8)
+    allowed = {0: [1, 2, 3, 5, 8, 11], 1: [4], 2: []}
+    for j in range(n_src):
+        for o in range(n_tgt):
+            if o not in allowed[j]:
+                forbidden[int(g.edge_off[e]) + o * n_src + j] = 1
+    n = 6000
+    for j in range(n_src):
+        hist, fallback_total = {}, 0
+        for a in range(n):
+            assign, fallbacks = O.sample_feasible(g, forbidden, 5, a, first_node=1, given=[j])
+            hist[assign[1]] = hist.get(assign[1], 0) + 1
+            fallback_total += fallbacks
+        if not allowed[j]:  # nothing allowed: the plain draw over all strategies, counted
+            assert fallback_total == n and len(hist) == n_tgt
+            assert all(O.plain_draw(5, a, 1, n_tgt) == O.sample_feasible(g, forbidden, 5, a, first_node=1, given=[j])[0][1]
+                       for a in range(50))
+            continue
+        assert fallback_total == 0 and sorted(hist) == allowed[j], (j, sorted(hist))
+        k = len(allowed[j])
+        chi2 = sum((hist[o] - n / k) ** 2 / (n / k) for o in allowed[j])
+        assert chi2 < 20.5, (j, chi2)  # 99.9th percentile of chi-square with 5 degrees of freedom
