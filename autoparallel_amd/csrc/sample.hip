@@ -11,7 +11,7 @@
 // flow rows holds by construction, as for the plain draws: an edge's inp_idx is
 // its producer's choice.
 //
-// One lane per assignment.  Lanes of a wave read the flags of the same edge
+// Large batches: one lane per assignment.  Lanes of a wave read the flags of the same edge
 // block and the same row, at the columns their producers' choices name: one or
 // two cache lines per load, out of L2.  The choice among the allowed strategies
 // is a reservoir walk (the k-th allowed one replaces the pick when a hash of
@@ -105,6 +105,63 @@ sample_feasible_kernel(apc_problem p, const uint8_t* __restrict__ flags, uint64_
   n_fallback[a] = fallbacks;
 }
 
+// Small batches: one wavefront per assignment, lanes over the strategies of the
+// node.  A lane finds out whether its strategy is allowed, the ballot of the wave
+// gives every allowed strategy its rank k in out_idx order, each lane evaluates the
+// reservoir's test for its own k, and the pick is the last strategy whose test
+// says "take": what the sequential walk ends with.  Same choices as the kernel
+// above, bit for bit; the lanes of a wave read one column of a block (a cache line
+// each) instead of sharing a row, which is the better trade while there are
+// fewer assignments than lanes on the chip.
+__global__ void __launch_bounds__(kBlock)
+sample_feasible_wave_kernel(apc_problem p, const uint8_t* __restrict__ flags, uint64_t seed, int64_t first,
+                            int64_t n_assign, const int32_t* __restrict__ node_gid, int first_node,
+                            uint16_t* __restrict__ assign, int32_t* __restrict__ n_fallback) {
+  const int64_t a = (int64_t)blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6);
+  if (a >= n_assign) return;  // wave-uniform
+  const int lane = threadIdx.x & 63;
+  const uint32_t h0 = assignment_hash(seed, first + a);
+  int fallbacks = 0;
+  for (int v = first_node; v < p.n_node; ++v) {
+    const int S = p.node_nstrat[v];
+    const int gid = node_gid ? node_gid[v] : v;
+    const int e0 = p.node_edge_off[v], e1 = p.node_edge_off[v + 1];
+    uint32_t count = 0;
+    int pick = -1;
+    for (int o0 = 0; o0 < S; o0 += 64) {
+      const int o = o0 + lane;
+      uint32_t bad = o < S ? 0u : (uint32_t)APC_ENTRY_NONFINITE;
+      if (o < S) {
+        for (int e = e0; e < e1; ++e) {
+          const apc_edge* ed = p.edges + e;  // wave-uniform: scalar loads
+          const int u = ed->src_node;
+          // the producer's choice was written by this wave (lane 0) or by the caller
+          const uint32_t j = u >= 0 ? (uint32_t)assign[(size_t)u * n_assign + a] : 0u;
+          bad |= flags[ed->off + (int64_t)o * ed->ssrc + j];
+        }
+      }
+      const bool allowed = !(bad & APC_ENTRY_NONFINITE);
+      const uint64_t mask = __ballot(allowed);
+      const uint32_t rank = count + (uint32_t)__popcll(mask & ((1ull << lane) - 1ull)) + 1u;
+      const uint64_t takes = __ballot(allowed && reservoir_takes(h0, gid, rank));
+      if (takes) pick = o0 + 63 - __clzll(takes);
+      count += (uint32_t)__popcll(mask);
+    }
+    if (count == 0) {
+      pick = (int)plain_draw(h0, gid, S);
+      ++fallbacks;
+    }
+    if (lane == 0) assign[(size_t)v * n_assign + a] = (uint16_t)pick;
+    // the next node may read this choice through the vector memory path of other lanes
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  }
+  if (lane == 0) n_fallback[a] = fallbacks;
+}
+
+constexpr int64_t kSampleWaveBelow = 65536;  // assignments: below, a wavefront each
+
 }  // namespace
 
 extern "C" {
@@ -118,6 +175,13 @@ int apc_sample_feasible(const apc_problem* p, const uint8_t* flags, uint64_t see
     return fail(APC_ERR_INVALID, "apc_sample_feasible: null argument%s");
   if (first_node < 0 || first_node > p->n_node)
     return fail(APC_ERR_INVALID, "apc_sample_feasible: first_node out of range%s");
+  if (n_assign < kSampleWaveBelow) {
+    const int64_t per = kBlock / 64;
+    hipLaunchKernelGGL(sample_feasible_wave_kernel, dim3((unsigned)((n_assign + per - 1) / per)), dim3(kBlock), 0,
+                       (hipStream_t)stream, *p, flags, seed, first, n_assign, node_gid, (int)first_node, assign,
+                       n_fallback);
+    return check_launch("sample_feasible_wave_kernel");
+  }
   hipLaunchKernelGGL(sample_feasible_kernel, dim3((unsigned)((n_assign + kBlock - 1) / kBlock)), dim3(kBlock), 0,
                      (hipStream_t)stream, *p, flags, seed, first, n_assign, node_gid, (int)first_node, assign,
                      n_fallback);

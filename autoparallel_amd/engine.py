@@ -717,6 +717,21 @@ class CostEngine:
         )
         return out
 
+    def score_window(self, assign: torch.Tensor, first_node: int, init: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """score() for a window of a larger graph: explicit assignments (uint16
+        [n_node, n_assign], stand-in nodes included), the first ``first_node``
+        nodes contribute nothing, and the sums continue from ``init``."""
+        assert self.built
+        assert assign.dim() == 2 and assign.shape[0] == self.g.num_nodes and assign.is_contiguous()
+        assert assign.dtype in (torch.int16, torch.uint16) and assign.device == self.comm.device
+        count = assign.shape[1]
+        assert 0 <= first_node <= self.g.num_nodes
+        assert init is None or (init.shape == (count, 6) and init.dtype == torch.float64 and init.is_contiguous())
+        out = torch.empty((count, 6), dtype=torch.float64, device=self.device)
+        if not self.packed_scoring:
+            raise _lib.ApcError("score_window needs a graph with entries")
+        return self._score_packed(assign, 0, 0, count, None, first_node, init, out)
+
     def sample_feasible(self, seed: int, first: int, count: int, node_gid: Optional[np.ndarray] = None,
                         first_node: int = 0, assign: Optional[torch.Tensor] = None):
         """``count`` assignments drawn node by node among the strategies that select

@@ -553,12 +553,21 @@ class PackedGraph:
         rec = np.zeros(L, self.SPEC_REC_DTYPE)
         assert rec.dtype.itemsize == 16
         rec["word"] = self.lists
-        some = self.lists != SPEC_NONE
-        w = self.lists[some].astype(np.int64)
+        if L == 0:
+            return rec
+        none = self.lists == SPEC_NONE
+        any_none = bool(none.any())
+        w = self.lists.astype(np.int64)
+        if any_none:
+            w[none] = 0
         plc = np.ascontiguousarray(self.tuple_plc).view("<u4").reshape(-1)
         nbytes, contig = self.meta_bytes_contiguous()
-        rec["plc"][some] = plc[w & (MAX_TUPLES - 1)]
-        rec["nbytes2"][some] = (nbytes[w >> TUPLE_BITS] << 1) | contig[w >> TUPLE_BITS]
+        per_meta = (nbytes << 1) | contig  # whole-array gathers: masked ones cost three times as much
+        rec["plc"] = plc[w & (MAX_TUPLES - 1)] if plc.shape[0] else 0
+        rec["nbytes2"] = per_meta[w >> TUPLE_BITS] if per_meta.shape[0] else 0
+        if any_none:
+            rec["plc"][none] = 0
+            rec["nbytes2"][none] = 0
         return rec
 
     LUT_TILE_DTYPE = np.dtype([

@@ -65,10 +65,15 @@ def score_in_windows(
     workers: int = 8,
     max_windows: Optional[int] = None,
     progress=None,
+    feasible: bool = False,
 ):
     """Scores ``n_assign`` on-device drawn assignments of the n_total-node stress
     DAG, window by window.  Returns (scores float64[n_assign, 6] on the host,
-    stats dict)."""
+    stats dict).  ``feasible``: the assignments are drawn node by node among the
+    strategies that select no forbidden entry against the producers' choices
+    (CostEngine.sample_feasible) instead of independently per node; the choices
+    of all nodes are then kept on the device (2 bytes per node and assignment),
+    since a later window's stand-in producers carry the choices of their nodes."""
     import torch
 
     from autoparallel_amd.engine import CostEngine
@@ -81,6 +86,12 @@ def score_in_windows(
              "build_device_s": 0.0, "score_device_s": 0.0, "wait_for_window_s": 0.0, "engine_construct_s": 0.0,
              "modes": {}}
     out = None
+    choices = fallbacks = None
+    if feasible:
+        # int16 storage of the uint16 choices: torch gathers rows of int16, not of uint16
+        choices = torch.zeros((n_total, n_assign), dtype=torch.int16, device="cuda")
+        fallbacks = torch.zeros(n_assign, dtype=torch.int64, device="cuda")
+        stats["sample_device_s"] = 0.0
     t_wall = time.perf_counter()
     pool = None
     if workers > 1 and len(tasks) > 1:
@@ -95,16 +106,29 @@ def score_in_windows(
             t_mark = time.perf_counter()
             eng = CostEngine(g)
             stats["engine_construct_s"] += time.perf_counter() - t_mark  # layout of the problem and its upload
-            ev = [torch.cuda.Event(enable_timing=True) for _ in range(3)]
+            ev = [torch.cuda.Event(enable_timing=True) for _ in range(4)]
             ev[0].record()
             eng.build(clamp_inf=True)
             ev[1].record()
-            out = eng.score_random_window(assign_seed, 0, n_assign, gid, n_standin, init=out)
-            ev[2].record()
+            if feasible:
+                # the stand-ins' rows are the choices made for their nodes in earlier windows
+                local = choices[torch.from_numpy(gid.astype(np.int64)).to(choices.device)].contiguous()
+                _, fb = eng.sample_feasible(assign_seed, 0, n_assign, node_gid=gid, first_node=n_standin,
+                                            assign=local.view(torch.uint16))
+                choices[lo:hi] = local[n_standin:]
+                fallbacks += fb
+                ev[2].record()
+                out = eng.score_window(local.view(torch.uint16), n_standin, init=out)
+            else:
+                ev[2].record()
+                out = eng.score_random_window(assign_seed, 0, n_assign, gid, n_standin, init=out)
+            ev[3].record()
             torch.cuda.synchronize()
             eng.check_status()
             stats["build_device_s"] += ev[0].elapsed_time(ev[1]) * 1e-3
-            stats["score_device_s"] += ev[1].elapsed_time(ev[2]) * 1e-3
+            if feasible:
+                stats["sample_device_s"] += ev[1].elapsed_time(ev[2]) * 1e-3
+            stats["score_device_s"] += ev[2].elapsed_time(ev[3]) * 1e-3
             real = g.edge_node >= n_standin  # the stand-ins' own input edges are not the DAG's
             stats["nodes"] += hi - lo
             stats["standin_nodes"] += n_standin
@@ -122,6 +146,11 @@ def score_in_windows(
             pool.terminate()
             pool.join()
     stats["wall_s"] = time.perf_counter() - t_wall
+    if feasible:
+        fb = fallbacks.cpu().numpy()
+        stats["fallback_nodes_per_assignment_mean"] = float(fb.mean())
+        stats["fallback_nodes_per_assignment_min"] = int(fb.min())
+        stats["assignments_without_fallback"] = int((fb == 0).sum())
     return out.cpu().numpy(), stats
 
 
@@ -133,6 +162,8 @@ def main():
     ap.add_argument("--workers", type=int, default=min(14, os.cpu_count() or 1))
     ap.add_argument("--max-windows", type=int, default=None)
     ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--feasible", action="store_true",
+                    help="draw the assignments node by node among the strategies without a forbidden entry")
     args = ap.parse_args()
 
     def progress(st, wall):
@@ -141,7 +172,8 @@ def main():
               file=sys.stderr, flush=True)
 
     scores, st = score_in_windows(args.nodes, args.window, args.assignments, seed=args.seed,
-                                  workers=args.workers, max_windows=args.max_windows, progress=progress)
+                                  workers=args.workers, max_windows=args.max_windows, progress=progress,
+                                  feasible=args.feasible)
     obj = scores[:, 4]
     st.update({
         "workload": f"stress DAG, {args.nodes} nodes, mesh (4,8,8), windows of {args.window}",

@@ -81,6 +81,9 @@ def main():
     ap.add_argument("--direct", action="store_true", help="evaluate every entry directly (no block table)")
     ap.add_argument("--table-mode", choices=["full", "compressed", "direct"], default=None,
                     help="force the block-table layout (default: chosen from the table sizes)")
+    ap.add_argument("--windowed", type=int, default=2048, metavar="ASSIGNMENTS",
+                    help="also build and score configs[4] at its full 200 000 nodes window by window with this many "
+                         "assignments, plain and feasible draws (about 30 s of wall time with 14 host workers; 0 = skip)")
     ap.add_argument("--calibration-copy-mib", type=int, default=0,
                     help="after the timed steps, also launch the plain copy kernel on this many MiB "
                          "(the known-traffic reference for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)")
@@ -438,6 +441,22 @@ def main():
             out["cpu_baseline"]["compiled_port"] = res
         except Exception as exc:  # the checker library is optional for the benchmark
             out["cpu_baseline"]["compiled_port"] = {"error": str(exc)}
+    if args.windowed > 0:
+        # configs[4] at full size: 2.4e10 entries, built and scored in windows of 3 000 nodes
+        from autoparallel_amd import windowed
+
+        legs = {}
+        for label, feasible in (("plain_draws", False), ("feasible_draws", True)):
+            scores, st = windowed.score_in_windows(200000, 3000, args.windowed, workers=14, feasible=feasible)
+            st.update({
+                "assignments": int(scores.shape[0]),
+                "entries_per_s_device_build": st["entries"] / st["build_device_s"],
+                "edge_terms_per_s_scoring": scores.shape[0] * st["edges"] / st["score_device_s"],
+                "fraction_without_forbidden_entry": float((scores[:, 5] == 0).mean()),
+                "objective_min": float(scores[:, 4].min()), "objective_mean": float(scores[:, 4].mean()),
+            })
+            legs[label] = st
+        out["windowed_stress_dag_200k"] = legs
     if args.fx_layers > 0 and args.workload == "llama3_8b_fwd_bwd_mesh8x8":
         # secondary figure: the same model through the reference-shaped interface, from
         # the traced joint graph to coefficients and ILP rows (strategy sets of the

@@ -58,6 +58,13 @@ def test_sampled_assignments_equal_the_oracles(CostEngine, name):
     # and the plain draws of the same counters do select forbidden variables on these graphs
     plain = eng.score_random(9, 1000, n).cpu().numpy()
     assert (plain[:, 5] > 0).mean() > (scores[:, 5] > 0).mean()
+    # a large batch takes the lane-per-assignment kernel (the one above a wavefront per
+    # assignment): the same choices for the same counters
+    big, big_fb = eng.sample_feasible(seed=9, first=1000, count=65536)
+    assert np.array_equal(big[:, :n].cpu().numpy(), assign) and np.array_equal(big_fb[:n].cpu().numpy(), fallback)
+    a = 65535
+    want, want_fb = O.sample_feasible(g, forbidden, 9, 1000 + a)
+    assert big[:, a].cpu().numpy().tolist() == want and int(big_fb[a]) == want_fb
 
 
 def test_sampler_continues_from_given_rows(CostEngine):

@@ -65,3 +65,41 @@ def test_a_window_of_the_full_dag_against_the_compiled_oracle():
     for k in ("comm", "cost", "compute"):
         assert (got[k].view(np.uint64) == want[k].view(np.uint64)).all(), k
     assert ((got["flags"] & 1) == want["transition"]).all()
+
+
+def test_feasible_draws_in_windows_equal_one_pass():
+    """Assignments drawn without forbidden entries where the graph allows it: the
+    windows carry the choices of earlier nodes along, and give the sample and the
+    sums of one pass over the whole graph, bit for bit."""
+    from autoparallel_amd.engine import CostEngine
+
+    n = 4096
+    g, gid, _ = graphgen.stress_dag_window(N_TOTAL, 0, N_TOTAL, (4, 8, 8), SEED, 4, S_MAX)
+    eng = CostEngine(g).build(clamp_inf=True)
+    assign, fb = eng.sample_feasible(1, 0, n)
+    whole = eng.score(assign).cpu().numpy()
+    plain = eng.score_random(1, 0, n).cpu().numpy()
+    assert (whole[:, 5] == 0).sum() >= (plain[:, 5] == 0).sum() and whole[:, 5].mean() < plain[:, 5].mean()
+    for window in (60, 97):
+        got, st = windowed.score_in_windows(N_TOTAL, window, n, seed=SEED, assign_seed=1, s_max=S_MAX, workers=1,
+                                            feasible=True)
+        assert (got.view(np.uint64) == whole.view(np.uint64)).all(), window
+        assert st["assignments_without_fallback"] == int((fb == 0).sum().item())
+        assert abs(st["fallback_nodes_per_assignment_mean"] - float(fb.double().mean().item())) < 1e-9
+
+
+def test_config5_at_full_size_in_windows():
+    """The planner stress DAG at its full 200 000 nodes (2.4e10 cost entries, more
+    than one GPU holds at once), built and scored window by window: sizes as the
+    generator defines them, every window with the compressed block table, finite
+    sums, and the same sums, bit for bit, from windows of another size."""
+    n = 2048
+    first, st = windowed.score_in_windows(200000, 3000, n, workers=14)
+    assert st["nodes"] == 200000 and st["edges"] == 360006 and st["entries"] == 23981186946, st
+    assert st["windows"] == 67 and st["modes"] == {"compressed": 67}
+    assert np.isfinite(first).all() and (first[:, 4] > 0).all()
+    print(f"  200k nodes in windows of 3000: wall {st['wall_s']:.1f} s, device build {st['build_device_s']:.2f} s, "
+          f"scoring {st['score_device_s']:.2f} s", flush=True)
+    second, st2 = windowed.score_in_windows(200000, 4500, n, workers=14)
+    assert st2["entries"] == st["entries"] and st2["windows"] == 45
+    assert (first.view(np.uint64) == second.view(np.uint64)).all()
