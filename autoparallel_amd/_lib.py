@@ -265,6 +265,10 @@ _SIGNATURES = {
         C.c_int,
         [C.POINTER(ApcModel), C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
     "apc_rw_times": (C.c_int, [C.POINTER(ApcModel), C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p]),
+    "apc_filter_strategies": (
+        C.c_int,
+        [C.POINTER(ApcModel), C.c_int32, C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p, C.c_int32, C.c_void_p,
+         C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p]),
     "apc_enumerate_input_options": (
         C.c_int,
         [C.POINTER(ApcModel), C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,

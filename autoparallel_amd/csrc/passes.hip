@@ -241,6 +241,89 @@ enumerate_kernel(apc_model m, int32_t n, const int32_t* __restrict__ rank,
 }
 
 // ---------------------------------------------------------------------------
+// Kernel: validity filter and de-duplication of operator strategies.  A set is the
+// candidate strategies of one node, a row of spec words per strategy (its input
+// specs, then its output specs; APC_SPEC_NONE where there is none).  A row is
+// valid when every spec passes the rule of enumerate_kernel: walking the mesh dims
+// in order, a Shard(d) needs the (already divided) size of dim d to be at least
+// the mesh size and divides it, rounding up.  Among the valid rows of a set, one
+// that repeats the words of an earlier valid row is dropped.  One workgroup per
+// set: a lane per row for the rule and a 64-bit hash of the row (LDS), then a
+// lane per row against the rows before it, hashes first.
+// ---------------------------------------------------------------------------
+constexpr int kFilterRows = 4096;  // rows of a set whose hashes fit the workgroup's LDS
+
+__device__ __forceinline__ uint64_t mix_word(uint64_t h, uint32_t w, int pos) {
+  uint64_t z = h ^ (((uint64_t)w << 8) + (uint64_t)(pos + 1)) * 0x9E3779B97F4A7C15ull;
+  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+  z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+  return z ^ (z >> 31);
+}
+
+__global__ void __launch_bounds__(kBlock)
+filter_strategies_kernel(apc_model m, const int32_t* __restrict__ meta_rank, const int64_t* __restrict__ meta_shape,
+                         const uint8_t* __restrict__ tuple_plc, const int64_t* __restrict__ set_row,
+                         const int32_t* __restrict__ set_width, const int64_t* __restrict__ set_word,
+                         const uint32_t* __restrict__ words, uint8_t* __restrict__ valid,
+                         uint8_t* __restrict__ keep) {
+  __shared__ uint64_t s_hash[kFilterRows];
+  __shared__ uint8_t s_valid[kFilterRows];
+  const int set = blockIdx.x;
+  const int64_t row0 = set_row[set];
+  const int n_rows = (int)(set_row[set + 1] - row0);
+  const int width = set_width[set];
+  const uint32_t* __restrict__ w0 = words + set_word[set];
+  for (int r = threadIdx.x; r < n_rows; r += kBlock) {
+    const uint32_t* __restrict__ row = w0 + (size_t)r * width;
+    bool ok = true;
+    uint64_t h = 0x243F6A8885A308D3ull;
+    for (int c = 0; c < width; ++c) {
+      const uint32_t w = row[c];
+      h = mix_word(h, w, c);
+      if (w == APC_SPEC_NONE) continue;
+      const uint32_t mid = w >> APC_TUPLE_BITS;
+      const uint32_t plc = load_tuple(tuple_plc, w & kTupleMask);
+      const int rank = meta_rank[mid];
+      int64_t sh[APC_MAX_RANK];
+#pragma unroll
+      for (int d = 0; d < APC_MAX_RANK; ++d) sh[d] = meta_shape[(size_t)mid * APC_MAX_RANK + d];
+      for (int i = 0; i < m.ndim; ++i) {
+        const int code = (plc >> (8 * i)) & 0xFF;
+        if ((code & kKindMask) != kShard) continue;
+        const int d = code & kArgMask;
+        const int64_t ms = m.mesh_shape[i];
+        if (d >= rank) { ok = false; continue; }  // a dim the tensor does not have (the packer refuses such a spec)
+#pragma unroll
+        for (int dd = 0; dd < APC_MAX_RANK; ++dd) {  // dynamic index kept in a loop so sh[] stays in registers
+          if (dd == d) {
+            if (sh[dd] >= ms) sh[dd] = (sh[dd] + ms - 1) / ms; else ok = false;
+          }
+        }
+      }
+    }
+    s_hash[r] = h;
+    s_valid[r] = ok ? 1 : 0;
+    valid[row0 + r] = ok ? 1 : 0;
+  }
+  __syncthreads();
+  for (int r = threadIdx.x; r < n_rows; r += kBlock) {
+    bool kept = s_valid[r] != 0;
+    if (kept) {
+      const uint64_t h = s_hash[r];
+      const uint32_t* __restrict__ row = w0 + (size_t)r * width;
+      for (int q = 0; q < r; ++q) {
+        if (!s_valid[q] || s_hash[q] != h) continue;
+        const uint32_t* __restrict__ other = w0 + (size_t)q * width;
+        bool same = true;
+        for (int c = 0; c < width && same; ++c) same = row[c] == other[c];
+        if (same) { kept = false; break; }
+      }
+    }
+    keep[row0 + r] = kept ? 1 : 0;
+  }
+}
+
+// ---------------------------------------------------------------------------
 // Kernels: scalar cost-model functions in batch form
 // ---------------------------------------------------------------------------
 // _get_sharded_shape_stride (compute_estimation.py:300-318), including its
@@ -415,6 +498,23 @@ int apc_enumerate_input_options(const apc_model* model, int32_t n, const int32_t
   hipLaunchKernelGGL(enumerate_kernel, dim3(grid_for((int64_t)n * 64, kBlock)), dim3(kBlock), 0,
                      (hipStream_t)stream, *model, n, rank, shape, cand_off, valid, plc);
   return check_launch("enumerate_kernel");
+}
+
+int apc_filter_strategies(const apc_model* model, int32_t n_meta, const int32_t* meta_rank,
+                          const int64_t* meta_shape, int32_t n_tuple, const uint8_t* tuple_plc, int32_t n_set,
+                          const int64_t* set_row, const int32_t* set_width, const int64_t* set_word,
+                          const uint32_t* words, int32_t max_rows, uint8_t* valid, uint8_t* keep, void* stream) {
+  if (!model || model->ndim < 1 || model->ndim > APC_MAX_MESH_DIMS)
+    return fail(APC_ERR_INVALID, "apc_filter_strategies: bad model%s");
+  if (n_set <= 0) return 0;
+  if (n_meta <= 0 || n_tuple <= 0 || !meta_rank || !meta_shape || !tuple_plc || !set_row || !set_width || !set_word ||
+      !words || !valid || !keep)
+    return fail(APC_ERR_INVALID, "apc_filter_strategies: null argument%s");
+  if (max_rows < 0 || max_rows > kFilterRows)
+    return fail(APC_ERR_INVALID, "apc_filter_strategies: a set has more than 4096 rows%s");
+  hipLaunchKernelGGL(filter_strategies_kernel, dim3((unsigned)n_set), dim3(kBlock), 0, (hipStream_t)stream, *model,
+                     meta_rank, meta_shape, tuple_plc, set_row, set_width, set_word, words, valid, keep);
+  return check_launch("filter_strategies_kernel");
 }
 
 }  // extern "C"

@@ -197,7 +197,15 @@ class SparseILP:
         n = indptr.shape[0] - 1
         if n <= 0:
             return []
-        coef = np.full(idx.shape[0], float(coef)) if np.isscalar(coef) else np.ascontiguousarray(coef, np.float64)
+        # coefficients that are all small whole numbers (the +-1 of the default rows) are kept
+        # as bytes: an eighth of the memory of a block; a row read out of the block is float64
+        if np.isscalar(coef):
+            small = float(coef) == int(coef) and -128 <= coef <= 127
+            coef = np.full(idx.shape[0], coef, np.int8 if small else np.float64)
+        else:
+            coef = np.ascontiguousarray(coef)
+            if coef.dtype != np.int8:
+                coef = np.ascontiguousarray(coef, np.float64)
         rhs = np.full(n, float(rhs)) if np.isscalar(rhs) else np.ascontiguousarray(rhs, np.float64)
         assert indptr[0] == 0 and indptr[-1] == idx.shape[0] == coef.shape[0] and (np.diff(indptr) >= 0).all()
         assert idx.size == 0 or (0 <= idx.min() and idx.max() < self.n_vars)
@@ -256,7 +264,7 @@ class SparseILP:
             r = b.rhs[keep]
             lo.append(r if b.sense != LE else np.full(r.shape[0], -np.inf))
             hi.append(r if b.sense != GE else np.full(r.shape[0], np.inf))
-        cat = lambda xs, dt: np.concatenate(xs) if xs else np.zeros(0, dt)
+        cat = lambda xs, dt: np.concatenate(xs).astype(dt, copy=False) if xs else np.zeros(0, dt)
         lens = cat(lens, np.int64)
         ptr = np.zeros(lens.shape[0] + 1, np.int64)
         np.cumsum(lens, out=ptr[1:])

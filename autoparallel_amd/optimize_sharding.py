@@ -19,6 +19,7 @@ import gc
 import logging
 import time
 import operator
+import weakref
 from typing import Any, Dict, Iterator, List, Optional, Tuple, Union
 
 import numpy as np
@@ -142,9 +143,26 @@ class DecisionVar:
         return "DecisionVar(" + ", ".join(f"{f}={getattr(self, f)!r}" for f in self._FIELDS) + ")"
 
 
-class DecisionVars(collections.abc.Mapping):
+class _OwnedByOptimizer:
+    """A view that the optimizer itself holds: it refers back weakly, so that the
+    optimizer and its million strategy objects are freed when the last reference to
+    it goes, not when the cyclic collector next walks the heap.  (The DecisionVar
+    views handed out to callers hold the optimizer strongly.)"""
+
+    def _bind(self, opt: "ShardingOptimizer") -> None:
+        self._opt_ref = weakref.ref(opt)
+
+    @property
+    def _opt(self) -> "ShardingOptimizer":
+        opt = self._opt_ref()
+        if opt is None:
+            raise ReferenceError("the ShardingOptimizer behind this mapping no longer exists")
+        return opt
+
+
+class DecisionVars(_OwnedByOptimizer, collections.abc.Mapping):
     def __init__(self, opt: "ShardingOptimizer"):
-        self._opt = opt
+        self._bind(opt)
         self._ordered_keys: Optional[np.ndarray] = None  # made when the mapping is first iterated
 
     def _col(self, key) -> int:
@@ -175,14 +193,15 @@ class DecisionVars(collections.abc.Mapping):
         return int(self._opt._packed.num_entries)
 
 
-class _ClusterLinks(collections.abc.Mapping):
+class _ClusterLinks(_OwnedByOptimizer, collections.abc.Mapping):
     """The reference's per-variable link table (linked key -> root key,
     autoparallel/optimize_sharding.py:356-378) as a view over the node-level
     links: a repeated node's key maps to the same (arg, out, inp) of its root.
     Keys are produced on iteration, not stored (a 32-layer model has millions)."""
 
     def __init__(self, opt: "ShardingOptimizer", node_links: Dict[int, int]):
-        self._opt, self._nodes = opt, dict(node_links)
+        self._bind(opt)
+        self._nodes = dict(node_links)
 
     def __getitem__(self, key):
         v, a, o, j = key
@@ -583,7 +602,7 @@ class ShardingOptimizer:
         # One template per strategy query: the repeated layers of a model ask the same
         # queries (same operator, arguments and candidates: same specs and program), and
         # a node then only adds its producers.  Everything else is array work in pack().
-        template_of: Dict[int, int] = {}
+        template_of: Dict[tuple, int] = {}
         strats, input_nodes_of = self.strats, self._all_input_nodes
         packed_nodes: List[torch.fx.Node] = []
         for node in self.nodes:
@@ -591,6 +610,11 @@ class ShardingOptimizer:
                 continue
             st: OpStrategy = strats[node]
             qkey = getattr(st, "_apc_query_id", None)
+            if qkey is not None:
+                # the answer of a query as it was handed out: a caller may have dropped or
+                # replaced strategies since (the specs of an answer are shared by its copies)
+                sts = st.strategies
+                qkey = (qkey, len(sts), id(sts[0].output_specs), id(sts[-1].output_specs))
             t = template_of.get(qkey) if qkey is not None else None
             if t is None:
                 desc = fx_programs.describe_node(node, st.strategies, b, name=node.name, memo=memo)

@@ -315,11 +315,19 @@ class PackedShardingOptimizer:
         count = np.asarray(count, np.int64)
         ptr = np.zeros(count.shape[0] + 1, np.int64)
         np.cumsum(count, out=ptr[1:])
-        seg = np.repeat(np.arange(count.shape[0], dtype=np.int64), count)
-        local = np.arange(int(ptr[-1]), dtype=np.int64) - ptr[:-1][seg]
-        if stride is not None:
-            local = local * np.asarray(stride, np.int64)[seg]
-        return start[seg] + local, ptr
+        total = int(ptr[-1])
+        if total == 0:
+            return np.zeros(0, np.int64), ptr
+        # as a running sum of steps: the stride inside a piece, and at the first element of a
+        # piece the jump from the last element of the piece before (three passes over the
+        # output instead of six)
+        step = np.ones(total, np.int64) if stride is None else np.repeat(np.asarray(stride, np.int64), count)
+        some = count > 0
+        first, st, cn = ptr[:-1][some], start[some], count[some]
+        last = st + (cn - 1 if stride is None else (cn - 1) * np.asarray(stride, np.int64)[some])
+        step[first[0]] = st[0]
+        step[first[1:]] = st[1:] - last[:-1]
+        return np.cumsum(step), ptr
 
     def _add_difference_rows(self, prefix, plus_start, plus_count, minus_start, minus_count, minus_stride) -> None:
         """Rows  sum(plus piece) - sum(minus piece) = 0, one per pair of pieces."""
@@ -330,7 +338,7 @@ class PackedShardingOptimizer:
         count = np.empty(2 * n, np.int64); count[0::2] = plus_count; count[1::2] = minus_count
         stride = np.ones(2 * n, np.int64); stride[1::2] = minus_stride
         idx, ptr = self._segments(start, count, stride)
-        sign = np.ones(2 * n); sign[1::2] = -1.0
+        sign = np.ones(2 * n, np.int8); sign[1::2] = -1
         self.prob.add_rows(prefix, ptr[0::2], idx, np.repeat(sign, count), ilp.EQ, 0.0)
 
     def add_unique_decision_constraint(self) -> None:
@@ -433,14 +441,29 @@ class PackedShardingOptimizer:
     def _add_paired_output_constraint(self, a: int, b: int, name: str) -> None:
         pa, pb = self._out_placements(a), self._out_placements(b)
         ea, eb = int(self.g.node_edge_off[a]), int(self.g.node_edge_off[b])
+        # rows in strategy order; consecutive rows of one kind go in as one block (the names
+        # and their order are those of a row-by-row loop: a counter per prefix)
+        run_prefix, ptr, idx, coef = None, [0], [], []
+
+        def flush():
+            if run_prefix is not None and len(ptr) > 1:
+                self.prob.add_rows(run_prefix, np.asarray(ptr, np.int64), np.concatenate(idx), np.concatenate(coef),
+                                   ilp.EQ, 0.0)
+
         for o, t in enumerate(pa):
             va = self._row_vars(ea, o)
             if t not in pb:
-                self.prob.add_row(name + "_disable", va, 1.0, ilp.EQ, 0.0)
-                continue
-            vb = self._row_vars(eb, pb.index(t))
-            self.prob.add_row(name, np.concatenate([vb, va]),
-                              np.concatenate([np.ones(len(vb)), -np.ones(len(va))]), ilp.EQ, 0.0)
+                prefix, row_idx, row_coef = name + "_disable", [va], [np.ones(len(va))]
+            else:
+                vb = self._row_vars(eb, pb.index(t))
+                prefix, row_idx, row_coef = name, [vb, va], [np.ones(len(vb)), -np.ones(len(va))]
+            if prefix != run_prefix:
+                flush()
+                run_prefix, ptr, idx, coef = prefix, [0], [], []
+            idx += row_idx
+            coef += row_coef
+            ptr.append(ptr[-1] + sum(len(x) for x in row_idx))
+        flush()
 
     def add_forward_backward_consistency_constraints(self) -> None:
         for p, gnode in self.roles.param_grad:
@@ -454,16 +477,19 @@ class PackedShardingOptimizer:
                 self._add_paired_output_constraint(n, t, "grad_output_constraint")
 
     def add_grad_reduce_dtype_constraints(self) -> None:
-        keys = self.g.entry_keys()
-        comm_pos = self.coef.comm > 0
+        g = self.g
         for nodes, name, enabled in (
             (self.roles.fwd_pre_cast, "fwd_param_dtype", True),
             (self.roles.bwd_pre_cast, "grad_reduce_dtype", self.force_grad_reduce_in_higher_precision),
         ):
             if not enabled or not nodes:
                 continue
-            mask = np.isin(keys[:, 0], np.fromiter(nodes, np.int64)) & comm_pos & (self.prob.upper > 0)
-            i = np.nonzero(mask)[0]
+            # the variables of those nodes: the blocks their edges own, in variable order
+            marked = np.zeros(g.num_nodes, bool)
+            marked[np.fromiter(nodes, np.int64)] = True
+            e = np.nonzero(marked[g.edge_node] & (self.var_start[1:] > self.var_start[:-1]))[0]
+            i, _ = self._segments(self.var_start[e], self.var_start[e + 1] - self.var_start[e])
+            i = i[(self.coef.comm[i] > 0) & (self.prob.upper[i] > 0)]
             self.prob.add_rows(name, np.arange(i.shape[0] + 1), i, 1.0, ilp.EQ, 0.0)
 
     # -- user constraints -----------------------------------------------------------

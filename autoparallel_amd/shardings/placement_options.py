@@ -103,18 +103,34 @@ def enumerate_input_placements(mesh_shape: Sequence[int], shapes: Sequence[Seque
     return out
 
 
+# input / parameter options by (mesh, tensor meta): the specs (which nothing writes to: they
+# are complete) and the id of the answer, as for operator queries.  The parameters of a model
+# have a handful of distinct shapes; a spec object costs ten microseconds to make and an
+# enumeration a kernel launch.
+_input_options_cache: Dict[tuple, tuple] = {}
+_query_serial = itertools.count()  # never restarts: an id names one answer for the life of the process
+
+
 def _create_all_options(mesh, shape, tensor_meta=None, tensor=None) -> OpStrategy:
     if tensor is not None:
         tensor_meta = _tensor_meta(tensor)
     if tensor_meta is None:
         t = torch.empty(tuple(shape), device="meta")
         tensor_meta = _tensor_meta(t)
-    rows = enumerate_input_placements(tuple(mesh.shape), [tuple(shape)])[0]
-    strats = []
-    for plc in rows:
-        spec = DTensorSpec(mesh, plc, tensor_meta=tensor_meta)
-        strats.append(OpSpec(spec, input_specs=[spec], redistribute_cost=[[0.0]]))
-    return OpStrategy(strats)
+    try:
+        key = (mesh, tuple(shape), tensor_meta)
+        hit = _input_options_cache.get(key)
+    except TypeError:  # a symbolic size
+        key = hit = None
+    if hit is None:
+        rows = enumerate_input_placements(tuple(mesh.shape), [tuple(shape)])[0]
+        hit = ([DTensorSpec(mesh, plc, tensor_meta=tensor_meta) for plc in rows], next(_query_serial))
+        if key is not None:
+            _input_options_cache[key] = hit
+    specs, qid = hit
+    out = OpStrategy([OpSpec(spec, input_specs=[spec], redistribute_cost=[[0.0]]) for spec in specs])
+    out._apc_query_id = qid  # equal ids: equal strategies (what a packer may memoise on)
+    return out
 
 
 # ---------------------------------------------------------------------------
@@ -157,6 +173,121 @@ def keep_unique_configs(op_strat: OpStrategy) -> OpStrategy:
             pass
         kept.append(st)
     return OpStrategy(kept)
+
+
+class _SpecWords:
+    """Spec words (tensor-meta id << 12 | placement-tuple id, as in the packed
+    problem) of the DTensorSpecs of one mesh, interned by value, with the two
+    tables on the device; kept between queries."""
+
+    def __init__(self, mesh_shape):
+        from ..packed import GraphBuilder
+
+        self.b = GraphBuilder(tuple(mesh_shape))
+        self.meta_ids: Dict[object, int] = {}
+        self.tuple_ids: Dict[object, int] = {}
+        self.uploaded = (-1, -1)
+        self.d_rank = self.d_shape = self.d_plc = None
+
+    def word(self, spec) -> int:
+        from ..dtensor_bridge import placement_codes, tensor_meta_key
+        from ..packed import SPEC_NONE, spec_word
+
+        if spec is None:
+            return SPEC_NONE
+        tm, plc = spec.tensor_meta, spec.placements
+        m = self.meta_ids.get(tm)
+        if m is None:
+            m = self.meta_ids[tm] = self.b.meta(*tensor_meta_key(tm))
+        t = self.tuple_ids.get(plc)
+        if t is None:
+            t = self.tuple_ids[plc] = self.b.tuple_id(placement_codes(plc))
+        return spec_word(m, t)
+
+    def tables(self):
+        b = self.b
+        n = (len(b._meta_rows), len(b._tuple_rows))
+        if n != self.uploaded:
+            rank = np.asarray([len(r[0]) for r in b._meta_rows], np.int32)
+            shape = np.ones((n[0], 8), np.int64)
+            for i, r in enumerate(b._meta_rows):
+                shape[i, : len(r[0])] = r[0]
+            plc = np.zeros((n[1], 4), np.uint8)
+            for i, r in enumerate(b._tuple_rows):
+                plc[i, : len(r)] = r
+            self.d_rank, self.d_shape, self.d_plc = (torch.from_numpy(a).cuda() for a in (rank, shape, plc))
+            self.uploaded = n
+        return n, self.d_rank, self.d_shape, self.d_plc
+
+
+_spec_words: Dict[tuple, _SpecWords] = {}
+# sets of at least this many strategies are filtered on the device (below, the launch and
+# the two copies cost more than the loop over a few dozen OpSpecs)
+DEVICE_FILTER_FROM = 32
+
+
+def strategy_rows(strategies, table: _SpecWords) -> Optional[np.ndarray]:
+    """uint32[n, width]: per strategy the words of its input specs, then of its
+    output specs.  None when the set has no such form (strategies of different
+    widths, a spec without its tensor meta)."""
+    rows = []
+    for st in strategies:
+        outs = st.output_specs
+        outs = [outs] if isinstance(outs, DTensorSpec) else list(outs or [])
+        specs = (list(st.input_specs) if st.input_specs is not None else []) + outs
+        if any(sp is not None and sp.tensor_meta is None for sp in specs):
+            return None
+        rows.append([table.word(sp) for sp in specs])
+    if not rows or any(len(r) != len(rows[0]) for r in rows) or not rows[0]:
+        return None
+    return np.asarray(rows, np.int64).astype(np.uint32)
+
+
+def filter_masks_on_device(mesh_shape, sets: Sequence[np.ndarray], table: _SpecWords):
+    """(valid, keep) uint8 per row of every set (apc_filter_strategies), the sets'
+    rows one after the other."""
+    from ..cost_models.collective_runtime_estimation import _device_name
+    from ..engine import make_model
+
+    lib = _lib.load()
+    n_rows = np.asarray([r.shape[0] for r in sets], np.int64)
+    width = np.asarray([r.shape[1] for r in sets], np.int32)
+    set_row = np.zeros(len(sets) + 1, np.int64)
+    np.cumsum(n_rows, out=set_row[1:])
+    set_word = np.zeros(len(sets), np.int64)
+    np.cumsum((n_rows * width)[:-1], out=set_word[1:])
+    words = np.concatenate([r.reshape(-1) for r in sets]).view(np.int32)
+    (n_meta, n_tuple), d_rank, d_shape, d_plc = table.tables()
+    d = lambda a: torch.from_numpy(a).cuda()
+    t_row, t_width, t_word, t_words = d(set_row), d(width), d(set_word), d(words)
+    masks = torch.empty((2, int(set_row[-1])), dtype=torch.uint8, device="cuda")
+    model = make_model(tuple(mesh_shape), 1, _device_name())
+    _lib.check(lib.apc_filter_strategies(
+        C.byref(model), n_meta, d_rank.data_ptr(), d_shape.data_ptr(), n_tuple, d_plc.data_ptr(), len(sets),
+        t_row.data_ptr(), t_width.data_ptr(), t_word.data_ptr(), t_words.data_ptr(), int(n_rows.max()),
+        masks[0].data_ptr(), masks[1].data_ptr(), None), "apc_filter_strategies")
+    out = masks.cpu().numpy()
+    return out[0], out[1]
+
+
+def filter_strategies(out_strat: OpStrategy, mesh) -> OpStrategy:
+    """remove_invalid_configs then keep_unique_configs.  Sets of DEVICE_FILTER_FROM
+    strategies or more go through the device in packed form; smaller ones, and sets
+    without that form, through the two loops."""
+    sts = out_strat.strategies
+    if DEVICE_FILTER_FROM <= len(sts) <= 4096:
+        mesh_shape = tuple(mesh.shape)
+        table = _spec_words.get((mesh, mesh_shape))
+        if table is None:
+            table = _spec_words[(mesh, mesh_shape)] = _SpecWords(mesh_shape)
+        try:
+            rows = strategy_rows(sts, table)
+        except (TypeError, AssertionError):  # an unhashable size, a tensor of more dims than the tables hold
+            rows = None
+        if rows is not None:
+            _, keep = filter_masks_on_device(mesh_shape, [rows], table)
+            return OpStrategy([st for st, k in zip(sts, keep.tolist()) if k])
+    return keep_unique_configs(remove_invalid_configs(out_strat, mesh))
 
 
 def propagate_tensor_meta(node, arg_vals: List[torch.Tensor], out_strat: OpStrategy, mesh=None) -> None:
@@ -770,12 +901,13 @@ def _copy_strategy(src: OpStrategy) -> OpStrategy:
 # model repeat the same queries, and one answer from the propagator costs
 # milliseconds.  Values: (strategies, why the all-Replicate stand-in was used or None, id of the answer).
 _strategy_cache: Dict[tuple, tuple] = {}
-_query_serial = itertools.count()  # never restarts: an id names one answer for the life of the process
 strategy_cache_stats = {"hits": 0, "misses": 0}
 
 
 def reset_placement_options_cache() -> None:
     _strategy_cache.clear()
+    _input_options_cache.clear()
+    _spec_words.clear()
     _fp_intern.clear()
     strategy_cache_stats.update(hits=0, misses=0)
 
@@ -964,8 +1096,7 @@ def _placement_options_uncached_inner(mesh, node, producers, arg_vals, schema_ar
     _unshare_specs(out, producers)
     propagate_tensor_meta(node, arg_vals, out, mesh)
     fill_redistribute_cost(out, producers)
-    out = remove_invalid_configs(out, mesh)
-    out = keep_unique_configs(out)
+    out = filter_strategies(out, mesh)
     if not out.strategies:
         why = "no strategy is valid for the shapes"
         if not _stand_in_on_error:

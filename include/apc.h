@@ -753,6 +753,23 @@ int apc_score_table(const apc_problem* p, const double* per_arg, const double* t
                     const double* init, double* out, void* stream);
 int apc_score_table_tile(void);
 
+/* Replaces remove_invalid_configs (autoparallel/shardings/propagation_rules.py:127-158)
+ * and keep_unique_configs (autoparallel/shardings/placement_options.py:151-170) for the
+ * candidate strategies of n_set nodes in packed form.  Set s has rows
+ * [set_row[s], set_row[s + 1]), each of set_width[s] spec words (the strategy's
+ * input specs, then its output specs; APC_SPEC_NONE for a missing one) starting at
+ * words[set_word[s]], row-major.  valid[row] = 1 if every spec of the row keeps
+ * every sharded dim non-empty (walking the mesh dims in order, Shard(d) needs the
+ * size of dim d, already divided by the earlier mesh dims that shard it, to be at
+ * least the mesh size); keep[row] = valid and no earlier valid row of the set has
+ * the same words (equal words stand for equal specs when the words were interned
+ * by value).  max_rows: the largest set's row count, at most 4096.  Word layout
+ * and tables as in apc_problem (meta_shape: [n_meta][APC_MAX_RANK]). */
+int apc_filter_strategies(const apc_model* model, int32_t n_meta, const int32_t* meta_rank,
+                          const int64_t* meta_shape, int32_t n_tuple, const uint8_t* tuple_plc, int32_t n_set,
+                          const int64_t* set_row, const int32_t* set_width, const int64_t* set_word,
+                          const uint32_t* words, int32_t max_rows, uint8_t* valid, uint8_t* keep, void* stream);
+
 /* Replaces _get_sharded_shape_stride
  * (autoparallel/cost_models/compute_estimation.py:300-318) for n specs:
  * rank[i], shape/stride[i][APC_MAX_RANK], plc[i][APC_MAX_MESH_DIMS] ->

@@ -356,6 +356,35 @@ def test_prefetch_discount_on_joint_graph(mesh):
     assert opt.strats[opt.nodes[k[0]]].strategies[k[2]].redistribute_cost[k[1]][k[3]] == 0.0
 
 
+def test_an_optimizer_is_freed_with_its_last_reference(mesh):
+    """The mappings the optimizer holds (decision_vars, cluster_links) refer back
+    to it weakly: no reference cycle keeps its strategies and coefficient arrays
+    alive until the cyclic collector next runs."""
+    import gc
+    import weakref
+
+    from autoparallel_amd.optimize_sharding import ShardingOptimizer
+
+    gm = _joint_graph()
+    was = gc.isenabled()
+    gc.disable()
+    try:
+        opt = ShardingOptimizer(gm, mesh, devices_per_host=8, device_name="AMD Instinct MI355X",
+                                repeated_subgraphs=True)
+        dvs, ref = opt.decision_vars, weakref.ref(opt)
+        key = next(iter(dvs))
+        dv = dvs[key]  # a view handed out keeps the optimizer alive
+        del opt
+        assert ref() is not None and dv.cost == dvs[key].cost
+        del dv
+        assert ref() is None
+        with pytest.raises(ReferenceError):
+            len(dvs)
+    finally:
+        if was:
+            gc.enable()
+
+
 def test_rebuild_after_mutating_strategies(mesh):
     """_build_decision_vars is re-entrant (reference tests/test_paired_output_constraint.py:30-158):
     after removing one placement from a gradient node's strategies, the rebuilt
