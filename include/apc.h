@@ -764,7 +764,7 @@ int apc_score_table_tile(void);
  * least the mesh size); keep[row] = valid and no earlier valid row of the set has
  * the same words (equal words stand for equal specs when the words were interned
  * by value).  max_rows: the largest set's row count, at most 4096.  Word layout
- * and tables as in apc_problem (meta_shape: [n_meta][APC_MAX_RANK]). */
+ * and tables are those of an apc_problem; meta_shape is [n_meta][APC_MAX_RANK]. */
 int apc_filter_strategies(const apc_model* model, int32_t n_meta, const int32_t* meta_rank,
                           const int64_t* meta_shape, int32_t n_tuple, const uint8_t* tuple_plc, int32_t n_set,
                           const int64_t* set_row, const int32_t* set_width, const int64_t* set_word,
