@@ -177,6 +177,10 @@ class DecisionVars(_OwnedByOptimizer, collections.abc.Mapping):
         v, a, o, j = key
         if not (0 <= v < g.num_nodes) or not (0 <= o < g.node_nstrat[v]):
             raise KeyError(key)
+        # a repeated (linked) node owns no variables, as in the reference, where decision_vars
+        # holds the keys of cluster roots and cluster_links maps a linked key to its root's
+        if self._opt._core.linked[v]:
+            raise KeyError(key)
         e = int(g.node_edge_off[v]) + a
         if a < 0 or e >= int(g.node_edge_off[v + 1]) or not (0 <= j < g.edge_ssrc[e]):
             raise KeyError(key)
@@ -206,7 +210,7 @@ class _ClusterLinks(_OwnedByOptimizer, collections.abc.Mapping):
     def __getitem__(self, key):
         v, a, o, j = key
         r = self._nodes.get(int(v))
-        if r is None or key not in self._opt.decision_vars:
+        if r is None or (r, int(a), int(o), int(j)) not in self._opt.decision_vars:
             raise KeyError(key)
         return (r, int(a), int(o), int(j))
 
@@ -308,9 +312,10 @@ class _Variables(collections.abc.Mapping):
 
     def __getitem__(self, key):
         opt = self._opt
-        col = opt.decision_vars._col(opt.cluster_links.get(key, key)) if key in opt.decision_vars else None
-        if col is None:
+        root_key = opt.cluster_links.get(key, key)  # a repeated node's variable is its root's
+        if root_key not in opt.decision_vars:
             raise KeyError(key)
+        col = opt.decision_vars._col(root_key)
         v, a, o, j = key
         return self._Var(f"n={opt.nodes[v]},s={v},arg={a},output_p={o},input_p={j}", col, opt.prob)
 
@@ -466,7 +471,8 @@ class ShardingOptimizer:
         return self.pulp_variables[key]
 
     def _resolve_decision_var(self, key) -> DecisionVar:
-        return self.decision_vars[key]
+        """The variable that stands for a key: its own, or its cluster root's (:446-460)."""
+        return self.decision_vars[self.cluster_links.get(key, key)]
 
     @classmethod
     def load(cls, path: str):
@@ -912,7 +918,7 @@ class ShardingOptimizer:
         sol = self._core._extract()
         by_node: Dict[torch.fx.Node, List[DecisionVar]] = {}
         for key in self.selected_keys:
-            by_node.setdefault(self.nodes[key[0]], []).append(self.decision_vars[key])
+            by_node.setdefault(self.nodes[key[0]], []).append(self._resolve_decision_var(key))
         del sol
         return log_formatting.format_sharding_log(self.graph, by_node, colored, verbose,
                                                   self.get_violated_constraints_log())

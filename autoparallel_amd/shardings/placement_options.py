@@ -20,6 +20,7 @@ import ctypes as C
 import itertools
 import logging
 import operator
+import threading
 from typing import Dict, List, Optional, Sequence
 
 import numpy as np
@@ -37,6 +38,7 @@ logger = logging.getLogger(__name__)
 
 fallback_nodes: List[str] = []  # nodes that got the implicit all-Replicate strategy
 fallback_reasons: Dict[str, str] = {}  # node name -> why its operator strategy was not used
+refused_candidates: List[str] = []  # one line per query in which a strategy rule refused some of the candidates
 
 # An operator without a registered strategy function gets the all-Replicate
 # stand-in, with a warning, as the reference's driver arranges
@@ -525,7 +527,7 @@ def _one_strategy_at_a_time(fn, op, args, kwargs, producers: List[OpStrategy]) -
         return a
 
     sts = []
-    refused = None
+    refused, n_refused = None, 0
     for lead_st in lead.strategies:
         if not isinstance(lead_st.output_specs, DTensorSpec):
             return None
@@ -536,13 +538,22 @@ def _one_strategy_at_a_time(fn, op, args, kwargs, producers: List[OpStrategy]) -
             # the rule has no answer for this candidate (a mean over shards of unequal size, ...):
             # the operator offers nothing that follows it, and reaching what it does offer
             # from that candidate is priced like any other redistribution
-            refused = exc
+            if refused is None:
+                refused = exc
+            n_refused += 1
             continue
         if not isinstance(res, OpStrategy):
             return None
         sts.extend(res.strategies)
     if not sts and refused is not None:
         raise refused
+    if n_refused:
+        # said out loud: a rule that refuses candidates narrows what the node offers, and a
+        # rule that does so by mistake would otherwise change plans without a trace
+        note = (f"{n_refused} of {len(lead.strategies)} candidates refused by the rule of `{op}`; first: "
+                f"{type(refused).__name__}: {refused}")
+        logger.warning("%s", note)
+        refused_candidates.append(note)
     return OpStrategy(sts)
 
 
@@ -957,6 +968,7 @@ def _zero_cost_rows(src_strategy, dst_spec):
 
 _cost_row_users: List = []  # modules of torch's strategy functions that hold generate_redistribute_costs
 _cost_row_users_at = -1     # len(sys.modules) when the list was made
+_cost_row_lock = threading.RLock()  # the patch below is a change to module globals: one thread at a time
 
 
 @contextlib.contextmanager
@@ -969,19 +981,24 @@ def _without_torch_cost_rows():
     import sys
 
     global _cost_row_users, _cost_row_users_at
-    if _cost_row_users_at != len(sys.modules):  # strategy modules are imported lazily
-        _cost_row_users = [mod for name, mod in list(sys.modules.items())
-                           if name.startswith("torch.distributed.tensor._ops") and mod is not None
-                           and "generate_redistribute_costs" in getattr(mod, "__dict__", {})]
-        _cost_row_users_at = len(sys.modules)
-    saved = [(mod, mod.__dict__["generate_redistribute_costs"]) for mod in _cost_row_users]
-    for mod, _ in saved:
-        mod.generate_redistribute_costs = _zero_cost_rows
-    try:
-        yield
-    finally:
-        for mod, fn in saved:
-            mod.generate_redistribute_costs = fn
+    # Process-wide while it lasts: other threads that enumerate strategies wait here, and a
+    # thread that runs DTensor operators meanwhile would see rows of zeros in the strategies it
+    # is handed (their specs are unaffected: no strategy function of the installed torch selects
+    # by those rows, which tests/test_placement_options_host.py checks on the operators in use).
+    with _cost_row_lock:
+        if _cost_row_users_at != len(sys.modules):  # strategy modules are imported lazily
+            _cost_row_users = [mod for name, mod in list(sys.modules.items())
+                               if name.startswith("torch.distributed.tensor._ops") and mod is not None
+                               and "generate_redistribute_costs" in getattr(mod, "__dict__", {})]
+            _cost_row_users_at = len(sys.modules)
+        saved = [(mod, mod.__dict__["generate_redistribute_costs"]) for mod in _cost_row_users]
+        for mod, _ in saved:
+            mod.generate_redistribute_costs = _zero_cost_rows
+        try:
+            yield
+        finally:
+            for mod, fn in saved:
+                mod.generate_redistribute_costs = fn
 
 
 def _placement_options_uncached(mesh, node, producers, arg_vals, schema_args) -> OpStrategy:

@@ -314,6 +314,14 @@ def test_repeated_subgraphs_on_joint_graph(mesh):
     for linked, root in opt.cluster_links.items():
         assert linked[1:] == root[1:] and linked[0] != root[0]
         assert str(opt.nodes[linked[0]].target) == str(opt.nodes[root[0]].target)
+    # as in the reference, decision_vars holds the root keys only; a linked key is resolved through the links
+    linked, root = next(iter(opt.cluster_links.items()))
+    assert root in opt.decision_vars and linked not in opt.decision_vars
+    with pytest.raises(KeyError):
+        opt.decision_vars[linked]
+    assert opt._resolve_decision_var(linked).key == root
+    assert opt.pulp_variables[linked].index == opt.pulp_variables[root].index
+    assert all(k[0] not in opt._cluster_linked_node_idxs for k in opt.decision_vars)
     sol = opt.get_solution()
     for v in opt._cluster_linked_node_idxs:
         r = opt._core.root[v]
