@@ -522,6 +522,49 @@ def test_torch_cost_rows_are_restored(meshes):
     assert OU.generate_redistribute_costs is real and MO.generate_redistribute_costs is real
 
 
+def test_strategies_do_not_depend_on_torchs_cost_rows(meshes):
+    """The strategy functions of the installed torch fill in cost rows but do not
+    select or order by them: with the rows made of zeros (as during a query) and
+    with torch's own rows, the operators a transformer graph uses answer with the
+    same input and output specs, in the same order."""
+    from torch.distributed.tensor import DTensor
+    from torch.distributed.tensor._op_schema import OpSchema
+
+    from torch.distributed.tensor.placement_types import Partial
+
+    from autoparallel_amd.shardings import placement_options as PO
+
+    mesh = meshes[1]  # (32, 8)
+    R, S, P = Replicate(), Shard, Partial()
+    x = _candidates(mesh, (64, 32), [(R, R), (S(0), R), (S(1), S(0)), (P, R)])
+    y = _candidates(mesh, (64, 32), [(R, R), (S(0), R), (R, S(1))])
+    w = _candidates(mesh, (32, 48), [(R, R), (R, S(1)), (S(0), R)])
+    x3 = _candidates(mesh, (32, 64, 32), [(R, R), (S(0), S(1)), (S(2), R)])
+    aten = torch.ops.aten
+    queries = [
+        (aten.add.Tensor, (x, y), {}), (aten.mul.Tensor, (x, y), {}), (aten.mm.default, (x, w), {}),
+        (aten.silu.default, (x,), {}), (aten.sum.dim_IntList, (x, [1], True), {}), (aten.mean.dim, (x, [-1], True), {}),
+        (aten._softmax.default, (x, -1, False), {}), (aten.t.default, (x,), {}), (aten.transpose.int, (x3, 1, 2), {}),
+        (aten.clone.default, (x,), {}), (aten._to_copy.default, (x,), {"dtype": torch.bfloat16}),
+        (aten.rsqrt.default, (x,), {}), (aten.neg.default, (x,), {}), (aten.pow.Tensor_Scalar, (x, 2), {}),
+        (aten.bmm.default, (x3, _candidates(mesh, (32, 32, 16), [(R, R), (S(0), R)])), {}),
+    ]
+    funcs = DTensor._op_dispatcher.sharding_propagator.op_strategy_funcs
+    asked = nonzero = 0
+    for op, args, kwargs in queries:
+        fn = funcs.get(op)
+        if fn is None:
+            continue
+        plain = fn(OpSchema(op, args, kwargs))
+        with PO._without_torch_cost_rows():
+            zeroed = fn(OpSchema(op, args, kwargs))
+        summary = lambda st: [(str(s.input_specs), str(s.output_specs)) for s in st.strategies]
+        assert summary(plain) == summary(zeroed), op
+        nonzero += any(c != 0 for s in plain.strategies for row in (s.redistribute_cost or []) for c in row)
+        asked += 1
+    assert asked >= 12 and nonzero >= 6  # torch's own rows really differ from the zeros
+
+
 def test_strategy_summaries_keep_the_cache_hits(meshes):
     """A query key holds one token per argument strategy; strategies with the
     same output specs get the same token wherever they come from, and tokens
