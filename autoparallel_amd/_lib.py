@@ -251,6 +251,10 @@ _SIGNATURES = {
         C.c_int,
         [C.POINTER(ApcProblem), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint64,
          C.c_int64, C.c_int64, C.c_void_p, C.c_void_p]),
+    "apc_score_assignments_window": (
+        C.c_int,
+        [C.POINTER(ApcProblem), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int32,
+         C.c_void_p, C.c_void_p, C.c_void_p]),
     "apc_random_assignment": (C.c_uint32, [C.c_uint64, C.c_int64, C.c_int32, C.c_int32]),
     "apc_sample_feasible": (
         C.c_int,

@@ -90,6 +90,15 @@ score_kernel(apc_problem p, const double* __restrict__ per_arg, const double* __
   r[5] = forbidden;
 }
 
+// x + 1.0 n times over.  While x is a whole number below 2^52 every step is exact, and so
+// is x + n in one step (what the carried sums are in practice: counts); anything else is
+// added one by one, as a sequential walk does.
+__device__ __forceinline__ double add_ones(double x, uint32_t n) {
+  if (x == floor(x) && fabs(x) < 4503599627370496.0 - 4294967296.0) return x + (double)n;
+  for (uint32_t i = 0; i < n; ++i) x += 1.0;
+  return x;
+}
+
 // In-order fold of one value per lane into acc: acc = (..((acc + v0) + v1)..) + v63,
 // the association a sequential loop over 64 items has.
 __device__ __forceinline__ double fold_in_order(double acc, double v) {
@@ -107,14 +116,21 @@ __device__ __forceinline__ double fold_in_order(double acc, double v) {
 // gathers of a tile overlap.
 // score_kernel<true> over a window of a larger graph: global node ids for the
 // draw, sums continued from the previous window's.
+template <bool kRandom>
 __global__ void __launch_bounds__(kBlock)
 score_window_kernel(apc_problem p, const double* __restrict__ per_arg,
                     const double* __restrict__ comm, const double* __restrict__ cost,
-                    const uint8_t* __restrict__ flags, uint64_t seed, int64_t first,
+                    const uint8_t* __restrict__ flags, const uint16_t* __restrict__ assign, int64_t stride,
+                    uint64_t seed, int64_t first,
                     int64_t n_assign, const int32_t* __restrict__ node_gid, int first_node,
                     const double* __restrict__ init, double* __restrict__ out) {
   const int64_t a = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (a >= n_assign) return;
+  // the choice at node v: drawn from its id in the whole graph, or read from the matrix
+  auto choice = [&](int v, int nstrat) -> uint32_t {
+    return kRandom ? mix_assignment(seed, first + a, node_gid ? node_gid[v] : v, nstrat)
+                   : (uint32_t)assign[(size_t)v * stride + a];
+  };
   double t_compute = 0.0, t_comm = 0.0, t_trans = 0.0, obj = 0.0, forbidden = 0.0;
   if (init) {
     const double* r = init + a * 6;
@@ -124,7 +140,7 @@ score_window_kernel(apc_problem p, const double* __restrict__ per_arg,
   if (first_node < p.n_node && p.node_edge_off[first_node] < p.n_edge)
     nxt = load_edge(p.edges + p.node_edge_off[first_node]);
   for (int v = first_node; v < p.n_node; ++v) {
-    const uint32_t o = mix_assignment(seed, first + a, node_gid[v], p.node_nstrat[v]);
+    const uint32_t o = choice(v, p.node_nstrat[v]);
     const int nargs = p.node_nargs[v];
     const double pa = per_arg[p.node_comp_off[v] + o];
     t_compute += pa * (double)(nargs > 1 ? nargs : 1);
@@ -133,8 +149,7 @@ score_window_kernel(apc_problem p, const double* __restrict__ per_arg,
       const apc_edge ed = nxt;
       if (e + 1 < p.n_edge) nxt = load_edge(p.edges + e + 1);
       uint32_t j = 0;
-      if (ed.src_node >= 0)
-        j = mix_assignment(seed, first + a, node_gid[ed.src_node], ed.ssrc);
+      if (ed.src_node >= 0) j = choice(ed.src_node, ed.ssrc);
       const int64_t idx = ed.off + (int64_t)o * ed.ssrc + j;
       const uint8_t f = flags[idx];
       obj += cost[idx] * mult;
@@ -642,14 +657,6 @@ score_table_kernel(apc_problem p, const double* __restrict__ per_arg, const doub
     for (int k = 0; k < kPer; ++k) t_compute[k] += pa[k] * fargs;
   }
   __builtin_amdgcn_s_waitcnt(0);  // nothing is in flight towards LDS when the workgroup ends
-  // x + 1.0 n times over.  While x is a whole number below 2^52 every step is exact, and so
-  // is x + n in one step (what the carried sums are in practice: counts); anything else is
-  // added one by one, as the other scorers do.
-  auto add_ones = [](double x, uint32_t n) -> double {
-    if (x == floor(x) && fabs(x) < 4503599627370496.0 - 4294967296.0) return x + (double)n;
-    for (uint32_t i = 0; i < n; ++i) x += 1.0;
-    return x;
-  };
 #pragma unroll
   for (int k = 0; k < kPer; ++k) {
     if (t_raw + k * lanes >= n_assign) continue;
@@ -700,16 +707,24 @@ score_wave_kernel(apc_problem p, const double* __restrict__ per_arg,
                   const double* __restrict__ comm, const double* __restrict__ cost,
                   const uint8_t* __restrict__ flags, const uint16_t* __restrict__ assign,
                   int64_t stride, uint64_t seed, int64_t first, int64_t n_assign,
+                  const int32_t* __restrict__ node_gid, int first_node, const double* __restrict__ init,
                   double* __restrict__ out) {
   const int64_t a = (int64_t)blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6);
   if (a >= n_assign) return;  // wave-uniform
   const int lane = threadIdx.x & 63;
   auto choice = [&](int v) -> uint32_t {
-    return kRandom ? mix_assignment(seed, first + a, v, p.node_nstrat[v])
+    return kRandom ? mix_assignment(seed, first + a, node_gid ? node_gid[v] : v, p.node_nstrat[v])
                    : (uint32_t)assign[(size_t)v * stride + a];
   };
+  // a window of a larger graph: the nodes below first_node (stand-ins) contribute nothing,
+  // and the sums continue from init
   double t_compute = 0.0, t_comm = 0.0, t_trans = 0.0, obj = 0.0, forbidden = 0.0;
-  for (int v0 = 0; v0 < p.n_node; v0 += 64) {
+  if (init) {
+    const double* r = init + a * 6;
+    t_compute = r[1]; t_comm = r[2]; t_trans = r[3]; obj = r[4]; forbidden = r[5];
+  }
+  const int e_first = first_node < p.n_node ? p.node_edge_off[first_node] : p.n_edge;
+  for (int v0 = first_node; v0 < p.n_node; v0 += 64) {
     const int v = v0 + lane;
     double term = 0.0;
     if (v < p.n_node) {
@@ -718,7 +733,7 @@ score_wave_kernel(apc_problem p, const double* __restrict__ per_arg,
     }
     t_compute = fold_in_order(t_compute, term);  // + 0.0 for the lanes past the end
   }
-  for (int e0 = 0; e0 < p.n_edge; e0 += 64) {
+  for (int e0 = e_first; e0 < p.n_edge; e0 += 64) {
     const int e = e0 + lane;
     double c_term = 0.0, o_term = 0.0, tr = 0.0, fb = 0.0;
     if (e < p.n_edge) {
@@ -737,13 +752,13 @@ score_wave_kernel(apc_problem p, const double* __restrict__ per_arg,
     }
     t_comm = fold_in_order(t_comm, c_term);
     obj = fold_in_order(obj, o_term);
-    // small integers: any order is exact
+    // small integers: any order is exact; onto the carried sums as so many ones
     for (int off = 32; off > 0; off >>= 1) {
       tr += __shfl_xor(tr, off, 64);
       fb += __shfl_xor(fb, off, 64);
     }
-    t_trans += tr;
-    forbidden += fb;
+    t_trans = add_ones(t_trans, (uint32_t)tr);
+    forbidden = add_ones(forbidden + 0.0, (uint32_t)fb);  // a walk adds 0.0 or 1.0 per edge: a carried -0.0 loses its sign
   }
   if (lane == 0) {
     double* r = out + a * 6;
@@ -796,10 +811,10 @@ static int launch_score(const apc_problem* p, const double* per_arg, const doubl
       const unsigned grid = (unsigned)((n + (kBlock / 64) - 1) / (kBlock / 64));
       if (random)
         hipLaunchKernelGGL(score_wave_kernel<true>, dim3(grid), dim3(kBlock), 0, stream, *p, per_arg,
-                           comm, cost, flags, asg, n_assign, seed, first + a0, n, o);
+                           comm, cost, flags, asg, n_assign, seed, first + a0, n, nullptr, 0, nullptr, o);
       else
         hipLaunchKernelGGL(score_wave_kernel<false>, dim3(grid), dim3(kBlock), 0, stream, *p,
-                           per_arg, comm, cost, flags, asg, n_assign, seed, first + a0, n, o);
+                           per_arg, comm, cost, flags, asg, n_assign, seed, first + a0, n, nullptr, 0, nullptr, o);
     } else {
       const unsigned grid = (unsigned)((n + kBlock - 1) / kBlock);
       if (random)
@@ -846,12 +861,45 @@ int apc_score_random_window(const apc_problem* p, const double* per_arg, const d
     return fail(APC_ERR_INVALID, "apc_score_random_window: null argument%s");
   if (first_node < 0 || first_node > p->n_node)
     return fail(APC_ERR_INVALID, "apc_score_random_window: first_node out of range%s");
+  if (n_assign < kScoreWaveBelow) {  // a wavefront per assignment
+    hipLaunchKernelGGL(score_wave_kernel<true>, dim3((unsigned)((n_assign + (kBlock / 64) - 1) / (kBlock / 64))),
+                       dim3(kBlock), 0, (hipStream_t)stream, *p, per_arg, comm, cost, flags, nullptr, n_assign, seed,
+                       first, n_assign, node_gid, (int)first_node, init, out);
+    return check_launch("score_wave_kernel");
+  }
   const int64_t kChunk = 262144;  // as launch_score
   for (int64_t a0 = 0; a0 < n_assign; a0 += kChunk) {
     const int64_t n = (n_assign - a0 < kChunk) ? (n_assign - a0) : kChunk;
-    hipLaunchKernelGGL(score_window_kernel, dim3((unsigned)((n + kBlock - 1) / kBlock)), dim3(kBlock),
-                       0, (hipStream_t)stream, *p, per_arg, comm, cost, flags, seed, first + a0, n,
+    hipLaunchKernelGGL(score_window_kernel<true>, dim3((unsigned)((n + kBlock - 1) / kBlock)), dim3(kBlock),
+                       0, (hipStream_t)stream, *p, per_arg, comm, cost, flags, nullptr, 0, seed, first + a0, n,
                        node_gid, first_node, init ? init + a0 * 6 : nullptr, out + a0 * 6);
+    if (int rc = check_launch("score_window_kernel")) return rc;
+  }
+  return 0;
+}
+
+int apc_score_assignments_window(const apc_problem* p, const double* per_arg, const double* comm,
+                                 const double* cost, const uint8_t* flags, const uint16_t* assign,
+                                 int64_t n_assign, int32_t first_node, const double* init, double* out,
+                                 void* stream) {
+  if (int rc = validate_problem(p)) return rc;
+  if (n_assign <= 0) return 0;
+  if (!per_arg || !comm || !cost || !flags || !out || !assign || !p->node_multiplier)
+    return fail(APC_ERR_INVALID, "apc_score_assignments_window: null argument%s");
+  if (first_node < 0 || first_node > p->n_node)
+    return fail(APC_ERR_INVALID, "apc_score_assignments_window: first_node out of range%s");
+  if (n_assign < kScoreWaveBelow) {  // a wavefront per assignment
+    hipLaunchKernelGGL(score_wave_kernel<false>, dim3((unsigned)((n_assign + (kBlock / 64) - 1) / (kBlock / 64))),
+                       dim3(kBlock), 0, (hipStream_t)stream, *p, per_arg, comm, cost, flags, assign, n_assign, 0, 0,
+                       n_assign, nullptr, (int)first_node, init, out);
+    return check_launch("score_wave_kernel");
+  }
+  const int64_t kChunk = 262144;  // as launch_score
+  for (int64_t a0 = 0; a0 < n_assign; a0 += kChunk) {
+    const int64_t n = (n_assign - a0 < kChunk) ? (n_assign - a0) : kChunk;
+    hipLaunchKernelGGL(score_window_kernel<false>, dim3((unsigned)((n + kBlock - 1) / kBlock)), dim3(kBlock),
+                       0, (hipStream_t)stream, *p, per_arg, comm, cost, flags, assign + a0, n_assign, 0, 0, n,
+                       nullptr, first_node, init ? init + a0 * 6 : nullptr, out + a0 * 6);
     if (int rc = check_launch("score_window_kernel")) return rc;
   }
   return 0;

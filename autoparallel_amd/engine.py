@@ -20,6 +20,11 @@ _SCORE_LANES_FROM = 32768  # assignments: below, one wavefront per assignment (e
 _SCORE_FROM_TABLE = True  # the three ways of scoring a graph with large blocks can be switched off (tests do)
 _SCORE_COMPACT = True
 _SCORE_STAGE_TILES = 8  # matrices of up to this many LDS tiles go through LDS in the table scorer
+# The table scorer pays about 2 us per edge whatever the batch (a matrix copied into LDS on every CU), the
+# walks over records about 14 ns per edge and assignment: from this many assignments on the table wins
+# (measured on a 3 000-node window of the stress DAG: 18 ms per window from the table for any batch up to
+# 2^20, 78 ms from compact records for 2^20)
+_SCORE_TABLE_FROM = 131072
 _SCORE_PER_LANE = 0  # assignments per lane of the compact scorer; 0: the library chooses
 _READBACK_PINNED = True  # results() copies into pinned host memory (else pageable)
 _LUT_TABLE_FROM = 2048  # table units: larger tables are built tile by tile with per-source terms in LDS
@@ -540,7 +545,8 @@ class CostEngine:
         cost is (comm + per_arg) + transition or its clamp (checked on the device
         when the records are made); else the 32-byte records that carry the cost
         (apc_score_packed)."""
-        if self._table_clamp is not None and _SCORE_FROM_TABLE and (self.large_blocks or not _SCORE_COMPACT):
+        if (self._table_clamp is not None and _SCORE_FROM_TABLE and (self.large_blocks or not _SCORE_COMPACT)
+                and count >= _SCORE_TABLE_FROM):
             aux = self._score_edge_aux(d_gid)
             _lib.check(
                 self.lib.apc_score_table(
@@ -706,8 +712,9 @@ class CostEngine:
         assert init is None or (init.shape == (count, 6) and init.dtype == torch.float64 and init.is_contiguous())
         d_gid = torch.from_numpy(gid).to(self.device)
         out = torch.empty((count, 6), dtype=torch.float64, device=self.device)
-        if self.packed_scoring:
+        if self.packed_scoring and count >= _SCORE_LANES_FROM:
             return self._score_packed(None, seed, first, count, d_gid, first_node, init, out)
+        self.last_score_backend = "entry_arrays"
         _lib.check(
             self.lib.apc_score_random_window(
                 C.byref(self.problem), self._ptr(self.per_arg), self._ptr(self.comm), self._ptr(self.cost),
@@ -728,9 +735,16 @@ class CostEngine:
         assert 0 <= first_node <= self.g.num_nodes
         assert init is None or (init.shape == (count, 6) and init.dtype == torch.float64 and init.is_contiguous())
         out = torch.empty((count, 6), dtype=torch.float64, device=self.device)
-        if not self.packed_scoring:
-            raise _lib.ApcError("score_window needs a graph with entries")
-        return self._score_packed(assign, 0, 0, count, None, first_node, init, out)
+        if self.packed_scoring and count >= _SCORE_LANES_FROM:
+            return self._score_packed(assign, 0, 0, count, None, first_node, init, out)
+        _lib.check(
+            self.lib.apc_score_assignments_window(
+                C.byref(self.problem), self._ptr(self.per_arg), self._ptr(self.comm), self._ptr(self.cost),
+                self._ptr(self.flags), self._ptr(assign), count, int(first_node), self._ptr(init), self._ptr(out),
+                self._stream()),
+            "apc_score_assignments_window")
+        self.last_score_backend = "entry_arrays"
+        return out
 
     def sample_feasible(self, seed: int, first: int, count: int, node_gid: Optional[np.ndarray] = None,
                         first_node: int = 0, assign: Optional[torch.Tensor] = None):

@@ -672,6 +672,15 @@ int apc_score_random_window(const apc_problem* p, const double* per_arg, const d
                             int64_t first, int64_t n_assign, const int32_t* node_gid,
                             int32_t first_node, const double* init, double* out, void* stream);
 
+/* apc_score_assignments for a window of a larger graph: the first first_node
+ * nodes (stand-ins for producers outside the window, whose rows of assign carry
+ * the choices made for them) contribute nothing, and the sums continue from init
+ * (double[n_assign][6], or NULL to start from zero).  assign: uint16[n_node][n_assign]. */
+int apc_score_assignments_window(const apc_problem* p, const double* per_arg, const double* comm,
+                                 const double* cost, const uint8_t* flags, const uint16_t* assign,
+                                 int64_t n_assign, int32_t first_node, const double* init, double* out,
+                                 void* stream);
+
 /* The three entry arrays interleaved, for scoring graphs whose edge blocks are
  * large: a drawn entry then costs one 32-byte gather instead of three gathers in
  * three arrays (measured 2x on blocks of 65 k entries, nothing on blocks of

@@ -25,9 +25,13 @@ def E():
 
 @pytest.fixture()
 def knobs(E):
-    saved = (E._SCORE_FROM_TABLE, E._SCORE_COMPACT, E._SCORE_STAGE_TILES, E._SCORE_PER_LANE)
+    saved = (E._SCORE_FROM_TABLE, E._SCORE_COMPACT, E._SCORE_STAGE_TILES, E._SCORE_PER_LANE, E._SCORE_TABLE_FROM,
+             E._SCORE_LANES_FROM)
+    # the table scorer and the record walks whatever the batch size, where a test asks for them
+    E._SCORE_TABLE_FROM = 0
     yield E
-    E._SCORE_FROM_TABLE, E._SCORE_COMPACT, E._SCORE_STAGE_TILES, E._SCORE_PER_LANE = saved
+    (E._SCORE_FROM_TABLE, E._SCORE_COMPACT, E._SCORE_STAGE_TILES, E._SCORE_PER_LANE, E._SCORE_TABLE_FROM,
+     E._SCORE_LANES_FROM) = saved
 
 
 def _same(a, b):
@@ -191,6 +195,7 @@ def test_small_batches_and_node_ranges(knobs):
     g = GRAPHS["stress"]()
     eng = E.CostEngine(g).build(clamp_inf=True)
     gid = np.arange(g.num_nodes, dtype=np.int32) * 3 + 5
+    E._SCORE_LANES_FROM = 0  # the batch scorers for these small batches too
     for n in (1, 7, 1000):
         eng.packed_scoring = False
         want = eng.score_random_window(3, 11, n, gid, 0)

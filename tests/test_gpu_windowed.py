@@ -103,3 +103,29 @@ def test_config5_at_full_size_in_windows():
     second, st2 = windowed.score_in_windows(200000, 4500, n, workers=14)
     assert st2["entries"] == st["entries"] and st2["windows"] == 45
     assert (first.view(np.uint64) == second.view(np.uint64)).all()
+
+
+def test_small_batches_of_explicit_assignments_in_a_window():
+    """apc_score_assignments_window (entry arrays, a lane per assignment) gives the
+    sums of the batch scorers for the same window, stand-ins and carried sums
+    included."""
+    from autoparallel_amd import engine as E
+    from autoparallel_amd.engine import CostEngine
+
+    g, gid, n_standin = graphgen.stress_dag_window(N_TOTAL, 100, 200, (4, 8, 8), SEED, 4, S_MAX)
+    assert n_standin > 0
+    eng = CostEngine(g).build(clamp_inf=True)
+    n = 500
+    rng = np.random.default_rng(0)
+    assign = torch.from_numpy(np.stack([rng.integers(0, s, n) for s in g.node_nstrat]).astype(np.int16)).cuda()
+    init = torch.rand(n, 6, dtype=torch.float64, device="cuda")
+    got = eng.score_window(assign, n_standin, init=init)
+    assert eng.last_score_backend == "entry_arrays"
+    saved = E._SCORE_LANES_FROM
+    try:
+        E._SCORE_LANES_FROM = 0
+        want = eng.score_window(assign, n_standin, init=init)
+        assert eng.last_score_backend != "entry_arrays"
+    finally:
+        E._SCORE_LANES_FROM = saved
+    assert torch.equal(got.view(torch.int64), want.view(torch.int64))
