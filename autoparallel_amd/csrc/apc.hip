@@ -884,6 +884,135 @@ edge_cost_kernel(apc_problem p, const double* __restrict__ table,
   if (have) item_store(cur, cur_r, comm, cost, flags, clamp_inf);
 }
 
+// One wavefront per work item, nothing predicated: the form the launcher takes
+// whenever all three outputs are asked for and the grid can hold a wave per item
+// (it always can below 8.6e9 entries).  A wave's life is a chain of dependent
+// accesses (item record, index loads of a compressed matrix, matrix and per-arg
+// loads, stores) and the chip hides it with the waves it holds, so the body is
+// written for few registers: no loop state, and lanes outside the block (before
+// its first entry in the block's first item, past its last in the last one) repeat
+// the nearest entry of the block (same loads, same values stored to the same
+// place) instead of being switched off, which keeps every access of the wave
+// unconditional.
+//
+// What depends on an entry's row alone (the per-arg compute term, the row's index
+// in a compressed matrix) is not loaded per entry.  Lane r of the wave loads the
+// values of the item's r-th row, one coalesced load each, and an entry takes its
+// row's values from that lane through the cross-lane network; only an item of
+// more than 64 rows (rows shorter than 9 entries) loads per entry.  Measured on
+// MI355X (264 M entries of compressed matrices): a vector load whose lanes all
+// read one address costs about as much as a 64-way gather; with eight such loads
+// of the row index per lane the kernel took 1.11 ms, without them 0.86 ms.  (The
+// scalar cache is no way out for the per-arg terms: they are written by the
+// launch before this one, and scalar loads of them returned values of an earlier
+// build in a test.)
+template <bool kSqueezed, int kN>
+__global__ void __launch_bounds__(kBlock)
+edge_cost_item_kernel(apc_problem p, const double* __restrict__ table,
+                      const double* __restrict__ per_arg, double* __restrict__ comm,
+                      double* __restrict__ cost, uint8_t* __restrict__ flags, int clamp_inf) {
+  unsigned wg = blockIdx.x;
+  if (kN > kPerLane) {  // runs of workgroups per XCD: see edge_cost_kernel
+    const unsigned k = wg >> 3, xcd = wg & 7;
+    wg = ((k / kXcdRun) * 8 + xcd) * kXcdRun + (k % kXcdRun);
+  }
+  const int i = __builtin_amdgcn_readfirstlane((int)(wg * (kBlock / 64) + (threadIdx.x >> 6)));
+  if (i >= p.n_item) return;
+  const int lane = threadIdx.x & 63;
+  const apc_edge ed = p.items[i];
+  const uint32_t ssrc = (uint32_t)ed.ssrc;
+  const uint32_t last = ssrc * (uint32_t)ed.sdst - 1u;
+  const uint32_t last_row = (uint32_t)ed.sdst - 1u;
+  const bool compressed = kSqueezed && (ed.flags & APC_EDGE_COMPRESSED);  // wave-uniform
+  const uint32_t usrc = (uint32_t)ed.flags >> APC_EDGE_USRC_SHIFT;
+  const int32_t* __restrict__ list_uidx = p.list_uidx;
+  const double* __restrict__ matrix =  // wave-uniform
+      ed.table_off >= 0 ? table + ed.table_off : p.default_vals + ed.default_off;
+  uint32_t l[kN], o[kN], urow[kN];
+  double pa[kN];
+#pragma unroll
+  for (int k = 0; k < kN; ++k) {
+    // the first item of a block may start up to 48 slots before it (local0 negative
+    // modulo 2^32): those lanes repeat the block's first entry, the ones past its end the last
+    const int32_t lk = (int32_t)ed.local0 + (k * 64 + lane);
+    l[k] = (uint32_t)(lk < 0 ? 0 : (lk > (int32_t)last ? (int32_t)last : lk));
+    o[k] = ed.magic ? __umulhi(l[k], ed.magic) : l[k] / ssrc;
+    urow[k] = 0;
+  }
+  // rows of the item: from the row of its first entry (lane 0) to that of its last (lane 63)
+  const uint32_t o_first = (uint32_t)__builtin_amdgcn_readfirstlane((int)o[0]);
+  const uint32_t o_last = (uint32_t)__builtin_amdgcn_readlane((int)o[kN - 1], 63);
+  if (o_last - o_first < 64u) {
+    const uint32_t row = o_first + (uint32_t)lane < last_row ? o_first + (uint32_t)lane : last_row;
+    const double pa_row = per_arg[ed.comp_base + row];
+    const int pa_lo = (int)(uint32_t)__double_as_longlong(pa_row);
+    const int pa_hi = (int)(uint32_t)((uint64_t)__double_as_longlong(pa_row) >> 32);
+    const int u_row = compressed ? list_uidx[(size_t)ed.dst_list + row] : 0;
+    if (ssrc >= 64) {
+      // 64 consecutive entries of rows this long lie in two rows at most: that of lane 0's
+      // entry and the next, both read from their lanes by the whole wave
+#pragma unroll
+      for (int k = 0; k < kN; ++k) {
+        const int ra = (int)((uint32_t)__builtin_amdgcn_readfirstlane((int)o[k]) - o_first);
+        const int rb = ra < 63 ? ra + 1 : 63;
+        const bool first = (int)(o[k] - o_first) == ra;
+        const uint32_t lo = (uint32_t)(first ? __builtin_amdgcn_readlane(pa_lo, ra) : __builtin_amdgcn_readlane(pa_lo, rb));
+        const uint32_t hi = (uint32_t)(first ? __builtin_amdgcn_readlane(pa_hi, ra) : __builtin_amdgcn_readlane(pa_hi, rb));
+        pa[k] = __longlong_as_double((long long)(((uint64_t)hi << 32) | lo));
+        if (compressed)
+          urow[k] = (uint32_t)(first ? __builtin_amdgcn_readlane(u_row, ra) : __builtin_amdgcn_readlane(u_row, rb));
+      }
+    } else {
+#pragma unroll
+      for (int k = 0; k < kN; ++k) {
+        const int from = (int)((o[k] - o_first) << 2);  // byte address of the lane that holds the row
+        const uint32_t lo = (uint32_t)__builtin_amdgcn_ds_bpermute(from, pa_lo);
+        const uint32_t hi = (uint32_t)__builtin_amdgcn_ds_bpermute(from, pa_hi);
+        pa[k] = __longlong_as_double((long long)(((uint64_t)hi << 32) | lo));
+        if (compressed) urow[k] = (uint32_t)__builtin_amdgcn_ds_bpermute(from, u_row);
+      }
+    }
+  } else {
+#pragma unroll
+    for (int k = 0; k < kN; ++k) {
+      pa[k] = per_arg[ed.comp_base + o[k]];
+      if (compressed) urow[k] = (uint32_t)list_uidx[(size_t)ed.dst_list + o[k]];
+    }
+  }
+  uint32_t at[kN];
+  if (compressed) {
+    // the matrix has one row / column per distinct spec word of the two runs
+#pragma unroll
+    for (int k = 0; k < kN; ++k)
+      at[k] = urow[k] * usrc + (uint32_t)list_uidx[(size_t)ed.src_list + (l[k] - o[k] * ssrc)];
+  } else {
+#pragma unroll
+    for (int k = 0; k < kN; ++k) at[k] = l[k];
+  }
+  double raw[kN];
+#pragma unroll
+  for (int k = 0; k < kN; ++k) raw[k] = matrix[at[k]];
+#pragma unroll
+  for (int k = 0; k < kN; ++k) {
+    const int trans = (int)((uint64_t)__double_as_longlong(raw[k]) >> 63);
+    const double cm = fabs(raw[k]);
+    double c = (cm + pa[k]) + (double)trans;  // optimize_sharding.py:544
+    const bool finite = isfinite(c);
+    if (clamp_inf && !finite) c = 10000.0;
+    const int64_t idx = ed.off + l[k];
+    const uint8_t f = (uint8_t)(trans | (finite ? 0 : APC_ENTRY_NONFINITE));
+    if (kN > kPerLane) {  // outputs that stream past every cache: see item_store
+      __builtin_nontemporal_store(cm, comm + idx);
+      __builtin_nontemporal_store(c, cost + idx);
+      __builtin_nontemporal_store(f, flags + idx);
+    } else {
+      comm[idx] = cm;
+      cost[idx] = c;
+      flags[idx] = f;
+    }
+  }
+}
+
 // Plain copy kernel of known size: the reference point against which the
 // hardware traffic counters are scaled when a profile is taken.
 __global__ void __launch_bounds__(kBlock)
@@ -1081,7 +1210,25 @@ static int launch_edge_costs(const apc_problem* p, const double* table, const do
 #define APC_LAUNCH_EDGE(MODE, N)                                                                   \
   hipExtLaunchKernelGGL((edge_cost_kernel<MODE, N>), dim3(grid), dim3(kBlock), 0, stream, start,   \
                         stop, 0, *p, table, per_arg, comm, cost, flags, clamp_inf)
-  if (table && p->list_uidx) {
+#define APC_LAUNCH_ITEMS(SQ, N)                                                                    \
+  hipExtLaunchKernelGGL((edge_cost_item_kernel<SQ, N>), dim3(grid), dim3(kBlock), lds, stream,    \
+                        start, stop, 0, *p, table, per_arg, comm, cost, flags, clamp_inf)
+  const bool wave_per_item = table && comm && cost && flags && (unsigned)((p->n_item + 3) / 4) <= cap;
+  // Waves per SIMD of the wave-per-item kernel.  It fits eight, and a problem whose block
+  // table is far larger than the caches wants them all (264 M entries over a table of
+  // 100 MB and more: 0.95 ms with eight, 1.13 ms with four).  A large problem whose table
+  // the L2s can hold is bound by its stores alone and runs best with four (418 M entries,
+  // table of 15 MB: 1.19 ms against 1.27 ms with eight; a plain fill of the same bytes takes
+  // 1.18 ms).  The kernel uses no LDS, so a workgroup that asks for a quarter of a CU's
+  // 160 KB limits a CU to four workgroups: one wave per SIMD each.
+  const size_t lds = wide && (size_t)p->table_size * sizeof(double) <= ((size_t)32 << 20) ? (size_t)40 << 10 : 0;
+  if (wave_per_item) {
+    if (p->list_uidx) {
+      if (wide) APC_LAUNCH_ITEMS(true, 2 * kPerLane); else APC_LAUNCH_ITEMS(true, kPerLane);
+    } else {
+      if (wide) APC_LAUNCH_ITEMS(false, 2 * kPerLane); else APC_LAUNCH_ITEMS(false, kPerLane);
+    }
+  } else if (table && p->list_uidx) {
     if (wide) APC_LAUNCH_EDGE(2, 2 * kPerLane); else APC_LAUNCH_EDGE(2, kPerLane);
   } else if (table) {
     if (wide) APC_LAUNCH_EDGE(1, 2 * kPerLane); else APC_LAUNCH_EDGE(1, kPerLane);
@@ -1089,6 +1236,7 @@ static int launch_edge_costs(const apc_problem* p, const double* table, const do
     APC_LAUNCH_EDGE(0, kPerLane);
   }
 #undef APC_LAUNCH_EDGE
+#undef APC_LAUNCH_ITEMS
   return check_launch("edge_cost_kernel");
 }
 

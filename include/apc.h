@@ -354,9 +354,13 @@ typedef struct apc_problem {
  *                           the nodes only)
  *   apc_build_pair_table    the table part of the above alone
  *   apc_node_compute_costs  the node part of the above alone
- *   apc_edge_costs          with a table: edge_cost_kernel<1,n> (full matrices) or
- *                           <2,n> (compressed: list_uidx set), n = 4 or 8 entries per
- *                           lane by item_entries; table == NULL: lut_kernel<entries>
+ *   apc_edge_costs          with a table and all three outputs: edge_cost_item_kernel
+ *                           <compressed,n>, one wavefront per work item (compressed:
+ *                           list_uidx set; n = 4 or 8 entries per lane by
+ *                           item_entries); with an output left out (or more than
+ *                           16.7 M work items): edge_cost_kernel<1,n> / <2,n>, the same
+ *                           arithmetic in a loop of predicated accesses;
+ *                           table == NULL: lut_kernel<entries>
  *                           when the problem carries lut_entry_tiles, else
  *                           edge_cost_kernel<0,4>, the per-entry fold (the fallback
  *                           for problems without spec_recs; a third of the rate)

@@ -441,6 +441,39 @@ def test_work_items_of_512_entries(CostEngine, mode):
         CostEngine(g, table_mode="direct", item_entries=512, lut=False).build()
 
 
+@pytest.mark.parametrize("mode", ["full", "compressed"])
+@pytest.mark.parametrize("item_entries", [256, 512])
+def test_entry_kernel_with_an_output_left_out(CostEngine, mode, item_entries):
+    """With all three outputs apc_edge_costs runs a wavefront per work item, nothing
+    predicated; with one left out, the loop kernel.  Same bits in what both write,
+    and the one left out stays untouched."""
+    for make in (GRAPHS["llama_2d"], GRAPHS["stress_3d"], _edge_case_graph):
+        g = make()
+        eng = CostEngine(g, table_mode=mode, item_entries=item_entries).build(clamp_inf=True)
+        want = eng.results()
+        slots = np.zeros(g.num_slots, bool)  # the slots that hold an entry; blocks are padded to 16
+        for e in range(g.num_edges):
+            slots[int(g.edge_off[e]): int(g.edge_off[e]) + int(g.edge_sdst[e]) * int(g.edge_ssrc[e])] = True
+        for skip in (None, "comm", "flags"):
+            eng.comm.fill_(-7.0)
+            eng.cost.fill_(-7.0)
+            eng.flags.fill_(0x55)
+            eng.edge_costs(clamp_inf=True, want_comm=skip != "comm", want_flags=skip != "flags")
+            got = eng.results()
+            assert bits_equal(got["cost"][slots], want["cost"][slots])
+            if skip == "comm":
+                assert (got["comm"] == -7.0).all()
+            else:
+                assert bits_equal(got["comm"][slots], want["comm"][slots])
+            if skip == "flags":
+                assert (got["flags"] == 0x55).all()
+            else:
+                assert (got["flags"][slots] == want["flags"][slots]).all()
+            # neither kernel writes between the blocks (the lanes of the unpredicated one that
+            # fall outside a block repeat an entry of the block)
+            assert (got["cost"][~slots] == -7.0).all() and (got["flags"][~slots] == 0x55).all()
+
+
 @pytest.mark.parametrize("rank,n_args", [(1, 15), (2, 16)])
 def test_more_arguments_than_the_node_record_holds(CostEngine, rank, n_args):
     """Arguments past the 14 runs kept in a node's record are found through the
