@@ -128,17 +128,27 @@ sample_feasible_wave_kernel(apc_problem p, const uint8_t* __restrict__ flags, ui
     const int e0 = p.node_edge_off[v], e1 = p.node_edge_off[v + 1];
     uint32_t count = 0;
     int pick = -1;
+    // The producers' choices (written by this wave's lane 0, or by the caller): lane i reads
+    // that of argument row i, and the wave takes them from there.  One load whose 64 lanes
+    // all read the same address costs as much as a 64-way gather on this chip.
+    int j_of = 0;
+    if (e0 + lane < e1) {
+      const int u = p.edges[e0 + lane].src_node;
+      j_of = u >= 0 ? (int)assign[(size_t)u * n_assign + a] : 0;
+    }
     for (int o0 = 0; o0 < S; o0 += 64) {
       const int o = o0 + lane;
       uint32_t bad = o < S ? 0u : (uint32_t)APC_ENTRY_NONFINITE;
-      if (o < S) {
-        for (int e = e0; e < e1; ++e) {
-          const apc_edge* ed = p.edges + e;  // wave-uniform: scalar loads
+      for (int e = e0; e < e1; ++e) {
+        const apc_edge* ed = p.edges + e;  // wave-uniform: scalar loads
+        uint32_t j;
+        if (e - e0 < 64) {
+          j = (uint32_t)__builtin_amdgcn_readlane(j_of, e - e0);
+        } else {  // more argument rows than lanes
           const int u = ed->src_node;
-          // the producer's choice was written by this wave (lane 0) or by the caller
-          const uint32_t j = u >= 0 ? (uint32_t)assign[(size_t)u * n_assign + a] : 0u;
-          bad |= flags[ed->off + (int64_t)o * ed->ssrc + j];
+          j = u >= 0 ? (uint32_t)assign[(size_t)u * n_assign + a] : 0u;
         }
+        if (o < S) bad |= flags[ed->off + (int64_t)o * ed->ssrc + j];
       }
       const bool allowed = !(bad & APC_ENTRY_NONFINITE);
       const uint64_t mask = __ballot(allowed);
