@@ -896,16 +896,17 @@ edge_cost_kernel(apc_problem p, const double* __restrict__ table,
 // unconditional.
 //
 // What depends on an entry's row alone (the per-arg compute term, the row's index
-// in a compressed matrix) is not loaded per entry.  Lane r of the wave loads the
-// values of the item's r-th row, one coalesced load each, and an entry takes its
-// row's values from that lane through the cross-lane network; only an item of
-// more than 64 rows (rows shorter than 9 entries) loads per entry.  Measured on
-// MI355X (264 M entries of compressed matrices): a vector load whose lanes all
-// read one address costs about as much as a 64-way gather; with eight such loads
-// of the row index per lane the kernel took 1.11 ms, without them 0.86 ms.  (The
-// scalar cache is no way out for the per-arg terms: they are written by the
-// launch before this one, and scalar loads of them returned values of an earlier
-// build in a test.)
+// in a compressed matrix) is not loaded per entry with one vector load whose lanes
+// all read the same address: such a load costs about as much as a 64-way gather
+// on this chip.  Measured on MI355X (264 M entries of compressed matrices): with
+// eight such loads of the row index per lane the kernel took 1.11 ms, without them
+// 0.86 ms.  Rows of 64 entries and more: 64 consecutive entries lie in two rows
+// at most, the same two for the whole wave, so their values come through the
+// scalar cache and a lane picks one of the two (0.86 ms).  Shorter rows: lane r of
+// the wave loads the values of the item's r-th row, one coalesced load each, and an
+// entry takes its row's values from that lane through the cross-lane network
+// (0.95 ms when rows of every length go this way); only an item of more than 64 rows
+// (rows shorter than 9 entries) loads per entry.
 template <bool kSqueezed, int kN>
 __global__ void __launch_bounds__(kBlock)
 edge_cost_item_kernel(apc_problem p, const double* __restrict__ table,
@@ -942,35 +943,36 @@ edge_cost_item_kernel(apc_problem p, const double* __restrict__ table,
   // rows of the item: from the row of its first entry (lane 0) to that of its last (lane 63)
   const uint32_t o_first = (uint32_t)__builtin_amdgcn_readfirstlane((int)o[0]);
   const uint32_t o_last = (uint32_t)__builtin_amdgcn_readlane((int)o[kN - 1], 63);
-  if (o_last - o_first < 64u) {
+  if (ssrc >= 64) {
+    // 64 consecutive entries of rows this long lie in two rows at most, that of lane 0's
+    // entry and the next: the same two addresses for the whole wave, read through the
+    // scalar cache, and a lane picks one of the two values
+#pragma unroll
+    for (int k = 0; k < kN; ++k) {
+      const uint32_t oa = (uint32_t)__builtin_amdgcn_readfirstlane((int)o[k]);
+      const uint32_t ob = oa < last_row ? oa + 1u : last_row;
+      const double pa_a = per_arg[ed.comp_base + oa], pa_b = per_arg[ed.comp_base + ob];
+      pa[k] = o[k] == oa ? pa_a : pa_b;
+      if (compressed) {
+        const uint32_t u_a = (uint32_t)list_uidx[(size_t)ed.dst_list + oa];
+        const uint32_t u_b = (uint32_t)list_uidx[(size_t)ed.dst_list + ob];
+        urow[k] = o[k] == oa ? u_a : u_b;
+      }
+    }
+  } else if (o_last - o_first < 64u) {
+    // lane r loads the values of the item's r-th row; an entry takes its row's from there
     const uint32_t row = o_first + (uint32_t)lane < last_row ? o_first + (uint32_t)lane : last_row;
     const double pa_row = per_arg[ed.comp_base + row];
     const int pa_lo = (int)(uint32_t)__double_as_longlong(pa_row);
     const int pa_hi = (int)(uint32_t)((uint64_t)__double_as_longlong(pa_row) >> 32);
     const int u_row = compressed ? list_uidx[(size_t)ed.dst_list + row] : 0;
-    if (ssrc >= 64) {
-      // 64 consecutive entries of rows this long lie in two rows at most: that of lane 0's
-      // entry and the next, both read from their lanes by the whole wave
 #pragma unroll
-      for (int k = 0; k < kN; ++k) {
-        const int ra = (int)((uint32_t)__builtin_amdgcn_readfirstlane((int)o[k]) - o_first);
-        const int rb = ra < 63 ? ra + 1 : 63;
-        const bool first = (int)(o[k] - o_first) == ra;
-        const uint32_t lo = (uint32_t)(first ? __builtin_amdgcn_readlane(pa_lo, ra) : __builtin_amdgcn_readlane(pa_lo, rb));
-        const uint32_t hi = (uint32_t)(first ? __builtin_amdgcn_readlane(pa_hi, ra) : __builtin_amdgcn_readlane(pa_hi, rb));
-        pa[k] = __longlong_as_double((long long)(((uint64_t)hi << 32) | lo));
-        if (compressed)
-          urow[k] = (uint32_t)(first ? __builtin_amdgcn_readlane(u_row, ra) : __builtin_amdgcn_readlane(u_row, rb));
-      }
-    } else {
-#pragma unroll
-      for (int k = 0; k < kN; ++k) {
-        const int from = (int)((o[k] - o_first) << 2);  // byte address of the lane that holds the row
-        const uint32_t lo = (uint32_t)__builtin_amdgcn_ds_bpermute(from, pa_lo);
-        const uint32_t hi = (uint32_t)__builtin_amdgcn_ds_bpermute(from, pa_hi);
-        pa[k] = __longlong_as_double((long long)(((uint64_t)hi << 32) | lo));
-        if (compressed) urow[k] = (uint32_t)__builtin_amdgcn_ds_bpermute(from, u_row);
-      }
+    for (int k = 0; k < kN; ++k) {
+      const int from = (int)((o[k] - o_first) << 2);  // byte address of the lane that holds the row
+      const uint32_t lo = (uint32_t)__builtin_amdgcn_ds_bpermute(from, pa_lo);
+      const uint32_t hi = (uint32_t)__builtin_amdgcn_ds_bpermute(from, pa_hi);
+      pa[k] = __longlong_as_double((long long)(((uint64_t)hi << 32) | lo));
+      if (compressed) urow[k] = (uint32_t)__builtin_amdgcn_ds_bpermute(from, u_row);
     }
   } else {
 #pragma unroll
