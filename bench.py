@@ -48,9 +48,9 @@ def workloads():
 
 
 def read_traffic(workload):
-    """HBM bytes per launch of edge_cost_kernel from the committed rocprofv3
-    counter summary (profiles/edge_cost_kernel_<workload>_traffic.txt), if any."""
-    path = os.path.join(ROOT, "profiles", f"edge_cost_kernel_{workload}_traffic.txt")
+    """HBM bytes per launch of the entry kernel from the committed rocprofv3
+    counter summary (profiles/edge_cost_item_kernel_<workload>_traffic.txt), if any."""
+    path = os.path.join(ROOT, "profiles", f"edge_cost_item_kernel_{workload}_traffic.txt")
     if not os.path.exists(path):
         return None
     for line in open(path):
@@ -293,7 +293,8 @@ def main():
             "phases_s": e2e,
         },
         "roofline": {
-            "kernel": "edge_cost_kernel" if eng.use_table or eng._lut_tiles is None else "lut_kernel<entries>",
+            "kernel": "edge_cost_item_kernel" if eng.use_table else
+                      ("edge_cost_kernel<0,4>" if eng._lut_tiles is None else "lut_kernel<entries>"),
             "bound": "hbm",
             "achieved": achieved,
             "peak": HBM_PEAK_GBS,
@@ -311,7 +312,7 @@ def main():
             "frac_at_8B": (8 * E + desc_bytes) / t_edge / 1e9 / HBM_PEAK_GBS,
             "step_frac_at_8B": (8 * E + desc_bytes) / (elapsed / args.steps) / 1e9 / HBM_PEAK_GBS,
             "traffic": read_traffic(args.workload),
-            "traffic_source": "profiles/edge_cost_kernel_%s_traffic.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE "
+            "traffic_source": "profiles/edge_cost_item_kernel_%s_traffic.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE "
                               "runs of this command, scaled by the copy kernel; not a quantity of this run)"
                               % args.workload,
         },
