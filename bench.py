@@ -339,6 +339,27 @@ def main():
                                "construction: each edge's inp_idx is its producer's draw), not ILP-feasible plans",
             "fraction_without_forbidden_entry": float((scores[:, 5] == 0).double().mean().item()),
         }
+        # The bound that applies to this launch.  Its inputs are the 16-byte records of the
+        # entries (one per slot) and 48 B of sums per assignment: that is all HBM has to
+        # deliver, once.  An assignment then reads one record per edge at a position its
+        # draws decide: random 16-byte reads served by L2 and the memory-side cache, at
+        # the rate at which a CU gets cache misses served.  Counted against HBM the
+        # requested bytes exceed the peak, which is why no HBM fraction is claimed.
+        reads = n * g.num_edges
+        hbm_bytes = 16 * g.num_slots + 48 * n
+        out["scoring"]["roofline"] = {
+            "kernel": "score_compact_kernel" if eng.last_score_backend == "compact_records" else eng.last_score_backend,
+            "bound": "cache-miss service rate (random 16-byte reads of records resident in L2 and the "
+                     "memory-side cache); not HBM, not MFMA",
+            "achieved": reads / t_score,
+            "unit": "random reads/s",
+            "per_cu_per_ns": reads / t_score / 256 / 1e9,
+            "peak": None,
+            "requested_bytes_per_s": 16 * reads / t_score,
+            "requested_bytes_over_hbm_peak": 16 * reads / t_score / (HBM_PEAK_GBS * 1e9),
+            "hbm_bytes_per_launch": hbm_bytes,
+            "hbm_frac": hbm_bytes / t_score / (HBM_PEAK_GBS * 1e9),
+        }
         # the same batch drawn so that no forbidden (non-finite) entry is selected where the
         # graph allows it: node by node, uniformly among the strategies allowed against the
         # producers' choices (apc_sample_feasible), then scored from the assignment matrix
