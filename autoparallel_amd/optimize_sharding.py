@@ -664,7 +664,12 @@ class ShardingOptimizer:
                 if k is of_node:
                     v = a.meta.get("val")
                     if isinstance(v, torch.Tensor):
-                        k = (tuple(str(d) for d in v.shape), tuple(str(d) for d in v.stride()), str(v.dtype))
+                        shape, stride = v.shape, v.stride()
+                        try:  # plain integers: the tuples themselves (equal exactly when their texts are)
+                            hash(shape), hash(stride)
+                            k = (tuple(shape), stride, v.dtype)
+                        except TypeError:  # a symbolic size has no hash: by its text
+                            k = (tuple(str(d) for d in shape), tuple(str(d) for d in stride), v.dtype)
                     else:
                         k = None if v is None else str(v)
                     of_node[a] = k
@@ -672,12 +677,19 @@ class ShardingOptimizer:
             return a if isinstance(a, int) else None
 
         ids: Dict[tuple, int] = {}
+        names: Dict[object, str] = {}  # an operator's name is asked once
         out = np.empty(len(nodes), np.int32)
         for i, n in enumerate(nodes):
-            kw = sorted(n.kwargs.items(), key=lambda kv: kv[0])
-            flat = _flat_args(kw, _flat_args(n.args, []))
-            key = (str(n.target), n.meta.get("partitioner_tag"), n.meta.get("stack_trace"),
-                   tuple(k for k, _ in kw), tuple(arg_key(a) for a in flat))
+            kwargs = n.kwargs
+            kw = sorted(kwargs.items(), key=lambda kv: kv[0]) if kwargs else ()
+            flat = _flat_args(kw, _flat_args(n.args, [])) if kw else _flat_args(n.args, [])
+            target = n.target
+            name = names.get(target)
+            if name is None:
+                name = names[target] = str(target)
+            meta = n.meta
+            key = (name, meta.get("partitioner_tag"), meta.get("stack_trace"),
+                   tuple(k for k, _ in kw), tuple([arg_key(a) for a in flat]))
             out[i] = ids.setdefault(key, len(ids))
         return out
 
