@@ -376,6 +376,13 @@ class CostEngine:
             "apc_node_compute_costs",
         )
 
+    def mark_results_edited(self) -> None:
+        """To be called by a caller that has written into comm / cost / flags / per_arg
+        itself: scoring then reads the arrays as they are (records are made again on the
+        next large batch, and the block table no longer stands for the arrays)."""
+        self._recs_valid = False
+        self._table_clamp = None
+
     def edge_costs(self, clamp_inf: bool = True, want_comm: bool = True, want_flags: bool = True):
         self._recs_valid = False
         self._table_clamp = None

@@ -329,6 +329,43 @@ def test_scoring(CostEngine):
         assert tuple(out[i, :4]) == tuple(float(x) for x in want)
 
 
+def test_device_scorers_on_a_hand_made_plan(CostEngine):
+    """Every device scorer against totals worked out by hand from the text of the reference's
+    _compute_solution_cost (helpers.hand_made_plan): the entry arrays of an engine are overwritten with
+    the literal numbers of that case, so nothing of the cost model is involved."""
+    from helpers import hand_made_plan
+
+    g, comm, transition, compute, assign, want = hand_made_plan()
+    eng = CostEngine(g, use_table=False).build(clamp_inf=True)
+    nargs = np.repeat(g.node_nargs, 2).astype(np.float64)
+    per_arg = compute / nargs
+    eng.per_arg.copy_(torch.from_numpy(per_arg))
+    eng.compute.copy_(torch.from_numpy(compute))
+    eng.comm.copy_(torch.from_numpy(comm))
+    # cost as the build forms it, (comm + per_arg) + transition, clamped; flags: transition | non-finite << 1
+    cost = np.zeros(g.num_slots)
+    flags = transition.copy()
+    for e in range(g.num_edges):
+        v, off, ssrc, sdst = int(g.edge_node[e]), int(g.edge_off[e]), int(g.edge_ssrc[e]), int(g.edge_sdst[e])
+        for o in range(sdst):
+            for j in range(ssrc):
+                c = (comm[off + o * ssrc + j] + per_arg[int(g.node_comp_off[v]) + o]) + float(transition[off + o * ssrc + j])
+                if not np.isfinite(c):
+                    c, flags[off + o * ssrc + j] = 10000.0, flags[off + o * ssrc + j] | 2
+                cost[off + o * ssrc + j] = c
+    eng.cost.copy_(torch.from_numpy(cost))
+    eng.flags.copy_(torch.from_numpy(flags))
+    eng.mark_results_edited()
+    # objective: the selected cost of every argument row, placeholders' own rows included;
+    # one selected variable is forbidden (C <- Q)
+    obj = 2.0 + 4.0 + (0.5 + 16.0) + 10000.0 + (0.25 + 64.0 + 1.0) + (0.125 + 256.0 + 1.0)
+    col = np.asarray(assign, np.int16)[:, None]
+    for count in (1, 70, 33000, 140000):  # wave per assignment, lanes, records
+        out = eng.score(torch.from_numpy(np.ascontiguousarray(np.tile(col, (1, count)))).cuda()).cpu().numpy()
+        assert tuple(out[0, :4]) == want and tuple(out[-1, :4]) == want, (count, eng.last_score_backend, out[0])
+        assert out[0, 4] == obj and out[0, 5] == 1.0 and bits_equal(out[0], out[-1])
+
+
 def test_scoring_from_interleaved_records(CostEngine, monkeypatch):
     """apc_score_packed against the scorers that read the three entry arrays:
     explicit assignments, drawn ones, a window with continued sums; and the

@@ -199,6 +199,20 @@ def test_scorer_matches_reference_mock_totals():
     assert (obj, viol) == (3.0, 0)
 
 
+def test_scorer_known_answers_of_a_hand_made_plan():
+    """The three rules of the reference's _compute_solution_cost that a sum of selected
+    entries would miss (optimize_sharding.py:1081-1101): compute_cost * num_args per node,
+    non-finite comm skipped, no transition through a producer whose output is a tuple of
+    specs.  The expected totals are worked out by hand in helpers.hand_made_plan."""
+    from helpers import hand_made_plan
+
+    g, comm, transition, compute, assign, want = hand_made_plan()
+    assert tuple(float(x) for x in O.score_assignment(g, comm, transition, compute, assign)) == want
+    # the other strategy of G (same placement as T[0]'s element): no comm term 0.125, nothing else changes
+    total, comp, cm, tr = O.score_assignment(g, comm, transition, compute, [1, 0, 1, 0, 0])
+    assert (float(total), float(comp), float(cm), float(tr)) == (358.0 - 256.0 + 128.0 + 0.75 + 2.0, 230.0, 0.75, 2.0)
+
+
 def test_scorer_on_graph(small_llama):
     g = small_llama
     r = O.GraphOracle(g).build()
