@@ -19,7 +19,11 @@ _UPLOAD_ARENA_MAX_ARRAY = 2 << 20
 _SCORE_LANES_FROM = 32768  # assignments: below, one wavefront per assignment (entry arrays as they are)
 _SCORE_FROM_TABLE = True  # the three ways of scoring a graph with large blocks can be switched off (tests do)
 _SCORE_COMPACT = True
-_SCORE_STAGE_TILES = 8  # matrices of up to this many LDS tiles go through LDS in the table scorer
+# Matrices of up to this many LDS tiles (64 KB each) go through LDS in the table scorer, larger
+# ones are read in place.  Measured on a 3 000-node window of the stress DAG, 2^20 assignments:
+# 17.9 ms with 1, 17.4 with 2, 18.0 with 4, 18.35 with 8 or 16.  (A lower bound, small matrices
+# read in place to save their barrier, only cost time: 17.4 -> 18.9 ms at 1 024 doubles.)
+_SCORE_STAGE_TILES = 2
 # The table scorer pays about 2 us per edge whatever the batch (a matrix copied into LDS on every CU), the
 # walks over records about 14 ns per edge and assignment: from this many assignments on the table wins
 # (measured on a 3 000-node window of the stress DAG: 18 ms per window from the table for any batch up to
