@@ -209,21 +209,33 @@ def describe_node(node, strategies, b: GraphBuilder, name: Optional[str] = None,
     meta_ids = memo.setdefault("meta_ids", {}) if memo is not None else {}
     tuple_ids = memo.setdefault("tuple_ids", {}) if memo is not None else {}
 
+    # ... and by object first: the specs of one answer mostly share their tensor-meta and
+    # placement objects (kept alive by the specs, which outlive the memo), and hashing a
+    # tensor meta walks its shape and stride tuples
+    by_id = memo.setdefault("by_id", {}) if memo is not None else {}
+
     def word(s) -> int:
-        if s is None or s.tensor_meta is None:
+        if s is None:
             return -1
         w = words.get(id(s))
         if w is None:
             tm, plc = s.tensor_meta, s.placements
-            try:
-                m = meta_ids.get(tm)
-                if m is None:
-                    m = meta_ids[tm] = b.meta(*tensor_meta_key(tm))
-                t = tuple_ids.get(plc)
-                if t is None:
-                    t = tuple_ids[plc] = b.tuple_id(placement_codes(plc))
-            except TypeError:  # a size without a hash
-                m, t = b.meta(*tensor_meta_key(tm)), b.tuple_id(placement_codes(plc))
+            if tm is None:
+                return -1
+            m = by_id.get(id(tm))
+            t = by_id.get(id(plc))
+            if m is None or t is None:
+                try:
+                    m = meta_ids.get(tm)
+                    if m is None:
+                        m = meta_ids[tm] = b.meta(*tensor_meta_key(tm))
+                    t = tuple_ids.get(plc)
+                    if t is None:
+                        t = tuple_ids[plc] = b.tuple_id(placement_codes(plc))
+                except TypeError:  # a size without a hash
+                    m, t = b.meta(*tensor_meta_key(tm)), b.tuple_id(placement_codes(plc))
+                by_id[id(tm)] = m
+                by_id[id(plc)] = t
             w = spec_word(m, t)
             words[id(s)] = w
         return w

@@ -611,8 +611,12 @@ class ShardingOptimizer:
         template_of: Dict[tuple, int] = {}
         strats, input_nodes_of = self.strats, self._all_input_nodes
         packed_nodes: List[torch.fx.Node] = []
+        kinds: List[int] = []   # 1 placeholder, 2 get_attr, 0 anything else
+        phases: List[int] = []  # 1: tagged as backward by the partitioner
+        getitem_target = operator.getitem
         for node in self.nodes:
-            if node.op == "output":
+            op = node.op
+            if op == "output":
                 continue
             st: OpStrategy = strats[node]
             qkey = getattr(st, "_apc_query_id", None)
@@ -631,19 +635,19 @@ class ShardingOptimizer:
                 t = b.add_template(desc)
                 if qkey is not None:
                     template_of[qkey] = t
-            getitem = int(node.args[1]) if node.op == "call_function" and node.target is operator.getitem else None
+            getitem = int(node.args[1]) if op == "call_function" and node.target is getitem_target else None
             index_of[node] = b.add_instance(t, [index_of[x] for x in input_nodes_of(node)], getitem, node.name)
             packed_nodes.append(node)
+            kinds.append(1 if op == "placeholder" else (2 if op == "get_attr" else 0))
+            phases.append(1 if node.meta.get("partitioner_tag") == "is_backward" else 0)
         # default rows: what a strategy carried before the engine ran; the packer reads them
         # where an edge has no producer or a spec is missing
         g = b.pack(default_rows_of=lambda v: [s.redistribute_cost for s in strats[packed_nodes[v]].strategies])
         assert self.nodes[:len(packed_nodes)] == packed_nodes, "node order must be preserved"
         g.roles = self._roles()
         g.edge_prefetchable = self._prefetchable(g, packed_nodes)
-        g.node_kind = np.asarray([1 if n.op == "placeholder" else (2 if n.op == "get_attr" else 0)
-                                  for n in packed_nodes], np.uint8)
-        g.node_phase = np.asarray([1 if n.meta.get("partitioner_tag") == "is_backward" else 0
-                                   for n in packed_nodes], np.int32)
+        g.node_kind = np.asarray(kinds, np.uint8)
+        g.node_phase = np.asarray(phases, np.int32)
         if self.repeated_subgraphs:
             g.node_cluster_key = self._cluster_keys(packed_nodes)
         return g
