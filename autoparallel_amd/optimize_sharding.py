@@ -393,13 +393,25 @@ def _gc_paused():
     collector walk all of it again (measured on the Llama-3-8B graph: 1.5-1.7 s for
     the constructor with it, 0.73 s without; strategy enumeration alone 0.94 s
     against 0.22 s).  Reference counting frees as usual; the collector resumes on
-    exit, if it was on."""
+    exit, if it was on.
+
+    What was allocated meanwhile and is still alive (the strategies and their cost
+    rows: 0.6 M tracked objects for that graph) lives as long as the optimizer.  Left
+    in the youngest generation, all of it is walked at the first allocation after the
+    collector resumes (0.1 s, a quarter of the constructor).  freeze() followed by
+    unfreeze() hands every tracked object to the oldest generation without walking it
+    (two list splices), where the next full collection finds it as it finds every other
+    long-lived object.  Not done when the caller keeps a frozen generation of its own,
+    which unfreeze() would release."""
     was = gc.isenabled()
     gc.disable()
     try:
         yield
     finally:
         if was:
+            if gc.get_freeze_count() == 0:
+                gc.freeze()
+                gc.unfreeze()
             gc.enable()
 
 
@@ -718,7 +730,7 @@ class ShardingOptimizer:
         self.phase_s["write_back_redistribute_cost"] = time.perf_counter() - t0
         return DecisionVars(self)
 
-    def _write_back_redistribute_costs(self) -> None:
+    def _write_back_redistribute_costs(self, as_built: bool = True) -> None:
         """strategy.redistribute_cost[argi][inp_idx] = comm, as the reference's
         loop does in place (:540)."""
         g, comm = self._packed, self._core.coef.comm
@@ -726,12 +738,30 @@ class ShardingOptimizer:
         nodes, strats = self.nodes, self.strats
         edge_node, edge_arg, edge_ssrc = g.edge_node.tolist(), g.edge_arg.tolist(), g.edge_ssrc.tolist()
         vs, alias = np.asarray(vs).tolist(), np.asarray(alias).tolist()
+        # Edges that read one matrix of the block table have the same block of comm values
+        # while the arrays are as the build wrote them (the entry kernel copies the matrix): the
+        # floats are made once per matrix, and an edge gets lists of its own over them.  Without a
+        # block table, or after a pass that changed comm edge by edge, every edge converts its own.
+        engine = getattr(self._core, "engine", None)
+        if as_built and engine is not None and engine.table_mode != "direct":
+            matrix_of = g.block_table(engine.table_mode == "compressed")[3].tolist()
+        else:
+            matrix_of = [-1] * g.num_edges
+        by_matrix: Dict[int, list] = {}
         made: Dict[int, list] = {}  # rows of the edges that own a block, as lists
         for e in range(g.num_edges):
             r = alias[e]  # a repeated node's rows are its root's (:554-571)
             block = made.get(r)
             if block is None:
-                block = made[r] = comm[vs[r] : vs[r + 1]].reshape(-1, edge_ssrc[e]).tolist()
+                m = matrix_of[r]
+                shared = by_matrix.get(m) if m >= 0 else None
+                if shared is None:
+                    block = comm[vs[r] : vs[r + 1]].reshape(-1, edge_ssrc[e]).tolist()
+                    if m >= 0:
+                        by_matrix[m] = block
+                else:
+                    block = [row[:] for row in shared]
+                made[r] = block
                 rows = block
             else:  # lists of its own over the same numbers (:569-571)
                 rows = [row[:] for row in block]
@@ -851,7 +881,7 @@ class ShardingOptimizer:
 
     def apply_prefetch_discount(self, scale: float = 0.0) -> int:
         n = self._core.apply_prefetch_discount(scale)
-        self._write_back_redistribute_costs()
+        self._write_back_redistribute_costs(as_built=False)  # the discount is per edge, not per matrix
         return n
 
     # -- solve ------------------------------------------------------------------------------
