@@ -193,7 +193,9 @@ class SparseILP:
         right-hand side ``rhs`` (an array or one value).  Names continue the
         prefix's counter.  Returns the names."""
         indptr = np.ascontiguousarray(indptr, np.int64)
-        idx = np.ascontiguousarray(idx, np.int64)
+        idx = np.ascontiguousarray(idx)
+        if idx.dtype != np.int32:  # 32-bit indices are kept as they come: half the bytes of a large block
+            idx = np.ascontiguousarray(idx, np.int64)
         n = indptr.shape[0] - 1
         if n <= 0:
             return []

@@ -308,26 +308,32 @@ class PackedShardingOptimizer:
         self.add_grad_reduce_dtype_constraints()
 
     @staticmethod
-    def _segments(start, count, stride=None):
+    def _segments(start, count, stride=None, dtype=np.int64):
         """Concatenation of start[k] + stride[k] * arange(count[k]) over k, and
-        the offsets of the pieces."""
+        the offsets of the pieces.  ``dtype``: of the concatenation (int32 halves the
+        bytes the passes below move when every value fits)."""
         start = np.asarray(start, np.int64)
         count = np.asarray(count, np.int64)
         ptr = np.zeros(count.shape[0] + 1, np.int64)
         np.cumsum(count, out=ptr[1:])
         total = int(ptr[-1])
         if total == 0:
-            return np.zeros(0, np.int64), ptr
+            return np.zeros(0, dtype), ptr
         # as a running sum of steps: the stride inside a piece, and at the first element of a
         # piece the jump from the last element of the piece before (three passes over the
         # output instead of six)
-        step = np.ones(total, np.int64) if stride is None else np.repeat(np.asarray(stride, np.int64), count)
+        step = np.ones(total, dtype) if stride is None else np.repeat(np.asarray(stride, dtype), count)
         some = count > 0
         first, st, cn = ptr[:-1][some], start[some], count[some]
         last = st + (cn - 1 if stride is None else (cn - 1) * np.asarray(stride, np.int64)[some])
         step[first[0]] = st[0]
         step[first[1:]] = st[1:] - last[:-1]
-        return np.cumsum(step), ptr
+        return np.cumsum(step, dtype=dtype), ptr
+
+    @property
+    def _idx_dtype(self):
+        """Variable indices of the row blocks: 32 bits while they fit."""
+        return np.int32 if self.n_vars < 2**31 - 1 else np.int64
 
     def _add_difference_rows(self, prefix, plus_start, plus_count, minus_start, minus_count, minus_stride) -> None:
         """Rows  sum(plus piece) - sum(minus piece) = 0, one per pair of pieces."""
@@ -337,7 +343,7 @@ class PackedShardingOptimizer:
         start = np.empty(2 * n, np.int64); start[0::2] = plus_start; start[1::2] = minus_start
         count = np.empty(2 * n, np.int64); count[0::2] = plus_count; count[1::2] = minus_count
         stride = np.ones(2 * n, np.int64); stride[1::2] = minus_stride
-        idx, ptr = self._segments(start, count, stride)
+        idx, ptr = self._segments(start, count, stride, self._idx_dtype)
         sign = np.ones(2 * n, np.int8); sign[1::2] = -1
         self.prob.add_rows(prefix, ptr[0::2], idx, np.repeat(sign, count), ilp.EQ, 0.0)
 
@@ -345,7 +351,7 @@ class PackedShardingOptimizer:
         # for every (node, arg): exactly one (out, inp) pair
         g = self.g
         e = np.nonzero(~self.linked[g.edge_node])[0]
-        idx, ptr = self._segments(self.var_start[e], self.var_start[e + 1] - self.var_start[e])
+        idx, ptr = self._segments(self.var_start[e], self.var_start[e + 1] - self.var_start[e], None, self._idx_dtype)
         self.prob.add_rows("unique_decision", ptr, idx, 1.0, ilp.EQ, 1.0)
 
     def _num_input_nodes(self, v: int) -> int:
@@ -366,13 +372,14 @@ class PackedShardingOptimizer:
         if later.size == 0:
             return
         S = g.node_nstrat[v[later]].astype(np.int64)
-        e = np.repeat(later, S)
         o = np.arange(int(S.sum()), dtype=np.int64) - np.repeat(np.cumsum(S) - S, S)
-        e0 = self.edge_alias[first[v[e]]]
-        ek = self.edge_alias[e]
+        # per edge first, then one value per (edge, strategy)
+        e0 = self.edge_alias[first[v[later]]]
+        ek = self.edge_alias[later]
         s0, sk = g.edge_ssrc[e0].astype(np.int64), g.edge_ssrc[ek].astype(np.int64)
-        self._add_difference_rows("same_across_args", self.var_start[e0] + o * s0, s0,
-                                  self.var_start[ek] + o * sk, sk, np.ones_like(sk))
+        s0r, skr = np.repeat(s0, S), np.repeat(sk, S)
+        self._add_difference_rows("same_across_args", np.repeat(self.var_start[e0], S) + o * s0r, s0r,
+                                  np.repeat(self.var_start[ek], S) + o * skr, skr, np.ones_like(skr))
 
     def add_output_input_consistent_constraint(self) -> None:
         # producer's chosen output strategy == the input strategy its consumer assumes:
@@ -401,13 +408,15 @@ class PackedShardingOptimizer:
             edges = edges[np.sort(firsts)]
         assert (g.edge_ssrc[edges] == g.node_nstrat[u[edges]]).all()
         S = g.node_nstrat[u[edges]].astype(np.int64)
-        e = np.repeat(edges, S)
         k = np.arange(int(S.sum()), dtype=np.int64) - np.repeat(np.cumsum(S) - S, S)
-        eu = self.edge_alias[g.node_edge_off[u[e]].astype(np.int64)]  # argument 0 of the producer
-        ev = self.edge_alias[e]
-        su, sv = g.edge_ssrc[eu].astype(np.int64), g.edge_ssrc[ev].astype(np.int64)
-        self._add_difference_rows("output_input_consistent", self.var_start[eu] + k * su, su,
-                                  self.var_start[ev] + k, g.edge_sdst[ev].astype(np.int64), sv)
+        # per edge first, then one value per (edge, strategy of the producer)
+        eu = self.edge_alias[g.node_edge_off[u[edges]].astype(np.int64)]  # argument 0 of the producer
+        ev = self.edge_alias[edges]
+        su = np.repeat(g.edge_ssrc[eu].astype(np.int64), S)
+        sv = np.repeat(g.edge_ssrc[ev].astype(np.int64), S)
+        self._add_difference_rows("output_input_consistent", np.repeat(self.var_start[eu], S) + k * su, su,
+                                  np.repeat(self.var_start[ev], S) + k,
+                                  np.repeat(g.edge_sdst[ev].astype(np.int64), S), sv)
 
     def add_inf_cost_constraint(self) -> None:
         # the engine already wrote 10000.0 into cost; pin those variables to 0
