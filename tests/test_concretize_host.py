@@ -94,3 +94,43 @@ def test_graph_without_symbols_is_recognised():
 ])
 def test_produces_tensor(val, want):
     assert _produces_tensor(val) is want
+
+
+def test_collector_pause_hands_long_lived_objects_over_without_a_walk():
+    """_gc_paused: the collector is off inside, on again after (if it was on), and what was
+    allocated inside does not sit in the youngest generation afterwards; a frozen generation
+    of the caller's own is left as it is."""
+    import gc
+
+    from autoparallel_amd.optimize_sharding import _gc_paused
+
+    class Box:
+        def __init__(self):
+            self.ref = [self]  # a container the collector tracks
+
+    assert gc.isenabled()
+    gc.collect()
+    with _gc_paused():
+        assert not gc.isenabled()
+        keep = [Box() for _ in range(5000)]
+    assert gc.isenabled() and gc.get_freeze_count() == 0
+    assert gc.get_count()[0] < 5000  # the 10 000 new containers are not counted as young
+    assert len(keep) == 5000
+    # nested use and a collector that was off before: left off
+    gc.disable()
+    try:
+        with _gc_paused():
+            pass
+        assert not gc.isenabled()
+    finally:
+        gc.enable()
+    # the caller's frozen generation survives
+    gc.freeze()
+    try:
+        frozen = gc.get_freeze_count()
+        assert frozen > 0
+        with _gc_paused():
+            more = [Box() for _ in range(100)]
+        assert gc.get_freeze_count() == frozen and gc.isenabled() and len(more) == 100
+    finally:
+        gc.unfreeze()
