@@ -48,20 +48,41 @@ schedule_metrics_kernel(apc_schedule s, const int32_t* __restrict__ order, int64
   int64_t live = s.initial_bytes, peak = s.initial_bytes;
   const int32_t* ord = kIdentity ? nullptr : order + b * N;
 
+  // What a step needs to know about its node is requested one step ahead, before the
+  // step's own stores to the scratch arrays (which the compiler must assume to alias
+  // the schedule's arrays): a step is a chain of dependent gathers (order -> node
+  // attributes -> storages -> scratch), and with one wavefront per CU nothing else hides
+  // them.
+  struct NodeAttr { int v; double dur; int tid, fl, u0, u1, a0, a1, wait_src; };
+  auto load_attr = [&](int v) -> NodeAttr {
+    NodeAttr n;
+    n.v = v; n.dur = s.dur[v]; n.tid = s.stream[v]; n.fl = s.flags[v];
+    n.u0 = s.use_off[v]; n.u1 = s.use_off[v + 1];
+    n.a0 = s.alloc_off[v]; n.a1 = s.alloc_off[v + 1];
+    n.wait_src = s.wait_src[v];
+    return n;
+  };
+  NodeAttr nxt = {};
+  int v_after = 0;  // the node of step t + 2
+  if (N > 0) nxt = load_attr(kIdentity ? 0 : ord[0]);
+  if (N > 1) v_after = kIdentity ? 1 : ord[1];
   for (int t = 0; t < N; ++t) {
-    const int v = kIdentity ? t : ord[t];
-    const double dur = s.dur[v];
-    const int tid = s.stream[v];
-    const int fl = s.flags[v];
+    const NodeAttr cur_n = nxt;
+    if (t + 1 < N) nxt = load_attr(v_after);
+    if (t + 2 < N) v_after = kIdentity ? t + 2 : ord[t + 2];
+    const int v = cur_n.v;
+    const double dur = cur_n.dur;
+    const int tid = cur_n.tid;
+    const int fl = cur_n.fl;
 
     // ---- memory (MemoryTracker.schedule_node)
-    const int u0 = s.use_off[v], u1 = s.use_off[v + 1];
+    const int u0 = cur_n.u0, u1 = cur_n.u1;
     for (int q = u0; q < u1; ++q) {  // this reader is now scheduled
       const int64_t at = (int64_t)s.use_st[q] * n_sched + b;
       remaining[at] = remaining[at] - 1;
     }
     if (!(fl & APC_SCHED_NO_MEM)) {
-      for (int q = s.alloc_off[v]; q < s.alloc_off[v + 1]; ++q) live += s.st_bytes[s.alloc_st[q]];
+      for (int q = cur_n.a0; q < cur_n.a1; ++q) live += s.st_bytes[s.alloc_st[q]];
       peak = live > peak ? live : peak;
       for (int q = u0; q < u1; ++q) {
         const int k = s.use_st[q];
@@ -78,7 +99,7 @@ schedule_metrics_kernel(apc_schedule s, const int32_t* __restrict__ order, int64
     if (!known) ct = c0;  // a stream starts at the compute stream's present time
     if (fl & APC_SCHED_COMM) {
       if (tid == 0 && (fl & APC_SCHED_WAIT)) {
-        const int src = s.wait_src[v];
+        const int src = cur_n.wait_src;
         double end = c0;
         if (src >= 0) {
           const double e = end_time[(int64_t)src * n_sched + b];
