@@ -478,6 +478,46 @@ def test_work_items_of_512_entries(CostEngine, mode):
         CostEngine(g, table_mode="direct", item_entries=512, lut=False).build()
 
 
+def _sized_blocks_graph(sizes):
+    """A chain of producer/consumer pairs whose edge blocks have the given (S_src, S_dst):
+    rows shorter than, exactly and longer than a wavefront, single rows and single columns,
+    behind small blocks, so that blocks start at every offset inside a 64-slot group."""
+    import itertools
+
+    b = GraphBuilder((2, 2, 2, 2), 8)
+    m = b.meta((8, 16, 32, 64), (32768, 2048, 64, 1), 4, packed.DT_F32)
+    codes = [0x00, 0x40, 0x41, 0x42, 0x43, 0x80]
+    tuples = list(itertools.product(codes, repeat=4))  # 1 296 distinct placement tuples
+    rng = np.random.default_rng(7)
+    for k, (ssrc, sdst) in enumerate(sizes):
+        src = [b.spec(m, tuples[i]) for i in rng.choice(len(tuples), ssrc, replace=False)]
+        dst = [b.spec(m, tuples[i]) for i in rng.choice(len(tuples), sdst, replace=False)]
+        p = b.add_node(NodeDesc(f"p{k}", in_specs=[[x] for x in src], out_specs=[[x] for x in src], inputs=[],
+                                default_rows=[[[0.0]] for _ in src]))
+        b.add_node(NodeDesc(f"c{k}", in_specs=[[x] for x in dst], out_specs=[[x] for x in dst], inputs=[p]))
+    return b.pack()
+
+
+@pytest.mark.parametrize("mode", ["full", "compressed"])
+@pytest.mark.parametrize("item_entries", [256, 512])
+def test_entry_kernel_on_blocks_of_chosen_sizes(CostEngine, mode, item_entries):
+    """The wave-per-item kernel picks the row values of an entry three ways (two candidate rows
+    for rows of 64 entries and more, one lane per row below, a load per entry for items of more
+    than 64 rows) and repeats an entry of the block in the lanes that fall outside it: blocks on
+    every side of those limits, every entry against the oracle."""
+    sizes = [(63, 5), (3, 2), (64, 7), (5, 1), (65, 9), (128, 1), (1, 300), (512, 3), (7, 200), (2, 700),
+             (200, 64), (64, 64), (9, 60), (8, 65), (300, 2), (1, 1), (130, 130)]
+    g = _sized_blocks_graph(sizes)
+    assert len({int(o) % 64 for o in g.edge_off[:-1]}) >= 3  # blocks start at several offsets of a 64-slot group
+    eng = CostEngine(g, table_mode=mode, item_entries=item_entries).build(clamp_inf=False)
+    got = eng.results()
+    ref = O.GraphOracle(g).build()
+    assert bits_equal(got["comm"], ref["comm"]), first_mismatch(got["comm"], ref["comm"])
+    assert bits_equal(got["cost"], ref["cost"]), first_mismatch(got["cost"], ref["cost"])
+    assert ((got["flags"] & 1) == ref["transition"]).all()
+    assert (((got["flags"] >> 1) & 1) == ~np.isfinite(ref["cost"])).all()
+
+
 @pytest.mark.parametrize("mode", ["full", "compressed"])
 @pytest.mark.parametrize("item_entries", [256, 512])
 def test_entry_kernel_with_an_output_left_out(CostEngine, mode, item_entries):
