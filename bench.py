@@ -217,6 +217,19 @@ def main():
         after.append(ms.value * 1e-3)
     eng.lib.apc_timer_destroy(timer)
     t_edge_after = float(np.mean(after))
+    # and the same launch 100 times back to back between two events on the stream: no event
+    # pair inside, so no launch carries the system-scope release a timed one ends with
+    # (the entry kernel alone: table and per-arg terms are those of the last build)
+    n_b2b = 100
+    ev_a, ev_b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    for _ in range(5):
+        eng.edge_costs(clamp_inf=True)
+    ev_a.record()
+    for _ in range(n_b2b):
+        eng.edge_costs(clamp_inf=True)
+    ev_b.record()
+    torch.cuda.synchronize()
+    t_edge_b2b = ev_a.elapsed_time(ev_b) * 1e-3 / n_b2b
 
     if args.calibration_copy_mib > 0:
         nbytes = args.calibration_copy_mib << 20
@@ -306,6 +319,9 @@ def main():
             "timed_launches": n_timed,
             "avg_launch_s_after_region": t_edge_after,
             "timed_launches_after_region": n_after,
+            "avg_launch_s_back_to_back": t_edge_b2b,
+            "launches_back_to_back": n_b2b,
+            "frac_back_to_back": algo_bytes / t_edge_b2b / 1e9 / HBM_PEAK_GBS,
             # the same bytes over the whole step (prepare launch included), and both
             # with 8 B per entry (the cost alone) instead of the 17 B this build writes
             "step_frac": algo_bytes / (elapsed / args.steps) / 1e9 / HBM_PEAK_GBS,
