@@ -256,11 +256,13 @@ _SIGNATURES = {
         [C.POINTER(ApcProblem), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int32,
          C.c_void_p, C.c_void_p, C.c_void_p]),
     "apc_random_assignment": (C.c_uint32, [C.c_uint64, C.c_int64, C.c_int32, C.c_int32]),
+    "apc_pack_allowed_columns": (
+        C.c_int, [C.POINTER(ApcProblem), C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p, C.c_void_p]),
     "apc_sample_feasible": (
         C.c_int,
-        [C.POINTER(ApcProblem), C.c_void_p, C.c_uint64, C.c_int64, C.c_int64, C.c_void_p, C.c_int32, C.c_void_p,
-         C.c_void_p, C.c_void_p]),
-    "apc_sample_takes": (C.c_int32, [C.c_uint64, C.c_int64, C.c_int32, C.c_uint32]),
+        [C.POINTER(ApcProblem), C.c_void_p, C.c_void_p, C.c_uint64, C.c_int64, C.c_int64, C.c_void_p, C.c_int32,
+         C.c_void_p, C.c_void_p, C.c_void_p]),
+    "apc_sample_rank": (C.c_uint32, [C.c_uint64, C.c_int64, C.c_int32, C.c_uint32]),
     "apc_local_shapes": (
         C.c_int,
         [C.POINTER(ApcModel), C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
@@ -314,7 +316,7 @@ EXPORTED_SYMBOLS = tuple(_SIGNATURES)
 _lib = None
 
 
-ABI_VERSION = 4  # apc_version() of the library whose struct layouts this module mirrors
+ABI_VERSION = 5  # apc_version() of the library whose struct layouts this module mirrors
 
 
 class ApcError(RuntimeError):

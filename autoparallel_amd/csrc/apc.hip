@@ -1072,7 +1072,7 @@ int launch_prepare(const apc_problem* p, double* table, bool do_nodes, double* c
 
 extern "C" {
 
-int apc_version(void) { return 4; }
+int apc_version(void) { return 5; }
 
 const char* apc_last_error(void) { return g_err; }
 

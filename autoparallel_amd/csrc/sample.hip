@@ -11,17 +11,22 @@
 // flow rows holds by construction, as for the plain draws: an edge's inp_idx is
 // its producer's choice.
 //
-// Large batches: one lane per assignment.  Lanes of a wave read the flags of the same edge
-// block and the same row, at the columns their producers' choices name: one or
-// two cache lines per load, out of L2.  The choice among the allowed strategies
-// is a reservoir walk (the k-th allowed one replaces the pick when a hash of
-// (seed, assignment, node, k) scaled to [0, k) is zero), so the flags are read
-// once and the draw is a function of counters alone: a host can repeat it.
+// Two steps.  apc_pack_allowed_columns turns the flags of a build into bit
+// columns: for an argument row (edge) and a choice j of its producer, one bit per
+// strategy of the consumer, set where the entry is finite.  The strategies a node
+// may take are then the AND of one column per argument row, a few 64-bit words,
+// instead of a walk over the flag bytes of every strategy; their number is a
+// population count, and the draw is the r-th set bit with r one hash of (seed,
+// assignment, node) scaled to the count: a function of counters alone, which a
+// host can repeat.  (When a lane walked the flag bytes and hashed once per allowed
+// strategy, a reservoir walk, 2^20 assignments of the 5.5 M-entry Llama-3-8B graph
+// took 136 ms on MI355X.)
 #include "apc_device.h"
 
 namespace {
 
-constexpr int kSampleArgs = 6;  // argument rows of a node whose bases a lane keeps in registers
+constexpr int kSampleArgs = 6;   // argument rows of a node whose columns a lane keeps in registers
+constexpr int kSampleWords = 8;  // words of a node's strategies a lane keeps in registers (512 strategies)
 
 __host__ __device__ __forceinline__ uint32_t finalise32(uint32_t h) {
   h ^= h >> 16;
@@ -46,14 +51,73 @@ __host__ __device__ __forceinline__ uint32_t plain_draw(uint32_t h0, int32_t gid
   return (uint32_t)(((uint64_t)h * (uint64_t)(uint32_t)nstrat) >> 32);
 }
 
-// Whether the k-th allowed strategy (k >= 1) replaces the pick: probability 1 / k.
-__host__ __device__ __forceinline__ bool reservoir_takes(uint32_t h0, int32_t gid, uint32_t k) {
-  const uint32_t h = finalise32(h0 ^ ((uint32_t)(gid + 1) * 0xC2B2AE3Du) ^ (k * 0x9E3779B1u) ^ 0x68E31DA4u);
-  return (uint32_t)(((uint64_t)h * (uint64_t)k) >> 32) == 0u;
+// Which of the count allowed strategies of a node is taken, counted in out_idx order:
+// uniform in [0, count), from a hash of its own (not the plain draw's).
+__host__ __device__ __forceinline__ uint32_t rank_draw(uint32_t h0, int32_t gid, uint32_t count) {
+  const uint32_t h = finalise32(h0 ^ ((uint32_t)(gid + 1) * 0xC2B2AE3Du) ^ 0x68E31DA4u);
+  return (uint32_t)(((uint64_t)h * (uint64_t)count) >> 32);
 }
 
+// position of the r-th set bit of m (r < popcount(m)): six halvings
+__device__ __forceinline__ int select_bit(uint64_t m, uint32_t r) {
+  int base = 0;
+#pragma unroll
+  for (int s = 32; s >= 1; s >>= 1) {
+    const uint64_t low = m & ((1ull << s) - 1ull);
+    const uint32_t c = (uint32_t)__popcll(low);
+    if (r >= c) {
+      r -= c;
+      m >>= s;
+      base += s;
+    } else {
+      m = low;
+    }
+  }
+  return base;
+}
+
+// the strategies of word w of a node with S strategies
+__device__ __forceinline__ uint64_t word_mask(int S, int w) {
+  const int left = S - 64 * w;
+  return left >= 64 ? ~0ull : (left <= 0 ? 0ull : ((1ull << left) - 1ull));
+}
+
+// One wavefront per (argument row e, 64 strategies of the consumer).  lane = choice j of the
+// producer, so a load reads 64 consecutive flag bytes of one row of the block; a walk over the
+// 64 strategies o fills, one bit a step, the word every lane keeps of its own column.
 __global__ void __launch_bounds__(kBlock)
-sample_feasible_kernel(apc_problem p, const uint8_t* __restrict__ flags, uint64_t seed, int64_t first,
+pack_allowed_columns_kernel(apc_problem p, const uint8_t* __restrict__ flags,
+                            const int64_t* __restrict__ col_off, int max_words,
+                            uint64_t* __restrict__ colbits) {
+  const int64_t unit = (int64_t)blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6);
+  const int e = __builtin_amdgcn_readfirstlane((int)(unit / max_words));
+  const int w = __builtin_amdgcn_readfirstlane((int)(unit % max_words));
+  if (e >= p.n_edge) return;
+  const apc_edge* ed = p.edges + e;  // wave-uniform: scalar loads
+  const int sdst = ed->sdst, ssrc = ed->ssrc;
+  const int W = (sdst + 63) >> 6;
+  if (w >= W) return;
+  const int lane = threadIdx.x & 63;
+  const int rows = min(64, sdst - 64 * w);
+  const uint8_t* __restrict__ tile = flags + ed->off + (int64_t)(64 * w) * ssrc;
+  uint64_t* __restrict__ out = colbits + col_off[e] + w;
+  for (int j0 = 0; j0 < ssrc; j0 += 64) {
+    const int j = j0 + lane;
+    const bool mine = j < ssrc;
+    const uint8_t* __restrict__ col = tile + (mine ? j : 0);
+    uint64_t m = 0;
+#pragma unroll 8
+    for (int k = 0; k < rows; ++k)
+      m |= (uint64_t)((col[(int64_t)k * ssrc] & APC_ENTRY_NONFINITE) == 0) << k;
+    if (mine) out[(int64_t)j * W] = m;
+  }
+}
+
+// One lane per assignment.  The lanes of a wave read, per argument row and word, the column
+// their producer's choice names: 8-byte gathers inside one block of columns.
+__global__ void __launch_bounds__(kBlock)
+sample_feasible_kernel(apc_problem p, const uint64_t* __restrict__ colbits,
+                       const int64_t* __restrict__ col_off, uint64_t seed, int64_t first,
                        int64_t n_assign, const int32_t* __restrict__ node_gid, int first_node,
                        uint16_t* __restrict__ assign, int32_t* __restrict__ n_fallback) {
   const int64_t a = (int64_t)blockIdx.x * kBlock + threadIdx.x;
@@ -64,40 +128,70 @@ sample_feasible_kernel(apc_problem p, const uint8_t* __restrict__ flags, uint64_
     const int S = p.node_nstrat[v];
     const int gid = node_gid ? node_gid[v] : v;
     const int e0 = p.node_edge_off[v], e1 = p.node_edge_off[v + 1];
-    // slot of (row 0, the producer's choice) in every argument's block, and the row length
-    int64_t base[kSampleArgs];
-    int32_t ssrc[kSampleArgs];
+    const int W = (S + 63) >> 6;
+    // the column of every argument row: that of the producer's choice
+    const uint64_t* col[kSampleArgs];
 #pragma unroll
     for (int i = 0; i < kSampleArgs; ++i) {
-      base[i] = 0;
-      ssrc[i] = 0;
+      col[i] = colbits;
       if (e0 + i < e1) {
-        const apc_edge* ed = p.edges + (e0 + i);
-        const int u = ed->src_node;
-        const uint32_t j = u >= 0 ? (uint32_t)assign[(size_t)u * n_assign + a] : 0u;
-        base[i] = ed->off + j;
-        ssrc[i] = ed->ssrc;
+        const int u = p.edges[e0 + i].src_node;
+        const int64_t j = u >= 0 ? (int64_t)assign[(size_t)u * n_assign + a] : 0;
+        col[i] = colbits + col_off[e0 + i] + j * W;
       }
     }
-    uint32_t count = 0, pick = 0;
-    for (int o = 0; o < S; ++o) {
-      uint32_t bad = 0;
+    // word w of the node's allowed strategies
+    auto allowed_word = [&](int w) -> uint64_t {
+      uint64_t m = word_mask(S, w);
 #pragma unroll
       for (int i = 0; i < kSampleArgs; ++i)
-        if (e0 + i < e1) bad |= flags[base[i] + (int64_t)o * ssrc[i]];
+        if (e0 + i < e1) m &= col[i][w];
       for (int e = e0 + kSampleArgs; e < e1; ++e) {  // a node with more argument rows than the registers hold
-        const apc_edge* ed = p.edges + e;
-        const int u = ed->src_node;
-        const uint32_t j = u >= 0 ? (uint32_t)assign[(size_t)u * n_assign + a] : 0u;
-        bad |= flags[ed->off + (int64_t)o * ed->ssrc + j];
+        const int u = p.edges[e].src_node;
+        const int64_t j = u >= 0 ? (int64_t)assign[(size_t)u * n_assign + a] : 0;
+        m &= colbits[col_off[e] + j * W + w];
       }
-      if (!(bad & APC_ENTRY_NONFINITE)) {
-        ++count;
-        if (reservoir_takes(h0, gid, count)) pick = (uint32_t)o;
+      return m;
+    };
+    uint32_t count = 0;
+    int pick = 0;
+    if (W <= kSampleWords) {  // wave-uniform: the words stay in registers
+      uint64_t m[kSampleWords];
+#pragma unroll
+      for (int w = 0; w < kSampleWords; ++w) {
+        m[w] = w < W ? allowed_word(w) : 0ull;
+        count += (uint32_t)__popcll(m[w]);
+      }
+      if (count > 0) {
+        uint32_t r = rank_draw(h0, gid, count);
+        bool found = false;
+#pragma unroll
+        for (int w = 0; w < kSampleWords; ++w) {
+          const uint32_t c = (uint32_t)__popcll(m[w]);
+          if (!found && r < c) {
+            pick = 64 * w + select_bit(m[w], r);
+            found = true;
+          }
+          if (!found) r -= c;
+        }
+      }
+    } else {  // more than 512 strategies: the words are formed twice
+      for (int w = 0; w < W; ++w) count += (uint32_t)__popcll(allowed_word(w));
+      if (count > 0) {
+        uint32_t r = rank_draw(h0, gid, count);
+        for (int w = 0; w < W; ++w) {
+          const uint64_t m = allowed_word(w);
+          const uint32_t c = (uint32_t)__popcll(m);
+          if (r < c) {
+            pick = 64 * w + select_bit(m, r);
+            break;
+          }
+          r -= c;
+        }
       }
     }
     if (count == 0) {
-      pick = plain_draw(h0, gid, S);
+      pick = (int)plain_draw(h0, gid, S);
       ++fallbacks;
     }
     assign[(size_t)v * n_assign + a] = (uint16_t)pick;
@@ -105,101 +199,42 @@ sample_feasible_kernel(apc_problem p, const uint8_t* __restrict__ flags, uint64_
   n_fallback[a] = fallbacks;
 }
 
-// Small batches: one wavefront per assignment, lanes over the strategies of the
-// node.  A lane finds out whether its strategy is allowed, the ballot of the wave
-// gives every allowed strategy its rank k in out_idx order, each lane evaluates the
-// reservoir's test for its own k, and the pick is the last strategy whose test
-// says "take": what the sequential walk ends with.  Same choices as the kernel
-// above, bit for bit; the lanes of a wave read one column of a block (a cache line
-// each) instead of sharing a row, which is the better trade while there are
-// fewer assignments than lanes on the chip.
-__global__ void __launch_bounds__(kBlock)
-sample_feasible_wave_kernel(apc_problem p, const uint8_t* __restrict__ flags, uint64_t seed, int64_t first,
-                            int64_t n_assign, const int32_t* __restrict__ node_gid, int first_node,
-                            uint16_t* __restrict__ assign, int32_t* __restrict__ n_fallback) {
-  const int64_t a = (int64_t)blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6);
-  if (a >= n_assign) return;  // wave-uniform
-  const int lane = threadIdx.x & 63;
-  const uint32_t h0 = assignment_hash(seed, first + a);
-  int fallbacks = 0;
-  for (int v = first_node; v < p.n_node; ++v) {
-    const int S = p.node_nstrat[v];
-    const int gid = node_gid ? node_gid[v] : v;
-    const int e0 = p.node_edge_off[v], e1 = p.node_edge_off[v + 1];
-    uint32_t count = 0;
-    int pick = -1;
-    // The producers' choices (written by this wave's lane 0, or by the caller): lane i reads
-    // that of argument row i, and the wave takes them from there.  One load whose 64 lanes
-    // all read the same address costs as much as a 64-way gather on this chip.
-    int j_of = 0;
-    if (e0 + lane < e1) {
-      const int u = p.edges[e0 + lane].src_node;
-      j_of = u >= 0 ? (int)assign[(size_t)u * n_assign + a] : 0;
-    }
-    for (int o0 = 0; o0 < S; o0 += 64) {
-      const int o = o0 + lane;
-      uint32_t bad = o < S ? 0u : (uint32_t)APC_ENTRY_NONFINITE;
-      for (int e = e0; e < e1; ++e) {
-        const apc_edge* ed = p.edges + e;  // wave-uniform: scalar loads
-        uint32_t j;
-        if (e - e0 < 64) {
-          j = (uint32_t)__builtin_amdgcn_readlane(j_of, e - e0);
-        } else {  // more argument rows than lanes
-          const int u = ed->src_node;
-          j = u >= 0 ? (uint32_t)assign[(size_t)u * n_assign + a] : 0u;
-        }
-        if (o < S) bad |= flags[ed->off + (int64_t)o * ed->ssrc + j];
-      }
-      const bool allowed = !(bad & APC_ENTRY_NONFINITE);
-      const uint64_t mask = __ballot(allowed);
-      const uint32_t rank = count + (uint32_t)__popcll(mask & ((1ull << lane) - 1ull)) + 1u;
-      const uint64_t takes = __ballot(allowed && reservoir_takes(h0, gid, rank));
-      if (takes) pick = o0 + 63 - __clzll(takes);
-      count += (uint32_t)__popcll(mask);
-    }
-    if (count == 0) {
-      pick = (int)plain_draw(h0, gid, S);
-      ++fallbacks;
-    }
-    if (lane == 0) assign[(size_t)v * n_assign + a] = (uint16_t)pick;
-    // the next node may read this choice through the vector memory path of other lanes
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-  }
-  if (lane == 0) n_fallback[a] = fallbacks;
-}
-
-constexpr int64_t kSampleWaveBelow = 65536;  // assignments: below, a wavefront each
-
 }  // namespace
 
 extern "C" {
 
-int apc_sample_feasible(const apc_problem* p, const uint8_t* flags, uint64_t seed, int64_t first,
-                        int64_t n_assign, const int32_t* node_gid, int32_t first_node, uint16_t* assign,
-                        int32_t* n_fallback, void* stream) {
+int apc_pack_allowed_columns(const apc_problem* p, const uint8_t* flags, const int64_t* col_off,
+                             int32_t max_words, uint64_t* colbits, void* stream) {
+  if (int rc = validate_problem(p)) return rc;
+  if (p->n_edge == 0 || p->n_entry == 0) return 0;
+  if (!flags || !col_off || !colbits || max_words <= 0)
+    return fail(APC_ERR_INVALID, "apc_pack_allowed_columns: null argument or max_words <= 0%s");
+  const int64_t units = (int64_t)p->n_edge * max_words;
+  const int64_t grid = (units + (kBlock / 64) - 1) / (kBlock / 64);
+  if (grid > 0x7FFFFFFF)
+    return fail(APC_ERR_INVALID, "apc_pack_allowed_columns: too many argument rows for one launch%s");
+  hipLaunchKernelGGL(pack_allowed_columns_kernel, dim3((unsigned)grid), dim3(kBlock), 0, (hipStream_t)stream, *p,
+                     flags, col_off, (int)max_words, colbits);
+  return check_launch("pack_allowed_columns_kernel");
+}
+
+int apc_sample_feasible(const apc_problem* p, const uint64_t* colbits, const int64_t* col_off, uint64_t seed,
+                        int64_t first, int64_t n_assign, const int32_t* node_gid, int32_t first_node,
+                        uint16_t* assign, int32_t* n_fallback, void* stream) {
   if (int rc = validate_problem(p)) return rc;
   if (n_assign <= 0) return 0;
-  if (!assign || !n_fallback || (p->n_entry > 0 && !flags))
+  if (!assign || !n_fallback || (p->n_entry > 0 && (!colbits || !col_off)))
     return fail(APC_ERR_INVALID, "apc_sample_feasible: null argument%s");
   if (first_node < 0 || first_node > p->n_node)
     return fail(APC_ERR_INVALID, "apc_sample_feasible: first_node out of range%s");
-  if (n_assign < kSampleWaveBelow) {
-    const int64_t per = kBlock / 64;
-    hipLaunchKernelGGL(sample_feasible_wave_kernel, dim3((unsigned)((n_assign + per - 1) / per)), dim3(kBlock), 0,
-                       (hipStream_t)stream, *p, flags, seed, first, n_assign, node_gid, (int)first_node, assign,
-                       n_fallback);
-    return check_launch("sample_feasible_wave_kernel");
-  }
   hipLaunchKernelGGL(sample_feasible_kernel, dim3((unsigned)((n_assign + kBlock - 1) / kBlock)), dim3(kBlock), 0,
-                     (hipStream_t)stream, *p, flags, seed, first, n_assign, node_gid, (int)first_node, assign,
-                     n_fallback);
+                     (hipStream_t)stream, *p, colbits, col_off, seed, first, n_assign, node_gid, (int)first_node,
+                     assign, n_fallback);
   return check_launch("sample_feasible_kernel");
 }
 
-int32_t apc_sample_takes(uint64_t seed, int64_t a, int32_t node, uint32_t k) {
-  return reservoir_takes(assignment_hash(seed, a), node, k) ? 1 : 0;
+uint32_t apc_sample_rank(uint64_t seed, int64_t a, int32_t node, uint32_t count) {
+  return count ? rank_draw(assignment_hash(seed, a), node, count) : 0u;
 }
 
 }  // extern "C"

@@ -757,14 +757,41 @@ class CostEngine:
         self.last_score_backend = "entry_arrays"
         return out
 
+    def _allowed_columns(self):
+        """(colbits, col_off, max_words) of apc_pack_allowed_columns for the flags as they
+        are now: the layout is made once per engine, the bits on every call (one pass over
+        the flags; any build or pass may have rewritten them)."""
+        g = self.g
+        lay = self._keep.get("column_layout")
+        if lay is None:
+            words = (g.edge_sdst.astype(np.int64) + 63) >> 6
+            size = g.edge_ssrc.astype(np.int64) * words
+            own = np.ones(g.num_edges, bool) if g.edge_alias is None else g.priced
+            off = np.zeros(g.num_edges, np.int64)
+            off[own] = np.cumsum(size[own]) - size[own]
+            if g.edge_alias is not None:  # an edge without a block of its own reads its root's columns
+                off[~own] = off[g.edge_alias[~own]]
+            total = int(size[own].sum())
+            lay = self._keep["column_layout"] = (
+                torch.from_numpy(off).to(self.device), max(int(words.max()) if g.num_edges else 1, 1),
+                torch.empty(max(total, 1), dtype=torch.int64, device=self.device))
+        d_off, max_words, colbits = lay
+        _lib.check(
+            self.lib.apc_pack_allowed_columns(
+                C.byref(self.problem), self._ptr(self.flags), self._ptr(d_off), int(max_words), self._ptr(colbits),
+                self._stream()),
+            "apc_pack_allowed_columns")
+        return colbits, d_off, max_words
+
     def sample_feasible(self, seed: int, first: int, count: int, node_gid: Optional[np.ndarray] = None,
                         first_node: int = 0, assign: Optional[torch.Tensor] = None):
         """``count`` assignments drawn node by node among the strategies that select
         no forbidden (non-finite) entry against the choices made for the node's
-        producers (apc_sample_feasible).  Returns (assign uint16[n_node, count] on
-        the device, n_fallback int32[count]: nodes that had no such strategy and
-        took the plain draw).  ``assign``/``first_node``: rows below first_node are
-        given (a window of a larger graph); ``node_gid``: ids for the hashes."""
+        producers (apc_pack_allowed_columns, then apc_sample_feasible).  Returns
+        (assign uint16[n_node, count] on the device, n_fallback int32[count]: nodes
+        that had no such strategy and took the plain draw).  ``assign``/``first_node``:
+        rows below first_node are given (a window of a larger graph); ``node_gid``:
+        ids for the hashes."""
         assert self.built
         N = self.g.num_nodes
         if assign is None:
@@ -775,10 +802,11 @@ class CostEngine:
         if node_gid is not None:
             d_gid = torch.from_numpy(np.ascontiguousarray(node_gid, np.int32)).to(self.device)
         fallback = torch.empty(count, dtype=torch.int32, device=self.device)
+        colbits, d_off, _ = self._allowed_columns()
         _lib.check(
             self.lib.apc_sample_feasible(
-                C.byref(self.problem), self._ptr(self.flags), int(seed), int(first), int(count), self._ptr(d_gid),
-                int(first_node), self._ptr(assign), self._ptr(fallback), self._stream()),
+                C.byref(self.problem), self._ptr(colbits), self._ptr(d_off), int(seed), int(first), int(count),
+                self._ptr(d_gid), int(first_node), self._ptr(assign), self._ptr(fallback), self._stream()),
             "apc_sample_feasible")
         return assign, fallback
 

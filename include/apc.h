@@ -368,7 +368,7 @@ typedef struct apc_problem {
  *   apc_build_pair_table_lut / apc_edge_costs_lut   lut_kernel over a list passed as
  *                           an argument instead of the problem's own
  *
- * Version of the ABI (struct layouts and signatures of this header): 4. */
+ * Version of the ABI (struct layouts and signatures of this header): 5. */
 int apc_version(void);
 const char* apc_last_error(void);
 
@@ -646,22 +646,35 @@ uint32_t apc_random_assignment(uint64_t seed, int64_t a, int32_t node, int32_t n
  * it.  No function of the reference does this; "forbidden" is the reference's own
  * notion: a decision variable whose cost is not finite, which
  * add_inf_cost_constraint pins to zero (autoparallel/optimize_sharding.py:803-812;
- * the APC_ENTRY_NONFINITE bit of flags).  For assignment a (counter first + a) the
- * nodes from first_node on are walked in order and node v gets, uniformly, one of
- * the strategies out_idx whose entries (v, arg, out_idx, choice of the producer of
- * arg) are all finite; a node without such a strategy takes the plain draw of
- * apc_random_assignment and is counted in n_fallback[a].  The choice among the
- * allowed strategies is a reservoir walk in out_idx order: the k-th allowed one
- * replaces the pick when apc_sample_takes(seed, first + a, id of v, k) is 1.
+ * the APC_ENTRY_NONFINITE bit of flags).  Two calls.
+ *
+ * apc_pack_allowed_columns writes, for every argument row (edge) e and every
+ * choice j of its producer, the bit column of the consumer's strategies whose entry
+ * (e, out_idx, j) is finite: words colbits[col_off[e] + j * W + w], W =
+ * ceil(S_dst / 64), bit (out_idx mod 64) of word out_idx / 64; bits past S_dst are
+ * zero.  col_off: int64[n_edge], the caller's layout (S_src * W words per edge;
+ * edges that share a block may share their columns); max_words: the largest W.
+ * To be called again after anything that rewrites flags.
+ *
+ * apc_sample_feasible: for assignment a (counter first + a) the nodes from
+ * first_node on are walked in order and node v gets, uniformly, one of the
+ * strategies out_idx whose entries (v, arg, out_idx, choice of the producer of arg)
+ * are all finite: the AND of one column per argument row; with `count` of them
+ * it is the one of rank apc_sample_rank(seed, first + a, id of v, count) in out_idx
+ * order.  A node without such a strategy takes the plain draw of
+ * apc_random_assignment and is counted in n_fallback[a].
  * assign: uint16[n_node][n_assign], written for v >= first_node; the rows below
  * first_node are read (choices made earlier, e.g. for the stand-in nodes of a
  * window of a larger graph).  node_gid: id of every node for the hashes (NULL:
  * its index).  Score the result with apc_score_assignments or the batch scorers
- * that take explicit assignments: element 5 of a row is 0 where n_fallback is. */
-int apc_sample_feasible(const apc_problem* p, const uint8_t* flags, uint64_t seed, int64_t first,
-                        int64_t n_assign, const int32_t* node_gid, int32_t first_node, uint16_t* assign,
-                        int32_t* n_fallback, void* stream);
-int32_t apc_sample_takes(uint64_t seed, int64_t a, int32_t node, uint32_t k);
+ * that take explicit assignments: element 5 of a row is 0 where n_fallback is.
+ * One lane per assignment. */
+int apc_pack_allowed_columns(const apc_problem* p, const uint8_t* flags, const int64_t* col_off,
+                             int32_t max_words, uint64_t* colbits, void* stream);
+int apc_sample_feasible(const apc_problem* p, const uint64_t* colbits, const int64_t* col_off, uint64_t seed,
+                        int64_t first, int64_t n_assign, const int32_t* node_gid, int32_t first_node,
+                        uint16_t* assign, int32_t* n_fallback, void* stream);
+uint32_t apc_sample_rank(uint64_t seed, int64_t a, int32_t node, uint32_t count);
 
 /* apc_score_random_assignments for a graph too large to keep its coefficients
  * resident: the problem holds a window of the graph's nodes (preceded by

@@ -669,11 +669,12 @@ def plain_draw(seed: int, a: int, gid: int, nstrat: int) -> int:
     return (h * nstrat) >> 32
 
 
-def reservoir_takes(seed: int, a: int, gid: int, k: int) -> bool:
-    """Whether the k-th allowed strategy (k >= 1) of node gid replaces the pick."""
-    h = _finalise32(_assignment_hash(seed, a) ^ (((gid + 1) * 0xC2B2AE3D) & _M32) ^ ((k * 0x9E3779B1) & _M32)
-                    ^ 0x68E31DA4)
-    return ((h * k) >> 32) == 0
+def sample_rank(seed: int, a: int, gid: int, count: int) -> int:
+    """Which of the ``count`` allowed strategies of node gid is taken, counted in
+    out_idx order: a 32-bit mix of (seed, assignment, node) of its own, scaled to
+    [0, count) by a multiply-high."""
+    h = _finalise32(_assignment_hash(seed, a) ^ (((gid + 1) * 0xC2B2AE3D) & _M32) ^ 0x68E31DA4)
+    return (h * count) >> 32
 
 
 def sample_feasible(g, forbidden, seed: int, a: int, node_gid=None, first_node: int = 0, given=None):
@@ -691,8 +692,8 @@ def sample_feasible(g, forbidden, seed: int, a: int, node_gid=None, first_node: 
     for v in range(first_node, N):
         gid = int(node_gid[v]) if node_gid is not None else v
         S = int(g.node_nstrat[v])
-        count, pick = 0, 0
         edges = range(int(g.node_edge_off[v]), int(g.node_edge_off[v + 1]))
+        allowed = []
         for o in range(S):
             ok = True
             for e in edges:
@@ -702,9 +703,10 @@ def sample_feasible(g, forbidden, seed: int, a: int, node_gid=None, first_node: 
                     ok = False
                     break
             if ok:
-                count += 1
-                if reservoir_takes(seed, a, gid, count):
-                    pick = o
+                allowed.append(o)
+        count, pick = len(allowed), 0
+        if count:
+            pick = allowed[sample_rank(seed, a, gid, count)]
         if count == 0:
             pick = plain_draw(seed, a, gid, S)
             fallbacks += 1

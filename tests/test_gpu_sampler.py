@@ -58,8 +58,7 @@ def test_sampled_assignments_equal_the_oracles(CostEngine, name):
     # and the plain draws of the same counters do select forbidden variables on these graphs
     plain = eng.score_random(9, 1000, n).cpu().numpy()
     assert (plain[:, 5] > 0).mean() > (scores[:, 5] > 0).mean()
-    # a large batch takes the lane-per-assignment kernel (the one above a wavefront per
-    # assignment): the same choices for the same counters
+    # a large batch: the same choices for the same counters
     big, big_fb = eng.sample_feasible(seed=9, first=1000, count=65536)
     assert np.array_equal(big[:, :n].cpu().numpy(), assign) and np.array_equal(big_fb[:n].cpu().numpy(), fallback)
     a = 65535
@@ -82,3 +81,68 @@ def test_sampler_continues_from_given_rows(CostEngine):
     assert torch.equal(part, whole)
     # the tail's fallbacks are a part of the whole's
     assert bool((fb_part <= fb_whole).all())
+
+
+def _wide_graph():
+    """A consumer with 700 strategies (more than a lane keeps in registers: the words are
+    formed twice), one with eight argument rows (more than the six a lane keeps), and a
+    small one, over producers of a few strategies each."""
+    import itertools
+
+    from autoparallel_amd import packed
+    from autoparallel_amd.packed import GraphBuilder, NodeDesc
+
+    b = GraphBuilder((2, 2, 2, 2), 8)
+    m = b.meta((8, 16, 32, 64), (32768, 2048, 64, 1), 4, packed.DT_F32)
+    codes = [0x00, 0x40, 0x41, 0x42, 0x43, 0x80]
+    tuples = list(itertools.product(codes, repeat=4))
+    rng = np.random.default_rng(3)
+
+    def specs(n):
+        return [b.spec(m, tuples[i]) for i in rng.choice(len(tuples), n, replace=False)]
+
+    prods = []
+    for k in range(8):
+        s = specs(5 + k)
+        prods.append(b.add_node(NodeDesc(f"p{k}", in_specs=[[x] for x in s], out_specs=[[x] for x in s], inputs=[],
+                                         default_rows=[[[0.0]] for _ in s])))
+    wide = specs(700)
+    b.add_node(NodeDesc("wide", in_specs=[[x] for x in wide], out_specs=[[x] for x in wide], inputs=[prods[0]]))
+    many = specs(40)
+    b.add_node(NodeDesc("many_args", in_specs=[[x] * 8 for x in many], out_specs=[[x] for x in many], inputs=prods))
+    small = specs(9)
+    b.add_node(NodeDesc("small", in_specs=[[x, x] for x in small], out_specs=[[x] for x in small],
+                        inputs=[len(prods), len(prods) + 1]))
+    return b.pack()
+
+
+def test_bit_columns_are_the_flags_and_wide_nodes_sample_like_the_oracle(CostEngine):
+    g = _wide_graph()
+    eng = CostEngine(g).build(clamp_inf=True)
+    ref = O.GraphOracle(g).build()
+    _, forbidden = O.clamp_inf(ref["cost"])
+    assert forbidden.any() and not forbidden.all()
+    # the packed columns, bit by bit, against the flags they were made from
+    colbits, d_off, max_words = eng._allowed_columns()
+    torch.cuda.synchronize()
+    bits, off = colbits.cpu().numpy().view(np.uint64), d_off.cpu().numpy()
+    flags = eng.results()["flags"]
+    assert max_words == (700 + 63) // 64
+    for e in range(g.num_edges):
+        sdst, ssrc, base = int(g.edge_sdst[e]), int(g.edge_ssrc[e]), int(g.edge_off[e])
+        W = (sdst + 63) // 64
+        block = (flags[base: base + sdst * ssrc].reshape(sdst, ssrc) & 2) == 0  # [o][j]: allowed
+        for j in range(ssrc):
+            words = bits[off[e] + j * W: off[e] + (j + 1) * W]
+            got = np.unpackbits(words.view(np.uint8), bitorder="little")[: W * 64].astype(bool)
+            assert np.array_equal(got[:sdst], block[:, j]) and not got[sdst:].any(), (e, j)
+    # and the draws
+    n = 200
+    assign, fallback = eng.sample_feasible(seed=21, first=7, count=n)
+    assign, fallback = assign.cpu().numpy(), fallback.cpu().numpy()
+    picked_high = False
+    for a in range(n):
+        want, want_fb = O.sample_feasible(g, forbidden, 21, 7 + a)
+        assert assign[:, a].tolist() == want and int(fallback[a]) == want_fb, a
+        picked_high |= want[8] >= 512  # the 700-strategy node reaches its last words
+    assert picked_high

@@ -246,7 +246,7 @@ def test_abi_exports_every_declared_symbol():
     for name in sorted(declared):
         assert hasattr(lib, name), f"{name} declared in apc.h but not exported"
     assert set(_lib.EXPORTED_SYMBOLS) == declared
-    assert lib.apc_version() == _lib.ABI_VERSION == 4
+    assert lib.apc_version() == _lib.ABI_VERSION == 5
     # struct sizes agree between the header's layout and the ctypes mirror
     assert packed.PackedGraph.EDGE_DTYPE.itemsize == 64
 
