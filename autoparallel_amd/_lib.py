@@ -174,6 +174,8 @@ class ApcSchedule(C.Structure):
         ("use_off", C.c_void_p),
         ("use_st", C.c_void_p),
         ("initial_bytes", C.c_int64),
+        ("comm_slot", C.c_void_p),
+        ("n_comm", C.c_int32),
     ]
 
 

@@ -324,6 +324,10 @@ class ScheduleEstimator:
         for name in ("dur", "stream", "flags", "wait_src", "st_bytes", "st_freeable", "st_users",
                      "alloc_off", "alloc_st", "use_off", "use_st"):
             setattr(s, name, up(name, getattr(ps, name)))
+        # the nodes whose end time the walk keeps (those on a stream of their own), numbered
+        on_stream = ps.stream != 0
+        slot = np.where(on_stream, np.cumsum(on_stream) - 1, -1).astype(np.int32)
+        s.comm_slot, s.n_comm = up("comm_slot", slot), int(on_stream.sum())
         self.sched = s
 
     def evaluate(self, orders: Optional[np.ndarray] = None):
@@ -336,10 +340,14 @@ class ScheduleEstimator:
         else:
             orders = np.ascontiguousarray(orders, np.int32)
             assert orders.ndim == 2 and orders.shape[1] == N
-            # each row a permutation: the kernel indexes node arrays with it
-            assert (np.sort(orders, axis=1) == np.arange(N, dtype=np.int32)).all(), "not permutations"
             B = orders.shape[0]
             d_orders = torch.from_numpy(orders).to(self.device)
+            # each row a permutation: the kernel indexes node arrays with it (checked on the
+            # device, where sorting the rows of a large batch takes a fraction of the host's time)
+            rows_sorted = torch.sort(d_orders, dim=1).values
+            assert bool((rows_sorted == torch.arange(N, dtype=torch.int32, device=self.device)).all().item()), \
+                "not permutations"
+            del rows_sorted
             order_ptr = C.c_void_p(d_orders.data_ptr())
         end = torch.empty(max(B * N, 1), dtype=torch.float64, device=self.device)
         rem = torch.empty(max(B * S, 1), dtype=torch.int32, device=self.device)

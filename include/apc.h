@@ -858,6 +858,14 @@ typedef struct apc_schedule {
   const int32_t* use_off;     /* [n_node+1] into use_st: storages the node reads       */
   const int32_t* use_st;
   int64_t initial_bytes;      /* live before the first node (graph inputs, attributes) */
+  /* optional accelerator, derived from `stream` by the host (NULL: end times stay
+   * in end_scratch): comm_slot[v] numbers the nodes that run on a stream other
+   * than 0, the only ones whose end time is kept, 0 .. n_comm-1 in any order; -1
+   * for the others.  With it, and when 48 B per node, 264 B per storage (plus
+   * one) and 512 B per such node (plus two) fit in the 160 KB of a CU's LDS, the
+   * walk touches global memory for the orders alone. */
+  const int32_t* comm_slot;   /* [n_node] or NULL                                     */
+  int32_t n_comm;
 } apc_schedule;
 
 /* Replaces estimate_graph_metrics
@@ -872,8 +880,10 @@ typedef struct apc_schedule {
  * its allocator is scheduled and freed at the last scheduled of its readers).
  * times[b * 4 ..] = total_time, compute_time, communication_time,
  * exposed_comm_time; peak[b] = peak_memory.  Scratch, device memory the caller
- * provides and the call overwrites: end_scratch double[n_sched * n_node],
- * remaining_scratch int32[n_sched * n_storage].  Every order must be a
+ * provides and the call may overwrite: end_scratch double[n_sched * n_node],
+ * remaining_scratch int32[n_sched * n_storage] (a graph small enough for a
+ * CU's LDS is walked from there by schedule_metrics_lds_kernel and leaves one
+ * or both untouched; schedule_metrics_kernel uses both).  Every order must be a
  * permutation that schedules a storage's allocator before its readers. */
 int apc_schedule_metrics(const apc_schedule* s, const int32_t* order, int64_t n_sched,
                          double* end_scratch, int32_t* remaining_scratch, double* times,

@@ -59,18 +59,24 @@ def test_batch_of_orders_matches_oracle(golden):
         assert len({float(t) for t in times[:, 0]}) > 1
 
 
-def test_large_batch_properties(golden):
-    """20 000 orders of the largest graph: invariants that hold for any order."""
+@pytest.mark.parametrize("copies", [100, 350])
+def test_large_batch_properties(golden, copies):
+    """20 000 and 70 000 orders of the largest graph (a workgroup's 64 orders on two
+    wavefronts and on one: the launch has several workgroups for every CU): the oracle's
+    numbers for the distinct orders, and invariants that hold for any order."""
     case = golden["cases"][-1]
     gm, est = SG.build_graph(case["desc"])
     ps = SM.pack_schedule(gm, est)
     base = ps.random_orders(200, seed=7)
-    orders = np.tile(base, (100, 1))
+    orders = np.tile(base, (copies, 1))
     times, peak = SM.ScheduleEstimator(ps).evaluate(orders)
-    assert times.shape == (20000, 4)
+    assert times.shape == (200 * copies, 4)
+    for b in range(0, 200, 7):
+        want = SO.schedule_metrics(ps, base[b])
+        assert tuple(times[b]) == want[:4] and int(peak[b]) == want[4], (b, times[b], want)
     # replicas of an order agree bit for bit wherever they sit in the batch
-    assert (times.reshape(100, 200, 4) == times[:200][None]).all()
-    assert (peak.reshape(100, 200) == peak[:200][None]).all()
+    assert (times.reshape(copies, 200, 4) == times[:200][None]).all()
+    assert (peak.reshape(copies, 200) == peak[:200][None]).all()
     launch = ps.n_node  # every node adds 1 us to its own stream
     comp = times[:, 1]
     assert np.allclose(comp, comp[0], rtol=1e-12)  # same terms, another order of summation
@@ -201,3 +207,49 @@ def test_runtime_estimator_of_a_lowered_graph():
         dist.destroy_process_group()
         if had:
             dist.init_process_group("fake", store=FakeStore(), rank=0, world_size=8)
+
+
+@pytest.mark.parametrize("n_layers", [32, 45, 80])
+def test_synthetic_schedule_from_lds_and_from_scratch_memory(n_layers):
+    """A graph whose records and reader counts fit a CU's LDS is walked from there (with
+    the end times of its collectives when those fit too), a larger one from the caller's
+    scratch arrays: each against the oracle, with a last wavefront that is only partly
+    filled."""
+    ps = SM.synthetic_schedule(n_layers, seed=3)
+    state = 48 * ps.n_node + 264 * (ps.n_storage + 1)
+    ends = 512 * (int((ps.stream != 0).sum()) + 2)
+    assert (state <= 160 * 1024) == (n_layers < 80) and (state + ends <= 160 * 1024) == (n_layers == 32)
+    orders = ps.random_orders(130, seed=5)
+    print(f"  {ps.n_node} nodes, {ps.n_storage} storages, {state} + {ends} bytes", flush=True)
+    times, peak = SM.ScheduleEstimator(ps).evaluate(orders)
+    for b, order in enumerate(orders):
+        want = SO.schedule_metrics(ps, order)
+        assert tuple(times[b]) == want[:4] and int(peak[b]) == want[4], (b, times[b], peak[b], want)
+    assert len({int(x) for x in peak}) > 1
+
+
+def test_a_node_that_reads_more_storages_than_its_record_names():
+    """Seven producers and one node that reads all of them (a record in LDS names four
+    of a node's storages; the rest come from the use list)."""
+    n_prod = 7
+    N = n_prod + 3
+    deps = [[] for _ in range(n_prod)] + [list(range(n_prod)), [n_prod], [n_prod + 1]]
+    use_off = np.concatenate([[0], np.cumsum([len(d) for d in deps])]).astype(np.int32)
+    use_st = np.asarray([u for d in deps for u in d], np.int32)
+    flags = np.zeros(N, np.uint8)
+    flags[-1] = SM.SCHED_NO_MEM
+    alloc_st = np.arange(N - 1, dtype=np.int32)
+    ps = SM.PackedSchedule(
+        dur=np.arange(1.0, N + 1.0), stream=np.zeros(N, np.int32), flags=flags, wait_src=np.full(N, -1, np.int32),
+        n_stream=1, st_bytes=(np.arange(N, dtype=np.int64) + 1) * 1000, st_freeable=np.ones(N, np.uint8),
+        st_users=np.bincount(use_st, minlength=N).astype(np.int32),
+        alloc_off=np.minimum(np.arange(N + 1), N - 1).astype(np.int32), alloc_st=alloc_st,
+        use_off=use_off, use_st=use_st, initial_bytes=500, dep_off=use_off.copy(), dep_node=use_st.copy())
+    ps.validate()
+    orders = ps.random_orders(70, seed=1)
+    times, peak = SM.ScheduleEstimator(ps).evaluate(orders)
+    for b, order in enumerate(orders):
+        want = SO.schedule_metrics(ps, order)
+        assert tuple(times[b]) == want[:4] and int(peak[b]) == want[4], (b, order, peak[b], want)
+    # all seven producers live when the reader allocates, then only its own output and its reader's
+    assert int(peak[0]) == 500 + sum(1000 * (k + 1) for k in range(n_prod + 1))
