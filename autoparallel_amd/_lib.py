@@ -263,7 +263,7 @@ _SIGNATURES = {
     "apc_sample_feasible": (
         C.c_int,
         [C.POINTER(ApcProblem), C.c_void_p, C.c_void_p, C.c_uint64, C.c_int64, C.c_int64, C.c_void_p, C.c_int32,
-         C.c_void_p, C.c_void_p, C.c_void_p]),
+         C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
     "apc_sample_rank": (C.c_uint32, [C.c_uint64, C.c_int64, C.c_int32, C.c_uint32]),
     "apc_local_shapes": (
         C.c_int,

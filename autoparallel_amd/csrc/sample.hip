@@ -121,6 +121,7 @@ __global__ void __launch_bounds__(kBlock)
 sample_feasible_kernel(apc_problem p, const uint64_t* __restrict__ colbits,
                        const int64_t* __restrict__ col_off, uint64_t seed, int64_t first,
                        int64_t n_assign, const int32_t* __restrict__ node_gid, int first_node,
+                       const uint64_t* __restrict__ row_filter, const int64_t* __restrict__ filter_off,
                        uint16_t* __restrict__ assign, int32_t* __restrict__ n_fallback) {
   const int64_t a = (int64_t)blockIdx.x * kBlock + threadIdx.x;
   if (a >= n_assign) return;
@@ -134,6 +135,7 @@ sample_feasible_kernel(apc_problem p, const uint64_t* __restrict__ colbits,
   // assignments of the same window: 62 -> 72 ms), so it runs without.
   struct Head {
     int S, gid, e0, e1;
+    int64_t keep;  // first word of the node's filter, or -1
     int src[kSampleArgs];
     int64_t off[kSampleArgs];
   };
@@ -143,6 +145,7 @@ sample_feasible_kernel(apc_problem p, const uint64_t* __restrict__ colbits,
     h.gid = node_gid ? node_gid[v] : v;
     h.e0 = p.node_edge_off[v];
     h.e1 = p.node_edge_off[v + 1];
+    h.keep = filter_off ? filter_off[v] : -1;
     if (kAhead) {
 #pragma unroll
       for (int i = 0; i < kSampleArgs; ++i) {
@@ -177,6 +180,7 @@ sample_feasible_kernel(apc_problem p, const uint64_t* __restrict__ colbits,
     // word w of the node's allowed strategies
     auto allowed_word = [&](int w) -> uint64_t {
       uint64_t m = word_mask(S, w);
+      if (head.keep >= 0) m &= row_filter[head.keep + w];  // the strategies the node may take at all
 #pragma unroll
       for (int i = 0; i < kSampleArgs; ++i)
         if (e0 + i < e1) m &= col[i][w];
@@ -254,20 +258,23 @@ int apc_pack_allowed_columns(const apc_problem* p, const uint8_t* flags, const i
 
 int apc_sample_feasible(const apc_problem* p, const uint64_t* colbits, const int64_t* col_off, uint64_t seed,
                         int64_t first, int64_t n_assign, const int32_t* node_gid, int32_t first_node,
-                        uint16_t* assign, int32_t* n_fallback, void* stream) {
+                        const uint64_t* row_filter, const int64_t* filter_off, uint16_t* assign,
+                        int32_t* n_fallback, void* stream) {
   if (int rc = validate_problem(p)) return rc;
   if (n_assign <= 0) return 0;
   if (!assign || !n_fallback || (p->n_entry > 0 && (!colbits || !col_off)))
     return fail(APC_ERR_INVALID, "apc_sample_feasible: null argument%s");
   if (first_node < 0 || first_node > p->n_node)
     return fail(APC_ERR_INVALID, "apc_sample_feasible: first_node out of range%s");
+  if ((row_filter == nullptr) != (filter_off == nullptr))
+    return fail(APC_ERR_INVALID, "apc_sample_feasible: row_filter and filter_off come together%s");
   const dim3 grid((unsigned)((n_assign + kBlock - 1) / kBlock));
   if (n_assign < 65536)  // fewer wavefronts than SIMDs
     hipLaunchKernelGGL(sample_feasible_kernel<true>, grid, dim3(kBlock), 0, (hipStream_t)stream, *p, colbits, col_off,
-                       seed, first, n_assign, node_gid, (int)first_node, assign, n_fallback);
+                       seed, first, n_assign, node_gid, (int)first_node, row_filter, filter_off, assign, n_fallback);
   else
     hipLaunchKernelGGL(sample_feasible_kernel<false>, grid, dim3(kBlock), 0, (hipStream_t)stream, *p, colbits, col_off,
-                       seed, first, n_assign, node_gid, (int)first_node, assign, n_fallback);
+                       seed, first, n_assign, node_gid, (int)first_node, row_filter, filter_off, assign, n_fallback);
   return check_launch("sample_feasible_kernel");
 }
 

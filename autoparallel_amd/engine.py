@@ -784,14 +784,16 @@ class CostEngine:
         return colbits, d_off, max_words
 
     def sample_feasible(self, seed: int, first: int, count: int, node_gid: Optional[np.ndarray] = None,
-                        first_node: int = 0, assign: Optional[torch.Tensor] = None):
+                        first_node: int = 0, assign: Optional[torch.Tensor] = None,
+                        row_filter: Optional[dict] = None):
         """``count`` assignments drawn node by node among the strategies that select
         no forbidden (non-finite) entry against the choices made for the node's
         producers (apc_pack_allowed_columns, then apc_sample_feasible).  Returns
         (assign uint16[n_node, count] on the device, n_fallback int32[count]: nodes
         that had no such strategy and took the plain draw).  ``assign``/``first_node``:
         rows below first_node are given (a window of a larger graph); ``node_gid``:
-        ids for the hashes."""
+        ids for the hashes; ``row_filter``: {node: bool per strategy}, the strategies a
+        node may take at all (feasible_plan.plan_filters)."""
         assert self.built
         N = self.g.num_nodes
         if assign is None:
@@ -803,10 +805,28 @@ class CostEngine:
             d_gid = torch.from_numpy(np.ascontiguousarray(node_gid, np.int32)).to(self.device)
         fallback = torch.empty(count, dtype=torch.int32, device=self.device)
         colbits, d_off, _ = self._allowed_columns()
+        d_keep = d_keep_off = None
+        if row_filter:
+            # bit out_idx mod 64 of word out_idx / 64, the words of the filtered nodes one after the other
+            keep_off = np.full(N, -1, np.int64)
+            words = []
+            at = 0
+            for v in sorted(row_filter):
+                keep = np.asarray(row_filter[v], bool)
+                assert keep.shape == (int(self.g.node_nstrat[v]),)
+                padded = np.zeros(-(-keep.shape[0] // 64) * 64, np.uint8)
+                padded[: keep.shape[0]] = keep
+                w = np.packbits(padded, bitorder="little").view(np.uint64)
+                keep_off[v] = at
+                at += w.shape[0]
+                words.append(w)
+            d_keep = torch.from_numpy(np.concatenate(words).view(np.int64)).to(self.device)
+            d_keep_off = torch.from_numpy(keep_off).to(self.device)
         _lib.check(
             self.lib.apc_sample_feasible(
                 C.byref(self.problem), self._ptr(colbits), self._ptr(d_off), int(seed), int(first), int(count),
-                self._ptr(d_gid), int(first_node), self._ptr(assign), self._ptr(fallback), self._stream()),
+                self._ptr(d_gid), int(first_node), self._ptr(d_keep), self._ptr(d_keep_off), self._ptr(assign),
+                self._ptr(fallback), self._stream()),
             "apc_sample_feasible")
         return assign, fallback
 

@@ -37,6 +37,7 @@ from .packed import (
     OP_ZERO,
     PARTIAL_SUM,
     PARTIAL_AVG,
+    PLC_KIND_MASK,
     PLC_PARTIAL,
     PLC_R,
     GraphBuilder,
@@ -1163,6 +1164,59 @@ def _stress_header(seed: int, v: int, nd: int, s_min: int, s_max: int):
     return r, shape, dt, out
 
 
+def _stress_body(seed: int, v: int, nd: int, header):
+    """(op class, producers, placement codes int[S, nd] of the input spec per producer and
+    strategy, the node's generator for what else it draws) of node v, from (seed, v) and the
+    headers of its producers alone."""
+    rng = np.random.default_rng([seed, v, 1])
+    op = ("matmul", "elementwise", "reduction", "view")[int(rng.integers(0, 4))]
+    if v == 0:
+        want_in = 0
+    elif op == "matmul":
+        want_in = 3 if rng.random() < 0.7 else 2  # with or without a bias
+    elif op == "elementwise":
+        want_in = int(rng.integers(1, 5))
+    else:
+        want_in = 1
+    inputs = [int(rng.integers(0, v)) for _ in range(want_in)]
+    S = len(header(v)[3])
+    in_codes = []
+    for u in inputs:
+        ru = header(u)[0]
+        codes = np.asarray([R] + [shard(d) for d in range(ru)] + [P])
+        in_codes.append(codes[rng.integers(0, len(codes), size=(S, nd))])
+    return op, inputs, in_codes, rng
+
+
+def stress_dag_partial_masks(n_total: int, lo: int, hi: int, mesh_shape: Sequence[int] = (4, 8, 8), seed: int = 0,
+                             s_min: int = 4, s_max: int = 512):
+    """{v: feasible_plan.NodeMasks} for the nodes [lo, hi) of the stress DAG, without
+    building their window: which mesh dims hold a Partial in the output spec of every
+    strategy and in its input spec per producer (what feasible_plan.window_masks reads
+    off the packed window)."""
+    from .feasible_plan import NodeMasks
+
+    assert 0 <= lo < hi <= n_total
+    nd = len(mesh_shape)
+    headers = {}
+
+    def header(v):
+        if v not in headers:
+            headers[v] = _stress_header(seed, v, nd, s_min, s_max)
+        return headers[v]
+
+    weights = 1 << np.arange(nd)
+
+    def mask(codes):
+        return (((codes & PLC_KIND_MASK) == PLC_PARTIAL) * weights).sum(axis=1).astype(np.uint8)
+
+    out = {}
+    for v in range(lo, hi):
+        _, inputs, in_codes, _ = _stress_body(seed, v, nd, header)
+        out[v] = NodeMasks(out=mask(header(v)[3]), producers=list(inputs), wants=[mask(c) for c in in_codes]).finish()
+    return out
+
+
 def stress_dag_window(
     n_total: int,
     lo: int,
@@ -1194,19 +1248,9 @@ def stress_dag_window(
     bodies = []
     external = set()
     for v in range(lo, hi):
-        rng = np.random.default_rng([seed, v, 1])
-        op = ("matmul", "elementwise", "reduction", "view")[int(rng.integers(0, 4))]
-        if v == 0:
-            want_in = 0
-        elif op == "matmul":
-            want_in = 3 if rng.random() < 0.7 else 2  # with or without a bias
-        elif op == "elementwise":
-            want_in = int(rng.integers(1, 5))
-        else:
-            want_in = 1
-        inputs = [int(rng.integers(0, v)) for _ in range(want_in)]
+        op, inputs, in_codes, rng = _stress_body(seed, v, nd, header)
         external.update(u for u in inputs if u < lo)
-        bodies.append((v, op, inputs, rng))
+        bodies.append((v, op, inputs, in_codes, rng))
     standins = sorted(external)
     local = {u: i for i, u in enumerate(standins)}
     local.update({v: len(standins) + (v - lo) for v in range(lo, hi)})
@@ -1228,18 +1272,14 @@ def stress_dag_window(
 
     for u in standins:
         add_input(u)
-    for v, op, inputs, rng in bodies:
+    for v, op, inputs, in_codes, rng in bodies:
         r, shape, dt, out_tuples = header(v)
         if not inputs:
             add_input(v)
             continue
         S = len(out_tuples)
         out_specs = [[w] for w in specs_of(v, out_tuples)]
-        cols = []
-        for u in inputs:
-            ru = header(u)[0]
-            codes = np.asarray([R] + [shard(d) for d in range(ru)] + [P])
-            cols.append(specs_of(u, codes[rng.integers(0, len(codes), size=(S, nd))]))
+        cols = [specs_of(u, codes) for u, codes in zip(inputs, in_codes)]
         in_specs = [list(row) for row in zip(*cols)]
         loc = [local[u] for u in inputs]
         isz = _ITEMSIZE[dt]

@@ -53,6 +53,13 @@ def _make_window(task):
     return lo, hi, g, gid, n_standin
 
 
+def _window_masks(task):
+    from autoparallel_amd import graphgen
+
+    n_total, lo, hi, mesh, seed, s_min, s_max = task
+    return graphgen.stress_dag_partial_masks(n_total, lo, hi, mesh, seed, s_min, s_max)
+
+
 def score_in_windows(
     n_total: int,
     window: int,
@@ -66,6 +73,7 @@ def score_in_windows(
     max_windows: Optional[int] = None,
     progress=None,
     feasible: bool = False,
+    plan: bool = True,
 ):
     """Scores ``n_assign`` on-device drawn assignments of the n_total-node stress
     DAG, window by window.  Returns (scores float64[n_assign, 6] on the host,
@@ -73,7 +81,11 @@ def score_in_windows(
     strategies that select no forbidden entry against the producers' choices
     (CostEngine.sample_feasible) instead of independently per node; the choices
     of all nodes are then kept on the device (2 bytes per node and assignment),
-    since a later window's stand-in producers carry the choices of their nodes."""
+    since a later window's stand-in producers carry the choices of their nodes.
+    ``plan`` (with ``feasible``): before the first window, the nodes that could run
+    out of strategies are found from the spec words of the whole DAG and their
+    producers confined to the strategies that serve them (feasible_plan), so that
+    no node falls back to the plain draw."""
     import torch
 
     from autoparallel_amd.engine import CostEngine
@@ -96,10 +108,24 @@ def score_in_windows(
     pool = None
     if workers > 1 and len(tasks) > 1:
         pool = mp.get_context("spawn").Pool(min(workers, len(tasks)))
-        results = pool.imap(_make_window, tasks)
-    else:
-        results = map(_make_window, tasks)
+    filters = {}
     try:
+        if feasible and plan:
+            from autoparallel_amd import feasible_plan
+
+            t_mark = time.perf_counter()
+            masks = {}
+            for part in (pool.imap_unordered(_window_masks, tasks) if pool else map(_window_masks, tasks)):
+                masks.update(part)
+            filters, stuck = feasible_plan.plan_filters(masks)
+            stats["plan_s"] = time.perf_counter() - t_mark
+            stats["plan_confined_nodes"] = len(filters)
+            stats["plan_stuck_nodes"] = len(stuck)
+            # nodes that no assignment of the graph can serve: none of their strategies finds,
+            # for every argument, a producer's strategy that offers the Partials it asks for
+            stats["unservable_nodes"] = [v for v in stuck if feasible_plan.unservable(masks, v)]
+            del masks
+        results = pool.imap(_make_window, tasks) if pool else map(_make_window, tasks)
         t_mark = time.perf_counter()
         for lo, hi, g, gid, n_standin in results:
             stats["wait_for_window_s"] += time.perf_counter() - t_mark  # the host's generation and packing
@@ -113,8 +139,9 @@ def score_in_windows(
             if feasible:
                 # the stand-ins' rows are the choices made for their nodes in earlier windows
                 local = choices[torch.from_numpy(gid.astype(np.int64)).to(choices.device)].contiguous()
+                keep = {i: filters[int(gid[i])] for i in range(n_standin, g.num_nodes) if int(gid[i]) in filters}
                 _, fb = eng.sample_feasible(assign_seed, 0, n_assign, node_gid=gid, first_node=n_standin,
-                                            assign=local.view(torch.uint16))
+                                            assign=local.view(torch.uint16), row_filter=keep)
                 choices[lo:hi] = local[n_standin:]
                 fallbacks += fb
                 ev[2].record()
@@ -164,6 +191,8 @@ def main():
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--feasible", action="store_true",
                     help="draw the assignments node by node among the strategies without a forbidden entry")
+    ap.add_argument("--no-plan", action="store_true",
+                    help="with --feasible: do not confine the producers of the nodes that could run out of strategies")
     args = ap.parse_args()
 
     def progress(st, wall):
@@ -173,7 +202,7 @@ def main():
 
     scores, st = score_in_windows(args.nodes, args.window, args.assignments, seed=args.seed,
                                   workers=args.workers, max_windows=args.max_windows, progress=progress,
-                                  feasible=args.feasible)
+                                  feasible=args.feasible, plan=not args.no_plan)
     obj = scores[:, 4]
     st.update({
         "workload": f"stress DAG, {args.nodes} nodes, mesh (4,8,8), windows of {args.window}",

@@ -491,8 +491,13 @@ def main():
                 "entries_per_s_device_build": st["entries"] / st["build_device_s"],
                 "edge_terms_per_s_scoring": scores.shape[0] * st["edges"] / st["score_device_s"],
                 "fraction_without_forbidden_entry": float((scores[:, 5] == 0).mean()),
+                "forbidden_entries_per_assignment_mean": float(scores[:, 5].mean()),
                 "objective_min": float(scores[:, 4].min()), "objective_mean": float(scores[:, 4].mean()),
             })
+            if feasible:
+                st["note"] = ("unservable_nodes: none of their strategies finds, for every argument, a strategy of "
+                              "the producer that offers the Partial placements it asks for; they select a forbidden "
+                              "entry in every assignment of this DAG, so no assignment of it is free of them")
             legs[label] = st
         out["windowed_stress_dag_200k"] = legs
     if args.fx_layers > 0 and args.workload == "llama3_8b_fwd_bwd_mesh8x8":

@@ -666,14 +666,22 @@ uint32_t apc_random_assignment(uint64_t seed, int64_t a, int32_t node, int32_t n
  * assign: uint16[n_node][n_assign], written for v >= first_node; the rows below
  * first_node are read (choices made earlier, e.g. for the stand-in nodes of a
  * window of a larger graph).  node_gid: id of every node for the hashes (NULL:
- * its index).  Score the result with apc_score_assignments or the batch scorers
+ * its index).  row_filter / filter_off (both or neither): strategies a node may
+ * take at all, whatever its producers chose; filter_off[v] is the first of the W
+ * words of node v's filter in row_filter (bit out_idx mod 64 of word out_idx / 64),
+ * or -1 for a node without one.  With filters that confine the producers of the
+ * nodes that would otherwise run out of strategies (autoparallel_amd/feasible_plan.py
+ * makes them on the host), no node of the planner stress DAG falls back.  The
+ * plain draw of a node that does fall back ignores its filter.
+ * Score the result with apc_score_assignments or the batch scorers
  * that take explicit assignments: element 5 of a row is 0 where n_fallback is.
  * One lane per assignment. */
 int apc_pack_allowed_columns(const apc_problem* p, const uint8_t* flags, const int64_t* col_off,
                              int32_t max_words, uint64_t* colbits, void* stream);
 int apc_sample_feasible(const apc_problem* p, const uint64_t* colbits, const int64_t* col_off, uint64_t seed,
                         int64_t first, int64_t n_assign, const int32_t* node_gid, int32_t first_node,
-                        uint16_t* assign, int32_t* n_fallback, void* stream);
+                        const uint64_t* row_filter, const int64_t* filter_off, uint16_t* assign,
+                        int32_t* n_fallback, void* stream);
 uint32_t apc_sample_rank(uint64_t seed, int64_t a, int32_t node, uint32_t count);
 
 /* apc_score_random_assignments for a graph too large to keep its coefficients

@@ -677,13 +677,16 @@ def sample_rank(seed: int, a: int, gid: int, count: int) -> int:
     return (h * count) >> 32
 
 
-def sample_feasible(g, forbidden, seed: int, a: int, node_gid=None, first_node: int = 0, given=None):
+def sample_feasible(g, forbidden, seed: int, a: int, node_gid=None, first_node: int = 0, given=None,
+                    row_filter=None):
     """One assignment, node by node in graph order: node v gets, uniformly, one of
     its strategies whose entries against the choices of its producers are all
     allowed (``forbidden``: uint8 per slot, the non-finite costs that
     add_inf_cost_constraint pins to zero, optimize_sharding.py:803-812); a node
     without one takes the plain draw and is counted.  ``given``: the choices of
-    the nodes below first_node.  Returns (choices per node, number of fallbacks)."""
+    the nodes below first_node.  ``row_filter``: {node: bool per strategy}, the
+    strategies a node may take at all.  Returns (choices per node, number of
+    fallbacks)."""
     N = g.num_nodes
     assign = [0] * N
     for v in range(first_node):
@@ -694,9 +697,12 @@ def sample_feasible(g, forbidden, seed: int, a: int, node_gid=None, first_node: 
         S = int(g.node_nstrat[v])
         edges = range(int(g.node_edge_off[v]), int(g.node_edge_off[v + 1]))
         allowed = []
+        keep = row_filter.get(v) if row_filter else None
         for o in range(S):
-            ok = True
+            ok = keep is None or bool(keep[o])
             for e in edges:
+                if not ok:
+                    break
                 u = int(g.edge_src_node[e])
                 j = assign[u] if u >= 0 else 0
                 if forbidden[int(g.edge_off[e]) + o * int(g.edge_ssrc[e]) + j]:

@@ -146,3 +146,31 @@ def test_bit_columns_are_the_flags_and_wide_nodes_sample_like_the_oracle(CostEng
         assert assign[:, a].tolist() == want and int(fallback[a]) == want_fb, a
         picked_high |= want[8] >= 512  # the 700-strategy node reaches its last words
     assert picked_high
+
+
+def test_filtered_draws_equal_the_oracle_and_never_fall_back(CostEngine):
+    """Row filters from the plan (feasible_plan): the device's draws equal the oracle's
+    with the same filters, no node falls back and no forbidden entry is selected, where
+    the walk without filters falls back several times per assignment."""
+    from autoparallel_amd import feasible_plan as FP
+    from autoparallel_amd import graphgen
+
+    g, _, _ = graphgen.stress_dag_window(600, 0, 600, (4, 8, 8), 0, 4, 48)
+    filters, stuck = FP.plan_filters(FP.window_masks(g))
+    assert filters and not stuck
+    eng = CostEngine(g).build(clamp_inf=True)
+    ref = O.GraphOracle(g).build()
+    _, forbidden = O.clamp_inf(ref["cost"])
+    n = 300
+    plain, plain_fb = eng.sample_feasible(seed=4, first=0, count=n)
+    assign, fallback = eng.sample_feasible(seed=4, first=0, count=n, row_filter=filters)
+    assert int(plain_fb.sum().item()) > n and int(fallback.sum().item()) == 0
+    scores = eng.score(assign).cpu().numpy()
+    assert (scores[:, 5] == 0).all()
+    assign = assign.cpu().numpy()
+    for a in range(0, n, 7):
+        want, want_fb = O.sample_feasible(g, forbidden, 4, a, row_filter=filters)
+        assert assign[:, a].tolist() == want and want_fb == 0, a
+    # the launch that fills the chip (another instance of the kernel): the same draws
+    big, big_fb = eng.sample_feasible(seed=4, first=0, count=65536, row_filter=filters)
+    assert int(big_fb.sum().item()) == 0 and (big[:, :n].cpu().numpy() == assign).all()

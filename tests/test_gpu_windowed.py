@@ -70,22 +70,35 @@ def test_a_window_of_the_full_dag_against_the_compiled_oracle():
 def test_feasible_draws_in_windows_equal_one_pass():
     """Assignments drawn without forbidden entries where the graph allows it: the
     windows carry the choices of earlier nodes along, and give the sample and the
-    sums of one pass over the whole graph, bit for bit."""
+    sums of one pass over the whole graph, bit for bit; without the plan, where nodes
+    fall back, and with it, where none does."""
+    from autoparallel_amd import feasible_plan
     from autoparallel_amd.engine import CostEngine
 
     n = 4096
     g, gid, _ = graphgen.stress_dag_window(N_TOTAL, 0, N_TOTAL, (4, 8, 8), SEED, 4, S_MAX)
     eng = CostEngine(g).build(clamp_inf=True)
-    assign, fb = eng.sample_feasible(1, 0, n)
-    whole = eng.score(assign).cpu().numpy()
     plain = eng.score_random(1, 0, n).cpu().numpy()
-    assert (whole[:, 5] == 0).sum() >= (plain[:, 5] == 0).sum() and whole[:, 5].mean() < plain[:, 5].mean()
-    for window in (60, 97):
-        got, st = windowed.score_in_windows(N_TOTAL, window, n, seed=SEED, assign_seed=1, s_max=S_MAX, workers=1,
-                                            feasible=True)
-        assert (got.view(np.uint64) == whole.view(np.uint64)).all(), window
-        assert st["assignments_without_fallback"] == int((fb == 0).sum().item())
-        assert abs(st["fallback_nodes_per_assignment_mean"] - float(fb.double().mean().item())) < 1e-9
+    # with at most 24 strategies per node the plan cannot serve every node of this graph
+    filters, stuck = feasible_plan.plan_filters(feasible_plan.window_masks(g))
+    fallbacks = {}
+    for plan in (False, True):
+        assign, fb = eng.sample_feasible(1, 0, n, row_filter=filters if plan else None)
+        whole = eng.score(assign).cpu().numpy()
+        assert (whole[:, 5] == 0).sum() >= (plain[:, 5] == 0).sum() and whole[:, 5].mean() < plain[:, 5].mean()
+        fallbacks[plan] = int(fb.sum().item())
+        if plan and not stuck:
+            assert fallbacks[plan] == 0 and (whole[:, 5] == 0).all()
+        for window in (60, 97):
+            got, st = windowed.score_in_windows(N_TOTAL, window, n, seed=SEED, assign_seed=1, s_max=S_MAX, workers=1,
+                                                feasible=True, plan=plan)
+            assert (got.view(np.uint64) == whole.view(np.uint64)).all(), (plan, window)
+            assert st["assignments_without_fallback"] == int((fb == 0).sum().item())
+            assert abs(st["fallback_nodes_per_assignment_mean"] - float(fb.double().mean().item())) < 1e-9
+            assert ("plan_confined_nodes" in st) == plan
+            if plan:
+                assert st["plan_confined_nodes"] == len(filters) and st["plan_stuck_nodes"] == len(stuck)
+    assert fallbacks[True] < fallbacks[False] / 2
 
 
 def test_config5_at_full_size_in_windows():
@@ -103,6 +116,40 @@ def test_config5_at_full_size_in_windows():
     second, st2 = windowed.score_in_windows(200000, 4500, n, workers=14)
     assert st2["entries"] == st["entries"] and st2["windows"] == 45
     assert (first.view(np.uint64) == second.view(np.uint64)).all()
+    # and drawn node by node with the plan that confines the producers of the nodes that
+    # would run out of strategies.  One node of this DAG (194 348: four strategies, each asking
+    # a producer for Partials that none of the producer's strategies offers) selects a forbidden
+    # entry whatever anyone chooses, so no assignment of the DAG is free of them; every other
+    # node is served in every assignment.
+    planned, st3 = windowed.score_in_windows(200000, 3000, n, workers=14, feasible=True)
+    print(f"  planned draws: {st3['plan_confined_nodes']} confined nodes, plan {st3['plan_s']:.1f} s, "
+          f"sampling {st3['sample_device_s']:.2f} s, {st3['fallback_nodes_per_assignment_mean']} fallbacks", flush=True)
+    assert st3["plan_stuck_nodes"] == 1 and st3["unservable_nodes"] == [194348]
+    assert st3["fallback_nodes_per_assignment_mean"] == 1.0 and st3["fallback_nodes_per_assignment_min"] == 1
+    assert (planned[:, 5] >= 1).all() and (planned[:, 5] <= 4).all() and (first[:, 5] > 100).all()
+    assert np.isfinite(planned).all()
+
+
+def test_the_node_of_config5_that_no_assignment_can_serve():
+    """Node 194 348 of the 200 000-node DAG, with its producers as stand-ins, from the
+    flags the device writes: each of its strategies has an argument whose entries are
+    forbidden against every strategy of the producer.  (So every assignment of the DAG
+    selects a forbidden entry, and the ILP over it has no solution.)"""
+    from autoparallel_amd.engine import CostEngine
+
+    g, gid, n_standin = graphgen.stress_dag_window(200000, 194348, 194349)
+    v = g.num_nodes - 1
+    assert int(gid[v]) == 194348 and n_standin == v
+    flags = CostEngine(g).build(clamp_inf=True).results()["flags"]
+    S = int(g.node_nstrat[v])
+    edges = range(int(g.node_edge_off[v]), int(g.node_edge_off[v + 1]))
+    assert S == 4 and len(edges) >= 1
+    for o in range(S):
+        dead = []
+        for e in edges:
+            ssrc, off = int(g.edge_ssrc[e]), int(g.edge_off[e])
+            dead.append(bool(((flags[off + o * ssrc: off + (o + 1) * ssrc] & 2) != 0).all()))
+        assert any(dead), (o, dead)
 
 
 def test_small_batches_of_explicit_assignments_in_a_window():
