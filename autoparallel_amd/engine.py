@@ -793,8 +793,16 @@ class CostEngine:
         that had no such strategy and took the plain draw).  ``assign``/``first_node``:
         rows below first_node are given (a window of a larger graph); ``node_gid``:
         ids for the hashes; ``row_filter``: {node: bool per strategy}, the strategies a
-        node may take at all (feasible_plan.plan_filters)."""
+        node may take at all, or "plan" for the filters feasible_plan.plan_filters makes
+        for this graph (made once per engine)."""
         assert self.built
+        if isinstance(row_filter, str):
+            assert row_filter == "plan" and first_node == 0
+            if "row_filter_plan" not in self._keep:
+                from . import feasible_plan
+
+                self._keep["row_filter_plan"] = feasible_plan.plan_filters(feasible_plan.window_masks(self.g))[0]
+            row_filter = self._keep["row_filter_plan"]
         N = self.g.num_nodes
         if assign is None:
             assert first_node == 0

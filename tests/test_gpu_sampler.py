@@ -165,6 +165,7 @@ def test_filtered_draws_equal_the_oracle_and_never_fall_back(CostEngine):
     plain, plain_fb = eng.sample_feasible(seed=4, first=0, count=n)
     assign, fallback = eng.sample_feasible(seed=4, first=0, count=n, row_filter=filters)
     assert int(plain_fb.sum().item()) > n and int(fallback.sum().item()) == 0
+    assert (eng.sample_feasible(seed=4, first=0, count=n, row_filter="plan")[0] == assign).all()
     scores = eng.score(assign).cpu().numpy()
     assert (scores[:, 5] == 0).all()
     assign = assign.cpu().numpy()
