@@ -484,8 +484,12 @@ def main():
         from autoparallel_amd import windowed
 
         legs = {}
-        for label, feasible in (("plain_draws", False), ("feasible_draws", True)):
-            scores, st = windowed.score_in_windows(200000, 3000, args.windowed, workers=14, feasible=feasible)
+        # the third leg: the same generator with another seed, a DAG of the same size whose every node
+        # can be served (seed 0, the configuration's, has one that cannot)
+        for label, feasible, dag_seed in (("plain_draws", False, 0), ("feasible_draws", True, 0),
+                                          ("feasible_draws_dag_seed_1", True, 1)):
+            scores, st = windowed.score_in_windows(200000, 3000, args.windowed, workers=14, feasible=feasible,
+                                                   seed=dag_seed)
             st.update({
                 "assignments": int(scores.shape[0]),
                 "entries_per_s_device_build": st["entries"] / st["build_device_s"],
@@ -494,7 +498,7 @@ def main():
                 "forbidden_entries_per_assignment_mean": float(scores[:, 5].mean()),
                 "objective_min": float(scores[:, 4].min()), "objective_mean": float(scores[:, 4].mean()),
             })
-            if feasible:
+            if feasible and st.get("unservable_nodes"):
                 st["note"] = ("unservable_nodes: none of their strategies finds, for every argument, a strategy of "
                               "the producer that offers the Partial placements it asks for; they select a forbidden "
                               "entry in every assignment of this DAG, so no assignment of it is free of them")

@@ -130,6 +130,20 @@ def test_config5_at_full_size_in_windows():
     assert np.isfinite(planned).all()
 
 
+def test_planned_draws_on_a_dag_of_the_same_size_that_has_feasible_assignments():
+    """The same generator with seed 1: 200 000 nodes, every one of which can be served.
+    With the plan no node of any assignment falls back and no forbidden entry is selected."""
+    n = 1024
+    scores, st = windowed.score_in_windows(200000, 3000, n, workers=14, feasible=True, seed=1)
+    print(f"  seed 1: {st['entries']} entries, {st['plan_confined_nodes']} confined nodes, "
+          f"sampling {st['sample_device_s']:.2f} s", flush=True)
+    assert st["nodes"] == 200000 and st["windows"] == 67 and st["entries"] > 2e10
+    assert st["plan_stuck_nodes"] == 0 and st["unservable_nodes"] == []
+    assert st["assignments_without_fallback"] == n and st["fallback_nodes_per_assignment_mean"] == 0.0
+    assert (scores[:, 5] == 0).all() and np.isfinite(scores).all()
+    assert len({float(x) for x in scores[:, 4]}) == n  # and they are different assignments
+
+
 def test_the_node_of_config5_that_no_assignment_can_serve():
     """Node 194 348 of the 200 000-node DAG, with its producers as stand-ins, from the
     flags the device writes: each of its strategies has an argument whose entries are
