@@ -74,6 +74,7 @@ def score_in_windows(
     progress=None,
     feasible: bool = False,
     plan: bool = True,
+    first: int = 0,
 ):
     """Scores ``n_assign`` on-device drawn assignments of the n_total-node stress
     DAG, window by window.  Returns (scores float64[n_assign, 6] on the host,
@@ -85,7 +86,9 @@ def score_in_windows(
     ``plan`` (with ``feasible``): before the first window, the nodes that could run
     out of strategies are found from the spec words of the whole DAG and their
     producers confined to the strategies that serve them (feasible_plan), so that
-    no node falls back to the plain draw."""
+    no node falls back to the plain draw.  ``first``: counter of the first assignment
+    (assignment a is drawn from the counter first + a), for a large sample taken in
+    several runs."""
     import torch
 
     from autoparallel_amd.engine import CostEngine
@@ -100,6 +103,14 @@ def score_in_windows(
     out = None
     choices = fallbacks = None
     if feasible:
+        need = 2 * n_total * n_assign
+        free = torch.cuda.mem_get_info()[0]
+        if need > 0.5 * free:
+            raise MemoryError(
+                f"feasible draws keep the choice of every node for every assignment on the device: {need / 2**30:.0f} GiB "
+                f"for {n_total} nodes x {n_assign} assignments, with {free / 2**30:.0f} GiB free of which the windows "
+                f"need half; take the sample in runs of at most {int(0.5 * free) // (2 * n_total)} assignments "
+                f"(first=...)")
         # int16 storage of the uint16 choices: torch gathers rows of int16, not of uint16
         choices = torch.zeros((n_total, n_assign), dtype=torch.int16, device="cuda")
         fallbacks = torch.zeros(n_assign, dtype=torch.int64, device="cuda")
@@ -140,7 +151,7 @@ def score_in_windows(
                 # the stand-ins' rows are the choices made for their nodes in earlier windows
                 local = choices[torch.from_numpy(gid.astype(np.int64)).to(choices.device)].contiguous()
                 keep = {i: filters[int(gid[i])] for i in range(n_standin, g.num_nodes) if int(gid[i]) in filters}
-                _, fb = eng.sample_feasible(assign_seed, 0, n_assign, node_gid=gid, first_node=n_standin,
+                _, fb = eng.sample_feasible(assign_seed, first, n_assign, node_gid=gid, first_node=n_standin,
                                             assign=local.view(torch.uint16), row_filter=keep)
                 choices[lo:hi] = local[n_standin:]
                 fallbacks += fb
@@ -148,7 +159,7 @@ def score_in_windows(
                 out = eng.score_window(local.view(torch.uint16), n_standin, init=out)
             else:
                 ev[2].record()
-                out = eng.score_random_window(assign_seed, 0, n_assign, gid, n_standin, init=out)
+                out = eng.score_random_window(assign_seed, first, n_assign, gid, n_standin, init=out)
             ev[3].record()
             torch.cuda.synchronize()
             eng.check_status()
@@ -189,6 +200,7 @@ def main():
     ap.add_argument("--workers", type=int, default=min(14, os.cpu_count() or 1))
     ap.add_argument("--max-windows", type=int, default=None)
     ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--first", type=int, default=0, help="counter of the first assignment")
     ap.add_argument("--feasible", action="store_true",
                     help="draw the assignments node by node among the strategies without a forbidden entry")
     ap.add_argument("--no-plan", action="store_true",
@@ -202,7 +214,7 @@ def main():
 
     scores, st = score_in_windows(args.nodes, args.window, args.assignments, seed=args.seed,
                                   workers=args.workers, max_windows=args.max_windows, progress=progress,
-                                  feasible=args.feasible, plan=not args.no_plan)
+                                  feasible=args.feasible, plan=not args.no_plan, first=args.first)
     obj = scores[:, 4]
     st.update({
         "workload": f"stress DAG, {args.nodes} nodes, mesh (4,8,8), windows of {args.window}",

@@ -99,6 +99,12 @@ def test_feasible_draws_in_windows_equal_one_pass():
             if plan:
                 assert st["plan_confined_nodes"] == len(filters) and st["plan_stuck_nodes"] == len(stuck)
     assert fallbacks[True] < fallbacks[False] / 2
+    # a sample taken in several runs: assignments 100 .. 163 by themselves are those of the run from 0
+    part, _ = windowed.score_in_windows(N_TOTAL, 60, 64, seed=SEED, assign_seed=1, s_max=S_MAX, workers=1,
+                                        feasible=True, first=100)
+    assert (part.view(np.uint64) == whole[100:164].view(np.uint64)).all()
+    part, _ = windowed.score_in_windows(N_TOTAL, 60, 64, seed=SEED, assign_seed=1, s_max=S_MAX, workers=1, first=100)
+    assert (part.view(np.uint64) == plain[100:164].view(np.uint64)).all()
 
 
 def test_config5_at_full_size_in_windows():
