@@ -75,6 +75,7 @@ def score_in_windows(
     feasible: bool = False,
     plan: bool = True,
     first: int = 0,
+    max_batch: Optional[int] = None,
 ):
     """Scores ``n_assign`` on-device drawn assignments of the n_total-node stress
     DAG, window by window.  Returns (scores float64[n_assign, 6] on the host,
@@ -87,8 +88,9 @@ def score_in_windows(
     out of strategies are found from the spec words of the whole DAG and their
     producers confined to the strategies that serve them (feasible_plan), so that
     no node falls back to the plain draw.  ``first``: counter of the first assignment
-    (assignment a is drawn from the counter first + a), for a large sample taken in
-    several runs."""
+    (assignment a is drawn from the counter first + a).  ``max_batch``: the largest
+    number of assignments of a pass of feasible draws (default: what 45 % of the
+    free device memory holds the choices of)."""
     import torch
 
     from autoparallel_amd.engine import CostEngine
@@ -100,21 +102,22 @@ def score_in_windows(
     stats = {"nodes": 0, "edges": 0, "entries": 0, "standin_nodes": 0, "windows": 0, "table_doubles": 0,
              "build_device_s": 0.0, "score_device_s": 0.0, "wait_for_window_s": 0.0, "engine_construct_s": 0.0,
              "modes": {}}
-    out = None
-    choices = fallbacks = None
+    # Feasible draws keep the choice of every node for every assignment on the device (a later
+    # window's stand-ins carry them): a sample too large for that is taken in batches, each a
+    # pass over all windows, which are kept on the host after the first pass.
+    batch = n_assign
     if feasible:
-        need = 2 * n_total * n_assign
         free = torch.cuda.mem_get_info()[0]
-        if need > 0.5 * free:
-            raise MemoryError(
-                f"feasible draws keep the choice of every node for every assignment on the device: {need / 2**30:.0f} GiB "
-                f"for {n_total} nodes x {n_assign} assignments, with {free / 2**30:.0f} GiB free of which the windows "
-                f"need half; take the sample in runs of at most {int(0.5 * free) // (2 * n_total)} assignments "
-                f"(first=...)")
-        # int16 storage of the uint16 choices: torch gathers rows of int16, not of uint16
-        choices = torch.zeros((n_total, n_assign), dtype=torch.int16, device="cuda")
-        fallbacks = torch.zeros(n_assign, dtype=torch.int64, device="cuda")
+        cap = max(1, int(0.45 * free) // (2 * n_total))
+        if max_batch is not None:
+            cap = max(1, min(cap, int(max_batch)))
+        if n_assign > cap:
+            batch = 1 << (cap.bit_length() - 1)
         stats["sample_device_s"] = 0.0
+    n_batches = -(-n_assign // batch)
+    stats["assignment_batches"] = n_batches
+    kept = [] if n_batches > 1 else None
+    outs, fbs = [], []
     t_wall = time.perf_counter()
     pool = None
     if workers > 1 and len(tasks) > 1:
@@ -136,60 +139,80 @@ def score_in_windows(
             # for every argument, a producer's strategy that offers the Partials it asks for
             stats["unservable_nodes"] = [v for v in stuck if feasible_plan.unservable(masks, v)]
             del masks
-        results = pool.imap(_make_window, tasks) if pool else map(_make_window, tasks)
-        t_mark = time.perf_counter()
-        for lo, hi, g, gid, n_standin in results:
-            stats["wait_for_window_s"] += time.perf_counter() - t_mark  # the host's generation and packing
-            t_mark = time.perf_counter()
-            eng = CostEngine(g)
-            stats["engine_construct_s"] += time.perf_counter() - t_mark  # layout of the problem and its upload
-            ev = [torch.cuda.Event(enable_timing=True) for _ in range(4)]
-            ev[0].record()
-            eng.build(clamp_inf=True)
-            ev[1].record()
+        for b in range(n_batches):
+            first_b, n_b = first + b * batch, min(batch, n_assign - b * batch)
+            out = None
+            choices = fallbacks = None
             if feasible:
-                # the stand-ins' rows are the choices made for their nodes in earlier windows
-                local = choices[torch.from_numpy(gid.astype(np.int64)).to(choices.device)].contiguous()
-                keep = {i: filters[int(gid[i])] for i in range(n_standin, g.num_nodes) if int(gid[i]) in filters}
-                _, fb = eng.sample_feasible(assign_seed, first, n_assign, node_gid=gid, first_node=n_standin,
-                                            assign=local.view(torch.uint16), row_filter=keep)
-                choices[lo:hi] = local[n_standin:]
-                fallbacks += fb
-                ev[2].record()
-                out = eng.score_window(local.view(torch.uint16), n_standin, init=out)
+                # int16 storage of the uint16 choices: torch gathers rows of int16, not of uint16
+                choices = torch.zeros((n_total, n_b), dtype=torch.int16, device="cuda")
+                fallbacks = torch.zeros(n_b, dtype=torch.int64, device="cuda")
+            if b == 0:
+                results = pool.imap(_make_window, tasks) if pool else map(_make_window, tasks)
             else:
-                ev[2].record()
-                out = eng.score_random_window(assign_seed, first, n_assign, gid, n_standin, init=out)
-            ev[3].record()
-            torch.cuda.synchronize()
-            eng.check_status()
-            stats["build_device_s"] += ev[0].elapsed_time(ev[1]) * 1e-3
-            if feasible:
-                stats["sample_device_s"] += ev[1].elapsed_time(ev[2]) * 1e-3
-            stats["score_device_s"] += ev[2].elapsed_time(ev[3]) * 1e-3
-            real = g.edge_node >= n_standin  # the stand-ins' own input edges are not the DAG's
-            stats["nodes"] += hi - lo
-            stats["standin_nodes"] += n_standin
-            stats["edges"] += int(real.sum())
-            stats["entries"] += int((g.edge_sdst.astype(np.int64) * g.edge_ssrc)[real].sum())
-            stats["table_doubles"] += 0 if eng.table is None else int(eng.table.numel())
-            stats["modes"][eng.table_mode] = stats["modes"].get(eng.table_mode, 0) + 1
-            stats["windows"] += 1
-            if progress:
-                progress(stats, time.perf_counter() - t_wall)
-            del eng
+                results = kept
             t_mark = time.perf_counter()
+            for item in results:
+                lo, hi, g, gid, n_standin = item
+                if b == 0 and kept is not None:
+                    kept.append(item)
+                stats["wait_for_window_s"] += time.perf_counter() - t_mark  # the host's generation and packing
+                t_mark = time.perf_counter()
+                eng = CostEngine(g)
+                stats["engine_construct_s"] += time.perf_counter() - t_mark  # layout of the problem and its upload
+                ev = [torch.cuda.Event(enable_timing=True) for _ in range(4)]
+                ev[0].record()
+                eng.build(clamp_inf=True)
+                ev[1].record()
+                if feasible:
+                    # the stand-ins' rows are the choices made for their nodes in earlier windows
+                    local = choices[torch.from_numpy(gid.astype(np.int64)).to(choices.device)].contiguous()
+                    keep = {i: filters[int(gid[i])] for i in range(n_standin, g.num_nodes) if int(gid[i]) in filters}
+                    _, fb = eng.sample_feasible(assign_seed, first_b, n_b, node_gid=gid, first_node=n_standin,
+                                                assign=local.view(torch.uint16), row_filter=keep)
+                    choices[lo:hi] = local[n_standin:]
+                    fallbacks += fb
+                    ev[2].record()
+                    out = eng.score_window(local.view(torch.uint16), n_standin, init=out)
+                    del local
+                else:
+                    ev[2].record()
+                    out = eng.score_random_window(assign_seed, first_b, n_b, gid, n_standin, init=out)
+                ev[3].record()
+                torch.cuda.synchronize()
+                eng.check_status()
+                stats["build_device_s"] += ev[0].elapsed_time(ev[1]) * 1e-3
+                if feasible:
+                    stats["sample_device_s"] += ev[1].elapsed_time(ev[2]) * 1e-3
+                stats["score_device_s"] += ev[2].elapsed_time(ev[3]) * 1e-3
+                if b == 0:
+                    real = g.edge_node >= n_standin  # the stand-ins' own input edges are not the DAG's
+                    stats["nodes"] += hi - lo
+                    stats["standin_nodes"] += n_standin
+                    stats["edges"] += int(real.sum())
+                    stats["entries"] += int((g.edge_sdst.astype(np.int64) * g.edge_ssrc)[real].sum())
+                    stats["table_doubles"] += 0 if eng.table is None else int(eng.table.numel())
+                    stats["modes"][eng.table_mode] = stats["modes"].get(eng.table_mode, 0) + 1
+                    stats["windows"] += 1
+                if progress:
+                    progress(stats, time.perf_counter() - t_wall)
+                del eng
+                t_mark = time.perf_counter()
+            outs.append(out.cpu().numpy())
+            if feasible:
+                fbs.append(fallbacks.cpu().numpy())
+            del out, choices, fallbacks
     finally:
         if pool is not None:
             pool.terminate()
             pool.join()
     stats["wall_s"] = time.perf_counter() - t_wall
     if feasible:
-        fb = fallbacks.cpu().numpy()
+        fb = np.concatenate(fbs)
         stats["fallback_nodes_per_assignment_mean"] = float(fb.mean())
         stats["fallback_nodes_per_assignment_min"] = int(fb.min())
         stats["assignments_without_fallback"] = int((fb == 0).sum())
-    return out.cpu().numpy(), stats
+    return np.concatenate(outs), stats
 
 
 def main():
@@ -219,7 +242,7 @@ def main():
     st.update({
         "workload": f"stress DAG, {args.nodes} nodes, mesh (4,8,8), windows of {args.window}",
         "assignments": int(scores.shape[0]),
-        "entries_per_s_device_build": st["entries"] / st["build_device_s"],
+        "entries_per_s_device_build": st["entries"] * st["assignment_batches"] / st["build_device_s"],
         "entries_per_s_wall": st["entries"] / st["wall_s"],
         "edge_terms_per_s_scoring": scores.shape[0] * st["edges"] / st["score_device_s"],
         "coefficient_bytes_if_resident": 17 * st["entries"],

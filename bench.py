@@ -492,7 +492,7 @@ def main():
                                                    seed=dag_seed)
             st.update({
                 "assignments": int(scores.shape[0]),
-                "entries_per_s_device_build": st["entries"] / st["build_device_s"],
+                "entries_per_s_device_build": st["entries"] * st["assignment_batches"] / st["build_device_s"],
                 "edge_terms_per_s_scoring": scores.shape[0] * st["edges"] / st["score_device_s"],
                 "fraction_without_forbidden_entry": float((scores[:, 5] == 0).mean()),
                 "forbidden_entries_per_assignment_mean": float(scores[:, 5].mean()),

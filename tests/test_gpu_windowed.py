@@ -99,6 +99,11 @@ def test_feasible_draws_in_windows_equal_one_pass():
             if plan:
                 assert st["plan_confined_nodes"] == len(filters) and st["plan_stuck_nodes"] == len(stuck)
     assert fallbacks[True] < fallbacks[False] / 2
+    # a sample too large for the device is taken in batches, each a pass over the kept windows
+    got, st = windowed.score_in_windows(N_TOTAL, 60, n, seed=SEED, assign_seed=1, s_max=S_MAX, workers=1,
+                                        feasible=True, max_batch=1000)
+    assert st["assignment_batches"] == 8 and (got.view(np.uint64) == whole.view(np.uint64)).all()
+    assert st["nodes"] == N_TOTAL and st["entries"] == g.num_entries
     # a sample taken in several runs: assignments 100 .. 163 by themselves are those of the run from 0
     part, _ = windowed.score_in_windows(N_TOTAL, 60, 64, seed=SEED, assign_seed=1, s_max=S_MAX, workers=1,
                                         feasible=True, first=100)
