@@ -361,7 +361,7 @@ schedule_metrics_lds_kernel(apc_schedule s, const int32_t* __restrict__ order, i
   // steps is for the loads of the block before and not for the ones just issued.
   auto entry = [&](int t) -> int {
     const int tc = t < N ? t : N - 1;
-    return kIdentity ? tc : ord[tc];
+    return (kIdentity || N == 0) ? tc : ord[tc];  // (an empty graph has no entries to read)
   };
   int nxt[kAhead];
 #pragma unroll

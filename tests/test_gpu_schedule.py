@@ -85,6 +85,15 @@ def test_large_batch_properties(golden, copies):
     assert (peak >= ps.initial_bytes).all() and (peak <= ps.initial_bytes + ps.st_bytes.sum()).all()
 
 
+def test_an_empty_graph_takes_no_time():
+    from test_oracle_schedule import _manual
+
+    ps = _manual([], [], [], n_stream=1)
+    times, peak = SM.ScheduleEstimator(ps).evaluate()
+    assert times.tolist() == [[0.0, 0.0, 0.0, 0.0]] and peak.tolist() == [0]
+    assert SO.schedule_metrics(ps)[:4] == (0.0, 0.0, 0.0, 0.0)
+
+
 def _constant_estimator(dur):
     return lambda node: dur if node.op == "call_function" else 0
 
