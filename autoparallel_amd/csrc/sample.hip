@@ -27,6 +27,7 @@ namespace {
 
 constexpr int kSampleArgs = 6;   // argument rows of a node whose columns a lane keeps in registers
 constexpr int kSampleWords = 8;  // words of a node's strategies a lane keeps in registers (512 strategies)
+typedef uint64_t u64x2_t __attribute__((ext_vector_type(2)));
 
 __host__ __device__ __forceinline__ uint32_t finalise32(uint32_t h) {
   h ^= h >> 16;
@@ -97,6 +98,7 @@ pack_allowed_columns_kernel(apc_problem p, const uint8_t* __restrict__ flags,
   const int sdst = ed->sdst, ssrc = ed->ssrc;
   const int W = (sdst + 63) >> 6;
   if (w >= W) return;
+  const int Wc = (W + 1) & ~1;  // words from one column to the next: whole pairs
   const int lane = threadIdx.x & 63;
   const int rows = min(64, sdst - 64 * w);
   const uint8_t* __restrict__ tile = flags + ed->off + (int64_t)(64 * w) * ssrc;
@@ -109,7 +111,7 @@ pack_allowed_columns_kernel(apc_problem p, const uint8_t* __restrict__ flags,
 #pragma unroll 8
     for (int k = 0; k < rows; ++k)
       m |= (uint64_t)((col[(int64_t)k * ssrc] & APC_ENTRY_NONFINITE) == 0) << k;
-    if (mine) out[(int64_t)j * W] = m;
+    if (mine) out[(int64_t)j * Wc] = m;
   }
 }
 
@@ -166,39 +168,60 @@ sample_feasible_kernel(apc_problem p, const uint64_t* __restrict__ colbits,
     if (kAhead && v + 1 < p.n_node) next = load_head(v + 1);
     const int S = head.S, gid = head.gid, e0 = head.e0, e1 = head.e1;
     const int W = (S + 63) >> 6;
+    const int Wc = (W + 1) & ~1;  // words from one column to the next: whole pairs, 16-byte aligned
     // the column of every argument row: that of the producer's choice
-    const uint64_t* col[kSampleArgs];
+    const u64x2_t* col[kSampleArgs];
 #pragma unroll
     for (int i = 0; i < kSampleArgs; ++i) {
-      col[i] = colbits;
+      col[i] = reinterpret_cast<const u64x2_t*>(colbits);
       if (e0 + i < e1) {
         const int u = kAhead ? head.src[i] : p.edges[e0 + i].src_node;
         const int64_t j = u >= 0 ? (int64_t)assign[(size_t)u * n_assign + a] : 0;
-        col[i] = colbits + (kAhead ? head.off[i] : col_off[e0 + i]) + j * W;
+        col[i] = reinterpret_cast<const u64x2_t*>(colbits + (kAhead ? head.off[i] : col_off[e0 + i]) + j * Wc);
       }
     }
-    // word w of the node's allowed strategies
-    auto allowed_word = [&](int w) -> uint64_t {
-      uint64_t m = word_mask(S, w);
-      if (head.keep >= 0) m &= row_filter[head.keep + w];  // the strategies the node may take at all
+    // words 2 q and 2 q + 1 of the node's allowed strategies: a lane reads its columns 16 bytes at
+    // a time (the lanes of a wave read different columns, and such a load costs the same for 8
+    // bytes as for 16)
+    auto allowed_pair = [&](int q) -> u64x2_t {
+      u64x2_t m = {word_mask(S, 2 * q), word_mask(S, 2 * q + 1)};
+      if (head.keep >= 0) {  // the strategies the node may take at all
+        m.x &= row_filter[head.keep + 2 * q];
+        if (2 * q + 1 < W) m.y &= row_filter[head.keep + 2 * q + 1];
+      }
 #pragma unroll
       for (int i = 0; i < kSampleArgs; ++i)
-        if (e0 + i < e1) m &= col[i][w];
+        if (e0 + i < e1) m &= col[i][q];
       for (int e = e0 + kSampleArgs; e < e1; ++e) {  // a node with more argument rows than the registers hold
         const int u = p.edges[e].src_node;
         const int64_t j = u >= 0 ? (int64_t)assign[(size_t)u * n_assign + a] : 0;
-        m &= colbits[col_off[e] + j * W + w];
+        m &= reinterpret_cast<const u64x2_t*>(colbits + col_off[e] + j * Wc)[q];
       }
       return m;
     };
     uint32_t count = 0;
     int pick = 0;
-    if (W <= kSampleWords) {  // wave-uniform: the words stay in registers
+    if (W == 1) {  // up to 64 strategies (most nodes of a traced model): one word, read by itself
+      uint64_t m = word_mask(S, 0);
+      if (head.keep >= 0) m &= row_filter[head.keep];
+#pragma unroll
+      for (int i = 0; i < kSampleArgs; ++i)
+        if (e0 + i < e1) m &= reinterpret_cast<const uint64_t*>(col[i])[0];
+      for (int e = e0 + kSampleArgs; e < e1; ++e) {
+        const int u = p.edges[e].src_node;
+        const int64_t j = u >= 0 ? (int64_t)assign[(size_t)u * n_assign + a] : 0;
+        m &= colbits[col_off[e] + j * Wc];
+      }
+      count = (uint32_t)__popcll(m);
+      if (count > 0) pick = select_bit(m, rank_draw(h0, gid, count));
+    } else if (W <= kSampleWords) {  // wave-uniform: the words stay in registers
       uint64_t m[kSampleWords];
 #pragma unroll
-      for (int w = 0; w < kSampleWords; ++w) {
-        m[w] = w < W ? allowed_word(w) : 0ull;
-        count += (uint32_t)__popcll(m[w]);
+      for (int q = 0; q < kSampleWords / 2; ++q) {
+        const u64x2_t mm = 2 * q < W ? allowed_pair(q) : u64x2_t{0ull, 0ull};
+        m[2 * q] = mm.x;
+        m[2 * q + 1] = mm.y;
+        count += (uint32_t)__popcll(mm.x) + (uint32_t)__popcll(mm.y);
       }
       if (count > 0) {
         uint32_t r = rank_draw(h0, gid, count);
@@ -214,17 +237,25 @@ sample_feasible_kernel(apc_problem p, const uint64_t* __restrict__ colbits,
         }
       }
     } else {  // more than 512 strategies: the words are formed twice
-      for (int w = 0; w < W; ++w) count += (uint32_t)__popcll(allowed_word(w));
+      for (int q = 0; 2 * q < W; ++q) {
+        const u64x2_t mm = allowed_pair(q);
+        count += (uint32_t)__popcll(mm.x) + (uint32_t)__popcll(mm.y);
+      }
       if (count > 0) {
         uint32_t r = rank_draw(h0, gid, count);
-        for (int w = 0; w < W; ++w) {
-          const uint64_t m = allowed_word(w);
-          const uint32_t c = (uint32_t)__popcll(m);
-          if (r < c) {
-            pick = 64 * w + select_bit(m, r);
+        for (int q = 0; 2 * q < W; ++q) {
+          const u64x2_t mm = allowed_pair(q);
+          const uint32_t cx = (uint32_t)__popcll(mm.x), cy = (uint32_t)__popcll(mm.y);
+          if (r < cx) {
+            pick = 128 * q + select_bit(mm.x, r);
             break;
           }
-          r -= c;
+          r -= cx;
+          if (r < cy) {
+            pick = 128 * q + 64 + select_bit(mm.y, r);
+            break;
+          }
+          r -= cy;
         }
       }
     }

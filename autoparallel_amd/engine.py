@@ -765,7 +765,7 @@ class CostEngine:
         lay = self._keep.get("column_layout")
         if lay is None:
             words = (g.edge_sdst.astype(np.int64) + 63) >> 6
-            size = g.edge_ssrc.astype(np.int64) * words
+            size = g.edge_ssrc.astype(np.int64) * ((words + 1) & ~1)  # a column: whole pairs of words
             own = np.ones(g.num_edges, bool) if g.edge_alias is None else g.priced
             off = np.zeros(g.num_edges, np.int64)
             off[own] = np.cumsum(size[own]) - size[own]

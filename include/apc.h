@@ -650,9 +650,12 @@ uint32_t apc_random_assignment(uint64_t seed, int64_t a, int32_t node, int32_t n
  *
  * apc_pack_allowed_columns writes, for every argument row (edge) e and every
  * choice j of its producer, the bit column of the consumer's strategies whose entry
- * (e, out_idx, j) is finite: words colbits[col_off[e] + j * W + w], W =
+ * (e, out_idx, j) is finite: words colbits[col_off[e] + j * Wc + w], w < W =
  * ceil(S_dst / 64), bit (out_idx mod 64) of word out_idx / 64; bits past S_dst are
- * zero.  col_off: int64[n_edge], the caller's layout (S_src * W words per edge;
+ * zero.  Wc = W rounded up to an even number: a column is whole pairs of words, and
+ * with colbits 16-byte aligned and every col_off even the sampler reads it 16 bytes
+ * at a time (the odd word of a column with an odd W is never written and may hold
+ * anything).  col_off: int64[n_edge], the caller's layout (S_src * Wc words per edge;
  * edges that share a block may share their columns); max_words: the largest W.
  * To be called again after anything that rewrites flags.
  *

@@ -131,9 +131,11 @@ def test_bit_columns_are_the_flags_and_wide_nodes_sample_like_the_oracle(CostEng
     for e in range(g.num_edges):
         sdst, ssrc, base = int(g.edge_sdst[e]), int(g.edge_ssrc[e]), int(g.edge_off[e])
         W = (sdst + 63) // 64
+        Wc = (W + 1) & ~1  # a column is whole pairs of words
+        assert off[e] % 2 == 0
         block = (flags[base: base + sdst * ssrc].reshape(sdst, ssrc) & 2) == 0  # [o][j]: allowed
         for j in range(ssrc):
-            words = bits[off[e] + j * W: off[e] + (j + 1) * W]
+            words = bits[off[e] + j * Wc: off[e] + j * Wc + W]
             got = np.unpackbits(words.view(np.uint8), bitorder="little")[: W * 64].astype(bool)
             assert np.array_equal(got[:sdst], block[:, j]) and not got[sdst:].any(), (e, j)
     # and the draws
